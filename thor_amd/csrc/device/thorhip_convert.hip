@@ -1,0 +1,380 @@
+// Type-converter kernels for gfx950 and the thorhip_convert entry point.
+//
+// Replaces TypeConverter::gpuConvertType and its 16 size-specialised kernels
+// (Utilities/TensorOperations/DataTypeConversions/TypeConverterKernels.cu:39-823,906-936,965-1338,1340-1433).
+//
+// Design for MI355X: the conversion is a pure HBM stream (6 B/element for fp32<->16-bit), so each lane moves whole
+// 16-byte words -- two dwordx4 loads and one dwordx4 store per slot for fp32->fp16 -- through a grid-stride loop
+// sized to a few resident waves per SIMD, with two slots in flight per lane.  A slot is a fixed, index-aligned group
+// of VEC elements; slots that straddle the [begin, end) range are handled element-wise, so nothing outside the range
+// is touched (the reference kernels over-read and over-write up to 15 elements into the tensor's 128-byte pad).
+#include "thorhip.h"
+#include "thorhip_internal.h"
+#include "thorhip_numeric.h"
+
+#include <cstdlib>
+#include <mutex>
+
+namespace {
+
+using namespace thor;
+
+constexpr int kBlockThreads = 256;
+
+template <int BYTES>
+struct Word;
+template <>
+struct Word<1> {
+    typedef u8 type;
+};
+template <>
+struct Word<2> {
+    typedef u16 type;
+};
+template <>
+struct Word<4> {
+    typedef u32 type;
+};
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+template <>
+struct Word<8> {
+    typedef u32x2 type;
+};
+template <>
+struct Word<16> {
+    typedef u32x4 type;
+};
+
+// VEC elements of T moved as whole machine words of up to 16 bytes.
+template <typename T, int VEC>
+struct alignas((sizeof(T) * VEC) >= 16 ? 16 : (sizeof(T) * VEC)) Pack {
+    static constexpr int kBytes = sizeof(T) * VEC;
+    static constexpr int kWordBytes = kBytes >= 16 ? 16 : kBytes;
+    static constexpr int kWords = kBytes / kWordBytes;
+    typedef typename Word<kWordBytes>::type word_t;
+    T v[VEC];
+
+    __device__ __forceinline__ void load(const T* p) {
+        const word_t* wp = reinterpret_cast<const word_t*>(p);
+        word_t* mine = reinterpret_cast<word_t*>(v);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) mine[w] = __builtin_nontemporal_load(wp + w);
+    }
+    __device__ __forceinline__ void store(T* p) const {
+        word_t* wp = reinterpret_cast<word_t*>(p);
+        const word_t* mine = reinterpret_cast<const word_t*>(v);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) __builtin_nontemporal_store(mine[w], wp + w);
+    }
+};
+
+template <typename From, typename To>
+struct Slot {
+    static constexpr int kMin = sizeof(From) < sizeof(To) ? sizeof(From) : sizeof(To);
+    static constexpr int kMax = sizeof(From) < sizeof(To) ? sizeof(To) : sizeof(From);
+    static constexpr int kA = 16 / kMin;
+    static constexpr int kB = 64 / kMax;
+    static constexpr int kVec = kA < kB ? kA : kB;
+};
+
+// Index-aligned slots [firstSlot, lastSlot) cover elements [begin, end).  UNROLL slots are in flight per lane.
+template <typename From, typename To, int VEC, int UNROLL>
+__global__ __launch_bounds__(kBlockThreads) void convertSlots(const From* src, To* dst, long begin, long end, long firstSlot,
+                                                               long lastSlot) {
+    const long stride = (long)gridDim.x * kBlockThreads;
+    for (long s0 = firstSlot + (long)blockIdx.x * kBlockThreads + threadIdx.x; s0 < lastSlot; s0 += stride * UNROLL) {
+        Pack<From, VEC> in[UNROLL];
+        bool whole[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const long s = s0 + (long)u * stride;
+            const long e0 = s * VEC;
+            whole[u] = (s < lastSlot) && (e0 >= begin) && (e0 + VEC <= end);
+            if (whole[u]) in[u].load(src + e0);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const long s = s0 + (long)u * stride;
+            const long e0 = s * VEC;
+            if (whole[u]) {
+                Pack<To, VEC> out;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) out.v[k] = convertElement<To>(in[u].v[k]);
+                out.store(dst + e0);
+            } else if (s < lastSlot) {
+                // ragged first / last slot: element-wise, and read everything before writing so that an in-place
+                // conversion between equally sized types stays correct
+                From tmp[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const long e = e0 + k;
+                    if (e >= begin && e < end) tmp[k] = src[e];
+                }
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const long e = e0 + k;
+                    if (e >= begin && e < end) dst[e] = convertElement<To>(tmp[k]);
+                }
+            }
+        }
+    }
+}
+
+// Element-wise fallback for buffers whose base address is not word aligned.
+template <typename From, typename To>
+__global__ __launch_bounds__(kBlockThreads) void convertScalar(const From* src, To* dst, long begin, long end) {
+    const long stride = (long)gridDim.x * kBlockThreads;
+    for (long e = begin + (long)blockIdx.x * kBlockThreads + threadIdx.x; e < end; e += stride) dst[e] = convertElement<To>(src[e]);
+}
+
+// One block converts [0, count) in place between differently sized types: every lane reads all of its elements, the
+// block synchronises, then every lane writes.  count is at most kStagedElements.
+constexpr int kStagedPerThread = 8;
+constexpr int kStagedElements = kBlockThreads * kStagedPerThread;
+template <typename From, typename To>
+__global__ __launch_bounds__(kBlockThreads) void convertStagedInPlace(const From* src, To* dst, long count) {
+    From tmp[kStagedPerThread];
+#pragma unroll
+    for (int k = 0; k < kStagedPerThread; ++k) {
+        const long e = (long)k * kBlockThreads + threadIdx.x;
+        if (e < count) tmp[k] = src[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kStagedPerThread; ++k) {
+        const long e = (long)k * kBlockThreads + threadIdx.x;
+        if (e < count) dst[e] = convertElement<To>(tmp[k]);
+    }
+}
+
+struct LaunchShape {
+    int compute_units = 0;
+    int blocks_per_cu = 0;
+};
+
+LaunchShape& launchShape() {
+    static LaunchShape shape;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+            shape.compute_units = prop.multiProcessorCount;
+        } else {
+            (void)hipGetLastError();
+            shape.compute_units = 256;
+        }
+        // Resident blocks of 256 threads per CU the grid-stride loop is sized for.  8 blocks = 32 waves = 8 per SIMD.
+        shape.blocks_per_cu = 8;
+        if (const char* env = std::getenv("THORHIP_CONVERT_BLOCKS_PER_CU")) {
+            const int v = std::atoi(env);
+            if (v >= 1 && v <= 64) shape.blocks_per_cu = v;
+        }
+    });
+    return shape;
+}
+
+unsigned gridFor(long work_items, int unroll) {
+    const LaunchShape& shape = launchShape();
+    const long per_block = (long)kBlockThreads * unroll;
+    long blocks = (work_items + per_block - 1) / per_block;
+    const long cap = (long)shape.compute_units * shape.blocks_per_cu;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return (unsigned)blocks;
+}
+
+template <typename T>
+bool alignedTo(const T* p, size_t bytes) {
+    return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
+}
+
+// Out-of-place (or same-size in-place) conversion of elements [begin, end).
+template <typename From, typename To>
+int launchRange(const From* src, To* dst, long begin, long end, hipStream_t stream) {
+    if (end <= begin) return 0;
+    constexpr int VEC = Slot<From, To>::kVec;
+    constexpr int UNROLL = 2;
+    const size_t src_word = sizeof(From) * VEC >= 16 ? 16 : sizeof(From) * VEC;
+    const size_t dst_word = sizeof(To) * VEC >= 16 ? 16 : sizeof(To) * VEC;
+    if (alignedTo(src, src_word) && alignedTo(dst, dst_word)) {
+        const long firstSlot = begin / VEC;
+        const long lastSlot = (end + VEC - 1) / VEC;
+        const unsigned grid = gridFor(lastSlot - firstSlot, UNROLL);
+        hipLaunchKernelGGL((convertSlots<From, To, VEC, UNROLL>), dim3(grid), dim3(kBlockThreads), 0, stream, src, dst, begin, end,
+                           firstSlot, lastSlot);
+    } else {
+        const unsigned grid = gridFor(end - begin, 1);
+        hipLaunchKernelGGL((convertScalar<From, To>), dim3(grid), dim3(kBlockThreads), 0, stream, src, dst, begin, end);
+    }
+    THORHIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// In-place conversion between differently sized types.  Element i's destination bytes overlap the source bytes of other
+// elements, so the range is cut into launches whose destination span is disjoint from their own source span; stream
+// order between launches does the rest.  Narrowing walks upward from a staged first chunk with spans growing by the
+// size ratio; widening walks downward and finishes with the staged chunk
+// (TypeConverterKernels.cu:826-904,939-962 use the same geometric schedule).
+template <typename From, typename To>
+int launchInPlace(const From* src, To* dst, long n, hipStream_t stream) {
+    constexpr long ss = sizeof(From), ds = sizeof(To);
+    if (ds < ss) {
+        long done = n < kStagedElements ? n : kStagedElements;
+        hipLaunchKernelGGL((convertStagedInPlace<From, To>), dim3(1), dim3(kBlockThreads), 0, stream, src, dst, done);
+        THORHIP_TRY(hipGetLastError());
+        while (done < n) {
+            // [done, next): destination bytes end at next*ds <= done*ss, the start of this launch's source bytes
+            long next = done * ss / ds;
+            if (next > n) next = n;
+            if (int rc = launchRange<From, To>(src, dst, done, next, stream)) return rc;
+            done = next;
+        }
+    } else {
+        long top = n;
+        while (top > kStagedElements) {
+            // [low, top): destination bytes start at low*ds >= top*ss, the end of this launch's source bytes
+            long low = (top * ss + ds - 1) / ds;
+            if (low < kStagedElements) low = kStagedElements;  // a later start keeps the spans disjoint
+            if (int rc = launchRange<From, To>(src, dst, low, top, stream)) return rc;
+            top = low;
+        }
+        hipLaunchKernelGGL((convertStagedInPlace<From, To>), dim3(1), dim3(kBlockThreads), 0, stream, src, dst, top);
+        THORHIP_TRY(hipGetLastError());
+    }
+    return 0;
+}
+
+template <typename From, typename To>
+int convertPair(const void* src_v, void* dst_v, long n, hipStream_t stream) {
+    const From* src = static_cast<const From*>(src_v);
+    To* dst = static_cast<To*>(dst_v);
+    if (src_v == dst_v) {
+        if (sizeof(From) == sizeof(To)) return launchRange<From, To>(src, dst, 0, n, stream);
+        return launchInPlace<From, To>(src, dst, n, stream);
+    }
+    const char* sb = static_cast<const char*>(src_v);
+    const char* se = sb + n * (long)sizeof(From);
+    const char* db = static_cast<const char*>(dst_v);
+    const char* de = db + n * (long)sizeof(To);
+    if (sb < de && db < se) {
+        return thorhip::fail(-1, "thorhip_convert: source and destination overlap without being the same buffer");
+    }
+    return launchRange<From, To>(src, dst, 0, n, stream);
+}
+
+template <typename From>
+int dispatchDst(const void* src, void* dst, int dst_dtype, long n, hipStream_t stream) {
+    switch (dst_dtype) {
+        case THORHIP_FP16:
+            return convertPair<From, f16>(src, dst, n, stream);
+        case THORHIP_BF16:
+            return convertPair<From, bf16>(src, dst, n, stream);
+        case THORHIP_FP8_E4M3:
+            return convertPair<From, e4m3>(src, dst, n, stream);
+        case THORHIP_FP8_E5M2:
+            return convertPair<From, e5m2>(src, dst, n, stream);
+        case THORHIP_FP32:
+            return convertPair<From, float>(src, dst, n, stream);
+        case THORHIP_FP64:
+            return convertPair<From, double>(src, dst, n, stream);
+        case THORHIP_INT8:
+            return convertPair<From, i8>(src, dst, n, stream);
+        case THORHIP_INT16:
+            return convertPair<From, i16>(src, dst, n, stream);
+        case THORHIP_INT32:
+            return convertPair<From, i32>(src, dst, n, stream);
+        case THORHIP_INT64:
+            return convertPair<From, i64>(src, dst, n, stream);
+        case THORHIP_UINT8:
+            return convertPair<From, u8>(src, dst, n, stream);
+        case THORHIP_UINT16:
+            return convertPair<From, u16>(src, dst, n, stream);
+        case THORHIP_UINT32:
+            return convertPair<From, u32>(src, dst, n, stream);
+        case THORHIP_UINT64:
+            return convertPair<From, u64>(src, dst, n, stream);
+        case THORHIP_BOOLEAN:
+            return convertPair<From, boolean>(src, dst, n, stream);
+        default:
+            return thorhip::fail(-1, "thorhip_convert: unknown destination dtype %d", dst_dtype);
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int thorhip_dtype_size(int dtype) {
+    switch (dtype) {
+        case THORHIP_FP8_E4M3:
+        case THORHIP_FP8_E5M2:
+        case THORHIP_INT8:
+        case THORHIP_UINT8:
+        case THORHIP_BOOLEAN:
+            return 1;
+        case THORHIP_FP16:
+        case THORHIP_BF16:
+        case THORHIP_INT16:
+        case THORHIP_UINT16:
+            return 2;
+        case THORHIP_FP32:
+        case THORHIP_INT32:
+        case THORHIP_UINT32:
+            return 4;
+        case THORHIP_FP64:
+        case THORHIP_INT64:
+        case THORHIP_UINT64:
+            return 8;
+        default:
+            return -1;
+    }
+}
+
+int thorhip_convert(const void* src, void* dst, int src_dtype, int dst_dtype, int64_t num_elements, void* stream_v) {
+    THORHIP_REQUIRE(num_elements >= 0, "thorhip_convert: negative element count %lld", (long long)num_elements);
+    THORHIP_REQUIRE(src_dtype != dst_dtype, "thorhip_convert: source and destination dtype are both %d", src_dtype);
+    THORHIP_REQUIRE(thorhip_dtype_size(src_dtype) > 0, "thorhip_convert: unknown source dtype %d", src_dtype);
+    THORHIP_REQUIRE(thorhip_dtype_size(dst_dtype) > 0, "thorhip_convert: unknown destination dtype %d", dst_dtype);
+    if (num_elements == 0) return 0;
+    THORHIP_REQUIRE(src != nullptr && dst != nullptr, "thorhip_convert: NULL buffer");
+    hipStream_t stream = (hipStream_t)stream_v;
+    const long n = (long)num_elements;
+    switch (src_dtype) {
+        case THORHIP_FP16:
+            return dispatchDst<f16>(src, dst, dst_dtype, n, stream);
+        case THORHIP_BF16:
+            return dispatchDst<bf16>(src, dst, dst_dtype, n, stream);
+        case THORHIP_FP8_E4M3:
+            return dispatchDst<e4m3>(src, dst, dst_dtype, n, stream);
+        case THORHIP_FP8_E5M2:
+            return dispatchDst<e5m2>(src, dst, dst_dtype, n, stream);
+        case THORHIP_FP32:
+            return dispatchDst<float>(src, dst, dst_dtype, n, stream);
+        case THORHIP_FP64:
+            return dispatchDst<double>(src, dst, dst_dtype, n, stream);
+        case THORHIP_INT8:
+            return dispatchDst<i8>(src, dst, dst_dtype, n, stream);
+        case THORHIP_INT16:
+            return dispatchDst<i16>(src, dst, dst_dtype, n, stream);
+        case THORHIP_INT32:
+            return dispatchDst<i32>(src, dst, dst_dtype, n, stream);
+        case THORHIP_INT64:
+            return dispatchDst<i64>(src, dst, dst_dtype, n, stream);
+        case THORHIP_UINT8:
+            return dispatchDst<u8>(src, dst, dst_dtype, n, stream);
+        case THORHIP_UINT16:
+            return dispatchDst<u16>(src, dst, dst_dtype, n, stream);
+        case THORHIP_UINT32:
+            return dispatchDst<u32>(src, dst, dst_dtype, n, stream);
+        case THORHIP_UINT64:
+            return dispatchDst<u64>(src, dst, dst_dtype, n, stream);
+        case THORHIP_BOOLEAN:
+            return dispatchDst<boolean>(src, dst, dst_dtype, n, stream);
+        default:
+            return thorhip::fail(-1, "thorhip_convert: unknown source dtype %d", src_dtype);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,349 @@
+// Device runtime half of the thorhip C ABI: devices, memory, streams, events, hipRTC compilation, module loading and
+// kernel launch.  This is the MI355X counterpart of the function table the reference dlopen()s from the CUDA driver
+// (Utilities/CudaDriver/CudaDrivertApi.h:9-158) plus its NVRTC/nvJitLink pipeline
+// (Utilities/Expression/EquationCompiler.cpp:1756-1908).
+#include "thorhip.h"
+#include "thorhip_internal.h"
+
+#include <hip/hiprtc.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace thorhip {
+std::string& lastError() {
+    static thread_local std::string slot;
+    return slot;
+}
+}  // namespace thorhip
+
+using thorhip::fail;
+
+extern "C" {
+
+int thorhip_abi_version(void) { return THORHIP_ABI_VERSION; }
+
+const char* thorhip_last_error(void) { return thorhip::lastError().c_str(); }
+
+// ---- devices ---------------------------------------------------------------------------------------------------------
+int thorhip_device_count(int* count) {
+    THORHIP_REQUIRE(count != nullptr, "thorhip_device_count: count is NULL");
+    int n = 0;
+    hipError_t err = hipGetDeviceCount(&n);
+    if (err == hipErrorNoDevice) {
+        (void)hipGetLastError();
+        *count = 0;
+        return 0;
+    }
+    THORHIP_TRY(err);
+    *count = n;
+    return 0;
+}
+
+int thorhip_set_device(int device) {
+    THORHIP_TRY(hipSetDevice(device));
+    return 0;
+}
+
+int thorhip_get_device(int* device) {
+    THORHIP_REQUIRE(device != nullptr, "thorhip_get_device: device is NULL");
+    THORHIP_TRY(hipGetDevice(device));
+    return 0;
+}
+
+int thorhip_device_get_info(int device, thorhip_device_info* info) {
+    THORHIP_REQUIRE(info != nullptr, "thorhip_device_get_info: info is NULL");
+    hipDeviceProp_t prop;
+    THORHIP_TRY(hipGetDeviceProperties(&prop, device));
+    std::memset(info, 0, sizeof *info);
+    info->compute_units = prop.multiProcessorCount;
+    info->wavefront_size = prop.warpSize;
+    info->max_threads_per_block = prop.maxThreadsPerBlock;
+    info->lds_bytes_per_block = (int)prop.sharedMemPerBlock;
+    info->l2_bytes = prop.l2CacheSize;
+    info->clock_khz = prop.clockRate;
+    info->memory_clock_khz = prop.memoryClockRate;
+    info->memory_bus_width_bits = prop.memoryBusWidth;
+    info->total_global_mem = prop.totalGlobalMem;
+    std::snprintf(info->arch_name, sizeof info->arch_name, "%s", prop.gcnArchName);
+    std::snprintf(info->name, sizeof info->name, "%s", prop.name);
+    return 0;
+}
+
+int thorhip_device_synchronize(void) {
+    THORHIP_TRY(hipDeviceSynchronize());
+    return 0;
+}
+
+// ---- memory ----------------------------------------------------------------------------------------------------------
+int thorhip_malloc(void** ptr, size_t bytes) {
+    THORHIP_REQUIRE(ptr != nullptr, "thorhip_malloc: ptr is NULL");
+    *ptr = nullptr;
+    if (bytes == 0) return 0;
+    hipError_t err = hipMalloc(ptr, bytes);
+    if (err != hipSuccess) {
+        size_t free_b = 0, total_b = 0;
+        (void)hipMemGetInfo(&free_b, &total_b);
+        (void)hipGetLastError();
+        return fail(-(int)err - 1000, "hipMalloc(%zu bytes) failed: %s; device memory free %zu of %zu bytes", bytes,
+                    hipGetErrorName(err), free_b, total_b);
+    }
+    return 0;
+}
+
+int thorhip_free(void* ptr) {
+    if (ptr == nullptr) return 0;
+    THORHIP_TRY(hipFree(ptr));
+    return 0;
+}
+
+int thorhip_host_malloc(void** ptr, size_t bytes) {
+    THORHIP_REQUIRE(ptr != nullptr, "thorhip_host_malloc: ptr is NULL");
+    *ptr = nullptr;
+    if (bytes == 0) return 0;
+    THORHIP_TRY(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+    return 0;
+}
+
+int thorhip_host_free(void* ptr) {
+    if (ptr == nullptr) return 0;
+    THORHIP_TRY(hipHostFree(ptr));
+    return 0;
+}
+
+int thorhip_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream) {
+    if (bytes == 0) return 0;
+    THORHIP_REQUIRE(dst != nullptr && src != nullptr, "thorhip_memcpy_async: NULL pointer");
+    hipMemcpyKind k;
+    switch (kind) {
+        case THORHIP_H2D:
+            k = hipMemcpyHostToDevice;
+            break;
+        case THORHIP_D2H:
+            k = hipMemcpyDeviceToHost;
+            break;
+        case THORHIP_D2D:
+            k = hipMemcpyDeviceToDevice;
+            break;
+        default:
+            return fail(-1, "thorhip_memcpy_async: unknown copy kind %d", kind);
+    }
+    THORHIP_TRY(hipMemcpyAsync(dst, src, bytes, k, (hipStream_t)stream));
+    return 0;
+}
+
+int thorhip_memset_async(void* dst, int byte_value, size_t bytes, void* stream) {
+    if (bytes == 0) return 0;
+    THORHIP_REQUIRE(dst != nullptr, "thorhip_memset_async: dst is NULL");
+    THORHIP_TRY(hipMemsetAsync(dst, byte_value, bytes, (hipStream_t)stream));
+    return 0;
+}
+
+int thorhip_mem_get_info(size_t* free_bytes, size_t* total_bytes) {
+    size_t f = 0, t = 0;
+    THORHIP_TRY(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return 0;
+}
+
+// ---- streams / events ------------------------------------------------------------------------------------------------
+int thorhip_stream_create(void** stream) {
+    THORHIP_REQUIRE(stream != nullptr, "thorhip_stream_create: stream is NULL");
+    hipStream_t s = nullptr;
+    THORHIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return 0;
+}
+
+int thorhip_stream_destroy(void* stream) {
+    if (stream == nullptr) return 0;
+    THORHIP_TRY(hipStreamDestroy((hipStream_t)stream));
+    return 0;
+}
+
+int thorhip_stream_synchronize(void* stream) {
+    THORHIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int thorhip_stream_wait_event(void* stream, void* event) {
+    THORHIP_REQUIRE(event != nullptr, "thorhip_stream_wait_event: event is NULL");
+    THORHIP_TRY(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0));
+    return 0;
+}
+
+int thorhip_stream_enqueue_host_function(void* stream, thorhip_host_fn fn, void* user_data) {
+    THORHIP_REQUIRE(fn != nullptr, "thorhip_stream_enqueue_host_function: fn is NULL");
+    THORHIP_TRY(hipLaunchHostFunc((hipStream_t)stream, fn, user_data));
+    return 0;
+}
+
+int thorhip_event_create(void** event, int enable_timing) {
+    THORHIP_REQUIRE(event != nullptr, "thorhip_event_create: event is NULL");
+    hipEvent_t e = nullptr;
+    THORHIP_TRY(hipEventCreateWithFlags(&e, enable_timing ? hipEventDefault : hipEventDisableTiming));
+    *event = e;
+    return 0;
+}
+
+int thorhip_event_destroy(void* event) {
+    if (event == nullptr) return 0;
+    THORHIP_TRY(hipEventDestroy((hipEvent_t)event));
+    return 0;
+}
+
+int thorhip_event_record(void* event, void* stream) {
+    THORHIP_REQUIRE(event != nullptr, "thorhip_event_record: event is NULL");
+    THORHIP_TRY(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+    return 0;
+}
+
+int thorhip_event_synchronize(void* event) {
+    THORHIP_REQUIRE(event != nullptr, "thorhip_event_synchronize: event is NULL");
+    THORHIP_TRY(hipEventSynchronize((hipEvent_t)event));
+    return 0;
+}
+
+int thorhip_event_elapsed_ms(float* ms, void* start, void* stop) {
+    THORHIP_REQUIRE(ms != nullptr && start != nullptr && stop != nullptr, "thorhip_event_elapsed_ms: NULL argument");
+    THORHIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return 0;
+}
+
+// ---- run-time compilation ---------------------------------------------------------------------------------------------
+static void copyLog(hiprtcProgram prog, char* log, size_t cap) {
+    if (log == nullptr || cap == 0) return;
+    log[0] = '\0';
+    size_t n = 0;
+    if (hiprtcGetProgramLogSize(prog, &n) != HIPRTC_SUCCESS || n == 0) return;
+    std::string text(n, '\0');
+    if (hiprtcGetProgramLog(prog, text.data()) != HIPRTC_SUCCESS) return;
+    std::snprintf(log, cap, "%s", text.c_str());
+}
+
+int thorhip_compile(const char* source, const char* program_name, const char* arch, const char* const* options,
+                    int num_options, void** code, size_t* code_size, char* log, size_t log_capacity) {
+    THORHIP_REQUIRE(source != nullptr && code != nullptr && code_size != nullptr, "thorhip_compile: NULL argument");
+    *code = nullptr;
+    *code_size = 0;
+    if (log && log_capacity) log[0] = '\0';
+
+    std::string arch_name;
+    if (arch != nullptr && arch[0] != '\0') {
+        arch_name = arch;
+    } else {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.gcnArchName[0]) {
+            arch_name = prop.gcnArchName;
+        } else {
+            (void)hipGetLastError();
+            arch_name = "gfx950";
+        }
+    }
+    const std::string arch_flag = "--offload-arch=" + arch_name;
+
+    hiprtcProgram prog = nullptr;
+    hiprtcResult rc = hiprtcCreateProgram(&prog, source, program_name ? program_name : "thor_fused.hip", 0, nullptr, nullptr);
+    if (rc != HIPRTC_SUCCESS) return fail(-2, "hiprtcCreateProgram failed: %s", hiprtcGetErrorString(rc));
+
+    // Fixed flags: gfx950 code object, wave64 (the gfx9 default), -O3, and the packed-fp32 VALU forms switched off.
+    std::vector<const char*> flags = {arch_flag.c_str(), "-O3",    "-std=c++17",     "-Xclang",
+                                      "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    for (int i = 0; i < num_options; ++i) flags.push_back(options[i]);
+
+    rc = hiprtcCompileProgram(prog, (int)flags.size(), flags.data());
+    copyLog(prog, log, log_capacity);
+    if (rc != HIPRTC_SUCCESS) {
+        std::string text;
+        size_t n = 0;
+        if (hiprtcGetProgramLogSize(prog, &n) == HIPRTC_SUCCESS && n > 0) {
+            text.resize(n);
+            (void)hiprtcGetProgramLog(prog, text.data());
+        }
+        (void)hiprtcDestroyProgram(&prog);
+        return fail(-3, "hiprtcCompileProgram(%s) failed: %s\n%s", arch_name.c_str(), hiprtcGetErrorString(rc), text.c_str());
+    }
+    size_t n = 0;
+    rc = hiprtcGetCodeSize(prog, &n);
+    if (rc != HIPRTC_SUCCESS || n == 0) {
+        (void)hiprtcDestroyProgram(&prog);
+        return fail(-4, "hiprtcGetCodeSize failed: %s", hiprtcGetErrorString(rc));
+    }
+    void* blob = std::malloc(n);
+    if (blob == nullptr) {
+        (void)hiprtcDestroyProgram(&prog);
+        return fail(-5, "thorhip_compile: out of host memory for a %zu byte code object", n);
+    }
+    rc = hiprtcGetCode(prog, (char*)blob);
+    (void)hiprtcDestroyProgram(&prog);
+    if (rc != HIPRTC_SUCCESS) {
+        std::free(blob);
+        return fail(-6, "hiprtcGetCode failed: %s", hiprtcGetErrorString(rc));
+    }
+    *code = blob;
+    *code_size = n;
+    return 0;
+}
+
+int thorhip_code_free(void* code) {
+    std::free(code);
+    return 0;
+}
+
+int thorhip_module_load(void** module, const void* code, size_t code_size) {
+    THORHIP_REQUIRE(module != nullptr && code != nullptr && code_size > 0, "thorhip_module_load: bad argument");
+    hipModule_t m = nullptr;
+    THORHIP_TRY(hipModuleLoadData(&m, code));
+    *module = m;
+    return 0;
+}
+
+int thorhip_module_unload(void* module) {
+    if (module == nullptr) return 0;
+    THORHIP_TRY(hipModuleUnload((hipModule_t)module));
+    return 0;
+}
+
+int thorhip_module_get_function(void** function, void* module, const char* kernel_name) {
+    THORHIP_REQUIRE(function != nullptr && module != nullptr && kernel_name != nullptr, "thorhip_module_get_function: NULL argument");
+    hipFunction_t f = nullptr;
+    THORHIP_TRY(hipModuleGetFunction(&f, (hipModule_t)module, kernel_name));
+    *function = f;
+    return 0;
+}
+
+int thorhip_function_get_attributes(void* function, int* num_vgprs_hint, int* static_lds_bytes, int* max_threads_per_block) {
+    THORHIP_REQUIRE(function != nullptr, "thorhip_function_get_attributes: function is NULL");
+    int v = 0;
+    if (num_vgprs_hint) {
+        THORHIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_NUM_REGS, (hipFunction_t)function));
+        *num_vgprs_hint = v;
+    }
+    if (static_lds_bytes) {
+        THORHIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, (hipFunction_t)function));
+        *static_lds_bytes = v;
+    }
+    if (max_threads_per_block) {
+        THORHIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_MAX_THREADS_PER_BLOCK, (hipFunction_t)function));
+        *max_threads_per_block = v;
+    }
+    return 0;
+}
+
+int thorhip_launch(void* function, uint32_t grid_x, uint32_t grid_y, uint32_t grid_z, uint32_t block_x, uint32_t block_y,
+                   uint32_t block_z, uint32_t dynamic_lds_bytes, void* stream, void** args) {
+    THORHIP_REQUIRE(function != nullptr, "thorhip_launch: function is NULL");
+    THORHIP_REQUIRE(grid_x > 0 && grid_y > 0 && grid_z > 0 && block_x > 0 && block_y > 0 && block_z > 0,
+                    "thorhip_launch: empty grid or block (%u,%u,%u)x(%u,%u,%u)", grid_x, grid_y, grid_z, block_x, block_y, block_z);
+    THORHIP_REQUIRE((uint64_t)block_x * block_y * block_z <= 1024, "thorhip_launch: block of %llu threads exceeds 1024",
+                    (unsigned long long)block_x * block_y * block_z);
+    THORHIP_TRY(hipModuleLaunchKernel((hipFunction_t)function, grid_x, grid_y, grid_z, block_x, block_y, block_z,
+                                      dynamic_lds_bytes, (hipStream_t)stream, args, nullptr));
+    return 0;
+}
+
+}  // extern "C"
