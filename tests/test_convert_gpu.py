@@ -73,6 +73,20 @@ def test_all_16bit_codes_widen_exactly(gpu):
     assert_same_bits(got, oracle.convert(codes, oracle.BF16, oracle.FP32), DataType.fp32)
 
 
+UNSIGNED = (DataType.uint8, DataType.uint16, DataType.uint32, DataType.uint64)
+
+
+def _sample_for(src, dst, n, rng):
+    """Negative float -> unsigned is undefined in the reference (C++ cast): keep such pairs on non-negative inputs."""
+    x = _sample(src, n, rng)
+    if dst in UNSIGNED and src not in INTS:
+        xf = np.abs(x) if src in (DataType.fp32, DataType.fp64) else np.abs(oracle.to_f32(x, int(src)))
+        x = xf if src in (DataType.fp32, DataType.fp64) else oracle.convert(xf.astype(np.float32), oracle.FP32, int(src))
+    if dst in UNSIGNED and src in INTS and src != DataType.boolean:
+        x = np.abs(x).astype(numpy_carrier(src))
+    return x
+
+
 def _sample(dtype, n, rng):
     """Small, exactly representable magnitudes like the reference's converter test (TypeConverterTest.cpp:10-180) plus
     fractional values so that rounding and truncation are exercised."""
@@ -81,8 +95,7 @@ def _sample(dtype, n, rng):
     if dtype in INTS:
         info = np.iinfo(numpy_carrier(dtype))
         return rng.integers(max(info.min, -100), min(info.max, 100) + 1, n).astype(numpy_carrier(dtype))
-    lo = 0.0 if False else -20.0
-    vals = (rng.uniform(lo, 20.0, n)).astype(np.float32)
+    vals = rng.uniform(-20.0, 20.0, n).astype(np.float32)
     vals[::7] = np.round(vals[::7])
     if dtype == DataType.fp32:
         return vals
@@ -95,13 +108,7 @@ def _sample(dtype, n, rng):
 def test_every_pair_out_of_place(gpu, src, dst):
     rng = np.random.default_rng(int(src) * 100 + int(dst))
     n = 5003
-    x = _sample(src, n, rng)
-    if dst in (DataType.uint8, DataType.uint16, DataType.uint32, DataType.uint64) and src not in INTS:
-        # negative float -> unsigned is undefined in the reference (C++ cast); keep the domain defined
-        xf = np.abs(oracle.to_f32(x, int(src))) if src != DataType.fp64 else np.abs(x)
-        x = xf if src in (DataType.fp32, DataType.fp64) else oracle.convert(xf.astype(np.float32), oracle.FP32, int(src))
-    if dst in (DataType.uint8, DataType.uint16, DataType.uint32, DataType.uint64) and src in INTS and src != DataType.boolean:
-        x = np.abs(x).astype(numpy_carrier(src))
+    x = _sample_for(src, dst, n, rng)
     got = gpu.convert_array(x, src, dst)
     want = oracle.convert(x, int(src), int(dst))
     assert_same_bits(got, want, dst)
@@ -114,7 +121,7 @@ def test_every_pair_out_of_place(gpu, src, dst):
 def test_in_place(gpu, src, dst, n):
     from thor_amd.runtime import DeviceBuffer, TypeConverter
     rng = np.random.default_rng(n)
-    x = _sample(src, n, rng)
+    x = _sample_for(src, dst, n, rng)
     want = oracle.convert(x, int(src), int(dst))
     nbytes = n * max(size_of(src), size_of(dst))
     buf = DeviceBuffer(nbytes + 256)
