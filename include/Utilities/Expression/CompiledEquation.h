@@ -1,0 +1,44 @@
+// A kernel compiled at run time for one GPU: the loaded code object, the kernel function handle and its launch shape.
+// Shared through a process-wide LRU keyed by the generated source text, so equal stages compile once
+// (reference: Utilities/Expression/CompiledEquation.h:96-103 owns the CUmodule the same way;
+//  Utilities/Expression/EquationCompiler.cpp:1916-1988 keeps the global kernel cache).
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace ThorImplementation {
+
+// A loaded code object; unloaded when the last kernel handle that refers to it goes away (errors are swallowed).
+struct LoadedModule {
+    LoadedModule() = default;
+    LoadedModule(const LoadedModule&) = delete;
+    LoadedModule& operator=(const LoadedModule&) = delete;
+    ~LoadedModule();
+    void* module = nullptr;
+    int deviceNum = 0;
+};
+
+struct CompiledKernel {
+    std::shared_ptr<LoadedModule> module;
+    void* function = nullptr;
+    int deviceNum = 0;
+    std::string kernelName;
+    std::string source;  // kept for diagnostics and tests
+    int numRegisters = 0;
+    int staticLdsBytes = 0;
+
+    // Asynchronous launch on `stream` (a raw stream handle of the same GPU).
+    void launch(uint32_t gridX, uint32_t gridY, uint32_t gridZ, uint32_t blockX, void* stream, std::vector<void*>& args) const;
+};
+
+// Compiles (or fetches from the process-wide cache) `kernelName` from `source` for GPU `deviceNum`.  `fastContract`
+// selects -ffp-contract=fast (mul+add may fuse, matching the reference's -fmad=true) versus -ffp-contract=off.
+std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract);
+
+// Number of run-time compilations performed so far (cache misses); used by tests of the caching behaviour.
+uint64_t compiledKernelCount();
+
+}  // namespace ThorImplementation

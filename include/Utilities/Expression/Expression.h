@@ -1,0 +1,336 @@
+// Expression: an immutable DAG of elementwise, broadcast, cast, shape and reduction operations over named tensor
+// inputs, built with ordinary C++ operators and lowered by FusedEquation into gfx950 kernels.
+//
+// The public surface (class names, method names, argument meaning, the ExprOp numbering and the way activations
+// decompose into primitive nodes) follows the reference so that its callers compile against this header unchanged:
+// Utilities/Expression/Expression.h:32-148 (ops), :231-371 (node), :516-1075 (API), :1077-1115 (stable activations),
+// Utilities/Expression/Expression.cpp:4176-4193,5185-5190 (activation macros).
+//
+// Operations of the reference that sit outside the elementwise / reduction / cast hot path (matmul, convolution,
+// attention, RoPE, scans, ragged segments, embedding, cuDNN softmax, transposes, strided views, user kernels) keep their
+// ExprOp codes so serialized graphs stay readable, but have no builder here and are rejected by the compiler.
+#pragma once
+
+#include "DeepLearning/Implementation/Tensor/Tensor.h"
+
+#include <cstdint>
+#include <initializer_list>
+#include <memory>
+#include <optional>
+#include <set>
+#include <string>
+#include <unordered_map>
+#include <utility>
+#include <vector>
+
+namespace ThorImplementation {
+
+class Expression;
+class Outputs;
+
+// clang-format off
+enum class ExprOp : uint16_t {
+    INPUT = 3, RUNTIME_SCALAR, TENSOR_RUNTIME_SCALAR, SCALAR_FP,
+    ADD, SUB, MUL, DIV, POW,
+    EQUAL, NOT_EQUAL, LESS, LESS_EQUAL, GREATER, GREATER_EQUAL,
+    LOGICAL_AND, LOGICAL_OR, LOGICAL_NOT, CAST, WHERE,
+    NEG, ABS, CEIL, FLOOR, ROUND, TRUNC,
+    SIN, COS, TAN, ASIN, ACOS, ATAN, SINH, COSH, ASINH, ACOSH, ATANH,
+    ERF, ERFC, ERFCX, ERFINV, ERFCINV, TGAMMA, LGAMMA, DIGAMMA,
+    EXP, EXPM1, EXP2, EXP10, LN, LOG1P, LOG2, LOG10, SQRT, TANH, NORMCDF,
+    ROPE, SOFTMAX, FILL, RESHAPE, STRIDED_VIEW, STRIDED_VIEW_BACKWARD, UNSQUEEZE, SQUEEZE, TRANSPOSE, TAKE_ALONG_AXIS,
+    MIN, MAX, MIN_GRAD_LEFT, MIN_GRAD_RIGHT, MAX_GRAD_LEFT, MAX_GRAD_RIGHT,
+    MATMUL, GEMM, CONV2D, CONV2D_BACKWARD_DATA, CONV2D_BACKWARD_FILTER, CONV3D, CONV3D_BACKWARD_DATA, CONV3D_BACKWARD_FILTER,
+    REDUCE_SUM, REDUCE_PROD, REDUCE_MIN, REDUCE_MAX, REDUCE_ARGMIN, REDUCE_ARGMAX,
+    REDUCE_MIN_BACKWARD, REDUCE_MAX_BACKWARD, SCAN_MIN_BACKWARD, SCAN_MAX_BACKWARD,
+    SEGMENTED_SCAN_MIN_BACKWARD, SEGMENTED_SCAN_MAX_BACKWARD,
+    REDUCE_AVG, REDUCE_NORM1, REDUCE_NORM2,
+    SCAN, RMSNORM, RMSNORM_BACKWARD_X, RMSNORM_BACKWARD_SCALE,
+    ATTENTION, ATTENTION_BACKWARD_Q, ATTENTION_BACKWARD_K, ATTENTION_BACKWARD_V, ATTENTION_BACKWARD_BIAS,
+    EMBEDDING_LOOKUP, CUDA_KERNEL_OUTPUT, SEGMENTED_SCAN,
+    SEGMENTED_REDUCE_SUM, SEGMENTED_REDUCE_MIN, SEGMENTED_REDUCE_MAX, RAGGED_VALUEWISE_EXTENT, SEGMENTED_REDUCE_MEAN,
+    SEGMENTED_BROADCAST, SEGMENTED_REDUCE_MIN_BACKWARD, SEGMENTED_REDUCE_MAX_BACKWARD,
+};
+// clang-format on
+
+inline bool isValueReductionOp(ExprOp op) {
+    switch (op) {
+        case ExprOp::REDUCE_SUM:
+        case ExprOp::REDUCE_PROD:
+        case ExprOp::REDUCE_MIN:
+        case ExprOp::REDUCE_MAX:
+        case ExprOp::REDUCE_AVG:
+        case ExprOp::REDUCE_NORM1:
+        case ExprOp::REDUCE_NORM2:
+            return true;
+        default:
+            return false;
+    }
+}
+inline bool isArgReductionOp(ExprOp op) { return op == ExprOp::REDUCE_ARGMIN || op == ExprOp::REDUCE_ARGMAX; }
+inline bool isReductionOp(ExprOp op) { return isValueReductionOp(op) || isArgReductionOp(op); }
+
+// One vertex of the DAG.  Children are indices into PhysicalExpression::nodes and always precede their consumer.
+struct ExprNode {
+    ExprOp op = ExprOp::SCALAR_FP;
+    uint32_t lhs = UINT32_MAX;
+    uint32_t rhs = UINT32_MAX;
+    uint32_t aux = UINT32_MAX;         // third operand (WHERE: lhs = condition, rhs = true value, aux = false value)
+    uint32_t input_slot = UINT32_MAX;  // INPUT / RUNTIME_SCALAR only
+    double scalar_fp = 0.0;            // SCALAR_FP / FILL only
+
+    // INPUT / RUNTIME_SCALAR: dtype of the value actually bound at stamp time (filled in by dtype resolution).
+    std::optional<DataType> input_tensor_dtype;
+    // Value semantics: the dtype the node's value has in the graph, and the dtype its arithmetic runs in.
+    std::optional<DataType> output_dtype;
+    std::optional<DataType> compute_dtype;
+
+    std::vector<uint64_t> reduction_axes;  // reductions: empty = all axes
+    std::vector<uint64_t> squeeze_axes;    // reductions and SQUEEZE; {UINT64_MAX} = every singleton axis
+    std::vector<uint64_t> unsqueeze_axes;
+    std::vector<uint64_t> reshape_dims;    // one entry may be UINT64_MAX = inferred
+    std::vector<uint64_t> fill_dims;
+};
+
+struct NamedInput {
+    enum class Kind : uint8_t { Tensor, RuntimeScalarFp32, TensorRuntimeScalar };
+    std::string name;
+    uint32_t slot = 0;
+    Kind kind = Kind::Tensor;
+};
+
+struct NamedOutput {
+    std::string name;
+    uint32_t node_idx = UINT32_MAX;
+};
+
+struct PhysicalExpression {
+    std::vector<ExprNode> nodes;
+    std::vector<NamedInput> inputs;
+    uint32_t output_node = UINT32_MAX;
+
+    uint32_t numInputs() const { return static_cast<uint32_t>(inputs.size()); }
+    uint32_t getOrCreateInputSlot(const std::string& name, NamedInput::Kind kind = NamedInput::Kind::Tensor);
+    std::set<std::string> getInputNames() const {
+        std::set<std::string> names;
+        for (const NamedInput& in : inputs) names.insert(in.name);
+        return names;
+    }
+};
+
+struct PhysicalOutputs {
+    std::shared_ptr<PhysicalExpression> expr;
+    std::vector<NamedOutput> outputs;
+};
+
+class Outputs {
+   public:
+    const std::shared_ptr<PhysicalExpression>& expression() const { return expr; }
+    const std::vector<NamedOutput>& namedOutputs() const { return outputs; }
+    PhysicalOutputs physicalOutputs() const;
+    static Outputs fromPhysicalOutputs(PhysicalOutputs physicalOutputs);
+
+   private:
+    Outputs(std::shared_ptr<PhysicalExpression> expr, std::vector<NamedOutput> outputs) : expr(std::move(expr)), outputs(std::move(outputs)) {}
+    std::shared_ptr<PhysicalExpression> expr;
+    std::vector<NamedOutput> outputs;
+    friend class Expression;
+};
+
+class Expression {
+   public:
+    Expression(double value);  // implicit on purpose: `x + 2.0`
+
+    static Expression input(const std::string& name, std::optional<DataType> compute_dtype = std::nullopt,
+                            std::optional<DataType> output_dtype = std::nullopt);
+    static Expression runtimeScalar(const std::string& name, std::optional<DataType> compute_dtype = std::nullopt,
+                                    std::optional<DataType> output_dtype = std::nullopt);
+    static Expression constantScalar(double value);
+    static Expression fill(double value, const std::vector<uint64_t>& dims, std::optional<DataType> output_dtype = std::nullopt);
+
+    static Outputs outputs(const std::vector<std::pair<std::string, Expression>>& named_exprs);
+    static Outputs outputs(std::initializer_list<std::pair<std::string, Expression>> named_exprs);
+
+    static Expression fromPhysicalNode(std::shared_ptr<PhysicalExpression> expr, uint32_t nodeIndex);
+    PhysicalExpression expression() const;
+    std::set<std::string> getInputNames() const;
+    bool isSameLogicalNode(const Expression& other) const {
+        return expr && other.expr && expr.get() == other.expr.get() && nodeIndex == other.nodeIndex;
+    }
+
+    // ---- arithmetic, comparison, logic --------------------------------------------------------------------------
+    Expression operator+(const Expression& other) const;
+    Expression operator-(const Expression& other) const;
+    Expression operator*(const Expression& other) const;
+    Expression operator/(const Expression& other) const;
+    Expression operator-() const;
+    Expression operator!() const;
+    Expression operator==(const Expression& other) const;
+    Expression operator!=(const Expression& other) const;
+    Expression operator<(const Expression& other) const;
+    Expression operator<=(const Expression& other) const;
+    Expression operator>(const Expression& other) const;
+    Expression operator>=(const Expression& other) const;
+
+    Expression equal(const Expression& other) const;
+    Expression notEqual(const Expression& other) const;
+    Expression lessThan(const Expression& other) const;
+    Expression lessEqual(const Expression& other) const;
+    Expression greaterThan(const Expression& other) const;
+    Expression greaterEqual(const Expression& other) const;
+    Expression logicalAnd(const Expression& other) const;
+    Expression logicalOr(const Expression& other) const;
+    Expression logicalNot() const;
+    Expression pow(const Expression& exponent) const;
+    Expression min(const Expression& other) const;
+    Expression max(const Expression& other) const;
+    Expression cast(DataType output_dtype) const;
+    Expression select(const Expression& true_value, const Expression& false_value) const;
+
+    static Expression equal(const Expression& lhs, const Expression& rhs) { return lhs.equal(rhs); }
+    static Expression notEqual(const Expression& lhs, const Expression& rhs) { return lhs.notEqual(rhs); }
+    static Expression lessThan(const Expression& lhs, const Expression& rhs) { return lhs.lessThan(rhs); }
+    static Expression lessEqual(const Expression& lhs, const Expression& rhs) { return lhs.lessEqual(rhs); }
+    static Expression greaterThan(const Expression& lhs, const Expression& rhs) { return lhs.greaterThan(rhs); }
+    static Expression greaterEqual(const Expression& lhs, const Expression& rhs) { return lhs.greaterEqual(rhs); }
+    static Expression logicalAnd(const Expression& lhs, const Expression& rhs) { return lhs.logicalAnd(rhs); }
+    static Expression logicalOr(const Expression& lhs, const Expression& rhs) { return lhs.logicalOr(rhs); }
+    static Expression logicalNot(const Expression& input) { return input.logicalNot(); }
+    static Expression cast(const Expression& input, DataType output_dtype) { return input.cast(output_dtype); }
+    static Expression where(const Expression& condition, const Expression& true_value, const Expression& false_value);
+    static Expression select(const Expression& condition, const Expression& true_value, const Expression& false_value) {
+        return where(condition, true_value, false_value);
+    }
+
+    // ---- unary math: one primitive node each ----------------------------------------------------------------------
+    Expression abs() const;
+    Expression ceil() const;
+    Expression floor() const;
+    Expression round() const;
+    Expression trunc() const;
+    Expression sin() const;
+    Expression cos() const;
+    Expression tan() const;
+    Expression asin() const;
+    Expression acos() const;
+    Expression atan() const;
+    Expression sinh() const;
+    Expression cosh() const;
+    Expression tanh() const;
+    Expression asinh() const;
+    Expression acosh() const;
+    Expression atanh() const;
+    Expression erf() const;
+    Expression erfc() const;
+    Expression erfcx() const;
+    Expression erfinv() const;
+    Expression erfcinv() const;
+    Expression tgamma() const;
+    Expression lgamma() const;
+    Expression digamma() const;
+    Expression exp() const;
+    Expression expm1() const;
+    Expression exp2() const;
+    Expression exp10() const;
+    Expression ln() const;
+    Expression log1p() const;
+    Expression log2() const;
+    Expression log10() const;
+    Expression sqrt() const;
+    static Expression sqrt(const Expression& expr) { return expr.sqrt(); }
+    Expression normcdf() const;
+
+    // ---- compositions of the primitives above ---------------------------------------------------------------------
+    Expression csc() const;
+    Expression sec() const;
+    Expression cot() const;
+    Expression acsc() const;
+    Expression asec() const;
+    Expression acot() const;
+    Expression csch() const;
+    Expression sech() const;
+    Expression coth() const;
+    Expression acsch() const;
+    Expression asech() const;
+    Expression acoth() const;
+    Expression log(double base) const;
+    Expression clamp(const Expression& lower_bound, const Expression& upper_bound) const;
+    Expression clamp(double lower_bound, double upper_bound) const;
+    static Expression clamp(const Expression& input, const Expression& lower_bound, const Expression& upper_bound) {
+        return input.clamp(lower_bound, upper_bound);
+    }
+    static Expression clamp(const Expression& input, double lower_bound, double upper_bound) { return input.clamp(lower_bound, upper_bound); }
+
+    // Numerically stable activation shapes.
+    Expression sigmoid() const;
+    Expression softplus() const;
+    Expression elu(double alpha = 1.0) const;
+    Expression selu() const;
+    Expression gelu() const;
+    Expression mish() const;
+    Expression relu6() const;
+    Expression hardTanh(double min_value = -1.0, double max_value = 1.0) const;
+    Expression hardSwish() const;
+    Expression threshold(double threshold = 0.0, double value = 0.0) const;
+    Expression swish() const;
+
+    // ---- shape -------------------------------------------------------------------------------------------------------
+    Expression reshape(const std::vector<uint64_t>& new_dims) const;
+    Expression unsqueeze(const std::vector<uint64_t>& unsqueeze_axes) const;
+    Expression squeeze(const std::vector<uint64_t>& squeeze_axes) const;
+
+    // ---- reductions: fp32 accumulation, reduced axes kept as 1 unless listed in squeeze_axes ------------------------
+    Expression reduction(ExprOp op, const std::vector<uint64_t>& reduction_axes, const std::vector<uint64_t>& squeeze_axes,
+                         std::optional<DataType> compute_dtype) const;
+    Expression reduce_sum(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                          std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression reduce_prod(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                           std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression reduce_min(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                          std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression reduce_max(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                          std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression reduce_mean(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                           std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression reduce_norm1(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                            std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression reduce_norm2(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                            std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression argmin(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                      std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression argmax(const std::vector<uint64_t>& reduction_axes = {}, const std::vector<uint64_t>& squeeze_axes = {},
+                      std::optional<DataType> compute_dtype = std::nullopt) const;
+    Expression dotProduct(const Expression& other, std::optional<DataType> compute_dtype = std::nullopt) const;
+    static Expression dotProduct(const Expression& lhs, const Expression& rhs, std::optional<DataType> compute_dtype = std::nullopt);
+
+    // ---- dtype overrides on the root node ----------------------------------------------------------------------------
+    Expression withDTypes(std::optional<DataType> compute_dtype = std::nullopt, std::optional<DataType> output_dtype = std::nullopt) const;
+    Expression withComputeDType(DataType compute_dtype) const { return withDTypes(compute_dtype, std::nullopt); }
+    Expression withOutputDType(DataType output_dtype) const { return withDTypes(std::nullopt, output_dtype); }
+
+    static bool isLeafOp(ExprOp op);
+    static bool isUnaryOp(ExprOp op);
+    static bool isBinaryOp(ExprOp op);
+    static bool isTernaryOp(ExprOp op);
+
+   private:
+    Expression(std::shared_ptr<PhysicalExpression> expr, uint32_t nodeIndex) : expr(std::move(expr)), nodeIndex(nodeIndex) {}
+    static Expression unaryOp(const Expression& input, ExprOp op);
+    static Expression binaryOp(const Expression& lhs, const Expression& rhs, ExprOp op);
+    static Expression ternaryOp(const Expression& a, const Expression& b, const Expression& c, ExprOp op);
+
+    std::shared_ptr<PhysicalExpression> expr;
+    uint32_t nodeIndex = UINT32_MAX;
+};
+
+std::string opName(ExprOp op);
+bool isCommutative(ExprOp op);
+std::string formatFloatCanonical(double x);
+// Canonical text of the sub-DAG below `nodeIndex` (commutative operands ordered, shared sub-trees memoised): two graphs
+// with the same text compute the same function of the same input slots.
+std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex, std::unordered_map<uint32_t, std::string>& memo);
+std::string canonicalize(const PhysicalExpression& expr);
+std::string canonicalize(const PhysicalOutputs& outputs);
+std::string expressionHash(const PhysicalOutputs& outputs);
+
+}  // namespace ThorImplementation

@@ -1,0 +1,74 @@
+// FusedEquation: a compiled Expression.  compile() only captures the graph; the first stamp()/run() with concrete
+// tensors resolves dtypes, infers shapes, splits the graph into stages at reduction boundaries, generates gfx950
+// source for each fused stage, compiles it with hipRTC and binds tensors.  Plans are cached per (dtypes, shapes,
+// strides, alignment) and kernels process-wide per source text
+// (reference: Utilities/Expression/FusedEquation.h:574-632; FusedEquation.cpp:6828-6887,7014-7064,8885-9353,10760-10905).
+#pragma once
+
+#include "Utilities/Cache/LruCache.h"
+#include "Utilities/Expression/Expression.h"
+#include "Utilities/Expression/StampedEquation.h"
+
+#include <memory>
+#include <optional>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace ThorImplementation {
+
+struct PlannedGraph;  // dtype-resolved, de-duplicated graph with its stage split (internal)
+
+class FusedEquation {
+   public:
+    static FusedEquation compile(const PhysicalExpression& expr, int device_num);
+    static FusedEquation compile(const PhysicalOutputs& outputs, int device_num);
+
+    // Binds tensors and returns a plan whose run() only launches.  Outputs are allocated here unless the caller passes
+    // them in `preallocated_outputs` (shape and dtype are validated).
+    [[nodiscard]] StampedExecutionPlan stamp(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                             const std::unordered_map<std::string, Tensor>& preallocated_outputs = {}) const;
+    [[nodiscard]] StampedExecutionPlan stampSingleOutput(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                                         const std::optional<Tensor>& preallocated_output = {}) const;
+
+    // Convenience: bind, launch into caller-provided outputs.  Restricted, as in the reference, to expressions that
+    // lower to fused kernels only (no reduction stage) -- use stamp() otherwise.
+    void run(const Tensor& input, Tensor& output, Stream& stream) const;
+    void run(const std::unordered_map<std::string, Tensor>& inputs, Tensor& output, Stream& stream) const;
+    void run(const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, float>& scalar_inputs, Tensor& output,
+             Stream& stream) const;
+    void run(const Tensor& input, std::unordered_map<std::string, Tensor>& outputs, Stream& stream) const;
+    void run(const std::unordered_map<std::string, Tensor>& inputs, std::unordered_map<std::string, Tensor>& outputs, Stream& stream) const;
+    void run(const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, float>& scalar_inputs,
+             std::unordered_map<std::string, Tensor>& outputs, Stream& stream) const;
+
+    std::vector<std::string> getOutputNames() const;
+    [[nodiscard]] const PhysicalOutputs& physicalOutputs() const { return outputs_template; }
+
+    std::vector<uint64_t> getOutputShape(const Tensor& input) const;
+    std::vector<uint64_t> getOutputShape(const std::unordered_map<std::string, Tensor>& inputs) const;
+    std::unordered_map<std::string, std::vector<uint64_t>> getOutputShapes(const Tensor& input) const;
+    std::unordered_map<std::string, std::vector<uint64_t>> getOutputShapes(const std::unordered_map<std::string, Tensor>& inputs) const;
+    std::unordered_map<std::string, DataType> getOutputDataTypes(const std::unordered_map<std::string, Tensor>& inputs) const;
+
+    // NumPy-style right-aligned broadcast of the input shapes; returns true when any input needs broadcasting.
+    static bool resolveLayout(std::vector<Tensor>& inputs, std::vector<uint64_t>& outputDimensions);
+
+    int getDeviceNum() const { return device_num; }
+
+   private:
+    FusedEquation(PhysicalOutputs outputs_template, int device_num);
+
+    std::shared_ptr<PlannedGraph> plannedGraphFor(const std::vector<DataType>& root_dtypes) const;
+    std::vector<DataType> rootDTypes(const std::unordered_map<std::string, Tensor>& inputs) const;
+    StampedExecutionPlan stampImpl(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                   const std::unordered_map<std::string, Tensor>& preallocated_outputs, bool fusedKernelsOnly) const;
+
+    PhysicalOutputs outputs_template;
+    std::vector<NamedInput> root_inputs;
+    int device_num;
+    // dtype key -> planned graph; full binding key -> stamped plan recipe is rebuilt per stamp (allocation is per stamp)
+    std::shared_ptr<LruCacheThreadSafe<std::string, std::shared_ptr<PlannedGraph>>> planned_graph_cache;
+};
+
+}  // namespace ThorImplementation

@@ -1,0 +1,152 @@
+// Stamped (shape- and tensor-bound) pieces of a compiled expression and the plan that runs them in order
+// (reference: Utilities/Expression/StampedEquation.h:411-516 StampedEquation, :551-597 StampedReduction / StampedArgMinMax,
+//  :1659-1780 StampedExecutionPlan).  A stamped object owns copies of the Tensor handles it reads and writes, so
+// the storage outlives queued work; run() never allocates, compiles or re-plans.
+#pragma once
+
+#include "DeepLearning/Implementation/Tensor/Tensor.h"
+#include "Utilities/Common/Stream.h"
+#include "Utilities/Expression/CompiledEquation.h"
+#include "Utilities/TensorOperations/Cub/CubReduction.h"
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+namespace ThorImplementation {
+
+// One launch of a run-time compiled elementwise / broadcast kernel, or of a row-fused kernel that also holds the
+// reductions of its rows.
+class StampedEquation {
+   public:
+    struct ScalarArgument {
+        std::string name;  // runtime scalar input name
+        size_t argIndex;   // position in the kernel argument list
+    };
+
+    StampedEquation(std::shared_ptr<CompiledKernel> kernel, std::vector<Tensor> inputs, std::vector<Tensor> outputs,
+                    std::vector<ScalarArgument> scalars, std::vector<size_t> inputArgIndex, std::vector<size_t> outputArgIndex,
+                    size_t numArgs, bool passNumel, uint64_t numel, bool numelIs64, uint32_t gridX, uint32_t threads, uint64_t flops,
+                    std::string description);
+
+    void run(Stream& stream) const { runOn(stream, {}); }
+    void runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const;
+
+    uint32_t gpuNum() const;
+    Tensor getOutputTensor() const;
+    const std::vector<Tensor>& getOutputTensors() const { return outputs; }
+    const std::vector<Tensor>& getInputTensors() const { return inputs; }
+    const std::shared_ptr<CompiledKernel>& getCompiledKernel() const { return kernel; }
+    uint64_t flopCount() const { return flops; }
+    const std::string& getDescription() const { return description; }
+    std::unordered_set<std::string> runtimeScalarNames() const;
+
+    // Reduced axes become 1; the listed squeeze axes (or every singleton when squeeze_axes == {UINT64_MAX}) are removed.
+    static std::vector<uint64_t> computeReductionOutputDims(const std::vector<uint64_t>& input_dims, const std::vector<uint64_t>& reduction_axes,
+                                                            const std::vector<uint64_t>& squeeze_axes);
+
+   private:
+    std::shared_ptr<CompiledKernel> kernel;
+    std::vector<Tensor> inputs;
+    std::vector<Tensor> outputs;
+    std::vector<ScalarArgument> scalars;
+    std::vector<size_t> inputArgIndex, outputArgIndex;
+    size_t numArgs;
+    bool passNumel;
+    uint64_t numel;
+    bool numelIs64;
+    uint32_t gridX, threads;
+    uint64_t flops;
+    std::string description;
+};
+
+class StampedReduction {
+   public:
+    explicit StampedReduction(std::shared_ptr<StampedCubReduction> stamped) : stamped(std::move(stamped)) {}
+    void runOn(Stream& stream) const { stamped->runOn(stream); }
+    CubReductionPath getPath() const { return stamped->getPath(); }
+    Tensor getOutputTensor() const { return stamped->getOutputTensor(); }
+    uint64_t flopCount() const { return stamped->getGeometry().input_elements; }
+    const std::shared_ptr<StampedCubReduction>& getStamped() const { return stamped; }
+
+   private:
+    std::shared_ptr<StampedCubReduction> stamped;
+};
+
+class StampedArgMinMax {
+   public:
+    explicit StampedArgMinMax(std::shared_ptr<StampedCubArgReduction> stamped) : stamped(std::move(stamped)) {}
+    void runOn(Stream& stream) const { stamped->runOn(stream); }
+    CubReductionPath getPath() const { return stamped->getPath(); }
+    Tensor getOutputTensor() const { return stamped->getIndexOutputTensor().value(); }
+    uint64_t flopCount() const { return stamped->getGeometry().input_elements; }
+
+   private:
+    std::shared_ptr<StampedCubArgReduction> stamped;
+};
+
+struct StampedExecutionStage {
+    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy };
+    static std::string kindToString(Kind kind) {
+        switch (kind) {
+            case Kind::FusedKernel:
+                return "FusedKernel";
+            case Kind::Reduction:
+                return "Reduction";
+            case Kind::ArgMinMax:
+                return "ArgMinMax";
+            case Kind::FusedRowKernel:
+                return "FusedRowKernel";
+            case Kind::Copy:
+                return "Copy";
+        }
+        return "<unknown>";
+    }
+
+    Kind kind = Kind::FusedKernel;
+    std::vector<uint32_t> dependency_stage_indices;
+    uint32_t gpu_num = 0;
+    std::shared_ptr<StampedEquation> kernel;
+    std::shared_ptr<StampedReduction> reduction;
+    std::shared_ptr<StampedArgMinMax> arg_minmax;
+    // Kind::Copy: a named output that is only a view of an input is copied into the caller's tensor
+    Tensor copySource, copyDestination;
+
+    uint64_t flopCount() const;
+    void runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const;
+};
+
+class StampedExecutionPlan {
+   public:
+    StampedExecutionPlan(std::vector<StampedExecutionStage> steps, std::unordered_map<std::string, Tensor> final_outputs, const Stream& stream)
+        : steps(std::move(steps)), final_outputs(std::move(final_outputs)), stream(stream) {}
+
+    void run();
+    void run(const std::unordered_map<std::string, float>& runtime_scalars);
+    void runOn(Stream& run_stream) const;
+    void runOn(Stream& run_stream, const std::unordered_map<std::string, float>& runtime_scalars) const;
+
+    bool requiresRuntimeScalars() const { return !runtimeScalarNames().empty(); }
+    std::unordered_set<std::string> runtimeScalarNames() const;
+
+    uint64_t flopCount() const;
+    std::vector<uint64_t> stageFlopCounts() const;
+    std::vector<std::string> stageKindNames() const;
+    std::vector<std::vector<uint32_t>> stageDependencyIndices() const;
+    std::vector<CubReductionPath> reductionPaths() const;
+    const std::vector<StampedExecutionStage>& stages() const { return steps; }
+
+    Tensor output(const std::string& name) const;
+    Tensor output() const;
+    const std::unordered_map<std::string, Tensor>& getFinalOutputs() const { return final_outputs; }
+
+   private:
+    std::vector<StampedExecutionStage> steps;
+    std::unordered_map<std::string, Tensor> final_outputs;
+    Stream stream;
+};
+
+}  // namespace ThorImplementation

@@ -1,0 +1,187 @@
+/*
+ * thor_c_api.h -- flat C binding of the host-side Thor API of this backend (Tensor, Stream, TypeConverter,
+ * CubReduction / CubArgReduction, Expression, FusedEquation, StampedExecutionPlan).
+ *
+ * The reference exposes this surface to Python through a nanobind module
+ * (bindings/python/src/core/physical/expression.cpp:602-2866, physical_tensor.cpp); this header is what a cgo / JNI /
+ * ctypes / nanobind shim binds instead.  Each function names the C++ entry point of the reference it stands for.
+ *
+ * Conventions: opaque handles are created by *_create / builder functions and released with the matching *_destroy;
+ * handles are independent references (destroying a tensor handle does not free storage another handle still uses).
+ * Functions that can fail return 0 on success and a negative code otherwise, or NULL for handle-returning functions;
+ * thor_last_error() then holds the message of the C++ exception, prefixed with its type
+ * ("invalid_argument: ...", "runtime_error: ...", "logic_error: ...").
+ */
+#ifndef THOR_C_API_H
+#define THOR_C_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct thor_tensor* thor_tensor_t;
+typedef struct thor_stream* thor_stream_t;
+typedef struct thor_stamped_reduction* thor_stamped_reduction_t;
+typedef struct thor_stamped_arg_reduction* thor_stamped_arg_reduction_t;
+typedef struct thor_expr* thor_expr_t;
+typedef struct thor_outputs* thor_outputs_t;
+typedef struct thor_fused_equation* thor_fused_equation_t;
+typedef struct thor_plan* thor_plan_t;
+
+enum { THOR_DEVICE_CPU = 1, THOR_DEVICE_GPU = 2 }; /* TensorPlacement::MemDevices */
+
+const char* thor_last_error(void);
+
+/* ---- Stream (Utilities/Common/Stream.h:35-116) ----------------------------------------------------------------------- */
+thor_stream_t thor_stream_create(int gpu_num);
+void thor_stream_destroy(thor_stream_t stream);
+int thor_stream_synchronize(thor_stream_t stream);
+void* thor_stream_raw(thor_stream_t stream); /* the hipStream_t, for thorhip_* calls */
+int thor_stream_gpu_num(thor_stream_t stream);
+
+/* ---- Tensor (DeepLearning/Implementation/Tensor/Tensor.h:54-264) ------------------------------------------------------- */
+thor_tensor_t thor_tensor_create(int device_type, int device_num, int dtype, const uint64_t* dims, int rank);
+thor_tensor_t thor_tensor_clone_handle(thor_tensor_t tensor);
+void thor_tensor_destroy(thor_tensor_t tensor);
+void* thor_tensor_mem_ptr(thor_tensor_t tensor);
+int thor_tensor_dtype(thor_tensor_t tensor);
+int thor_tensor_rank(thor_tensor_t tensor);
+int thor_tensor_dims(thor_tensor_t tensor, uint64_t* dims_out);       /* rank entries */
+int thor_tensor_strides(thor_tensor_t tensor, uint64_t* strides_out); /* rank entries, in elements */
+uint64_t thor_tensor_num_elements(thor_tensor_t tensor);
+int thor_tensor_device_type(thor_tensor_t tensor);
+int thor_tensor_device_num(thor_tensor_t tensor);
+int thor_tensor_is_dense(thor_tensor_t tensor);
+/* Tensor::copyFromAsync: copies and, when dtypes differ, converts (Tensor.cpp:731-866) */
+int thor_tensor_copy_from_async(thor_tensor_t dest, thor_tensor_t source, thor_stream_t stream);
+int thor_tensor_memset_async(thor_tensor_t tensor, int byte_value, thor_stream_t stream);
+int thor_tensor_reshape(thor_tensor_t tensor, const uint64_t* dims, int rank);
+/* Tensor::aliasView (Tensor.cpp:617-660) */
+thor_tensor_t thor_tensor_alias_view(thor_tensor_t tensor, const uint64_t* dims, const uint64_t* strides_elements, int rank,
+                                     uint64_t element_offset);
+
+/* ---- TypeConverter::convertType (TypeConverter.h:30-46); device_num == -1 converts on the host inside the stream ------ */
+int thor_convert_type(void* source, void* dest, int source_dtype, int dest_dtype, int64_t num_elements, thor_stream_t stream,
+                      int device_num);
+/* synchronous host conversion, TypeConverter::cpuConvertTypeImpl (TypeConverter.cpp:899-942) */
+int thor_convert_type_cpu(const void* source, void* dest, int source_dtype, int dest_dtype, int64_t num_elements);
+
+/* ---- CubReduction (Utilities/TensorOperations/Cub/CubReduction.h:175-234,496-537) ------------------------------------- */
+typedef struct thor_reduction_geometry {
+    int path; /* CubReductionPath */
+    int reduced_axes_are_contiguous;
+    uint64_t outer_size, reduction_size, inner_size;
+    uint64_t input_elements, output_elements;
+    int rank;
+    uint64_t output_dimensions[16];
+    int squeezed_rank;
+    uint64_t squeezed_output_dimensions[16];
+    int device_transform_uses_affine_stride;
+    uint64_t affine_input_stride;
+} thor_reduction_geometry;
+
+/* CubReduction::analyzeGeometry; strides == NULL means dense row-major */
+int thor_reduction_analyze_geometry(const uint64_t* dims, const uint64_t* strides, int rank, const uint32_t* axes, int num_axes,
+                                    thor_reduction_geometry* out);
+/* CubReduction::mapLogicalReductionIndexToPhysicalIndex */
+int thor_reduction_map_index(const uint64_t* dims, const uint64_t* strides, int rank, const uint32_t* axes, int num_axes,
+                             uint64_t output_index, uint64_t reduction_index, uint64_t* physical_index);
+/* CubReduction(op, axes, output_dtype, scale).stamp(input[, preallocated_output], stream); output_dtype < 0 = input dtype */
+thor_stamped_reduction_t thor_reduction_stamp(int op, const uint32_t* axes, int num_axes, int output_dtype, float output_scale,
+                                              thor_tensor_t input, thor_tensor_t preallocated_output, thor_stream_t stream);
+void thor_stamped_reduction_destroy(thor_stamped_reduction_t r);
+int thor_stamped_reduction_run(thor_stamped_reduction_t r);
+int thor_stamped_reduction_run_scaled(thor_stamped_reduction_t r, float output_scale);
+int thor_stamped_reduction_run_on(thor_stamped_reduction_t r, thor_stream_t stream);
+thor_tensor_t thor_stamped_reduction_output(thor_stamped_reduction_t r);
+int thor_stamped_reduction_path(thor_stamped_reduction_t r);
+size_t thor_stamped_reduction_workspace_bytes(thor_stamped_reduction_t r);
+int thor_stamped_reduction_variant(thor_stamped_reduction_t r, char* buffer, size_t capacity);
+/* the generated HIP source for a geometry, without touching a GPU (host-only tests compile it with thorhip_compile) */
+int thor_reduction_generate_source(int is_arg, int op, int input_dtype, int output_dtype, int index_dtype, const uint64_t* dims,
+                                   const uint64_t* strides, int rank, const uint32_t* axes, int num_axes, char* buffer,
+                                   size_t capacity, size_t* needed);
+
+/* ---- CubArgReduction (CubReduction.h:412-487) ---------------------------------------------------------------------------- */
+thor_stamped_arg_reduction_t thor_arg_reduction_stamp(int op, const uint32_t* axes, int num_axes, int produce_value, int produce_index,
+                                                      int value_output_dtype, int index_output_dtype, thor_tensor_t input,
+                                                      thor_tensor_t preallocated_value, thor_tensor_t preallocated_index,
+                                                      thor_stream_t stream);
+void thor_stamped_arg_reduction_destroy(thor_stamped_arg_reduction_t r);
+int thor_stamped_arg_reduction_run(thor_stamped_arg_reduction_t r);
+thor_tensor_t thor_stamped_arg_reduction_value_output(thor_stamped_arg_reduction_t r); /* NULL when not produced */
+thor_tensor_t thor_stamped_arg_reduction_index_output(thor_stamped_arg_reduction_t r);
+int thor_stamped_arg_reduction_path(thor_stamped_arg_reduction_t r);
+
+/* ---- Expression (Utilities/Expression/Expression.h:516-1075) ------------------------------------------------------------- */
+/* dtype arguments: a DataType code, or -1 for "not specified" */
+thor_expr_t thor_expr_input(const char* name, int compute_dtype, int output_dtype);
+thor_expr_t thor_expr_runtime_scalar(const char* name, int compute_dtype, int output_dtype);
+thor_expr_t thor_expr_scalar(double value);
+thor_expr_t thor_expr_fill(double value, const uint64_t* dims, int rank, int output_dtype);
+/* `method` is the C++ method name: "add", "sub", "mul", "div", "pow", "min", "max", "equal", "notEqual", "lessThan",
+ * "lessEqual", "greaterThan", "greaterEqual", "logicalAnd", "logicalOr" (binary); "neg", "logicalNot", "abs", "exp",
+ * "sigmoid", "gelu", ... (unary; every unary method of Expression) */
+thor_expr_t thor_expr_binary(const char* method, thor_expr_t lhs, thor_expr_t rhs);
+thor_expr_t thor_expr_unary(const char* method, thor_expr_t input);
+/* methods with numeric parameters: "elu"(alpha), "hardTanh"(min,max), "threshold"(threshold,value), "log"(base),
+ * "clamp"(lo,hi) */
+thor_expr_t thor_expr_unary_params(const char* method, thor_expr_t input, double p0, double p1);
+thor_expr_t thor_expr_where(thor_expr_t condition, thor_expr_t true_value, thor_expr_t false_value);
+thor_expr_t thor_expr_cast(thor_expr_t input, int dtype);
+thor_expr_t thor_expr_with_dtypes(thor_expr_t input, int compute_dtype, int output_dtype);
+/* `method`: "reduce_sum", "reduce_prod", "reduce_min", "reduce_max", "reduce_mean", "reduce_norm1", "reduce_norm2",
+ * "argmin", "argmax"; num_axes == 0 reduces all axes; squeeze axis UINT64_MAX squeezes every singleton axis */
+thor_expr_t thor_expr_reduce(const char* method, thor_expr_t input, const uint64_t* axes, int num_axes, const uint64_t* squeeze_axes,
+                             int num_squeeze_axes);
+thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank);
+thor_expr_t thor_expr_unsqueeze(thor_expr_t input, const uint64_t* axes, int num_axes);
+thor_expr_t thor_expr_squeeze(thor_expr_t input, const uint64_t* axes, int num_axes);
+void thor_expr_destroy(thor_expr_t expr);
+int thor_expr_num_nodes(thor_expr_t expr);
+int thor_expr_canonical(thor_expr_t expr, char* buffer, size_t capacity, size_t* needed);
+
+/* Expression::outputs({{name, expr}, ...}) */
+thor_outputs_t thor_outputs_create(const char* const* names, const thor_expr_t* exprs, int count);
+void thor_outputs_destroy(thor_outputs_t outputs);
+
+/* ---- FusedEquation (Utilities/Expression/FusedEquation.h:574-632) --------------------------------------------------------- */
+thor_fused_equation_t thor_fused_equation_compile(thor_outputs_t outputs, int device_num);
+void thor_fused_equation_destroy(thor_fused_equation_t eq);
+int thor_fused_equation_num_outputs(thor_fused_equation_t eq);
+int thor_fused_equation_output_name(thor_fused_equation_t eq, int index, char* buffer, size_t capacity);
+/* FusedEquation::stamp(inputs, stream, {}, preallocated_outputs) */
+thor_plan_t thor_fused_equation_stamp(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs, int num_inputs,
+                                      const char* const* preallocated_names, const thor_tensor_t* preallocated, int num_preallocated,
+                                      thor_stream_t stream);
+/* FusedEquation::run(inputs, scalar_inputs, outputs, stream): compile-if-needed and launch into caller tensors */
+int thor_fused_equation_run(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs, int num_inputs,
+                            const char* const* scalar_names, const float* scalars, int num_scalars, const char* const* output_names,
+                            const thor_tensor_t* outputs, int num_outputs, thor_stream_t stream);
+/* FusedEquation::getOutputShapes / getOutputDataTypes for one named output */
+int thor_fused_equation_output_shape(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs, int num_inputs,
+                                     const char* output_name, uint64_t* dims_out, int* rank_out, int* dtype_out);
+
+/* ---- StampedExecutionPlan (Utilities/Expression/StampedEquation.h:1659-1780) ---------------------------------------------- */
+void thor_plan_destroy(thor_plan_t plan);
+int thor_plan_run(thor_plan_t plan);
+int thor_plan_run_with_scalars(thor_plan_t plan, const char* const* scalar_names, const float* scalars, int num_scalars);
+int thor_plan_run_on(thor_plan_t plan, thor_stream_t stream);
+thor_tensor_t thor_plan_output(thor_plan_t plan, const char* name);
+int thor_plan_num_stages(thor_plan_t plan);
+/* StampedExecutionPlan::stageKindNames: "FusedKernel", "Reduction", "ArgMinMax", ... */
+int thor_plan_stage_kind(thor_plan_t plan, int stage, char* buffer, size_t capacity);
+/* generated HIP source of a stage's kernel (diagnostics and tests) */
+int thor_plan_stage_source(thor_plan_t plan, int stage, char* buffer, size_t capacity, size_t* needed);
+int thor_plan_stage_description(thor_plan_t plan, int stage, char* buffer, size_t capacity);
+uint64_t thor_plan_flop_count(thor_plan_t plan);
+/* number of run-time compilations since process start (cache-behaviour tests) */
+uint64_t thor_compiled_kernel_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THOR_C_API_H */

@@ -1,2 +1,284 @@
 // Device-side building blocks shared by every run-time compiled kernel (placed after thorhip_numeric.h).
+//
+// wave64 throughout: a wavefront is 64 lanes, a 256-thread block is 4 wavefronts.  Reductions keep fp32 accumulators in
+// registers, fold lanes with cross-lane shuffles, fold wavefronts through a few words of LDS, and fold blocks through
+// a per-launch partials buffer whose last-arriving block (atomic ticket) produces the final values -- one launch, no
+// atomics on the data, bit-reproducible for a fixed shape.
 #pragma once
+
+namespace thor {
+
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// ---- machine-word loads / stores of VEC elements --------------------------------------------------------------------
+template <int BYTES>
+struct WordOf;
+template <>
+struct WordOf<1> {
+    typedef u8 type;
+};
+template <>
+struct WordOf<2> {
+    typedef u16 type;
+};
+template <>
+struct WordOf<4> {
+    typedef u32 type;
+};
+template <>
+struct WordOf<8> {
+    typedef u32x2 type;
+};
+template <>
+struct WordOf<16> {
+    typedef u32x4 type;
+};
+
+template <typename T, int VEC>
+struct alignas((sizeof(T) * VEC) >= 16 ? 16 : (sizeof(T) * VEC)) Pack {
+    static constexpr int kBytes = sizeof(T) * VEC;
+    static constexpr int kWordBytes = kBytes >= 16 ? 16 : kBytes;
+    static constexpr int kWords = kBytes / kWordBytes;
+    typedef typename WordOf<kWordBytes>::type word_t;
+    T v[VEC];
+
+    // streaming (non-temporal) access: data that is touched once should not displace reusable lines
+    __device__ __forceinline__ void loadStream(const T* p) {
+        const word_t* wp = reinterpret_cast<const word_t*>(p);
+        word_t* mine = reinterpret_cast<word_t*>(v);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) mine[w] = __builtin_nontemporal_load(wp + w);
+    }
+    __device__ __forceinline__ void load(const T* p) {
+        const word_t* wp = reinterpret_cast<const word_t*>(p);
+        word_t* mine = reinterpret_cast<word_t*>(v);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) mine[w] = wp[w];
+    }
+    __device__ __forceinline__ void storeStream(T* p) const {
+        word_t* wp = reinterpret_cast<word_t*>(p);
+        const word_t* mine = reinterpret_cast<const word_t*>(v);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) __builtin_nontemporal_store(mine[w], wp + w);
+    }
+    __device__ __forceinline__ void store(T* p) const {
+        word_t* wp = reinterpret_cast<word_t*>(p);
+        const word_t* mine = reinterpret_cast<const word_t*>(v);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) wp[w] = mine[w];
+    }
+};
+
+// ---- fp32 -> storage ---------------------------------------------------------------------------------------------------
+template <typename To>
+__device__ __forceinline__ To fromFloat(float x) {
+    return Store<To>::from(x);
+}
+__device__ __forceinline__ float toFloat(boolean v) { return v.bits ? 1.0f : 0.0f; }
+__device__ __forceinline__ float toFloat(u8 v) { return (float)v; }
+__device__ __forceinline__ float toFloat(i8 v) { return (float)v; }
+__device__ __forceinline__ float toFloat(u16 v) { return (float)v; }
+__device__ __forceinline__ float toFloat(i16 v) { return (float)v; }
+__device__ __forceinline__ float toFloat(u32 v) { return (float)v; }
+__device__ __forceinline__ float toFloat(i32 v) { return (float)v; }
+__device__ __forceinline__ float toFloat(u64 v) { return (float)v; }
+__device__ __forceinline__ float toFloat(i64 v) { return (float)v; }
+
+// fp16 values are held in native _Float16 registers inside fused kernels
+__device__ __forceinline__ _Float16 asHalf(f16 h) { return __builtin_bit_cast(_Float16, h.bits); }
+__device__ __forceinline__ f16 fromHalf(_Float16 h) {
+    f16 r;
+    r.bits = __builtin_bit_cast(u16, h);
+    return r;
+}
+__device__ __forceinline__ boolean makeBoolean(bool b) {
+    boolean r;
+    r.bits = b ? 1 : 0;
+    return r;
+}
+
+// value rounded through a 16-bit / 8-bit float and widened again (how a bf16 / fp8 compute step is modelled in fp32)
+__device__ __forceinline__ float roundBf16(float x) { return toFloat(toBf16(x)); }
+__device__ __forceinline__ float roundF16(float x) { return toFloat(toF16(x)); }
+__device__ __forceinline__ float roundE4m3(float x) { return toFloat(toE4m3(x)); }
+__device__ __forceinline__ float roundE5m2(float x) { return toFloat(toE5m2(x)); }
+
+// ---- reduction operators: fp32 accumulate -----------------------------------------------------------------------------
+// Min / Max return the NaN operand when either side is NaN (unlike fminf / fmaxf).
+struct SumOp {
+    __device__ __forceinline__ static float identity() { return 0.0f; }
+    __device__ __forceinline__ static float transform(float x) { return x; }
+    __device__ __forceinline__ static float combine(float a, float b) { return a + b; }
+};
+struct AbsSumOp {
+    __device__ __forceinline__ static float identity() { return 0.0f; }
+    __device__ __forceinline__ static float transform(float x) { return __builtin_fabsf(x); }
+    __device__ __forceinline__ static float combine(float a, float b) { return a + b; }
+};
+struct SquareSumOp {
+    __device__ __forceinline__ static float identity() { return 0.0f; }
+    __device__ __forceinline__ static float transform(float x) { return x * x; }
+    __device__ __forceinline__ static float combine(float a, float b) { return a + b; }
+};
+struct ProductOp {
+    __device__ __forceinline__ static float identity() { return 1.0f; }
+    __device__ __forceinline__ static float transform(float x) { return x; }
+    __device__ __forceinline__ static float combine(float a, float b) { return a * b; }
+};
+struct MinOp {
+    __device__ __forceinline__ static float identity() { return __builtin_inff(); }
+    __device__ __forceinline__ static float transform(float x) { return x; }
+    __device__ __forceinline__ static float combine(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fminf(a, b)); }
+};
+struct MaxOp {
+    __device__ __forceinline__ static float identity() { return -__builtin_inff(); }
+    __device__ __forceinline__ static float transform(float x) { return x; }
+    __device__ __forceinline__ static float combine(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fmaxf(a, b)); }
+};
+
+// Accumulator protocol used by every reduction kernel:
+//   reset(), add(x, index), merge(other), shuffleXor(mask), and the fields a partial is stored as.
+template <typename Op>
+struct ValueAcc {
+    float v;
+    __device__ __forceinline__ void reset() { v = Op::identity(); }
+    template <typename I>
+    __device__ __forceinline__ void add(float x, I) {
+        v = Op::combine(v, Op::transform(x));
+    }
+    __device__ __forceinline__ void merge(const ValueAcc& o) { v = Op::combine(v, o.v); }
+    __device__ __forceinline__ ValueAcc shuffleXor(int mask) const {
+        ValueAcc r;
+        r.v = __shfl_xor(v, mask, kWave);
+        return r;
+    }
+};
+
+// Candidate {value, index}: NaN beats every number, equal values (and two NaNs) keep the lower index.  The empty
+// candidate carries the all-ones index, so any real element wins against it.
+template <bool IS_MAX, typename IndexT>
+struct ArgAcc {
+    float v;
+    IndexT i;
+    __device__ __forceinline__ void reset() {
+        v = IS_MAX ? -__builtin_inff() : __builtin_inff();
+        i = ~(IndexT)0;
+    }
+    __device__ __forceinline__ static bool better(float av, IndexT ai, float bv, IndexT bi) {
+        // true when candidate a wins over candidate b
+        const bool an = av != av, bn = bv != bv;
+        if (an || bn) return (an && bn) ? (ai <= bi) : an;
+        if (IS_MAX ? (av > bv) : (av < bv)) return true;
+        if (IS_MAX ? (bv > av) : (bv < av)) return false;
+        return ai <= bi;
+    }
+    template <typename I>
+    __device__ __forceinline__ void add(float x, I index) {
+        if (!better(v, i, x, (IndexT)index)) {
+            v = x;
+            i = (IndexT)index;
+        }
+    }
+    __device__ __forceinline__ void merge(const ArgAcc& o) {
+        if (!better(v, i, o.v, o.i)) {
+            v = o.v;
+            i = o.i;
+        }
+    }
+    __device__ __forceinline__ ArgAcc shuffleXor(int mask) const {
+        ArgAcc r;
+        r.v = __shfl_xor(v, mask, kWave);
+        if (sizeof(IndexT) == 8) {
+            const u32 lo = __shfl_xor((u32)((u64)i & 0xffffffffu), mask, kWave);
+            const u32 hi = __shfl_xor((u32)((u64)i >> 32), mask, kWave);
+            r.i = (IndexT)(((u64)hi << 32) | lo);
+        } else {
+            r.i = (IndexT)__shfl_xor((u32)i, mask, kWave);
+        }
+        return r;
+    }
+};
+
+// Folds the LANES (power of two, <= 64) consecutive lanes that share a result; every lane of the group ends up with it.
+template <int LANES, typename Acc>
+__device__ __forceinline__ void groupReduce(Acc& acc) {
+#pragma unroll
+    for (int mask = LANES / 2; mask >= 1; mask >>= 1) acc.merge(acc.shuffleXor(mask));
+}
+
+// Folds a whole block of THREADS threads (multiple of 64).  Returns the result in every thread of wavefront 0 (and in
+// all threads when BROADCAST is set).  `scratch` must hold THREADS / 64 accumulators in LDS; without BROADCAST there is
+// no trailing barrier, so a second fold in the same kernel needs its own scratch.
+template <int THREADS, bool BROADCAST, typename Acc>
+__device__ __forceinline__ void blockReduce(Acc& acc, Acc* scratch) {
+    groupReduce<kWave>(acc);
+    if (THREADS > kWave) {
+        constexpr int kWaves = THREADS / kWave;
+        const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+        if (lane == 0) scratch[wave] = acc;
+        __syncthreads();
+        if (wave == 0 || BROADCAST) {
+            Acc other;
+            other.reset();
+            if (lane < kWaves) other = scratch[lane];
+            groupReduce<kWave>(other);
+            acc = other;
+        }
+        if (BROADCAST) __syncthreads();
+    }
+}
+
+// Block-uniform "am I the last block to arrive" test.  The caller has written its partial; the fence orders that write
+// before the ticket, and the block that draws the last ticket re-arms the counter for the next launch.
+__device__ __forceinline__ bool lastBlockArrived(u32* counter, u32 expected, u32* sharedFlag) {
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const u32 ticket = atomicAdd(counter, 1u);
+        const bool last = ticket == expected - 1u;
+        if (last) *counter = 0u;
+        *sharedFlag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    const bool last = *sharedFlag != 0u;
+    if (last) __threadfence();
+    return last;
+}
+
+// ---- result finalisation -----------------------------------------------------------------------------------------------
+// FINALIZE: 0 none, 1 divide by `divisor` (mean), 2 square root (L2 norm).  Then the fp32 scale, then one conversion.
+template <int FINALIZE>
+__device__ __forceinline__ float finalizeValue(float acc, float divisor, float scale) {
+    float r = acc;
+    if (FINALIZE == 1) r = (divisor == 0.0f) ? 0.0f : ((divisor == 1.0f) ? acc : acc / divisor);
+    if (FINALIZE == 2) r = __builtin_sqrtf(acc);
+    return r * scale;
+}
+
+// digamma for x of either sign: reflection for x < 0.5, upward recurrence to x >= 6, then the asymptotic series
+__device__ inline float digammaf(float x) {
+    if (x != x) return x;
+    float reflection = 0.0f;
+    bool reflect = false;
+    if (x <= 0.0f && x == __builtin_floorf(x)) return __builtin_nanf("");
+    if (x < 0.5f) {
+        const float pi = 3.14159265358979323846f;
+        reflection = pi / tanf(pi * x);
+        reflect = true;
+        x = 1.0f - x;
+    }
+    float shift = 0.0f;
+    while (x < 6.0f) {
+        shift += 1.0f / x;
+        x += 1.0f;
+    }
+    const float inv = 1.0f / x, inv2 = inv * inv;
+    float series = inv2 * (1.0f / 12.0f - inv2 * (1.0f / 120.0f - inv2 * (1.0f / 252.0f - inv2 * (1.0f / 240.0f - inv2 * (1.0f / 132.0f)))));
+    float r = logf(x) - 0.5f * inv - series - shift;
+    return reflect ? r - reflection : r;
+}
+
+}  // namespace thor

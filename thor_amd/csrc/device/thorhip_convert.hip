@@ -4,10 +4,12 @@
 // (Utilities/TensorOperations/DataTypeConversions/TypeConverterKernels.cu:39-823,906-936,965-1338,1340-1433).
 //
 // Design for MI355X: the conversion is a pure HBM stream (6 B/element for fp32<->16-bit), so each lane moves whole
-// 16-byte words -- two dwordx4 loads and one dwordx4 store per slot for fp32->fp16 -- through a grid-stride loop
-// sized to a few resident waves per SIMD, with two slots in flight per lane.  A slot is a fixed, index-aligned group
-// of VEC elements; slots that straddle the [begin, end) range are handled element-wise, so nothing outside the range
-// is touched (the reference kernels over-read and over-write up to 15 elements into the tensor's 128-byte pad).
+// 16-byte words -- two dwordx4 loads and one dwordx4 store per slot for fp32->fp16 -- with non-temporal hints, one slot
+// per lane and as many 256-thread blocks as there are slots.  Measured on MI355X at 2^28 elements this shape (6.15 TB/s)
+// beats grid-stride loops capped at a few blocks per CU (5.3-5.9 TB/s) and cached loads/stores (5.4 TB/s); the loop
+// remains so that a capped grid can be selected with THORHIP_CONVERT_BLOCKS_PER_CU.  A slot is a fixed, index-aligned
+// group of VEC elements; slots that straddle the [begin, end) range are handled element-wise, so nothing outside the
+// range is touched (the reference kernels over-read and over-write up to 15 elements into the tensor's 128-byte pad).
 #include "thorhip.h"
 #include "thorhip_internal.h"
 #include "thorhip_numeric.h"
@@ -165,11 +167,11 @@ LaunchShape& launchShape() {
             (void)hipGetLastError();
             shape.compute_units = 256;
         }
-        // Resident blocks of 256 threads per CU the grid-stride loop is sized for.  8 blocks = 32 waves = 8 per SIMD.
-        shape.blocks_per_cu = 8;
+        // 0 = one slot per lane (no cap); a positive value caps the grid at that many 256-thread blocks per CU.
+        shape.blocks_per_cu = 0;
         if (const char* env = std::getenv("THORHIP_CONVERT_BLOCKS_PER_CU")) {
             const int v = std::atoi(env);
-            if (v >= 1 && v <= 64) shape.blocks_per_cu = v;
+            if (v >= 0 && v <= 4096) shape.blocks_per_cu = v;
         }
     });
     return shape;
@@ -179,7 +181,7 @@ unsigned gridFor(long work_items, int unroll) {
     const LaunchShape& shape = launchShape();
     const long per_block = (long)kBlockThreads * unroll;
     long blocks = (work_items + per_block - 1) / per_block;
-    const long cap = (long)shape.compute_units * shape.blocks_per_cu;
+    const long cap = shape.blocks_per_cu > 0 ? (long)shape.compute_units * shape.blocks_per_cu : 0x7fffffffL;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     return (unsigned)blocks;
@@ -195,7 +197,7 @@ template <typename From, typename To>
 int launchRange(const From* src, To* dst, long begin, long end, hipStream_t stream) {
     if (end <= begin) return 0;
     constexpr int VEC = Slot<From, To>::kVec;
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = 1;
     const size_t src_word = sizeof(From) * VEC >= 16 ? 16 : sizeof(From) * VEC;
     const size_t dst_word = sizeof(To) * VEC >= 16 ? 16 : sizeof(To) * VEC;
     if (alignedTo(src, src_word) && alignedTo(dst, dst_word)) {

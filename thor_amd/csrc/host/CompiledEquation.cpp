@@ -1,0 +1,98 @@
+#include "Utilities/Expression/CompiledEquation.h"
+
+#include "Utilities/Cache/LruCache.h"
+#include "Utilities/Common/ScopedGpu.h"
+
+#include <atomic>
+#include <stdexcept>
+#include <vector>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <mutex>
+
+namespace ThorImplementation {
+
+namespace {
+std::atomic<uint64_t> compileCount{0};
+
+LruCacheThreadSafe<std::string, std::shared_ptr<CompiledKernel>>& kernelCache() {
+    static LruCacheThreadSafe<std::string, std::shared_ptr<CompiledKernel>> cache(10000);
+    return cache;
+}
+
+LruCacheThreadSafe<std::string, std::shared_ptr<LoadedModule>>& moduleCache() {
+    static LruCacheThreadSafe<std::string, std::shared_ptr<LoadedModule>> cache(10000);
+    return cache;
+}
+
+std::string archOf(int deviceNum) {
+    static std::mutex mutex;
+    static std::vector<std::string> names;
+    std::lock_guard<std::mutex> lock(mutex);
+    if ((int)names.size() <= deviceNum) names.resize(deviceNum + 1);
+    if (names[deviceNum].empty()) {
+        thorhip_device_info info;
+        THOR_HIP_CHECK(thorhip_device_get_info(deviceNum, &info));
+        names[deviceNum] = info.arch_name;
+    }
+    return names[deviceNum];
+}
+}  // namespace
+
+LoadedModule::~LoadedModule() {
+    if (module != nullptr) {
+        int previous = 0;
+        const bool known = thorhip_get_device(&previous) == 0;
+        if (known && previous != deviceNum) (void)thorhip_set_device(deviceNum);
+        (void)thorhip_module_unload(module);
+        if (known && previous != deviceNum) (void)thorhip_set_device(previous);
+    }
+}
+
+void CompiledKernel::launch(uint32_t gridX, uint32_t gridY, uint32_t gridZ, uint32_t blockX, void* stream, std::vector<void*>& args) const {
+    THOR_HIP_CHECK(thorhip_launch(function, gridX, gridY, gridZ, blockX, 1, 1, 0, stream, args.data()));
+}
+
+uint64_t compiledKernelCount() { return compileCount.load(); }
+
+std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract) {
+    const std::string moduleKey = std::to_string(deviceNum) + (fastContract ? "|fast|" : "|off|") + source;
+    const std::string kernelKey = kernelName + "|" + moduleKey;
+    return kernelCache().getOrCreate(kernelKey, [&] {
+        ScopedGpu scoped(deviceNum);
+        std::shared_ptr<LoadedModule> loaded = moduleCache().getOrCreate(moduleKey, [&] {
+            const std::string arch = archOf(deviceNum);
+            const char* options[] = {fastContract ? "-ffp-contract=fast" : "-ffp-contract=off"};
+            void* code = nullptr;
+            size_t codeSize = 0;
+            std::vector<char> log(16384, 0);
+            if (const char* dump = std::getenv("THOR_DUMP_KERNEL_SOURCE")) {
+                std::ofstream out(std::string(dump) + "/" + kernelName + "_" + std::to_string(compileCount.load()) + ".hip");
+                out << source;
+            }
+            const int rc = thorhip_compile(source.c_str(), (kernelName + ".hip").c_str(), arch.c_str(), options, 1, &code, &codeSize,
+                                           log.data(), log.size());
+            if (rc != 0) {
+                throw std::runtime_error("Run-time compilation of kernel '" + kernelName + "' failed: " + thorhip_last_error());
+            }
+            auto module = std::make_shared<LoadedModule>();
+            module->deviceNum = deviceNum;
+            const int loadRc = thorhip_module_load(&module->module, code, codeSize);
+            (void)thorhip_code_free(code);
+            hipCheck(loadRc, "thorhip_module_load");
+            compileCount.fetch_add(1);
+            return module;
+        });
+        auto kernel = std::make_shared<CompiledKernel>();
+        kernel->module = loaded;
+        kernel->deviceNum = deviceNum;
+        kernel->kernelName = kernelName;
+        kernel->source = source;
+        THOR_HIP_CHECK(thorhip_module_get_function(&kernel->function, loaded->module, kernelName.c_str()));
+        (void)thorhip_function_get_attributes(kernel->function, &kernel->numRegisters, &kernel->staticLdsBytes, nullptr);
+        return kernel;
+    });
+}
+
+}  // namespace ThorImplementation

@@ -1,0 +1,630 @@
+// Graph construction for Expression (reference behaviour: Utilities/Expression/Expression.cpp:3057-3296,3604-3722,
+// 4176-4193,5084-5310).  Every operator builds a fresh PhysicalExpression holding copies of its operands' sub-DAGs with
+// the input slots merged by name; nodes shared inside one operand are copied once.
+#include "Utilities/Expression/Expression.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <functional>
+#include <limits>
+#include <sstream>
+#include <stdexcept>
+#include <unordered_set>
+
+namespace ThorImplementation {
+
+uint32_t PhysicalExpression::getOrCreateInputSlot(const std::string& name, NamedInput::Kind kind) {
+    for (const NamedInput& in : inputs) {
+        if (in.name == name) {
+            if (in.kind != kind) throw std::runtime_error("Input kind mismatch for input: " + name);
+            return in.slot;
+        }
+    }
+    const uint32_t slot = static_cast<uint32_t>(inputs.size());
+    inputs.push_back(NamedInput{name, slot, kind});
+    return slot;
+}
+
+PhysicalOutputs Outputs::physicalOutputs() const {
+    if (!expr) throw std::runtime_error("Outputs has no backing expression graph.");
+    return PhysicalOutputs{expr, outputs};
+}
+
+Outputs Outputs::fromPhysicalOutputs(PhysicalOutputs physicalOutputs) {
+    if (!physicalOutputs.expr) throw std::runtime_error("Outputs::fromPhysicalOutputs requires a non-null PhysicalExpression.");
+    return Outputs(std::move(physicalOutputs.expr), std::move(physicalOutputs.outputs));
+}
+
+namespace {
+
+void validateUserInputName(const std::string& name) {
+    if (name.empty()) throw std::invalid_argument("Expression input names must not be empty.");
+    if (name.rfind("__", 0) == 0) throw std::invalid_argument("Expression input names starting with '__' are reserved: " + name);
+}
+
+// Copies sub-DAGs into `dst`, keeping one copy per (source graph, source node) and one input slot per name.
+class GraphMerger {
+   public:
+    explicit GraphMerger(PhysicalExpression& dst) : dst(dst) {
+        for (const NamedInput& in : dst.inputs) slotByName[in.name] = in.slot;
+    }
+
+    uint32_t absorb(const PhysicalExpression& src, uint32_t root) {
+        if (root >= src.nodes.size()) throw std::runtime_error("Expression node index is out of range.");
+        std::unordered_map<uint32_t, uint32_t>& memo = memos[&src];
+        // children precede parents, so an ascending sweep over the reachable set needs no recursion
+        std::vector<char> needed(root + 1, 0);
+        needed[root] = 1;
+        for (uint32_t i = root + 1; i-- > 0;) {
+            if (!needed[i]) continue;
+            const ExprNode& n = src.nodes[i];
+            for (uint32_t child : {n.lhs, n.rhs, n.aux}) {
+                if (child == UINT32_MAX) continue;
+                if (child >= i) throw std::runtime_error("Expression graph is not topologically ordered.");
+                needed[child] = 1;
+            }
+        }
+        for (uint32_t i = 0; i <= root; ++i) {
+            if (!needed[i] || memo.count(i)) continue;
+            ExprNode copy = src.nodes[i];
+            if (copy.lhs != UINT32_MAX) copy.lhs = memo.at(copy.lhs);
+            if (copy.rhs != UINT32_MAX) copy.rhs = memo.at(copy.rhs);
+            if (copy.aux != UINT32_MAX) copy.aux = memo.at(copy.aux);
+            if (copy.op == ExprOp::INPUT || copy.op == ExprOp::RUNTIME_SCALAR || copy.op == ExprOp::TENSOR_RUNTIME_SCALAR) {
+                if (copy.input_slot >= src.inputs.size()) throw std::runtime_error("Input slot out of range while combining expressions.");
+                const NamedInput& in = src.inputs[copy.input_slot];
+                auto it = slotByName.find(in.name);
+                if (it == slotByName.end()) {
+                    const uint32_t slot = static_cast<uint32_t>(dst.inputs.size());
+                    dst.inputs.push_back(NamedInput{in.name, slot, in.kind});
+                    it = slotByName.emplace(in.name, slot).first;
+                } else if (dst.inputs[it->second].kind != in.kind) {
+                    throw std::runtime_error("Input kind mismatch while combining expressions for input: " + in.name);
+                }
+                copy.input_slot = it->second;
+            }
+            memo[i] = static_cast<uint32_t>(dst.nodes.size());
+            dst.nodes.push_back(std::move(copy));
+        }
+        return memo.at(root);
+    }
+
+   private:
+    PhysicalExpression& dst;
+    std::unordered_map<std::string, uint32_t> slotByName;
+    std::unordered_map<const PhysicalExpression*, std::unordered_map<uint32_t, uint32_t>> memos;
+};
+
+std::vector<uint64_t> sortedUnique(std::vector<uint64_t> v) {
+    std::sort(v.begin(), v.end());
+    v.erase(std::unique(v.begin(), v.end()), v.end());
+    return v;
+}
+
+}  // namespace
+
+// ---- leaves ------------------------------------------------------------------------------------------------------------
+Expression::Expression(double value) {
+    expr = std::make_shared<PhysicalExpression>();
+    ExprNode node;
+    node.op = ExprOp::SCALAR_FP;
+    node.scalar_fp = value;
+    expr->nodes.push_back(node);
+    expr->output_node = nodeIndex = 0;
+}
+
+Expression Expression::constantScalar(double value) { return Expression(value); }
+
+static Expression makeLeaf(ExprOp op, NamedInput::Kind kind, const std::string& name, std::optional<DataType> compute_dtype,
+                           std::optional<DataType> output_dtype, std::shared_ptr<PhysicalExpression>& out) {
+    validateUserInputName(name);
+    out = std::make_shared<PhysicalExpression>();
+    ExprNode node;
+    node.op = op;
+    node.input_slot = out->getOrCreateInputSlot(name, kind);
+    node.output_dtype = output_dtype;
+    node.compute_dtype = compute_dtype;
+    out->nodes.push_back(node);
+    out->output_node = 0;
+    return Expression::fromPhysicalNode(out, 0);
+}
+
+Expression Expression::input(const std::string& name, std::optional<DataType> compute_dtype, std::optional<DataType> output_dtype) {
+    std::shared_ptr<PhysicalExpression> out;
+    return makeLeaf(ExprOp::INPUT, NamedInput::Kind::Tensor, name, compute_dtype, output_dtype, out);
+}
+
+Expression Expression::runtimeScalar(const std::string& name, std::optional<DataType> compute_dtype, std::optional<DataType> output_dtype) {
+    std::shared_ptr<PhysicalExpression> out;
+    return makeLeaf(ExprOp::RUNTIME_SCALAR, NamedInput::Kind::RuntimeScalarFp32, name, compute_dtype, output_dtype, out);
+}
+
+Expression Expression::fill(double value, const std::vector<uint64_t>& dims, std::optional<DataType> output_dtype) {
+    if (dims.empty()) throw std::invalid_argument("Expression::fill requires non-empty concrete dimensions; use constantScalar for a scalar.");
+    for (uint64_t d : dims) {
+        if (d == 0 || d == std::numeric_limits<uint64_t>::max()) throw std::invalid_argument("Expression::fill requires concrete non-zero dimensions.");
+    }
+    auto out = std::make_shared<PhysicalExpression>();
+    ExprNode node;
+    node.op = ExprOp::FILL;
+    node.scalar_fp = value;
+    node.fill_dims = dims;
+    node.output_dtype = output_dtype;
+    out->nodes.push_back(node);
+    out->output_node = 0;
+    return Expression(out, 0);
+}
+
+Expression Expression::fromPhysicalNode(std::shared_ptr<PhysicalExpression> expr, uint32_t nodeIndex) {
+    if (!expr) throw std::invalid_argument("Expression::fromPhysicalNode requires a non-null PhysicalExpression.");
+    if (nodeIndex >= expr->nodes.size()) throw std::out_of_range("Expression::fromPhysicalNode node index is out of range.");
+    return Expression(std::move(expr), nodeIndex);
+}
+
+PhysicalExpression Expression::expression() const {
+    if (!expr) throw std::runtime_error("Expression has no underlying graph.");
+    PhysicalExpression out = *expr;
+    out.output_node = nodeIndex;
+    return out;
+}
+
+std::set<std::string> Expression::getInputNames() const {
+    if (!expr) throw std::runtime_error("Expression has no underlying graph.");
+    // only the inputs reachable from this node
+    std::set<std::string> names;
+    std::vector<char> seen(nodeIndex + 1, 0);
+    seen[nodeIndex] = 1;
+    for (uint32_t i = nodeIndex + 1; i-- > 0;) {
+        if (!seen[i]) continue;
+        const ExprNode& n = expr->nodes[i];
+        for (uint32_t c : {n.lhs, n.rhs, n.aux})
+            if (c != UINT32_MAX) seen[c] = 1;
+        if (n.input_slot != UINT32_MAX) names.insert(expr->inputs.at(n.input_slot).name);
+    }
+    return names;
+}
+
+// ---- combinators -------------------------------------------------------------------------------------------------------
+Expression Expression::unaryOp(const Expression& input, ExprOp op) {
+    if (!input.expr) throw std::runtime_error("Cannot apply unary op to empty expression");
+    auto out = std::make_shared<PhysicalExpression>();
+    GraphMerger merger(*out);
+    ExprNode node;
+    node.op = op;
+    node.lhs = merger.absorb(*input.expr, input.nodeIndex);
+    out->nodes.push_back(node);
+    out->output_node = static_cast<uint32_t>(out->nodes.size() - 1);
+    return Expression(out, out->output_node);
+}
+
+Expression Expression::binaryOp(const Expression& lhs, const Expression& rhs, ExprOp op) {
+    if (!lhs.expr || !rhs.expr) throw std::runtime_error("Cannot combine empty expressions");
+    auto out = std::make_shared<PhysicalExpression>();
+    GraphMerger merger(*out);
+    ExprNode node;
+    node.op = op;
+    node.lhs = merger.absorb(*lhs.expr, lhs.nodeIndex);
+    node.rhs = merger.absorb(*rhs.expr, rhs.nodeIndex);
+    out->nodes.push_back(node);
+    out->output_node = static_cast<uint32_t>(out->nodes.size() - 1);
+    return Expression(out, out->output_node);
+}
+
+Expression Expression::ternaryOp(const Expression& a, const Expression& b, const Expression& c, ExprOp op) {
+    if (!a.expr || !b.expr || !c.expr) throw std::runtime_error("Cannot combine empty expressions");
+    auto out = std::make_shared<PhysicalExpression>();
+    GraphMerger merger(*out);
+    ExprNode node;
+    node.op = op;
+    node.lhs = merger.absorb(*a.expr, a.nodeIndex);
+    node.rhs = merger.absorb(*b.expr, b.nodeIndex);
+    node.aux = merger.absorb(*c.expr, c.nodeIndex);
+    out->nodes.push_back(node);
+    out->output_node = static_cast<uint32_t>(out->nodes.size() - 1);
+    return Expression(out, out->output_node);
+}
+
+Outputs Expression::outputs(const std::vector<std::pair<std::string, Expression>>& named_exprs) {
+    if (named_exprs.empty()) throw std::runtime_error("Expression::outputs requires at least one named output.");
+    auto merged = std::make_shared<PhysicalExpression>();
+    GraphMerger merger(*merged);
+    std::vector<NamedOutput> outs;
+    std::unordered_set<std::string> seen;
+    for (const auto& [name, e] : named_exprs) {
+        if (name.empty()) throw std::runtime_error("Output name cannot be empty.");
+        if (!seen.insert(name).second) throw std::runtime_error("Duplicate output name: " + name);
+        if (!e.expr) throw std::runtime_error("Output expression has no backing PhysicalExpression.");
+        outs.push_back(NamedOutput{name, merger.absorb(*e.expr, e.nodeIndex)});
+    }
+    merged->output_node = outs.back().node_idx;
+    return Outputs(std::move(merged), std::move(outs));
+}
+
+Outputs Expression::outputs(std::initializer_list<std::pair<std::string, Expression>> named_exprs) {
+    return outputs(std::vector<std::pair<std::string, Expression>>(named_exprs));
+}
+
+// ---- operators -----------------------------------------------------------------------------------------------------------
+Expression Expression::operator+(const Expression& o) const { return binaryOp(*this, o, ExprOp::ADD); }
+Expression Expression::operator-(const Expression& o) const { return binaryOp(*this, o, ExprOp::SUB); }
+Expression Expression::operator*(const Expression& o) const { return binaryOp(*this, o, ExprOp::MUL); }
+Expression Expression::operator/(const Expression& o) const { return binaryOp(*this, o, ExprOp::DIV); }
+Expression Expression::operator-() const { return unaryOp(*this, ExprOp::NEG); }
+Expression Expression::operator!() const { return logicalNot(); }
+Expression Expression::operator==(const Expression& o) const { return equal(o); }
+Expression Expression::operator!=(const Expression& o) const { return notEqual(o); }
+Expression Expression::operator<(const Expression& o) const { return lessThan(o); }
+Expression Expression::operator<=(const Expression& o) const { return lessEqual(o); }
+Expression Expression::operator>(const Expression& o) const { return greaterThan(o); }
+Expression Expression::operator>=(const Expression& o) const { return greaterEqual(o); }
+
+Expression Expression::equal(const Expression& o) const { return binaryOp(*this, o, ExprOp::EQUAL); }
+Expression Expression::notEqual(const Expression& o) const { return binaryOp(*this, o, ExprOp::NOT_EQUAL); }
+Expression Expression::lessThan(const Expression& o) const { return binaryOp(*this, o, ExprOp::LESS); }
+Expression Expression::lessEqual(const Expression& o) const { return binaryOp(*this, o, ExprOp::LESS_EQUAL); }
+Expression Expression::greaterThan(const Expression& o) const { return binaryOp(*this, o, ExprOp::GREATER); }
+Expression Expression::greaterEqual(const Expression& o) const { return binaryOp(*this, o, ExprOp::GREATER_EQUAL); }
+Expression Expression::logicalAnd(const Expression& o) const { return binaryOp(*this, o, ExprOp::LOGICAL_AND); }
+Expression Expression::logicalOr(const Expression& o) const { return binaryOp(*this, o, ExprOp::LOGICAL_OR); }
+Expression Expression::logicalNot() const { return unaryOp(*this, ExprOp::LOGICAL_NOT); }
+Expression Expression::pow(const Expression& e) const { return binaryOp(*this, e, ExprOp::POW); }
+Expression Expression::min(const Expression& o) const { return binaryOp(*this, o, ExprOp::MIN); }
+Expression Expression::max(const Expression& o) const { return binaryOp(*this, o, ExprOp::MAX); }
+
+Expression Expression::cast(DataType output_dtype) const {
+    Expression result = unaryOp(*this, ExprOp::CAST);
+    ExprNode& node = result.expr->nodes[result.nodeIndex];
+    node.output_dtype = output_dtype;
+    node.compute_dtype = output_dtype;
+    return result;
+}
+
+Expression Expression::where(const Expression& condition, const Expression& true_value, const Expression& false_value) {
+    return ternaryOp(condition, true_value, false_value, ExprOp::WHERE);
+}
+Expression Expression::select(const Expression& true_value, const Expression& false_value) const { return where(*this, true_value, false_value); }
+
+#define THOR_UNARY(method, OP) \
+    Expression Expression::method() const { return unaryOp(*this, ExprOp::OP); }
+THOR_UNARY(abs, ABS)
+THOR_UNARY(ceil, CEIL)
+THOR_UNARY(floor, FLOOR)
+THOR_UNARY(round, ROUND)
+THOR_UNARY(trunc, TRUNC)
+THOR_UNARY(sin, SIN)
+THOR_UNARY(cos, COS)
+THOR_UNARY(tan, TAN)
+THOR_UNARY(asin, ASIN)
+THOR_UNARY(acos, ACOS)
+THOR_UNARY(atan, ATAN)
+THOR_UNARY(sinh, SINH)
+THOR_UNARY(cosh, COSH)
+THOR_UNARY(tanh, TANH)
+THOR_UNARY(asinh, ASINH)
+THOR_UNARY(acosh, ACOSH)
+THOR_UNARY(atanh, ATANH)
+THOR_UNARY(erf, ERF)
+THOR_UNARY(erfc, ERFC)
+THOR_UNARY(erfcx, ERFCX)
+THOR_UNARY(erfinv, ERFINV)
+THOR_UNARY(erfcinv, ERFCINV)
+THOR_UNARY(tgamma, TGAMMA)
+THOR_UNARY(lgamma, LGAMMA)
+THOR_UNARY(digamma, DIGAMMA)
+THOR_UNARY(exp, EXP)
+THOR_UNARY(expm1, EXPM1)
+THOR_UNARY(exp2, EXP2)
+THOR_UNARY(exp10, EXP10)
+THOR_UNARY(ln, LN)
+THOR_UNARY(log1p, LOG1P)
+THOR_UNARY(log2, LOG2)
+THOR_UNARY(log10, LOG10)
+THOR_UNARY(sqrt, SQRT)
+THOR_UNARY(normcdf, NORMCDF)
+#undef THOR_UNARY
+
+// reciprocal / inverse-reciprocal trigonometry: 1 / f(x) and f(1 / x)
+Expression Expression::csc() const { return constantScalar(1.0) / sin(); }
+Expression Expression::sec() const { return constantScalar(1.0) / cos(); }
+Expression Expression::cot() const { return constantScalar(1.0) / tan(); }
+Expression Expression::csch() const { return constantScalar(1.0) / sinh(); }
+Expression Expression::sech() const { return constantScalar(1.0) / cosh(); }
+Expression Expression::coth() const { return constantScalar(1.0) / tanh(); }
+Expression Expression::acsc() const { return (constantScalar(1.0) / *this).asin(); }
+Expression Expression::asec() const { return (constantScalar(1.0) / *this).acos(); }
+Expression Expression::acot() const { return (constantScalar(1.0) / *this).atan(); }
+Expression Expression::acsch() const { return (constantScalar(1.0) / *this).asinh(); }
+Expression Expression::asech() const { return (constantScalar(1.0) / *this).acosh(); }
+Expression Expression::acoth() const { return (constantScalar(1.0) / *this).atanh(); }
+
+Expression Expression::log(double base) const {
+    if (base <= 0.0 || base == 1.0) {
+        throw std::runtime_error("log base must be positive and not equal to 1, received base = " + std::to_string(base));
+    }
+    return ln() / constantScalar(std::log(base));
+}
+
+Expression Expression::clamp(const Expression& lower_bound, const Expression& upper_bound) const { return max(lower_bound).min(upper_bound); }
+Expression Expression::clamp(double lower_bound, double upper_bound) const {
+    if (lower_bound > upper_bound) throw std::invalid_argument("Expression::clamp requires lower_bound <= upper_bound.");
+    return clamp(constantScalar(lower_bound), constantScalar(upper_bound));
+}
+
+// sigmoid(x) = exp(-max(-x, 0)) / (1 + exp(-|x|)): finite for both signs of large |x|
+Expression Expression::sigmoid() const {
+    const Expression negated = -*this;
+    const Expression numerator = (-negated.max(Expression(0.0))).exp();
+    const Expression denominator = Expression(1.0) + (-abs()).exp();
+    return numerator / denominator;
+}
+// log(1 + e^x) = max(x, 0) + log1p(e^-|x|)
+Expression Expression::softplus() const { return max(Expression(0.0)) + (-abs()).exp().log1p(); }
+// expm1 of min(x, 0) never evaluates e^x for positive x and keeps precision near zero
+Expression Expression::elu(double alpha) const { return max(Expression(0.0)) + (min(Expression(0.0)).expm1() * Expression(alpha)); }
+Expression Expression::selu() const {
+    return (max(Expression(0.0)) * Expression(1.05070098)) + (min(Expression(0.0)).expm1() * Expression(1.758099326));
+}
+Expression Expression::gelu() const { return *this * normcdf(); }
+Expression Expression::mish() const { return *this * softplus().tanh(); }
+Expression Expression::relu6() const { return max(Expression(0.0)).min(Expression(6.0)); }
+Expression Expression::hardTanh(double min_value, double max_value) const {
+    if (min_value > max_value) throw std::invalid_argument("Expression::hardTanh requires min_value <= max_value.");
+    return max(Expression(min_value)).min(Expression(max_value));
+}
+Expression Expression::hardSwish() const { return *this * ((*this + Expression(3.0)).relu6() / Expression(6.0)); }
+Expression Expression::threshold(double threshold, double value) const {
+    return where(*this > Expression(threshold), *this, Expression(value));
+}
+Expression Expression::swish() const { return *this * sigmoid(); }
+
+// ---- shape ---------------------------------------------------------------------------------------------------------------
+Expression Expression::reshape(const std::vector<uint64_t>& new_dims) const {
+    if (new_dims.empty()) throw std::invalid_argument("Expression::reshape requires at least one dimension.");
+    if (std::count(new_dims.begin(), new_dims.end(), std::numeric_limits<uint64_t>::max()) > 1) {
+        throw std::invalid_argument("Expression::reshape supports at most one infer-dimension marker.");
+    }
+    Expression out = unaryOp(*this, ExprOp::RESHAPE);
+    out.expr->nodes[out.nodeIndex].reshape_dims = new_dims;
+    return out;
+}
+
+Expression Expression::unsqueeze(const std::vector<uint64_t>& axes) const {
+    Expression out = unaryOp(*this, ExprOp::UNSQUEEZE);
+    out.expr->nodes[out.nodeIndex].unsqueeze_axes = sortedUnique(axes);
+    return out;
+}
+
+Expression Expression::squeeze(const std::vector<uint64_t>& axes) const {
+    Expression out = unaryOp(*this, ExprOp::SQUEEZE);
+    out.expr->nodes[out.nodeIndex].squeeze_axes = sortedUnique(axes);
+    return out;
+}
+
+// ---- reductions -----------------------------------------------------------------------------------------------------------
+Expression Expression::reduction(ExprOp op, const std::vector<uint64_t>& reduction_axes, const std::vector<uint64_t>& squeeze_axes,
+                                 std::optional<DataType> compute_dtype) const {
+    if (!isReductionOp(op)) throw std::invalid_argument("Expression::reduction requires a reduction op.");
+    if (compute_dtype.has_value() && compute_dtype.value() != DataType::FP32) {
+        throw std::runtime_error("Reductions accumulate in FP32; requested compute dtype " + std::string(dataTypeName(compute_dtype.value())) +
+                                 " is not supported.");
+    }
+    Expression out = unaryOp(*this, op);
+    ExprNode& node = out.expr->nodes[out.nodeIndex];
+    node.reduction_axes = reduction_axes;
+    node.squeeze_axes = squeeze_axes;
+    node.compute_dtype = DataType::FP32;
+    if (isArgReductionOp(op)) node.output_dtype = DataType::UINT32;
+    return out;
+}
+
+#define THOR_REDUCTION(method, OP)                                                                                           \
+    Expression Expression::method(const std::vector<uint64_t>& axes, const std::vector<uint64_t>& squeeze,                    \
+                                  std::optional<DataType> compute_dtype) const {                                              \
+        return reduction(ExprOp::OP, axes, squeeze, compute_dtype);                                                           \
+    }
+THOR_REDUCTION(reduce_sum, REDUCE_SUM)
+THOR_REDUCTION(reduce_prod, REDUCE_PROD)
+THOR_REDUCTION(reduce_min, REDUCE_MIN)
+THOR_REDUCTION(reduce_max, REDUCE_MAX)
+THOR_REDUCTION(reduce_mean, REDUCE_AVG)
+THOR_REDUCTION(reduce_norm1, REDUCE_NORM1)
+THOR_REDUCTION(reduce_norm2, REDUCE_NORM2)
+THOR_REDUCTION(argmin, REDUCE_ARGMIN)
+THOR_REDUCTION(argmax, REDUCE_ARGMAX)
+#undef THOR_REDUCTION
+
+Expression Expression::dotProduct(const Expression& other, std::optional<DataType> compute_dtype) const {
+    return dotProduct(*this, other, compute_dtype);
+}
+Expression Expression::dotProduct(const Expression& lhs, const Expression& rhs, std::optional<DataType> compute_dtype) {
+    return (lhs * rhs).reduce_sum({}, {UINT64_MAX}, compute_dtype);
+}
+
+Expression Expression::withDTypes(std::optional<DataType> compute_dtype, std::optional<DataType> output_dtype) const {
+    if (!expr) throw std::runtime_error("Cannot override dtypes on an empty expression");
+    auto out = std::make_shared<PhysicalExpression>();
+    GraphMerger merger(*out);
+    const uint32_t root = merger.absorb(*expr, nodeIndex);
+    out->output_node = root;
+    if (compute_dtype.has_value()) out->nodes[root].compute_dtype = compute_dtype;
+    if (output_dtype.has_value()) out->nodes[root].output_dtype = output_dtype;
+    return Expression(out, root);
+}
+
+// ---- op classification ---------------------------------------------------------------------------------------------------
+bool Expression::isLeafOp(ExprOp op) {
+    return op == ExprOp::INPUT || op == ExprOp::RUNTIME_SCALAR || op == ExprOp::TENSOR_RUNTIME_SCALAR || op == ExprOp::SCALAR_FP ||
+           op == ExprOp::FILL;
+}
+
+bool Expression::isBinaryOp(ExprOp op) {
+    switch (op) {
+        case ExprOp::ADD:
+        case ExprOp::SUB:
+        case ExprOp::MUL:
+        case ExprOp::DIV:
+        case ExprOp::POW:
+        case ExprOp::EQUAL:
+        case ExprOp::NOT_EQUAL:
+        case ExprOp::LESS:
+        case ExprOp::LESS_EQUAL:
+        case ExprOp::GREATER:
+        case ExprOp::GREATER_EQUAL:
+        case ExprOp::LOGICAL_AND:
+        case ExprOp::LOGICAL_OR:
+        case ExprOp::MIN:
+        case ExprOp::MAX:
+        case ExprOp::MIN_GRAD_LEFT:
+        case ExprOp::MIN_GRAD_RIGHT:
+        case ExprOp::MAX_GRAD_LEFT:
+        case ExprOp::MAX_GRAD_RIGHT:
+            return true;
+        default:
+            return false;
+    }
+}
+
+bool Expression::isTernaryOp(ExprOp op) { return op == ExprOp::WHERE; }
+
+bool Expression::isUnaryOp(ExprOp op) {
+    if (isLeafOp(op) || isBinaryOp(op) || isTernaryOp(op)) return false;
+    if (isReductionOp(op)) return true;
+    switch (op) {
+        case ExprOp::LOGICAL_NOT:
+        case ExprOp::CAST:
+        case ExprOp::RESHAPE:
+        case ExprOp::UNSQUEEZE:
+        case ExprOp::SQUEEZE:
+            return true;
+        default:
+            return op >= ExprOp::NEG && op <= ExprOp::NORMCDF;
+    }
+}
+
+// ---- canonical text -------------------------------------------------------------------------------------------------------
+std::string opName(ExprOp op) {
+    static const std::unordered_map<uint16_t, const char*> names = {
+        {(uint16_t)ExprOp::INPUT, "input"}, {(uint16_t)ExprOp::RUNTIME_SCALAR, "runtime_scalar"},
+        {(uint16_t)ExprOp::TENSOR_RUNTIME_SCALAR, "tensor_runtime_scalar"}, {(uint16_t)ExprOp::SCALAR_FP, "scalar"},
+        {(uint16_t)ExprOp::ADD, "add"}, {(uint16_t)ExprOp::SUB, "sub"}, {(uint16_t)ExprOp::MUL, "mul"}, {(uint16_t)ExprOp::DIV, "div"},
+        {(uint16_t)ExprOp::POW, "pow"}, {(uint16_t)ExprOp::EQUAL, "eq"}, {(uint16_t)ExprOp::NOT_EQUAL, "ne"}, {(uint16_t)ExprOp::LESS, "lt"},
+        {(uint16_t)ExprOp::LESS_EQUAL, "le"}, {(uint16_t)ExprOp::GREATER, "gt"}, {(uint16_t)ExprOp::GREATER_EQUAL, "ge"},
+        {(uint16_t)ExprOp::LOGICAL_AND, "and"}, {(uint16_t)ExprOp::LOGICAL_OR, "or"}, {(uint16_t)ExprOp::LOGICAL_NOT, "not"},
+        {(uint16_t)ExprOp::CAST, "cast"}, {(uint16_t)ExprOp::WHERE, "where"}, {(uint16_t)ExprOp::NEG, "neg"}, {(uint16_t)ExprOp::ABS, "abs"},
+        {(uint16_t)ExprOp::CEIL, "ceil"}, {(uint16_t)ExprOp::FLOOR, "floor"}, {(uint16_t)ExprOp::ROUND, "round"},
+        {(uint16_t)ExprOp::TRUNC, "trunc"}, {(uint16_t)ExprOp::SIN, "sin"}, {(uint16_t)ExprOp::COS, "cos"}, {(uint16_t)ExprOp::TAN, "tan"},
+        {(uint16_t)ExprOp::ASIN, "asin"}, {(uint16_t)ExprOp::ACOS, "acos"}, {(uint16_t)ExprOp::ATAN, "atan"}, {(uint16_t)ExprOp::SINH, "sinh"},
+        {(uint16_t)ExprOp::COSH, "cosh"}, {(uint16_t)ExprOp::ASINH, "asinh"}, {(uint16_t)ExprOp::ACOSH, "acosh"},
+        {(uint16_t)ExprOp::ATANH, "atanh"}, {(uint16_t)ExprOp::ERF, "erf"}, {(uint16_t)ExprOp::ERFC, "erfc"}, {(uint16_t)ExprOp::ERFCX, "erfcx"},
+        {(uint16_t)ExprOp::ERFINV, "erfinv"}, {(uint16_t)ExprOp::ERFCINV, "erfcinv"}, {(uint16_t)ExprOp::TGAMMA, "tgamma"},
+        {(uint16_t)ExprOp::LGAMMA, "lgamma"}, {(uint16_t)ExprOp::DIGAMMA, "digamma"}, {(uint16_t)ExprOp::EXP, "exp"},
+        {(uint16_t)ExprOp::EXPM1, "expm1"}, {(uint16_t)ExprOp::EXP2, "exp2"}, {(uint16_t)ExprOp::EXP10, "exp10"}, {(uint16_t)ExprOp::LN, "ln"},
+        {(uint16_t)ExprOp::LOG1P, "log1p"}, {(uint16_t)ExprOp::LOG2, "log2"}, {(uint16_t)ExprOp::LOG10, "log10"}, {(uint16_t)ExprOp::SQRT, "sqrt"},
+        {(uint16_t)ExprOp::TANH, "tanh"}, {(uint16_t)ExprOp::NORMCDF, "normcdf"}, {(uint16_t)ExprOp::FILL, "fill"},
+        {(uint16_t)ExprOp::RESHAPE, "reshape"}, {(uint16_t)ExprOp::UNSQUEEZE, "unsqueeze"}, {(uint16_t)ExprOp::SQUEEZE, "squeeze"},
+        {(uint16_t)ExprOp::MIN, "min"}, {(uint16_t)ExprOp::MAX, "max"}, {(uint16_t)ExprOp::MIN_GRAD_LEFT, "min_grad_left"},
+        {(uint16_t)ExprOp::MIN_GRAD_RIGHT, "min_grad_right"}, {(uint16_t)ExprOp::MAX_GRAD_LEFT, "max_grad_left"},
+        {(uint16_t)ExprOp::MAX_GRAD_RIGHT, "max_grad_right"}, {(uint16_t)ExprOp::REDUCE_SUM, "reduce_sum"},
+        {(uint16_t)ExprOp::REDUCE_PROD, "reduce_prod"}, {(uint16_t)ExprOp::REDUCE_MIN, "reduce_min"}, {(uint16_t)ExprOp::REDUCE_MAX, "reduce_max"},
+        {(uint16_t)ExprOp::REDUCE_ARGMIN, "argmin"}, {(uint16_t)ExprOp::REDUCE_ARGMAX, "argmax"}, {(uint16_t)ExprOp::REDUCE_AVG, "reduce_mean"},
+        {(uint16_t)ExprOp::REDUCE_NORM1, "reduce_norm1"}, {(uint16_t)ExprOp::REDUCE_NORM2, "reduce_norm2"},
+    };
+    auto it = names.find(static_cast<uint16_t>(op));
+    return it == names.end() ? "op" + std::to_string(static_cast<int>(op)) : it->second;
+}
+
+bool isCommutative(ExprOp op) {
+    switch (op) {
+        case ExprOp::ADD:
+        case ExprOp::MUL:
+        case ExprOp::MIN:
+        case ExprOp::MAX:
+        case ExprOp::EQUAL:
+        case ExprOp::NOT_EQUAL:
+        case ExprOp::LOGICAL_AND:
+        case ExprOp::LOGICAL_OR:
+            return true;
+        default:
+            return false;
+    }
+}
+
+std::string formatFloatCanonical(double x) {
+    char buffer[64];
+    std::snprintf(buffer, sizeof buffer, "%.17g", x);
+    return buffer;
+}
+
+static std::string axesText(const std::vector<uint64_t>& v) {
+    std::string s = "[";
+    for (size_t i = 0; i < v.size(); ++i) s += (i ? "," : "") + std::to_string(v[i]);
+    return s + "]";
+}
+
+std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex, std::unordered_map<uint32_t, std::string>& memo) {
+    auto hit = memo.find(nodeIndex);
+    if (hit != memo.end()) return hit->second;
+    const ExprNode& n = expr.nodes.at(nodeIndex);
+    std::string text = opName(n.op);
+    auto dtypes = [&] {
+        std::string s;
+        if (n.output_dtype) s += std::string(":o=") + dataTypeName(*n.output_dtype);
+        if (n.compute_dtype) s += std::string(":c=") + dataTypeName(*n.compute_dtype);
+        if (n.input_tensor_dtype) s += std::string(":i=") + dataTypeName(*n.input_tensor_dtype);
+        return s;
+    };
+    if (n.op == ExprOp::INPUT || n.op == ExprOp::RUNTIME_SCALAR || n.op == ExprOp::TENSOR_RUNTIME_SCALAR) {
+        text += "#" + std::to_string(n.input_slot) + dtypes();
+    } else if (n.op == ExprOp::SCALAR_FP) {
+        text += "(" + formatFloatCanonical(n.scalar_fp) + ")" + dtypes();
+    } else if (n.op == ExprOp::FILL) {
+        text += "(" + formatFloatCanonical(n.scalar_fp) + "," + axesText(n.fill_dims) + ")" + dtypes();
+    } else {
+        std::vector<std::string> kids;
+        for (uint32_t c : {n.lhs, n.rhs, n.aux})
+            if (c != UINT32_MAX) kids.push_back(canonicalizeNode(expr, c, memo));
+        if (isCommutative(n.op) && kids.size() == 2 && kids[1] < kids[0]) std::swap(kids[0], kids[1]);
+        text += dtypes();
+        if (isReductionOp(n.op)) text += ":axes=" + axesText(n.reduction_axes) + ":squeeze=" + axesText(n.squeeze_axes);
+        if (n.op == ExprOp::RESHAPE) text += ":dims=" + axesText(n.reshape_dims);
+        if (n.op == ExprOp::UNSQUEEZE) text += ":axes=" + axesText(n.unsqueeze_axes);
+        if (n.op == ExprOp::SQUEEZE) text += ":axes=" + axesText(n.squeeze_axes);
+        text += "(";
+        for (size_t i = 0; i < kids.size(); ++i) text += (i ? "," : "") + kids[i];
+        text += ")";
+    }
+    memo[nodeIndex] = text;
+    return text;
+}
+
+std::string canonicalize(const PhysicalExpression& expr) {
+    std::unordered_map<uint32_t, std::string> memo;
+    return canonicalizeNode(expr, expr.output_node, memo);
+}
+
+std::string canonicalize(const PhysicalOutputs& outputs) {
+    if (!outputs.expr) throw std::runtime_error("canonicalize requires a non-null expression graph.");
+    std::unordered_map<uint32_t, std::string> memo;
+    std::vector<std::string> parts;
+    for (const NamedOutput& o : outputs.outputs) parts.push_back(o.name + "=" + canonicalizeNode(*outputs.expr, o.node_idx, memo));
+    std::sort(parts.begin(), parts.end());
+    std::string text;
+    for (const std::string& p : parts) text += p + ";";
+    return text;
+}
+
+std::string expressionHash(const PhysicalOutputs& outputs) {
+    // FNV-1a over the canonical text, printed as 16 hex digits
+    const std::string text = canonicalize(outputs);
+    uint64_t h = 1469598103934665603ull;
+    for (unsigned char c : text) {
+        h ^= c;
+        h *= 1099511628211ull;
+    }
+    char buffer[32];
+    std::snprintf(buffer, sizeof buffer, "%016llx", static_cast<unsigned long long>(h));
+    return buffer;
+}
+
+}  // namespace ThorImplementation

@@ -1,0 +1,735 @@
+// Planning and stamping of compiled expressions: dtype resolution, de-duplication, the split into stages at reduction
+// boundaries, shape inference, output allocation and kernel generation per stage
+// (reference behaviour: Utilities/Expression/EquationCompiler.cpp:6572-7879 planExecution,
+//  Utilities/Expression/FusedEquation.cpp:666-710 broadcasting, :6828-6887 per-dtype compilation, :8885-9353 stamp,
+//  :10760-10905 convenience run).
+#include "Utilities/Expression/FusedEquation.h"
+
+#include "HipSourceEmitter.h"
+#include "ReductionPlanner.h"
+#include "RowFusion.h"
+#include "Utilities/Common/ScopedGpu.h"
+#include "Utilities/Expression/ExpressionDTypeResolution.h"
+
+#include <algorithm>
+#include <cstdlib>
+#include <limits>
+#include <map>
+#include <numeric>
+#include <sstream>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+struct PlannedGraph {
+    enum class Role : uint8_t { Inline, InputSource, Materialized, View };
+    PhysicalExpression expr;  // dtype-resolved, de-duplicated, reachable nodes only
+    std::vector<NamedOutput> outputs;
+    std::vector<Role> role;
+    std::vector<uint32_t> level;  // Materialized nodes: position in the dependency order
+};
+
+namespace {
+
+using Role = PlannedGraph::Role;
+
+bool isShapeOnly(ExprOp op) { return op == ExprOp::RESHAPE || op == ExprOp::UNSQUEEZE || op == ExprOp::SQUEEZE; }
+bool isReductionStorage(DataType d) {
+    return d == DataType::FP8_E4M3 || d == DataType::FP8_E5M2 || d == DataType::FP16 || d == DataType::BF16 || d == DataType::FP32;
+}
+
+std::string axesKey(const std::vector<uint64_t>& v) {
+    std::string s;
+    for (uint64_t a : v) s += std::to_string(a) + ",";
+    return s;
+}
+
+std::string structuralKey(const ExprNode& n) {
+    std::ostringstream k;
+    k << static_cast<int>(n.op) << "|" << n.lhs << "|" << n.rhs << "|" << n.aux << "|" << n.input_slot << "|" << formatFloatCanonical(n.scalar_fp)
+      << "|" << (n.input_tensor_dtype ? static_cast<int>(*n.input_tensor_dtype) : -1) << "|" << (n.output_dtype ? static_cast<int>(*n.output_dtype) : -1)
+      << "|" << (n.compute_dtype ? static_cast<int>(*n.compute_dtype) : -1) << "|" << axesKey(n.reduction_axes) << "|" << axesKey(n.squeeze_axes)
+      << "|" << axesKey(n.unsqueeze_axes) << "|" << axesKey(n.reshape_dims) << "|" << axesKey(n.fill_dims);
+    return k.str();
+}
+
+// Rebuilds the reachable part of a resolved graph without duplicate nodes and with explicit CAST nodes wherever a
+// tensor consumer (reduction, shape op, named output) needs an input in a dtype its bound tensor does not have.
+class GraphBuilder {
+   public:
+    explicit GraphBuilder(const PhysicalExpression& src) : src(src) { out.inputs = src.inputs; }
+
+    uint32_t add(ExprNode node) {
+        if (isCommutative(node.op) && node.rhs != UINT32_MAX && node.rhs < node.lhs) std::swap(node.lhs, node.rhs);
+        const std::string key = structuralKey(node);
+        auto it = byKey.find(key);
+        if (it != byKey.end()) return it->second;
+        const uint32_t idx = static_cast<uint32_t>(out.nodes.size());
+        out.nodes.push_back(std::move(node));
+        byKey.emplace(key, idx);
+        return idx;
+    }
+
+    uint32_t castOf(uint32_t child, DataType dtype) {
+        ExprNode cast;
+        cast.op = ExprOp::CAST;
+        cast.lhs = child;
+        cast.output_dtype = dtype;
+        cast.compute_dtype = dtype;
+        return add(cast);
+    }
+
+    // index (in the new graph) of a node that can stand for `child` as a tensor of its value dtype
+    uint32_t asTensorOperand(uint32_t child, bool forReduction) {
+        const ExprNode& c = out.nodes[child];
+        DataType valueDType = c.output_dtype.value();
+        if (forReduction && !isReductionStorage(valueDType)) return castOf(child, DataType::FP32);
+        if (c.op == ExprOp::INPUT && c.input_tensor_dtype.value() != valueDType) return castOf(child, valueDType);
+        return child;
+    }
+
+    uint32_t translate(uint32_t srcIndex) {
+        auto it = remap.find(srcIndex);
+        if (it != remap.end()) return it->second;
+        ExprNode node = src.nodes.at(srcIndex);
+        if (node.lhs != UINT32_MAX) node.lhs = translate(node.lhs);
+        if (node.rhs != UINT32_MAX) node.rhs = translate(node.rhs);
+        if (node.aux != UINT32_MAX) node.aux = translate(node.aux);
+        if (isReductionOp(node.op)) {
+            node.lhs = asTensorOperand(node.lhs, true);
+        } else if (isShapeOnly(node.op)) {
+            double folded;
+            if (!tryFoldConstant(out, node.lhs, folded)) node.lhs = asTensorOperand(node.lhs, false);
+        }
+        const uint32_t idx = add(std::move(node));
+        remap.emplace(srcIndex, idx);
+        return idx;
+    }
+
+    const PhysicalExpression& src;
+    PhysicalExpression out;
+    std::unordered_map<std::string, uint32_t> byKey;
+    std::unordered_map<uint32_t, uint32_t> remap;
+};
+
+bool isTensorRole(Role r) { return r != Role::Inline; }
+
+// Tensor sources (inputs, materialised values, views) that the value of `root` is computed from without crossing
+// another materialised value.
+void collectSources(const PlannedGraph& g, uint32_t root, std::vector<uint32_t>& sources, std::vector<uint32_t>& scalarSlots) {
+    std::vector<char> seen(g.expr.nodes.size(), 0);
+    std::vector<uint32_t> stack;
+    const ExprNode& r = g.expr.nodes[root];
+    for (uint32_t c : {r.lhs, r.rhs, r.aux})
+        if (c != UINT32_MAX) stack.push_back(c);
+    if (r.op == ExprOp::RUNTIME_SCALAR) scalarSlots.push_back(r.input_slot);
+    while (!stack.empty()) {
+        const uint32_t n = stack.back();
+        stack.pop_back();
+        if (seen[n]) continue;
+        seen[n] = 1;
+        if (isTensorRole(g.role[n])) {
+            sources.push_back(n);
+            continue;
+        }
+        const ExprNode& node = g.expr.nodes[n];
+        if (node.op == ExprOp::RUNTIME_SCALAR) scalarSlots.push_back(node.input_slot);
+        for (uint32_t c : {node.lhs, node.rhs, node.aux})
+            if (c != UINT32_MAX) stack.push_back(c);
+    }
+    std::sort(sources.begin(), sources.end());
+    sources.erase(std::unique(sources.begin(), sources.end()), sources.end());
+    std::sort(scalarSlots.begin(), scalarSlots.end());
+    scalarSlots.erase(std::unique(scalarSlots.begin(), scalarSlots.end()), scalarSlots.end());
+}
+
+uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
+    while (g.role[node] == Role::View) node = g.expr.nodes[node].lhs;
+    return node;
+}
+
+std::vector<uint64_t> broadcastDims(const std::vector<uint64_t>& a, const std::vector<uint64_t>& b) {
+    const size_t rank = std::max(a.size(), b.size());
+    std::vector<uint64_t> out(rank, 1);
+    for (size_t i = 0; i < rank; ++i) {
+        const uint64_t da = i < rank - a.size() ? 1 : a[i - (rank - a.size())];
+        const uint64_t db = i < rank - b.size() ? 1 : b[i - (rank - b.size())];
+        if (da != db && da != 1 && db != 1) {
+            throw std::runtime_error("Expression operands are not broadcast-compatible.");
+        }
+        out[i] = std::max(da, db);
+    }
+    return out;
+}
+
+std::vector<uint64_t> reshapeDims(const std::vector<uint64_t>& in, const std::vector<uint64_t>& requested) {
+    uint64_t total = 1, known = 1;
+    for (uint64_t d : in) total *= d;
+    std::vector<uint64_t> out = requested;
+    int infer = -1;
+    for (size_t i = 0; i < out.size(); ++i) {
+        if (out[i] == std::numeric_limits<uint64_t>::max()) {
+            infer = static_cast<int>(i);
+        } else {
+            known *= out[i];
+        }
+    }
+    if (infer >= 0) {
+        if (known == 0 || total % known != 0) throw std::runtime_error("Expression::reshape cannot infer the marked dimension.");
+        out[infer] = total / known;
+        known *= out[infer];
+    }
+    if (known != total) throw std::runtime_error("Expression::reshape changes the number of elements.");
+    return out;
+}
+
+std::vector<uint64_t> sortedAxesOrAll(const std::vector<uint64_t>& axes, size_t rank) {
+    std::vector<uint64_t> out = axes;
+    if (out.empty()) {
+        out.resize(rank);
+        std::iota(out.begin(), out.end(), 0);
+    } else {
+        std::sort(out.begin(), out.end());
+        out.erase(std::unique(out.begin(), out.end()), out.end());
+    }
+    for (uint64_t a : out)
+        if (a >= rank) throw std::runtime_error("Reduction axis out of range.");
+    return out;
+}
+
+std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std::vector<Tensor>& boundInputs) {
+    std::vector<std::vector<uint64_t>> dims(g.expr.nodes.size());
+    for (uint32_t i = 0; i < g.expr.nodes.size(); ++i) {
+        const ExprNode& n = g.expr.nodes[i];
+        switch (n.op) {
+            case ExprOp::INPUT:
+                dims[i] = boundInputs.at(n.input_slot).getDimensions();
+                break;
+            case ExprOp::RUNTIME_SCALAR:
+            case ExprOp::SCALAR_FP:
+                dims[i] = {};
+                break;
+            case ExprOp::FILL:
+                dims[i] = n.fill_dims;
+                break;
+            case ExprOp::RESHAPE:
+                dims[i] = reshapeDims(dims[n.lhs], n.reshape_dims);
+                break;
+            case ExprOp::UNSQUEEZE: {
+                const size_t rank = dims[n.lhs].size() + n.unsqueeze_axes.size();
+                std::vector<uint64_t> out;
+                size_t src = 0;
+                for (size_t a = 0; a < rank; ++a) {
+                    if (std::binary_search(n.unsqueeze_axes.begin(), n.unsqueeze_axes.end(), a)) {
+                        out.push_back(1);
+                    } else {
+                        if (src >= dims[n.lhs].size()) throw std::runtime_error("unsqueeze axes are invalid for the input rank.");
+                        out.push_back(dims[n.lhs][src++]);
+                    }
+                }
+                for (uint64_t a : n.unsqueeze_axes)
+                    if (a >= rank) throw std::runtime_error("unsqueeze axes are invalid for the input rank.");
+                dims[i] = out;
+                break;
+            }
+            case ExprOp::SQUEEZE:
+                dims[i] = StampedEquation::computeReductionOutputDims(dims[n.lhs], {}, n.squeeze_axes.empty() ? std::vector<uint64_t>{UINT64_MAX} : n.squeeze_axes);
+                break;
+            default:
+                if (isReductionOp(n.op)) {
+                    const std::vector<uint64_t> axes = sortedAxesOrAll(n.reduction_axes, dims[n.lhs].size());
+                    dims[i] = StampedEquation::computeReductionOutputDims(dims[n.lhs], axes, n.squeeze_axes);
+                } else if (n.op == ExprOp::WHERE) {
+                    dims[i] = broadcastDims(broadcastDims(dims[n.lhs], dims[n.rhs]), dims[n.aux]);
+                } else if (Expression::isBinaryOp(n.op)) {
+                    dims[i] = broadcastDims(dims[n.lhs], dims[n.rhs]);
+                } else {
+                    dims[i] = dims[n.lhs];
+                }
+        }
+    }
+    return dims;
+}
+
+std::vector<uint64_t> orScalarShape(const std::vector<uint64_t>& dims) { return dims.empty() ? std::vector<uint64_t>{1} : dims; }
+
+CubReductionOp valueReductionOp(ExprOp op) {
+    switch (op) {
+        case ExprOp::REDUCE_SUM: return CubReductionOp::Sum;
+        case ExprOp::REDUCE_PROD: return CubReductionOp::Product;
+        case ExprOp::REDUCE_MIN: return CubReductionOp::Min;
+        case ExprOp::REDUCE_MAX: return CubReductionOp::Max;
+        case ExprOp::REDUCE_AVG: return CubReductionOp::Mean;
+        case ExprOp::REDUCE_NORM1: return CubReductionOp::L1Norm;
+        case ExprOp::REDUCE_NORM2: return CubReductionOp::L2Norm;
+        default: break;
+    }
+    throw std::runtime_error("Not a value reduction op.");
+}
+
+bool rowFusionEnabled() {
+    const char* env = std::getenv("THOR_DISABLE_ROW_FUSION");
+    return !(env && env[0] == '1');
+}
+
+}  // namespace
+
+// ---- FusedEquation --------------------------------------------------------------------------------------------------------------
+FusedEquation::FusedEquation(PhysicalOutputs outputs, int device_num)
+    : outputs_template(std::move(outputs)),
+      root_inputs(outputs_template.expr ? outputs_template.expr->inputs : std::vector<NamedInput>{}),
+      device_num(device_num),
+      planned_graph_cache(std::make_shared<LruCacheThreadSafe<std::string, std::shared_ptr<PlannedGraph>>>(128)) {}
+
+FusedEquation FusedEquation::compile(const PhysicalExpression& expr, int device_num) {
+    if (expr.output_node >= expr.nodes.size()) throw std::runtime_error("FusedEquation::compile requires a valid output node.");
+    PhysicalOutputs outputs;
+    outputs.expr = std::make_shared<PhysicalExpression>(expr);
+    outputs.outputs.push_back(NamedOutput{"output", expr.output_node});
+    return compile(outputs, device_num);
+}
+
+FusedEquation FusedEquation::compile(const PhysicalOutputs& outputs, int device_num) {
+    if (!outputs.expr) throw std::runtime_error("FusedEquation::compile requires a non-null expression graph.");
+    if (outputs.outputs.empty()) throw std::runtime_error("FusedEquation::compile requires at least one output.");
+    for (const NamedOutput& o : outputs.outputs) {
+        if (o.node_idx >= outputs.expr->nodes.size()) throw std::runtime_error("FusedEquation::compile output node index is out of range.");
+    }
+    int count = 0;
+    THOR_HIP_CHECK(thorhip_device_count(&count));
+    if (device_num < 0 || (count > 0 && device_num >= count)) {
+        throw std::runtime_error("FusedEquation::compile: no such GPU: " + std::to_string(device_num));
+    }
+    // private copy: later edits of the caller's graph must not reach the compiled equation
+    PhysicalOutputs copy;
+    copy.expr = std::make_shared<PhysicalExpression>(*outputs.expr);
+    copy.outputs = outputs.outputs;
+    return FusedEquation(std::move(copy), device_num);
+}
+
+std::vector<std::string> FusedEquation::getOutputNames() const {
+    std::vector<std::string> names;
+    for (const NamedOutput& o : outputs_template.outputs) names.push_back(o.name);
+    return names;
+}
+
+std::vector<DataType> FusedEquation::rootDTypes(const std::unordered_map<std::string, Tensor>& inputs) const {
+    std::vector<DataType> dtypes(root_inputs.size(), DataType::FP32);
+    for (const NamedInput& in : root_inputs) {
+        if (in.kind == NamedInput::Kind::RuntimeScalarFp32) continue;
+        auto it = inputs.find(in.name);
+        if (it == inputs.end()) throw std::runtime_error("Missing required input tensor: " + in.name);
+        if (!it->second.isInitialized()) throw std::runtime_error("Input tensor is not initialized: " + in.name);
+        dtypes[in.slot] = it->second.getDataType();
+    }
+    for (const auto& [name, tensor] : inputs) {
+        (void)tensor;
+        bool known = false;
+        for (const NamedInput& in : root_inputs) known = known || in.name == name;
+        if (!known) throw std::runtime_error("Unexpected input tensor for this equation: " + name);
+    }
+    return dtypes;
+}
+
+std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<DataType>& root_dtypes) const {
+    std::string key;
+    for (DataType d : root_dtypes) key += std::to_string(static_cast<int>(d)) + ",";
+    return planned_graph_cache->getOrCreate(key, [&] {
+        PhysicalOutputs resolved;
+        resolved.expr = std::make_shared<PhysicalExpression>(*outputs_template.expr);
+        resolved.outputs = outputs_template.outputs;
+        resolveOutputsDTypesInPlace(resolved, root_dtypes);
+
+        auto graph = std::make_shared<PlannedGraph>();
+        GraphBuilder builder(*resolved.expr);
+        for (const NamedOutput& o : resolved.outputs) {
+            uint32_t idx = builder.translate(o.node_idx);
+            // a named output that is only an input in another dtype becomes an explicit cast
+            idx = builder.asTensorOperand(idx, false);
+            graph->outputs.push_back(NamedOutput{o.name, idx});
+        }
+        graph->expr = std::move(builder.out);
+        graph->expr.output_node = graph->outputs.back().node_idx;
+
+        const size_t count = graph->expr.nodes.size();
+        graph->role.assign(count, Role::Inline);
+        graph->level.assign(count, 0);
+        auto ensureTensor = [&](uint32_t n) {
+            if (graph->role[n] == Role::Inline) graph->role[n] = Role::Materialized;
+        };
+        for (uint32_t i = 0; i < count; ++i) {
+            const ExprNode& n = graph->expr.nodes[i];
+            if (n.op == ExprOp::INPUT) {
+                graph->role[i] = Role::InputSource;
+            } else if (isReductionOp(n.op)) {
+                graph->role[i] = Role::Materialized;
+                ensureTensor(n.lhs);
+            } else if (isShapeOnly(n.op)) {
+                double folded;
+                if (!tryFoldConstant(graph->expr, i, folded)) {
+                    ensureTensor(n.lhs);
+                    graph->role[i] = Role::View;
+                }
+            }
+        }
+        for (const NamedOutput& o : graph->outputs) ensureTensor(o.node_idx);
+
+        // dependency levels: a materialised value runs after every materialised value it reads
+        for (uint32_t i = 0; i < count; ++i) {
+            if (graph->role[i] != Role::Materialized) continue;
+            std::vector<uint32_t> sources, scalars;
+            if (isReductionOp(graph->expr.nodes[i].op)) {
+                sources.push_back(graph->expr.nodes[i].lhs);
+            } else {
+                collectSources(*graph, i, sources, scalars);
+            }
+            uint32_t level = 0;
+            for (uint32_t s : sources) {
+                const uint32_t base = baseOfView(*graph, s);
+                if (graph->role[base] == Role::Materialized) level = std::max(level, graph->level[base] + 1);
+            }
+            graph->level[i] = level;
+        }
+        return graph;
+    });
+}
+
+bool FusedEquation::resolveLayout(std::vector<Tensor>& inputs, std::vector<uint64_t>& outputDimensions) {
+    if (inputs.empty()) throw std::runtime_error("resolveLayout requires at least one input tensor.");
+    std::vector<uint64_t> dims;
+    for (const Tensor& t : inputs) dims = broadcastDims(dims, t.getDimensions());
+    outputDimensions = dims;
+    bool broadcast = false;
+    for (const Tensor& t : inputs) broadcast = broadcast || t.getDimensions() != dims;
+    return broadcast;
+}
+
+StampedExecutionPlan FusedEquation::stamp(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                          const std::unordered_map<std::string, Tensor>& preallocated_outputs) const {
+    return stampImpl(inputs, stream, preallocated_outputs, false);
+}
+
+StampedExecutionPlan FusedEquation::stampSingleOutput(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                                      const std::optional<Tensor>& preallocated_output) const {
+    if (outputs_template.outputs.size() != 1) throw std::runtime_error("stampSingleOutput requires an equation with exactly one output.");
+    std::unordered_map<std::string, Tensor> pre;
+    if (preallocated_output.has_value()) pre.emplace(outputs_template.outputs[0].name, preallocated_output.value());
+    return stampImpl(inputs, stream, pre, false);
+}
+
+StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                              const std::unordered_map<std::string, Tensor>& preallocated, bool fusedKernelsOnly) const {
+    if (!stream.isInitialized()) throw std::runtime_error("FusedEquation::stamp requires an initialized stream.");
+    if (stream.getGpuNum() != device_num) throw std::runtime_error("FusedEquation::stamp: the stream belongs to another GPU than the equation.");
+    const std::vector<DataType> dtypes = rootDTypes(inputs);
+    const std::shared_ptr<PlannedGraph> graph = plannedGraphFor(dtypes);
+    const PhysicalExpression& expr = graph->expr;
+    const TensorPlacement gpuPlacement(TensorPlacement::MemDevices::GPU, device_num);
+
+    std::vector<Tensor> bound(root_inputs.size());
+    for (const NamedInput& in : root_inputs) {
+        if (in.kind == NamedInput::Kind::RuntimeScalarFp32) continue;
+        const Tensor& t = inputs.at(in.name);
+        if (t.getPlacement() != gpuPlacement) throw std::runtime_error("Input tensor '" + in.name + "' does not live on the equation's GPU.");
+        bound[in.slot] = t;
+    }
+    for (const auto& [name, tensor] : preallocated) {
+        bool known = false;
+        for (const NamedOutput& o : graph->outputs) known = known || o.name == name;
+        if (!known) throw std::runtime_error("Preallocated output '" + name + "' is not an output of this equation.");
+        if (!tensor.isInitialized() || tensor.getPlacement() != gpuPlacement) {
+            throw std::runtime_error("Preallocated output '" + name + "' must be an initialized tensor on the equation's GPU.");
+        }
+    }
+
+    const std::vector<std::vector<uint64_t>> dims = inferShapes(*graph, bound);
+    ScopedGpu scoped(device_num);
+
+    // ---- tensors of every tensor-role node --------------------------------------------------------------------------
+    std::vector<Tensor> tensorOf(expr.nodes.size());
+    std::unordered_map<uint32_t, std::string> outputNameOfNode;
+    for (const NamedOutput& o : graph->outputs) outputNameOfNode.emplace(o.node_idx, o.name);  // first name wins for allocation
+
+    auto allocateFor = [&](uint32_t node) {
+        const DataType dtype = expr.nodes[node].output_dtype.value();
+        const std::vector<uint64_t> shape = orScalarShape(dims[node]);
+        auto named = outputNameOfNode.find(node);
+        if (named != outputNameOfNode.end()) {
+            auto pre = preallocated.find(named->second);
+            if (pre != preallocated.end()) {
+                const Tensor& t = pre->second;
+                if (t.getDataType() != dtype) {
+                    throw std::runtime_error("Preallocated output '" + named->second + "' has dtype " + dataTypeName(t.getDataType()) +
+                                             " but the expression produces " + dataTypeName(dtype) + ".");
+                }
+                if (t.getDimensions() != shape) {
+                    throw std::runtime_error("Preallocated output '" + named->second + "' has shape " + t.dimensionsToString() +
+                                             " but the expression produces " + TensorDescriptor(dtype, shape).toString() + ".");
+                }
+                if (!t.isDenseContiguous()) throw std::runtime_error("Preallocated output '" + named->second + "' must be dense.");
+                return t;
+            }
+        }
+        return Tensor(gpuPlacement, TensorDescriptor(dtype, shape));
+    };
+
+    auto viewOf = [&](uint32_t node) {
+        const Tensor& base = tensorOf[expr.nodes[node].lhs];
+        if (!base.isDenseContiguous()) throw std::runtime_error("Shape operations on a non-dense tensor view are not supported.");
+        Tensor view = base;
+        view.reshape(orScalarShape(dims[node]));
+        return view;
+    };
+
+    // ---- stages in level order -----------------------------------------------------------------------------------------
+    uint32_t maxLevel = 0;
+    for (uint32_t i = 0; i < expr.nodes.size(); ++i)
+        if (graph->role[i] == Role::Materialized) maxLevel = std::max(maxLevel, graph->level[i]);
+
+    for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
+        if (graph->role[i] == Role::InputSource) tensorOf[i] = bound[expr.nodes[i].input_slot];
+    }
+    // views of inputs can be resolved right away; views of materialised values are resolved after their stage
+    auto resolveViewsUpTo = [&]() {
+        for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
+            if (graph->role[i] == Role::View && !tensorOf[i].isInitialized() && tensorOf[expr.nodes[i].lhs].isInitialized()) tensorOf[i] = viewOf(i);
+        }
+    };
+    resolveViewsUpTo();
+
+    std::vector<StampedExecutionStage> stages;
+    std::vector<int> stageOfNode(expr.nodes.size(), -1);
+    auto dependenciesOf = [&](const std::vector<uint32_t>& sources) {
+        std::vector<uint32_t> deps;
+        for (uint32_t s : sources) {
+            const int st = stageOfNode[baseOfView(*graph, s)];
+            if (st >= 0) deps.push_back(static_cast<uint32_t>(st));
+        }
+        std::sort(deps.begin(), deps.end());
+        deps.erase(std::unique(deps.begin(), deps.end()), deps.end());
+        return deps;
+    };
+
+    std::vector<char> done(expr.nodes.size(), 0);
+    if (rowFusionEnabled() && !fusedKernelsOnly) {
+        // Recognise chains of last-axis reductions and row-wise elementwise work over one [rows, R] input and emit them
+        // as one kernel that keeps each row in registers.
+        std::vector<uint8_t> roles(graph->role.size());
+        for (size_t i = 0; i < roles.size(); ++i) roles[i] = static_cast<uint8_t>(graph->role[i]);
+        RowFusionContext context{expr, graph->outputs, root_inputs, roles, dims, tensorOf, done, stages, stageOfNode, allocateFor, device_num};
+        tryRowFusion(context);
+        resolveViewsUpTo();
+    }
+
+    for (uint32_t level = 0; level <= maxLevel; ++level) {
+        // fused values of this level, grouped by output shape so that one kernel shares the loads
+        std::map<std::vector<uint64_t>, std::vector<uint32_t>> fusedGroups;
+        for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
+            if (graph->role[i] != Role::Materialized || graph->level[i] != level || done[i]) continue;
+            const ExprNode& n = expr.nodes[i];
+            if (!isReductionOp(n.op)) {
+                fusedGroups[orScalarShape(dims[i])].push_back(i);
+                continue;
+            }
+            if (fusedKernelsOnly) {
+                throw std::runtime_error(
+                    "FusedEquation::run() only supports expressions that lower to fused kernels; this expression has a reduction stage. "
+                    "Use stamp() and run the returned plan.");
+            }
+            const Tensor& input = tensorOf[n.lhs];
+            std::vector<uint32_t> axes;
+            for (uint64_t a : sortedAxesOrAll(n.reduction_axes, dims[n.lhs].size())) axes.push_back(static_cast<uint32_t>(a));
+            Tensor output = allocateFor(i);
+            StampedExecutionStage stage;
+            stage.gpu_num = device_num;
+            stage.dependency_stage_indices = dependenciesOf({n.lhs});
+            if (isArgReductionOp(n.op)) {
+                CubArgReductionOutputOptions options;
+                options.produce_value = false;
+                options.produce_index = true;
+                options.index_output_dtype = n.output_dtype.value();
+                const CubArgReduction reduction(n.op == ExprOp::REDUCE_ARGMAX ? CubArgReductionOp::ArgMax : CubArgReductionOp::ArgMin, axes, options);
+                stage.kind = StampedExecutionStage::Kind::ArgMinMax;
+                stage.arg_minmax = std::make_shared<StampedArgMinMax>(reduction.stamp(input, std::nullopt, output, stream));
+            } else {
+                const CubReduction reduction(valueReductionOp(n.op), axes, n.output_dtype.value());
+                stage.kind = StampedExecutionStage::Kind::Reduction;
+                stage.reduction = std::make_shared<StampedReduction>(reduction.stamp(input, output, stream));
+            }
+            tensorOf[i] = output;
+            stageOfNode[i] = static_cast<int>(stages.size());
+            stages.push_back(std::move(stage));
+            done[i] = 1;
+        }
+
+        for (auto& [shape, nodes] : fusedGroups) {
+            FusedKernelRequest request;
+            request.expr = &expr;
+            request.outputDims = shape;
+            std::vector<uint32_t> sources, scalarSlots;
+            for (uint32_t node : nodes) {
+                std::vector<uint32_t> s, sc;
+                if (isTensorRole(graph->role[node]) && expr.nodes[node].op == ExprOp::INPUT) {
+                    s.push_back(node);
+                } else {
+                    collectSources(*graph, node, s, sc);
+                }
+                sources.insert(sources.end(), s.begin(), s.end());
+                scalarSlots.insert(scalarSlots.end(), sc.begin(), sc.end());
+            }
+            std::sort(sources.begin(), sources.end());
+            sources.erase(std::unique(sources.begin(), sources.end()), sources.end());
+            std::sort(scalarSlots.begin(), scalarSlots.end());
+            scalarSlots.erase(std::unique(scalarSlots.begin(), scalarSlots.end()), scalarSlots.end());
+
+            std::vector<Tensor> inputTensors;
+            for (uint32_t s : sources) {
+                const Tensor& t = tensorOf[s];
+                if (!t.isInitialized()) throw std::logic_error("Fused stage reads a value that has not been produced yet.");
+                KernelOperand operand;
+                operand.node = s;
+                operand.storageDType = t.getDataType();
+                operand.dims = orScalarShape(dims[s]);
+                operand.strides = t.getStridesElements();
+                if (operand.strides.size() != operand.dims.size()) throw std::logic_error("Operand rank does not match its tensor.");
+                operand.alignmentBytes = pointerAlignment(t.getMemPtr());
+                request.operands.push_back(operand);
+                inputTensors.push_back(t);
+            }
+            request.scalarSlots = scalarSlots;
+            std::vector<Tensor> outputTensors;
+            for (uint32_t node : nodes) {
+                Tensor out = allocateFor(node);
+                KernelOutput ko;
+                ko.node = node;
+                ko.storageDType = out.getDataType();
+                ko.alignmentBytes = pointerAlignment(out.getMemPtr());
+                request.outputs.push_back(ko);
+                outputTensors.push_back(out);
+                tensorOf[node] = out;
+            }
+            const EmittedKernel emitted = emitFusedKernel(request);
+            std::shared_ptr<CompiledKernel> kernel = compileKernel(emitted.source, emitted.kernelName, device_num, emitted.fastContract);
+
+            std::vector<size_t> inputArgIndex(inputTensors.size()), outputArgIndex(outputTensors.size());
+            std::iota(inputArgIndex.begin(), inputArgIndex.end(), 0);
+            std::vector<StampedEquation::ScalarArgument> scalarArgs;
+            size_t next = inputTensors.size();
+            for (uint32_t slot : scalarSlots) scalarArgs.push_back({root_inputs.at(slot).name, next++});
+            for (size_t o = 0; o < outputTensors.size(); ++o) outputArgIndex[o] = next++;
+
+            StampedExecutionStage stage;
+            stage.kind = StampedExecutionStage::Kind::FusedKernel;
+            stage.gpu_num = device_num;
+            stage.dependency_stage_indices = dependenciesOf(sources);
+            stage.kernel = std::make_shared<StampedEquation>(kernel, inputTensors, outputTensors, scalarArgs, inputArgIndex, outputArgIndex, next,
+                                                             emitted.passNumel, emitted.numel, emitted.numelIs64, emitted.gridX, emitted.threads,
+                                                             emitted.flopsPerElement * emitted.numel, emitted.description);
+            for (uint32_t node : nodes) {
+                stageOfNode[node] = static_cast<int>(stages.size());
+                done[node] = 1;
+            }
+            stages.push_back(std::move(stage));
+        }
+        resolveViewsUpTo();
+    }
+
+    // ---- final outputs ---------------------------------------------------------------------------------------------------
+    std::unordered_map<std::string, Tensor> finalOutputs;
+    for (const NamedOutput& o : graph->outputs) {
+        Tensor produced = tensorOf[o.node_idx];
+        if (!produced.isInitialized()) throw std::logic_error("Output '" + o.name + "' was not produced by any stage.");
+        auto pre = preallocated.find(o.name);
+        if (pre != preallocated.end() && pre->second != produced && pre->second.getMemPtr() != produced.getMemPtr()) {
+            // the value lives elsewhere (an input, a view, or another name's tensor): copy it into the caller's tensor
+            if (pre->second.getTotalNumElements() != produced.getTotalNumElements() || pre->second.getDataType() != produced.getDataType()) {
+                throw std::runtime_error("Preallocated output '" + o.name + "' does not match the shape or dtype the expression produces.");
+            }
+            StampedExecutionStage copy;
+            copy.kind = StampedExecutionStage::Kind::Copy;
+            copy.gpu_num = device_num;
+            copy.copySource = produced;
+            copy.copyDestination = pre->second;
+            const int st = stageOfNode[baseOfView(*graph, o.node_idx)];
+            if (st >= 0) copy.dependency_stage_indices.push_back(static_cast<uint32_t>(st));
+            stages.push_back(std::move(copy));
+            produced = pre->second;
+        }
+        finalOutputs.emplace(o.name, produced);
+    }
+    return StampedExecutionPlan(std::move(stages), std::move(finalOutputs), stream);
+}
+
+// ---- convenience run ---------------------------------------------------------------------------------------------------------------
+void FusedEquation::run(const Tensor& input, Tensor& output, Stream& stream) const {
+    if (root_inputs.size() != 1) throw std::runtime_error("run(input, output) requires an equation with exactly one input.");
+    run(std::unordered_map<std::string, Tensor>{{root_inputs[0].name, input}}, output, stream);
+}
+
+void FusedEquation::run(const std::unordered_map<std::string, Tensor>& inputs, Tensor& output, Stream& stream) const {
+    run(inputs, std::unordered_map<std::string, float>{}, output, stream);
+}
+
+void FusedEquation::run(const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, float>& scalar_inputs,
+                        Tensor& output, Stream& stream) const {
+    if (outputs_template.outputs.size() != 1) throw std::runtime_error("run(..., output) requires an equation with exactly one output.");
+    std::unordered_map<std::string, Tensor> outputs{{outputs_template.outputs[0].name, output}};
+    run(inputs, scalar_inputs, outputs, stream);
+}
+
+void FusedEquation::run(const Tensor& input, std::unordered_map<std::string, Tensor>& outputs, Stream& stream) const {
+    if (root_inputs.size() != 1) throw std::runtime_error("run(input, outputs) requires an equation with exactly one input.");
+    run(std::unordered_map<std::string, Tensor>{{root_inputs[0].name, input}}, outputs, stream);
+}
+
+void FusedEquation::run(const std::unordered_map<std::string, Tensor>& inputs, std::unordered_map<std::string, Tensor>& outputs, Stream& stream) const {
+    run(inputs, std::unordered_map<std::string, float>{}, outputs, stream);
+}
+
+void FusedEquation::run(const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, float>& scalar_inputs,
+                        std::unordered_map<std::string, Tensor>& outputs, Stream& stream) const {
+    for (const NamedOutput& o : outputs_template.outputs) {
+        if (!outputs.count(o.name)) throw std::runtime_error("Missing output tensor: " + o.name);
+    }
+    const StampedExecutionPlan plan = stampImpl(inputs, stream, outputs, true);
+    for (const std::string& name : plan.runtimeScalarNames()) {
+        if (!scalar_inputs.count(name)) throw std::runtime_error("Missing runtime scalar input: " + name);
+    }
+    plan.runOn(stream, scalar_inputs);
+}
+
+// ---- shape / dtype queries -----------------------------------------------------------------------------------------------------------
+std::unordered_map<std::string, std::vector<uint64_t>> FusedEquation::getOutputShapes(const std::unordered_map<std::string, Tensor>& inputs) const {
+    const std::shared_ptr<PlannedGraph> graph = plannedGraphFor(rootDTypes(inputs));
+    std::vector<Tensor> bound(root_inputs.size());
+    for (const NamedInput& in : root_inputs)
+        if (in.kind != NamedInput::Kind::RuntimeScalarFp32) bound[in.slot] = inputs.at(in.name);
+    const std::vector<std::vector<uint64_t>> dims = inferShapes(*graph, bound);
+    std::unordered_map<std::string, std::vector<uint64_t>> out;
+    for (const NamedOutput& o : graph->outputs) out.emplace(o.name, orScalarShape(dims[o.node_idx]));
+    return out;
+}
+
+std::unordered_map<std::string, std::vector<uint64_t>> FusedEquation::getOutputShapes(const Tensor& input) const {
+    if (root_inputs.size() != 1) throw std::runtime_error("getOutputShapes(input) requires an equation with exactly one input.");
+    return getOutputShapes(std::unordered_map<std::string, Tensor>{{root_inputs[0].name, input}});
+}
+
+std::vector<uint64_t> FusedEquation::getOutputShape(const std::unordered_map<std::string, Tensor>& inputs) const {
+    if (outputs_template.outputs.size() != 1) throw std::runtime_error("getOutputShape requires an equation with exactly one output.");
+    return getOutputShapes(inputs).begin()->second;
+}
+
+std::vector<uint64_t> FusedEquation::getOutputShape(const Tensor& input) const {
+    if (outputs_template.outputs.size() != 1) throw std::runtime_error("getOutputShape requires an equation with exactly one output.");
+    return getOutputShapes(input).begin()->second;
+}
+
+std::unordered_map<std::string, DataType> FusedEquation::getOutputDataTypes(const std::unordered_map<std::string, Tensor>& inputs) const {
+    const std::shared_ptr<PlannedGraph> graph = plannedGraphFor(rootDTypes(inputs));
+    std::unordered_map<std::string, DataType> out;
+    for (const NamedOutput& o : graph->outputs) out.emplace(o.name, graph->expr.nodes[o.node_idx].output_dtype.value());
+    return out;
+}
+
+}  // namespace ThorImplementation

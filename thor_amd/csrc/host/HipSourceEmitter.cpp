@@ -1,0 +1,654 @@
+#include "HipSourceEmitter.h"
+
+#include "ReductionPlanner.h"  // deviceTypeName
+#include "thorhip_numeric_embed.h"
+
+#include <algorithm>
+#include <iomanip>
+#include <limits>
+#include <optional>
+#include <sstream>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+namespace {
+
+bool isFloatHeld(DataType d) {  // dtypes whose in-kernel value lives in a `float`
+    return d == DataType::FP32 || d == DataType::BF16 || d == DataType::FP8_E4M3 || d == DataType::FP8_E5M2;
+}
+bool isIntegral(DataType d) {
+    switch (d) {
+        case DataType::INT8:
+        case DataType::INT16:
+        case DataType::INT32:
+        case DataType::INT64:
+        case DataType::UINT8:
+        case DataType::UINT16:
+        case DataType::UINT32:
+        case DataType::UINT64:
+            return true;
+        default:
+            return false;
+    }
+}
+
+const char* unaryFunction(ExprOp op) {
+    switch (op) {
+        case ExprOp::ABS: return "fabsf";
+        case ExprOp::CEIL: return "ceilf";
+        case ExprOp::FLOOR: return "floorf";
+        case ExprOp::ROUND: return "roundf";
+        case ExprOp::TRUNC: return "truncf";
+        case ExprOp::SIN: return "sinf";
+        case ExprOp::COS: return "cosf";
+        case ExprOp::TAN: return "tanf";
+        case ExprOp::ASIN: return "asinf";
+        case ExprOp::ACOS: return "acosf";
+        case ExprOp::ATAN: return "atanf";
+        case ExprOp::SINH: return "sinhf";
+        case ExprOp::COSH: return "coshf";
+        case ExprOp::ASINH: return "asinhf";
+        case ExprOp::ACOSH: return "acoshf";
+        case ExprOp::ATANH: return "atanhf";
+        case ExprOp::ERF: return "erff";
+        case ExprOp::ERFC: return "erfcf";
+        case ExprOp::ERFCX: return "erfcxf";
+        case ExprOp::ERFINV: return "erfinvf";
+        case ExprOp::ERFCINV: return "erfcinvf";
+        case ExprOp::TGAMMA: return "tgammaf";
+        case ExprOp::LGAMMA: return "lgammaf";
+        case ExprOp::DIGAMMA: return "thor::digammaf";
+        case ExprOp::EXP: return "expf";
+        case ExprOp::EXPM1: return "expm1f";
+        case ExprOp::EXP2: return "exp2f";
+        case ExprOp::EXP10: return "exp10f";
+        case ExprOp::LN: return "logf";
+        case ExprOp::LOG1P: return "log1pf";
+        case ExprOp::LOG2: return "log2f";
+        case ExprOp::LOG10: return "log10f";
+        case ExprOp::SQRT: return "sqrtf";
+        case ExprOp::TANH: return "tanhf";
+        case ExprOp::NORMCDF: return "normcdff";
+        default: return nullptr;
+    }
+}
+
+uint64_t opFlops(ExprOp op) {
+    switch (op) {
+        case ExprOp::ADD:
+        case ExprOp::SUB:
+        case ExprOp::MUL:
+        case ExprOp::NEG:
+        case ExprOp::ABS:
+        case ExprOp::MIN:
+        case ExprOp::MAX:
+            return 1;
+        case ExprOp::DIV:
+        case ExprOp::SQRT:
+            return 4;
+        case ExprOp::CAST:
+        case ExprOp::RESHAPE:
+        case ExprOp::SQUEEZE:
+        case ExprOp::UNSQUEEZE:
+            return 0;
+        default:
+            return unaryFunction(op) ? 8 : 1;
+    }
+}
+
+bool isConstZero(const PhysicalExpression& e, uint32_t n) {
+    double v;
+    return tryFoldConstant(e, n, v) && v == 0.0;
+}
+bool isConstOne(const PhysicalExpression& e, uint32_t n) {
+    double v;
+    return tryFoldConstant(e, n, v) && v == 1.0;
+}
+
+// x + 0, 0 + x, x - 0, x * 1, 1 * x, x / 1 and pure shape ops evaluate to their operand
+bool aliasSource(const PhysicalExpression& e, uint32_t nodeIndex, uint32_t& source) {
+    const ExprNode& n = e.nodes[nodeIndex];
+    switch (n.op) {
+        case ExprOp::RESHAPE:
+        case ExprOp::UNSQUEEZE:
+        case ExprOp::SQUEEZE:
+            source = n.lhs;
+            return true;
+        case ExprOp::ADD:
+            if (isConstZero(e, n.lhs)) return source = n.rhs, true;
+            if (isConstZero(e, n.rhs)) return source = n.lhs, true;
+            return false;
+        case ExprOp::SUB:
+            if (isConstZero(e, n.rhs)) return source = n.lhs, true;
+            return false;
+        case ExprOp::MUL:
+            if (isConstOne(e, n.lhs)) return source = n.rhs, true;
+            if (isConstOne(e, n.rhs)) return source = n.lhs, true;
+            return false;
+        case ExprOp::DIV:
+            if (isConstOne(e, n.rhs)) return source = n.lhs, true;
+            return false;
+        default:
+            return false;
+    }
+}
+
+}  // namespace
+
+const char* valueCType(DataType dtype) {
+    switch (dtype) {
+        case DataType::FP32:
+        case DataType::BF16:
+        case DataType::FP8_E4M3:
+        case DataType::FP8_E5M2:
+            return "float";
+        case DataType::FP16: return "_Float16";
+        case DataType::FP64: return "double";
+        case DataType::BOOLEAN: return "bool";
+        case DataType::INT8: return "thor::i8";
+        case DataType::INT16: return "thor::i16";
+        case DataType::INT32: return "thor::i32";
+        case DataType::INT64: return "thor::i64";
+        case DataType::UINT8: return "thor::u8";
+        case DataType::UINT16: return "thor::u16";
+        case DataType::UINT32: return "thor::u32";
+        case DataType::UINT64: return "thor::u64";
+        default: break;
+    }
+    throw std::runtime_error(std::string("No in-kernel value type for dtype ") + dataTypeName(dtype));
+}
+
+std::string floatLiteral(double value) {
+    // nine significant digits and an `f` suffix: the literal text the reference prints for the same constant
+    if (value != value) return "__builtin_nanf(\"\")";
+    if (value == std::numeric_limits<double>::infinity()) return "__builtin_inff()";
+    if (value == -std::numeric_limits<double>::infinity()) return "(-__builtin_inff())";
+    std::ostringstream oss;
+    oss << std::setprecision(9) << std::defaultfloat << value;
+    std::string s = oss.str();
+    if (s.find('.') == std::string::npos && s.find('e') == std::string::npos && s.find('E') == std::string::npos) s += ".0";
+    return s + "f";
+}
+
+std::string castValueExpr(const std::string& x, DataType from, DataType to) {
+    if (from == to) return x;
+    // every conversion goes through the fp32 image of the source value, as `static_cast` chains do in the reference
+    std::string asFloat;
+    if (isFloatHeld(from)) {
+        asFloat = x;
+    } else if (from == DataType::FP16 || isIntegral(from) || from == DataType::FP64) {
+        asFloat = "(float)(" + x + ")";
+    } else if (from == DataType::BOOLEAN) {
+        asFloat = "((" + x + ") ? 1.0f : 0.0f)";
+    } else {
+        throw std::runtime_error(std::string("Unsupported cast source dtype in fused stage emitter: ") + dataTypeName(from));
+    }
+    switch (to) {
+        case DataType::FP32: return asFloat;
+        case DataType::FP16: return "(_Float16)(" + asFloat + ")";
+        case DataType::BF16: return "thor::roundBf16(" + asFloat + ")";
+        case DataType::FP8_E4M3: return "thor::roundE4m3(" + asFloat + ")";
+        case DataType::FP8_E5M2: return "thor::roundE5m2(" + asFloat + ")";
+        case DataType::BOOLEAN: return "((" + asFloat + ") != 0.0f)";
+        case DataType::FP64: return "(double)(" + asFloat + ")";
+        default:
+            if (isIntegral(to)) {
+                if (isIntegral(from)) return std::string("(") + valueCType(to) + ")(" + x + ")";
+                return std::string("(") + valueCType(to) + ")(" + asFloat + ")";
+            }
+    }
+    throw std::runtime_error(std::string("Unsupported cast destination dtype in fused stage emitter: ") + dataTypeName(to));
+}
+
+std::string storageToValueExpr(const std::string& x, DataType dtype) {
+    switch (dtype) {
+        case DataType::FP16: return "thor::asHalf(" + x + ")";
+        case DataType::BF16:
+        case DataType::FP8_E4M3:
+        case DataType::FP8_E5M2:
+            return "thor::toFloat(" + x + ")";
+        case DataType::BOOLEAN: return "((" + x + ").bits != 0)";
+        default: return x;
+    }
+}
+
+std::string valueToStorageExpr(const std::string& x, DataType dtype) {
+    switch (dtype) {
+        case DataType::FP16: return "thor::fromHalf(" + x + ")";
+        case DataType::BF16: return "thor::toBf16(" + x + ")";
+        case DataType::FP8_E4M3: return "thor::toE4m3(" + x + ")";
+        case DataType::FP8_E5M2: return "thor::toE5m2(" + x + ")";
+        case DataType::BOOLEAN: return "thor::makeBoolean(" + x + ")";
+        default: return x;
+    }
+}
+
+DataType emittedValueDType(const ExprNode& node) {
+    if (Expression::isLeafOp(node.op)) {
+        if (!node.output_dtype) throw std::runtime_error("Leaf node without a resolved output dtype.");
+        return *node.output_dtype;
+    }
+    if (!node.compute_dtype) throw std::runtime_error("Node without a resolved compute dtype.");
+    return *node.compute_dtype;
+}
+
+bool tryFoldConstant(const PhysicalExpression& expr, uint32_t nodeIndex, double& value) {
+    const ExprNode& n = expr.nodes.at(nodeIndex);
+    switch (n.op) {
+        case ExprOp::SCALAR_FP:
+        case ExprOp::FILL:
+            value = n.scalar_fp;
+            return true;
+        case ExprOp::RESHAPE:
+        case ExprOp::UNSQUEEZE:
+        case ExprOp::SQUEEZE:
+            return tryFoldConstant(expr, n.lhs, value);
+        case ExprOp::NEG:
+            if (!tryFoldConstant(expr, n.lhs, value)) return false;
+            value = -value;
+            return true;
+        case ExprOp::ADD:
+        case ExprOp::SUB:
+        case ExprOp::MUL:
+        case ExprOp::DIV: {
+            double a, b;
+            if (!tryFoldConstant(expr, n.lhs, a) || !tryFoldConstant(expr, n.rhs, b)) return false;
+            value = n.op == ExprOp::ADD ? a + b : n.op == ExprOp::SUB ? a - b : n.op == ExprOp::MUL ? a * b : a / b;
+            return true;
+        }
+        default:
+            return false;
+    }
+}
+
+namespace {
+
+// Emits `const T tN = ...;` statements for a set of nodes.  Values of tensor sources (t<node> for operand nodes) are
+// defined by the caller; valueDType[] records the dtype every defined value has.
+class BodyEmitter {
+   public:
+    BodyEmitter(const PhysicalExpression& expr) : expr(expr), valueDType(expr.nodes.size()) {}
+
+    void defineSource(uint32_t node, DataType dtype) { valueDType[node] = dtype; }
+    bool defined(uint32_t node) const { return valueDType[node].has_value(); }
+    DataType dtypeOf(uint32_t node) const { return valueDType[node].value(); }
+
+    std::string ref(uint32_t child, DataType target) const {
+        double folded;
+        if (!valueDType[child].has_value() && tryFoldConstant(expr, child, folded)) {
+            return castValueExpr(floatLiteral(folded), DataType::FP32, target);
+        }
+        return castValueExpr("t" + std::to_string(child), valueDType[child].value(), target);
+    }
+
+    // nodes (ascending) needed to evaluate `roots`, stopping at already defined values and at constants
+    std::vector<uint32_t> collect(const std::vector<uint32_t>& roots) const {
+        std::vector<char> need(expr.nodes.size(), 0);
+        std::vector<uint32_t> stack(roots.begin(), roots.end());
+        while (!stack.empty()) {
+            const uint32_t n = stack.back();
+            stack.pop_back();
+            if (need[n] || valueDType[n].has_value()) continue;
+            double folded;
+            if (tryFoldConstant(expr, n, folded)) continue;
+            need[n] = 1;
+            const ExprNode& node = expr.nodes[n];
+            for (uint32_t c : {node.lhs, node.rhs, node.aux})
+                if (c != UINT32_MAX) stack.push_back(c);
+        }
+        std::vector<uint32_t> order;
+        for (uint32_t i = 0; i < need.size(); ++i)
+            if (need[i]) order.push_back(i);
+        return order;
+    }
+
+    uint64_t emit(std::string& out, uint32_t nodeIndex, const std::string& indent, const std::vector<uint32_t>& scalarSlots) {
+        const ExprNode& n = expr.nodes[nodeIndex];
+        const DataType dtype = emittedValueDType(n);
+        const std::string decl = indent + "const " + valueCType(dtype) + " t" + std::to_string(nodeIndex) + " = ";
+        valueDType[nodeIndex] = dtype;
+        if (n.op == ExprOp::RUNTIME_SCALAR) {
+            (void)scalarSlots;
+            out += decl + castValueExpr("s" + std::to_string(n.input_slot), DataType::FP32, dtype) + ";\n";
+            return 0;
+        }
+        if (n.op == ExprOp::INPUT) throw std::runtime_error("Fused stage reads an input that was not bound as a kernel operand.");
+        uint32_t source;
+        if (aliasSource(expr, nodeIndex, source)) {
+            out += decl + ref(source, dtype) + ";\n";
+            return 0;
+        }
+        const uint64_t flops = opFlops(n.op);
+        if (n.op == ExprOp::CAST) {
+            out += decl + ref(n.lhs, dtype) + ";\n";
+            return flops;
+        }
+        if (n.op == ExprOp::WHERE) {
+            out += decl + "(" + ref(n.lhs, DataType::BOOLEAN) + " ? " + ref(n.rhs, dtype) + " : " + ref(n.aux, dtype) + ");\n";
+            return flops;
+        }
+        if (Expression::isBinaryOp(n.op)) {
+            out += decl + binary(n, dtype) + ";\n";
+            return flops;
+        }
+        out += decl + unary(n, dtype) + ";\n";
+        return flops;
+    }
+
+   private:
+    std::string unary(const ExprNode& n, DataType c) const {
+        if (n.op == ExprOp::NEG) {
+            if (c == DataType::FP32 || c == DataType::FP16 || c == DataType::BF16) return "(-" + ref(n.lhs, c) + ")";
+            return castValueExpr("(-" + ref(n.lhs, DataType::FP32) + ")", DataType::FP32, c);
+        }
+        if (n.op == ExprOp::LOGICAL_NOT) {
+            if (c == DataType::BOOLEAN) return "(!" + ref(n.lhs, DataType::BOOLEAN) + ")";
+            return "(!(" + ref(n.lhs, DataType::FP32) + " != 0.0f))";
+        }
+        if (const char* fn = unaryFunction(n.op)) {
+            // evaluated on an fp32 copy of the operand and converted back to the compute dtype
+            return castValueExpr(std::string(fn) + "(" + ref(n.lhs, DataType::FP32) + ")", DataType::FP32, c);
+        }
+        throw std::runtime_error("Unsupported unary op in fused stage emitter: " + opName(n.op));
+    }
+
+    std::string binary(const ExprNode& n, DataType c) const {
+        const bool native = c == DataType::FP32 || c == DataType::FP16 || c == DataType::BF16;
+        auto arithmetic = [&](const char* op) {
+            if (native || (n.op == ExprOp::SUB && (c == DataType::UINT32 || c == DataType::UINT64))) {
+                const std::string text = "(" + ref(n.lhs, c) + " " + op + " " + ref(n.rhs, c) + ")";
+                // bf16 arithmetic: exact fp32 operation on bf16 operands, then one rounding to bf16
+                return c == DataType::BF16 ? "thor::roundBf16" + text : text;
+            }
+            return castValueExpr("(" + ref(n.lhs, DataType::FP32) + " " + op + " " + ref(n.rhs, DataType::FP32) + ")", DataType::FP32, c);
+        };
+        const std::string a = ref(n.lhs, DataType::FP32), b = ref(n.rhs, DataType::FP32);
+        switch (n.op) {
+            case ExprOp::ADD: return arithmetic("+");
+            case ExprOp::SUB: return arithmetic("-");
+            case ExprOp::MUL: return arithmetic("*");
+            case ExprOp::DIV: return arithmetic("/");
+            case ExprOp::POW: return castValueExpr("powf(" + a + ", " + b + ")", DataType::FP32, c);
+            case ExprOp::MIN: return castValueExpr("fminf(" + a + ", " + b + ")", DataType::FP32, c);
+            case ExprOp::MAX: return castValueExpr("fmaxf(" + a + ", " + b + ")", DataType::FP32, c);
+            case ExprOp::EQUAL: return "(" + a + " == " + b + ")";
+            case ExprOp::NOT_EQUAL: return "(" + a + " != " + b + ")";
+            case ExprOp::LESS: return "(" + a + " < " + b + ")";
+            case ExprOp::LESS_EQUAL: return "(" + a + " <= " + b + ")";
+            case ExprOp::GREATER: return "(" + a + " > " + b + ")";
+            case ExprOp::GREATER_EQUAL: return "(" + a + " >= " + b + ")";
+            case ExprOp::LOGICAL_AND:
+                if (c == DataType::BOOLEAN) return "(" + ref(n.lhs, c) + " && " + ref(n.rhs, c) + ")";
+                return "((" + a + " != 0.0f) && (" + b + " != 0.0f))";
+            case ExprOp::LOGICAL_OR:
+                if (c == DataType::BOOLEAN) return "(" + ref(n.lhs, c) + " || " + ref(n.rhs, c) + ")";
+                return "((" + a + " != 0.0f) || (" + b + " != 0.0f))";
+            case ExprOp::MIN_GRAD_LEFT:
+            case ExprOp::MAX_GRAD_RIGHT:
+                return castValueExpr("((" + a + " < " + b + ") ? 1.0f : ((" + a + " > " + b + ") ? 0.0f : 0.5f))", DataType::FP32, c);
+            case ExprOp::MIN_GRAD_RIGHT:
+            case ExprOp::MAX_GRAD_LEFT:
+                return castValueExpr("((" + a + " > " + b + ") ? 1.0f : ((" + a + " < " + b + ") ? 0.0f : 0.5f))", DataType::FP32, c);
+            default: break;
+        }
+        throw std::runtime_error("Unsupported binary op in fused stage emitter: " + opName(n.op));
+    }
+
+    const PhysicalExpression& expr;
+    std::vector<std::optional<DataType>> valueDType;
+};
+
+struct CollapsedLayout {
+    std::vector<uint64_t> dims;                       // collapsed output dims
+    std::vector<std::vector<uint64_t>> operandStride;  // [operand][axis]
+};
+
+// Right-aligns every operand against the output shape (stride 0 on broadcast axes), then merges neighbouring axes that
+// every operand and the dense output address as one longer axis.
+CollapsedLayout collapseForBroadcast(const FusedKernelRequest& r) {
+    const size_t rank = r.outputDims.size();
+    std::vector<std::vector<uint64_t>> strides(r.operands.size(), std::vector<uint64_t>(rank, 0));
+    for (size_t o = 0; o < r.operands.size(); ++o) {
+        const KernelOperand& op = r.operands[o];
+        if (op.dims.size() > rank) throw std::runtime_error("Fused stage operand has a higher rank than the stage output.");
+        const size_t shift = rank - op.dims.size();
+        for (size_t a = 0; a < op.dims.size(); ++a) {
+            const uint64_t d = op.dims[a], outDim = r.outputDims[a + shift];
+            if (d == outDim) {
+                strides[o][a + shift] = d == 1 ? 0 : op.strides[a];
+            } else if (d == 1) {
+                strides[o][a + shift] = 0;
+            } else {
+                throw std::runtime_error("Fused stage operand shape does not broadcast to the stage output shape.");
+            }
+        }
+    }
+    std::vector<uint64_t> outStride(rank, 1);
+    for (size_t a = rank; a-- > 1;) outStride[a - 1] = outStride[a] * r.outputDims[a];
+
+    CollapsedLayout c;
+    c.operandStride.assign(r.operands.size(), {});
+    std::vector<uint64_t> outC;
+    for (size_t a = 0; a < rank; ++a) {
+        const uint64_t d = r.outputDims[a];
+        if (d == 1) continue;
+        bool merge = !c.dims.empty();
+        if (merge) {
+            for (size_t o = 0; o < r.operands.size() && merge; ++o) merge = c.operandStride[o].back() == d * strides[o][a];
+            merge = merge && outC.back() == d * outStride[a];
+        }
+        if (merge) {
+            c.dims.back() *= d;
+            for (size_t o = 0; o < r.operands.size(); ++o) c.operandStride[o].back() = strides[o][a];
+            outC.back() = outStride[a];
+        } else {
+            c.dims.push_back(d);
+            for (size_t o = 0; o < r.operands.size(); ++o) c.operandStride[o].push_back(strides[o][a]);
+            outC.push_back(outStride[a]);
+        }
+    }
+    if (c.dims.empty()) {
+        c.dims.push_back(1);
+        for (auto& s : c.operandStride) s.push_back(0);
+    }
+    return c;
+}
+
+}  // namespace
+
+EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
+    if (!r.expr || r.outputs.empty()) throw std::runtime_error("Fused stage needs an expression and at least one output.");
+    const PhysicalExpression& expr = *r.expr;
+    EmittedKernel k;
+    k.numel = 1;
+    for (uint64_t d : r.outputDims) k.numel *= d;
+    k.numelIs64 = k.numel >= (1ull << 31);
+    const char* indexType = k.numelIs64 ? "unsigned long long" : "unsigned int";
+
+    // flat when every operand has the output's element count, is dense, and agrees on the non-singleton dims
+    auto stripOnes = [](const std::vector<uint64_t>& d) {
+        std::vector<uint64_t> out;
+        for (uint64_t v : d)
+            if (v != 1) out.push_back(v);
+        return out;
+    };
+    const std::vector<uint64_t> outCore = stripOnes(r.outputDims);
+    k.flat = true;
+    for (const KernelOperand& op : r.operands) {
+        uint64_t expected = 1;
+        bool dense = true;
+        for (size_t a = op.dims.size(); a-- > 0;) {
+            if (op.dims[a] != 1 && op.strides[a] != expected) dense = false;
+            expected *= op.dims[a];
+        }
+        if (!dense || stripOnes(op.dims) != outCore) k.flat = false;
+    }
+
+    // widest element decides the vector length: one 16-byte access for it, narrower operands move fewer bytes
+    uint32_t widest = 1;
+    for (const KernelOperand& op : r.operands) widest = std::max(widest, dataTypeSizeInBytes(op.storageDType));
+    for (const KernelOutput& out : r.outputs) widest = std::max(widest, dataTypeSizeInBytes(out.storageDType));
+    int vec = static_cast<int>(16 / widest);
+
+    CollapsedLayout layout;
+    if (!k.flat) layout = collapseForBroadcast(r);
+    auto fits = [&](int v) {
+        for (const KernelOutput& out : r.outputs)
+            if (out.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(out.storageDType)) != 0) return false;
+        if (k.flat) {
+            for (const KernelOperand& op : r.operands)
+                if (op.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(op.storageDType)) != 0) return false;
+            return true;
+        }
+        if (layout.dims.back() % v != 0) return false;
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            const std::vector<uint64_t>& s = layout.operandStride[o];
+            if (s.back() > 1) return false;  // neither contiguous nor broadcast along the innermost axis
+            if (s.back() == 1) {
+                if (r.operands[o].alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(r.operands[o].storageDType)) != 0) return false;
+                for (size_t a = 0; a + 1 < s.size(); ++a)
+                    if (s[a] % v != 0) return false;
+            }
+        }
+        return true;
+    };
+    while (vec > 1 && !fits(vec)) vec /= 2;
+    k.vec = vec;
+    k.passNumel = k.flat;
+
+    // 16-bit float arithmetic must round after every operation, so mul+add fusion is only allowed in all-fp32 kernels
+    k.fastContract = true;
+    BodyEmitter probe(expr);
+    for (const KernelOperand& op : r.operands) probe.defineSource(op.node, DataType::FP32);
+    std::vector<uint32_t> roots;
+    for (const KernelOutput& out : r.outputs) roots.push_back(out.node);
+    for (uint32_t n : probe.collect(roots)) {
+        const DataType c = emittedValueDType(expr.nodes[n]);
+        if (c == DataType::FP16 || c == DataType::BF16) k.fastContract = false;
+    }
+
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude;
+    s << "extern \"C\" __global__ __launch_bounds__(256) void fused_kernel(";
+    for (size_t o = 0; o < r.operands.size(); ++o) s << "const " << deviceTypeName(r.operands[o].storageDType) << "* in" << o << ", ";
+    for (uint32_t slot : r.scalarSlots) s << "float s" << slot << ", ";
+    for (size_t o = 0; o < r.outputs.size(); ++o) {
+        s << deviceTypeName(r.outputs[o].storageDType) << "* out" << o;
+        if (o + 1 < r.outputs.size() || k.passNumel) s << ", ";
+    }
+    if (k.passNumel) s << indexType << " numel";
+    s << ") {\n";
+    s << "    typedef " << indexType << " index_t;\n";
+    s << "    constexpr int V = " << vec << ";\n";
+
+    // body text for one element; `load(o)` and `store(o, value)` differ between the vector and the scalar form
+    uint64_t flops = 0;
+    auto emitBody = [&](const std::string& indent, auto loadExpr, auto storeStmt) {
+        std::string body;
+        BodyEmitter emitter(expr);
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            const KernelOperand& op = r.operands[o];
+            const ExprNode& node = expr.nodes[op.node];
+            const DataType valueDType = node.output_dtype.value();
+            std::string value = storageToValueExpr(loadExpr(o), op.storageDType);
+            value = castValueExpr(value, op.storageDType, valueDType);
+            body += indent + "const " + valueCType(valueDType) + " t" + std::to_string(op.node) + " = " + value + ";\n";
+            emitter.defineSource(op.node, valueDType);
+        }
+        uint64_t bodyFlops = 0;
+        for (uint32_t n : emitter.collect(roots)) bodyFlops += emitter.emit(body, n, indent, r.scalarSlots);
+        for (size_t o = 0; o < r.outputs.size(); ++o) {
+            const ExprNode& node = expr.nodes[r.outputs[o].node];
+            const DataType outDType = node.output_dtype.value();
+            if (outDType != r.outputs[o].storageDType) throw std::runtime_error("Fused stage output tensor dtype differs from the node's output dtype.");
+            const std::string value = emitter.ref(r.outputs[o].node, outDType);
+            body += indent + storeStmt(o, valueToStorageExpr(value, outDType)) + "\n";
+        }
+        flops = bodyFlops;
+        return body;
+    };
+
+    if (k.flat) {
+        s << "    const index_t base = ((index_t)blockIdx.x * 256u + threadIdx.x) * V;\n";
+        s << "    if (base >= numel) return;\n";
+        if (vec > 1) {
+            s << "    if (base + V <= numel) {\n";
+            for (size_t o = 0; o < r.operands.size(); ++o) {
+                s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n";
+                s << "        p" << o << ".loadStream(in" << o << " + base);\n";
+            }
+            for (size_t o = 0; o < r.outputs.size(); ++o) s << "        thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", V> q" << o << ";\n";
+            s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
+            s << emitBody(
+                "            ", [](size_t o) { return "p" + std::to_string(o) + ".v[k]"; },
+                [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; });
+            s << "        }\n";
+            for (size_t o = 0; o < r.outputs.size(); ++o) s << "        q" << o << ".storeStream(out" << o << " + base);\n";
+            s << "        return;\n    }\n";
+        }
+        s << "    const index_t end = (base + V < numel) ? base + V : numel;\n";
+        s << "    for (index_t e = base; e < end; ++e) {\n";
+        s << emitBody(
+            "        ", [](size_t o) { return "in" + std::to_string(o) + "[e]"; },
+            [](size_t o, const std::string& v) { return "out" + std::to_string(o) + "[e] = " + v + ";"; });
+        s << "    }\n";
+        const uint64_t lanes = (k.numel + vec - 1) / vec;
+        k.gridX = static_cast<uint32_t>(std::max<uint64_t>((lanes + 255) / 256, 1));
+        k.description = "flat(vec=" + std::to_string(vec) + ")";
+    } else {
+        std::vector<uint64_t> dims = layout.dims;
+        dims.back() /= vec;  // the innermost axis is walked in vectors
+        uint64_t lanes = 1;
+        for (uint64_t d : dims) lanes *= d;
+        s << "    const index_t lane = (index_t)blockIdx.x * 256u + threadIdx.x;\n";
+        s << "    if (lane >= " << lanes << "ull) return;\n";
+        s << "    index_t rest = lane;\n";
+        for (size_t a = dims.size(); a-- > 0;) {
+            if (a == 0) {
+                s << "    const index_t c0 = rest;\n";
+            } else {
+                s << "    const index_t c" << a << " = rest % " << dims[a] << "u;\n    rest /= " << dims[a] << "u;\n";
+            }
+        }
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            const std::vector<uint64_t>& st = layout.operandStride[o];
+            s << "    const unsigned long long off" << o << " = 0ull";
+            for (size_t a = 0; a < st.size(); ++a) {
+                if (st[a] == 0) continue;
+                const uint64_t step = (a + 1 == st.size()) ? st[a] * vec : st[a];
+                s << " + (unsigned long long)c" << a << " * " << step << "ull";
+            }
+            s << ";\n";
+        }
+        s << "    const unsigned long long outOff = (unsigned long long)lane * V;\n";
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            const bool contiguous = layout.operandStride[o].back() == 1;
+            const char* type = deviceTypeName(r.operands[o].storageDType);
+            if (contiguous && vec > 1) {
+                s << "    thor::Pack<" << type << ", V> p" << o << ";\n    p" << o << ".loadStream(in" << o << " + off" << o << ");\n";
+            } else {
+                s << "    const " << type << " b" << o << " = in" << o << "[off" << o << "];\n";
+            }
+        }
+        for (size_t o = 0; o < r.outputs.size(); ++o) s << "    thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", V> q" << o << ";\n";
+        s << "#pragma unroll\n    for (int k = 0; k < V; ++k) {\n";
+        s << emitBody(
+            "        ",
+            [&](size_t o) {
+                const bool contiguous = layout.operandStride[o].back() == 1;
+                return (contiguous && vec > 1) ? "p" + std::to_string(o) + ".v[k]" : "b" + std::to_string(o);
+            },
+            [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; });
+        s << "    }\n";
+        for (size_t o = 0; o < r.outputs.size(); ++o) s << "    q" << o << ".storeStream(out" << o << " + outOff);\n";
+        k.gridX = static_cast<uint32_t>(std::max<uint64_t>((lanes + 255) / 256, 1));
+        k.description = "broadcast(axes=" + std::to_string(dims.size()) + ",vec=" + std::to_string(vec) + ")";
+    }
+    s << "}\n";
+    k.source = s.str();
+    k.flopsPerElement = flops;
+    return k;
+}
+
+}  // namespace ThorImplementation

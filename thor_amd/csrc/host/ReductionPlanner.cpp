@@ -1,0 +1,358 @@
+#include "ReductionPlanner.h"
+
+#include "Utilities/Expression/CompiledEquation.h"
+#include "thorhip_numeric_embed.h"
+
+#include <algorithm>
+#include <sstream>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+namespace {
+
+constexpr uint64_t kTargetThreads = 256ull * 512ull;  // threads that keep 256 CUs busy with loads in flight
+constexpr uint64_t kMaxGridY = 65535;
+
+uint64_t pow2Ceil(uint64_t v) {
+    uint64_t p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+uint64_t ceilDiv(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+
+// Largest power-of-two element count whose byte size is <= 16, divides every listed extent and fits the alignment.
+int chooseVector(uint32_t elementBytes, uint64_t alignmentBytes, std::initializer_list<uint64_t> mustDivide) {
+    int vec = static_cast<int>(16 / elementBytes);
+    while (vec > 1) {
+        bool ok = alignmentBytes % (static_cast<uint64_t>(vec) * elementBytes) == 0;
+        for (uint64_t extent : mustDivide) ok = ok && (extent % vec == 0);
+        if (ok) break;
+        vec /= 2;
+    }
+    return vec;
+}
+
+size_t partialBytes(uint64_t slots, bool isArg, bool indexIs64) {
+    size_t bytes = ((slots * 4 + 7) / 8) * 8;
+    if (isArg) bytes += slots * (indexIs64 ? 8 : 4);
+    return bytes;
+}
+
+// Merges adjacent axes that address memory as one longer axis (outer stride == inner dim * inner stride) and drops
+// singleton axes.  Order is preserved, so row-major positions inside the collapsed domain are unchanged.
+void collapseAxes(std::vector<uint64_t>& dims, std::vector<uint64_t>& strides) {
+    std::vector<uint64_t> d, s;
+    for (size_t i = 0; i < dims.size(); ++i) {
+        if (dims[i] == 1) continue;
+        if (!d.empty() && s.back() == dims[i] * strides[i]) {
+            d.back() *= dims[i];
+            s.back() = strides[i];
+        } else {
+            d.push_back(dims[i]);
+            s.push_back(strides[i]);
+        }
+    }
+    dims = d;
+    strides = s;
+}
+
+const char* accumulatorType(const ReductionKernelRequest& r, bool indexIs64, int& finalize) {
+    finalize = 0;
+    if (r.isArg) {
+        if (r.argOp == CubArgReductionOp::ArgMax) return indexIs64 ? "ArgAcc<true, u64>" : "ArgAcc<true, u32>";
+        return indexIs64 ? "ArgAcc<false, u64>" : "ArgAcc<false, u32>";
+    }
+    switch (r.valueOp) {
+        case CubReductionOp::Sum:
+            return "ValueAcc<SumOp>";
+        case CubReductionOp::Mean:
+            finalize = 1;
+            return "ValueAcc<SumOp>";
+        case CubReductionOp::L1Norm:
+            return "ValueAcc<AbsSumOp>";
+        case CubReductionOp::L2Norm:
+            finalize = 2;
+            return "ValueAcc<SquareSumOp>";
+        case CubReductionOp::Product:
+            return "ValueAcc<ProductOp>";
+        case CubReductionOp::Min:
+            return "ValueAcc<MinOp>";
+        case CubReductionOp::Max:
+            return "ValueAcc<MaxOp>";
+    }
+    throw std::invalid_argument("Unsupported tensor reduction operation.");
+}
+
+std::string offsetFunction(const char* name, const std::vector<uint64_t>& dims, const std::vector<uint64_t>& strides) {
+    std::ostringstream out;
+    out << "    static __device__ __forceinline__ u64 " << name << "(u64 i) {\n        u64 offset = 0;\n";
+    for (size_t a = dims.size(); a-- > 0;) {
+        if (a == 0) {
+            out << "        offset += i * " << strides[a] << "ull;\n";
+        } else {
+            out << "        offset += (i % " << dims[a] << "ull) * " << strides[a] << "ull;\n        i /= " << dims[a] << "ull;\n";
+        }
+    }
+    out << "        return offset;\n    }\n";
+    return out.str();
+}
+
+}  // namespace
+
+uint64_t pointerAlignment(const void* p) {
+    const uint64_t address = reinterpret_cast<uint64_t>(p);
+    uint64_t alignment = 256;
+    while (alignment > 1 && address % alignment != 0) alignment /= 2;
+    return alignment;
+}
+
+const char* deviceTypeName(DataType dtype) {
+    switch (dtype) {
+        case DataType::FP16: return "thor::f16";
+        case DataType::BF16: return "thor::bf16";
+        case DataType::FP8_E4M3: return "thor::e4m3";
+        case DataType::FP8_E5M2: return "thor::e5m2";
+        case DataType::FP32: return "float";
+        case DataType::FP64: return "double";
+        case DataType::INT8: return "thor::i8";
+        case DataType::INT16: return "thor::i16";
+        case DataType::INT32: return "thor::i32";
+        case DataType::INT64: return "thor::i64";
+        case DataType::UINT8: return "thor::u8";
+        case DataType::UINT16: return "thor::u16";
+        case DataType::UINT32: return "thor::u32";
+        case DataType::UINT64: return "thor::u64";
+        case DataType::BOOLEAN: return "thor::boolean";
+        default: break;
+    }
+    throw std::invalid_argument(std::string("No device type for dtype ") + dataTypeName(dtype));
+}
+
+std::string ReductionShape::describe() const {
+    std::ostringstream out;
+    switch (kernel) {
+        case Kernel::All:
+            out << "all(blocks=" << blocks << ",unroll=" << unroll;
+            break;
+        case Kernel::Rows:
+            out << "rows(lanes_per_row=" << threadsPerRow << ",split=" << split;
+            break;
+        case Kernel::Columns:
+            out << "columns(split=" << split;
+            break;
+        case Kernel::Strided:
+            out << "strided(kept_rank=" << keptDims.size() << ",reduced_rank=" << reducedDims.size() << ",split=" << split;
+            break;
+    }
+    out << ",vec=" << vec << ",threads=" << threads << ",grid=" << gridX << "x" << gridY << ")";
+    return out.str();
+}
+
+ReductionShape planReductionShape(const ReductionKernelRequest& request) {
+    const CubReductionGeometry& g = request.geometry;
+    const uint32_t elementBytes = dataTypeSizeInBytes(request.inputDType);
+    ReductionShape shape;
+    shape.indexIs64 = g.input_elements >= (1ull << 31) || g.reduction_size >= (1ull << 31);
+
+    auto finishSplit = [&](uint64_t outputs) {
+        if (shape.split > 1) shape.workspaceBytes = partialBytes(outputs * shape.split, request.isArg, shape.indexIs64);
+    };
+
+    if (g.path == CubReductionPath::DeviceTransformReduce && !g.device_transform_uses_affine_stride) {
+        shape.kernel = ReductionShape::Kernel::All;
+        shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.input_elements});
+        shape.threads = 256;
+        shape.unroll = 4;
+        const uint64_t vectors = g.input_elements / shape.vec;
+        shape.blocks = std::min<uint64_t>(std::max<uint64_t>(ceilDiv(vectors, 256ull * shape.unroll), 1), 65536);
+        shape.gridX = static_cast<uint32_t>(shape.blocks);
+        if (shape.blocks > 1) {
+            const size_t partials = partialBytes(shape.blocks, request.isArg, shape.indexIs64);
+            shape.counterOffset = ((partials + 255) / 256) * 256;
+            shape.workspaceBytes = shape.counterOffset + 256;
+            shape.usesTicketCounter = true;
+        }
+        return shape;
+    }
+
+    if (g.path == CubReductionPath::ContiguousFixedSegment) {
+        shape.kernel = ReductionShape::Kernel::Rows;
+        shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.reduction_size});
+        const uint64_t vectorsPerRow = g.reduction_size / shape.vec;
+        // aim at about 8 vector loads in flight per lane
+        const uint64_t lanes = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(ceilDiv(vectorsPerRow, 8)), 1), 1024);
+        shape.threadsPerRow = static_cast<int>(lanes);
+        shape.threads = lanes <= 64 ? 256 : static_cast<int>(lanes);
+        const uint64_t totalThreads = g.outer_size * lanes;
+        if (totalThreads < kTargetThreads && vectorsPerRow > lanes * 16) {
+            shape.split = std::min<uint64_t>({ceilDiv(kTargetThreads, totalThreads), vectorsPerRow / (lanes * 8), kMaxGridY});
+            if (shape.split < 2) shape.split = 1;
+        }
+        const uint64_t rowsPerBlock = lanes <= 64 ? 256 / lanes : 1;
+        shape.gridX = static_cast<uint32_t>(ceilDiv(g.outer_size, rowsPerBlock));
+        shape.gridY = static_cast<uint32_t>(shape.split);
+        finishSplit(g.outer_size);
+        return shape;
+    }
+
+    if (g.path == CubReductionPath::TiledFixedSegment) {
+        shape.kernel = ReductionShape::Kernel::Columns;
+        shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.inner_size});
+        shape.threads = 256;
+        const uint64_t columns = g.outer_size * (g.inner_size / shape.vec);
+        if (columns < kTargetThreads && g.reduction_size >= 64) {
+            shape.split = std::min<uint64_t>({ceilDiv(kTargetThreads, columns), g.reduction_size / 16, kMaxGridY});
+            if (shape.split < 2) shape.split = 1;
+        }
+        shape.gridX = static_cast<uint32_t>(ceilDiv(columns, 256));
+        shape.gridY = static_cast<uint32_t>(shape.split);
+        finishSplit(g.output_elements);
+        return shape;
+    }
+
+    // Strided: arbitrary kept / reduced axes, including views and the affine rank-1 whole-tensor case.
+    shape.kernel = ReductionShape::Kernel::Strided;
+    shape.threads = 256;
+    for (size_t a = 0; a < g.indexing.retained_axes.size(); ++a) {
+        shape.keptDims.push_back(g.indexing.retained_dimensions[a]);
+        shape.keptStrides.push_back(g.indexing.input_strides[g.indexing.retained_axes[a]]);
+    }
+    for (size_t a = 0; a < g.indexing.reduced_axes.size(); ++a) {
+        shape.reducedDims.push_back(g.indexing.reduced_dimensions[a]);
+        shape.reducedStrides.push_back(g.indexing.input_strides[g.indexing.reduced_axes[a]]);
+    }
+    collapseAxes(shape.keptDims, shape.keptStrides);
+    collapseAxes(shape.reducedDims, shape.reducedStrides);
+    if (shape.keptDims.empty()) {
+        shape.keptDims = {1};
+        shape.keptStrides = {0};
+    }
+    if (shape.reducedDims.empty()) {
+        shape.reducedDims = {1};
+        shape.reducedStrides = {0};
+    }
+    shape.vec = 1;
+    if (shape.reducedStrides.back() == 1) {
+        int vec = static_cast<int>(16 / elementBytes);
+        while (vec > 1) {
+            bool ok = request.inputAlignmentBytes % (static_cast<uint64_t>(vec) * elementBytes) == 0 && shape.reducedDims.back() % vec == 0;
+            for (size_t a = 0; a + 1 < shape.reducedStrides.size(); ++a) ok = ok && shape.reducedStrides[a] % vec == 0;
+            for (uint64_t s : shape.keptStrides) ok = ok && s % vec == 0;
+            if (ok) break;
+            vec /= 2;
+        }
+        shape.vec = vec;
+    }
+    const uint64_t reductionVectors = g.reduction_size / shape.vec;
+    const uint64_t outputs = g.output_elements;
+    if (outputs < 2048 && reductionVectors > 256ull * 8) {
+        shape.split = std::min<uint64_t>({ceilDiv(4096, outputs), reductionVectors / (256ull * 4), kMaxGridY});
+        if (shape.split < 2) shape.split = 1;
+    }
+    shape.gridX = static_cast<uint32_t>(outputs);
+    shape.gridY = static_cast<uint32_t>(shape.split);
+    finishSplit(outputs);
+    return shape;
+}
+
+std::string generateReductionSource(const ReductionKernelRequest& request, const ReductionShape& shape) {
+    const CubReductionGeometry& g = request.geometry;
+    int finalize = 0;
+    const char* acc = accumulatorType(request, shape.indexIs64, finalize);
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude << thor_embed::kReduceKernels;
+    s << "namespace gen {\nusing namespace thor;\nstruct Cfg {\n";
+    s << "    typedef " << deviceTypeName(request.inputDType) << " In;\n";
+    s << "    typedef " << deviceTypeName(request.valueOutputDType) << " Out;\n";
+    s << "    typedef " << (shape.indexIs64 ? "u64" : "u32") << " IndexT;\n";
+    s << "    typedef " << (request.indexOutputDType == DataType::UINT64 ? "u64" : "u32") << " OutIndex;\n";
+    s << "    typedef " << acc << " Acc;\n";
+    s << "    static constexpr bool kIsArg = " << (request.isArg ? "true" : "false") << ";\n";
+    s << "    static constexpr bool kWriteValue = " << (request.writeValue ? "true" : "false") << ";\n";
+    s << "    static constexpr bool kWriteIndex = " << (request.writeIndex ? "true" : "false") << ";\n";
+    s << "    static constexpr int kFinalize = " << finalize << ";\n";
+    s << "    static constexpr float kDivisor = (float)" << g.reduction_size << "ull;\n";
+    s << "    static constexpr int kVec = " << shape.vec << ";\n";
+    s << "    static constexpr int kThreads = " << shape.threads << ";\n";
+    s << "    static constexpr u64 kSplit = " << shape.split << "ull;\n";
+    s << "    static constexpr u64 kOutputs = " << g.output_elements << "ull;\n";
+    const char* body = "";
+    switch (shape.kernel) {
+        case ReductionShape::Kernel::All:
+            s << "    static constexpr u64 kN = " << g.input_elements << "ull;\n";
+            s << "    static constexpr int kUnroll = " << shape.unroll << ";\n";
+            s << "    static constexpr u64 kBlocks = " << shape.blocks << "ull;\n";
+            body = "thor::reduceAll<gen::Cfg>(in, valueOut, indexOut, partials, counter, scale);";
+            break;
+        case ReductionShape::Kernel::Rows:
+            s << "    static constexpr u64 kOuter = " << g.outer_size << "ull;\n";
+            s << "    static constexpr u64 kR = " << g.reduction_size << "ull;\n";
+            s << "    static constexpr int kThreadsPerRow = " << shape.threadsPerRow << ";\n";
+            body = "thor::reduceRows<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
+            break;
+        case ReductionShape::Kernel::Columns:
+            s << "    static constexpr u64 kOuter = " << g.outer_size << "ull;\n";
+            s << "    static constexpr u64 kR = " << g.reduction_size << "ull;\n";
+            s << "    static constexpr u64 kInner = " << g.inner_size << "ull;\n";
+            s << "    static constexpr u64 kOutOuterStride = " << g.tiled_output_outer_stride << "ull;\n";
+            s << "    static constexpr u64 kOutInnerStride = " << g.tiled_output_inner_stride << "ull;\n";
+            body = "thor::reduceColumns<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
+            break;
+        case ReductionShape::Kernel::Strided: {
+            std::vector<uint64_t> rd = shape.reducedDims, rs = shape.reducedStrides;
+            if (shape.vec > 1) {
+                rd.back() /= shape.vec;
+                rs.back() = shape.vec;  // one step of the innermost axis = one vector
+            }
+            s << "    static constexpr u64 kReduction = " << (g.reduction_size / shape.vec) << "ull;\n";
+            s << offsetFunction("keptOffset", shape.keptDims, shape.keptStrides);
+            s << offsetFunction("reducedOffset", rd, rs);
+            body = "thor::reduceStrided<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
+            break;
+        }
+    }
+    // layout of the final store made by the second stage of split kernels
+    if (shape.kernel == ReductionShape::Kernel::Columns) {
+        s << "    static constexpr u64 kFinishInner = " << g.inner_size << "ull;\n";
+        s << "    static constexpr u64 kFinishOuterStride = " << g.tiled_output_outer_stride << "ull;\n";
+        s << "    static constexpr u64 kFinishInnerStride = " << g.tiled_output_inner_stride << "ull;\n";
+    } else {
+        s << "    static constexpr u64 kFinishInner = 1ull;\n    static constexpr u64 kFinishOuterStride = 1ull;\n"
+             "    static constexpr u64 kFinishInnerStride = 0ull;\n";
+    }
+    s << "};\n}  // namespace gen\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads
+      << ") void thor_reduce_main(const gen::Cfg::In* in, void* valueOut, void* indexOut, void* partials, unsigned int* counter, float scale) {\n"
+         "    (void)counter;\n    (void)partials;\n    "
+      << body << "\n}\n";
+    if (shape.split > 1) {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_reduce_finish(const void* partials, void* valueOut, void* indexOut, float "
+             "scale) {\n    thor::finishPartials<gen::Cfg>(partials, valueOut, indexOut, scale);\n}\n";
+    }
+    return s.str();
+}
+
+ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request) {
+    const ReductionShape shape = planReductionShape(request);
+    const std::string source = generateReductionSource(request, shape);
+    ReductionLaunchPlan plan;
+    // fp32 accumulation order is part of the result: never let the compiler fuse or reassociate across elements
+    plan.mainKernel = compileKernel(source, "thor_reduce_main", request.deviceNum, /*fastContract=*/false);
+    if (shape.split > 1) {
+        plan.finishKernel = compileKernel(source, "thor_reduce_finish", request.deviceNum, false);
+        plan.finishThreads = 256;
+        plan.finishGridX = static_cast<uint32_t>((request.geometry.output_elements * 64 + 255) / 256);
+    }
+    plan.mainGridX = shape.gridX;
+    plan.mainGridY = shape.gridY;
+    plan.mainThreads = static_cast<uint32_t>(shape.threads);
+    plan.usesTicketCounter = shape.usesTicketCounter;
+    plan.workspaceBytes = shape.workspaceBytes;
+    plan.counterOffset = shape.counterOffset;
+    plan.variant = shape.describe();
+    return plan;
+}
+
+}  // namespace ThorImplementation

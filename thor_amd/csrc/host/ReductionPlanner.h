@@ -1,0 +1,51 @@
+// Internal: turns a reduction geometry into a kernel shape (vector width, lanes per row, split factor, grid), generates
+// the traits struct that specialises the device templates for that shape, and compiles it.
+#pragma once
+
+#include "Utilities/TensorOperations/Cub/CubReduction.h"
+
+#include <cstdint>
+#include <string>
+
+namespace ThorImplementation {
+
+struct ReductionKernelRequest {
+    bool isArg = false;
+    CubReductionOp valueOp = CubReductionOp::Sum;
+    CubArgReductionOp argOp = CubArgReductionOp::ArgMax;
+    DataType inputDType = DataType::FP32;
+    DataType valueOutputDType = DataType::FP32;
+    DataType indexOutputDType = DataType::UINT32;
+    bool writeValue = true;
+    bool writeIndex = false;
+    CubReductionGeometry geometry;
+    uint64_t inputAlignmentBytes = 256;  // largest power of two (capped at 256) dividing the input base address
+    int deviceNum = 0;
+};
+
+struct ReductionShape {
+    enum class Kernel { All, Rows, Columns, Strided } kernel = Kernel::All;
+    int vec = 1;
+    int threads = 256;
+    int threadsPerRow = 64;
+    int unroll = 4;
+    uint64_t blocks = 1;
+    uint64_t split = 1;
+    bool indexIs64 = false;
+    uint32_t gridX = 1, gridY = 1;
+    size_t workspaceBytes = 0;
+    size_t counterOffset = 0;
+    bool usesTicketCounter = false;
+    // collapsed axes of the strided kernel
+    std::vector<uint64_t> keptDims, keptStrides, reducedDims, reducedStrides;
+    std::string describe() const;
+};
+
+uint64_t pointerAlignment(const void* p);
+ReductionShape planReductionShape(const ReductionKernelRequest& request);
+std::string generateReductionSource(const ReductionKernelRequest& request, const ReductionShape& shape);
+ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request);
+
+const char* deviceTypeName(DataType dtype);  // "thor::f16", "float", ...
+
+}  // namespace ThorImplementation

@@ -1,0 +1,213 @@
+#include "Utilities/Expression/StampedEquation.h"
+
+#include "Utilities/Common/ScopedGpu.h"
+
+#include <algorithm>
+#include <limits>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+StampedEquation::StampedEquation(std::shared_ptr<CompiledKernel> kernel, std::vector<Tensor> inputs, std::vector<Tensor> outputs,
+                                 std::vector<ScalarArgument> scalars, std::vector<size_t> inputArgIndex, std::vector<size_t> outputArgIndex,
+                                 size_t numArgs, bool passNumel, uint64_t numel, bool numelIs64, uint32_t gridX, uint32_t threads,
+                                 uint64_t flops, std::string description)
+    : kernel(std::move(kernel)), inputs(std::move(inputs)), outputs(std::move(outputs)), scalars(std::move(scalars)),
+      inputArgIndex(std::move(inputArgIndex)), outputArgIndex(std::move(outputArgIndex)), numArgs(numArgs), passNumel(passNumel),
+      numel(numel), numelIs64(numelIs64), gridX(gridX), threads(threads), flops(flops), description(std::move(description)) {
+    if (!this->kernel) throw std::runtime_error("StampedEquation requires a compiled kernel.");
+    if (this->outputs.empty()) throw std::runtime_error("StampedEquation requires at least one output tensor.");
+    for (const Tensor& t : this->inputs) {
+        if (t.getPlacement().getMemDevice() != TensorPlacement::MemDevices::GPU) {
+            throw std::runtime_error("Fused equation inputs must be GPU tensors.");
+        }
+    }
+}
+
+uint32_t StampedEquation::gpuNum() const { return outputs[0].getPlacement().getDeviceNum(); }
+
+Tensor StampedEquation::getOutputTensor() const {
+    if (outputs.size() != 1) {
+        throw std::runtime_error("getOutputTensor called but there are " + std::to_string(outputs.size()) +
+                                 " outputs. This function is only valid for single output equations.");
+    }
+    return outputs[0];
+}
+
+std::unordered_set<std::string> StampedEquation::runtimeScalarNames() const {
+    std::unordered_set<std::string> names;
+    for (const ScalarArgument& s : scalars) names.insert(s.name);
+    return names;
+}
+
+void StampedEquation::runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const {
+    if (!stream.isInitialized() || stream.getGpuNum() != static_cast<int>(gpuNum())) {
+        throw std::runtime_error("Stamped equation must run on a stream of the GPU its tensors live on.");
+    }
+    // argument storage: one slot per kernel argument, each holding either a pointer or a float / index value
+    std::vector<const void*> pointerSlots(numArgs, nullptr);
+    std::vector<float> floatSlots(numArgs, 0.0f);
+    std::vector<void*> args(numArgs + (passNumel ? 1 : 0), nullptr);
+    for (size_t i = 0; i < inputs.size(); ++i) {
+        pointerSlots[inputArgIndex[i]] = inputs[i].getMemPtr();
+        args[inputArgIndex[i]] = &pointerSlots[inputArgIndex[i]];
+    }
+    for (size_t i = 0; i < outputs.size(); ++i) {
+        pointerSlots[outputArgIndex[i]] = outputs[i].getMemPtr();
+        args[outputArgIndex[i]] = &pointerSlots[outputArgIndex[i]];
+    }
+    for (const ScalarArgument& s : scalars) {
+        auto it = runtime_scalars.find(s.name);
+        if (it == runtime_scalars.end()) throw std::runtime_error("Missing runtime scalar input: " + s.name);
+        floatSlots[s.argIndex] = it->second;
+        args[s.argIndex] = &floatSlots[s.argIndex];
+    }
+    uint32_t numel32 = static_cast<uint32_t>(numel);
+    uint64_t numel64 = numel;
+    if (passNumel) args[numArgs] = numelIs64 ? static_cast<void*>(&numel64) : static_cast<void*>(&numel32);
+    ScopedGpu scoped(stream.getGpuNum());
+    kernel->launch(gridX, 1, 1, threads, stream.getStream(), args);
+}
+
+std::vector<uint64_t> StampedEquation::computeReductionOutputDims(const std::vector<uint64_t>& input_dims,
+                                                                  const std::vector<uint64_t>& reduction_axes,
+                                                                  const std::vector<uint64_t>& squeeze_axes) {
+    std::vector<uint64_t> out = input_dims;
+    for (uint64_t axis : reduction_axes) {
+        if (axis >= out.size()) throw std::runtime_error("Reduction axis out of range.");
+        out[axis] = 1;
+    }
+    if (squeeze_axes.empty()) return out;
+    std::vector<uint64_t> squeezed;
+    if (squeeze_axes.size() == 1 && squeeze_axes[0] == std::numeric_limits<uint64_t>::max()) {
+        for (uint64_t d : out)
+            if (d != 1) squeezed.push_back(d);
+    } else {
+        std::vector<uint64_t> axes = squeeze_axes;
+        std::sort(axes.begin(), axes.end());
+        axes.erase(std::unique(axes.begin(), axes.end()), axes.end());
+        for (uint64_t axis : axes) {
+            if (axis >= out.size()) throw std::runtime_error("squeeze axes are invalid for the input rank.");
+            if (out[axis] != 1) {
+                throw std::runtime_error("Trying to squeeze axis " + std::to_string(axis) + " but it has size " + std::to_string(out[axis]) +
+                                         ", can only squeeze dimensions of size 1.");
+            }
+        }
+        for (uint64_t i = 0; i < out.size(); ++i)
+            if (!std::binary_search(axes.begin(), axes.end(), i)) squeezed.push_back(out[i]);
+    }
+    if (squeezed.empty()) squeezed.push_back(1);
+    return squeezed;
+}
+
+uint64_t StampedExecutionStage::flopCount() const {
+    switch (kind) {
+        case Kind::FusedKernel:
+        case Kind::FusedRowKernel:
+            return kernel ? kernel->flopCount() : 0;
+        case Kind::Reduction:
+            return reduction ? reduction->flopCount() : 0;
+        case Kind::ArgMinMax:
+            return arg_minmax ? arg_minmax->flopCount() : 0;
+        case Kind::Copy:
+            return 0;
+    }
+    return 0;
+}
+
+void StampedExecutionStage::runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const {
+    switch (kind) {
+        case Kind::FusedKernel:
+        case Kind::FusedRowKernel:
+            if (!kernel) throw std::runtime_error("Fused execution stage is missing its stamped kernel.");
+            kernel->runOn(stream, runtime_scalars);
+            return;
+        case Kind::Reduction:
+            if (!reduction) throw std::runtime_error("Reduction execution stage is missing its stamped reduction.");
+            reduction->runOn(stream);
+            return;
+        case Kind::ArgMinMax:
+            if (!arg_minmax) throw std::runtime_error("ArgMinMax execution stage is missing its stamped reduction.");
+            arg_minmax->runOn(stream);
+            return;
+        case Kind::Copy: {
+            Tensor destination = copyDestination;
+            destination.copyFromAsync(copySource, stream);
+            return;
+        }
+    }
+}
+
+void StampedExecutionPlan::run() { runOn(stream, {}); }
+void StampedExecutionPlan::run(const std::unordered_map<std::string, float>& runtime_scalars) { runOn(stream, runtime_scalars); }
+void StampedExecutionPlan::runOn(Stream& run_stream) const { runOn(run_stream, {}); }
+
+void StampedExecutionPlan::runOn(Stream& run_stream, const std::unordered_map<std::string, float>& runtime_scalars) const {
+    // Stages are stored in dependency order and issued on one stream: stream order is the synchronisation.
+    for (const StampedExecutionStage& step : steps) step.runOn(run_stream, runtime_scalars);
+}
+
+std::unordered_set<std::string> StampedExecutionPlan::runtimeScalarNames() const {
+    std::unordered_set<std::string> names;
+    for (const StampedExecutionStage& step : steps) {
+        if (step.kernel) {
+            for (const std::string& n : step.kernel->runtimeScalarNames()) names.insert(n);
+        }
+    }
+    return names;
+}
+
+uint64_t StampedExecutionPlan::flopCount() const {
+    uint64_t total = 0;
+    for (const StampedExecutionStage& step : steps) {
+        const uint64_t f = step.flopCount();
+        if (std::numeric_limits<uint64_t>::max() - total < f) throw std::runtime_error("StampedExecutionPlan::flopCount overflow.");
+        total += f;
+    }
+    return total;
+}
+
+std::vector<uint64_t> StampedExecutionPlan::stageFlopCounts() const {
+    std::vector<uint64_t> out;
+    for (const StampedExecutionStage& step : steps) out.push_back(step.flopCount());
+    return out;
+}
+
+std::vector<std::string> StampedExecutionPlan::stageKindNames() const {
+    std::vector<std::string> out;
+    for (const StampedExecutionStage& step : steps) out.push_back(StampedExecutionStage::kindToString(step.kind));
+    return out;
+}
+
+std::vector<std::vector<uint32_t>> StampedExecutionPlan::stageDependencyIndices() const {
+    std::vector<std::vector<uint32_t>> out;
+    for (const StampedExecutionStage& step : steps) out.push_back(step.dependency_stage_indices);
+    return out;
+}
+
+std::vector<CubReductionPath> StampedExecutionPlan::reductionPaths() const {
+    std::vector<CubReductionPath> out;
+    for (const StampedExecutionStage& step : steps) {
+        if (step.kind == StampedExecutionStage::Kind::Reduction) {
+            if (!step.reduction) throw std::runtime_error("Reduction execution stage is missing its stamped reduction.");
+            out.push_back(step.reduction->getPath());
+        }
+    }
+    return out;
+}
+
+Tensor StampedExecutionPlan::output(const std::string& name) const {
+    auto it = final_outputs.find(name);
+    if (it == final_outputs.end()) throw std::runtime_error("No such output in stamped execution plan: " + name);
+    return it->second;
+}
+
+Tensor StampedExecutionPlan::output() const {
+    if (final_outputs.size() != 1) {
+        throw std::runtime_error("StampedEquation.output() called to return the single output tensor, but there are " +
+                                 std::to_string(final_outputs.size()) + " output tensors.");
+    }
+    return final_outputs.begin()->second;
+}
+
+}  // namespace ThorImplementation

@@ -1,0 +1,242 @@
+// Flat C binding, part 1: errors, Stream, Tensor, TypeConverter, CubReduction, CubArgReduction.
+#include "capi_internal.h"
+
+#include "ReductionPlanner.h"
+#include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
+
+#include <cstring>
+
+using namespace ThorImplementation;
+
+namespace thor_capi {
+std::string& lastError() {
+    static thread_local std::string slot;
+    return slot;
+}
+
+void recordCurrentException() {
+    try {
+        throw;
+    } catch (const std::invalid_argument& e) {
+        lastError() = std::string("invalid_argument: ") + e.what();
+    } catch (const std::out_of_range& e) {
+        lastError() = std::string("out_of_range: ") + e.what();
+    } catch (const std::logic_error& e) {
+        lastError() = std::string("logic_error: ") + e.what();
+    } catch (const std::runtime_error& e) {
+        lastError() = std::string("runtime_error: ") + e.what();
+    } catch (const std::exception& e) {
+        lastError() = std::string("exception: ") + e.what();
+    } catch (...) {
+        lastError() = "exception: unknown";
+    }
+}
+
+int copyOut(const std::string& text, char* buffer, size_t capacity, size_t* needed) {
+    if (needed) *needed = text.size() + 1;
+    if (buffer == nullptr || capacity == 0) return needed ? 0 : -1;
+    const size_t n = std::min(text.size(), capacity - 1);
+    std::memcpy(buffer, text.data(), n);
+    buffer[n] = '\0';
+    return text.size() + 1 <= capacity ? 0 : -2;
+}
+}  // namespace thor_capi
+
+using namespace thor_capi;
+
+namespace {
+std::vector<uint32_t> axesOf(const uint32_t* axes, int n) { return std::vector<uint32_t>(axes, axes + (n > 0 ? n : 0)); }
+std::vector<uint64_t> dimsOf(const uint64_t* dims, int n) { return std::vector<uint64_t>(dims, dims + (n > 0 ? n : 0)); }
+
+CubReductionGeometry geometryOf(const uint64_t* dims, const uint64_t* strides, int rank, const uint32_t* axes, int num_axes) {
+    if (strides == nullptr) return CubReduction::analyzeGeometry(dimsOf(dims, rank), axesOf(axes, num_axes));
+    return CubReduction::analyzeGeometry(dimsOf(dims, rank), dimsOf(strides, rank), axesOf(axes, num_axes));
+}
+}  // namespace
+
+extern "C" {
+
+const char* thor_last_error(void) { return lastError().c_str(); }
+
+// ---- Stream ---------------------------------------------------------------------------------------------------------------
+thor_stream_t thor_stream_create(int gpu_num) {
+    THOR_CAPI_TRY_PTR(return new thor_stream{Stream(gpu_num)};)
+}
+void thor_stream_destroy(thor_stream_t stream) { delete stream; }
+int thor_stream_synchronize(thor_stream_t stream) {
+    THOR_CAPI_TRY_INT(require(stream, "stream"); stream->stream.synchronize();)
+}
+void* thor_stream_raw(thor_stream_t stream) { return stream ? stream->stream.getStream() : nullptr; }
+int thor_stream_gpu_num(thor_stream_t stream) { return stream ? stream->stream.getGpuNum() : -1; }
+
+// ---- Tensor ---------------------------------------------------------------------------------------------------------------
+thor_tensor_t thor_tensor_create(int device_type, int device_num, int dtype, const uint64_t* dims, int rank) {
+    THOR_CAPI_TRY_PTR(
+        if (rank <= 0 || dims == nullptr) throw std::invalid_argument("thor_tensor_create requires at least one dimension.");
+        for (int i = 0; i < rank; ++i)
+            if (dims[i] == 0) throw std::invalid_argument("Tensor dimensions must be non-zero.");
+        const TensorPlacement placement(device_type == THOR_DEVICE_GPU ? TensorPlacement::MemDevices::GPU : TensorPlacement::MemDevices::CPU,
+                                        device_type == THOR_DEVICE_GPU ? device_num : 0);
+        (void)dataTypeSizeInBytes(static_cast<DataType>(dtype));
+        return new thor_tensor{Tensor(placement, TensorDescriptor(static_cast<DataType>(dtype), dimsOf(dims, rank)))};)
+}
+thor_tensor_t thor_tensor_clone_handle(thor_tensor_t tensor) {
+    THOR_CAPI_TRY_PTR(require(tensor, "tensor"); return new thor_tensor{tensor->tensor};)
+}
+void thor_tensor_destroy(thor_tensor_t tensor) { delete tensor; }
+void* thor_tensor_mem_ptr(thor_tensor_t tensor) { return tensor ? tensor->tensor.getMemPtr() : nullptr; }
+int thor_tensor_dtype(thor_tensor_t tensor) { return tensor ? static_cast<int>(tensor->tensor.getDataType()) : -1; }
+int thor_tensor_rank(thor_tensor_t tensor) { return tensor ? static_cast<int>(tensor->tensor.getNumDimensions()) : -1; }
+int thor_tensor_dims(thor_tensor_t tensor, uint64_t* dims_out) {
+    THOR_CAPI_TRY_INT(require(tensor, "tensor"); const auto d = tensor->tensor.getDimensions(); std::copy(d.begin(), d.end(), dims_out);)
+}
+int thor_tensor_strides(thor_tensor_t tensor, uint64_t* strides_out) {
+    THOR_CAPI_TRY_INT(require(tensor, "tensor"); const auto s = tensor->tensor.getStridesElements(); std::copy(s.begin(), s.end(), strides_out);)
+}
+uint64_t thor_tensor_num_elements(thor_tensor_t tensor) { return tensor ? tensor->tensor.getTotalNumElements() : 0; }
+int thor_tensor_device_type(thor_tensor_t tensor) {
+    if (!tensor) return -1;
+    return tensor->tensor.getPlacement().getMemDevice() == TensorPlacement::MemDevices::GPU ? THOR_DEVICE_GPU : THOR_DEVICE_CPU;
+}
+int thor_tensor_device_num(thor_tensor_t tensor) { return tensor ? tensor->tensor.getPlacement().getDeviceNum() : -1; }
+int thor_tensor_is_dense(thor_tensor_t tensor) { return tensor && tensor->tensor.isDenseContiguous() ? 1 : 0; }
+int thor_tensor_copy_from_async(thor_tensor_t dest, thor_tensor_t source, thor_stream_t stream) {
+    THOR_CAPI_TRY_INT(require(dest, "dest"); require(source, "source"); require(stream, "stream");
+                      dest->tensor.copyFromAsync(source->tensor, stream->stream);)
+}
+int thor_tensor_memset_async(thor_tensor_t tensor, int byte_value, thor_stream_t stream) {
+    THOR_CAPI_TRY_INT(require(tensor, "tensor"); require(stream, "stream");
+                      tensor->tensor.memsetAsync(stream->stream, static_cast<int8_t>(byte_value));)
+}
+int thor_tensor_reshape(thor_tensor_t tensor, const uint64_t* dims, int rank) {
+    THOR_CAPI_TRY_INT(require(tensor, "tensor"); tensor->tensor.reshape(dimsOf(dims, rank));)
+}
+thor_tensor_t thor_tensor_alias_view(thor_tensor_t tensor, const uint64_t* dims, const uint64_t* strides, int rank, uint64_t element_offset) {
+    THOR_CAPI_TRY_PTR(require(tensor, "tensor");
+                      return new thor_tensor{tensor->tensor.aliasView(dimsOf(dims, rank), dimsOf(strides, rank), element_offset)};)
+}
+
+// ---- TypeConverter ----------------------------------------------------------------------------------------------------------
+int thor_convert_type(void* source, void* dest, int source_dtype, int dest_dtype, int64_t num_elements, thor_stream_t stream, int device_num) {
+    THOR_CAPI_TRY_INT(require(stream, "stream");
+                      if (source_dtype == dest_dtype) throw std::invalid_argument("convertType requires two different dtypes.");
+                      if (num_elements < 0) throw std::invalid_argument("convertType requires a non-negative element count.");
+                      TypeConverter::convertType(source, dest, static_cast<DataType>(source_dtype), static_cast<DataType>(dest_dtype),
+                                                 static_cast<long>(num_elements), stream->stream, device_num);)
+}
+int thor_convert_type_cpu(const void* source, void* dest, int source_dtype, int dest_dtype, int64_t num_elements) {
+    THOR_CAPI_TRY_INT(if (source_dtype == dest_dtype) throw std::invalid_argument("convertType requires two different dtypes.");
+                      if (num_elements < 0) throw std::invalid_argument("convertType requires a non-negative element count.");
+                      TypeConverter::cpuConvertNow(source, dest, static_cast<DataType>(source_dtype), static_cast<DataType>(dest_dtype),
+                                                   static_cast<long>(num_elements));)
+}
+
+// ---- CubReduction -------------------------------------------------------------------------------------------------------------
+int thor_reduction_analyze_geometry(const uint64_t* dims, const uint64_t* strides, int rank, const uint32_t* axes, int num_axes,
+                                    thor_reduction_geometry* out) {
+    THOR_CAPI_TRY_INT(
+        if (out == nullptr) throw std::invalid_argument("thor_reduction_analyze_geometry: out is NULL");
+        const CubReductionGeometry g = geometryOf(dims, strides, rank, axes, num_axes);
+        if (g.rank > 16) throw std::invalid_argument("thor_reduction_analyze_geometry reports at most 16 dimensions.");
+        std::memset(out, 0, sizeof *out);
+        out->path = static_cast<int>(g.path);
+        out->reduced_axes_are_contiguous = g.reduced_axes_are_contiguous;
+        out->outer_size = g.outer_size;
+        out->reduction_size = g.reduction_size;
+        out->inner_size = g.inner_size;
+        out->input_elements = g.input_elements;
+        out->output_elements = g.output_elements;
+        out->rank = static_cast<int>(g.rank);
+        std::copy(g.output_dimensions.begin(), g.output_dimensions.end(), out->output_dimensions);
+        out->squeezed_rank = static_cast<int>(g.squeezed_output_dimensions.size());
+        std::copy(g.squeezed_output_dimensions.begin(), g.squeezed_output_dimensions.end(), out->squeezed_output_dimensions);
+        out->device_transform_uses_affine_stride = g.device_transform_uses_affine_stride;
+        out->affine_input_stride = g.affine_input_stride;)
+}
+
+int thor_reduction_map_index(const uint64_t* dims, const uint64_t* strides, int rank, const uint32_t* axes, int num_axes,
+                             uint64_t output_index, uint64_t reduction_index, uint64_t* physical_index) {
+    THOR_CAPI_TRY_INT(const CubReductionGeometry g = geometryOf(dims, strides, rank, axes, num_axes);
+                      *physical_index = CubReduction::mapLogicalReductionIndexToPhysicalIndex(g, output_index, reduction_index);)
+}
+
+thor_stamped_reduction_t thor_reduction_stamp(int op, const uint32_t* axes, int num_axes, int output_dtype, float output_scale,
+                                              thor_tensor_t input, thor_tensor_t preallocated_output, thor_stream_t stream) {
+    THOR_CAPI_TRY_PTR(
+        require(input, "input"); require(stream, "stream");
+        std::optional<DataType> out;
+        if (output_dtype >= 0) out = static_cast<DataType>(output_dtype);
+        const CubReduction reduction(static_cast<CubReductionOp>(op), axesOf(axes, num_axes), out, output_scale);
+        auto stamped = preallocated_output ? reduction.stamp(input->tensor, preallocated_output->tensor, stream->stream)
+                                           : reduction.stamp(input->tensor, stream->stream);
+        return new thor_stamped_reduction{stamped};)
+}
+void thor_stamped_reduction_destroy(thor_stamped_reduction_t r) { delete r; }
+int thor_stamped_reduction_run(thor_stamped_reduction_t r) { THOR_CAPI_TRY_INT(require(r, "reduction"); r->stamped->run();) }
+int thor_stamped_reduction_run_scaled(thor_stamped_reduction_t r, float scale) {
+    THOR_CAPI_TRY_INT(require(r, "reduction"); r->stamped->run(scale);)
+}
+int thor_stamped_reduction_run_on(thor_stamped_reduction_t r, thor_stream_t stream) {
+    THOR_CAPI_TRY_INT(require(r, "reduction"); require(stream, "stream"); r->stamped->runOn(stream->stream);)
+}
+thor_tensor_t thor_stamped_reduction_output(thor_stamped_reduction_t r) {
+    THOR_CAPI_TRY_PTR(require(r, "reduction"); return new thor_tensor{r->stamped->getOutputTensor()};)
+}
+int thor_stamped_reduction_path(thor_stamped_reduction_t r) { return r ? static_cast<int>(r->stamped->getPath()) : -1; }
+size_t thor_stamped_reduction_workspace_bytes(thor_stamped_reduction_t r) { return r ? r->stamped->getWorkspaceSizeInBytes() : 0; }
+int thor_stamped_reduction_variant(thor_stamped_reduction_t r, char* buffer, size_t capacity) {
+    THOR_CAPI_TRY_INT(require(r, "reduction"); copyOut(r->stamped->getKernelVariant(), buffer, capacity, nullptr);)
+}
+
+int thor_reduction_generate_source(int is_arg, int op, int input_dtype, int output_dtype, int index_dtype, const uint64_t* dims,
+                                   const uint64_t* strides, int rank, const uint32_t* axes, int num_axes, char* buffer, size_t capacity,
+                                   size_t* needed) {
+    THOR_CAPI_TRY_INT(
+        ReductionKernelRequest request;
+        request.isArg = is_arg != 0;
+        if (is_arg) {
+            request.argOp = static_cast<CubArgReductionOp>(op);
+            request.writeIndex = true;
+            request.writeValue = true;
+        } else {
+            request.valueOp = static_cast<CubReductionOp>(op);
+        }
+        request.inputDType = static_cast<DataType>(input_dtype);
+        request.valueOutputDType = static_cast<DataType>(output_dtype);
+        request.indexOutputDType = static_cast<DataType>(index_dtype);
+        request.geometry = geometryOf(dims, strides, rank, axes, num_axes);
+        const ReductionShape shape = planReductionShape(request);
+        copyOut(generateReductionSource(request, shape), buffer, capacity, needed);)
+}
+
+// ---- CubArgReduction --------------------------------------------------------------------------------------------------------------
+thor_stamped_arg_reduction_t thor_arg_reduction_stamp(int op, const uint32_t* axes, int num_axes, int produce_value, int produce_index,
+                                                      int value_output_dtype, int index_output_dtype, thor_tensor_t input,
+                                                      thor_tensor_t preallocated_value, thor_tensor_t preallocated_index,
+                                                      thor_stream_t stream) {
+    THOR_CAPI_TRY_PTR(
+        require(input, "input"); require(stream, "stream");
+        CubArgReductionOutputOptions options;
+        options.produce_value = produce_value != 0;
+        options.produce_index = produce_index != 0;
+        if (value_output_dtype >= 0) options.value_output_dtype = static_cast<DataType>(value_output_dtype);
+        if (index_output_dtype >= 0) options.index_output_dtype = static_cast<DataType>(index_output_dtype);
+        const CubArgReduction reduction(static_cast<CubArgReductionOp>(op), axesOf(axes, num_axes), options);
+        std::optional<Tensor> value, index;
+        if (preallocated_value) value = preallocated_value->tensor;
+        if (preallocated_index) index = preallocated_index->tensor;
+        return new thor_stamped_arg_reduction{reduction.stamp(input->tensor, value, index, stream->stream)};)
+}
+void thor_stamped_arg_reduction_destroy(thor_stamped_arg_reduction_t r) { delete r; }
+int thor_stamped_arg_reduction_run(thor_stamped_arg_reduction_t r) { THOR_CAPI_TRY_INT(require(r, "arg reduction"); r->stamped->run();) }
+thor_tensor_t thor_stamped_arg_reduction_value_output(thor_stamped_arg_reduction_t r) {
+    if (!r || !r->stamped->getValueOutputTensor().has_value()) return nullptr;
+    return new thor_tensor{r->stamped->getValueOutputTensor().value()};
+}
+thor_tensor_t thor_stamped_arg_reduction_index_output(thor_stamped_arg_reduction_t r) {
+    if (!r || !r->stamped->getIndexOutputTensor().has_value()) return nullptr;
+    return new thor_tensor{r->stamped->getIndexOutputTensor().value()};
+}
+int thor_stamped_arg_reduction_path(thor_stamped_arg_reduction_t r) { return r ? static_cast<int>(r->stamped->getPath()) : -1; }
+
+}  // extern "C"

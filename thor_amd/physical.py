@@ -1,0 +1,729 @@
+"""Python mirror of the reference's `thor.physical` surface for the hot path -- Expression, FusedEquation ("compile"),
+Equation (the stamped plan), PhysicalTensor, Stream, Placement -- bound to libthor_amd.so through include/thor_c_api.h.
+
+The shapes of the calls follow bindings/python/src/core/physical/expression.cpp:602-2866 of the reference so that its
+test helpers (`_copy_numpy_to_gpu`, `_run_expr`, `_run_staged_expr`) read the same here.  Nothing is computed in Python.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+from typing import Dict, Iterable, List, Optional, Sequence, Union
+
+import numpy as np
+
+from . import _lib
+from .dtypes import DataType, numpy_carrier
+
+_vp, _i, _u64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_size_t
+_u64p = ctypes.POINTER(ctypes.c_uint64)
+_u32p = ctypes.POINTER(ctypes.c_uint32)
+_cp = ctypes.c_char_p
+_cpp = ctypes.POINTER(ctypes.c_char_p)
+_vpp = ctypes.POINTER(ctypes.c_void_p)
+_fp = ctypes.POINTER(ctypes.c_float)
+UINT64_MAX = (1 << 64) - 1
+
+
+class ReductionGeometry(ctypes.Structure):
+    _fields_ = [
+        ("path", _i), ("reduced_axes_are_contiguous", _i),
+        ("outer_size", _u64), ("reduction_size", _u64), ("inner_size", _u64),
+        ("input_elements", _u64), ("output_elements", _u64),
+        ("rank", _i), ("output_dimensions", _u64 * 16),
+        ("squeezed_rank", _i), ("squeezed_output_dimensions", _u64 * 16),
+        ("device_transform_uses_affine_stride", _i), ("affine_input_stride", _u64),
+    ]
+
+
+PROTOTYPES = {
+    "thor_last_error": (_cp, []),
+    "thor_stream_create": (_vp, [_i]), "thor_stream_destroy": (None, [_vp]), "thor_stream_synchronize": (_i, [_vp]),
+    "thor_stream_raw": (_vp, [_vp]), "thor_stream_gpu_num": (_i, [_vp]),
+    "thor_tensor_create": (_vp, [_i, _i, _i, _u64p, _i]), "thor_tensor_clone_handle": (_vp, [_vp]), "thor_tensor_destroy": (None, [_vp]),
+    "thor_tensor_mem_ptr": (_vp, [_vp]), "thor_tensor_dtype": (_i, [_vp]), "thor_tensor_rank": (_i, [_vp]),
+    "thor_tensor_dims": (_i, [_vp, _u64p]), "thor_tensor_strides": (_i, [_vp, _u64p]), "thor_tensor_num_elements": (_u64, [_vp]),
+    "thor_tensor_device_type": (_i, [_vp]), "thor_tensor_device_num": (_i, [_vp]), "thor_tensor_is_dense": (_i, [_vp]),
+    "thor_tensor_copy_from_async": (_i, [_vp, _vp, _vp]), "thor_tensor_memset_async": (_i, [_vp, _i, _vp]),
+    "thor_tensor_reshape": (_i, [_vp, _u64p, _i]), "thor_tensor_alias_view": (_vp, [_vp, _u64p, _u64p, _i, _u64]),
+    "thor_convert_type": (_i, [_vp, _vp, _i, _i, ctypes.c_int64, _vp, _i]),
+    "thor_convert_type_cpu": (_i, [_vp, _vp, _i, _i, ctypes.c_int64]),
+    "thor_reduction_analyze_geometry": (_i, [_u64p, _u64p, _i, _u32p, _i, ctypes.POINTER(ReductionGeometry)]),
+    "thor_reduction_map_index": (_i, [_u64p, _u64p, _i, _u32p, _i, _u64, _u64, _u64p]),
+    "thor_reduction_stamp": (_vp, [_i, _u32p, _i, _i, ctypes.c_float, _vp, _vp, _vp]),
+    "thor_stamped_reduction_destroy": (None, [_vp]), "thor_stamped_reduction_run": (_i, [_vp]),
+    "thor_stamped_reduction_run_scaled": (_i, [_vp, ctypes.c_float]), "thor_stamped_reduction_run_on": (_i, [_vp, _vp]),
+    "thor_stamped_reduction_output": (_vp, [_vp]), "thor_stamped_reduction_path": (_i, [_vp]),
+    "thor_stamped_reduction_workspace_bytes": (_sz, [_vp]), "thor_stamped_reduction_variant": (_i, [_vp, _cp, _sz]),
+    "thor_reduction_generate_source": (_i, [_i, _i, _i, _i, _i, _u64p, _u64p, _i, _u32p, _i, _cp, _sz, ctypes.POINTER(_sz)]),
+    "thor_arg_reduction_stamp": (_vp, [_i, _u32p, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "thor_stamped_arg_reduction_destroy": (None, [_vp]), "thor_stamped_arg_reduction_run": (_i, [_vp]),
+    "thor_stamped_arg_reduction_value_output": (_vp, [_vp]), "thor_stamped_arg_reduction_index_output": (_vp, [_vp]),
+    "thor_stamped_arg_reduction_path": (_i, [_vp]),
+    "thor_expr_input": (_vp, [_cp, _i, _i]), "thor_expr_runtime_scalar": (_vp, [_cp, _i, _i]), "thor_expr_scalar": (_vp, [ctypes.c_double]),
+    "thor_expr_fill": (_vp, [ctypes.c_double, _u64p, _i, _i]), "thor_expr_binary": (_vp, [_cp, _vp, _vp]), "thor_expr_unary": (_vp, [_cp, _vp]),
+    "thor_expr_unary_params": (_vp, [_cp, _vp, ctypes.c_double, ctypes.c_double]), "thor_expr_where": (_vp, [_vp, _vp, _vp]),
+    "thor_expr_cast": (_vp, [_vp, _i]), "thor_expr_with_dtypes": (_vp, [_vp, _i, _i]),
+    "thor_expr_reduce": (_vp, [_cp, _vp, _u64p, _i, _u64p, _i]), "thor_expr_reshape": (_vp, [_vp, _u64p, _i]),
+    "thor_expr_unsqueeze": (_vp, [_vp, _u64p, _i]), "thor_expr_squeeze": (_vp, [_vp, _u64p, _i]), "thor_expr_destroy": (None, [_vp]),
+    "thor_expr_num_nodes": (_i, [_vp]), "thor_expr_canonical": (_i, [_vp, _cp, _sz, ctypes.POINTER(_sz)]),
+    "thor_outputs_create": (_vp, [_cpp, _vpp, _i]), "thor_outputs_destroy": (None, [_vp]),
+    "thor_fused_equation_compile": (_vp, [_vp, _i]), "thor_fused_equation_destroy": (None, [_vp]),
+    "thor_fused_equation_num_outputs": (_i, [_vp]), "thor_fused_equation_output_name": (_i, [_vp, _i, _cp, _sz]),
+    "thor_fused_equation_stamp": (_vp, [_vp, _cpp, _vpp, _i, _cpp, _vpp, _i, _vp]),
+    "thor_fused_equation_run": (_i, [_vp, _cpp, _vpp, _i, _cpp, _fp, _i, _cpp, _vpp, _i, _vp]),
+    "thor_fused_equation_output_shape": (_i, [_vp, _cpp, _vpp, _i, _cp, _u64p, ctypes.POINTER(_i), ctypes.POINTER(_i)]),
+    "thor_plan_destroy": (None, [_vp]), "thor_plan_run": (_i, [_vp]), "thor_plan_run_with_scalars": (_i, [_vp, _cpp, _fp, _i]),
+    "thor_plan_run_on": (_i, [_vp, _vp]), "thor_plan_output": (_vp, [_vp, _cp]), "thor_plan_num_stages": (_i, [_vp]),
+    "thor_plan_stage_kind": (_i, [_vp, _i, _cp, _sz]), "thor_plan_stage_source": (_i, [_vp, _i, _cp, _sz, ctypes.POINTER(_sz)]),
+    "thor_plan_stage_description": (_i, [_vp, _i, _cp, _sz]), "thor_plan_flop_count": (_u64, [_vp]),
+    "thor_compiled_kernel_count": (_u64, []),
+}
+
+_bound = None
+
+
+def lib():
+    global _bound
+    if _bound is None:
+        L = _lib.load()
+        for name, (restype, argtypes) in PROTOTYPES.items():
+            fn = getattr(L, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _bound = L
+    return _bound
+
+
+_ERROR_TYPES = {"invalid_argument": ValueError, "out_of_range": IndexError, "logic_error": AssertionError}
+
+
+def _raise_last(what: str):
+    msg = (lib().thor_last_error() or b"").decode("utf-8", "replace")
+    kind, _, text = msg.partition(": ")
+    raise _ERROR_TYPES.get(kind, RuntimeError)(f"{what}: {text or msg}")
+
+
+def _check(rc: int, what: str):
+    if rc != 0:
+        _raise_last(what)
+
+
+def _handle(ptr, what: str):
+    if not ptr:
+        _raise_last(what)
+    return ptr
+
+
+def _u64_array(values: Sequence[int]):
+    values = [int(v) for v in values]
+    return (ctypes.c_uint64 * max(1, len(values)))(*values), len(values)
+
+
+def _u32_array(values: Sequence[int]):
+    values = [int(v) for v in values]
+    return (ctypes.c_uint32 * max(1, len(values)))(*values), len(values)
+
+
+def _names(names: Sequence[str]):
+    return (ctypes.c_char_p * max(1, len(names)))(*[n.encode() for n in names])
+
+
+def _ptrs(handles: Sequence[int]):
+    return (ctypes.c_void_p * max(1, len(handles)))(*handles)
+
+
+def _dtype_code(dtype: Optional[DataType]) -> int:
+    return -1 if dtype is None else int(dtype)
+
+
+class DeviceType(enum.IntEnum):
+    cpu = 1
+    gpu = 2
+
+
+class Placement:
+    def __init__(self, device_type: DeviceType, device_num: int = 0):
+        self.device_type = DeviceType(device_type)
+        self.device_num = device_num
+
+    def __eq__(self, other):
+        return isinstance(other, Placement) and (self.device_type, self.device_num) == (other.device_type, other.device_num)
+
+    def __repr__(self):
+        return "CPU" if self.device_type == DeviceType.cpu else f"GPU:{self.device_num}"
+
+
+class Stream:
+    """Stream(gpu_num): shared handle of one HIP stream (Utilities/Common/Stream.h:35-116)."""
+
+    def __init__(self, gpu_num: int = 0):
+        self._h = _handle(lib().thor_stream_create(gpu_num), "Stream")
+        self.gpu_num = gpu_num
+
+    @property
+    def handle(self):  # raw hipStream_t, accepted by thor_amd.runtime helpers
+        return lib().thor_stream_raw(self._h)
+
+    def synchronize(self):
+        _check(lib().thor_stream_synchronize(self._h), "Stream.synchronize")
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_stream_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class PhysicalTensor:
+    class Descriptor:
+        def __init__(self, dtype: DataType, dimensions: Sequence[int]):
+            self.dtype = DataType(dtype)
+            self.dimensions = [int(d) for d in dimensions]
+
+        def get_dimensions(self) -> List[int]:
+            return list(self.dimensions)
+
+        def get_data_type(self) -> DataType:
+            return self.dtype
+
+    def __init__(self, placement: Placement, descriptor: "PhysicalTensor.Descriptor", _handle_ptr=None):
+        if _handle_ptr is not None:
+            self._h = _handle_ptr
+        else:
+            dims, rank = _u64_array(descriptor.dimensions)
+            self._h = _handle(lib().thor_tensor_create(int(placement.device_type), placement.device_num, int(descriptor.dtype), dims, rank),
+                              "PhysicalTensor")
+
+    @classmethod
+    def _wrap(cls, ptr) -> "PhysicalTensor":
+        return cls(None, None, _handle_ptr=_handle(ptr, "tensor handle"))
+
+    def get_descriptor(self) -> "PhysicalTensor.Descriptor":
+        return PhysicalTensor.Descriptor(self.get_data_type(), self.get_dimensions())
+
+    def get_data_type(self) -> DataType:
+        return DataType(lib().thor_tensor_dtype(self._h))
+
+    def get_dimensions(self) -> List[int]:
+        rank = lib().thor_tensor_rank(self._h)
+        out = (ctypes.c_uint64 * rank)()
+        _check(lib().thor_tensor_dims(self._h, out), "get_dimensions")
+        return list(out)
+
+    def get_strides_elements(self) -> List[int]:
+        rank = lib().thor_tensor_rank(self._h)
+        out = (ctypes.c_uint64 * rank)()
+        _check(lib().thor_tensor_strides(self._h, out), "get_strides_elements")
+        return list(out)
+
+    def get_placement(self) -> Placement:
+        return Placement(DeviceType(lib().thor_tensor_device_type(self._h)), lib().thor_tensor_device_num(self._h))
+
+    def get_total_num_elements(self) -> int:
+        return lib().thor_tensor_num_elements(self._h)
+
+    def is_dense_contiguous(self) -> bool:
+        return bool(lib().thor_tensor_is_dense(self._h))
+
+    def mem_ptr(self) -> int:
+        return lib().thor_tensor_mem_ptr(self._h) or 0
+
+    def numpy(self) -> np.ndarray:
+        """Zero-copy view of a CPU tensor in its numpy carrier dtype (bf16 / fp8 appear as raw unsigned integers)."""
+        if self.get_placement().device_type != DeviceType.cpu:
+            raise RuntimeError("numpy() is only available for CPU tensors")
+        if not self.is_dense_contiguous():
+            raise RuntimeError("numpy() requires a dense tensor")
+        carrier = numpy_carrier(self.get_data_type())
+        n = self.get_total_num_elements()
+        buf = (ctypes.c_char * (n * carrier.itemsize)).from_address(self.mem_ptr())
+        arr = np.frombuffer(buf, dtype=carrier, count=n).reshape(self.get_dimensions())
+        arr.flags.writeable = True
+        self._keepalive = buf
+        return arr
+
+    def copy_from_async(self, source: "PhysicalTensor", stream: Stream):
+        _check(lib().thor_tensor_copy_from_async(self._h, source._h, stream._h), "copy_from_async")
+
+    def memset_async(self, value: int, stream: Stream):
+        _check(lib().thor_tensor_memset_async(self._h, value, stream._h), "memset_async")
+
+    def reshape(self, dimensions: Sequence[int]):
+        dims, rank = _u64_array(dimensions)
+        _check(lib().thor_tensor_reshape(self._h, dims, rank), "reshape")
+
+    def alias_view(self, dimensions: Sequence[int], strides_elements: Sequence[int], element_offset: int = 0) -> "PhysicalTensor":
+        dims, rank = _u64_array(dimensions)
+        strides, _ = _u64_array(strides_elements)
+        return PhysicalTensor._wrap(lib().thor_tensor_alias_view(self._h, dims, strides, rank, element_offset))
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_tensor_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+def convert_type_cpu(values: np.ndarray, source_dtype: DataType, dest_dtype: DataType) -> np.ndarray:
+    """TypeConverter's host path (TypeConverter::cpuConvertTypeImpl) on a numpy carrier array."""
+    values = np.ascontiguousarray(values)
+    assert values.dtype == numpy_carrier(source_dtype)
+    out = np.empty(values.shape, dtype=numpy_carrier(dest_dtype))
+    _check(lib().thor_convert_type_cpu(values.ctypes.data, out.ctypes.data, int(source_dtype), int(dest_dtype), values.size), "convert_type_cpu")
+    return out
+
+
+# ---- reductions ------------------------------------------------------------------------------------------------------------
+class CubReductionOp(enum.IntEnum):
+    Sum = 0
+    Min = 1
+    Max = 2
+    Product = 3
+    Mean = 4
+    L1Norm = 5
+    L2Norm = 6
+
+
+class CubArgReductionOp(enum.IntEnum):
+    ArgMin = 0
+    ArgMax = 1
+
+
+class CubReductionPath(enum.IntEnum):
+    DeviceTransformReduce = 0
+    ContiguousFixedSegment = 1
+    TiledFixedSegment = 2
+    StridedFixedSegment = 3
+    OffsetSegmented = 4
+
+
+def analyze_geometry(dims: Sequence[int], axes: Union[int, Sequence[int]], strides: Optional[Sequence[int]] = None) -> ReductionGeometry:
+    axes = [axes] if isinstance(axes, int) else list(axes)
+    d, rank = _u64_array(dims)
+    a, na = _u32_array(axes)
+    s = _u64_array(strides)[0] if strides is not None else None
+    out = ReductionGeometry()
+    _check(lib().thor_reduction_analyze_geometry(d, s, len(dims), a, na, ctypes.byref(out)), "analyzeGeometry")
+    return out
+
+
+def map_logical_reduction_index(dims, axes, output_index, reduction_index, strides=None) -> int:
+    d, _ = _u64_array(dims)
+    a, na = _u32_array(axes)
+    s = _u64_array(strides)[0] if strides is not None else None
+    out = ctypes.c_uint64()
+    _check(lib().thor_reduction_map_index(d, s, len(dims), a, na, output_index, reduction_index, ctypes.byref(out)), "mapLogicalReductionIndex")
+    return out.value
+
+
+def reduction_source(is_arg: bool, op: int, input_dtype: DataType, output_dtype: DataType, dims, axes, strides=None,
+                     index_dtype: DataType = DataType.uint32) -> str:
+    d, _ = _u64_array(dims)
+    a, na = _u32_array(axes)
+    s = _u64_array(strides)[0] if strides is not None else None
+    cap = 1 << 20
+    buf = ctypes.create_string_buffer(cap)
+    need = ctypes.c_size_t()
+    _check(lib().thor_reduction_generate_source(int(is_arg), int(op), int(input_dtype), int(output_dtype), int(index_dtype), d, s, len(dims), a, na,
+                                                buf, cap, ctypes.byref(need)), "reduction_source")
+    return buf.value.decode()
+
+
+class StampedCubReduction:
+    def __init__(self, ptr):
+        self._h = ptr
+
+    def run(self, output_scale: Optional[float] = None):
+        if output_scale is None:
+            _check(lib().thor_stamped_reduction_run(self._h), "StampedCubReduction.run")
+        else:
+            _check(lib().thor_stamped_reduction_run_scaled(self._h, output_scale), "StampedCubReduction.run")
+
+    def run_on(self, stream: Stream):
+        _check(lib().thor_stamped_reduction_run_on(self._h, stream._h), "StampedCubReduction.runOn")
+
+    def get_output_tensor(self) -> PhysicalTensor:
+        return PhysicalTensor._wrap(lib().thor_stamped_reduction_output(self._h))
+
+    def get_path(self) -> CubReductionPath:
+        return CubReductionPath(lib().thor_stamped_reduction_path(self._h))
+
+    def get_workspace_size_in_bytes(self) -> int:
+        return lib().thor_stamped_reduction_workspace_bytes(self._h)
+
+    def get_kernel_variant(self) -> str:
+        buf = ctypes.create_string_buffer(512)
+        _check(lib().thor_stamped_reduction_variant(self._h, buf, 512), "variant")
+        return buf.value.decode()
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_stamped_reduction_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class CubReduction:
+    """CubReduction(op, axes, output_dtype=None, output_scale=1.0).stamp(input, stream[, preallocated_output])."""
+
+    def __init__(self, op: CubReductionOp, axes: Union[int, Sequence[int]], output_dtype: Optional[DataType] = None, output_scale: float = 1.0):
+        self.op, self.axes = int(op), ([axes] if isinstance(axes, int) else list(axes))
+        self.output_dtype, self.output_scale = output_dtype, float(output_scale)
+
+    def stamp(self, input: PhysicalTensor, stream: Stream, preallocated_output: Optional[PhysicalTensor] = None) -> StampedCubReduction:
+        a, na = _u32_array(self.axes)
+        ptr = lib().thor_reduction_stamp(self.op, a, na, _dtype_code(self.output_dtype), self.output_scale, input._h,
+                                         preallocated_output._h if preallocated_output else None, stream._h)
+        return StampedCubReduction(_handle(ptr, "CubReduction.stamp"))
+
+
+class StampedCubArgReduction:
+    def __init__(self, ptr):
+        self._h = ptr
+
+    def run(self):
+        _check(lib().thor_stamped_arg_reduction_run(self._h), "StampedCubArgReduction.run")
+
+    def get_value_output_tensor(self) -> Optional[PhysicalTensor]:
+        ptr = lib().thor_stamped_arg_reduction_value_output(self._h)
+        return PhysicalTensor._wrap(ptr) if ptr else None
+
+    def get_index_output_tensor(self) -> Optional[PhysicalTensor]:
+        ptr = lib().thor_stamped_arg_reduction_index_output(self._h)
+        return PhysicalTensor._wrap(ptr) if ptr else None
+
+    def get_path(self) -> CubReductionPath:
+        return CubReductionPath(lib().thor_stamped_arg_reduction_path(self._h))
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_stamped_arg_reduction_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class CubArgReduction:
+    def __init__(self, op: CubArgReductionOp, axes: Union[int, Sequence[int]], produce_value: bool = True, produce_index: bool = True,
+                 value_output_dtype: Optional[DataType] = None, index_output_dtype: DataType = DataType.uint32):
+        self.op, self.axes = int(op), ([axes] if isinstance(axes, int) else list(axes))
+        self.produce_value, self.produce_index = produce_value, produce_index
+        self.value_output_dtype, self.index_output_dtype = value_output_dtype, index_output_dtype
+
+    def stamp(self, input: PhysicalTensor, stream: Stream, preallocated_value: Optional[PhysicalTensor] = None,
+              preallocated_index: Optional[PhysicalTensor] = None) -> StampedCubArgReduction:
+        a, na = _u32_array(self.axes)
+        ptr = lib().thor_arg_reduction_stamp(self.op, a, na, int(self.produce_value), int(self.produce_index), _dtype_code(self.value_output_dtype),
+                                             int(self.index_output_dtype), input._h, preallocated_value._h if preallocated_value else None,
+                                             preallocated_index._h if preallocated_index else None, stream._h)
+        return StampedCubArgReduction(_handle(ptr, "CubArgReduction.stamp"))
+
+
+# ---- expressions -------------------------------------------------------------------------------------------------------------
+def _as_expr(value) -> "Expression":
+    if isinstance(value, Expression):
+        return value
+    if isinstance(value, (int, float, np.floating, np.integer)):
+        return Expression.constant_scalar(float(value))
+    raise TypeError(f"cannot use {type(value).__name__} as an Expression operand")
+
+
+def _parse_axes(axis) -> List[int]:
+    if axis is None:
+        return []
+    if isinstance(axis, (int, np.integer)):
+        return [int(axis)]
+    return [int(a) for a in axis]
+
+
+def _parse_squeeze(squeeze) -> List[int]:
+    if squeeze is True:
+        return [UINT64_MAX]
+    if squeeze is False or squeeze is None:
+        return []
+    if isinstance(squeeze, (int, np.integer)):
+        return [int(squeeze)]
+    return [int(a) for a in squeeze]
+
+
+class Expression:
+    """Expression graph node; static builders mirror `thor.physical.Expression` (`ex.input`, `ex.exp`, `ex.reduce_sum`, ...)."""
+
+    def __init__(self, ptr):
+        self._h = _handle(ptr, "Expression")
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_expr_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    # -- leaves
+    @staticmethod
+    def input(name: str, compute_dtype: Optional[DataType] = None, output_dtype: Optional[DataType] = None) -> "Expression":
+        return Expression(lib().thor_expr_input(name.encode(), _dtype_code(compute_dtype), _dtype_code(output_dtype)))
+
+    @staticmethod
+    def runtime_scalar(name: str, compute_dtype: Optional[DataType] = None, output_dtype: Optional[DataType] = None) -> "Expression":
+        return Expression(lib().thor_expr_runtime_scalar(name.encode(), _dtype_code(compute_dtype), _dtype_code(output_dtype)))
+
+    @staticmethod
+    def constant_scalar(value: float) -> "Expression":
+        return Expression(lib().thor_expr_scalar(float(value)))
+
+    @staticmethod
+    def fill(value: float, dims: Sequence[int], output_dtype: Optional[DataType] = None) -> "Expression":
+        d, rank = _u64_array(dims)
+        return Expression(lib().thor_expr_fill(float(value), d, rank, _dtype_code(output_dtype)))
+
+    # -- generic dispatch
+    def _binary(self, method: str, other, reflected: bool = False) -> "Expression":
+        other = _as_expr(other)
+        lhs, rhs = (other, self) if reflected else (self, other)
+        return Expression(lib().thor_expr_binary(method.encode(), lhs._h, rhs._h))
+
+    def _unary(self, method: str) -> "Expression":
+        return Expression(lib().thor_expr_unary(method.encode(), self._h))
+
+    def __add__(self, o): return self._binary("add", o)
+    def __radd__(self, o): return self._binary("add", o, True)
+    def __sub__(self, o): return self._binary("sub", o)
+    def __rsub__(self, o): return self._binary("sub", o, True)
+    def __mul__(self, o): return self._binary("mul", o)
+    def __rmul__(self, o): return self._binary("mul", o, True)
+    def __truediv__(self, o): return self._binary("div", o)
+    def __rtruediv__(self, o): return self._binary("div", o, True)
+    def __pow__(self, o): return self._binary("pow", o)
+    def __rpow__(self, o): return self._binary("pow", o, True)
+    def __neg__(self): return self._unary("neg")
+    def __lt__(self, o): return self._binary("lessThan", o)
+    def __le__(self, o): return self._binary("lessEqual", o)
+    def __gt__(self, o): return self._binary("greaterThan", o)
+    def __ge__(self, o): return self._binary("greaterEqual", o)
+    def __eq__(self, o): return self._binary("equal", o)  # type: ignore[override]
+    def __ne__(self, o): return self._binary("notEqual", o)  # type: ignore[override]
+    __hash__ = None  # type: ignore[assignment]
+
+    def min(self, o): return self._binary("min", o)
+    def max(self, o): return self._binary("max", o)
+    def pow(self, o): return self._binary("pow", o)
+    def logical_and(self, o): return self._binary("logicalAnd", o)
+    def logical_or(self, o): return self._binary("logicalOr", o)
+    def logical_not(self): return self._unary("logicalNot")
+    def dot_product(self, o): return self._binary("dotProduct", o)
+
+    def cast(self, dtype: DataType) -> "Expression":
+        return Expression(lib().thor_expr_cast(self._h, int(dtype)))
+
+    def with_dtypes(self, compute_dtype: Optional[DataType] = None, output_dtype: Optional[DataType] = None) -> "Expression":
+        return Expression(lib().thor_expr_with_dtypes(self._h, _dtype_code(compute_dtype), _dtype_code(output_dtype)))
+
+    def with_compute_dtype(self, dtype: DataType) -> "Expression":
+        return self.with_dtypes(compute_dtype=dtype)
+
+    def with_output_dtype(self, dtype: DataType) -> "Expression":
+        return self.with_dtypes(output_dtype=dtype)
+
+    @staticmethod
+    def where(condition, true_value, false_value) -> "Expression":
+        return Expression(lib().thor_expr_where(_as_expr(condition)._h, _as_expr(true_value)._h, _as_expr(false_value)._h))
+
+    select = where
+
+    def elu(self, alpha: float = 1.0): return Expression(lib().thor_expr_unary_params(b"elu", self._h, alpha, 0.0))
+    def hard_tanh(self, min_value=-1.0, max_value=1.0): return Expression(lib().thor_expr_unary_params(b"hardTanh", self._h, min_value, max_value))
+    def threshold(self, threshold=0.0, value=0.0): return Expression(lib().thor_expr_unary_params(b"threshold", self._h, threshold, value))
+    def log(self, base: float): return Expression(lib().thor_expr_unary_params(b"log", self._h, base, 0.0))
+    def clamp(self, lo: float, hi: float): return Expression(lib().thor_expr_unary_params(b"clamp", self._h, lo, hi))
+
+    def reshape(self, dims: Sequence[int]) -> "Expression":
+        d, rank = _u64_array([UINT64_MAX if v == -1 else v for v in dims])
+        return Expression(lib().thor_expr_reshape(self._h, d, rank))
+
+    def unsqueeze(self, axes) -> "Expression":
+        a, n = _u64_array(_parse_axes(axes))
+        return Expression(lib().thor_expr_unsqueeze(self._h, a, n))
+
+    def squeeze(self, axes) -> "Expression":
+        a, n = _u64_array(_parse_axes(axes))
+        return Expression(lib().thor_expr_squeeze(self._h, a, n))
+
+    def _reduce(self, method: str, axis=None, squeeze=False, output_dtype: Optional[DataType] = None) -> "Expression":
+        axes, na = _u64_array(_parse_axes(axis))
+        sq, ns = _u64_array(_parse_squeeze(squeeze))
+        out = Expression(lib().thor_expr_reduce(method.encode(), self._h, axes, na, sq, ns))
+        return out.with_output_dtype(output_dtype) if output_dtype is not None else out
+
+    def num_nodes(self) -> int:
+        return lib().thor_expr_num_nodes(self._h)
+
+    def canonical(self) -> str:
+        need = ctypes.c_size_t()
+        cap = 1 << 16
+        buf = ctypes.create_string_buffer(cap)
+        _check(lib().thor_expr_canonical(self._h, buf, cap, ctypes.byref(need)), "canonical")
+        return buf.value.decode()
+
+    # -- compile (thor.physical.Expression.compile)
+    @staticmethod
+    def outputs(named: Dict[str, "Expression"]) -> "Outputs":
+        return Outputs(named)
+
+    @staticmethod
+    def compile(expr_or_outputs, device_num: int = 0) -> "FusedEquation":
+        outputs = expr_or_outputs if isinstance(expr_or_outputs, Outputs) else Outputs({"output": _as_expr(expr_or_outputs)})
+        return FusedEquation(_handle(lib().thor_fused_equation_compile(outputs._h, device_num), "Expression.compile"))
+
+
+_UNARY_NAMES = ["abs", "ceil", "floor", "round", "trunc", "sin", "cos", "tan", "csc", "sec", "cot", "asin", "acos", "atan", "acsc", "asec", "acot",
+                "sinh", "cosh", "tanh", "csch", "sech", "coth", "asinh", "acosh", "atanh", "acsch", "asech", "acoth", "erf", "erfc", "erfcx",
+                "erfinv", "erfcinv", "tgamma", "lgamma", "digamma", "ln", "log1p", "log2", "log10", "exp", "expm1", "exp2", "exp10", "sqrt",
+                "normcdf", "sigmoid", "softplus", "selu", "gelu", "mish", "relu6", "swish"]
+for _name in _UNARY_NAMES:
+    setattr(Expression, _name, (lambda n: lambda self: self._unary(n))(_name))
+Expression.hard_swish = lambda self: self._unary("hardSwish")
+Expression.relu = lambda self: self.max(0.0)  # ReLU is spelled max(x, 0) in the reference (Api/Layers/Activations/Relu.h:21-22)
+
+_REDUCTIONS = ["reduce_sum", "reduce_prod", "reduce_min", "reduce_max", "reduce_mean", "reduce_norm1", "reduce_norm2"]
+for _name in _REDUCTIONS:
+    setattr(Expression, _name, (lambda n: lambda self, axis=None, squeeze=False, compute_dtype=DataType.fp32, output_dtype=DataType.fp32:
+                                self._reduce(n, axis, squeeze, output_dtype))(_name))
+Expression.argmin = lambda self, axis=None, squeeze=False: self._reduce("argmin", axis, squeeze)
+Expression.argmax = lambda self, axis=None, squeeze=False: self._reduce("argmax", axis, squeeze)
+
+
+class Outputs:
+    def __init__(self, named: Dict[str, Expression]):
+        names = list(named.keys())
+        self._h = _handle(lib().thor_outputs_create(_names(names), _ptrs([named[n]._h for n in names]), len(names)), "Expression.outputs")
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_outputs_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class Equation:
+    """A stamped execution plan (StampedExecutionPlan): run() only launches."""
+
+    def __init__(self, ptr):
+        self._h = ptr
+
+    def run(self, runtime_scalars: Optional[Dict[str, float]] = None):
+        if runtime_scalars:
+            names = list(runtime_scalars)
+            vals = (ctypes.c_float * len(names))(*[runtime_scalars[n] for n in names])
+            _check(lib().thor_plan_run_with_scalars(self._h, _names(names), vals, len(names)), "Equation.run")
+        else:
+            _check(lib().thor_plan_run(self._h), "Equation.run")
+
+    def run_on(self, stream: Stream):
+        _check(lib().thor_plan_run_on(self._h, stream._h), "Equation.runOn")
+
+    def output(self, name: Optional[str] = None) -> PhysicalTensor:
+        return PhysicalTensor._wrap(lib().thor_plan_output(self._h, name.encode() if name is not None else None))
+
+    def stage_kind_names(self) -> List[str]:
+        out = []
+        for s in range(lib().thor_plan_num_stages(self._h)):
+            buf = ctypes.create_string_buffer(64)
+            _check(lib().thor_plan_stage_kind(self._h, s, buf, 64), "stageKindNames")
+            out.append(buf.value.decode())
+        return out
+
+    def stage_descriptions(self) -> List[str]:
+        out = []
+        for s in range(lib().thor_plan_num_stages(self._h)):
+            buf = ctypes.create_string_buffer(512)
+            _check(lib().thor_plan_stage_description(self._h, s, buf, 512), "stage description")
+            out.append(buf.value.decode())
+        return out
+
+    def stage_source(self, stage: int) -> str:
+        cap = 1 << 20
+        buf = ctypes.create_string_buffer(cap)
+        need = ctypes.c_size_t()
+        _check(lib().thor_plan_stage_source(self._h, stage, buf, cap, ctypes.byref(need)), "stage source")
+        return buf.value.decode()
+
+    def flop_count(self) -> int:
+        return lib().thor_plan_flop_count(self._h)
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_plan_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class FusedEquation:
+    def __init__(self, ptr):
+        self._h = ptr
+
+    def output_names(self) -> List[str]:
+        out = []
+        for i in range(lib().thor_fused_equation_num_outputs(self._h)):
+            buf = ctypes.create_string_buffer(256)
+            _check(lib().thor_fused_equation_output_name(self._h, i, buf, 256), "getOutputNames")
+            out.append(buf.value.decode())
+        return out
+
+    def stamp(self, inputs: Dict[str, PhysicalTensor], stream: Stream, preallocated_outputs: Optional[Dict[str, PhysicalTensor]] = None) -> Equation:
+        names = list(inputs)
+        pre = preallocated_outputs or {}
+        pre_names = list(pre)
+        ptr = lib().thor_fused_equation_stamp(self._h, _names(names), _ptrs([inputs[n]._h for n in names]), len(names), _names(pre_names),
+                                              _ptrs([pre[n]._h for n in pre_names]), len(pre_names), stream._h)
+        return Equation(_handle(ptr, "FusedEquation.stamp"))
+
+    def run(self, inputs: Union[PhysicalTensor, Dict[str, PhysicalTensor]], outputs: Union[PhysicalTensor, Dict[str, PhysicalTensor]], stream: Stream,
+            scalar_inputs: Optional[Dict[str, float]] = None):
+        if isinstance(outputs, PhysicalTensor):
+            out_names = self.output_names()
+            if len(out_names) != 1:
+                raise RuntimeError("run(..., output) requires an equation with exactly one output")
+            outputs = {out_names[0]: outputs}
+        if isinstance(inputs, PhysicalTensor):
+            raise TypeError("pass inputs as a {name: tensor} dict")
+        in_names, out_names = list(inputs), list(outputs)
+        scalars = scalar_inputs or {}
+        s_names = list(scalars)
+        s_vals = (ctypes.c_float * max(1, len(s_names)))(*[scalars[n] for n in s_names])
+        _check(lib().thor_fused_equation_run(self._h, _names(in_names), _ptrs([inputs[n]._h for n in in_names]), len(in_names), _names(s_names), s_vals,
+                                             len(s_names), _names(out_names), _ptrs([outputs[n]._h for n in out_names]), len(out_names), stream._h),
+               "FusedEquation.run")
+
+    def get_output_shape(self, inputs: Dict[str, PhysicalTensor], output_name: str = "output"):
+        names = list(inputs)
+        dims = (ctypes.c_uint64 * 16)()
+        rank, dtype = ctypes.c_int(), ctypes.c_int()
+        _check(lib().thor_fused_equation_output_shape(self._h, _names(names), _ptrs([inputs[n]._h for n in names]), len(names), output_name.encode(), dims,
+                                                      ctypes.byref(rank), ctypes.byref(dtype)), "getOutputShape")
+        return list(dims[: rank.value]), DataType(dtype.value)
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_fused_equation_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+def compiled_kernel_count() -> int:
+    return lib().thor_compiled_kernel_count()
