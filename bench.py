@@ -57,6 +57,114 @@ def cpu_baseline(seconds_budget: float = 12.0):
             "sample": f"{elems // (4 * n)} passes of the 4 conversions over 2^25 elements ({dt:.1f} s)"}
 
 
+def bench_other_configs(stream_raw_unused=None, iters=20):
+    """BASELINE configs 1, 3, 4, 5 through the Expression / reduction API: GB/s on algorithmic bytes, HIP-event timed."""
+    from thor_amd import physical as ph
+    from thor_amd.dtypes import DataType
+    from thor_amd.physical import Expression as ex
+    from thor_amd.runtime import Event
+
+    import oracle
+    stream = ph.Stream(0)
+    results = {}
+
+    class RawStream:  # Event.record wants an object with .handle
+        handle = stream.handle
+
+    def gpu_from(values, dtype):
+        carrier = values if dtype == DataType.fp32 else oracle.convert(np.ascontiguousarray(values, dtype=np.float32), oracle.FP32, int(dtype))
+        shape = list(carrier.shape)
+        cpu = ph.PhysicalTensor(ph.Placement(ph.DeviceType.cpu), ph.PhysicalTensor.Descriptor(dtype, shape))
+        cpu.numpy()[...] = carrier
+        gpu = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(dtype, shape))
+        gpu.copy_from_async(cpu, stream)
+        stream.synchronize()
+        return gpu
+
+    def timed(name, run, nbytes, elements, note=""):
+        for _ in range(3):
+            run()
+        stream.synchronize()
+        a, b = Event(), Event()
+        a.record(RawStream)
+        for _ in range(iters):
+            run()
+        b.record(RawStream)
+        b.synchronize()
+        ms = a.elapsed_ms(b) / iters
+        results[name] = {"ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1), "pct_hbm_peak": round(100 * nbytes / ms / 1e6 / HBM_PEAK_GBPS, 1),
+                         "Gelem/s": round(elements / ms / 1e6, 2), "plan": note}
+
+    rng = np.random.default_rng(1234)
+    # ---- config 1: out = (a*b+c)*sigmoid(d), fp32, 2^20 (cache resident) and 2^28 (HBM)
+    for log2n in (20, 28):
+        n = 1 << log2n
+        block = rng.uniform(-1, 1, min(n, 1 << 22)).astype(np.float32)
+        tensors = {}
+        for k in "abcd":
+            t = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [n]))
+            src = gpu_from(np.roll(block, ord(k)), DataType.fp32)
+            from thor_amd import _lib
+            for off in range(0, n, block.size):
+                _lib.check(_lib.load().thorhip_memcpy_async(t.mem_ptr() + off * 4, src.mem_ptr(), block.nbytes, 3, stream.handle), "d2d")
+            stream.synchronize()
+            tensors[k] = t
+        ea, eb, ec, ed = (ex.input(k) for k in "abcd")
+        plan = ex.compile((ea * eb + ec) * ed.sigmoid(), 0).stamp(tensors, stream)
+        timed(f"c1_fused_elementwise_fp32_2^{log2n}", plan.run, 20 * n, n, "+".join(plan.stage_descriptions()))
+        del tensors, plan
+
+    # ---- config 3: fp32 [8192, 8192]
+    x = gpu_from(rng.standard_normal((8192, 8192), dtype=np.float32), DataType.fp32)
+    n = 8192 * 8192
+    for name, stamped in (("c3_full_sum", ph.CubReduction(ph.CubReductionOp.Sum, [0, 1], DataType.fp32).stamp(x, stream)),
+                          ("c3_row_sum", ph.CubReduction(ph.CubReductionOp.Sum, 1, DataType.fp32).stamp(x, stream)),
+                          ("c3_row_max", ph.CubReduction(ph.CubReductionOp.Max, 1, DataType.fp32).stamp(x, stream))):
+        timed(name, stamped.run, 4 * n, n, stamped.get_kernel_variant())
+    amax = ph.CubArgReduction(ph.CubArgReductionOp.ArgMax, 1, produce_value=False).stamp(x, stream)
+    timed("c3_row_argmax", amax.run, 4 * n, n)
+    del x
+
+    # ---- config 4: bf16 [16384, 4096] softmax (fp32 out), fp32 [32768, 1024] mean/variance normalise
+    xs = gpu_from((rng.standard_normal((16384, 4096), dtype=np.float32) * 3), DataType.bf16)
+    ix = ex.input("x")
+    e = (ix - ix.reduce_max(axis=1)).exp()
+    soft = ex.compile(e / e.reduce_sum(axis=1), 0)
+    n = 16384 * 4096
+    for label, env in (("staged", "1"), ("fused", "0")):
+        os.environ["THOR_DISABLE_ROW_FUSION"] = env
+        plan = soft.stamp({"x": xs}, stream)
+        timed(f"c4_softmax_bf16_{label}", plan.run, 6 * n, n, ">".join(plan.stage_kind_names()))
+    del xs, plan
+    xn = gpu_from(rng.standard_normal((32768, 1024), dtype=np.float32), DataType.fp32)
+    mean = ix.reduce_mean(axis=1)
+    cen = ix - mean
+    var = (cen * cen).reduce_mean(axis=1)
+    norm = ex.compile(cen / (var + 1e-5).sqrt(), 0)
+    n = 32768 * 1024
+    for label, env in (("staged", "1"), ("fused", "0")):
+        os.environ["THOR_DISABLE_ROW_FUSION"] = env
+        plan = norm.stamp({"x": xn}, stream)
+        timed(f"c4_normalize_fp32_{label}", plan.run, 8 * n, n, ">".join(plan.stage_kind_names()))
+    os.environ.pop("THOR_DISABLE_ROW_FUSION", None)
+    del xn, plan
+
+    # ---- config 5: fp16 NCHW [64,256,56,56]
+    shape = (64, 256, 56, 56)
+    xc = gpu_from(rng.standard_normal(shape, dtype=np.float32), DataType.fp16)
+    scale = gpu_from(rng.uniform(0.5, 1.5, (1, 256, 1, 1)).astype(np.float32), DataType.fp16)
+    bias = gpu_from(rng.uniform(-0.1, 0.1, (1, 256, 1, 1)).astype(np.float32), DataType.fp16)
+    n = int(np.prod(shape))
+    plan = ex.compile((ex.input("x") * ex.input("scale") + ex.input("bias")).max(0.0), 0).stamp({"x": xc, "scale": scale, "bias": bias}, stream)
+    timed("c5_relu_scale_bias_fp16", plan.run, 4 * n, n, "+".join(plan.stage_descriptions()))
+    csum = ph.CubReduction(ph.CubReductionOp.Sum, [0, 2, 3], DataType.fp32).stamp(xc, stream)
+    timed("c5_channel_sum_fp16", csum.run, 2 * n, n, csum.get_kernel_variant())
+    stats = ex.compile(ex.outputs({"sum": ix.reduce_sum(axis=[0, 2, 3], squeeze=True), "sumsq": (ix * ix).reduce_sum(axis=[0, 2, 3], squeeze=True)}), 0)
+    plan = stats.stamp({"x": xc}, stream)
+    timed("c5_channel_sum_and_sumsq_fp16", plan.run, 2 * n, n, ">".join(plan.stage_kind_names()))
+    return results
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -64,6 +172,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--log2-elements", type=int, default=28)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the secondary lines for BASELINE configs 1, 3, 4, 5")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -138,6 +247,10 @@ def main():
                      "kernel": "convertSlots<float, f16> (fp32->fp16)", "kernel_avg_ms": round(kernel_avg_ms, 4),
                      "algorithmic_bytes_per_launch": n * BYTES_PER_ELEMENT},
     }
+    for b_ in (src, f16, b16, w16, wb16):
+        b_.free()
+    if not args.no_other_configs:
+        result["other_configs"] = bench_other_configs()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

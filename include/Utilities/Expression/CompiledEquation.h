@@ -35,7 +35,8 @@ struct CompiledKernel {
 };
 
 // Compiles (or fetches from the process-wide cache) `kernelName` from `source` for GPU `deviceNum`.  `fastContract`
-// selects -ffp-contract=fast (mul+add may fuse, matching the reference's -fmad=true) versus -ffp-contract=off.
+// keeps the compiler's default contraction (a*b+c inside one expression may fuse, matching the reference's
+// -fmad=true); false compiles with -ffp-contract=off so every operation rounds on its own.
 std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract);
 
 // Number of run-time compilations performed so far (cache misses); used by tests of the caching behaviour.

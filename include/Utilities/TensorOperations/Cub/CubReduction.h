@@ -18,6 +18,7 @@
 #include <limits>
 #include <memory>
 #include <optional>
+#include <string>
 #include <vector>
 
 namespace ThorImplementation {
@@ -152,9 +153,7 @@ struct ReductionLaunchPlan {
     std::shared_ptr<CompiledKernel> finishKernel;  // null unless the reduction domain was split across blocks
     uint32_t mainGridX = 1, mainGridY = 1, mainThreads = 256;
     uint32_t finishGridX = 1, finishThreads = 256;
-    bool usesTicketCounter = false;
-    size_t workspaceBytes = 0;  // partials (+ a 4-byte ticket counter at the end when used)
-    size_t counterOffset = 0;
+    size_t workspaceBytes = 0;  // per-block / per-share partials
     std::string variant;        // human-readable description of the chosen kernel shape
 };
 

@@ -1,0 +1,204 @@
+"""Single-pass row kernels (chains of last-axis reductions and the elementwise work between them, kept in registers)
+against the staged plan of the same expression and against closed forms in float64.
+
+The staged plan is what the reference produces for these expressions (test/Utilities/Expression/CommonInputFusionTest.cpp:281-327:
+softmax lowers to Reduction, Fused, Reduction, Fused); the row kernel must give the same values up to the rounding
+freedom of the fp32 accumulation order, and exactly the same values where no accumulation order is involved."""
+from __future__ import annotations
+
+import os
+
+import numpy as np
+import pytest
+
+from helpers import copy_gpu_to_numpy, copy_numpy_to_gpu, from_storage, run_staged, to_storage
+from thor_amd import physical as ph
+from thor_amd.dtypes import DataType
+from thor_amd.physical import Expression as ex
+
+pytestmark = pytest.mark.gpu
+
+
+def staged(expr, inputs, dtypes, scalars=None):
+    os.environ["THOR_DISABLE_ROW_FUSION"] = "1"
+    try:
+        return run_staged(expr, inputs, dtypes, scalars=scalars)
+    finally:
+        os.environ.pop("THOR_DISABLE_ROW_FUSION", None)
+
+
+def softmax_expr():
+    ix = ex.input("x")
+    e = (ix - ix.reduce_max(axis=1)).exp()
+    return e / e.reduce_sum(axis=1)
+
+
+TOL = {DataType.fp32: (3e-6, 1e-9), DataType.fp16: (2e-3, 1e-6), DataType.bf16: (1.6e-2, 1e-6)}
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)
+@pytest.mark.parametrize("shape", [(33, 200), (5, 2), (3, 7), (1000, 4096), (64, 4100), (9, 16384), (2, 32768), (300, 64), (4097, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_softmax_single_pass_matches_staged_and_closed_form(gpu, dtype, shape):
+    rng = np.random.default_rng(1237)
+    x = to_storage((rng.standard_normal(shape) * 3).astype(np.float32), dtype)
+    plan, outs = run_staged(softmax_expr(), {"x": x}, dtype)
+    assert plan.stage_kind_names() == ["FusedRowKernel"], plan.stage_descriptions()
+    plan_s, outs_s = staged(softmax_expr(), {"x": x}, dtype)
+    assert plan_s.stage_kind_names() == ["Reduction", "FusedKernel", "Reduction", "FusedKernel"]
+    got, ref = outs["output"], outs_s["output"]
+    assert got.dtype == ref.dtype and got.shape == ref.shape == shape
+    xf = from_storage(x, dtype).astype(np.float64)
+    p = np.exp(xf - xf.max(axis=1, keepdims=True))
+    want = p / p.sum(axis=1, keepdims=True)
+    rtol, atol = TOL[dtype]
+    np.testing.assert_allclose(got.astype(np.float64), want, rtol=rtol, atol=atol)
+    # against the staged plan: same values up to the order of the fp32 row sum (and, for 16-bit compute, one rounding step)
+    np.testing.assert_allclose(got.astype(np.float64), ref.astype(np.float64), rtol=rtol, atol=atol)
+    np.testing.assert_allclose(got.astype(np.float64).sum(axis=1), 1.0, rtol=max(rtol, 1e-5))
+
+
+def test_row_longer_than_the_register_budget_falls_back_to_the_staged_plan(gpu):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, 70001)).astype(np.float32)
+    plan, outs = run_staged(softmax_expr(), {"x": x}, DataType.fp32)
+    assert plan.stage_kind_names() == ["Reduction", "FusedKernel", "Reduction", "FusedKernel"]
+    x64 = x.astype(np.float64)
+    p = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(outs["output"], p / p.sum(axis=1, keepdims=True), rtol=3e-6, atol=1e-12)
+
+
+def test_order_independent_parts_are_bit_identical_to_the_staged_plan(gpu):
+    """x - rowmax and rowmax itself involve no accumulation order: both plans must agree bit for bit."""
+    rng = np.random.default_rng(77)
+    x = to_storage(rng.standard_normal((257, 1000)).astype(np.float32) * 10, DataType.fp16)
+    ix = ex.input("x")
+    m = ix.reduce_max(axis=1)
+    lo = ix.reduce_min(axis=1)
+    outputs = ex.outputs({"centered": (ix - m) / (m - lo + 1.0), "rowmax": m.squeeze([1]), "range": m - lo})
+    plan, outs = run_staged(outputs, {"x": x}, DataType.fp16)
+    assert plan.stage_kind_names() == ["FusedRowKernel"], plan.stage_descriptions()
+    _, outs_s = staged(outputs, {"x": x}, DataType.fp16)
+    for name in ("centered", "rowmax", "range"):
+        assert outs[name].shape == outs_s[name].shape
+        np.testing.assert_array_equal(outs[name].view(np.uint8), outs_s[name].view(np.uint8), err_msg=name)
+    xf = from_storage(x, DataType.fp16)
+    assert outs["rowmax"].dtype == np.float32  # reductions produce fp32 unless told otherwise
+    np.testing.assert_array_equal(outs["rowmax"], xf.max(axis=1))
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)
+@pytest.mark.parametrize("shape", [(8, 3, 130), (2048, 1024), (17, 4096)], ids=lambda s: "x".join(map(str, s)))
+def test_mean_variance_normalisation_single_pass(gpu, dtype, shape):
+    """y = (x - mean) / sqrt(var + eps) * gamma + beta over the last axis, gamma/beta of shape [R]."""
+    rng = np.random.default_rng(99)
+    R = shape[-1]
+    last = len(shape) - 1
+    x = to_storage((rng.standard_normal(shape) * 2 + 0.5).astype(np.float32), dtype)
+    gamma = to_storage(rng.uniform(0.5, 1.5, R).astype(np.float32), dtype)
+    beta = to_storage(rng.uniform(-1, 1, R).astype(np.float32), dtype)
+    ix, ig, ib = ex.input("x"), ex.input("gamma"), ex.input("beta")
+    mean = ix.reduce_mean(axis=last)
+    centered = ix - mean
+    var = (centered * centered).reduce_mean(axis=last)
+    expr = centered / (var + 1e-5).sqrt() * ig + ib
+    inputs = {"x": x, "gamma": gamma, "beta": beta}
+    plan, outs = run_staged(expr, inputs, dtype)
+    assert plan.stage_kind_names() == ["FusedRowKernel"], plan.stage_descriptions()
+    _, outs_s = staged(expr, inputs, dtype)
+    xf = from_storage(x, dtype).astype(np.float64)
+    g, b = from_storage(gamma, dtype).astype(np.float64), from_storage(beta, dtype).astype(np.float64)
+    mu = xf.mean(axis=last, keepdims=True)
+    v = ((xf - mu) ** 2).mean(axis=last, keepdims=True)
+    want = (xf - mu) / np.sqrt(v + 1e-5) * g + b
+    rtol, atol = {DataType.fp32: (2e-5, 2e-5), DataType.fp16: (6e-3, 6e-3), DataType.bf16: (4e-2, 4e-2)}[dtype]
+    got = outs["output"].astype(np.float64)
+    assert got.shape == tuple(shape)
+    np.testing.assert_allclose(got, want, rtol=rtol, atol=atol)
+    np.testing.assert_allclose(got, outs_s["output"].astype(np.float64), rtol=rtol, atol=atol)
+
+
+def test_values_needed_by_later_stages_are_written_and_everything_else_stays_on_chip(gpu):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((96, 384)).astype(np.float32)
+    ix = ex.input("x")
+    e = (ix - ix.reduce_max(axis=1)).exp()
+    row_sum = e.reduce_sum(axis=1)               # [96, 1]
+    total = row_sum.reduce_sum(axis=0)           # [1, 1]: a reduction over rows, outside the row kernel
+    outputs = ex.outputs({"softmax": e / row_sum, "total": total, "lse": row_sum.ln() + ix.reduce_max(axis=1)})
+    plan, outs = run_staged(outputs, {"x": x}, DataType.fp32)
+    kinds = plan.stage_kind_names()
+    assert kinds[0] == "FusedRowKernel" and kinds.count("FusedRowKernel") == 1 and "Reduction" in kinds[1:], kinds
+    x64 = x.astype(np.float64)
+    m = x64.max(axis=1, keepdims=True)
+    p = np.exp(x64 - m)
+    np.testing.assert_allclose(outs["softmax"], p / p.sum(axis=1, keepdims=True), rtol=3e-6)
+    np.testing.assert_allclose(outs["total"].reshape(()), p.sum(), rtol=1e-5)
+    np.testing.assert_allclose(outs["lse"], np.log(p.sum(axis=1, keepdims=True)) + m, rtol=1e-6)
+
+
+def test_runtime_scalar_and_squeezed_results(gpu):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((40, 333)).astype(np.float32)
+    ix, t = ex.input("x"), ex.runtime_scalar("t")
+    scaled = ix * t
+    e = (scaled - scaled.reduce_max(axis=1)).exp()
+    outputs = ex.outputs({"p": e / e.reduce_sum(axis=1), "sumsq": (scaled * scaled).reduce_sum(axis=1, squeeze=True) * 0.5})
+    for temperature in (0.5, 2.0):
+        plan, outs = run_staged(outputs, {"x": x}, DataType.fp32, scalars={"t": temperature})
+        assert plan.stage_kind_names() == ["FusedRowKernel"], plan.stage_descriptions()
+        s = x.astype(np.float64) * temperature
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        np.testing.assert_allclose(outs["p"], p / p.sum(axis=1, keepdims=True), rtol=3e-6)
+        assert outs["sumsq"].shape == (40,)
+        np.testing.assert_allclose(outs["sumsq"], 0.5 * (s * s).sum(axis=1), rtol=1e-5)
+
+
+def test_nan_and_inf_rows_behave_like_the_staged_plan(gpu):
+    x = np.zeros((4, 96), np.float32)
+    x[0, 5] = np.nan
+    x[1, 7] = np.inf
+    x[2, :] = -np.inf
+    x[3, :] = np.linspace(-50, 50, 96)
+    plan, outs = run_staged(softmax_expr(), {"x": x}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedRowKernel"]
+    _, outs_s = staged(softmax_expr(), {"x": x}, DataType.fp32)
+    np.testing.assert_array_equal(np.isnan(outs["output"]), np.isnan(outs_s["output"]))
+    ok = ~np.isnan(outs_s["output"])
+    np.testing.assert_allclose(outs["output"][ok], outs_s["output"][ok], rtol=2e-6, atol=1e-30)
+
+
+def test_config4_full_size_properties(gpu):
+    """softmax over [8192, 4096] bf16 -> fp32 and normalisation over [32768, 1024] fp32 at their full sizes."""
+    rng = np.random.default_rng(1237)
+    stream = ph.Stream(0)
+    x = to_storage((rng.standard_normal((8192, 4096), dtype=np.float32) * 3), DataType.bf16)
+    eq = ex.compile(softmax_expr(), 0)
+    tx = copy_numpy_to_gpu(x, stream, DataType.bf16)
+    plan = eq.stamp({"x": tx}, stream)
+    assert plan.stage_kind_names() == ["FusedRowKernel"]
+    plan.run()
+    got = copy_gpu_to_numpy(plan.output(), stream)
+    assert got.dtype == np.float32 and got.shape == (8192, 4096)
+    xf = from_storage(x, DataType.bf16)
+    assert np.all(got >= 0) and np.all(got <= 1)
+    np.testing.assert_allclose(got.astype(np.float64).sum(axis=1), 1.0, rtol=2e-2)
+    # the maximum of every row stays its maximum (ties allowed), and a sample of rows matches the closed form
+    assert np.all(got[np.arange(8192), xf.argmax(axis=1)] == got.max(axis=1))
+    rows = rng.choice(8192, 64, replace=False)
+    s = xf[rows].astype(np.float64)
+    p = np.exp(s - s.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(got[rows], p / p.sum(axis=1, keepdims=True), rtol=1.6e-2, atol=1e-7)
+
+    y = rng.standard_normal((32768, 1024), dtype=np.float32) * 4 + 1
+    iy = ex.input("y")
+    centered = iy - iy.reduce_mean(axis=1)
+    expr = centered / ((centered * centered).reduce_mean(axis=1) + 1e-5).sqrt()
+    plan, outs = run_staged(expr, {"y": y}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedRowKernel"]
+    z = outs["output"].astype(np.float64)
+    np.testing.assert_allclose(z.mean(axis=1), 0.0, atol=2e-6)
+    np.testing.assert_allclose((z * z).mean(axis=1), 1.0, rtol=2e-5)
+    y64 = y[rows].astype(np.float64)
+    mu = y64.mean(axis=1, keepdims=True)
+    np.testing.assert_allclose(z[rows], (y64 - mu) / np.sqrt(((y64 - mu) ** 2).mean(axis=1, keepdims=True) + 1e-5), rtol=2e-5, atol=2e-6)

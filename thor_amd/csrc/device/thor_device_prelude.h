@@ -2,8 +2,7 @@
 //
 // wave64 throughout: a wavefront is 64 lanes, a 256-thread block is 4 wavefronts.  Reductions keep fp32 accumulators in
 // registers, fold lanes with cross-lane shuffles, fold wavefronts through a few words of LDS, and fold blocks through
-// a per-launch partials buffer whose last-arriving block (atomic ticket) produces the final values -- one launch, no
-// atomics on the data, bit-reproducible for a fixed shape.
+// a per-launch partials buffer that a small second launch folds -- no atomics, bit-reproducible for a fixed shape.
 #pragma once
 
 namespace thor {
@@ -231,23 +230,6 @@ __device__ __forceinline__ void blockReduce(Acc& acc, Acc* scratch) {
     }
 }
 
-// Block-uniform "am I the last block to arrive" test.  The caller has written its partial; the fence orders that write
-// before the ticket, and the block that draws the last ticket re-arms the counter for the next launch.
-__device__ __forceinline__ bool lastBlockArrived(u32* counter, u32 expected, u32* sharedFlag) {
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const u32 ticket = atomicAdd(counter, 1u);
-        const bool last = ticket == expected - 1u;
-        if (last) *counter = 0u;
-        *sharedFlag = last ? 1u : 0u;
-    }
-    __syncthreads();
-    const bool last = *sharedFlag != 0u;
-    if (last) __threadfence();
-    return last;
-}
-
 // ---- result finalisation -----------------------------------------------------------------------------------------------
 // FINALIZE: 0 none, 1 divide by `divisor` (mean), 2 square root (L2 norm).  Then the fp32 scale, then one conversion.
 template <int FINALIZE>
@@ -258,27 +240,32 @@ __device__ __forceinline__ float finalizeValue(float acc, float divisor, float s
     return r * scale;
 }
 
-// digamma for x of either sign: reflection for x < 0.5, upward recurrence to x >= 6, then the asymptotic series
+// digamma(x) in fp32 with the reference's recipe (its emitted helper, Utilities/Expression/CudaSourceEmitter.cpp:679-722):
+// poles at the non-positive integers give NaN, x <= 0 is reflected through psi(1-x) - pi/tan(pi x), the argument is
+// walked up to x >= 8 with psi(x) = psi(x+1) - 1/x, and the asymptotic series is summed to the 1/x^10 term in the
+// same order, so the rounding behaviour matches term for term.
 __device__ inline float digammaf(float x) {
     if (x != x) return x;
-    float reflection = 0.0f;
-    bool reflect = false;
-    if (x <= 0.0f && x == __builtin_floorf(x)) return __builtin_nanf("");
-    if (x < 0.5f) {
-        const float pi = 3.14159265358979323846f;
-        reflection = pi / tanf(pi * x);
-        reflect = true;
+    if (__builtin_isinf(x)) return x > 0.0f ? x : __builtin_nanf("");
+    const float pi = 3.14159265358979323846f;
+    float acc = 0.0f;
+    if (x <= 0.0f) {
+        if (x == floorf(x)) return __builtin_nanf("");
+        acc -= pi / tanf(pi * x);
         x = 1.0f - x;
     }
-    float shift = 0.0f;
-    while (x < 6.0f) {
-        shift += 1.0f / x;
-        x += 1.0f;
-    }
-    const float inv = 1.0f / x, inv2 = inv * inv;
-    float series = inv2 * (1.0f / 12.0f - inv2 * (1.0f / 120.0f - inv2 * (1.0f / 252.0f - inv2 * (1.0f / 240.0f - inv2 * (1.0f / 132.0f)))));
-    float r = logf(x) - 0.5f * inv - series - shift;
-    return reflect ? r - reflection : r;
+    for (; x < 8.0f; x += 1.0f) acc -= 1.0f / x;
+    const float r = 1.0f / x;
+    const float r2 = r * r, r4 = r2 * r2;
+    const float r6 = r4 * r2, r8 = r4 * r4;
+    const float r10 = r8 * r2;
+    acc += logf(x) - 0.5f * r;
+    acc -= r2 * (1.0f / 12.0f);
+    acc += r4 * (1.0f / 120.0f);
+    acc -= r6 * (1.0f / 252.0f);
+    acc += r8 * (1.0f / 240.0f);
+    acc -= r10 * (1.0f / 132.0f);
+    return acc;
 }
 
 }  // namespace thor

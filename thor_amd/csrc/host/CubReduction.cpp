@@ -266,9 +266,6 @@ std::shared_ptr<StampedCubReduction> CubReduction::stamp(const Tensor& input, co
     std::optional<Tensor> workspace;
     if (plan.workspaceBytes > 0) {
         workspace = Tensor(input.getPlacement(), TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
-        if (plan.usesTicketCounter) {
-            THOR_HIP_CHECK(thorhip_memset_async(workspace->getMemPtr<char>() + plan.counterOffset, 0, 4, stream.getStream()));
-        }
     }
     return std::shared_ptr<StampedCubReduction>(
         new StampedCubReduction(op, geometry, input, output, std::move(plan), std::move(workspace), output_scale, stream));
@@ -279,9 +276,8 @@ void launchPlan(const ReductionLaunchPlan& plan, const void* in, void* valueOut,
                 float scale, void* stream) {
     char* ws = workspace.has_value() ? const_cast<Tensor&>(workspace.value()).getMemPtr<char>() : nullptr;
     void* partials = ws;
-    void* counter = (ws != nullptr && plan.usesTicketCounter) ? ws + plan.counterOffset : nullptr;
     const void* input = in;
-    std::vector<void*> args = {&input, &valueOut, &indexOut, &partials, &counter, &scale};
+    std::vector<void*> args = {&input, &valueOut, &indexOut, &partials, &scale};
     plan.mainKernel->launch(plan.mainGridX, plan.mainGridY, 1, plan.mainThreads, stream, args);
     if (plan.finishKernel) {
         const void* constPartials = partials;
@@ -377,9 +373,6 @@ std::shared_ptr<StampedCubArgReduction> CubArgReduction::stamp(const Tensor& inp
     std::optional<Tensor> workspace;
     if (plan.workspaceBytes > 0) {
         workspace = Tensor(input.getPlacement(), TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
-        if (plan.usesTicketCounter) {
-            THOR_HIP_CHECK(thorhip_memset_async(workspace->getMemPtr<char>() + plan.counterOffset, 0, 4, stream.getStream()));
-        }
     }
     return std::shared_ptr<StampedCubArgReduction>(
         new StampedCubArgReduction(op, geometry, input, std::move(value), std::move(index), std::move(plan), std::move(workspace), stream));

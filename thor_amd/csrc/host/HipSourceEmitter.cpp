@@ -262,142 +262,136 @@ bool tryFoldConstant(const PhysicalExpression& expr, uint32_t nodeIndex, double&
     }
 }
 
-namespace {
+BodyEmitter::BodyEmitter(const PhysicalExpression& expr) : expr(expr), valueDType(expr.nodes.size()), names(expr.nodes.size()) {}
 
-// Emits `const T tN = ...;` statements for a set of nodes.  Values of tensor sources (t<node> for operand nodes) are
-// defined by the caller; valueDType[] records the dtype every defined value has.
-class BodyEmitter {
-   public:
-    BodyEmitter(const PhysicalExpression& expr) : expr(expr), valueDType(expr.nodes.size()) {}
+void BodyEmitter::defineSource(uint32_t node, DataType dtype, const std::string& name) {
+    valueDType[node] = dtype;
+    names[node] = name.empty() ? "t" + std::to_string(node) : name;
+}
 
-    void defineSource(uint32_t node, DataType dtype) { valueDType[node] = dtype; }
-    bool defined(uint32_t node) const { return valueDType[node].has_value(); }
-    DataType dtypeOf(uint32_t node) const { return valueDType[node].value(); }
+std::string BodyEmitter::ref(uint32_t child, DataType target) const {
+    double folded;
+    if (!valueDType[child].has_value() && tryFoldConstant(expr, child, folded)) {
+        return castValueExpr(floatLiteral(folded), DataType::FP32, target);
+    }
+    if (!valueDType[child].has_value()) throw std::logic_error("Fused stage emitter referenced a value before its definition.");
+    return castValueExpr(names[child], valueDType[child].value(), target);
+}
 
-    std::string ref(uint32_t child, DataType target) const {
+std::vector<uint32_t> BodyEmitter::collect(const std::vector<uint32_t>& roots) const {
+    std::vector<char> need(expr.nodes.size(), 0);
+    std::vector<uint32_t> stack(roots.begin(), roots.end());
+    while (!stack.empty()) {
+        const uint32_t n = stack.back();
+        stack.pop_back();
+        if (need[n] || valueDType[n].has_value()) continue;
         double folded;
-        if (!valueDType[child].has_value() && tryFoldConstant(expr, child, folded)) {
-            return castValueExpr(floatLiteral(folded), DataType::FP32, target);
-        }
-        return castValueExpr("t" + std::to_string(child), valueDType[child].value(), target);
+        if (tryFoldConstant(expr, n, folded)) continue;
+        need[n] = 1;
+        const ExprNode& node = expr.nodes[n];
+        for (uint32_t c : {node.lhs, node.rhs, node.aux})
+            if (c != UINT32_MAX) stack.push_back(c);
     }
+    std::vector<uint32_t> order;
+    for (uint32_t i = 0; i < need.size(); ++i)
+        if (need[i]) order.push_back(i);
+    return order;
+}
 
-    // nodes (ascending) needed to evaluate `roots`, stopping at already defined values and at constants
-    std::vector<uint32_t> collect(const std::vector<uint32_t>& roots) const {
-        std::vector<char> need(expr.nodes.size(), 0);
-        std::vector<uint32_t> stack(roots.begin(), roots.end());
-        while (!stack.empty()) {
-            const uint32_t n = stack.back();
-            stack.pop_back();
-            if (need[n] || valueDType[n].has_value()) continue;
-            double folded;
-            if (tryFoldConstant(expr, n, folded)) continue;
-            need[n] = 1;
-            const ExprNode& node = expr.nodes[n];
-            for (uint32_t c : {node.lhs, node.rhs, node.aux})
-                if (c != UINT32_MAX) stack.push_back(c);
-        }
-        std::vector<uint32_t> order;
-        for (uint32_t i = 0; i < need.size(); ++i)
-            if (need[i]) order.push_back(i);
-        return order;
-    }
-
-    uint64_t emit(std::string& out, uint32_t nodeIndex, const std::string& indent, const std::vector<uint32_t>& scalarSlots) {
-        const ExprNode& n = expr.nodes[nodeIndex];
-        const DataType dtype = emittedValueDType(n);
-        const std::string decl = indent + "const " + valueCType(dtype) + " t" + std::to_string(nodeIndex) + " = ";
+uint64_t BodyEmitter::emit(std::string& out, uint32_t nodeIndex, const std::string& indent) {
+    const ExprNode& n = expr.nodes[nodeIndex];
+    const DataType dtype = emittedValueDType(n);
+    const std::string name = "t" + std::to_string(nodeIndex);
+    const std::string decl = indent + "const " + valueCType(dtype) + " " + name + " = ";
+    auto define = [&] {
         valueDType[nodeIndex] = dtype;
-        if (n.op == ExprOp::RUNTIME_SCALAR) {
-            (void)scalarSlots;
-            out += decl + castValueExpr("s" + std::to_string(n.input_slot), DataType::FP32, dtype) + ";\n";
-            return 0;
-        }
-        if (n.op == ExprOp::INPUT) throw std::runtime_error("Fused stage reads an input that was not bound as a kernel operand.");
-        uint32_t source;
-        if (aliasSource(expr, nodeIndex, source)) {
-            out += decl + ref(source, dtype) + ";\n";
-            return 0;
-        }
-        const uint64_t flops = opFlops(n.op);
-        if (n.op == ExprOp::CAST) {
-            out += decl + ref(n.lhs, dtype) + ";\n";
-            return flops;
-        }
-        if (n.op == ExprOp::WHERE) {
-            out += decl + "(" + ref(n.lhs, DataType::BOOLEAN) + " ? " + ref(n.rhs, dtype) + " : " + ref(n.aux, dtype) + ");\n";
-            return flops;
-        }
-        if (Expression::isBinaryOp(n.op)) {
-            out += decl + binary(n, dtype) + ";\n";
-            return flops;
-        }
+        names[nodeIndex] = name;
+    };
+    if (n.op == ExprOp::RUNTIME_SCALAR) {
+        out += decl + castValueExpr("s" + std::to_string(n.input_slot), DataType::FP32, dtype) + ";\n";
+        define();
+        return 0;
+    }
+    if (n.op == ExprOp::INPUT) throw std::runtime_error("Fused stage reads an input that was not bound as a kernel operand.");
+    uint32_t source;
+    uint64_t flops = 0;
+    if (aliasSource(expr, nodeIndex, source)) {
+        out += decl + ref(source, dtype) + ";\n";
+    } else if (n.op == ExprOp::CAST) {
+        out += decl + ref(n.lhs, dtype) + ";\n";
+    } else if (n.op == ExprOp::WHERE) {
+        out += decl + "(" + ref(n.lhs, DataType::BOOLEAN) + " ? " + ref(n.rhs, dtype) + " : " + ref(n.aux, dtype) + ");\n";
+        flops = 1;
+    } else if (Expression::isBinaryOp(n.op)) {
+        out += decl + binary(n, dtype) + ";\n";
+        flops = opFlops(n.op);
+    } else {
         out += decl + unary(n, dtype) + ";\n";
-        return flops;
+        flops = opFlops(n.op);
     }
+    define();
+    return flops;
+}
 
-   private:
-    std::string unary(const ExprNode& n, DataType c) const {
-        if (n.op == ExprOp::NEG) {
-            if (c == DataType::FP32 || c == DataType::FP16 || c == DataType::BF16) return "(-" + ref(n.lhs, c) + ")";
-            return castValueExpr("(-" + ref(n.lhs, DataType::FP32) + ")", DataType::FP32, c);
-        }
-        if (n.op == ExprOp::LOGICAL_NOT) {
-            if (c == DataType::BOOLEAN) return "(!" + ref(n.lhs, DataType::BOOLEAN) + ")";
-            return "(!(" + ref(n.lhs, DataType::FP32) + " != 0.0f))";
-        }
-        if (const char* fn = unaryFunction(n.op)) {
-            // evaluated on an fp32 copy of the operand and converted back to the compute dtype
-            return castValueExpr(std::string(fn) + "(" + ref(n.lhs, DataType::FP32) + ")", DataType::FP32, c);
-        }
-        throw std::runtime_error("Unsupported unary op in fused stage emitter: " + opName(n.op));
+std::string BodyEmitter::unary(const ExprNode& n, DataType c) const {
+    if (n.op == ExprOp::NEG) {
+        if (c == DataType::FP32 || c == DataType::FP16 || c == DataType::BF16) return "(-" + ref(n.lhs, c) + ")";
+        return castValueExpr("(-" + ref(n.lhs, DataType::FP32) + ")", DataType::FP32, c);
     }
-
-    std::string binary(const ExprNode& n, DataType c) const {
-        const bool native = c == DataType::FP32 || c == DataType::FP16 || c == DataType::BF16;
-        auto arithmetic = [&](const char* op) {
-            if (native || (n.op == ExprOp::SUB && (c == DataType::UINT32 || c == DataType::UINT64))) {
-                const std::string text = "(" + ref(n.lhs, c) + " " + op + " " + ref(n.rhs, c) + ")";
-                // bf16 arithmetic: exact fp32 operation on bf16 operands, then one rounding to bf16
-                return c == DataType::BF16 ? "thor::roundBf16" + text : text;
-            }
-            return castValueExpr("(" + ref(n.lhs, DataType::FP32) + " " + op + " " + ref(n.rhs, DataType::FP32) + ")", DataType::FP32, c);
-        };
-        const std::string a = ref(n.lhs, DataType::FP32), b = ref(n.rhs, DataType::FP32);
-        switch (n.op) {
-            case ExprOp::ADD: return arithmetic("+");
-            case ExprOp::SUB: return arithmetic("-");
-            case ExprOp::MUL: return arithmetic("*");
-            case ExprOp::DIV: return arithmetic("/");
-            case ExprOp::POW: return castValueExpr("powf(" + a + ", " + b + ")", DataType::FP32, c);
-            case ExprOp::MIN: return castValueExpr("fminf(" + a + ", " + b + ")", DataType::FP32, c);
-            case ExprOp::MAX: return castValueExpr("fmaxf(" + a + ", " + b + ")", DataType::FP32, c);
-            case ExprOp::EQUAL: return "(" + a + " == " + b + ")";
-            case ExprOp::NOT_EQUAL: return "(" + a + " != " + b + ")";
-            case ExprOp::LESS: return "(" + a + " < " + b + ")";
-            case ExprOp::LESS_EQUAL: return "(" + a + " <= " + b + ")";
-            case ExprOp::GREATER: return "(" + a + " > " + b + ")";
-            case ExprOp::GREATER_EQUAL: return "(" + a + " >= " + b + ")";
-            case ExprOp::LOGICAL_AND:
-                if (c == DataType::BOOLEAN) return "(" + ref(n.lhs, c) + " && " + ref(n.rhs, c) + ")";
-                return "((" + a + " != 0.0f) && (" + b + " != 0.0f))";
-            case ExprOp::LOGICAL_OR:
-                if (c == DataType::BOOLEAN) return "(" + ref(n.lhs, c) + " || " + ref(n.rhs, c) + ")";
-                return "((" + a + " != 0.0f) || (" + b + " != 0.0f))";
-            case ExprOp::MIN_GRAD_LEFT:
-            case ExprOp::MAX_GRAD_RIGHT:
-                return castValueExpr("((" + a + " < " + b + ") ? 1.0f : ((" + a + " > " + b + ") ? 0.0f : 0.5f))", DataType::FP32, c);
-            case ExprOp::MIN_GRAD_RIGHT:
-            case ExprOp::MAX_GRAD_LEFT:
-                return castValueExpr("((" + a + " > " + b + ") ? 1.0f : ((" + a + " < " + b + ") ? 0.0f : 0.5f))", DataType::FP32, c);
-            default: break;
-        }
-        throw std::runtime_error("Unsupported binary op in fused stage emitter: " + opName(n.op));
+    if (n.op == ExprOp::LOGICAL_NOT) {
+        if (c == DataType::BOOLEAN) return "(!" + ref(n.lhs, DataType::BOOLEAN) + ")";
+        return "(!(" + ref(n.lhs, DataType::FP32) + " != 0.0f))";
     }
+    if (const char* fn = unaryFunction(n.op)) {
+        // evaluated on an fp32 copy of the operand and converted back to the compute dtype
+        return castValueExpr(std::string(fn) + "(" + ref(n.lhs, DataType::FP32) + ")", DataType::FP32, c);
+    }
+    throw std::runtime_error("Unsupported unary op in fused stage emitter: " + opName(n.op));
+}
 
-    const PhysicalExpression& expr;
-    std::vector<std::optional<DataType>> valueDType;
-};
+std::string BodyEmitter::binary(const ExprNode& n, DataType c) const {
+    const bool native = c == DataType::FP32 || c == DataType::FP16 || c == DataType::BF16;
+    auto arithmetic = [&](const char* op) {
+        if (native || (n.op == ExprOp::SUB && (c == DataType::UINT32 || c == DataType::UINT64))) {
+            const std::string text = "(" + ref(n.lhs, c) + " " + op + " " + ref(n.rhs, c) + ")";
+            // bf16 arithmetic: exact fp32 operation on bf16 operands, then one rounding to bf16
+            return c == DataType::BF16 ? "thor::roundBf16" + text : text;
+        }
+        return castValueExpr("(" + ref(n.lhs, DataType::FP32) + " " + op + " " + ref(n.rhs, DataType::FP32) + ")", DataType::FP32, c);
+    };
+    const std::string a = ref(n.lhs, DataType::FP32), b = ref(n.rhs, DataType::FP32);
+    switch (n.op) {
+        case ExprOp::ADD: return arithmetic("+");
+        case ExprOp::SUB: return arithmetic("-");
+        case ExprOp::MUL: return arithmetic("*");
+        case ExprOp::DIV: return arithmetic("/");
+        case ExprOp::POW: return castValueExpr("powf(" + a + ", " + b + ")", DataType::FP32, c);
+        case ExprOp::MIN: return castValueExpr("fminf(" + a + ", " + b + ")", DataType::FP32, c);
+        case ExprOp::MAX: return castValueExpr("fmaxf(" + a + ", " + b + ")", DataType::FP32, c);
+        case ExprOp::EQUAL: return "(" + a + " == " + b + ")";
+        case ExprOp::NOT_EQUAL: return "(" + a + " != " + b + ")";
+        case ExprOp::LESS: return "(" + a + " < " + b + ")";
+        case ExprOp::LESS_EQUAL: return "(" + a + " <= " + b + ")";
+        case ExprOp::GREATER: return "(" + a + " > " + b + ")";
+        case ExprOp::GREATER_EQUAL: return "(" + a + " >= " + b + ")";
+        case ExprOp::LOGICAL_AND:
+            if (c == DataType::BOOLEAN) return "(" + ref(n.lhs, c) + " && " + ref(n.rhs, c) + ")";
+            return "((" + a + " != 0.0f) && (" + b + " != 0.0f))";
+        case ExprOp::LOGICAL_OR:
+            if (c == DataType::BOOLEAN) return "(" + ref(n.lhs, c) + " || " + ref(n.rhs, c) + ")";
+            return "((" + a + " != 0.0f) || (" + b + " != 0.0f))";
+        case ExprOp::MIN_GRAD_LEFT:
+        case ExprOp::MAX_GRAD_RIGHT:
+            return castValueExpr("((" + a + " < " + b + ") ? 1.0f : ((" + a + " > " + b + ") ? 0.0f : 0.5f))", DataType::FP32, c);
+        case ExprOp::MIN_GRAD_RIGHT:
+        case ExprOp::MAX_GRAD_LEFT:
+            return castValueExpr("((" + a + " > " + b + ") ? 1.0f : ((" + a + " < " + b + ") ? 0.0f : 0.5f))", DataType::FP32, c);
+        default: break;
+    }
+    throw std::runtime_error("Unsupported binary op in fused stage emitter: " + opName(n.op));
+}
+
+namespace {
 
 struct CollapsedLayout {
     std::vector<uint64_t> dims;                       // collapsed output dims
@@ -557,7 +551,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
             emitter.defineSource(op.node, valueDType);
         }
         uint64_t bodyFlops = 0;
-        for (uint32_t n : emitter.collect(roots)) bodyFlops += emitter.emit(body, n, indent, r.scalarSlots);
+        for (uint32_t n : emitter.collect(roots)) bodyFlops += emitter.emit(body, n, indent);
         for (size_t o = 0; o < r.outputs.size(); ++o) {
             const ExprNode& node = expr.nodes[r.outputs[o].node];
             const DataType outDType = node.output_dtype.value();

@@ -14,6 +14,7 @@
 #include "Utilities/Expression/Expression.h"
 
 #include <cstdint>
+#include <optional>
 #include <string>
 #include <vector>
 
@@ -71,5 +72,30 @@ std::string floatLiteral(double value);
 // dtype of the value a node evaluates to inside a kernel: leaves carry their output dtype, everything else its compute dtype
 DataType emittedValueDType(const ExprNode& node);
 bool tryFoldConstant(const PhysicalExpression& expr, uint32_t nodeIndex, double& value);
+
+// Emits `const T tN = ...;` statements for elementwise nodes.  Values that already exist (kernel operands, results of
+// earlier statements) are registered with their dtype and the C name that holds them; constants are folded on the host
+// and printed as literals; x+0, x*1, x/1 and pure shape ops become aliases of their operand.
+class BodyEmitter {
+   public:
+    explicit BodyEmitter(const PhysicalExpression& expr);
+    void defineSource(uint32_t node, DataType dtype, const std::string& name = "");
+    bool defined(uint32_t node) const { return valueDType[node].has_value(); }
+    DataType dtypeOf(uint32_t node) const { return valueDType[node].value(); }
+    const std::string& nameOf(uint32_t node) const { return names[node]; }
+    // expression reading the value of `child` converted to dtype `target`
+    std::string ref(uint32_t child, DataType target) const;
+    // nodes (ascending) needed to evaluate `roots`, stopping at already defined values and at host-foldable constants
+    std::vector<uint32_t> collect(const std::vector<uint32_t>& roots) const;
+    // appends the statement for one node (operands must be defined); returns the flops it costs per element
+    uint64_t emit(std::string& out, uint32_t nodeIndex, const std::string& indent);
+
+   private:
+    std::string unary(const ExprNode& n, DataType c) const;
+    std::string binary(const ExprNode& n, DataType c) const;
+    const PhysicalExpression& expr;
+    std::vector<std::optional<DataType>> valueDType;
+    std::vector<std::string> names;
+};
 
 }  // namespace ThorImplementation

@@ -168,12 +168,7 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
         const uint64_t vectors = g.input_elements / shape.vec;
         shape.blocks = std::min<uint64_t>(std::max<uint64_t>(ceilDiv(vectors, 256ull * shape.unroll), 1), 65536);
         shape.gridX = static_cast<uint32_t>(shape.blocks);
-        if (shape.blocks > 1) {
-            const size_t partials = partialBytes(shape.blocks, request.isArg, shape.indexIs64);
-            shape.counterOffset = ((partials + 255) / 256) * 256;
-            shape.workspaceBytes = shape.counterOffset + 256;
-            shape.usesTicketCounter = true;
-        }
+        if (shape.blocks > 1) shape.workspaceBytes = partialBytes(shape.blocks, request.isArg, shape.indexIs64);
         return shape;
     }
 
@@ -284,7 +279,8 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             s << "    static constexpr u64 kN = " << g.input_elements << "ull;\n";
             s << "    static constexpr int kUnroll = " << shape.unroll << ";\n";
             s << "    static constexpr u64 kBlocks = " << shape.blocks << "ull;\n";
-            body = "thor::reduceAll<gen::Cfg>(in, valueOut, indexOut, partials, counter, scale);";
+            s << "    static constexpr int kFinishThreads = 1024;\n";
+            body = "thor::reduceAll<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
             break;
         case ReductionShape::Kernel::Rows:
             s << "    static constexpr u64 kOuter = " << g.outer_size << "ull;\n";
@@ -324,10 +320,13 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     }
     s << "};\n}  // namespace gen\n";
     s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads
-      << ") void thor_reduce_main(const gen::Cfg::In* in, void* valueOut, void* indexOut, void* partials, unsigned int* counter, float scale) {\n"
-         "    (void)counter;\n    (void)partials;\n    "
+      << ") void thor_reduce_main(const gen::Cfg::In* in, void* valueOut, void* indexOut, void* partials, float scale) {\n"
+         "    (void)partials;\n    "
       << body << "\n}\n";
-    if (shape.split > 1) {
+    if (shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1) {
+        s << "extern \"C\" __global__ __launch_bounds__(1024) void thor_reduce_finish(const void* partials, void* valueOut, void* indexOut, float "
+             "scale) {\n    thor::finishAll<gen::Cfg>(partials, valueOut, indexOut, scale);\n}\n";
+    } else if (shape.split > 1) {
         s << "extern \"C\" __global__ __launch_bounds__(256) void thor_reduce_finish(const void* partials, void* valueOut, void* indexOut, float "
              "scale) {\n    thor::finishPartials<gen::Cfg>(partials, valueOut, indexOut, scale);\n}\n";
     }
@@ -340,7 +339,11 @@ ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request)
     ReductionLaunchPlan plan;
     // fp32 accumulation order is part of the result: never let the compiler fuse or reassociate across elements
     plan.mainKernel = compileKernel(source, "thor_reduce_main", request.deviceNum, /*fastContract=*/false);
-    if (shape.split > 1) {
+    if (shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1) {
+        plan.finishKernel = compileKernel(source, "thor_reduce_finish", request.deviceNum, false);
+        plan.finishThreads = 1024;
+        plan.finishGridX = 1;
+    } else if (shape.split > 1) {
         plan.finishKernel = compileKernel(source, "thor_reduce_finish", request.deviceNum, false);
         plan.finishThreads = 256;
         plan.finishGridX = static_cast<uint32_t>((request.geometry.output_elements * 64 + 255) / 256);
@@ -348,9 +351,7 @@ ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request)
     plan.mainGridX = shape.gridX;
     plan.mainGridY = shape.gridY;
     plan.mainThreads = static_cast<uint32_t>(shape.threads);
-    plan.usesTicketCounter = shape.usesTicketCounter;
     plan.workspaceBytes = shape.workspaceBytes;
-    plan.counterOffset = shape.counterOffset;
     plan.variant = shape.describe();
     return plan;
 }

@@ -34,8 +34,6 @@ struct ReductionShape {
     bool indexIs64 = false;
     uint32_t gridX = 1, gridY = 1;
     size_t workspaceBytes = 0;
-    size_t counterOffset = 0;
-    bool usesTicketCounter = false;
     // collapsed axes of the strided kernel
     std::vector<uint64_t> keptDims, keptStrides, reducedDims, reducedStrides;
     std::string describe() const;
