@@ -19,6 +19,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E published peak
+# HBM bytes one fp32->fp16 launch over 2^28 elements moves, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs scaled by the
+# same counters' readings for a plain copy kernel of known size (profiles/convert_round_trip_2p28_hbm_traffic.txt).
+MEASURED_TRAFFIC_BYTES_2P28 = 1572374 * 1024
 BYTES_PER_ELEMENT = 6   # fp32 <-> 16-bit: 4 + 2
 
 
@@ -81,22 +84,31 @@ def bench_other_configs(stream_raw_unused=None, iters=20):
         stream.synchronize()
         return gpu
 
-    def timed(name, run, nbytes, elements, note=""):
-        for _ in range(3):
-            run()
+    def clone(t):
+        c = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(t.get_data_type(), t.get_dimensions()))
+        c.copy_from_async(t, stream)
+        stream.synchronize()
+        return c
+
+    def timed(name, runs, nbytes, elements, note=""):
+        if callable(runs):
+            runs = [runs]
+        reps = max(iters, len(runs) * 2)
+        for k in range(max(3, len(runs))):
+            runs[k % len(runs)]()
         stream.synchronize()
         a, b = Event(), Event()
         a.record(RawStream)
-        for _ in range(iters):
-            run()
+        for k in range(reps):
+            runs[k % len(runs)]()
         b.record(RawStream)
         b.synchronize()
-        ms = a.elapsed_ms(b) / iters
+        ms = a.elapsed_ms(b) / reps
         results[name] = {"ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1), "pct_hbm_peak": round(100 * nbytes / ms / 1e6 / HBM_PEAK_GBPS, 1),
-                         "Gelem/s": round(elements / ms / 1e6, 2), "plan": note}
+                         "Gelem/s": round(elements / ms / 1e6, 2), "rotating_buffers": len(runs), "plan": note}
 
     rng = np.random.default_rng(1234)
-    # ---- config 1: out = (a*b+c)*sigmoid(d), fp32, 2^20 (cache resident) and 2^28 (HBM)
+    # ---- config 1: out = (a*b+c)*sigmoid(d), fp32, 2^20 (cache resident by construction) and 2^28 (5 GiB per launch)
     for log2n in (20, 28):
         n = 1 << log2n
         block = rng.uniform(-1, 1, min(n, 1 << 22)).astype(np.float32)
@@ -114,16 +126,17 @@ def bench_other_configs(stream_raw_unused=None, iters=20):
         timed(f"c1_fused_elementwise_fp32_2^{log2n}", plan.run, 20 * n, n, "+".join(plan.stage_descriptions()))
         del tensors, plan
 
-    # ---- config 3: fp32 [8192, 8192]
+    # ---- config 3: fp32 [8192, 8192] (256 MiB per input; rotated over 6 copies)
     x = gpu_from(rng.standard_normal((8192, 8192), dtype=np.float32), DataType.fp32)
     n = 8192 * 8192
-    for name, stamped in (("c3_full_sum", ph.CubReduction(ph.CubReductionOp.Sum, [0, 1], DataType.fp32).stamp(x, stream)),
-                          ("c3_row_sum", ph.CubReduction(ph.CubReductionOp.Sum, 1, DataType.fp32).stamp(x, stream)),
-                          ("c3_row_max", ph.CubReduction(ph.CubReductionOp.Max, 1, DataType.fp32).stamp(x, stream))):
-        timed(name, stamped.run, 4 * n, n, stamped.get_kernel_variant())
-    amax = ph.CubArgReduction(ph.CubArgReductionOp.ArgMax, 1, produce_value=False).stamp(x, stream)
-    timed("c3_row_argmax", amax.run, 4 * n, n)
-    del x
+    xs3 = [x] + [clone(x) for _ in range(5)]
+    for name, op, axes in (("c3_full_sum", ph.CubReductionOp.Sum, [0, 1]), ("c3_row_sum", ph.CubReductionOp.Sum, 1),
+                           ("c3_row_max", ph.CubReductionOp.Max, 1), ("c3_col_sum", ph.CubReductionOp.Sum, 0)):
+        stamps = [ph.CubReduction(op, axes, DataType.fp32).stamp(t, stream) for t in xs3]
+        timed(name, [st.run for st in stamps], 4 * n, n, stamps[0].get_kernel_variant())
+    amax = [ph.CubArgReduction(ph.CubArgReductionOp.ArgMax, 1, produce_value=False).stamp(t, stream) for t in xs3]
+    timed("c3_row_argmax", [a.run for a in amax], 4 * n, n)
+    del x, xs3, stamps, amax
 
     # ---- config 4: bf16 [16384, 4096] softmax (fp32 out), fp32 [32768, 1024] mean/variance normalise
     xs = gpu_from((rng.standard_normal((16384, 4096), dtype=np.float32) * 3), DataType.bf16)
@@ -131,37 +144,43 @@ def bench_other_configs(stream_raw_unused=None, iters=20):
     e = (ix - ix.reduce_max(axis=1)).exp()
     soft = ex.compile(e / e.reduce_sum(axis=1), 0)
     n = 16384 * 4096
+    xs4 = [xs] + [clone(xs) for _ in range(3)]
     for label, env in (("staged", "1"), ("fused", "0")):
         os.environ["THOR_DISABLE_ROW_FUSION"] = env
-        plan = soft.stamp({"x": xs}, stream)
-        timed(f"c4_softmax_bf16_{label}", plan.run, 6 * n, n, ">".join(plan.stage_kind_names()))
-    del xs, plan
+        plans = [soft.stamp({"x": t}, stream) for t in xs4]
+        timed(f"c4_softmax_bf16_{label}", [p_.run for p_ in plans], 6 * n, n, ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
+        del plans
+    del xs, xs4
     xn = gpu_from(rng.standard_normal((32768, 1024), dtype=np.float32), DataType.fp32)
     mean = ix.reduce_mean(axis=1)
     cen = ix - mean
     var = (cen * cen).reduce_mean(axis=1)
     norm = ex.compile(cen / (var + 1e-5).sqrt(), 0)
     n = 32768 * 1024
+    xn4 = [xn] + [clone(xn) for _ in range(5)]
     for label, env in (("staged", "1"), ("fused", "0")):
         os.environ["THOR_DISABLE_ROW_FUSION"] = env
-        plan = norm.stamp({"x": xn}, stream)
-        timed(f"c4_normalize_fp32_{label}", plan.run, 8 * n, n, ">".join(plan.stage_kind_names()))
+        plans = [norm.stamp({"x": t}, stream) for t in xn4]
+        timed(f"c4_normalize_fp32_{label}", [p_.run for p_ in plans], 8 * n, n, ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
+        del plans
     os.environ.pop("THOR_DISABLE_ROW_FUSION", None)
-    del xn, plan
+    del xn, xn4
 
-    # ---- config 5: fp16 NCHW [64,256,56,56]
+    # ---- config 5: fp16 NCHW [64,256,56,56] (98 MiB per tensor; rotated over 8 copies)
     shape = (64, 256, 56, 56)
     xc = gpu_from(rng.standard_normal(shape, dtype=np.float32), DataType.fp16)
     scale = gpu_from(rng.uniform(0.5, 1.5, (1, 256, 1, 1)).astype(np.float32), DataType.fp16)
     bias = gpu_from(rng.uniform(-0.1, 0.1, (1, 256, 1, 1)).astype(np.float32), DataType.fp16)
     n = int(np.prod(shape))
-    plan = ex.compile((ex.input("x") * ex.input("scale") + ex.input("bias")).max(0.0), 0).stamp({"x": xc, "scale": scale, "bias": bias}, stream)
-    timed("c5_relu_scale_bias_fp16", plan.run, 4 * n, n, "+".join(plan.stage_descriptions()))
-    csum = ph.CubReduction(ph.CubReductionOp.Sum, [0, 2, 3], DataType.fp32).stamp(xc, stream)
-    timed("c5_channel_sum_fp16", csum.run, 2 * n, n, csum.get_kernel_variant())
+    xc8 = [xc] + [clone(xc) for _ in range(7)]
+    relu = ex.compile((ex.input("x") * ex.input("scale") + ex.input("bias")).max(0.0), 0)
+    plans = [relu.stamp({"x": t, "scale": scale, "bias": bias}, stream) for t in xc8]
+    timed("c5_relu_scale_bias_fp16", [p_.run for p_ in plans], 4 * n, n, "+".join(plans[0].stage_descriptions()))
+    csum = [ph.CubReduction(ph.CubReductionOp.Sum, [0, 2, 3], DataType.fp32).stamp(t, stream) for t in xc8]
+    timed("c5_channel_sum_fp16", [c.run for c in csum], 2 * n, n, csum[0].get_kernel_variant())
     stats = ex.compile(ex.outputs({"sum": ix.reduce_sum(axis=[0, 2, 3], squeeze=True), "sumsq": (ix * ix).reduce_sum(axis=[0, 2, 3], squeeze=True)}), 0)
-    plan = stats.stamp({"x": xc}, stream)
-    timed("c5_channel_sum_and_sumsq_fp16", plan.run, 2 * n, n, ">".join(plan.stage_kind_names()))
+    plans = [stats.stamp({"x": t}, stream) for t in xc8]
+    timed("c5_channel_sum_and_sumsq_fp16", [p_.run for p_ in plans], 2 * n, n, ">".join(plans[0].stage_kind_names()))
     return results
 
 
@@ -173,6 +192,9 @@ def main():
     ap.add_argument("--log2-elements", type=int, default=28)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="skip the secondary lines for BASELINE configs 1, 3, 4, 5")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="before the timed region, launch a plain copy kernel of known size (uint32->int32 over the same element count: "
+                         "4 B read + 4 B written per element) so that hardware counters of a profiled run can be scaled against it")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -205,6 +227,10 @@ def main():
         TypeConverter.convert_type(src.ptr, b16.ptr, DataType.fp32, DataType.bf16, n, stream)
         TypeConverter.convert_type(b16.ptr, wb16.ptr, DataType.bf16, DataType.fp32, n, stream)
 
+    if args.calibration_copy:
+        for _ in range(3):
+            TypeConverter.convert_type(src.ptr, w16.ptr, DataType.uint32, DataType.int32, n, stream)
+        stream.synchronize()
     for _ in range(args.warmup):
         step()
     stream.synchronize()
@@ -243,8 +269,9 @@ def main():
         "gelem_per_s": round(4 * n * args.steps / elapsed / 1e9, 3),
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "convertSlots<float, f16> (fp32->fp16)", "kernel_avg_ms": round(kernel_avg_ms, 4),
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES_2P28 if args.log2_elements == 28 else None,
+                     "kernel": "convertSlots<float, thor::f16, 4, 1> (fp32->fp16)", "kernel_avg_ms": round(kernel_avg_ms, 4),
                      "algorithmic_bytes_per_launch": n * BYTES_PER_ELEMENT},
     }
     for b_ in (src, f16, b16, w16, wb16):

@@ -11,7 +11,7 @@ import os
 import numpy as np
 import pytest
 
-from helpers import copy_gpu_to_numpy, copy_numpy_to_gpu, from_storage, run_staged, to_storage
+from helpers import copy_gpu_to_numpy, copy_numpy_to_gpu, from_storage, run_staged, to_storage, ulp_distance_f32
 from thor_amd import physical as ph
 from thor_amd.dtypes import DataType
 from thor_amd.physical import Expression as ex
@@ -69,13 +69,15 @@ def test_row_longer_than_the_register_budget_falls_back_to_the_staged_plan(gpu):
 
 
 def test_order_independent_parts_are_bit_identical_to_the_staged_plan(gpu):
-    """x - rowmax and rowmax itself involve no accumulation order: both plans must agree bit for bit."""
+    """x - rowmax, rowmax and rowmax - rowmin involve no accumulation order: both plans must agree bit for bit.  Division by a
+    per-row value uses one reciprocal per row plus a fused correction step in the row kernel: within 1 ulp of the IEEE
+    quotient of the staged plan, and equal to it almost everywhere."""
     rng = np.random.default_rng(77)
     x = to_storage(rng.standard_normal((257, 1000)).astype(np.float32) * 10, DataType.fp16)
     ix = ex.input("x")
     m = ix.reduce_max(axis=1)
     lo = ix.reduce_min(axis=1)
-    outputs = ex.outputs({"centered": (ix - m) / (m - lo + 1.0), "rowmax": m.squeeze([1]), "range": m - lo})
+    outputs = ex.outputs({"centered": (ix - m) * 0.25, "rowmax": m.squeeze([1]), "range": m - lo, "scaled": (ix - m) / (m - lo + 1.0)})
     plan, outs = run_staged(outputs, {"x": x}, DataType.fp16)
     assert plan.stage_kind_names() == ["FusedRowKernel"], plan.stage_descriptions()
     _, outs_s = staged(outputs, {"x": x}, DataType.fp16)
@@ -85,6 +87,32 @@ def test_order_independent_parts_are_bit_identical_to_the_staged_plan(gpu):
     xf = from_storage(x, DataType.fp16)
     assert outs["rowmax"].dtype == np.float32  # reductions produce fp32 unless told otherwise
     np.testing.assert_array_equal(outs["rowmax"], xf.max(axis=1))
+    assert outs["scaled"].dtype == np.float32
+    distance = ulp_distance_f32(outs["scaled"], outs_s["scaled"])
+    assert distance.max() <= 1 and (distance != 0).mean() < 1e-3
+    x64 = xf.astype(np.float64)
+    exact = (x64 - x64.max(axis=1, keepdims=True)) / (x64.max(axis=1, keepdims=True) - x64.min(axis=1, keepdims=True) + 1.0)
+    assert ulp_distance_f32(outs["scaled"], exact.astype(np.float32)).max() <= 2
+
+
+def test_row_divisor_special_values(gpu):
+    """Zeros, infinities, NaNs, huge and tiny divisors and dividends give the same results as the staged plan's IEEE division."""
+    rows = np.array([[1.0, -2.0, 0.0, -0.0, np.inf, -np.inf, np.nan, 3e38, 1e-45, 1.5e-39, 7.0, 1e30],
+                     [1e38, 2e38, 3e38, 1.0, 0.0, -1.0, 5.0, 6.0, 7.0, 8.0, 9.0, 10.0],
+                     [1e-30, 2e-30, 1e-38, 1.0e-35, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0],
+                     [0.0] * 12,
+                     [np.inf, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0, 9.0, 10.0, 11.0],
+                     [3.0, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0, 9.0, 10.0, 11.0]], dtype=np.float32)
+    ix = ex.input("x")
+    expr = ix / ix.reduce_max(axis=1) + (ix * ix) / ix.reduce_norm1(axis=1)
+    plan, outs = run_staged(expr, {"x": rows}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedRowKernel"], plan.stage_descriptions()
+    _, outs_s = staged(expr, {"x": rows}, DataType.fp32)
+    got, ref = outs["output"], outs_s["output"]
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(ref))
+    np.testing.assert_array_equal(np.isinf(got), np.isinf(ref))
+    finite = np.isfinite(ref)
+    assert ulp_distance_f32(got[finite], ref[finite]).max() <= 2
 
 
 @pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)

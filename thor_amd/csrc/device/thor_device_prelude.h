@@ -101,9 +101,38 @@ __device__ __forceinline__ boolean makeBoolean(bool b) {
 
 // value rounded through a 16-bit / 8-bit float and widened again (how a bf16 / fp8 compute step is modelled in fp32)
 __device__ __forceinline__ float roundBf16(float x) { return toFloat(toBf16(x)); }
+// Storage form of a float that already holds a bf16 value (every bf16-typed value inside a kernel does: loads widen
+// exactly and every arithmetic result passes through roundBf16): the upper half of its bits; NaN stays canonical.
+__device__ __forceinline__ bf16 bf16FromExact(float x) {
+    bf16 r;
+    r.bits = (x != x) ? (u16)0x7fffu : (u16)(f32Bits(x) >> 16);
+    return r;
+}
 __device__ __forceinline__ float roundF16(float x) { return toFloat(toF16(x)); }
 __device__ __forceinline__ float roundE4m3(float x) { return toFloat(toE4m3(x)); }
 __device__ __forceinline__ float roundE5m2(float x) { return toFloat(toE5m2(x)); }
+
+// Division of many values by one divisor that a whole row shares (a row sum, a standard deviation).  The reciprocal is
+// taken once; each quotient is then x * r corrected by one fused residual step, with v_div_fixup supplying the IEEE
+// results for zeros, infinities, NaNs and exponent overflow / underflow.  The result is within one unit in the last
+// place of x / d and equal to it in all but rare cases, for a third of the instructions of a full division; divisors
+// whose reciprocal would leave the normal range take the full division.
+struct RowDivisor {
+    float d, r;
+    bool fast;
+    __device__ __forceinline__ explicit RowDivisor(float divisor) : d(divisor), r(1.0f / divisor) {
+        const float a = __builtin_fabsf(divisor);
+        fast = a >= 0x1p-100f && a <= 0x1p100f;
+    }
+    __device__ __forceinline__ float divide(float x) const {
+        if (fast) {
+            const float q = x * r;
+            const float residual = __builtin_fmaf(-d, q, x);
+            return __builtin_amdgcn_div_fixupf(__builtin_fmaf(residual, r, q), d, x);
+        }
+        return x / d;
+    }
+};
 
 // ---- reduction operators: fp32 accumulate -----------------------------------------------------------------------------
 // Min / Max return the NaN operand when either side is NaN (unlike fminf / fmaxf).

@@ -216,7 +216,7 @@ std::string storageToValueExpr(const std::string& x, DataType dtype) {
 std::string valueToStorageExpr(const std::string& x, DataType dtype) {
     switch (dtype) {
         case DataType::FP16: return "thor::fromHalf(" + x + ")";
-        case DataType::BF16: return "thor::toBf16(" + x + ")";
+        case DataType::BF16: return "thor::bf16FromExact(" + x + ")";  // bf16 values are held as floats that need no rounding
         case DataType::FP8_E4M3: return "thor::toE4m3(" + x + ")";
         case DataType::FP8_E5M2: return "thor::toE5m2(" + x + ")";
         case DataType::BOOLEAN: return "thor::makeBoolean(" + x + ")";
@@ -262,7 +262,8 @@ bool tryFoldConstant(const PhysicalExpression& expr, uint32_t nodeIndex, double&
     }
 }
 
-BodyEmitter::BodyEmitter(const PhysicalExpression& expr) : expr(expr), valueDType(expr.nodes.size()), names(expr.nodes.size()) {}
+BodyEmitter::BodyEmitter(const PhysicalExpression& expr)
+    : expr(expr), valueDType(expr.nodes.size()), names(expr.nodes.size()), rowDivisors(expr.nodes.size()) {}
 
 void BodyEmitter::defineSource(uint32_t node, DataType dtype, const std::string& name) {
     valueDType[node] = dtype;
@@ -364,7 +365,9 @@ std::string BodyEmitter::binary(const ExprNode& n, DataType c) const {
         case ExprOp::ADD: return arithmetic("+");
         case ExprOp::SUB: return arithmetic("-");
         case ExprOp::MUL: return arithmetic("*");
-        case ExprOp::DIV: return arithmetic("/");
+        case ExprOp::DIV:
+            if (c == DataType::FP32 && !rowDivisors[n.rhs].empty()) return rowDivisors[n.rhs] + ".divide(" + a + ")";
+            return arithmetic("/");
         case ExprOp::POW: return castValueExpr("powf(" + a + ", " + b + ")", DataType::FP32, c);
         case ExprOp::MIN: return castValueExpr("fminf(" + a + ", " + b + ")", DataType::FP32, c);
         case ExprOp::MAX: return castValueExpr("fmaxf(" + a + ", " + b + ")", DataType::FP32, c);

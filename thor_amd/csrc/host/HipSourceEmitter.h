@@ -87,6 +87,8 @@ class BodyEmitter {
     std::string ref(uint32_t child, DataType target) const;
     // nodes (ascending) needed to evaluate `roots`, stopping at already defined values and at host-foldable constants
     std::vector<uint32_t> collect(const std::vector<uint32_t>& roots) const;
+    // fp32 divisions by `node` are emitted as `name.divide(x)` (a thor::RowDivisor built once from the divisor's value)
+    void defineRowDivisor(uint32_t node, const std::string& name) { rowDivisors[node] = name; }
     // appends the statement for one node (operands must be defined); returns the flops it costs per element
     uint64_t emit(std::string& out, uint32_t nodeIndex, const std::string& indent);
 
@@ -96,6 +98,7 @@ class BodyEmitter {
     const PhysicalExpression& expr;
     std::vector<std::optional<DataType>> valueDType;
     std::vector<std::string> names;
+    std::vector<std::string> rowDivisors;
 };
 
 }  // namespace ThorImplementation

