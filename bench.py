@@ -135,7 +135,7 @@ def bench_other_configs(stream_raw_unused=None, iters=20):
         stamps = [ph.CubReduction(op, axes, DataType.fp32).stamp(t, stream) for t in xs3]
         timed(name, [st.run for st in stamps], 4 * n, n, stamps[0].get_kernel_variant())
     amax = [ph.CubArgReduction(ph.CubArgReductionOp.ArgMax, 1, produce_value=False).stamp(t, stream) for t in xs3]
-    timed("c3_row_argmax", [a.run for a in amax], 4 * n, n)
+    timed("c3_row_argmax", [a.run for a in amax], 4 * n, n, amax[0].get_kernel_variant())
     del x, xs3, stamps, amax
 
     # ---- config 4: bf16 [16384, 4096] softmax (fp32 out), fp32 [32768, 1024] mean/variance normalise

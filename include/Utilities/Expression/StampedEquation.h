@@ -11,6 +11,7 @@
 
 #include <cstdint>
 #include <memory>
+#include <optional>
 #include <string>
 #include <unordered_map>
 #include <unordered_set>
@@ -88,8 +89,32 @@ class StampedArgMinMax {
     std::shared_ptr<StampedCubArgReduction> stamped;
 };
 
+// Several value reductions over one geometry evaluated in a single pass over their common sources, with the
+// elementwise work that feeds them computed in registers (sum(x) and sum(x*x) of one tensor: one read of x).
+class StampedFusedReduction {
+   public:
+    StampedFusedReduction(ReductionLaunchPlan plan, std::vector<Tensor> inputs, std::vector<std::string> scalarNames, std::vector<Tensor> outputs,
+                          std::optional<Tensor> workspace, uint64_t flops)
+        : plan(std::move(plan)), inputs(std::move(inputs)), scalarNames(std::move(scalarNames)), outputs(std::move(outputs)),
+          workspace(std::move(workspace)), flops(flops) {}
+    void runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const;
+    const std::vector<Tensor>& getOutputTensors() const { return outputs; }
+    const std::vector<std::string>& runtimeScalarNames() const { return scalarNames; }
+    uint64_t flopCount() const { return flops; }
+    const std::string& getDescription() const { return plan.variant; }
+    const ReductionLaunchPlan& getLaunchPlan() const { return plan; }
+
+   private:
+    ReductionLaunchPlan plan;
+    std::vector<Tensor> inputs;
+    std::vector<std::string> scalarNames;
+    std::vector<Tensor> outputs;
+    std::optional<Tensor> workspace;
+    uint64_t flops;
+};
+
 struct StampedExecutionStage {
-    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy };
+    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction };
     static std::string kindToString(Kind kind) {
         switch (kind) {
             case Kind::FusedKernel:
@@ -102,6 +127,8 @@ struct StampedExecutionStage {
                 return "FusedRowKernel";
             case Kind::Copy:
                 return "Copy";
+            case Kind::FusedReduction:
+                return "FusedReduction";
         }
         return "<unknown>";
     }
@@ -112,6 +139,7 @@ struct StampedExecutionStage {
     std::shared_ptr<StampedEquation> kernel;
     std::shared_ptr<StampedReduction> reduction;
     std::shared_ptr<StampedArgMinMax> arg_minmax;
+    std::shared_ptr<StampedFusedReduction> fused_reduction;
     // Kind::Copy: a named output that is only a view of an input is copied into the caller's tensor
     Tensor copySource, copyDestination;
 

@@ -115,6 +115,7 @@ int thor_stamped_arg_reduction_run(thor_stamped_arg_reduction_t r);
 thor_tensor_t thor_stamped_arg_reduction_value_output(thor_stamped_arg_reduction_t r); /* NULL when not produced */
 thor_tensor_t thor_stamped_arg_reduction_index_output(thor_stamped_arg_reduction_t r);
 int thor_stamped_arg_reduction_path(thor_stamped_arg_reduction_t r);
+int thor_stamped_arg_reduction_variant(thor_stamped_arg_reduction_t r, char* buffer, size_t capacity);
 
 /* ---- Expression (Utilities/Expression/Expression.h:516-1075) ------------------------------------------------------------- */
 /* dtype arguments: a DataType code, or -1 for "not specified" */

@@ -183,6 +183,10 @@ struct ValueAcc {
         r.v = __shfl_xor(v, mask, kWave);
         return r;
     }
+    // A partial of `slots` accumulators is one float array of that length.
+    __device__ __forceinline__ static u64 partialBytes(u64 slots) { return ((slots * 4 + 7) / 8) * 8; }
+    __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64) const { static_cast<float*>(partials)[slot] = v; }
+    __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64) { v = static_cast<const float*>(partials)[slot]; }
 };
 
 // Candidate {value, index}: NaN beats every number, equal values (and two NaNs) keep the lower index.  The empty
@@ -227,6 +231,16 @@ struct ArgAcc {
             r.i = (IndexT)__shfl_xor((u32)i, mask, kWave);
         }
         return r;
+    }
+    // A partial of `slots` candidates is a float array followed by an IndexT array of the same length.
+    __device__ __forceinline__ static u64 partialBytes(u64 slots) { return ((slots * 4 + 7) / 8) * 8 + slots * sizeof(IndexT); }
+    __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64 slots) const {
+        static_cast<float*>(partials)[slot] = v;
+        reinterpret_cast<IndexT*>(static_cast<char*>(partials) + ((slots * 4 + 7) / 8) * 8)[slot] = i;
+    }
+    __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64 slots) {
+        v = static_cast<const float*>(partials)[slot];
+        i = reinterpret_cast<const IndexT*>(static_cast<const char*>(partials) + ((slots * 4 + 7) / 8) * 8)[slot];
     }
 };
 

@@ -2,13 +2,16 @@
 // prelude at run-time compilation).  They replace cub::DeviceReduce / DeviceSegmentedReduce and the reference's tiled
 // kernels (Utilities/TensorOperations/Cub/CubReductionOperation.cuh:2482-3054, CubArgReductionOperation.cuh:1054-1186).
 //
-// Cfg provides
-//   In, Out                       storage types of the input and of the value output
-//   Acc                           ValueAcc<Op> or ArgAcc<IS_MAX, IndexT>
+// One kernel may reduce several values at once from several tensors of the same layout: the generated Cfg describes
+// what is read at an element offset, how the loaded words turn into the values that are accumulated (an elementwise
+// prologue evaluated in registers), and where the results go.  Cfg provides
+//   Sources                       the tensors (and by-value scalars) the prologue reads
+//   Loaded                        the words loaded for one vector position: Cfg::load(sources, elementOffset, loaded)
+//   Acc                           ValueAcc<Op>, ArgAcc<IS_MAX, IndexT> or a generated struct of several ValueAcc members with
+//                                 the same protocol (reset, merge, shuffleXor, storePartial, loadPartial, partialBytes)
+//   accumulateOne(acc, loaded, sources, k, index)   evaluates element k of a loaded vector and adds it under `index`
+//   Outputs, store(acc, outIndex, outputs, scale)   finalises (mean divide, L2 square root), scales, converts, stores
 //   IndexT                        u32 or u64: type of element offsets and of arg indices inside the kernel
-//   OutIndex                      u32 or u64: storage type of the arg index output
-//   kIsArg, kWriteValue, kWriteIndex
-//   kFinalize, kDivisor           0 none / 1 divide by kDivisor / 2 square root
 //   kVec                          elements per vector load (all shapes and base addresses are multiples of it)
 //   kThreads                      threads per block
 // plus the geometry constants each kernel names below.  Shapes are compile-time constants: trip counts are known, loops
@@ -16,46 +19,6 @@
 #pragma once
 
 namespace thor {
-
-template <typename Cfg>
-__device__ __forceinline__ void loadAsFloat(const typename Cfg::In* p, float (&x)[Cfg::kVec]) {
-    Pack<typename Cfg::In, Cfg::kVec> pack;
-    pack.loadStream(p);
-#pragma unroll
-    for (int k = 0; k < Cfg::kVec; ++k) x[k] = toFloat(pack.v[k]);
-}
-
-template <typename Cfg>
-__device__ __forceinline__ void storeResult(const typename Cfg::Acc& acc, u64 outIndex, void* valueOut, void* indexOut, float scale) {
-    if constexpr (Cfg::kIsArg) {
-        if (Cfg::kWriteValue) static_cast<typename Cfg::Out*>(valueOut)[outIndex] = fromFloat<typename Cfg::Out>(acc.v);
-        if (Cfg::kWriteIndex) static_cast<typename Cfg::OutIndex*>(indexOut)[outIndex] = (typename Cfg::OutIndex)acc.i;
-    } else {
-        static_cast<typename Cfg::Out*>(valueOut)[outIndex] =
-            fromFloat<typename Cfg::Out>(finalizeValue<Cfg::kFinalize>(acc.v, Cfg::kDivisor, scale));
-    }
-}
-
-// Partials live in a float array followed (arg reductions only) by an IndexT array of the same length.
-template <typename Cfg>
-__device__ __forceinline__ void storePartial(const typename Cfg::Acc& acc, void* partials, u64 slot, u64 slots) {
-    static_cast<float*>(partials)[slot] = acc.v;
-    if constexpr (Cfg::kIsArg) {
-        typename Cfg::IndexT* ip = reinterpret_cast<typename Cfg::IndexT*>(static_cast<char*>(partials) + ((slots * 4 + 7) / 8) * 8);
-        ip[slot] = acc.i;
-    }
-}
-template <typename Cfg>
-__device__ __forceinline__ typename Cfg::Acc loadPartial(const void* partials, u64 slot, u64 slots) {
-    typename Cfg::Acc acc;
-    acc.v = static_cast<const float*>(partials)[slot];
-    if constexpr (Cfg::kIsArg) {
-        const typename Cfg::IndexT* ip =
-            reinterpret_cast<const typename Cfg::IndexT*>(static_cast<const char*>(partials) + ((slots * 4 + 7) / 8) * 8);
-        acc.i = ip[slot];
-    }
-    return acc;
-}
 
 // ---- whole tensor -> one value ------------------------------------------------------------------------------------------
 // Cfg: kN (elements), kUnroll (vectors in flight per thread), kBlocks (grid size).
@@ -65,7 +28,7 @@ __device__ __forceinline__ typename Cfg::Acc loadPartial(const void* partials, u
 // a device-scope release per block has to write back a non-coherent per-XCD L2, and 16 384 tickets serialise on one
 // address.  Two launches cost a few microseconds.
 template <typename Cfg>
-__device__ __forceinline__ void reduceAll(const typename Cfg::In* in, void* valueOut, void* indexOut, void* partials, float scale) {
+__device__ __forceinline__ void reduceAll(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* partials, float scale) {
     typedef typename Cfg::IndexT IndexT;
     typedef typename Cfg::Acc Acc;
     constexpr IndexT kVectors = (IndexT)(Cfg::kN / Cfg::kVec);
@@ -74,43 +37,47 @@ __device__ __forceinline__ void reduceAll(const typename Cfg::In* in, void* valu
     Acc acc;
     acc.reset();
     for (IndexT base = (IndexT)blockIdx.x * kChunk; base < kVectors; base += (IndexT)Cfg::kBlocks * kChunk) {
-        float x[Cfg::kUnroll][Cfg::kVec];
+        typename Cfg::Loaded x[Cfg::kUnroll];
         bool live[Cfg::kUnroll];
 #pragma unroll
         for (int u = 0; u < Cfg::kUnroll; ++u) {
             const IndexT v = base + (IndexT)u * Cfg::kThreads + threadIdx.x;
             live[u] = v < kVectors;
-            if (live[u]) loadAsFloat<Cfg>(in + v * Cfg::kVec, x[u]);
+            if (live[u]) Cfg::load(src, (u64)v * Cfg::kVec, x[u]);
         }
 #pragma unroll
         for (int u = 0; u < Cfg::kUnroll; ++u) {
             if (live[u]) {
                 const IndexT v = base + (IndexT)u * Cfg::kThreads + threadIdx.x;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) acc.add(x[u][k], v * Cfg::kVec + k);
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, k, (IndexT)(v * Cfg::kVec + k));
             }
         }
     }
     blockReduce<Cfg::kThreads, false>(acc, scratch);
     if (threadIdx.x == 0) {
         if (Cfg::kBlocks == 1) {
-            storeResult<Cfg>(acc, 0, valueOut, indexOut, scale);
+            Cfg::store(acc, 0, out, scale);
         } else {
-            storePartial<Cfg>(acc, partials, blockIdx.x, Cfg::kBlocks);
+            acc.storePartial(partials, blockIdx.x, Cfg::kBlocks);
         }
     }
 }
 
 // One block of kFinishThreads threads folds the kBlocks partials of reduceAll.
 template <typename Cfg>
-__device__ __forceinline__ void finishAll(const void* partials, void* valueOut, void* indexOut, float scale) {
+__device__ __forceinline__ void finishAll(const void* partials, const typename Cfg::Outputs& out, float scale) {
     typedef typename Cfg::Acc Acc;
     __shared__ Acc scratch[Cfg::kFinishThreads / kWave];
     Acc total;
     total.reset();
-    for (u32 b = threadIdx.x; b < (u32)Cfg::kBlocks; b += Cfg::kFinishThreads) total.merge(loadPartial<Cfg>(partials, b, Cfg::kBlocks));
+    for (u32 b = threadIdx.x; b < (u32)Cfg::kBlocks; b += Cfg::kFinishThreads) {
+        Acc part;
+        part.loadPartial(partials, b, Cfg::kBlocks);
+        total.merge(part);
+    }
     blockReduce<Cfg::kFinishThreads, false>(total, scratch);
-    if (threadIdx.x == 0) storeResult<Cfg>(total, 0, valueOut, indexOut, scale);
+    if (threadIdx.x == 0) Cfg::store(total, 0, out, scale);
 }
 
 // ---- contiguous rows: [kOuter, kR] -> [kOuter] ----------------------------------------------------------------------------
@@ -118,7 +85,7 @@ __device__ __forceinline__ void finishAll(const void* partials, void* valueOut, 
 // and kThreads == kThreadsPerRow), kSplit (row segments; 1 = whole row).  With kSplit > 1 the block at (x = row,
 // y = segment) writes a partial and finishPartials folds them.
 template <typename Cfg>
-__device__ __forceinline__ void reduceRows(const typename Cfg::In* in, void* valueOut, void* indexOut, void* partials, float scale) {
+__device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* partials, float scale) {
     typedef typename Cfg::IndexT IndexT;
     typedef typename Cfg::Acc Acc;
     constexpr int TPR = Cfg::kThreadsPerRow;
@@ -141,26 +108,26 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::In* in, void* val
     const u64 vBegin = segment * kVectorsPerSegment;
     const u64 vEnd = (vBegin + kVectorsPerSegment < kVectorsPerRow) ? vBegin + kVectorsPerSegment : kVectorsPerRow;
     const bool rowLive = row < Cfg::kOuter;
-    const typename Cfg::In* rowPtr = in + (rowLive ? row : 0) * Cfg::kR;
+    const u64 rowBase = (rowLive ? row : 0) * Cfg::kR;
 
     Acc acc;
     acc.reset();
     constexpr int kBatch = kIters >= 8 ? 8 : (int)(kIters > 0 ? kIters : 1);
     for (u64 it = 0; it < kIters; it += kBatch) {
-        float x[kBatch][Cfg::kVec];
+        typename Cfg::Loaded x[kBatch];
         bool live[kBatch];
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const u64 v = vBegin + (it + u) * TPR + lane;
             live[u] = rowLive && v < vEnd;
-            if (live[u]) loadAsFloat<Cfg>(rowPtr + v * Cfg::kVec, x[u]);
+            if (live[u]) Cfg::load(src, rowBase + v * Cfg::kVec, x[u]);
         }
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             if (live[u]) {
                 const u64 v = vBegin + (it + u) * TPR + lane;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) acc.add(x[u][k], (IndexT)(v * Cfg::kVec + k));
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, k, (IndexT)(v * Cfg::kVec + k));
             }
         }
     }
@@ -172,55 +139,83 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::In* in, void* val
     }
     if (lane == 0 && rowLive) {
         if (Cfg::kSplit > 1) {
-            storePartial<Cfg>(acc, partials, row * Cfg::kSplit + segment, Cfg::kOuter * Cfg::kSplit);
+            acc.storePartial(partials, row * Cfg::kSplit + segment, Cfg::kOuter * Cfg::kSplit);
         } else {
-            storeResult<Cfg>(acc, row, valueOut, indexOut, scale);
+            Cfg::store(acc, row, out, scale);
         }
     }
 }
 
 // ---- middle axis: [kOuter, kR, kInner] -> [kOuter, kInner] ------------------------------------------------------------------
-// One thread owns kVec adjacent inner positions and walks its share of the kR rows; adjacent threads read adjacent
-// memory.  Cfg: kOuter, kR, kInner, kSplit (shares of kR, grid y), kOutOuterStride / kOutInnerStride (output layout).
+// A block is kLanesX columns wide (a column = kVec adjacent inner positions; adjacent lanes read adjacent memory) and
+// kThreads / kLanesX row groups deep: row group g of share s walks rows rBegin + g, rBegin + g + groups, ...; the groups
+// are then folded through LDS, so the depth adds parallelism without adding partials.  Cfg: kOuter, kR, kInner,
+// kLanesX (power of two <= 64), kBatch (rows in flight per thread), kSplit (shares of kR, grid y),
+// kOutOuterStride / kOutInnerStride (output layout).
 template <typename Cfg>
-__device__ __forceinline__ void reduceColumns(const typename Cfg::In* in, void* valueOut, void* indexOut, void* partials, float scale) {
+__device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* partials, float scale) {
     typedef typename Cfg::IndexT IndexT;
     typedef typename Cfg::Acc Acc;
     constexpr u64 kInnerVectors = Cfg::kInner / Cfg::kVec;
     constexpr u64 kColumns = Cfg::kOuter * kInnerVectors;
     constexpr u64 kRowsPerShare = (Cfg::kR + Cfg::kSplit - 1) / Cfg::kSplit;
-    const u64 column = (u64)blockIdx.x * Cfg::kThreads + threadIdx.x;
-    if (column >= kColumns) return;
-    const u64 outer = column / kInnerVectors, iv = column % kInnerVectors;
+    constexpr int kGroups = Cfg::kThreads / Cfg::kLanesX;
+    constexpr int kBatch = Cfg::kBatch;
+    const int lx = threadIdx.x % Cfg::kLanesX, group = threadIdx.x / Cfg::kLanesX;
+    const u64 column = (u64)blockIdx.x * Cfg::kLanesX + lx;
+    const bool columnLive = column < kColumns;
+    const u64 safeColumn = columnLive ? column : 0;
+    const u64 outer = safeColumn / kInnerVectors, iv = safeColumn % kInnerVectors;
     const u64 share = Cfg::kSplit > 1 ? blockIdx.y : 0;
     const u64 rBegin = share * kRowsPerShare;
     const u64 rEnd = (rBegin + kRowsPerShare < Cfg::kR) ? rBegin + kRowsPerShare : Cfg::kR;
-    const typename Cfg::In* base = in + outer * Cfg::kR * Cfg::kInner + iv * Cfg::kVec;
+    const u64 base = outer * Cfg::kR * Cfg::kInner + iv * Cfg::kVec;
 
     Acc acc[Cfg::kVec];
 #pragma unroll
     for (int k = 0; k < Cfg::kVec; ++k) acc[k].reset();
-    constexpr int kBatch = 4;
-    for (u64 r = rBegin; r < rEnd; r += kBatch) {
-        float x[kBatch][Cfg::kVec];
+    for (u64 r0 = rBegin + group; r0 < rEnd; r0 += (u64)kGroups * kBatch) {
+        typename Cfg::Loaded x[kBatch];
+        bool live[kBatch];
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u)
-            if (r + u < rEnd) loadAsFloat<Cfg>(base + (r + u) * Cfg::kInner, x[u]);
+        for (int u = 0; u < kBatch; ++u) {
+            const u64 r = r0 + (u64)u * kGroups;
+            live[u] = columnLive && r < rEnd;
+            if (live[u]) Cfg::load(src, base + r * Cfg::kInner, x[u]);
+        }
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u)
-            if (r + u < rEnd) {
+        for (int u = 0; u < kBatch; ++u) {
+            if (live[u]) {
+                const u64 r = r0 + (u64)u * kGroups;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) acc[k].add(x[u][k], (IndexT)(r + u));
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, k, (IndexT)r);
             }
+        }
     }
+    if (kGroups > 1) {
+        // fold the row groups: group g > 0 parks its accumulators, group 0 merges them in group order
+        __shared__ Acc parked[(kGroups > 1 ? kGroups - 1 : 1) * Cfg::kLanesX * Cfg::kVec];
+        if (group > 0) {
+#pragma unroll
+            for (int k = 0; k < Cfg::kVec; ++k) parked[((group - 1) * Cfg::kLanesX + lx) * Cfg::kVec + k] = acc[k];
+        }
+        __syncthreads();
+        if (group == 0) {
+            for (int g = 1; g < kGroups; ++g) {
+#pragma unroll
+                for (int k = 0; k < Cfg::kVec; ++k) acc[k].merge(parked[((g - 1) * Cfg::kLanesX + lx) * Cfg::kVec + k]);
+            }
+        }
+    }
+    if (group != 0 || !columnLive) return;
 #pragma unroll
     for (int k = 0; k < Cfg::kVec; ++k) {
         const u64 inner = iv * Cfg::kVec + k;
         if (Cfg::kSplit > 1) {
             const u64 logical = outer * Cfg::kInner + inner;
-            storePartial<Cfg>(acc[k], partials, logical * Cfg::kSplit + share, Cfg::kOuter * Cfg::kInner * Cfg::kSplit);
+            acc[k].storePartial(partials, logical * Cfg::kSplit + share, Cfg::kOuter * Cfg::kInner * Cfg::kSplit);
         } else {
-            storeResult<Cfg>(acc[k], outer * Cfg::kOutOuterStride + inner * Cfg::kOutInnerStride, valueOut, indexOut, scale);
+            Cfg::store(acc[k], outer * Cfg::kOutOuterStride + inner * Cfg::kOutInnerStride, out, scale);
         }
     }
 }
@@ -230,7 +225,7 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::In* in, void* 
 // reduced axes (the innermost reduced axis is counted in vectors of kVec when it is contiguous) -- kOutputs, kReduction
 // (vector count of the reduction domain), kSplit (shares of the reduction domain, grid y; outputs on grid x).
 template <typename Cfg>
-__device__ __forceinline__ void reduceStrided(const typename Cfg::In* in, void* valueOut, void* indexOut, void* partials, float scale) {
+__device__ __forceinline__ void reduceStrided(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* partials, float scale) {
     typedef typename Cfg::IndexT IndexT;
     typedef typename Cfg::Acc Acc;
     constexpr u64 kPerShare = (Cfg::kReduction + Cfg::kSplit - 1) / Cfg::kSplit;
@@ -238,36 +233,36 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::In* in, void* 
     const u64 share = blockIdx.y;
     const u64 rBegin = share * kPerShare;
     const u64 rEnd = (rBegin + kPerShare < Cfg::kReduction) ? rBegin + kPerShare : Cfg::kReduction;
-    const typename Cfg::In* base = in + Cfg::keptOffset(output);
+    const u64 base = Cfg::keptOffset(output);
     __shared__ Acc scratch[Cfg::kThreads / kWave];
 
     Acc acc;
     acc.reset();
     constexpr int kBatch = 4;
     for (u64 r0 = rBegin + threadIdx.x; r0 < rEnd; r0 += (u64)Cfg::kThreads * kBatch) {
-        float x[kBatch][Cfg::kVec];
+        typename Cfg::Loaded x[kBatch];
         bool live[kBatch];
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const u64 r = r0 + (u64)u * Cfg::kThreads;
             live[u] = r < rEnd;
-            if (live[u]) loadAsFloat<Cfg>(base + Cfg::reducedOffset(r), x[u]);
+            if (live[u]) Cfg::load(src, base + Cfg::reducedOffset(r), x[u]);
         }
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             if (live[u]) {
                 const u64 r = r0 + (u64)u * Cfg::kThreads;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) acc.add(x[u][k], (IndexT)(r * Cfg::kVec + k));
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, k, (IndexT)(r * Cfg::kVec + k));
             }
         }
     }
     blockReduce<Cfg::kThreads, false>(acc, scratch);
     if (threadIdx.x == 0) {
         if (Cfg::kSplit > 1) {
-            storePartial<Cfg>(acc, partials, output * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
+            acc.storePartial(partials, output * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
         } else {
-            storeResult<Cfg>(acc, output, valueOut, indexOut, scale);
+            Cfg::store(acc, output, out, scale);
         }
     }
 }
@@ -276,7 +271,7 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::In* in, void* 
 // One wavefront per output.  Cfg: kOutputs, kSplit, kFinishOuterStride/kFinishInnerStride/kFinishInner (output layout:
 // logical index o = outer * kFinishInner + inner is stored at outer * kFinishOuterStride + inner * kFinishInnerStride).
 template <typename Cfg>
-__device__ __forceinline__ void finishPartials(const void* partials, void* valueOut, void* indexOut, float scale) {
+__device__ __forceinline__ void finishPartials(const void* partials, const typename Cfg::Outputs& out, float scale) {
     typedef typename Cfg::Acc Acc;
     const u64 output = ((u64)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
     const int lane = threadIdx.x % kWave;
@@ -284,12 +279,16 @@ __device__ __forceinline__ void finishPartials(const void* partials, void* value
     Acc acc;
     acc.reset();
     if (live) {
-        for (u64 s = lane; s < Cfg::kSplit; s += kWave) acc.merge(loadPartial<Cfg>(partials, output * Cfg::kSplit + s, Cfg::kOutputs * Cfg::kSplit));
+        for (u64 s = lane; s < Cfg::kSplit; s += kWave) {
+            Acc part;
+            part.loadPartial(partials, output * Cfg::kSplit + s, Cfg::kOutputs * Cfg::kSplit);
+            acc.merge(part);
+        }
     }
     groupReduce<kWave>(acc);
     if (live && lane == 0) {
         const u64 outer = output / Cfg::kFinishInner, inner = output % Cfg::kFinishInner;
-        storeResult<Cfg>(acc, outer * Cfg::kFinishOuterStride + inner * Cfg::kFinishInnerStride, valueOut, indexOut, scale);
+        Cfg::store(acc, outer * Cfg::kFinishOuterStride + inner * Cfg::kFinishInnerStride, out, scale);
     }
 }
 

@@ -6,6 +6,7 @@
 #include <atomic>
 #include <stdexcept>
 #include <vector>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
@@ -56,11 +57,46 @@ void CompiledKernel::launch(uint32_t gridX, uint32_t gridY, uint32_t gridZ, uint
 
 uint64_t compiledKernelCount() { return compileCount.load(); }
 
+namespace {
+// Every generated kernel gets a name of its own, <base>_<8 hex digits of a hash of the source>, so that profiles tell the
+// kernels of different shapes apart.  All extern "C" kernels of one source share the tag.
+std::string sourceTag(const std::string& source) {
+    uint32_t h = 2166136261u;  // FNV-1a
+    for (unsigned char ch : source) {
+        h ^= ch;
+        h *= 16777619u;
+    }
+    char text[16];
+    std::snprintf(text, sizeof text, "%08x", h);
+    return text;
+}
+
+std::string withTaggedKernelNames(const std::string& source, const std::string& tag) {
+    static const std::string marker = "extern \"C\" __global__";
+    std::string out;
+    size_t pos = 0;
+    while (true) {
+        const size_t at = source.find(marker, pos);
+        if (at == std::string::npos) break;
+        const size_t paren = source.find('(', source.find(" void ", at));
+        if (paren == std::string::npos) break;
+        out.append(source, pos, paren - pos);
+        out += "_" + tag;
+        pos = paren;
+    }
+    out.append(source, pos, std::string::npos);
+    return out;
+}
+}  // namespace
+
 std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract) {
     const std::string moduleKey = std::to_string(deviceNum) + (fastContract ? "|contract|" : "|off|") + source;
     const std::string kernelKey = kernelName + "|" + moduleKey;
     return kernelCache().getOrCreate(kernelKey, [&] {
         ScopedGpu scoped(deviceNum);
+        const std::string tag = sourceTag(source);
+        const std::string taggedName = kernelName + "_" + tag;
+        const std::string taggedSource = withTaggedKernelNames(source, tag);
         std::shared_ptr<LoadedModule> loaded = moduleCache().getOrCreate(moduleKey, [&] {
             const std::string arch = archOf(deviceNum);
             // "fast" contraction would also rewrite the error-compensated sequences inside the device math library (expf drops
@@ -72,10 +108,10 @@ std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const s
             size_t codeSize = 0;
             std::vector<char> log(16384, 0);
             if (const char* dump = std::getenv("THOR_DUMP_KERNEL_SOURCE")) {
-                std::ofstream out(std::string(dump) + "/" + kernelName + "_" + std::to_string(compileCount.load()) + ".hip");
-                out << source;
+                std::ofstream out(std::string(dump) + "/" + taggedName + ".hip");
+                out << taggedSource;
             }
-            const int rc = thorhip_compile(source.c_str(), (kernelName + ".hip").c_str(), arch.c_str(), options, numOptions, &code, &codeSize,
+            const int rc = thorhip_compile(taggedSource.c_str(), (taggedName + ".hip").c_str(), arch.c_str(), options, numOptions, &code, &codeSize,
                                            log.data(), log.size());
             if (rc != 0) {
                 throw std::runtime_error("Run-time compilation of kernel '" + kernelName + "' failed: " + thorhip_last_error());
@@ -91,9 +127,9 @@ std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const s
         auto kernel = std::make_shared<CompiledKernel>();
         kernel->module = loaded;
         kernel->deviceNum = deviceNum;
-        kernel->kernelName = kernelName;
-        kernel->source = source;
-        THOR_HIP_CHECK(thorhip_module_get_function(&kernel->function, loaded->module, kernelName.c_str()));
+        kernel->kernelName = taggedName;
+        kernel->source = taggedSource;
+        THOR_HIP_CHECK(thorhip_module_get_function(&kernel->function, loaded->module, taggedName.c_str()));
         (void)thorhip_function_get_attributes(kernel->function, &kernel->numRegisters, &kernel->staticLdsBytes, nullptr);
         return kernel;
     });

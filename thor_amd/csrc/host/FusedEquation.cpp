@@ -267,9 +267,14 @@ CubReductionOp valueReductionOp(ExprOp op) {
     throw std::runtime_error("Not a value reduction op.");
 }
 
-bool rowFusionEnabled() {
-    const char* env = std::getenv("THOR_DISABLE_ROW_FUSION");
-    return !(env && env[0] == '1');
+// THOR_DISABLE_ROW_FUSION=1 (or THOR_DISABLE_STAGE_FUSION=1) selects the staged plan: one stage per reduction and per
+// elementwise group, like the reference's lowering.
+bool stageFusionEnabled() {
+    for (const char* name : {"THOR_DISABLE_ROW_FUSION", "THOR_DISABLE_STAGE_FUSION"}) {
+        const char* env = std::getenv(name);
+        if (env && env[0] == '1') return false;
+    }
+    return true;
 }
 
 }  // namespace
@@ -511,17 +516,24 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     };
 
     std::vector<char> done(expr.nodes.size(), 0);
-    if (rowFusionEnabled() && !fusedKernelsOnly) {
+    const bool stageFusion = stageFusionEnabled() && !fusedKernelsOnly;
+    std::vector<uint8_t> roles(graph->role.size());
+    for (size_t i = 0; i < roles.size(); ++i) roles[i] = static_cast<uint8_t>(graph->role[i]);
+    RowFusionContext context{expr, graph->outputs, root_inputs, roles, dims, tensorOf, done, stages, stageOfNode, allocateFor, device_num};
+    if (stageFusion) {
         // Recognise chains of last-axis reductions and row-wise elementwise work over one [rows, R] input and emit them
         // as one kernel that keeps each row in registers.
-        std::vector<uint8_t> roles(graph->role.size());
-        for (size_t i = 0; i < roles.size(); ++i) roles[i] = static_cast<uint8_t>(graph->role[i]);
-        RowFusionContext context{expr, graph->outputs, root_inputs, roles, dims, tensorOf, done, stages, stageOfNode, allocateFor, device_num};
         tryRowFusion(context);
         resolveViewsUpTo();
     }
 
     for (uint32_t level = 0; level <= maxLevel; ++level) {
+        if (stageFusion) {
+            // Reductions over one shape and axes whose inputs exist by now (or are elementwise functions of such tensors
+            // that nothing else needs) run as one pass.
+            tryReductionFusion(context);
+            resolveViewsUpTo();
+        }
         // fused values of this level, grouped by output shape so that one kernel shares the loads
         std::map<std::vector<uint64_t>, std::vector<uint32_t>> fusedGroups;
         for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
@@ -624,7 +636,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             stage.dependency_stage_indices = dependenciesOf(sources);
             stage.kernel = std::make_shared<StampedEquation>(kernel, inputTensors, outputTensors, scalarArgs, inputArgIndex, outputArgIndex, next,
                                                              emitted.passNumel, emitted.numel, emitted.numelIs64, emitted.gridX, emitted.threads,
-                                                             emitted.flopsPerElement * emitted.numel, emitted.description);
+                                                             emitted.flopsPerElement * emitted.numel, emitted.description + " [" + kernel->kernelName + "]");
             for (uint32_t node : nodes) {
                 stageOfNode[node] = static_cast<int>(stages.size());
                 done[node] = 1;

@@ -58,13 +58,20 @@ void collapseAxes(std::vector<uint64_t>& dims, std::vector<uint64_t>& strides) {
     strides = s;
 }
 
+const char* valueAccumulatorType(CubReductionOp op, int& finalize);
+
 const char* accumulatorType(const ReductionKernelRequest& r, bool indexIs64, int& finalize) {
     finalize = 0;
     if (r.isArg) {
         if (r.argOp == CubArgReductionOp::ArgMax) return indexIs64 ? "ArgAcc<true, u64>" : "ArgAcc<true, u32>";
         return indexIs64 ? "ArgAcc<false, u64>" : "ArgAcc<false, u32>";
     }
-    switch (r.valueOp) {
+    return valueAccumulatorType(r.valueOp, finalize);
+}
+
+const char* valueAccumulatorType(CubReductionOp op, int& finalize) {
+    finalize = 0;
+    switch (op) {
         case CubReductionOp::Sum:
             return "ValueAcc<SumOp>";
         case CubReductionOp::Mean:
@@ -140,7 +147,7 @@ std::string ReductionShape::describe() const {
             out << "rows(lanes_per_row=" << threadsPerRow << ",split=" << split;
             break;
         case Kernel::Columns:
-            out << "columns(split=" << split;
+            out << "columns(lanes_x=" << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
             break;
         case Kernel::Strided:
             out << "strided(kept_rank=" << keptDims.size() << ",reduced_rank=" << reducedDims.size() << ",split=" << split;
@@ -152,12 +159,18 @@ std::string ReductionShape::describe() const {
 
 ReductionShape planReductionShape(const ReductionKernelRequest& request) {
     const CubReductionGeometry& g = request.geometry;
-    const uint32_t elementBytes = dataTypeSizeInBytes(request.inputDType);
+    uint32_t elementBytes = dataTypeSizeInBytes(request.inputDType);
+    if (!request.values.empty()) {
+        elementBytes = 1;
+        for (const ReductionKernelRequest::Source& source : request.sources)
+            if (!source.scalar) elementBytes = std::max(elementBytes, dataTypeSizeInBytes(source.storage));
+    }
+    const uint64_t accumulators = request.values.empty() ? 1 : request.values.size();
     ReductionShape shape;
     shape.indexIs64 = g.input_elements >= (1ull << 31) || g.reduction_size >= (1ull << 31);
 
     auto finishSplit = [&](uint64_t outputs) {
-        if (shape.split > 1) shape.workspaceBytes = partialBytes(outputs * shape.split, request.isArg, shape.indexIs64);
+        if (shape.split > 1) shape.workspaceBytes = accumulators * partialBytes(outputs * shape.split, request.isArg, shape.indexIs64);
     };
 
     if (g.path == CubReductionPath::DeviceTransformReduce && !g.device_transform_uses_affine_stride) {
@@ -168,7 +181,7 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
         const uint64_t vectors = g.input_elements / shape.vec;
         shape.blocks = std::min<uint64_t>(std::max<uint64_t>(ceilDiv(vectors, 256ull * shape.unroll), 1), 65536);
         shape.gridX = static_cast<uint32_t>(shape.blocks);
-        if (shape.blocks > 1) shape.workspaceBytes = partialBytes(shape.blocks, request.isArg, shape.indexIs64);
+        if (shape.blocks > 1) shape.workspaceBytes = accumulators * partialBytes(shape.blocks, request.isArg, shape.indexIs64);
         return shape;
     }
 
@@ -196,12 +209,20 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
         shape.kernel = ReductionShape::Kernel::Columns;
         shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.inner_size});
         shape.threads = 256;
+        shape.unroll = 8;  // rows in flight per thread
         const uint64_t columns = g.outer_size * (g.inner_size / shape.vec);
-        if (columns < kTargetThreads && g.reduction_size >= 64) {
-            shape.split = std::min<uint64_t>({ceilDiv(kTargetThreads, columns), g.reduction_size / 16, kMaxGridY});
+        // a block is up to one wavefront of columns wide; the rest of its threads are row groups folded through LDS
+        shape.threadsPerRow = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(columns)));
+        const uint64_t groups = 256 / shape.threadsPerRow;
+        // enough threads to keep loads in flight on every CU, but at least 16 rows per thread and partials that stay small
+        // next to the input (measured on 8192 x 8192 fp32: 512 Ki threads reach 5.3 TB/s, 128 Ki threads 3.8 TB/s)
+        const uint64_t wantedThreads = 4 * kTargetThreads;
+        if (columns * groups < wantedThreads && g.reduction_size >= groups * 32) {
+            shape.split = std::min<uint64_t>({ceilDiv(wantedThreads, columns * groups), g.reduction_size / (groups * 16), kMaxGridY});
             if (shape.split < 2) shape.split = 1;
         }
-        shape.gridX = static_cast<uint32_t>(ceilDiv(columns, 256));
+        const uint64_t columnsNow = g.outer_size * (g.inner_size / shape.vec);
+        shape.gridX = static_cast<uint32_t>(ceilDiv(columnsNow, shape.threadsPerRow));
         shape.gridY = static_cast<uint32_t>(shape.split);
         finishSplit(g.output_elements);
         return shape;
@@ -254,25 +275,105 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
 
 std::string generateReductionSource(const ReductionKernelRequest& request, const ReductionShape& shape) {
     const CubReductionGeometry& g = request.geometry;
-    int finalize = 0;
-    const char* acc = accumulatorType(request, shape.indexIs64, finalize);
+    // the plain request is the fused form with one source and the value itself
+    std::vector<ReductionKernelRequest::Source> sources = request.sources;
+    std::vector<ReductionKernelRequest::Value> values = request.values;
+    std::string prologue = request.prologue;
+    if (values.empty()) {
+        sources = {{request.inputDType, false}};
+        values = {{request.valueOp, request.valueOutputDType, "x0"}};
+        prologue = "        const float x0 = toFloat(l.p0.v[k]);\n";
+    } else if (request.isArg) {
+        throw std::invalid_argument("Arg reductions cannot be fused with other reductions.");
+    }
+    const char* indexType = shape.indexIs64 ? "u64" : "u32";
+
     std::ostringstream s;
     s << thor_embed::kDevicePrelude << thor_embed::kReduceKernels;
     s << "namespace gen {\nusing namespace thor;\nstruct Cfg {\n";
-    s << "    typedef " << deviceTypeName(request.inputDType) << " In;\n";
-    s << "    typedef " << deviceTypeName(request.valueOutputDType) << " Out;\n";
-    s << "    typedef " << (shape.indexIs64 ? "u64" : "u32") << " IndexT;\n";
-    s << "    typedef " << (request.indexOutputDType == DataType::UINT64 ? "u64" : "u32") << " OutIndex;\n";
-    s << "    typedef " << acc << " Acc;\n";
-    s << "    static constexpr bool kIsArg = " << (request.isArg ? "true" : "false") << ";\n";
-    s << "    static constexpr bool kWriteValue = " << (request.writeValue ? "true" : "false") << ";\n";
-    s << "    static constexpr bool kWriteIndex = " << (request.writeIndex ? "true" : "false") << ";\n";
-    s << "    static constexpr int kFinalize = " << finalize << ";\n";
-    s << "    static constexpr float kDivisor = (float)" << g.reduction_size << "ull;\n";
+    s << "    typedef " << indexType << " IndexT;\n";
     s << "    static constexpr int kVec = " << shape.vec << ";\n";
     s << "    static constexpr int kThreads = " << shape.threads << ";\n";
     s << "    static constexpr u64 kSplit = " << shape.split << "ull;\n";
     s << "    static constexpr u64 kOutputs = " << g.output_elements << "ull;\n";
+    s << "    static constexpr float kDivisor = (float)" << g.reduction_size << "ull;\n";
+
+    // what the prologue reads
+    s << "    struct Sources {\n";
+    for (size_t i = 0; i < sources.size(); ++i) s << "        const " << deviceTypeName(sources[i].storage) << "* in" << i << ";\n";
+    for (uint32_t slot : request.scalarSlots) s << "        float s" << slot << ";\n";
+    s << "    };\n    struct Loaded {\n";
+    for (size_t i = 0; i < sources.size(); ++i) {
+        if (sources[i].scalar) {
+            s << "        " << deviceTypeName(sources[i].storage) << " z" << i << ";\n";
+        } else {
+            s << "        Pack<" << deviceTypeName(sources[i].storage) << ", kVec> p" << i << ";\n";
+        }
+    }
+    s << "    };\n";
+    s << "    static __device__ __forceinline__ void load(const Sources& s, u64 offset, Loaded& l) {\n";
+    for (size_t i = 0; i < sources.size(); ++i) {
+        if (sources[i].scalar) {
+            s << "        l.z" << i << " = s.in" << i << "[0];\n";
+        } else {
+            s << "        l.p" << i << ".loadStream(s.in" << i << " + offset);\n";
+        }
+    }
+    s << "        (void)offset;\n    }\n";
+
+    // accumulators
+    std::vector<int> finalize(values.size(), 0);
+    if (request.isArg) {
+        int f = 0;
+        s << "    typedef " << accumulatorType(request, shape.indexIs64, f) << " Acc;\n";
+    } else if (values.size() == 1) {
+        s << "    typedef " << valueAccumulatorType(values[0].op, finalize[0]) << " Acc;\n";
+    } else {
+        s << "    struct Acc {\n";
+        for (size_t j = 0; j < values.size(); ++j) s << "        " << valueAccumulatorType(values[j].op, finalize[j]) << " a" << j << ";\n";
+        s << "        __device__ __forceinline__ void reset() {";
+        for (size_t j = 0; j < values.size(); ++j) s << " a" << j << ".reset();";
+        s << " }\n        __device__ __forceinline__ void merge(const Acc& o) {";
+        for (size_t j = 0; j < values.size(); ++j) s << " a" << j << ".merge(o.a" << j << ");";
+        s << " }\n        __device__ __forceinline__ Acc shuffleXor(int mask) const {\n            Acc r;\n";
+        for (size_t j = 0; j < values.size(); ++j) s << "            r.a" << j << " = a" << j << ".shuffleXor(mask);\n";
+        s << "            return r;\n        }\n";
+        // partials: one float array per member, back to back
+        s << "        __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64 slots) const {\n"
+             "            char* base = static_cast<char*>(partials);\n            const u64 stride = ((slots * 4 + 7) / 8) * 8;\n";
+        for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".storePartial(base + " << j << " * stride, slot, slots);\n";
+        s << "        }\n        __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64 slots) {\n"
+             "            const char* base = static_cast<const char*>(partials);\n            const u64 stride = ((slots * 4 + 7) / 8) * 8;\n";
+        for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".loadPartial(base + " << j << " * stride, slot, slots);\n";
+        s << "        }\n    };\n";
+    }
+    s << "    static __device__ __forceinline__ void accumulateOne(Acc& acc, const Loaded& l, const Sources& s, int k, IndexT index) {\n";
+    s << prologue;
+    if (request.isArg || values.size() == 1) {
+        s << "        acc.add(" << values[0].expression << ", index);\n";
+    } else {
+        for (size_t j = 0; j < values.size(); ++j) s << "        acc.a" << j << ".add(" << values[j].expression << ", index);\n";
+    }
+    s << "        (void)l; (void)s; (void)k; (void)index;\n    }\n";
+
+    // results
+    s << "    struct Outputs {\n";
+    for (size_t j = 0; j < values.size(); ++j) s << "        " << deviceTypeName(values[j].outputDType) << "* out" << j << ";\n";
+    s << "        " << (request.indexOutputDType == DataType::UINT64 ? "u64" : "u32") << "* indexOut;\n    };\n";
+    s << "    static __device__ __forceinline__ void store(const Acc& acc, u64 outIndex, const Outputs& o, float scale) {\n";
+    if (request.isArg) {
+        if (request.writeValue) s << "        o.out0[outIndex] = fromFloat<" << deviceTypeName(values[0].outputDType) << ">(acc.v);\n";
+        if (request.writeIndex) s << "        o.indexOut[outIndex] = (" << (request.indexOutputDType == DataType::UINT64 ? "u64" : "u32") << ")acc.i;\n";
+        s << "        (void)scale;\n";
+    } else {
+        for (size_t j = 0; j < values.size(); ++j) {
+            const std::string member = values.size() == 1 ? "acc.v" : "acc.a" + std::to_string(j) + ".v";
+            s << "        o.out" << j << "[outIndex] = fromFloat<" << deviceTypeName(values[j].outputDType) << ">(finalizeValue<" << finalize[j] << ">("
+              << member << ", kDivisor, scale));\n";
+        }
+    }
+    s << "        (void)acc; (void)outIndex; (void)o;\n    }\n";
+
     const char* body = "";
     switch (shape.kernel) {
         case ReductionShape::Kernel::All:
@@ -280,13 +381,13 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             s << "    static constexpr int kUnroll = " << shape.unroll << ";\n";
             s << "    static constexpr u64 kBlocks = " << shape.blocks << "ull;\n";
             s << "    static constexpr int kFinishThreads = 1024;\n";
-            body = "thor::reduceAll<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
+            body = "thor::reduceAll<gen::Cfg>(src, out, partials, scale);";
             break;
         case ReductionShape::Kernel::Rows:
             s << "    static constexpr u64 kOuter = " << g.outer_size << "ull;\n";
             s << "    static constexpr u64 kR = " << g.reduction_size << "ull;\n";
             s << "    static constexpr int kThreadsPerRow = " << shape.threadsPerRow << ";\n";
-            body = "thor::reduceRows<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
+            body = "thor::reduceRows<gen::Cfg>(src, out, partials, scale);";
             break;
         case ReductionShape::Kernel::Columns:
             s << "    static constexpr u64 kOuter = " << g.outer_size << "ull;\n";
@@ -294,7 +395,9 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             s << "    static constexpr u64 kInner = " << g.inner_size << "ull;\n";
             s << "    static constexpr u64 kOutOuterStride = " << g.tiled_output_outer_stride << "ull;\n";
             s << "    static constexpr u64 kOutInnerStride = " << g.tiled_output_inner_stride << "ull;\n";
-            body = "thor::reduceColumns<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
+            s << "    static constexpr int kBatch = " << shape.unroll << ";\n";
+            s << "    static constexpr int kLanesX = " << shape.threadsPerRow << ";\n";
+            body = "thor::reduceColumns<gen::Cfg>(src, out, partials, scale);";
             break;
         case ReductionShape::Kernel::Strided: {
             std::vector<uint64_t> rd = shape.reducedDims, rs = shape.reducedStrides;
@@ -305,7 +408,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             s << "    static constexpr u64 kReduction = " << (g.reduction_size / shape.vec) << "ull;\n";
             s << offsetFunction("keptOffset", shape.keptDims, shape.keptStrides);
             s << offsetFunction("reducedOffset", rd, rs);
-            body = "thor::reduceStrided<gen::Cfg>(in, valueOut, indexOut, partials, scale);";
+            body = "thor::reduceStrided<gen::Cfg>(src, out, partials, scale);";
             break;
         }
     }
@@ -319,16 +422,27 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
              "    static constexpr u64 kFinishInnerStride = 0ull;\n";
     }
     s << "};\n}  // namespace gen\n";
-    s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads
-      << ") void thor_reduce_main(const gen::Cfg::In* in, void* valueOut, void* indexOut, void* partials, float scale) {\n"
-         "    (void)partials;\n    "
-      << body << "\n}\n";
-    if (shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1) {
-        s << "extern \"C\" __global__ __launch_bounds__(1024) void thor_reduce_finish(const void* partials, void* valueOut, void* indexOut, float "
-             "scale) {\n    thor::finishAll<gen::Cfg>(partials, valueOut, indexOut, scale);\n}\n";
-    } else if (shape.split > 1) {
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_reduce_finish(const void* partials, void* valueOut, void* indexOut, float "
-             "scale) {\n    thor::finishPartials<gen::Cfg>(partials, valueOut, indexOut, scale);\n}\n";
+
+    // kernel signatures: sources, runtime scalars, outputs, index output, partials, scale
+    std::ostringstream outputParams, outputInit;
+    for (size_t j = 0; j < values.size(); ++j) {
+        outputParams << deviceTypeName(values[j].outputDType) << "* out" << j << ", ";
+        outputInit << "out" << j << ", ";
+    }
+    outputParams << "void* indexOut";
+    outputInit << "static_cast<decltype(gen::Cfg::Outputs::indexOut)>(indexOut)";
+    s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads << ") void thor_reduce_main(";
+    for (size_t i = 0; i < sources.size(); ++i) s << "const " << deviceTypeName(sources[i].storage) << "* in" << i << ", ";
+    for (uint32_t slot : request.scalarSlots) s << "float s" << slot << ", ";
+    s << outputParams.str() << ", void* partials, float scale) {\n    const gen::Cfg::Sources src{";
+    for (size_t i = 0; i < sources.size(); ++i) s << (i ? ", " : "") << "in" << i;
+    for (uint32_t slot : request.scalarSlots) s << ", s" << slot;
+    s << "};\n    const gen::Cfg::Outputs out{" << outputInit.str() << "};\n    (void)partials;\n    " << body << "\n}\n";
+    const bool twoStageAll = shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1;
+    if (twoStageAll || shape.split > 1) {
+        s << "extern \"C\" __global__ __launch_bounds__(" << (twoStageAll ? 1024 : 256) << ") void thor_reduce_finish(const void* partials, "
+          << outputParams.str() << ", float scale) {\n    const gen::Cfg::Outputs out{" << outputInit.str() << "};\n    thor::"
+          << (twoStageAll ? "finishAll" : "finishPartials") << "<gen::Cfg>(partials, out, scale);\n}\n";
     }
     return s.str();
 }
@@ -352,7 +466,7 @@ ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request)
     plan.mainGridY = shape.gridY;
     plan.mainThreads = static_cast<uint32_t>(shape.threads);
     plan.workspaceBytes = shape.workspaceBytes;
-    plan.variant = shape.describe();
+    plan.variant = shape.describe() + " [" + plan.mainKernel->kernelName + "]";
     return plan;
 }
 

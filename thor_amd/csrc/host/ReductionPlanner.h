@@ -6,6 +6,7 @@
 
 #include <cstdint>
 #include <string>
+#include <vector>
 
 namespace ThorImplementation {
 
@@ -19,8 +20,26 @@ struct ReductionKernelRequest {
     bool writeValue = true;
     bool writeIndex = false;
     CubReductionGeometry geometry;
-    uint64_t inputAlignmentBytes = 256;  // largest power of two (capped at 256) dividing the input base address
+    uint64_t inputAlignmentBytes = 256;  // largest power of two (capped at 256) dividing every source base address
     int deviceNum = 0;
+
+    // ---- fused form: several value reductions over the same geometry, fed by an elementwise prologue ------------------
+    // When `values` is empty the request is the plain one above: one source of inputDType, the value itself reduced.
+    struct Source {
+        DataType storage = DataType::FP32;
+        bool scalar = false;  // a one-element tensor read at [0] instead of at the element offset
+    };
+    struct Value {
+        CubReductionOp op = CubReductionOp::Sum;
+        DataType outputDType = DataType::FP32;
+        std::string expression;  // fp32 C expression of the value to accumulate, in terms of the prologue's names
+    };
+    std::vector<Source> sources;         // kernel arguments in0, in1, ... ; vector sources share the reduction input's layout
+    std::vector<uint32_t> scalarSlots;   // runtime scalars passed by value as float s<slot>, after the sources
+    // Statements evaluated once per element before the values are accumulated.  Element k of vector source i is
+    // `l.p<i>.v[k]`, scalar source i is `l.z<i>`, runtime scalars are `s.s<slot>`.
+    std::string prologue;
+    std::vector<Value> values;           // outputs out0, out1, ... in this order
 };
 
 struct ReductionShape {

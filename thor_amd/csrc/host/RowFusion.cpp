@@ -676,7 +676,7 @@ void tryRowFusion(RowFusionContext& ctx) {
             if (st >= 0) stage.dependency_stage_indices.push_back(static_cast<uint32_t>(st));
         }
         stage.kernel = std::make_shared<StampedEquation>(kernel, inputs, outputs, scalarArgs, inputArgIndex, outputArgIndex, next, false,
-                                                         rg.rows * rg.R, false, em.gridX, em.threads, em.flops, em.description);
+                                                         rg.rows * rg.R, false, em.gridX, em.threads, em.flops, em.description + " [" + kernel->kernelName + "]");
         const int stageIndex = static_cast<int>(ctx.stages.size());
         for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
             if (!rg.member[i]) continue;

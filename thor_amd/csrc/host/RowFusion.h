@@ -30,4 +30,9 @@ struct RowFusionContext {
 // Appends FusedRowKernel stages for every group it recognises and marks the nodes they produce as done.
 void tryRowFusion(RowFusionContext& ctx);
 
+// Groups the remaining value reductions that run over the same shape and axes and whose inputs are tensors that already
+// exist (or elementwise functions of such tensors that nothing else needs) into FusedReduction stages: one pass over the
+// sources feeds every accumulator, and the elementwise work happens in registers instead of a materialised tensor.
+void tryReductionFusion(RowFusionContext& ctx);
+
 }  // namespace ThorImplementation

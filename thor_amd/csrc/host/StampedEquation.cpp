@@ -100,6 +100,47 @@ std::vector<uint64_t> StampedEquation::computeReductionOutputDims(const std::vec
     return squeezed;
 }
 
+void StampedFusedReduction::runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const {
+    if (!stream.isInitialized() || outputs.empty() || stream.getGpuNum() != static_cast<int>(outputs[0].getPlacement().getDeviceNum())) {
+        throw std::runtime_error("Stamped reduction must run on a stream of the GPU its tensors live on.");
+    }
+    // main kernel: sources, runtime scalars, outputs, index output (unused), partials, scale
+    std::vector<const void*> sourcePointers(inputs.size());
+    std::vector<float> scalarValues(scalarNames.size());
+    std::vector<void*> outputPointers(outputs.size());
+    void* indexOut = nullptr;
+    void* partials = workspace.has_value() ? const_cast<Tensor&>(workspace.value()).getMemPtr<char>() : nullptr;
+    float scale = 1.0f;
+    std::vector<void*> args;
+    for (size_t i = 0; i < inputs.size(); ++i) {
+        sourcePointers[i] = inputs[i].getMemPtr();
+        args.push_back(&sourcePointers[i]);
+    }
+    for (size_t i = 0; i < scalarNames.size(); ++i) {
+        auto it = runtime_scalars.find(scalarNames[i]);
+        if (it == runtime_scalars.end()) throw std::runtime_error("Missing runtime scalar input: " + scalarNames[i]);
+        scalarValues[i] = it->second;
+        args.push_back(&scalarValues[i]);
+    }
+    for (size_t i = 0; i < outputs.size(); ++i) {
+        outputPointers[i] = const_cast<Tensor&>(outputs[i]).getMemPtr();
+        args.push_back(&outputPointers[i]);
+    }
+    args.push_back(&indexOut);
+    args.push_back(&partials);
+    args.push_back(&scale);
+    ScopedGpu scoped(stream.getGpuNum());
+    plan.mainKernel->launch(plan.mainGridX, plan.mainGridY, 1, plan.mainThreads, stream.getStream(), args);
+    if (plan.finishKernel) {
+        const void* constPartials = partials;
+        std::vector<void*> finishArgs = {&constPartials};
+        for (size_t i = 0; i < outputs.size(); ++i) finishArgs.push_back(&outputPointers[i]);
+        finishArgs.push_back(&indexOut);
+        finishArgs.push_back(&scale);
+        plan.finishKernel->launch(plan.finishGridX, 1, 1, plan.finishThreads, stream.getStream(), finishArgs);
+    }
+}
+
 uint64_t StampedExecutionStage::flopCount() const {
     switch (kind) {
         case Kind::FusedKernel:
@@ -111,6 +152,8 @@ uint64_t StampedExecutionStage::flopCount() const {
             return arg_minmax ? arg_minmax->flopCount() : 0;
         case Kind::Copy:
             return 0;
+        case Kind::FusedReduction:
+            return fused_reduction ? fused_reduction->flopCount() : 0;
     }
     return 0;
 }
@@ -135,6 +178,10 @@ void StampedExecutionStage::runOn(Stream& stream, const std::unordered_map<std::
             destination.copyFromAsync(copySource, stream);
             return;
         }
+        case Kind::FusedReduction:
+            if (!fused_reduction) throw std::runtime_error("Fused reduction stage is missing its stamped reduction.");
+            fused_reduction->runOn(stream, runtime_scalars);
+            return;
     }
 }
 
@@ -152,6 +199,9 @@ std::unordered_set<std::string> StampedExecutionPlan::runtimeScalarNames() const
     for (const StampedExecutionStage& step : steps) {
         if (step.kernel) {
             for (const std::string& n : step.kernel->runtimeScalarNames()) names.insert(n);
+        }
+        if (step.fused_reduction) {
+            for (const std::string& n : step.fused_reduction->runtimeScalarNames()) names.insert(n);
         }
     }
     return names;

@@ -238,5 +238,8 @@ thor_tensor_t thor_stamped_arg_reduction_index_output(thor_stamped_arg_reduction
     return new thor_tensor{r->stamped->getIndexOutputTensor().value()};
 }
 int thor_stamped_arg_reduction_path(thor_stamped_arg_reduction_t r) { return r ? static_cast<int>(r->stamped->getPath()) : -1; }
+int thor_stamped_arg_reduction_variant(thor_stamped_arg_reduction_t r, char* buffer, size_t capacity) {
+    THOR_CAPI_TRY_INT(require(r, "arg reduction"); copyOut(r->stamped->getKernelVariant(), buffer, capacity, nullptr);)
+}
 
 }  // extern "C"

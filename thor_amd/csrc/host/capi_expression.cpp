@@ -237,7 +237,9 @@ int thor_plan_stage_kind(thor_plan_t plan, int stage, char* buffer, size_t capac
 }
 int thor_plan_stage_source(thor_plan_t plan, int stage, char* buffer, size_t capacity, size_t* needed) {
     THOR_CAPI_TRY_INT(require(plan, "plan"); const StampedExecutionStage& s = plan->plan.stages().at(stage);
-                      copyOut(s.kernel ? s.kernel->getCompiledKernel()->source : std::string(), buffer, capacity, needed);)
+                      copyOut(s.kernel ? s.kernel->getCompiledKernel()->source
+                                       : (s.fused_reduction ? s.fused_reduction->getLaunchPlan().mainKernel->source : std::string()),
+                              buffer, capacity, needed);)
 }
 int thor_plan_stage_description(thor_plan_t plan, int stage, char* buffer, size_t capacity) {
     THOR_CAPI_TRY_INT(
@@ -245,6 +247,7 @@ int thor_plan_stage_description(thor_plan_t plan, int stage, char* buffer, size_
         std::string text;
         if (s.kernel) text = s.kernel->getDescription();
         if (s.reduction) text = s.reduction->getStamped()->getKernelVariant();
+        if (s.fused_reduction) text = s.fused_reduction->getDescription();
         copyOut(text, buffer, capacity, nullptr);)
 }
 uint64_t thor_plan_flop_count(thor_plan_t plan) { return plan ? plan->plan.flopCount() : 0; }

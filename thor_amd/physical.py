@@ -55,6 +55,7 @@ PROTOTYPES = {
     "thor_stamped_reduction_run_scaled": (_i, [_vp, ctypes.c_float]), "thor_stamped_reduction_run_on": (_i, [_vp, _vp]),
     "thor_stamped_reduction_output": (_vp, [_vp]), "thor_stamped_reduction_path": (_i, [_vp]),
     "thor_stamped_reduction_workspace_bytes": (_sz, [_vp]), "thor_stamped_reduction_variant": (_i, [_vp, _cp, _sz]),
+    "thor_stamped_arg_reduction_variant": (_i, [_vp, _cp, _sz]),
     "thor_reduction_generate_source": (_i, [_i, _i, _i, _i, _i, _u64p, _u64p, _i, _u32p, _i, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_arg_reduction_stamp": (_vp, [_i, _u32p, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "thor_stamped_arg_reduction_destroy": (None, [_vp]), "thor_stamped_arg_reduction_run": (_i, [_vp]),
@@ -401,6 +402,11 @@ class StampedCubArgReduction:
 
     def get_path(self) -> CubReductionPath:
         return CubReductionPath(lib().thor_stamped_arg_reduction_path(self._h))
+
+    def get_kernel_variant(self) -> str:
+        buf = ctypes.create_string_buffer(512)
+        _check(lib().thor_stamped_arg_reduction_variant(self._h, buf, 512), "variant")
+        return buf.value.decode()
 
     def __del__(self):
         try:
