@@ -60,7 +60,7 @@ def cpu_baseline(seconds_budget: float = 12.0):
             "sample": f"{elems // (4 * n)} passes of the 4 conversions over 2^25 elements ({dt:.1f} s)"}
 
 
-def bench_other_configs(stream_raw_unused=None, iters=20):
+def bench_other_configs():
     """BASELINE configs 1, 3, 4, 5 through the Expression / reduction API: GB/s on algorithmic bytes, HIP-event timed."""
     from thor_amd import physical as ph
     from thor_amd.dtypes import DataType
@@ -91,19 +91,24 @@ def bench_other_configs(stream_raw_unused=None, iters=20):
         return c
 
     def timed(name, runs, nbytes, elements, note=""):
+        """Median of 5 samples; a sample is one pass over every rotating buffer (at least 8 launches), bracketed by events on
+        the launch stream (the reference's protocol: warm-up, >= 5 samples x >= 4 iterations, median)."""
         if callable(runs):
             runs = [runs]
-        reps = max(iters, len(runs) * 2)
+        reps = max(8, len(runs))
         for k in range(max(3, len(runs))):
             runs[k % len(runs)]()
         stream.synchronize()
-        a, b = Event(), Event()
-        a.record(RawStream)
-        for k in range(reps):
-            runs[k % len(runs)]()
-        b.record(RawStream)
-        b.synchronize()
-        ms = a.elapsed_ms(b) / reps
+        samples = []
+        for _ in range(5):
+            a, b = Event(), Event()
+            a.record(RawStream)
+            for k in range(reps):
+                runs[k % len(runs)]()
+            b.record(RawStream)
+            b.synchronize()
+            samples.append(a.elapsed_ms(b) / reps)
+        ms = float(np.median(samples))
         results[name] = {"ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1), "pct_hbm_peak": round(100 * nbytes / ms / 1e6 / HBM_PEAK_GBPS, 1),
                          "Gelem/s": round(elements / ms / 1e6, 2), "rotating_buffers": len(runs), "plan": note}
 
@@ -180,7 +185,7 @@ def bench_other_configs(stream_raw_unused=None, iters=20):
     timed("c5_channel_sum_fp16", [c.run for c in csum], 2 * n, n, csum[0].get_kernel_variant())
     stats = ex.compile(ex.outputs({"sum": ix.reduce_sum(axis=[0, 2, 3], squeeze=True), "sumsq": (ix * ix).reduce_sum(axis=[0, 2, 3], squeeze=True)}), 0)
     plans = [stats.stamp({"x": t}, stream) for t in xc8]
-    timed("c5_channel_sum_and_sumsq_fp16", [p_.run for p_ in plans], 2 * n, n, ">".join(plans[0].stage_kind_names()))
+    timed("c5_channel_sum_and_sumsq_fp16", [p_.run for p_ in plans], 2 * n, n, ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
     return results
 
 
