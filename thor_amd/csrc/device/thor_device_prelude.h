@@ -207,9 +207,12 @@ struct ArgAcc {
         if (IS_MAX ? (bv > av) : (bv < av)) return false;
         return ai <= bi;
     }
+    // Adds the next element of one thread's walk.  Every kernel visits its elements in increasing index order, so an
+    // equal value never replaces the candidate: only a strictly better value, the first NaN, or the first element at all.
     template <typename I>
     __device__ __forceinline__ void add(float x, I index) {
-        if (!better(v, i, x, (IndexT)index)) {
+        const bool strictlyBetter = IS_MAX ? (x > v) : (x < v);
+        if (strictlyBetter || ((x != x) && (v == v)) || i == ~(IndexT)0) {
             v = x;
             i = (IndexT)index;
         }
