@@ -40,6 +40,10 @@ class Stream {
 
     typedef void (*HostFn)(void*);
     void enqueueHostFunction(HostFn function, std::unique_ptr<HostFunctionArgsBase>&& args);
+    // The arguments of a finished host function (and the tensors they keep alive) are destroyed on an application thread,
+    // never on the runtime's callback thread, where releasing device or pinned memory is not allowed.  synchronize(),
+    // enqueueHostFunction() and tensor allocation drain the list; it may also be drained explicitly.
+    static void drainFinishedHostCalls();
 
     bool operator==(const Stream& other) const { return state != nullptr && state == other.state; }
     int getGpuNum() const;

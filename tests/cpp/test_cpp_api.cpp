@@ -1,0 +1,319 @@
+// Exercises the C++ API (namespace ThorImplementation) directly, the way the reference's gtest suites do
+// (test/Utilities/TensorOperations/CubReductionValueOperationsTest.cpp, CubArgReductionTest.cpp,
+//  CubReductionGeometryTest.cpp, test/Utilities/Expression/CommonInputFusionTest.cpp,
+//  test/Utilities/TensorOperations/DataTypeConversions).  Plain asserts instead of gtest: the image has no gtest.
+// Usage: test_cpp_api [host|gpu]   (host: the cases that need no GPU)
+#include "DeepLearning/Implementation/Tensor/Tensor.h"
+#include "Utilities/Common/Stream.h"
+#include "Utilities/Expression/Expression.h"
+#include "Utilities/Expression/ExpressionDTypeResolution.h"
+#include "Utilities/Expression/FusedEquation.h"
+#include "Utilities/TensorOperations/Cub/CubReduction.h"
+#include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <limits>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+using namespace ThorImplementation;
+
+static int failures = 0;
+static int checks = 0;
+#define CHECK(cond)                                                                     \
+    do {                                                                                \
+        ++checks;                                                                       \
+        if (!(cond)) {                                                                  \
+            ++failures;                                                                 \
+            std::printf("  CHECK failed %s:%d: %s\n", __FILE__, __LINE__, #cond);       \
+        }                                                                               \
+    } while (0)
+#define CHECK_NEAR(a, b, tol) CHECK(std::fabs(double(a) - double(b)) <= (tol))
+template <typename E, typename F>
+static bool throwsAs(F&& f) {
+    try {
+        f();
+    } catch (const E&) {
+        return true;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+static const TensorPlacement cpuPlacement(TensorPlacement::MemDevices::CPU);
+static const TensorPlacement gpuPlacement(TensorPlacement::MemDevices::GPU, 0);
+
+static Tensor gpuFrom(const std::vector<float>& values, const std::vector<uint64_t>& dims, Stream& stream, DataType dtype = DataType::FP32) {
+    Tensor host(cpuPlacement, TensorDescriptor(DataType::FP32, dims));
+    std::memcpy(host.getMemPtr<float>(), values.data(), values.size() * sizeof(float));
+    Tensor device(gpuPlacement, TensorDescriptor(dtype, dims));
+    device.copyFromAsync(host, stream);  // converts when the dtypes differ
+    stream.synchronize();
+    return device;
+}
+
+static std::vector<float> toHostF32(const Tensor& t, Stream& stream) {
+    Tensor host(cpuPlacement, TensorDescriptor(DataType::FP32, t.getDimensions()));
+    host.copyFromAsync(t, stream);
+    stream.synchronize();
+    const float* p = host.getMemPtr<float>();
+    return std::vector<float>(p, p + host.getTotalNumElements());
+}
+
+template <typename T>
+static std::vector<T> toHostRaw(const Tensor& t, Stream& stream) {
+    Tensor host(cpuPlacement, TensorDescriptor(t.getDataType(), t.getDimensions()));
+    host.copyFromAsync(t, stream);
+    stream.synchronize();
+    const T* p = host.getMemPtr<T>();
+    return std::vector<T>(p, p + host.getTotalNumElements());
+}
+
+// ---- host-only cases -----------------------------------------------------------------------------------------------------
+static void geometryPathsAndErrors() {
+    // CubReductionGeometryTest.cpp: path selection and argument validation by exception type
+    CHECK(CubReduction::analyzeGeometry({8192, 8192}, std::vector<uint32_t>{0, 1}).path == CubReductionPath::DeviceTransformReduce);
+    const CubReductionGeometry rows = CubReduction::analyzeGeometry({8192, 4096}, 1);
+    CHECK(rows.path == CubReductionPath::ContiguousFixedSegment && rows.outer_size == 8192 && rows.reduction_size == 4096 && rows.inner_size == 1);
+    const CubReductionGeometry tiled = CubReduction::analyzeGeometry({4, 5, 6}, 1);
+    CHECK(tiled.path == CubReductionPath::TiledFixedSegment && tiled.outer_size == 4 && tiled.reduction_size == 5 && tiled.inner_size == 6);
+    const CubReductionGeometry strided = CubReduction::analyzeGeometry({64, 256, 56, 56}, std::vector<uint32_t>{0, 2, 3});
+    CHECK(strided.path == CubReductionPath::StridedFixedSegment && strided.output_elements == 256 && strided.reduction_size == 64ull * 56 * 56);
+    CHECK((strided.squeezed_output_dimensions == std::vector<uint64_t>{256}));
+    CHECK(throwsAs<std::invalid_argument>([] { CubReduction::analyzeGeometry({4, 5}, 2); }));
+    CHECK(throwsAs<std::invalid_argument>([] { CubReduction::analyzeGeometry({4, 5}, std::vector<uint32_t>{1, 1}); }));
+    CHECK(throwsAs<std::invalid_argument>([] { CubReduction::analyzeGeometry({}, 0); }));
+    CHECK(CubReduction::getFp32EmptyReductionValue(CubReductionOp::Product) == 1.0f);
+    CHECK(CubReduction::getFp32EmptyReductionValue(CubReductionOp::Min) == std::numeric_limits<float>::infinity());
+    CHECK(CubArgReduction::getEmptyReductionIndex() == std::numeric_limits<uint64_t>::max());
+    // logical (output, reduction) coordinates -> physical offsets on a [2,3,2] tensor reduced over {0,2}
+    const CubReductionGeometry g = CubReduction::analyzeGeometry({2, 3, 2}, std::vector<uint32_t>{0, 2});
+    CHECK(CubReduction::mapLogicalReductionIndexToPhysicalIndex(g, 1, 0) == 2);
+    CHECK(CubReduction::mapLogicalReductionIndexToPhysicalIndex(g, 1, 3) == 6 + 2 + 1);
+}
+
+static void dtypeResolutionAndStageSplit() {
+    // CommonInputFusionTest.cpp:281-303: a reduction boundary splits stages; dtype rules of ExpressionDTypeResolution.cpp
+    Expression x = Expression::input("x"), y = Expression::input("y");
+    Expression trunk = x + y;
+    Outputs outs = Expression::outputs({{"trunk", trunk}, {"sum_last", trunk.reduce_sum({1}, {})}});
+    PhysicalOutputs physical = outs.physicalOutputs();
+    resolveOutputsDTypesInPlace(physical, {DataType::FP16, DataType::BF16});
+    for (const NamedOutput& o : physical.outputs) {
+        const ExprNode& node = physical.expr->nodes[o.node_idx];
+        if (o.name == "trunk") CHECK(node.output_dtype == DataType::FP32);  // fp16 with bf16 promotes to fp32
+        if (o.name == "sum_last") CHECK(node.output_dtype == DataType::FP32 && node.compute_dtype == DataType::FP32);
+    }
+    Expression s = Expression::input("d").sigmoid();
+    const PhysicalExpression p = s.expression();
+    CHECK(canonicalize(p) == "div(exp(neg(max(neg(input#0),scalar(0)))),add(exp(neg(abs(input#0))),scalar(1)))");
+    CHECK(throwsAs<std::runtime_error>([&] {
+        PhysicalOutputs bad = Expression::outputs({{"o", x + y}}).physicalOutputs();
+        resolveOutputsDTypesInPlace(bad, {DataType::UINT8, DataType::FP16});
+    }));
+}
+
+static void cpuTypeConverter() {
+    // the reference's CPU path (TypeConverter.cpp:899-942): RNE, +-Inf on overflow, gradual underflow, fp8 satfinite
+    const std::vector<float> in = {1.0f, 65504.0f, 65520.0f, 1e5f, -1e5f, 5.9604645e-8f, 2.9802322e-8f, 1e-40f, 448.0f, 1e6f};
+    std::vector<uint16_t> h(in.size()), b(in.size());
+    std::vector<uint8_t> e4(in.size()), e5(in.size());
+    TypeConverter::cpuConvertNow(in.data(), h.data(), DataType::FP32, DataType::FP16, in.size());
+    TypeConverter::cpuConvertNow(in.data(), b.data(), DataType::FP32, DataType::BF16, in.size());
+    TypeConverter::cpuConvertNow(in.data(), e4.data(), DataType::FP32, DataType::FP8_E4M3, in.size());
+    TypeConverter::cpuConvertNow(in.data(), e5.data(), DataType::FP32, DataType::FP8_E5M2, in.size());
+    CHECK(h[0] == 0x3C00 && h[1] == 0x7BFF && h[2] == 0x7C00 && h[3] == 0x7C00 && h[4] == 0xFC00);
+    CHECK(h[5] == 0x0001 && h[6] == 0x0000 && h[7] == 0x0000);  // 2^-24 is the smallest subnormal; 2^-25 ties to even (zero)
+    CHECK(b[0] == 0x3F80 && b[3] == 0x47C3 && b[7] == 0x0001);  // 1e5 -> 0x47C35000 rounds to 0x47C3 ; 1e-40 is a bf16 subnormal
+    CHECK(e4[8] == 0x7E && e4[9] == 0x7E);                      // 448 is the largest e4m3 value and everything above saturates to it
+    CHECK(e5[9] == 0x7B);                                       // 57344 saturating
+    std::vector<float> back(in.size());
+    TypeConverter::cpuConvertNow(h.data(), back.data(), DataType::FP16, DataType::FP32, in.size());
+    CHECK(back[0] == 1.0f && back[1] == 65504.0f && std::isinf(back[2]) && back[5] == 5.9604645e-8f);
+}
+
+// ---- GPU cases -------------------------------------------------------------------------------------------------------------
+static void valueReductionsSmallExact(Stream& stream) {
+    // CubReductionValueOperationsTest.cpp: small integers, exact in fp32 whatever the order
+    Tensor v = gpuFrom({-2.0f, 3.0f, -4.0f}, {3}, stream);
+    auto run = [&](CubReductionOp op, const Tensor& t, std::vector<uint32_t> axes, float scale = 1.0f) {
+        auto stamped = CubReduction(op, axes, DataType::FP32, scale).stamp(t, stream);
+        stamped->run();
+        return toHostF32(stamped->getOutputTensor(), stream);
+    };
+    CHECK(run(CubReductionOp::Sum, v, {0})[0] == -3.0f);
+    CHECK(run(CubReductionOp::Min, v, {0})[0] == -4.0f);
+    CHECK(run(CubReductionOp::Max, v, {0})[0] == 3.0f);
+    CHECK(run(CubReductionOp::Product, v, {0})[0] == 24.0f);
+    CHECK(run(CubReductionOp::Mean, v, {0})[0] == -1.0f);
+    CHECK(run(CubReductionOp::L1Norm, v, {0})[0] == 9.0f);
+    CHECK_NEAR(run(CubReductionOp::L2Norm, v, {0})[0], std::sqrt(29.0), 1e-6);
+    CHECK(run(CubReductionOp::Sum, v, {0}, 0.5f)[0] == -1.5f);
+    Tensor m = gpuFrom({-1, 2, -3, 4, -5, 6}, {2, 3}, stream);
+    CHECK((run(CubReductionOp::Sum, m, {1}) == std::vector<float>{-2, 5}));
+    CHECK((run(CubReductionOp::Sum, m, {0}) == std::vector<float>{3, -3, 3}));
+    CHECK((run(CubReductionOp::Max, m, {0, 1}) == std::vector<float>{6}));
+    Tensor nan = gpuFrom({1.0f, std::nanf(""), 3.0f}, {3}, stream);
+    CHECK(std::isnan(run(CubReductionOp::Max, nan, {0})[0]) && std::isnan(run(CubReductionOp::Min, nan, {0})[0]));
+    // output dtype and satfinite for fp8 (CubReductionDTypeAndLifecycleTest.cpp:205-222)
+    Tensor big = gpuFrom({400.0f, 400.0f}, {2}, stream);
+    auto e4 = CubReduction(CubReductionOp::Sum, 0u, DataType::FP8_E4M3).stamp(big, stream);
+    e4->run();
+    CHECK(toHostF32(e4->getOutputTensor(), stream)[0] == 448.0f);
+    CHECK(e4->getOutputDataType() == DataType::FP8_E4M3 && e4->getAccumulatorDataType() == DataType::FP32);
+    CHECK(throwsAs<std::invalid_argument>([&] { CubReduction(CubReductionOp::Sum, 3u).stamp(m, stream); }));
+}
+
+static void argReductionsTiesAndNaN(Stream& stream) {
+    // CubArgReductionTest.cpp: lowest index wins ties, NaN wins, index is the position inside the reduction domain
+    Tensor t = gpuFrom({1, 1, 3, 1, std::nanf(""), 0, std::nanf(""), -4}, {2, 4}, stream);
+    CubArgReductionOutputOptions options;
+    options.produce_value = true;
+    auto amin = CubArgReduction(CubArgReductionOp::ArgMin, 1u, options).stamp(t, stream);
+    amin->run();
+    CHECK((toHostRaw<uint32_t>(amin->getIndexOutputTensor().value(), stream) == std::vector<uint32_t>{0, 0}));
+    const std::vector<float> values = toHostF32(amin->getValueOutputTensor().value(), stream);
+    CHECK(values[0] == 1.0f && std::isnan(values[1]));
+    Tensor u = gpuFrom({5, 5, 3, 5, -1, std::nanf(""), std::nanf(""), 8}, {2, 4}, stream);
+    options.produce_value = false;
+    options.index_output_dtype = DataType::UINT64;
+    auto amax = CubArgReduction(CubArgReductionOp::ArgMax, 1u, options).stamp(u, stream);
+    amax->run();
+    CHECK((toHostRaw<uint64_t>(amax->getIndexOutputTensor().value(), stream) == std::vector<uint64_t>{0, 1}));
+    CHECK(!amax->getValueOutputTensor().has_value());
+}
+
+static void expressionConfig1AndRuntimeScalars(Stream& stream) {
+    const size_t n = 1000;
+    std::vector<float> a(n), b(n), c(n), d(n);
+    for (size_t i = 0; i < n; ++i) {
+        a[i] = std::sin(0.1f * i);
+        b[i] = std::cos(0.3f * i);
+        c[i] = 0.001f * i - 0.5f;
+        d[i] = 0.02f * i - 10.0f;
+    }
+    Expression ea = Expression::input("a"), eb = Expression::input("b"), ec = Expression::input("c"), ed = Expression::input("d");
+    FusedEquation eq = FusedEquation::compile(((ea * eb + ec) * ed.sigmoid()).expression(), 0);
+    std::unordered_map<std::string, Tensor> inputs = {{"a", gpuFrom(a, {n}, stream)}, {"b", gpuFrom(b, {n}, stream)}, {"c", gpuFrom(c, {n}, stream)},
+                                                      {"d", gpuFrom(d, {n}, stream)}};
+    StampedExecutionPlan plan = eq.stamp(inputs, stream);
+    CHECK((plan.stageKindNames() == std::vector<std::string>{"FusedKernel"}));
+    plan.run();
+    const std::vector<float> got = toHostF32(plan.output(), stream);
+    for (size_t i = 0; i < n; i += 37) {
+        const double want = (double(a[i]) * b[i] + c[i]) / (1.0 + std::exp(-double(d[i])));
+        CHECK_NEAR(got[i], want, 4e-7 * std::max(1.0, std::fabs(want)) + 2e-7);
+    }
+    // convenience run into a caller-provided tensor, with a runtime scalar
+    Expression scaled = Expression::input("x") * Expression::runtimeScalar("alpha") + 1.0;
+    FusedEquation eq2 = FusedEquation::compile(scaled.expression(), 0);
+    Tensor x = gpuFrom({1, 2, 3, 4}, {4}, stream);
+    Tensor out(gpuPlacement, TensorDescriptor(DataType::FP32, {4}));
+    eq2.run({{"x", x}}, {{"alpha", 2.5f}}, out, stream);
+    CHECK((toHostF32(out, stream) == std::vector<float>{3.5f, 6.0f, 8.5f, 11.0f}));
+    CHECK(throwsAs<std::runtime_error>([&] { eq2.run({{"x", x}}, out, stream); }));  // missing runtime scalar
+}
+
+static void softmaxPlansAndRowKernel(Stream& stream) {
+    const uint64_t rows = 7, cols = 130;
+    std::vector<float> x(rows * cols);
+    for (size_t i = 0; i < x.size(); ++i) x[i] = 3.0f * std::sin(0.37f * i);
+    Tensor tx = gpuFrom(x, {rows, cols}, stream, DataType::BF16);
+    const std::vector<float> xb = toHostF32(tx, stream);  // the bf16-rounded values the kernels see
+    Expression ix = Expression::input("x");
+    Expression e = (ix - ix.reduce_max({1})).exp();
+    FusedEquation eq = FusedEquation::compile((e / e.reduce_sum({1})).expression(), 0);
+    auto check = [&](const StampedExecutionPlan& plan) {
+        const std::vector<float> got = toHostF32(plan.output(), stream);
+        for (uint64_t r = 0; r < rows; ++r) {
+            double m = -1e30, sum = 0;
+            for (uint64_t c = 0; c < cols; ++c) m = std::max<double>(m, xb[r * cols + c]);
+            for (uint64_t c = 0; c < cols; ++c) sum += std::exp(xb[r * cols + c] - m);
+            for (uint64_t c = 0; c < cols; c += 11) CHECK_NEAR(got[r * cols + c], std::exp(xb[r * cols + c] - m) / sum, 2e-6);
+        }
+    };
+    StampedExecutionPlan fused = eq.stamp({{"x", tx}}, stream);
+    CHECK((fused.stageKindNames() == std::vector<std::string>{"FusedRowKernel"}));
+    CHECK(fused.output().getDataType() == DataType::FP32);
+    fused.run();
+    check(fused);
+    setenv("THOR_DISABLE_ROW_FUSION", "1", 1);
+    StampedExecutionPlan staged = eq.stamp({{"x", tx}}, stream);
+    unsetenv("THOR_DISABLE_ROW_FUSION");
+    // the reference's lowering (CommonInputFusionTest.cpp:281-327)
+    CHECK((staged.stageKindNames() == std::vector<std::string>{"Reduction", "FusedKernel", "Reduction", "FusedKernel"}));
+    CHECK((staged.reductionPaths() == std::vector<CubReductionPath>{CubReductionPath::ContiguousFixedSegment, CubReductionPath::ContiguousFixedSegment}));
+    staged.run();
+    check(staged);
+}
+
+static void typeConverterOnGpuAndTensorViews(Stream& stream) {
+    const uint64_t n = 100003;
+    std::vector<float> x(n);
+    for (uint64_t i = 0; i < n; ++i) x[i] = (i % 100 == 0 ? 1e5f : 1.0f) * std::sin(0.001f * i) * (i % 100 == 1 ? 1e-40f : 1.0f);
+    Tensor src = gpuFrom(x, {n}, stream);
+    Tensor half(gpuPlacement, TensorDescriptor(DataType::FP16, {n}));
+    TypeConverter::convertType(src.getMemPtr(), half.getMemPtr(), DataType::FP32, DataType::FP16, (long)n, stream, 0);
+    const std::vector<uint16_t> got = toHostRaw<uint16_t>(half, stream);
+    std::vector<uint16_t> want(n);
+    TypeConverter::cpuConvertNow(x.data(), want.data(), DataType::FP32, DataType::FP16, (long)n);
+    CHECK(got == want);
+    // in place, widening back (walks backwards)
+    Tensor wide(gpuPlacement, TensorDescriptor(DataType::FP32, {n}));
+    wide.copyFromAsync(half, stream);  // device-to-device copy with conversion
+    const std::vector<float> back = toHostF32(wide, stream);
+    std::vector<float> wantBack(n);
+    TypeConverter::cpuConvertNow(want.data(), wantBack.data(), DataType::FP16, DataType::FP32, (long)n);
+    CHECK(std::memcmp(back.data(), wantBack.data(), n * 4) == 0);
+    // a transposed view reduces through the strided path
+    Tensor m = gpuFrom({1, 2, 3, 4, 5, 6}, {2, 3}, stream);
+    Tensor view = m.aliasView({3, 2}, {1, 3});
+    auto stamped = CubReduction(CubReductionOp::Sum, 1u).stamp(view, stream);
+    stamped->run();
+    CHECK((toHostF32(stamped->getOutputTensor(), stream) == std::vector<float>{5, 7, 9}));
+    CHECK(throwsAs<std::invalid_argument>([&] { Tensor outside = m.aliasView({4, 2}, {1, 3}); }));  // would read past the allocation
+}
+
+int main(int argc, char** argv) {
+    const std::string mode = argc > 1 ? argv[1] : "gpu";
+    struct Case {
+        const char* name;
+        std::function<void()> body;
+    };
+    std::vector<Case> cases = {{"geometryPathsAndErrors", geometryPathsAndErrors},
+                               {"dtypeResolutionAndStageSplit", dtypeResolutionAndStageSplit},
+                               {"cpuTypeConverter", cpuTypeConverter}};
+    if (mode == "gpu") {
+        auto withStream = [](void (*f)(Stream&)) {
+            return [f] {
+                Stream stream(0);
+                f(stream);
+            };
+        };
+        cases.push_back({"valueReductionsSmallExact", withStream(valueReductionsSmallExact)});
+        cases.push_back({"argReductionsTiesAndNaN", withStream(argReductionsTiesAndNaN)});
+        cases.push_back({"expressionConfig1AndRuntimeScalars", withStream(expressionConfig1AndRuntimeScalars)});
+        cases.push_back({"softmaxPlansAndRowKernel", withStream(softmaxPlansAndRowKernel)});
+        cases.push_back({"typeConverterOnGpuAndTensorViews", withStream(typeConverterOnGpuAndTensorViews)});
+    }
+    for (const Case& c : cases) {
+        const int before = failures;
+        std::printf("[ RUN  ] %s\n", c.name);
+        std::fflush(stdout);
+        try {
+            c.body();
+        } catch (const std::exception& e) {
+            ++failures;
+            std::printf("  unexpected exception: %s\n", e.what());
+        }
+        std::printf("[ %s ] %s\n", failures == before ? " OK " : "FAIL", c.name);
+    }
+    std::printf("%d checks, %d failures\n", checks, failures);
+    return failures == 0 ? 0 : 1;
+}

@@ -1,6 +1,7 @@
 #include "Utilities/Common/Stream.h"
 
 #include <atomic>
+#include <vector>
 
 using ThorImplementation::ScopedGpu;
 
@@ -23,6 +24,29 @@ struct Stream::PendingHostCall {
 };
 
 static std::atomic<uint64_t> nextStreamId{1};
+
+// Finished host calls wait here until an application thread destroys them.  Never destructed: callbacks may still arrive
+// while the process shuts down.
+namespace {
+struct FinishedCalls {
+    std::mutex mutex;
+    std::vector<void*> calls;
+};
+FinishedCalls& finishedCalls() {
+    static FinishedCalls* list = new FinishedCalls;
+    return *list;
+}
+}  // namespace
+
+void Stream::drainFinishedHostCalls() {
+    std::vector<void*> calls;
+    {
+        FinishedCalls& list = finishedCalls();
+        std::lock_guard<std::mutex> lock(list.mutex);
+        calls.swap(list.calls);
+    }
+    for (void* raw : calls) delete static_cast<PendingHostCall*>(raw);
+}
 
 Stream::Stream(int gpuNum, Priority) {
     // Priorities are accepted for source compatibility; every stream is created at the default priority.
@@ -71,6 +95,7 @@ void Stream::waitEvent(Event event) const {
 void Stream::synchronize() const {
     THOR_THROW_IF_FALSE(state != nullptr);
     THOR_HIP_CHECK(thorhip_stream_synchronize(state->handle));
+    drainFinishedHostCalls();
     std::exception_ptr failure;
     {
         std::lock_guard<std::mutex> lock(state->failureMutex);
@@ -85,17 +110,27 @@ void Stream::deviceSynchronize(int gpuNum) {
 }
 
 void Stream::hostFunctionTrampoline(void* raw) noexcept {
-    std::unique_ptr<PendingHostCall> call(static_cast<PendingHostCall*>(raw));
+    PendingHostCall* call = static_cast<PendingHostCall*>(raw);
     try {
         call->function(call->args.get());
     } catch (...) {
         std::lock_guard<std::mutex> lock(call->owner->failureMutex);
         if (!call->owner->firstFailure) call->owner->firstFailure = std::current_exception();
     }
+    // This runs on the runtime's callback thread: destroying the arguments here could free device or pinned memory (the
+    // tensors a copy keeps alive), which blocks on the very stream that is executing this callback.  Park them instead.
+    try {
+        FinishedCalls& list = finishedCalls();
+        std::lock_guard<std::mutex> lock(list.mutex);
+        list.calls.push_back(call);
+    } catch (...) {
+        // out of memory while parking: leak the call rather than release memory on this thread
+    }
 }
 
 void Stream::enqueueHostFunction(HostFn function, std::unique_ptr<HostFunctionArgsBase>&& args) {
     THOR_THROW_IF_FALSE(state != nullptr && function != nullptr);
+    drainFinishedHostCalls();
     auto* call = new PendingHostCall{function, std::move(args), state};
     const int rc = thorhip_stream_enqueue_host_function(state->handle, &Stream::hostFunctionTrampoline, call);
     if (rc != 0) {

@@ -39,6 +39,7 @@ Tensor::Tensor(TensorPlacement placement, TensorDescriptor descriptor, uint32_t 
     : placement(placement), descriptor(descriptor) {
     THOR_THROW_IF_FALSE(placement.getMemDevice() != TensorPlacement::MemDevices::INVALID);
     THOR_THROW_IF_FALSE(descriptor.getTotalNumElements() > 0);
+    Stream::drainFinishedHostCalls();  // release what finished copies kept alive before asking for more memory
     auto memory = std::make_shared<BackingMemory>();
     memory->placement = placement;
     const size_t bytes = descriptor.getArraySizeInBytes() + kTailPadBytes;
