@@ -188,6 +188,42 @@ def test_views_diagonal_and_broadcast_alias(stream):
     assert copy_gpu_to_numpy(amax.get_index_output_tensor(), stream).reshape(-1).tolist() == [4] * 5
 
 
+PERMUTED = [
+    # (storage shape, permutation giving the view, reduced view axes)
+    ((96, 200), (1, 0), [1]),            # transposed matrix, reduce along the view's rows = the storage's columns
+    ((40, 33, 64), (2, 0, 1), [1]),      # contiguous storage axis first in the view, reduce a middle storage axis
+    ((40, 33, 64), (2, 0, 1), [1, 2]),   # ... and both other axes
+    ((12, 16, 48), (0, 2, 1), [2]),      # batch kept, inner two swapped
+    ((7, 130), (1, 0), [1]),             # lane axis not a multiple of the vector width
+]
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16], ids=lambda d: d.name)
+@pytest.mark.parametrize("shape,perm,axes", PERMUTED, ids=[f"{s}-{p}-{a}".replace(" ", "") for s, p, a in PERMUTED])
+def test_permuted_views_reduce_with_lanes_on_the_contiguous_kept_axis(stream, shape, perm, axes, dtype):
+    """Dense tensors seen through a permuted view (what Expression transposes hand to reductions): values and arg indices
+    must equal those of the materialised permutation."""
+    rng = np.random.default_rng(12)
+    x = rng.integers(-8, 9, shape).astype(np.float32)  # small integers: sums are exact in any order
+    storage = to_storage(x, dtype)
+    t = copy_numpy_to_gpu(storage, stream, dtype)
+    strides = [int(np.prod(shape[i + 1:])) for i in range(len(shape))]
+    view = t.alias_view([shape[p] for p in perm], [strides[p] for p in perm])
+    logical = np.ascontiguousarray(np.transpose(x, perm))
+    for name in ("Sum", "Max", "Min", "L1Norm"):
+        stamped = ph.CubReduction(OPS[name][0], axes, DataType.fp32).stamp(view, stream)
+        stamped.run()
+        want = oracle.reduce(OPS[name][1], logical, oracle.FP32, axes)
+        np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream).reshape(want.shape), want, err_msg=f"{name} {stamped.get_kernel_variant()}")
+    assert "view_columns" in stamped.get_kernel_variant()
+    for op, oracle_op in ((ph.CubArgReductionOp.ArgMax, oracle.ARGMAX), (ph.CubArgReductionOp.ArgMin, oracle.ARGMIN)):
+        arg = ph.CubArgReduction(op, axes, value_output_dtype=DataType.fp32).stamp(view, stream)
+        arg.run()
+        want_index, want_value = oracle.arg_reduce(oracle_op, logical, oracle.FP32, axes)
+        np.testing.assert_array_equal(copy_gpu_to_numpy(arg.get_index_output_tensor(), stream).reshape(want_index.shape).astype(np.uint64), want_index)
+        np.testing.assert_array_equal(gpu_to_f32(arg.get_value_output_tensor(), stream).reshape(want_value.shape), want_value)
+
+
 def test_config3_full_size_properties(stream):
     """BASELINE config 3, fp32 [8192, 8192] N(0,1): full sum, row sum, row max, row argmax.  Checked at full size against
     the float64 oracle (rows are independent, so the oracle finishes in seconds) and through invariants."""

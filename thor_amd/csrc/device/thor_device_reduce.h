@@ -146,30 +146,29 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
     }
 }
 
-// ---- middle axis: [kOuter, kR, kInner] -> [kOuter, kInner] ------------------------------------------------------------------
-// A block is kLanesX columns wide (a column = kVec adjacent inner positions; adjacent lanes read adjacent memory) and
-// kThreads / kLanesX row groups deep: row group g of share s walks rows rBegin + g, rBegin + g + groups, ...; the groups
-// are then folded through LDS, so the depth adds parallelism without adding partials.  Cfg: kOuter, kR, kInner,
-// kLanesX (power of two <= 64), kBatch (rows in flight per thread), kSplit (shares of kR, grid y),
-// kOutOuterStride / kOutInnerStride (output layout).
+// ---- lanes across outputs: [kOuter, kR, kInner] -> [kOuter, kInner], and views whose kept axis is the contiguous one --------
+// A column is kVec outputs that are adjacent in memory; adjacent lanes own adjacent columns, so a wavefront reads up to
+// 1 KiB of contiguous memory per step of the reduction.  A block is kLanesX columns wide and kThreads / kLanesX row
+// groups deep: row group g of share s walks reduction positions rBegin + g, rBegin + g + groups, ...; the groups are
+// then folded through LDS, so the depth adds parallelism without adding partials.
+// Cfg: kColumns, kR (reduction positions), kLanesX (power of two <= 64), kBatch (positions in flight per thread), kSplit
+// (shares of kR, grid y), and the generated address functions columnBase(column), rowOffset(r), outputIndex(column, k)
+// (where element k of the column is stored) and partialSlot(column, k) (its row-major output number).
 template <typename Cfg>
 __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* partials, float scale) {
     typedef typename Cfg::IndexT IndexT;
     typedef typename Cfg::Acc Acc;
-    constexpr u64 kInnerVectors = Cfg::kInner / Cfg::kVec;
-    constexpr u64 kColumns = Cfg::kOuter * kInnerVectors;
     constexpr u64 kRowsPerShare = (Cfg::kR + Cfg::kSplit - 1) / Cfg::kSplit;
     constexpr int kGroups = Cfg::kThreads / Cfg::kLanesX;
     constexpr int kBatch = Cfg::kBatch;
     const int lx = threadIdx.x % Cfg::kLanesX, group = threadIdx.x / Cfg::kLanesX;
     const u64 column = (u64)blockIdx.x * Cfg::kLanesX + lx;
-    const bool columnLive = column < kColumns;
+    const bool columnLive = column < Cfg::kColumns;
     const u64 safeColumn = columnLive ? column : 0;
-    const u64 outer = safeColumn / kInnerVectors, iv = safeColumn % kInnerVectors;
     const u64 share = Cfg::kSplit > 1 ? blockIdx.y : 0;
     const u64 rBegin = share * kRowsPerShare;
     const u64 rEnd = (rBegin + kRowsPerShare < Cfg::kR) ? rBegin + kRowsPerShare : Cfg::kR;
-    const u64 base = outer * Cfg::kR * Cfg::kInner + iv * Cfg::kVec;
+    const u64 base = Cfg::columnBase(safeColumn);
 
     Acc acc[Cfg::kVec];
 #pragma unroll
@@ -181,7 +180,7 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
         for (int u = 0; u < kBatch; ++u) {
             const u64 r = r0 + (u64)u * kGroups;
             live[u] = columnLive && r < rEnd;
-            if (live[u]) Cfg::load(src, base + r * Cfg::kInner, x[u]);
+            if (live[u]) Cfg::load(src, base + Cfg::rowOffset(r), x[u]);
         }
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
@@ -210,12 +209,10 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
     if (group != 0 || !columnLive) return;
 #pragma unroll
     for (int k = 0; k < Cfg::kVec; ++k) {
-        const u64 inner = iv * Cfg::kVec + k;
         if (Cfg::kSplit > 1) {
-            const u64 logical = outer * Cfg::kInner + inner;
-            acc[k].storePartial(partials, logical * Cfg::kSplit + share, Cfg::kOuter * Cfg::kInner * Cfg::kSplit);
+            acc[k].storePartial(partials, Cfg::partialSlot(column, k) * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
         } else {
-            Cfg::store(acc[k], outer * Cfg::kOutOuterStride + inner * Cfg::kOutInnerStride, out, scale);
+            Cfg::store(acc[k], Cfg::outputIndex(column, k), out, scale);
         }
     }
 }

@@ -147,7 +147,7 @@ std::string ReductionShape::describe() const {
             out << "rows(lanes_per_row=" << threadsPerRow << ",split=" << split;
             break;
         case Kernel::Columns:
-            out << "columns(lanes_x=" << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
+            out << (laneAxis < 0 ? "columns(lanes_x=" : "view_columns(lanes_x=") << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
             break;
         case Kernel::Strided:
             out << "strided(kept_rank=" << keptDims.size() << ",reduced_rank=" << reducedDims.size() << ",split=" << split;
@@ -250,6 +250,42 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
     if (shape.reducedDims.empty()) {
         shape.reducedDims = {1};
         shape.reducedStrides = {0};
+    }
+    // A view whose contiguous axis is a kept one (a transposed matrix reduced along its rows): lanes go across that axis,
+    // every lane owns outputs, and memory is still read in contiguous runs.  Lanes across the reduction domain, below,
+    // would read one element per cache line.
+    int laneAxis = -1;
+    bool reducedContiguous = false;
+    for (size_t a = 0; a < shape.reducedDims.size(); ++a) reducedContiguous = reducedContiguous || (shape.reducedStrides[a] == 1 && shape.reducedDims[a] > 1);
+    if (!reducedContiguous) {
+        for (size_t a = 0; a < shape.keptDims.size(); ++a)
+            if (shape.keptStrides[a] == 1 && shape.keptDims[a] >= 16) laneAxis = static_cast<int>(a);
+    }
+    if (laneAxis >= 0) {
+        shape.kernel = ReductionShape::Kernel::Columns;
+        shape.laneAxis = laneAxis;
+        int vec = static_cast<int>(16 / elementBytes);
+        while (vec > 1) {
+            bool ok = request.inputAlignmentBytes % (static_cast<uint64_t>(vec) * elementBytes) == 0 && shape.keptDims[laneAxis] % vec == 0;
+            for (size_t a = 0; a < shape.keptStrides.size(); ++a) ok = ok && (static_cast<int>(a) == laneAxis || shape.keptStrides[a] % vec == 0);
+            for (uint64_t st : shape.reducedStrides) ok = ok && st % vec == 0;
+            if (ok) break;
+            vec /= 2;
+        }
+        shape.vec = vec;
+        shape.unroll = 8;
+        const uint64_t columns = g.output_elements / vec;
+        shape.threadsPerRow = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(columns)));
+        const uint64_t groups = 256 / shape.threadsPerRow;
+        const uint64_t wantedThreads = 4 * kTargetThreads;
+        if (columns * groups < wantedThreads && g.reduction_size >= groups * 32) {
+            shape.split = std::min<uint64_t>({ceilDiv(wantedThreads, columns * groups), g.reduction_size / (groups * 16), kMaxGridY});
+            if (shape.split < 2) shape.split = 1;
+        }
+        shape.gridX = static_cast<uint32_t>(ceilDiv(columns, shape.threadsPerRow));
+        shape.gridY = static_cast<uint32_t>(shape.split);
+        finishSplit(g.output_elements);
+        return shape;
     }
     shape.vec = 1;
     if (shape.reducedStrides.back() == 1) {
@@ -392,13 +428,44 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             body = "thor::reduceRows<gen::Cfg>(src, out, partials, scale);";
             break;
         case ReductionShape::Kernel::Columns:
-            s << "    static constexpr u64 kOuter = " << g.outer_size << "ull;\n";
             s << "    static constexpr u64 kR = " << g.reduction_size << "ull;\n";
-            s << "    static constexpr u64 kInner = " << g.inner_size << "ull;\n";
-            s << "    static constexpr u64 kOutOuterStride = " << g.tiled_output_outer_stride << "ull;\n";
-            s << "    static constexpr u64 kOutInnerStride = " << g.tiled_output_inner_stride << "ull;\n";
             s << "    static constexpr int kBatch = " << shape.unroll << ";\n";
             s << "    static constexpr int kLanesX = " << shape.threadsPerRow << ";\n";
+            s << "    static constexpr u64 kColumns = " << (g.output_elements / shape.vec) << "ull;\n";
+            if (shape.laneAxis < 0) {
+                // dense [outer, R, inner]
+                const uint64_t innerVectors = g.inner_size / shape.vec;
+                s << "    static __device__ __forceinline__ u64 columnBase(u64 c) { return (c / " << innerVectors << "ull) * " << (g.reduction_size * g.inner_size)
+                  << "ull + (c % " << innerVectors << "ull) * " << shape.vec << "ull; }\n";
+                s << "    static __device__ __forceinline__ u64 rowOffset(u64 r) { return r * " << g.inner_size << "ull; }\n";
+                s << "    static __device__ __forceinline__ u64 partialSlot(u64 c, int k) { return (c / " << innerVectors << "ull) * " << g.inner_size
+                  << "ull + (c % " << innerVectors << "ull) * " << shape.vec << "ull + k; }\n";
+                s << "    static __device__ __forceinline__ u64 outputIndex(u64 c, int k) { return (c / " << innerVectors << "ull) * "
+                  << g.tiled_output_outer_stride << "ull + ((c % " << innerVectors << "ull) * " << shape.vec << "ull + k) * " << g.tiled_output_inner_stride
+                  << "ull; }\n";
+            } else {
+                // a view: columns enumerate the kept coordinates with the contiguous axis fastest (in vectors); outputs are
+                // numbered row-major over the kept axes in their logical order
+                const size_t lane = static_cast<size_t>(shape.laneAxis);
+                std::vector<uint64_t> logicalStride(shape.keptDims.size(), 1);
+                for (size_t a = shape.keptDims.size(); a-- > 1;) logicalStride[a - 1] = logicalStride[a] * shape.keptDims[a];
+                const uint64_t laneVectors = shape.keptDims[lane] / shape.vec;
+                std::ostringstream base, slot;
+                base << "    static __device__ __forceinline__ u64 columnBase(u64 c) {\n        u64 offset = (c % " << laneVectors << "ull) * " << shape.vec
+                     << "ull;\n        c /= " << laneVectors << "ull;\n";
+                slot << "    static __device__ __forceinline__ u64 partialSlot(u64 c, int k) {\n        u64 index = ((c % " << laneVectors << "ull) * " << shape.vec
+                     << "ull + k) * " << logicalStride[lane] << "ull;\n        c /= " << laneVectors << "ull;\n";
+                for (size_t a = shape.keptDims.size(); a-- > 0;) {
+                    if (a == lane) continue;
+                    base << "        offset += (c % " << shape.keptDims[a] << "ull) * " << shape.keptStrides[a] << "ull;\n        c /= " << shape.keptDims[a] << "ull;\n";
+                    slot << "        index += (c % " << shape.keptDims[a] << "ull) * " << logicalStride[a] << "ull;\n        c /= " << shape.keptDims[a] << "ull;\n";
+                }
+                base << "        return offset;\n    }\n";
+                slot << "        return index;\n    }\n";
+                s << base.str() << slot.str();
+                s << "    static __device__ __forceinline__ u64 outputIndex(u64 c, int k) { return partialSlot(c, k); }\n";
+                s << offsetFunction("rowOffset", shape.reducedDims, shape.reducedStrides);
+            }
             body = "thor::reduceColumns<gen::Cfg>(src, out, partials, scale);";
             break;
         case ReductionShape::Kernel::Strided: {
@@ -415,7 +482,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
         }
     }
     // layout of the final store made by the second stage of split kernels
-    if (shape.kernel == ReductionShape::Kernel::Columns) {
+    if (shape.kernel == ReductionShape::Kernel::Columns && shape.laneAxis < 0) {
         s << "    static constexpr u64 kFinishInner = " << g.inner_size << "ull;\n";
         s << "    static constexpr u64 kFinishOuterStride = " << g.tiled_output_outer_stride << "ull;\n";
         s << "    static constexpr u64 kFinishInnerStride = " << g.tiled_output_inner_stride << "ull;\n";

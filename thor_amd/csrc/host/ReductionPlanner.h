@@ -55,6 +55,9 @@ struct ReductionShape {
     size_t workspaceBytes = 0;
     // collapsed axes of the strided kernel
     std::vector<uint64_t> keptDims, keptStrides, reducedDims, reducedStrides;
+    // Columns kernel over a view: index (into keptDims) of the kept axis that is contiguous in memory, or -1 for the
+    // dense [outer, R, inner] layout
+    int laneAxis = -1;
     std::string describe() const;
 };
 
