@@ -186,6 +186,11 @@ def bench_other_configs():
     stats = ex.compile(ex.outputs({"sum": ix.reduce_sum(axis=[0, 2, 3], squeeze=True), "sumsq": (ix * ix).reduce_sum(axis=[0, 2, 3], squeeze=True)}), 0)
     plans = [stats.stamp({"x": t}, stream) for t in xc8]
     timed("c5_channel_sum_and_sumsq_fp16", [p_.run for p_ in plans], 2 * n, n, ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
+    y = (ex.input("x") * ex.input("scale") + ex.input("bias")).max(0.0)
+    all3 = ex.compile(ex.outputs({"y": y, "sum": ix.reduce_sum(axis=[0, 2, 3], squeeze=True), "sumsq": (ix * ix).reduce_sum(axis=[0, 2, 3], squeeze=True)}), 0)
+    plans = [all3.stamp({"x": t, "scale": scale, "bias": bias}, stream) for t in xc8]
+    timed("c5_relu_and_channel_statistics_one_pass_fp16", [p_.run for p_ in plans], 4 * n, n,
+          ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
     return results
 
 

@@ -90,13 +90,14 @@ class StampedArgMinMax {
 };
 
 // Several value reductions over one geometry evaluated in a single pass over their common sources, with the
-// elementwise work that feeds them computed in registers (sum(x) and sum(x*x) of one tensor: one read of x).
+// elementwise work that feeds them computed in registers (sum(x) and sum(x*x) of one tensor: one read of x), optionally
+// writing same-shaped elementwise results of those sources in the same pass.
 class StampedFusedReduction {
    public:
     StampedFusedReduction(ReductionLaunchPlan plan, std::vector<Tensor> inputs, std::vector<std::string> scalarNames, std::vector<Tensor> outputs,
-                          std::optional<Tensor> workspace, uint64_t flops)
+                          std::vector<Tensor> elementwiseOutputs, std::optional<Tensor> workspace, uint64_t flops)
         : plan(std::move(plan)), inputs(std::move(inputs)), scalarNames(std::move(scalarNames)), outputs(std::move(outputs)),
-          workspace(std::move(workspace)), flops(flops) {}
+          elementwiseOutputs(std::move(elementwiseOutputs)), workspace(std::move(workspace)), flops(flops) {}
     void runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const;
     const std::vector<Tensor>& getOutputTensors() const { return outputs; }
     const std::vector<std::string>& runtimeScalarNames() const { return scalarNames; }
@@ -109,6 +110,7 @@ class StampedFusedReduction {
     std::vector<Tensor> inputs;
     std::vector<std::string> scalarNames;
     std::vector<Tensor> outputs;
+    std::vector<Tensor> elementwiseOutputs;  // tensors of the input's shape written by the same pass
     std::optional<Tensor> workspace;
     uint64_t flops;
 };

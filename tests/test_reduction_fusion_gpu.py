@@ -88,7 +88,7 @@ def test_mixed_operations_scalars_and_output_dtypes(gpu):
         np.testing.assert_allclose(outs["sum16"].reshape(-1).astype(np.float64), v64.sum(axis=0), rtol=1e-3)
 
 
-def test_values_that_something_else_needs_are_still_materialised(gpu):
+def test_values_that_something_else_needs_are_written_by_the_same_pass(gpu):
     rng = np.random.default_rng(6)
     x = rng.standard_normal((32, 48)).astype(np.float32)
     ix = ex.input("x")
@@ -96,10 +96,72 @@ def test_values_that_something_else_needs_are_still_materialised(gpu):
     outputs = ex.outputs({"sq": sq, "colsum": sq.reduce_sum(axis=0), "colmax": sq.reduce_max(axis=0)})
     plan, outs = run_staged(outputs, {"x": x}, DataType.fp32)
     kinds = plan.stage_kind_names()
-    assert kinds == ["FusedKernel", "FusedReduction"], kinds  # sq is an output: written once, then both reductions read it together
+    assert kinds == ["FusedReduction"], kinds  # sq is an output: the pass that reduces it also writes it
+    assert "elementwise_outputs=1" in plan.stage_descriptions()[0]
     np.testing.assert_array_equal(outs["sq"], x * x)
     np.testing.assert_allclose(outs["colsum"].reshape(-1), (x.astype(np.float64) ** 2).sum(axis=0), rtol=1e-5)
     np.testing.assert_array_equal(outs["colmax"].reshape(-1), (x * x).max(axis=0))
+    _, outs_s = staged(outputs, {"x": x}, DataType.fp32)
+    np.testing.assert_array_equal(outs["sq"], outs_s["sq"])
+    np.testing.assert_array_equal(outs["colmax"], outs_s["colmax"])
+
+
+@pytest.mark.parametrize("stats_of", ["input", "output"])
+@pytest.mark.parametrize("shape", [(4, 16, 6, 10), (3, 8, 7, 9)], ids=lambda s: "x".join(map(str, s)))
+def test_per_channel_scale_bias_relu_with_statistics_in_one_pass(gpu, shape, stats_of):
+    """BASELINE config 5's three results from one read of x: y = relu(x*scale+bias) with [1,C,1,1] scale and bias, plus
+    per-channel sum and sum of squares (of x, or of y)."""
+    rng = np.random.default_rng(1238)
+    C = shape[1]
+    x = to_storage(rng.standard_normal(shape).astype(np.float32), DataType.fp16)
+    scale = to_storage(rng.uniform(0.5, 1.5, (1, C, 1, 1)).astype(np.float32), DataType.fp16)
+    bias = to_storage(rng.uniform(-0.1, 0.1, (1, C, 1, 1)).astype(np.float32), DataType.fp16)
+    ix, isc, ib = ex.input("x"), ex.input("scale"), ex.input("bias")
+    y = (ix * isc + ib).max(0.0)
+    v = ix if stats_of == "input" else y
+    outputs = ex.outputs({"y": y, "sum": v.reduce_sum(axis=[0, 2, 3], squeeze=True), "sumsq": (v * v).reduce_sum(axis=[0, 2, 3], squeeze=True)})
+    inputs = {"x": x, "scale": scale, "bias": bias}
+    plan, outs = run_staged(outputs, inputs, DataType.fp16)
+    assert plan.stage_kind_names() == ["FusedReduction"], plan.stage_descriptions()
+    plan_s, outs_s = staged(outputs, inputs, DataType.fp16)
+    assert len(plan_s.stage_kind_names()) >= 3
+    # the elementwise result involves no accumulation: bit-identical to the staged plan and to fp16 arithmetic rounded per operation
+    np.testing.assert_array_equal(outs["y"].view(np.uint16), outs_s["y"].view(np.uint16))
+    xf, sf, bf = (from_storage(a, DataType.fp16) for a in (x, scale, bias))
+    h = lambda a: from_storage(to_storage(a, DataType.fp16), DataType.fp16)
+    want_y = np.maximum(h(h(xf * sf) + bf), 0)
+    np.testing.assert_array_equal(from_storage(outs["y"], DataType.fp16), want_y)
+    vf = xf if stats_of == "input" else want_y
+    want_sum = vf.astype(np.float64).sum(axis=(0, 2, 3))
+    want_sq = h(vf * vf).astype(np.float64).sum(axis=(0, 2, 3))
+    assert np.all(np.abs(outs["sum"].astype(np.float64) - want_sum) <= 1e-5 * np.abs(vf).astype(np.float64).sum(axis=(0, 2, 3)) + 1e-30)
+    np.testing.assert_allclose(outs["sumsq"].astype(np.float64), want_sq, rtol=1e-5)
+    for name in ("sum", "sumsq"):
+        np.testing.assert_allclose(outs[name], outs_s[name], rtol=2e-5, atol=1e-4)
+
+
+def test_per_row_and_scalar_operands_in_row_and_column_geometries(gpu):
+    rng = np.random.default_rng(15)
+    x = rng.standard_normal((48, 100003)).astype(np.float32)   # rows too long for the register-resident row kernel
+    w = rng.uniform(0.5, 2.0, (48, 1)).astype(np.float32)      # one weight per row: a kept operand of the row reduction
+    c = np.array([0.75], dtype=np.float32)
+    ix, iw, ic = ex.input("x"), ex.input("w"), ex.input("c")
+    v = ix * iw + ic
+    outputs = ex.outputs({"rowsum": v.reduce_sum(axis=1), "rowmax": v.reduce_max(axis=1)})
+    plan, outs = run_staged(outputs, {"x": x, "w": w, "c": c}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedReduction"], plan.stage_descriptions()
+    v64 = x.astype(np.float64) * w + 0.75
+    np.testing.assert_allclose(outs["rowsum"].reshape(-1), v64.sum(axis=1), rtol=1e-5, atol=1e-2)
+    np.testing.assert_allclose(outs["rowmax"].reshape(-1), v64.max(axis=1), rtol=1e-6)
+    # column geometry: one weight per column
+    y = rng.standard_normal((1000, 96)).astype(np.float32)
+    g = rng.uniform(0.5, 2.0, (96,)).astype(np.float32)
+    iy, ig = ex.input("y"), ex.input("g")
+    outputs = ex.outputs({"colsum": (iy * ig).reduce_sum(axis=0, squeeze=True), "colsq": (iy * iy).reduce_sum(axis=0, squeeze=True)})
+    plan, outs = run_staged(outputs, {"y": y, "g": g}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedReduction"], plan.stage_descriptions()
+    np.testing.assert_allclose(outs["colsum"], (y.astype(np.float64) * g).sum(axis=0), rtol=1e-5, atol=1e-3)
+    np.testing.assert_allclose(outs["colsq"], (y.astype(np.float64) ** 2).sum(axis=0), rtol=1e-5)
 
 
 def test_config5_per_channel_statistics_at_full_size(gpu):

@@ -58,11 +58,12 @@ def test_softmax_single_pass_matches_staged_and_closed_form(gpu, dtype, shape):
     np.testing.assert_allclose(got.astype(np.float64).sum(axis=1), 1.0, rtol=max(rtol, 1e-5))
 
 
-def test_row_longer_than_the_register_budget_falls_back_to_the_staged_plan(gpu):
+def test_row_longer_than_the_register_budget_uses_streaming_stages(gpu):
     rng = np.random.default_rng(5)
     x = rng.standard_normal((3, 70001)).astype(np.float32)
     plan, outs = run_staged(softmax_expr(), {"x": x}, DataType.fp32)
-    assert plan.stage_kind_names() == ["Reduction", "FusedKernel", "Reduction", "FusedKernel"]
+    # no register-resident row kernel; the row sum and the exp that feeds it still share one pass
+    assert plan.stage_kind_names() == ["Reduction", "FusedReduction", "FusedKernel"], plan.stage_descriptions()
     x64 = x.astype(np.float64)
     p = np.exp(x64 - x64.max(axis=1, keepdims=True))
     np.testing.assert_allclose(outs["output"], p / p.sum(axis=1, keepdims=True), rtol=3e-6, atol=1e-12)

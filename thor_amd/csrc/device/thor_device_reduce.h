@@ -9,7 +9,10 @@
 //   Loaded                        the words loaded for one vector position: Cfg::load(sources, elementOffset, loaded)
 //   Acc                           ValueAcc<Op>, ArgAcc<IS_MAX, IndexT> or a generated struct of several ValueAcc members with
 //                                 the same protocol (reset, merge, shuffleXor, storePartial, loadPartial, partialBytes)
-//   accumulateOne(acc, loaded, sources, k, index)   evaluates element k of a loaded vector and adds it under `index`
+//   Kept, loadKept(sources, outputSlot, kept)       values that depend only on the output (per-channel scale, scalars)
+//   accumulateOne(acc, loaded, sources, kept, k, index)   evaluates element k of a loaded vector and adds it under `index`
+//   elementwise<KS>(sources, outputs, offset, loaded, kept)   optional same-shaped outputs computed from the loaded vector
+//                                 and stored at the same offset (element k uses kept[k * KS])
 //   Outputs, store(acc, outIndex, outputs, scale)   finalises (mean divide, L2 square root), scales, converts, stores
 //   IndexT                        u32 or u64: type of element offsets and of arg indices inside the kernel
 //   kVec                          elements per vector load (all shapes and base addresses are multiples of it)
@@ -36,6 +39,8 @@ __device__ __forceinline__ void reduceAll(const typename Cfg::Sources& src, cons
     __shared__ Acc scratch[Cfg::kThreads / kWave];
     Acc acc;
     acc.reset();
+    typename Cfg::Kept kept;
+    Cfg::loadKept(src, 0, kept);
     for (IndexT base = (IndexT)blockIdx.x * kChunk; base < kVectors; base += (IndexT)Cfg::kBlocks * kChunk) {
         typename Cfg::Loaded x[Cfg::kUnroll];
         bool live[Cfg::kUnroll];
@@ -50,7 +55,8 @@ __device__ __forceinline__ void reduceAll(const typename Cfg::Sources& src, cons
             if (live[u]) {
                 const IndexT v = base + (IndexT)u * Cfg::kThreads + threadIdx.x;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, k, (IndexT)(v * Cfg::kVec + k));
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, kept, k, (IndexT)(v * Cfg::kVec + k));
+                Cfg::template elementwise<0>(src, out, (u64)v * Cfg::kVec, x[u], &kept);
             }
         }
     }
@@ -112,6 +118,8 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
 
     Acc acc;
     acc.reset();
+    typename Cfg::Kept kept;
+    Cfg::loadKept(src, rowLive ? row : 0, kept);
     constexpr int kBatch = kIters >= 8 ? 8 : (int)(kIters > 0 ? kIters : 1);
     for (u64 it = 0; it < kIters; it += kBatch) {
         typename Cfg::Loaded x[kBatch];
@@ -127,7 +135,8 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
             if (live[u]) {
                 const u64 v = vBegin + (it + u) * TPR + lane;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, k, (IndexT)(v * Cfg::kVec + k));
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, kept, k, (IndexT)(v * Cfg::kVec + k));
+                Cfg::template elementwise<0>(src, out, rowBase + v * Cfg::kVec, x[u], &kept);
             }
         }
     }
@@ -171,8 +180,12 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
     const u64 base = Cfg::columnBase(safeColumn);
 
     Acc acc[Cfg::kVec];
+    typename Cfg::Kept kept[Cfg::kVec];
 #pragma unroll
-    for (int k = 0; k < Cfg::kVec; ++k) acc[k].reset();
+    for (int k = 0; k < Cfg::kVec; ++k) {
+        acc[k].reset();
+        Cfg::loadKept(src, Cfg::partialSlot(safeColumn, k), kept[k]);
+    }
     for (u64 r0 = rBegin + group; r0 < rEnd; r0 += (u64)kGroups * kBatch) {
         typename Cfg::Loaded x[kBatch];
         bool live[kBatch];
@@ -187,7 +200,8 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
             if (live[u]) {
                 const u64 r = r0 + (u64)u * kGroups;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, k, (IndexT)r);
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, (IndexT)r);
+                Cfg::template elementwise<1>(src, out, base + Cfg::rowOffset(r), x[u], kept);
             }
         }
     }
@@ -235,6 +249,8 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::Sources& src, 
 
     Acc acc;
     acc.reset();
+    typename Cfg::Kept kept;
+    Cfg::loadKept(src, output, kept);
     constexpr int kBatch = 4;
     for (u64 r0 = rBegin + threadIdx.x; r0 < rEnd; r0 += (u64)Cfg::kThreads * kBatch) {
         typename Cfg::Loaded x[kBatch];
@@ -250,7 +266,8 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::Sources& src, 
             if (live[u]) {
                 const u64 r = r0 + (u64)u * Cfg::kThreads;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, k, (IndexT)(r * Cfg::kVec + k));
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, kept, k, (IndexT)(r * Cfg::kVec + k));
+                Cfg::template elementwise<0>(src, out, base + Cfg::reducedOffset(r), x[u], &kept);
             }
         }
     }

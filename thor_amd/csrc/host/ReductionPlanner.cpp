@@ -163,7 +163,8 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
     if (!request.values.empty()) {
         elementBytes = 1;
         for (const ReductionKernelRequest::Source& source : request.sources)
-            if (!source.scalar) elementBytes = std::max(elementBytes, dataTypeSizeInBytes(source.storage));
+            if (source.kind == ReductionKernelRequest::Source::Kind::Vector) elementBytes = std::max(elementBytes, dataTypeSizeInBytes(source.storage));
+        for (const ReductionKernelRequest::Elementwise& e : request.elementwise) elementBytes = std::max(elementBytes, dataTypeSizeInBytes(e.outputDType));
     }
     const uint64_t accumulators = request.values.empty() ? 1 : request.values.size();
     ReductionShape shape;
@@ -318,7 +319,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     std::vector<ReductionKernelRequest::Value> values = request.values;
     std::string prologue = request.prologue;
     if (values.empty()) {
-        sources = {{request.inputDType, false}};
+        sources = {{request.inputDType, ReductionKernelRequest::Source::Kind::Vector}};
         values = {{request.valueOp, request.valueOutputDType, "x0"}};
         prologue = "        const float x0 = toFloat(l.p0.v[k]);\n";
     } else if (request.isArg) {
@@ -337,27 +338,29 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     s << "    static constexpr float kDivisor = (float)" << g.reduction_size << "ull;\n";
 
     // what the prologue reads
+    typedef ReductionKernelRequest::Source::Kind SourceKind;
     s << "    struct Sources {\n";
     for (size_t i = 0; i < sources.size(); ++i) s << "        const " << deviceTypeName(sources[i].storage) << "* in" << i << ";\n";
     for (uint32_t slot : request.scalarSlots) s << "        float s" << slot << ";\n";
     s << "    };\n    struct Loaded {\n";
-    for (size_t i = 0; i < sources.size(); ++i) {
-        if (sources[i].scalar) {
-            s << "        " << deviceTypeName(sources[i].storage) << " z" << i << ";\n";
-        } else {
-            s << "        Pack<" << deviceTypeName(sources[i].storage) << ", kVec> p" << i << ";\n";
-        }
-    }
+    for (size_t i = 0; i < sources.size(); ++i)
+        if (sources[i].kind == SourceKind::Vector) s << "        Pack<" << deviceTypeName(sources[i].storage) << ", kVec> p" << i << ";\n";
     s << "    };\n";
     s << "    static __device__ __forceinline__ void load(const Sources& s, u64 offset, Loaded& l) {\n";
+    for (size_t i = 0; i < sources.size(); ++i)
+        if (sources[i].kind == SourceKind::Vector) s << "        l.p" << i << ".loadStream(s.in" << i << " + offset);\n";
+    s << "        (void)s; (void)offset; (void)l;\n    }\n";
+    // values that depend only on the output
+    s << "    struct Kept {\n";
+    for (size_t i = 0; i < sources.size(); ++i)
+        if (sources[i].kind != SourceKind::Vector) s << "        " << deviceTypeName(sources[i].storage) << " z" << i << ";\n";
+    s << "    };\n";
+    s << "    static __device__ __forceinline__ void loadKept(const Sources& s, u64 slot, Kept& kk) {\n";
     for (size_t i = 0; i < sources.size(); ++i) {
-        if (sources[i].scalar) {
-            s << "        l.z" << i << " = s.in" << i << "[0];\n";
-        } else {
-            s << "        l.p" << i << ".loadStream(s.in" << i << " + offset);\n";
-        }
+        if (sources[i].kind == SourceKind::Scalar) s << "        kk.z" << i << " = s.in" << i << "[0];\n";
+        if (sources[i].kind == SourceKind::Kept) s << "        kk.z" << i << " = s.in" << i << "[slot];\n";
     }
-    s << "        (void)offset;\n    }\n";
+    s << "        (void)s; (void)slot; (void)kk;\n    }\n";
 
     // accumulators
     std::vector<int> finalize(values.size(), 0);
@@ -385,19 +388,32 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
         for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".loadPartial(base + " << j << " * stride, slot, slots);\n";
         s << "        }\n    };\n";
     }
-    s << "    static __device__ __forceinline__ void accumulateOne(Acc& acc, const Loaded& l, const Sources& s, int k, IndexT index) {\n";
+    s << "    static __device__ __forceinline__ void accumulateOne(Acc& acc, const Loaded& l, const Sources& s, const Kept& kk, int k, IndexT index) {\n";
     s << prologue;
     if (request.isArg || values.size() == 1) {
         s << "        acc.add(" << values[0].expression << ", index);\n";
     } else {
         for (size_t j = 0; j < values.size(); ++j) s << "        acc.a" << j << ".add(" << values[j].expression << ", index);\n";
     }
-    s << "        (void)l; (void)s; (void)k; (void)index;\n    }\n";
+    s << "        (void)l; (void)s; (void)kk; (void)k; (void)index;\n    }\n";
 
     // results
     s << "    struct Outputs {\n";
     for (size_t j = 0; j < values.size(); ++j) s << "        " << deviceTypeName(values[j].outputDType) << "* out" << j << ";\n";
+    for (size_t j = 0; j < request.elementwise.size(); ++j) s << "        " << deviceTypeName(request.elementwise[j].outputDType) << "* e" << j << ";\n";
     s << "        " << (request.indexOutputDType == DataType::UINT64 ? "u64" : "u32") << "* indexOut;\n    };\n";
+    // same-shaped outputs written by the pass that reads the sources
+    s << "    template <int KS>\n    static __device__ __forceinline__ void elementwise(const Sources& s, const Outputs& o, u64 offset, const Loaded& l, "
+         "const Kept* kept) {\n";
+    if (!request.elementwise.empty()) {
+        for (size_t j = 0; j < request.elementwise.size(); ++j)
+            s << "        Pack<" << deviceTypeName(request.elementwise[j].outputDType) << ", kVec> q" << j << ";\n";
+        s << "#pragma unroll\n        for (int k = 0; k < kVec; ++k) {\n        const Kept& kk = kept[k * KS];\n" << prologue;
+        for (size_t j = 0; j < request.elementwise.size(); ++j) s << "        q" << j << ".v[k] = " << request.elementwise[j].expression << ";\n";
+        s << "        }\n";
+        for (size_t j = 0; j < request.elementwise.size(); ++j) s << "        q" << j << ".storeStream(o.e" << j << " + offset);\n";
+    }
+    s << "        (void)s; (void)o; (void)offset; (void)l; (void)kept;\n    }\n";
     s << "    static __device__ __forceinline__ void store(const Acc& acc, u64 outIndex, const Outputs& o, float scale) {\n";
     if (request.isArg) {
         if (request.writeValue) s << "        o.out0[outIndex] = fromFloat<" << deviceTypeName(values[0].outputDType) << ">(acc.v);\n";
@@ -492,14 +508,23 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     }
     s << "};\n}  // namespace gen\n";
 
-    // kernel signatures: sources, runtime scalars, outputs, index output, partials, scale
-    std::ostringstream outputParams, outputInit;
+    // kernel signatures: sources, runtime scalars, reduction outputs, elementwise outputs, index output, partials, scale
+    std::ostringstream outputParams, outputInit, finishParams, finishInit;
     for (size_t j = 0; j < values.size(); ++j) {
         outputParams << deviceTypeName(values[j].outputDType) << "* out" << j << ", ";
         outputInit << "out" << j << ", ";
     }
+    finishParams << outputParams.str();
+    finishInit << outputInit.str();
+    for (size_t j = 0; j < request.elementwise.size(); ++j) {
+        outputParams << deviceTypeName(request.elementwise[j].outputDType) << "* e" << j << ", ";
+        outputInit << "e" << j << ", ";
+        finishInit << "nullptr, ";
+    }
     outputParams << "void* indexOut";
+    finishParams << "void* indexOut";
     outputInit << "static_cast<decltype(gen::Cfg::Outputs::indexOut)>(indexOut)";
+    finishInit << "static_cast<decltype(gen::Cfg::Outputs::indexOut)>(indexOut)";
     s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads << ") void thor_reduce_main(";
     for (size_t i = 0; i < sources.size(); ++i) s << "const " << deviceTypeName(sources[i].storage) << "* in" << i << ", ";
     for (uint32_t slot : request.scalarSlots) s << "float s" << slot << ", ";
@@ -510,7 +535,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     const bool twoStageAll = shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1;
     if (twoStageAll || shape.split > 1) {
         s << "extern \"C\" __global__ __launch_bounds__(" << (twoStageAll ? 1024 : 256) << ") void thor_reduce_finish(const void* partials, "
-          << outputParams.str() << ", float scale) {\n    const gen::Cfg::Outputs out{" << outputInit.str() << "};\n    thor::"
+          << finishParams.str() << ", float scale) {\n    const gen::Cfg::Outputs out{" << finishInit.str() << "};\n    thor::"
           << (twoStageAll ? "finishAll" : "finishPartials") << "<gen::Cfg>(partials, out, scale);\n}\n";
     }
     return s.str();

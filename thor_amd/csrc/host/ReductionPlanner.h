@@ -26,20 +26,31 @@ struct ReductionKernelRequest {
     // ---- fused form: several value reductions over the same geometry, fed by an elementwise prologue ------------------
     // When `values` is empty the request is the plain one above: one source of inputDType, the value itself reduced.
     struct Source {
+        enum class Kind : uint8_t {
+            Vector,  // same layout as the reduction input: read at the element offset
+            Scalar,  // one element, read at [0]
+            Kept,    // one element per output (numbered row-major over the kept axes), read at [output]: a per-channel scale
+        };
         DataType storage = DataType::FP32;
-        bool scalar = false;  // a one-element tensor read at [0] instead of at the element offset
+        Kind kind = Kind::Vector;
     };
     struct Value {
         CubReductionOp op = CubReductionOp::Sum;
         DataType outputDType = DataType::FP32;
         std::string expression;  // fp32 C expression of the value to accumulate, in terms of the prologue's names
     };
-    std::vector<Source> sources;         // kernel arguments in0, in1, ... ; vector sources share the reduction input's layout
+    struct Elementwise {
+        DataType outputDType = DataType::FP32;
+        std::string expression;  // storage-typed C expression of the element to store, in terms of the prologue's names
+    };
+    std::vector<Source> sources;         // kernel arguments in0, in1, ...
     std::vector<uint32_t> scalarSlots;   // runtime scalars passed by value as float s<slot>, after the sources
     // Statements evaluated once per element before the values are accumulated.  Element k of vector source i is
-    // `l.p<i>.v[k]`, scalar source i is `l.z<i>`, runtime scalars are `s.s<slot>`.
+    // `l.p<i>.v[k]`, scalar and kept source i is `kk.z<i>`, runtime scalars are `s.s<slot>`.
     std::string prologue;
     std::vector<Value> values;           // outputs out0, out1, ... in this order
+    // Tensors of the reduction input's shape written by the same pass (arguments e0, e1, ... after the reduction outputs).
+    std::vector<Elementwise> elementwise;
 };
 
 struct ReductionShape {

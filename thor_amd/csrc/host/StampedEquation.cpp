@@ -126,6 +126,11 @@ void StampedFusedReduction::runOn(Stream& stream, const std::unordered_map<std::
         outputPointers[i] = const_cast<Tensor&>(outputs[i]).getMemPtr();
         args.push_back(&outputPointers[i]);
     }
+    std::vector<void*> elementwisePointers(elementwiseOutputs.size());
+    for (size_t i = 0; i < elementwiseOutputs.size(); ++i) {
+        elementwisePointers[i] = const_cast<Tensor&>(elementwiseOutputs[i]).getMemPtr();
+        args.push_back(&elementwisePointers[i]);
+    }
     args.push_back(&indexOut);
     args.push_back(&partials);
     args.push_back(&scale);
