@@ -60,6 +60,43 @@ def cpu_baseline(seconds_budget: float = 12.0):
             "sample": f"{elems // (4 * n)} passes of the 4 conversions over 2^25 elements ({dt:.1f} s)"}
 
 
+def cpu_baseline_other_configs(seconds_each: float = 1.5):
+    """The oracle's host restatements of configs 1, 3, 4, 5 (OpenMP over all host cores) on bounded samples of the same
+    workloads; GB/s on the same algorithmic bytes as the GPU lines."""
+    import oracle
+    oracle.build()
+    rng = np.random.default_rng(99)
+    out = {}
+
+    def timed(name, fn, nbytes, sample):
+        threads = fn()  # warm-up, also pages the buffers in
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            threads = fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= seconds_each:
+                break
+        out[name] = {"GB/s": round(nbytes * reps / dt / 1e9, 2), "cores": int(threads), "kind": "port", "sample": f"{reps} passes over {sample} ({dt:.1f} s)"}
+
+    n = 1 << 24
+    a, b, c, d = (rng.uniform(-1, 1, n).astype(np.float32) for _ in range(4))
+    timed("c1_fused_elementwise_fp32", lambda: oracle.expr_config1(a, b, c, d)[1], 20 * n, "2^24 elements")
+    del a, b, c, d
+    x = rng.standard_normal((2048, 8192), dtype=np.float32)
+    timed("c3_row_sum_max_argmax_fp32", lambda: oracle.rows_f32(x)[3], 4 * x.size, "[2048, 8192] (sum, max and argmax in one pass)")
+    xs = oracle.convert((rng.standard_normal((2048, 4096), dtype=np.float32) * 3), oracle.FP32, oracle.BF16)
+    timed("c4_softmax_bf16", lambda: oracle.softmax_rows_bf16(xs)[1], 6 * xs.size, "[2048, 4096]")
+    xn = rng.standard_normal((8192, 1024), dtype=np.float32)
+    timed("c4_normalize_fp32", lambda: oracle.normalize_rows_f32(xn)[1], 8 * xn.size, "[8192, 1024]")
+    xc = rng.standard_normal((8, 256, 56, 56), dtype=np.float32).astype(np.float16)
+    sc = rng.uniform(0.5, 1.5, 256).astype(np.float16)
+    bi = rng.uniform(-0.1, 0.1, 256).astype(np.float16)
+    timed("c5_relu_scale_bias_fp16", lambda: oracle.relu_scale_bias_f16(xc, sc, bi)[1], 4 * xc.size, "[8, 256, 56, 56]")
+    timed("c5_channel_sum_and_sumsq_fp16", lambda: oracle.channel_stats_f16(xc)[2], 2 * xc.size, "[8, 256, 56, 56]")
+    return out
+
+
 def bench_other_configs():
     """BASELINE configs 1, 3, 4, 5 through the Expression / reduction API: GB/s on algorithmic bytes, HIP-event timed."""
     from thor_amd import physical as ph
@@ -290,6 +327,8 @@ def main():
         result["other_configs"] = bench_other_configs()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
+        if not args.no_other_configs:
+            result["cpu_baseline_other_configs"] = cpu_baseline_other_configs()
     print(json.dumps(result))
 
 

@@ -33,8 +33,8 @@ CARRIER = {
 
 def build(force: bool = False) -> str:
     """Compile libthor_oracle.so with gcc when missing (or when force is set)."""
-    src = os.path.join(_HERE, "thor_oracle.c")
-    stale = (not os.path.exists(_LIB_PATH)) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src)
+    sources = [os.path.join(_HERE, name) for name in ("thor_oracle.c", "thor_oracle_expr.c", "thor_oracle.h")]
+    stale = (not os.path.exists(_LIB_PATH)) or any(os.path.getmtime(_LIB_PATH) < os.path.getmtime(src) for src in sources)
     if force or stale:
         subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"], stdout=subprocess.DEVNULL)
     return _LIB_PATH
@@ -61,6 +61,13 @@ def lib() -> ctypes.CDLL:
         L.oracle_arg_reduce.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, u64p, u64p, ctypes.c_int, u32p, ctypes.c_int,
                                         ctypes.c_void_p, ctypes.c_void_p]
         L.oracle_dtype_size.argtypes = [ctypes.c_int]
+        vp, lg = ctypes.c_void_p, ctypes.c_long
+        L.oracle_expr_config1.argtypes = [vp, vp, vp, vp, vp, lg]
+        L.oracle_softmax_rows_bf16.argtypes = [vp, vp, lg, lg]
+        L.oracle_normalize_rows_f32.argtypes = [vp, vp, lg, lg, ctypes.c_float]
+        L.oracle_relu_scale_bias_f16.argtypes = [vp, vp, vp, vp, lg, lg, lg]
+        L.oracle_channel_stats_f16.argtypes = [vp, vp, vp, lg, lg, lg]
+        L.oracle_rows_f32.argtypes = [vp, vp, vp, vp, lg, lg]
         _lib = L
     return _lib
 
@@ -142,3 +149,62 @@ def arg_reduce(op: int, arr: np.ndarray, in_dtype: int, axes):
     if rc:
         raise ValueError("oracle_arg_reduce rejected the arguments")
     return idx, val
+
+
+# ---- BASELINE expression workloads on the host cores (thor_oracle_expr.c) ------------------------------------------------------
+def _c(a, dtype):
+    a = np.ascontiguousarray(a)
+    assert a.dtype == np.dtype(dtype), (a.dtype, dtype)
+    return a
+
+
+def expr_config1(a, b, c, d):
+    """out = (a*b + c) * sigmoid(d) in fp32; returns (out, threads)."""
+    a, b, c, d = (_c(v, np.float32) for v in (a, b, c, d))
+    out = np.empty_like(a)
+    threads = lib().oracle_expr_config1(a.ctypes.data, b.ctypes.data, c.ctypes.data, d.ctypes.data, out.ctypes.data, a.size)
+    return out, threads
+
+
+def softmax_rows_bf16(x_bits):
+    x_bits = _c(x_bits, np.uint16)
+    rows, cols = x_bits.shape
+    out = np.empty((rows, cols), dtype=np.float32)
+    threads = lib().oracle_softmax_rows_bf16(x_bits.ctypes.data, out.ctypes.data, rows, cols)
+    return out, threads
+
+
+def normalize_rows_f32(x, eps=1e-5):
+    x = _c(x, np.float32)
+    rows, cols = x.shape
+    out = np.empty_like(x)
+    threads = lib().oracle_normalize_rows_f32(x.ctypes.data, out.ctypes.data, rows, cols, eps)
+    return out, threads
+
+
+def relu_scale_bias_f16(x, scale, bias):
+    """x: float16 [N,C,H,W]; scale, bias: float16 with C elements."""
+    x, scale, bias = (_c(v, np.float16) for v in (x, scale, bias))
+    n, c = x.shape[0], x.shape[1]
+    hw = x.size // (n * c)
+    out = np.empty_like(x)
+    threads = lib().oracle_relu_scale_bias_f16(x.ctypes.data, scale.ctypes.data, bias.ctypes.data, out.ctypes.data, n, c, hw)
+    return out, threads
+
+
+def channel_stats_f16(x):
+    x = _c(x, np.float16)
+    n, c = x.shape[0], x.shape[1]
+    hw = x.size // (n * c)
+    total, squares = np.empty(c, np.float32), np.empty(c, np.float32)
+    threads = lib().oracle_channel_stats_f16(x.ctypes.data, total.ctypes.data, squares.ctypes.data, n, c, hw)
+    return total, squares, threads
+
+
+def rows_f32(x):
+    """row sums, row maxima and row argmax (uint32) of an fp32 matrix."""
+    x = _c(x, np.float32)
+    rows, cols = x.shape
+    s, m, a = np.empty(rows, np.float32), np.empty(rows, np.float32), np.empty(rows, np.uint32)
+    threads = lib().oracle_rows_f32(x.ctypes.data, s.ctypes.data, m.ctypes.data, a.ctypes.data, rows, cols)
+    return s, m, a, threads

@@ -92,6 +92,14 @@ int oracle_reduce_f64(int op, const void* in, int in_dtype, const uint64_t* dims
 int oracle_arg_reduce(int op, const void* in, int in_dtype, const uint64_t* dims, const uint64_t* strides, int rank,
                       const uint32_t* axes, int naxes, uint64_t* index_out, float* value_out);
 
+/* BASELINE expression workloads restated on the host (thor_oracle_expr.c); each returns the OpenMP thread count used. */
+int oracle_expr_config1(const float* a, const float* b, const float* c, const float* d, float* out, long n);
+int oracle_softmax_rows_bf16(const uint16_t* x, float* out, long rows, long cols);
+int oracle_normalize_rows_f32(const float* x, float* out, long rows, long cols, float eps);
+int oracle_relu_scale_bias_f16(const uint16_t* x, const uint16_t* scale, const uint16_t* bias, uint16_t* out, long n, long c, long hw);
+int oracle_channel_stats_f16(const uint16_t* x, float* sum, float* sumsq, long n, long c, long hw);
+int oracle_rows_f32(const float* x, float* row_sum, float* row_max, uint32_t* row_argmax, long rows, long cols);
+
 #ifdef __cplusplus
 }
 #endif
