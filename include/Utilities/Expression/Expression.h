@@ -67,6 +67,14 @@ inline bool isValueReductionOp(ExprOp op) {
             return false;
     }
 }
+// Softmax spellings of the reference (it takes cuDNN's enums: Expression.h:736-738 there).  Channel = over axis 1 for every
+// other coordinate (NCHW semantics; the last axis of an [N, C] matrix), Instance = over every axis but the first.
+enum class SoftmaxAlgorithm : uint8_t { Fast = 0, Accurate = 1, Log = 2 };
+enum class SoftmaxMode : uint8_t { Instance = 0, Channel = 1 };
+
+// reduction_axes entry standing for "every axis except axis 0"
+constexpr uint64_t kReduceAllAxesButFirst = UINT64_MAX - 1;
+
 inline bool isArgReductionOp(ExprOp op) { return op == ExprOp::REDUCE_ARGMIN || op == ExprOp::REDUCE_ARGMAX; }
 inline bool isReductionOp(ExprOp op) { return isValueReductionOp(op) || isArgReductionOp(op); }
 
@@ -90,7 +98,12 @@ struct ExprNode {
     std::vector<uint64_t> unsqueeze_axes;
     std::vector<uint64_t> reshape_dims;    // one entry may be UINT64_MAX = inferred
     std::vector<uint64_t> fill_dims;
+    SoftmaxAlgorithm softmax_algorithm = SoftmaxAlgorithm::Accurate;  // SOFTMAX only
+    SoftmaxMode softmax_mode = SoftmaxMode::Channel;
 };
+
+// The axes a reduction node reduces for an input of `rank` dimensions: sorted, unique, validated ({} = all).
+std::vector<uint64_t> resolveReductionAxes(const std::vector<uint64_t>& reduction_axes, size_t rank);
 
 struct NamedInput {
     enum class Kind : uint8_t { Tensor, RuntimeScalarFp32, TensorRuntimeScalar };
@@ -273,6 +286,12 @@ class Expression {
     Expression hardSwish() const;
     Expression threshold(double threshold = 0.0, double value = 0.0) const;
     Expression swish() const;
+
+    // softmax / log-softmax over the channel axis (or over everything but the batch axis), fp32 arithmetic, result in
+    // the input's dtype (fp16 for fp8 inputs).  Lowered to max / exp / sum / divide, which a [N, C] input runs as one
+    // register-resident row kernel.
+    Expression softmax(SoftmaxAlgorithm algorithm = SoftmaxAlgorithm::Accurate, SoftmaxMode mode = SoftmaxMode::Channel) const;
+    Expression logSoftmax(SoftmaxMode mode = SoftmaxMode::Channel) const;
 
     // ---- shape -------------------------------------------------------------------------------------------------------
     Expression reshape(const std::vector<uint64_t>& new_dims) const;

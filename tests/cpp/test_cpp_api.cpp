@@ -251,6 +251,15 @@ static void softmaxPlansAndRowKernel(Stream& stream) {
     CHECK((staged.reductionPaths() == std::vector<CubReductionPath>{CubReductionPath::ContiguousFixedSegment, CubReductionPath::ContiguousFixedSegment}));
     staged.run();
     check(staged);
+    // Expression::softmax(): the same function, result in the input's dtype (the reference's softmax stage keeps it)
+    FusedEquation method = FusedEquation::compile(ix.softmax().expression(), 0);
+    StampedExecutionPlan viaMethod = method.stamp({{"x", tx}}, stream);
+    CHECK((viaMethod.stageKindNames() == std::vector<std::string>{"FusedRowKernel"}));
+    CHECK(viaMethod.output().getDataType() == DataType::BF16);
+    viaMethod.run();
+    const std::vector<float> rounded = toHostF32(viaMethod.output(), stream), exact = toHostF32(fused.output(), stream);
+    for (size_t i = 0; i < rounded.size(); i += 7) CHECK_NEAR(rounded[i], exact[i], 4e-3 * exact[i] + 1e-9);
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)ix.softmax(SoftmaxAlgorithm::Log); }));
 }
 
 static void typeConverterOnGpuAndTensorViews(Stream& stream) {

@@ -231,3 +231,46 @@ def test_config4_full_size_properties(gpu):
     y64 = y[rows].astype(np.float64)
     mu = y64.mean(axis=1, keepdims=True)
     np.testing.assert_allclose(z[rows], (y64 - mu) / np.sqrt(((y64 - mu) ** 2).mean(axis=1, keepdims=True) + 1e-5), rtol=2e-5, atol=2e-6)
+
+
+# ---- Expression.softmax() / log_softmax(): the reference lowers these to a cuDNN stage (Expression.cpp:3724-3750); here they
+# ---- lower to the composed form and, for [N, C] inputs, to one row kernel --------------------------------------------------
+def _softmax64(x, axes, log=False):
+    m = x.max(axis=axes, keepdims=True)
+    p = np.exp(x - m)
+    s = p.sum(axis=axes, keepdims=True)
+    return (x - m) - np.log(s) if log else p / s
+
+
+SOFTMAX_OUT_TOL = {DataType.fp32: 3e-6, DataType.fp16: 1.2e-3, DataType.bf16: 9e-3, DataType.fp8_e4m3: 1.2e-3}
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.bf16, DataType.fp8_e4m3], ids=lambda d: d.name)
+def test_softmax_method_on_matrices_is_one_row_kernel_and_keeps_the_input_dtype(gpu, dtype):
+    rng = np.random.default_rng(31)
+    x = to_storage((rng.standard_normal((65, 777)) * 2).astype(np.float32), dtype)
+    xf = from_storage(x, dtype).astype(np.float64)
+    out_dtype = DataType.fp16 if dtype == DataType.fp8_e4m3 else dtype  # fp8 inputs produce fp16, like the reference's softmax stage
+    for build, want in ((lambda e: e.softmax(), _softmax64(xf, 1)), (lambda e: e.softmax("fast"), _softmax64(xf, 1)),
+                        (lambda e: e.softmax("accurate", "instance"), _softmax64(xf, 1)), (lambda e: e.log_softmax(), _softmax64(xf, 1, log=True))):
+        plan, outs = run_staged(build(ex.input("x")), {"x": x}, dtype)
+        assert plan.stage_kind_names() == ["FusedRowKernel"], plan.stage_descriptions()
+        assert plan.output().get_data_type() == out_dtype
+        got = from_storage(outs["output"], out_dtype).astype(np.float64)
+        tol = SOFTMAX_OUT_TOL[dtype]
+        np.testing.assert_allclose(got, want, rtol=tol, atol=tol * 1e-2 if want.min() >= 0 else tol * 8)
+
+
+def test_softmax_channel_and_instance_modes_on_nchw(gpu):
+    rng = np.random.default_rng(32)
+    x = rng.standard_normal((3, 6, 5, 7)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    plan, outs = run_staged(ex.input("x").softmax(), {"x": x}, DataType.fp32)           # over C for every (n, h, w)
+    assert "FusedRowKernel" not in plan.stage_kind_names()
+    np.testing.assert_allclose(outs["output"], _softmax64(x64, 1), rtol=3e-6, atol=1e-9)
+    plan, outs = run_staged(ex.input("x").softmax("accurate", "instance"), {"x": x}, DataType.fp32)  # over C*H*W per sample
+    np.testing.assert_allclose(outs["output"], _softmax64(x64, (1, 2, 3)), rtol=3e-6, atol=1e-9)
+    plan, outs = run_staged(ex.input("x").log_softmax("instance"), {"x": x}, DataType.fp32)
+    np.testing.assert_allclose(outs["output"], _softmax64(x64, (1, 2, 3), log=True), rtol=3e-6, atol=3e-6)
+    with pytest.raises(RuntimeError, match="axis"):
+        run_staged(ex.input("x").softmax(), {"x": x.reshape(-1)}, DataType.fp32)

@@ -378,6 +378,40 @@ Expression Expression::threshold(double threshold, double value) const {
 }
 Expression Expression::swish() const { return *this * sigmoid(); }
 
+Expression Expression::softmax(SoftmaxAlgorithm algorithm, SoftmaxMode mode) const {
+    if (algorithm == SoftmaxAlgorithm::Log) {
+        throw std::invalid_argument("Expression::softmax computes ordinary softmax; use Expression::logSoftmax for the log form.");
+    }
+    Expression out = unaryOp(*this, ExprOp::SOFTMAX);
+    out.expr->nodes[out.nodeIndex].softmax_algorithm = algorithm;
+    out.expr->nodes[out.nodeIndex].softmax_mode = mode;
+    return out;
+}
+
+Expression Expression::logSoftmax(SoftmaxMode mode) const {
+    Expression out = unaryOp(*this, ExprOp::SOFTMAX);
+    out.expr->nodes[out.nodeIndex].softmax_algorithm = SoftmaxAlgorithm::Log;
+    out.expr->nodes[out.nodeIndex].softmax_mode = mode;
+    return out;
+}
+
+std::vector<uint64_t> resolveReductionAxes(const std::vector<uint64_t>& reduction_axes, size_t rank) {
+    std::vector<uint64_t> out;
+    if (reduction_axes.empty()) {
+        for (uint64_t a = 0; a < rank; ++a) out.push_back(a);
+    } else if (reduction_axes.size() == 1 && reduction_axes[0] == kReduceAllAxesButFirst) {
+        if (rank < 2) throw std::runtime_error("Reduction axis out of range.");
+        for (uint64_t a = 1; a < rank; ++a) out.push_back(a);
+    } else {
+        out = reduction_axes;
+        std::sort(out.begin(), out.end());
+        out.erase(std::unique(out.begin(), out.end()), out.end());
+    }
+    for (uint64_t a : out)
+        if (a >= rank) throw std::runtime_error("Reduction axis out of range.");
+    return out;
+}
+
 // ---- shape ---------------------------------------------------------------------------------------------------------------
 Expression Expression::reshape(const std::vector<uint64_t>& new_dims) const {
     if (new_dims.empty()) throw std::invalid_argument("Expression::reshape requires at least one dimension.");
@@ -496,6 +530,7 @@ bool Expression::isUnaryOp(ExprOp op) {
         case ExprOp::RESHAPE:
         case ExprOp::UNSQUEEZE:
         case ExprOp::SQUEEZE:
+        case ExprOp::SOFTMAX:
             return true;
         default:
             return op >= ExprOp::NEG && op <= ExprOp::NORMCDF;
@@ -521,7 +556,7 @@ std::string opName(ExprOp op) {
         {(uint16_t)ExprOp::LGAMMA, "lgamma"}, {(uint16_t)ExprOp::DIGAMMA, "digamma"}, {(uint16_t)ExprOp::EXP, "exp"},
         {(uint16_t)ExprOp::EXPM1, "expm1"}, {(uint16_t)ExprOp::EXP2, "exp2"}, {(uint16_t)ExprOp::EXP10, "exp10"}, {(uint16_t)ExprOp::LN, "ln"},
         {(uint16_t)ExprOp::LOG1P, "log1p"}, {(uint16_t)ExprOp::LOG2, "log2"}, {(uint16_t)ExprOp::LOG10, "log10"}, {(uint16_t)ExprOp::SQRT, "sqrt"},
-        {(uint16_t)ExprOp::TANH, "tanh"}, {(uint16_t)ExprOp::NORMCDF, "normcdf"}, {(uint16_t)ExprOp::FILL, "fill"},
+        {(uint16_t)ExprOp::TANH, "tanh"}, {(uint16_t)ExprOp::NORMCDF, "normcdf"}, {(uint16_t)ExprOp::SOFTMAX, "softmax"}, {(uint16_t)ExprOp::FILL, "fill"},
         {(uint16_t)ExprOp::RESHAPE, "reshape"}, {(uint16_t)ExprOp::UNSQUEEZE, "unsqueeze"}, {(uint16_t)ExprOp::SQUEEZE, "squeeze"},
         {(uint16_t)ExprOp::MIN, "min"}, {(uint16_t)ExprOp::MAX, "max"}, {(uint16_t)ExprOp::MIN_GRAD_LEFT, "min_grad_left"},
         {(uint16_t)ExprOp::MIN_GRAD_RIGHT, "min_grad_right"}, {(uint16_t)ExprOp::MAX_GRAD_LEFT, "max_grad_left"},
@@ -590,6 +625,9 @@ std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex,
         if (n.op == ExprOp::RESHAPE) text += ":dims=" + axesText(n.reshape_dims);
         if (n.op == ExprOp::UNSQUEEZE) text += ":axes=" + axesText(n.unsqueeze_axes);
         if (n.op == ExprOp::SQUEEZE) text += ":axes=" + axesText(n.squeeze_axes);
+        if (n.op == ExprOp::SOFTMAX) {
+            text += std::string(":alg=") + std::to_string(static_cast<int>(n.softmax_algorithm)) + ":mode=" + std::to_string(static_cast<int>(n.softmax_mode));
+        }
         text += "(";
         for (size_t i = 0; i < kids.size(); ++i) text += (i ? "," : "") + kids[i];
         text += ")";

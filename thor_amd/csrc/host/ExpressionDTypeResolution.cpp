@@ -70,6 +70,13 @@ DataType nodeOutputDType(const ExprNode& node, const std::vector<ExprNode>& node
         return out;
     }
     if (isComparison(node.op) || isLogical(node.op)) return node.output_dtype.value_or(DataType::BOOLEAN);
+    if (node.op == ExprOp::SOFTMAX) {
+        // the input's dtype, fp8 widened to fp16 (the reference's toSupportedInputDType for its softmax stage,
+        // Utilities/Expression/ExpressionDTypeResolution.cpp:259-272)
+        const DataType in = resolved[node.lhs];
+        if (!isSupportedFusionFloatingType(in)) throw std::runtime_error("Softmax requires a floating-point input.");
+        return node.output_dtype.value_or(isFp8Type(in) ? DataType::FP16 : in);
+    }
     if (node.op == ExprOp::WHERE) {
         if (resolved[node.lhs] != DataType::BOOLEAN) {
             throw std::runtime_error(std::string("Where condition must have BOOLEAN dtype, received: ") + dataTypeName(resolved[node.lhs]));
@@ -144,7 +151,7 @@ void propagateMaterialisedDTypes(PhysicalExpression& expr, const std::vector<uin
         auto toParent = [&](uint32_t p) { seed(required.at(p), flowing); };
         if (node.op == ExprOp::CAST) {
             // an explicit conversion boundary: the source keeps its own compute dtype
-        } else if (isReductionOp(node.op)) {
+        } else if (isReductionOp(node.op) || node.op == ExprOp::SOFTMAX) {
             // the reduction's mandatory fp32 stays inside the reduction; its producer keeps its own policy
             const ExprNode& producer = expr.nodes.at(node.lhs);
             if (producer.compute_dtype) {
@@ -197,6 +204,8 @@ void resolveInPlace(PhysicalExpression& expr, const std::vector<DataType>& rootD
         DataType requested;
         if (node.op == ExprOp::CAST || isShapeOnly(node.op)) {
             requested = out;
+        } else if (node.op == ExprOp::SOFTMAX) {
+            requested = DataType::FP32;  // fp32 arithmetic whatever the storage
         } else if (node.op == ExprOp::SUB && (logicalIn == DataType::UINT32 || logicalIn == DataType::UINT64) && logicalIn == out) {
             requested = logicalIn;  // exact unsigned differences stay in the integer domain
         } else if (isComparison(node.op)) {
@@ -282,7 +291,7 @@ DataType toSupportedComputeDType(ExprOp op, DataType requested) {
     }
     if (op == ExprOp::SUB && (requested == DataType::UINT32 || requested == DataType::UINT64)) return requested;
     if (!isSupportedFusionFloatingType(requested)) throw std::runtime_error("Unsupported dtype in toSupportedComputeDType.");
-    if (isReductionOp(op)) return DataType::FP32;
+    if (isReductionOp(op) || op == ExprOp::SOFTMAX) return DataType::FP32;
     if (isFp8Type(requested) || requested == DataType::FP16) return DataType::FP16;
     return requested;  // bf16 or fp32
 }

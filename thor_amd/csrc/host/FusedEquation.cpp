@@ -88,6 +88,30 @@ class GraphBuilder {
         return child;
     }
 
+    // softmax(x) = exp(x - max) / sum(exp(x - max)) over the channel axis (or every axis but the first), in fp32, converted
+    // once to the node's output dtype; Fast skips the max, Log returns (x - max) - ln(sum).  `node.lhs` is already translated.
+    uint32_t lowerSoftmax(const ExprNode& node) {
+        const uint32_t x = asTensorOperand(node.lhs, true);
+        const std::vector<uint64_t> axes = node.softmax_mode == SoftmaxMode::Channel ? std::vector<uint64_t>{1} : std::vector<uint64_t>{kReduceAllAxesButFirst};
+        auto make = [&](ExprOp op, uint32_t lhs, uint32_t rhs = UINT32_MAX) {
+            ExprNode n;
+            n.op = op;
+            n.lhs = lhs;
+            n.rhs = rhs;
+            n.compute_dtype = DataType::FP32;
+            n.output_dtype = DataType::FP32;
+            if (isReductionOp(op)) n.reduction_axes = axes;
+            return add(n);
+        };
+        uint32_t shifted = x;
+        if (node.softmax_algorithm != SoftmaxAlgorithm::Fast) shifted = make(ExprOp::SUB, x, make(ExprOp::REDUCE_MAX, x));
+        const uint32_t e = make(ExprOp::EXP, shifted);
+        const uint32_t sum = make(ExprOp::REDUCE_SUM, e);
+        const uint32_t result = node.softmax_algorithm == SoftmaxAlgorithm::Log ? make(ExprOp::SUB, shifted, make(ExprOp::LN, sum)) : make(ExprOp::DIV, e, sum);
+        const DataType outDType = node.output_dtype.value();
+        return outDType == DataType::FP32 ? result : castOf(result, outDType);
+    }
+
     uint32_t translate(uint32_t srcIndex) {
         auto it = remap.find(srcIndex);
         if (it != remap.end()) return it->second;
@@ -95,6 +119,11 @@ class GraphBuilder {
         if (node.lhs != UINT32_MAX) node.lhs = translate(node.lhs);
         if (node.rhs != UINT32_MAX) node.rhs = translate(node.rhs);
         if (node.aux != UINT32_MAX) node.aux = translate(node.aux);
+        if (node.op == ExprOp::SOFTMAX) {
+            const uint32_t idx = lowerSoftmax(node);
+            remap.emplace(srcIndex, idx);
+            return idx;
+        }
         if (isReductionOp(node.op)) {
             node.lhs = asTensorOperand(node.lhs, true);
         } else if (isShapeOnly(node.op)) {
@@ -183,19 +212,7 @@ std::vector<uint64_t> reshapeDims(const std::vector<uint64_t>& in, const std::ve
     return out;
 }
 
-std::vector<uint64_t> sortedAxesOrAll(const std::vector<uint64_t>& axes, size_t rank) {
-    std::vector<uint64_t> out = axes;
-    if (out.empty()) {
-        out.resize(rank);
-        std::iota(out.begin(), out.end(), 0);
-    } else {
-        std::sort(out.begin(), out.end());
-        out.erase(std::unique(out.begin(), out.end()), out.end());
-    }
-    for (uint64_t a : out)
-        if (a >= rank) throw std::runtime_error("Reduction axis out of range.");
-    return out;
-}
+std::vector<uint64_t> sortedAxesOrAll(const std::vector<uint64_t>& axes, size_t rank) { return resolveReductionAxes(axes, rank); }
 
 std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std::vector<Tensor>& boundInputs) {
     std::vector<std::vector<uint64_t>> dims(g.expr.nodes.size());

@@ -131,11 +131,7 @@ void tryReductionFusion(RowFusionContext& ctx) {
         if (ctx.done[i] || !isValueReductionOp(n.op) || ctx.role[i] != Role::Materialized) continue;
         const std::vector<uint64_t>& shape = ctx.dims[n.lhs];
         if (shape.empty() || product(shape) < 2) continue;
-        std::vector<uint64_t> axes = n.reduction_axes;
-        if (axes.empty())
-            for (uint64_t a = 0; a < shape.size(); ++a) axes.push_back(a);
-        std::sort(axes.begin(), axes.end());
-        axes.erase(std::unique(axes.begin(), axes.end()), axes.end());
+        const std::vector<uint64_t> axes = resolveReductionAxes(n.reduction_axes, shape.size());
         groups[Key(shape, axes)].push_back(i);
     }
 

@@ -79,6 +79,8 @@ struct Region {
 
 bool isLastAxisReduction(const ExprNode& n, const std::vector<uint64_t>& inDims) {
     if (!isValueReductionOp(n.op) || inDims.empty()) return false;
+    if (n.reduction_axes.empty()) return inDims.size() == 1;
+    if (n.reduction_axes.size() == 1 && n.reduction_axes[0] == kReduceAllAxesButFirst) return inDims.size() == 2;
     std::vector<uint64_t> axes = n.reduction_axes;
     std::sort(axes.begin(), axes.end());
     axes.erase(std::unique(axes.begin(), axes.end()), axes.end());

@@ -125,6 +125,12 @@ thor_expr_t thor_expr_unary_params(const char* method, thor_expr_t input, double
         if (m == "threshold") return new thor_expr{input->expr.threshold(p0, p1)};
         if (m == "log") return new thor_expr{input->expr.log(p0)};
         if (m == "clamp") return new thor_expr{input->expr.clamp(p0, p1)};
+        if (m == "softmax" || m == "logSoftmax") {  // p0: 0 fast, 1 accurate; p1: 0 instance, 1 channel
+            if ((p0 != 0.0 && p0 != 1.0) || (p1 != 0.0 && p1 != 1.0)) throw std::invalid_argument("Unknown softmax algorithm or mode.");
+            const SoftmaxMode mode = p1 == 0.0 ? SoftmaxMode::Instance : SoftmaxMode::Channel;
+            if (m == "logSoftmax") return new thor_expr{input->expr.logSoftmax(mode)};
+            return new thor_expr{input->expr.softmax(p0 == 0.0 ? SoftmaxAlgorithm::Fast : SoftmaxAlgorithm::Accurate, mode)};
+        }
         throw std::invalid_argument("Unknown parameterised Expression method: " + m);)
 }
 

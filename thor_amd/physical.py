@@ -552,6 +552,13 @@ class Expression:
     def log(self, base: float): return Expression(lib().thor_expr_unary_params(b"log", self._h, base, 0.0))
     def clamp(self, lo: float, hi: float): return Expression(lib().thor_expr_unary_params(b"clamp", self._h, lo, hi))
 
+    def softmax(self, algorithm: str = "accurate", mode: str = "channel") -> "Expression":
+        """Softmax over axis 1 ("channel") or over every axis but the first ("instance"); "fast" skips the max subtraction."""
+        return Expression(lib().thor_expr_unary_params(b"softmax", self._h, {"fast": 0.0, "accurate": 1.0}[algorithm], {"instance": 0.0, "channel": 1.0}[mode]))
+
+    def log_softmax(self, mode: str = "channel") -> "Expression":
+        return Expression(lib().thor_expr_unary_params(b"logSoftmax", self._h, 1.0, {"instance": 0.0, "channel": 1.0}[mode]))
+
     def reshape(self, dims: Sequence[int]) -> "Expression":
         d, rank = _u64_array([UINT64_MAX if v == -1 else v for v in dims])
         return Expression(lib().thor_expr_reshape(self._h, d, rank))
