@@ -36,10 +36,11 @@ struct CubArgReductionOutputOptions {
 };
 
 // Which kernel family a geometry maps to.  The names are the reference's; here they mean:
-//   DeviceTransformReduce   whole tensor (or a rank-1 strided view) -> one value, single launch with a last-block fold
+//   DeviceTransformReduce   whole tensor (or a rank-1 strided view) -> one value: per-block partials, then a one-block finishing launch
 //   ContiguousFixedSegment  [outer, R] rows, R contiguous: 1..64 lanes or one block per row
 //   TiledFixedSegment       [outer, R, inner] with inner > 1: one lane per inner vector, R optionally split
 //   StridedFixedSegment     anything else (disjoint axes, views): generated address arithmetic, R optionally split
+//   OffsetSegmented         [N, D...] rows reduced over runtime row ranges (CubSegmentedReduction below)
 enum class CubReductionPath : uint8_t {
     DeviceTransformReduce = 0,
     ContiguousFixedSegment = 1,
@@ -147,10 +148,69 @@ class CubArgReduction {
     CubArgReductionOutputOptions outputs;
 };
 
+class StampedCubSegmentedReduction;
+class StampedCubSegmentedArgReduction;
+
+// Offset-segmented reduction of dense values [N, D...] -> [B, D...] (reference: CubReduction.h:236-330).  Segment i is the
+// half-open row range [offsets[i], offsets[i + 1]) of a rank-1 UINT32 / UINT64 offsets tensor with B + 1 entries.  Inputs
+// convert to fp32, all arithmetic is fp32.  Empty segments give getFp32EmptyReductionValue(); a mean divides by the
+// segment's row count and is 0 for an empty segment.  Supported: sum, mean, min, max.  stamp() reads and validates the
+// offsets (zero based, non-decreasing, within N); stampRuntimeOffsets() only checks shapes and dtypes, for offsets that
+// are filled in later.  Either way the kernels read the offsets when they run, so the partition may change between runs.
+class CubSegmentedReduction {
+   public:
+    explicit CubSegmentedReduction(CubReductionOp op, std::optional<DataType> output_dtype = std::nullopt);
+
+    CubReductionOp getOperation() const { return op; }
+    std::optional<DataType> getConfiguredOutputDataType() const { return output_dtype; }
+    DataType resolveOutputDataType(DataType input_dtype) const { return output_dtype.value_or(input_dtype); }
+    static bool isInputDataTypeSupported(DataType dtype);
+    static bool isOffsetDataTypeSupported(DataType dtype) { return dtype == DataType::UINT32 || dtype == DataType::UINT64; }
+
+    std::shared_ptr<StampedCubSegmentedReduction> stamp(const Tensor& input, const Tensor& segment_offsets, const Stream& stream) const;
+    std::shared_ptr<StampedCubSegmentedReduction> stamp(const Tensor& input, const Tensor& preallocated_output, const Tensor& segment_offsets,
+                                                        const Stream& stream) const;
+    std::shared_ptr<StampedCubSegmentedReduction> stampRuntimeOffsets(const Tensor& input, const Tensor& preallocated_output,
+                                                                      const Tensor& segment_offsets, const Stream& stream) const;
+
+   private:
+    std::shared_ptr<StampedCubSegmentedReduction> stampValidated(const Tensor& input, const Tensor& output, const Tensor& segment_offsets,
+                                                                 const Stream& stream) const;
+    CubReductionOp op;
+    std::optional<DataType> output_dtype;
+};
+
+// Offset-segmented argmin / argmax over packed values [N, D...]: winners are global packed indices row * D + d, UINT64
+// (default) or UINT32; NaN wins, the lowest index wins ties, empty segments give the all-ones index of the output dtype
+// (reference: CubReduction.h:331-400).
+class CubSegmentedArgReduction {
+   public:
+    explicit CubSegmentedArgReduction(CubArgReductionOp op, DataType index_output_dtype = DataType::UINT64);
+
+    CubArgReductionOp getOperation() const { return op; }
+    DataType getIndexOutputDataType() const { return index_output_dtype; }
+    static bool isInputDataTypeSupported(DataType dtype) { return CubSegmentedReduction::isInputDataTypeSupported(dtype); }
+    static bool isOffsetDataTypeSupported(DataType dtype) { return CubSegmentedReduction::isOffsetDataTypeSupported(dtype); }
+
+    std::shared_ptr<StampedCubSegmentedArgReduction> stamp(const Tensor& input, const Tensor& segment_offsets, const Stream& stream) const;
+    std::shared_ptr<StampedCubSegmentedArgReduction> stamp(const Tensor& input, const Tensor& preallocated_index_output,
+                                                           const Tensor& segment_offsets, const Stream& stream) const;
+    std::shared_ptr<StampedCubSegmentedArgReduction> stampRuntimeOffsets(const Tensor& input, const Tensor& preallocated_index_output,
+                                                                         const Tensor& segment_offsets, const Stream& stream) const;
+
+   private:
+    std::shared_ptr<StampedCubSegmentedArgReduction> stampValidated(const Tensor& input, const Tensor& index_output, const Tensor& segment_offsets,
+                                                                    const Stream& stream) const;
+    CubArgReductionOp op;
+    DataType index_output_dtype;
+};
+
 // The launch recipe a stamp produced: up to two kernels (main + fold of split partials) with fixed grids.
 struct ReductionLaunchPlan {
     std::shared_ptr<CompiledKernel> mainKernel;
     std::shared_ptr<CompiledKernel> finishKernel;  // null unless the reduction domain was split across blocks
+    std::shared_ptr<CompiledKernel> prepareKernel; // offset-segmented reductions over several chunks: runs before the main kernel
+    uint32_t prepareGridX = 1, prepareThreads = 256;
     uint32_t mainGridX = 1, mainGridY = 1, mainThreads = 256;
     uint32_t finishGridX = 1, finishThreads = 256;
     size_t workspaceBytes = 0;  // per-block / per-share partials
@@ -223,6 +283,76 @@ class StampedCubArgReduction {
     const Tensor input;
     mutable std::optional<Tensor> value_output;
     mutable std::optional<Tensor> index_output;
+    ReductionLaunchPlan plan;
+    std::optional<Tensor> workspace;
+    Stream stream;
+};
+
+// Concrete offset-segmented reductions: run() launches only.
+class StampedCubSegmentedReduction {
+   public:
+    void run() { runOn(stream); }
+    void runOn(Stream& run_stream) const;
+
+    uint32_t gpuNum() const { return input.getPlacement().getDeviceNum(); }
+    Tensor getOutputTensor() const { return output; }
+    CubReductionOp getOperation() const { return op; }
+    CubReductionPath getPath() const { return CubReductionPath::OffsetSegmented; }
+    DataType getInputDataType() const { return input.getDataType(); }
+    DataType getOutputDataType() const { return output.getDataType(); }
+    DataType getAccumulatorDataType() const { return DataType::FP32; }
+    DataType getOffsetDataType() const { return segment_offsets.getDataType(); }
+    uint64_t getNumItems() const { return num_items; }
+    uint64_t getNumSegments() const { return num_segments; }
+    size_t getWorkspaceSizeInBytes() const { return plan.workspaceBytes; }
+    const std::string& getKernelVariant() const { return plan.variant; }
+
+   private:
+    friend class CubSegmentedReduction;
+    StampedCubSegmentedReduction(CubReductionOp op, const Tensor& input, const Tensor& output, const Tensor& segment_offsets, uint64_t num_items,
+                                 uint64_t num_segments, ReductionLaunchPlan plan, std::optional<Tensor> workspace, const Stream& stream)
+        : op(op), input(input), output(output), segment_offsets(segment_offsets), num_items(num_items), num_segments(num_segments),
+          plan(std::move(plan)), workspace(std::move(workspace)), stream(stream) {}
+
+    CubReductionOp op;
+    const Tensor input;
+    mutable Tensor output;
+    const Tensor segment_offsets;
+    const uint64_t num_items, num_segments;
+    ReductionLaunchPlan plan;
+    std::optional<Tensor> workspace;
+    Stream stream;
+};
+
+class StampedCubSegmentedArgReduction {
+   public:
+    void run() { runOn(stream); }
+    void runOn(Stream& run_stream) const;
+
+    uint32_t gpuNum() const { return input.getPlacement().getDeviceNum(); }
+    Tensor getIndexOutputTensor() const { return index_output; }
+    CubArgReductionOp getOperation() const { return op; }
+    CubReductionPath getPath() const { return CubReductionPath::OffsetSegmented; }
+    DataType getInputDataType() const { return input.getDataType(); }
+    DataType getOffsetDataType() const { return segment_offsets.getDataType(); }
+    uint64_t getNumItems() const { return num_items; }
+    uint64_t getNumSegments() const { return num_segments; }
+    size_t getWorkspaceSizeInBytes() const { return plan.workspaceBytes; }
+    const std::string& getKernelVariant() const { return plan.variant; }
+
+   private:
+    friend class CubSegmentedArgReduction;
+    StampedCubSegmentedArgReduction(CubArgReductionOp op, const Tensor& input, const Tensor& index_output, const Tensor& segment_offsets,
+                                    uint64_t num_items, uint64_t num_segments, ReductionLaunchPlan plan, std::optional<Tensor> workspace,
+                                    const Stream& stream)
+        : op(op), input(input), index_output(index_output), segment_offsets(segment_offsets), num_items(num_items), num_segments(num_segments),
+          plan(std::move(plan)), workspace(std::move(workspace)), stream(stream) {}
+
+    CubArgReductionOp op;
+    const Tensor input;
+    mutable Tensor index_output;
+    const Tensor segment_offsets;
+    const uint64_t num_items, num_segments;
     ReductionLaunchPlan plan;
     std::optional<Tensor> workspace;
     Stream stream;

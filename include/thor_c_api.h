@@ -26,6 +26,7 @@ typedef struct thor_tensor* thor_tensor_t;
 typedef struct thor_stream* thor_stream_t;
 typedef struct thor_stamped_reduction* thor_stamped_reduction_t;
 typedef struct thor_stamped_arg_reduction* thor_stamped_arg_reduction_t;
+typedef struct thor_stamped_segmented_reduction* thor_stamped_segmented_reduction_t;
 typedef struct thor_expr* thor_expr_t;
 typedef struct thor_outputs* thor_outputs_t;
 typedef struct thor_fused_equation* thor_fused_equation_t;
@@ -116,6 +117,18 @@ thor_tensor_t thor_stamped_arg_reduction_value_output(thor_stamped_arg_reduction
 thor_tensor_t thor_stamped_arg_reduction_index_output(thor_stamped_arg_reduction_t r);
 int thor_stamped_arg_reduction_path(thor_stamped_arg_reduction_t r);
 int thor_stamped_arg_reduction_variant(thor_stamped_arg_reduction_t r, char* buffer, size_t capacity);
+
+/* CubSegmentedReduction / CubSegmentedArgReduction (CubReduction.h:236-400 of the reference): values [N, D...] reduced over the row
+ * ranges [offsets[i], offsets[i+1]) of a UINT32 / UINT64 offsets tensor.  is_arg = 0: op is a CubReductionOp (sum, mean, min, max),
+ * dtype the output dtype (-1 = input dtype); is_arg = 1: op is a CubArgReductionOp, dtype the index dtype (UINT32 / UINT64, -1 = UINT64).
+ * preallocated_output may be NULL unless runtime_offsets is set (then the offsets are not read at stamp time). */
+thor_stamped_segmented_reduction_t thor_segmented_reduction_stamp(int is_arg, int op, int dtype, thor_tensor_t input, thor_tensor_t segment_offsets,
+                                                                  thor_tensor_t preallocated_output, int runtime_offsets, thor_stream_t stream);
+void thor_stamped_segmented_reduction_destroy(thor_stamped_segmented_reduction_t r);
+int thor_stamped_segmented_reduction_run(thor_stamped_segmented_reduction_t r);
+thor_tensor_t thor_stamped_segmented_reduction_output(thor_stamped_segmented_reduction_t r);
+size_t thor_stamped_segmented_reduction_workspace_bytes(thor_stamped_segmented_reduction_t r);
+int thor_stamped_segmented_reduction_variant(thor_stamped_segmented_reduction_t r, char* buffer, size_t capacity);
 
 /* ---- Expression (Utilities/Expression/Expression.h:516-1075) ------------------------------------------------------------- */
 /* dtype arguments: a DataType code, or -1 for "not specified" */

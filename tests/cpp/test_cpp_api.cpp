@@ -170,6 +170,65 @@ static void valueReductionsSmallExact(Stream& stream) {
     CHECK(throwsAs<std::invalid_argument>([&] { CubReduction(CubReductionOp::Sum, 3u).stamp(m, stream); }));
 }
 
+static Tensor gpuOffsets(const std::vector<uint64_t>& values, Stream& stream, DataType dtype = DataType::UINT32) {
+    Tensor host(cpuPlacement, TensorDescriptor(dtype, {values.size()}));
+    for (size_t i = 0; i < values.size(); ++i) {
+        if (dtype == DataType::UINT64)
+            host.getMemPtr<uint64_t>()[i] = values[i];
+        else
+            host.getMemPtr<uint32_t>()[i] = static_cast<uint32_t>(values[i]);
+    }
+    Tensor device(gpuPlacement, TensorDescriptor(dtype, {values.size()}));
+    device.copyFromAsync(host, stream);
+    stream.synchronize();
+    return device;
+}
+
+static void offsetSegmentedReductions(Stream& stream) {
+    const float inf = std::numeric_limits<float>::infinity();
+    // CubOffsetSegmentedReductionTest.cpp:29-45: scalar rows, an empty segment, skewed lengths
+    Tensor x = gpuFrom({1, -2, 4, 5, 7, -1, 8, 99, 100}, {9}, stream);
+    Tensor offsets = gpuOffsets({0, 3, 3, 5, 7}, stream);
+    auto run = [&](CubReductionOp op) {
+        auto stamped = CubSegmentedReduction(op, DataType::FP32).stamp(x, offsets, stream);
+        CHECK(stamped->getPath() == CubReductionPath::OffsetSegmented);
+        stamped->run();
+        return toHostF32(stamped->getOutputTensor(), stream);
+    };
+    CHECK((run(CubReductionOp::Sum) == std::vector<float>{3, 0, 12, 7}));
+    CHECK((run(CubReductionOp::Mean) == std::vector<float>{1, 0, 6, 3.5f}));
+    CHECK((run(CubReductionOp::Min) == std::vector<float>{-2, inf, 5, -1}));
+    CHECK((run(CubReductionOp::Max) == std::vector<float>{4, -inf, 7, 8}));
+    // :116-157: vector values, packed indices row * D + d, NaN wins, lowest index wins ties, all-ones for empty segments
+    Tensor v = gpuFrom({2, 7, 5, -1, 7, 6, -1, 4, std::nanf(""), 6, 1, 9, 5, 1, 8}, {5, 3}, stream);
+    Tensor vOffsets = gpuOffsets({0, 3, 3, 5}, stream, DataType::UINT64);
+    const uint64_t none = std::numeric_limits<uint64_t>::max();
+    auto argMin = CubSegmentedArgReduction(CubArgReductionOp::ArgMin).stamp(v, vOffsets, stream);
+    argMin->run();
+    CHECK((toHostRaw<uint64_t>(argMin->getIndexOutputTensor(), stream) == std::vector<uint64_t>{3, 7, 8, none, none, none, 12, 10, 14}));
+    auto argMax = CubSegmentedArgReduction(CubArgReductionOp::ArgMax, DataType::UINT32).stamp(v, vOffsets, stream);
+    argMax->run();
+    const uint32_t none32 = std::numeric_limits<uint32_t>::max();
+    CHECK((toHostRaw<uint32_t>(argMax->getIndexOutputTensor(), stream) == std::vector<uint32_t>{0, 1, 8, none32, none32, none32, 9, 10, 11}));
+    // :239-295: runtime offsets are read by the kernels, not by the stamp
+    Tensor y = gpuFrom({1, 2, 3, 4, 5, 6}, {6}, stream);
+    Tensor runtimeOffsets = gpuOffsets({9, 9, 9, 9}, stream);
+    Tensor out(gpuPlacement, TensorDescriptor(DataType::FP32, {3}));
+    CHECK(throwsAs<std::invalid_argument>([&] { CubSegmentedReduction(CubReductionOp::Mean, DataType::FP32).stamp(y, out, runtimeOffsets, stream); }));
+    auto dynamic = CubSegmentedReduction(CubReductionOp::Mean, DataType::FP32).stampRuntimeOffsets(y, out, runtimeOffsets, stream);
+    runtimeOffsets.copyFromAsync(gpuOffsets({0, 2, 2, 6}, stream), stream);
+    dynamic->run();
+    CHECK((toHostF32(out, stream) == std::vector<float>{1.5f, 0.0f, 4.5f}));
+    runtimeOffsets.copyFromAsync(gpuOffsets({0, 1, 4, 6}, stream), stream);
+    dynamic->run();
+    CHECK((toHostF32(out, stream) == std::vector<float>{1.0f, 3.0f, 5.5f}));
+    // :457-511: contract violations
+    CHECK(throwsAs<std::invalid_argument>([&] { CubSegmentedReduction(CubReductionOp::Product); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { CubSegmentedReduction(CubReductionOp::Sum).stamp(x, gpuOffsets({1, 3, 9}, stream), stream); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { CubSegmentedReduction(CubReductionOp::Sum).stamp(x, gpuOffsets({0, 5, 3}, stream), stream); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { CubSegmentedReduction(CubReductionOp::Sum).stamp(x, gpuOffsets({0, 5, 10}, stream), stream); }));
+}
+
 static void argReductionsTiesAndNaN(Stream& stream) {
     // CubArgReductionTest.cpp: lowest index wins ties, NaN wins, index is the position inside the reduction domain
     Tensor t = gpuFrom({1, 1, 3, 1, std::nanf(""), 0, std::nanf(""), -4}, {2, 4}, stream);
@@ -307,6 +366,7 @@ int main(int argc, char** argv) {
         };
         cases.push_back({"valueReductionsSmallExact", withStream(valueReductionsSmallExact)});
         cases.push_back({"argReductionsTiesAndNaN", withStream(argReductionsTiesAndNaN)});
+        cases.push_back({"offsetSegmentedReductions", withStream(offsetSegmentedReductions)});
         cases.push_back({"expressionConfig1AndRuntimeScalars", withStream(expressionConfig1AndRuntimeScalars)});
         cases.push_back({"softmaxPlansAndRowKernel", withStream(softmaxPlansAndRowKernel)});
         cases.push_back({"typeConverterOnGpuAndTensorViews", withStream(typeConverterOnGpuAndTensorViews)});

@@ -281,6 +281,275 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::Sources& src, 
     }
 }
 
+// ---- offset-segmented rows: values [N, D] and offsets [B + 1] -> [B, D] ---------------------------------------------------------
+// Segment b is the row range [offsets[b], offsets[b + 1]); the offsets are read when the kernels run, so a stamped
+// reduction follows whatever partition is in the tensor at that moment (replaces cub::DeviceSegmentedReduce and the
+// reference's vector-valued segmented kernels, Utilities/TensorOperations/Cub/CubReductionOffsetSegmented.cu).
+//
+// Work is split by rows, not by segments, so the load of a block does not depend on the partition.  Three launches:
+//   prepareSegments  writes, for every chunk of kChunkRows rows, the first segment that touches it
+//   reduceSegments   block (chunk, column tile) hands the pieces [segment ∩ chunk] to teams of threads; the team size is
+//                    picked per chunk from the number of pieces: the whole block inside a long segment, teams of
+//                    kMinTeam lanes when the chunk holds many short segments.  A piece that is a whole segment is
+//                    finalised and stored at once; a piece of a segment that began in an earlier chunk goes to the
+//                    chunk's `head` partial, a piece of a segment that continues into the next chunk to its `tail` partial
+//   finishSegments   folds tail[c] with head[c + 1 .. c1] for every segment that spans chunks
+// Offsets are clamped to the row count, so an invalid partition gives meaningless results but never reads outside the
+// values tensor.  An element's index (arg reductions) is its packed position row * kD + d; empty segments keep the
+// accumulator's identity (sum 0, min +inf, max -inf, index all-ones) and a mean over zero rows is 0.
+// Workspace: accumulators [kChunks][2][kD]; u64 tails[kChunks] (the segment whose tail the chunk holds, or all-ones);
+// u64 firstSegment[kChunks].
+// Cfg: kD, kRows, kSegments, kColumnTiles, kLanesX, kBatch, kChunkRows, kChunks, kMinTeam, kFinishLanes, kFinishThreads,
+// OffsetT (u32 or u64).
+template <typename Cfg>
+__device__ __forceinline__ u64 segmentOffset(const typename Cfg::OffsetT* offsets, u64 s) {
+    const u64 o = (u64)offsets[s];
+    return o < Cfg::kRows ? o : Cfg::kRows;
+}
+
+template <typename Cfg>
+struct SegmentWorkspace {
+    static constexpr u64 kPartialSlots = Cfg::kChunks * 2 * Cfg::kD;
+    __device__ __forceinline__ static u64* tails(void* workspace) {
+        return reinterpret_cast<u64*>(static_cast<char*>(workspace) + Cfg::Acc::partialBytes(kPartialSlots));
+    }
+    __device__ __forceinline__ static u64* firstSegment(void* workspace) { return tails(workspace) + Cfg::kChunks; }
+};
+
+__device__ __forceinline__ u64 shuffleFrom(u64 v, int sourceLane) {
+    const u32 lo = __shfl((u32)(v & 0xffffffffu), sourceLane, kWave);
+    const u32 hi = __shfl((u32)(v >> 32), sourceLane, kWave);
+    return ((u64)hi << 32) | lo;
+}
+
+// firstSegment[c] = the first segment that touches chunk c: the first one that ends after the chunk's first row or begins
+// at or after it (an empty segment belongs to the chunk its position lies in); bit 63 is set when that segment began
+// before the chunk.  One thread per segment (and one for "no segment") writes the entries of the chunks it is first in:
+// with reach(s) = the last row position that still belongs to s (last - 1, or first for an empty segment), those are
+// the chunks whose first row lies in (reach(s - 1), reach(s)].  Most threads own no chunk; a long range is written by
+// the whole wavefront.  Launched with 256 threads per block over kSegments + 1 threads.
+template <typename Cfg>
+__device__ __forceinline__ void prepareSegments(void* workspace, const typename Cfg::OffsetT* offsets) {
+    constexpr u64 kStraddles = (u64)1 << 63;
+    u64* table = SegmentWorkspace<Cfg>::firstSegment(workspace);
+    const u64 s = (u64)blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = threadIdx.x % kWave;
+    u64 chunkLo = 0, count = 0, first = 0;
+    if (s <= Cfg::kSegments) {
+        u64 afterPrevious = 0;  // reach(s - 1) + 1
+        if (s > 0) {
+            const u64 f = segmentOffset<Cfg>(offsets, s - 1), l = segmentOffset<Cfg>(offsets, s);
+            afterPrevious = l > f ? l : f + 1;
+        }
+        u64 chunkEnd = Cfg::kChunks;  // the thread after the last segment takes every chunk that is left
+        if (s < Cfg::kSegments) {
+            first = segmentOffset<Cfg>(offsets, s);
+            const u64 last = segmentOffset<Cfg>(offsets, s + 1);
+            const u64 reach = last > first ? last - 1 : first;
+            chunkEnd = reach / Cfg::kChunkRows + 1;
+            if (chunkEnd > Cfg::kChunks) chunkEnd = Cfg::kChunks;
+        } else {
+            first = Cfg::kRows;
+        }
+        chunkLo = (afterPrevious + Cfg::kChunkRows - 1) / Cfg::kChunkRows;
+        count = chunkEnd > chunkLo ? chunkEnd - chunkLo : 0;
+    }
+    if (count <= 4) {
+        for (u64 i = 0; i < count; ++i) table[chunkLo + i] = s | (first < (chunkLo + i) * Cfg::kChunkRows ? kStraddles : 0);
+    }
+    u64 longRanges = __builtin_amdgcn_ballot_w64(count > 4);
+    while (longRanges) {
+        const int owner = __builtin_ctzll(longRanges);
+        longRanges &= longRanges - 1;
+        const u64 lo = shuffleFrom(chunkLo, owner), n = shuffleFrom(count, owner), value = shuffleFrom(s, owner), begin = shuffleFrom(first, owner);
+        for (u64 i = lane; i < n; i += kWave) table[lo + i] = value | (begin < (lo + i) * Cfg::kChunkRows ? kStraddles : 0);
+    }
+}
+
+constexpr __device__ int floorLog2(int x) { return x <= 1 ? 0 : 1 + floorLog2(x / 2); }
+
+// Folds the threads of a team of 2^teamBits consecutive threads that share a column (thread-in-team modulo LANES_X):
+// shuffles inside a wavefront, then LDS between the wavefronts of a team.  The result is valid in the team's first
+// LANES_X threads.  teamBits must be the same for the whole block; `parked` holds THREADS / 64 * LANES_X * VEC accumulators.
+template <int THREADS, int LANES_X, int VEC, typename Acc>
+__device__ __forceinline__ void teamReduce(Acc (&acc)[VEC], int teamBits, Acc* parked) {
+    const int inWave = teamBits < 6 ? (1 << teamBits) : kWave;
+    for (int mask = inWave / 2; mask >= LANES_X; mask >>= 1) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k].merge(acc[k].shuffleXor(mask));
+    }
+    if (THREADS > kWave && teamBits > 6) {
+        const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+        const int wavesPerTeam = 1 << (teamBits - 6);
+        const int waveInTeam = wave & (wavesPerTeam - 1);
+        if (waveInTeam != 0 && lane < LANES_X) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) parked[(wave * LANES_X + lane) * VEC + k] = acc[k];
+        }
+        __syncthreads();
+        if (waveInTeam == 0 && lane < LANES_X) {
+            for (int w = 1; w < wavesPerTeam; ++w) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k].merge(parked[((wave + w) * LANES_X + lane) * VEC + k]);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <typename Cfg>
+__device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* workspace, float scale,
+                                               const typename Cfg::OffsetT* offsets) {
+    typedef typename Cfg::IndexT IndexT;
+    typedef typename Cfg::Acc Acc;
+    typedef SegmentWorkspace<Cfg> Workspace;
+    constexpr u64 kColumnsPerRow = Cfg::kD / Cfg::kVec;
+    constexpr int kBatch = Cfg::kBatch;
+    constexpr int kThreadBits = floorLog2(Cfg::kThreads);
+    constexpr int kMaxTeamBits = kThreadBits - floorLog2(Cfg::kMinTeam);
+    __shared__ Acc parked[Cfg::kThreads / kWave * Cfg::kLanesX * Cfg::kVec];
+
+    const u64 chunk = blockIdx.x / Cfg::kColumnTiles, tile = blockIdx.x % Cfg::kColumnTiles;
+    const u64 cBegin = chunk * Cfg::kChunkRows;
+    const u64 cEnd = cBegin + Cfg::kChunkRows < Cfg::kRows ? cBegin + Cfg::kChunkRows : Cfg::kRows;
+    // segments [sLo, sEnd) touch the chunk: from the prepared first one up to the first one that begins at or after the
+    // chunk's end, which is the next chunk's first one unless that one began before the boundary; the last chunk also
+    // takes the empty segments at the very end
+    u64 sLo = 0, sEnd = Cfg::kSegments;
+    if (Cfg::kChunks > 1) {
+        constexpr u64 kStraddles = (u64)1 << 63;
+        sLo = Workspace::firstSegment(workspace)[chunk] & ~kStraddles;
+        if (sLo > Cfg::kSegments) sLo = Cfg::kSegments;
+        if (chunk + 1 < Cfg::kChunks) {
+            const u64 entry = Workspace::firstSegment(workspace)[chunk + 1];
+            sEnd = (entry & ~kStraddles) + (entry >> 63);
+            if (sEnd > Cfg::kSegments) sEnd = Cfg::kSegments;
+        }
+    }
+    const u64 pieces = sEnd > sLo ? sEnd - sLo : 0;
+
+    // one team per piece: as many teams as pieces (a power of two), teams never smaller than kMinTeam threads
+    int teamCountBits = 0;
+    while (teamCountBits < kMaxTeamBits && ((u64)1 << teamCountBits) < pieces) ++teamCountBits;
+    const int teamBits = kThreadBits - teamCountBits;
+    const u64 team = threadIdx.x >> teamBits;
+    const int inTeam = threadIdx.x & ((1 << teamBits) - 1);
+    const int lx = inTeam % Cfg::kLanesX;
+    const u64 rowLane = inTeam / Cfg::kLanesX, rowLanes = (u64)(1 << teamBits) / Cfg::kLanesX;
+    const u64 column = tile * Cfg::kLanesX + lx;
+    const bool columnLive = column < kColumnsPerRow;
+    const u64 columnOffset = (columnLive ? column : 0) * Cfg::kVec;  // dead lanes read column 0 and store nothing
+    const u64 passes = (pieces + ((u64)1 << teamCountBits) - 1) >> teamCountBits;
+
+    for (u64 pass = 0; pass < passes; ++pass) {
+        const u64 segment = sLo + (pass << teamCountBits) + team;
+        const bool pieceLive = segment < sEnd;
+        u64 first = 0, last = 0;
+        if (pieceLive) {
+            first = segmentOffset<Cfg>(offsets, segment);
+            last = segmentOffset<Cfg>(offsets, segment + 1);
+            if (last < first) last = first;
+        }
+        const u64 pBegin = first > cBegin ? first : cBegin;
+        const u64 pEnd = last < cEnd ? last : cEnd;
+
+        Acc acc[Cfg::kVec];
+        typename Cfg::Kept kept;
+        Cfg::loadKept(src, pieceLive ? segment : 0, kept);
+#pragma unroll
+        for (int k = 0; k < Cfg::kVec; ++k) acc[k].reset();
+        for (u64 r0 = pBegin + rowLane; r0 < pEnd; r0 += rowLanes * kBatch) {
+            typename Cfg::Loaded x[kBatch];
+            if (r0 + (u64)(kBatch - 1) * rowLanes < pEnd) {
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) Cfg::load(src, (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset, x[u]);
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const u64 base = (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset;
+#pragma unroll
+                    for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept, k, (IndexT)(base + k));
+                }
+            } else {
+                bool live[kBatch];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const u64 r = r0 + (u64)u * rowLanes;
+                    live[u] = r < pEnd;
+                    if (live[u]) Cfg::load(src, r * Cfg::kD + columnOffset, x[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    if (live[u]) {
+                        const u64 base = (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset;
+#pragma unroll
+                        for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept, k, (IndexT)(base + k));
+                    }
+                }
+            }
+        }
+        teamReduce<Cfg::kThreads, Cfg::kLanesX, Cfg::kVec>(acc, teamBits, parked);
+        if (pieceLive && rowLane == 0 && columnLive) {
+#pragma unroll
+            for (int k = 0; k < Cfg::kVec; ++k) {
+                const u64 d = column * Cfg::kVec + k;
+                if (first < cBegin) {
+                    acc[k].storePartial(workspace, (chunk * 2 + 0) * Cfg::kD + d, Workspace::kPartialSlots);
+                } else if (last > cEnd) {
+                    acc[k].storePartial(workspace, (chunk * 2 + 1) * Cfg::kD + d, Workspace::kPartialSlots);
+                } else {
+                    Cfg::store(acc[k], segment * Cfg::kD + d, out, scale, (float)(last - first));
+                }
+            }
+        }
+    }
+    if (Cfg::kChunks > 1 && tile == 0 && threadIdx.x == 0) {
+        u64 tailSegment = ~(u64)0;
+        if (pieces > 0) {
+            const u64 first = segmentOffset<Cfg>(offsets, sEnd - 1), last = segmentOffset<Cfg>(offsets, sEnd);
+            if (first >= cBegin && first < cEnd && last > cEnd) tailSegment = sEnd - 1;
+        }
+        Workspace::tails(workspace)[chunk] = tailSegment;
+    }
+}
+
+// Last launch: block (c, column tile) finishes the segment whose tail chunk c holds, if any: tail[c] and the heads of the
+// chunks the segment runs on into, spread over the block's kFinishThreads / kFinishLanes row lanes.  The mean's divisor is
+// the row count the offsets hold now.  kFinishLanes = columns (single trailing elements) per block, a power of two <= 64.
+template <typename Cfg>
+__device__ __forceinline__ void finishSegments(const void* workspace, const typename Cfg::Outputs& out, float scale, const typename Cfg::OffsetT* offsets) {
+    typedef typename Cfg::Acc Acc;
+    typedef SegmentWorkspace<Cfg> Workspace;
+    constexpr int kThreads = Cfg::kFinishThreads;  // threads that finish one segment: 64, or the whole block of 256
+    constexpr u64 kTiles = (Cfg::kD + Cfg::kFinishLanes - 1) / Cfg::kFinishLanes;
+    __shared__ Acc parked[kThreads / kWave * Cfg::kFinishLanes];
+    const u64 job = ((u64)blockIdx.x * blockDim.x + threadIdx.x) / kThreads;
+    const u64 chunk = job / kTiles, tile = job % kTiles;
+    if (chunk >= Cfg::kChunks) return;  // (groups of kThreads leave together: barriers are only used when that is the block)
+    const u64 segment = Workspace::tails(const_cast<void*>(workspace))[chunk];
+    if (segment >= Cfg::kSegments) return;  // no segment continues past this chunk
+    const u64 first = segmentOffset<Cfg>(offsets, segment), last = segmentOffset<Cfg>(offsets, segment + 1);
+    if (last <= first) return;
+    u64 lastChunk = (last - 1) / Cfg::kChunkRows;
+    if (lastChunk >= Cfg::kChunks) lastChunk = Cfg::kChunks - 1;
+    const int lx = threadIdx.x % Cfg::kFinishLanes;
+    const u64 rowLane = (threadIdx.x % kThreads) / Cfg::kFinishLanes, rowLanes = kThreads / Cfg::kFinishLanes;
+    const u64 d = tile * Cfg::kFinishLanes + lx;
+    const bool columnLive = d < Cfg::kD;
+    Acc acc[1];
+    acc[0].reset();
+    if (columnLive) {
+        if (rowLane == 0) acc[0].loadPartial(workspace, (chunk * 2 + 1) * Cfg::kD + d, Workspace::kPartialSlots);
+#pragma unroll 4
+        for (u64 c = chunk + 1 + rowLane; c <= lastChunk; c += rowLanes) {
+            Acc part;
+            part.loadPartial(workspace, (c * 2 + 0) * Cfg::kD + d, Workspace::kPartialSlots);
+            acc[0].merge(part);
+        }
+    }
+    teamReduce<kThreads, Cfg::kFinishLanes, 1>(acc, floorLog2(kThreads), parked);
+    if (rowLane == 0 && columnLive) Cfg::store(acc[0], segment * Cfg::kD + d, out, scale, (float)(last - first));
+}
+
 // ---- second stage of the split kernels: [kOutputs, kSplit] partials -> [kOutputs] -------------------------------------------
 // One wavefront per output.  Cfg: kOutputs, kSplit, kFinishOuterStride/kFinishInnerStride/kFinishInner (output layout:
 // logical index o = outer * kFinishInner + inner is stored at outer * kFinishOuterStride + inner * kFinishInnerStride).

@@ -149,6 +149,9 @@ std::string ReductionShape::describe() const {
         case Kernel::Columns:
             out << (laneAxis < 0 ? "columns(lanes_x=" : "view_columns(lanes_x=") << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
             break;
+        case Kernel::Segments:
+            out << "segments(lanes_x=" << threadsPerRow << ",rows_in_flight=" << unroll << ",chunk_rows=" << chunkRows << ",min_team=" << minTeam;
+            break;
         case Kernel::Strided:
             out << "strided(kept_rank=" << keptDims.size() << ",reduced_rank=" << reducedDims.size() << ",split=" << split;
             break;
@@ -173,6 +176,40 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
     auto finishSplit = [&](uint64_t outputs) {
         if (shape.split > 1) shape.workspaceBytes = accumulators * partialBytes(outputs * shape.split, request.isArg, shape.indexIs64);
     };
+
+    if (request.segmented) {
+        shape.kernel = ReductionShape::Kernel::Segments;
+        shape.indexIs64 = true;  // packed global indices; the all-ones sentinel must survive the conversion to a 64-bit output
+        shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {request.trailing});
+        shape.threads = 256;
+        shape.unroll = 8;
+        const uint64_t columnsPerRow = request.trailing / shape.vec;
+        shape.threadsPerRow = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(columnsPerRow)));
+        const uint64_t lanesX = static_cast<uint64_t>(shape.threadsPerRow);
+        const uint64_t tiles = ceilDiv(columnsPerRow, lanesX);
+        // A block streams a chunk of rows whatever the partition is.  Chunks are about as long as an average segment, so
+        // that the teams of one block get pieces of similar length, between one pass of the block and about 128 KiB;
+        // shorter while that leaves fewer than eight blocks per CU.
+        const uint64_t averageRows = std::max<uint64_t>(request.segmentedRows / std::max<uint64_t>(request.segments, 1), 1);
+        const uint64_t rowsPerPass = (256 / lanesX) * shape.unroll;
+        const uint64_t passBytes = rowsPerPass * lanesX * shape.vec * elementBytes;
+        uint64_t passesPerChunk = std::min<uint64_t>(std::max<uint64_t>(131072 / passBytes, 1), std::max<uint64_t>(pow2Ceil(averageRows / rowsPerPass + 1) / 2, 1));
+        while (passesPerChunk > 1 && ceilDiv(request.segmentedRows, rowsPerPass * passesPerChunk) * tiles < 2048) passesPerChunk /= 2;
+        shape.chunkRows = rowsPerPass * passesPerChunk;
+        shape.chunks = std::max<uint64_t>(ceilDiv(request.segmentedRows, shape.chunkRows), 1);
+        // the smallest team that shares one segment: eight rows in flight per lane should cover an average segment
+        const uint64_t rowLanes = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(averageRows) / shape.unroll, 1), 8);
+        shape.minTeam = static_cast<int>(std::min<uint64_t>(lanesX * rowLanes, 256));
+        shape.finishLanes = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(request.trailing)));
+        // a segment of average length runs over averageRows / chunkRows chunks, folded by finishThreads / finishLanes row
+        // lanes: one wavefront while that leaves each lane a handful of partials, else a block
+        shape.finishThreads = (averageRows / shape.chunkRows) * shape.finishLanes > 8 * 64 ? 256 : 64;
+        shape.blocks = tiles;
+        shape.gridX = static_cast<uint32_t>(shape.chunks * tiles);
+        shape.gridY = 1;
+        if (shape.chunks > 1) shape.workspaceBytes = partialBytes(shape.chunks * 2 * request.trailing, request.isArg, true) + shape.chunks * 16;
+        return shape;
+    }
 
     if (g.path == CubReductionPath::DeviceTransformReduce && !g.device_transform_uses_affine_stride) {
         shape.kernel = ReductionShape::Kernel::All;
@@ -414,7 +451,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
         for (size_t j = 0; j < request.elementwise.size(); ++j) s << "        q" << j << ".storeStream(o.e" << j << " + offset);\n";
     }
     s << "        (void)s; (void)o; (void)offset; (void)l; (void)kept;\n    }\n";
-    s << "    static __device__ __forceinline__ void store(const Acc& acc, u64 outIndex, const Outputs& o, float scale) {\n";
+    s << "    static __device__ __forceinline__ void store(const Acc& acc, u64 outIndex, const Outputs& o, float scale, float divisor = kDivisor) {\n";
     if (request.isArg) {
         if (request.writeValue) s << "        o.out0[outIndex] = fromFloat<" << deviceTypeName(values[0].outputDType) << ">(acc.v);\n";
         if (request.writeIndex) s << "        o.indexOut[outIndex] = (" << (request.indexOutputDType == DataType::UINT64 ? "u64" : "u32") << ")acc.i;\n";
@@ -423,10 +460,10 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
         for (size_t j = 0; j < values.size(); ++j) {
             const std::string member = values.size() == 1 ? "acc.v" : "acc.a" + std::to_string(j) + ".v";
             s << "        o.out" << j << "[outIndex] = fromFloat<" << deviceTypeName(values[j].outputDType) << ">(finalizeValue<" << finalize[j] << ">("
-              << member << ", kDivisor, scale));\n";
+              << member << ", divisor, scale));\n";
         }
     }
-    s << "        (void)acc; (void)outIndex; (void)o;\n    }\n";
+    s << "        (void)acc; (void)outIndex; (void)o; (void)divisor;\n    }\n";
 
     const char* body = "";
     switch (shape.kernel) {
@@ -484,6 +521,21 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             }
             body = "thor::reduceColumns<gen::Cfg>(src, out, partials, scale);";
             break;
+        case ReductionShape::Kernel::Segments:
+            s << "    typedef " << (request.offsetsAre64 ? "u64" : "u32") << " OffsetT;\n";
+            s << "    static constexpr u64 kD = " << request.trailing << "ull;\n";
+            s << "    static constexpr u64 kSegments = " << request.segments << "ull;\n";
+            s << "    static constexpr u64 kColumnTiles = " << shape.blocks << "ull;\n";
+            s << "    static constexpr int kBatch = " << shape.unroll << ";\n";
+            s << "    static constexpr int kLanesX = " << shape.threadsPerRow << ";\n";
+            s << "    static constexpr u64 kRows = " << request.segmentedRows << "ull;\n";
+            s << "    static constexpr u64 kChunkRows = " << shape.chunkRows << "ull;\n";
+            s << "    static constexpr u64 kChunks = " << shape.chunks << "ull;\n";
+            s << "    static constexpr int kMinTeam = " << shape.minTeam << ";\n";
+            s << "    static constexpr int kFinishLanes = " << shape.finishLanes << ";\n";
+            s << "    static constexpr int kFinishThreads = " << shape.finishThreads << ";\n";
+            body = "thor::reduceSegments<gen::Cfg>(src, out, partials, scale, static_cast<const gen::Cfg::OffsetT*>(offsets));";
+            break;
         case ReductionShape::Kernel::Strided: {
             std::vector<uint64_t> rd = shape.reducedDims, rs = shape.reducedStrides;
             if (shape.vec > 1) {
@@ -528,12 +580,18 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads << ") void thor_reduce_main(";
     for (size_t i = 0; i < sources.size(); ++i) s << "const " << deviceTypeName(sources[i].storage) << "* in" << i << ", ";
     for (uint32_t slot : request.scalarSlots) s << "float s" << slot << ", ";
-    s << outputParams.str() << ", void* partials, float scale) {\n    const gen::Cfg::Sources src{";
+    s << outputParams.str() << ", void* partials, float scale" << (request.segmented ? ", const void* offsets" : "") << ") {\n    const gen::Cfg::Sources src{";
     for (size_t i = 0; i < sources.size(); ++i) s << (i ? ", " : "") << "in" << i;
     for (uint32_t slot : request.scalarSlots) s << ", s" << slot;
     s << "};\n    const gen::Cfg::Outputs out{" << outputInit.str() << "};\n    (void)partials;\n    " << body << "\n}\n";
     const bool twoStageAll = shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1;
-    if (twoStageAll || shape.split > 1) {
+    if (request.segmented && shape.chunks > 1) {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_reduce_finish(const void* partials, "
+          << finishParams.str() << ", float scale, const void* offsets) {\n    const gen::Cfg::Outputs out{" << finishInit.str()
+          << "};\n    thor::finishSegments<gen::Cfg>(partials, out, scale, static_cast<const gen::Cfg::OffsetT*>(offsets));\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_reduce_prepare(void* partials, const void* offsets) {\n"
+             "    thor::prepareSegments<gen::Cfg>(partials, static_cast<const gen::Cfg::OffsetT*>(offsets));\n}\n";
+    } else if (twoStageAll || shape.split > 1) {
         s << "extern \"C\" __global__ __launch_bounds__(" << (twoStageAll ? 1024 : 256) << ") void thor_reduce_finish(const void* partials, "
           << finishParams.str() << ", float scale) {\n    const gen::Cfg::Outputs out{" << finishInit.str() << "};\n    thor::"
           << (twoStageAll ? "finishAll" : "finishPartials") << "<gen::Cfg>(partials, out, scale);\n}\n";
@@ -551,6 +609,16 @@ ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request)
         plan.finishKernel = compileKernel(source, "thor_reduce_finish", request.deviceNum, false);
         plan.finishThreads = 1024;
         plan.finishGridX = 1;
+    } else if (shape.kernel == ReductionShape::Kernel::Segments) {
+        if (shape.chunks > 1) {
+            plan.prepareKernel = compileKernel(source, "thor_reduce_prepare", request.deviceNum, false);
+            plan.prepareThreads = 256;
+            plan.prepareGridX = static_cast<uint32_t>(ceilDiv(request.segments + 1, 256));
+            plan.finishKernel = compileKernel(source, "thor_reduce_finish", request.deviceNum, false);
+            plan.finishThreads = 256;
+            plan.finishGridX = static_cast<uint32_t>(
+                ceilDiv(shape.chunks * ceilDiv(request.trailing, static_cast<uint64_t>(shape.finishLanes)) * shape.finishThreads, 256));
+        }
     } else if (shape.split > 1) {
         plan.finishKernel = compileKernel(source, "thor_reduce_finish", request.deviceNum, false);
         plan.finishThreads = 256;

@@ -23,6 +23,13 @@ struct ReductionKernelRequest {
     uint64_t inputAlignmentBytes = 256;  // largest power of two (capped at 256) dividing every source base address
     int deviceNum = 0;
 
+    // ---- offset-segmented form: values [rows, trailing] reduced over row ranges given by an offsets tensor at run time ----
+    // geometry.output_elements = segments * trailing, geometry.input_elements = rows * trailing; the kernels take the
+    // offsets pointer as their last argument.
+    bool segmented = false;
+    uint64_t segments = 0, segmentedRows = 0, trailing = 1;
+    bool offsetsAre64 = false;
+
     // ---- fused form: several value reductions over the same geometry, fed by an elementwise prologue ------------------
     // When `values` is empty the request is the plain one above: one source of inputDType, the value itself reduced.
     struct Source {
@@ -54,7 +61,7 @@ struct ReductionKernelRequest {
 };
 
 struct ReductionShape {
-    enum class Kernel { All, Rows, Columns, Strided } kernel = Kernel::All;
+    enum class Kernel { All, Rows, Columns, Strided, Segments } kernel = Kernel::All;
     int vec = 1;
     int threads = 256;
     int threadsPerRow = 64;
@@ -69,6 +76,10 @@ struct ReductionShape {
     // Columns kernel over a view: index (into keptDims) of the kept axis that is contiguous in memory, or -1 for the
     // dense [outer, R, inner] layout
     int laneAxis = -1;
+    // Segments kernel: rows per block, number of such chunks, smallest team of threads that shares a segment, columns per
+    // block of the finishing launch
+    uint64_t chunkRows = 0, chunks = 1;
+    int minTeam = 1, finishLanes = 1, finishThreads = 256;
     std::string describe() const;
 };
 

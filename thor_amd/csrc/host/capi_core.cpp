@@ -242,4 +242,49 @@ int thor_stamped_arg_reduction_variant(thor_stamped_arg_reduction_t r, char* buf
     THOR_CAPI_TRY_INT(require(r, "arg reduction"); copyOut(r->stamped->getKernelVariant(), buffer, capacity, nullptr);)
 }
 
+thor_stamped_segmented_reduction_t thor_segmented_reduction_stamp(int is_arg, int op, int dtype, thor_tensor_t input, thor_tensor_t segment_offsets,
+                                                                  thor_tensor_t preallocated_output, int runtime_offsets, thor_stream_t stream) {
+    THOR_CAPI_TRY_PTR(
+        require(input, "input"); require(segment_offsets, "segment offsets"); require(stream, "stream");
+        if (runtime_offsets && !preallocated_output) throw std::invalid_argument("stampRuntimeOffsets requires a preallocated output.");
+        auto handle = std::make_unique<thor_stamped_segmented_reduction>();
+        if (is_arg) {
+            const CubSegmentedArgReduction reduction(static_cast<CubArgReductionOp>(op), dtype >= 0 ? static_cast<DataType>(dtype) : DataType::UINT64);
+            if (runtime_offsets) {
+                handle->arg = reduction.stampRuntimeOffsets(input->tensor, preallocated_output->tensor, segment_offsets->tensor, stream->stream);
+            } else if (preallocated_output) {
+                handle->arg = reduction.stamp(input->tensor, preallocated_output->tensor, segment_offsets->tensor, stream->stream);
+            } else {
+                handle->arg = reduction.stamp(input->tensor, segment_offsets->tensor, stream->stream);
+            }
+        } else {
+            const CubSegmentedReduction reduction(static_cast<CubReductionOp>(op),
+                                                  dtype >= 0 ? std::optional<DataType>(static_cast<DataType>(dtype)) : std::nullopt);
+            if (runtime_offsets) {
+                handle->value = reduction.stampRuntimeOffsets(input->tensor, preallocated_output->tensor, segment_offsets->tensor, stream->stream);
+            } else if (preallocated_output) {
+                handle->value = reduction.stamp(input->tensor, preallocated_output->tensor, segment_offsets->tensor, stream->stream);
+            } else {
+                handle->value = reduction.stamp(input->tensor, segment_offsets->tensor, stream->stream);
+            }
+        }
+        return handle.release();)
+}
+void thor_stamped_segmented_reduction_destroy(thor_stamped_segmented_reduction_t r) { delete r; }
+int thor_stamped_segmented_reduction_run(thor_stamped_segmented_reduction_t r) {
+    THOR_CAPI_TRY_INT(require(r, "segmented reduction"); if (r->value) r->value->run(); else r->arg->run();)
+}
+thor_tensor_t thor_stamped_segmented_reduction_output(thor_stamped_segmented_reduction_t r) {
+    if (!r) return nullptr;
+    return new thor_tensor{r->value ? r->value->getOutputTensor() : r->arg->getIndexOutputTensor()};
+}
+size_t thor_stamped_segmented_reduction_workspace_bytes(thor_stamped_segmented_reduction_t r) {
+    if (!r) return 0;
+    return r->value ? r->value->getWorkspaceSizeInBytes() : r->arg->getWorkspaceSizeInBytes();
+}
+int thor_stamped_segmented_reduction_variant(thor_stamped_segmented_reduction_t r, char* buffer, size_t capacity) {
+    THOR_CAPI_TRY_INT(require(r, "segmented reduction");
+                      copyOut(r->value ? r->value->getKernelVariant() : r->arg->getKernelVariant(), buffer, capacity, nullptr);)
+}
+
 }  // extern "C"

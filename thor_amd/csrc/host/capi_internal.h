@@ -24,6 +24,10 @@ struct thor_stamped_reduction {
 struct thor_stamped_arg_reduction {
     std::shared_ptr<ThorImplementation::StampedCubArgReduction> stamped;
 };
+struct thor_stamped_segmented_reduction {
+    std::shared_ptr<ThorImplementation::StampedCubSegmentedReduction> value;     // exactly one of the two is set
+    std::shared_ptr<ThorImplementation::StampedCubSegmentedArgReduction> arg;
+};
 
 namespace thor_capi {
 std::string& lastError();

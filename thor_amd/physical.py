@@ -56,6 +56,10 @@ PROTOTYPES = {
     "thor_stamped_reduction_output": (_vp, [_vp]), "thor_stamped_reduction_path": (_i, [_vp]),
     "thor_stamped_reduction_workspace_bytes": (_sz, [_vp]), "thor_stamped_reduction_variant": (_i, [_vp, _cp, _sz]),
     "thor_stamped_arg_reduction_variant": (_i, [_vp, _cp, _sz]),
+    "thor_segmented_reduction_stamp": (_vp, [_i, _i, _i, _vp, _vp, _vp, _i, _vp]),
+    "thor_stamped_segmented_reduction_destroy": (None, [_vp]), "thor_stamped_segmented_reduction_run": (_i, [_vp]),
+    "thor_stamped_segmented_reduction_output": (_vp, [_vp]), "thor_stamped_segmented_reduction_workspace_bytes": (_sz, [_vp]),
+    "thor_stamped_segmented_reduction_variant": (_i, [_vp, _cp, _sz]),
     "thor_reduction_generate_source": (_i, [_i, _i, _i, _i, _i, _u64p, _u64p, _i, _u32p, _i, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_arg_reduction_stamp": (_vp, [_i, _u32p, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "thor_stamped_arg_reduction_destroy": (None, [_vp]), "thor_stamped_arg_reduction_run": (_i, [_vp]),
@@ -431,6 +435,74 @@ class CubArgReduction:
                                              int(self.index_output_dtype), input._h, preallocated_value._h if preallocated_value else None,
                                              preallocated_index._h if preallocated_index else None, stream._h)
         return StampedCubArgReduction(_handle(ptr, "CubArgReduction.stamp"))
+
+
+class StampedCubSegmentedReduction:
+    def __init__(self, ptr):
+        self._h = ptr
+
+    def run(self):
+        _check(lib().thor_stamped_segmented_reduction_run(self._h), "StampedCubSegmentedReduction.run")
+
+    def get_output_tensor(self) -> PhysicalTensor:
+        return PhysicalTensor._wrap(_handle(lib().thor_stamped_segmented_reduction_output(self._h), "getOutputTensor"))
+
+    get_index_output_tensor = get_output_tensor
+
+    def get_path(self) -> CubReductionPath:
+        return CubReductionPath.OffsetSegmented
+
+    def get_workspace_size_in_bytes(self) -> int:
+        return lib().thor_stamped_segmented_reduction_workspace_bytes(self._h)
+
+    def get_kernel_variant(self) -> str:
+        buf = ctypes.create_string_buffer(512)
+        _check(lib().thor_stamped_segmented_reduction_variant(self._h, buf, 512), "variant")
+        return buf.value.decode()
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_stamped_segmented_reduction_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class CubSegmentedReduction:
+    """Values [N, D...] reduced over the row ranges [offsets[i], offsets[i+1]) -> [B, D...] (sum, mean, min, max)."""
+
+    def __init__(self, op: CubReductionOp, output_dtype: Optional[DataType] = None):
+        self.op, self.output_dtype = op, output_dtype
+
+    def _stamp(self, input, offsets, stream, preallocated, runtime):
+        ptr = lib().thor_segmented_reduction_stamp(0, int(self.op), -1 if self.output_dtype is None else int(self.output_dtype), input._h, offsets._h,
+                                                   preallocated._h if preallocated is not None else None, 1 if runtime else 0, stream._h)
+        return StampedCubSegmentedReduction(_handle(ptr, "CubSegmentedReduction.stamp"))
+
+    def stamp(self, input: PhysicalTensor, segment_offsets: PhysicalTensor, stream: Stream, preallocated_output: Optional[PhysicalTensor] = None):
+        return self._stamp(input, segment_offsets, stream, preallocated_output, False)
+
+    def stamp_runtime_offsets(self, input: PhysicalTensor, preallocated_output: PhysicalTensor, segment_offsets: PhysicalTensor, stream: Stream):
+        return self._stamp(input, segment_offsets, stream, preallocated_output, True)
+
+
+class CubSegmentedArgReduction:
+    """Winner indices (packed row * D + d) of argmin / argmax over the same row ranges; empty segments give the all-ones index."""
+
+    def __init__(self, op: CubArgReductionOp, index_output_dtype: DataType = DataType.uint64):
+        self.op, self.index_output_dtype = op, index_output_dtype
+
+    def _stamp(self, input, offsets, stream, preallocated, runtime):
+        ptr = lib().thor_segmented_reduction_stamp(1, int(self.op), int(self.index_output_dtype), input._h, offsets._h,
+                                                   preallocated._h if preallocated is not None else None, 1 if runtime else 0, stream._h)
+        return StampedCubSegmentedReduction(_handle(ptr, "CubSegmentedArgReduction.stamp"))
+
+    def stamp(self, input: PhysicalTensor, segment_offsets: PhysicalTensor, stream: Stream, preallocated_index_output: Optional[PhysicalTensor] = None):
+        return self._stamp(input, segment_offsets, stream, preallocated_index_output, False)
+
+    def stamp_runtime_offsets(self, input: PhysicalTensor, preallocated_index_output: PhysicalTensor, segment_offsets: PhysicalTensor, stream: Stream):
+        return self._stamp(input, segment_offsets, stream, preallocated_index_output, True)
 
 
 # ---- expressions -------------------------------------------------------------------------------------------------------------
