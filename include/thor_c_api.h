@@ -130,6 +130,12 @@ thor_tensor_t thor_stamped_segmented_reduction_output(thor_stamped_segmented_red
 size_t thor_stamped_segmented_reduction_workspace_bytes(thor_stamped_segmented_reduction_t r);
 int thor_stamped_segmented_reduction_variant(thor_stamped_segmented_reduction_t r, char* buffer, size_t capacity);
 
+/* ---- segmented broadcast (Utilities/Expression/SegmentedBroadcastKernel.h:8-12) ------------------------------------------- */
+/* output[r, :] = per_segment_values[b, :] for the rows r of segment b (divided by the segment length when
+ * normalize_by_segment_length is nonzero); rows of no segment are left untouched.  Enqueued on `stream`. */
+int thor_segmented_broadcast(thor_tensor_t per_segment_values, thor_tensor_t segment_offsets, thor_tensor_t output,
+                             int normalize_by_segment_length, thor_stream_t stream);
+
 /* ---- Expression (Utilities/Expression/Expression.h:516-1075) ------------------------------------------------------------- */
 /* dtype arguments: a DataType code, or -1 for "not specified" */
 thor_expr_t thor_expr_input(const char* name, int compute_dtype, int output_dtype);

@@ -550,6 +550,123 @@ __device__ __forceinline__ void finishSegments(const void* workspace, const type
     if (rowLane == 0 && columnLive) Cfg::store(acc[0], segment * Cfg::kD + d, out, scale, (float)(last - first));
 }
 
+// ---- segmented broadcast: per-segment values [B, E] -> rows [N, E] ---------------------------------------------------------------
+// out[r, :] = values[b, :] for every row r of segment b = [offsets[b], offsets[b + 1]), optionally divided by the
+// segment's length in fp32 and rounded once to the storage type (reference: Utilities/Expression/SegmentedBroadcastKernel.cu:82-104,
+// one block per segment).  Rows that belong to no segment are left untouched.  Here the *output* is split into chunks of
+// rows, so the stores stream at the same rate whatever the partition is: a block searches the offsets once for the
+// first segment that reaches into its chunk, stages a window of kWindow + 1 offsets in LDS, and every thread finds the
+// segment of the vector it writes with a binary search in that window (further windows follow while segments are
+// shorter than kChunkRows / kWindow on average).
+// First s in [0, n] for which pred(s) holds, for a predicate that is false up to some point and true from there on
+// (pred(n) is taken as true).  A wavefront with all 64 lanes active runs the search: each round probes 64 evenly spaced
+// candidates, so the depth is log64(n) dependent loads instead of log2(n).
+template <typename Pred>
+__device__ __forceinline__ u64 waveLowerBound(u64 n, Pred pred) {
+    const u64 lane = threadIdx.x % kWave;
+    u64 lo = 0, hi = n;
+    while (hi > lo) {
+        const u64 step = (hi - lo + kWave - 1) / kWave;
+        const u64 probe = lo + lane * step;
+        const bool holds = probe < hi ? pred(probe) : true;
+        const u64 mask = __builtin_amdgcn_ballot_w64(holds);
+        const u64 firstTrue = mask ? (u64)__builtin_ctzll(mask) : (u64)kWave;
+        if (firstTrue == 0) return lo;
+        const u64 newLo = lo + (firstTrue - 1) * step + 1;
+        const u64 newHi = lo + firstTrue * step;
+        lo = newLo;
+        hi = newHi < hi ? newHi : hi;
+    }
+    return lo;
+}
+
+// Cfg: T (storage type), OffsetT, kE (elements per value), kRows, kSegments, kChunkRows, kVec (elements per store; kChunkRows * kE
+// is a multiple of it), kThreads, kWindow (a power of two), kNormalize, kViaHalf (round through fp16 first: e5m2).
+template <typename Cfg>
+__device__ __forceinline__ typename Cfg::T broadcastValue(typename Cfg::T value, u64 length) {
+    if constexpr (!Cfg::kNormalize) {
+        return value;
+    } else {
+        float x = toFloat(value) / (float)length;
+        if (Cfg::kViaHalf) x = roundF16(x);
+        return fromFloat<typename Cfg::T>(x);
+    }
+}
+
+template <typename Cfg>
+__device__ __forceinline__ void broadcastSegments(const typename Cfg::T* values, const typename Cfg::OffsetT* offsets, typename Cfg::T* out) {
+    typedef typename Cfg::T T;
+    constexpr int kWindow = Cfg::kWindow;
+    constexpr u64 kE = Cfg::kE;
+    constexpr int kVec = Cfg::kVec;
+    constexpr bool kRowVectors = kE % kVec == 0;  // a vector never crosses a row
+    __shared__ u64 bounds[kWindow + 1];
+    const u64 cBegin = (u64)blockIdx.x * Cfg::kChunkRows;
+    const u64 cEnd = cBegin + Cfg::kChunkRows < Cfg::kRows ? cBegin + Cfg::kChunkRows : Cfg::kRows;
+    u64 window = waveLowerBound(Cfg::kSegments, [&](u64 s) { return segmentOffset<Cfg>(offsets, s + 1) > cBegin; });
+    while (window < Cfg::kSegments) {
+        for (int i = threadIdx.x; i <= kWindow; i += Cfg::kThreads) {
+            const u64 s = window + i;
+            bounds[i] = segmentOffset<Cfg>(offsets, s < Cfg::kSegments ? s : Cfg::kSegments);
+        }
+        __syncthreads();
+        const u64 rLo = bounds[0] > cBegin ? bounds[0] : cBegin;
+        const u64 rHi = bounds[kWindow] < cEnd ? bounds[kWindow] : cEnd;
+        if (rLo < rHi) {
+            const u64 vLo = rLo * kE / kVec, vHi = (rHi * kE + kVec - 1) / kVec;
+            for (u64 v = vLo + threadIdx.x; v < vHi; v += Cfg::kThreads) {
+                const u64 e0 = v * kVec;
+                u64 row = e0 / kE;
+                u64 component = e0 % kE;
+                const u64 searched = row > rLo ? row : rLo;
+                int j = 0;  // bounds[j] <= searched < bounds[j + step] holds throughout
+#pragma unroll
+                for (int step = kWindow / 2; step >= 1; step /= 2) {
+                    if (bounds[j + step] <= searched) j += step;
+                }
+                if (kRowVectors) {
+                    if (row >= rLo && row < rHi) {
+                        const u64 length = bounds[j + 1] - bounds[j];
+                        Pack<T, kVec> x;
+                        x.load(values + (window + j) * kE + component);
+#pragma unroll
+                        for (int k = 0; k < kVec; ++k) x.v[k] = broadcastValue<Cfg>(x.v[k], length);
+                        x.storeStream(out + e0);
+                    }
+                } else {
+                    Pack<T, kVec> x;
+                    bool live[kVec];
+                    bool all = true;
+#pragma unroll
+                    for (int k = 0; k < kVec; ++k) {
+                        live[k] = row >= rLo && row < rHi;
+                        all = all && live[k];
+                        if (live[k]) {
+                            while (bounds[j + 1] <= row) ++j;
+                            x.v[k] = broadcastValue<Cfg>(values[(window + j) * kE + component], bounds[j + 1] - bounds[j]);
+                        }
+                        if (++component == kE) {
+                            component = 0;
+                            ++row;
+                        }
+                    }
+                    if (all) {
+                        x.storeStream(out + e0);
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < kVec; ++k)
+                            if (live[k]) out[e0 + k] = x.v[k];
+                    }
+                }
+            }
+        }
+        const bool finished = bounds[kWindow] >= cEnd;
+        __syncthreads();
+        if (finished) break;
+        window += kWindow;
+    }
+}
+
 // ---- second stage of the split kernels: [kOutputs, kSplit] partials -> [kOutputs] -------------------------------------------
 // One wavefront per output.  Cfg: kOutputs, kSplit, kFinishOuterStride/kFinishInnerStride/kFinishInner (output layout:
 // logical index o = outer * kFinishInner + inner is stored at outer * kFinishOuterStride + inner * kFinishInnerStride).

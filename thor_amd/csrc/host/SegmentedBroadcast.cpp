@@ -1,0 +1,104 @@
+// Segmented broadcast: validation, kernel specialisation and launch (kernel: thor_device_reduce.h broadcastSegments).
+#include "Utilities/Expression/SegmentedBroadcastKernel.h"
+
+#include "ReductionPlanner.h"
+#include "Utilities/Common/ScopedGpu.h"
+#include "Utilities/Expression/CompiledEquation.h"
+#include "thorhip_numeric_embed.h"
+
+#include <algorithm>
+#include <limits>
+#include <sstream>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+namespace {
+
+uint64_t pow2Floor(uint64_t v) {
+    uint64_t p = 1;
+    while (p * 2 <= v) p *= 2;
+    return p;
+}
+
+uint64_t pow2Ceil(uint64_t v) {
+    uint64_t p = 1;
+    while (p < v) p *= 2;
+    return p;
+}
+
+const char* rawWordName(uint32_t bytes) { return bytes == 1 ? "thor::u8" : bytes == 2 ? "thor::u16" : "thor::u32"; }
+
+}  // namespace
+
+void launchSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, Tensor& output, bool normalize_by_segment_length,
+                              Stream& stream) {
+    if (!per_segment_values.isInitialized() || !segment_offsets.isInitialized() || !output.isInitialized()) {
+        throw std::runtime_error("Segmented broadcast requires initialized tensors.");
+    }
+    if (per_segment_values.getPlacement() != segment_offsets.getPlacement() || per_segment_values.getPlacement() != output.getPlacement()) {
+        throw std::runtime_error("Segmented broadcast tensors must share one placement.");
+    }
+    if (per_segment_values.getPlacement().getMemDevice() != TensorPlacement::MemDevices::GPU || !stream.isInitialized() ||
+        per_segment_values.getPlacement().getDeviceNum() != stream.getGpuNum()) {
+        throw std::runtime_error("Segmented broadcast requires tensors on the execution GPU.");
+    }
+    if (per_segment_values.getDimensions().empty() || segment_offsets.getDimensions().size() != 1 || output.getDimensions().empty()) {
+        throw std::runtime_error("Segmented broadcast requires per-segment values [B,D...], offsets [B+1], and output [N,D...].");
+    }
+    const uint64_t segments = per_segment_values.getDimensions()[0];
+    if (segments == 0 || segments > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) {
+        throw std::runtime_error("Segmented broadcast batch size is zero or exceeds the supported number of segments.");
+    }
+    if (segment_offsets.getDimensions()[0] != segments + 1) throw std::runtime_error("Segmented broadcast offsets must have shape [batch_size + 1].");
+    if (per_segment_values.getDataType() != output.getDataType()) throw std::runtime_error("Segmented broadcast input and output dtypes must match.");
+    if (!per_segment_values.isDenseContiguous() || !segment_offsets.isDenseContiguous() || !output.isDenseContiguous()) {
+        throw std::runtime_error("Segmented broadcast requires dense tensors.");
+    }
+    const DataType offsetType = segment_offsets.getDataType();
+    if (offsetType != DataType::UINT32 && offsetType != DataType::UINT64) throw std::runtime_error("Segmented broadcast offsets must use UINT32 or UINT64.");
+    const DataType dtype = per_segment_values.getDataType();
+    if (dtype != DataType::FP8_E4M3 && dtype != DataType::FP8_E5M2 && dtype != DataType::FP16 && dtype != DataType::BF16 && dtype != DataType::FP32) {
+        throw std::runtime_error("Segmented broadcast requires a floating-point expression dtype.");
+    }
+    // Trailing dimensions may be reshaped between the two tensors ([B, 4] against [N, 2, 2]); the elements per value are
+    // what has to agree.
+    const uint64_t rows = output.getDimensions()[0];
+    const uint64_t elementsPerValue = per_segment_values.getTotalNumElements() / segments;
+    if (elementsPerValue == 0 || rows == 0 || output.getTotalNumElements() % rows != 0 || output.getTotalNumElements() / rows != elementsPerValue) {
+        throw std::runtime_error("Segmented broadcast trailing dimensions produce an invalid elements-per-value extent.");
+    }
+
+    const uint32_t elementBytes = dataTypeSizeInBytes(dtype);
+    const uint64_t alignment = std::min(pointerAlignment(per_segment_values.getMemPtr()), pointerAlignment(output.getMemPtr()));
+    int vec = static_cast<int>(16 / elementBytes);
+    while (vec > 1 && alignment % (static_cast<uint64_t>(vec) * elementBytes) != 0) vec /= 2;
+    // about 128 KiB of output per block, fewer rows while that leaves under eight blocks per CU; always a multiple of 16 rows
+    uint64_t chunkRows = std::max<uint64_t>(pow2Floor(std::max<uint64_t>(131072 / (elementsPerValue * elementBytes), 1)), 16);
+    while (chunkRows > 16 && (rows + chunkRows - 1) / chunkRows < 2048) chunkRows /= 2;
+    const uint64_t chunks = (rows + chunkRows - 1) / chunkRows;
+    const uint64_t averageRows = std::max<uint64_t>(rows / segments, 1);
+    const uint64_t window = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(2 * chunkRows / averageRows + 2), 16), 1024);
+
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude << thor_embed::kReduceKernels;
+    const std::string typeName = normalize_by_segment_length ? deviceTypeName(dtype) : rawWordName(elementBytes);
+    s << "namespace gen {\nstruct Cfg {\n    typedef " << typeName << " T;\n    typedef " << (offsetType == DataType::UINT64 ? "thor::u64" : "thor::u32")
+      << " OffsetT;\n    static constexpr thor::u64 kE = " << elementsPerValue << "ull;\n    static constexpr thor::u64 kRows = " << rows
+      << "ull;\n    static constexpr thor::u64 kSegments = " << segments << "ull;\n    static constexpr thor::u64 kChunkRows = " << chunkRows
+      << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = 256;\n    static constexpr int kWindow = " << window
+      << ";\n    static constexpr bool kNormalize = " << (normalize_by_segment_length ? "true" : "false")
+      << ";\n    static constexpr bool kViaHalf = " << (dtype == DataType::FP8_E5M2 ? "true" : "false") << ";\n};\n}  // namespace gen\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_segmented_broadcast(const gen::Cfg::T* values, const void* offsets, gen::Cfg::T* out) "
+         "{\n    thor::broadcastSegments<gen::Cfg>(values, static_cast<const gen::Cfg::OffsetT*>(offsets), out);\n}\n";
+    const std::shared_ptr<CompiledKernel> kernel = compileKernel(s.str(), "thor_segmented_broadcast", stream.getGpuNum(), /*fastContract=*/false);
+
+    ScopedGpu scoped(stream.getGpuNum());
+    const void* values = per_segment_values.getMemPtr();
+    const void* offsets = segment_offsets.getMemPtr();
+    void* out = output.getMemPtr();
+    std::vector<void*> args = {&values, &offsets, &out};
+    kernel->launch(static_cast<uint32_t>(chunks), 1, 1, 256, stream.getStream(), args);
+}
+
+}  // namespace ThorImplementation

@@ -2,6 +2,7 @@
 #include "capi_internal.h"
 
 #include "ReductionPlanner.h"
+#include "Utilities/Expression/SegmentedBroadcastKernel.h"
 #include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
 
 #include <cstring>
@@ -285,6 +286,14 @@ size_t thor_stamped_segmented_reduction_workspace_bytes(thor_stamped_segmented_r
 int thor_stamped_segmented_reduction_variant(thor_stamped_segmented_reduction_t r, char* buffer, size_t capacity) {
     THOR_CAPI_TRY_INT(require(r, "segmented reduction");
                       copyOut(r->value ? r->value->getKernelVariant() : r->arg->getKernelVariant(), buffer, capacity, nullptr);)
+}
+
+int thor_segmented_broadcast(thor_tensor_t per_segment_values, thor_tensor_t segment_offsets, thor_tensor_t output, int normalize_by_segment_length,
+                             thor_stream_t stream) {
+    THOR_CAPI_TRY_INT(require(per_segment_values, "per-segment values"); require(segment_offsets, "segment offsets"); require(output, "output");
+                      require(stream, "stream");
+                      launchSegmentedBroadcast(per_segment_values->tensor, segment_offsets->tensor, output->tensor, normalize_by_segment_length != 0,
+                                               stream->stream);)
 }
 
 }  // extern "C"

@@ -60,6 +60,7 @@ PROTOTYPES = {
     "thor_stamped_segmented_reduction_destroy": (None, [_vp]), "thor_stamped_segmented_reduction_run": (_i, [_vp]),
     "thor_stamped_segmented_reduction_output": (_vp, [_vp]), "thor_stamped_segmented_reduction_workspace_bytes": (_sz, [_vp]),
     "thor_stamped_segmented_reduction_variant": (_i, [_vp, _cp, _sz]),
+    "thor_segmented_broadcast": (_i, [_vp, _vp, _vp, _i, _vp]),
     "thor_reduction_generate_source": (_i, [_i, _i, _i, _i, _i, _u64p, _u64p, _i, _u32p, _i, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_arg_reduction_stamp": (_vp, [_i, _u32p, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "thor_stamped_arg_reduction_destroy": (None, [_vp]), "thor_stamped_arg_reduction_run": (_i, [_vp]),
@@ -503,6 +504,14 @@ class CubSegmentedArgReduction:
 
     def stamp_runtime_offsets(self, input: PhysicalTensor, preallocated_index_output: PhysicalTensor, segment_offsets: PhysicalTensor, stream: Stream):
         return self._stamp(input, segment_offsets, stream, preallocated_index_output, True)
+
+
+def segmented_broadcast(per_segment_values: PhysicalTensor, segment_offsets: PhysicalTensor, output: PhysicalTensor,
+                        normalize_by_segment_length: bool, stream: Stream) -> None:
+    """output[r] = per_segment_values[b] for the rows r of segment b = [offsets[b], offsets[b + 1]), divided by the segment's
+    length when asked; rows of no segment keep their contents (reference: SegmentedBroadcastKernel.h launchSegmentedBroadcast)."""
+    _check(lib().thor_segmented_broadcast(per_segment_values._h, segment_offsets._h, output._h, 1 if normalize_by_segment_length else 0, stream._h),
+           "segmented_broadcast")
 
 
 # ---- expressions -------------------------------------------------------------------------------------------------------------
