@@ -78,6 +78,16 @@ constexpr uint64_t kReduceAllAxesButFirst = UINT64_MAX - 1;
 inline bool isArgReductionOp(ExprOp op) { return op == ExprOp::REDUCE_ARGMIN || op == ExprOp::REDUCE_ARGMAX; }
 inline bool isReductionOp(ExprOp op) { return isValueReductionOp(op) || isArgReductionOp(op); }
 
+// Ops over a ragged batch: lhs holds values, rhs the row-partition offsets [B + 1] (UINT32 / UINT64), which are structure,
+// not data: they take no part in dtype promotion or broadcasting.
+inline bool isSegmentedReduceOp(ExprOp op) {
+    return op == ExprOp::SEGMENTED_REDUCE_SUM || op == ExprOp::SEGMENTED_REDUCE_MIN || op == ExprOp::SEGMENTED_REDUCE_MAX ||
+           op == ExprOp::SEGMENTED_REDUCE_MEAN;
+}
+inline bool isRaggedOp(ExprOp op) {
+    return isSegmentedReduceOp(op) || op == ExprOp::SEGMENTED_BROADCAST || op == ExprOp::RAGGED_VALUEWISE_EXTENT;
+}
+
 // One vertex of the DAG.  Children are indices into PhysicalExpression::nodes and always precede their consumer.
 struct ExprNode {
     ExprOp op = ExprOp::SCALAR_FP;
@@ -100,6 +110,14 @@ struct ExprNode {
     std::vector<uint64_t> fill_dims;
     SoftmaxAlgorithm softmax_algorithm = SoftmaxAlgorithm::Accurate;  // SOFTMAX only
     SoftmaxMode softmax_mode = SoftmaxMode::Channel;
+
+    // Ragged ops (reference: Expression.h:336-343 there): the batch size B, the capacity of the packed values tensor in
+    // rows, and the elements one row holds.  Zero batch size = not given (segmented reductions take both from the bound
+    // tensors then).
+    uint64_t ragged_runtime_batch_size = 0;
+    uint64_t ragged_runtime_max_active_values = 0;
+    uint64_t ragged_runtime_elements_per_value = 1;
+    bool segmented_broadcast_normalize_by_length = false;
 };
 
 // The axes a reduction node reduces for an input of `rank` dimensions: sorted, unique, validated ({} = all).
@@ -321,6 +339,26 @@ class Expression {
                       std::optional<DataType> compute_dtype = std::nullopt) const;
     Expression dotProduct(const Expression& other, std::optional<DataType> compute_dtype = std::nullopt) const;
     static Expression dotProduct(const Expression& lhs, const Expression& rhs, std::optional<DataType> compute_dtype = std::nullopt);
+
+    // ---- ragged batches: values [N, D...] packed row after row, offsets [B + 1] read on the device at run time -------------
+    // Per-segment sum / min / max / mean -> [B, D...] in the values' dtype, fp32 accumulation (reference: Expression.cpp:3962-4008).
+    static Expression segmentedReduceWithRaggedMetadata(const Expression& input, const Expression& offsets, ExprOp op, uint64_t ragged_batch_size,
+                                                        uint64_t ragged_max_active_values, uint64_t ragged_elements_per_value = 1);
+    Expression segmentedReduceSum(const Expression& offsets) const { return segmentedReduceSum(*this, offsets); }
+    Expression segmentedReduceMin(const Expression& offsets) const { return segmentedReduceMin(*this, offsets); }
+    Expression segmentedReduceMax(const Expression& offsets) const { return segmentedReduceMax(*this, offsets); }
+    Expression segmentedReduceMean(const Expression& offsets) const { return segmentedReduceMean(*this, offsets); }
+    static Expression segmentedReduceSum(const Expression& input, const Expression& offsets);
+    static Expression segmentedReduceMin(const Expression& input, const Expression& offsets);
+    static Expression segmentedReduceMax(const Expression& input, const Expression& offsets);
+    static Expression segmentedReduceMean(const Expression& input, const Expression& offsets);
+    // Per-segment values [B, D...] -> rows [max_active_values, D...]: every row of segment b receives values[b] (divided by
+    // the segment's length on request); rows of no segment are undefined (RaggedExpression.cpp:421-430 there).
+    static Expression segmentedBroadcast(const Expression& per_segment_values, const Expression& offsets, uint64_t batch_size,
+                                         uint64_t max_active_values, uint64_t elements_per_value, bool normalize_by_segment_length);
+    // Identity on the values that limits the kernel producing them to the first offsets[batch_size] rows; the rest of the
+    // output tensor keeps its contents (Expression.cpp:4010-4032 there).  `offsets` has to be a direct input.
+    Expression withRaggedRuntimeExtent(const Expression& offsets, uint64_t batch_size, uint64_t max_active_values, uint64_t elements_per_value) const;
 
     // ---- dtype overrides on the root node ----------------------------------------------------------------------------
     Expression withDTypes(std::optional<DataType> compute_dtype = std::nullopt, std::optional<DataType> output_dtype = std::nullopt) const;

@@ -9,7 +9,33 @@
 #include "DeepLearning/Implementation/Tensor/Tensor.h"
 #include "Utilities/Common/Stream.h"
 
+#include <memory>
+#include <string>
+
 namespace ThorImplementation {
+
+struct CompiledKernel;
+
+// The validated, compiled form: stampSegmentedBroadcast() does everything launchSegmentedBroadcast() does except the
+// launch; runOn() only launches (what a stamped execution plan keeps per broadcast stage).
+class StampedSegmentedBroadcast {
+   public:
+    StampedSegmentedBroadcast(std::shared_ptr<CompiledKernel> kernel, Tensor values, Tensor offsets, Tensor output, uint32_t gridX, std::string variant)
+        : kernel(std::move(kernel)), values(std::move(values)), offsets(std::move(offsets)), output(std::move(output)), gridX(gridX),
+          variant(std::move(variant)) {}
+    void runOn(Stream& stream) const;
+    Tensor getOutputTensor() const { return output; }
+    const std::string& getKernelVariant() const { return variant; }
+
+   private:
+    std::shared_ptr<CompiledKernel> kernel;
+    Tensor values, offsets, output;
+    uint32_t gridX;
+    std::string variant;
+};
+
+std::shared_ptr<StampedSegmentedBroadcast> stampSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, const Tensor& output,
+                                                                   bool normalize_by_segment_length, const Stream& stream);
 
 void launchSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, Tensor& output, bool normalize_by_segment_length,
                               Stream& stream);

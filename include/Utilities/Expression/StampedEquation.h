@@ -7,6 +7,7 @@
 #include "DeepLearning/Implementation/Tensor/Tensor.h"
 #include "Utilities/Common/Stream.h"
 #include "Utilities/Expression/CompiledEquation.h"
+#include "Utilities/Expression/SegmentedBroadcastKernel.h"
 #include "Utilities/TensorOperations/Cub/CubReduction.h"
 
 #include <cstdint>
@@ -115,8 +116,21 @@ class StampedFusedReduction {
     uint64_t flops;
 };
 
+// Per-segment reduction over a ragged batch; the offsets are read on the device each time the stage runs.
+class StampedSegmentedReductionStage {
+   public:
+    explicit StampedSegmentedReductionStage(std::shared_ptr<StampedCubSegmentedReduction> stamped) : stamped(std::move(stamped)) {}
+    void runOn(Stream& stream) const { stamped->runOn(stream); }
+    Tensor getOutputTensor() const { return stamped->getOutputTensor(); }
+    uint64_t flopCount() const { return stamped->getNumItems(); }
+    const std::shared_ptr<StampedCubSegmentedReduction>& getStamped() const { return stamped; }
+
+   private:
+    std::shared_ptr<StampedCubSegmentedReduction> stamped;
+};
+
 struct StampedExecutionStage {
-    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction };
+    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction, SegmentedReduction, SegmentedBroadcast };
     static std::string kindToString(Kind kind) {
         switch (kind) {
             case Kind::FusedKernel:
@@ -131,6 +145,10 @@ struct StampedExecutionStage {
                 return "Copy";
             case Kind::FusedReduction:
                 return "FusedReduction";
+            case Kind::SegmentedReduction:
+                return "SegmentedReduction";
+            case Kind::SegmentedBroadcast:
+                return "SegmentedBroadcast";
         }
         return "<unknown>";
     }
@@ -142,6 +160,8 @@ struct StampedExecutionStage {
     std::shared_ptr<StampedReduction> reduction;
     std::shared_ptr<StampedArgMinMax> arg_minmax;
     std::shared_ptr<StampedFusedReduction> fused_reduction;
+    std::shared_ptr<StampedSegmentedReductionStage> segmented_reduction;
+    std::shared_ptr<StampedSegmentedBroadcast> segmented_broadcast;
     // Kind::Copy: a named output that is only a view of an input is copied into the caller's tensor
     Tensor copySource, copyDestination;
 

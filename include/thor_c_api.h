@@ -146,6 +146,11 @@ thor_expr_t thor_expr_fill(double value, const uint64_t* dims, int rank, int out
  * "lessEqual", "greaterThan", "greaterEqual", "logicalAnd", "logicalOr" (binary); "neg", "logicalNot", "abs", "exp",
  * "sigmoid", "gelu", ... (unary; every unary method of Expression) */
 thor_expr_t thor_expr_binary(const char* method, thor_expr_t lhs, thor_expr_t rhs);
+/* Ragged batches (Expression::segmentedReduceWithRaggedMetadata / segmentedBroadcast / withRaggedRuntimeExtent): `method` is
+ * "segment_sum", "segment_min", "segment_max", "segment_mean" (batch_size and max_active_values both zero = take them from the
+ * bound tensors), "segmented_broadcast", "segmented_broadcast_normalized" or "ragged_extent". */
+thor_expr_t thor_expr_ragged(const char* method, thor_expr_t values, thor_expr_t offsets, uint64_t batch_size, uint64_t max_active_values,
+                             uint64_t elements_per_value);
 thor_expr_t thor_expr_unary(const char* method, thor_expr_t input);
 /* methods with numeric parameters: "elu"(alpha), "hardTanh"(min,max), "threshold"(threshold,value), "log"(base),
  * "clamp"(lo,hi) */

@@ -1,0 +1,168 @@
+"""Ragged-batch Expression ops (segmented reductions, segmented broadcast, runtime-extent kernels) through compile / stamp / run,
+with the reference's RaggedExpressionTest.cpp execution cases as known answers and numpy loops over the segments otherwise."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+
+from helpers import copy_gpu_to_numpy, copy_numpy_to_gpu, from_storage, gpu_tensor, to_storage
+from thor_amd import physical as ph
+from thor_amd.dtypes import DataType
+from thor_amd.physical import Expression as ex
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def stream(gpu):
+    return ph.Stream(0)
+
+
+class Ragged:
+    """The composition rules of the reference's RaggedExpression (RaggedExpression.cpp:204-330) spelled with Expression primitives."""
+
+    def __init__(self, name, batch, capacity, trailing=()):
+        self.values, self.offsets = ex.input(name + ".values"), ex.input(name + ".offsets")
+        self.batch, self.capacity, self.trailing = batch, capacity, tuple(trailing)
+        self.elements = int(np.prod(trailing)) if trailing else 1
+
+    def wrap(self, values):
+        return values.with_ragged_runtime_extent(self.offsets, self.batch, self.capacity, self.elements)
+
+    def reduce(self, values, kind):
+        return getattr(values, "segment_" + kind)(self.offsets, self.batch, self.capacity, self.elements)
+
+    def spread(self, per_segment, normalize=False):
+        return per_segment.segmented_broadcast(self.offsets, self.batch, self.capacity, self.elements, normalize)
+
+    def softmax(self, log=False):
+        shifted = self.values - self.spread(self.reduce(self.values, "max"))
+        e = shifted.exp()
+        total = self.spread(self.reduce(e, "sum"))
+        return self.wrap(shifted - total.ln() if log else e / total)
+
+
+def run(expr_or_outputs, inputs, stream, preallocated=None):
+    eq = ex.compile(expr_or_outputs, device_num=0)
+    plan = eq.stamp(inputs, stream, preallocated_outputs=preallocated)
+    plan.run()
+    return plan, eq
+
+
+def test_segment_sum_min_max_mean_for_empty_and_skewed_rows(stream):
+    """RaggedExpressionTest.cpp:1795-1824."""
+    r = Ragged("x", 4, 9)
+    inputs = {"x.values": copy_numpy_to_gpu(np.array([1, -2, 4, 5, 7, -1, 8, 99, 100], np.float32), stream, DataType.fp32),
+              "x.offsets": copy_numpy_to_gpu(np.array([0, 3, 3, 5, 7], np.uint32), stream, DataType.uint32)}
+    outputs = ex.outputs({k: r.reduce(r.values, k) for k in ("sum", "min", "max", "mean")})
+    plan, eq = run(outputs, inputs, stream)
+    assert sorted(plan.stage_kind_names()) == ["SegmentedReduction"] * 4
+    got = {k: copy_gpu_to_numpy(plan.output(k), stream) for k in ("sum", "min", "max", "mean")}
+    np.testing.assert_array_equal(got["sum"], np.array([3, 0, 12, 7], np.float32))
+    np.testing.assert_array_equal(got["mean"], np.array([1, 0, 6, 3.5], np.float32))
+    np.testing.assert_array_equal(got["min"], np.array([-2, np.inf, 5, -1], np.float32))
+    np.testing.assert_array_equal(got["max"], np.array([4, -np.inf, 7, 8], np.float32))
+
+
+@pytest.mark.parametrize("log", [False, True], ids=["softmax", "log_softmax"])
+def test_segment_softmax_per_row_leaves_unused_capacity_untouched(stream, log):
+    """RaggedExpressionTest.cpp:1826-1884: scalar values, an empty row, three rows of capacity nobody owns."""
+    r = Ragged("x", 3, 8)
+    x = np.array([1, 2, 0, -1, 1, 50, 60, 70], np.float32)
+    inputs = {"x.values": copy_numpy_to_gpu(x, stream, DataType.fp32), "x.offsets": copy_numpy_to_gpu(np.array([0, 2, 2, 5], np.uint32), stream, DataType.uint32)}
+    out = copy_numpy_to_gpu(np.full(8, 321.0, np.float32), stream, DataType.fp32)
+    plan, _ = run(ex.outputs({"y": r.softmax(log)}), inputs, stream, {"y": out})
+    got = copy_gpu_to_numpy(plan.output("y"), stream)
+    want = np.full(8, 321.0, np.float64)
+    for lo, hi in ((0, 2), (2, 5)):
+        e = np.exp(x[lo:hi].astype(np.float64) - x[lo:hi].max())
+        want[lo:hi] = np.log(e / e.sum()) if log else e / e.sum()
+    np.testing.assert_allclose(got, want, rtol=0, atol=2e-5)
+    assert np.array_equal(got[5:], np.full(3, 321.0, np.float32))
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16, DataType.fp16], ids=lambda d: d.name)
+def test_vector_segment_softmax_per_component(stream, dtype):
+    """RaggedExpressionTest.cpp:1940-1981: [32, 2] capacity, five active rows in four segments, fp16 / bf16 / fp32."""
+    capacity = 32
+    values = np.full((capacity, 2), 91.0, np.float32)
+    values[:5] = np.array([[1, 10], [3, 6], [-1, 4], [5, -2], [7, 8]], np.float32)
+    r = Ragged("x", 4, capacity, (2,))
+    inputs = {"x.values": copy_numpy_to_gpu(to_storage(values, dtype), stream, dtype),
+              "x.offsets": copy_numpy_to_gpu(np.array([0, 2, 2, 3, 5], np.uint32), stream, DataType.uint32)}
+    out = copy_numpy_to_gpu(to_storage(np.full((capacity, 2), 77.0, np.float32), dtype), stream, dtype)
+    plan, _ = run(ex.outputs({"y": r.softmax()}), inputs, stream, {"y": out})
+    got = from_storage(copy_gpu_to_numpy(plan.output("y"), stream), dtype)
+    e2, e10, e6 = np.exp(2.0), np.exp(10.0), np.exp(6.0)
+    want = np.full((capacity, 2), 77.0)
+    want[:5] = [[1 / (1 + e2), e10 / (e10 + e6)], [e2 / (1 + e2), e6 / (e10 + e6)], [1, 1], [1 / (1 + e2), 1 / (1 + e10)], [e2 / (1 + e2), e10 / (1 + e10)]]
+    np.testing.assert_allclose(got, want, rtol=0, atol=3e-5 if dtype == DataType.fp32 else 2e-2)
+
+
+def test_valuewise_kernels_follow_the_offsets_of_each_run(stream):
+    """RaggedExpressionTest.cpp:1758-1793: the active extent is read on the device, so one stamped plan serves every partition."""
+    r = Ragged("x", 3, 1000, (3,))
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((1000, 3)).astype(np.float32)
+    offsets = copy_numpy_to_gpu(np.array([0, 10, 10, 40], np.uint32), stream, DataType.uint32)
+    inputs = {"x.values": copy_numpy_to_gpu(x, stream, DataType.fp32), "x.offsets": offsets}
+    out = gpu_tensor([1000, 3], DataType.fp32)
+    plan, _ = run(ex.outputs({"y": r.wrap((r.values * 2.0 + 1.0).abs())}), inputs, stream, {"y": out})
+    assert plan.stage_kind_names() == ["FusedKernel"]
+    for active in (40, 7, 1000, 0, 333):
+        out.copy_from_async(copy_numpy_to_gpu(np.full((1000, 3), -5.0, np.float32), stream, DataType.fp32), stream)
+        offsets.copy_from_async(copy_numpy_to_gpu(np.array([0, min(active, 3), min(active, 3), active], np.uint32), stream, DataType.uint32), stream)
+        plan.run()
+        got = copy_gpu_to_numpy(out, stream)
+        np.testing.assert_array_equal(got[:active], np.abs(x[:active] * np.float32(2.0) + np.float32(1.0)))
+        assert np.all(got[active:] == -5.0), active
+
+
+SHAPES = [((5000,), 37), ((4096, 8), 300), ((3000, 3, 5), 12), ((20000, 64), 2000)]
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16], ids=lambda d: d.name)
+@pytest.mark.parametrize("shape,segments", SHAPES, ids=[f"{s}-{b}" for s, b in SHAPES])
+def test_random_ragged_softmax_and_centering_against_numpy(stream, shape, segments, dtype):
+    rng = np.random.default_rng(segments)
+    capacity = shape[0]
+    active = capacity - capacity // 5
+    cuts = np.sort(rng.integers(0, active + 1, segments - 1))
+    offsets = np.concatenate([[0], cuts, [active]]).astype(np.int64)
+    x = to_storage(rng.standard_normal(shape).astype(np.float32) * 3, dtype)
+    xf = from_storage(x, dtype).astype(np.float64)
+    r = Ragged("x", segments, capacity, shape[1:])
+    inputs = {"x.values": copy_numpy_to_gpu(x, stream, dtype), "x.offsets": copy_numpy_to_gpu(offsets.astype(np.uint32), stream, DataType.uint32)}
+    centered = r.wrap(r.values - r.spread(r.reduce(r.values, "sum"), normalize=True))
+    filler = to_storage(np.full(shape, 9.0, np.float32), dtype)
+    pre = {"softmax": copy_numpy_to_gpu(filler, stream, dtype), "centered": copy_numpy_to_gpu(filler, stream, dtype)}
+    plan, _ = run(ex.outputs({"softmax": r.softmax(), "centered": centered}), inputs, stream, pre)
+    got_softmax = from_storage(copy_gpu_to_numpy(plan.output("softmax"), stream), dtype).astype(np.float64)
+    got_centered = from_storage(copy_gpu_to_numpy(plan.output("centered"), stream), dtype).astype(np.float64)
+    want_softmax, want_centered = np.full(shape, 9.0), np.full(shape, 9.0)
+    for b in range(segments):
+        lo, hi = offsets[b], offsets[b + 1]
+        if hi > lo:
+            e = np.exp(xf[lo:hi] - xf[lo:hi].max(axis=0))
+            want_softmax[lo:hi] = e / e.sum(axis=0)
+            want_centered[lo:hi] = xf[lo:hi] - xf[lo:hi].mean(axis=0)
+    tolerance = 2e-5 if dtype == DataType.fp32 else 3e-2
+    np.testing.assert_allclose(got_softmax, want_softmax, rtol=0, atol=tolerance)
+    np.testing.assert_allclose(got_centered, want_centered, rtol=0, atol=tolerance * 4)
+
+
+def test_dtype_and_shape_rules(stream):
+    x = copy_numpy_to_gpu(np.zeros((6, 2), np.float32), stream, DataType.fp16)
+    offsets = copy_numpy_to_gpu(np.array([0, 2, 6], np.uint32), stream, DataType.uint32)
+    v, o = ex.input("v"), ex.input("o")
+    eq = ex.compile(ex.outputs({"s": v.segment_sum(o)}), device_num=0)
+    plan = eq.stamp({"v": x, "o": offsets}, stream)
+    assert plan.output("s").get_data_type() == DataType.fp16 and plan.output("s").get_dimensions() == [2, 2]
+    with pytest.raises(RuntimeError, match="offsets must have UINT32 or UINT64"):
+        ex.compile(ex.outputs({"s": v.segment_sum(o)}), device_num=0).stamp({"v": x, "o": copy_numpy_to_gpu(np.zeros(3, np.float32), stream, DataType.fp32)}, stream)
+    with pytest.raises(RuntimeError, match="output dtype to match input dtype"):
+        ex.compile(ex.outputs({"s": v.segment_sum(o).with_output_dtype(DataType.fp32)}), device_num=0).stamp({"v": x, "o": offsets}, stream)
+    with pytest.raises(ValueError, match="direct input"):
+        v.with_ragged_runtime_extent(o + 1.0, 2, 6, 2)
+    with pytest.raises(RuntimeError, match="batch size \\+ 1"):
+        ex.compile(ex.outputs({"s": v.segment_sum(o, 5, 6, 2)}), device_num=0).stamp({"v": x, "o": offsets}, stream)

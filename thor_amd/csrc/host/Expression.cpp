@@ -486,6 +486,68 @@ Expression Expression::withDTypes(std::optional<DataType> compute_dtype, std::op
     return Expression(out, root);
 }
 
+// ---- ragged batches ------------------------------------------------------------------------------------------------------
+Expression Expression::segmentedReduceWithRaggedMetadata(const Expression& input, const Expression& offsets, ExprOp op, uint64_t ragged_batch_size,
+                                                         uint64_t ragged_max_active_values, uint64_t ragged_elements_per_value) {
+    if (!isSegmentedReduceOp(op)) throw std::invalid_argument("segmentedReduceWithRaggedMetadata requires a segmented reduction op.");
+    if ((ragged_batch_size == 0) != (ragged_max_active_values == 0)) {
+        throw std::invalid_argument("Segmented reduction ragged metadata requires both batch size and max active values, or neither.");
+    }
+    if (ragged_elements_per_value == 0) throw std::invalid_argument("Segmented reduction ragged elements-per-value metadata must be non-zero.");
+    Expression out = binaryOp(input, offsets, op);
+    if (ragged_batch_size != 0) {
+        ExprNode& node = out.expr->nodes.at(out.nodeIndex);
+        node.ragged_runtime_batch_size = ragged_batch_size;
+        node.ragged_runtime_max_active_values = ragged_max_active_values;
+        node.ragged_runtime_elements_per_value = ragged_elements_per_value;
+    }
+    return out;
+}
+
+Expression Expression::segmentedReduceSum(const Expression& input, const Expression& offsets) {
+    return segmentedReduceWithRaggedMetadata(input, offsets, ExprOp::SEGMENTED_REDUCE_SUM, 0, 0);
+}
+Expression Expression::segmentedReduceMin(const Expression& input, const Expression& offsets) {
+    return segmentedReduceWithRaggedMetadata(input, offsets, ExprOp::SEGMENTED_REDUCE_MIN, 0, 0);
+}
+Expression Expression::segmentedReduceMax(const Expression& input, const Expression& offsets) {
+    return segmentedReduceWithRaggedMetadata(input, offsets, ExprOp::SEGMENTED_REDUCE_MAX, 0, 0);
+}
+Expression Expression::segmentedReduceMean(const Expression& input, const Expression& offsets) {
+    return segmentedReduceWithRaggedMetadata(input, offsets, ExprOp::SEGMENTED_REDUCE_MEAN, 0, 0);
+}
+
+Expression Expression::segmentedBroadcast(const Expression& per_segment_values, const Expression& offsets, uint64_t batch_size,
+                                          uint64_t max_active_values, uint64_t elements_per_value, bool normalize_by_segment_length) {
+    if (batch_size == 0 || max_active_values == 0 || elements_per_value == 0) {
+        throw std::invalid_argument("Expression::segmentedBroadcast requires non-zero batch size, row capacity and elements per value.");
+    }
+    Expression out = binaryOp(per_segment_values, offsets, ExprOp::SEGMENTED_BROADCAST);
+    ExprNode& node = out.expr->nodes.at(out.nodeIndex);
+    node.ragged_runtime_batch_size = batch_size;
+    node.ragged_runtime_max_active_values = max_active_values;
+    node.ragged_runtime_elements_per_value = elements_per_value;
+    node.segmented_broadcast_normalize_by_length = normalize_by_segment_length;
+    return out;
+}
+
+Expression Expression::withRaggedRuntimeExtent(const Expression& offsets, uint64_t batch_size, uint64_t max_active_values,
+                                               uint64_t elements_per_value) const {
+    if (batch_size + 1 <= batch_size) throw std::invalid_argument("Expression::withRaggedRuntimeExtent batch size overflows offsets element count.");
+    if (max_active_values == 0 || elements_per_value == 0) {
+        throw std::invalid_argument("Expression::withRaggedRuntimeExtent requires non-zero maximum extent metadata.");
+    }
+    if (!offsets.expr || offsets.expr->nodes.at(offsets.nodeIndex).op != ExprOp::INPUT) {
+        throw std::invalid_argument("Expression::withRaggedRuntimeExtent currently requires offsets to be a direct input expression.");
+    }
+    Expression out = binaryOp(*this, offsets, ExprOp::RAGGED_VALUEWISE_EXTENT);
+    ExprNode& node = out.expr->nodes.at(out.nodeIndex);
+    node.ragged_runtime_batch_size = batch_size;
+    node.ragged_runtime_max_active_values = max_active_values;
+    node.ragged_runtime_elements_per_value = elements_per_value;
+    return out;
+}
+
 // ---- op classification ---------------------------------------------------------------------------------------------------
 bool Expression::isLeafOp(ExprOp op) {
     return op == ExprOp::INPUT || op == ExprOp::RUNTIME_SCALAR || op == ExprOp::TENSOR_RUNTIME_SCALAR || op == ExprOp::SCALAR_FP ||
@@ -564,6 +626,9 @@ std::string opName(ExprOp op) {
         {(uint16_t)ExprOp::REDUCE_PROD, "reduce_prod"}, {(uint16_t)ExprOp::REDUCE_MIN, "reduce_min"}, {(uint16_t)ExprOp::REDUCE_MAX, "reduce_max"},
         {(uint16_t)ExprOp::REDUCE_ARGMIN, "argmin"}, {(uint16_t)ExprOp::REDUCE_ARGMAX, "argmax"}, {(uint16_t)ExprOp::REDUCE_AVG, "reduce_mean"},
         {(uint16_t)ExprOp::REDUCE_NORM1, "reduce_norm1"}, {(uint16_t)ExprOp::REDUCE_NORM2, "reduce_norm2"},
+        {(uint16_t)ExprOp::SEGMENTED_REDUCE_SUM, "segmented_reduce_sum"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MIN, "segmented_reduce_min"},
+        {(uint16_t)ExprOp::SEGMENTED_REDUCE_MAX, "segmented_reduce_max"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MEAN, "segmented_reduce_mean"},
+        {(uint16_t)ExprOp::SEGMENTED_BROADCAST, "segmented_broadcast"}, {(uint16_t)ExprOp::RAGGED_VALUEWISE_EXTENT, "ragged_valuewise_extent"},
     };
     auto it = names.find(static_cast<uint16_t>(op));
     return it == names.end() ? "op" + std::to_string(static_cast<int>(op)) : it->second;
@@ -625,6 +690,11 @@ std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex,
         if (n.op == ExprOp::RESHAPE) text += ":dims=" + axesText(n.reshape_dims);
         if (n.op == ExprOp::UNSQUEEZE) text += ":axes=" + axesText(n.unsqueeze_axes);
         if (n.op == ExprOp::SQUEEZE) text += ":axes=" + axesText(n.squeeze_axes);
+        if (isRaggedOp(n.op)) {
+            text += ":ragged=[" + std::to_string(n.ragged_runtime_batch_size) + "," + std::to_string(n.ragged_runtime_max_active_values) + "," +
+                    std::to_string(n.ragged_runtime_elements_per_value) + "]";
+            if (n.op == ExprOp::SEGMENTED_BROADCAST) text += n.segmented_broadcast_normalize_by_length ? ":normalized" : "";
+        }
         if (n.op == ExprOp::SOFTMAX) {
             text += std::string(":alg=") + std::to_string(static_cast<int>(n.softmax_algorithm)) + ":mode=" + std::to_string(static_cast<int>(n.softmax_mode));
         }

@@ -29,6 +29,7 @@ bool isBindableInputDType(DataType dtype) {
 }
 
 void rejectUnsupportedOp(ExprOp op) {
+    if (isRaggedOp(op)) return;
     if (Expression::isLeafOp(op) || Expression::isUnaryOp(op) || Expression::isBinaryOp(op) || Expression::isTernaryOp(op)) {
         if (op != ExprOp::TENSOR_RUNTIME_SCALAR) return;
     }
@@ -37,6 +38,7 @@ void rejectUnsupportedOp(ExprOp op) {
 
 std::vector<DataType> tensorParentDTypes(const ExprNode& node, const std::vector<ExprNode>& nodes, const std::vector<DataType>& resolved) {
     std::vector<DataType> out;
+    if (isRaggedOp(node.op)) return {resolved.at(node.lhs)};  // the offsets are structure, not a value
     auto add = [&](uint32_t parent) {
         if (parent >= nodes.size()) throw std::runtime_error("Parent node index out of range during dtype resolution.");
         if (!isScalarLeaf(nodes[parent].op)) out.push_back(resolved[parent]);
@@ -59,7 +61,33 @@ DataType promoteWhereBranches(const std::vector<DataType>& dtypes) {
     throw std::runtime_error("Where branch dtypes must either match exactly or be supported floating dtypes.");
 }
 
+const char* raggedOpLabel(ExprOp op) {
+    if (op == ExprOp::SEGMENTED_BROADCAST) return "segmented-broadcast";
+    if (op == ExprOp::RAGGED_VALUEWISE_EXTENT) return "ragged valuewise extent";
+    return "segmented-reduction";
+}
+
+// Reference rules (Utilities/Expression/ExpressionDTypeResolution.cpp:635-646,705-733 there): offsets are UINT32 / UINT64, the
+// result has the values' dtype, and segmented reductions / broadcasts take floating-point values only.
+DataType raggedOutputDType(const ExprNode& node, const std::vector<DataType>& resolved) {
+    const DataType offsets = resolved.at(node.rhs);
+    if (offsets != DataType::UINT32 && offsets != DataType::UINT64) {
+        throw std::runtime_error(std::string(raggedOpLabel(node.op)) + " offsets must have UINT32 or UINT64 dtype, received: " + dataTypeName(offsets));
+    }
+    const DataType values = resolved.at(node.lhs);
+    if (node.op == ExprOp::RAGGED_VALUEWISE_EXTENT) return node.output_dtype.value_or(values);
+    if (!isSupportedFusionFloatingType(values)) {
+        throw std::runtime_error(std::string("Unsupported ") + raggedOpLabel(node.op) + " dtype: " + dataTypeName(values));
+    }
+    if (node.output_dtype.has_value() && node.output_dtype.value() != values) {
+        throw std::runtime_error(std::string("Expression ") + (node.op == ExprOp::SEGMENTED_BROADCAST ? "segmented broadcast" : "segmented reduction") +
+                                 " currently requires output dtype to match input dtype.");
+    }
+    return values;
+}
+
 DataType nodeOutputDType(const ExprNode& node, const std::vector<ExprNode>& nodes, const std::vector<DataType>& resolved) {
+    if (isRaggedOp(node.op)) return raggedOutputDType(node, resolved);
     if (isArgReductionOp(node.op)) return DataType::UINT32;
     if (isValueReductionOp(node.op)) {
         // fp32 accumulate and finalise, then one conversion to the requested storage dtype (fp32 unless overridden)
@@ -151,7 +179,9 @@ void propagateMaterialisedDTypes(PhysicalExpression& expr, const std::vector<uin
         auto toParent = [&](uint32_t p) { seed(required.at(p), flowing); };
         if (node.op == ExprOp::CAST) {
             // an explicit conversion boundary: the source keeps its own compute dtype
-        } else if (isReductionOp(node.op) || node.op == ExprOp::SOFTMAX) {
+        } else if (node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST) {
+            toParent(node.lhs);  // never into the offsets
+        } else if (isReductionOp(node.op) || node.op == ExprOp::SOFTMAX || isSegmentedReduceOp(node.op)) {
             // the reduction's mandatory fp32 stays inside the reduction; its producer keeps its own policy
             const ExprNode& producer = expr.nodes.at(node.lhs);
             if (producer.compute_dtype) {
@@ -202,8 +232,10 @@ void resolveInPlace(PhysicalExpression& expr, const std::vector<DataType>& rootD
         const DataType out = nodeOutputDType(node, expr.nodes, resolved);
         const DataType logicalIn = nodeLogicalInputDType(node, expr.nodes, resolved);
         DataType requested;
-        if (node.op == ExprOp::CAST || isShapeOnly(node.op)) {
-            requested = out;
+        if (node.op == ExprOp::CAST || isShapeOnly(node.op) || node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST) {
+            requested = out;  // values pass through unchanged (a normalised broadcast divides in fp32 and rounds once)
+        } else if (isSegmentedReduceOp(node.op)) {
+            requested = DataType::FP32;
         } else if (node.op == ExprOp::SOFTMAX) {
             requested = DataType::FP32;  // fp32 arithmetic whatever the storage
         } else if (node.op == ExprOp::SUB && (logicalIn == DataType::UINT32 || logicalIn == DataType::UINT64) && logicalIn == out) {
@@ -285,13 +317,13 @@ DataType toSupportedComputeDType(ExprOp op, DataType requested) {
         if (isSupportedFusionFloatingType(requested)) return toSupportedComputeDType(ExprOp::ADD, requested);
         throw std::runtime_error("Unsupported boolean/comparison/where dtype in toSupportedComputeDType.");
     }
-    if (op == ExprOp::CAST || isShapeOnly(op)) {
+    if (op == ExprOp::CAST || isShapeOnly(op) || op == ExprOp::RAGGED_VALUEWISE_EXTENT || op == ExprOp::SEGMENTED_BROADCAST) {
         if (isBindableInputDType(requested)) return requested;
         throw std::runtime_error("Unsupported passthrough dtype in toSupportedComputeDType.");
     }
     if (op == ExprOp::SUB && (requested == DataType::UINT32 || requested == DataType::UINT64)) return requested;
     if (!isSupportedFusionFloatingType(requested)) throw std::runtime_error("Unsupported dtype in toSupportedComputeDType.");
-    if (isReductionOp(op) || op == ExprOp::SOFTMAX) return DataType::FP32;
+    if (isReductionOp(op) || op == ExprOp::SOFTMAX || isSegmentedReduceOp(op)) return DataType::FP32;
     if (isFp8Type(requested) || requested == DataType::FP16) return DataType::FP16;
     return requested;  // bf16 or fp32
 }

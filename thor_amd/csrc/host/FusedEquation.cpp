@@ -49,7 +49,8 @@ std::string structuralKey(const ExprNode& n) {
     k << static_cast<int>(n.op) << "|" << n.lhs << "|" << n.rhs << "|" << n.aux << "|" << n.input_slot << "|" << formatFloatCanonical(n.scalar_fp)
       << "|" << (n.input_tensor_dtype ? static_cast<int>(*n.input_tensor_dtype) : -1) << "|" << (n.output_dtype ? static_cast<int>(*n.output_dtype) : -1)
       << "|" << (n.compute_dtype ? static_cast<int>(*n.compute_dtype) : -1) << "|" << axesKey(n.reduction_axes) << "|" << axesKey(n.squeeze_axes)
-      << "|" << axesKey(n.unsqueeze_axes) << "|" << axesKey(n.reshape_dims) << "|" << axesKey(n.fill_dims);
+      << "|" << axesKey(n.unsqueeze_axes) << "|" << axesKey(n.reshape_dims) << "|" << axesKey(n.fill_dims) << "|" << n.ragged_runtime_batch_size << "|"
+      << n.ragged_runtime_max_active_values << "|" << n.ragged_runtime_elements_per_value << "|" << n.segmented_broadcast_normalize_by_length;
     return k.str();
 }
 
@@ -124,8 +125,10 @@ class GraphBuilder {
             remap.emplace(srcIndex, idx);
             return idx;
         }
-        if (isReductionOp(node.op)) {
+        if (isReductionOp(node.op) || isSegmentedReduceOp(node.op)) {
             node.lhs = asTensorOperand(node.lhs, true);
+        } else if (node.op == ExprOp::SEGMENTED_BROADCAST) {
+            node.lhs = asTensorOperand(node.lhs, false);
         } else if (isShapeOnly(node.op)) {
             double folded;
             if (!tryFoldConstant(out, node.lhs, folded)) node.lhs = asTensorOperand(node.lhs, false);
@@ -149,7 +152,11 @@ void collectSources(const PlannedGraph& g, uint32_t root, std::vector<uint32_t>&
     std::vector<char> seen(g.expr.nodes.size(), 0);
     std::vector<uint32_t> stack;
     const ExprNode& r = g.expr.nodes[root];
-    for (uint32_t c : {r.lhs, r.rhs, r.aux})
+    // the offsets under a runtime-extent marker are the kernel's extent, not one of its value sources
+    auto valueChildren = [](const ExprNode& n) {
+        return n.op == ExprOp::RAGGED_VALUEWISE_EXTENT ? std::vector<uint32_t>{n.lhs} : std::vector<uint32_t>{n.lhs, n.rhs, n.aux};
+    };
+    for (uint32_t c : valueChildren(r))
         if (c != UINT32_MAX) stack.push_back(c);
     if (r.op == ExprOp::RUNTIME_SCALAR) scalarSlots.push_back(r.input_slot);
     while (!stack.empty()) {
@@ -163,7 +170,7 @@ void collectSources(const PlannedGraph& g, uint32_t root, std::vector<uint32_t>&
         }
         const ExprNode& node = g.expr.nodes[n];
         if (node.op == ExprOp::RUNTIME_SCALAR) scalarSlots.push_back(node.input_slot);
-        for (uint32_t c : {node.lhs, node.rhs, node.aux})
+        for (uint32_t c : valueChildren(node))
             if (c != UINT32_MAX) stack.push_back(c);
     }
     std::sort(sources.begin(), sources.end());
@@ -252,6 +259,34 @@ std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std:
             case ExprOp::SQUEEZE:
                 dims[i] = StampedEquation::computeReductionOutputDims(dims[n.lhs], {}, n.squeeze_axes.empty() ? std::vector<uint64_t>{UINT64_MAX} : n.squeeze_axes);
                 break;
+            case ExprOp::RAGGED_VALUEWISE_EXTENT:
+                dims[i] = dims[n.lhs];
+                break;
+            case ExprOp::SEGMENTED_REDUCE_SUM:
+            case ExprOp::SEGMENTED_REDUCE_MIN:
+            case ExprOp::SEGMENTED_REDUCE_MAX:
+            case ExprOp::SEGMENTED_REDUCE_MEAN: {
+                // values [N, D...] and offsets [B + 1] -> [B, D...]
+                if (dims[n.lhs].empty() || dims[n.rhs].size() != 1 || dims[n.rhs][0] < 2) {
+                    throw std::runtime_error("Segmented reduction requires values [N, D...] and offsets [B + 1] with at least one segment.");
+                }
+                if (n.ragged_runtime_batch_size != 0 && dims[n.rhs][0] != n.ragged_runtime_batch_size + 1) {
+                    throw std::runtime_error("Segmented reduction offsets do not have the ragged descriptor's batch size + 1 entries.");
+                }
+                dims[i] = dims[n.lhs];
+                dims[i][0] = dims[n.rhs][0] - 1;
+                break;
+            }
+            case ExprOp::SEGMENTED_BROADCAST: {
+                // per-segment values [B, D...] -> rows [capacity, D...]
+                if (dims[n.lhs].empty() || dims[n.rhs].size() != 1 || dims[n.rhs][0] != dims[n.lhs][0] + 1) {
+                    throw std::runtime_error("Segmented broadcast requires per-segment values [B, D...] and offsets [B + 1].");
+                }
+                if (n.ragged_runtime_max_active_values == 0) throw std::runtime_error("Segmented broadcast is missing its row capacity.");
+                dims[i] = dims[n.lhs];
+                dims[i][0] = n.ragged_runtime_max_active_values;
+                break;
+            }
             default:
                 if (isReductionOp(n.op)) {
                     const std::vector<uint64_t> axes = sortedAxesOrAll(n.reduction_axes, dims[n.lhs].size());
@@ -386,6 +421,14 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             } else if (isReductionOp(n.op)) {
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
+            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
+                graph->role[i] = Role::Materialized;
+                ensureTensor(n.lhs);
+                ensureTensor(n.rhs);
+            } else if (n.op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
+                // the kernel that produces these values stops at the rows the partition covers
+                graph->role[i] = Role::Materialized;
+                ensureTensor(n.rhs);
             } else if (isShapeOnly(n.op)) {
                 double folded;
                 if (!tryFoldConstant(graph->expr, i, folded)) {
@@ -402,6 +445,9 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             std::vector<uint32_t> sources, scalars;
             if (isReductionOp(graph->expr.nodes[i].op)) {
                 sources.push_back(graph->expr.nodes[i].lhs);
+            } else if (isSegmentedReduceOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST) {
+                sources.push_back(graph->expr.nodes[i].lhs);
+                sources.push_back(graph->expr.nodes[i].rhs);
             } else {
                 collectSources(*graph, i, sources, scalars);
             }
@@ -556,8 +602,47 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
         for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
             if (graph->role[i] != Role::Materialized || graph->level[i] != level || done[i]) continue;
             const ExprNode& n = expr.nodes[i];
+            if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
+                if (fusedKernelsOnly) {
+                    throw std::runtime_error(
+                        "FusedEquation::run() only supports expressions that lower to fused kernels; this expression has a segmented stage. "
+                        "Use stamp() and run the returned plan.");
+                }
+                const Tensor& values = tensorOf[n.lhs];
+                const Tensor& offsets = tensorOf[n.rhs];
+                Tensor output = allocateFor(i);
+                StampedExecutionStage stage;
+                stage.gpu_num = device_num;
+                stage.dependency_stage_indices = dependenciesOf({n.lhs, n.rhs});
+                if (n.op == ExprOp::SEGMENTED_BROADCAST) {
+                    stage.kind = StampedExecutionStage::Kind::SegmentedBroadcast;
+                    stage.segmented_broadcast = stampSegmentedBroadcast(values, offsets, output, n.segmented_broadcast_normalize_by_length, stream);
+                } else {
+                    const CubReductionOp op = n.op == ExprOp::SEGMENTED_REDUCE_SUM   ? CubReductionOp::Sum
+                                              : n.op == ExprOp::SEGMENTED_REDUCE_MIN ? CubReductionOp::Min
+                                              : n.op == ExprOp::SEGMENTED_REDUCE_MAX ? CubReductionOp::Max
+                                                                                     : CubReductionOp::Mean;
+                    stage.kind = StampedExecutionStage::Kind::SegmentedReduction;
+                    // the partition is read on the device every time the plan runs: nothing about it is fixed here
+                    stage.segmented_reduction = std::make_shared<StampedSegmentedReductionStage>(
+                        CubSegmentedReduction(op, n.output_dtype.value()).stampRuntimeOffsets(values, output, offsets, stream));
+                }
+                tensorOf[i] = output;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(stage));
+                done[i] = 1;
+                continue;
+            }
             if (!isReductionOp(n.op)) {
-                fusedGroups[orScalarShape(dims[i])].push_back(i);
+                // kernels of ragged values stop at the partition's last row, so they are grouped by partition as well
+                std::vector<uint64_t> key = orScalarShape(dims[i]);
+                if (n.op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
+                    key.push_back(UINT64_MAX);
+                    key.push_back(n.rhs);
+                    key.push_back(n.ragged_runtime_batch_size);
+                    key.push_back(n.ragged_runtime_elements_per_value);
+                }
+                fusedGroups[key].push_back(i);
                 continue;
             }
             if (fusedKernelsOnly) {
@@ -591,10 +676,27 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             done[i] = 1;
         }
 
-        for (auto& [shape, nodes] : fusedGroups) {
+        for (auto& [groupKey, nodes] : fusedGroups) {
             FusedKernelRequest request;
             request.expr = &expr;
+            const std::vector<uint64_t> shape = orScalarShape(dims[nodes.front()]);
             request.outputDims = shape;
+            std::optional<Tensor> extentOffsets;
+            if (expr.nodes[nodes.front()].op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
+                const ExprNode& marker = expr.nodes[nodes.front()];
+                extentOffsets = tensorOf[marker.rhs];
+                if (!extentOffsets->isInitialized() || !extentOffsets->isDenseContiguous() ||
+                    extentOffsets->getTotalNumElements() != marker.ragged_runtime_batch_size + 1) {
+                    throw std::runtime_error("Ragged runtime extent offsets must be a dense tensor with batch size + 1 entries.");
+                }
+                uint64_t elements = 1;
+                for (uint64_t d : shape) elements *= d;
+                if (elements != marker.ragged_runtime_max_active_values * marker.ragged_runtime_elements_per_value) {
+                    throw std::runtime_error("Ragged values do not have the shape [max active values, elements per value] their descriptor states.");
+                }
+                request.extent = RaggedExtent{marker.ragged_runtime_batch_size, marker.ragged_runtime_elements_per_value,
+                                              extentOffsets->getDataType() == DataType::UINT64};
+            }
             std::vector<uint32_t> sources, scalarSlots;
             for (uint32_t node : nodes) {
                 std::vector<uint32_t> s, sc;
@@ -640,6 +742,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             const EmittedKernel emitted = emitFusedKernel(request);
             std::shared_ptr<CompiledKernel> kernel = compileKernel(emitted.source, emitted.kernelName, device_num, emitted.fastContract);
 
+            if (extentOffsets.has_value()) inputTensors.push_back(extentOffsets.value());  // the pointer argument after the operands
             std::vector<size_t> inputArgIndex(inputTensors.size()), outputArgIndex(outputTensors.size());
             std::iota(inputArgIndex.begin(), inputArgIndex.end(), 0);
             std::vector<StampedEquation::ScalarArgument> scalarArgs;

@@ -114,6 +114,7 @@ bool aliasSource(const PhysicalExpression& e, uint32_t nodeIndex, uint32_t& sour
         case ExprOp::RESHAPE:
         case ExprOp::UNSQUEEZE:
         case ExprOp::SQUEEZE:
+        case ExprOp::RAGGED_VALUEWISE_EXTENT:  // the values themselves; the extent limits the kernel, not the arithmetic
             source = n.lhs;
             return true;
         case ExprOp::ADD:
@@ -291,6 +292,10 @@ std::vector<uint32_t> BodyEmitter::collect(const std::vector<uint32_t>& roots) c
         if (tryFoldConstant(expr, n, folded)) continue;
         need[n] = 1;
         const ExprNode& node = expr.nodes[n];
+        if (node.op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
+            stack.push_back(node.lhs);  // the offsets are read as the kernel's extent, not as a value
+            continue;
+        }
         for (uint32_t c : {node.lhs, node.rhs, node.aux})
             if (c != UINT32_MAX) stack.push_back(c);
     }
@@ -532,14 +537,23 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
     k.threads = static_cast<uint32_t>(threads);
     s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void fused_kernel(";
     for (size_t o = 0; o < r.operands.size(); ++o) s << "const " << deviceTypeName(r.operands[o].storageDType) << "* in" << o << ", ";
+    if (r.extent.has_value()) {
+        if (!k.flat) throw std::runtime_error("A ragged runtime extent needs operands of the output's own dense shape (no broadcasting).");
+        s << "const " << (r.extent->offsetsAre64 ? "unsigned long long" : "unsigned int") << "* extentOffsets, ";
+    }
     for (uint32_t slot : r.scalarSlots) s << "float s" << slot << ", ";
     for (size_t o = 0; o < r.outputs.size(); ++o) {
         s << deviceTypeName(r.outputs[o].storageDType) << "* out" << o;
         if (o + 1 < r.outputs.size() || k.passNumel) s << ", ";
     }
-    if (k.passNumel) s << indexType << " numel";
+    if (k.passNumel) s << indexType << (r.extent.has_value() ? " capacity" : " numel");
     s << ") {\n";
     s << "    typedef " << indexType << " index_t;\n";
+    if (r.extent.has_value()) {
+        // only the rows the partition covers now are computed; the rest of the outputs keeps its contents
+        s << "    const unsigned long long active = (unsigned long long)extentOffsets[" << r.extent->batchSize << "ull] * " << r.extent->elementsPerValue
+          << "ull;\n    const index_t numel = active < (unsigned long long)capacity ? (index_t)active : capacity;\n";
+    }
     s << "    constexpr int V = " << vec << ";\n";
 
     // body text for one element; `load(o)` and `store(o, value)` differ between the vector and the scalar form

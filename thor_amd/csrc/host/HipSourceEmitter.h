@@ -35,9 +35,18 @@ struct KernelOutput {
     uint64_t alignmentBytes = 256;
 };
 
+// Kernels of a ragged batch compute only the first offsets[batchSize] * elementsPerValue elements; `offsets` is passed as a
+// pointer after the operands and read on the device.
+struct RaggedExtent {
+    uint64_t batchSize = 0;
+    uint64_t elementsPerValue = 1;
+    bool offsetsAre64 = false;
+};
+
 struct FusedKernelRequest {
     const PhysicalExpression* expr = nullptr;
     std::vector<KernelOperand> operands;   // kernel arguments, in order
+    std::optional<RaggedExtent> extent;    // then the offsets pointer of the runtime extent, when there is one
     std::vector<uint32_t> scalarSlots;     // runtime scalar input slots passed by value (float), after the operands
     std::vector<KernelOutput> outputs;     // then the outputs
     std::vector<uint64_t> outputDims;      // common logical shape of every output

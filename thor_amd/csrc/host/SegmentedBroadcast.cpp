@@ -31,8 +31,8 @@ const char* rawWordName(uint32_t bytes) { return bytes == 1 ? "thor::u8" : bytes
 
 }  // namespace
 
-void launchSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, Tensor& output, bool normalize_by_segment_length,
-                              Stream& stream) {
+std::shared_ptr<StampedSegmentedBroadcast> stampSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, const Tensor& output,
+                                                                   bool normalize_by_segment_length, const Stream& stream) {
     if (!per_segment_values.isInitialized() || !segment_offsets.isInitialized() || !output.isInitialized()) {
         throw std::runtime_error("Segmented broadcast requires initialized tensors.");
     }
@@ -93,12 +93,27 @@ void launchSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& se
          "{\n    thor::broadcastSegments<gen::Cfg>(values, static_cast<const gen::Cfg::OffsetT*>(offsets), out);\n}\n";
     const std::shared_ptr<CompiledKernel> kernel = compileKernel(s.str(), "thor_segmented_broadcast", stream.getGpuNum(), /*fastContract=*/false);
 
+    std::ostringstream variant;
+    variant << "segmented_broadcast(chunk_rows=" << chunkRows << ",window=" << window << ",vec=" << vec << ",grid=" << chunks << ") [" << kernel->kernelName
+            << "]";
+    return std::make_shared<StampedSegmentedBroadcast>(kernel, per_segment_values, segment_offsets, output, static_cast<uint32_t>(chunks), variant.str());
+}
+
+void StampedSegmentedBroadcast::runOn(Stream& stream) const {
+    if (!stream.isInitialized() || stream.getGpuNum() != static_cast<int>(output.getPlacement().getDeviceNum())) {
+        throw std::runtime_error("Segmented broadcast requires tensors on the execution GPU.");
+    }
     ScopedGpu scoped(stream.getGpuNum());
-    const void* values = per_segment_values.getMemPtr();
-    const void* offsets = segment_offsets.getMemPtr();
-    void* out = output.getMemPtr();
-    std::vector<void*> args = {&values, &offsets, &out};
-    kernel->launch(static_cast<uint32_t>(chunks), 1, 1, 256, stream.getStream(), args);
+    const void* valuePointer = values.getMemPtr();
+    const void* offsetPointer = offsets.getMemPtr();
+    void* out = const_cast<Tensor&>(output).getMemPtr();
+    std::vector<void*> args = {&valuePointer, &offsetPointer, &out};
+    kernel->launch(gridX, 1, 1, 256, stream.getStream(), args);
+}
+
+void launchSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, Tensor& output, bool normalize_by_segment_length,
+                              Stream& stream) {
+    stampSegmentedBroadcast(per_segment_values, segment_offsets, output, normalize_by_segment_length, stream)->runOn(stream);
 }
 
 }  // namespace ThorImplementation

@@ -159,6 +159,10 @@ uint64_t StampedExecutionStage::flopCount() const {
             return 0;
         case Kind::FusedReduction:
             return fused_reduction ? fused_reduction->flopCount() : 0;
+        case Kind::SegmentedReduction:
+            return segmented_reduction ? segmented_reduction->flopCount() : 0;
+        case Kind::SegmentedBroadcast:
+            return 0;
     }
     return 0;
 }
@@ -186,6 +190,14 @@ void StampedExecutionStage::runOn(Stream& stream, const std::unordered_map<std::
         case Kind::FusedReduction:
             if (!fused_reduction) throw std::runtime_error("Fused reduction stage is missing its stamped reduction.");
             fused_reduction->runOn(stream, runtime_scalars);
+            return;
+        case Kind::SegmentedReduction:
+            if (!segmented_reduction) throw std::runtime_error("Segmented reduction stage is missing its stamped reduction.");
+            segmented_reduction->runOn(stream);
+            return;
+        case Kind::SegmentedBroadcast:
+            if (!segmented_broadcast) throw std::runtime_error("Segmented broadcast stage is missing its stamped broadcast.");
+            segmented_broadcast->runOn(stream);
             return;
     }
 }

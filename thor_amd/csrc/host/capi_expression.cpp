@@ -109,6 +109,27 @@ thor_expr_t thor_expr_binary(const char* method, thor_expr_t lhs, thor_expr_t rh
                       return new thor_expr{it->second(lhs->expr, rhs->expr)};)
 }
 
+thor_expr_t thor_expr_ragged(const char* method, thor_expr_t values, thor_expr_t offsets, uint64_t batch_size, uint64_t max_active_values,
+                             uint64_t elements_per_value) {
+    THOR_CAPI_TRY_PTR(
+        require(values, "expression"); require(offsets, "expression"); const std::string m = method ? method : "";
+        if (m == "segmented_broadcast" || m == "segmented_broadcast_normalized") {
+            return new thor_expr{Expression::segmentedBroadcast(values->expr, offsets->expr, batch_size, max_active_values, elements_per_value,
+                                                                m == "segmented_broadcast_normalized")};
+        }
+        if (m == "ragged_extent") {
+            return new thor_expr{values->expr.withRaggedRuntimeExtent(offsets->expr, batch_size, max_active_values, elements_per_value)};
+        }
+        ExprOp op;
+        if (m == "segment_sum") op = ExprOp::SEGMENTED_REDUCE_SUM;
+        else if (m == "segment_min") op = ExprOp::SEGMENTED_REDUCE_MIN;
+        else if (m == "segment_max") op = ExprOp::SEGMENTED_REDUCE_MAX;
+        else if (m == "segment_mean") op = ExprOp::SEGMENTED_REDUCE_MEAN;
+        else throw std::invalid_argument("Unknown ragged Expression method: " + m);
+        return new thor_expr{Expression::segmentedReduceWithRaggedMetadata(values->expr, offsets->expr, op, batch_size, max_active_values,
+                                                                           elements_per_value == 0 ? 1 : elements_per_value)};)
+}
+
 thor_expr_t thor_expr_unary(const char* method, thor_expr_t input) {
     THOR_CAPI_TRY_PTR(require(input, "expression");
                       auto it = unaryMethods().find(method ? method : "");
@@ -254,6 +275,8 @@ int thor_plan_stage_description(thor_plan_t plan, int stage, char* buffer, size_
         if (s.kernel) text = s.kernel->getDescription();
         if (s.reduction) text = s.reduction->getStamped()->getKernelVariant();
         if (s.fused_reduction) text = s.fused_reduction->getDescription();
+        if (s.segmented_reduction) text = s.segmented_reduction->getStamped()->getKernelVariant();
+        if (s.segmented_broadcast) text = s.segmented_broadcast->getKernelVariant();
         copyOut(text, buffer, capacity, nullptr);)
 }
 uint64_t thor_plan_flop_count(thor_plan_t plan) { return plan ? plan->plan.flopCount() : 0; }

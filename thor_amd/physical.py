@@ -67,7 +67,8 @@ PROTOTYPES = {
     "thor_stamped_arg_reduction_value_output": (_vp, [_vp]), "thor_stamped_arg_reduction_index_output": (_vp, [_vp]),
     "thor_stamped_arg_reduction_path": (_i, [_vp]),
     "thor_expr_input": (_vp, [_cp, _i, _i]), "thor_expr_runtime_scalar": (_vp, [_cp, _i, _i]), "thor_expr_scalar": (_vp, [ctypes.c_double]),
-    "thor_expr_fill": (_vp, [ctypes.c_double, _u64p, _i, _i]), "thor_expr_binary": (_vp, [_cp, _vp, _vp]), "thor_expr_unary": (_vp, [_cp, _vp]),
+    "thor_expr_fill": (_vp, [ctypes.c_double, _u64p, _i, _i]), "thor_expr_binary": (_vp, [_cp, _vp, _vp]),
+    "thor_expr_ragged": (_vp, [_cp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64]), "thor_expr_unary": (_vp, [_cp, _vp]),
     "thor_expr_unary_params": (_vp, [_cp, _vp, ctypes.c_double, ctypes.c_double]), "thor_expr_where": (_vp, [_vp, _vp, _vp]),
     "thor_expr_cast": (_vp, [_vp, _i]), "thor_expr_with_dtypes": (_vp, [_vp, _i, _i]),
     "thor_expr_reduce": (_vp, [_cp, _vp, _u64p, _i, _u64p, _i]), "thor_expr_reshape": (_vp, [_vp, _u64p, _i]),
@@ -639,6 +640,32 @@ class Expression:
 
     def log_softmax(self, mode: str = "channel") -> "Expression":
         return Expression(lib().thor_expr_unary_params(b"logSoftmax", self._h, 1.0, {"instance": 0.0, "channel": 1.0}[mode]))
+
+    # -- ragged batches: values [N, D...] packed row after row, offsets [B + 1] read on the device when the plan runs
+    def _ragged(self, method: str, offsets: "Expression", batch_size: int, max_active_values: int, elements_per_value: int) -> "Expression":
+        return Expression(lib().thor_expr_ragged(method.encode(), self._h, offsets._h, batch_size, max_active_values, elements_per_value))
+
+    def segment_sum(self, offsets, batch_size=0, max_active_values=0, elements_per_value=1):
+        """Per-segment sum -> [B, D...] in the values' dtype (fp32 accumulation); empty segments give 0."""
+        return self._ragged("segment_sum", offsets, batch_size, max_active_values, elements_per_value)
+
+    def segment_min(self, offsets, batch_size=0, max_active_values=0, elements_per_value=1):
+        return self._ragged("segment_min", offsets, batch_size, max_active_values, elements_per_value)
+
+    def segment_max(self, offsets, batch_size=0, max_active_values=0, elements_per_value=1):
+        return self._ragged("segment_max", offsets, batch_size, max_active_values, elements_per_value)
+
+    def segment_mean(self, offsets, batch_size=0, max_active_values=0, elements_per_value=1):
+        return self._ragged("segment_mean", offsets, batch_size, max_active_values, elements_per_value)
+
+    def segmented_broadcast(self, offsets, batch_size: int, max_active_values: int, elements_per_value: int = 1, normalize_by_segment_length: bool = False):
+        """Per-segment values [B, D...] -> rows [max_active_values, D...]; rows of no segment are undefined."""
+        method = "segmented_broadcast_normalized" if normalize_by_segment_length else "segmented_broadcast"
+        return self._ragged(method, offsets, batch_size, max_active_values, elements_per_value)
+
+    def with_ragged_runtime_extent(self, offsets, batch_size: int, max_active_values: int, elements_per_value: int = 1):
+        """The same values, computed only for the first offsets[batch_size] rows; the rest of the output keeps its contents."""
+        return self._ragged("ragged_extent", offsets, batch_size, max_active_values, elements_per_value)
 
     def reshape(self, dims: Sequence[int]) -> "Expression":
         d, rank = _u64_array([UINT64_MAX if v == -1 else v for v in dims])
