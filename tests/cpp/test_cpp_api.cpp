@@ -8,6 +8,7 @@
 #include "Utilities/Expression/Expression.h"
 #include "Utilities/Expression/ExpressionDTypeResolution.h"
 #include "Utilities/Expression/FusedEquation.h"
+#include "Utilities/Expression/RaggedExpression.h"
 #include "Utilities/TensorOperations/Cub/CubReduction.h"
 #include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
 
@@ -17,8 +18,11 @@
 #include <cstring>
 #include <functional>
 #include <limits>
+#include <optional>
+#include <set>
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 using namespace ThorImplementation;
@@ -229,6 +233,109 @@ static void offsetSegmentedReductions(Stream& stream) {
     CHECK(throwsAs<std::invalid_argument>([&] { CubSegmentedReduction(CubReductionOp::Sum).stamp(x, gpuOffsets({0, 5, 10}, stream), stream); }));
 }
 
+static void raggedExpressionStructure() {
+    // RaggedExpressionTest.cpp:739-795,907-957,2037-2055 there: names, descriptors and markers, no device work
+    const RaggedTensorDescriptor descriptor(DataType::FP32, {4}, 3, 9);
+    CHECK(descriptor.getValuesDimensions() == (std::vector<uint64_t>{9, 4}) && descriptor.getOffsetsDescriptor().getDimensions() == (std::vector<uint64_t>{4}));
+    CHECK(descriptor.getOffsetsDataType() == DataType::UINT32);
+    CHECK(throwsAs<std::invalid_argument>([] { RaggedTensorDescriptor(DataType::FP32, {4}, 3, 0); }));
+    CHECK(throwsAs<std::invalid_argument>([] { RowPartitionDescriptor(3, 9, DataType::INT32); }));
+    CHECK(throwsAs<std::invalid_argument>([] { RowPartitionDescriptor(3, 1ull << 33, DataType::UINT32); }));
+
+    const RaggedExpression x = RaggedExpression::input("x", descriptor);
+    CHECK((x.getInputNames() == std::set<std::string>{"x.values", "x.offsets"}));
+    CHECK((x.getMetadataInputNames() == std::set<std::string>{"x.offsets"}));
+    CHECK((x.getDifferentiableInputNames() == std::set<std::string>{"x.values"}));
+    CHECK(x.getRuntimeExtent().maxLaunchElements() == 36);
+    const PhysicalExpression marked = x.mapValues([](const Expression& v) { return (v.swish() + Expression(0.25)).tanh(); }).getValues().expression();
+    const ExprNode& marker = marked.nodes.at(marked.output_node);
+    CHECK(marker.op == ExprOp::RAGGED_VALUEWISE_EXTENT && marker.ragged_runtime_batch_size == 3 && marker.ragged_runtime_max_active_values == 9 &&
+          marker.ragged_runtime_elements_per_value == 4);
+    CHECK(marked.nodes.at(marker.lhs).op == ExprOp::TANH && marked.nodes.at(marker.rhs).op == ExprOp::INPUT);
+
+    const Expression shared = Expression::input("shared.offsets");
+    const RaggedExpression a(Expression::input("a.values"), shared, descriptor), b(Expression::input("b.values"), shared, descriptor);
+    const RaggedExpression sum = a + b;
+    CHECK(sum.getOffsets().isSameLogicalNode(shared) && sum.getDescriptor() == descriptor);
+    const RaggedExpression less = a.lessThan(b);
+    CHECK(less.getValuesDataType() == DataType::BOOLEAN && less.getOffsets().isSameLogicalNode(shared));
+    CHECK(a.cast(DataType::FP16).getValuesDataType() == DataType::FP16 && a.cast(DataType::FP16).getRuntimeExtent().elementsPerValue == 4);
+    const RaggedExpression other(Expression::input("c.values"), Expression::input("c.offsets"), descriptor);
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)(a + other); }));
+    const RaggedExpression wider(Expression::input("d.values"), shared, RaggedTensorDescriptor(DataType::FP32, {5}, 3, 9));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)(a + wider); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)a.withValues(Expression::input("e"), RaggedTensorDescriptor(DataType::FP32, {4}, 2, 9)); }));
+    CHECK(throwsAs<std::runtime_error>([] { (void)RaggedExpression().getValues(); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)RaggedExpression::input("i", RaggedTensorDescriptor(DataType::INT32, {}, 3, 9)).segment_mean(); }));
+
+    const PhysicalExpression reduced = x.reduce_sum().expression();
+    const ExprNode& reduction = reduced.nodes.at(reduced.output_node);
+    CHECK(reduction.op == ExprOp::SEGMENTED_REDUCE_SUM && reduction.ragged_runtime_elements_per_value == 4 && reduction.ragged_runtime_batch_size == 3);
+    CHECK(canonicalize(reduced).find("segmented_reduce_sum:ragged=[3,9,4]") != std::string::npos);
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)(Expression::input("v") + 1.0).withRaggedRuntimeExtent(Expression::input("o") + 1.0, 3, 9, 4); }));
+}
+
+static void raggedExpressionExecution(Stream& stream) {
+    // RaggedExpressionTest.cpp:1795-1824 there: empty and skewed rows
+    auto runOne = [&](const Expression& e, const std::unordered_map<std::string, Tensor>& inputs, const std::optional<Tensor>& into = std::nullopt) {
+        FusedEquation eq = FusedEquation::compile(Expression::outputs({{"out", e}}).physicalOutputs(), 0);
+        std::unordered_map<std::string, Tensor> pre;
+        if (into.has_value()) pre.emplace("out", into.value());
+        StampedExecutionPlan plan = eq.stamp(inputs, stream, pre);
+        plan.run();
+        return plan.output("out");
+    };
+    const float inf = std::numeric_limits<float>::infinity();
+    {
+        const RaggedExpression x = RaggedExpression::input("x", RaggedTensorDescriptor(DataType::FP32, {}, 4, 9));
+        const std::unordered_map<std::string, Tensor> inputs{{"x.values", gpuFrom({1, -2, 4, 5, 7, -1, 8, 99, 100}, {9}, stream)},
+                                                            {"x.offsets", gpuOffsets({0, 3, 3, 5, 7}, stream)}};
+        CHECK((toHostF32(runOne(x.segment_sum(), inputs), stream) == std::vector<float>{3, 0, 12, 7}));
+        CHECK((toHostF32(runOne(x.segment_mean(), inputs), stream) == std::vector<float>{1, 0, 6, 3.5f}));
+        CHECK((toHostF32(runOne(x.segment_min(), inputs), stream) == std::vector<float>{-2, inf, 5, -1}));
+        CHECK((toHostF32(runOne(x.segment_max(), inputs), stream) == std::vector<float>{4, -inf, 7, 8}));
+    }
+    {
+        // :1983-2035 there: [6, 2, 2] values, UINT64 offsets, one empty row, one row of capacity nobody owns
+        const RaggedExpression x = RaggedExpression::input("x", RaggedTensorDescriptor(DataType::FP32, {2, 2}, 3, 6, DataType::UINT64));
+        const std::unordered_map<std::string, Tensor> inputs{
+            {"x.values", gpuFrom({1, 2, 3, 4, 5, 6, 7, 8, -1, -2, -3, -4, 9, 10, 11, 12, 13, 14, 15, 16, 101, 102, 103, 104}, {6, 2, 2}, stream)},
+            {"x.offsets", gpuOffsets({0, 2, 2, 5}, stream, DataType::UINT64)}};
+        const Tensor sum = runOne(x.segment_sum(), inputs);
+        CHECK((sum.getDimensions() == std::vector<uint64_t>{3, 2, 2}));
+        CHECK((toHostF32(sum, stream) == std::vector<float>{6, 8, 10, 12, 0, 0, 0, 0, 21, 22, 23, 24}));
+        const float small = 1.0f / (1.0f + std::exp(4.0f)), large = 1.0f - small;
+        const Tensor softmax = runOne(x.segment_softmax().getValues(), inputs, gpuFrom(std::vector<float>(24, 555.0f), {6, 2, 2}, stream));
+        const std::vector<float> p = toHostF32(softmax, stream);
+        for (int c = 0; c < 4; ++c) {
+            CHECK_NEAR(p[c], small, 3e-5);
+            CHECK_NEAR(p[4 + c], large, 3e-5);
+        }
+        for (int i = 20; i < 24; ++i) CHECK(p[i] == 555.0f);
+        const Tensor logSoftmax = runOne(x.segment_log_softmax().getValues(), inputs, gpuFrom(std::vector<float>(24, -555.0f), {6, 2, 2}, stream));
+        const std::vector<float> lp = toHostF32(logSoftmax, stream);
+        for (int c = 0; c < 4; ++c) {
+            CHECK_NEAR(lp[c], std::log(small), 3e-5);
+            CHECK_NEAR(lp[4 + c], std::log(large), 3e-5);
+        }
+        for (int i = 20; i < 24; ++i) CHECK(lp[i] == -555.0f);
+    }
+    {
+        // :1826-1854 there: scalar values
+        const RaggedExpression x = RaggedExpression::input("x", RaggedTensorDescriptor(DataType::FP32, {}, 3, 8));
+        const std::unordered_map<std::string, Tensor> inputs{{"x.values", gpuFrom({1, 2, 0, -1, 1, 50, 60, 70}, {8}, stream)},
+                                                            {"x.offsets", gpuOffsets({0, 2, 2, 5}, stream)}};
+        const std::vector<float> p = toHostF32(runOne(x.softmax().getValues(), inputs, gpuFrom(std::vector<float>(8, 321.0f), {8}, stream)), stream);
+        const float d0 = std::exp(1.0f) + std::exp(2.0f), d2 = std::exp(0.0f) + std::exp(-1.0f) + std::exp(1.0f);
+        const std::vector<float> want{std::exp(1.0f) / d0, std::exp(2.0f) / d0, std::exp(0.0f) / d2, std::exp(-1.0f) / d2, std::exp(1.0f) / d2, 321, 321, 321};
+        for (size_t i = 0; i < want.size(); ++i) CHECK_NEAR(p[i], want[i], 2e-5);
+        // relu and a comparison, valuewise, over the active rows only
+        const RaggedExpression y = x.relu() * x.relu();
+        const std::vector<float> q = toHostF32(runOne(y.getValues(), inputs, gpuFrom(std::vector<float>(8, -7.0f), {8}, stream)), stream);
+        CHECK((q == std::vector<float>{1, 4, 0, 0, 1, -7, -7, -7}));
+    }
+}
+
 static void argReductionsTiesAndNaN(Stream& stream) {
     // CubArgReductionTest.cpp: lowest index wins ties, NaN wins, index is the position inside the reduction domain
     Tensor t = gpuFrom({1, 1, 3, 1, std::nanf(""), 0, std::nanf(""), -4}, {2, 4}, stream);
@@ -356,7 +463,8 @@ int main(int argc, char** argv) {
     };
     std::vector<Case> cases = {{"geometryPathsAndErrors", geometryPathsAndErrors},
                                {"dtypeResolutionAndStageSplit", dtypeResolutionAndStageSplit},
-                               {"cpuTypeConverter", cpuTypeConverter}};
+                               {"cpuTypeConverter", cpuTypeConverter},
+                               {"raggedExpressionStructure", raggedExpressionStructure}};
     if (mode == "gpu") {
         auto withStream = [](void (*f)(Stream&)) {
             return [f] {
@@ -367,6 +475,7 @@ int main(int argc, char** argv) {
         cases.push_back({"valueReductionsSmallExact", withStream(valueReductionsSmallExact)});
         cases.push_back({"argReductionsTiesAndNaN", withStream(argReductionsTiesAndNaN)});
         cases.push_back({"offsetSegmentedReductions", withStream(offsetSegmentedReductions)});
+        cases.push_back({"raggedExpressionExecution", withStream(raggedExpressionExecution)});
         cases.push_back({"expressionConfig1AndRuntimeScalars", withStream(expressionConfig1AndRuntimeScalars)});
         cases.push_back({"softmaxPlansAndRowKernel", withStream(softmaxPlansAndRowKernel)});
         cases.push_back({"typeConverterOnGpuAndTensorViews", withStream(typeConverterOnGpuAndTensorViews)});
