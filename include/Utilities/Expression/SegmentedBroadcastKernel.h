@@ -37,6 +37,10 @@ class StampedSegmentedBroadcast {
 std::shared_ptr<StampedSegmentedBroadcast> stampSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, const Tensor& output,
                                                                    bool normalize_by_segment_length, const Stream& stream);
 
+// ids[r] = the segment row r belongs to, for every row inside a segment (UINT32 [N]; other rows keep their contents).  The
+// index fused kernels read per-segment values through.
+std::shared_ptr<StampedSegmentedBroadcast> stampSegmentIds(const Tensor& segment_offsets, const Tensor& ids, const Stream& stream);
+
 void launchSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, Tensor& output, bool normalize_by_segment_length,
                               Stream& stream);
 

@@ -581,7 +581,8 @@ __device__ __forceinline__ u64 waveLowerBound(u64 n, Pred pred) {
 }
 
 // Cfg: T (storage type), OffsetT, kE (elements per value), kRows, kSegments, kChunkRows, kVec (elements per store; kChunkRows * kE
-// is a multiple of it), kThreads, kWindow (a power of two), kNormalize, kViaHalf (round through fp16 first: e5m2).
+// is a multiple of it), kThreads, kWindow (a power of two), kNormalize, kViaHalf (round through fp16 first: e5m2), kIds (write
+// the segment's number instead of a value: the row -> segment index that fused kernels gather per-segment values through).
 template <typename Cfg>
 __device__ __forceinline__ typename Cfg::T broadcastValue(typename Cfg::T value, u64 length) {
     if constexpr (!Cfg::kNormalize) {
@@ -624,7 +625,7 @@ __device__ __forceinline__ void broadcastSegments(const typename Cfg::T* values,
                 for (int step = kWindow / 2; step >= 1; step /= 2) {
                     if (bounds[j + step] <= searched) j += step;
                 }
-                if (kRowVectors) {
+                if (kRowVectors && !Cfg::kIds) {
                     if (row >= rLo && row < rHi) {
                         const u64 length = bounds[j + 1] - bounds[j];
                         Pack<T, kVec> x;
@@ -643,7 +644,11 @@ __device__ __forceinline__ void broadcastSegments(const typename Cfg::T* values,
                         all = all && live[k];
                         if (live[k]) {
                             while (bounds[j + 1] <= row) ++j;
-                            x.v[k] = broadcastValue<Cfg>(values[(window + j) * kE + component], bounds[j + 1] - bounds[j]);
+                            if constexpr (Cfg::kIds) {
+                                x.v[k] = (T)(window + j);
+                            } else {
+                                x.v[k] = broadcastValue<Cfg>(values[(window + j) * kE + component], bounds[j + 1] - bounds[j]);
+                            }
                         }
                         if (++component == kE) {
                             component = 0;

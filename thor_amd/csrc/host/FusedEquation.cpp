@@ -22,7 +22,9 @@
 namespace ThorImplementation {
 
 struct PlannedGraph {
-    enum class Role : uint8_t { Inline, InputSource, Materialized, View };
+    // Gather: a SEGMENTED_BROADCAST that only fused kernels consume: they read the per-segment tensor through a
+    // row -> segment index instead of a materialised [rows, E] copy
+    enum class Role : uint8_t { Inline, InputSource, Materialized, View, Gather };
     PhysicalExpression expr;  // dtype-resolved, de-duplicated, reachable nodes only
     std::vector<NamedOutput> outputs;
     std::vector<Role> role;
@@ -180,8 +182,16 @@ void collectSources(const PlannedGraph& g, uint32_t root, std::vector<uint32_t>&
 }
 
 uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
-    while (g.role[node] == Role::View) node = g.expr.nodes[node].lhs;
+    // the tensor a source stands on: views and gathers lead to the tensor they read
+    while (g.role[node] == Role::View || g.role[node] == Role::Gather) node = g.expr.nodes[node].lhs;
     return node;
+}
+
+// Can the consumer read a per-segment value through the segment index?  Only work that ends up inside a flat fused kernel.
+bool consumesGather(const ExprNode& consumer) {
+    if (consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT || consumer.op == ExprOp::WHERE || consumer.op == ExprOp::CAST) return true;
+    if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX) return false;
+    return Expression::isBinaryOp(consumer.op) || Expression::isUnaryOp(consumer.op);
 }
 
 std::vector<uint64_t> broadcastDims(const std::vector<uint64_t>& a, const std::vector<uint64_t>& b) {
@@ -439,6 +449,22 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
         }
         for (const NamedOutput& o : graph->outputs) ensureTensor(o.node_idx);
 
+        if (stageFusionEnabled()) {
+            std::vector<char> named(count, 0), fusable(count, 1), used(count, 0);
+            for (const NamedOutput& o : graph->outputs) named[o.node_idx] = 1;
+            for (uint32_t i = 0; i < count; ++i) {
+                const ExprNode& n = graph->expr.nodes[i];
+                for (uint32_t c : {n.lhs, n.rhs, n.aux}) {
+                    if (c == UINT32_MAX || graph->expr.nodes[c].op != ExprOp::SEGMENTED_BROADCAST) continue;
+                    used[c] = 1;
+                    if (!consumesGather(n) || (n.op == ExprOp::RAGGED_VALUEWISE_EXTENT && n.rhs == c)) fusable[c] = 0;
+                }
+            }
+            for (uint32_t i = 0; i < count; ++i) {
+                if (graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST && used[i] && fusable[i] && !named[i]) graph->role[i] = Role::Gather;
+            }
+        }
+
         // dependency levels: a materialised value runs after every materialised value it reads
         for (uint32_t i = 0; i < count; ++i) {
             if (graph->role[i] != Role::Materialized) continue;
@@ -579,6 +605,8 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     };
 
     std::vector<char> done(expr.nodes.size(), 0);
+    std::map<std::pair<uint32_t, uint64_t>, std::pair<Tensor, uint32_t>> segmentIds;  // (offsets node, row capacity) -> index tensor, its stage
+    std::unordered_map<uint32_t, uint32_t> materialisedGather;                        // gather node -> the stage that wrote its rows
     const bool stageFusion = stageFusionEnabled() && !fusedKernelsOnly;
     std::vector<uint8_t> roles(graph->role.size());
     for (size_t i = 0; i < roles.size(); ++i) roles[i] = static_cast<uint8_t>(graph->role[i]);
@@ -713,8 +741,71 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             std::sort(scalarSlots.begin(), scalarSlots.end());
             scalarSlots.erase(std::unique(scalarSlots.begin(), scalarSlots.end()), scalarSlots.end());
 
-            std::vector<Tensor> inputTensors;
+            // Per-segment values reach a flat kernel through the row -> segment index; a kernel that broadcasts other operands
+            // gets them as a materialised [rows, E] tensor instead.
+            auto stripOnes = [](const std::vector<uint64_t>& d) {
+                std::vector<uint64_t> out;
+                for (uint64_t v : d)
+                    if (v != 1) out.push_back(v);
+                return out;
+            };
+            bool flatGroup = true;
             for (uint32_t s : sources) {
+                if (graph->role[s] == Role::Gather) continue;
+                flatGroup = flatGroup && tensorOf[s].isInitialized() && tensorOf[s].isDenseContiguous() && stripOnes(orScalarShape(dims[s])) == stripOnes(shape);
+            }
+            std::vector<uint32_t> extraDependencies;
+            std::vector<Tensor> inputTensors, gatherTensors;
+            for (uint32_t s : sources) {
+                if (graph->role[s] == Role::Gather && !tensorOf[s].isInitialized()) {
+                    const ExprNode& g = expr.nodes[s];
+                    const Tensor& perSegment = tensorOf[g.lhs];
+                    const Tensor& offsets = tensorOf[g.rhs];
+                    if (!perSegment.isInitialized() || !offsets.isInitialized()) throw std::logic_error("Gathered per-segment values have not been produced yet.");
+                    if (flatGroup && perSegment.isDenseContiguous() && offsets.isDenseContiguous()) {
+                        const uint64_t capacity = g.ragged_runtime_max_active_values;
+                        auto key = std::make_pair(g.rhs, capacity);
+                        auto found = segmentIds.find(key);
+                        if (found == segmentIds.end()) {
+                            Tensor ids(gpuPlacement, TensorDescriptor(DataType::UINT32, {capacity}));
+                            StampedExecutionStage stage;
+                            stage.kind = StampedExecutionStage::Kind::SegmentedBroadcast;
+                            stage.gpu_num = device_num;
+                            stage.segmented_broadcast = stampSegmentIds(offsets, ids, stream);
+                            found = segmentIds.emplace(key, std::make_pair(ids, static_cast<uint32_t>(stages.size()))).first;
+                            stages.push_back(std::move(stage));
+                        }
+                        GatherOperand gather;
+                        gather.node = s;
+                        gather.storageDType = perSegment.getDataType();
+                        gather.elementsPerValue = g.ragged_runtime_elements_per_value;
+                        gather.segments = g.ragged_runtime_batch_size;
+                        gather.normalize = g.segmented_broadcast_normalize_by_length;
+                        gather.offsetsAre64 = offsets.getDataType() == DataType::UINT64;
+                        gather.alignmentBytes = pointerAlignment(perSegment.getMemPtr());
+                        if (perSegment.getTotalNumElements() != gather.segments * gather.elementsPerValue ||
+                            offsets.getTotalNumElements() != gather.segments + 1) {
+                            throw std::runtime_error("Segmented broadcast operands do not have the shapes [B, E] and [B + 1] of their ragged descriptor.");
+                        }
+                        request.gathers.push_back(gather);
+                        gatherTensors.push_back(perSegment);
+                        gatherTensors.push_back(found->second.first);
+                        if (gather.normalize) gatherTensors.push_back(offsets);
+                        extraDependencies.push_back(found->second.second);
+                        continue;
+                    }
+                    // not a flat kernel: materialise the broadcast once and read it like any other tensor
+                    Tensor rows(gpuPlacement, TensorDescriptor(g.output_dtype.value(), orScalarShape(dims[s])));
+                    StampedExecutionStage stage;
+                    stage.kind = StampedExecutionStage::Kind::SegmentedBroadcast;
+                    stage.gpu_num = device_num;
+                    stage.dependency_stage_indices = dependenciesOf({g.lhs, g.rhs});
+                    stage.segmented_broadcast = stampSegmentedBroadcast(perSegment, offsets, rows, g.segmented_broadcast_normalize_by_length, stream);
+                    tensorOf[s] = rows;
+                    materialisedGather[s] = static_cast<uint32_t>(stages.size());
+                    stages.push_back(std::move(stage));
+                }
+                if (materialisedGather.count(s)) extraDependencies.push_back(materialisedGather.at(s));
                 const Tensor& t = tensorOf[s];
                 if (!t.isInitialized()) throw std::logic_error("Fused stage reads a value that has not been produced yet.");
                 KernelOperand operand;
@@ -742,7 +833,8 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             const EmittedKernel emitted = emitFusedKernel(request);
             std::shared_ptr<CompiledKernel> kernel = compileKernel(emitted.source, emitted.kernelName, device_num, emitted.fastContract);
 
-            if (extentOffsets.has_value()) inputTensors.push_back(extentOffsets.value());  // the pointer argument after the operands
+            inputTensors.insert(inputTensors.end(), gatherTensors.begin(), gatherTensors.end());  // pointer arguments after the operands
+            if (extentOffsets.has_value()) inputTensors.push_back(extentOffsets.value());
             std::vector<size_t> inputArgIndex(inputTensors.size()), outputArgIndex(outputTensors.size());
             std::iota(inputArgIndex.begin(), inputArgIndex.end(), 0);
             std::vector<StampedEquation::ScalarArgument> scalarArgs;
@@ -754,6 +846,10 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             stage.kind = StampedExecutionStage::Kind::FusedKernel;
             stage.gpu_num = device_num;
             stage.dependency_stage_indices = dependenciesOf(sources);
+            stage.dependency_stage_indices.insert(stage.dependency_stage_indices.end(), extraDependencies.begin(), extraDependencies.end());
+            std::sort(stage.dependency_stage_indices.begin(), stage.dependency_stage_indices.end());
+            stage.dependency_stage_indices.erase(std::unique(stage.dependency_stage_indices.begin(), stage.dependency_stage_indices.end()),
+                                                 stage.dependency_stage_indices.end());
             stage.kernel = std::make_shared<StampedEquation>(kernel, inputTensors, outputTensors, scalarArgs, inputArgIndex, outputArgIndex, next,
                                                              emitted.passNumel, emitted.numel, emitted.numelIs64, emitted.gridX, emitted.threads,
                                                              emitted.flopsPerElement * emitted.numel, emitted.description + " [" + kernel->kernelName + "]");

@@ -524,6 +524,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
     k.fastContract = true;
     BodyEmitter probe(expr);
     for (const KernelOperand& op : r.operands) probe.defineSource(op.node, DataType::FP32);
+    for (const GatherOperand& g : r.gathers) probe.defineSource(g.node, DataType::FP32);
     std::vector<uint32_t> roots;
     for (const KernelOutput& out : r.outputs) roots.push_back(out.node);
     for (uint32_t n : probe.collect(roots)) {
@@ -537,6 +538,11 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
     k.threads = static_cast<uint32_t>(threads);
     s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void fused_kernel(";
     for (size_t o = 0; o < r.operands.size(); ++o) s << "const " << deviceTypeName(r.operands[o].storageDType) << "* in" << o << ", ";
+    if (!r.gathers.empty() && !k.flat) throw std::runtime_error("Gathered per-segment operands need a kernel without broadcasting.");
+    for (size_t g = 0; g < r.gathers.size(); ++g) {
+        s << "const " << deviceTypeName(r.gathers[g].storageDType) << "* g" << g << ", const unsigned int* gid" << g << ", ";
+        if (r.gathers[g].normalize) s << "const " << (r.gathers[g].offsetsAre64 ? "unsigned long long" : "unsigned int") << "* goff" << g << ", ";
+    }
     if (r.extent.has_value()) {
         if (!k.flat) throw std::runtime_error("A ragged runtime extent needs operands of the output's own dense shape (no broadcasting).");
         s << "const " << (r.extent->offsetsAre64 ? "unsigned long long" : "unsigned int") << "* extentOffsets, ";
@@ -558,9 +564,30 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
 
     // body text for one element; `load(o)` and `store(o, value)` differ between the vector and the scalar form
     uint64_t flops = 0;
-    auto emitBody = [&](const std::string& indent, auto loadExpr, auto storeStmt) {
+    // the element a gathered operand contributes at flat index `index`: the storage word, and the segment it came from
+    auto gatherValue = [&](size_t g, const std::string& word, const std::string& segment) {
+        const GatherOperand& op = r.gathers[g];
+        std::string value = storageToValueExpr(word, op.storageDType);
+        if (op.normalize) {
+            // fp32 division by the segment's length, rounded once to the storage dtype (through fp16 for e5m2), as the
+            // materialised broadcast stores it
+            std::string quotient = "(" + castValueExpr(value, op.storageDType, DataType::FP32) + " / (float)(goff" + std::to_string(g) + "[" + segment +
+                                   " + 1] - goff" + std::to_string(g) + "[" + segment + "]))";
+            if (op.storageDType == DataType::FP8_E5M2) quotient = "thor::roundF16(" + quotient + ")";
+            value = storageToValueExpr(valueToStorageExpr(castValueExpr(quotient, DataType::FP32, op.storageDType), op.storageDType), op.storageDType);
+        }
+        return value;
+    };
+    auto emitBody = [&](const std::string& indent, auto loadExpr, auto storeStmt, auto gatherExpr) {
         std::string body;
         BodyEmitter emitter(expr);
+        for (size_t g = 0; g < r.gathers.size(); ++g) {
+            const GatherOperand& op = r.gathers[g];
+            const DataType valueDType = expr.nodes[op.node].output_dtype.value();
+            const std::string value = castValueExpr(gatherExpr(g, body, indent), op.storageDType, valueDType);
+            body += indent + "const " + valueCType(valueDType) + " t" + std::to_string(op.node) + " = " + value + ";\n";
+            emitter.defineSource(op.node, valueDType);
+        }
         for (size_t o = 0; o < r.operands.size(); ++o) {
             const KernelOperand& op = r.operands[o];
             const ExprNode& node = expr.nodes[op.node];
@@ -583,11 +610,43 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         return body;
     };
 
+    // segment of flat element `index` for gather g (clamped: rows outside every segment hold no defined index)
+    auto segmentOf = [&](size_t g, const std::string& index) {
+        const GatherOperand& op = r.gathers[g];
+        const std::string id = "gid" + std::to_string(g) + "[(unsigned long long)(" + index + ") / " + std::to_string(op.elementsPerValue) + "ull]";
+        return "((unsigned long long)(" + id + " < " + std::to_string(op.segments) + "u ? " + id + " : " + std::to_string(op.segments - 1) + "u))";
+    };
+    auto gatherPerElement = [&](const std::string& index) {
+        return [&, index](size_t g, std::string& body, const std::string& indent) {
+            const std::string seg = "gs" + std::to_string(g);
+            body += indent + "const unsigned long long " + seg + " = " + segmentOf(g, index) + ";\n";
+            const std::string word = "g" + std::to_string(g) + "[" + seg + " * " + std::to_string(r.gathers[g].elementsPerValue) + "ull + (unsigned long long)(" +
+                                     index + ") % " + std::to_string(r.gathers[g].elementsPerValue) + "ull]";
+            return gatherValue(g, word, seg);
+        };
+    };
+    auto noGather = [](size_t, std::string&, const std::string&) -> std::string { throw std::logic_error("gather in a broadcast kernel"); };
+
     if (k.flat) {
         s << "    const index_t base = ((index_t)blockIdx.x * " << threads << "u + threadIdx.x) * V;\n";
         s << "    if (base >= numel) return;\n";
         if (vec > 1) {
             s << "    if (base + V <= numel) {\n";
+            // a whole vector lies in one row when the row length is a multiple of the vector: one index read, one vector load
+            std::vector<char> hoisted(r.gathers.size(), 0);
+            for (size_t g = 0; g < r.gathers.size(); ++g) {
+                const GatherOperand& op = r.gathers[g];
+                hoisted[g] = op.elementsPerValue % vec == 0 && op.alignmentBytes % (static_cast<uint64_t>(vec) * dataTypeSizeInBytes(op.storageDType)) == 0;
+                if (!hoisted[g]) continue;
+                s << "        const unsigned long long gs" << g << " = " << segmentOf(g, "base") << ";\n";
+                s << "        thor::Pack<" << deviceTypeName(op.storageDType) << ", V> gp" << g << ";\n";
+                s << "        gp" << g << ".load(g" << g << " + gs" << g << " * " << op.elementsPerValue << "ull + (unsigned long long)base % " << op.elementsPerValue
+                  << "ull);\n";
+            }
+            auto gatherInVector = [&](size_t g, std::string& body, const std::string& indent) {
+                if (hoisted[g]) return gatherValue(g, "gp" + std::to_string(g) + ".v[k]", "gs" + std::to_string(g));
+                return gatherPerElement("base + k")(g, body, indent);
+            };
             for (size_t o = 0; o < r.operands.size(); ++o) {
                 s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n";
                 s << "        p" << o << ".loadStream(in" << o << " + base);\n";
@@ -596,7 +655,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
             s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
             s << emitBody(
                 "            ", [](size_t o) { return "p" + std::to_string(o) + ".v[k]"; },
-                [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; });
+                [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; }, gatherInVector);
             s << "        }\n";
             for (size_t o = 0; o < r.outputs.size(); ++o) s << "        q" << o << ".storeStream(out" << o << " + base);\n";
             s << "        return;\n    }\n";
@@ -605,7 +664,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         s << "    for (index_t e = base; e < end; ++e) {\n";
         s << emitBody(
             "        ", [](size_t o) { return "in" + std::to_string(o) + "[e]"; },
-            [](size_t o, const std::string& v) { return "out" + std::to_string(o) + "[e] = " + v + ";"; });
+            [](size_t o, const std::string& v) { return "out" + std::to_string(o) + "[e] = " + v + ";"; }, gatherPerElement("e"));
         s << "    }\n";
         const uint64_t lanes = (k.numel + vec - 1) / vec;
         k.gridX = static_cast<uint32_t>(std::max<uint64_t>((lanes + threads - 1) / threads, 1));
@@ -653,7 +712,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
                 const bool contiguous = layout.operandStride[o].back() == 1;
                 return (contiguous && vec > 1) ? "p" + std::to_string(o) + ".v[k]" : "b" + std::to_string(o);
             },
-            [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; });
+            [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; }, noGather);
         s << "    }\n";
         for (size_t o = 0; o < r.outputs.size(); ++o) s << "    q" << o << ".storeStream(out" << o << " + outOff);\n";
         k.gridX = static_cast<uint32_t>(std::max<uint64_t>((lanes + threads - 1) / threads, 1));

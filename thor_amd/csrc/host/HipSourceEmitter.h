@@ -43,9 +43,23 @@ struct RaggedExtent {
     bool offsetsAre64 = false;
 };
 
+// A per-segment tensor [B, E] read through a row -> segment index: element e of the output takes values[ids[e / E] * E + e % E]
+// (the value a SEGMENTED_BROADCAST node would have materialised), divided by the segment's length when `normalize` is set.
+// Kernel arguments: `const T* g<i>, const unsigned int* gid<i>` and, when normalised, `const OffsetT* goff<i>`.
+struct GatherOperand {
+    uint32_t node = UINT32_MAX;  // the SEGMENTED_BROADCAST node this stands for
+    DataType storageDType = DataType::FP32;
+    uint64_t elementsPerValue = 1;
+    uint64_t segments = 1;
+    bool normalize = false;
+    bool offsetsAre64 = false;
+    uint64_t alignmentBytes = 256;
+};
+
 struct FusedKernelRequest {
     const PhysicalExpression* expr = nullptr;
     std::vector<KernelOperand> operands;   // kernel arguments, in order
+    std::vector<GatherOperand> gathers;    // then the gathered per-segment tensors (flat kernels only)
     std::optional<RaggedExtent> extent;    // then the offsets pointer of the runtime extent, when there is one
     std::vector<uint32_t> scalarSlots;     // runtime scalar input slots passed by value (float), after the operands
     std::vector<KernelOutput> outputs;     // then the outputs

@@ -31,8 +31,31 @@ const char* rawWordName(uint32_t bytes) { return bytes == 1 ? "thor::u8" : bytes
 
 }  // namespace
 
+namespace {
+std::shared_ptr<StampedSegmentedBroadcast> stampImpl(const Tensor& per_segment_values, const Tensor& segment_offsets, const Tensor& output,
+                                                     bool normalize_by_segment_length, bool ids, const Stream& stream);
+}
+
 std::shared_ptr<StampedSegmentedBroadcast> stampSegmentedBroadcast(const Tensor& per_segment_values, const Tensor& segment_offsets, const Tensor& output,
                                                                    bool normalize_by_segment_length, const Stream& stream) {
+    return stampImpl(per_segment_values, segment_offsets, output, normalize_by_segment_length, false, stream);
+}
+
+std::shared_ptr<StampedSegmentedBroadcast> stampSegmentIds(const Tensor& segment_offsets, const Tensor& ids, const Stream& stream) {
+    if (!ids.isInitialized() || ids.getDataType() != DataType::UINT32 || ids.getDimensions().size() != 1) {
+        throw std::runtime_error("Segment ids must be a UINT32 tensor of shape [rows].");
+    }
+    if (!segment_offsets.isInitialized() || segment_offsets.getDimensions().size() != 1 || segment_offsets.getDimensions()[0] < 2) {
+        throw std::runtime_error("Segment ids require offsets [B+1] with at least one segment.");
+    }
+    // the values operand is not read in this mode; a [B] view of the ids tensor's dtype stands in for the shape checks
+    Tensor standIn(ids.getPlacement(), TensorDescriptor(DataType::UINT32, {segment_offsets.getDimensions()[0] - 1}));
+    return stampImpl(standIn, segment_offsets, ids, false, true, stream);
+}
+
+namespace {
+std::shared_ptr<StampedSegmentedBroadcast> stampImpl(const Tensor& per_segment_values, const Tensor& segment_offsets, const Tensor& output,
+                                                     bool normalize_by_segment_length, bool ids, const Stream& stream) {
     if (!per_segment_values.isInitialized() || !segment_offsets.isInitialized() || !output.isInitialized()) {
         throw std::runtime_error("Segmented broadcast requires initialized tensors.");
     }
@@ -58,7 +81,7 @@ std::shared_ptr<StampedSegmentedBroadcast> stampSegmentedBroadcast(const Tensor&
     const DataType offsetType = segment_offsets.getDataType();
     if (offsetType != DataType::UINT32 && offsetType != DataType::UINT64) throw std::runtime_error("Segmented broadcast offsets must use UINT32 or UINT64.");
     const DataType dtype = per_segment_values.getDataType();
-    if (dtype != DataType::FP8_E4M3 && dtype != DataType::FP8_E5M2 && dtype != DataType::FP16 && dtype != DataType::BF16 && dtype != DataType::FP32) {
+    if (!ids && dtype != DataType::FP8_E4M3 && dtype != DataType::FP8_E5M2 && dtype != DataType::FP16 && dtype != DataType::BF16 && dtype != DataType::FP32) {
         throw std::runtime_error("Segmented broadcast requires a floating-point expression dtype.");
     }
     // Trailing dimensions may be reshaped between the two tensors ([B, 4] against [N, 2, 2]); the elements per value are
@@ -88,16 +111,18 @@ std::shared_ptr<StampedSegmentedBroadcast> stampSegmentedBroadcast(const Tensor&
       << "ull;\n    static constexpr thor::u64 kSegments = " << segments << "ull;\n    static constexpr thor::u64 kChunkRows = " << chunkRows
       << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = 256;\n    static constexpr int kWindow = " << window
       << ";\n    static constexpr bool kNormalize = " << (normalize_by_segment_length ? "true" : "false")
-      << ";\n    static constexpr bool kViaHalf = " << (dtype == DataType::FP8_E5M2 ? "true" : "false") << ";\n};\n}  // namespace gen\n";
+      << ";\n    static constexpr bool kViaHalf = " << (dtype == DataType::FP8_E5M2 ? "true" : "false") << ";\n    static constexpr bool kIds = "
+      << (ids ? "true" : "false") << ";\n};\n}  // namespace gen\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_segmented_broadcast(const gen::Cfg::T* values, const void* offsets, gen::Cfg::T* out) "
          "{\n    thor::broadcastSegments<gen::Cfg>(values, static_cast<const gen::Cfg::OffsetT*>(offsets), out);\n}\n";
     const std::shared_ptr<CompiledKernel> kernel = compileKernel(s.str(), "thor_segmented_broadcast", stream.getGpuNum(), /*fastContract=*/false);
 
     std::ostringstream variant;
-    variant << "segmented_broadcast(chunk_rows=" << chunkRows << ",window=" << window << ",vec=" << vec << ",grid=" << chunks << ") [" << kernel->kernelName
+    variant << (ids ? "segment_ids(chunk_rows=" : "segmented_broadcast(chunk_rows=") << chunkRows << ",window=" << window << ",vec=" << vec << ",grid=" << chunks << ") [" << kernel->kernelName
             << "]";
     return std::make_shared<StampedSegmentedBroadcast>(kernel, per_segment_values, segment_offsets, output, static_cast<uint32_t>(chunks), variant.str());
 }
+}  // namespace
 
 void StampedSegmentedBroadcast::runOn(Stream& stream) const {
     if (!stream.isInitialized() || stream.getGpuNum() != static_cast<int>(output.getPlacement().getDeviceNum())) {
