@@ -95,10 +95,12 @@ class StampedArgMinMax {
 // writing same-shaped elementwise results of those sources in the same pass.
 class StampedFusedReduction {
    public:
+    // `segmentOffsets`: the reduction runs per segment of a ragged batch; the kernels read this offsets tensor at every run.
     StampedFusedReduction(ReductionLaunchPlan plan, std::vector<Tensor> inputs, std::vector<std::string> scalarNames, std::vector<Tensor> outputs,
-                          std::vector<Tensor> elementwiseOutputs, std::optional<Tensor> workspace, uint64_t flops)
+                          std::vector<Tensor> elementwiseOutputs, std::optional<Tensor> workspace, uint64_t flops,
+                          std::optional<Tensor> segmentOffsets = std::nullopt)
         : plan(std::move(plan)), inputs(std::move(inputs)), scalarNames(std::move(scalarNames)), outputs(std::move(outputs)),
-          elementwiseOutputs(std::move(elementwiseOutputs)), workspace(std::move(workspace)), flops(flops) {}
+          elementwiseOutputs(std::move(elementwiseOutputs)), workspace(std::move(workspace)), flops(flops), segmentOffsets(std::move(segmentOffsets)) {}
     void runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const;
     const std::vector<Tensor>& getOutputTensors() const { return outputs; }
     const std::vector<std::string>& runtimeScalarNames() const { return scalarNames; }
@@ -114,6 +116,7 @@ class StampedFusedReduction {
     std::vector<Tensor> elementwiseOutputs;  // tensors of the input's shape written by the same pass
     std::optional<Tensor> workspace;
     uint64_t flops;
+    std::optional<Tensor> segmentOffsets;
 };
 
 // Per-segment reduction over a ragged batch; the offsets are read on the device each time the stage runs.

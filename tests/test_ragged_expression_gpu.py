@@ -166,3 +166,82 @@ def test_dtype_and_shape_rules(stream):
         v.with_ragged_runtime_extent(o + 1.0, 2, 6, 2)
     with pytest.raises(RuntimeError, match="batch size \\+ 1"):
         ex.compile(ex.outputs({"s": v.segment_sum(o, 5, 6, 2)}), device_num=0).stamp({"v": x, "o": offsets}, stream)
+
+
+def staged(run_it):
+    """The same expression with stage fusion off: one stage per segmented reduction, broadcast and elementwise group."""
+    import os
+    os.environ["THOR_DISABLE_STAGE_FUSION"] = "1"
+    try:
+        return run_it()
+    finally:
+        os.environ.pop("THOR_DISABLE_STAGE_FUSION", None)
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16], ids=lambda d: d.name)
+def test_fused_and_staged_softmax_plans_agree(stream, dtype):
+    """Fused: the exponentials are never stored (the sum's kernel evaluates them with the per-segment maximum read once per
+    segment; the last kernel recomputes them), per-segment values are read through the row -> segment index."""
+    rng = np.random.default_rng(11)
+    capacity, trailing, segments = 6000, (16,), 200
+    offsets = np.concatenate([[0], np.sort(rng.integers(0, 5000, segments - 1)), [5000]]).astype(np.uint32)
+    x = to_storage(rng.standard_normal((capacity,) + trailing).astype(np.float32) * 2, dtype)
+    r = Ragged("x", segments, capacity, trailing)
+    inputs = {"x.values": copy_numpy_to_gpu(x, stream, dtype), "x.offsets": copy_numpy_to_gpu(offsets, stream, DataType.uint32)}
+
+    def both():
+        out = {}
+        for name, e in (("softmax", r.softmax()), ("log_softmax", r.softmax(True))):
+            filler = copy_numpy_to_gpu(to_storage(np.zeros((capacity,) + trailing, np.float32), dtype), stream, dtype)
+            plan, _ = run(ex.outputs({"y": e}), inputs, stream, {"y": filler})
+            out[name] = (plan.stage_kind_names(), from_storage(copy_gpu_to_numpy(plan.output("y"), stream), dtype))
+        return out
+
+    fused, reference = both(), staged(both)
+    assert fused["softmax"][0] == ["SegmentedReduction", "FusedReduction", "SegmentedBroadcast", "FusedKernel"]
+    assert reference["softmax"][0] == ["SegmentedReduction", "SegmentedBroadcast", "FusedKernel", "SegmentedReduction", "SegmentedBroadcast", "FusedKernel"]
+    tolerance = 1e-6 if dtype == DataType.fp32 else 2e-3
+    for name in ("softmax", "log_softmax"):
+        np.testing.assert_allclose(fused[name][1], reference[name][1], rtol=0, atol=tolerance, err_msg=name)
+
+
+def test_kernels_that_broadcast_other_operands_take_materialised_rows(stream):
+    """A per-channel bias makes the elementwise kernel a broadcasting one: the per-segment values reach it as a stored
+    [rows, E] tensor; the segmented reduction then squares the stored rows in registers."""
+    rng = np.random.default_rng(5)
+    capacity, e_per, segments = 700, 12, 9
+    offsets = np.array([0, 50, 50, 120, 300, 301, 420, 600, 650, 700], np.uint32)
+    x = rng.standard_normal((capacity, e_per)).astype(np.float32)
+    bias = rng.standard_normal((1, e_per)).astype(np.float32)
+    r = Ragged("x", segments, capacity, (e_per,))
+    b = ex.input("bias")
+    inputs = {"x.values": copy_numpy_to_gpu(x, stream, DataType.fp32), "x.offsets": copy_numpy_to_gpu(offsets, stream, DataType.uint32),
+              "bias": copy_numpy_to_gpu(bias, stream, DataType.fp32)}
+    centred = r.values - r.spread(r.reduce(r.values, "mean")) + b
+    outputs = ex.outputs({"rows": centred, "energy": r.reduce(centred * centred, "sum")})
+    plan, _ = run(outputs, inputs, stream)
+    means = np.stack([x[lo:hi].mean(axis=0) if hi > lo else np.zeros(e_per) for lo, hi in zip(offsets[:-1], offsets[1:])])
+    want_rows = x - np.repeat(means, np.diff(offsets), axis=0) + bias
+    np.testing.assert_allclose(copy_gpu_to_numpy(plan.output("rows"), stream), want_rows, rtol=1e-5, atol=1e-5)
+    want_energy = np.stack([(want_rows[lo:hi] ** 2).sum(axis=0) for lo, hi in zip(offsets[:-1], offsets[1:])])
+    np.testing.assert_allclose(copy_gpu_to_numpy(plan.output("energy"), stream), want_energy, rtol=1e-4, atol=1e-4)
+    assert plan.stage_kind_names() == ["SegmentedReduction", "SegmentedBroadcast", "FusedKernel", "FusedReduction"]
+
+
+def test_segmented_reduction_of_an_expression_with_scalars_and_means(stream):
+    """sum((x - mean)^2 * w) per segment with a runtime scalar: one kernel over x after the mean, nothing stored in between."""
+    rng = np.random.default_rng(8)
+    capacity, segments = 50000, 300
+    offsets = np.concatenate([[0], np.sort(rng.integers(0, capacity, segments - 1)), [capacity]]).astype(np.uint64)
+    x = rng.standard_normal((capacity, 4)).astype(np.float32)
+    r = Ragged("x", segments, capacity, (4,))
+    w = ex.runtime_scalar("w")
+    deviation = r.values - r.spread(r.reduce(r.values, "mean"))
+    outputs = ex.outputs({"scatter": r.reduce(deviation * deviation * w, "sum")})
+    eq = ex.compile(outputs, device_num=0)
+    plan = eq.stamp({"x.values": copy_numpy_to_gpu(x, stream, DataType.fp32), "x.offsets": copy_numpy_to_gpu(offsets, stream, DataType.uint64)}, stream)
+    assert plan.stage_kind_names() == ["SegmentedReduction", "FusedReduction"]
+    plan.run({"w": 0.5})
+    want = np.stack([((x[lo:hi] - x[lo:hi].mean(axis=0)) ** 2).sum(axis=0) * 0.5 if hi > lo else np.zeros(4)
+                     for lo, hi in zip(offsets[:-1].astype(int), offsets[1:].astype(int))])
+    np.testing.assert_allclose(copy_gpu_to_numpy(plan.output("scatter"), stream), want, rtol=2e-5, atol=1e-5)

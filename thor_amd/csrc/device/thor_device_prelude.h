@@ -88,6 +88,16 @@ __device__ __forceinline__ float toFloat(i64 v) { return (float)v; }
 
 // fp16 values are held in native _Float16 registers inside fused kernels
 __device__ __forceinline__ _Float16 asHalf(f16 h) { return __builtin_bit_cast(_Float16, h.bits); }
+// fp32 -> fp16 value (round to nearest even, the hardware conversion), spelled as the instruction itself.  A plain
+// `(_Float16)x` lets the vectoriser pair two conversions that feed packed fp16 arithmetic into a <2 x float> truncation,
+// which this compiler cannot select once packed fp32 operations are switched off (it aborts: "Cannot select: v2f32 =
+// bitcast", seen for x - ln(y) over fp16 vectors); the instruction keeps each conversion scalar and leaves the packed
+// fp16 arithmetic around it alone.
+__device__ __forceinline__ _Float16 halfFromFloat(float x) {
+    _Float16 h;
+    asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(x));
+    return h;
+}
 __device__ __forceinline__ f16 fromHalf(_Float16 h) {
     f16 r;
     r.bits = __builtin_bit_cast(u16, h);

@@ -454,10 +454,12 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
         const u64 pEnd = last < cEnd ? last : cEnd;
 
         Acc acc[Cfg::kVec];
-        typename Cfg::Kept kept;
-        Cfg::loadKept(src, pieceLive ? segment : 0, kept);
+        typename Cfg::Kept kept[Cfg::kVec];  // per-output operands: one element per (segment, trailing element)
 #pragma unroll
-        for (int k = 0; k < Cfg::kVec; ++k) acc[k].reset();
+        for (int k = 0; k < Cfg::kVec; ++k) {
+            Cfg::loadKept(src, (pieceLive ? segment : 0) * Cfg::kD + columnOffset + k, kept[k]);
+            acc[k].reset();
+        }
         for (u64 r0 = pBegin + rowLane; r0 < pEnd; r0 += rowLanes * kBatch) {
             typename Cfg::Loaded x[kBatch];
             if (r0 + (u64)(kBatch - 1) * rowLanes < pEnd) {
@@ -467,7 +469,7 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
                 for (int u = 0; u < kBatch; ++u) {
                     const u64 base = (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset;
 #pragma unroll
-                    for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept, k, (IndexT)(base + k));
+                    for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, (IndexT)(base + k));
                 }
             } else {
                 bool live[kBatch];
@@ -482,7 +484,7 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
                     if (live[u]) {
                         const u64 base = (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset;
 #pragma unroll
-                        for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept, k, (IndexT)(base + k));
+                        for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, (IndexT)(base + k));
                     }
                 }
             }

@@ -463,6 +463,47 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             for (uint32_t i = 0; i < count; ++i) {
                 if (graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST && used[i] && fusable[i] && !named[i]) graph->role[i] = Role::Gather;
             }
+            // An elementwise value that only segmented reductions over one partition need as a tensor is never stored: the
+            // reduction evaluates it in registers (per-segment values of the same partition are read once per segment), and
+            // elementwise consumers recompute it.
+            for (uint32_t r = 0; r < count; ++r) {
+                const ExprNode& reduce = graph->expr.nodes[r];
+                if (!isSegmentedReduceOp(reduce.op)) continue;
+                const uint32_t m = reduce.lhs;
+                const ExprNode& operand = graph->expr.nodes[m];
+                const bool elementwise = Expression::isBinaryOp(operand.op) || operand.op == ExprOp::WHERE || operand.op == ExprOp::CAST ||
+                                         (Expression::isUnaryOp(operand.op) && !isReductionOp(operand.op) && !isShapeOnly(operand.op) && operand.op != ExprOp::SOFTMAX);
+                if (graph->role[m] != Role::Materialized || named[m] || !elementwise) continue;
+                bool ok = true;
+                for (uint32_t j = 0; j < count && ok; ++j) {
+                    const ExprNode& consumer = graph->expr.nodes[j];
+                    if (consumer.lhs != m && consumer.rhs != m && consumer.aux != m) continue;
+                    if (isSegmentedReduceOp(consumer.op)) {
+                        ok = consumer.lhs == m && consumer.rhs == reduce.rhs;
+                    } else {
+                        ok = consumesGather(consumer) && !(consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT && consumer.rhs == m);
+                    }
+                }
+                // everything below m, down to tensors: elementwise work and broadcasts over the same partition
+                std::vector<uint32_t> stack{m};
+                std::vector<char> seen(count, 0);
+                while (ok && !stack.empty()) {
+                    const uint32_t v = stack.back();
+                    stack.pop_back();
+                    if (seen[v]) continue;
+                    seen[v] = 1;
+                    const ExprNode& node = graph->expr.nodes[v];
+                    if (node.op == ExprOp::SEGMENTED_BROADCAST) {
+                        ok = graph->role[v] != Role::Gather || (node.rhs == reduce.rhs && !node.segmented_broadcast_normalize_by_length);
+                        continue;
+                    }
+                    if (v != m && graph->role[v] != Role::Inline) continue;
+                    if (node.op == ExprOp::FILL || node.op == ExprOp::RAGGED_VALUEWISE_EXTENT) ok = false;
+                    for (uint32_t c : {node.lhs, node.rhs, node.aux})
+                        if (c != UINT32_MAX) stack.push_back(c);
+                }
+                if (ok) graph->role[m] = Role::Inline;
+            }
         }
 
         // dependency levels: a materialised value runs after every materialised value it reads
@@ -472,7 +513,12 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             if (isReductionOp(graph->expr.nodes[i].op)) {
                 sources.push_back(graph->expr.nodes[i].lhs);
             } else if (isSegmentedReduceOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST) {
-                sources.push_back(graph->expr.nodes[i].lhs);
+                const uint32_t operand = graph->expr.nodes[i].lhs;
+                if (graph->role[operand] == Role::Inline) {
+                    collectSources(*graph, operand, sources, scalars);  // evaluated inside the reduction
+                } else {
+                    sources.push_back(operand);
+                }
                 sources.push_back(graph->expr.nodes[i].rhs);
             } else {
                 collectSources(*graph, i, sources, scalars);
@@ -618,6 +664,282 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
         resolveViewsUpTo();
     }
 
+    // One fused elementwise kernel for values of one shape (and one ragged extent): gathers its sources, emits and compiles the
+    // kernel, allocates the outputs and appends the stage.
+    auto emitFusedGroup = [&](const std::vector<uint32_t>& nodes) {
+        FusedKernelRequest request;
+        request.expr = &expr;
+        const std::vector<uint64_t> shape = orScalarShape(dims[nodes.front()]);
+        request.outputDims = shape;
+        std::optional<Tensor> extentOffsets;
+        if (expr.nodes[nodes.front()].op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
+            const ExprNode& marker = expr.nodes[nodes.front()];
+            extentOffsets = tensorOf[marker.rhs];
+            if (!extentOffsets->isInitialized() || !extentOffsets->isDenseContiguous() ||
+                extentOffsets->getTotalNumElements() != marker.ragged_runtime_batch_size + 1) {
+                throw std::runtime_error("Ragged runtime extent offsets must be a dense tensor with batch size + 1 entries.");
+            }
+            uint64_t elements = 1;
+            for (uint64_t d : shape) elements *= d;
+            if (elements != marker.ragged_runtime_max_active_values * marker.ragged_runtime_elements_per_value) {
+                throw std::runtime_error("Ragged values do not have the shape [max active values, elements per value] their descriptor states.");
+            }
+            request.extent = RaggedExtent{marker.ragged_runtime_batch_size, marker.ragged_runtime_elements_per_value,
+                                          extentOffsets->getDataType() == DataType::UINT64};
+        }
+        std::vector<uint32_t> sources, scalarSlots;
+        for (uint32_t node : nodes) {
+            std::vector<uint32_t> s, sc;
+            if (isTensorRole(graph->role[node]) && expr.nodes[node].op == ExprOp::INPUT) {
+                s.push_back(node);
+            } else {
+                collectSources(*graph, node, s, sc);
+            }
+            sources.insert(sources.end(), s.begin(), s.end());
+            scalarSlots.insert(scalarSlots.end(), sc.begin(), sc.end());
+        }
+        std::sort(sources.begin(), sources.end());
+        sources.erase(std::unique(sources.begin(), sources.end()), sources.end());
+        std::sort(scalarSlots.begin(), scalarSlots.end());
+        scalarSlots.erase(std::unique(scalarSlots.begin(), scalarSlots.end()), scalarSlots.end());
+
+        // Per-segment values reach a flat kernel through the row -> segment index; a kernel that broadcasts other operands
+        // gets them as a materialised [rows, E] tensor instead.
+        auto stripOnes = [](const std::vector<uint64_t>& d) {
+            std::vector<uint64_t> out;
+            for (uint64_t v : d)
+                if (v != 1) out.push_back(v);
+            return out;
+        };
+        bool flatGroup = true;
+        for (uint32_t s : sources) {
+            if (graph->role[s] == Role::Gather) continue;
+            flatGroup = flatGroup && tensorOf[s].isInitialized() && tensorOf[s].isDenseContiguous() && stripOnes(orScalarShape(dims[s])) == stripOnes(shape);
+        }
+        std::vector<uint32_t> extraDependencies;
+        std::vector<Tensor> inputTensors, gatherTensors;
+        for (uint32_t s : sources) {
+            if (graph->role[s] == Role::Gather && !tensorOf[s].isInitialized()) {
+                const ExprNode& g = expr.nodes[s];
+                const Tensor& perSegment = tensorOf[g.lhs];
+                const Tensor& offsets = tensorOf[g.rhs];
+                if (!perSegment.isInitialized() || !offsets.isInitialized()) throw std::logic_error("Gathered per-segment values have not been produced yet.");
+                if (flatGroup && perSegment.isDenseContiguous() && offsets.isDenseContiguous()) {
+                    const uint64_t capacity = g.ragged_runtime_max_active_values;
+                    auto key = std::make_pair(g.rhs, capacity);
+                    auto found = segmentIds.find(key);
+                    if (found == segmentIds.end()) {
+                        Tensor ids(gpuPlacement, TensorDescriptor(DataType::UINT32, {capacity}));
+                        StampedExecutionStage stage;
+                        stage.kind = StampedExecutionStage::Kind::SegmentedBroadcast;
+                        stage.gpu_num = device_num;
+                        stage.segmented_broadcast = stampSegmentIds(offsets, ids, stream);
+                        found = segmentIds.emplace(key, std::make_pair(ids, static_cast<uint32_t>(stages.size()))).first;
+                        stages.push_back(std::move(stage));
+                    }
+                    GatherOperand gather;
+                    gather.node = s;
+                    gather.storageDType = perSegment.getDataType();
+                    gather.elementsPerValue = g.ragged_runtime_elements_per_value;
+                    gather.segments = g.ragged_runtime_batch_size;
+                    gather.normalize = g.segmented_broadcast_normalize_by_length;
+                    gather.offsetsAre64 = offsets.getDataType() == DataType::UINT64;
+                    gather.alignmentBytes = pointerAlignment(perSegment.getMemPtr());
+                    if (perSegment.getTotalNumElements() != gather.segments * gather.elementsPerValue ||
+                        offsets.getTotalNumElements() != gather.segments + 1) {
+                        throw std::runtime_error("Segmented broadcast operands do not have the shapes [B, E] and [B + 1] of their ragged descriptor.");
+                    }
+                    request.gathers.push_back(gather);
+                    gatherTensors.push_back(perSegment);
+                    gatherTensors.push_back(found->second.first);
+                    if (gather.normalize) gatherTensors.push_back(offsets);
+                    extraDependencies.push_back(found->second.second);
+                    continue;
+                }
+                // not a flat kernel: materialise the broadcast once and read it like any other tensor
+                Tensor rows(gpuPlacement, TensorDescriptor(g.output_dtype.value(), orScalarShape(dims[s])));
+                StampedExecutionStage stage;
+                stage.kind = StampedExecutionStage::Kind::SegmentedBroadcast;
+                stage.gpu_num = device_num;
+                stage.dependency_stage_indices = dependenciesOf({g.lhs, g.rhs});
+                stage.segmented_broadcast = stampSegmentedBroadcast(perSegment, offsets, rows, g.segmented_broadcast_normalize_by_length, stream);
+                tensorOf[s] = rows;
+                materialisedGather[s] = static_cast<uint32_t>(stages.size());
+                stages.push_back(std::move(stage));
+            }
+            if (materialisedGather.count(s)) extraDependencies.push_back(materialisedGather.at(s));
+            const Tensor& t = tensorOf[s];
+            if (!t.isInitialized()) throw std::logic_error("Fused stage reads a value that has not been produced yet.");
+            KernelOperand operand;
+            operand.node = s;
+            operand.storageDType = t.getDataType();
+            operand.dims = orScalarShape(dims[s]);
+            operand.strides = t.getStridesElements();
+            if (operand.strides.size() != operand.dims.size()) throw std::logic_error("Operand rank does not match its tensor.");
+            operand.alignmentBytes = pointerAlignment(t.getMemPtr());
+            request.operands.push_back(operand);
+            inputTensors.push_back(t);
+        }
+        request.scalarSlots = scalarSlots;
+        std::vector<Tensor> outputTensors;
+        for (uint32_t node : nodes) {
+            Tensor out = allocateFor(node);
+            KernelOutput ko;
+            ko.node = node;
+            ko.storageDType = out.getDataType();
+            ko.alignmentBytes = pointerAlignment(out.getMemPtr());
+            request.outputs.push_back(ko);
+            outputTensors.push_back(out);
+            tensorOf[node] = out;
+        }
+        const EmittedKernel emitted = emitFusedKernel(request);
+        std::shared_ptr<CompiledKernel> kernel = compileKernel(emitted.source, emitted.kernelName, device_num, emitted.fastContract);
+
+        inputTensors.insert(inputTensors.end(), gatherTensors.begin(), gatherTensors.end());  // pointer arguments after the operands
+        if (extentOffsets.has_value()) inputTensors.push_back(extentOffsets.value());
+        std::vector<size_t> inputArgIndex(inputTensors.size()), outputArgIndex(outputTensors.size());
+        std::iota(inputArgIndex.begin(), inputArgIndex.end(), 0);
+        std::vector<StampedEquation::ScalarArgument> scalarArgs;
+        size_t next = inputTensors.size();
+        for (uint32_t slot : scalarSlots) scalarArgs.push_back({root_inputs.at(slot).name, next++});
+        for (size_t o = 0; o < outputTensors.size(); ++o) outputArgIndex[o] = next++;
+
+        StampedExecutionStage stage;
+        stage.kind = StampedExecutionStage::Kind::FusedKernel;
+        stage.gpu_num = device_num;
+        stage.dependency_stage_indices = dependenciesOf(sources);
+        stage.dependency_stage_indices.insert(stage.dependency_stage_indices.end(), extraDependencies.begin(), extraDependencies.end());
+        std::sort(stage.dependency_stage_indices.begin(), stage.dependency_stage_indices.end());
+        stage.dependency_stage_indices.erase(std::unique(stage.dependency_stage_indices.begin(), stage.dependency_stage_indices.end()),
+                                             stage.dependency_stage_indices.end());
+        stage.kernel = std::make_shared<StampedEquation>(kernel, inputTensors, outputTensors, scalarArgs, inputArgIndex, outputArgIndex, next,
+                                                         emitted.passNumel, emitted.numel, emitted.numelIs64, emitted.gridX, emitted.threads,
+                                                         emitted.flopsPerElement * emitted.numel, emitted.description + " [" + kernel->kernelName + "]");
+        for (uint32_t node : nodes) {
+            stageOfNode[node] = static_cast<int>(stages.size());
+            done[node] = 1;
+        }
+        stages.push_back(std::move(stage));
+    };
+
+    // A segmented reduction whose operand is an elementwise expression: the reduction kernel evaluates the expression in
+    // registers.  Sources are tensors of the operand's shape, single elements, and per-segment tensors that the expression
+    // broadcasts over the same partition (read once per segment and trailing element).  False = cannot be done this way.
+    auto stampSegmentedReductionOfExpression = [&](uint32_t node) -> bool {
+        const ExprNode& n = expr.nodes[node];
+        const uint32_t operand = n.lhs;
+        const Tensor& offsets = tensorOf[n.rhs];
+        std::vector<uint32_t> sources, scalarSlots;
+        collectSources(*graph, operand, sources, scalarSlots);
+        const std::vector<uint64_t> valueShape = orScalarShape(dims[operand]);
+        if (valueShape.empty() || !offsets.isInitialized() || !offsets.isDenseContiguous()) return false;
+        uint64_t trailing = 1;
+        for (size_t a = 1; a < valueShape.size(); ++a) trailing *= valueShape[a];
+        const uint64_t rows = valueShape[0], segments = offsets.getTotalNumElements() - 1;
+        auto stripOnes = [](const std::vector<uint64_t>& d) {
+            std::vector<uint64_t> out;
+            for (uint64_t v : d)
+                if (v != 1) out.push_back(v);
+            return out;
+        };
+        using SourceKind = ReductionKernelRequest::Source::Kind;
+        ReductionKernelRequest request;
+        request.segmented = true;
+        request.segments = segments;
+        request.segmentedRows = rows;
+        request.trailing = trailing;
+        request.offsetsAre64 = offsets.getDataType() == DataType::UINT64;
+        request.deviceNum = device_num;
+        request.inputAlignmentBytes = 256;
+        request.geometry.path = CubReductionPath::OffsetSegmented;
+        request.geometry.rank = static_cast<uint32_t>(valueShape.size());
+        request.geometry.input_elements = rows * trailing;
+        request.geometry.output_elements = segments * trailing;
+        request.geometry.reduction_size = rows;
+        request.geometry.output_dimensions = orScalarShape(dims[node]);
+        request.geometry.squeezed_output_dimensions = request.geometry.output_dimensions;
+        request.scalarSlots = scalarSlots;
+
+        BodyEmitter body(expr);
+        std::string text;
+        for (uint32_t slot : scalarSlots) text += "        const float s" + std::to_string(slot) + " = s.s" + std::to_string(slot) + ";\n";
+        std::vector<Tensor> inputs;
+        bool anyVector = false;
+        for (uint32_t s : sources) {
+            Tensor t;
+            SourceKind kind;
+            if (graph->role[s] == Role::Gather && !tensorOf[s].isInitialized()) {
+                const ExprNode& g = expr.nodes[s];
+                t = tensorOf[g.lhs];
+                if (g.rhs != n.rhs || g.segmented_broadcast_normalize_by_length || !t.isInitialized() || !t.isDenseContiguous() ||
+                    t.getTotalNumElements() != segments * trailing) {
+                    return false;
+                }
+                kind = SourceKind::Kept;
+            } else {
+                t = tensorOf[s];
+                if (!t.isInitialized() || !t.isDenseContiguous()) return false;
+                if (stripOnes(orScalarShape(dims[s])) == stripOnes(valueShape)) {
+                    kind = SourceKind::Vector;
+                } else if (t.getTotalNumElements() == 1) {
+                    kind = SourceKind::Scalar;
+                } else {
+                    return false;
+                }
+            }
+            const size_t index = inputs.size();
+            ReductionKernelRequest::Source source;
+            source.storage = t.getDataType();
+            source.kind = kind;
+            request.sources.push_back(source);
+            if (kind == SourceKind::Vector) {
+                request.inputAlignmentBytes = std::min(request.inputAlignmentBytes, pointerAlignment(t.getMemPtr()));
+                anyVector = true;
+            }
+            inputs.push_back(t);
+            const DataType valueDType = expr.nodes[s].output_dtype.value();
+            const std::string raw = kind == SourceKind::Vector ? "l.p" + std::to_string(index) + ".v[k]" : "kk.z" + std::to_string(index);
+            text += "        const " + std::string(valueCType(valueDType)) + " t" + std::to_string(s) + " = " +
+                    castValueExpr(storageToValueExpr(raw, t.getDataType()), t.getDataType(), valueDType) + ";\n";
+            body.defineSource(s, valueDType);
+        }
+        if (!anyVector) return false;
+        uint64_t flopsPerElement = 1;
+        for (uint32_t v : body.collect({operand})) flopsPerElement += body.emit(text, v, "        ");
+        // the staged plan would have stored the operand in its output dtype: round there before accumulating in fp32
+        const DataType storedDType = expr.nodes[operand].output_dtype.value();
+        ReductionKernelRequest::Value value;
+        value.op = n.op == ExprOp::SEGMENTED_REDUCE_SUM   ? CubReductionOp::Sum
+                   : n.op == ExprOp::SEGMENTED_REDUCE_MIN ? CubReductionOp::Min
+                   : n.op == ExprOp::SEGMENTED_REDUCE_MAX ? CubReductionOp::Max
+                                                          : CubReductionOp::Mean;
+        value.outputDType = n.output_dtype.value();
+        value.expression = castValueExpr(body.ref(operand, storedDType), storedDType, DataType::FP32);
+        request.values.push_back(value);
+        request.prologue = text;
+        request.inputDType = inputs.front().getDataType();
+
+        ReductionLaunchPlan plan = buildReductionKernels(request);
+        std::optional<Tensor> workspace;
+        if (plan.workspaceBytes > 0) workspace = Tensor(gpuPlacement, TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
+        Tensor output = allocateFor(node);
+        std::vector<std::string> scalarNames;
+        for (uint32_t slot : scalarSlots) scalarNames.push_back(root_inputs.at(slot).name);
+        StampedExecutionStage stage;
+        stage.kind = StampedExecutionStage::Kind::FusedReduction;
+        stage.gpu_num = device_num;
+        sources.push_back(n.rhs);
+        stage.dependency_stage_indices = dependenciesOf(sources);
+        plan.variant = "fused_segmented_reduction(sources=" + std::to_string(inputs.size()) + ") " + plan.variant;
+        stage.fused_reduction = std::make_shared<StampedFusedReduction>(std::move(plan), inputs, scalarNames, std::vector<Tensor>{output}, std::vector<Tensor>{},
+                                                                        workspace, flopsPerElement * rows * trailing, offsets);
+        tensorOf[node] = output;
+        stageOfNode[node] = static_cast<int>(stages.size());
+        stages.push_back(std::move(stage));
+        done[node] = 1;
+        return true;
+    };
+
     for (uint32_t level = 0; level <= maxLevel; ++level) {
         if (stageFusion) {
             // Reductions over one shape and axes whose inputs exist by now (or are elementwise functions of such tensors
@@ -635,6 +957,10 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                     throw std::runtime_error(
                         "FusedEquation::run() only supports expressions that lower to fused kernels; this expression has a segmented stage. "
                         "Use stamp() and run the returned plan.");
+                }
+                if (isSegmentedReduceOp(n.op) && graph->role[n.lhs] == Role::Inline) {
+                    if (stampSegmentedReductionOfExpression(i)) continue;
+                    emitFusedGroup({n.lhs});  // operands the reduction cannot evaluate by itself: store the values first
                 }
                 const Tensor& values = tensorOf[n.lhs];
                 const Tensor& offsets = tensorOf[n.rhs];
@@ -704,161 +1030,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             done[i] = 1;
         }
 
-        for (auto& [groupKey, nodes] : fusedGroups) {
-            FusedKernelRequest request;
-            request.expr = &expr;
-            const std::vector<uint64_t> shape = orScalarShape(dims[nodes.front()]);
-            request.outputDims = shape;
-            std::optional<Tensor> extentOffsets;
-            if (expr.nodes[nodes.front()].op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
-                const ExprNode& marker = expr.nodes[nodes.front()];
-                extentOffsets = tensorOf[marker.rhs];
-                if (!extentOffsets->isInitialized() || !extentOffsets->isDenseContiguous() ||
-                    extentOffsets->getTotalNumElements() != marker.ragged_runtime_batch_size + 1) {
-                    throw std::runtime_error("Ragged runtime extent offsets must be a dense tensor with batch size + 1 entries.");
-                }
-                uint64_t elements = 1;
-                for (uint64_t d : shape) elements *= d;
-                if (elements != marker.ragged_runtime_max_active_values * marker.ragged_runtime_elements_per_value) {
-                    throw std::runtime_error("Ragged values do not have the shape [max active values, elements per value] their descriptor states.");
-                }
-                request.extent = RaggedExtent{marker.ragged_runtime_batch_size, marker.ragged_runtime_elements_per_value,
-                                              extentOffsets->getDataType() == DataType::UINT64};
-            }
-            std::vector<uint32_t> sources, scalarSlots;
-            for (uint32_t node : nodes) {
-                std::vector<uint32_t> s, sc;
-                if (isTensorRole(graph->role[node]) && expr.nodes[node].op == ExprOp::INPUT) {
-                    s.push_back(node);
-                } else {
-                    collectSources(*graph, node, s, sc);
-                }
-                sources.insert(sources.end(), s.begin(), s.end());
-                scalarSlots.insert(scalarSlots.end(), sc.begin(), sc.end());
-            }
-            std::sort(sources.begin(), sources.end());
-            sources.erase(std::unique(sources.begin(), sources.end()), sources.end());
-            std::sort(scalarSlots.begin(), scalarSlots.end());
-            scalarSlots.erase(std::unique(scalarSlots.begin(), scalarSlots.end()), scalarSlots.end());
-
-            // Per-segment values reach a flat kernel through the row -> segment index; a kernel that broadcasts other operands
-            // gets them as a materialised [rows, E] tensor instead.
-            auto stripOnes = [](const std::vector<uint64_t>& d) {
-                std::vector<uint64_t> out;
-                for (uint64_t v : d)
-                    if (v != 1) out.push_back(v);
-                return out;
-            };
-            bool flatGroup = true;
-            for (uint32_t s : sources) {
-                if (graph->role[s] == Role::Gather) continue;
-                flatGroup = flatGroup && tensorOf[s].isInitialized() && tensorOf[s].isDenseContiguous() && stripOnes(orScalarShape(dims[s])) == stripOnes(shape);
-            }
-            std::vector<uint32_t> extraDependencies;
-            std::vector<Tensor> inputTensors, gatherTensors;
-            for (uint32_t s : sources) {
-                if (graph->role[s] == Role::Gather && !tensorOf[s].isInitialized()) {
-                    const ExprNode& g = expr.nodes[s];
-                    const Tensor& perSegment = tensorOf[g.lhs];
-                    const Tensor& offsets = tensorOf[g.rhs];
-                    if (!perSegment.isInitialized() || !offsets.isInitialized()) throw std::logic_error("Gathered per-segment values have not been produced yet.");
-                    if (flatGroup && perSegment.isDenseContiguous() && offsets.isDenseContiguous()) {
-                        const uint64_t capacity = g.ragged_runtime_max_active_values;
-                        auto key = std::make_pair(g.rhs, capacity);
-                        auto found = segmentIds.find(key);
-                        if (found == segmentIds.end()) {
-                            Tensor ids(gpuPlacement, TensorDescriptor(DataType::UINT32, {capacity}));
-                            StampedExecutionStage stage;
-                            stage.kind = StampedExecutionStage::Kind::SegmentedBroadcast;
-                            stage.gpu_num = device_num;
-                            stage.segmented_broadcast = stampSegmentIds(offsets, ids, stream);
-                            found = segmentIds.emplace(key, std::make_pair(ids, static_cast<uint32_t>(stages.size()))).first;
-                            stages.push_back(std::move(stage));
-                        }
-                        GatherOperand gather;
-                        gather.node = s;
-                        gather.storageDType = perSegment.getDataType();
-                        gather.elementsPerValue = g.ragged_runtime_elements_per_value;
-                        gather.segments = g.ragged_runtime_batch_size;
-                        gather.normalize = g.segmented_broadcast_normalize_by_length;
-                        gather.offsetsAre64 = offsets.getDataType() == DataType::UINT64;
-                        gather.alignmentBytes = pointerAlignment(perSegment.getMemPtr());
-                        if (perSegment.getTotalNumElements() != gather.segments * gather.elementsPerValue ||
-                            offsets.getTotalNumElements() != gather.segments + 1) {
-                            throw std::runtime_error("Segmented broadcast operands do not have the shapes [B, E] and [B + 1] of their ragged descriptor.");
-                        }
-                        request.gathers.push_back(gather);
-                        gatherTensors.push_back(perSegment);
-                        gatherTensors.push_back(found->second.first);
-                        if (gather.normalize) gatherTensors.push_back(offsets);
-                        extraDependencies.push_back(found->second.second);
-                        continue;
-                    }
-                    // not a flat kernel: materialise the broadcast once and read it like any other tensor
-                    Tensor rows(gpuPlacement, TensorDescriptor(g.output_dtype.value(), orScalarShape(dims[s])));
-                    StampedExecutionStage stage;
-                    stage.kind = StampedExecutionStage::Kind::SegmentedBroadcast;
-                    stage.gpu_num = device_num;
-                    stage.dependency_stage_indices = dependenciesOf({g.lhs, g.rhs});
-                    stage.segmented_broadcast = stampSegmentedBroadcast(perSegment, offsets, rows, g.segmented_broadcast_normalize_by_length, stream);
-                    tensorOf[s] = rows;
-                    materialisedGather[s] = static_cast<uint32_t>(stages.size());
-                    stages.push_back(std::move(stage));
-                }
-                if (materialisedGather.count(s)) extraDependencies.push_back(materialisedGather.at(s));
-                const Tensor& t = tensorOf[s];
-                if (!t.isInitialized()) throw std::logic_error("Fused stage reads a value that has not been produced yet.");
-                KernelOperand operand;
-                operand.node = s;
-                operand.storageDType = t.getDataType();
-                operand.dims = orScalarShape(dims[s]);
-                operand.strides = t.getStridesElements();
-                if (operand.strides.size() != operand.dims.size()) throw std::logic_error("Operand rank does not match its tensor.");
-                operand.alignmentBytes = pointerAlignment(t.getMemPtr());
-                request.operands.push_back(operand);
-                inputTensors.push_back(t);
-            }
-            request.scalarSlots = scalarSlots;
-            std::vector<Tensor> outputTensors;
-            for (uint32_t node : nodes) {
-                Tensor out = allocateFor(node);
-                KernelOutput ko;
-                ko.node = node;
-                ko.storageDType = out.getDataType();
-                ko.alignmentBytes = pointerAlignment(out.getMemPtr());
-                request.outputs.push_back(ko);
-                outputTensors.push_back(out);
-                tensorOf[node] = out;
-            }
-            const EmittedKernel emitted = emitFusedKernel(request);
-            std::shared_ptr<CompiledKernel> kernel = compileKernel(emitted.source, emitted.kernelName, device_num, emitted.fastContract);
-
-            inputTensors.insert(inputTensors.end(), gatherTensors.begin(), gatherTensors.end());  // pointer arguments after the operands
-            if (extentOffsets.has_value()) inputTensors.push_back(extentOffsets.value());
-            std::vector<size_t> inputArgIndex(inputTensors.size()), outputArgIndex(outputTensors.size());
-            std::iota(inputArgIndex.begin(), inputArgIndex.end(), 0);
-            std::vector<StampedEquation::ScalarArgument> scalarArgs;
-            size_t next = inputTensors.size();
-            for (uint32_t slot : scalarSlots) scalarArgs.push_back({root_inputs.at(slot).name, next++});
-            for (size_t o = 0; o < outputTensors.size(); ++o) outputArgIndex[o] = next++;
-
-            StampedExecutionStage stage;
-            stage.kind = StampedExecutionStage::Kind::FusedKernel;
-            stage.gpu_num = device_num;
-            stage.dependency_stage_indices = dependenciesOf(sources);
-            stage.dependency_stage_indices.insert(stage.dependency_stage_indices.end(), extraDependencies.begin(), extraDependencies.end());
-            std::sort(stage.dependency_stage_indices.begin(), stage.dependency_stage_indices.end());
-            stage.dependency_stage_indices.erase(std::unique(stage.dependency_stage_indices.begin(), stage.dependency_stage_indices.end()),
-                                                 stage.dependency_stage_indices.end());
-            stage.kernel = std::make_shared<StampedEquation>(kernel, inputTensors, outputTensors, scalarArgs, inputArgIndex, outputArgIndex, next,
-                                                             emitted.passNumel, emitted.numel, emitted.numelIs64, emitted.gridX, emitted.threads,
-                                                             emitted.flopsPerElement * emitted.numel, emitted.description + " [" + kernel->kernelName + "]");
-            for (uint32_t node : nodes) {
-                stageOfNode[node] = static_cast<int>(stages.size());
-                done[node] = 1;
-            }
-            stages.push_back(std::move(stage));
-        }
+        for (auto& [groupKey, nodes] : fusedGroups) emitFusedGroup(nodes);
         resolveViewsUpTo();
     }
 

@@ -188,7 +188,7 @@ std::string castValueExpr(const std::string& x, DataType from, DataType to) {
     }
     switch (to) {
         case DataType::FP32: return asFloat;
-        case DataType::FP16: return "(_Float16)(" + asFloat + ")";
+        case DataType::FP16: return "thor::halfFromFloat(" + asFloat + ")";
         case DataType::BF16: return "thor::roundBf16(" + asFloat + ")";
         case DataType::FP8_E4M3: return "thor::roundE4m3(" + asFloat + ")";
         case DataType::FP8_E5M2: return "thor::roundE5m2(" + asFloat + ")";

@@ -134,7 +134,13 @@ void StampedFusedReduction::runOn(Stream& stream, const std::unordered_map<std::
     args.push_back(&indexOut);
     args.push_back(&partials);
     args.push_back(&scale);
+    const void* offsetPointer = segmentOffsets.has_value() ? segmentOffsets->getMemPtr() : nullptr;
+    if (segmentOffsets.has_value()) args.push_back(&offsetPointer);
     ScopedGpu scoped(stream.getGpuNum());
+    if (plan.prepareKernel) {
+        std::vector<void*> prepareArgs = {&partials, &offsetPointer};
+        plan.prepareKernel->launch(plan.prepareGridX, 1, 1, plan.prepareThreads, stream.getStream(), prepareArgs);
+    }
     plan.mainKernel->launch(plan.mainGridX, plan.mainGridY, 1, plan.mainThreads, stream.getStream(), args);
     if (plan.finishKernel) {
         const void* constPartials = partials;
@@ -142,6 +148,7 @@ void StampedFusedReduction::runOn(Stream& stream, const std::unordered_map<std::
         for (size_t i = 0; i < outputs.size(); ++i) finishArgs.push_back(&outputPointers[i]);
         finishArgs.push_back(&indexOut);
         finishArgs.push_back(&scale);
+        if (segmentOffsets.has_value()) finishArgs.push_back(&offsetPointer);
         plan.finishKernel->launch(plan.finishGridX, 1, 1, plan.finishThreads, stream.getStream(), finishArgs);
     }
 }
