@@ -1,0 +1,143 @@
+// Stamps a matrix of expressions without a GPU: this program defines the device C-ABI entry points for memory, streams,
+// modules and launches itself (the dynamic linker binds the library's calls to these definitions), so planning, source
+// generation and the run-time compilation for gfx950 run exactly as on a GPU box while nothing is launched.  What it
+// guards: every kernel variant the planner can emit for these expressions compiles.  A compiler failure inside the
+// in-process compiler aborts the process, so each case prints its name first.
+#include "thorhip.h"
+
+#include "Utilities/Expression/FusedEquation.h"
+#include "Utilities/Expression/RaggedExpression.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+extern "C" {
+int thorhip_device_count(int* count) { return *count = 1, 0; }
+int thorhip_set_device(int) { return 0; }
+int thorhip_get_device(int* device) { return *device = 0, 0; }
+int thorhip_device_get_info(int, thorhip_device_info* info) {
+    std::memset(info, 0, sizeof *info);
+    info->compute_units = 256;
+    info->wavefront_size = 64;
+    info->max_threads_per_block = 1024;
+    std::strcpy(info->arch_name, "gfx950");
+    return 0;
+}
+int thorhip_device_synchronize(void) { return 0; }
+int thorhip_malloc(void** ptr, size_t bytes) { return posix_memalign(ptr, 256, bytes ? bytes : 256) ? -1 : 0; }
+int thorhip_free(void* ptr) { return std::free(ptr), 0; }
+int thorhip_host_malloc(void** ptr, size_t bytes) { return posix_memalign(ptr, 256, bytes ? bytes : 256) ? -1 : 0; }
+int thorhip_host_free(void* ptr) { return std::free(ptr), 0; }
+int thorhip_memcpy_async(void* dst, const void* src, size_t bytes, int, void*) { return std::memcpy(dst, src, bytes), 0; }
+int thorhip_memset_async(void* dst, int value, size_t bytes, void*) { return std::memset(dst, value, bytes), 0; }
+int thorhip_mem_get_info(size_t* free_bytes, size_t* total_bytes) { return *free_bytes = *total_bytes = size_t(1) << 38, 0; }
+int thorhip_stream_create(void** stream) { return *stream = std::malloc(8), 0; }
+int thorhip_stream_destroy(void* stream) { return std::free(stream), 0; }
+int thorhip_stream_synchronize(void*) { return 0; }
+int thorhip_stream_wait_event(void*, void*) { return 0; }
+int thorhip_stream_enqueue_host_function(void*, thorhip_host_fn fn, void* user_data) { return fn(user_data), 0; }
+int thorhip_event_create(void** event, int) { return *event = std::malloc(8), 0; }
+int thorhip_event_destroy(void* event) { return std::free(event), 0; }
+int thorhip_event_record(void*, void*) { return 0; }
+int thorhip_event_synchronize(void*) { return 0; }
+int thorhip_event_elapsed_ms(float* ms, void*, void*) { return *ms = 0.0f, 0; }
+int thorhip_module_load(void** module, const void*, size_t) { return *module = std::malloc(8), 0; }
+int thorhip_module_unload(void* module) { return std::free(module), 0; }
+int thorhip_module_get_function(void** function, void* module, const char*) { return *function = module, 0; }
+int thorhip_function_get_attributes(void*, int* vgprs, int* lds, int* threads) {
+    if (vgprs) *vgprs = 0;
+    if (lds) *lds = 0;
+    if (threads) *threads = 1024;
+    return 0;
+}
+int thorhip_launch(void*, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, void*, void**) { return 0; }
+}
+
+using namespace ThorImplementation;
+
+static const TensorPlacement gpuPlacement(TensorPlacement::MemDevices::GPU, 0);
+static int stamped = 0;
+
+static void stampOne(const std::string& name, const Expression& e, const std::unordered_map<std::string, Tensor>& inputs, Stream& stream,
+                     const char* expectKinds = nullptr) {
+    std::printf("[ RUN  ] %s\n", name.c_str());
+    std::fflush(stdout);
+    FusedEquation eq = FusedEquation::compile(Expression::outputs({{"y", e}}).physicalOutputs(), 0);
+    std::unordered_map<std::string, Tensor> used;
+    for (const std::string& input : e.getInputNames()) used.emplace(input, inputs.at(input));
+    StampedExecutionPlan plan = eq.stamp(used, stream);
+    std::string kinds;
+    for (const std::string& k : plan.stageKindNames()) kinds += (kinds.empty() ? "" : ",") + k;
+    if (expectKinds && kinds != expectKinds) {
+        std::printf("  unexpected plan: %s (wanted %s)\n", kinds.c_str(), expectKinds);
+        std::exit(1);
+    }
+    ++stamped;
+}
+
+static int runAll();
+
+int main() {
+    try {
+        return runAll();
+    } catch (const std::exception& e) {
+        std::printf("  exception: %s\n", e.what());
+        return 1;
+    }
+}
+
+static int runAll() {
+    Stream stream(0);
+    const std::vector<std::pair<const char*, DataType>> floats = {{"fp16", DataType::FP16}, {"bf16", DataType::BF16}, {"fp32", DataType::FP32},
+                                                                  {"e4m3", DataType::FP8_E4M3}};
+    // a unary function feeding arithmetic with another tensor, flat kernels, every float dtype (16-bit float arithmetic is
+    // where conversions meet packed instructions)
+    const std::vector<std::pair<const char*, std::function<Expression(const Expression&)>>> unary = {
+        {"exp", [](const Expression& v) { return v.exp(); }},       {"ln", [](const Expression& v) { return v.ln(); }},
+        {"sqrt", [](const Expression& v) { return v.sqrt(); }},     {"tanh", [](const Expression& v) { return v.tanh(); }},
+        {"sin", [](const Expression& v) { return v.sin(); }},       {"erf", [](const Expression& v) { return v.erf(); }},
+        {"lgamma", [](const Expression& v) { return v.lgamma(); }}, {"sigmoid", [](const Expression& v) { return v.sigmoid(); }},
+        {"gelu", [](const Expression& v) { return v.gelu(); }},     {"softplus", [](const Expression& v) { return v.softplus(); }},
+        {"normcdf", [](const Expression& v) { return v.normcdf(); }}, {"log1p", [](const Expression& v) { return v.log1p(); }},
+        {"abs", [](const Expression& v) { return v.abs(); }},       {"floor", [](const Expression& v) { return v.floor(); }}};
+    for (const auto& [dtypeName, dtype] : floats) {
+        Tensor a(gpuPlacement, TensorDescriptor(dtype, {4096, 24})), b(gpuPlacement, TensorDescriptor(dtype, {4096, 24}));
+        const std::unordered_map<std::string, Tensor> inputs{{"a", a}, {"b", b}};
+        const Expression x = Expression::input("a"), y = Expression::input("b");
+        for (const auto& [opName, op] : unary) {
+            stampOne(std::string("flat ") + dtypeName + " a - " + opName + "(b)", x - op(y), inputs, stream, "FusedKernel");
+            stampOne(std::string("flat ") + dtypeName + " " + opName + "(a) * b + a", op(x) * y + x, inputs, stream, "FusedKernel");
+        }
+        stampOne(std::string("rows ") + dtypeName + " softmax", x.softmax(), inputs, stream);
+        stampOne(std::string("rows ") + dtypeName + " log softmax", x.logSoftmax(), inputs, stream);
+        stampOne(std::string("rows ") + dtypeName + " standardise",
+                 (x - x.reduce_mean({1})) / ((x - x.reduce_mean({1})) * (x - x.reduce_mean({1}))).reduce_mean({1}).sqrt(), inputs, stream);
+        stampOne(std::string("columns ") + dtypeName + " sum of a * ln(b)", (x * y.abs().ln()).reduce_sum({0}), inputs, stream);
+    }
+    // ragged batches: scalar and vector values, both offset dtypes, fused and index-gather paths
+    for (const auto& [dtypeName, dtype] : floats) {
+        if (dtype == DataType::FP8_E4M3) continue;
+        for (uint64_t elements : {uint64_t(1), uint64_t(16), uint64_t(3)}) {
+            for (DataType offsetsType : {DataType::UINT32, DataType::UINT64}) {
+                const std::vector<uint64_t> trailing = elements > 1 ? std::vector<uint64_t>{elements} : std::vector<uint64_t>{};
+                const RaggedExpression r = RaggedExpression::input("x", RaggedTensorDescriptor(dtype, trailing, 200, 6000, offsetsType));
+                std::vector<uint64_t> dims{6000};
+                if (elements > 1) dims.push_back(elements);
+                const std::unordered_map<std::string, Tensor> inputs{{"x.values", Tensor(gpuPlacement, TensorDescriptor(dtype, dims))},
+                                                                    {"x.offsets", Tensor(gpuPlacement, TensorDescriptor(offsetsType, {201}))}};
+                const std::string tag = std::string("ragged ") + dtypeName + " E=" + std::to_string(elements) + (offsetsType == DataType::UINT64 ? " u64 " : " u32 ");
+                stampOne(tag + "softmax", r.segment_softmax().getValues(), inputs, stream, "SegmentedReduction,FusedReduction,SegmentedBroadcast,FusedKernel");
+                stampOne(tag + "log softmax", r.segment_log_softmax().getValues(), inputs, stream,
+                         "SegmentedReduction,FusedReduction,SegmentedBroadcast,FusedKernel");
+                stampOne(tag + "mean", r.segment_mean(), inputs, stream, "SegmentedReduction");
+                stampOne(tag + "relu * exp", (r.relu() * r.exp()).getValues(), inputs, stream, "FusedKernel");
+            }
+        }
+    }
+    std::printf("%d expressions stamped, 0 failures\n", stamped);
+    return 0;
+}
