@@ -228,6 +228,49 @@ def bench_other_configs():
     plans = [all3.stamp({"x": t, "scale": scale, "bias": bias}, stream) for t in xc8]
     timed("c5_relu_and_channel_statistics_one_pass_fp16", [p_.run for p_ in plans], 4 * n, n,
           ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
+    del xc, xc8, plans, csum
+
+    # ---- ragged batches (the rows next to the dense path): [2^22, 64] fp32 values (1 GiB) in 65 536 segments of log-normal
+    # length; bytes counted are the values read once (reductions), written once (broadcast), read + written once (softmax)
+    rows, width, segments = 1 << 22, 64, 1 << 16
+    weights = rng.lognormal(0.0, 1.0, segments)
+    cuts = np.floor(np.cumsum(weights) / weights.sum() * rows).astype(np.int64)
+    host_offsets = ph.PhysicalTensor(ph.Placement(ph.DeviceType.cpu), ph.PhysicalTensor.Descriptor(DataType.uint32, [segments + 1]))
+    host_offsets.numpy()[...] = np.concatenate([[0], cuts[:-1], [rows]]).astype(np.uint32)
+    offsets_u32 = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.uint32, [segments + 1]))
+    offsets_u32.copy_from_async(host_offsets, stream)
+    stream.synchronize()
+    from thor_amd import _lib
+    block = gpu_from(rng.standard_normal((1 << 16, width), dtype=np.float32), DataType.fp32)
+    values = []
+    for _ in range(3):
+        t = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [rows, width]))
+        for off in range(0, rows * width, (1 << 16) * width):
+            _lib.check(_lib.load().thorhip_memcpy_async(t.mem_ptr() + off * 4, block.mem_ptr(), (1 << 16) * width * 4, 3, stream.handle), "d2d")
+        values.append(t)
+    stream.synchronize()
+    n = rows * width
+    sums = [ph.CubSegmentedReduction(ph.CubReductionOp.Sum, DataType.fp32).stamp_runtime_offsets(
+        t, ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [segments, width])), offsets_u32, stream)
+        for t in values]
+    timed("ragged_segment_sum_fp32", [s_.run for s_ in sums], 4 * n, n, sums[0].get_kernel_variant())
+    args = [ph.CubSegmentedArgReduction(ph.CubArgReductionOp.ArgMax).stamp_runtime_offsets(
+        t, ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.uint64, [segments, width])), offsets_u32, stream)
+        for t in values]
+    timed("ragged_segment_argmax_fp32", [a_.run for a_ in args], 4 * n, n, args[0].get_kernel_variant())
+    per_segment = sums[0].get_output_tensor()
+    timed("ragged_segmented_broadcast_fp32", [(lambda t=t: ph.segmented_broadcast(per_segment, offsets_u32, t, False, stream)) for t in values], 4 * n, n)
+    rv, ro = ex.input("x.values"), ex.input("x.offsets")
+    spread = lambda v: v.segmented_broadcast(ro, segments, rows, width)
+    shifted = rv - spread(rv.segment_max(ro, segments, rows, width))
+    soft = (shifted.exp() / spread(shifted.exp().segment_sum(ro, segments, rows, width))).with_ragged_runtime_extent(ro, segments, rows, width)
+    ragged = ex.compile(ex.outputs({"y": soft}), 0)
+    for label, env in (("staged", "1"), ("fused", "0")):
+        os.environ["THOR_DISABLE_STAGE_FUSION"] = env
+        plans = [ragged.stamp({"x.values": t, "x.offsets": offsets_u32}, stream) for t in values[:2]]
+        timed(f"ragged_segment_softmax_fp32_{label}", [p_.run for p_ in plans], 8 * n, n, ">".join(plans[0].stage_kind_names()))
+        del plans
+    os.environ.pop("THOR_DISABLE_STAGE_FUSION", None)
     return results
 
 

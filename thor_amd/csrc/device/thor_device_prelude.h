@@ -222,10 +222,9 @@ struct ArgAcc {
     template <typename I>
     __device__ __forceinline__ void add(float x, I index) {
         const bool strictlyBetter = IS_MAX ? (x > v) : (x < v);
-        if (strictlyBetter || ((x != x) && (v == v)) || i == ~(IndexT)0) {
-            v = x;
-            i = (IndexT)index;
-        }
+        const bool take = strictlyBetter | ((x != x) & (v == v)) | (i == ~(IndexT)0);
+        v = take ? x : v;  // selects, not branches: lanes of a wavefront rarely agree
+        i = take ? (IndexT)index : i;
     }
     __device__ __forceinline__ void merge(const ArgAcc& o) {
         if (!better(v, i, o.v, o.i)) {

@@ -399,7 +399,7 @@ std::vector<DataType> FusedEquation::rootDTypes(const std::unordered_map<std::st
 }
 
 std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<DataType>& root_dtypes) const {
-    std::string key;
+    std::string key = stageFusionEnabled() ? "fused:" : "staged:";  // roles differ between the two kinds of plan
     for (DataType d : root_dtypes) key += std::to_string(static_cast<int>(d)) + ",";
     return planned_graph_cache->getOrCreate(key, [&] {
         PhysicalOutputs resolved;
