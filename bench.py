@@ -259,7 +259,8 @@ def bench_other_configs():
         for t in values]
     timed("ragged_segment_argmax_fp32", [a_.run for a_ in args], 4 * n, n, args[0].get_kernel_variant())
     per_segment = sums[0].get_output_tensor()
-    timed("ragged_segmented_broadcast_fp32", [(lambda t=t: ph.segmented_broadcast(per_segment, offsets_u32, t, False, stream)) for t in values], 4 * n, n)
+    timed("ragged_segmented_broadcast_fp32", [(lambda t=t: ph.segmented_broadcast(per_segment, offsets_u32, t, False, stream)) for t in values], 4 * n, n,
+          "thor_segmented_broadcast (output-chunked, LDS window of offsets)")
     rv, ro = ex.input("x.values"), ex.input("x.offsets")
     spread = lambda v: v.segmented_broadcast(ro, segments, rows, width)
     shifted = rv - spread(rv.segment_max(ro, segments, rows, width))
@@ -268,7 +269,8 @@ def bench_other_configs():
     for label, env in (("staged", "1"), ("fused", "0")):
         os.environ["THOR_DISABLE_STAGE_FUSION"] = env
         plans = [ragged.stamp({"x.values": t, "x.offsets": offsets_u32}, stream) for t in values[:2]]
-        timed(f"ragged_segment_softmax_fp32_{label}", [p_.run for p_ in plans], 8 * n, n, ">".join(plans[0].stage_kind_names()))
+        timed(f"ragged_segment_softmax_fp32_{label}", [p_.run for p_ in plans], 8 * n, n,
+              ">".join(plans[0].stage_kind_names()) + " " + " | ".join(plans[0].stage_descriptions()))
         del plans
     os.environ.pop("THOR_DISABLE_STAGE_FUSION", None)
     return results

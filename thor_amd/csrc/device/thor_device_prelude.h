@@ -169,12 +169,13 @@ struct ProductOp {
 struct MinOp {
     __device__ __forceinline__ static float identity() { return __builtin_inff(); }
     __device__ __forceinline__ static float transform(float x) { return x; }
-    __device__ __forceinline__ static float combine(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fminf(a, b)); }
+    // b replaces a when it is smaller or NaN; a NaN in a stays (no comparison with it holds): two compares and a select
+    __device__ __forceinline__ static float combine(float a, float b) { return ((b < a) | (b != b)) ? b : a; }
 };
 struct MaxOp {
     __device__ __forceinline__ static float identity() { return -__builtin_inff(); }
     __device__ __forceinline__ static float transform(float x) { return x; }
-    __device__ __forceinline__ static float combine(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fmaxf(a, b)); }
+    __device__ __forceinline__ static float combine(float a, float b) { return ((b > a) | (b != b)) ? b : a; }
 };
 
 // Accumulator protocol used by every reduction kernel:
@@ -210,12 +211,12 @@ struct ArgAcc {
         i = ~(IndexT)0;
     }
     __device__ __forceinline__ static bool better(float av, IndexT ai, float bv, IndexT bi) {
-        // true when candidate a wins over candidate b
+        // true when candidate a wins over candidate b.  Spelled without control flow: the lanes of a wavefront rarely agree.
         const bool an = av != av, bn = bv != bv;
-        if (an || bn) return (an && bn) ? (ai <= bi) : an;
-        if (IS_MAX ? (av > bv) : (av < bv)) return true;
-        if (IS_MAX ? (bv > av) : (bv < av)) return false;
-        return ai <= bi;
+        const bool strictA = IS_MAX ? (av > bv) : (av < bv);  // false whenever a NaN is involved
+        const bool strictB = IS_MAX ? (bv > av) : (bv < av);
+        const bool onlyA = an & !bn, onlyB = bn & !an;
+        return onlyA | (!onlyB & (strictA | (!strictB & (ai <= bi))));
     }
     // Adds the next element of one thread's walk.  Every kernel visits its elements in increasing index order, so an
     // equal value never replaces the candidate: only a strictly better value, the first NaN, or the first element at all.
@@ -227,10 +228,9 @@ struct ArgAcc {
         i = take ? (IndexT)index : i;
     }
     __device__ __forceinline__ void merge(const ArgAcc& o) {
-        if (!better(v, i, o.v, o.i)) {
-            v = o.v;
-            i = o.i;
-        }
+        const bool keep = better(v, i, o.v, o.i);
+        v = keep ? v : o.v;
+        i = keep ? i : o.i;
     }
     __device__ __forceinline__ ArgAcc shuffleXor(int mask) const {
         ArgAcc r;

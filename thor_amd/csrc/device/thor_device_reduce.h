@@ -479,6 +479,7 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
                     live[u] = r < pEnd;
                     if (live[u]) Cfg::load(src, r * Cfg::kD + columnOffset, x[u]);
                 }
+                // (selects over re-read rows instead of these branches measured 15-25 % slower for sums of short segments)
 #pragma unroll
                 for (int u = 0; u < kBatch; ++u) {
                     if (live[u]) {
