@@ -84,6 +84,8 @@ inline bool isSegmentedReduceOp(ExprOp op) {
     return op == ExprOp::SEGMENTED_REDUCE_SUM || op == ExprOp::SEGMENTED_REDUCE_MIN || op == ExprOp::SEGMENTED_REDUCE_MAX ||
            op == ExprOp::SEGMENTED_REDUCE_MEAN;
 }
+// Views of the operand's storage: nothing is computed, consumers read through the view's strides.
+inline bool isStorageViewOp(ExprOp op) { return op == ExprOp::STRIDED_VIEW || op == ExprOp::TRANSPOSE; }
 inline bool isRaggedOp(ExprOp op) {
     return isSegmentedReduceOp(op) || op == ExprOp::SEGMENTED_BROADCAST || op == ExprOp::RAGGED_VALUEWISE_EXTENT;
 }
@@ -108,6 +110,9 @@ struct ExprNode {
     std::vector<uint64_t> unsqueeze_axes;
     std::vector<uint64_t> reshape_dims;    // one entry may be UINT64_MAX = inferred
     std::vector<uint64_t> fill_dims;
+    // STRIDED_VIEW: shape, strides and first element of the view, in elements of the operand's storage
+    std::vector<uint64_t> view_dims, view_strides;
+    uint64_t view_element_offset = 0;
     SoftmaxAlgorithm softmax_algorithm = SoftmaxAlgorithm::Accurate;  // SOFTMAX only
     SoftmaxMode softmax_mode = SoftmaxMode::Channel;
 
@@ -315,6 +320,15 @@ class Expression {
     Expression reshape(const std::vector<uint64_t>& new_dims) const;
     Expression unsqueeze(const std::vector<uint64_t>& unsqueeze_axes) const;
     Expression squeeze(const std::vector<uint64_t>& squeeze_axes) const;
+    // A view of the operand's storage (reference: Expression.cpp:3769-3787 there): `strides_elements` and `element_offset`
+    // address the storage of the tensor the operand resolves to, not the logical index space of an earlier view.  Nothing is
+    // copied; kernels read through the strides.
+    Expression stridedView(const std::vector<uint64_t>& dims, const std::vector<uint64_t>& strides_elements, uint64_t element_offset = 0) const;
+    Expression aliasView(const std::vector<uint64_t>& dims, const std::vector<uint64_t>& strides_elements, uint64_t element_offset = 0) const {
+        return stridedView(dims, strides_elements, element_offset);
+    }
+    // The last two axes exchanged (rank >= 2), as a view.
+    Expression transpose() const;
 
     // ---- reductions: fp32 accumulation, reduced axes kept as 1 unless listed in squeeze_axes ------------------------
     Expression reduction(ExprOp op, const std::vector<uint64_t>& reduction_axes, const std::vector<uint64_t>& squeeze_axes,

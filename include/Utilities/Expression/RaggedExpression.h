@@ -6,7 +6,7 @@
 //
 // Differences from the reference on this backend: segment_softmax / segment_log_softmax use the segment maximum and sum
 // broadcast back over the rows for scalar values too (the reference runs segmented scans there; the values agree to fp32
-// rounding), and trailing-dimension slices are not available (the Expression graph here has no strided views).
+// rounding); RaggedExpressionRuntimeExtent carries no activeValueCount expression (the kernels read offsets[B] themselves).
 #pragma once
 
 #include "DeepLearning/Implementation/Tensor/RaggedTensorDescriptor.h"
@@ -57,6 +57,11 @@ class RaggedExpression {
     RaggedExpression withValues(Expression new_values, RaggedTensorDescriptor new_descriptor) const;
     // any shape-preserving function of the unwrapped packed values
     RaggedExpression mapValues(const std::function<Expression(const Expression&)>& mapper) const;
+    // [start, start + length) of one trailing axis, as a strided view of the packed values: consecutive slices compose into
+    // one view of the original storage (reference: RaggedExpression.cpp:143-203 there).  The values have to resolve to a
+    // dense tensor (an input or a stored value).
+    RaggedExpression sliceTrailingDimension(uint64_t trailing_axis, uint64_t start, uint64_t length) const;
+    RaggedExpression sliceLastDimension(uint64_t start, uint64_t length) const;
     RaggedExpression cast(DataType output_dtype) const;
 
     RaggedExpression operator+(const RaggedExpression& other) const;
@@ -94,6 +99,15 @@ class RaggedExpression {
     Expression overRows(const Expression& per_segment_values, bool normalize_by_segment_length) const;
     RaggedExpression compare(const RaggedExpression& other, Comparison which, const char* caller) const;
     RaggedExpression shiftedExponentials(Expression& shifted) const;
+
+    // a slice remembers the storage it views, so that the next slice re-views that storage with composed strides
+    struct SliceOrigin {
+        Expression source = Expression::constantScalar(0.0);
+        std::vector<uint64_t> strides;
+        uint64_t offset = 0;
+        bool valid = false;
+    };
+    SliceOrigin sliceOrigin;
 
     Expression values = Expression::constantScalar(0.0);           // what ragged operations compose on
     Expression executionValues = Expression::constantScalar(0.0);  // values under the runtime-extent marker

@@ -162,6 +162,8 @@ thor_expr_t thor_expr_with_dtypes(thor_expr_t input, int compute_dtype, int outp
  * "argmin", "argmax"; num_axes == 0 reduces all axes; squeeze axis UINT64_MAX squeezes every singleton axis */
 thor_expr_t thor_expr_reduce(const char* method, thor_expr_t input, const uint64_t* axes, int num_axes, const uint64_t* squeeze_axes,
                              int num_squeeze_axes);
+/* Expression::stridedView: dims / strides / offset in elements of the operand's storage ("transpose" is a unary method). */
+thor_expr_t thor_expr_strided_view(thor_expr_t input, const uint64_t* dims, const uint64_t* strides, int rank, uint64_t element_offset);
 thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank);
 thor_expr_t thor_expr_unsqueeze(thor_expr_t input, const uint64_t* axes, int num_axes);
 thor_expr_t thor_expr_squeeze(thor_expr_t input, const uint64_t* axes, int num_axes);

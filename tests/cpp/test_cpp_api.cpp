@@ -273,6 +273,20 @@ static void raggedExpressionStructure() {
     CHECK(reduction.op == ExprOp::SEGMENTED_REDUCE_SUM && reduction.ragged_runtime_elements_per_value == 4 && reduction.ragged_runtime_batch_size == 3);
     CHECK(canonicalize(reduced).find("segmented_reduce_sum:ragged=[3,9,4]") != std::string::npos);
     CHECK(throwsAs<std::invalid_argument>([&] { (void)(Expression::input("v") + 1.0).withRaggedRuntimeExtent(Expression::input("o") + 1.0, 3, 9, 4); }));
+
+    // RaggedExpressionTest.cpp:800-871 there: trailing slices keep the partition and use storage strides; nested slices compose
+    const RaggedExpression wide = RaggedExpression::input("w", RaggedTensorDescriptor(DataType::FP32, {2, 6}, 3, 9));
+    const RaggedExpression inner = wide.sliceLastDimension(2, 4).sliceLastDimension(1, 2);
+    CHECK((inner.getValuesDimensions() == std::vector<uint64_t>{9, 2, 2}) && inner.getRuntimeExtent().elementsPerValue == 4);
+    const PhysicalExpression sliced = inner.getValues().expression();
+    const ExprNode& view = sliced.nodes.at(sliced.nodes.at(sliced.output_node).lhs);
+    CHECK(view.op == ExprOp::STRIDED_VIEW && (view.view_strides == std::vector<uint64_t>{12, 6, 1}) && view.view_element_offset == 3);
+    CHECK(sliced.nodes.at(view.lhs).op == ExprOp::INPUT);  // one view of the original storage, not a view of a view
+    const RaggedExpression outer = wide.sliceTrailingDimension(0, 1, 1);
+    CHECK((outer.getValuesDimensions() == std::vector<uint64_t>{9, 1, 6}));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)wide.sliceLastDimension(4, 3); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)wide.sliceTrailingDimension(2, 0, 1); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)wide.sliceLastDimension(0, 0); }));
 }
 
 static void raggedExpressionExecution(Stream& stream) {
@@ -333,6 +347,18 @@ static void raggedExpressionExecution(Stream& stream) {
         const RaggedExpression y = x.relu() * x.relu();
         const std::vector<float> q = toHostF32(runOne(y.getValues(), inputs, gpuFrom(std::vector<float>(8, -7.0f), {8}, stream)), stream);
         CHECK((q == std::vector<float>{1, 4, 0, 0, 1, -7, -7, -7}));
+    }
+    {
+        // trailing slices of [6, 4] values compose and only the active rows are computed (:1348-1404 there)
+        const RaggedExpression x = RaggedExpression::input("x", RaggedTensorDescriptor(DataType::FP32, {4}, 2, 6));
+        std::vector<float> host(24);
+        for (size_t i = 0; i < host.size(); ++i) host[i] = static_cast<float>(i);
+        const std::unordered_map<std::string, Tensor> inputs{{"x.values", gpuFrom(host, {6, 4}, stream)}, {"x.offsets", gpuOffsets({0, 1, 4}, stream)}};
+        const RaggedExpression product = x.sliceLastDimension(0, 2) * x.sliceLastDimension(2, 2);
+        const std::vector<float> p = toHostF32(runOne(product.getValues(), inputs, gpuFrom(std::vector<float>(12, -1.0f), {6, 2}, stream)), stream);
+        CHECK((p == std::vector<float>{0 * 2, 1 * 3, 4 * 6, 5 * 7, 8 * 10, 9 * 11, 12 * 14, 13 * 15, -1, -1, -1, -1}));
+        const std::vector<float> sums = toHostF32(runOne(x.sliceLastDimension(1, 2).sliceLastDimension(1, 1).segment_sum(), inputs), stream);
+        CHECK((sums == std::vector<float>{2, 6 + 10 + 14}));
     }
 }
 

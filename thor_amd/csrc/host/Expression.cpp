@@ -486,6 +486,28 @@ Expression Expression::withDTypes(std::optional<DataType> compute_dtype, std::op
     return Expression(out, root);
 }
 
+Expression Expression::stridedView(const std::vector<uint64_t>& dims, const std::vector<uint64_t>& strides_elements, uint64_t element_offset) const {
+    if (!expr) throw std::runtime_error("Cannot create a strided view from an empty expression");
+    if (dims.empty() || dims.size() != strides_elements.size()) {
+        throw std::invalid_argument("Expression::stridedView requires dimensions and strides with the same non-zero rank.");
+    }
+    for (uint64_t d : dims) {
+        if (d == std::numeric_limits<uint64_t>::max()) throw std::invalid_argument("Expression::stridedView does not support infer-dimension markers.");
+        if (d == 0) throw std::invalid_argument("Expression::stridedView does not support zero-sized dimensions.");
+    }
+    Expression out = unaryOp(*this, ExprOp::STRIDED_VIEW);
+    ExprNode& node = out.expr->nodes[out.nodeIndex];
+    node.view_dims = dims;
+    node.view_strides = strides_elements;
+    node.view_element_offset = element_offset;
+    return out;
+}
+
+Expression Expression::transpose() const {
+    if (!expr) throw std::runtime_error("Cannot transpose an empty expression");
+    return unaryOp(*this, ExprOp::TRANSPOSE);
+}
+
 // ---- ragged batches ------------------------------------------------------------------------------------------------------
 Expression Expression::segmentedReduceWithRaggedMetadata(const Expression& input, const Expression& offsets, ExprOp op, uint64_t ragged_batch_size,
                                                          uint64_t ragged_max_active_values, uint64_t ragged_elements_per_value) {
@@ -628,6 +650,7 @@ std::string opName(ExprOp op) {
         {(uint16_t)ExprOp::REDUCE_NORM1, "reduce_norm1"}, {(uint16_t)ExprOp::REDUCE_NORM2, "reduce_norm2"},
         {(uint16_t)ExprOp::SEGMENTED_REDUCE_SUM, "segmented_reduce_sum"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MIN, "segmented_reduce_min"},
         {(uint16_t)ExprOp::SEGMENTED_REDUCE_MAX, "segmented_reduce_max"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MEAN, "segmented_reduce_mean"},
+        {(uint16_t)ExprOp::STRIDED_VIEW, "strided_view"}, {(uint16_t)ExprOp::TRANSPOSE, "transpose"},
         {(uint16_t)ExprOp::SEGMENTED_BROADCAST, "segmented_broadcast"}, {(uint16_t)ExprOp::RAGGED_VALUEWISE_EXTENT, "ragged_valuewise_extent"},
     };
     auto it = names.find(static_cast<uint16_t>(op));
@@ -690,6 +713,9 @@ std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex,
         if (n.op == ExprOp::RESHAPE) text += ":dims=" + axesText(n.reshape_dims);
         if (n.op == ExprOp::UNSQUEEZE) text += ":axes=" + axesText(n.unsqueeze_axes);
         if (n.op == ExprOp::SQUEEZE) text += ":axes=" + axesText(n.squeeze_axes);
+        if (n.op == ExprOp::STRIDED_VIEW) {
+            text += ":dims=" + axesText(n.view_dims) + ":strides=" + axesText(n.view_strides) + ":offset=" + std::to_string(n.view_element_offset);
+        }
         if (isRaggedOp(n.op)) {
             text += ":ragged=[" + std::to_string(n.ragged_runtime_batch_size) + "," + std::to_string(n.ragged_runtime_max_active_values) + "," +
                     std::to_string(n.ragged_runtime_elements_per_value) + "]";

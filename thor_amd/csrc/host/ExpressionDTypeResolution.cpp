@@ -8,7 +8,7 @@ namespace {
 
 bool isComparison(ExprOp op) { return op >= ExprOp::EQUAL && op <= ExprOp::GREATER_EQUAL; }
 bool isLogical(ExprOp op) { return op == ExprOp::LOGICAL_AND || op == ExprOp::LOGICAL_OR || op == ExprOp::LOGICAL_NOT; }
-bool isShapeOnly(ExprOp op) { return op == ExprOp::RESHAPE || op == ExprOp::UNSQUEEZE || op == ExprOp::SQUEEZE; }
+bool isShapeOnly(ExprOp op) { return op == ExprOp::RESHAPE || op == ExprOp::UNSQUEEZE || op == ExprOp::SQUEEZE || isStorageViewOp(op); }
 bool isScalarLeaf(ExprOp op) { return op == ExprOp::SCALAR_FP || op == ExprOp::RUNTIME_SCALAR || op == ExprOp::TENSOR_RUNTIME_SCALAR; }
 
 bool isBindableInputDType(DataType dtype) {
@@ -29,7 +29,7 @@ bool isBindableInputDType(DataType dtype) {
 }
 
 void rejectUnsupportedOp(ExprOp op) {
-    if (isRaggedOp(op)) return;
+    if (isRaggedOp(op) || isStorageViewOp(op)) return;
     if (Expression::isLeafOp(op) || Expression::isUnaryOp(op) || Expression::isBinaryOp(op) || Expression::isTernaryOp(op)) {
         if (op != ExprOp::TENSOR_RUNTIME_SCALAR) return;
     }

@@ -35,7 +35,7 @@ namespace {
 
 using Role = PlannedGraph::Role;
 
-bool isShapeOnly(ExprOp op) { return op == ExprOp::RESHAPE || op == ExprOp::UNSQUEEZE || op == ExprOp::SQUEEZE; }
+bool isShapeOnly(ExprOp op) { return op == ExprOp::RESHAPE || op == ExprOp::UNSQUEEZE || op == ExprOp::SQUEEZE || isStorageViewOp(op); }
 bool isReductionStorage(DataType d) {
     return d == DataType::FP8_E4M3 || d == DataType::FP8_E5M2 || d == DataType::FP16 || d == DataType::BF16 || d == DataType::FP32;
 }
@@ -52,7 +52,8 @@ std::string structuralKey(const ExprNode& n) {
       << "|" << (n.input_tensor_dtype ? static_cast<int>(*n.input_tensor_dtype) : -1) << "|" << (n.output_dtype ? static_cast<int>(*n.output_dtype) : -1)
       << "|" << (n.compute_dtype ? static_cast<int>(*n.compute_dtype) : -1) << "|" << axesKey(n.reduction_axes) << "|" << axesKey(n.squeeze_axes)
       << "|" << axesKey(n.unsqueeze_axes) << "|" << axesKey(n.reshape_dims) << "|" << axesKey(n.fill_dims) << "|" << n.ragged_runtime_batch_size << "|"
-      << n.ragged_runtime_max_active_values << "|" << n.ragged_runtime_elements_per_value << "|" << n.segmented_broadcast_normalize_by_length;
+      << n.ragged_runtime_max_active_values << "|" << n.ragged_runtime_elements_per_value << "|" << n.segmented_broadcast_normalize_by_length << "|"
+      << axesKey(n.view_dims) << "|" << axesKey(n.view_strides) << "|" << n.view_element_offset;
     return k.str();
 }
 
@@ -134,6 +135,10 @@ class GraphBuilder {
         } else if (isShapeOnly(node.op)) {
             double folded;
             if (!tryFoldConstant(out, node.lhs, folded)) node.lhs = asTensorOperand(node.lhs, false);
+        }
+        if ((isSegmentedReduceOp(node.op) || node.op == ExprOp::SEGMENTED_BROADCAST) && isStorageViewOp(out.nodes[node.lhs].op)) {
+            // the segment kernels stream dense rows: a strided view is gathered into a dense tensor first (an identity kernel)
+            node.lhs = castOf(node.lhs, out.nodes[node.lhs].output_dtype.value());
         }
         const uint32_t idx = add(std::move(node));
         remap.emplace(srcIndex, idx);
@@ -266,6 +271,14 @@ std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std:
                 dims[i] = out;
                 break;
             }
+            case ExprOp::STRIDED_VIEW:
+                dims[i] = n.view_dims;
+                break;
+            case ExprOp::TRANSPOSE:
+                if (dims[n.lhs].size() < 2) throw std::runtime_error("Expression::transpose requires a tensor of rank 2 or more.");
+                dims[i] = dims[n.lhs];
+                std::swap(dims[i][dims[i].size() - 1], dims[i][dims[i].size() - 2]);
+                break;
             case ExprOp::SQUEEZE:
                 dims[i] = StampedEquation::computeReductionOutputDims(dims[n.lhs], {}, n.squeeze_axes.empty() ? std::vector<uint64_t>{UINT64_MAX} : n.squeeze_axes);
                 break;
@@ -441,7 +454,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
                 ensureTensor(n.rhs);
             } else if (isShapeOnly(n.op)) {
                 double folded;
-                if (!tryFoldConstant(graph->expr, i, folded)) {
+                if (isStorageViewOp(n.op) || !tryFoldConstant(graph->expr, i, folded)) {
                     ensureTensor(n.lhs);
                     graph->role[i] = Role::View;
                 }
@@ -615,6 +628,19 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
 
     auto viewOf = [&](uint32_t node) {
         const Tensor& base = tensorOf[expr.nodes[node].lhs];
+        const ExprNode& v = expr.nodes[node];
+        if (v.op == ExprOp::STRIDED_VIEW) {
+            // strides and offset address the storage the operand resolves to
+            if (!base.isDenseContiguous()) throw std::runtime_error("Expression::stridedView needs a dense operand: compose the strides of nested views first.");
+            return base.aliasView(v.view_dims, v.view_strides, v.view_element_offset);
+        }
+        if (v.op == ExprOp::TRANSPOSE) {
+            std::vector<uint64_t> d = base.getDimensions(), st = base.getStridesElements();
+            if (d.size() < 2) throw std::runtime_error("Expression::transpose requires a tensor of rank 2 or more.");
+            std::swap(d[d.size() - 1], d[d.size() - 2]);
+            std::swap(st[st.size() - 1], st[st.size() - 2]);
+            return base.aliasView(d, st, 0);
+        }
         if (!base.isDenseContiguous()) throw std::runtime_error("Shape operations on a non-dense tensor view are not supported.");
         Tensor view = base;
         view.reshape(orScalarShape(dims[node]));

@@ -505,6 +505,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
             return true;
         }
         if (layout.dims.back() % v != 0) return false;
+        if (r.extent.has_value() && r.extent->elementsPerValue % v != 0) return false;  // a vector never straddles the last active row
         for (size_t o = 0; o < r.operands.size(); ++o) {
             const std::vector<uint64_t>& s = layout.operandStride[o];
             if (s.back() > 1) return false;  // neither contiguous nor broadcast along the innermost axis
@@ -543,10 +544,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         s << "const " << deviceTypeName(r.gathers[g].storageDType) << "* g" << g << ", const unsigned int* gid" << g << ", ";
         if (r.gathers[g].normalize) s << "const " << (r.gathers[g].offsetsAre64 ? "unsigned long long" : "unsigned int") << "* goff" << g << ", ";
     }
-    if (r.extent.has_value()) {
-        if (!k.flat) throw std::runtime_error("A ragged runtime extent needs operands of the output's own dense shape (no broadcasting).");
-        s << "const " << (r.extent->offsetsAre64 ? "unsigned long long" : "unsigned int") << "* extentOffsets, ";
-    }
+    if (r.extent.has_value()) s << "const " << (r.extent->offsetsAre64 ? "unsigned long long" : "unsigned int") << "* extentOffsets, ";
     for (uint32_t slot : r.scalarSlots) s << "float s" << slot << ", ";
     for (size_t o = 0; o < r.outputs.size(); ++o) {
         s << deviceTypeName(r.outputs[o].storageDType) << "* out" << o;
@@ -558,7 +556,8 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
     if (r.extent.has_value()) {
         // only the rows the partition covers now are computed; the rest of the outputs keeps its contents
         s << "    const unsigned long long active = (unsigned long long)extentOffsets[" << r.extent->batchSize << "ull] * " << r.extent->elementsPerValue
-          << "ull;\n    const index_t numel = active < (unsigned long long)capacity ? (index_t)active : capacity;\n";
+          << "ull;\n";
+        if (k.flat) s << "    const index_t numel = active < (unsigned long long)capacity ? (index_t)active : capacity;\n";
     }
     s << "    constexpr int V = " << vec << ";\n";
 
@@ -676,6 +675,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         for (uint64_t d : dims) lanes *= d;
         s << "    const index_t lane = (index_t)blockIdx.x * " << threads << "u + threadIdx.x;\n";
         s << "    if (lane >= " << lanes << "ull) return;\n";
+        if (r.extent.has_value()) s << "    if ((unsigned long long)lane * V >= active) return;\n";
         s << "    index_t rest = lane;\n";
         for (size_t a = dims.size(); a-- > 0;) {
             if (a == 0) {

@@ -110,6 +110,40 @@ RaggedExpression RaggedExpression::mapValues(const std::function<Expression(cons
     return withValues(mapper(values), descriptor);
 }
 
+RaggedExpression RaggedExpression::sliceTrailingDimension(uint64_t trailing_axis, uint64_t start, uint64_t length) const {
+    requireInitialized("sliceTrailingDimension");
+    const std::vector<uint64_t> trailing = descriptor.getTrailingDimensions();
+    if (trailing_axis >= trailing.size()) throw std::invalid_argument("RaggedExpression::sliceTrailingDimension trailing axis is out of range.");
+    if (length == 0) throw std::invalid_argument("RaggedExpression::sliceTrailingDimension requires a non-zero slice length.");
+    if (start >= trailing[trailing_axis] || length > trailing[trailing_axis] - start) {
+        throw std::invalid_argument("RaggedExpression::sliceTrailingDimension slice exceeds the source trailing dimension.");
+    }
+    std::vector<uint64_t> dims = descriptor.getValuesDimensions();
+    // strides address storage, not the index space of an earlier view: a slice of a slice re-views the first slice's source
+    SliceOrigin origin = sliceOrigin;
+    if (!origin.valid) {
+        origin.source = values;
+        origin.strides.assign(dims.size(), 1);
+        for (size_t a = dims.size() - 1; a-- > 0;) origin.strides[a] = origin.strides[a + 1] * dims[a + 1];
+        origin.offset = 0;
+        origin.valid = true;
+    }
+    origin.offset += start * origin.strides[trailing_axis + 1];
+    dims[trailing_axis + 1] = length;
+    RaggedExpression out = withValues(origin.source.stridedView(dims, origin.strides, origin.offset),
+                                      RaggedTensorDescriptor(TensorDescriptor(descriptor.getValuesDataType(), dims), descriptor.getRowPartition(),
+                                                             descriptor.getRaggedRank()));
+    out.sliceOrigin = origin;
+    return out;
+}
+
+RaggedExpression RaggedExpression::sliceLastDimension(uint64_t start, uint64_t length) const {
+    requireInitialized("sliceLastDimension");
+    const size_t rank = descriptor.getTrailingDimensions().size();
+    if (rank == 0) throw std::invalid_argument("RaggedExpression::sliceLastDimension requires at least one trailing value dimension.");
+    return sliceTrailingDimension(rank - 1, start, length);
+}
+
 RaggedExpression RaggedExpression::cast(DataType output_dtype) const {
     requireInitialized("cast");
     return withValues(values.cast(output_dtype), withValuesDataType(descriptor, output_dtype));

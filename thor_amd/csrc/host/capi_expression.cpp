@@ -40,7 +40,7 @@ const std::unordered_map<std::string, std::function<Expression(const Expression&
         M(asec), M(acot), M(sinh), M(cosh), M(tanh), M(csch), M(sech), M(coth), M(asinh), M(acosh), M(atanh), M(acsch), M(asech), M(acoth),
         M(erf), M(erfc), M(erfcx), M(erfinv), M(erfcinv), M(tgamma), M(lgamma), M(digamma), M(ln), M(log1p), M(log2), M(log10), M(exp), M(expm1),
         M(exp2), M(exp10), M(sqrt), M(normcdf), M(sigmoid), M(softplus), M(selu), M(gelu), M(mish), M(relu6), M(hardSwish), M(swish),
-        M(logicalNot),
+        M(logicalNot), M(transpose),
 #undef M
         {"neg", [](const Expression& e) { return -e; }},
         {"elu", [](const Expression& e) { return e.elu(); }},
@@ -179,6 +179,11 @@ thor_expr_t thor_expr_reduce(const char* method, thor_expr_t input, const uint64
         auto it = ops.find(method ? method : "");
         if (it == ops.end()) throw std::invalid_argument(std::string("Unknown reduction method: ") + (method ? method : "(null)"));
         return new thor_expr{input->expr.reduction(it->second, u64s(axes, num_axes), u64s(squeeze_axes, num_squeeze_axes), std::nullopt)};)
+}
+thor_expr_t thor_expr_strided_view(thor_expr_t input, const uint64_t* dims, const uint64_t* strides, int rank, uint64_t element_offset) {
+    THOR_CAPI_TRY_PTR(require(input, "expression"); if (rank < 0 || (rank > 0 && (!dims || !strides))) throw std::invalid_argument("strided view needs dims and strides.");
+                      return new thor_expr{input->expr.stridedView(std::vector<uint64_t>(dims, dims + rank), std::vector<uint64_t>(strides, strides + rank),
+                                                                   element_offset)};)
 }
 thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank) {
     THOR_CAPI_TRY_PTR(require(input, "expression"); return new thor_expr{input->expr.reshape(u64s(dims, rank))};)

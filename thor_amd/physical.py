@@ -72,6 +72,7 @@ PROTOTYPES = {
     "thor_expr_unary_params": (_vp, [_cp, _vp, ctypes.c_double, ctypes.c_double]), "thor_expr_where": (_vp, [_vp, _vp, _vp]),
     "thor_expr_cast": (_vp, [_vp, _i]), "thor_expr_with_dtypes": (_vp, [_vp, _i, _i]),
     "thor_expr_reduce": (_vp, [_cp, _vp, _u64p, _i, _u64p, _i]), "thor_expr_reshape": (_vp, [_vp, _u64p, _i]),
+    "thor_expr_strided_view": (_vp, [_vp, _u64p, _u64p, _i, ctypes.c_uint64]),
     "thor_expr_unsqueeze": (_vp, [_vp, _u64p, _i]), "thor_expr_squeeze": (_vp, [_vp, _u64p, _i]), "thor_expr_destroy": (None, [_vp]),
     "thor_expr_num_nodes": (_i, [_vp]), "thor_expr_canonical": (_i, [_vp, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_outputs_create": (_vp, [_cpp, _vpp, _i]), "thor_outputs_destroy": (None, [_vp]),
@@ -666,6 +667,20 @@ class Expression:
     def with_ragged_runtime_extent(self, offsets, batch_size: int, max_active_values: int, elements_per_value: int = 1):
         """The same values, computed only for the first offsets[batch_size] rows; the rest of the output keeps its contents."""
         return self._ragged("ragged_extent", offsets, batch_size, max_active_values, elements_per_value)
+
+    def transpose(self) -> "Expression":
+        """The last two axes exchanged, as a view of the operand's storage."""
+        return self._unary("transpose")
+
+    def strided_view(self, dims: Sequence[int], strides_elements: Sequence[int], element_offset: int = 0) -> "Expression":
+        """A view of the operand's storage: strides and offset are in elements of the tensor the operand resolves to."""
+        d, rank = _u64_array(dims)
+        st, rank2 = _u64_array(strides_elements)
+        if rank != rank2:
+            raise ValueError("strided_view needs one stride per dimension")
+        return Expression(lib().thor_expr_strided_view(self._h, d, st, rank, int(element_offset)))
+
+    alias_view = strided_view
 
     def reshape(self, dims: Sequence[int]) -> "Expression":
         d, rank = _u64_array([UINT64_MAX if v == -1 else v for v in dims])
