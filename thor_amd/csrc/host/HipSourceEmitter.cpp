@@ -518,6 +518,28 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         return true;
     };
     while (vec > 1 && !fits(vec)) vec /= 2;
+
+    // Operands whose contiguous axis is another axis of the output than the innermost one (transposes, permuted views): read
+    // through LDS tiles, so that both the operand and the output are addressed along their own contiguous axis.
+    int tileAxis = -1;
+    std::vector<char> viaTile(r.operands.size(), 0);
+    if (!k.flat && layout.dims.size() >= 2 && !r.extent.has_value() && r.gathers.empty()) {
+        bool consistent = true;
+        for (size_t o = 0; o < r.operands.size() && consistent; ++o) {
+            const std::vector<uint64_t>& st = layout.operandStride[o];
+            if (st.back() <= 1) continue;
+            int axis = -1;
+            for (size_t a = 0; a + 1 < st.size(); ++a)
+                if (st[a] == 1 && layout.dims[a] > 1) axis = static_cast<int>(a);
+            if (axis < 0) continue;  // contiguous nowhere: strided scalar reads
+            if (tileAxis >= 0 && tileAxis != axis) consistent = false;
+            tileAxis = axis;
+            viaTile[o] = 1;
+        }
+        if (!consistent || tileAxis < 0 || layout.dims[tileAxis] < 16 || layout.dims.back() < 16) tileAxis = -1;
+    }
+    const bool tiled = tileAxis >= 0;
+    if (tiled) vec = 1;
     k.vec = vec;
     k.passNumel = k.flat;
 
@@ -668,6 +690,97 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         const uint64_t lanes = (k.numel + vec - 1) / vec;
         k.gridX = static_cast<uint32_t>(std::max<uint64_t>((lanes + threads - 1) / threads, 1));
         k.description = "flat(vec=" + std::to_string(vec) + ")";
+    } else if (tiled) {
+        // block = one 64 x (64 * VB) tile of the (tile axis, innermost axis) plane at fixed other coordinates; 256 threads = 4 rows
+        // of 64; a thread handles VB adjacent innermost elements (4 bytes of the widest type) per row
+        const std::vector<uint64_t>& dims = layout.dims;
+        const size_t rank = dims.size(), A = static_cast<size_t>(tileAxis), B = rank - 1;
+        std::vector<uint64_t> outStride(rank, 1);
+        for (size_t a = rank; a-- > 1;) outStride[a - 1] = outStride[a] * dims[a];
+        int vb = std::max(1, 4 / static_cast<int>(widest));
+        auto vectorFits = [&](int v) {
+            if (dims[B] % v != 0) return false;
+            for (const KernelOutput& out : r.outputs)
+                if (out.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(out.storageDType)) != 0) return false;
+            for (size_t o = 0; o < r.operands.size(); ++o) {
+                const std::vector<uint64_t>& st = layout.operandStride[o];
+                if (viaTile[o] || st[B] != 1) continue;
+                if (r.operands[o].alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(r.operands[o].storageDType)) != 0) return false;
+                for (size_t a = 0; a < B; ++a)
+                    if (st[a] % v != 0) return false;
+            }
+            return true;
+        };
+        while (vb > 1 && !vectorFits(vb)) vb /= 2;
+        const uint64_t tileB = 64ull * vb;
+        const uint64_t tilesA = (dims[A] + 63) / 64, tilesB = (dims[B] + tileB - 1) / tileB;
+        uint64_t blocks = tilesA * tilesB;
+        s << "    constexpr int PITCH = 65;\n    constexpr int VB = " << vb << ";\n";
+        s << "    const unsigned tx = threadIdx.x % 64u, ty = threadIdx.x / 64u;\n";
+        s << "    unsigned long long rest = blockIdx.x;\n";
+        // tiles are numbered along diagonals: blocks that run together then differ in both coordinates, so neither the
+        // reads (rows a pitch apart) nor the writes of a power-of-two matrix queue up on one memory channel
+        s << "    const unsigned long long tileB = rest % " << tilesB << "ull;\n    rest /= " << tilesB << "ull;\n";
+        s << "    const unsigned long long b0 = tileB * " << tileB << "ull;\n";
+        s << "    const unsigned long long a0 = ((rest + tileB) % " << tilesA << "ull) * 64ull;\n    rest /= " << tilesA << "ull;\n";
+        for (size_t a = rank; a-- > 0;) {
+            if (a == A || a == B) continue;
+            s << "    const unsigned long long c" << a << " = rest % " << dims[a] << "ull;\n    rest /= " << dims[a] << "ull;\n";
+            blocks *= dims[a];
+        }
+        auto baseOf = [&](const std::vector<uint64_t>& st) {
+            std::string text = "0ull";
+            for (size_t a = 0; a < rank; ++a)
+                if (a != A && a != B && st[a] != 0) text += " + c" + std::to_string(a) + " * " + std::to_string(st[a]) + "ull";
+            return text;
+        };
+        for (size_t o = 0; o < r.operands.size(); ++o) s << "    const unsigned long long base" << o << " = " << baseOf(layout.operandStride[o]) << ";\n";
+        s << "    const unsigned long long outBase = " << baseOf(outStride) << ";\n";
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            if (!viaTile[o]) continue;
+            const char* type = deviceTypeName(r.operands[o].storageDType);
+            s << "    __shared__ " << type << " tile" << o << "[64 * VB * PITCH];\n";
+            s << "#pragma unroll\n    for (int i = 0; i < 16 * VB; ++i) {\n";
+            s << "        const unsigned long long a = a0 + tx, b = b0 + ty + 4u * i;\n";
+            s << "        if (a < " << dims[A] << "ull && b < " << dims[B] << "ull) tile" << o << "[(ty + 4u * i) * PITCH + tx] = in" << o << "[base" << o
+              << " + a + b * " << layout.operandStride[o][B] << "ull];\n    }\n";
+        }
+        s << "    __syncthreads();\n";
+        s << "#pragma unroll 4\n    for (int i = 0; i < 16; ++i) {\n";
+        s << "        const unsigned long long a = a0 + ty + 4u * i, b = b0 + tx * VB;\n";
+        s << "        if (a >= " << dims[A] << "ull || b >= " << dims[B] << "ull) continue;\n";
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            if (viaTile[o]) continue;
+            const std::vector<uint64_t>& st = layout.operandStride[o];
+            const char* type = deviceTypeName(r.operands[o].storageDType);
+            const std::string address = "in" + std::to_string(o) + " + base" + std::to_string(o) + " + a * " + std::to_string(st[A]) + "ull + b * " +
+                                        std::to_string(st[B]) + "ull";
+            if (st[B] == 1) {
+                s << "        thor::Pack<" << type << ", VB> p" << o << ";\n        p" << o << ".loadStream(" << address << ");\n";
+            } else if (st[B] == 0) {
+                s << "        const " << type << " b" << o << " = *(" << address << ");\n";
+            }
+        }
+        for (size_t o = 0; o < r.outputs.size(); ++o) s << "        thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", VB> q" << o << ";\n";
+        s << "#pragma unroll\n        for (int k = 0; k < VB; ++k) {\n";
+        s << emitBody(
+            "            ",
+            [&](size_t o) {
+                const std::vector<uint64_t>& st = layout.operandStride[o];
+                if (viaTile[o]) return "tile" + std::to_string(o) + "[(tx * VB + k) * PITCH + ty + 4u * i]";
+                if (st[B] == 1) return "p" + std::to_string(o) + ".v[k]";
+                if (st[B] == 0) return "b" + std::to_string(o);
+                return "in" + std::to_string(o) + "[base" + std::to_string(o) + " + a * " + std::to_string(st[A]) + "ull + (b + k) * " + std::to_string(st[B]) + "ull]";
+            },
+            [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; }, noGather);
+        s << "        }\n";
+        for (size_t o = 0; o < r.outputs.size(); ++o)
+            s << "        q" << o << ".storeStream(out" << o << " + outBase + a * " << outStride[A] << "ull + b);\n";
+        s << "    }\n";
+        if (blocks >= (1ull << 31)) throw std::runtime_error("Tiled fused kernel would need more blocks than a grid holds.");
+        k.gridX = static_cast<uint32_t>(blocks);
+        k.vec = vb;
+        k.description = "tiled(axis=" + std::to_string(tileAxis) + "/" + std::to_string(rank) + ",tile=64x" + std::to_string(tileB) + ")";
     } else {
         std::vector<uint64_t> dims = layout.dims;
         dims.back() /= vec;  // the innermost axis is walked in vectors
