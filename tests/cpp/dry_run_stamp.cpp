@@ -117,6 +117,15 @@ static int runAll() {
         stampOne(std::string("rows ") + dtypeName + " standardise",
                  (x - x.reduce_mean({1})) / ((x - x.reduce_mean({1})) * (x - x.reduce_mean({1}))).reduce_mean({1}).sqrt(), inputs, stream);
         stampOne(std::string("columns ") + dtypeName + " sum of a * ln(b)", (x * y.abs().ln()).reduce_sum({0}), inputs, stream);
+        // transposed and sliced operands: LDS-tiled and broadcast-form kernels, reductions over views
+        Tensor t(gpuPlacement, TensorDescriptor(dtype, {24, 4096}));
+        const std::unordered_map<std::string, Tensor> withT{{"a", a}, {"b", b}, {"t", t}};
+        const Expression z = Expression::input("t");
+        stampOne(std::string("tiled ") + dtypeName + " exp(t^T) - a", z.transpose().exp() - x, withT, stream, "FusedKernel");
+        stampOne(std::string("tiled ") + dtypeName + " (a + t^T)^T", (x + z.transpose()).transpose() * z, withT, stream);
+        stampOne(std::string("view ") + dtypeName + " half columns", x.stridedView({4096, 12}, {24, 1}, 12).tanh() * y.stridedView({4096, 12}, {24, 1}, 0),
+                 withT, stream, "FusedKernel");
+        stampOne(std::string("view ") + dtypeName + " row sums of t^T", z.transpose().reduce_sum({1}), withT, stream);
     }
     // ragged batches: scalar and vector values, both offset dtypes, fused and index-gather paths
     for (const auto& [dtypeName, dtype] : floats) {
@@ -135,6 +144,10 @@ static int runAll() {
                          "SegmentedReduction,FusedReduction,SegmentedBroadcast,FusedKernel");
                 stampOne(tag + "mean", r.segment_mean(), inputs, stream, "SegmentedReduction");
                 stampOne(tag + "relu * exp", (r.relu() * r.exp()).getValues(), inputs, stream, "FusedKernel");
+                if (elements == 16) {
+                    stampOne(tag + "sliced gate", (r.sliceLastDimension(0, 8).exp() * r.sliceLastDimension(8, 8)).getValues(), inputs, stream, "FusedKernel");
+                    stampOne(tag + "sliced sum", r.sliceLastDimension(4, 8).segment_sum(), inputs, stream);
+                }
             }
         }
     }
