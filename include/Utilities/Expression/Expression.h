@@ -84,6 +84,9 @@ inline bool isSegmentedReduceOp(ExprOp op) {
     return op == ExprOp::SEGMENTED_REDUCE_SUM || op == ExprOp::SEGMENTED_REDUCE_MIN || op == ExprOp::SEGMENTED_REDUCE_MAX ||
            op == ExprOp::SEGMENTED_REDUCE_MEAN;
 }
+// Gradient of a min/max reduction: lhs is the reduced operand, rhs the gradient of the reduction's output; the element of each
+// reduction window that won (the first in logical order among equals) takes the window's gradient, every other element 0.
+inline bool isWinnerRoutingOp(ExprOp op) { return op == ExprOp::REDUCE_MIN_BACKWARD || op == ExprOp::REDUCE_MAX_BACKWARD; }
 // Views of the operand's storage: nothing is computed, consumers read through the view's strides.
 inline bool isStorageViewOp(ExprOp op) { return op == ExprOp::STRIDED_VIEW || op == ExprOp::TRANSPOSE; }
 inline bool isRaggedOp(ExprOp op) {

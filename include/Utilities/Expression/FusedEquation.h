@@ -42,6 +42,18 @@ class FusedEquation {
     void run(const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, float>& scalar_inputs,
              std::unordered_map<std::string, Tensor>& outputs, Stream& stream) const;
 
+    // The equation of the gradients of this equation's outputs with respect to the named tensor inputs (all of them when
+    // `wrt_names` is empty): outputs "<input>_grad", inputs the forward inputs plus one upstream gradient per forward
+    // output (named by the caller; with no name given, a single output's upstream gradient is implicit ones) and, with
+    // `accumulate_grad_outputs`, the running "<input>_grad" tensors the new gradients are added to.  The gradient graph is
+    // built when tensors are bound, since undoing broadcasts needs their shapes; names are validated here.
+    [[nodiscard]] FusedEquation compileBackward(const std::vector<std::string>& wrt_names = {},
+                                                const std::optional<std::string>& upstream_input_name = std::nullopt,
+                                                bool accumulate_grad_outputs = false) const;
+    [[nodiscard]] FusedEquation compileBackward(const std::vector<std::string>& wrt_names,
+                                                const std::unordered_map<std::string, std::string>& upstream_input_names_by_output,
+                                                bool accumulate_grad_outputs = false) const;
+
     std::vector<std::string> getOutputNames() const;
     [[nodiscard]] const PhysicalOutputs& physicalOutputs() const { return outputs_template; }
 
@@ -64,6 +76,13 @@ class FusedEquation {
     StampedExecutionPlan stampImpl(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
                                    const std::unordered_map<std::string, Tensor>& preallocated_outputs, bool fusedKernelsOnly) const;
 
+    struct BackwardRecipe;  // a backward equation before shapes are known: the forward graph and what to differentiate
+    FusedEquation(std::shared_ptr<BackwardRecipe> recipe, int device_num);
+    // the equation for the shapes and dtypes of `inputs`, and the subset of `inputs` it reads
+    std::shared_ptr<const FusedEquation> backwardFor(const std::unordered_map<std::string, Tensor>& inputs,
+                                                     std::unordered_map<std::string, Tensor>& used) const;
+
+    std::shared_ptr<BackwardRecipe> backward;  // set on equations made by compileBackward; outputs_template is empty then
     PhysicalOutputs outputs_template;
     std::vector<NamedInput> root_inputs;
     int device_num;

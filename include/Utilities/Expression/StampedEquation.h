@@ -133,7 +133,7 @@ class StampedSegmentedReductionStage {
 };
 
 struct StampedExecutionStage {
-    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction, SegmentedReduction, SegmentedBroadcast };
+    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction, SegmentedReduction, SegmentedBroadcast, ReduceMinMaxBackward };
     static std::string kindToString(Kind kind) {
         switch (kind) {
             case Kind::FusedKernel:
@@ -152,6 +152,8 @@ struct StampedExecutionStage {
                 return "SegmentedReduction";
             case Kind::SegmentedBroadcast:
                 return "SegmentedBroadcast";
+            case Kind::ReduceMinMaxBackward:
+                return "ReduceMinMaxBackward";
         }
         return "<unknown>";
     }
@@ -159,7 +161,7 @@ struct StampedExecutionStage {
     Kind kind = Kind::FusedKernel;
     std::vector<uint32_t> dependency_stage_indices;
     uint32_t gpu_num = 0;
-    std::shared_ptr<StampedEquation> kernel;
+    std::shared_ptr<StampedEquation> kernel;  // also the routing kernel of Kind::ReduceMinMaxBackward (its winners come from an ArgMinMax stage)
     std::shared_ptr<StampedReduction> reduction;
     std::shared_ptr<StampedArgMinMax> arg_minmax;
     std::shared_ptr<StampedFusedReduction> fused_reduction;

@@ -177,6 +177,13 @@ void thor_outputs_destroy(thor_outputs_t outputs);
 
 /* ---- FusedEquation (Utilities/Expression/FusedEquation.h:574-632) --------------------------------------------------------- */
 thor_fused_equation_t thor_fused_equation_compile(thor_outputs_t outputs, int device_num);
+/* FusedEquation::compileBackward (Utilities/Expression/FusedEquation.h:580-586): the equation of the gradients "<input>_grad"
+ * of `wrt_names` (all tensor inputs when num_wrt is 0).  num_upstream == 0: implicit ones as the upstream gradient of the single
+ * output.  upstream_output_names == NULL and num_upstream == 1: upstream_input_names[0] names the upstream gradient input of the
+ * single output.  Otherwise upstream_input_names[i] is the upstream gradient input of forward output upstream_output_names[i]. */
+thor_fused_equation_t thor_fused_equation_compile_backward(thor_fused_equation_t eq, const char* const* wrt_names, int num_wrt,
+                                                           const char* const* upstream_output_names, const char* const* upstream_input_names,
+                                                           int num_upstream, int accumulate_grad_outputs);
 void thor_fused_equation_destroy(thor_fused_equation_t eq);
 int thor_fused_equation_num_outputs(thor_fused_equation_t eq);
 int thor_fused_equation_output_name(thor_fused_equation_t eq, int index, char* buffer, size_t capacity);

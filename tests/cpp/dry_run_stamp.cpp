@@ -79,6 +79,25 @@ static void stampOne(const std::string& name, const Expression& e, const std::un
     ++stamped;
 }
 
+// the gradients of `e` with respect to every tensor input, for an upstream gradient of the output's shape
+static void stampBackward(const std::string& name, const Expression& e, std::unordered_map<std::string, Tensor> inputs, const Tensor& upstream, Stream& stream,
+                          const char* expectKinds = nullptr) {
+    std::printf("[ RUN  ] %s\n", name.c_str());
+    std::fflush(stdout);
+    const FusedEquation forward = FusedEquation::compile(Expression::outputs({{"y", e}}).physicalOutputs(), 0);
+    const FusedEquation backward = forward.compileBackward({}, std::string("__grad_output"));
+    std::unordered_map<std::string, Tensor> used{{"__grad_output", upstream}};
+    for (const std::string& input : e.getInputNames()) used.emplace(input, inputs.at(input));
+    StampedExecutionPlan plan = backward.stamp(used, stream);
+    std::string kinds;
+    for (const std::string& k : plan.stageKindNames()) kinds += (kinds.empty() ? "" : ",") + k;
+    if (expectKinds && kinds != expectKinds) {
+        std::printf("  unexpected plan: %s (wanted %s)\n", kinds.c_str(), expectKinds);
+        std::exit(1);
+    }
+    ++stamped;
+}
+
 static int runAll();
 
 int main() {
@@ -117,6 +136,16 @@ static int runAll() {
         stampOne(std::string("rows ") + dtypeName + " standardise",
                  (x - x.reduce_mean({1})) / ((x - x.reduce_mean({1})) * (x - x.reduce_mean({1}))).reduce_mean({1}).sqrt(), inputs, stream);
         stampOne(std::string("columns ") + dtypeName + " sum of a * ln(b)", (x * y.abs().ln()).reduce_sum({0}), inputs, stream);
+        // backward equations: gradients of fused chains, row kernels that recompute the forward value, winner routing
+        Tensor rowGradient(gpuPlacement, TensorDescriptor(dtype, {4096})), fullGradient(gpuPlacement, TensorDescriptor(dtype, {4096, 24}));
+        stampBackward(std::string("backward ") + dtypeName + " tanh(a) * b + exp(a)", x.tanh() * y + x.exp(), inputs, fullGradient, stream, "FusedKernel");
+        stampBackward(std::string("backward ") + dtypeName + " gelu(a) / softplus(b)", x.gelu() / y.softplus(), inputs, fullGradient, stream, "FusedKernel");
+        stampBackward(std::string("backward ") + dtypeName + " softmax", x.softmax(), inputs, fullGradient, stream, "FusedRowKernel");
+        stampBackward(std::string("backward ") + dtypeName + " log softmax", x.logSoftmax(), inputs, fullGradient, stream, "FusedRowKernel");
+        stampBackward(std::string("backward ") + dtypeName + " row norms of a * b", (x * y).reduce_norm2({1}, {1}), inputs, rowGradient, stream);
+        stampBackward(std::string("backward ") + dtypeName + " row max", x.reduce_max({1}, {1}), inputs, rowGradient, stream);
+        stampBackward(std::string("backward ") + dtypeName + " column min of exp", x.exp().reduce_min({0}, {}),
+                      inputs, Tensor(gpuPlacement, TensorDescriptor(dtype, {1, 24})), stream);
         // transposed and sliced operands: LDS-tiled and broadcast-form kernels, reductions over views
         Tensor t(gpuPlacement, TensorDescriptor(dtype, {24, 4096}));
         const std::unordered_map<std::string, Tensor> withT{{"a", a}, {"b", b}, {"t", t}};
@@ -143,6 +172,14 @@ static int runAll() {
                 stampOne(tag + "log softmax", r.segment_log_softmax().getValues(), inputs, stream,
                          "SegmentedReduction,FusedReduction,SegmentedBroadcast,FusedKernel");
                 stampOne(tag + "mean", r.segment_mean(), inputs, stream, "SegmentedReduction");
+                {
+                    std::vector<uint64_t> perSegment{200};
+                    if (elements > 1) perSegment.push_back(elements);
+                    stampBackward(tag + "backward of mean", r.segment_mean(), inputs, Tensor(gpuPlacement, TensorDescriptor(dtype, perSegment)), stream);
+                    stampBackward(tag + "backward of exp(sum) spread over rows",
+                                  r.getValues().exp() * Expression::segmentedBroadcast(r.segment_sum(), r.getOffsets(), 200, 6000, elements, false), inputs,
+                                  Tensor(gpuPlacement, TensorDescriptor(dtype, dims)), stream);
+                }
                 stampOne(tag + "relu * exp", (r.relu() * r.exp()).getValues(), inputs, stream, "FusedKernel");
                 if (elements == 16) {
                     stampOne(tag + "sliced gate", (r.sliceLastDimension(0, 8).exp() * r.sliceLastDimension(8, 8)).getValues(), inputs, stream, "FusedKernel");

@@ -7,6 +7,7 @@
 #include "Utilities/Common/Stream.h"
 #include "Utilities/Expression/Expression.h"
 #include "Utilities/Expression/ExpressionDTypeResolution.h"
+#include "Utilities/Expression/AutoDiff.h"
 #include "Utilities/Expression/FusedEquation.h"
 #include "Utilities/Expression/RaggedExpression.h"
 #include "Utilities/TensorOperations/Cub/CubReduction.h"
@@ -233,6 +234,47 @@ static void offsetSegmentedReductions(Stream& stream) {
     CHECK(throwsAs<std::invalid_argument>([&] { CubSegmentedReduction(CubReductionOp::Sum).stamp(x, gpuOffsets({0, 5, 10}, stream), stream); }));
 }
 
+static void autodiffGraphStructure() {
+    // buildBackwardOutputs builds gradients as one more expression graph (AutoDiff.h:15-27, AutoDiff.cpp:2486-2581 there)
+    const Expression x = Expression::input("x"), w = Expression::input("w");
+    const PhysicalOutputs forward = Expression::outputs({{"y", (x * w).tanh()}}).physicalOutputs();
+    const std::unordered_map<std::string, std::vector<uint64_t>> dims{{"x", {4, 3}}, {"w", {3}}};
+    const PhysicalOutputs backward = buildBackwardOutputs(forward, {"x", "w"}, std::string(DEFAULT_BACKWARD_UPSTREAM_INPUT_NAME), dims);
+    CHECK(backward.outputs.size() == 2 && backward.outputs[0].name == "x_grad" && backward.outputs[1].name == "w_grad");
+    CHECK((backward.expr->getInputNames() == std::set<std::string>{"x", "w", "__grad_output"}));
+    auto count = [&](ExprOp op) {
+        int n = 0;
+        for (const ExprNode& node : backward.expr->nodes) n += node.op == op;
+        return n;
+    };
+    CHECK(count(ExprOp::TANH) == 1);        // the forward value is copied once and shared by both gradients
+    CHECK(count(ExprOp::REDUCE_SUM) == 1);  // w was broadcast over rows: its gradient is summed back to [3]
+    for (const ExprNode& node : backward.expr->nodes) {
+        if (node.op == ExprOp::REDUCE_SUM) CHECK(node.reduction_axes == (std::vector<uint64_t>{0}) && node.squeeze_axes == (std::vector<uint64_t>{0}));
+    }
+    // implicit upstream: ones of the output's shape; a gradient nothing reaches is zeros of the input's shape
+    const PhysicalOutputs implicit = buildBackwardOutputs(Expression::outputs({{"y", x.exp()}, }).physicalOutputs(), {"x"}, std::nullopt, dims);
+    bool seeded = false;
+    for (const ExprNode& node : implicit.expr->nodes) seeded = seeded || (node.op == ExprOp::FILL && node.scalar_fp == 1.0 && node.fill_dims == dims.at("x"));
+    CHECK(seeded);
+    CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"x"}, std::string("w"), dims); }));        // collides with an input
+    CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"nope"}, std::nullopt, dims); }));         // unknown input
+    CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"x", "x"}, std::nullopt, dims); }));       // duplicate
+    CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"x"}, std::nullopt, std::nullopt); }));    // shapes are required
+    CHECK(throwsAs<std::runtime_error>([&] {
+        (void)buildBackwardOutputs(Expression::outputs({{"y", x.floor() * w}}).physicalOutputs(), {"x"}, std::nullopt, dims);  // no rule for floor
+    }));
+    const PhysicalOutputs two = Expression::outputs({{"a", x + w}, {"b", x - w}}).physicalOutputs();
+    CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(two, {"x"}, std::nullopt, dims); }));  // several outputs need a seed map
+    const PhysicalOutputs partial = buildBackwardOutputs(two, {"w"}, std::unordered_map<std::string, std::string>{{"b", "__gb"}}, dims);
+    CHECK((partial.expr->getInputNames() == std::set<std::string>{"__gb"}));  // d(x - w)/dw = -g, summed over rows: no forward value needed
+    // offsets of a ragged batch are structure
+    const Expression offsets = Expression::input("offsets");
+    const PhysicalOutputs ragged = Expression::outputs({{"s", Expression::segmentedReduceSum(x, offsets)}}).physicalOutputs();
+    CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(ragged, {"offsets"}, std::nullopt, {{{"x", {4, 3}}, {"offsets", {3}}}}); }));
+    CHECK((normalizeBackwardWrtNames(*ragged.expr, {}) == std::vector<std::string>{"x"}));
+}
+
 static void raggedExpressionStructure() {
     // RaggedExpressionTest.cpp:739-795,907-957,2037-2055 there: names, descriptors and markers, no device work
     const RaggedTensorDescriptor descriptor(DataType::FP32, {4}, 3, 9);
@@ -412,6 +454,51 @@ static void expressionConfig1AndRuntimeScalars(Stream& stream) {
     CHECK(throwsAs<std::runtime_error>([&] { eq2.run({{"x", x}}, out, stream); }));  // missing runtime scalar
 }
 
+static void autodiffExecution(Stream& stream) {
+    // d/dx, d/dw of sum(tanh(x * w)) with w broadcast over rows; then the same with an explicit upstream gradient
+    const std::vector<float> xv{0.5f, -1.0f, 2.0f, 1.5f, 0.25f, -0.75f}, wv{2.0f, -0.5f, 1.0f}, gv{1.0f, 2.0f, -1.0f, 0.5f, 0.0f, 3.0f};
+    const Expression x = Expression::input("x"), w = Expression::input("w");
+    const FusedEquation forward = FusedEquation::compile(Expression::outputs({{"y", (x * w).tanh()}}).physicalOutputs(), 0);
+    const std::unordered_map<std::string, Tensor> inputs{{"x", gpuFrom(xv, {2, 3}, stream)}, {"w", gpuFrom(wv, {3}, stream)}};
+    const FusedEquation implicit = forward.compileBackward({"x", "w"});
+    CHECK((implicit.getOutputNames() == std::vector<std::string>{"x_grad", "w_grad"}));
+    CHECK((implicit.getOutputShapes(inputs).at("w_grad") == std::vector<uint64_t>{3}));
+    StampedExecutionPlan plan = implicit.stamp(inputs, stream);
+    plan.run();
+    std::vector<float> gx = toHostF32(plan.output("x_grad"), stream), gw = toHostF32(plan.output("w_grad"), stream);
+    for (int r = 0; r < 2; ++r) {
+        for (int c = 0; c < 3; ++c) {
+            const double t = std::tanh(double(xv[r * 3 + c]) * wv[c]);
+            CHECK_NEAR(gx[r * 3 + c], (1 - t * t) * wv[c], 1e-6);
+        }
+    }
+    for (int c = 0; c < 3; ++c) {
+        double want = 0;
+        for (int r = 0; r < 2; ++r) {
+            const double t = std::tanh(double(xv[r * 3 + c]) * wv[c]);
+            want += (1 - t * t) * xv[r * 3 + c];
+        }
+        CHECK_NEAR(gw[c], want, 1e-6);
+    }
+    std::unordered_map<std::string, Tensor> withUpstream = inputs;
+    withUpstream.emplace("__grad_output", gpuFrom(gv, {2, 3}, stream));
+    StampedExecutionPlan seeded = forward.compileBackward({"x"}, std::string(DEFAULT_BACKWARD_UPSTREAM_INPUT_NAME)).stamp(withUpstream, stream);
+    seeded.run();
+    gx = toHostF32(seeded.output("x_grad"), stream);
+    for (int i = 0; i < 6; ++i) {
+        const double t = std::tanh(double(xv[i]) * wv[i % 3]);
+        CHECK_NEAR(gx[i], gv[i] * (1 - t * t) * wv[i % 3], 1e-6);
+    }
+    // min/max reductions hand the gradient to the first winner
+    const FusedEquation rowMax = FusedEquation::compile(Expression::outputs({{"m", x.reduce_max({1}, {1})}}).physicalOutputs(), 0);
+    StampedExecutionPlan routed = rowMax.compileBackward({"x"}).stamp({{"x", gpuFrom({1, 3, 3, 2, 2, 0}, {2, 3}, stream)}}, stream);
+    CHECK((routed.stageKindNames() == std::vector<std::string>{"FusedKernel", "ArgMinMax", "ReduceMinMaxBackward"}));
+    routed.run();
+    CHECK((toHostF32(routed.output("x_grad"), stream) == std::vector<float>{0, 1, 0, 1, 0, 0}));
+    CHECK(throwsAs<std::runtime_error>([&] { (void)forward.compileBackward({"x"}, std::string("w")); }));
+    CHECK(throwsAs<std::runtime_error>([&] { (void)implicit.compileBackward({"x"}); }));  // no second derivative of a backward equation
+}
+
 static void softmaxPlansAndRowKernel(Stream& stream) {
     const uint64_t rows = 7, cols = 130;
     std::vector<float> x(rows * cols);
@@ -490,7 +577,8 @@ int main(int argc, char** argv) {
     std::vector<Case> cases = {{"geometryPathsAndErrors", geometryPathsAndErrors},
                                {"dtypeResolutionAndStageSplit", dtypeResolutionAndStageSplit},
                                {"cpuTypeConverter", cpuTypeConverter},
-                               {"raggedExpressionStructure", raggedExpressionStructure}};
+                               {"raggedExpressionStructure", raggedExpressionStructure},
+                               {"autodiffGraphStructure", autodiffGraphStructure}};
     if (mode == "gpu") {
         auto withStream = [](void (*f)(Stream&)) {
             return [f] {
@@ -504,6 +592,7 @@ int main(int argc, char** argv) {
         cases.push_back({"raggedExpressionExecution", withStream(raggedExpressionExecution)});
         cases.push_back({"expressionConfig1AndRuntimeScalars", withStream(expressionConfig1AndRuntimeScalars)});
         cases.push_back({"softmaxPlansAndRowKernel", withStream(softmaxPlansAndRowKernel)});
+        cases.push_back({"autodiffExecution", withStream(autodiffExecution)});
         cases.push_back({"typeConverterOnGpuAndTensorViews", withStream(typeConverterOnGpuAndTensorViews)});
     }
     for (const Case& c : cases) {

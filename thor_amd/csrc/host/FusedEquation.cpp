@@ -5,14 +5,18 @@
 //  :10760-10905 convenience run).
 #include "Utilities/Expression/FusedEquation.h"
 
+#include "AutoDiffInternal.h"
 #include "HipSourceEmitter.h"
 #include "ReductionPlanner.h"
 #include "RowFusion.h"
+#include "ShapeInference.h"
+#include "WinnerRouting.h"
 #include "Utilities/Common/ScopedGpu.h"
 #include "Utilities/Expression/ExpressionDTypeResolution.h"
 
 #include <algorithm>
 #include <cstdlib>
+#include <functional>
 #include <limits>
 #include <map>
 #include <numeric>
@@ -128,8 +132,20 @@ class GraphBuilder {
             remap.emplace(srcIndex, idx);
             return idx;
         }
+        if (node.op == ExprOp::CAST) {
+            // a conversion of a computed value to the dtype it already has is that value (inputs and views keep theirs: it
+            // is what copies them into a tensor of their own)
+            const ExprNode& child = out.nodes[node.lhs];
+            if (!Expression::isLeafOp(child.op) && !isShapeOnly(child.op) && child.output_dtype == node.output_dtype) {
+                remap.emplace(srcIndex, node.lhs);
+                return node.lhs;
+            }
+        }
         if (isReductionOp(node.op) || isSegmentedReduceOp(node.op)) {
             node.lhs = asTensorOperand(node.lhs, true);
+        } else if (isWinnerRoutingOp(node.op)) {
+            node.lhs = asTensorOperand(node.lhs, true);  // read by an arg reduction
+            node.rhs = asTensorOperand(node.rhs, false);
         } else if (node.op == ExprOp::SEGMENTED_BROADCAST) {
             node.lhs = asTensorOperand(node.lhs, false);
         } else if (isShapeOnly(node.op)) {
@@ -195,7 +211,9 @@ uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
 // Can the consumer read a per-segment value through the segment index?  Only work that ends up inside a flat fused kernel.
 bool consumesGather(const ExprNode& consumer) {
     if (consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT || consumer.op == ExprOp::WHERE || consumer.op == ExprOp::CAST) return true;
-    if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX) return false;
+    if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX || isWinnerRoutingOp(consumer.op)) {
+        return false;
+    }
     return Expression::isBinaryOp(consumer.op) || Expression::isUnaryOp(consumer.op);
 }
 
@@ -236,13 +254,16 @@ std::vector<uint64_t> reshapeDims(const std::vector<uint64_t>& in, const std::ve
 
 std::vector<uint64_t> sortedAxesOrAll(const std::vector<uint64_t>& axes, size_t rank) { return resolveReductionAxes(axes, rank); }
 
-std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std::vector<Tensor>& boundInputs) {
-    std::vector<std::vector<uint64_t>> dims(g.expr.nodes.size());
-    for (uint32_t i = 0; i < g.expr.nodes.size(); ++i) {
-        const ExprNode& n = g.expr.nodes[i];
+}  // namespace
+
+std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpression& expr,
+                                                           const std::function<std::vector<uint64_t>(uint32_t)>& inputDims) {
+    std::vector<std::vector<uint64_t>> dims(expr.nodes.size());
+    for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
+        const ExprNode& n = expr.nodes[i];
         switch (n.op) {
             case ExprOp::INPUT:
-                dims[i] = boundInputs.at(n.input_slot).getDimensions();
+                dims[i] = inputDims(n.input_slot);
                 break;
             case ExprOp::RUNTIME_SCALAR:
             case ExprOp::SCALAR_FP:
@@ -310,6 +331,18 @@ std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std:
                 dims[i][0] = n.ragged_runtime_max_active_values;
                 break;
             }
+            case ExprOp::REDUCE_MIN_BACKWARD:
+            case ExprOp::REDUCE_MAX_BACKWARD: {
+                // operand-shaped; the gradient holds one element per reduction window
+                const std::vector<uint64_t> windows = StampedEquation::computeReductionOutputDims(
+                    dims[n.lhs], sortedAxesOrAll(n.reduction_axes, dims[n.lhs].size()), n.squeeze_axes);
+                uint64_t expected = 1, got = 1;
+                for (uint64_t d : windows) expected *= d;
+                for (uint64_t d : dims[n.rhs]) got *= d;
+                if (expected != got) throw std::runtime_error("Min/max reduction backward: the gradient does not have the reduction's output shape.");
+                dims[i] = dims[n.lhs];
+                break;
+            }
             default:
                 if (isReductionOp(n.op)) {
                     const std::vector<uint64_t> axes = sortedAxesOrAll(n.reduction_axes, dims[n.lhs].size());
@@ -324,6 +357,12 @@ std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std:
         }
     }
     return dims;
+}
+
+namespace {
+
+std::vector<std::vector<uint64_t>> inferShapes(const PlannedGraph& g, const std::vector<Tensor>& boundInputs) {
+    return inferExpressionShapes(g.expr, [&](uint32_t slot) { return boundInputs.at(slot).getDimensions(); });
 }
 
 std::vector<uint64_t> orScalarShape(const std::vector<uint64_t>& dims) { return dims.empty() ? std::vector<uint64_t>{1} : dims; }
@@ -444,7 +483,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             } else if (isReductionOp(n.op)) {
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
-            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
+            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(n.op)) {
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
                 ensureTensor(n.rhs);
@@ -525,6 +564,9 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             std::vector<uint32_t> sources, scalars;
             if (isReductionOp(graph->expr.nodes[i].op)) {
                 sources.push_back(graph->expr.nodes[i].lhs);
+            } else if (isWinnerRoutingOp(graph->expr.nodes[i].op)) {
+                sources.push_back(graph->expr.nodes[i].lhs);
+                sources.push_back(graph->expr.nodes[i].rhs);
             } else if (isSegmentedReduceOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST) {
                 const uint32_t operand = graph->expr.nodes[i].lhs;
                 if (graph->role[operand] == Role::Inline) {
@@ -574,6 +616,11 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                                               const std::unordered_map<std::string, Tensor>& preallocated, bool fusedKernelsOnly) const {
     if (!stream.isInitialized()) throw std::runtime_error("FusedEquation::stamp requires an initialized stream.");
     if (stream.getGpuNum() != device_num) throw std::runtime_error("FusedEquation::stamp: the stream belongs to another GPU than the equation.");
+    if (backward) {
+        std::unordered_map<std::string, Tensor> used;
+        const std::shared_ptr<const FusedEquation> equation = backwardFor(inputs, used);
+        return equation->stampImpl(used, stream, preallocated, fusedKernelsOnly);
+    }
     const std::vector<DataType> dtypes = rootDTypes(inputs);
     const std::shared_ptr<PlannedGraph> graph = plannedGraphFor(dtypes);
     const PhysicalExpression& expr = graph->expr;
@@ -1013,6 +1060,46 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 done[i] = 1;
                 continue;
             }
+            if (isWinnerRoutingOp(n.op)) {
+                if (fusedKernelsOnly) {
+                    throw std::runtime_error(
+                        "FusedEquation::run() only supports expressions that lower to fused kernels; this expression has a reduction stage. "
+                        "Use stamp() and run the returned plan.");
+                }
+                // winners of the forward reduction (an index per window), then one pass that spreads the gradient
+                const Tensor& operand = tensorOf[n.lhs];
+                const std::vector<uint64_t> axes64 = sortedAxesOrAll(n.reduction_axes, dims[n.lhs].size());
+                std::vector<uint32_t> axes(axes64.begin(), axes64.end());
+                CubArgReductionOutputOptions options;
+                options.produce_value = false;
+                options.produce_index = true;
+                options.index_output_dtype = DataType::UINT32;
+                const CubArgReduction reduction(n.op == ExprOp::REDUCE_MAX_BACKWARD ? CubArgReductionOp::ArgMax : CubArgReductionOp::ArgMin, axes, options);
+                Tensor winners(gpuPlacement, TensorDescriptor(DataType::UINT32, StampedEquation::computeReductionOutputDims(dims[n.lhs], axes64, {})));
+                StampedExecutionStage find;
+                find.kind = StampedExecutionStage::Kind::ArgMinMax;
+                find.gpu_num = device_num;
+                find.dependency_stage_indices = dependenciesOf({n.lhs});
+                find.arg_minmax = std::make_shared<StampedArgMinMax>(reduction.stamp(operand, std::nullopt, winners, stream));
+                const uint32_t findStage = static_cast<uint32_t>(stages.size());
+                stages.push_back(std::move(find));
+
+                Tensor gradient = tensorOf[n.rhs];
+                if (!gradient.isDenseContiguous()) throw std::runtime_error("Min/max reduction backward needs a dense gradient tensor.");
+                Tensor routed = allocateFor(i);
+                StampedExecutionStage spread;
+                spread.kind = StampedExecutionStage::Kind::ReduceMinMaxBackward;
+                spread.gpu_num = device_num;
+                spread.dependency_stage_indices = dependenciesOf({n.rhs});
+                spread.dependency_stage_indices.push_back(findStage);
+                std::sort(spread.dependency_stage_indices.begin(), spread.dependency_stage_indices.end());
+                spread.kernel = stampWinnerRouting(winners, gradient, routed, dims[n.lhs], axes64, device_num);
+                tensorOf[i] = routed;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(spread));
+                done[i] = 1;
+                continue;
+            }
             if (!isReductionOp(n.op)) {
                 // kernels of ragged values stop at the partition's last row, so they are grouped by partition as well
                 std::vector<uint64_t> key = orScalarShape(dims[i]);
@@ -1086,6 +1173,110 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     return StampedExecutionPlan(std::move(stages), std::move(finalOutputs), stream);
 }
 
+// ---- backward equations -------------------------------------------------------------------------------------------------------------
+struct FusedEquation::BackwardRecipe {
+    PhysicalOutputs forward;
+    std::vector<std::string> wrt;
+    std::optional<std::unordered_map<std::string, std::string>> upstreamByOutput;
+    bool accumulate = false;
+    // shapes and dtypes of the forward inputs -> the equation differentiated for them
+    LruCacheThreadSafe<std::string, std::shared_ptr<const FusedEquation>> specialised{64};
+};
+
+FusedEquation::FusedEquation(std::shared_ptr<BackwardRecipe> recipe, int device_num)
+    : backward(std::move(recipe)),
+      device_num(device_num),
+      planned_graph_cache(std::make_shared<LruCacheThreadSafe<std::string, std::shared_ptr<PlannedGraph>>>(1)) {
+    // what may be bound: the forward inputs, the upstream gradients and the running gradients; what is produced
+    root_inputs = backward->forward.expr->inputs;
+    auto addInput = [&](const std::string& name) {
+        for (const NamedInput& in : root_inputs)
+            if (in.name == name) return;
+        root_inputs.push_back(NamedInput{name, static_cast<uint32_t>(root_inputs.size()), NamedInput::Kind::Tensor});
+    };
+    if (backward->upstreamByOutput.has_value()) {
+        for (const NamedOutput& o : backward->forward.outputs) {
+            auto it = backward->upstreamByOutput->find(o.name);
+            if (it != backward->upstreamByOutput->end()) addInput(it->second);
+        }
+    }
+    for (const std::string& name : backward->wrt) {
+        if (backward->accumulate) addInput(name + "_grad");
+        outputs_template.outputs.push_back(NamedOutput{name + "_grad", UINT32_MAX});
+    }
+}
+
+FusedEquation FusedEquation::compileBackward(const std::vector<std::string>& wrt_names, const std::optional<std::string>& upstream_input_name,
+                                             bool accumulate_grad_outputs) const {
+    if (backward) throw std::runtime_error("compileBackward of a backward equation is not supported.");
+    auto recipe = std::make_shared<BackwardRecipe>();
+    recipe->forward = outputs_template;
+    recipe->wrt = normalizeBackwardWrtNames(*outputs_template.expr, wrt_names);
+    recipe->upstreamByOutput = normalizeBackwardUpstreamNames(outputs_template, upstream_input_name);
+    recipe->accumulate = accumulate_grad_outputs;
+    if (outputs_template.outputs.size() > 1 && !recipe->upstreamByOutput.has_value()) {
+        throw std::runtime_error(
+            "buildBackwardOutputs for multi-output forward equations requires an explicit upstream seed map. The map may be partial when "
+            "some outputs have no incoming gradient.");
+    }
+    return FusedEquation(std::move(recipe), device_num);
+}
+
+FusedEquation FusedEquation::compileBackward(const std::vector<std::string>& wrt_names,
+                                             const std::unordered_map<std::string, std::string>& upstream_input_names_by_output,
+                                             bool accumulate_grad_outputs) const {
+    if (backward) throw std::runtime_error("compileBackward of a backward equation is not supported.");
+    auto recipe = std::make_shared<BackwardRecipe>();
+    recipe->forward = outputs_template;
+    recipe->wrt = normalizeBackwardWrtNames(*outputs_template.expr, wrt_names);
+    recipe->upstreamByOutput = normalizeBackwardUpstreamNames(outputs_template, upstream_input_names_by_output);
+    if (recipe->upstreamByOutput->empty()) {
+        throw std::runtime_error("buildBackwardOutputs explicit upstream seed map must contain at least one forward output.");
+    }
+    recipe->accumulate = accumulate_grad_outputs;
+    return FusedEquation(std::move(recipe), device_num);
+}
+
+std::shared_ptr<const FusedEquation> FusedEquation::backwardFor(const std::unordered_map<std::string, Tensor>& inputs,
+                                                                std::unordered_map<std::string, Tensor>& used) const {
+    const PhysicalExpression& forward = *backward->forward.expr;
+    for (const auto& [name, tensor] : inputs) {
+        (void)tensor;
+        bool known = false;
+        for (const NamedInput& in : root_inputs) known = known || in.name == name;
+        if (!known) throw std::runtime_error("Unexpected input tensor for this equation: " + name);
+    }
+    // the forward inputs fix the shapes and dtypes the gradients are built for
+    std::string key;
+    std::vector<DataType> dtypes(forward.inputs.size(), DataType::FP32);
+    std::unordered_map<std::string, std::vector<uint64_t>> dimsByName;
+    for (const NamedInput& in : forward.inputs) {
+        if (in.kind == NamedInput::Kind::RuntimeScalarFp32) continue;
+        auto it = inputs.find(in.name);
+        if (it == inputs.end()) throw std::runtime_error("Missing required input tensor: " + in.name);
+        if (!it->second.isInitialized()) throw std::runtime_error("Input tensor is not initialized: " + in.name);
+        dtypes[in.slot] = it->second.getDataType();
+        dimsByName[in.name] = it->second.getDimensions();
+        key += in.name + ":" + std::to_string(static_cast<int>(dtypes[in.slot])) + ":" + axesKey(it->second.getDimensions()) + ";";
+    }
+    const std::shared_ptr<const FusedEquation> equation = backward->specialised.getOrCreate(key, [&] {
+        PhysicalOutputs typed;
+        typed.expr = std::make_shared<PhysicalExpression>(forward);
+        typed.outputs = backward->forward.outputs;
+        resolveOutputsDTypesInPlace(typed, dtypes);
+        const PhysicalOutputs gradients =
+            buildBackwardOutputsTyped(backward->forward, *typed.expr, backward->wrt, backward->upstreamByOutput, dimsByName, backward->accumulate);
+        return std::shared_ptr<const FusedEquation>(new FusedEquation(compile(gradients, device_num)));
+    });
+    for (const NamedInput& in : equation->root_inputs) {
+        if (in.kind == NamedInput::Kind::RuntimeScalarFp32) continue;
+        auto it = inputs.find(in.name);
+        if (it == inputs.end()) throw std::runtime_error("Missing required input tensor: " + in.name);
+        used.emplace(in.name, it->second);
+    }
+    return equation;
+}
+
 // ---- convenience run ---------------------------------------------------------------------------------------------------------------
 void FusedEquation::run(const Tensor& input, Tensor& output, Stream& stream) const {
     if (root_inputs.size() != 1) throw std::runtime_error("run(input, output) requires an equation with exactly one input.");
@@ -1126,6 +1317,11 @@ void FusedEquation::run(const std::unordered_map<std::string, Tensor>& inputs, c
 
 // ---- shape / dtype queries -----------------------------------------------------------------------------------------------------------
 std::unordered_map<std::string, std::vector<uint64_t>> FusedEquation::getOutputShapes(const std::unordered_map<std::string, Tensor>& inputs) const {
+    if (backward) {
+        std::unordered_map<std::string, Tensor> used;
+        const std::shared_ptr<const FusedEquation> equation = backwardFor(inputs, used);
+        return equation->getOutputShapes(used);
+    }
     const std::shared_ptr<PlannedGraph> graph = plannedGraphFor(rootDTypes(inputs));
     std::vector<Tensor> bound(root_inputs.size());
     for (const NamedInput& in : root_inputs)
@@ -1152,6 +1348,11 @@ std::vector<uint64_t> FusedEquation::getOutputShape(const Tensor& input) const {
 }
 
 std::unordered_map<std::string, DataType> FusedEquation::getOutputDataTypes(const std::unordered_map<std::string, Tensor>& inputs) const {
+    if (backward) {
+        std::unordered_map<std::string, Tensor> used;
+        const std::shared_ptr<const FusedEquation> equation = backwardFor(inputs, used);
+        return equation->getOutputDataTypes(used);
+    }
     const std::shared_ptr<PlannedGraph> graph = plannedGraphFor(rootDTypes(inputs));
     std::unordered_map<std::string, DataType> out;
     for (const NamedOutput& o : graph->outputs) out.emplace(o.name, graph->expr.nodes[o.node_idx].output_dtype.value());

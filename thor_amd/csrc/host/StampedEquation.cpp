@@ -157,6 +157,7 @@ uint64_t StampedExecutionStage::flopCount() const {
     switch (kind) {
         case Kind::FusedKernel:
         case Kind::FusedRowKernel:
+        case Kind::ReduceMinMaxBackward:
             return kernel ? kernel->flopCount() : 0;
         case Kind::Reduction:
             return reduction ? reduction->flopCount() : 0;
@@ -178,6 +179,7 @@ void StampedExecutionStage::runOn(Stream& stream, const std::unordered_map<std::
     switch (kind) {
         case Kind::FusedKernel:
         case Kind::FusedRowKernel:
+        case Kind::ReduceMinMaxBackward:
             if (!kernel) throw std::runtime_error("Fused execution stage is missing its stamped kernel.");
             kernel->runOn(stream, runtime_scalars);
             return;

@@ -215,6 +215,21 @@ void thor_outputs_destroy(thor_outputs_t outputs) { delete outputs; }
 thor_fused_equation_t thor_fused_equation_compile(thor_outputs_t outputs, int device_num) {
     THOR_CAPI_TRY_PTR(require(outputs, "outputs"); return new thor_fused_equation{FusedEquation::compile(outputs->outputs.physicalOutputs(), device_num)};)
 }
+thor_fused_equation_t thor_fused_equation_compile_backward(thor_fused_equation_t eq, const char* const* wrt_names, int num_wrt,
+                                                           const char* const* upstream_output_names, const char* const* upstream_input_names,
+                                                           int num_upstream, int accumulate_grad_outputs) {
+    THOR_CAPI_TRY_PTR(
+        require(eq, "equation"); std::vector<std::string> wrt; for (int i = 0; i < num_wrt; ++i) wrt.emplace_back(wrt_names[i]);
+        if (num_upstream == 0) return new thor_fused_equation{eq->equation.compileBackward(wrt, std::nullopt, accumulate_grad_outputs != 0)};
+        if (!upstream_input_names) throw std::invalid_argument("upstream_input_names is null");
+        if (!upstream_output_names) {
+            if (num_upstream != 1) throw std::invalid_argument("a single upstream input name needs num_upstream == 1");
+            return new thor_fused_equation{eq->equation.compileBackward(wrt, std::string(upstream_input_names[0]), accumulate_grad_outputs != 0)};
+        }
+        std::unordered_map<std::string, std::string> byOutput;
+        for (int i = 0; i < num_upstream; ++i) byOutput[upstream_output_names[i]] = upstream_input_names[i];
+        return new thor_fused_equation{eq->equation.compileBackward(wrt, byOutput, accumulate_grad_outputs != 0)};)
+}
 void thor_fused_equation_destroy(thor_fused_equation_t eq) { delete eq; }
 int thor_fused_equation_num_outputs(thor_fused_equation_t eq) { return eq ? static_cast<int>(eq->equation.getOutputNames().size()) : -1; }
 int thor_fused_equation_output_name(thor_fused_equation_t eq, int index, char* buffer, size_t capacity) {

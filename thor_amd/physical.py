@@ -77,6 +77,7 @@ PROTOTYPES = {
     "thor_expr_num_nodes": (_i, [_vp]), "thor_expr_canonical": (_i, [_vp, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_outputs_create": (_vp, [_cpp, _vpp, _i]), "thor_outputs_destroy": (None, [_vp]),
     "thor_fused_equation_compile": (_vp, [_vp, _i]), "thor_fused_equation_destroy": (None, [_vp]),
+    "thor_fused_equation_compile_backward": (_vp, [_vp, _cpp, _i, _cpp, _cpp, _i, _i]),
     "thor_fused_equation_num_outputs": (_i, [_vp]), "thor_fused_equation_output_name": (_i, [_vp, _i, _cp, _sz]),
     "thor_fused_equation_stamp": (_vp, [_vp, _cpp, _vpp, _i, _cpp, _vpp, _i, _vp]),
     "thor_fused_equation_run": (_i, [_vp, _cpp, _vpp, _i, _cpp, _fp, _i, _cpp, _vpp, _i, _vp]),
@@ -818,6 +819,28 @@ class FusedEquation:
             _check(lib().thor_fused_equation_output_name(self._h, i, buf, 256), "getOutputNames")
             out.append(buf.value.decode())
         return out
+
+    def compile_backward(self, wrt_names: Optional[List[str]] = None,
+                         error_input_name: Union[None, str, Dict[str, str]] = None, accumulate_grad_outputs: bool = False) -> "FusedEquation":
+        """Equation of the gradients ``<input>_grad`` of ``wrt_names`` (all tensor inputs when empty).
+
+        ``error_input_name`` names the upstream gradient input of a single-output equation, or maps forward output names to
+        upstream gradient input names; None means implicit ones for a single output.  (reference:
+        bindings/python/src/core/physical/expression.cpp:2638-2720)
+        """
+        wrt = list(wrt_names or [])
+        if isinstance(error_input_name, dict):
+            if len(error_input_name) == 0:
+                raise RuntimeError("Cannot compute backward expression with no error inputs.")
+            outs = list(error_input_name)
+            ptr = lib().thor_fused_equation_compile_backward(self._h, _names(wrt), len(wrt), _names(outs), _names([error_input_name[o] for o in outs]),
+                                                             len(outs), int(accumulate_grad_outputs))
+        elif error_input_name is None:
+            ptr = lib().thor_fused_equation_compile_backward(self._h, _names(wrt), len(wrt), None, None, 0, int(accumulate_grad_outputs))
+        else:
+            ptr = lib().thor_fused_equation_compile_backward(self._h, _names(wrt), len(wrt), None, _names([error_input_name]), 1,
+                                                             int(accumulate_grad_outputs))
+        return FusedEquation(_handle(ptr, "FusedEquation.compile_backward"))
 
     def stamp(self, inputs: Dict[str, PhysicalTensor], stream: Stream, preallocated_outputs: Optional[Dict[str, PhysicalTensor]] = None) -> Equation:
         names = list(inputs)
