@@ -273,6 +273,36 @@ def bench_other_configs():
               ">".join(plans[0].stage_kind_names()) + " " + " | ".join(plans[0].stage_descriptions()))
         del plans
     os.environ.pop("THOR_DISABLE_STAGE_FUSION", None)
+    del values, sums, args, per_segment, block
+
+    # ---- backward equations (compile_backward): bytes counted are every operand and the upstream gradient read once and every
+    # gradient written once
+    n = 1 << 26
+    fill = gpu_from(rng.uniform(0.5, 1.5, 1 << 22).astype(np.float32), DataType.fp32)
+    tensors = {}
+    for k in ("a", "b", "c", "d", "__grad_output"):
+        t = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [n]))
+        for off in range(0, n, 1 << 22):
+            _lib.check(_lib.load().thorhip_memcpy_async(t.mem_ptr() + off * 4, fill.mem_ptr(), 4 << 22, 3, stream.handle), "d2d")
+        tensors[k] = t
+    stream.synchronize()
+    ea, eb, ec, ed = (ex.input(k) for k in "abcd")
+    plan = ex.compile((ea * eb + ec) * ed.sigmoid(), 0).compile_backward(["a", "b", "c", "d"], error_input_name="__grad_output").stamp(tensors, stream)
+    timed("backward_c1_four_gradients_fp32_2^26", plan.run, 36 * n, n, ">".join(plan.stage_kind_names()) + " " + plan.stage_descriptions()[0])
+    del tensors, plan, fill
+    xs = gpu_from((rng.standard_normal((16384, 4096), dtype=np.float32) * 3), DataType.bf16)
+    gs = gpu_from(rng.standard_normal((16384, 4096), dtype=np.float32), DataType.bf16)
+    n = 16384 * 4096
+    pairs = [(xs, gs), (clone(xs), clone(gs)), (clone(xs), clone(gs))]
+    soft_backward = ex.compile(ex.input("x").softmax(), 0).compile_backward(["x"], error_input_name="__grad_output")
+    plans = [soft_backward.stamp({"x": a_, "__grad_output": g_}, stream) for a_, g_ in pairs]
+    timed("backward_c4_softmax_bf16", [p_.run for p_ in plans], 6 * n, n, ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
+    del xs, gs, pairs, plans
+    x = gpu_from(rng.standard_normal((8192, 8192), dtype=np.float32), DataType.fp32)
+    n = 8192 * 8192
+    row_max_backward = ex.compile(ex.input("x").reduce_max(axis=1, squeeze=[1]), 0).compile_backward(["x"])
+    plans = [row_max_backward.stamp({"x": t}, stream) for t in (x, clone(x), clone(x))]
+    timed("backward_c3_row_max_fp32", [p_.run for p_ in plans], 8 * n, n, ">".join(plans[0].stage_kind_names()) + " " + " | ".join(plans[0].stage_descriptions()))
     return results
 
 

@@ -695,9 +695,61 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     };
 
     // ---- stages in level order -----------------------------------------------------------------------------------------
+    // Elementwise values are grouped into kernels by shape (and ragged extent).  With the shapes known, a stored value that
+    // another value of the same group reads directly need not come back from memory: both run in one kernel, which keeps the
+    // producer's value in registers and stores it as well.  That holds when the stored value is the computed one (storage
+    // dtype = arithmetic dtype) and the consumer does not read it through a view.
+    auto groupKeyOf = [&](uint32_t i) {
+        const ExprNode& n = expr.nodes[i];
+        std::vector<uint64_t> key = orScalarShape(dims[i]);
+        if (n.op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
+            // kernels of ragged values stop at the partition's last row, so they are grouped by partition as well
+            key.push_back(UINT64_MAX);
+            key.push_back(n.rhs);
+            key.push_back(n.ragged_runtime_batch_size);
+            key.push_back(n.ragged_runtime_elements_per_value);
+        }
+        return key;
+    };
+    auto runsInFusedKernel = [&](uint32_t i) {
+        const ExprOp op = expr.nodes[i].op;
+        return graph->role[i] == Role::Materialized && !isReductionOp(op) && !isSegmentedReduceOp(op) && op != ExprOp::SEGMENTED_BROADCAST &&
+               !isWinnerRoutingOp(op) && op != ExprOp::INPUT;
+    };
+    std::vector<uint32_t> levelOf = graph->level;
+    if (stageFusionEnabled()) {
+        for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
+            if (graph->role[i] != Role::Materialized) continue;
+            const ExprNode& n = expr.nodes[i];
+            std::vector<uint32_t> sources, scalars;
+            if (isReductionOp(n.op)) {
+                sources.push_back(n.lhs);
+            } else if (isWinnerRoutingOp(n.op)) {
+                sources = {n.lhs, n.rhs};
+            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
+                if (graph->role[n.lhs] == Role::Inline) {
+                    collectSources(*graph, n.lhs, sources, scalars);
+                } else {
+                    sources.push_back(n.lhs);
+                }
+                sources.push_back(n.rhs);
+            } else {
+                collectSources(*graph, i, sources, scalars);
+            }
+            uint32_t level = 0;
+            for (uint32_t s : sources) {
+                const uint32_t base = baseOfView(*graph, s);
+                if (graph->role[base] != Role::Materialized) continue;
+                const bool sameKernel = s == base && runsInFusedKernel(i) && runsInFusedKernel(base) && groupKeyOf(base) == groupKeyOf(i) &&
+                                        expr.nodes[base].output_dtype.value() == emittedValueDType(expr.nodes[base]);
+                level = std::max(level, levelOf[base] + (sameKernel ? 0 : 1));
+            }
+            levelOf[i] = level;
+        }
+    }
     uint32_t maxLevel = 0;
     for (uint32_t i = 0; i < expr.nodes.size(); ++i)
-        if (graph->role[i] == Role::Materialized) maxLevel = std::max(maxLevel, graph->level[i]);
+        if (graph->role[i] == Role::Materialized) maxLevel = std::max(maxLevel, levelOf[i]);
 
     for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
         if (graph->role[i] == Role::InputSource) tensorOf[i] = bound[expr.nodes[i].input_slot];
@@ -773,6 +825,12 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
         }
         std::sort(sources.begin(), sources.end());
         sources.erase(std::unique(sources.begin(), sources.end()), sources.end());
+        // a value this kernel computes itself is used from registers (its own sources are listed through its membership)
+        sources.erase(std::remove_if(sources.begin(), sources.end(),
+                                     [&](uint32_t s) {
+                                         return graph->role[s] == Role::Materialized && !done[s] && std::find(nodes.begin(), nodes.end(), s) != nodes.end();
+                                     }),
+                      sources.end());
         std::sort(scalarSlots.begin(), scalarSlots.end());
         scalarSlots.erase(std::unique(scalarSlots.begin(), scalarSlots.end()), scalarSlots.end());
 
@@ -1023,7 +1081,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
         // fused values of this level, grouped by output shape so that one kernel shares the loads
         std::map<std::vector<uint64_t>, std::vector<uint32_t>> fusedGroups;
         for (uint32_t i = 0; i < expr.nodes.size(); ++i) {
-            if (graph->role[i] != Role::Materialized || graph->level[i] != level || done[i]) continue;
+            if (graph->role[i] != Role::Materialized || levelOf[i] != level || done[i]) continue;
             const ExprNode& n = expr.nodes[i];
             if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
                 if (fusedKernelsOnly) {
@@ -1101,15 +1159,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 continue;
             }
             if (!isReductionOp(n.op)) {
-                // kernels of ragged values stop at the partition's last row, so they are grouped by partition as well
-                std::vector<uint64_t> key = orScalarShape(dims[i]);
-                if (n.op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
-                    key.push_back(UINT64_MAX);
-                    key.push_back(n.rhs);
-                    key.push_back(n.ragged_runtime_batch_size);
-                    key.push_back(n.ragged_runtime_elements_per_value);
-                }
-                fusedGroups[key].push_back(i);
+                fusedGroups[groupKeyOf(i)].push_back(i);
                 continue;
             }
             if (fusedKernelsOnly) {
