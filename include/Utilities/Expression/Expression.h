@@ -332,6 +332,11 @@ class Expression {
     }
     // The last two axes exchanged (rank >= 2), as a view.
     Expression transpose() const;
+    // Gather along one axis (the last one for axis = -1): the result has the shape of `indices` (UINT32 / UINT64), which
+    // matches this tensor on every other axis; result[c] = this[c with the axis coordinate replaced by indices[c]]
+    // (Expression.h:676-677, Expression.cpp:3856-3865 there).  The axis is kept in reduction_axes ({UINT64_MAX} = last).
+    Expression takeAlongAxis(const Expression& indices, int64_t axis = -1) const;
+    static Expression takeAlongAxis(const Expression& input, const Expression& indices, int64_t axis = -1) { return input.takeAlongAxis(indices, axis); }
 
     // ---- reductions: fp32 accumulation, reduced axes kept as 1 unless listed in squeeze_axes ------------------------
     Expression reduction(ExprOp op, const std::vector<uint64_t>& reduction_axes, const std::vector<uint64_t>& squeeze_axes,

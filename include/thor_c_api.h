@@ -164,6 +164,8 @@ thor_expr_t thor_expr_reduce(const char* method, thor_expr_t input, const uint64
                              int num_squeeze_axes);
 /* Expression::stridedView: dims / strides / offset in elements of the operand's storage ("transpose" is a unary method). */
 thor_expr_t thor_expr_strided_view(thor_expr_t input, const uint64_t* dims, const uint64_t* strides, int rank, uint64_t element_offset);
+/* Expression::takeAlongAxis(indices, axis) (Expression.h:676-677 there); axis = -1 is the last axis */
+thor_expr_t thor_expr_take_along_axis(thor_expr_t input, thor_expr_t indices, int64_t axis);
 thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank);
 thor_expr_t thor_expr_unsqueeze(thor_expr_t input, const uint64_t* axes, int num_axes);
 thor_expr_t thor_expr_squeeze(thor_expr_t input, const uint64_t* axes, int num_axes);

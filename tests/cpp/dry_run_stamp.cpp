@@ -146,6 +146,9 @@ static int runAll() {
         stampBackward(std::string("backward ") + dtypeName + " row max", x.reduce_max({1}, {1}), inputs, rowGradient, stream);
         stampBackward(std::string("backward ") + dtypeName + " column min of exp", x.exp().reduce_min({0}, {}),
                       inputs, Tensor(gpuPlacement, TensorDescriptor(dtype, {1, 24})), stream);
+        // gathers along an axis, with indices the same equation computes
+        stampOne(std::string("gather ") + dtypeName + " value at the row argmax", (x * y).takeAlongAxis(x.argmax({1}, {}), 1), inputs, stream);
+        stampOne(std::string("gather ") + dtypeName + " column picks", x.takeAlongAxis(y.argmin({0}, {}), 0) + 1.0, inputs, stream);
         // transposed and sliced operands: LDS-tiled and broadcast-form kernels, reductions over views
         Tensor t(gpuPlacement, TensorDescriptor(dtype, {24, 4096}));
         const std::unordered_map<std::string, Tensor> withT{{"a", a}, {"b", b}, {"t", t}};

@@ -268,6 +268,19 @@ static void autodiffGraphStructure() {
     CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(two, {"x"}, std::nullopt, dims); }));  // several outputs need a seed map
     const PhysicalOutputs partial = buildBackwardOutputs(two, {"w"}, std::unordered_map<std::string, std::string>{{"b", "__gb"}}, dims);
     CHECK((partial.expr->getInputNames() == std::set<std::string>{"__gb"}));  // d(x - w)/dw = -g, summed over rows: no forward value needed
+    // take_along_axis is an index-aware binary op: the axis rides in reduction_axes, indices must be integral
+    // (ExpressionConvenienceOpsTest.cpp:357-383 there)
+    PhysicalOutputs take = Expression::outputs({{"y", x.takeAlongAxis(w, 1)}}).physicalOutputs();
+    const ExprNode& takeNode = take.expr->nodes.at(take.outputs[0].node_idx);
+    CHECK(takeNode.op == ExprOp::TAKE_ALONG_AXIS && takeNode.reduction_axes == (std::vector<uint64_t>{1}));
+    CHECK(take.expr->nodes.at(takeNode.lhs).op == ExprOp::INPUT && take.expr->nodes.at(takeNode.rhs).op == ExprOp::INPUT);
+    CHECK(throwsAs<std::runtime_error>([&] {
+        PhysicalOutputs floatIndices = Expression::outputs({{"y", x.takeAlongAxis(w, 1)}}).physicalOutputs();
+        resolveOutputsDTypesInPlace(floatIndices, {DataType::FP32, DataType::FP32});
+    }));
+    resolveOutputsDTypesInPlace(take, {DataType::FP16, DataType::UINT32});
+    CHECK(take.expr->nodes.at(take.outputs[0].node_idx).output_dtype == DataType::FP16);
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)x.takeAlongAxis(w, -2); }));
     // offsets of a ragged batch are structure
     const Expression offsets = Expression::input("offsets");
     const PhysicalOutputs ragged = Expression::outputs({{"s", Expression::segmentedReduceSum(x, offsets)}}).physicalOutputs();

@@ -86,3 +86,61 @@ def test_ragged_kernel_over_a_slice_of_the_packed_values(stream, dtype):
     want[:700] = (1.0 / (1.0 + np.exp(-xf[:700, :width].astype(np.float64)))) * xf[:700, width:]
     np.testing.assert_allclose(got, want, rtol=0, atol=1e-5 if dtype == DataType.fp32 else 3e-2)
     assert np.all(got[700:] == -3.0)
+
+
+# ---- take_along_axis (ExpressionConvenienceOpsTest.cpp:357-409 there) ---------------------------------------------------------------
+def test_take_along_axis_known_answers(stream):
+    values = copy_numpy_to_gpu(np.array([[10, 11, 12, 13], [20, 21, 22, 23]], np.float32), stream, DataType.fp32)
+    indices = copy_numpy_to_gpu(np.array([[3, 0, 2], [1, 1, 0]], np.uint32), stream, DataType.uint32)
+    plan = run({"y": ex.input("values").take_along_axis(ex.input("indices"))}, {"values": values, "indices": indices}, stream)
+    assert plan.output("y").get_dimensions() == [2, 3] and plan.stage_kind_names() == ["FusedKernel"]
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("y"), stream), [[13, 10, 12], [21, 21, 20]])
+    values = copy_numpy_to_gpu(np.array([[1, 2], [3, 4], [5, 6]], np.float32), stream, DataType.fp32)
+    indices = copy_numpy_to_gpu(np.array([[2, 0], [0, 1]], np.uint32), stream, DataType.uint32)
+    plan = run({"y": ex.input("values").take_along_axis(ex.input("indices"), 0)}, {"values": values, "indices": indices}, stream)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("y"), stream), [[5, 2], [1, 4]])
+
+
+@pytest.mark.parametrize("index_dtype", [DataType.uint32, DataType.uint64], ids=lambda d: d.name)
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.fp8_e4m3], ids=lambda d: d.name)
+@pytest.mark.parametrize("shape,axis,taken", [((7, 50, 33), 1, 9), ((7, 50, 33), 2, 64), ((7, 50, 33), 0, 3), ((4096, 130), -1, 130), ((5,), 0, 11)], ids=str)
+def test_take_along_axis_matches_numpy(stream, shape, axis, taken, dtype, index_dtype):
+    rng = np.random.default_rng(21)
+    x = to_storage(rng.standard_normal(shape).astype(np.float32), dtype)
+    index_shape = list(shape)
+    index_shape[axis] = taken
+    chosen = rng.integers(0, shape[axis], index_shape).astype(np.uint32 if index_dtype == DataType.uint32 else np.uint64)
+    plan = run({"y": ex.input("x").take_along_axis(ex.input("i"), axis)}, {"x": copy_numpy_to_gpu(x, stream, dtype), "i": copy_numpy_to_gpu(chosen, stream, index_dtype)},
+               stream)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("y"), stream), np.take_along_axis(x, chosen.astype(np.int64), axis))  # a copy: bit-exact
+
+
+def test_take_along_axis_of_computed_operands(stream):
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((300, 77)).astype(np.float32)
+    ix = ex.input("x")
+    # the value at the row's argmax is the row's max; a transposed operand is gathered from a dense copy
+    outputs = {"at_argmax": (ix * 2.0).take_along_axis(ix.argmax(axis=1), 1), "row_max": ix.reduce_max(axis=1) * 2.0,
+               "of_transpose": ix.transpose().take_along_axis(ix.transpose().argmin(axis=0), 0)}
+    plan = run(outputs, {"x": copy_numpy_to_gpu(x, stream, DataType.fp32)}, stream)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("at_argmax"), stream), copy_gpu_to_numpy(plan.output("row_max"), stream))
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("of_transpose"), stream), x.min(axis=1)[None, :])
+    # indices past the end read the last element of the axis instead of leaving the tensor
+    far = copy_numpy_to_gpu(np.full((300, 2), 1000, np.uint32), stream, DataType.uint32)
+    plan = run({"y": ix.take_along_axis(ex.input("i"))}, {"x": copy_numpy_to_gpu(x, stream, DataType.fp32), "i": far}, stream)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("y"), stream), np.repeat(x[:, -1:], 2, axis=1))
+
+
+def test_take_along_axis_validation(stream):
+    x = copy_numpy_to_gpu(np.zeros((4, 6), np.float32), stream, DataType.fp32)
+    ix, ii = ex.input("x"), ex.input("i")
+    with pytest.raises(RuntimeError, match="indices must have UINT32 or UINT64 dtype, received"):
+        run({"y": ix.take_along_axis(ii)}, {"x": x, "i": x}, stream)
+    with pytest.raises(RuntimeError, match="must have the same rank"):
+        run({"y": ix.take_along_axis(ii)}, {"x": x, "i": copy_numpy_to_gpu(np.zeros((4,), np.uint32), stream, DataType.uint32)}, stream)
+    with pytest.raises(RuntimeError, match="must match except on the selected axis"):
+        run({"y": ix.take_along_axis(ii, 1)}, {"x": x, "i": copy_numpy_to_gpu(np.zeros((3, 2), np.uint32), stream, DataType.uint32)}, stream)
+    with pytest.raises(RuntimeError, match="axis is out of range"):
+        run({"y": ix.take_along_axis(ii, 2)}, {"x": x, "i": copy_numpy_to_gpu(np.zeros((4, 2), np.uint32), stream, DataType.uint32)}, stream)
+    with pytest.raises(ValueError, match="only axis=-1 or an explicit non-negative axis"):
+        ix.take_along_axis(ii, -2)

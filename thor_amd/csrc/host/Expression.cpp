@@ -503,6 +503,13 @@ Expression Expression::stridedView(const std::vector<uint64_t>& dims, const std:
     return out;
 }
 
+Expression Expression::takeAlongAxis(const Expression& indices, int64_t axis) const {
+    if (axis < -1) throw std::invalid_argument("Expression::takeAlongAxis currently supports only axis=-1 or an explicit non-negative axis.");
+    Expression out = binaryOp(*this, indices, ExprOp::TAKE_ALONG_AXIS);
+    out.expr->nodes[out.nodeIndex].reduction_axes = {axis < 0 ? UINT64_MAX : static_cast<uint64_t>(axis)};
+    return out;
+}
+
 Expression Expression::transpose() const {
     if (!expr) throw std::runtime_error("Cannot transpose an empty expression");
     return unaryOp(*this, ExprOp::TRANSPOSE);
@@ -651,7 +658,7 @@ std::string opName(ExprOp op) {
         {(uint16_t)ExprOp::SEGMENTED_REDUCE_SUM, "segmented_reduce_sum"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MIN, "segmented_reduce_min"},
         {(uint16_t)ExprOp::SEGMENTED_REDUCE_MAX, "segmented_reduce_max"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MEAN, "segmented_reduce_mean"},
         {(uint16_t)ExprOp::STRIDED_VIEW, "strided_view"}, {(uint16_t)ExprOp::TRANSPOSE, "transpose"},
-        {(uint16_t)ExprOp::REDUCE_MIN_BACKWARD, "reduce_min_backward"}, {(uint16_t)ExprOp::REDUCE_MAX_BACKWARD, "reduce_max_backward"},
+        {(uint16_t)ExprOp::TAKE_ALONG_AXIS, "take_along_axis"}, {(uint16_t)ExprOp::REDUCE_MIN_BACKWARD, "reduce_min_backward"}, {(uint16_t)ExprOp::REDUCE_MAX_BACKWARD, "reduce_max_backward"},
         {(uint16_t)ExprOp::SEGMENTED_BROADCAST, "segmented_broadcast"}, {(uint16_t)ExprOp::RAGGED_VALUEWISE_EXTENT, "ragged_valuewise_extent"},
     };
     auto it = names.find(static_cast<uint16_t>(op));
@@ -710,6 +717,7 @@ std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex,
             if (c != UINT32_MAX) kids.push_back(canonicalizeNode(expr, c, memo));
         if (isCommutative(n.op) && kids.size() == 2 && kids[1] < kids[0]) std::swap(kids[0], kids[1]);
         text += dtypes();
+        if (n.op == ExprOp::TAKE_ALONG_AXIS) text += ":axis=" + axesText(n.reduction_axes);
         if (isReductionOp(n.op) || isWinnerRoutingOp(n.op)) text += ":axes=" + axesText(n.reduction_axes) + ":squeeze=" + axesText(n.squeeze_axes);
         if (n.op == ExprOp::RESHAPE) text += ":dims=" + axesText(n.reshape_dims);
         if (n.op == ExprOp::UNSQUEEZE) text += ":axes=" + axesText(n.unsqueeze_axes);

@@ -7,6 +7,7 @@
 
 #include "AutoDiffInternal.h"
 #include "HipSourceEmitter.h"
+#include "IndexGather.h"
 #include "ReductionPlanner.h"
 #include "RowFusion.h"
 #include "ShapeInference.h"
@@ -146,6 +147,12 @@ class GraphBuilder {
         } else if (isWinnerRoutingOp(node.op)) {
             node.lhs = asTensorOperand(node.lhs, true);  // read by an arg reduction
             node.rhs = asTensorOperand(node.rhs, false);
+        } else if (node.op == ExprOp::TAKE_ALONG_AXIS) {
+            node.lhs = asTensorOperand(node.lhs, false);
+            node.rhs = asTensorOperand(node.rhs, false);
+            // the gather addresses dense storage: a strided view is copied into a dense tensor first
+            if (isStorageViewOp(out.nodes[node.lhs].op)) node.lhs = castOf(node.lhs, out.nodes[node.lhs].output_dtype.value());
+            if (isStorageViewOp(out.nodes[node.rhs].op)) node.rhs = castOf(node.rhs, out.nodes[node.rhs].output_dtype.value());
         } else if (node.op == ExprOp::SEGMENTED_BROADCAST) {
             node.lhs = asTensorOperand(node.lhs, false);
         } else if (isShapeOnly(node.op)) {
@@ -211,7 +218,8 @@ uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
 // Can the consumer read a per-segment value through the segment index?  Only work that ends up inside a flat fused kernel.
 bool consumesGather(const ExprNode& consumer) {
     if (consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT || consumer.op == ExprOp::WHERE || consumer.op == ExprOp::CAST) return true;
-    if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX || isWinnerRoutingOp(consumer.op)) {
+    if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX || isWinnerRoutingOp(consumer.op) ||
+        consumer.op == ExprOp::TAKE_ALONG_AXIS) {
         return false;
     }
     return Expression::isBinaryOp(consumer.op) || Expression::isUnaryOp(consumer.op);
@@ -331,6 +339,11 @@ std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpressio
                 dims[i][0] = n.ragged_runtime_max_active_values;
                 break;
             }
+            case ExprOp::TAKE_ALONG_AXIS:
+                if (dims[n.lhs].empty() || dims[n.rhs].empty()) throw std::runtime_error("take_along_axis requires non-scalar input and indices tensors.");
+                if (dims[n.lhs].size() != dims[n.rhs].size()) throw std::runtime_error("take_along_axis input and indices must have the same rank.");
+                dims[i] = dims[n.rhs];
+                break;
             case ExprOp::REDUCE_MIN_BACKWARD:
             case ExprOp::REDUCE_MAX_BACKWARD: {
                 // operand-shaped; the gradient holds one element per reduction window
@@ -483,7 +496,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             } else if (isReductionOp(n.op)) {
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
-            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(n.op)) {
+            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS) {
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
                 ensureTensor(n.rhs);
@@ -564,7 +577,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             std::vector<uint32_t> sources, scalars;
             if (isReductionOp(graph->expr.nodes[i].op)) {
                 sources.push_back(graph->expr.nodes[i].lhs);
-            } else if (isWinnerRoutingOp(graph->expr.nodes[i].op)) {
+            } else if (isWinnerRoutingOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::TAKE_ALONG_AXIS) {
                 sources.push_back(graph->expr.nodes[i].lhs);
                 sources.push_back(graph->expr.nodes[i].rhs);
             } else if (isSegmentedReduceOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST) {
@@ -714,7 +727,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     auto runsInFusedKernel = [&](uint32_t i) {
         const ExprOp op = expr.nodes[i].op;
         return graph->role[i] == Role::Materialized && !isReductionOp(op) && !isSegmentedReduceOp(op) && op != ExprOp::SEGMENTED_BROADCAST &&
-               !isWinnerRoutingOp(op) && op != ExprOp::INPUT;
+               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && op != ExprOp::INPUT;
     };
     std::vector<uint32_t> levelOf = graph->level;
     if (stageFusionEnabled()) {
@@ -724,7 +737,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             std::vector<uint32_t> sources, scalars;
             if (isReductionOp(n.op)) {
                 sources.push_back(n.lhs);
-            } else if (isWinnerRoutingOp(n.op)) {
+            } else if (isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS) {
                 sources = {n.lhs, n.rhs};
             } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
                 if (graph->role[n.lhs] == Role::Inline) {
@@ -1113,6 +1126,22 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                         CubSegmentedReduction(op, n.output_dtype.value()).stampRuntimeOffsets(values, output, offsets, stream));
                 }
                 tensorOf[i] = output;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(stage));
+                done[i] = 1;
+                continue;
+            }
+            if (n.op == ExprOp::TAKE_ALONG_AXIS) {
+                const uint64_t rank = dims[n.lhs].size();
+                const uint64_t axis = n.reduction_axes.empty() || n.reduction_axes.front() == UINT64_MAX ? rank - 1 : n.reduction_axes.front();
+                if (axis >= rank) throw std::runtime_error("take_along_axis axis is out of range for the input rank.");
+                Tensor gathered = allocateFor(i);
+                StampedExecutionStage stage;
+                stage.kind = StampedExecutionStage::Kind::FusedKernel;
+                stage.gpu_num = device_num;
+                stage.dependency_stage_indices = dependenciesOf({n.lhs, n.rhs});
+                stage.kernel = stampTakeAlongAxis(tensorOf[n.lhs], tensorOf[n.rhs], gathered, axis, device_num);
+                tensorOf[i] = gathered;
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
                 done[i] = 1;

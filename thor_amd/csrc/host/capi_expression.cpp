@@ -185,6 +185,9 @@ thor_expr_t thor_expr_strided_view(thor_expr_t input, const uint64_t* dims, cons
                       return new thor_expr{input->expr.stridedView(std::vector<uint64_t>(dims, dims + rank), std::vector<uint64_t>(strides, strides + rank),
                                                                    element_offset)};)
 }
+thor_expr_t thor_expr_take_along_axis(thor_expr_t input, thor_expr_t indices, int64_t axis) {
+    THOR_CAPI_TRY_PTR(require(input, "input"); require(indices, "indices"); return new thor_expr{input->expr.takeAlongAxis(indices->expr, axis)};)
+}
 thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank) {
     THOR_CAPI_TRY_PTR(require(input, "expression"); return new thor_expr{input->expr.reshape(u64s(dims, rank))};)
 }

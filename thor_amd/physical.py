@@ -73,6 +73,7 @@ PROTOTYPES = {
     "thor_expr_cast": (_vp, [_vp, _i]), "thor_expr_with_dtypes": (_vp, [_vp, _i, _i]),
     "thor_expr_reduce": (_vp, [_cp, _vp, _u64p, _i, _u64p, _i]), "thor_expr_reshape": (_vp, [_vp, _u64p, _i]),
     "thor_expr_strided_view": (_vp, [_vp, _u64p, _u64p, _i, ctypes.c_uint64]),
+    "thor_expr_take_along_axis": (_vp, [_vp, _vp, ctypes.c_int64]),
     "thor_expr_unsqueeze": (_vp, [_vp, _u64p, _i]), "thor_expr_squeeze": (_vp, [_vp, _u64p, _i]), "thor_expr_destroy": (None, [_vp]),
     "thor_expr_num_nodes": (_i, [_vp]), "thor_expr_canonical": (_i, [_vp, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_outputs_create": (_vp, [_cpp, _vpp, _i]), "thor_outputs_destroy": (None, [_vp]),
@@ -668,6 +669,10 @@ class Expression:
     def with_ragged_runtime_extent(self, offsets, batch_size: int, max_active_values: int, elements_per_value: int = 1):
         """The same values, computed only for the first offsets[batch_size] rows; the rest of the output keeps its contents."""
         return self._ragged("ragged_extent", offsets, batch_size, max_active_values, elements_per_value)
+
+    def take_along_axis(self, indices: "Expression", axis: int = -1) -> "Expression":
+        """Gather along one axis with UINT32 / UINT64 indices; the result has the shape of ``indices``."""
+        return Expression(_handle(lib().thor_expr_take_along_axis(self._h, indices._h, axis), "take_along_axis"))
 
     def transpose(self) -> "Expression":
         """The last two axes exchanged, as a view of the operand's storage."""
