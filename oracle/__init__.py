@@ -208,3 +208,105 @@ def rows_f32(x):
     s, m, a = np.empty(rows, np.float32), np.empty(rows, np.float32), np.empty(rows, np.uint32)
     threads = lib().oracle_rows_f32(x.ctypes.data, s.ctypes.data, m.ctypes.data, a.ctypes.data, rows, cols)
     return s, m, a, threads
+
+
+# ---- prefix scans --------------------------------------------------------------------------------------------------------------
+SCAN_SUM, SCAN_MIN, SCAN_MAX, SCAN_PRODUCT, SCAN_ARGMIN, SCAN_ARGMAX = range(6)
+
+
+def _scan_segment_fast(x, base, integer, dtype):
+    """Inclusive forward scan of one segment with NumPy's sequential accumulate routines, for the cases where they perform the
+    same operations in the same order as the element-by-element walk: returns (values, winner positions) or None."""
+    if x.size == 0:
+        return x.copy(), np.zeros(0, np.int64)
+    if base in (SCAN_MIN, SCAN_MAX):
+        if not integer and np.isnan(x).any():
+            return None
+        running = (np.minimum if base == SCAN_MIN else np.maximum).accumulate(x)
+        changed = np.concatenate([[True], running[1:] != running[:-1]])  # a new running value is set by a strictly better element
+        positions = np.maximum.accumulate(np.where(changed, np.arange(x.size), 0))
+        return x[positions], positions  # the winner's own bits (-0.0 and +0.0 compare equal: the earlier one stays)
+    if integer:
+        if base == SCAN_SUM:
+            return np.cumsum(x, dtype=np.uint64) & np.uint64(0xFFFFFFFF), None
+        return None
+    if dtype == FP32:
+        return (np.cumsum(x, dtype=np.float32) if base == SCAN_SUM else np.cumprod(x, dtype=np.float32)), None
+    if dtype == FP16:
+        with np.errstate(over="ignore", invalid="ignore"):
+            half = x.astype(np.float16)
+            return (np.cumsum(half, dtype=np.float16) if base == SCAN_SUM else np.cumprod(half, dtype=np.float16)).astype(np.float32), None
+    return None
+
+
+def scan(values: np.ndarray, op: int, inclusive: bool = True, reverse: bool = False, segment_size: int = 0, offsets=None, dtype: int = FP32,
+         fast: bool = True):
+    """Sequential restatement of the reference's scans over a flat array of `dtype` carriers
+    (Utilities/TensorOperations/Cub/CubScan.cu:47-93 operators, :106-196 identities; CubSegmentedScan.cu for segments).
+
+    Every combine rounds to the element type (16-bit floats add and multiply in fp32, then round); min / max keep the earlier
+    element unless the later one is strictly smaller / larger; the first element of a segment is taken as it is.  Exclusive
+    scans start with 0, 1, the largest / smallest value (+-inf for floats); arg scans return UINT32 flattened indices, with
+    0xFFFFFFFF where the prefix is empty.  Segments: `segment_size` > 0 -> consecutive runs of that length; `offsets` -> the
+    ranges [offsets[s], offsets[s + 1]); neither -> one scan.  Elements outside every segment keep 0.  `reverse` scans every
+    segment from its end.  Value scans return carriers of `dtype`.  `fast` lets NumPy's sequential accumulate routines stand in
+    for the walk where they do the same operations in the same order (the tests hold the two against each other)."""
+    flat = np.ascontiguousarray(values).reshape(-1)
+    n = flat.size
+    arg = op in (SCAN_ARGMIN, SCAN_ARGMAX)
+    base = {SCAN_ARGMIN: SCAN_MIN, SCAN_ARGMAX: SCAN_MAX}.get(op, op)
+    integer = dtype == UINT32
+    work = flat.astype(np.uint64) if integer else to_f32(flat, dtype).astype(np.float32)
+
+    def rounded(x):
+        if integer:
+            return np.uint64(int(x) & 0xFFFFFFFF)
+        return to_f32(from_f32(np.array([x], np.float32), dtype), dtype)[0]
+
+    identity = {SCAN_SUM: 0, SCAN_PRODUCT: 1, SCAN_MIN: 0xFFFFFFFF if integer else np.inf, SCAN_MAX: 0 if integer else -np.inf}[base]
+    if offsets is not None:
+        bounds = [(int(offsets[s]), int(offsets[s + 1])) for s in range(len(offsets) - 1)]
+    elif segment_size:
+        bounds = [(b, b + segment_size) for b in range(0, n, segment_size)]
+    else:
+        bounds = [(0, n)]
+    out_values = np.zeros(n, np.uint64 if integer else np.float32)
+    out_index = np.zeros(n, np.uint32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        for begin, end in bounds:
+            quick = _scan_segment_fast(work[begin:end][::-1] if reverse else work[begin:end], base, integer, dtype) if fast else None
+            if quick is not None and end > begin:
+                running_values, positions = quick
+                if positions is None:
+                    positions = np.zeros(end - begin, np.int64)
+                where = (end - 1 - positions) if reverse else (begin + positions)
+                if not inclusive:
+                    running_values = np.concatenate([[identity], running_values[:-1]]).astype(running_values.dtype)
+                    where = np.concatenate([[0xFFFFFFFF], where[:-1]])
+                target = slice(begin, end)
+                out_values[target] = running_values[::-1] if reverse else running_values
+                out_index[target] = (where[::-1] if reverse else where).astype(np.uint32)
+                continue
+            order = range(end - 1, begin - 1, -1) if reverse else range(begin, end)
+            running, winner = None, 0xFFFFFFFF
+            for i in order:
+                x = work[i]
+                if not inclusive:
+                    out_values[i] = identity if running is None else running
+                    out_index[i] = winner
+                if running is None:
+                    running, winner = x, i
+                elif base == SCAN_SUM:
+                    running = rounded(np.float32(running) + np.float32(x)) if not integer else rounded(int(running) + int(x))
+                elif base == SCAN_PRODUCT:
+                    running = rounded(np.float32(running) * np.float32(x)) if not integer else rounded(int(running) * int(x))
+                elif (x < running) if base == SCAN_MIN else (running < x):
+                    running, winner = x, i
+                if inclusive:
+                    out_values[i] = running
+                    out_index[i] = winner
+    if arg:
+        return out_index.reshape(np.shape(values))
+    if integer:
+        return out_values.astype(np.uint32).reshape(np.shape(values))
+    return from_f32(out_values.astype(np.float32), dtype).reshape(np.shape(values))

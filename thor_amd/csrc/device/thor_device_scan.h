@@ -1,0 +1,317 @@
+// Prefix scans (sum / product / min / max and arg-min / arg-max) over one logical sequence that segment heads cut into
+// independent scans: rows of equal length, the segments of a row partition, or nothing (one flat scan).  Instantiated by
+// run-time generated traits structs (placed after thor_device_prelude.h).
+//
+// A block owns a chunk of consecutive logical positions and keeps it in registers: lane-interleaved 16-byte vectors, so
+// loads and stores coalesce.  Order inside the chunk is (vector round, thread, element).  Each thread scans its vectors
+// serially, the per-vector totals are scanned across the wavefront with shuffles, the wavefront totals across the block
+// through a few words of LDS, and the prefix is folded back into the elements: one read and one write per element.  The
+// state that flows is {value, index of the value (arg scans), "a head lies in the summarised range"}; combining an earlier
+// state with a later one keeps the later one alone when it holds a head.
+//
+// Chunks that start inside a segment need the state of what precedes them.  That takes three launches, none of which
+// waits on another block: the same kernel without stores writes each chunk's total, one block turns the totals into
+// carries, the full kernel applies them.  When segments are rows that chunks hold whole, the single launch is enough.
+//
+// A reverse scan walks the same code over mirrored positions (logical p = total - 1 - physical q).
+//
+// Cfg: T (storage), Acc (u32 for UINT32, float otherwise), kUnsigned, kOp (0 sum, 1 min, 2 max, 3 product), kArg, kInclusive, kReverse,
+// kTotal, kRow (row length; 0 = heads come from a bitmap), kThreads, kVec, kItems, kChunkElems (positions per block, a
+// multiple of kVec, at most kThreads * kVec * kItems), kChunks, kCarry, kWriteValue, kWriteIndex.
+#pragma once
+
+namespace thor {
+
+constexpr u32 kNoIndex = 0xffffffffu;
+
+template <typename Cfg>
+struct ScanState {
+    typename Cfg::Acc v;
+    u32 i;
+    u32 head;
+};
+
+template <typename Cfg>
+__device__ __forceinline__ typename Cfg::Acc scanIdentity() {
+    typedef typename Cfg::Acc Acc;
+    if (Cfg::kOp == 0) return (Acc)0;
+    if (Cfg::kOp == 3) return (Acc)1;
+    if (Cfg::kUnsigned) return Cfg::kOp == 1 ? (Acc)0xffffffffu : (Acc)0;  // largest / smallest value
+    return Cfg::kOp == 1 ? (Acc)__builtin_inff() : (Acc)(-__builtin_inff());
+}
+
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanEmpty() {
+    ScanState<Cfg> s;
+    s.v = scanIdentity<Cfg>();
+    s.i = kNoIndex;
+    s.head = 0;
+    return s;
+}
+
+// `a` summarises positions before those of `b`.  Min / max keep the earlier value unless the later one is strictly better
+// (so equal values keep the first index); an empty earlier state loses against any element.
+template <typename Cfg>
+__device__ __forceinline__ void scanOp(typename Cfg::Acc av, u32 ai, typename Cfg::Acc bv, u32 bi, typename Cfg::Acc& rv, u32& ri) {
+    if (Cfg::kOp == 0) {
+        rv = av + bv;
+        ri = kNoIndex;
+    } else if (Cfg::kOp == 3) {
+        rv = av * bv;
+        ri = kNoIndex;
+    } else {
+        // an index also says "holds an element": the first element of a scan is taken as it is, whatever its value (a NaN
+        // that comes first stays, one that comes later never wins: no comparison with it holds)
+        const bool takeLater = ((Cfg::kOp == 1 ? (bv < av) : (av < bv)) | (ai == kNoIndex)) & (bi != kNoIndex);
+        rv = takeLater ? bv : av;
+        ri = takeLater ? bi : ai;
+    }
+}
+
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanCombine(const ScanState<Cfg>& a, const ScanState<Cfg>& b) {
+    ScanState<Cfg> r;
+    scanOp<Cfg>(a.v, a.i, b.v, b.i, r.v, r.i);
+    r.v = b.head ? b.v : r.v;
+    r.i = b.head ? b.i : r.i;
+    r.head = a.head | b.head;
+    return r;
+}
+
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanShuffleUp(const ScanState<Cfg>& s, int delta) {
+    ScanState<Cfg> r;
+    r.v = __shfl_up(s.v, delta, kWave);
+    r.i = (Cfg::kOp == 1 || Cfg::kOp == 2) ? __shfl_up(s.i, delta, kWave) : kNoIndex;
+    r.head = __shfl_up(s.head, delta, kWave);
+    return r;
+}
+
+// inclusive scan of one state per lane across the wavefront
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanWave(ScanState<Cfg> s, int lane) {
+#pragma unroll
+    for (int delta = 1; delta < kWave; delta *= 2) {
+        const ScanState<Cfg> earlier = scanShuffleUp<Cfg>(s, delta);
+        const ScanState<Cfg> merged = scanCombine<Cfg>(earlier, s);
+        if (lane >= delta) s = merged;
+    }
+    return s;
+}
+
+__device__ __forceinline__ float scanLoad(float x) { return x; }
+__device__ __forceinline__ float scanLoad(f16 x) { return toFloat(x); }
+__device__ __forceinline__ float scanLoad(bf16 x) { return toFloat(x); }
+__device__ __forceinline__ u32 scanLoad(u32 x) { return x; }
+template <typename T>
+__device__ __forceinline__ T scanStore(float x) {
+    return fromFloat<T>(x);
+}
+template <typename T>
+__device__ __forceinline__ T scanStore(u32 x) {
+    return (T)x;
+}
+
+// chunk states in memory: kChunks values, then kChunks indices, then kChunks head words
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanLoadState(const void* buffer, u64 slot) {
+    ScanState<Cfg> s;
+    const u32* words = static_cast<const u32*>(buffer);
+    s.v = __builtin_bit_cast(typename Cfg::Acc, words[slot]);
+    s.i = words[Cfg::kChunks + slot];
+    s.head = words[2 * Cfg::kChunks + slot];
+    return s;
+}
+template <typename Cfg>
+__device__ __forceinline__ void scanStoreState(void* buffer, u64 slot, const ScanState<Cfg>& s) {
+    u32* words = static_cast<u32*>(buffer);
+    words[slot] = __builtin_bit_cast(u32, s.v);
+    words[Cfg::kChunks + slot] = s.i;
+    words[2 * Cfg::kChunks + slot] = s.head;
+}
+
+// bit k set: logical position p + k starts a segment (p is a multiple of kVec)
+template <typename Cfg>
+__device__ __forceinline__ u32 scanHeadBits(const u32* heads, u64 p) {
+    constexpr int V = Cfg::kVec;
+    if (Cfg::kRow == 0) return (heads[p / 32] >> (p % 32)) & ((1u << V) - 1u);
+    if (Cfg::kRow % V == 0) return p % Cfg::kRow == 0 ? 1u : 0u;
+    u32 bits = 0;
+#pragma unroll
+    for (int k = 0; k < V; ++k) bits |= ((p + k) % Cfg::kRow == 0 ? 1u : 0u) << k;
+    return bits;
+}
+
+// AGGREGATE_ONLY: write the chunk's total to `aggregates` and nothing else.  Otherwise: take the chunk's carry from
+// `carries` (when Cfg::kCarry) and write the scanned values and / or indices.
+template <typename Cfg, bool AGGREGATE_ONLY>
+__device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* heads, const void* carries, void* aggregates,
+                                          typename Cfg::T* outValue, u32* outIndex) {
+    typedef typename Cfg::T T;
+    typedef typename Cfg::Acc Acc;
+    typedef ScanState<Cfg> S;
+    constexpr int V = Cfg::kVec, ITEMS = Cfg::kItems, THREADS = Cfg::kThreads, WAVES = THREADS / kWave;
+    static_assert(ITEMS * WAVES <= kWave, "the wavefront totals of a chunk are scanned by one wavefront");
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const u64 chunkBase = (u64)blockIdx.x * Cfg::kChunkElems;
+
+    __shared__ u32 totalValue[ITEMS * WAVES], totalIndex[ITEMS * WAVES], totalHead[ITEMS * WAVES];
+
+    Acc pre[ITEMS][V];
+    u32 preIndex[ITEMS][V];
+    u32 sealed[ITEMS];
+    bool live[ITEMS];
+    u64 physical[ITEMS];  // first element of the vector in memory
+    S laneExclusive[ITEMS];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const u64 local = ((u64)it * THREADS + threadIdx.x) * V;
+        const u64 p = chunkBase + local;
+        live[it] = local < Cfg::kChunkElems && p < Cfg::kTotal;
+        physical[it] = Cfg::kReverse ? Cfg::kTotal - (live[it] ? p : 0) - V : (live[it] ? p : 0);
+        Pack<T, V> x;
+        u32 headBits = 0;
+        if (live[it]) {
+            x.loadStream(in + physical[it]);
+            headBits = scanHeadBits<Cfg>(heads, p);
+        }
+        S run = scanEmpty<Cfg>();
+        sealed[it] = 0;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            S e;
+            e.v = live[it] ? scanLoad(x.v[Cfg::kReverse ? V - 1 - k : k]) : scanIdentity<Cfg>();
+            e.i = live[it] ? (u32)(physical[it] + (Cfg::kReverse ? V - 1 - k : k)) : kNoIndex;
+            e.head = (headBits >> k) & 1u;
+            if (!Cfg::kInclusive) {
+                pre[it][k] = e.head ? scanIdentity<Cfg>() : run.v;
+                preIndex[it][k] = e.head ? kNoIndex : run.i;
+                sealed[it] |= (run.head | e.head) << k;
+            }
+            run = scanCombine<Cfg>(run, e);
+            if (Cfg::kInclusive) {
+                pre[it][k] = run.v;
+                preIndex[it][k] = run.i;
+                sealed[it] |= run.head << k;
+            }
+        }
+        const S inclusive = scanWave<Cfg>(run, lane);
+        laneExclusive[it] = scanShuffleUp<Cfg>(inclusive, 1);
+        if (lane == 0) laneExclusive[it] = scanEmpty<Cfg>();
+        if (lane == kWave - 1) {
+            totalValue[it * WAVES + wave] = __builtin_bit_cast(u32, inclusive.v);
+            totalIndex[it * WAVES + wave] = inclusive.i;
+            totalHead[it * WAVES + wave] = inclusive.head;
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        S mine = scanEmpty<Cfg>();
+        if (lane < ITEMS * WAVES) {
+            mine.v = __builtin_bit_cast(Acc, totalValue[lane]);
+            mine.i = totalIndex[lane];
+            mine.head = totalHead[lane];
+        }
+        const S inclusive = scanWave<Cfg>(mine, lane);
+        if (AGGREGATE_ONLY) {
+            if (lane == kWave - 1) scanStoreState<Cfg>(aggregates, blockIdx.x, inclusive);
+        } else {
+            S before = scanShuffleUp<Cfg>(inclusive, 1);
+            if (lane == 0) before = scanEmpty<Cfg>();
+            if (Cfg::kCarry) before = scanCombine<Cfg>(scanLoadState<Cfg>(carries, blockIdx.x), before);
+            if (lane < ITEMS * WAVES) {
+                totalValue[lane] = __builtin_bit_cast(u32, before.v);
+                totalIndex[lane] = before.i;
+                totalHead[lane] = before.head;
+            }
+        }
+    }
+    if (AGGREGATE_ONLY) return;
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        if (!live[it]) continue;
+        S base;
+        base.v = __builtin_bit_cast(Acc, totalValue[it * WAVES + wave]);
+        base.i = totalIndex[it * WAVES + wave];
+        base.head = totalHead[it * WAVES + wave];
+        base = scanCombine<Cfg>(base, laneExclusive[it]);
+        Pack<T, V> values;
+        Pack<u32, V> indices;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            Acc v;
+            u32 i;
+            scanOp<Cfg>(base.v, base.i, pre[it][k], preIndex[it][k], v, i);
+            const bool own = (sealed[it] >> k) & 1u;
+            v = own ? pre[it][k] : v;
+            i = own ? preIndex[it][k] : i;
+            values.v[Cfg::kReverse ? V - 1 - k : k] = scanStore<T>(v);
+            indices.v[Cfg::kReverse ? V - 1 - k : k] = i;
+        }
+        if (Cfg::kWriteValue) values.storeStream(outValue + physical[it]);
+        if (Cfg::kWriteIndex) indices.storeStream(outIndex + physical[it]);
+    }
+}
+
+// One block: the totals of kChunks chunks -> the state that precedes each chunk.  A thread owns a run of consecutive chunks.
+template <typename Cfg>
+__device__ __forceinline__ void scanCarries(const void* aggregates, void* carries) {
+    typedef ScanState<Cfg> S;
+    constexpr int THREADS = 1024, WAVES = THREADS / kWave;
+    constexpr u64 PER = (Cfg::kChunks + THREADS - 1) / THREADS;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const u64 first = (u64)threadIdx.x * PER;
+    __shared__ u32 totalValue[WAVES], totalIndex[WAVES], totalHead[WAVES];
+    S run = scanEmpty<Cfg>();
+    for (u64 c = first; c < first + PER && c < Cfg::kChunks; ++c) run = scanCombine<Cfg>(run, scanLoadState<Cfg>(aggregates, c));
+    const S inclusive = scanWave<Cfg>(run, lane);
+    S before = scanShuffleUp<Cfg>(inclusive, 1);
+    if (lane == 0) before = scanEmpty<Cfg>();
+    if (lane == kWave - 1) {
+        totalValue[wave] = __builtin_bit_cast(u32, inclusive.v);
+        totalIndex[wave] = inclusive.i;
+        totalHead[wave] = inclusive.head;
+    }
+    __syncthreads();
+    S earlierWaves = scanEmpty<Cfg>();
+    for (int w = 0; w < wave; ++w) {
+        S t;
+        t.v = __builtin_bit_cast(typename Cfg::Acc, totalValue[w]);
+        t.i = totalIndex[w];
+        t.head = totalHead[w];
+        earlierWaves = scanCombine<Cfg>(earlierWaves, t);
+    }
+    run = scanCombine<Cfg>(earlierWaves, before);
+    for (u64 c = first; c < first + PER && c < Cfg::kChunks; ++c) {
+        scanStoreState<Cfg>(carries, c, run);
+        run = scanCombine<Cfg>(run, scanLoadState<Cfg>(aggregates, c));
+    }
+}
+
+// Segment heads of a row partition as one bit per logical position.  The bitmap is cleared by scanClearHeads first.
+// Cfg: OffsetT, kSegments, kTotal, kReverse.
+template <typename Cfg>
+__device__ __forceinline__ void scanClearHeads(u32* heads) {
+    const u64 word = (u64)blockIdx.x * blockDim.x + threadIdx.x;
+    if (word < (Cfg::kTotal + 31) / 32) heads[word] = 0;
+}
+template <typename Cfg>
+__device__ __forceinline__ void scanMarkHeads(const typename Cfg::OffsetT* offsets, u32* heads) {
+    const u64 s = (u64)blockIdx.x * blockDim.x + threadIdx.x;
+    if (s > Cfg::kSegments) return;
+    u64 begin = (u64)offsets[s];
+    begin = begin < Cfg::kTotal ? begin : Cfg::kTotal;
+    if (s == Cfg::kSegments) {
+        // rows past the partition form a segment of their own, so nothing of theirs flows into a real one
+        if (!Cfg::kReverse && begin < Cfg::kTotal) atomicOr(&heads[begin / 32], 1u << (begin % 32));
+        return;
+    }
+    u64 end = (u64)offsets[s + 1];
+    end = end < Cfg::kTotal ? end : Cfg::kTotal;
+    if (end <= begin) return;
+    const u64 position = Cfg::kReverse ? Cfg::kTotal - end : begin;
+    atomicOr(&heads[position / 32], 1u << (position % 32));
+}
+
+}  // namespace thor

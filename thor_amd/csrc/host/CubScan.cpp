@@ -1,0 +1,381 @@
+// Prefix scans: validation, kernel specialisation and launch (kernels: device/thor_device_scan.h; reference behaviour:
+// Utilities/TensorOperations/Cub/CubScan.cu:47-196 operators and identities, :314-420 plan / run protocol,
+// CubSegmentedScan.cu for the uniform-segment and offset-segment forms).
+#include "CubScanInternal.h"
+
+#include "ReductionPlanner.h"
+#include "Utilities/Common/ScopedGpu.h"
+#include "thorhip_numeric_embed.h"
+
+#include <algorithm>
+#include <numeric>
+#include <sstream>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+namespace {
+
+size_t roundUp(size_t v, size_t to) { return (v + to - 1) / to * to; }
+
+const char* scanStorageName(DataType dtype) {
+    switch (dtype) {
+        case DataType::UINT32: return "thor::u32";
+        case DataType::FP16: return "thor::f16";
+        case DataType::BF16: return "thor::bf16";
+        case DataType::FP32: return "float";
+        default: break;
+    }
+    throw std::invalid_argument(std::string("Unsupported CUB scan dtype ") + dataTypeName(dtype) + ".");
+}
+
+}  // namespace
+
+bool isCubScanDTypeSupported(DataType dtype) {
+    return dtype == DataType::UINT32 || dtype == DataType::FP16 || dtype == DataType::BF16 || dtype == DataType::FP32;
+}
+bool isCubSegmentOffsetDTypeSupported(DataType dtype) { return dtype == DataType::UINT32 || dtype == DataType::UINT64; }
+
+Tensor allocateCubTemporaryStorage(const TensorPlacement& placement, size_t bytes) {
+    if (placement.getMemDevice() != TensorPlacement::MemDevices::GPU) throw std::invalid_argument("CUB temporary storage must be planned on GPU placement.");
+    return Tensor(placement, TensorDescriptor(DataType::UINT8, {std::max<uint64_t>(bytes, 1)}));
+}
+
+std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r) {
+    if (!isCubScanDTypeSupported(r.dtype)) throw std::invalid_argument(std::string("Unsupported CUB scan dtype ") + dataTypeName(r.dtype) + ".");
+    if (r.total == 0) throw std::invalid_argument("CUB scan requires at least one element.");
+    if ((r.writeIndex || r.op == 1 || r.op == 2) && r.total > 0xfffffffeull) {
+        throw std::invalid_argument("CUB min / max / arg scans index elements with UINT32: too many elements.");
+    }
+    const bool ragged = r.row == 0;
+    if (!ragged && r.total % r.row != 0) throw std::invalid_argument("CUB uniform segmented scan requires num_items == num_segments * segment_size.");
+
+    auto kernels = std::make_shared<CubScanKernels>();
+    CubScanKernels& k = *kernels;
+    k.request = r;
+    const uint32_t elementBytes = dataTypeSizeInBytes(r.dtype);
+    uint64_t vec = 16 / elementBytes;
+    while (vec > 1 && (r.total % vec != 0 || r.alignmentBytes % (vec * std::max<uint32_t>(elementBytes, r.writeIndex ? 4 : elementBytes)) != 0)) vec /= 2;
+    const uint64_t threads = 256, lanesWorth = threads * vec;
+    uint64_t items = 4;
+    uint64_t chunkElems = lanesWorth * items;
+    k.carry = true;
+    if (!ragged && r.row <= lanesWorth * 16) {
+        // chunks of whole rows: every chunk starts at a head and needs nothing from its predecessors
+        const uint64_t step = vec / std::gcd(r.row, vec);  // rows per chunk must keep chunk starts on vector boundaries
+        uint64_t rowsPerChunk = std::max<uint64_t>(lanesWorth * 4 / r.row / step * step, step);
+        if (rowsPerChunk * r.row <= lanesWorth * 16) {
+            chunkElems = rowsPerChunk * r.row;
+            items = (chunkElems + lanesWorth - 1) / lanesWorth;
+            k.carry = false;
+        }
+    }
+    if (k.carry) {
+        items = 8;
+        chunkElems = lanesWorth * items;
+    }
+    k.chunks = (r.total + chunkElems - 1) / chunkElems;
+    if (k.chunks == 1) k.carry = false;
+    if (k.chunks > 0x7fffffffull) throw std::invalid_argument("CUB scan: too many elements for one launch.");
+
+    // temporary storage: head bitmap (ragged), chunk totals, chunk carries
+    k.headsBytes = ragged ? roundUp((r.total + 31) / 32 * 4, 256) : 0;
+    k.statesBytes = k.carry ? roundUp(3 * k.chunks * 4, 256) : 0;
+    k.tempBytes = std::max<size_t>(k.headsBytes + 2 * k.statesBytes, 1);
+
+    const bool isUnsigned = r.dtype == DataType::UINT32;
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude << thor_embed::kScanKernels;
+    s << "namespace gen {\nstruct Cfg {\n    typedef " << scanStorageName(r.dtype) << " T;\n    typedef " << (isUnsigned ? "thor::u32" : "float")
+      << " Acc;\n    typedef " << (r.offsets64 ? "thor::u64" : "thor::u32") << " OffsetT;\n"
+      << "    static constexpr bool kUnsigned = " << (isUnsigned ? "true" : "false") << ";\n    static constexpr int kOp = " << r.op
+      << ";\n    static constexpr bool kArg = " << (r.writeIndex ? "true" : "false") << ";\n    static constexpr bool kInclusive = "
+      << (r.inclusive ? "true" : "false") << ";\n    static constexpr bool kReverse = " << (r.reverse ? "true" : "false")
+      << ";\n    static constexpr thor::u64 kTotal = " << r.total << "ull;\n    static constexpr thor::u64 kRow = " << r.row
+      << "ull;\n    static constexpr thor::u64 kSegments = " << r.segments << "ull;\n    static constexpr int kThreads = " << threads
+      << ";\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kItems = " << items
+      << ";\n    static constexpr thor::u64 kChunkElems = " << chunkElems << "ull;\n    static constexpr thor::u64 kChunks = " << k.chunks
+      << "ull;\n    static constexpr bool kCarry = " << (k.carry ? "true" : "false") << ";\n    static constexpr bool kWriteValue = "
+      << (r.writeValue ? "true" : "false") << ";\n    static constexpr bool kWriteIndex = " << (r.writeIndex ? "true" : "false") << ";\n};\n}  // namespace gen\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_main(const gen::Cfg::T* in, const thor::u32* heads, const void* carries, "
+         "gen::Cfg::T* outValue, thor::u32* outIndex) {\n    thor::scanChunk<gen::Cfg, false>(in, heads, carries, nullptr, outValue, outIndex);\n}\n";
+    if (k.carry) {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_totals(const gen::Cfg::T* in, const thor::u32* heads, void* totals) {\n"
+             "    thor::scanChunk<gen::Cfg, true>(in, heads, nullptr, totals, nullptr, nullptr);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(1024) void thor_scan_carries(const void* totals, void* carries) {\n"
+             "    thor::scanCarries<gen::Cfg>(totals, carries);\n}\n";
+    }
+    if (ragged) {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_clear_heads(thor::u32* heads) { thor::scanClearHeads<gen::Cfg>(heads); }\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_mark_heads(const void* offsets, thor::u32* heads) {\n"
+             "    thor::scanMarkHeads<gen::Cfg>(static_cast<const gen::Cfg::OffsetT*>(offsets), heads);\n}\n";
+    }
+    const std::string source = s.str();
+    k.mainKernel = compileKernel(source, "thor_scan_main", r.deviceNum, /*fastContract=*/false);
+    if (k.carry) {
+        k.totalsKernel = compileKernel(source, "thor_scan_totals", r.deviceNum, false);
+        k.carriesKernel = compileKernel(source, "thor_scan_carries", r.deviceNum, false);
+    }
+    if (ragged) {
+        k.clearKernel = compileKernel(source, "thor_scan_clear_heads", r.deviceNum, false);
+        k.markKernel = compileKernel(source, "thor_scan_mark_heads", r.deviceNum, false);
+    }
+    std::ostringstream variant;
+    variant << (ragged ? "segments" : r.row == r.total ? "flat" : "rows") << "(chunk=" << chunkElems << ",vec=" << vec << ",items=" << items
+            << ",grid=" << k.chunks << (k.carry ? ",passes=totals+carries+scan" : ",passes=scan") << (r.reverse ? ",reverse" : "") << ") ["
+            << k.mainKernel->kernelName << "]";
+    k.variant = variant.str();
+    return kernels;
+}
+
+void launchScan(const CubScanKernels& k, const void* input, const void* offsets, void* temp, size_t tempBytes, void* outValue, void* outIndex,
+                Stream& stream) {
+    if (!stream.isInitialized() || stream.getGpuNum() != k.request.deviceNum) throw std::invalid_argument("CUB scan stream must live on the plan's GPU.");
+    if (tempBytes < k.tempBytes || (k.tempBytes > 1 && temp == nullptr)) throw std::invalid_argument("CUB scan temporary storage is too small for the plan.");
+    ScopedGpu scoped(k.request.deviceNum);
+    char* base = static_cast<char*>(temp);
+    void* heads = k.headsBytes ? base : nullptr;
+    void* totals = k.statesBytes ? base + k.headsBytes : nullptr;
+    void* carries = k.statesBytes ? base + k.headsBytes + k.statesBytes : nullptr;
+    void* raw = stream.getStream();
+    if (k.clearKernel) {
+        if (offsets == nullptr) throw std::invalid_argument("CUB segmented scan requires segment offsets.");
+        const uint64_t words = (k.request.total + 31) / 32;
+        std::vector<void*> clearArgs = {&heads};
+        k.clearKernel->launch(static_cast<uint32_t>((words + 255) / 256), 1, 1, 256, raw, clearArgs);
+        std::vector<void*> markArgs = {&offsets, &heads};
+        k.markKernel->launch(static_cast<uint32_t>((k.request.segments + 1 + 255) / 256), 1, 1, 256, raw, markArgs);
+    }
+    if (k.carry) {
+        std::vector<void*> totalsArgs = {&input, &heads, &totals};
+        k.totalsKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, 256, raw, totalsArgs);
+        std::vector<void*> carriesArgs = {&totals, &carries};
+        k.carriesKernel->launch(1, 1, 1, 1024, raw, carriesArgs);
+    }
+    std::vector<void*> mainArgs = {&input, &heads, &carries, &outValue, &outIndex};
+    k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, 256, raw, mainArgs);
+}
+
+std::string cubScanKernelVariant(const std::shared_ptr<const CubScanKernels>& kernels) { return kernels ? kernels->variant : std::string(); }
+
+// ---- the reference's plan / run entry points ----------------------------------------------------------------------------------
+namespace {
+
+struct Checked {
+    ScanRequest request;
+    TensorPlacement placement;
+};
+
+// shared validation (reference: validateExclusiveSum and the checks of each prepare function)
+Checked check(const Tensor& input, const Tensor& output, const Tensor* offsets, uint64_t numItems, uint64_t numSegments, uint64_t segmentSize,
+              bool uniform, bool arg) {
+    if (!input.isInitialized() || !output.isInitialized()) throw std::invalid_argument("CUB scan requires initialized input and output tensors.");
+    if (input.getPlacement().getMemDevice() != TensorPlacement::MemDevices::GPU || input.getPlacement() != output.getPlacement()) {
+        throw std::invalid_argument("CUB scan input and output must live on the same GPU.");
+    }
+    if (!isCubScanDTypeSupported(input.getDataType())) {
+        throw std::invalid_argument(std::string("Unsupported CUB scan dtype ") + dataTypeName(input.getDataType()) + ".");
+    }
+    if (arg ? output.getDataType() != DataType::UINT32 : output.getDataType() != input.getDataType()) {
+        throw std::invalid_argument(arg ? "CUB arg scan output must be UINT32." : "CUB scan input and output dtypes must match.");
+    }
+    if (numItems == 0) throw std::invalid_argument("CUB scan requires at least one element.");
+    if (input.getTotalNumElements() < numItems || output.getTotalNumElements() < numItems) {
+        throw std::invalid_argument("CUB scan num_items exceeds the input or output tensor.");
+    }
+    if (!input.isDenseContiguous() || !output.isDenseContiguous()) throw std::invalid_argument("CUB scan requires dense tensors.");
+    Checked c;
+    c.placement = input.getPlacement();
+    ScanRequest& r = c.request;
+    r.dtype = input.getDataType();
+    r.total = numItems;
+    r.deviceNum = static_cast<int>(input.getPlacement().getDeviceNum());
+    r.alignmentBytes = std::min(pointerAlignment(input.getMemPtr()), pointerAlignment(output.getMemPtr()));
+    if (offsets) {
+        if (!offsets->isInitialized() || offsets->getPlacement() != input.getPlacement() || !offsets->isDenseContiguous()) {
+            throw std::invalid_argument("CUB segmented scan offsets must be a dense tensor on the input's GPU.");
+        }
+        if (!isCubSegmentOffsetDTypeSupported(offsets->getDataType())) throw std::invalid_argument("CUB segmented scan offsets must be UINT32 or UINT64.");
+        if (numSegments == 0 || offsets->getTotalNumElements() < numSegments + 1) {
+            throw std::invalid_argument("CUB segmented scan offsets must hold num_segments + 1 entries.");
+        }
+        r.row = 0;
+        r.segments = numSegments;
+        r.offsets64 = offsets->getDataType() == DataType::UINT64;
+    } else if (uniform) {
+        if (numSegments == 0 || segmentSize == 0 || numSegments * segmentSize != numItems) {
+            throw std::invalid_argument("CUB uniform segmented scan requires num_items == num_segments * segment_size.");
+        }
+        r.row = segmentSize;
+        r.segments = numSegments;
+    } else {
+        r.row = numItems;
+        r.segments = 1;
+    }
+    return c;
+}
+
+void fill(ScanRequest& r, CubScanOp op, CubScanMode mode, CubScanDirection direction) {
+    r.op = static_cast<int>(op);
+    r.writeValue = true;
+    r.writeIndex = false;
+    r.inclusive = mode == CubScanMode::Inclusive;
+    r.reverse = direction == CubScanDirection::Reverse;
+}
+void fill(ScanRequest& r, CubArgScanOp op, CubScanMode mode, CubScanDirection direction) {
+    r.op = op == CubArgScanOp::ArgMin ? 1 : 2;
+    r.writeValue = false;
+    r.writeIndex = true;
+    r.inclusive = mode == CubScanMode::Inclusive;
+    r.reverse = direction == CubScanDirection::Reverse;
+}
+
+template <typename Plan>
+void run(const Plan& plan, const Tensor& temp, const Tensor& input, Tensor& output, const Tensor* offsets, bool arg, Stream& stream) {
+    if (!plan.kernels) throw std::invalid_argument("CUB scan plan was not prepared.");
+    if (input.getDataType() != plan.dtype || input.getPlacement() != plan.placement || output.getPlacement() != plan.placement ||
+        input.getTotalNumElements() < plan.num_items || output.getTotalNumElements() < plan.num_items) {
+        throw std::invalid_argument("CUB scan tensors do not match the plan.");
+    }
+    if (std::min(pointerAlignment(input.getMemPtr()), pointerAlignment(output.getMemPtr())) < plan.kernels->request.alignmentBytes) {
+        throw std::invalid_argument("CUB scan tensors are less aligned than the tensors the plan was prepared for.");
+    }
+    if (plan.temp_storage_bytes > 1 && (!temp.isInitialized() || temp.getPlacement() != plan.placement ||
+                                        temp.getTotalNumElements() * dataTypeSizeInBytes(temp.getDataType()) < plan.temp_storage_bytes)) {
+        throw std::invalid_argument("CUB scan temporary storage is too small for the plan.");
+    }
+    void* tempPtr = temp.isInitialized() ? const_cast<Tensor&>(temp).getMemPtr() : nullptr;
+    const size_t tempBytes = temp.isInitialized() ? temp.getTotalNumElements() * dataTypeSizeInBytes(temp.getDataType()) : 1;
+    launchScan(*plan.kernels, input.getMemPtr(), offsets ? offsets->getMemPtr() : nullptr, tempPtr, tempBytes, arg ? nullptr : output.getMemPtr(),
+               arg ? output.getMemPtr() : nullptr, stream);
+}
+
+}  // namespace
+
+#define THOR_SCAN_PLAN_COMMON(plan, checked, opValue, modeValue, directionValue) \
+    plan.placement = checked.placement;                                          \
+    plan.dtype = checked.request.dtype;                                          \
+    plan.num_items = numItems;                                                   \
+    plan.op = opValue;                                                           \
+    plan.mode = modeValue;                                                       \
+    plan.direction = directionValue;                                             \
+    plan.kernels = buildScanKernels(checked.request);                            \
+    plan.temp_storage_bytes = plan.kernels->tempBytes
+
+CubDeviceScanPlan prepareCubDeviceScan(const Tensor& input, const Tensor& output, uint64_t numItems, CubScanOp op, CubScanMode mode,
+                                       CubScanDirection direction) {
+    Checked c = check(input, output, nullptr, numItems, 1, numItems, false, false);
+    fill(c.request, op, mode, direction);
+    CubDeviceScanPlan plan;
+    THOR_SCAN_PLAN_COMMON(plan, c, op, mode, direction);
+    return plan;
+}
+size_t cubDeviceScanTempBytes(const Tensor& input, const Tensor& output, uint64_t numItems, CubScanOp op, CubScanMode mode, CubScanDirection direction) {
+    return prepareCubDeviceScan(input, output, numItems, op, mode, direction).temp_storage_bytes;
+}
+void cubDeviceScan(const CubDeviceScanPlan& plan, const Tensor& temp, const Tensor& input, Tensor& output, Stream& stream) {
+    run(plan, temp, input, output, nullptr, false, stream);
+}
+
+CubDeviceArgScanPlan prepareCubDeviceArgScan(const Tensor& input, const Tensor& output, uint64_t numItems, CubArgScanOp op, CubScanMode mode,
+                                             CubScanDirection direction) {
+    Checked c = check(input, output, nullptr, numItems, 1, numItems, false, true);
+    fill(c.request, op, mode, direction);
+    CubDeviceArgScanPlan plan;
+    THOR_SCAN_PLAN_COMMON(plan, c, op, mode, direction);
+    return plan;
+}
+size_t cubDeviceArgScanTempBytes(const Tensor& input, const Tensor& output, uint64_t numItems, CubArgScanOp op, CubScanMode mode,
+                                 CubScanDirection direction) {
+    return prepareCubDeviceArgScan(input, output, numItems, op, mode, direction).temp_storage_bytes;
+}
+void cubDeviceArgScan(const CubDeviceArgScanPlan& plan, const Tensor& temp, const Tensor& input, Tensor& output, Stream& stream) {
+    run(plan, temp, input, output, nullptr, true, stream);
+}
+
+CubDeviceSegmentedUniformScanPlan prepareCubDeviceSegmentedUniformScan(const Tensor& input, const Tensor& output, uint64_t numItems,
+                                                                       uint64_t numSegments, uint64_t segmentSize, CubScanOp op, CubScanMode mode,
+                                                                       CubScanDirection direction) {
+    Checked c = check(input, output, nullptr, numItems, numSegments, segmentSize, true, false);
+    fill(c.request, op, mode, direction);
+    CubDeviceSegmentedUniformScanPlan plan;
+    THOR_SCAN_PLAN_COMMON(plan, c, op, mode, direction);
+    plan.num_segments = numSegments;
+    plan.segment_size = segmentSize;
+    return plan;
+}
+size_t cubDeviceSegmentedUniformScanTempBytes(const Tensor& input, const Tensor& output, uint64_t numItems, uint64_t numSegments, uint64_t segmentSize,
+                                              CubScanOp op, CubScanMode mode, CubScanDirection direction) {
+    return prepareCubDeviceSegmentedUniformScan(input, output, numItems, numSegments, segmentSize, op, mode, direction).temp_storage_bytes;
+}
+void cubDeviceSegmentedUniformScan(const CubDeviceSegmentedUniformScanPlan& plan, const Tensor& temp, const Tensor& input, Tensor& output,
+                                   Stream& stream) {
+    run(plan, temp, input, output, nullptr, false, stream);
+}
+
+CubDeviceSegmentedUniformArgScanPlan prepareCubDeviceSegmentedUniformArgScan(const Tensor& input, const Tensor& output, uint64_t numItems,
+                                                                             uint64_t numSegments, uint64_t segmentSize, CubArgScanOp op,
+                                                                             CubScanMode mode, CubScanDirection direction) {
+    Checked c = check(input, output, nullptr, numItems, numSegments, segmentSize, true, true);
+    fill(c.request, op, mode, direction);
+    CubDeviceSegmentedUniformArgScanPlan plan;
+    THOR_SCAN_PLAN_COMMON(plan, c, op, mode, direction);
+    plan.num_segments = numSegments;
+    plan.segment_size = segmentSize;
+    return plan;
+}
+size_t cubDeviceSegmentedUniformArgScanTempBytes(const Tensor& input, const Tensor& output, uint64_t numItems, uint64_t numSegments,
+                                                 uint64_t segmentSize, CubArgScanOp op, CubScanMode mode, CubScanDirection direction) {
+    return prepareCubDeviceSegmentedUniformArgScan(input, output, numItems, numSegments, segmentSize, op, mode, direction).temp_storage_bytes;
+}
+void cubDeviceSegmentedUniformArgScan(const CubDeviceSegmentedUniformArgScanPlan& plan, const Tensor& temp, const Tensor& input, Tensor& output,
+                                      Stream& stream) {
+    run(plan, temp, input, output, nullptr, true, stream);
+}
+
+CubDeviceSegmentedScanPlan prepareCubDeviceSegmentedScan(const Tensor& input, const Tensor& output, const Tensor& offsets, uint64_t numItems,
+                                                         uint64_t numSegments, CubScanOp op, CubScanMode mode, CubScanDirection direction) {
+    Checked c = check(input, output, &offsets, numItems, numSegments, 0, false, false);
+    fill(c.request, op, mode, direction);
+    CubDeviceSegmentedScanPlan plan;
+    THOR_SCAN_PLAN_COMMON(plan, c, op, mode, direction);
+    plan.num_segments = numSegments;
+    plan.offset_dtype = offsets.getDataType();
+    return plan;
+}
+size_t cubDeviceSegmentedScanTempBytes(const Tensor& input, const Tensor& output, const Tensor& offsets, uint64_t numItems, uint64_t numSegments,
+                                       CubScanOp op, CubScanMode mode, CubScanDirection direction) {
+    return prepareCubDeviceSegmentedScan(input, output, offsets, numItems, numSegments, op, mode, direction).temp_storage_bytes;
+}
+void cubDeviceSegmentedScan(const CubDeviceSegmentedScanPlan& plan, const Tensor& temp, const Tensor& input, Tensor& output, const Tensor& offsets,
+                            Stream& stream) {
+    if (offsets.getDataType() != plan.offset_dtype || offsets.getTotalNumElements() < plan.num_segments + 1) {
+        throw std::invalid_argument("CUB segmented scan offsets do not match the plan.");
+    }
+    run(plan, temp, input, output, &offsets, false, stream);
+}
+
+CubDeviceSegmentedArgScanPlan prepareCubDeviceSegmentedArgScan(const Tensor& input, const Tensor& output, const Tensor& offsets, uint64_t numItems,
+                                                               uint64_t numSegments, CubArgScanOp op, CubScanMode mode,
+                                                               CubScanDirection direction) {
+    Checked c = check(input, output, &offsets, numItems, numSegments, 0, false, true);
+    fill(c.request, op, mode, direction);
+    CubDeviceSegmentedArgScanPlan plan;
+    THOR_SCAN_PLAN_COMMON(plan, c, op, mode, direction);
+    plan.num_segments = numSegments;
+    plan.offset_dtype = offsets.getDataType();
+    return plan;
+}
+size_t cubDeviceSegmentedArgScanTempBytes(const Tensor& input, const Tensor& output, const Tensor& offsets, uint64_t numItems, uint64_t numSegments,
+                                          CubArgScanOp op, CubScanMode mode, CubScanDirection direction) {
+    return prepareCubDeviceSegmentedArgScan(input, output, offsets, numItems, numSegments, op, mode, direction).temp_storage_bytes;
+}
+void cubDeviceSegmentedArgScan(const CubDeviceSegmentedArgScanPlan& plan, const Tensor& temp, const Tensor& input, Tensor& output,
+                               const Tensor& offsets, Stream& stream) {
+    if (offsets.getDataType() != plan.offset_dtype || offsets.getTotalNumElements() < plan.num_segments + 1) {
+        throw std::invalid_argument("CUB segmented scan offsets do not match the plan.");
+    }
+    run(plan, temp, input, output, &offsets, true, stream);
+}
+
+}  // namespace ThorImplementation

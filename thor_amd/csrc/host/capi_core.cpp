@@ -3,6 +3,7 @@
 
 #include "ReductionPlanner.h"
 #include "Utilities/Expression/SegmentedBroadcastKernel.h"
+#include "Utilities/TensorOperations/Cub/CubDevicePrimitives.h"
 #include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
 
 #include <cstring>
@@ -294,6 +295,50 @@ int thor_segmented_broadcast(thor_tensor_t per_segment_values, thor_tensor_t seg
                       require(stream, "stream");
                       launchSegmentedBroadcast(per_segment_values->tensor, segment_offsets->tensor, output->tensor, normalize_by_segment_length != 0,
                                                stream->stream);)
+}
+
+int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments, uint64_t segment_size,
+              int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity) {
+    THOR_CAPI_TRY_INT(
+        require(input, "input"); require(output, "output"); require(stream, "stream");
+        if (op < 0 || op > 3 || (arg != 0 && op != 1 && op != 2)) throw std::invalid_argument("scan op must be 0..3 (1 or 2 for arg scans)");
+        const CubScanMode mode = inclusive ? CubScanMode::Inclusive : CubScanMode::Exclusive;
+        const CubScanDirection direction = reverse ? CubScanDirection::Reverse : CubScanDirection::Forward;
+        const CubScanOp valueOp = static_cast<CubScanOp>(op);
+        const CubArgScanOp argOp = op == 1 ? CubArgScanOp::ArgMin : CubArgScanOp::ArgMax;
+        const Tensor& in = input->tensor;
+        Tensor& out = output->tensor;
+        std::shared_ptr<const CubScanKernels> kernels;
+        if (offsets) {
+            if (arg) {
+                const auto plan = prepareCubDeviceSegmentedArgScan(in, out, offsets->tensor, num_items, num_segments, argOp, mode, direction);
+                cubDeviceSegmentedArgScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, offsets->tensor, stream->stream);
+                kernels = plan.kernels;
+            } else {
+                const auto plan = prepareCubDeviceSegmentedScan(in, out, offsets->tensor, num_items, num_segments, valueOp, mode, direction);
+                cubDeviceSegmentedScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, offsets->tensor, stream->stream);
+                kernels = plan.kernels;
+            }
+        } else if (segment_size > 0) {
+            if (arg) {
+                const auto plan = prepareCubDeviceSegmentedUniformArgScan(in, out, num_items, num_items / segment_size, segment_size, argOp, mode, direction);
+                cubDeviceSegmentedUniformArgScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+                kernels = plan.kernels;
+            } else {
+                const auto plan = prepareCubDeviceSegmentedUniformScan(in, out, num_items, num_items / segment_size, segment_size, valueOp, mode, direction);
+                cubDeviceSegmentedUniformScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+                kernels = plan.kernels;
+            }
+        } else if (arg) {
+            const auto plan = prepareCubDeviceArgScan(in, out, num_items, argOp, mode, direction);
+            cubDeviceArgScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+            kernels = plan.kernels;
+        } else {
+            const auto plan = prepareCubDeviceScan(in, out, num_items, valueOp, mode, direction);
+            cubDeviceScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+            kernels = plan.kernels;
+        }
+        if (variant) copyOut(cubScanKernelVariant(kernels), variant, variant_capacity, nullptr);)
 }
 
 }  // extern "C"
