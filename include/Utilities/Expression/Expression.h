@@ -72,6 +72,12 @@ inline bool isValueReductionOp(ExprOp op) {
 enum class SoftmaxAlgorithm : uint8_t { Fast = 0, Accurate = 1, Log = 2 };
 enum class SoftmaxMode : uint8_t { Instance = 0, Channel = 1 };
 
+// Prefix scans along the last axis (Expression.h:181-193 there).  ArgMin / ArgMax return the UINT32 flattened index of the
+// element that holds the running minimum / maximum (the first one among equals), 0xFFFFFFFF where the prefix is empty.
+enum class ScanOp : uint8_t { Sum = 0, Min = 1, Max = 2, Product = 3, ArgMin = 4, ArgMax = 5 };
+enum class ScanMode : uint8_t { Exclusive = 0, Inclusive = 1 };
+inline bool isArgScanOp(ScanOp op) { return op == ScanOp::ArgMin || op == ScanOp::ArgMax; }
+
 // reduction_axes entry standing for "every axis except axis 0"
 constexpr uint64_t kReduceAllAxesButFirst = UINT64_MAX - 1;
 
@@ -89,6 +95,9 @@ inline bool isSegmentedReduceOp(ExprOp op) {
 inline bool isWinnerRoutingOp(ExprOp op) { return op == ExprOp::REDUCE_MIN_BACKWARD || op == ExprOp::REDUCE_MAX_BACKWARD; }
 // Views of the operand's storage: nothing is computed, consumers read through the view's strides.
 inline bool isStorageViewOp(ExprOp op) { return op == ExprOp::STRIDED_VIEW || op == ExprOp::TRANSPOSE; }
+// SCAN: lhs scanned along its last axis.  SEGMENTED_SCAN: lhs = values [N], rhs = row-partition offsets [B + 1]; every segment
+// is scanned on its own.
+inline bool isScanOp(ExprOp op) { return op == ExprOp::SCAN || op == ExprOp::SEGMENTED_SCAN; }
 inline bool isRaggedOp(ExprOp op) {
     return isSegmentedReduceOp(op) || op == ExprOp::SEGMENTED_BROADCAST || op == ExprOp::RAGGED_VALUEWISE_EXTENT;
 }
@@ -116,6 +125,11 @@ struct ExprNode {
     // STRIDED_VIEW: shape, strides and first element of the view, in elements of the operand's storage
     std::vector<uint64_t> view_dims, view_strides;
     uint64_t view_element_offset = 0;
+    // SCAN / SEGMENTED_SCAN: scan_axis UINT64_MAX = the last axis
+    ScanOp scan_op = ScanOp::Sum;
+    ScanMode scan_mode = ScanMode::Inclusive;
+    uint64_t scan_axis = UINT64_MAX;
+    bool scan_reverse = false;
     SoftmaxAlgorithm softmax_algorithm = SoftmaxAlgorithm::Accurate;  // SOFTMAX only
     SoftmaxMode softmax_mode = SoftmaxMode::Channel;
 
@@ -332,6 +346,21 @@ class Expression {
     }
     // The last two axes exchanged (rank >= 2), as a view.
     Expression transpose() const;
+    // Prefix scans along the last axis (axis = -1 or the index of the last axis), and over the segments of a row partition
+    // (values [N], offsets [B + 1]); `reverse` scans from the end of every row / segment.  Values are UINT32, FP16, BF16 or
+    // FP32 and keep their dtype; arg scans return UINT32 (Expression.h:640-700, Expression.cpp:3866-3960 there).
+    Expression scan(ScanOp op = ScanOp::Sum, int64_t axis = -1, bool inclusive = true) const;
+    static Expression scan(const Expression& input, ScanOp op, int64_t axis = -1, bool inclusive = true) { return input.scan(op, axis, inclusive); }
+    Expression reverseScan(ScanOp op, int64_t axis = -1, bool inclusive = true) const;
+    Expression prefixCount(bool inclusive = true, int64_t axis = -1) const;  // running count of non-zero elements, UINT32
+    std::pair<Expression, Expression> scanWithIndices(ScanOp op, int64_t axis = -1, bool inclusive = true) const;  // {values, indices}, Min / Max
+    Expression segmentedScan(const Expression& offsets, ScanOp op = ScanOp::Sum, bool inclusive = true, bool reverse = false) const;
+    static Expression segmentedScan(const Expression& input, const Expression& offsets, ScanOp op, bool inclusive = true, bool reverse = false) {
+        return input.segmentedScan(offsets, op, inclusive, reverse);
+    }
+    static Expression segmentedScanWithRaggedMetadata(const Expression& input, const Expression& offsets, ScanOp op, bool inclusive, bool reverse,
+                                                      uint64_t ragged_batch_size, uint64_t ragged_max_active_values);
+    std::pair<Expression, Expression> segmentedScanWithIndices(const Expression& offsets, ScanOp op, bool inclusive = true, bool reverse = false) const;
     // Gather along one axis (the last one for axis = -1): the result has the shape of `indices` (UINT32 / UINT64), which
     // matches this tensor on every other axis; result[c] = this[c with the axis coordinate replaced by indices[c]]
     // (Expression.h:676-677, Expression.cpp:3856-3865 there).  The axis is kept in reduction_axes ({UINT64_MAX} = last).

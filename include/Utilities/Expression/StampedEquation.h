@@ -132,8 +132,27 @@ class StampedSegmentedReductionStage {
     std::shared_ptr<StampedCubSegmentedReduction> stamped;
 };
 
+// A prefix scan bound to its tensors: values along the last axis, or over the segments of an offsets tensor read at every run.
+struct CubScanKernels;
+class StampedScan {
+   public:
+    StampedScan(std::shared_ptr<const CubScanKernels> kernels, Tensor input, std::optional<Tensor> offsets, Tensor temp, Tensor output, bool indexOutput)
+        : kernels(std::move(kernels)), input(std::move(input)), offsets(std::move(offsets)), temp(std::move(temp)), output(std::move(output)),
+          indexOutput(indexOutput) {}
+    void runOn(Stream& stream) const;
+    Tensor getOutputTensor() const { return output; }
+    std::string getKernelVariant() const;
+
+   private:
+    std::shared_ptr<const CubScanKernels> kernels;
+    Tensor input;
+    std::optional<Tensor> offsets;
+    Tensor temp, output;
+    bool indexOutput;
+};
+
 struct StampedExecutionStage {
-    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction, SegmentedReduction, SegmentedBroadcast, ReduceMinMaxBackward };
+    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction, SegmentedReduction, SegmentedBroadcast, ReduceMinMaxBackward, Scan };
     static std::string kindToString(Kind kind) {
         switch (kind) {
             case Kind::FusedKernel:
@@ -154,6 +173,8 @@ struct StampedExecutionStage {
                 return "SegmentedBroadcast";
             case Kind::ReduceMinMaxBackward:
                 return "ReduceMinMaxBackward";
+            case Kind::Scan:
+                return "Scan";
         }
         return "<unknown>";
     }
@@ -167,6 +188,7 @@ struct StampedExecutionStage {
     std::shared_ptr<StampedFusedReduction> fused_reduction;
     std::shared_ptr<StampedSegmentedReductionStage> segmented_reduction;
     std::shared_ptr<StampedSegmentedBroadcast> segmented_broadcast;
+    std::shared_ptr<StampedScan> scan;
     // Kind::Copy: a named output that is only a view of an input is copied into the caller's tensor
     Tensor copySource, copyDestination;
 

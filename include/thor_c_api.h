@@ -171,6 +171,9 @@ thor_expr_t thor_expr_reduce(const char* method, thor_expr_t input, const uint64
                              int num_squeeze_axes);
 /* Expression::stridedView: dims / strides / offset in elements of the operand's storage ("transpose" is a unary method). */
 thor_expr_t thor_expr_strided_view(thor_expr_t input, const uint64_t* dims, const uint64_t* strides, int rank, uint64_t element_offset);
+/* Expression::scan / segmentedScan (Expression.h:640-700 there): op 0 sum, 1 min, 2 max, 3 product, 4 arg-min, 5 arg-max;
+ * offsets == NULL: scan along the last axis (axis -1 or its index); else a scan over the segments of the offsets expression */
+thor_expr_t thor_expr_scan(thor_expr_t input, thor_expr_t offsets, int op, int64_t axis, int inclusive, int reverse);
 /* Expression::takeAlongAxis(indices, axis) (Expression.h:676-677 there); axis = -1 is the last axis */
 thor_expr_t thor_expr_take_along_axis(thor_expr_t input, thor_expr_t indices, int64_t axis);
 thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank);

@@ -209,6 +209,21 @@ class BackwardGraph {
         d[0] = rows;
         return push(std::move(n), d);
     }
+    // the scan `like` describes, over `values` (and the same offsets), in the other direction
+    uint32_t oppositeScan(uint32_t values, uint32_t offsets, const ExprNode& like) {
+        ExprNode n;
+        n.op = like.op;
+        n.lhs = values;
+        n.rhs = offsets;
+        n.scan_op = like.scan_op;
+        n.scan_mode = like.scan_mode;
+        n.scan_axis = like.scan_axis;
+        n.scan_reverse = !like.scan_reverse;
+        n.ragged_runtime_batch_size = like.ragged_runtime_batch_size;
+        n.ragged_runtime_max_active_values = like.ragged_runtime_max_active_values;
+        n.ragged_runtime_elements_per_value = like.ragged_runtime_elements_per_value;
+        return push(std::move(n), dims[values]);
+    }
     uint32_t raggedExtent(uint32_t values, uint32_t offsets, const ExprNode& like) {
         ExprNode n;
         n.op = ExprOp::RAGGED_VALUEWISE_EXTENT;
@@ -257,7 +272,7 @@ class BackwardGraph {
 
 std::string noRule(ExprOp op) { return "Thor expressions autodiff does not support backward for op " + opName(op) + "."; }
 
-bool usesRowPartition(ExprOp op) { return isRaggedOp(op); }
+bool usesRowPartition(ExprOp op) { return isRaggedOp(op) || op == ExprOp::SEGMENTED_SCAN; }
 
 // input names that feed row-partition offsets: structure, not data
 std::unordered_set<std::string> rowPartitionInputs(const PhysicalExpression& forward) {
@@ -513,6 +528,13 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
                 break;
             case ExprOp::RAGGED_VALUEWISE_EXTENT:
                 contribute(n.lhs, b.raggedExtent(g, b.value(n.rhs), n));
+                break;
+            case ExprOp::SCAN:
+            case ExprOp::SEGMENTED_SCAN:
+                // element j feeds every later prefix (the later ones only, when exclusive): its gradient is the same scan of the
+                // upstream gradient run from the other end
+                if (n.scan_op != ScanOp::Sum) throw std::runtime_error(noRule(n.op) + " Only sum scans are differentiable here.");
+                contribute(n.lhs, b.oppositeScan(g, n.op == ExprOp::SEGMENTED_SCAN ? b.value(n.rhs) : kNone, n));
                 break;
 
             default:

@@ -3,6 +3,8 @@
 // CubSegmentedScan.cu for the uniform-segment and offset-segment forms).
 #include "CubScanInternal.h"
 
+#include "Utilities/Expression/StampedEquation.h"
+
 #include "ReductionPlanner.h"
 #include "Utilities/Common/ScopedGpu.h"
 #include "thorhip_numeric_embed.h"
@@ -155,6 +157,13 @@ void launchScan(const CubScanKernels& k, const void* input, const void* offsets,
     std::vector<void*> mainArgs = {&input, &heads, &carries, &outValue, &outIndex};
     k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, 256, raw, mainArgs);
 }
+
+void StampedScan::runOn(Stream& stream) const {
+    Tensor& out = const_cast<Tensor&>(output);
+    launchScan(*kernels, input.getMemPtr(), offsets.has_value() ? offsets->getMemPtr() : nullptr, const_cast<Tensor&>(temp).getMemPtr(),
+               temp.getTotalNumElements(), indexOutput ? nullptr : out.getMemPtr(), indexOutput ? out.getMemPtr() : nullptr, stream);
+}
+std::string StampedScan::getKernelVariant() const { return kernels->variant; }
 
 std::string cubScanKernelVariant(const std::shared_ptr<const CubScanKernels>& kernels) { return kernels ? kernels->variant : std::string(); }
 

@@ -503,6 +503,73 @@ Expression Expression::stridedView(const std::vector<uint64_t>& dims, const std:
     return out;
 }
 
+// ---- scans -----------------------------------------------------------------------------------------------------------------
+namespace {
+void validateScanOp(ScanOp op, const char* api) {
+    if (static_cast<uint8_t>(op) > static_cast<uint8_t>(ScanOp::ArgMax)) throw std::invalid_argument(std::string(api) + " received an unsupported ScanOp.");
+}
+ScanOp indexOpOf(ScanOp op, const char* api) {
+    if (op == ScanOp::Min) return ScanOp::ArgMin;
+    if (op == ScanOp::Max) return ScanOp::ArgMax;
+    throw std::invalid_argument(std::string(api) + " supports only ScanOp::Min and ScanOp::Max.");
+}
+}  // namespace
+
+Expression Expression::scan(ScanOp op, int64_t axis, bool inclusive) const {
+    if (axis < -1) throw std::invalid_argument("Expression::scan currently supports only axis=-1 or an explicit non-negative final axis.");
+    validateScanOp(op, "Expression::scan");
+    Expression out = unaryOp(*this, ExprOp::SCAN);
+    ExprNode& node = out.expr->nodes[out.nodeIndex];
+    node.scan_op = op;
+    node.scan_mode = inclusive ? ScanMode::Inclusive : ScanMode::Exclusive;
+    node.scan_axis = axis < 0 ? UINT64_MAX : static_cast<uint64_t>(axis);
+    return out;
+}
+
+Expression Expression::reverseScan(ScanOp op, int64_t axis, bool inclusive) const {
+    Expression out = scan(op, axis, inclusive);
+    out.expr->nodes[out.nodeIndex].scan_reverse = true;
+    return out;
+}
+
+Expression Expression::prefixCount(bool inclusive, int64_t axis) const { return cast(DataType::UINT32).scan(ScanOp::Sum, axis, inclusive); }
+
+std::pair<Expression, Expression> Expression::scanWithIndices(ScanOp op, int64_t axis, bool inclusive) const {
+    const ScanOp indexOp = indexOpOf(op, "Expression::scanWithIndices");
+    return {scan(op, axis, inclusive), scan(indexOp, axis, inclusive)};
+}
+
+Expression Expression::segmentedScan(const Expression& offsets, ScanOp op, bool inclusive, bool reverse) const {
+    validateScanOp(op, "Expression::segmentedScan");
+    Expression out = binaryOp(*this, offsets, ExprOp::SEGMENTED_SCAN);
+    ExprNode& node = out.expr->nodes[out.nodeIndex];
+    node.scan_op = op;
+    node.scan_mode = inclusive ? ScanMode::Inclusive : ScanMode::Exclusive;
+    node.scan_axis = UINT64_MAX;
+    node.scan_reverse = reverse;
+    return out;
+}
+
+Expression Expression::segmentedScanWithRaggedMetadata(const Expression& input, const Expression& offsets, ScanOp op, bool inclusive, bool reverse,
+                                                       uint64_t ragged_batch_size, uint64_t ragged_max_active_values) {
+    if ((ragged_batch_size == 0) != (ragged_max_active_values == 0)) {
+        throw std::invalid_argument("Segmented scan ragged metadata requires both batch size and max active values, or neither.");
+    }
+    Expression out = input.segmentedScan(offsets, op, inclusive, reverse);
+    if (ragged_batch_size != 0) {
+        ExprNode& node = out.expr->nodes.at(out.nodeIndex);
+        node.ragged_runtime_batch_size = ragged_batch_size;
+        node.ragged_runtime_max_active_values = ragged_max_active_values;
+        node.ragged_runtime_elements_per_value = 1;
+    }
+    return out;
+}
+
+std::pair<Expression, Expression> Expression::segmentedScanWithIndices(const Expression& offsets, ScanOp op, bool inclusive, bool reverse) const {
+    const ScanOp indexOp = indexOpOf(op, "Expression::segmentedScanWithIndices");
+    return {segmentedScan(offsets, op, inclusive, reverse), segmentedScan(offsets, indexOp, inclusive, reverse)};
+}
+
 Expression Expression::takeAlongAxis(const Expression& indices, int64_t axis) const {
     if (axis < -1) throw std::invalid_argument("Expression::takeAlongAxis currently supports only axis=-1 or an explicit non-negative axis.");
     Expression out = binaryOp(*this, indices, ExprOp::TAKE_ALONG_AXIS);
@@ -658,7 +725,7 @@ std::string opName(ExprOp op) {
         {(uint16_t)ExprOp::SEGMENTED_REDUCE_SUM, "segmented_reduce_sum"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MIN, "segmented_reduce_min"},
         {(uint16_t)ExprOp::SEGMENTED_REDUCE_MAX, "segmented_reduce_max"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MEAN, "segmented_reduce_mean"},
         {(uint16_t)ExprOp::STRIDED_VIEW, "strided_view"}, {(uint16_t)ExprOp::TRANSPOSE, "transpose"},
-        {(uint16_t)ExprOp::TAKE_ALONG_AXIS, "take_along_axis"}, {(uint16_t)ExprOp::REDUCE_MIN_BACKWARD, "reduce_min_backward"}, {(uint16_t)ExprOp::REDUCE_MAX_BACKWARD, "reduce_max_backward"},
+        {(uint16_t)ExprOp::TAKE_ALONG_AXIS, "take_along_axis"}, {(uint16_t)ExprOp::SCAN, "scan"}, {(uint16_t)ExprOp::SEGMENTED_SCAN, "segmented_scan"}, {(uint16_t)ExprOp::REDUCE_MIN_BACKWARD, "reduce_min_backward"}, {(uint16_t)ExprOp::REDUCE_MAX_BACKWARD, "reduce_max_backward"},
         {(uint16_t)ExprOp::SEGMENTED_BROADCAST, "segmented_broadcast"}, {(uint16_t)ExprOp::RAGGED_VALUEWISE_EXTENT, "ragged_valuewise_extent"},
     };
     auto it = names.find(static_cast<uint16_t>(op));
@@ -718,6 +785,11 @@ std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex,
         if (isCommutative(n.op) && kids.size() == 2 && kids[1] < kids[0]) std::swap(kids[0], kids[1]);
         text += dtypes();
         if (n.op == ExprOp::TAKE_ALONG_AXIS) text += ":axis=" + axesText(n.reduction_axes);
+        if (isScanOp(n.op)) {
+            static const char* const scanNames[] = {"sum", "min", "max", "product", "arg_min", "arg_max"};
+            text += std::string(":") + scanNames[static_cast<int>(n.scan_op)] + (n.scan_mode == ScanMode::Inclusive ? ":inclusive" : ":exclusive") +
+                    (n.scan_reverse ? ":reverse" : "") + ":axis=" + (n.scan_axis == UINT64_MAX ? std::string("last") : std::to_string(n.scan_axis));
+        }
         if (isReductionOp(n.op) || isWinnerRoutingOp(n.op)) text += ":axes=" + axesText(n.reduction_axes) + ":squeeze=" + axesText(n.squeeze_axes);
         if (n.op == ExprOp::RESHAPE) text += ":dims=" + axesText(n.reshape_dims);
         if (n.op == ExprOp::UNSQUEEZE) text += ":axes=" + axesText(n.unsqueeze_axes);

@@ -29,7 +29,7 @@ bool isBindableInputDType(DataType dtype) {
 }
 
 void rejectUnsupportedOp(ExprOp op) {
-    if (isRaggedOp(op) || isStorageViewOp(op) || isWinnerRoutingOp(op) || op == ExprOp::TAKE_ALONG_AXIS) return;
+    if (isRaggedOp(op) || isStorageViewOp(op) || isWinnerRoutingOp(op) || op == ExprOp::TAKE_ALONG_AXIS || isScanOp(op)) return;
     if (Expression::isLeafOp(op) || Expression::isUnaryOp(op) || Expression::isBinaryOp(op) || Expression::isTernaryOp(op)) {
         if (op != ExprOp::TENSOR_RUNTIME_SCALAR) return;
     }
@@ -39,7 +39,7 @@ void rejectUnsupportedOp(ExprOp op) {
 std::vector<DataType> tensorParentDTypes(const ExprNode& node, const std::vector<ExprNode>& nodes, const std::vector<DataType>& resolved) {
     std::vector<DataType> out;
     if (isRaggedOp(node.op)) return {resolved.at(node.lhs)};  // the offsets are structure, not a value
-    if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS) return {resolved.at(node.lhs)};
+    if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(node.op)) return {resolved.at(node.lhs)};
     auto add = [&](uint32_t parent) {
         if (parent >= nodes.size()) throw std::runtime_error("Parent node index out of range during dtype resolution.");
         if (!isScalarLeaf(nodes[parent].op)) out.push_back(resolved[parent]);
@@ -89,6 +89,22 @@ DataType raggedOutputDType(const ExprNode& node, const std::vector<DataType>& re
 
 DataType nodeOutputDType(const ExprNode& node, const std::vector<ExprNode>& nodes, const std::vector<DataType>& resolved) {
     if (isRaggedOp(node.op)) return raggedOutputDType(node, resolved);
+    if (isScanOp(node.op)) {
+        // values keep their dtype, arg scans return flattened UINT32 indices; offsets are structure
+        const DataType in = resolved[node.lhs];
+        if (in != DataType::UINT32 && in != DataType::FP16 && in != DataType::BF16 && in != DataType::FP32) {
+            throw std::runtime_error(std::string("Expression scan requires UINT32, FP16, BF16 or FP32 values, received: ") + dataTypeName(in));
+        }
+        if (node.op == ExprOp::SEGMENTED_SCAN && resolved[node.rhs] != DataType::UINT32 && resolved[node.rhs] != DataType::UINT64) {
+            throw std::runtime_error(std::string("Expression segmented-scan offsets must have UINT32 or UINT64 dtype, received: ") +
+                                     dataTypeName(resolved[node.rhs]));
+        }
+        const DataType out = isArgScanOp(node.scan_op) ? DataType::UINT32 : in;
+        if (node.output_dtype.has_value() && node.output_dtype.value() != out) {
+            throw std::runtime_error("Expression scan output dtype is fixed by its input (UINT32 for arg scans).");
+        }
+        return out;
+    }
     if (node.op == ExprOp::TAKE_ALONG_AXIS) {
         const DataType indexType = resolved[node.rhs];
         if (indexType != DataType::UINT32 && indexType != DataType::UINT64) {
@@ -197,8 +213,8 @@ void propagateMaterialisedDTypes(PhysicalExpression& expr, const std::vector<uin
             // an explicit conversion boundary: the source keeps its own compute dtype
         } else if (node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST) {
             toParent(node.lhs);  // never into the offsets
-        } else if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS) {
-            // both operands are read as stored tensors: nothing to widen
+        } else if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(node.op)) {
+            // the operands are read as stored tensors: nothing to widen
         } else if (isReductionOp(node.op) || node.op == ExprOp::SOFTMAX || isSegmentedReduceOp(node.op)) {
             // the reduction's mandatory fp32 stays inside the reduction; its producer keeps its own policy
             const ExprNode& producer = expr.nodes.at(node.lhs);
@@ -251,7 +267,7 @@ void resolveInPlace(PhysicalExpression& expr, const std::vector<DataType>& rootD
         const DataType logicalIn = nodeLogicalInputDType(node, expr.nodes, resolved);
         DataType requested;
         if (node.op == ExprOp::CAST || isShapeOnly(node.op) || node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST ||
-            isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS) {
+            isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(node.op)) {
             requested = out;  // values pass through unchanged (a normalised broadcast divides in fp32 and rounds once)
         } else if (isSegmentedReduceOp(node.op)) {
             requested = DataType::FP32;
@@ -337,7 +353,7 @@ DataType toSupportedComputeDType(ExprOp op, DataType requested) {
         throw std::runtime_error("Unsupported boolean/comparison/where dtype in toSupportedComputeDType.");
     }
     if (op == ExprOp::CAST || isShapeOnly(op) || op == ExprOp::RAGGED_VALUEWISE_EXTENT || op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(op) ||
-        op == ExprOp::TAKE_ALONG_AXIS) {
+        op == ExprOp::TAKE_ALONG_AXIS || isScanOp(op)) {
         if (isBindableInputDType(requested)) return requested;
         throw std::runtime_error("Unsupported passthrough dtype in toSupportedComputeDType.");
     }

@@ -6,6 +6,7 @@
 #include "Utilities/Expression/FusedEquation.h"
 
 #include "AutoDiffInternal.h"
+#include "CubScanInternal.h"
 #include "HipSourceEmitter.h"
 #include "IndexGather.h"
 #include "ReductionPlanner.h"
@@ -58,7 +59,8 @@ std::string structuralKey(const ExprNode& n) {
       << "|" << (n.compute_dtype ? static_cast<int>(*n.compute_dtype) : -1) << "|" << axesKey(n.reduction_axes) << "|" << axesKey(n.squeeze_axes)
       << "|" << axesKey(n.unsqueeze_axes) << "|" << axesKey(n.reshape_dims) << "|" << axesKey(n.fill_dims) << "|" << n.ragged_runtime_batch_size << "|"
       << n.ragged_runtime_max_active_values << "|" << n.ragged_runtime_elements_per_value << "|" << n.segmented_broadcast_normalize_by_length << "|"
-      << axesKey(n.view_dims) << "|" << axesKey(n.view_strides) << "|" << n.view_element_offset;
+      << axesKey(n.view_dims) << "|" << axesKey(n.view_strides) << "|" << n.view_element_offset << "|" << static_cast<int>(n.scan_op) << "|"
+      << static_cast<int>(n.scan_mode) << "|" << n.scan_axis << "|" << n.scan_reverse;
     return k.str();
 }
 
@@ -147,6 +149,11 @@ class GraphBuilder {
         } else if (isWinnerRoutingOp(node.op)) {
             node.lhs = asTensorOperand(node.lhs, true);  // read by an arg reduction
             node.rhs = asTensorOperand(node.rhs, false);
+        } else if (isScanOp(node.op)) {
+            // the scan kernels stream dense storage
+            node.lhs = asTensorOperand(node.lhs, false);
+            if (isStorageViewOp(out.nodes[node.lhs].op)) node.lhs = castOf(node.lhs, out.nodes[node.lhs].output_dtype.value());
+            if (node.op == ExprOp::SEGMENTED_SCAN) node.rhs = asTensorOperand(node.rhs, false);
         } else if (node.op == ExprOp::TAKE_ALONG_AXIS) {
             node.lhs = asTensorOperand(node.lhs, false);
             node.rhs = asTensorOperand(node.rhs, false);
@@ -219,7 +226,7 @@ uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
 bool consumesGather(const ExprNode& consumer) {
     if (consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT || consumer.op == ExprOp::WHERE || consumer.op == ExprOp::CAST) return true;
     if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX || isWinnerRoutingOp(consumer.op) ||
-        consumer.op == ExprOp::TAKE_ALONG_AXIS) {
+        consumer.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(consumer.op)) {
         return false;
     }
     return Expression::isBinaryOp(consumer.op) || Expression::isUnaryOp(consumer.op);
@@ -337,6 +344,25 @@ std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpressio
                 if (n.ragged_runtime_max_active_values == 0) throw std::runtime_error("Segmented broadcast is missing its row capacity.");
                 dims[i] = dims[n.lhs];
                 dims[i][0] = n.ragged_runtime_max_active_values;
+                break;
+            }
+            case ExprOp::SCAN:
+                if (dims[n.lhs].empty()) throw std::runtime_error("Expression::scan requires a tensor of rank 1 or more.");
+                if (n.scan_axis != UINT64_MAX && n.scan_axis != dims[n.lhs].size() - 1) {
+                    throw std::runtime_error("Expression::scan currently supports only axis=-1 or an explicit non-negative final axis.");
+                }
+                dims[i] = dims[n.lhs];
+                break;
+            case ExprOp::SEGMENTED_SCAN: {
+                uint64_t elements = 1;
+                for (uint64_t d : dims[n.lhs]) elements *= d;
+                if (dims[n.lhs].empty() || elements != dims[n.lhs][0] || dims[n.rhs].size() != 1 || dims[n.rhs][0] < 2) {
+                    throw std::runtime_error("Segmented scan requires values [N] (one element per row) and offsets [B + 1] with at least one segment.");
+                }
+                if (n.ragged_runtime_batch_size != 0 && dims[n.rhs][0] != n.ragged_runtime_batch_size + 1) {
+                    throw std::runtime_error("Segmented scan offsets do not have the ragged descriptor's batch size + 1 entries.");
+                }
+                dims[i] = dims[n.lhs];
                 break;
             }
             case ExprOp::TAKE_ALONG_AXIS:
@@ -496,7 +522,11 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             } else if (isReductionOp(n.op)) {
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
-            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS) {
+            } else if (n.op == ExprOp::SCAN) {
+                graph->role[i] = Role::Materialized;
+                ensureTensor(n.lhs);
+            } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS ||
+                       n.op == ExprOp::SEGMENTED_SCAN) {
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
                 ensureTensor(n.rhs);
@@ -577,7 +607,10 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             std::vector<uint32_t> sources, scalars;
             if (isReductionOp(graph->expr.nodes[i].op)) {
                 sources.push_back(graph->expr.nodes[i].lhs);
-            } else if (isWinnerRoutingOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::TAKE_ALONG_AXIS) {
+            } else if (graph->expr.nodes[i].op == ExprOp::SCAN) {
+                sources.push_back(graph->expr.nodes[i].lhs);
+            } else if (isWinnerRoutingOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::TAKE_ALONG_AXIS ||
+                       graph->expr.nodes[i].op == ExprOp::SEGMENTED_SCAN) {
                 sources.push_back(graph->expr.nodes[i].lhs);
                 sources.push_back(graph->expr.nodes[i].rhs);
             } else if (isSegmentedReduceOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST) {
@@ -727,7 +760,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     auto runsInFusedKernel = [&](uint32_t i) {
         const ExprOp op = expr.nodes[i].op;
         return graph->role[i] == Role::Materialized && !isReductionOp(op) && !isSegmentedReduceOp(op) && op != ExprOp::SEGMENTED_BROADCAST &&
-               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && op != ExprOp::INPUT;
+               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && !isScanOp(op) && op != ExprOp::INPUT;
     };
     std::vector<uint32_t> levelOf = graph->level;
     if (stageFusionEnabled()) {
@@ -737,7 +770,9 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             std::vector<uint32_t> sources, scalars;
             if (isReductionOp(n.op)) {
                 sources.push_back(n.lhs);
-            } else if (isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS) {
+            } else if (n.op == ExprOp::SCAN) {
+                sources = {n.lhs};
+            } else if (isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS || n.op == ExprOp::SEGMENTED_SCAN) {
                 sources = {n.lhs, n.rhs};
             } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
                 if (graph->role[n.lhs] == Role::Inline) {
@@ -1126,6 +1161,52 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                         CubSegmentedReduction(op, n.output_dtype.value()).stampRuntimeOffsets(values, output, offsets, stream));
                 }
                 tensorOf[i] = output;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(stage));
+                done[i] = 1;
+                continue;
+            }
+            if (isScanOp(n.op)) {
+                if (fusedKernelsOnly) {
+                    throw std::runtime_error(
+                        "FusedEquation::run() only supports expressions that lower to fused kernels; this expression has a scan stage. "
+                        "Use stamp() and run the returned plan.");
+                }
+                const Tensor& values = tensorOf[n.lhs];
+                if (!values.isDenseContiguous()) throw std::runtime_error("Expression scan needs a dense operand.");
+                Tensor scanned = allocateFor(i);
+                ScanRequest request;
+                request.dtype = values.getDataType();
+                request.total = values.getTotalNumElements();
+                request.deviceNum = device_num;
+                const bool arg = isArgScanOp(n.scan_op);
+                request.op = arg ? (n.scan_op == ScanOp::ArgMin ? 1 : 2) : static_cast<int>(n.scan_op);
+                request.writeValue = !arg;
+                request.writeIndex = arg;
+                request.inclusive = n.scan_mode == ScanMode::Inclusive;
+                request.reverse = n.scan_reverse;
+                request.alignmentBytes = std::min(pointerAlignment(values.getMemPtr()), pointerAlignment(scanned.getMemPtr()));
+                std::optional<Tensor> offsets;
+                std::vector<uint32_t> stageSources{n.lhs};
+                if (n.op == ExprOp::SEGMENTED_SCAN) {
+                    offsets = tensorOf[n.rhs];
+                    if (!offsets->isDenseContiguous()) throw std::runtime_error("Segmented scan needs dense offsets.");
+                    request.row = 0;
+                    request.segments = offsets->getTotalNumElements() - 1;
+                    request.offsets64 = offsets->getDataType() == DataType::UINT64;
+                    stageSources.push_back(n.rhs);
+                } else {
+                    request.row = dims[n.lhs].back();
+                    request.segments = request.total / request.row;
+                }
+                const std::shared_ptr<const CubScanKernels> kernels = buildScanKernels(request);
+                Tensor temp(gpuPlacement, TensorDescriptor(DataType::UINT8, {std::max<uint64_t>(kernels->tempBytes, 1)}));
+                StampedExecutionStage stage;
+                stage.kind = StampedExecutionStage::Kind::Scan;
+                stage.gpu_num = device_num;
+                stage.dependency_stage_indices = dependenciesOf(stageSources);
+                stage.scan = std::make_shared<StampedScan>(kernels, values, offsets, temp, scanned, arg);
+                tensorOf[i] = scanned;
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
                 done[i] = 1;

@@ -170,6 +170,7 @@ uint64_t StampedExecutionStage::flopCount() const {
         case Kind::SegmentedReduction:
             return segmented_reduction ? segmented_reduction->flopCount() : 0;
         case Kind::SegmentedBroadcast:
+        case Kind::Scan:
             return 0;
     }
     return 0;
@@ -207,6 +208,10 @@ void StampedExecutionStage::runOn(Stream& stream, const std::unordered_map<std::
         case Kind::SegmentedBroadcast:
             if (!segmented_broadcast) throw std::runtime_error("Segmented broadcast stage is missing its stamped broadcast.");
             segmented_broadcast->runOn(stream);
+            return;
+        case Kind::Scan:
+            if (!scan) throw std::runtime_error("Scan stage is missing its stamped scan.");
+            scan->runOn(stream);
             return;
     }
 }

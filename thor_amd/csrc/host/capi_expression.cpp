@@ -185,6 +185,12 @@ thor_expr_t thor_expr_strided_view(thor_expr_t input, const uint64_t* dims, cons
                       return new thor_expr{input->expr.stridedView(std::vector<uint64_t>(dims, dims + rank), std::vector<uint64_t>(strides, strides + rank),
                                                                    element_offset)};)
 }
+thor_expr_t thor_expr_scan(thor_expr_t input, thor_expr_t offsets, int op, int64_t axis, int inclusive, int reverse) {
+    THOR_CAPI_TRY_PTR(require(input, "input"); if (op < 0 || op > 5) throw std::invalid_argument("scan op must be 0..5");
+                      const ScanOp scanOp = static_cast<ScanOp>(op);
+                      if (offsets) return new thor_expr{input->expr.segmentedScan(offsets->expr, scanOp, inclusive != 0, reverse != 0)};
+                      return new thor_expr{reverse ? input->expr.reverseScan(scanOp, axis, inclusive != 0) : input->expr.scan(scanOp, axis, inclusive != 0)};)
+}
 thor_expr_t thor_expr_take_along_axis(thor_expr_t input, thor_expr_t indices, int64_t axis) {
     THOR_CAPI_TRY_PTR(require(input, "input"); require(indices, "indices"); return new thor_expr{input->expr.takeAlongAxis(indices->expr, axis)};)
 }
@@ -300,6 +306,7 @@ int thor_plan_stage_description(thor_plan_t plan, int stage, char* buffer, size_
         if (s.fused_reduction) text = s.fused_reduction->getDescription();
         if (s.segmented_reduction) text = s.segmented_reduction->getStamped()->getKernelVariant();
         if (s.segmented_broadcast) text = s.segmented_broadcast->getKernelVariant();
+        if (s.scan) text = s.scan->getKernelVariant();
         copyOut(text, buffer, capacity, nullptr);)
 }
 uint64_t thor_plan_flop_count(thor_plan_t plan) { return plan ? plan->plan.flopCount() : 0; }

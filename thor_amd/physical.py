@@ -75,6 +75,7 @@ PROTOTYPES = {
     "thor_expr_reduce": (_vp, [_cp, _vp, _u64p, _i, _u64p, _i]), "thor_expr_reshape": (_vp, [_vp, _u64p, _i]),
     "thor_expr_strided_view": (_vp, [_vp, _u64p, _u64p, _i, ctypes.c_uint64]),
     "thor_expr_take_along_axis": (_vp, [_vp, _vp, ctypes.c_int64]),
+    "thor_expr_scan": (_vp, [_vp, _vp, _i, ctypes.c_int64, _i, _i]),
     "thor_expr_unsqueeze": (_vp, [_vp, _u64p, _i]), "thor_expr_squeeze": (_vp, [_vp, _u64p, _i]), "thor_expr_destroy": (None, [_vp]),
     "thor_expr_num_nodes": (_i, [_vp]), "thor_expr_canonical": (_i, [_vp, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_outputs_create": (_vp, [_cpp, _vpp, _i]), "thor_outputs_destroy": (None, [_vp]),
@@ -695,6 +696,30 @@ class Expression:
     def with_ragged_runtime_extent(self, offsets, batch_size: int, max_active_values: int, elements_per_value: int = 1):
         """The same values, computed only for the first offsets[batch_size] rows; the rest of the output keeps its contents."""
         return self._ragged("ragged_extent", offsets, batch_size, max_active_values, elements_per_value)
+
+    def scan(self, op: "ScanOp" = None, axis: int = -1, inclusive: bool = True, reverse: bool = False) -> "Expression":
+        """Prefix scan along the last axis; values keep their dtype, ``ScanOp.arg_min`` / ``arg_max`` return UINT32 flattened
+        indices (thor.physical.Expression.scan)."""
+        op = ScanOp.sum if op is None else op
+        return Expression(_handle(lib().thor_expr_scan(self._h, None, int(op), axis, int(inclusive), int(reverse)), "scan"))
+
+    def segmented_scan(self, offsets: "Expression", op: "ScanOp" = None, inclusive: bool = True, reverse: bool = False) -> "Expression":
+        op = ScanOp.sum if op is None else op
+        return Expression(_handle(lib().thor_expr_scan(self._h, offsets._h, int(op), -1, int(inclusive), int(reverse)), "segmented_scan"))
+
+    def scan_with_indices(self, op: "ScanOp", axis: int = -1, inclusive: bool = True):
+        if op not in (ScanOp.min, ScanOp.max):
+            raise ValueError("scan_with_indices supports only ScanOp.min and ScanOp.max")
+        return self.scan(op, axis, inclusive), self.scan(ScanOp.arg_min if op == ScanOp.min else ScanOp.arg_max, axis, inclusive)
+
+    def segmented_scan_with_indices(self, offsets: "Expression", op: "ScanOp", inclusive: bool = True, reverse: bool = False):
+        if op not in (ScanOp.min, ScanOp.max):
+            raise ValueError("segmented_scan_with_indices supports only ScanOp.min and ScanOp.max")
+        return (self.segmented_scan(offsets, op, inclusive, reverse),
+                self.segmented_scan(offsets, ScanOp.arg_min if op == ScanOp.min else ScanOp.arg_max, inclusive, reverse))
+
+    def prefix_count(self, inclusive: bool = True, axis: int = -1) -> "Expression":
+        return self.cast(DataType.uint32).scan(ScanOp.sum, axis, inclusive)
 
     def take_along_axis(self, indices: "Expression", axis: int = -1) -> "Expression":
         """Gather along one axis with UINT32 / UINT64 indices; the result has the shape of ``indices``."""
