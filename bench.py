@@ -303,6 +303,36 @@ def bench_other_configs():
     row_max_backward = ex.compile(ex.input("x").reduce_max(axis=1, squeeze=[1]), 0).compile_backward(["x"])
     plans = [row_max_backward.stamp({"x": t}, stream) for t in (x, clone(x), clone(x))]
     timed("backward_c3_row_max_fp32", [p_.run for p_ in plans], 8 * n, n, ">".join(plans[0].stage_kind_names()) + " " + " | ".join(plans[0].stage_descriptions()))
+    del plans
+
+    # ---- prefix scans (Expression.scan): bytes counted are the values read once and the result written once
+    from thor_amd.physical import ScanOp
+    xs3 = [x, clone(x), clone(x)]
+    row_sum = ex.compile(ex.input("x").scan(ScanOp.sum), 0)
+    plans = [row_sum.stamp({"x": t}, stream) for t in xs3]
+    timed("scan_c3_row_cumsum_fp32", [p_.run for p_ in plans], 8 * n, n, plans[0].stage_descriptions()[0])
+    row_argmax = ex.compile(ex.input("x").scan(ScanOp.arg_max), 0)
+    plans = [row_argmax.stamp({"x": t}, stream) for t in xs3]
+    timed("scan_c3_row_running_argmax_fp32", [p_.run for p_ in plans], 8 * n, n, plans[0].stage_descriptions()[0])
+    flat = ex.compile(ex.input("x").reshape([n]).scan(ScanOp.sum), 0)
+    plans = [flat.stamp({"x": t}, stream) for t in xs3]
+    timed("scan_flat_cumsum_fp32_2^26", [p_.run for p_ in plans], 8 * n, n, plans[0].stage_descriptions()[0])
+    del plans, xs3, x
+    xb = gpu_from(rng.standard_normal((16384, 4096), dtype=np.float32), DataType.bf16)
+    nb = 16384 * 4096
+    xb3 = [xb, clone(xb), clone(xb)]
+    plans = [row_sum.stamp({"x": t}, stream) for t in xb3]
+    timed("scan_c4_row_cumsum_bf16", [p_.run for p_ in plans], 4 * nb, nb, plans[0].stage_descriptions()[0])
+    del plans, xb3, xb
+    scalars = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [rows * 16]))
+    wide_offsets = ph.PhysicalTensor(ph.Placement(ph.DeviceType.cpu), ph.PhysicalTensor.Descriptor(DataType.uint32, [segments + 1]))
+    wide_offsets.numpy()[...] = host_offsets.numpy() * 16
+    ragged_offsets = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.uint32, [segments + 1]))
+    ragged_offsets.copy_from_async(wide_offsets, stream)
+    stream.synchronize()
+    ragged_sum = ex.compile(ex.input("v").segmented_scan(ex.input("o"), ScanOp.sum), 0)
+    plan = ragged_sum.stamp({"v": scalars, "o": ragged_offsets}, stream)
+    timed("scan_ragged_cumsum_fp32_2^26", plan.run, 8 * rows * 16, rows * 16, plan.stage_descriptions()[0])
     return results
 
 

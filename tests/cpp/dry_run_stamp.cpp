@@ -146,6 +146,13 @@ static int runAll() {
         stampBackward(std::string("backward ") + dtypeName + " row max", x.reduce_max({1}, {1}), inputs, rowGradient, stream);
         stampBackward(std::string("backward ") + dtypeName + " column min of exp", x.exp().reduce_min({0}, {}),
                       inputs, Tensor(gpuPlacement, TensorDescriptor(dtype, {1, 24})), stream);
+        // scans along the last axis, forward and as the backward of a sum scan; arg scans
+        if (dtype != DataType::FP8_E4M3) {
+            stampOne(std::string("scan ") + dtypeName + " running max of a * b", (x * y).scan(ScanOp::Max), inputs, stream, "FusedKernel,Scan");
+            stampOne(std::string("scan ") + dtypeName + " exclusive sum - argmin", x.scan(ScanOp::Sum, -1, false), inputs, stream, "Scan");
+            stampOne(std::string("scan ") + dtypeName + " argmin", x.scan(ScanOp::ArgMin), inputs, stream, "Scan");
+            stampBackward(std::string("backward ") + dtypeName + " sum scan", x.scan(ScanOp::Sum), inputs, fullGradient, stream, "Scan");
+        }
         // gathers along an axis, with indices the same equation computes
         stampOne(std::string("gather ") + dtypeName + " value at the row argmax", (x * y).takeAlongAxis(x.argmax({1}, {}), 1), inputs, stream);
         stampOne(std::string("gather ") + dtypeName + " column picks", x.takeAlongAxis(y.argmin({0}, {}), 0) + 1.0, inputs, stream);

@@ -10,6 +10,7 @@
 #include "Utilities/Expression/AutoDiff.h"
 #include "Utilities/Expression/FusedEquation.h"
 #include "Utilities/Expression/RaggedExpression.h"
+#include "Utilities/TensorOperations/Cub/CubDevicePrimitives.h"
 #include "Utilities/TensorOperations/Cub/CubReduction.h"
 #include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
 
@@ -288,6 +289,41 @@ static void autodiffGraphStructure() {
     CHECK((normalizeBackwardWrtNames(*ragged.expr, {}) == std::vector<std::string>{"x"}));
 }
 
+static void scanExpressionStructure() {
+    // Expression::scan builds a SCAN node that carries op, mode and axis (Expression.cpp:3908-3922 there); arg scans resolve to
+    // UINT32, value scans keep the input dtype; segmented scans take offsets as structure
+    const Expression x = Expression::input("x"), offsets = Expression::input("offsets");
+    PhysicalOutputs scan = Expression::outputs({{"y", x.scan(ScanOp::Max, -1, false)}}).physicalOutputs();
+    const ExprNode& node = scan.expr->nodes.at(scan.outputs[0].node_idx);
+    CHECK(node.op == ExprOp::SCAN && node.scan_op == ScanOp::Max && node.scan_mode == ScanMode::Exclusive && node.scan_axis == UINT64_MAX && !node.scan_reverse);
+    resolveOutputsDTypesInPlace(scan, {DataType::BF16});
+    CHECK(scan.expr->nodes.at(scan.outputs[0].node_idx).output_dtype == DataType::BF16);
+    PhysicalOutputs arg = Expression::outputs({{"y", x.segmentedScan(offsets, ScanOp::ArgMin, true, true)}}).physicalOutputs();
+    const ExprNode& argNode = arg.expr->nodes.at(arg.outputs[0].node_idx);
+    CHECK(argNode.op == ExprOp::SEGMENTED_SCAN && argNode.scan_reverse && arg.expr->nodes.at(argNode.rhs).op == ExprOp::INPUT);
+    resolveOutputsDTypesInPlace(arg, {DataType::FP32, DataType::UINT64});
+    CHECK(arg.expr->nodes.at(arg.outputs[0].node_idx).output_dtype == DataType::UINT32);
+    CHECK(throwsAs<std::runtime_error>([&] {
+        PhysicalOutputs bad = Expression::outputs({{"y", x.scan(ScanOp::Sum)}}).physicalOutputs();
+        resolveOutputsDTypesInPlace(bad, {DataType::INT32});
+    }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)x.scan(ScanOp::Sum, -2); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)x.scanWithIndices(ScanOp::Sum); }));
+    const auto [values, indices] = x.scanWithIndices(ScanOp::Min);
+    CHECK(values.expression().nodes.back().scan_op == ScanOp::Min && indices.expression().nodes.back().scan_op == ScanOp::ArgMin);
+    const PhysicalExpression count = (x > Expression(0.0)).prefixCount().expression();
+    CHECK(count.nodes.back().op == ExprOp::SCAN && count.nodes.at(count.nodes.back().lhs).op == ExprOp::CAST);
+    // the gradient of a sum scan is the scan from the other end (AutoDiff.cpp there: reverse-scan lowering)
+    const PhysicalOutputs forward = Expression::outputs({{"y", x.scan(ScanOp::Sum, -1, false)}}).physicalOutputs();
+    const PhysicalOutputs backward = buildBackwardOutputs(forward, {"x"}, std::string("__grad_output"), {{{"x", {3, 5}}}});
+    bool reversed = false;
+    for (const ExprNode& n : backward.expr->nodes) reversed = reversed || (n.op == ExprOp::SCAN && n.scan_reverse && n.scan_mode == ScanMode::Exclusive);
+    CHECK(reversed);
+    CHECK(throwsAs<std::runtime_error>([&] {
+        (void)buildBackwardOutputs(Expression::outputs({{"y", x.scan(ScanOp::Max)}}).physicalOutputs(), {"x"}, std::nullopt, {{{"x", {3, 5}}}});
+    }));
+}
+
 static void raggedExpressionStructure() {
     // RaggedExpressionTest.cpp:739-795,907-957,2037-2055 there: names, descriptors and markers, no device work
     const RaggedTensorDescriptor descriptor(DataType::FP32, {4}, 3, 9);
@@ -512,6 +548,64 @@ static void autodiffExecution(Stream& stream) {
     CHECK(throwsAs<std::runtime_error>([&] { (void)implicit.compileBackward({"x"}); }));  // no second derivative of a backward equation
 }
 
+static void devicePrefixScans(Stream& stream) {
+    // cubDeviceScan / cubDeviceSegmentedUniformScan / cubDeviceSegmentedScan and arg forms: plan, temporary storage, run
+    // (CubDevicePrimitivesTest.cpp there; literal vectors of test_expression_scan.py / test_expression_segmented_scan.py)
+    auto upload = [&](const std::vector<uint32_t>& v, const std::vector<uint64_t>& dims) {
+        Tensor host(cpuPlacement, TensorDescriptor(DataType::UINT32, dims));
+        std::memcpy(host.getMemPtr<uint32_t>(), v.data(), v.size() * 4);
+        Tensor device(gpuPlacement, TensorDescriptor(DataType::UINT32, dims));
+        device.copyFromAsync(host, stream);
+        stream.synchronize();
+        return device;
+    };
+    const Tensor rows = upload({2, 3, 1, 4, 5, 1, 2, 3}, {2, 4});
+    Tensor out(gpuPlacement, TensorDescriptor(DataType::UINT32, {2, 4}));
+    auto uniform = [&](CubScanOp op, CubScanMode mode, CubScanDirection direction = CubScanDirection::Forward) {
+        const CubDeviceSegmentedUniformScanPlan plan = prepareCubDeviceSegmentedUniformScan(rows, out, 8, 2, 4, op, mode, direction);
+        CHECK(plan.temp_storage_bytes >= 1 && plan.num_segments == 2 && plan.segment_size == 4 && plan.dtype == DataType::UINT32);
+        CHECK(cubDeviceSegmentedUniformScanTempBytes(rows, out, 8, 2, 4, op, mode, direction) == plan.temp_storage_bytes);
+        const Tensor temp = allocateCubTemporaryStorage(gpuPlacement, plan.temp_storage_bytes);
+        cubDeviceSegmentedUniformScan(plan, temp, rows, out, stream);
+        return toHostRaw<uint32_t>(out, stream);
+    };
+    CHECK((uniform(CubScanOp::Sum, CubScanMode::Inclusive) == std::vector<uint32_t>{2, 5, 6, 10, 5, 6, 8, 11}));
+    CHECK((uniform(CubScanOp::Sum, CubScanMode::Exclusive) == std::vector<uint32_t>{0, 2, 5, 6, 0, 5, 6, 8}));
+    CHECK((uniform(CubScanOp::Min, CubScanMode::Exclusive) == std::vector<uint32_t>{0xffffffffu, 2, 2, 1, 0xffffffffu, 5, 1, 1}));
+    CHECK((uniform(CubScanOp::Max, CubScanMode::Inclusive) == std::vector<uint32_t>{2, 3, 3, 4, 5, 5, 5, 5}));
+    CHECK((uniform(CubScanOp::Product, CubScanMode::Inclusive) == std::vector<uint32_t>{2, 6, 6, 24, 5, 5, 10, 30}));
+    CHECK((uniform(CubScanOp::Sum, CubScanMode::Inclusive, CubScanDirection::Reverse) == std::vector<uint32_t>{10, 8, 5, 4, 11, 6, 5, 3}));
+    // one flat scan over the same eight elements
+    const CubDeviceScanPlan flat = prepareCubDeviceScan(rows, out, 8, CubScanOp::Sum, CubScanMode::Inclusive);
+    cubDeviceScan(flat, allocateCubTemporaryStorage(gpuPlacement, flat.temp_storage_bytes), rows, out, stream);
+    CHECK((toHostRaw<uint32_t>(out, stream) == std::vector<uint32_t>{2, 5, 6, 10, 15, 16, 18, 21}));
+    // segments of an offsets tensor, and the flattened index of the running maximum
+    const Tensor values = upload({8, 6, 7, 5, 3, 2, 9}, {7}), offsets = upload({0, 2, 5, 7}, {4});
+    Tensor ragged(gpuPlacement, TensorDescriptor(DataType::UINT32, {7}));
+    const CubDeviceSegmentedScanPlan segmented = prepareCubDeviceSegmentedScan(values, ragged, offsets, 7, 3, CubScanOp::Max, CubScanMode::Exclusive);
+    CHECK(segmented.offset_dtype == DataType::UINT32 && segmented.num_segments == 3);
+    cubDeviceSegmentedScan(segmented, allocateCubTemporaryStorage(gpuPlacement, segmented.temp_storage_bytes), values, ragged, offsets, stream);
+    CHECK((toHostRaw<uint32_t>(ragged, stream) == std::vector<uint32_t>{0, 8, 0, 7, 7, 0, 2}));
+    const CubDeviceSegmentedArgScanPlan winners = prepareCubDeviceSegmentedArgScan(values, ragged, offsets, 7, 3, CubArgScanOp::ArgMin, CubScanMode::Inclusive);
+    cubDeviceSegmentedArgScan(winners, allocateCubTemporaryStorage(gpuPlacement, winners.temp_storage_bytes), values, ragged, offsets, stream);
+    CHECK((toHostRaw<uint32_t>(ragged, stream) == std::vector<uint32_t>{0, 1, 2, 3, 4, 5, 5}));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceSegmentedUniformScan(rows, out, 8, 3, 3, CubScanOp::Sum, CubScanMode::Inclusive); }));
+    CHECK(throwsAs<std::invalid_argument>([&] {
+        cubDeviceScan(flat, allocateCubTemporaryStorage(gpuPlacement, 1), rows, out, stream);  // flat over 8 elements needs no storage: one chunk
+        const Tensor big(gpuPlacement, TensorDescriptor(DataType::UINT32, {1 << 20}));
+        Tensor bigOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {1 << 20}));
+        const CubDeviceScanPlan carried = prepareCubDeviceScan(big, bigOut, 1 << 20, CubScanOp::Sum, CubScanMode::Inclusive);
+        cubDeviceScan(carried, allocateCubTemporaryStorage(gpuPlacement, 1), big, bigOut, stream);  // too little temporary storage
+    }));
+    CHECK(isCubScanDTypeSupported(DataType::BF16) && !isCubScanDTypeSupported(DataType::INT32) && isCubSegmentOffsetDTypeSupported(DataType::UINT64));
+    // through the Expression: one Scan stage
+    const FusedEquation running = FusedEquation::compile(Expression::outputs({{"y", Expression::input("x").scan(ScanOp::Max)}}).physicalOutputs(), 0);
+    StampedExecutionPlan plan = running.stamp({{"x", rows}}, stream);
+    CHECK((plan.stageKindNames() == std::vector<std::string>{"Scan"}));
+    plan.run();
+    CHECK((toHostRaw<uint32_t>(plan.output("y"), stream) == std::vector<uint32_t>{2, 3, 3, 4, 5, 5, 5, 5}));
+}
+
 static void softmaxPlansAndRowKernel(Stream& stream) {
     const uint64_t rows = 7, cols = 130;
     std::vector<float> x(rows * cols);
@@ -591,7 +685,8 @@ int main(int argc, char** argv) {
                                {"dtypeResolutionAndStageSplit", dtypeResolutionAndStageSplit},
                                {"cpuTypeConverter", cpuTypeConverter},
                                {"raggedExpressionStructure", raggedExpressionStructure},
-                               {"autodiffGraphStructure", autodiffGraphStructure}};
+                               {"autodiffGraphStructure", autodiffGraphStructure},
+                               {"scanExpressionStructure", scanExpressionStructure}};
     if (mode == "gpu") {
         auto withStream = [](void (*f)(Stream&)) {
             return [f] {
@@ -606,6 +701,7 @@ int main(int argc, char** argv) {
         cases.push_back({"expressionConfig1AndRuntimeScalars", withStream(expressionConfig1AndRuntimeScalars)});
         cases.push_back({"softmaxPlansAndRowKernel", withStream(softmaxPlansAndRowKernel)});
         cases.push_back({"autodiffExecution", withStream(autodiffExecution)});
+        cases.push_back({"devicePrefixScans", withStream(devicePrefixScans)});
         cases.push_back({"typeConverterOnGpuAndTensorViews", withStream(typeConverterOnGpuAndTensorViews)});
     }
     for (const Case& c : cases) {
