@@ -68,7 +68,7 @@ def check(got, carrier, dtype, op, inclusive, reverse, **segments):
     slack = magnitude.astype(np.float64).reshape(-1) * unit * 2 + (64 * 2.0 ** -24) * magnitude.astype(np.float64).reshape(-1) + 1e-30
     assert np.all(np.abs(gotf - reference.astype(np.float64).reshape(-1)) <= slack)
 
-SHAPES = [("rows", (300, 64)), ("rows", (9, 1000)), ("rows", (5, 4099)), ("rows", (3, 70000)), ("rows", (2048, 3)), ("flat", (1, 100003)), ("flat", (1, 1 << 20))]
+SHAPES = [("rows", (300, 64)), ("rows", (5, 4099)), ("rows", (3, 70000)), ("rows", (2048, 3)), ("flat", (1, 1 << 20))]
 
 
 @pytest.mark.parametrize("reverse", [False, True], ids=["forward", "reverse"])

@@ -87,15 +87,34 @@ __device__ __forceinline__ ScanState<Cfg> scanShuffleUp(const ScanState<Cfg>& s,
     return r;
 }
 
-// inclusive scan of one state per lane across the wavefront
-template <typename Cfg>
-__device__ __forceinline__ ScanState<Cfg> scanWave(ScanState<Cfg> s, int lane) {
-#pragma unroll
-    for (int delta = 1; delta < kWave; delta *= 2) {
-        const ScanState<Cfg> earlier = scanShuffleUp<Cfg>(s, delta);
-        const ScanState<Cfg> merged = scanCombine<Cfg>(earlier, s);
-        if (lane >= delta) s = merged;
-    }
+// Lane-to-lane moves of the data-parallel primitive kind: the value of the lane `shift` places earlier inside a row of 16
+// lanes (CTRL 0x110 + shift), lane 15 of the previous row (0x142, rows 1 and 3) or lane 31 (0x143, rows 2 and 3).  Lanes
+// with no source, and rows outside ROW_MASK, receive `empty`.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ u32 scanMoveBits(u32 empty, u32 x) {
+    return (u32)__builtin_amdgcn_update_dpp((int)empty, (int)x, CTRL, ROW_MASK, 0xf, false);
+}
+template <typename Cfg, bool WITH_HEAD, int CTRL, int ROW_MASK>
+__device__ __forceinline__ ScanState<Cfg> scanStep(const ScanState<Cfg>& s) {
+    typedef typename Cfg::Acc Acc;
+    ScanState<Cfg> earlier;
+    earlier.v = __builtin_bit_cast(Acc, scanMoveBits<CTRL, ROW_MASK>(__builtin_bit_cast(u32, scanIdentity<Cfg>()), __builtin_bit_cast(u32, s.v)));
+    earlier.i = (Cfg::kOp == 1 || Cfg::kOp == 2) ? scanMoveBits<CTRL, ROW_MASK>(kNoIndex, s.i) : kNoIndex;
+    earlier.head = WITH_HEAD ? scanMoveBits<CTRL, ROW_MASK>(0u, s.head) : 0u;
+    return scanCombine<Cfg>(earlier, s);  // an empty earlier state leaves s as it is
+}
+
+// Inclusive scan of one state per lane across the wavefront: four steps inside rows of 16 lanes, then the total of row 0
+// into row 1 and of row 2 into row 3, then the total of the lower half into the upper half.  WITH_HEAD = false: no state
+// holds a segment head except possibly lane 0's (which nothing is combined into), so the head words stay where they are.
+template <typename Cfg, bool WITH_HEAD = true>
+__device__ __forceinline__ ScanState<Cfg> scanWave(ScanState<Cfg> s) {
+    s = scanStep<Cfg, WITH_HEAD, 0x111, 0xf>(s);
+    s = scanStep<Cfg, WITH_HEAD, 0x112, 0xf>(s);
+    s = scanStep<Cfg, WITH_HEAD, 0x114, 0xf>(s);
+    s = scanStep<Cfg, WITH_HEAD, 0x118, 0xf>(s);
+    s = scanStep<Cfg, WITH_HEAD, 0x142, 0xa>(s);
+    s = scanStep<Cfg, WITH_HEAD, 0x143, 0xc>(s);
     return s;
 }
 
@@ -152,6 +171,8 @@ __device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* 
     typedef ScanState<Cfg> S;
     constexpr int V = Cfg::kVec, ITEMS = Cfg::kItems, THREADS = Cfg::kThreads, WAVES = THREADS / kWave;
     static_assert(ITEMS * WAVES <= kWave, "the wavefront totals of a chunk are scanned by one wavefront");
+    // rows that start only where a round of the block starts (or one flat scan): heads need not travel between lanes
+    constexpr bool kPlain = Cfg::kRow != 0 && (Cfg::kRow % ((u64)THREADS * V) == 0 || Cfg::kRow == Cfg::kTotal);
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const u64 chunkBase = (u64)blockIdx.x * Cfg::kChunkElems;
 
@@ -195,7 +216,15 @@ __device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* 
                 sealed[it] |= run.head << k;
             }
         }
-        const S inclusive = scanWave<Cfg>(run, lane);
+        S inclusive;
+        if (kPlain) {
+            // only the first lane of the block can hold a head in this round, and nothing is combined into it
+            const u32 roundHead = (chunkBase + (u64)it * THREADS * V) % Cfg::kRow == 0 ? 1u : 0u;
+            inclusive = scanWave<Cfg, false>(run);
+            inclusive.head = wave == 0 ? roundHead : 0u;
+        } else {
+            inclusive = scanWave<Cfg, true>(run);
+        }
         laneExclusive[it] = scanShuffleUp<Cfg>(inclusive, 1);
         if (lane == 0) laneExclusive[it] = scanEmpty<Cfg>();
         if (lane == kWave - 1) {
@@ -212,7 +241,7 @@ __device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* 
             mine.i = totalIndex[lane];
             mine.head = totalHead[lane];
         }
-        const S inclusive = scanWave<Cfg>(mine, lane);
+        const S inclusive = scanWave<Cfg>(mine);
         if (AGGREGATE_ONLY) {
             if (lane == kWave - 1) scanStoreState<Cfg>(aggregates, blockIdx.x, inclusive);
         } else {
@@ -263,9 +292,21 @@ __device__ __forceinline__ void scanCarries(const void* aggregates, void* carrie
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const u64 first = (u64)threadIdx.x * PER;
     __shared__ u32 totalValue[WAVES], totalIndex[WAVES], totalHead[WAVES];
+    // a thread's totals are loaded at once (independent loads), then folded from registers
+    constexpr bool kHeld = PER <= 32;
+    S held[kHeld ? PER : 1];
+    if (kHeld) {
+#pragma unroll
+        for (u64 j = 0; j < PER; ++j) held[j] = first + j < Cfg::kChunks ? scanLoadState<Cfg>(aggregates, first + j) : scanEmpty<Cfg>();
+    }
     S run = scanEmpty<Cfg>();
-    for (u64 c = first; c < first + PER && c < Cfg::kChunks; ++c) run = scanCombine<Cfg>(run, scanLoadState<Cfg>(aggregates, c));
-    const S inclusive = scanWave<Cfg>(run, lane);
+    if (kHeld) {
+#pragma unroll
+        for (u64 j = 0; j < PER; ++j) run = scanCombine<Cfg>(run, held[j]);
+    } else {
+        for (u64 c = first; c < first + PER && c < Cfg::kChunks; ++c) run = scanCombine<Cfg>(run, scanLoadState<Cfg>(aggregates, c));
+    }
+    const S inclusive = scanWave<Cfg>(run);
     S before = scanShuffleUp<Cfg>(inclusive, 1);
     if (lane == 0) before = scanEmpty<Cfg>();
     if (lane == kWave - 1) {
@@ -283,9 +324,17 @@ __device__ __forceinline__ void scanCarries(const void* aggregates, void* carrie
         earlierWaves = scanCombine<Cfg>(earlierWaves, t);
     }
     run = scanCombine<Cfg>(earlierWaves, before);
-    for (u64 c = first; c < first + PER && c < Cfg::kChunks; ++c) {
-        scanStoreState<Cfg>(carries, c, run);
-        run = scanCombine<Cfg>(run, scanLoadState<Cfg>(aggregates, c));
+    if (kHeld) {
+#pragma unroll
+        for (u64 j = 0; j < PER; ++j) {
+            if (first + j < Cfg::kChunks) scanStoreState<Cfg>(carries, first + j, run);
+            run = scanCombine<Cfg>(run, held[j]);
+        }
+    } else {
+        for (u64 c = first; c < first + PER && c < Cfg::kChunks; ++c) {
+            scanStoreState<Cfg>(carries, c, run);
+            run = scanCombine<Cfg>(run, scanLoadState<Cfg>(aggregates, c));
+        }
     }
 }
 

@@ -10,6 +10,7 @@
 #include "thorhip_numeric_embed.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <numeric>
 #include <sstream>
 #include <stdexcept>
@@ -58,24 +59,30 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r) {
     const uint32_t elementBytes = dataTypeSizeInBytes(r.dtype);
     uint64_t vec = 16 / elementBytes;
     while (vec > 1 && (r.total % vec != 0 || r.alignmentBytes % (vec * std::max<uint32_t>(elementBytes, r.writeIndex ? 4 : elementBytes)) != 0)) vec /= 2;
-    const uint64_t threads = 256, lanesWorth = threads * vec;
+    uint64_t threads = 256;
+    if (const char* env = std::getenv("THOR_SCAN_THREADS")) {  // tuning switch: 256, 512 or 1024 threads per block
+        const long requested = std::atol(env);
+        if (requested == 256 || requested == 512 || requested == 1024) threads = static_cast<uint64_t>(requested);
+    }
+    const uint64_t lanesWorth = threads * vec, maxItems = 64 / (threads / 64) < 16 ? 64 / (threads / 64) : 16;
     uint64_t items = 4;
     uint64_t chunkElems = lanesWorth * items;
     k.carry = true;
-    if (!ragged && r.row <= lanesWorth * 16) {
+    if (!ragged && r.row <= lanesWorth * maxItems) {
         // chunks of whole rows: every chunk starts at a head and needs nothing from its predecessors
         const uint64_t step = vec / std::gcd(r.row, vec);  // rows per chunk must keep chunk starts on vector boundaries
         uint64_t rowsPerChunk = std::max<uint64_t>(lanesWorth * 4 / r.row / step * step, step);
-        if (rowsPerChunk * r.row <= lanesWorth * 16) {
+        if (rowsPerChunk * r.row <= lanesWorth * maxItems) {
             chunkElems = rowsPerChunk * r.row;
             items = (chunkElems + lanesWorth - 1) / lanesWorth;
             k.carry = false;
         }
     }
     if (k.carry) {
-        items = 8;
+        items = std::min<uint64_t>(8, maxItems);
         chunkElems = lanesWorth * items;
     }
+    k.threads = static_cast<uint32_t>(threads);
     k.chunks = (r.total + chunkElems - 1) / chunkElems;
     if (k.chunks == 1) k.carry = false;
     if (k.chunks > 0x7fffffffull) throw std::invalid_argument("CUB scan: too many elements for one launch.");
@@ -99,10 +106,10 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r) {
       << ";\n    static constexpr thor::u64 kChunkElems = " << chunkElems << "ull;\n    static constexpr thor::u64 kChunks = " << k.chunks
       << "ull;\n    static constexpr bool kCarry = " << (k.carry ? "true" : "false") << ";\n    static constexpr bool kWriteValue = "
       << (r.writeValue ? "true" : "false") << ";\n    static constexpr bool kWriteIndex = " << (r.writeIndex ? "true" : "false") << ";\n};\n}  // namespace gen\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_main(const gen::Cfg::T* in, const thor::u32* heads, const void* carries, "
+    s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void thor_scan_main(const gen::Cfg::T* in, const thor::u32* heads, const void* carries, "
          "gen::Cfg::T* outValue, thor::u32* outIndex) {\n    thor::scanChunk<gen::Cfg, false>(in, heads, carries, nullptr, outValue, outIndex);\n}\n";
     if (k.carry) {
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_totals(const gen::Cfg::T* in, const thor::u32* heads, void* totals) {\n"
+        s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void thor_scan_totals(const gen::Cfg::T* in, const thor::u32* heads, void* totals) {\n"
              "    thor::scanChunk<gen::Cfg, true>(in, heads, nullptr, totals, nullptr, nullptr);\n}\n";
         s << "extern \"C\" __global__ __launch_bounds__(1024) void thor_scan_carries(const void* totals, void* carries) {\n"
              "    thor::scanCarries<gen::Cfg>(totals, carries);\n}\n";
@@ -123,7 +130,7 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r) {
         k.markKernel = compileKernel(source, "thor_scan_mark_heads", r.deviceNum, false);
     }
     std::ostringstream variant;
-    variant << (ragged ? "segments" : r.row == r.total ? "flat" : "rows") << "(chunk=" << chunkElems << ",vec=" << vec << ",items=" << items
+    variant << (ragged ? "segments" : r.row == r.total ? "flat" : "rows") << "(chunk=" << chunkElems << ",vec=" << vec << ",items=" << items << ",threads=" << threads
             << ",grid=" << k.chunks << (k.carry ? ",passes=totals+carries+scan" : ",passes=scan") << (r.reverse ? ",reverse" : "") << ") ["
             << k.mainKernel->kernelName << "]";
     k.variant = variant.str();
@@ -150,12 +157,12 @@ void launchScan(const CubScanKernels& k, const void* input, const void* offsets,
     }
     if (k.carry) {
         std::vector<void*> totalsArgs = {&input, &heads, &totals};
-        k.totalsKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, 256, raw, totalsArgs);
+        k.totalsKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, totalsArgs);
         std::vector<void*> carriesArgs = {&totals, &carries};
         k.carriesKernel->launch(1, 1, 1, 1024, raw, carriesArgs);
     }
     std::vector<void*> mainArgs = {&input, &heads, &carries, &outValue, &outIndex};
-    k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, 256, raw, mainArgs);
+    k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, mainArgs);
 }
 
 void StampedScan::runOn(Stream& stream) const {

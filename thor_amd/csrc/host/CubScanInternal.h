@@ -27,6 +27,7 @@ struct CubScanKernels {
     ScanRequest request;
     std::shared_ptr<CompiledKernel> mainKernel, totalsKernel, carriesKernel, clearKernel, markKernel;
     uint64_t chunks = 1;
+    uint32_t threads = 256;
     bool carry = false;
     size_t headsBytes = 0, statesBytes = 0, tempBytes = 1;
     std::string variant;
