@@ -136,19 +136,24 @@ class StampedSegmentedReductionStage {
 struct CubScanKernels;
 class StampedScan {
    public:
+    // one output: the scanned values, or (indexOutput) the UINT32 indices of an arg scan
     StampedScan(std::shared_ptr<const CubScanKernels> kernels, Tensor input, std::optional<Tensor> offsets, Tensor temp, Tensor output, bool indexOutput)
-        : kernels(std::move(kernels)), input(std::move(input)), offsets(std::move(offsets)), temp(std::move(temp)), output(std::move(output)),
-          indexOutput(indexOutput) {}
+        : kernels(std::move(kernels)), input(std::move(input)), offsets(std::move(offsets)), temp(std::move(temp)) {
+        (indexOutput ? indices : values) = std::move(output);
+    }
+    // a min / max scan that writes the running values and the indices that hold them in one pass
+    StampedScan(std::shared_ptr<const CubScanKernels> kernels, Tensor input, std::optional<Tensor> offsets, Tensor temp, Tensor values, Tensor indices)
+        : kernels(std::move(kernels)), input(std::move(input)), offsets(std::move(offsets)), temp(std::move(temp)), values(std::move(values)),
+          indices(std::move(indices)) {}
     void runOn(Stream& stream) const;
-    Tensor getOutputTensor() const { return output; }
+    Tensor getOutputTensor() const { return values.isInitialized() ? values : indices; }
     std::string getKernelVariant() const;
 
    private:
     std::shared_ptr<const CubScanKernels> kernels;
     Tensor input;
     std::optional<Tensor> offsets;
-    Tensor temp, output;
-    bool indexOutput;
+    Tensor temp, values, indices;
 };
 
 struct StampedExecutionStage {

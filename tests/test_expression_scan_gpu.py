@@ -44,7 +44,7 @@ def test_scan_with_indices_returns_values_and_flattened_winner_indices(stream, n
     values = np.array([[3.0, 1.0, 4.0, 1.0], [2.0, 5.0, 0.0, 0.0]], np.float32)
     found, indices = ex.input("x").scan_with_indices(op=ScanOp[name], axis=-1, inclusive=inclusive)
     plan = stamp_run({"values": found, "indices": indices}, {"x": copy_numpy_to_gpu(values, stream, DataType.fp32)}, stream)
-    assert plan.stage_kind_names() == ["Scan", "Scan"]
+    assert plan.stage_kind_names() == ["Scan"]  # values and indices come from one pass
     expected_indices = oracle.scan(values, ORACLE_OP[ScanOp["arg_" + name]], inclusive, segment_size=4)
     np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("indices"), stream), expected_indices)
     np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("values"), stream), oracle.scan(values, ORACLE_OP[ScanOp[name]], inclusive, segment_size=4))
@@ -167,3 +167,18 @@ def test_validation(stream):
     with pytest.raises(RuntimeError, match="Only sum scans are differentiable"):
         ex.compile(ix.scan(ScanOp.max), device_num=0).compile_backward(["x"]).stamp({"x": x}, stream)
     stamp_run(ix.scan(ScanOp.sum, axis=1), {"x": x}, stream)  # the index of the last axis is accepted
+
+
+@pytest.mark.parametrize("inclusive", [True, False])
+@pytest.mark.parametrize("name", ["min", "max"])
+def test_segmented_scan_with_indices_is_one_stage(stream, name, inclusive):
+    """test_expression_arg_scan.py:180-228 there."""
+    values = np.array([8, 6, 7, 5, 3, 2, 9], np.uint32)
+    offsets = np.array([0, 2, 5, 7], np.uint32)
+    found, indices = ex.input("x").segmented_scan_with_indices(ex.input("offsets"), op=ScanOp[name], inclusive=inclusive)
+    plan = stamp_run({"values": found, "indices": indices},
+                     {"x": copy_numpy_to_gpu(values, stream, DataType.uint32), "offsets": copy_numpy_to_gpu(offsets, stream, DataType.uint32)}, stream)
+    assert plan.stage_kind_names() == ["Scan"]
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("values"), stream), oracle.scan(values, ORACLE_OP[ScanOp[name]], inclusive, offsets=offsets, dtype=oracle.UINT32))
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("indices"), stream),
+                                  oracle.scan(values, ORACLE_OP[ScanOp["arg_" + name]], inclusive, offsets=offsets, dtype=oracle.UINT32))

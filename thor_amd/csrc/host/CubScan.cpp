@@ -166,9 +166,9 @@ void launchScan(const CubScanKernels& k, const void* input, const void* offsets,
 }
 
 void StampedScan::runOn(Stream& stream) const {
-    Tensor& out = const_cast<Tensor&>(output);
     launchScan(*kernels, input.getMemPtr(), offsets.has_value() ? offsets->getMemPtr() : nullptr, const_cast<Tensor&>(temp).getMemPtr(),
-               temp.getTotalNumElements(), indexOutput ? nullptr : out.getMemPtr(), indexOutput ? out.getMemPtr() : nullptr, stream);
+               temp.getTotalNumElements(), values.isInitialized() ? const_cast<Tensor&>(values).getMemPtr() : nullptr,
+               indices.isInitialized() ? const_cast<Tensor&>(indices).getMemPtr() : nullptr, stream);
 }
 std::string StampedScan::getKernelVariant() const { return kernels->variant; }
 

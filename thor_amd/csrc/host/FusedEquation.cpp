@@ -1183,9 +1183,27 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 request.op = arg ? (n.scan_op == ScanOp::ArgMin ? 1 : 2) : static_cast<int>(n.scan_op);
                 request.writeValue = !arg;
                 request.writeIndex = arg;
+                // a min / max scan and the arg scan of the same operand (scanWithIndices) are one pass with two outputs
+                uint32_t partner = UINT32_MAX;
+                if (request.op == 1 || request.op == 2) {
+                    const ScanOp wanted = arg ? (request.op == 1 ? ScanOp::Min : ScanOp::Max) : (request.op == 1 ? ScanOp::ArgMin : ScanOp::ArgMax);
+                    for (uint32_t j = i + 1; j < expr.nodes.size() && partner == UINT32_MAX; ++j) {
+                        const ExprNode& m = expr.nodes[j];
+                        if (!done[j] && graph->role[j] == Role::Materialized && levelOf[j] == level && m.op == n.op && m.lhs == n.lhs && m.rhs == n.rhs &&
+                            m.scan_op == wanted && m.scan_mode == n.scan_mode && m.scan_reverse == n.scan_reverse) {
+                            partner = j;
+                        }
+                    }
+                }
+                Tensor partnerOutput;
+                if (partner != UINT32_MAX) {
+                    partnerOutput = allocateFor(partner);
+                    request.writeValue = request.writeIndex = true;
+                }
                 request.inclusive = n.scan_mode == ScanMode::Inclusive;
                 request.reverse = n.scan_reverse;
                 request.alignmentBytes = std::min(pointerAlignment(values.getMemPtr()), pointerAlignment(scanned.getMemPtr()));
+                if (partner != UINT32_MAX) request.alignmentBytes = std::min(request.alignmentBytes, pointerAlignment(partnerOutput.getMemPtr()));
                 std::optional<Tensor> offsets;
                 std::vector<uint32_t> stageSources{n.lhs};
                 if (n.op == ExprOp::SEGMENTED_SCAN) {
@@ -1205,7 +1223,14 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 stage.kind = StampedExecutionStage::Kind::Scan;
                 stage.gpu_num = device_num;
                 stage.dependency_stage_indices = dependenciesOf(stageSources);
-                stage.scan = std::make_shared<StampedScan>(kernels, values, offsets, temp, scanned, arg);
+                if (partner != UINT32_MAX) {
+                    stage.scan = std::make_shared<StampedScan>(kernels, values, offsets, temp, arg ? partnerOutput : scanned, arg ? scanned : partnerOutput);
+                    tensorOf[partner] = partnerOutput;
+                    stageOfNode[partner] = static_cast<int>(stages.size());
+                    done[partner] = 1;
+                } else {
+                    stage.scan = std::make_shared<StampedScan>(kernels, values, offsets, temp, scanned, arg);
+                }
                 tensorOf[i] = scanned;
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
