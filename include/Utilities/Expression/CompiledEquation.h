@@ -4,12 +4,22 @@
 //  Utilities/Expression/EquationCompiler.cpp:1916-1988 keeps the global kernel cache).
 #pragma once
 
+#include "DeepLearning/Implementation/Tensor/Tensor.h"
+
 #include <cstdint>
 #include <memory>
 #include <string>
 #include <vector>
 
 namespace ThorImplementation {
+
+// A scalar that lives in device memory: one element of `sourceDType` at `byteOffset` inside `buffer`, read by the kernels at
+// every run, so a stamped plan follows a value that other GPU work updates (reference: CompiledEquation.h:15-19 there).
+struct TensorScalarBinding {
+    Tensor buffer;
+    uint64_t byteOffset = 0;
+    DataType sourceDType = DataType::FP32;
+};
 
 // A loaded code object; unloaded when the last kernel handle that refers to it goes away (errors are swallowed).
 struct LoadedModule {

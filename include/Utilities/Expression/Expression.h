@@ -198,6 +198,10 @@ class Expression {
                             std::optional<DataType> output_dtype = std::nullopt);
     static Expression runtimeScalar(const std::string& name, std::optional<DataType> compute_dtype = std::nullopt,
                                     std::optional<DataType> output_dtype = std::nullopt);
+    // A scalar read from device memory at every run (bound with a TensorScalarBinding at stamp time); like a runtime scalar
+    // it takes no part in dtype promotion (Expression.cpp:3101-3120 there).
+    static Expression tensorRuntimeScalar(const std::string& name, std::optional<DataType> compute_dtype = std::nullopt,
+                                          std::optional<DataType> output_dtype = std::nullopt);
     static Expression constantScalar(double value);
     static Expression fill(double value, const std::vector<uint64_t>& dims, std::optional<DataType> output_dtype = std::nullopt);
 

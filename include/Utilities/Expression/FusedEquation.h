@@ -6,6 +6,7 @@
 #pragma once
 
 #include "Utilities/Cache/LruCache.h"
+#include "Utilities/Expression/CompiledEquation.h"
 #include "Utilities/Expression/Expression.h"
 #include "Utilities/Expression/StampedEquation.h"
 
@@ -26,9 +27,12 @@ class FusedEquation {
 
     // Binds tensors and returns a plan whose run() only launches.  Outputs are allocated here unless the caller passes
     // them in `preallocated_outputs` (shape and dtype are validated).
+    // `tensor_scalar_inputs` binds the equation's tensorRuntimeScalar inputs to elements of device buffers.
     [[nodiscard]] StampedExecutionPlan stamp(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                             const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs = {},
                                              const std::unordered_map<std::string, Tensor>& preallocated_outputs = {}) const;
     [[nodiscard]] StampedExecutionPlan stampSingleOutput(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                                         const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs = {},
                                                          const std::optional<Tensor>& preallocated_output = {}) const;
 
     // Convenience: bind, launch into caller-provided outputs.  Restricted, as in the reference, to expressions that
@@ -61,7 +65,11 @@ class FusedEquation {
     std::vector<uint64_t> getOutputShape(const std::unordered_map<std::string, Tensor>& inputs) const;
     std::unordered_map<std::string, std::vector<uint64_t>> getOutputShapes(const Tensor& input) const;
     std::unordered_map<std::string, std::vector<uint64_t>> getOutputShapes(const std::unordered_map<std::string, Tensor>& inputs) const;
+    std::unordered_map<std::string, std::vector<uint64_t>> getOutputShapes(
+        const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs) const;
     std::unordered_map<std::string, DataType> getOutputDataTypes(const std::unordered_map<std::string, Tensor>& inputs) const;
+    std::unordered_map<std::string, DataType> getOutputDataTypes(const std::unordered_map<std::string, Tensor>& inputs,
+                                                                 const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs) const;
 
     // NumPy-style right-aligned broadcast of the input shapes; returns true when any input needs broadcasting.
     static bool resolveLayout(std::vector<Tensor>& inputs, std::vector<uint64_t>& outputDimensions);
@@ -71,6 +79,9 @@ class FusedEquation {
    private:
     FusedEquation(PhysicalOutputs outputs_template, int device_num);
 
+    // `inputs` plus one single-element view per tensor-scalar binding (validated)
+    std::unordered_map<std::string, Tensor> withTensorScalars(const std::unordered_map<std::string, Tensor>& inputs,
+                                                              const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs) const;
     std::shared_ptr<PlannedGraph> plannedGraphFor(const std::vector<DataType>& root_dtypes) const;
     std::vector<DataType> rootDTypes(const std::unordered_map<std::string, Tensor>& inputs) const;
     StampedExecutionPlan stampImpl(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,

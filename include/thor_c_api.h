@@ -203,6 +203,15 @@ int thor_fused_equation_output_name(thor_fused_equation_t eq, int index, char* b
 thor_plan_t thor_fused_equation_stamp(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs, int num_inputs,
                                       const char* const* preallocated_names, const thor_tensor_t* preallocated, int num_preallocated,
                                       thor_stream_t stream);
+/* The same with tensorRuntimeScalar inputs bound to one element of a device buffer each (TensorScalarBinding,
+ * Utilities/Expression/CompiledEquation.h:15-19 there): scalar_buffers[i] at scalar_byte_offsets[i], read as scalar_dtypes[i]. */
+thor_plan_t thor_fused_equation_stamp_with_tensor_scalars(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs,
+                                                          int num_inputs, const char* const* scalar_names, const thor_tensor_t* scalar_buffers,
+                                                          const uint64_t* scalar_byte_offsets, const int* scalar_dtypes, int num_scalars,
+                                                          const char* const* preallocated_names, const thor_tensor_t* preallocated,
+                                                          int num_preallocated, thor_stream_t stream);
+/* Expression::tensorRuntimeScalar(name, compute_dtype, output_dtype) */
+thor_expr_t thor_expr_tensor_runtime_scalar(const char* name, int compute_dtype, int output_dtype);
 /* FusedEquation::run(inputs, scalar_inputs, outputs, stream): compile-if-needed and launch into caller tensors */
 int thor_fused_equation_run(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs, int num_inputs,
                             const char* const* scalar_names, const float* scalars, int num_scalars, const char* const* output_names,

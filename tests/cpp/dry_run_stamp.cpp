@@ -153,6 +153,19 @@ static int runAll() {
             stampOne(std::string("scan ") + dtypeName + " argmin", x.scan(ScanOp::ArgMin), inputs, stream, "Scan");
             stampBackward(std::string("backward ") + dtypeName + " sum scan", x.scan(ScanOp::Sum), inputs, fullGradient, stream, "Scan");
         }
+        // a scalar kept in device memory next to flat operands
+        {
+            std::printf("[ RUN  ] tensor scalar %s\n", dtypeName);
+            std::fflush(stdout);
+            const FusedEquation eq = FusedEquation::compile(Expression::outputs({{"y", (x * Expression::tensorRuntimeScalar("step") + y).tanh()}}).physicalOutputs(), 0);
+            Tensor buffer(gpuPlacement, TensorDescriptor(DataType::FP32, {4}));
+            StampedExecutionPlan plan = eq.stamp(inputs, stream, {{"step", TensorScalarBinding{buffer, 8, DataType::FP32}}});
+            if (plan.stageKindNames() != std::vector<std::string>{"FusedKernel"}) {
+                std::printf("  unexpected plan\n");
+                std::exit(1);
+            }
+            ++stamped;
+        }
         // gathers along an axis, with indices the same equation computes
         stampOne(std::string("gather ") + dtypeName + " value at the row argmax", (x * y).takeAlongAxis(x.argmax({1}, {}), 1), inputs, stream);
         stampOne(std::string("gather ") + dtypeName + " column picks", x.takeAlongAxis(y.argmin({0}, {}), 0) + 1.0, inputs, stream);

@@ -386,7 +386,7 @@ static void raggedExpressionExecution(Stream& stream) {
         FusedEquation eq = FusedEquation::compile(Expression::outputs({{"out", e}}).physicalOutputs(), 0);
         std::unordered_map<std::string, Tensor> pre;
         if (into.has_value()) pre.emplace("out", into.value());
-        StampedExecutionPlan plan = eq.stamp(inputs, stream, pre);
+        StampedExecutionPlan plan = eq.stamp(inputs, stream, {}, pre);
         plan.run();
         return plan.output("out");
     };
@@ -492,6 +492,24 @@ static void expressionConfig1AndRuntimeScalars(Stream& stream) {
     for (size_t i = 0; i < n; i += 37) {
         const double want = (double(a[i]) * b[i] + c[i]) / (1.0 + std::exp(-double(d[i])));
         CHECK_NEAR(got[i], want, 4e-7 * std::max(1.0, std::fabs(want)) + 2e-7);
+    }
+    // a scalar kept in device memory: read at every run through a TensorScalarBinding (CompiledEquation.h:15-19 there), bound as
+    // the third argument of stamp like in the reference
+    {
+        const Expression stepped = Expression::input("x") * Expression::tensorRuntimeScalar("step") + 1.0;
+        const FusedEquation eq3 = FusedEquation::compile(stepped.expression(), 0);
+        Tensor xs = gpuFrom({1, 2, 3, 4}, {4}, stream), buffer = gpuFrom({123.0f, 0.25f}, {2}, stream);
+        StampedExecutionPlan byOffset = eq3.stamp({{"x", xs}}, stream, {{"step", TensorScalarBinding{buffer, 4, DataType::FP32}}});
+        CHECK((byOffset.stageKindNames() == std::vector<std::string>{"FusedKernel"}));
+        byOffset.run();
+        CHECK((toHostF32(byOffset.output(), stream) == std::vector<float>{1.25f, 1.5f, 1.75f, 2.0f}));
+        buffer.copyFromAsync(gpuFrom({123.0f, -1.5f}, {2}, stream), stream);
+        byOffset.run();
+        CHECK((toHostF32(byOffset.output(), stream) == std::vector<float>{-0.5f, -2.0f, -3.5f, -5.0f}));
+        CHECK(throwsAs<std::runtime_error>([&] { (void)eq3.stamp({{"x", xs}}, stream); }));                                                          // unbound
+        CHECK(throwsAs<std::runtime_error>([&] { (void)eq3.stamp({{"x", xs}}, stream, {{"step", TensorScalarBinding{buffer, 2, DataType::FP32}}}); }));  // misaligned
+        CHECK(throwsAs<std::runtime_error>([&] { (void)eq3.stamp({{"x", xs}}, stream, {{"step", TensorScalarBinding{buffer, 8, DataType::FP32}}}); }));  // past the end
+        CHECK(throwsAs<std::runtime_error>([&] { (void)eq3.stamp({{"x", xs}}, stream, {{"step", TensorScalarBinding{buffer, 0, DataType::FP16}}}); }));  // dtype
     }
     // convenience run into a caller-provided tensor, with a runtime scalar
     Expression scaled = Expression::input("x") * Expression::runtimeScalar("alpha") + 1.0;

@@ -140,6 +140,11 @@ Expression Expression::runtimeScalar(const std::string& name, std::optional<Data
     return makeLeaf(ExprOp::RUNTIME_SCALAR, NamedInput::Kind::RuntimeScalarFp32, name, compute_dtype, output_dtype, out);
 }
 
+Expression Expression::tensorRuntimeScalar(const std::string& name, std::optional<DataType> compute_dtype, std::optional<DataType> output_dtype) {
+    std::shared_ptr<PhysicalExpression> out;
+    return makeLeaf(ExprOp::TENSOR_RUNTIME_SCALAR, NamedInput::Kind::TensorRuntimeScalar, name, compute_dtype, output_dtype, out);
+}
+
 Expression Expression::fill(double value, const std::vector<uint64_t>& dims, std::optional<DataType> output_dtype) {
     if (dims.empty()) throw std::invalid_argument("Expression::fill requires non-empty concrete dimensions; use constantScalar for a scalar.");
     for (uint64_t d : dims) {

@@ -30,9 +30,7 @@ bool isBindableInputDType(DataType dtype) {
 
 void rejectUnsupportedOp(ExprOp op) {
     if (isRaggedOp(op) || isStorageViewOp(op) || isWinnerRoutingOp(op) || op == ExprOp::TAKE_ALONG_AXIS || isScanOp(op)) return;
-    if (Expression::isLeafOp(op) || Expression::isUnaryOp(op) || Expression::isBinaryOp(op) || Expression::isTernaryOp(op)) {
-        if (op != ExprOp::TENSOR_RUNTIME_SCALAR) return;
-    }
+    if (Expression::isLeafOp(op) || Expression::isUnaryOp(op) || Expression::isBinaryOp(op) || Expression::isTernaryOp(op)) return;
     throw std::runtime_error("Expression op '" + opName(op) + "' is outside the elementwise / reduction / cast path of this backend.");
 }
 
@@ -244,7 +242,7 @@ void resolveInPlace(PhysicalExpression& expr, const std::vector<DataType>& rootD
     for (uint32_t idx = 0; idx < expr.nodes.size(); ++idx) {
         ExprNode& node = expr.nodes[idx];
         rejectUnsupportedOp(node.op);
-        if (node.op == ExprOp::INPUT || node.op == ExprOp::RUNTIME_SCALAR) {
+        if (node.op == ExprOp::INPUT || node.op == ExprOp::RUNTIME_SCALAR || node.op == ExprOp::TENSOR_RUNTIME_SCALAR) {
             if (node.input_slot >= rootDTypes.size()) throw std::runtime_error("Input slot out of range during dtype resolution.");
             const DataType actual = rootDTypes[node.input_slot];
             if (!isBindableInputDType(actual)) {

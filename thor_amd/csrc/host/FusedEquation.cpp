@@ -127,6 +127,8 @@ class GraphBuilder {
         auto it = remap.find(srcIndex);
         if (it != remap.end()) return it->second;
         ExprNode node = src.nodes.at(srcIndex);
+        // a scalar in device memory is bound as a one-element tensor: from here on an input like any other
+        if (node.op == ExprOp::TENSOR_RUNTIME_SCALAR) node.op = ExprOp::INPUT;
         if (node.lhs != UINT32_MAX) node.lhs = translate(node.lhs);
         if (node.rhs != UINT32_MAX) node.rhs = translate(node.rhs);
         if (node.aux != UINT32_MAX) node.aux = translate(node.aux);
@@ -278,6 +280,7 @@ std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpressio
         const ExprNode& n = expr.nodes[i];
         switch (n.op) {
             case ExprOp::INPUT:
+            case ExprOp::TENSOR_RUNTIME_SCALAR:  // bound as a one-element tensor
                 dims[i] = inputDims(n.input_slot);
                 break;
             case ExprOp::RUNTIME_SCALAR:
@@ -645,17 +648,46 @@ bool FusedEquation::resolveLayout(std::vector<Tensor>& inputs, std::vector<uint6
     return broadcast;
 }
 
+std::unordered_map<std::string, Tensor> FusedEquation::withTensorScalars(const std::unordered_map<std::string, Tensor>& inputs,
+                                                                         const std::unordered_map<std::string, TensorScalarBinding>& bindings) const {
+    if (bindings.empty()) return inputs;
+    std::unordered_map<std::string, Tensor> merged = inputs;
+    for (const auto& [name, binding] : bindings) {
+        bool declared = false;
+        for (const NamedInput& in : root_inputs) declared = declared || (in.name == name && in.kind == NamedInput::Kind::TensorRuntimeScalar);
+        if (!declared) throw std::runtime_error("Unexpected tensor-runtime-scalar input for this equation: " + name);
+        if (inputs.count(name)) throw std::runtime_error("Input '" + name + "' is bound both as a tensor and as a tensor-runtime-scalar.");
+        if (!binding.buffer.isInitialized()) throw std::runtime_error("Tensor-runtime-scalar buffer is not initialized for " + name + ".");
+        if (binding.buffer.getDataType() != binding.sourceDType) {
+            throw std::runtime_error("Tensor-runtime-scalar binding for " + name + " must use a backing buffer with the same dtype as the scalar source dtype.");
+        }
+        const uint64_t elementBytes = dataTypeSizeInBytes(binding.sourceDType);
+        if (elementBytes == 0 || binding.byteOffset % elementBytes != 0) {
+            throw std::runtime_error("Tensor-runtime-scalar binding byte offset is not element-aligned for " + name + ".");
+        }
+        if (!binding.buffer.isDenseContiguous() || binding.byteOffset + elementBytes > binding.buffer.getTotalNumElements() * elementBytes) {
+            throw std::runtime_error("Tensor-runtime-scalar binding exceeds backing buffer size for " + name + ".");
+        }
+        Tensor flat = binding.buffer;
+        flat.reshape({binding.buffer.getTotalNumElements()});
+        merged.emplace(name, flat.aliasView({1}, {1}, binding.byteOffset / elementBytes));
+    }
+    return merged;
+}
+
 StampedExecutionPlan FusedEquation::stamp(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                          const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs,
                                           const std::unordered_map<std::string, Tensor>& preallocated_outputs) const {
-    return stampImpl(inputs, stream, preallocated_outputs, false);
+    return stampImpl(withTensorScalars(inputs, tensor_scalar_inputs), stream, preallocated_outputs, false);
 }
 
 StampedExecutionPlan FusedEquation::stampSingleOutput(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
+                                                      const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs,
                                                       const std::optional<Tensor>& preallocated_output) const {
     if (outputs_template.outputs.size() != 1) throw std::runtime_error("stampSingleOutput requires an equation with exactly one output.");
     std::unordered_map<std::string, Tensor> pre;
     if (preallocated_output.has_value()) pre.emplace(outputs_template.outputs[0].name, preallocated_output.value());
-    return stampImpl(inputs, stream, pre, false);
+    return stampImpl(withTensorScalars(inputs, tensor_scalar_inputs), stream, pre, false);
 }
 
 StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
@@ -1530,6 +1562,15 @@ std::vector<uint64_t> FusedEquation::getOutputShape(const std::unordered_map<std
 std::vector<uint64_t> FusedEquation::getOutputShape(const Tensor& input) const {
     if (outputs_template.outputs.size() != 1) throw std::runtime_error("getOutputShape requires an equation with exactly one output.");
     return getOutputShapes(input).begin()->second;
+}
+
+std::unordered_map<std::string, std::vector<uint64_t>> FusedEquation::getOutputShapes(
+    const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs) const {
+    return getOutputShapes(withTensorScalars(inputs, tensor_scalar_inputs));
+}
+std::unordered_map<std::string, DataType> FusedEquation::getOutputDataTypes(
+    const std::unordered_map<std::string, Tensor>& inputs, const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs) const {
+    return getOutputDataTypes(withTensorScalars(inputs, tensor_scalar_inputs));
 }
 
 std::unordered_map<std::string, DataType> FusedEquation::getOutputDataTypes(const std::unordered_map<std::string, Tensor>& inputs) const {

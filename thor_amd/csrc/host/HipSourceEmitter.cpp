@@ -478,7 +478,16 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
     };
     const std::vector<uint64_t> outCore = stripOnes(r.outputDims);
     k.flat = true;
-    for (const KernelOperand& op : r.operands) {
+    // a single-element operand (a scalar kept in device memory) is read at [0] and does not decide the kernel's form
+    std::vector<char> single(r.operands.size(), 0);
+    for (size_t o = 0; o < r.operands.size(); ++o) {
+        uint64_t count = 1;
+        for (uint64_t d : r.operands[o].dims) count *= d;
+        single[o] = count == 1 && k.numel > 1;
+    }
+    for (size_t o = 0; o < r.operands.size(); ++o) {
+        const KernelOperand& op = r.operands[o];
+        if (single[o]) continue;
         uint64_t expected = 1;
         bool dense = true;
         for (size_t a = op.dims.size(); a-- > 0;) {
@@ -490,7 +499,8 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
 
     // widest element decides the vector length: one 16-byte access for it, narrower operands move fewer bytes
     uint32_t widest = 1;
-    for (const KernelOperand& op : r.operands) widest = std::max(widest, dataTypeSizeInBytes(op.storageDType));
+    for (size_t o = 0; o < r.operands.size(); ++o)
+        if (!single[o]) widest = std::max(widest, dataTypeSizeInBytes(r.operands[o].storageDType));
     for (const KernelOutput& out : r.outputs) widest = std::max(widest, dataTypeSizeInBytes(out.storageDType));
     int vec = static_cast<int>(16 / widest);
 
@@ -500,8 +510,10 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         for (const KernelOutput& out : r.outputs)
             if (out.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(out.storageDType)) != 0) return false;
         if (k.flat) {
-            for (const KernelOperand& op : r.operands)
-                if (op.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(op.storageDType)) != 0) return false;
+            for (size_t o = 0; o < r.operands.size(); ++o) {
+                const KernelOperand& op = r.operands[o];
+                if (!single[o] && op.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(op.storageDType)) != 0) return false;
+            }
             return true;
         }
         if (layout.dims.back() % v != 0) return false;
@@ -669,13 +681,14 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
                 return gatherPerElement("base + k")(g, body, indent);
             };
             for (size_t o = 0; o < r.operands.size(); ++o) {
+                if (single[o]) continue;
                 s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n";
                 s << "        p" << o << ".loadStream(in" << o << " + base);\n";
             }
             for (size_t o = 0; o < r.outputs.size(); ++o) s << "        thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", V> q" << o << ";\n";
             s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
             s << emitBody(
-                "            ", [](size_t o) { return "p" + std::to_string(o) + ".v[k]"; },
+                "            ", [&](size_t o) { return single[o] ? "in" + std::to_string(o) + "[0]" : "p" + std::to_string(o) + ".v[k]"; },
                 [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; }, gatherInVector);
             s << "        }\n";
             for (size_t o = 0; o < r.outputs.size(); ++o) s << "        q" << o << ".storeStream(out" << o << " + base);\n";
@@ -684,7 +697,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         s << "    const index_t end = (base + V < numel) ? base + V : numel;\n";
         s << "    for (index_t e = base; e < end; ++e) {\n";
         s << emitBody(
-            "        ", [](size_t o) { return "in" + std::to_string(o) + "[e]"; },
+            "        ", [&](size_t o) { return "in" + std::to_string(o) + (single[o] ? "[0]" : "[e]"); },
             [](size_t o, const std::string& v) { return "out" + std::to_string(o) + "[e] = " + v + ";"; }, gatherPerElement("e"));
         s << "    }\n";
         const uint64_t lanes = (k.numel + vec - 1) / vec;

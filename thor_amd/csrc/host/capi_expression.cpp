@@ -97,6 +97,9 @@ thor_expr_t thor_expr_input(const char* name, int compute_dtype, int output_dtyp
 thor_expr_t thor_expr_runtime_scalar(const char* name, int compute_dtype, int output_dtype) {
     THOR_CAPI_TRY_PTR(return new thor_expr{Expression::runtimeScalar(name ? name : "", optionalDType(compute_dtype), optionalDType(output_dtype))};)
 }
+thor_expr_t thor_expr_tensor_runtime_scalar(const char* name, int compute_dtype, int output_dtype) {
+    THOR_CAPI_TRY_PTR(return new thor_expr{Expression::tensorRuntimeScalar(name ? name : "", optionalDType(compute_dtype), optionalDType(output_dtype))};)
+}
 thor_expr_t thor_expr_scalar(double value) { THOR_CAPI_TRY_PTR(return new thor_expr{Expression(value)};) }
 thor_expr_t thor_expr_fill(double value, const uint64_t* dims, int rank, int output_dtype) {
     THOR_CAPI_TRY_PTR(return new thor_expr{Expression::fill(value, u64s(dims, rank), optionalDType(output_dtype))};)
@@ -249,8 +252,22 @@ thor_plan_t thor_fused_equation_stamp(thor_fused_equation_t eq, const char* cons
                                       const char* const* preallocated_names, const thor_tensor_t* preallocated, int num_preallocated,
                                       thor_stream_t stream) {
     THOR_CAPI_TRY_PTR(require(eq, "equation"); require(stream, "stream");
-                      return new thor_plan{eq->equation.stamp(tensorMap(input_names, inputs, num_inputs), stream->stream,
+                      return new thor_plan{eq->equation.stamp(tensorMap(input_names, inputs, num_inputs), stream->stream, {},
                                                               tensorMap(preallocated_names, preallocated, num_preallocated))};)
+}
+
+thor_plan_t thor_fused_equation_stamp_with_tensor_scalars(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs,
+                                                          int num_inputs, const char* const* scalar_names, const thor_tensor_t* scalar_buffers,
+                                                          const uint64_t* scalar_byte_offsets, const int* scalar_dtypes, int num_scalars,
+                                                          const char* const* preallocated_names, const thor_tensor_t* preallocated,
+                                                          int num_preallocated, thor_stream_t stream) {
+    THOR_CAPI_TRY_PTR(require(eq, "equation"); require(stream, "stream"); std::unordered_map<std::string, TensorScalarBinding> bindings;
+                      for (int i = 0; i < num_scalars; ++i) {
+                          require(scalar_buffers[i], "tensor scalar buffer");
+                          bindings[scalar_names[i]] = TensorScalarBinding{scalar_buffers[i]->tensor, scalar_byte_offsets ? scalar_byte_offsets[i] : 0,
+                                                                          static_cast<DataType>(scalar_dtypes[i])};
+                      } return new thor_plan{eq->equation.stamp(tensorMap(input_names, inputs, num_inputs), stream->stream, bindings,
+                                                                tensorMap(preallocated_names, preallocated, num_preallocated))};)
 }
 
 int thor_fused_equation_run(thor_fused_equation_t eq, const char* const* input_names, const thor_tensor_t* inputs, int num_inputs,

@@ -83,6 +83,8 @@ PROTOTYPES = {
     "thor_fused_equation_compile_backward": (_vp, [_vp, _cpp, _i, _cpp, _cpp, _i, _i]),
     "thor_fused_equation_num_outputs": (_i, [_vp]), "thor_fused_equation_output_name": (_i, [_vp, _i, _cp, _sz]),
     "thor_fused_equation_stamp": (_vp, [_vp, _cpp, _vpp, _i, _cpp, _vpp, _i, _vp]),
+    "thor_fused_equation_stamp_with_tensor_scalars": (_vp, [_vp, _cpp, _vpp, _i, _cpp, _vpp, _u64p, ctypes.POINTER(_i), _i, _cpp, _vpp, _i, _vp]),
+    "thor_expr_tensor_runtime_scalar": (_vp, [_cp, _i, _i]),
     "thor_fused_equation_run": (_i, [_vp, _cpp, _vpp, _i, _cpp, _fp, _i, _cpp, _vpp, _i, _vp]),
     "thor_fused_equation_output_shape": (_i, [_vp, _cpp, _vpp, _i, _cp, _u64p, ctypes.POINTER(_i), ctypes.POINTER(_i)]),
     "thor_plan_destroy": (None, [_vp]), "thor_plan_run": (_i, [_vp]), "thor_plan_run_with_scalars": (_i, [_vp, _cpp, _fp, _i]),
@@ -596,6 +598,12 @@ class Expression:
         return Expression(lib().thor_expr_runtime_scalar(name.encode(), _dtype_code(compute_dtype), _dtype_code(output_dtype)))
 
     @staticmethod
+    def tensor_runtime_scalar(name: str, compute_dtype: Optional[DataType] = None, output_dtype: Optional[DataType] = None) -> "Expression":
+        """A scalar read from device memory at every run; bound at stamp time with a TensorScalarBinding."""
+        return Expression(_handle(lib().thor_expr_tensor_runtime_scalar(name.encode(), _dtype_code(compute_dtype), _dtype_code(output_dtype)),
+                                  "tensor_runtime_scalar"))
+
+    @staticmethod
     def constant_scalar(value: float) -> "Expression":
         return Expression(lib().thor_expr_scalar(float(value)))
 
@@ -864,6 +872,15 @@ class Equation:
             pass
 
 
+class TensorScalarBinding:
+    """thor.physical.TensorScalarBinding: one element of ``source_dtype`` at ``byte_offset`` inside ``buffer``."""
+
+    def __init__(self, buffer: Optional[PhysicalTensor] = None, byte_offset: int = 0, source_dtype: DataType = DataType.fp32):
+        self.buffer = buffer
+        self.byte_offset = byte_offset
+        self.source_dtype = source_dtype
+
+
 class FusedEquation:
     def __init__(self, ptr):
         self._h = ptr
@@ -898,10 +915,20 @@ class FusedEquation:
                                                              int(accumulate_grad_outputs))
         return FusedEquation(_handle(ptr, "FusedEquation.compile_backward"))
 
-    def stamp(self, inputs: Dict[str, PhysicalTensor], stream: Stream, preallocated_outputs: Optional[Dict[str, PhysicalTensor]] = None) -> Equation:
+    def stamp(self, inputs: Dict[str, PhysicalTensor], stream: Stream, preallocated_outputs: Optional[Dict[str, PhysicalTensor]] = None,
+              tensor_scalar_inputs: Optional[Dict[str, TensorScalarBinding]] = None) -> Equation:
         names = list(inputs)
         pre = preallocated_outputs or {}
         pre_names = list(pre)
+        if tensor_scalar_inputs:
+            s_names = list(tensor_scalar_inputs)
+            bindings = [tensor_scalar_inputs[n] for n in s_names]
+            offsets = (ctypes.c_uint64 * len(s_names))(*[int(b.byte_offset) for b in bindings])
+            dtypes = (ctypes.c_int * len(s_names))(*[int(b.source_dtype) for b in bindings])
+            ptr = lib().thor_fused_equation_stamp_with_tensor_scalars(
+                self._h, _names(names), _ptrs([inputs[n]._h for n in names]), len(names), _names(s_names), _ptrs([b.buffer._h for b in bindings]), offsets,
+                dtypes, len(s_names), _names(pre_names), _ptrs([pre[n]._h for n in pre_names]), len(pre_names), stream._h)
+            return Equation(_handle(ptr, "FusedEquation.stamp"))
         ptr = lib().thor_fused_equation_stamp(self._h, _names(names), _ptrs([inputs[n]._h for n in names]), len(names), _names(pre_names),
                                               _ptrs([pre[n]._h for n in pre_names]), len(pre_names), stream._h)
         return Equation(_handle(ptr, "FusedEquation.stamp"))
