@@ -110,7 +110,8 @@ __device__ __forceinline__ boolean makeBoolean(bool b) {
 }
 
 // value rounded through a 16-bit / 8-bit float and widened again (how a bf16 / fp8 compute step is modelled in fp32)
-__device__ __forceinline__ float roundBf16(float x) { return toFloat(toBf16(x)); }
+// (a NaN stays a NaN of the hardware's choosing here; bf16FromExact writes the canonical one when the value is stored)
+__device__ __forceinline__ float roundBf16(float x) { return bitsF32((u32)bf16BitsRne(x) << 16); }
 // Storage form of a float that already holds a bf16 value (every bf16-typed value inside a kernel does: loads widen
 // exactly and every arithmetic result passes through roundBf16): the upper half of its bits; NaN stays canonical.
 __device__ __forceinline__ bf16 bf16FromExact(float x) {

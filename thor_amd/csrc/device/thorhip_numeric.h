@@ -77,11 +77,14 @@ __device__ __forceinline__ f16 toF16(float x) {
     return r;
 }
 
+// v_cvt_pk_bf16_f32 (what the compiler selects for a float -> __bf16 truncation on gfx950): round-to-nearest-even with
+// gradual underflow, equal to the integer formula (b + 0x7fff + ((b >> 16) & 1)) >> 16 on every one of the 2^32 - 2^24
+// inputs that are not NaN; a NaN comes out as a quiet NaN that keeps its sign and upper payload.
+__device__ __forceinline__ u16 bf16BitsRne(float x) { return __builtin_bit_cast(u16, (__bf16)x); }
+
 __device__ __forceinline__ bf16 toBf16(float x) {
-    const u32 b = f32Bits(x);
-    const u32 rounded = (b + 0x7fffu + ((b >> 16) & 1u)) >> 16;
     bf16 r;
-    r.bits = (x != x) ? (u16)0x7fffu : (u16)rounded;
+    r.bits = (x != x) ? (u16)0x7fffu : bf16BitsRne(x);
     return r;
 }
 
