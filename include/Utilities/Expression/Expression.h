@@ -78,6 +78,33 @@ enum class ScanOp : uint8_t { Sum = 0, Min = 1, Max = 2, Product = 3, ArgMin = 4
 enum class ScanMode : uint8_t { Exclusive = 0, Inclusive = 1 };
 inline bool isArgScanOp(ScanOp op) { return op == ScanOp::ArgMin || op == ScanOp::ArgMax; }
 
+// Rotary position embedding (Expression.h:150-218 there).  Pair j of the rotary part of the head dimension turns by
+// position * frequency(j); the scaling kinds only change the frequencies (and, for Linear, the position).
+enum class RotaryScalingKind : uint8_t { None = 0, Linear = 1, DynamicNTK = 2, Yarn = 3, LongRope = 4, Llama3 = 5 };
+struct RotaryPositionEmbeddingOptions {
+    uint32_t sequence_axis = 2;
+    uint32_t head_dim_axis = 3;
+    uint64_t rotary_dim = 0;  // 0 = the whole head dimension
+    double base = 10000.0;
+    int64_t position_offset = 0;
+    bool interleaved = false;  // pairs (2j, 2j + 1) instead of (j, j + rotary_dim / 2)
+    bool inverse = false;      // turns the other way (the transpose of the rotation)
+    RotaryScalingKind scaling_kind = RotaryScalingKind::None;
+    double scaling_factor = 1.0;
+    uint64_t original_max_position_embeddings = 0;
+    std::optional<double> attention_factor = std::nullopt;
+    double yarn_beta_fast = 32.0;
+    double yarn_beta_slow = 1.0;
+    double llama3_low_freq_factor = 1.0;
+    double llama3_high_freq_factor = 4.0;
+    std::vector<double> long_rope_short_factors;
+    std::vector<double> long_rope_long_factors;
+    std::optional<DataType> output_dtype = std::nullopt;
+    std::optional<DataType> compute_dtype = std::nullopt;
+    // Accepted for source compatibility; the rotation always writes a tensor of its own here.
+    bool allow_in_place_materialization = false;
+};
+
 // reduction_axes entry standing for "every axis except axis 0"
 constexpr uint64_t kReduceAllAxesButFirst = UINT64_MAX - 1;
 
@@ -130,6 +157,26 @@ struct ExprNode {
     ScanMode scan_mode = ScanMode::Inclusive;
     uint64_t scan_axis = UINT64_MAX;
     bool scan_reverse = false;
+    // ROPE (Expression.h:293-318 there): lhs = values; rhs = position ids (rope_position_ids_node there: one absolute
+    // position per element of the sequence axis) and aux = effective sequence length (rope_effective_sequence_length_node
+    // there: one element, read on the device at run time), UINT32_MAX where absent.
+    uint32_t rope_sequence_axis = 2;
+    uint32_t rope_head_dim_axis = 3;
+    uint64_t rope_rotary_dim = 0;
+    double rope_base = 10000.0;
+    int64_t rope_position_offset = 0;
+    bool rope_interleaved = false;
+    bool rope_inverse = false;
+    RotaryScalingKind rope_scaling_kind = RotaryScalingKind::None;
+    double rope_scaling_factor = 1.0;
+    uint64_t rope_original_max_position_embeddings = 0;
+    double rope_attention_factor = 1.0;
+    double rope_yarn_beta_fast = 32.0;
+    double rope_yarn_beta_slow = 1.0;
+    double rope_llama3_low_freq_factor = 1.0;
+    double rope_llama3_high_freq_factor = 4.0;
+    std::vector<double> rope_long_rope_short_factors;
+    std::vector<double> rope_long_rope_long_factors;
     SoftmaxAlgorithm softmax_algorithm = SoftmaxAlgorithm::Accurate;  // SOFTMAX only
     SoftmaxMode softmax_mode = SoftmaxMode::Channel;
 
@@ -371,6 +418,23 @@ class Expression {
     Expression takeAlongAxis(const Expression& indices, int64_t axis = -1) const;
     static Expression takeAlongAxis(const Expression& input, const Expression& indices, int64_t axis = -1) { return input.takeAlongAxis(indices, axis); }
 
+    // Rotary position embedding of every [sequence, head dimension] plane of the operand (Expression.h:650-675,
+    // Expression.cpp:4334-4507 there).  Explicit position ids (any numeric dtype, one per element of the sequence axis) replace
+    // coordinate + position_offset; the effective sequence length (one element) replaces the extent of the sequence axis in
+    // the Dynamic-NTK and LongRoPE rules.  Arithmetic is fp32; the result has output_dtype or the operand's dtype.
+    Expression rotaryPositionEmbedding(RotaryPositionEmbeddingOptions options = {}) const;
+    Expression rope(RotaryPositionEmbeddingOptions options = {}) const { return rotaryPositionEmbedding(std::move(options)); }
+    static Expression rotaryPositionEmbedding(const Expression& input, RotaryPositionEmbeddingOptions options = {}) {
+        return input.rotaryPositionEmbedding(std::move(options));
+    }
+    static Expression rope(const Expression& input, RotaryPositionEmbeddingOptions options = {}) { return input.rotaryPositionEmbedding(std::move(options)); }
+    Expression rotaryPositionEmbeddingWithEffectiveSequenceLength(const Expression& effective_sequence_length,
+                                                                  RotaryPositionEmbeddingOptions options = {}) const;
+    Expression rotaryPositionEmbeddingWithPositionIds(const Expression& position_ids, RotaryPositionEmbeddingOptions options = {}) const;
+    Expression rotaryPositionEmbeddingWithPositionIdsAndEffectiveSequenceLength(const Expression& position_ids,
+                                                                                const Expression& effective_sequence_length,
+                                                                                RotaryPositionEmbeddingOptions options = {}) const;
+
     // ---- reductions: fp32 accumulation, reduced axes kept as 1 unless listed in squeeze_axes ------------------------
     Expression reduction(ExprOp op, const std::vector<uint64_t>& reduction_axes, const std::vector<uint64_t>& squeeze_axes,
                          std::optional<DataType> compute_dtype) const;
@@ -430,6 +494,7 @@ class Expression {
     static Expression unaryOp(const Expression& input, ExprOp op);
     static Expression binaryOp(const Expression& lhs, const Expression& rhs, ExprOp op);
     static Expression ternaryOp(const Expression& a, const Expression& b, const Expression& c, ExprOp op);
+    static Expression ropeOp(const Expression& input, const Expression* position_ids, const Expression* effective_sequence_length, ExprNode node);
 
     std::shared_ptr<PhysicalExpression> expr;
     uint32_t nodeIndex = UINT32_MAX;
@@ -438,6 +503,8 @@ class Expression {
 std::string opName(ExprOp op);
 bool isCommutative(ExprOp op);
 std::string formatFloatCanonical(double x);
+// Every parameter of a ROPE node as text (two rotations with the same text and operands are the same computation).
+std::string ropeKey(const ExprNode& n);
 // Canonical text of the sub-DAG below `nodeIndex` (commutative operands ordered, shared sub-trees memoised): two graphs
 // with the same text compute the same function of the same input slots.
 std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex, std::unordered_map<uint32_t, std::string>& memo);

@@ -176,6 +176,33 @@ thor_expr_t thor_expr_strided_view(thor_expr_t input, const uint64_t* dims, cons
 thor_expr_t thor_expr_scan(thor_expr_t input, thor_expr_t offsets, int op, int64_t axis, int inclusive, int reverse);
 /* Expression::takeAlongAxis(indices, axis) (Expression.h:676-677 there); axis = -1 is the last axis */
 thor_expr_t thor_expr_take_along_axis(thor_expr_t input, thor_expr_t indices, int64_t axis);
+/* Expression::rotaryPositionEmbedding and its WithPositionIds / WithEffectiveSequenceLength forms (Expression.h:196-218 options,
+ * :650-675 builders there).  position_ids and effective_sequence_length may be NULL.  scaling_kind: 0 none, 1 linear, 2 dynamic
+ * NTK, 3 YaRN, 4 LongRoPE, 5 Llama 3.  attention_factor <= 0 asks for the scaling kind's own; output_dtype / compute_dtype < 0
+ * leave the choice to dtype resolution. */
+typedef struct thor_rope_options {
+    uint32_t sequence_axis;
+    uint32_t head_dim_axis;
+    uint64_t rotary_dim;
+    double base;
+    int64_t position_offset;
+    int interleaved;
+    int inverse;
+    int scaling_kind;
+    double scaling_factor;
+    uint64_t original_max_position_embeddings;
+    double attention_factor;
+    double yarn_beta_fast;
+    double yarn_beta_slow;
+    double llama3_low_freq_factor;
+    double llama3_high_freq_factor;
+    const double* long_rope_short_factors;
+    const double* long_rope_long_factors;
+    uint64_t num_long_rope_factors;
+    int output_dtype;
+    int compute_dtype;
+} thor_rope_options;
+thor_expr_t thor_expr_rope(thor_expr_t input, thor_expr_t position_ids, thor_expr_t effective_sequence_length, const thor_rope_options* options);
 thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank);
 thor_expr_t thor_expr_unsqueeze(thor_expr_t input, const uint64_t* axes, int num_axes);
 thor_expr_t thor_expr_squeeze(thor_expr_t input, const uint64_t* axes, int num_axes);

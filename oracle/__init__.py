@@ -6,6 +6,7 @@ Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import 
 from __future__ import annotations
 
 import ctypes
+import math
 import os
 import subprocess
 
@@ -310,3 +311,114 @@ def scan(values: np.ndarray, op: int, inclusive: bool = True, reverse: bool = Fa
     if integer:
         return out_values.astype(np.uint32).reshape(np.shape(values))
     return from_f32(out_values.astype(np.float32), dtype).reshape(np.shape(values))
+
+
+# ---- rotary position embedding -------------------------------------------------------------------------------------------
+ROPE_NONE, ROPE_LINEAR, ROPE_DYNAMIC_NTK, ROPE_YARN, ROPE_LONGROPE, ROPE_LLAMA3 = 0, 1, 2, 3, 4, 5
+
+
+def rope_attention_factor(scaling_kind=ROPE_NONE, scaling_factor=1.0, original_max_position_embeddings=0, attention_factor=None):
+    """The magnitude correction a ROPE node carries (Utilities/Expression/Expression.cpp:4398-4413): the caller's, else
+    0.1 ln(s) + 1 for YaRN and sqrt(1 + ln(s) / ln(original_max)) for LongRoPE when s > 1, else 1."""
+    if attention_factor is not None:
+        return float(attention_factor)
+    if scaling_kind == ROPE_YARN:
+        return 1.0 if scaling_factor <= 1.0 else 0.1 * math.log(scaling_factor) + 1.0
+    if scaling_kind == ROPE_LONGROPE:
+        return 1.0 if scaling_factor <= 1.0 else math.sqrt(1.0 + math.log(scaling_factor) / math.log(float(original_max_position_embeddings)))
+    return 1.0
+
+
+def rope_frequencies(rotary_dim, base=10000.0, scaling_kind=ROPE_NONE, scaling_factor=1.0, original_max_position_embeddings=0,
+                     yarn_beta_fast=32.0, yarn_beta_slow=1.0, llama3_low_freq_factor=1.0, llama3_high_freq_factor=4.0,
+                     long_rope_short_factors=None, long_rope_long_factors=None, sequence_length=1.0):
+    """fp32 frequency of every pair, operation by operation as the generated kernel of the reference computes it
+    (Utilities/Expression/CudaSourceEmitter.cpp:3607-3690).  `sequence_length` is max(effective length + max(offset, 0), 1),
+    which only the Dynamic-NTK and LongRoPE rules read.  Linear scaling leaves the frequencies alone (it divides the position)."""
+    f = np.float32
+    pairs = np.arange(rotary_dim // 2, dtype=np.float32)
+    rot = f(rotary_dim)
+    b = f(base)
+    s = f(scaling_factor)
+    original = f(original_max_position_embeddings)
+    seq_len = f(sequence_length)
+    if scaling_kind == ROPE_DYNAMIC_NTK:
+        if seq_len > original and rotary_dim > 2:
+            ratio = f(f(f(s * seq_len) / original) - f(s - f(1.0)))
+            b = f(b * np.power(ratio, f(rot / f(rotary_dim - 2)), dtype=np.float32))
+        return np.power(b, (f(-2.0) * pairs) / rot, dtype=np.float32)
+    if scaling_kind == ROPE_YARN:
+        pos_freq = np.power(b, (f(2.0) * pairs) / rot, dtype=np.float32)
+        extrapolated = f(1.0) / pos_freq
+        interpolated = f(1.0) / (s * pos_freq)
+        log_base = np.log(b, dtype=np.float32)
+        two_pi = f(6.2831853071795864769)
+        low = f(rot * np.log(f(original / f(f(yarn_beta_fast) * two_pi)), dtype=np.float32)) / f(f(2.0) * log_base)
+        high = f(rot * np.log(f(original / f(f(yarn_beta_slow) * two_pi)), dtype=np.float32)) / f(f(2.0) * log_base)
+        low = max(f(np.floor(low)), f(0.0))
+        high = min(f(np.ceil(high)), f(rotary_dim - 1))
+        if low == high:
+            high = f(high + f(0.001))
+        ramp = np.minimum(np.maximum((pairs - low) / f(high - low), f(0.0)), f(1.0)).astype(np.float32)
+        return (interpolated * ramp + extrapolated * (f(1.0) - ramp)).astype(np.float32)
+    if scaling_kind == ROPE_LONGROPE:
+        stretch = np.asarray(long_rope_long_factors if seq_len > original else long_rope_short_factors, dtype=np.float32)
+        return (f(1.0) / (stretch * np.power(b, (f(2.0) * pairs) / rot, dtype=np.float32))).astype(np.float32)
+    plain = np.power(b, (f(-2.0) * pairs) / rot, dtype=np.float32)
+    if scaling_kind == ROPE_LLAMA3:
+        two_pi = f(6.2831853071795864769)
+        wavelength = two_pi / plain
+        low_wavelength = f(original / f(llama3_low_freq_factor))
+        high_wavelength = f(original / f(llama3_high_freq_factor))
+        smooth = (original / wavelength - f(llama3_low_freq_factor)) / f(f(llama3_high_freq_factor) - f(llama3_low_freq_factor))
+        blended = (f(1.0) - smooth) * (plain / s) + smooth * plain
+        return np.where(wavelength > low_wavelength, plain / s, np.where(wavelength < high_wavelength, plain, blended)).astype(np.float32)
+    return plain
+
+
+def rope(x: np.ndarray, dtype: int = FP32, *, sequence_axis=2, head_dim_axis=3, rotary_dim=0, base=10000.0, position_offset=0, interleaved=False,
+         inverse=False, scaling_kind=ROPE_NONE, scaling_factor=1.0, original_max_position_embeddings=0, attention_factor=None, yarn_beta_fast=32.0,
+         yarn_beta_slow=1.0, llama3_low_freq_factor=1.0, llama3_high_freq_factor=4.0, long_rope_short_factors=None, long_rope_long_factors=None,
+         position_ids=None, effective_sequence_length=None, out_dtype=None):
+    """Rotary position embedding of carriers `x` of `dtype`, in fp32, restating the reference's generated kernel
+    (Utilities/Expression/CudaSourceEmitter.cpp:3538-3697): the first element a and second element b of pair j at position p
+    become a cos(t) - b sin(t) and a sin(t) + b cos(t), t = p * frequency(j), sine and cosine scaled by the attention factor and
+    the sine negated for the inverse; p = coordinate + offset (divided by the factor for linear scaling) or the given position
+    ids; the pairs are (j, j + rotary/2), or (2j, 2j + 1) when interleaved; coordinates of the head dimension beyond rotary_dim
+    pass through.  Returns carriers of `out_dtype` (default: `dtype`)."""
+    out_dtype = dtype if out_dtype is None else out_dtype
+    f = np.float32
+    values = to_f32(np.ascontiguousarray(x).reshape(-1), dtype).astype(np.float32).reshape(np.shape(x))
+    moved = np.moveaxis(values, (sequence_axis, head_dim_axis), (-2, -1))  # [..., S, D] view
+    seq, head_dim = moved.shape[-2], moved.shape[-1]
+    rotary = head_dim if rotary_dim == 0 else rotary_dim
+    assert 0 < rotary <= head_dim and rotary % 2 == 0
+    half = rotary // 2
+    if position_ids is not None:
+        positions = np.asarray(position_ids).reshape(-1).astype(np.float32)
+        assert position_offset == 0 and positions.size == seq
+    else:
+        positions = np.arange(seq, dtype=np.float32) + f(position_offset)
+    if scaling_kind == ROPE_LINEAR:
+        positions = positions / f(scaling_factor)
+    extent = f(seq) if effective_sequence_length is None else f(effective_sequence_length)
+    seq_len = max(f(extent + f(max(0, position_offset))), f(1.0))
+    freq = rope_frequencies(rotary, base, scaling_kind, scaling_factor, original_max_position_embeddings, yarn_beta_fast, yarn_beta_slow,
+                            llama3_low_freq_factor, llama3_high_freq_factor, long_rope_short_factors, long_rope_long_factors, seq_len)
+    theta = (positions[:, None] * freq[None, :]).astype(np.float32)
+    # sine and cosine of the fp32 angle, correctly rounded to fp32 (device libraries stay within 2 ulp of this)
+    sn = np.sin(theta.astype(np.float64)).astype(np.float32)
+    cs = np.cos(theta.astype(np.float64)).astype(np.float32)
+    factor = rope_attention_factor(scaling_kind, scaling_factor, original_max_position_embeddings, attention_factor)
+    if factor != 1.0:
+        sn, cs = sn * f(factor), cs * f(factor)
+    if inverse:
+        sn = -sn
+    first = np.arange(0, rotary, 2) if interleaved else np.arange(half)
+    second = first + 1 if interleaved else first + half
+    a, b = moved[..., first], moved[..., second]
+    result = moved.copy()
+    result[..., first] = a * cs - b * sn
+    result[..., second] = a * sn + b * cs
+    result = np.moveaxis(result, (-2, -1), (sequence_axis, head_dim_axis))
+    return from_f32(np.ascontiguousarray(result, dtype=np.float32).reshape(-1), out_dtype).reshape(np.shape(x))

@@ -169,6 +169,51 @@ static int runAll() {
         // gathers along an axis, with indices the same equation computes
         stampOne(std::string("gather ") + dtypeName + " value at the row argmax", (x * y).takeAlongAxis(x.argmax({1}, {}), 1), inputs, stream);
         stampOne(std::string("gather ") + dtypeName + " column picks", x.takeAlongAxis(y.argmin({0}, {}), 0) + 1.0, inputs, stream);
+        // rotary position embedding: vector and scalar layouts, every scaling rule, explicit positions, backward
+        {
+            Tensor q(gpuPlacement, TensorDescriptor(dtype, {2, 4, 48, 64})), odd(gpuPlacement, TensorDescriptor(dtype, {3, 30, 7, 5}));
+            Tensor positions(gpuPlacement, TensorDescriptor(DataType::UINT32, {48})), length(gpuPlacement, TensorDescriptor(DataType::INT32, {1}));
+            const std::unordered_map<std::string, Tensor> ropeInputs{{"q", q}, {"odd", odd}, {"positions", positions}, {"length", length}};
+            const Expression iq = Expression::input("q"), iodd = Expression::input("odd");
+            RotaryPositionEmbeddingOptions o;
+            stampOne(std::string("rope ") + dtypeName + " plain", iq.rope(o) * 2.0, ropeInputs, stream);
+            o.interleaved = true;
+            o.rotary_dim = 32;
+            stampOne(std::string("rope ") + dtypeName + " interleaved partial", (iq + 1.0).rope(o), ropeInputs, stream);
+            o = {};
+            o.sequence_axis = 3;
+            o.head_dim_axis = 1;
+            stampOne(std::string("rope ") + dtypeName + " head dimension before sequence", iodd.rope(o), ropeInputs, stream);
+            o = {};
+            o.scaling_kind = RotaryScalingKind::Linear;
+            o.scaling_factor = 2.0;
+            stampOne(std::string("rope ") + dtypeName + " linear with ids", iq.rotaryPositionEmbeddingWithPositionIds(Expression::input("positions"), o), ropeInputs, stream);
+            o.scaling_kind = RotaryScalingKind::DynamicNTK;
+            o.original_max_position_embeddings = 16;
+            stampOne(std::string("rope ") + dtypeName + " dynamic ntk with length",
+                     iq.rotaryPositionEmbeddingWithEffectiveSequenceLength(Expression::input("length"), o), ropeInputs, stream);
+            o.scaling_kind = RotaryScalingKind::Yarn;
+            o.scaling_factor = 4.0;
+            stampOne(std::string("rope ") + dtypeName + " yarn", iq.rope(o), ropeInputs, stream);
+            o.scaling_kind = RotaryScalingKind::Llama3;
+            o.inverse = true;
+            stampOne(std::string("rope ") + dtypeName + " llama3 inverse", iq.rope(o), ropeInputs, stream);
+            o = {};
+            o.scaling_kind = RotaryScalingKind::LongRope;
+            o.rotary_dim = 8;
+            o.scaling_factor = 4.0;
+            o.original_max_position_embeddings = 16;
+            o.long_rope_short_factors = {1.0, 1.1, 1.2, 1.3};
+            o.long_rope_long_factors = {2.0, 2.2, 2.4, 2.6};
+            stampOne(std::string("rope ") + dtypeName + " longrope with ids and length",
+                     iq.rotaryPositionEmbeddingWithPositionIdsAndEffectiveSequenceLength(Expression::input("positions"), Expression::input("length"), o),
+                     ropeInputs, stream);
+            if (dtype != DataType::FP8_E4M3) {
+                Tensor upstream(gpuPlacement, TensorDescriptor(dtype, {2, 4, 48, 64}));
+                stampBackward(std::string("backward rope ") + dtypeName + " longrope with ids", (iq * 3.0).rotaryPositionEmbeddingWithPositionIds(Expression::input("positions"), o),
+                              ropeInputs, upstream, stream);
+            }
+        }
         // transposed and sliced operands: LDS-tiled and broadcast-form kernels, reductions over views
         Tensor t(gpuPlacement, TensorDescriptor(dtype, {24, 4096}));
         const std::unordered_map<std::string, Tensor> withT{{"a", a}, {"b", b}, {"t", t}};

@@ -189,3 +189,21 @@ def test_full_size_round_trip_properties(gpu):
         for b_ in (narrow, wide, again):
             b_.free()
     src.free()
+
+
+def test_every_fp32_bit_pattern_narrows_to_bf16_like_the_oracle(gpu):
+    """All 2^32 fp32 inputs, 2^26 at a time: the device's fp32 -> bf16 (the hardware conversion, canonical NaN) equals the
+    oracle's round-to-nearest-even on every one of them, subnormals, halfway cases, infinities and NaNs included."""
+    from thor_amd.runtime import DeviceBuffer, TypeConverter
+    n = 1 << 26
+    src, dst = DeviceBuffer(n * 4), DeviceBuffer(n * 2)
+    for chunk in range(64):
+        bits = np.arange(chunk * n, (chunk + 1) * n, dtype=np.uint64).astype(np.uint32)
+        src.upload(bits.view(np.float32))
+        TypeConverter.convert_type(src.ptr, dst.ptr, DataType.fp32, DataType.bf16, n)
+        got = dst.download(np.uint16, n)
+        want = oracle.convert(bits.view(np.float32), oracle.FP32, oracle.BF16).view(np.uint16)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, f"chunk {chunk}: {bad.size} mismatches, first input {int(bits[bad[0]]):#010x}: got {got[bad[0]]:#x} want {want[bad[0]]:#x}"
+    src.free()
+    dst.free()

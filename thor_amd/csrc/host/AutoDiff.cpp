@@ -224,6 +224,17 @@ class BackwardGraph {
         n.ragged_runtime_elements_per_value = like.ragged_runtime_elements_per_value;
         return push(std::move(n), dims[values]);
     }
+    // the rotation `like` describes turned the other way, over `values` (same position ids and effective length)
+    uint32_t oppositeRope(uint32_t values, uint32_t positionIds, uint32_t effectiveLength, const ExprNode& like) {
+        ExprNode n = like;
+        n.lhs = values;
+        n.rhs = positionIds;
+        n.aux = effectiveLength;
+        n.rope_inverse = !like.rope_inverse;
+        n.output_dtype.reset();
+        n.input_tensor_dtype.reset();
+        return push(std::move(n), dims[values]);
+    }
     uint32_t raggedExtent(uint32_t values, uint32_t offsets, const ExprNode& like) {
         ExprNode n;
         n.op = ExprOp::RAGGED_VALUEWISE_EXTENT;
@@ -337,7 +348,8 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
         }
         // offsets are structure: nothing flows through the rhs of a ragged op
         const bool ragged = usesRowPartition(n.op);
-        for (uint32_t c : {n.lhs, ragged ? kNone : n.rhs, n.aux})
+        const bool rope = n.op == ExprOp::ROPE;  // position ids and the effective length are structure as well
+        for (uint32_t c : {n.lhs, ragged || rope ? kNone : n.rhs, rope ? kNone : n.aux})
             if (c != kNone && reaches[c]) reaches[i] = 1;
     }
 
@@ -535,6 +547,12 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
                 // upstream gradient run from the other end
                 if (n.scan_op != ScanOp::Sum) throw std::runtime_error(noRule(n.op) + " Only sum scans are differentiable here.");
                 contribute(n.lhs, b.oppositeScan(g, n.op == ExprOp::SEGMENTED_SCAN ? b.value(n.rhs) : kNone, n));
+                break;
+
+            case ExprOp::ROPE:
+                // y = a R x with R a rotation: the gradient is a R^T g, the same rotation turned the other way
+                // (Utilities/Expression/AutoDiff.cpp:4672-4693 there)
+                contribute(n.lhs, b.oppositeRope(g, n.rhs != kNone ? b.value(n.rhs) : kNone, n.aux != kNone ? b.value(n.aux) : kNone, n));
                 break;
 
             default:

@@ -582,6 +582,141 @@ Expression Expression::takeAlongAxis(const Expression& indices, int64_t axis) co
     return out;
 }
 
+// ---- rotary position embedding (Expression.cpp:4334-4507 there) -----------------------------------------------------------
+namespace {
+ExprNode ropeNodeFrom(const RotaryPositionEmbeddingOptions& options) {
+    if (options.base <= 0.0) throw std::runtime_error("RoPE base must be positive.");
+    if (options.scaling_factor <= 0.0) throw std::runtime_error("RoPE scaling factor must be positive.");
+    if (options.attention_factor.has_value() && options.attention_factor.value() <= 0.0) throw std::runtime_error("RoPE attention_factor must be positive.");
+    if (options.rotary_dim != 0 && (options.rotary_dim & 1ull) != 0) throw std::runtime_error("RoPE rotary_dim must be even.");
+    if (options.scaling_kind == RotaryScalingKind::DynamicNTK && options.original_max_position_embeddings == 0) {
+        throw std::runtime_error("Dynamic-NTK RoPE scaling requires original_max_position_embeddings.");
+    }
+    if ((options.scaling_kind == RotaryScalingKind::Yarn || options.scaling_kind == RotaryScalingKind::LongRope ||
+         options.scaling_kind == RotaryScalingKind::Llama3) &&
+        options.original_max_position_embeddings == 0) {
+        throw std::runtime_error("This RoPE scaling kind requires original_max_position_embeddings.");
+    }
+    if (options.scaling_kind == RotaryScalingKind::Yarn && (options.yarn_beta_fast <= 0.0 || options.yarn_beta_slow <= 0.0)) {
+        throw std::runtime_error("YaRN RoPE scaling requires positive beta parameters.");
+    }
+    if (options.scaling_kind == RotaryScalingKind::Llama3 &&
+        (options.llama3_low_freq_factor <= 0.0 || options.llama3_high_freq_factor <= 0.0 ||
+         options.llama3_high_freq_factor <= options.llama3_low_freq_factor)) {
+        throw std::runtime_error("Llama3 RoPE scaling requires 0 < low_freq_factor < high_freq_factor.");
+    }
+    if (options.scaling_kind == RotaryScalingKind::LongRope) {
+        if (options.rotary_dim == 0) throw std::runtime_error("LongRoPE scaling requires an explicit rotary_dim.");
+        const uint64_t expected = options.rotary_dim / 2;
+        if (options.long_rope_short_factors.size() != expected || options.long_rope_long_factors.size() != expected) {
+            throw std::runtime_error("LongRoPE scaling requires short/long factor lists of length rotary_dim / 2.");
+        }
+        for (double f : options.long_rope_short_factors)
+            if (f <= 0.0) throw std::runtime_error("LongRoPE short factors must be positive.");
+        for (double f : options.long_rope_long_factors)
+            if (f <= 0.0) throw std::runtime_error("LongRoPE long factors must be positive.");
+    }
+    ExprNode node;
+    node.op = ExprOp::ROPE;
+    node.rope_sequence_axis = options.sequence_axis;
+    node.rope_head_dim_axis = options.head_dim_axis;
+    node.rope_rotary_dim = options.rotary_dim;
+    node.rope_base = options.base;
+    node.rope_position_offset = options.position_offset;
+    node.rope_interleaved = options.interleaved;
+    node.rope_inverse = options.inverse;
+    node.rope_scaling_kind = options.scaling_kind;
+    node.rope_scaling_factor = options.scaling_factor;
+    node.rope_original_max_position_embeddings = options.original_max_position_embeddings;
+    // the magnitude correction that goes with the stretched frequencies, unless the caller names one
+    if (options.attention_factor.has_value()) {
+        node.rope_attention_factor = options.attention_factor.value();
+    } else if (options.scaling_kind == RotaryScalingKind::Yarn) {
+        node.rope_attention_factor = options.scaling_factor <= 1.0 ? 1.0 : 0.1 * std::log(options.scaling_factor) + 1.0;
+    } else if (options.scaling_kind == RotaryScalingKind::LongRope) {
+        node.rope_attention_factor =
+            options.scaling_factor <= 1.0
+                ? 1.0
+                : std::sqrt(1.0 + std::log(options.scaling_factor) / std::log(static_cast<double>(options.original_max_position_embeddings)));
+    } else {
+        node.rope_attention_factor = 1.0;
+    }
+    node.rope_yarn_beta_fast = options.yarn_beta_fast;
+    node.rope_yarn_beta_slow = options.yarn_beta_slow;
+    node.rope_llama3_low_freq_factor = options.llama3_low_freq_factor;
+    node.rope_llama3_high_freq_factor = options.llama3_high_freq_factor;
+    node.rope_long_rope_short_factors = options.long_rope_short_factors;
+    node.rope_long_rope_long_factors = options.long_rope_long_factors;
+    node.output_dtype = options.output_dtype;
+    node.compute_dtype = options.compute_dtype;
+    return node;
+}
+}  // namespace
+
+Expression Expression::ropeOp(const Expression& input, const Expression* position_ids, const Expression* effective_sequence_length, ExprNode node) {
+    if (!input.expr) throw std::runtime_error("Cannot build RoPE from an empty expression.");
+    auto out = std::make_shared<PhysicalExpression>();
+    GraphMerger merger(*out);
+    // metadata first, so every operand precedes the rotation in the graph
+    if (effective_sequence_length != nullptr) node.aux = merger.absorb(*effective_sequence_length->expr, effective_sequence_length->nodeIndex);
+    if (position_ids != nullptr) node.rhs = merger.absorb(*position_ids->expr, position_ids->nodeIndex);
+    node.lhs = merger.absorb(*input.expr, input.nodeIndex);
+    out->nodes.push_back(std::move(node));
+    out->output_node = static_cast<uint32_t>(out->nodes.size() - 1);
+    return Expression(out, out->output_node);
+}
+
+Expression Expression::rotaryPositionEmbedding(RotaryPositionEmbeddingOptions options) const {
+    if (!expr) throw std::runtime_error("Cannot build RoPE from an empty expression.");
+    return ropeOp(*this, nullptr, nullptr, ropeNodeFrom(options));
+}
+
+Expression Expression::rotaryPositionEmbeddingWithEffectiveSequenceLength(const Expression& effective_sequence_length,
+                                                                          RotaryPositionEmbeddingOptions options) const {
+    if (!effective_sequence_length.expr) throw std::runtime_error("RoPE effective sequence length cannot be an empty expression.");
+    // the scaling rules take the length as a floating-point number, whatever dtype the caller's metadata has
+    const Expression length = effective_sequence_length.cast(DataType::FP32);
+    return ropeOp(*this, nullptr, &length, ropeNodeFrom(options));
+}
+
+Expression Expression::rotaryPositionEmbeddingWithPositionIds(const Expression& position_ids, RotaryPositionEmbeddingOptions options) const {
+    if (!position_ids.expr) throw std::runtime_error("RoPE position ids cannot be an empty expression.");
+    if (options.position_offset != 0) {
+        throw std::runtime_error("RoPE explicit position ids require position_offset == 0 because the ids are absolute positions.");
+    }
+    const Expression ids = position_ids.cast(DataType::FP32);
+    return ropeOp(*this, &ids, nullptr, ropeNodeFrom(options));
+}
+
+Expression Expression::rotaryPositionEmbeddingWithPositionIdsAndEffectiveSequenceLength(const Expression& position_ids,
+                                                                                        const Expression& effective_sequence_length,
+                                                                                        RotaryPositionEmbeddingOptions options) const {
+    if (!position_ids.expr) throw std::runtime_error("RoPE position ids cannot be an empty expression.");
+    if (!effective_sequence_length.expr) throw std::runtime_error("RoPE effective sequence length cannot be an empty expression.");
+    if (options.position_offset != 0) {
+        throw std::runtime_error("RoPE explicit position ids require position_offset == 0 because the ids are absolute positions.");
+    }
+    const Expression ids = position_ids.cast(DataType::FP32);
+    const Expression length = effective_sequence_length.cast(DataType::FP32);
+    return ropeOp(*this, &ids, &length, ropeNodeFrom(options));
+}
+
+std::string ropeKey(const ExprNode& n) {
+    std::string k = "seq=" + std::to_string(n.rope_sequence_axis) + ",dim=" + std::to_string(n.rope_head_dim_axis) + ",rotary=" + std::to_string(n.rope_rotary_dim) +
+                    ",base=" + formatFloatCanonical(n.rope_base) + ",offset=" + std::to_string(n.rope_position_offset) +
+                    (n.rope_interleaved ? ",interleaved" : "") + (n.rope_inverse ? ",inverse" : "") + ",kind=" + std::to_string(static_cast<int>(n.rope_scaling_kind)) +
+                    ",factor=" + formatFloatCanonical(n.rope_scaling_factor) + ",max=" + std::to_string(n.rope_original_max_position_embeddings) +
+                    ",attention=" + formatFloatCanonical(n.rope_attention_factor) + ",yarn=" + formatFloatCanonical(n.rope_yarn_beta_fast) + "/" +
+                    formatFloatCanonical(n.rope_yarn_beta_slow) + ",llama3=" + formatFloatCanonical(n.rope_llama3_low_freq_factor) + "/" +
+                    formatFloatCanonical(n.rope_llama3_high_freq_factor) + ",short=";
+    for (double f : n.rope_long_rope_short_factors) k += formatFloatCanonical(f) + ";";
+    k += ",long=";
+    for (double f : n.rope_long_rope_long_factors) k += formatFloatCanonical(f) + ";";
+    // which of the two optional operands is which (both ride in rhs / aux)
+    k += std::string(",ids=") + (n.rhs != UINT32_MAX ? "1" : "0") + ",length=" + (n.aux != UINT32_MAX ? "1" : "0");
+    return k;
+}
+
 Expression Expression::transpose() const {
     if (!expr) throw std::runtime_error("Cannot transpose an empty expression");
     return unaryOp(*this, ExprOp::TRANSPOSE);
@@ -719,7 +854,7 @@ std::string opName(ExprOp op) {
         {(uint16_t)ExprOp::LGAMMA, "lgamma"}, {(uint16_t)ExprOp::DIGAMMA, "digamma"}, {(uint16_t)ExprOp::EXP, "exp"},
         {(uint16_t)ExprOp::EXPM1, "expm1"}, {(uint16_t)ExprOp::EXP2, "exp2"}, {(uint16_t)ExprOp::EXP10, "exp10"}, {(uint16_t)ExprOp::LN, "ln"},
         {(uint16_t)ExprOp::LOG1P, "log1p"}, {(uint16_t)ExprOp::LOG2, "log2"}, {(uint16_t)ExprOp::LOG10, "log10"}, {(uint16_t)ExprOp::SQRT, "sqrt"},
-        {(uint16_t)ExprOp::TANH, "tanh"}, {(uint16_t)ExprOp::NORMCDF, "normcdf"}, {(uint16_t)ExprOp::SOFTMAX, "softmax"}, {(uint16_t)ExprOp::FILL, "fill"},
+        {(uint16_t)ExprOp::TANH, "tanh"}, {(uint16_t)ExprOp::NORMCDF, "normcdf"}, {(uint16_t)ExprOp::SOFTMAX, "softmax"}, {(uint16_t)ExprOp::ROPE, "rope"}, {(uint16_t)ExprOp::FILL, "fill"},
         {(uint16_t)ExprOp::RESHAPE, "reshape"}, {(uint16_t)ExprOp::UNSQUEEZE, "unsqueeze"}, {(uint16_t)ExprOp::SQUEEZE, "squeeze"},
         {(uint16_t)ExprOp::MIN, "min"}, {(uint16_t)ExprOp::MAX, "max"}, {(uint16_t)ExprOp::MIN_GRAD_LEFT, "min_grad_left"},
         {(uint16_t)ExprOp::MIN_GRAD_RIGHT, "min_grad_right"}, {(uint16_t)ExprOp::MAX_GRAD_LEFT, "max_grad_left"},
@@ -790,6 +925,7 @@ std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex,
         if (isCommutative(n.op) && kids.size() == 2 && kids[1] < kids[0]) std::swap(kids[0], kids[1]);
         text += dtypes();
         if (n.op == ExprOp::TAKE_ALONG_AXIS) text += ":axis=" + axesText(n.reduction_axes);
+        if (n.op == ExprOp::ROPE) text += ":" + ropeKey(n);
         if (isScanOp(n.op)) {
             static const char* const scanNames[] = {"sum", "min", "max", "product", "arg_min", "arg_max"};
             text += std::string(":") + scanNames[static_cast<int>(n.scan_op)] + (n.scan_mode == ScanMode::Inclusive ? ":inclusive" : ":exclusive") +

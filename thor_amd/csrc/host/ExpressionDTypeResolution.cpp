@@ -29,7 +29,7 @@ bool isBindableInputDType(DataType dtype) {
 }
 
 void rejectUnsupportedOp(ExprOp op) {
-    if (isRaggedOp(op) || isStorageViewOp(op) || isWinnerRoutingOp(op) || op == ExprOp::TAKE_ALONG_AXIS || isScanOp(op)) return;
+    if (isRaggedOp(op) || isStorageViewOp(op) || isWinnerRoutingOp(op) || op == ExprOp::TAKE_ALONG_AXIS || op == ExprOp::ROPE || isScanOp(op)) return;
     if (Expression::isLeafOp(op) || Expression::isUnaryOp(op) || Expression::isBinaryOp(op) || Expression::isTernaryOp(op)) return;
     throw std::runtime_error("Expression op '" + opName(op) + "' is outside the elementwise / reduction / cast path of this backend.");
 }
@@ -37,7 +37,7 @@ void rejectUnsupportedOp(ExprOp op) {
 std::vector<DataType> tensorParentDTypes(const ExprNode& node, const std::vector<ExprNode>& nodes, const std::vector<DataType>& resolved) {
     std::vector<DataType> out;
     if (isRaggedOp(node.op)) return {resolved.at(node.lhs)};  // the offsets are structure, not a value
-    if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(node.op)) return {resolved.at(node.lhs)};
+    if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScanOp(node.op)) return {resolved.at(node.lhs)};
     auto add = [&](uint32_t parent) {
         if (parent >= nodes.size()) throw std::runtime_error("Parent node index out of range during dtype resolution.");
         if (!isScalarLeaf(nodes[parent].op)) out.push_back(resolved[parent]);
@@ -109,6 +109,14 @@ DataType nodeOutputDType(const ExprNode& node, const std::vector<ExprNode>& node
             throw std::runtime_error(std::string("take_along_axis indices must have UINT32 or UINT64 dtype, received: ") + dataTypeName(indexType));
         }
         return node.output_dtype.value_or(resolved[node.lhs]);
+    }
+    if (node.op == ExprOp::ROPE) {
+        // fp32 arithmetic on stored values; the result keeps the operand's dtype unless the node names another
+        const DataType out = node.output_dtype.value_or(resolved[node.lhs]);
+        if (!isSupportedFusionFloatingType(resolved[node.lhs]) || !isSupportedFusionFloatingType(out)) {
+            throw std::runtime_error("RoPE requires floating-point input and output dtypes.");
+        }
+        return out;
     }
     if (isWinnerRoutingOp(node.op)) {
         // the gradient of the reduced operand, in the operand's dtype unless the node names another
@@ -211,7 +219,7 @@ void propagateMaterialisedDTypes(PhysicalExpression& expr, const std::vector<uin
             // an explicit conversion boundary: the source keeps its own compute dtype
         } else if (node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST) {
             toParent(node.lhs);  // never into the offsets
-        } else if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(node.op)) {
+        } else if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScanOp(node.op)) {
             // the operands are read as stored tensors: nothing to widen
         } else if (isReductionOp(node.op) || node.op == ExprOp::SOFTMAX || isSegmentedReduceOp(node.op)) {
             // the reduction's mandatory fp32 stays inside the reduction; its producer keeps its own policy
@@ -265,7 +273,7 @@ void resolveInPlace(PhysicalExpression& expr, const std::vector<DataType>& rootD
         const DataType logicalIn = nodeLogicalInputDType(node, expr.nodes, resolved);
         DataType requested;
         if (node.op == ExprOp::CAST || isShapeOnly(node.op) || node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST ||
-            isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(node.op)) {
+            isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScanOp(node.op)) {
             requested = out;  // values pass through unchanged (a normalised broadcast divides in fp32 and rounds once)
         } else if (isSegmentedReduceOp(node.op)) {
             requested = DataType::FP32;
@@ -351,7 +359,7 @@ DataType toSupportedComputeDType(ExprOp op, DataType requested) {
         throw std::runtime_error("Unsupported boolean/comparison/where dtype in toSupportedComputeDType.");
     }
     if (op == ExprOp::CAST || isShapeOnly(op) || op == ExprOp::RAGGED_VALUEWISE_EXTENT || op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(op) ||
-        op == ExprOp::TAKE_ALONG_AXIS || isScanOp(op)) {
+        op == ExprOp::TAKE_ALONG_AXIS || op == ExprOp::ROPE || isScanOp(op)) {
         if (isBindableInputDType(requested)) return requested;
         throw std::runtime_error("Unsupported passthrough dtype in toSupportedComputeDType.");
     }

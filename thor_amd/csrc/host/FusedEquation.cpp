@@ -9,6 +9,7 @@
 #include "CubScanInternal.h"
 #include "HipSourceEmitter.h"
 #include "IndexGather.h"
+#include "RotaryEmbedding.h"
 #include "ReductionPlanner.h"
 #include "RowFusion.h"
 #include "ShapeInference.h"
@@ -61,6 +62,7 @@ std::string structuralKey(const ExprNode& n) {
       << n.ragged_runtime_max_active_values << "|" << n.ragged_runtime_elements_per_value << "|" << n.segmented_broadcast_normalize_by_length << "|"
       << axesKey(n.view_dims) << "|" << axesKey(n.view_strides) << "|" << n.view_element_offset << "|" << static_cast<int>(n.scan_op) << "|"
       << static_cast<int>(n.scan_mode) << "|" << n.scan_axis << "|" << n.scan_reverse;
+    if (n.op == ExprOp::ROPE) k << "|" << ropeKey(n);
     return k.str();
 }
 
@@ -156,6 +158,13 @@ class GraphBuilder {
             node.lhs = asTensorOperand(node.lhs, false);
             if (isStorageViewOp(out.nodes[node.lhs].op)) node.lhs = castOf(node.lhs, out.nodes[node.lhs].output_dtype.value());
             if (node.op == ExprOp::SEGMENTED_SCAN) node.rhs = asTensorOperand(node.rhs, false);
+        } else if (node.op == ExprOp::ROPE) {
+            // the rotation kernel addresses dense storage; position ids and the effective length are small tensors it reads
+            for (uint32_t* operand : {&node.lhs, &node.rhs, &node.aux}) {
+                if (*operand == UINT32_MAX) continue;
+                *operand = asTensorOperand(*operand, false);
+                if (isStorageViewOp(out.nodes[*operand].op)) *operand = castOf(*operand, out.nodes[*operand].output_dtype.value());
+            }
         } else if (node.op == ExprOp::TAKE_ALONG_AXIS) {
             node.lhs = asTensorOperand(node.lhs, false);
             node.rhs = asTensorOperand(node.rhs, false);
@@ -228,7 +237,7 @@ uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
 bool consumesGather(const ExprNode& consumer) {
     if (consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT || consumer.op == ExprOp::WHERE || consumer.op == ExprOp::CAST) return true;
     if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX || isWinnerRoutingOp(consumer.op) ||
-        consumer.op == ExprOp::TAKE_ALONG_AXIS || isScanOp(consumer.op)) {
+        consumer.op == ExprOp::TAKE_ALONG_AXIS || consumer.op == ExprOp::ROPE || isScanOp(consumer.op)) {
         return false;
     }
     return Expression::isBinaryOp(consumer.op) || Expression::isUnaryOp(consumer.op);
@@ -366,6 +375,31 @@ std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpressio
                     throw std::runtime_error("Segmented scan offsets do not have the ragged descriptor's batch size + 1 entries.");
                 }
                 dims[i] = dims[n.lhs];
+                break;
+            }
+            case ExprOp::ROPE: {
+                const std::vector<uint64_t>& in = dims[n.lhs];
+                if (n.rope_sequence_axis >= in.size() || n.rope_head_dim_axis >= in.size() || n.rope_sequence_axis == n.rope_head_dim_axis) {
+                    throw std::runtime_error("RoPE sequence and head-dimension axes must be distinct axes of the input.");
+                }
+                const uint64_t headDim = in[n.rope_head_dim_axis];
+                const uint64_t rotary = n.rope_rotary_dim == 0 ? headDim : n.rope_rotary_dim;
+                if (rotary == 0 || rotary > headDim || (rotary & 1ull) != 0) {
+                    throw std::runtime_error("RoPE rotary_dim must be even and no larger than the head dimension.");
+                }
+                if (n.rope_scaling_kind == RotaryScalingKind::LongRope && n.rope_long_rope_short_factors.size() != rotary / 2) {
+                    throw std::runtime_error("LongRoPE scaling requires short/long factor lists of length rotary_dim / 2.");
+                }
+                auto elements = [&](uint32_t node) {
+                    uint64_t e = 1;
+                    for (uint64_t d : dims[node]) e *= d;
+                    return e;
+                };
+                if (n.rhs != UINT32_MAX && elements(n.rhs) != in[n.rope_sequence_axis]) {
+                    throw std::runtime_error("RoPE position ids must hold one position per element of the sequence axis.");
+                }
+                if (n.aux != UINT32_MAX && elements(n.aux) != 1) throw std::runtime_error("RoPE effective sequence length must be a single element.");
+                dims[i] = in;
                 break;
             }
             case ExprOp::TAKE_ALONG_AXIS:
@@ -533,6 +567,10 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
                 ensureTensor(n.rhs);
+            } else if (n.op == ExprOp::ROPE) {
+                graph->role[i] = Role::Materialized;
+                for (uint32_t operand : {n.lhs, n.rhs, n.aux})
+                    if (operand != UINT32_MAX) ensureTensor(operand);
             } else if (n.op == ExprOp::RAGGED_VALUEWISE_EXTENT) {
                 // the kernel that produces these values stops at the rows the partition covers
                 graph->role[i] = Role::Materialized;
@@ -612,6 +650,9 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
                 sources.push_back(graph->expr.nodes[i].lhs);
             } else if (graph->expr.nodes[i].op == ExprOp::SCAN) {
                 sources.push_back(graph->expr.nodes[i].lhs);
+            } else if (graph->expr.nodes[i].op == ExprOp::ROPE) {
+                for (uint32_t operand : {graph->expr.nodes[i].lhs, graph->expr.nodes[i].rhs, graph->expr.nodes[i].aux})
+                    if (operand != UINT32_MAX) sources.push_back(operand);
             } else if (isWinnerRoutingOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::TAKE_ALONG_AXIS ||
                        graph->expr.nodes[i].op == ExprOp::SEGMENTED_SCAN) {
                 sources.push_back(graph->expr.nodes[i].lhs);
@@ -792,7 +833,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     auto runsInFusedKernel = [&](uint32_t i) {
         const ExprOp op = expr.nodes[i].op;
         return graph->role[i] == Role::Materialized && !isReductionOp(op) && !isSegmentedReduceOp(op) && op != ExprOp::SEGMENTED_BROADCAST &&
-               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && !isScanOp(op) && op != ExprOp::INPUT;
+               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && op != ExprOp::ROPE && !isScanOp(op) && op != ExprOp::INPUT;
     };
     std::vector<uint32_t> levelOf = graph->level;
     if (stageFusionEnabled()) {
@@ -804,6 +845,9 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 sources.push_back(n.lhs);
             } else if (n.op == ExprOp::SCAN) {
                 sources = {n.lhs};
+            } else if (n.op == ExprOp::ROPE) {
+                for (uint32_t operand : {n.lhs, n.rhs, n.aux})
+                    if (operand != UINT32_MAX) sources.push_back(operand);
             } else if (isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS || n.op == ExprOp::SEGMENTED_SCAN) {
                 sources = {n.lhs, n.rhs};
             } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
@@ -1264,6 +1308,23 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                     stage.scan = std::make_shared<StampedScan>(kernels, values, offsets, temp, scanned, arg);
                 }
                 tensorOf[i] = scanned;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(stage));
+                done[i] = 1;
+                continue;
+            }
+            if (n.op == ExprOp::ROPE) {
+                Tensor rotated = allocateFor(i);
+                StampedExecutionStage stage;
+                stage.kind = StampedExecutionStage::Kind::FusedKernel;
+                stage.gpu_num = device_num;
+                std::vector<uint32_t> operands = {n.lhs};
+                if (n.rhs != UINT32_MAX) operands.push_back(n.rhs);
+                if (n.aux != UINT32_MAX) operands.push_back(n.aux);
+                stage.dependency_stage_indices = dependenciesOf(operands);
+                stage.kernel = stampRotaryEmbedding(tensorOf[n.lhs], n.rhs != UINT32_MAX ? std::optional<Tensor>(tensorOf[n.rhs]) : std::nullopt,
+                                                    n.aux != UINT32_MAX ? std::optional<Tensor>(tensorOf[n.aux]) : std::nullopt, rotated, n, device_num);
+                tensorOf[i] = rotated;
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
                 done[i] = 1;

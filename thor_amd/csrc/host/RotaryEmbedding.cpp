@@ -1,0 +1,268 @@
+// Expression::rotaryPositionEmbedding: pairs of the head dimension turned by an angle that grows with the position
+// (reference behaviour: Utilities/Expression/CudaSourceEmitter.cpp:3538-3697 angle, frequency rules and the rotation;
+// Expression.cpp:4334-4426 parameters).
+//
+// The angle depends on the position and the pair only, so a thread owns one (position, group of pairs) item, works its sines
+// and cosines out once and keeps them in registers while it walks every other coordinate of the tensor (batch, heads): the
+// transcendental work is spread over that walk and the kernel stays a stream of 16-byte loads and stores.  The tensor is read
+// as [O, first special axis, M, second special axis, I] whichever order the sequence and head-dimension axes come in; when the
+// head dimension is the last axis a thread moves whole vectors along it, otherwise single elements.
+#include "RotaryEmbedding.h"
+
+#include "HipSourceEmitter.h"
+#include "ReductionPlanner.h"
+#include "Utilities/Expression/CompiledEquation.h"
+#include "thorhip_numeric_embed.h"
+
+#include <algorithm>
+#include <sstream>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+namespace {
+
+std::string floatArray(const std::vector<double>& values) {
+    std::string s = "{";
+    for (size_t i = 0; i < values.size(); ++i) s += (i ? ", " : "") + floatLiteral(values[i]);
+    return s + "}";
+}
+
+// Statements that leave the frequency of pair `j` (a float expression) in `freq`; every rule in fp32, operation by operation as
+// the reference emits it.
+std::string frequencyStatements(const ExprNode& n, uint64_t rotary, const std::string& j, const std::string& ind) {
+    std::ostringstream s;
+    const std::string rot = "(float)" + std::to_string(rotary) + "ull";
+    const std::string base = floatLiteral(n.rope_base), factor = floatLiteral(n.rope_scaling_factor);
+    const std::string originalMax = floatLiteral(static_cast<double>(n.rope_original_max_position_embeddings));
+    switch (n.rope_scaling_kind) {
+        case RotaryScalingKind::DynamicNTK:
+            s << ind << "float base = " << base << ";\n";
+            s << ind << "if (seqLen > " << originalMax << " && " << rotary << "ull > 2ull) {\n";
+            s << ind << "    const float ratio = (" << factor << " * seqLen / " << originalMax << ") - (" << factor << " - 1.0f);\n";
+            s << ind << "    base = base * powf(ratio, " << rot << " / (float)" << (rotary - 2) << "ull);\n";
+            s << ind << "}\n";
+            s << ind << "freq = powf(base, -2.0f * " << j << " / " << rot << ");\n";
+            break;
+        case RotaryScalingKind::Yarn:
+            s << ind << "const float posFreq = powf(" << base << ", 2.0f * " << j << " / " << rot << ");\n";
+            s << ind << "const float extrapolated = 1.0f / posFreq;\n";
+            s << ind << "const float interpolated = 1.0f / (" << factor << " * posFreq);\n";
+            s << ind << "const float logBase = logf(" << base << ");\n";
+            s << ind << "float low = (" << rot << " * logf(" << originalMax << " / (" << floatLiteral(n.rope_yarn_beta_fast)
+              << " * 6.2831853071795864769f))) / (2.0f * logBase);\n";
+            s << ind << "float high = (" << rot << " * logf(" << originalMax << " / (" << floatLiteral(n.rope_yarn_beta_slow)
+              << " * 6.2831853071795864769f))) / (2.0f * logBase);\n";
+            s << ind << "low = fmaxf(floorf(low), 0.0f);\n";
+            s << ind << "high = fminf(ceilf(high), (float)" << (rotary - 1) << "ull);\n";
+            s << ind << "if (low == high) high += 0.001f;\n";
+            s << ind << "const float ramp = fminf(fmaxf((" << j << " - low) / (high - low), 0.0f), 1.0f);\n";
+            s << ind << "freq = interpolated * ramp + extrapolated * (1.0f - ramp);\n";
+            break;
+        case RotaryScalingKind::LongRope:
+            s << ind << "const float stretch = seqLen > " << originalMax << " ? thor_rope_long_factors[pair] : thor_rope_short_factors[pair];\n";
+            s << ind << "freq = 1.0f / (stretch * powf(" << base << ", 2.0f * " << j << " / " << rot << "));\n";
+            break;
+        case RotaryScalingKind::Llama3: {
+            const std::string lowFactor = floatLiteral(n.rope_llama3_low_freq_factor), highFactor = floatLiteral(n.rope_llama3_high_freq_factor);
+            s << ind << "const float plain = powf(" << base << ", -2.0f * " << j << " / " << rot << ");\n";
+            s << ind << "const float wavelength = 6.2831853071795864769f / plain;\n";
+            s << ind << "const float lowWavelength = " << originalMax << " / " << lowFactor << ";\n";
+            s << ind << "const float highWavelength = " << originalMax << " / " << highFactor << ";\n";
+            s << ind << "if (wavelength > lowWavelength) {\n";
+            s << ind << "    freq = plain / " << factor << ";\n";
+            s << ind << "} else if (wavelength < highWavelength) {\n";
+            s << ind << "    freq = plain;\n";
+            s << ind << "} else {\n";
+            s << ind << "    const float smooth = (" << originalMax << " / wavelength - " << lowFactor << ") / (" << highFactor << " - " << lowFactor << ");\n";
+            s << ind << "    freq = (1.0f - smooth) * (plain / " << factor << ") + smooth * plain;\n";
+            s << ind << "}\n";
+            break;
+        }
+        case RotaryScalingKind::None:
+        case RotaryScalingKind::Linear:
+            s << ind << "freq = powf(" << base << ", -2.0f * " << j << " / " << rot << ");\n";
+            break;
+    }
+    return s.str();
+}
+
+}  // namespace
+
+std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, const std::optional<Tensor>& positionIds,
+                                                      const std::optional<Tensor>& effectiveLength, const Tensor& output, const ExprNode& n,
+                                                      int deviceNum) {
+    if (!values.isInitialized() || !output.isInitialized()) throw std::runtime_error("RoPE requires initialized tensors.");
+    const std::vector<uint64_t>& dims = values.getDimensions();
+    const uint32_t seqAxis = n.rope_sequence_axis, dimAxis = n.rope_head_dim_axis;
+    if (seqAxis >= dims.size() || dimAxis >= dims.size() || seqAxis == dimAxis) {
+        throw std::runtime_error("RoPE sequence and head-dimension axes must be distinct axes of the input.");
+    }
+    if (output.getDimensions() != dims) throw std::runtime_error("RoPE output must have the shape of its input.");
+    for (uint64_t d : dims)
+        if (d == 0) throw std::runtime_error("RoPE does not support zero-sized dimensions.");
+    if (!values.isDenseContiguous() || !output.isDenseContiguous()) throw std::runtime_error("RoPE requires dense tensors.");
+    const uint64_t seq = dims[seqAxis], headDim = dims[dimAxis];
+    const uint64_t rotary = n.rope_rotary_dim == 0 ? headDim : n.rope_rotary_dim;
+    if (rotary == 0 || rotary > headDim || (rotary & 1ull) != 0) throw std::runtime_error("RoPE rotary_dim must be even and no larger than the head dimension.");
+    const uint64_t half = rotary / 2;
+    if (n.rope_base <= 0.0 || n.rope_scaling_factor <= 0.0) throw std::runtime_error("Invalid RoPE base/scaling factor during code generation.");
+    if (n.rope_scaling_kind == RotaryScalingKind::LongRope &&
+        (n.rope_long_rope_short_factors.size() != half || n.rope_long_rope_long_factors.size() != half)) {
+        throw std::runtime_error("LongRoPE code generation requires short/long factor lists of length rotary_dim / 2.");
+    }
+    if (positionIds.has_value()) {
+        if (!positionIds->isInitialized() || !positionIds->isDenseContiguous() || positionIds->getTotalNumElements() != seq) {
+            throw std::runtime_error("RoPE position ids must hold one position per element of the sequence axis.");
+        }
+    }
+    if (effectiveLength.has_value()) {
+        if (!effectiveLength->isInitialized() || effectiveLength->getTotalNumElements() != 1) {
+            throw std::runtime_error("RoPE effective sequence length must be a single element.");
+        }
+    }
+
+    // [O, first, M, second, I] around the two special axes
+    const uint32_t firstAxis = std::min(seqAxis, dimAxis), secondAxis = std::max(seqAxis, dimAxis);
+    uint64_t outerCount = 1, middleCount = 1, innerCount = 1;
+    for (size_t d = 0; d < dims.size(); ++d) {
+        if (d < firstAxis) outerCount *= dims[d];
+        if (d > firstAxis && d < secondAxis) middleCount *= dims[d];
+        if (d > secondAxis) innerCount *= dims[d];
+    }
+    auto strideOf = [&](uint32_t axis) {
+        uint64_t s = 1;
+        for (size_t d = axis + 1; d < dims.size(); ++d) s *= dims[d];
+        return s;
+    };
+    const uint64_t seqStride = strideOf(seqAxis), dimStride = strideOf(dimAxis);
+    const uint64_t middleStride = dims[secondAxis] * innerCount, outerStride = dims[firstAxis] * middleCount * middleStride;
+    const uint64_t walk = outerCount * middleCount * innerCount;  // coordinates a thread visits with one set of angles
+    const uint64_t total = walk * seq * headDim;
+
+    const uint32_t inBytes = dataTypeSizeInBytes(values.getDataType()), outBytes = dataTypeSizeInBytes(output.getDataType());
+    const uint64_t tail = headDim - rotary;
+    int vec = dimStride == 1 ? static_cast<int>(16 / std::max(inBytes, outBytes)) : 1;
+    auto fits = [&](int v) {
+        if (v == 1) return true;
+        if (tail % v != 0) return false;
+        if (n.rope_interleaved ? rotary % v != 0 : half % v != 0) return false;
+        return pointerAlignment(values.getMemPtr()) % (static_cast<uint64_t>(v) * inBytes) == 0 &&
+               pointerAlignment(output.getMemPtr()) % (static_cast<uint64_t>(v) * outBytes) == 0;
+    };
+    while (!fits(vec)) vec /= 2;
+    const bool pairsInsideVector = n.rope_interleaved && vec > 1;
+    const uint64_t pairSlots = n.rope_interleaved ? (vec > 1 ? rotary / vec : half) : half / vec;
+    const int pairsPerThread = n.rope_interleaved ? (vec > 1 ? vec / 2 : 1) : vec;
+    const uint64_t slots = pairSlots + tail / vec;
+    const uint64_t items = seq * slots;
+    const uint32_t threads = 256;
+    const uint64_t blocksPerChunk = (items + threads - 1) / threads;
+    // enough blocks to fill the chip, each walking as long a stretch as that leaves
+    uint64_t chunks = std::min<uint64_t>(walk, std::max<uint64_t>(1, (4096 + blocksPerChunk - 1) / blocksPerChunk));
+    const uint64_t walkPerChunk = (walk + chunks - 1) / chunks;
+    chunks = (walk + walkPerChunk - 1) / walkPerChunk;
+    const uint64_t blocks = blocksPerChunk * chunks;
+    if (blocks > 0x7fffffffull) throw std::runtime_error("RoPE: the tensor is too large for one launch.");
+
+    const std::string inType = deviceTypeName(values.getDataType()), outType = deviceTypeName(output.getDataType());
+    const bool needsLength = n.rope_scaling_kind == RotaryScalingKind::DynamicNTK || n.rope_scaling_kind == RotaryScalingKind::LongRope;
+
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude;
+    if (n.rope_scaling_kind == RotaryScalingKind::LongRope) {
+        s << "__device__ const float thor_rope_short_factors[" << half << "] = " << floatArray(n.rope_long_rope_short_factors) << ";\n";
+        s << "__device__ const float thor_rope_long_factors[" << half << "] = " << floatArray(n.rope_long_rope_long_factors) << ";\n";
+    }
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_rope(const " << inType << "* x";
+    if (positionIds.has_value()) s << ", const " << deviceTypeName(positionIds->getDataType()) << "* ids";
+    if (effectiveLength.has_value()) s << ", const " << deviceTypeName(effectiveLength->getDataType()) << "* length";
+    s << ", " << outType << "* out) {\n";
+    s << "    constexpr int V = " << vec << ", P = " << pairsPerThread << ";\n";
+    s << "    const thor::u64 chunk = blockIdx.x / " << blocksPerChunk << "u;\n";
+    s << "    const thor::u64 item = (thor::u64)(blockIdx.x % " << blocksPerChunk << "u) * " << threads << " + threadIdx.x;\n";
+    s << "    if (item >= " << items << "ull) return;\n";
+    s << "    const thor::u64 position = item / " << slots << "ull, slot = item % " << slots << "ull;\n";
+    s << "    const thor::u64 walkFirst = chunk * " << walkPerChunk << "ull;\n";
+    s << "    const thor::u64 walkLast = walkFirst + " << walkPerChunk << "ull < " << walk << "ull ? walkFirst + " << walkPerChunk << "ull : " << walk << "ull;\n";
+    // address of (walk coordinate w, this position, head-dimension coordinate d)
+    s << "    auto at = [&](thor::u64 w, thor::u64 d) {\n";
+    s << "        const thor::u64 i = w % " << innerCount << "ull, m = (w / " << innerCount << "ull) % " << middleCount << "ull, o = w / " << innerCount * middleCount
+      << "ull;\n";
+    s << "        return o * " << outerStride << "ull + m * " << middleStride << "ull + i + position * " << seqStride << "ull + d * " << dimStride << "ull;\n";
+    s << "    };\n";
+    if (tail != 0) {
+        s << "    if (slot >= " << pairSlots << "ull) {\n";
+        s << "        // beyond the rotary part: a copy\n";
+        s << "        const thor::u64 d = " << rotary << "ull + (slot - " << pairSlots << "ull) * V;\n";
+        s << "        for (thor::u64 w = walkFirst; w < walkLast; ++w) {\n";
+        s << "            thor::Pack<" << inType << ", V> p;\n            p.loadStream(x + at(w, d));\n";
+        s << "            thor::Pack<" << outType << ", V> q;\n";
+        s << "#pragma unroll\n            for (int k = 0; k < V; ++k) q.v[k] = thor::fromFloat<" << outType << ">(thor::toFloat(p.v[k]));\n";
+        s << "            q.storeStream(out + at(w, d));\n        }\n        return;\n    }\n";
+    }
+    s << "    const thor::u64 firstPair = slot * P;\n";
+    if (positionIds.has_value()) {
+        s << "    float angleBase = thor::toFloat(ids[position]);\n";
+    } else {
+        s << "    float angleBase = (float)position + " << floatLiteral(static_cast<double>(n.rope_position_offset)) << ";\n";
+    }
+    if (n.rope_scaling_kind == RotaryScalingKind::Linear) s << "    angleBase = angleBase / " << floatLiteral(n.rope_scaling_factor) << ";\n";
+    if (needsLength) {
+        const std::string extent = effectiveLength.has_value() ? std::string("thor::toFloat(length[0])") : floatLiteral(static_cast<double>(seq));
+        s << "    const float seqLen = fmaxf(" << extent << " + " << floatLiteral(static_cast<double>(std::max<int64_t>(0, n.rope_position_offset)))
+          << ", 1.0f);\n";
+    }
+    s << "    float sn[P], cs[P];\n";
+    s << "#pragma unroll\n    for (int k = 0; k < P; ++k) {\n";
+    s << "        const thor::u64 pair = firstPair + k;\n";
+    s << "        float freq = 0.0f;\n";
+    s << "        {\n" << frequencyStatements(n, rotary, "(float)pair", "            ") << "        }\n";
+    s << "        const float theta = angleBase * freq;\n";
+    s << "        sn[k] = sinf(theta);\n        cs[k] = cosf(theta);\n";
+    if (n.rope_attention_factor != 1.0) {
+        s << "        sn[k] *= " << floatLiteral(n.rope_attention_factor) << ";\n        cs[k] *= " << floatLiteral(n.rope_attention_factor) << ";\n";
+    }
+    if (n.rope_inverse) s << "        sn[k] = -sn[k];\n";
+    s << "    }\n";
+    s << "    for (thor::u64 w = walkFirst; w < walkLast; ++w) {\n";
+    if (pairsInsideVector) {
+        s << "        const thor::u64 e = at(w, firstPair * 2);\n";
+        s << "        thor::Pack<" << inType << ", V> p;\n        p.loadStream(x + e);\n";
+        s << "        thor::Pack<" << outType << ", V> q;\n";
+        s << "#pragma unroll\n        for (int k = 0; k < P; ++k) {\n";
+        s << "            const float a = thor::toFloat(p.v[2 * k]), b = thor::toFloat(p.v[2 * k + 1]);\n";
+        s << "            q.v[2 * k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
+        s << "            q.v[2 * k + 1] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
+        s << "        }\n        q.storeStream(out + e);\n";
+    } else {
+        // the two elements of a pair lie `apart` coordinates from each other along the head dimension
+        const uint64_t apart = n.rope_interleaved ? 1 : half;
+        const std::string firstCoordinate = n.rope_interleaved ? "firstPair * 2" : "firstPair";
+        s << "        const thor::u64 ea = at(w, " << firstCoordinate << "), eb = at(w, " << firstCoordinate << " + " << apart << "ull);\n";
+        s << "        thor::Pack<" << inType << ", V> pa, pb;\n        pa.loadStream(x + ea);\n        pb.loadStream(x + eb);\n";
+        s << "        thor::Pack<" << outType << ", V> qa, qb;\n";
+        s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
+        s << "            const float a = thor::toFloat(pa.v[k]), b = thor::toFloat(pb.v[k]);\n";
+        s << "            qa.v[k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
+        s << "            qb.v[k] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
+        s << "        }\n        qa.storeStream(out + ea);\n        qb.storeStream(out + eb);\n";
+    }
+    s << "    }\n}\n";
+
+    const std::shared_ptr<CompiledKernel> kernel = compileKernel(s.str(), "thor_rope", deviceNum, /*fastContract=*/false);
+    std::ostringstream description;
+    description << "rope(seq=" << seq << ",head_dim=" << headDim << ",rotary=" << rotary << (n.rope_interleaved ? ",interleaved" : "")
+                << (n.rope_inverse ? ",inverse" : "") << ",walk=" << walk << "/" << chunks << ",vec=" << vec << ",grid=" << blocks << ") [" << kernel->kernelName
+                << "]";
+    std::vector<Tensor> inputs = {values};
+    if (positionIds.has_value()) inputs.push_back(*positionIds);
+    if (effectiveLength.has_value()) inputs.push_back(*effectiveLength);
+    std::vector<size_t> inputArgs;
+    for (size_t i = 0; i < inputs.size(); ++i) inputArgs.push_back(i);
+    return std::make_shared<StampedEquation>(kernel, inputs, std::vector<Tensor>{output}, std::vector<StampedEquation::ScalarArgument>{}, inputArgs,
+                                             std::vector<size_t>{inputs.size()}, inputs.size() + 1, /*passNumel=*/false, total, total > UINT32_MAX,
+                                             static_cast<uint32_t>(blocks), threads, /*flops=*/0, description.str());
+}
+
+}  // namespace ThorImplementation

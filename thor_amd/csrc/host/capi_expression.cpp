@@ -197,6 +197,33 @@ thor_expr_t thor_expr_scan(thor_expr_t input, thor_expr_t offsets, int op, int64
 thor_expr_t thor_expr_take_along_axis(thor_expr_t input, thor_expr_t indices, int64_t axis) {
     THOR_CAPI_TRY_PTR(require(input, "input"); require(indices, "indices"); return new thor_expr{input->expr.takeAlongAxis(indices->expr, axis)};)
 }
+thor_expr_t thor_expr_rope(thor_expr_t input, thor_expr_t position_ids, thor_expr_t effective_sequence_length, const thor_rope_options* options) {
+    THOR_CAPI_TRY_PTR(
+        require(input, "input"); if (!options) throw std::invalid_argument("rope needs options.");
+        if (options->scaling_kind < 0 || options->scaling_kind > 5) throw std::invalid_argument("rope scaling_kind must be 0..5");
+        if (options->num_long_rope_factors > 0 && (!options->long_rope_short_factors || !options->long_rope_long_factors)) {
+            throw std::invalid_argument("rope needs both LongRoPE factor lists.");
+        }
+        RotaryPositionEmbeddingOptions o;
+        o.sequence_axis = options->sequence_axis; o.head_dim_axis = options->head_dim_axis; o.rotary_dim = options->rotary_dim; o.base = options->base;
+        o.position_offset = options->position_offset; o.interleaved = options->interleaved != 0; o.inverse = options->inverse != 0;
+        o.scaling_kind = static_cast<RotaryScalingKind>(options->scaling_kind); o.scaling_factor = options->scaling_factor;
+        o.original_max_position_embeddings = options->original_max_position_embeddings;
+        if (options->attention_factor > 0.0) o.attention_factor = options->attention_factor;
+        o.yarn_beta_fast = options->yarn_beta_fast; o.yarn_beta_slow = options->yarn_beta_slow;
+        o.llama3_low_freq_factor = options->llama3_low_freq_factor; o.llama3_high_freq_factor = options->llama3_high_freq_factor;
+        if (options->num_long_rope_factors > 0) {
+            o.long_rope_short_factors.assign(options->long_rope_short_factors, options->long_rope_short_factors + options->num_long_rope_factors);
+            o.long_rope_long_factors.assign(options->long_rope_long_factors, options->long_rope_long_factors + options->num_long_rope_factors);
+        }
+        o.output_dtype = optionalDType(options->output_dtype); o.compute_dtype = optionalDType(options->compute_dtype);
+        if (position_ids && effective_sequence_length) {
+            return new thor_expr{input->expr.rotaryPositionEmbeddingWithPositionIdsAndEffectiveSequenceLength(position_ids->expr, effective_sequence_length->expr, o)};
+        }
+        if (position_ids) return new thor_expr{input->expr.rotaryPositionEmbeddingWithPositionIds(position_ids->expr, o)};
+        if (effective_sequence_length) return new thor_expr{input->expr.rotaryPositionEmbeddingWithEffectiveSequenceLength(effective_sequence_length->expr, o)};
+        return new thor_expr{input->expr.rotaryPositionEmbedding(o)};)
+}
 thor_expr_t thor_expr_reshape(thor_expr_t input, const uint64_t* dims, int rank) {
     THOR_CAPI_TRY_PTR(require(input, "expression"); return new thor_expr{input->expr.reshape(u64s(dims, rank))};)
 }

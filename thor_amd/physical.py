@@ -75,6 +75,7 @@ PROTOTYPES = {
     "thor_expr_reduce": (_vp, [_cp, _vp, _u64p, _i, _u64p, _i]), "thor_expr_reshape": (_vp, [_vp, _u64p, _i]),
     "thor_expr_strided_view": (_vp, [_vp, _u64p, _u64p, _i, ctypes.c_uint64]),
     "thor_expr_take_along_axis": (_vp, [_vp, _vp, ctypes.c_int64]),
+    "thor_expr_rope": (_vp, [_vp, _vp, _vp, _vp]),
     "thor_expr_scan": (_vp, [_vp, _vp, _i, ctypes.c_int64, _i, _i]),
     "thor_expr_unsqueeze": (_vp, [_vp, _u64p, _i]), "thor_expr_squeeze": (_vp, [_vp, _u64p, _i]), "thor_expr_destroy": (None, [_vp]),
     "thor_expr_num_nodes": (_i, [_vp]), "thor_expr_canonical": (_i, [_vp, _cp, _sz, ctypes.POINTER(_sz)]),
@@ -522,6 +523,27 @@ def segmented_broadcast(per_segment_values: PhysicalTensor, segment_offsets: Phy
            "segmented_broadcast")
 
 
+class RotaryScalingKind(enum.IntEnum):
+    """thor.physical.RotaryScalingKind (Utilities/Expression/Expression.h:150-157 there)."""
+    none = 0
+    linear = 1
+    dynamic_ntk = 2
+    yarn = 3
+    longrope = 4
+    llama3 = 5
+
+
+class _RopeOptions(ctypes.Structure):
+    """thor_rope_options of the C-ABI."""
+    _fields_ = [("sequence_axis", ctypes.c_uint32), ("head_dim_axis", ctypes.c_uint32), ("rotary_dim", ctypes.c_uint64), ("base", ctypes.c_double),
+                ("position_offset", ctypes.c_int64), ("interleaved", ctypes.c_int), ("inverse", ctypes.c_int), ("scaling_kind", ctypes.c_int),
+                ("scaling_factor", ctypes.c_double), ("original_max_position_embeddings", ctypes.c_uint64), ("attention_factor", ctypes.c_double),
+                ("yarn_beta_fast", ctypes.c_double), ("yarn_beta_slow", ctypes.c_double), ("llama3_low_freq_factor", ctypes.c_double),
+                ("llama3_high_freq_factor", ctypes.c_double), ("long_rope_short_factors", ctypes.POINTER(ctypes.c_double)),
+                ("long_rope_long_factors", ctypes.POINTER(ctypes.c_double)), ("num_long_rope_factors", ctypes.c_uint64), ("output_dtype", ctypes.c_int),
+                ("compute_dtype", ctypes.c_int)]
+
+
 class ScanOp(enum.IntEnum):
     """thor.physical.ScanOp (Utilities/Expression/Expression.h:181-188 there)."""
     sum = 0
@@ -732,6 +754,36 @@ class Expression:
     def take_along_axis(self, indices: "Expression", axis: int = -1) -> "Expression":
         """Gather along one axis with UINT32 / UINT64 indices; the result has the shape of ``indices``."""
         return Expression(_handle(lib().thor_expr_take_along_axis(self._h, indices._h, axis), "take_along_axis"))
+
+    def rope(self, sequence_axis: int = 2, head_dim_axis: int = 3, rotary_dim: int = 0, base: float = 10000.0, position_offset: int = 0,
+             interleaved: bool = False, inverse: bool = False, scaling_kind: "RotaryScalingKind" = None, scaling_factor: float = 1.0,
+             original_max_position_embeddings: int = 0, attention_factor: Optional[float] = None, yarn_beta_fast: float = 32.0,
+             yarn_beta_slow: float = 1.0, llama3_low_freq_factor: float = 1.0, llama3_high_freq_factor: float = 4.0,
+             long_rope_short_factors: Sequence[float] = (), long_rope_long_factors: Sequence[float] = (), output_dtype: Optional[DataType] = None,
+             compute_dtype: Optional[DataType] = None, allow_in_place_materialization: bool = False, position_ids: Optional["Expression"] = None,
+             effective_sequence_length: Optional["Expression"] = None) -> "Expression":
+        """Rotary position embedding (thor.physical.Expression.rope / rotary_position_embedding: bindings/python/src/core/physical/
+        expression.cpp:1233-1385 there).  ``rotary_dim=0`` turns the whole head dimension.  ``position_ids`` (one absolute position
+        per element of the sequence axis) and ``effective_sequence_length`` (one element) are the C++ API's WithPositionIds /
+        WithEffectiveSequenceLength forms."""
+        if attention_factor is not None and attention_factor <= 0:
+            raise RuntimeError("RoPE attention_factor must be positive.")
+        if len(long_rope_short_factors) != len(long_rope_long_factors):
+            raise RuntimeError("LongRoPE scaling requires short/long factor lists of length rotary_dim / 2.")
+        count = len(long_rope_short_factors)
+        short = (ctypes.c_double * max(count, 1))(*[float(v) for v in long_rope_short_factors])
+        long_ = (ctypes.c_double * max(count, 1))(*[float(v) for v in long_rope_long_factors])
+        options = _RopeOptions(int(sequence_axis), int(head_dim_axis), int(rotary_dim), float(base), int(position_offset), int(bool(interleaved)),
+                               int(bool(inverse)), int(RotaryScalingKind.none if scaling_kind is None else scaling_kind), float(scaling_factor),
+                               int(original_max_position_embeddings), float(attention_factor) if attention_factor is not None else 0.0,
+                               float(yarn_beta_fast), float(yarn_beta_slow), float(llama3_low_freq_factor), float(llama3_high_freq_factor),
+                               ctypes.cast(short, ctypes.POINTER(ctypes.c_double)), ctypes.cast(long_, ctypes.POINTER(ctypes.c_double)), count,
+                               -1 if output_dtype is None else int(output_dtype), -1 if compute_dtype is None else int(compute_dtype))
+        ids = position_ids._h if position_ids is not None else None
+        length = effective_sequence_length._h if effective_sequence_length is not None else None
+        return Expression(_handle(lib().thor_expr_rope(self._h, ids, length, ctypes.byref(options)), "rope"))
+
+    rotary_position_embedding = rope
 
     def transpose(self) -> "Expression":
         """The last two axes exchanged, as a view of the operand's storage."""
