@@ -333,6 +333,24 @@ def bench_other_configs():
     ragged_sum = ex.compile(ex.input("v").segmented_scan(ex.input("o"), ScanOp.sum), 0)
     plan = ragged_sum.stamp({"v": scalars, "o": ragged_offsets}, stream)
     timed("scan_ragged_cumsum_fp32_2^26", plan.run, 8 * rows * 16, rows * 16, plan.stage_descriptions()[0])
+    del plan, scalars
+
+    # ---- rotary position embedding (Expression.rope): every element read once and written once
+    from thor_amd.dtypes import size_of
+    from thor_amd.physical import RotaryScalingKind
+    plane = rng.standard_normal((4096, 128), dtype=np.float32)
+    for label, dtype, shape, options in (
+            ("rope_bf16_bhsd_8x32x4096x128", DataType.bf16, (8, 32, 4096, 128), {}),
+            ("rope_bf16_bshd_llama3_8x4096x32x128", DataType.bf16, (8, 4096, 32, 128),
+             {"sequence_axis": 1, "head_dim_axis": 3, "scaling_kind": RotaryScalingKind.llama3, "scaling_factor": 8.0, "original_max_position_embeddings": 8192,
+              "base": 500000.0}),
+            ("rope_fp32_bhsd_interleaved_4x32x4096x128", DataType.fp32, (4, 32, 4096, 128), {"interleaved": True})):
+        q = gpu_from(np.resize(plane, shape), dtype)
+        count = int(np.prod(shape))
+        rope = ex.compile(ex.input("q").rope(**options), 0)
+        plans = [rope.stamp({"q": t}, stream) for t in (q, clone(q))]
+        timed(label, [p_.run for p_ in plans], 2 * size_of(dtype) * count, count, plans[0].stage_descriptions()[0])
+        del plans, q
     return results
 
 

@@ -207,6 +207,25 @@ def test_backward_is_the_rotation_turned_back(stream, case):
     assert abs(float((y * g32).sum()) - float((x32.astype(np.float64) * got).sum())) < 1e-3
 
 
+def test_walking_and_tiled_kernels_agree(stream, monkeypatch):
+    """Layouts with heads between the sequence and the head dimension run the LDS-tiled kernel; switched off, the walking kernel
+    takes them: the two work the same angles out and must agree to the last bit.  Different block counts change nothing either."""
+    rng = np.random.default_rng(38)
+    x = to_storage(rng.standard_normal((3, 130, 5, 64)).astype(np.float32), DataType.bf16)
+    t = copy_numpy_to_gpu(x, stream, DataType.bf16)
+    options = {"sequence_axis": 1, "head_dim_axis": 3, "rotary_dim": 48, "position_offset": 7}
+    results = []
+    for env in ({}, {"THOR_ROPE_NO_TILES": "1"}, {"THOR_ROPE_NO_TILES": "1", "THOR_ROPE_BLOCKS": "1"}):
+        for name in ("THOR_ROPE_NO_TILES", "THOR_ROPE_BLOCKS"):
+            monkeypatch.delenv(name, raising=False)
+        for name, value in env.items():
+            monkeypatch.setenv(name, value)
+        plan = run({"y": ex.input("x").rope(**options)}, {"x": t}, stream)
+        results.append((plan.stage_descriptions()[-1], copy_gpu_to_numpy(plan.output("y"), stream)))
+    assert "tile=" in results[0][0] and "walk=" in results[1][0] and "walk=15/1," in results[2][0]
+    assert np.array_equal(results[0][1], results[1][1]) and np.array_equal(results[1][1], results[2][1])
+
+
 def test_rotation_inside_a_larger_graph(stream):
     rng = np.random.default_rng(35)
     x32 = rng.standard_normal((2, 3, 40, 32)).astype(np.float32)

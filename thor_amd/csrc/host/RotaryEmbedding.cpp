@@ -15,6 +15,7 @@
 #include "thorhip_numeric_embed.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <sstream>
 #include <stdexcept>
 
@@ -158,15 +159,31 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     const uint64_t items = seq * slots;
     const uint32_t threads = 256;
     const uint64_t blocksPerChunk = (items + threads - 1) / threads;
-    // enough blocks to fill the chip, each walking as long a stretch as that leaves
-    uint64_t chunks = std::min<uint64_t>(walk, std::max<uint64_t>(1, (4096 + blocksPerChunk - 1) / blocksPerChunk));
+    // Many blocks, each thread walking at least two coordinates with its angles (measured on [8, 32, 4096, 128] bf16: 88 us
+    // with walks of 2 in 16384 blocks, 97 us with walks of 8, 136 us with walks of 1, where the sines are not shared at all).
+    uint64_t wantedBlocks = 32768;
+    if (const char* text = std::getenv("THOR_ROPE_BLOCKS")) {
+        const long long asked = std::atoll(text);
+        if (asked >= 1 && asked <= (1 << 24)) wantedBlocks = static_cast<uint64_t>(asked);
+    }
+    uint64_t chunks = std::min<uint64_t>(std::max<uint64_t>(1, walk / 2), std::max<uint64_t>(1, (wantedBlocks + blocksPerChunk - 1) / blocksPerChunk));
     const uint64_t walkPerChunk = (walk + chunks - 1) / chunks;
     chunks = (walk + walkPerChunk - 1) / walkPerChunk;
-    const uint64_t blocks = blocksPerChunk * chunks;
+    // Heads between the sequence axis and a last-axis head dimension ([.., S, heads.., D]): everything at one position is one
+    // contiguous run, so a block takes a few consecutive positions, leaves their sines and cosines in LDS (one per thread) and
+    // streams the run, every head reading the same table.
+    const bool tiled = middleCount > 1 && innerCount == 1 && dimStride == 1 && seqAxis < dimAxis && std::getenv("THOR_ROPE_NO_TILES") == nullptr;
+    uint64_t tilePositions = std::max<uint64_t>(1, threads / half);
+    while (tilePositions * middleCount * slots < 2 * threads && tilePositions * 2 * half <= 4096) tilePositions *= 2;
+    tilePositions = std::min(tilePositions, seq);
+    const uint64_t tiles = (seq + tilePositions - 1) / tilePositions;
+    const uint64_t blocks = tiled ? outerCount * tiles : blocksPerChunk * chunks;
     if (blocks > 0x7fffffffull) throw std::runtime_error("RoPE: the tensor is too large for one launch.");
 
     const std::string inType = deviceTypeName(values.getDataType()), outType = deviceTypeName(output.getDataType());
     const bool needsLength = n.rope_scaling_kind == RotaryScalingKind::DynamicNTK || n.rope_scaling_kind == RotaryScalingKind::LongRope;
+    // a block shares the table of frequencies when that saves work: more than one thread of the block per pair
+    const bool sharedFrequencies = half <= 8192 && items >= 2 * half;
 
     std::ostringstream s;
     s << thor_embed::kDevicePrelude;
@@ -174,11 +191,89 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "__device__ const float thor_rope_short_factors[" << half << "] = " << floatArray(n.rope_long_rope_short_factors) << ";\n";
         s << "__device__ const float thor_rope_long_factors[" << half << "] = " << floatArray(n.rope_long_rope_long_factors) << ";\n";
     }
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_rope(const " << inType << "* x";
-    if (positionIds.has_value()) s << ", const " << deviceTypeName(positionIds->getDataType()) << "* ids";
-    if (effectiveLength.has_value()) s << ", const " << deviceTypeName(effectiveLength->getDataType()) << "* length";
-    s << ", " << outType << "* out) {\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_rope(const " << inType << "* __restrict__ x";
+    if (positionIds.has_value()) s << ", const " << deviceTypeName(positionIds->getDataType()) << "* __restrict__ ids";
+    if (effectiveLength.has_value()) s << ", const " << deviceTypeName(effectiveLength->getDataType()) << "* __restrict__ length";
+    s << ", " << outType << "* __restrict__ out) {\n";
     s << "    constexpr int V = " << vec << ", P = " << pairsPerThread << ";\n";
+    if (needsLength) {
+        const std::string extent = effectiveLength.has_value() ? std::string("thor::toFloat(length[0])") : floatLiteral(static_cast<double>(seq));
+        s << "    const float seqLen = fmaxf(" << extent << " + " << floatLiteral(static_cast<double>(std::max<int64_t>(0, n.rope_position_offset)))
+          << ", 1.0f);\n";
+    }
+    const std::string attention = floatLiteral(n.rope_attention_factor);
+    // the two elements of a pair lie `apart` coordinates from each other along the head dimension
+    const uint64_t apart = n.rope_interleaved ? 1 : half;
+    if (tiled) {
+        const uint64_t table = tilePositions * half;
+        s << "    __shared__ float sines[" << table << "], cosines[" << table << "];\n";
+        s << "    const thor::u64 outer = blockIdx.x / " << tiles << "u, firstPosition = (thor::u64)(blockIdx.x % " << tiles << "u) * " << tilePositions << "ull;\n";
+        s << "    for (thor::u32 t = threadIdx.x; t < " << table << "u; t += " << threads << "u) {\n";
+        s << "        const thor::u32 pair = t % " << half << "u;\n";
+        s << "        const thor::u64 position = firstPosition + t / " << half << "u;\n";
+        s << "        float sn = 0.0f, cs = 0.0f;\n";
+        s << "        if (position < " << seq << "ull) {\n";
+        if (positionIds.has_value()) {
+            s << "            float angleBase = thor::toFloat(ids[position]);\n";
+        } else {
+            s << "            float angleBase = (float)position + " << floatLiteral(static_cast<double>(n.rope_position_offset)) << ";\n";
+        }
+        if (n.rope_scaling_kind == RotaryScalingKind::Linear) s << "            angleBase = angleBase / " << floatLiteral(n.rope_scaling_factor) << ";\n";
+        s << "            float freq = 0.0f;\n";
+        s << "            {\n" << frequencyStatements(n, rotary, "(float)pair", "                ") << "            }\n";
+        s << "            const float theta = angleBase * freq;\n";
+        s << "            sn = sinf(theta);\n            cs = cosf(theta);\n";
+        if (n.rope_attention_factor != 1.0) s << "            sn *= " << attention << ";\n            cs *= " << attention << ";\n";
+        if (n.rope_inverse) s << "            sn = -sn;\n";
+        s << "        }\n        sines[t] = sn;\n        cosines[t] = cs;\n    }\n";
+        s << "    __syncthreads();\n";
+        s << "    const thor::u64 base = outer * " << outerStride << "ull + firstPosition * " << seqStride << "ull;\n";
+        s << "    const thor::u64 left = " << seq << "ull - firstPosition;\n";
+        s << "    const thor::u32 liveItems = (thor::u32)(left < " << tilePositions << "ull ? left : " << tilePositions << "ull) * " << middleCount * slots << "u;\n";
+        s << "    for (thor::u32 item = threadIdx.x; item < liveItems; item += " << threads << "u) {\n";
+        s << "        const thor::u32 row = item / " << slots << "u, slot = item % " << slots << "u;\n";
+        s << "        const thor::u64 rowBase = base + (thor::u64)row * " << headDim << "ull;\n";
+        if (tail != 0) {
+            s << "        if (slot >= " << pairSlots << "u) {\n";
+            s << "            const thor::u64 e = rowBase + " << rotary << "ull + (slot - " << pairSlots << "u) * V;\n";
+            s << "            thor::Pack<" << inType << ", V> p;\n            p.loadStream(x + e);\n";
+            s << "            thor::Pack<" << outType << ", V> q;\n";
+            s << "#pragma unroll\n            for (int k = 0; k < V; ++k) q.v[k] = thor::fromFloat<" << outType << ">(thor::toFloat(p.v[k]));\n";
+            s << "            q.storeStream(out + e);\n            continue;\n        }\n";
+        }
+        s << "        const thor::u32 firstPair = slot * P;\n";
+        s << "        const float* sn = sines + (row / " << middleCount << "u) * " << half << "u + firstPair;\n";
+        s << "        const float* cs = cosines + (row / " << middleCount << "u) * " << half << "u + firstPair;\n";
+        if (pairsInsideVector) {
+            s << "        const thor::u64 e = rowBase + firstPair * 2;\n";
+            s << "        thor::Pack<" << inType << ", V> p;\n        p.loadStream(x + e);\n";
+            s << "        thor::Pack<" << outType << ", V> q;\n";
+            s << "#pragma unroll\n        for (int k = 0; k < P; ++k) {\n";
+            s << "            const float a = thor::toFloat(p.v[2 * k]), b = thor::toFloat(p.v[2 * k + 1]);\n";
+            s << "            q.v[2 * k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
+            s << "            q.v[2 * k + 1] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
+            s << "        }\n        q.storeStream(out + e);\n";
+        } else {
+            s << "        const thor::u64 ea = rowBase + " << (n.rope_interleaved ? "firstPair * 2" : "firstPair") << ", eb = ea + " << apart << "ull;\n";
+            s << "        thor::Pack<" << inType << ", V> pa, pb;\n        pa.loadStream(x + ea);\n        pb.loadStream(x + eb);\n";
+            s << "        thor::Pack<" << outType << ", V> qa, qb;\n";
+            s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
+            s << "            const float a = thor::toFloat(pa.v[k]), b = thor::toFloat(pb.v[k]);\n";
+            s << "            qa.v[k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
+            s << "            qb.v[k] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
+            s << "        }\n        qa.storeStream(out + ea);\n        qb.storeStream(out + eb);\n";
+        }
+        s << "    }\n}\n";
+    } else {
+    if (sharedFrequencies) {
+        // one frequency per pair, worked out once per block
+        s << "    __shared__ float frequencies[" << half << "];\n";
+        s << "    for (thor::u32 pair = threadIdx.x; pair < " << half << "u; pair += " << threads << "u) {\n";
+        s << "        float freq = 0.0f;\n";
+        s << "        {\n" << frequencyStatements(n, rotary, "(float)pair", "            ") << "        }\n";
+        s << "        frequencies[pair] = freq;\n    }\n";
+        s << "    __syncthreads();\n";
+    }
     s << "    const thor::u64 chunk = blockIdx.x / " << blocksPerChunk << "u;\n";
     s << "    const thor::u64 item = (thor::u64)(blockIdx.x % " << blocksPerChunk << "u) * " << threads << " + threadIdx.x;\n";
     s << "    if (item >= " << items << "ull) return;\n";
@@ -208,16 +303,15 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "    float angleBase = (float)position + " << floatLiteral(static_cast<double>(n.rope_position_offset)) << ";\n";
     }
     if (n.rope_scaling_kind == RotaryScalingKind::Linear) s << "    angleBase = angleBase / " << floatLiteral(n.rope_scaling_factor) << ";\n";
-    if (needsLength) {
-        const std::string extent = effectiveLength.has_value() ? std::string("thor::toFloat(length[0])") : floatLiteral(static_cast<double>(seq));
-        s << "    const float seqLen = fmaxf(" << extent << " + " << floatLiteral(static_cast<double>(std::max<int64_t>(0, n.rope_position_offset)))
-          << ", 1.0f);\n";
-    }
     s << "    float sn[P], cs[P];\n";
     s << "#pragma unroll\n    for (int k = 0; k < P; ++k) {\n";
     s << "        const thor::u64 pair = firstPair + k;\n";
-    s << "        float freq = 0.0f;\n";
-    s << "        {\n" << frequencyStatements(n, rotary, "(float)pair", "            ") << "        }\n";
+    if (sharedFrequencies) {
+        s << "        const float freq = frequencies[pair];\n";
+    } else {
+        s << "        float freq = 0.0f;\n";
+        s << "        {\n" << frequencyStatements(n, rotary, "(float)pair", "            ") << "        }\n";
+    }
     s << "        const float theta = angleBase * freq;\n";
     s << "        sn[k] = sinf(theta);\n        cs[k] = cosf(theta);\n";
     if (n.rope_attention_factor != 1.0) {
@@ -225,6 +319,7 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     }
     if (n.rope_inverse) s << "        sn[k] = -sn[k];\n";
     s << "    }\n";
+    s << "#pragma unroll 1\n";
     s << "    for (thor::u64 w = walkFirst; w < walkLast; ++w) {\n";
     if (pairsInsideVector) {
         s << "        const thor::u64 e = at(w, firstPair * 2);\n";
@@ -236,8 +331,6 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "            q.v[2 * k + 1] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
         s << "        }\n        q.storeStream(out + e);\n";
     } else {
-        // the two elements of a pair lie `apart` coordinates from each other along the head dimension
-        const uint64_t apart = n.rope_interleaved ? 1 : half;
         const std::string firstCoordinate = n.rope_interleaved ? "firstPair * 2" : "firstPair";
         s << "        const thor::u64 ea = at(w, " << firstCoordinate << "), eb = at(w, " << firstCoordinate << " + " << apart << "ull);\n";
         s << "        thor::Pack<" << inType << ", V> pa, pb;\n        pa.loadStream(x + ea);\n        pb.loadStream(x + eb);\n";
@@ -249,12 +342,18 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "        }\n        qa.storeStream(out + ea);\n        qb.storeStream(out + eb);\n";
     }
     s << "    }\n}\n";
+    }
 
     const std::shared_ptr<CompiledKernel> kernel = compileKernel(s.str(), "thor_rope", deviceNum, /*fastContract=*/false);
     std::ostringstream description;
     description << "rope(seq=" << seq << ",head_dim=" << headDim << ",rotary=" << rotary << (n.rope_interleaved ? ",interleaved" : "")
-                << (n.rope_inverse ? ",inverse" : "") << ",walk=" << walk << "/" << chunks << ",vec=" << vec << ",grid=" << blocks << ") [" << kernel->kernelName
-                << "]";
+                << (n.rope_inverse ? ",inverse" : "");
+    if (tiled) {
+        description << ",tile=" << tilePositions << "x" << middleCount;
+    } else {
+        description << ",walk=" << walk << "/" << chunks;
+    }
+    description << ",vec=" << vec << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
     std::vector<Tensor> inputs = {values};
     if (positionIds.has_value()) inputs.push_back(*positionIds);
     if (effectiveLength.has_value()) inputs.push_back(*effectiveLength);
