@@ -324,6 +324,54 @@ static void scanExpressionStructure() {
     }));
 }
 
+static void ropeExpressionStructure() {
+    // ROPE nodes carry every option; explicit positions and the effective length ride as operands that precede the rotation and
+    // are cast to fp32 (Expression.cpp:4334-4507, ExpressionConvenienceOpsTest.cpp:3670-3700 there)
+    RotaryPositionEmbeddingOptions options;
+    options.sequence_axis = 1;
+    options.head_dim_axis = 2;
+    options.rotary_dim = 4;
+    options.scaling_kind = RotaryScalingKind::Yarn;
+    options.scaling_factor = 4.0;
+    options.original_max_position_embeddings = 16;
+    const Expression x = Expression::input("x");
+    PhysicalOutputs outputs =
+        Expression::outputs({{"y", x.rotaryPositionEmbeddingWithPositionIds(Expression::input("positions"), options)}}).physicalOutputs();
+    const ExprNode& node = outputs.expr->nodes.at(outputs.outputs[0].node_idx);
+    CHECK(node.op == ExprOp::ROPE && node.rhs != UINT32_MAX && node.aux == UINT32_MAX && node.rhs < outputs.outputs[0].node_idx);
+    CHECK(outputs.expr->nodes.at(node.rhs).op == ExprOp::CAST && outputs.expr->nodes.at(node.rhs).output_dtype == DataType::FP32);
+    CHECK(node.rope_sequence_axis == 1 && node.rope_head_dim_axis == 2 && node.rope_rotary_dim == 4 && node.rope_scaling_kind == RotaryScalingKind::Yarn);
+    CHECK(std::fabs(node.rope_attention_factor - (0.1 * std::log(4.0) + 1.0)) < 1e-15);  // YaRN's own magnitude correction
+    resolveOutputsDTypesInPlace(outputs, {DataType::UINT32, DataType::BF16});  // slots in order of appearance: positions come first
+    CHECK(outputs.expr->nodes.at(outputs.outputs[0].node_idx).output_dtype == DataType::BF16);
+    options.position_offset = 1;
+    CHECK(throwsAs<std::runtime_error>([&] { (void)x.rotaryPositionEmbeddingWithPositionIds(Expression::input("positions"), options); }));
+    options.position_offset = 0;
+    options.rotary_dim = 3;
+    CHECK(throwsAs<std::runtime_error>([&] { (void)x.rope(options); }));
+    options.rotary_dim = 4;
+    options.scaling_kind = RotaryScalingKind::LongRope;
+    CHECK(throwsAs<std::runtime_error>([&] { (void)x.rope(options); }));  // factor lists missing
+    options.long_rope_short_factors = {1.0, 1.0};
+    options.long_rope_long_factors = {2.0, 2.0};
+    const PhysicalExpression both =
+        x.rotaryPositionEmbeddingWithPositionIdsAndEffectiveSequenceLength(Expression::input("positions"), Expression::input("lengths"), options).expression();
+    CHECK(both.nodes.back().op == ExprOp::ROPE && both.nodes.back().rhs != UINT32_MAX && both.nodes.back().aux != UINT32_MAX);
+    CHECK(std::fabs(both.nodes.back().rope_attention_factor - std::sqrt(1.0 + std::log(4.0) / std::log(16.0))) < 1e-15);
+    // equal parameters, equal text; any parameter tells two rotations apart
+    RotaryPositionEmbeddingOptions a, b;
+    b.base = 500000.0;
+    CHECK(canonicalize(x.rope(a).expression()) == canonicalize(x.rope(a).expression()));
+    CHECK(canonicalize(x.rope(a).expression()) != canonicalize(x.rope(b).expression()));
+    // the gradient is the same rotation turned the other way, positions and all (AutoDiff.cpp:4672-4693 there)
+    options.inverse = false;
+    const PhysicalOutputs forward = Expression::outputs({{"y", x.rotaryPositionEmbeddingWithPositionIds(Expression::input("positions"), options)}}).physicalOutputs();
+    const PhysicalOutputs backward = buildBackwardOutputs(forward, {"x"}, std::string("__grad_output"), {{{"x", {2, 5, 8}}, {"positions", {5}}}});
+    int turnedBack = 0;
+    for (const ExprNode& n : backward.expr->nodes) turnedBack += n.op == ExprOp::ROPE && n.rope_inverse && n.rhs != UINT32_MAX && n.rope_rotary_dim == 4;
+    CHECK(turnedBack == 1);
+}
+
 static void raggedExpressionStructure() {
     // RaggedExpressionTest.cpp:739-795,907-957,2037-2055 there: names, descriptors and markers, no device work
     const RaggedTensorDescriptor descriptor(DataType::FP32, {4}, 3, 9);
@@ -566,6 +614,62 @@ static void autodiffExecution(Stream& stream) {
     CHECK(throwsAs<std::runtime_error>([&] { (void)implicit.compileBackward({"x"}); }));  // no second derivative of a backward equation
 }
 
+static void ropeExecution(Stream& stream) {
+    // the equivalences ExpressionConvenienceOpsTest.cpp:3503-3668 there asserts, and the closed form of the first pair
+    std::vector<float> values(1 * 2 * 8 * 8);
+    for (size_t i = 0; i < values.size(); ++i) values[i] = 0.25f * static_cast<float>(static_cast<int>(i % 17) - 8);
+    const Tensor x = gpuFrom(values, {1, 2, 8, 8}, stream);
+    auto run = [&](const Expression& e, std::unordered_map<std::string, Tensor> inputs) {
+        FusedEquation eq = FusedEquation::compile(Expression::outputs({{"y", e}}).physicalOutputs(), 0);
+        StampedExecutionPlan plan = eq.stamp(inputs, stream);
+        plan.run();
+        return toHostF32(plan.output("y"), stream);
+    };
+    const Expression ix = Expression::input("x");
+    RotaryPositionEmbeddingOptions plainOptions;
+    plainOptions.rotary_dim = 4;
+    const std::vector<float> plain = run(ix.rope(plainOptions), {{"x", x}});
+    // pair 0 turns by the position itself: (a, b) -> (a cos p - b sin p, a sin p + b cos p); the tail is untouched
+    for (int p = 0; p < 8; ++p) {
+        const float a = values[p * 8 + 0], b = values[p * 8 + 2];
+        CHECK(std::fabs(plain[p * 8 + 0] - (a * std::cos((float)p) - b * std::sin((float)p))) < 1e-5f);
+        CHECK(std::fabs(plain[p * 8 + 2] - (a * std::sin((float)p) + b * std::cos((float)p))) < 1e-5f);
+        for (int d = 4; d < 8; ++d) CHECK(plain[p * 8 + d] == values[p * 8 + d]);
+    }
+    Tensor lengthHost(cpuPlacement, TensorDescriptor(DataType::UINT32, {1}));
+    lengthHost.getMemPtr<uint32_t>()[0] = 3;
+    Tensor length(gpuPlacement, TensorDescriptor(DataType::UINT32, {1}));
+    length.copyFromAsync(lengthHost, stream);
+    stream.synchronize();
+    RotaryPositionEmbeddingOptions ntk = plainOptions;
+    ntk.scaling_kind = RotaryScalingKind::DynamicNTK;
+    ntk.scaling_factor = 2.0;
+    ntk.original_max_position_embeddings = 4;
+    // a short effective length leaves Dynamic NTK unscaled; the physical extent (8 > 4) does not
+    CHECK(run(ix.rotaryPositionEmbeddingWithEffectiveSequenceLength(Expression::input("length"), ntk), {{"x", x}, {"length", length}}) == plain);
+    CHECK(run(ix.rope(ntk), {{"x", x}}) != plain);
+    RotaryPositionEmbeddingOptions longRope = plainOptions;
+    longRope.scaling_kind = RotaryScalingKind::LongRope;
+    longRope.original_max_position_embeddings = 4;
+    longRope.long_rope_short_factors = {1.0, 1.0};
+    longRope.long_rope_long_factors = {2.0, 2.0};
+    CHECK(run(ix.rotaryPositionEmbeddingWithEffectiveSequenceLength(Expression::input("length"), longRope), {{"x", x}, {"length", length}}) == plain);
+    CHECK(run(ix.rope(longRope), {{"x", x}}) != plain);
+    // explicit absolute positions equal the offset they spell out; turning back returns the input
+    Tensor idsHost(cpuPlacement, TensorDescriptor(DataType::UINT32, {8}));
+    for (uint32_t p = 0; p < 8; ++p) idsHost.getMemPtr<uint32_t>()[p] = p + 5;
+    Tensor ids(gpuPlacement, TensorDescriptor(DataType::UINT32, {8}));
+    ids.copyFromAsync(idsHost, stream);
+    stream.synchronize();
+    RotaryPositionEmbeddingOptions shifted = plainOptions;
+    shifted.position_offset = 5;
+    CHECK(run(ix.rotaryPositionEmbeddingWithPositionIds(Expression::input("positions"), plainOptions), {{"x", x}, {"positions", ids}}) == run(ix.rope(shifted), {{"x", x}}));
+    RotaryPositionEmbeddingOptions back = shifted;
+    back.inverse = true;
+    const std::vector<float> round = run(ix.rope(shifted).rope(back), {{"x", x}});
+    for (size_t i = 0; i < values.size(); ++i) CHECK(std::fabs(round[i] - values[i]) < 2e-6f);
+}
+
 static void devicePrefixScans(Stream& stream) {
     // cubDeviceScan / cubDeviceSegmentedUniformScan / cubDeviceSegmentedScan and arg forms: plan, temporary storage, run
     // (CubDevicePrimitivesTest.cpp there; literal vectors of test_expression_scan.py / test_expression_segmented_scan.py)
@@ -704,7 +808,8 @@ int main(int argc, char** argv) {
                                {"cpuTypeConverter", cpuTypeConverter},
                                {"raggedExpressionStructure", raggedExpressionStructure},
                                {"autodiffGraphStructure", autodiffGraphStructure},
-                               {"scanExpressionStructure", scanExpressionStructure}};
+                               {"scanExpressionStructure", scanExpressionStructure},
+                               {"ropeExpressionStructure", ropeExpressionStructure}};
     if (mode == "gpu") {
         auto withStream = [](void (*f)(Stream&)) {
             return [f] {
@@ -720,6 +825,7 @@ int main(int argc, char** argv) {
         cases.push_back({"softmaxPlansAndRowKernel", withStream(softmaxPlansAndRowKernel)});
         cases.push_back({"autodiffExecution", withStream(autodiffExecution)});
         cases.push_back({"devicePrefixScans", withStream(devicePrefixScans)});
+        cases.push_back({"ropeExecution", withStream(ropeExecution)});
         cases.push_back({"typeConverterOnGpuAndTensorViews", withStream(typeConverterOnGpuAndTensorViews)});
     }
     for (const Case& c : cases) {
