@@ -125,6 +125,13 @@ inline bool isStorageViewOp(ExprOp op) { return op == ExprOp::STRIDED_VIEW || op
 // SCAN: lhs scanned along its last axis.  SEGMENTED_SCAN: lhs = values [N], rhs = row-partition offsets [B + 1]; every segment
 // is scanned on its own.
 inline bool isScanOp(ExprOp op) { return op == ExprOp::SCAN || op == ExprOp::SEGMENTED_SCAN; }
+// Gradient of a min / max scan (AutoDiff.cpp:5743-5760 there): lhs = the scanned operand, rhs = the FP32 gradient of the scan's
+// output, aux = the offsets of a segmented scan.  Every position's gradient goes to the element that held the running
+// minimum / maximum there (the first among equals); the result is FP32, shaped like the operand.
+inline bool isScanBackwardOp(ExprOp op) {
+    return op == ExprOp::SCAN_MIN_BACKWARD || op == ExprOp::SCAN_MAX_BACKWARD || op == ExprOp::SEGMENTED_SCAN_MIN_BACKWARD ||
+           op == ExprOp::SEGMENTED_SCAN_MAX_BACKWARD;
+}
 inline bool isRaggedOp(ExprOp op) {
     return isSegmentedReduceOp(op) || op == ExprOp::SEGMENTED_BROADCAST || op == ExprOp::RAGGED_VALUEWISE_EXTENT;
 }

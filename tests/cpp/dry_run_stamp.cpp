@@ -169,6 +169,12 @@ static int runAll() {
         // gathers along an axis, with indices the same equation computes
         stampOne(std::string("gather ") + dtypeName + " value at the row argmax", (x * y).takeAlongAxis(x.argmax({1}, {}), 1), inputs, stream);
         stampOne(std::string("gather ") + dtypeName + " column picks", x.takeAlongAxis(y.argmin({0}, {}), 0) + 1.0, inputs, stream);
+        // min / max scans backward: arg scan, cleared FP32 tensor, scatter-add
+        if (dtype != DataType::FP8_E4M3) {
+            Tensor upstream(gpuPlacement, TensorDescriptor(dtype, {4096, 24}));
+            stampBackward(std::string("backward ") + dtypeName + " running max", x.scan(ScanOp::Max) * y, inputs, upstream, stream);
+            stampBackward(std::string("backward ") + dtypeName + " exclusive reverse running min", x.reverseScan(ScanOp::Min, -1, false), inputs, upstream, stream);
+        }
         // rotary position embedding: vector and scalar layouts, every scaling rule, explicit positions, backward
         {
             Tensor q(gpuPlacement, TensorDescriptor(dtype, {2, 4, 48, 64})), odd(gpuPlacement, TensorDescriptor(dtype, {3, 30, 7, 5}));

@@ -319,8 +319,25 @@ static void scanExpressionStructure() {
     bool reversed = false;
     for (const ExprNode& n : backward.expr->nodes) reversed = reversed || (n.op == ExprOp::SCAN && n.scan_reverse && n.scan_mode == ScanMode::Exclusive);
     CHECK(reversed);
+    // min / max scans route every position's gradient to the running winner: an FP32 SCAN_MAX_BACKWARD node over the operand and
+    // the FP32 gradient (AutoDiff.cpp:5743-5760 there); product scans have no rule
+    const PhysicalOutputs maxBackward =
+        buildBackwardOutputs(Expression::outputs({{"y", x.scan(ScanOp::Max, -1, false)}}).physicalOutputs(), {"x"}, std::nullopt, {{{"x", {3, 5}}}});
+    int routed = 0;
+    for (const ExprNode& n : maxBackward.expr->nodes) {
+        if (n.op != ExprOp::SCAN_MAX_BACKWARD) continue;
+        ++routed;
+        CHECK(n.scan_mode == ScanMode::Exclusive && !n.scan_reverse && n.aux == UINT32_MAX && n.output_dtype == DataType::FP32);
+        CHECK(maxBackward.expr->nodes.at(n.lhs).op == ExprOp::INPUT && maxBackward.expr->nodes.at(n.rhs).output_dtype == DataType::FP32);
+    }
+    CHECK(routed == 1);
+    const PhysicalOutputs raggedMin = buildBackwardOutputs(Expression::outputs({{"y", x.segmentedScan(offsets, ScanOp::Min)}}).physicalOutputs(), {"x"},
+                                                           std::string("__grad_output"), {{{"x", {9}}, {"offsets", {4}}}});
+    bool segmentedRouting = false;
+    for (const ExprNode& n : raggedMin.expr->nodes) segmentedRouting = segmentedRouting || (n.op == ExprOp::SEGMENTED_SCAN_MIN_BACKWARD && n.aux != UINT32_MAX);
+    CHECK(segmentedRouting);
     CHECK(throwsAs<std::runtime_error>([&] {
-        (void)buildBackwardOutputs(Expression::outputs({{"y", x.scan(ScanOp::Max)}}).physicalOutputs(), {"x"}, std::nullopt, {{{"x", {3, 5}}}});
+        (void)buildBackwardOutputs(Expression::outputs({{"y", x.scan(ScanOp::Product)}}).physicalOutputs(), {"x"}, std::nullopt, {{{"x", {3, 5}}}});
     }));
 }
 

@@ -164,8 +164,8 @@ def test_validation(stream):
                                                                 "o": copy_numpy_to_gpu(np.zeros(3, np.float32), stream, DataType.fp32)}, stream)
     with pytest.raises(ValueError, match="supports only ScanOp.min and ScanOp.max"):
         ix.scan_with_indices(ScanOp.sum)
-    with pytest.raises(RuntimeError, match="Only sum scans are differentiable"):
-        ex.compile(ix.scan(ScanOp.max), device_num=0).compile_backward(["x"]).stamp({"x": x}, stream)
+    with pytest.raises(RuntimeError, match="supports backward only for sum/min/max scan"):
+        ex.compile(ix.scan(ScanOp.product), device_num=0).compile_backward(["x"]).stamp({"x": x}, stream)
     stamp_run(ix.scan(ScanOp.sum, axis=1), {"x": x}, stream)  # the index of the last axis is accepted
 
 
@@ -182,3 +182,92 @@ def test_segmented_scan_with_indices_is_one_stage(stream, name, inclusive):
     np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("values"), stream), oracle.scan(values, ORACLE_OP[ScanOp[name]], inclusive, offsets=offsets, dtype=oracle.UINT32))
     np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("indices"), stream),
                                   oracle.scan(values, ORACLE_OP[ScanOp["arg_" + name]], inclusive, offsets=offsets, dtype=oracle.UINT32))
+
+
+# ---- min / max scans backward: every position's gradient goes to the element that held the running extreme there -----------------
+MINMAX_BACKWARD_EXPECTED = {  # worked out by hand for the vectors of test_segmented_minmax_scan_backward_uses_arg_scan_and_flat_scatter_add there
+    ("min", True): [0.5, -0.75, 0.0, 2.0, 0.75, 0.0, 1.5], ("max", True): [-0.25, 0.0, 0.0, 4.25, 0.0, 0.0, 0.0],
+    ("min", False): [-1.0, 0.25, 0.0, 1.25, 1.0, 0.0, 0.0], ("max", False): [-0.75, 0.0, 0.0, 2.25, 0.0, 0.0, 0.0]}
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp16, DataType.bf16, DataType.fp32], ids=lambda d: d.name)
+@pytest.mark.parametrize("inclusive", [True, False])
+@pytest.mark.parametrize("name", ["min", "max"])
+def test_segmented_minmax_scan_backward_uses_arg_scan_and_scatter_add(stream, name, inclusive, dtype):
+    values = to_storage(np.array([3.0, 1.0, 1.0, 4.0, 2.0, 2.0, 0.0], np.float32), dtype)
+    grad = to_storage(np.array([0.5, -1.0, 0.25, 2.0, 1.25, -0.5, 1.5], np.float32), dtype)
+    offsets = np.array([0, 3, 3, 7], np.uint32)
+    fwd = ex.compile(ex.input("x").segmented_scan(ex.input("offsets"), op=ScanOp[name], inclusive=inclusive), device_num=0)
+    bwd = fwd.compile_backward(["x"], error_input_name="__grad_output")
+    assert bwd.output_names() == ["x_grad"]
+    plan = bwd.stamp({"x": copy_numpy_to_gpu(values, stream, dtype), "offsets": copy_numpy_to_gpu(offsets, stream, DataType.uint32),
+                      "__grad_output": copy_numpy_to_gpu(grad, stream, dtype)}, stream)
+    plan.run()
+    assert plan.stage_kind_names().count("Scan") == 1 and sum("scatter_add" in d for d in plan.stage_descriptions()) == 1
+    assert plan.output("x_grad").get_data_type() == dtype
+    got = from_storage(copy_gpu_to_numpy(plan.output("x_grad"), stream), dtype)
+    np.testing.assert_allclose(got, MINMAX_BACKWARD_EXPECTED[(name, inclusive)], rtol=1e-5, atol=1e-6)
+
+
+def winners_gradient(values, grad, op, inclusive, reverse=False, segment_size=0, offsets=None, dtype=oracle.FP32):
+    """Scatter of `grad` by the oracle's arg scan, in float64."""
+    winners = oracle.scan(values, op, inclusive, reverse, segment_size=segment_size, offsets=offsets, dtype=dtype).reshape(-1)
+    live = np.ones(winners.size, bool)
+    if offsets is not None:
+        live[:] = False
+        live[int(offsets[0]):int(offsets[-1])] = True
+    live &= winners != 0xFFFFFFFF
+    expected = np.zeros(winners.size, np.float64)
+    np.add.at(expected, winners[live].astype(np.int64), grad.reshape(-1).astype(np.float64)[live])
+    return expected.reshape(values.shape)
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16], ids=lambda d: d.name)
+@pytest.mark.parametrize("inclusive,reverse", [(True, False), (False, False), (True, True)])
+@pytest.mark.parametrize("name", ["min", "max"])
+@pytest.mark.parametrize("shape", [(64, 1000), (3, 20000), (1, 7)], ids=str)
+def test_row_minmax_scan_backward(stream, shape, name, inclusive, reverse, dtype):
+    rng = np.random.default_rng(61)
+    # few distinct values: long runs of one winner, and ties that the first occurrence must win
+    values = to_storage(rng.integers(-6, 7, shape).astype(np.float32) * 0.5, dtype)
+    grad = to_storage(rng.integers(-8, 9, shape).astype(np.float32) * 0.25, dtype)  # sums of these are exact in fp32
+    ix = ex.input("x")
+    scanned = ix.scan(ScanOp[name], inclusive=inclusive, reverse=reverse)
+    bwd = ex.compile(scanned, device_num=0).compile_backward(["x"], error_input_name="__grad_output")
+    plan = bwd.stamp({"x": copy_numpy_to_gpu(values, stream, dtype), "__grad_output": copy_numpy_to_gpu(grad, stream, dtype)}, stream)
+    plan.run()
+    expected = winners_gradient(values, from_storage(grad, dtype), ORACLE_OP[ScanOp["arg_" + name]], inclusive, reverse, segment_size=shape[-1], dtype=int(dtype))
+    got = from_storage(copy_gpu_to_numpy(plan.output("x_grad"), stream), dtype).astype(np.float64)
+    if dtype == DataType.fp32:
+        np.testing.assert_array_equal(got, expected)  # exact sums: the order of the additions cannot show
+    else:
+        np.testing.assert_allclose(got, from_storage(to_storage(expected.astype(np.float32), dtype), dtype), rtol=0, atol=0)
+
+
+def test_ragged_minmax_scan_backward_and_chain_rule(stream):
+    rng = np.random.default_rng(62)
+    n = 50_000
+    cuts = np.sort(rng.choice(np.arange(1, n - 500), 300, replace=False))
+    offsets = np.concatenate([[0], cuts, [n - 500]]).astype(np.uint64)  # the last 500 values belong to no segment
+    values = (rng.integers(-50, 51, n).astype(np.float32)) * 0.125
+    grad = rng.integers(-8, 9, n).astype(np.float32) * 0.25
+    v, o = ex.input("v"), ex.input("o")
+    fwd = ex.compile(v.segmented_scan(o, ScanOp.max, inclusive=True, reverse=True), device_num=0)
+    plan = fwd.compile_backward(["v"], error_input_name="__grad_output").stamp(
+        {"v": copy_numpy_to_gpu(values, stream, DataType.fp32), "o": copy_numpy_to_gpu(offsets, stream, DataType.uint64),
+         "__grad_output": copy_numpy_to_gpu(grad, stream, DataType.fp32)}, stream)
+    plan.run()
+    expected = winners_gradient(values, grad, oracle.SCAN_ARGMAX, True, True, offsets=offsets)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("v_grad"), stream), expected)
+    assert np.all(expected[n - 500:] == 0)
+    # through elementwise work on both sides: d/dx sum(w * cummax(x^2)) = 2 x * scatter(w)
+    x32 = rng.uniform(0.5, 2.0, (30, 257)).astype(np.float32)
+    w32 = rng.integers(-4, 5, (30, 257)).astype(np.float32)
+    x, w = ex.input("x"), ex.input("w")
+    loss = ((x * x).scan(ScanOp.max) * w).reduce_sum(axis=[0, 1])
+    plan = ex.compile(loss, device_num=0).compile_backward(["x"]).stamp({"x": copy_numpy_to_gpu(x32, stream, DataType.fp32), "w": copy_numpy_to_gpu(w32, stream, DataType.fp32)},
+                                                                        stream)
+    plan.run()
+    squares = x32 * x32
+    expected = 2.0 * x32.astype(np.float64) * winners_gradient(squares, w32, oracle.SCAN_ARGMAX, True, segment_size=257)
+    np.testing.assert_allclose(copy_gpu_to_numpy(plan.output("x_grad"), stream), expected, rtol=1e-6, atol=1e-6)

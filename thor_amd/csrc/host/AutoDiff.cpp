@@ -224,6 +224,25 @@ class BackwardGraph {
         n.ragged_runtime_elements_per_value = like.ragged_runtime_elements_per_value;
         return push(std::move(n), dims[values]);
     }
+    // the gradient of the min / max scan `like`: operand, FP32 upstream gradient, offsets of a segmented scan
+    uint32_t scanWinnerGradient(uint32_t operand, uint32_t gradient, uint32_t offsets, const ExprNode& like) {
+        ExprNode n;
+        const bool smallest = like.scan_op == ScanOp::Min;
+        n.op = like.op == ExprOp::SEGMENTED_SCAN ? (smallest ? ExprOp::SEGMENTED_SCAN_MIN_BACKWARD : ExprOp::SEGMENTED_SCAN_MAX_BACKWARD)
+                                                 : (smallest ? ExprOp::SCAN_MIN_BACKWARD : ExprOp::SCAN_MAX_BACKWARD);
+        n.lhs = operand;
+        n.rhs = gradient;
+        n.aux = offsets;
+        n.scan_op = like.scan_op;
+        n.scan_mode = like.scan_mode;
+        n.scan_axis = like.scan_axis;
+        n.scan_reverse = like.scan_reverse;
+        n.ragged_runtime_batch_size = like.ragged_runtime_batch_size;
+        n.ragged_runtime_max_active_values = like.ragged_runtime_max_active_values;
+        n.ragged_runtime_elements_per_value = like.ragged_runtime_elements_per_value;
+        n.output_dtype = DataType::FP32;
+        return push(std::move(n), dims[operand]);
+    }
     // the rotation `like` describes turned the other way, over `values` (same position ids and effective length)
     uint32_t oppositeRope(uint32_t values, uint32_t positionIds, uint32_t effectiveLength, const ExprNode& like) {
         ExprNode n = like;
@@ -545,8 +564,15 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
             case ExprOp::SEGMENTED_SCAN:
                 // element j feeds every later prefix (the later ones only, when exclusive): its gradient is the same scan of the
                 // upstream gradient run from the other end
-                if (n.scan_op != ScanOp::Sum) throw std::runtime_error(noRule(n.op) + " Only sum scans are differentiable here.");
-                contribute(n.lhs, b.oppositeScan(g, n.op == ExprOp::SEGMENTED_SCAN ? b.value(n.rhs) : kNone, n));
+                if (n.scan_op == ScanOp::Sum) {
+                    contribute(n.lhs, b.oppositeScan(g, n.op == ExprOp::SEGMENTED_SCAN ? b.value(n.rhs) : kNone, n));
+                } else if (n.scan_op == ScanOp::Min || n.scan_op == ScanOp::Max) {
+                    // every position hands its gradient to the element that held the running minimum / maximum there
+                    // (Utilities/Expression/AutoDiff.cpp:5743-5760 there)
+                    contribute(n.lhs, b.scanWinnerGradient(x(), b.cast(g, DataType::FP32), n.op == ExprOp::SEGMENTED_SCAN ? b.value(n.rhs) : kNone, n));
+                } else {
+                    throw std::runtime_error("Thor expressions autodiff currently supports backward only for sum/min/max scan.");
+                }
                 break;
 
             case ExprOp::ROPE:

@@ -10,6 +10,7 @@
 #include "HipSourceEmitter.h"
 #include "IndexGather.h"
 #include "RotaryEmbedding.h"
+#include "ScatterAdd.h"
 #include "ReductionPlanner.h"
 #include "RowFusion.h"
 #include "ShapeInference.h"
@@ -158,7 +159,7 @@ class GraphBuilder {
             node.lhs = asTensorOperand(node.lhs, false);
             if (isStorageViewOp(out.nodes[node.lhs].op)) node.lhs = castOf(node.lhs, out.nodes[node.lhs].output_dtype.value());
             if (node.op == ExprOp::SEGMENTED_SCAN) node.rhs = asTensorOperand(node.rhs, false);
-        } else if (node.op == ExprOp::ROPE) {
+        } else if (node.op == ExprOp::ROPE || isScanBackwardOp(node.op)) {
             // the rotation kernel addresses dense storage; position ids and the effective length are small tensors it reads
             for (uint32_t* operand : {&node.lhs, &node.rhs, &node.aux}) {
                 if (*operand == UINT32_MAX) continue;
@@ -237,7 +238,7 @@ uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
 bool consumesGather(const ExprNode& consumer) {
     if (consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT || consumer.op == ExprOp::WHERE || consumer.op == ExprOp::CAST) return true;
     if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX || isWinnerRoutingOp(consumer.op) ||
-        consumer.op == ExprOp::TAKE_ALONG_AXIS || consumer.op == ExprOp::ROPE || isScanOp(consumer.op)) {
+        consumer.op == ExprOp::TAKE_ALONG_AXIS || consumer.op == ExprOp::ROPE || isScanBackwardOp(consumer.op) || isScanOp(consumer.op)) {
         return false;
     }
     return Expression::isBinaryOp(consumer.op) || Expression::isUnaryOp(consumer.op);
@@ -373,6 +374,19 @@ std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpressio
                 }
                 if (n.ragged_runtime_batch_size != 0 && dims[n.rhs][0] != n.ragged_runtime_batch_size + 1) {
                     throw std::runtime_error("Segmented scan offsets do not have the ragged descriptor's batch size + 1 entries.");
+                }
+                dims[i] = dims[n.lhs];
+                break;
+            }
+            case ExprOp::SCAN_MIN_BACKWARD:
+            case ExprOp::SCAN_MAX_BACKWARD:
+            case ExprOp::SEGMENTED_SCAN_MIN_BACKWARD:
+            case ExprOp::SEGMENTED_SCAN_MAX_BACKWARD: {
+                if (dims[n.rhs] != dims[n.lhs]) throw std::runtime_error("Scan min/max backward requires a gradient shaped like the scanned operand.");
+                const bool segmented = n.op == ExprOp::SEGMENTED_SCAN_MIN_BACKWARD || n.op == ExprOp::SEGMENTED_SCAN_MAX_BACKWARD;
+                if (segmented != (n.aux != UINT32_MAX)) throw std::runtime_error("Scan min/max backward: offsets go with segmented scans only.");
+                if (!segmented && n.scan_axis != UINT64_MAX && n.scan_axis != dims[n.lhs].size() - 1) {
+                    throw std::runtime_error("Expression::scan currently supports only the last axis.");
                 }
                 dims[i] = dims[n.lhs];
                 break;
@@ -567,7 +581,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
                 ensureTensor(n.rhs);
-            } else if (n.op == ExprOp::ROPE) {
+            } else if (n.op == ExprOp::ROPE || isScanBackwardOp(n.op)) {
                 graph->role[i] = Role::Materialized;
                 for (uint32_t operand : {n.lhs, n.rhs, n.aux})
                     if (operand != UINT32_MAX) ensureTensor(operand);
@@ -650,7 +664,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
                 sources.push_back(graph->expr.nodes[i].lhs);
             } else if (graph->expr.nodes[i].op == ExprOp::SCAN) {
                 sources.push_back(graph->expr.nodes[i].lhs);
-            } else if (graph->expr.nodes[i].op == ExprOp::ROPE) {
+            } else if (graph->expr.nodes[i].op == ExprOp::ROPE || isScanBackwardOp(graph->expr.nodes[i].op)) {
                 for (uint32_t operand : {graph->expr.nodes[i].lhs, graph->expr.nodes[i].rhs, graph->expr.nodes[i].aux})
                     if (operand != UINT32_MAX) sources.push_back(operand);
             } else if (isWinnerRoutingOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::TAKE_ALONG_AXIS ||
@@ -833,7 +847,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     auto runsInFusedKernel = [&](uint32_t i) {
         const ExprOp op = expr.nodes[i].op;
         return graph->role[i] == Role::Materialized && !isReductionOp(op) && !isSegmentedReduceOp(op) && op != ExprOp::SEGMENTED_BROADCAST &&
-               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && op != ExprOp::ROPE && !isScanOp(op) && op != ExprOp::INPUT;
+               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && op != ExprOp::ROPE && !isScanBackwardOp(op) && !isScanOp(op) && op != ExprOp::INPUT;
     };
     std::vector<uint32_t> levelOf = graph->level;
     if (stageFusionEnabled()) {
@@ -845,7 +859,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 sources.push_back(n.lhs);
             } else if (n.op == ExprOp::SCAN) {
                 sources = {n.lhs};
-            } else if (n.op == ExprOp::ROPE) {
+            } else if (n.op == ExprOp::ROPE || isScanBackwardOp(n.op)) {
                 for (uint32_t operand : {n.lhs, n.rhs, n.aux})
                     if (operand != UINT32_MAX) sources.push_back(operand);
             } else if (isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS || n.op == ExprOp::SEGMENTED_SCAN) {
@@ -1310,6 +1324,71 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 tensorOf[i] = scanned;
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
+                done[i] = 1;
+                continue;
+            }
+            if (isScanBackwardOp(n.op)) {
+                if (fusedKernelsOnly) {
+                    throw std::runtime_error(
+                        "FusedEquation::run() only supports expressions that lower to fused kernels; this expression has a scan stage. "
+                        "Use stamp() and run the returned plan.");
+                }
+                // which element held the running minimum / maximum at every position (an arg scan), then every position's gradient
+                // added into that element of a cleared FP32 tensor
+                const Tensor& values = tensorOf[n.lhs];
+                const Tensor& gradient = tensorOf[n.rhs];
+                if (!values.isDenseContiguous() || !gradient.isDenseContiguous()) throw std::runtime_error("Scan min/max backward needs dense operands.");
+                const bool segmented = n.aux != UINT32_MAX;
+                Tensor winners(gpuPlacement, TensorDescriptor(DataType::UINT32, values.getDimensions()));
+                ScanRequest request;
+                request.dtype = values.getDataType();
+                request.total = values.getTotalNumElements();
+                request.deviceNum = device_num;
+                request.op = (n.op == ExprOp::SCAN_MIN_BACKWARD || n.op == ExprOp::SEGMENTED_SCAN_MIN_BACKWARD) ? 1 : 2;
+                request.writeValue = false;
+                request.writeIndex = true;
+                request.inclusive = n.scan_mode == ScanMode::Inclusive;
+                request.reverse = n.scan_reverse;
+                request.alignmentBytes = std::min(pointerAlignment(values.getMemPtr()), pointerAlignment(winners.getMemPtr()));
+                std::optional<Tensor> offsets;
+                std::vector<uint32_t> scanSources{n.lhs};
+                if (segmented) {
+                    offsets = tensorOf[n.aux];
+                    if (!offsets->isDenseContiguous()) throw std::runtime_error("Segmented scan needs dense offsets.");
+                    request.row = 0;
+                    request.segments = offsets->getTotalNumElements() - 1;
+                    request.offsets64 = offsets->getDataType() == DataType::UINT64;
+                    scanSources.push_back(n.aux);
+                } else {
+                    request.row = dims[n.lhs].back();
+                    request.segments = request.total / request.row;
+                }
+                const std::shared_ptr<const CubScanKernels> kernels = buildScanKernels(request);
+                Tensor temp(gpuPlacement, TensorDescriptor(DataType::UINT8, {std::max<uint64_t>(kernels->tempBytes, 1)}));
+                StampedExecutionStage scanStage;
+                scanStage.kind = StampedExecutionStage::Kind::Scan;
+                scanStage.gpu_num = device_num;
+                scanStage.dependency_stage_indices = dependenciesOf(scanSources);
+                scanStage.scan = std::make_shared<StampedScan>(kernels, values, offsets, temp, winners, /*indexOutput=*/true);
+                const uint32_t scanIndex = static_cast<uint32_t>(stages.size());
+                stages.push_back(std::move(scanStage));
+                Tensor routed = allocateFor(i);
+                StampedExecutionStage clearStage;
+                clearStage.kind = StampedExecutionStage::Kind::FusedKernel;
+                clearStage.gpu_num = device_num;
+                clearStage.kernel = stampScatterClear(routed, device_num);
+                const uint32_t clearIndex = static_cast<uint32_t>(stages.size());
+                stages.push_back(std::move(clearStage));
+                StampedExecutionStage addStage;
+                addStage.kind = StampedExecutionStage::Kind::FusedKernel;
+                addStage.gpu_num = device_num;
+                addStage.dependency_stage_indices = dependenciesOf({n.rhs});
+                addStage.dependency_stage_indices.push_back(scanIndex);
+                addStage.dependency_stage_indices.push_back(clearIndex);
+                addStage.kernel = stampScatterAdd(gradient, winners, routed, offsets, device_num);
+                tensorOf[i] = routed;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(addStage));
                 done[i] = 1;
                 continue;
             }

@@ -1,0 +1,122 @@
+// Flat scatter-add: output[indices[i]] += updates[i] (the reference's contract: Utilities/Expression/FlatScatterAddKernel.h:17-30
+// there, which sorts the destinations, reduces equal ones and applies the result with a sparse-vector library call).
+//
+// Here the destinations come from arg scans, so equal destinations sit next to each other in long runs (a running maximum
+// changes rarely).  A wavefront first adds up every run of equal neighbouring destinations among its 64 elements with shuffles,
+// then the last lane of each run issues one hardware fp32 atomic add; a row whose maximum never changes costs one atomic per
+// wavefront instead of 64.  Sums of more than one wavefront's worth of values are added in the order the atomics arrive.
+#include "ScatterAdd.h"
+
+#include "ReductionPlanner.h"
+#include "Utilities/Expression/CompiledEquation.h"
+#include "thorhip_numeric_embed.h"
+
+#include <sstream>
+#include <stdexcept>
+
+namespace ThorImplementation {
+
+namespace {
+
+std::string clearSource(uint64_t outputs, int clearVec) {
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude;
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scatter_clear(float* __restrict__ out) {\n";
+    s << "    const thor::u64 vector = (thor::u64)blockIdx.x * 256 + threadIdx.x;\n";
+    s << "    if (vector >= " << outputs / clearVec << "ull) return;\n";
+    s << "    thor::Pack<float, " << clearVec << "> zero = {};\n";
+    s << "    zero.store(out + vector * " << clearVec << ");\n}\n";
+    return s.str();
+}
+
+// offsetsType: empty = every update counts; else the updates outside [offsets[0], offsets[segments]) are skipped
+std::string addSource(uint64_t updates, uint64_t outputs, const std::string& offsetsType, uint64_t segments) {
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude;
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scatter_add(const float* __restrict__ updates, const thor::u32* __restrict__ indices,\n";
+    s << "                                                                   ";
+    if (!offsetsType.empty()) s << "const " << offsetsType << "* __restrict__ offsets, ";
+    s << "float* __restrict__ out) {\n";
+    s << "    const thor::u64 i = (thor::u64)blockIdx.x * 256 + threadIdx.x;\n";
+    s << "    thor::u32 key = 0xffffffffu;\n    float v = 0.0f;\n";
+    if (offsetsType.empty()) {
+        s << "    if (i < " << updates << "ull) {\n        key = indices[i];\n        v = updates[i];\n    }\n";
+    } else {
+        s << "    const thor::u64 first = (thor::u64)offsets[0], end = (thor::u64)offsets[" << segments << "];\n";
+        s << "    if (i < " << updates << "ull && i >= first && i < end) {\n        key = indices[i];\n        v = updates[i];\n    }\n";
+    }
+    s << "    if (key >= " << outputs << "ull) key = 0xffffffffu;\n";
+    s << "    const int lane = threadIdx.x & 63;\n";
+    // runs of equal neighbouring destinations inside the wavefront: bit l of `heads` = lane l starts a run
+    s << "    const thor::u32 before = __shfl_up(key, 1);\n";
+    s << "    const thor::u64 heads = __ballot(lane == 0 || before != key);\n";
+    s << "    const int start = 63 - __builtin_clzll(heads & (~0ull >> (63 - lane)));\n";
+    s << "#pragma unroll\n    for (int off = 1; off < 64; off <<= 1) {\n";
+    s << "        const float other = __shfl_up(v, off);\n";
+    s << "        if (lane - off >= start) v += other;\n    }\n";
+    s << "    const bool last = lane == 63 || ((heads >> (lane + 1)) & 1ull) != 0;\n";
+    s << "    if (last && key != 0xffffffffu) unsafeAtomicAdd(out + key, v);\n}\n";
+    return s.str();
+}
+
+void requireDense(const Tensor& t, DataType dtype, const char* what) {
+    if (!t.isInitialized() || !t.isDenseContiguous() || t.getDataType() != dtype) {
+        throw std::runtime_error(std::string("Scatter-add requires a dense ") + dataTypeName(dtype) + " " + what + " tensor.");
+    }
+}
+
+int clearVectorOf(const Tensor& output) {
+    int vec = 4;
+    while (vec > 1 && (output.getTotalNumElements() % vec != 0 || pointerAlignment(output.getMemPtr()) % (4ull * vec) != 0)) vec /= 2;
+    return vec;
+}
+
+}  // namespace
+
+std::shared_ptr<StampedEquation> stampScatterClear(const Tensor& output, int deviceNum) {
+    requireDense(output, DataType::FP32, "output");
+    const uint64_t outputs = output.getTotalNumElements();
+    const int vec = clearVectorOf(output);
+    const uint64_t blocks = (outputs / vec + 255) / 256;
+    if (blocks > 0x7fffffffull) throw std::runtime_error("Scatter-add: the output is too large for one launch.");
+    const std::shared_ptr<CompiledKernel> kernel = compileKernel(clearSource(outputs, vec), "thor_scatter_clear", deviceNum, /*fastContract=*/false);
+    std::ostringstream description;
+    description << "scatter_clear(n=" << outputs << ",vec=" << vec << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
+    return std::make_shared<StampedEquation>(kernel, std::vector<Tensor>{}, std::vector<Tensor>{output}, std::vector<StampedEquation::ScalarArgument>{},
+                                             std::vector<size_t>{}, std::vector<size_t>{0}, 1, /*passNumel=*/false, outputs, outputs > UINT32_MAX,
+                                             static_cast<uint32_t>(blocks), 256, /*flops=*/0, description.str());
+}
+
+std::shared_ptr<StampedEquation> stampScatterAdd(const Tensor& updates, const Tensor& indices, const Tensor& output, const std::optional<Tensor>& offsets,
+                                                 int deviceNum) {
+    requireDense(updates, DataType::FP32, "updates");
+    requireDense(indices, DataType::UINT32, "indices");
+    requireDense(output, DataType::FP32, "output");
+    const uint64_t count = updates.getTotalNumElements(), outputs = output.getTotalNumElements();
+    if (indices.getTotalNumElements() != count) throw std::runtime_error("Scatter-add requires one index per update.");
+    if (outputs >= 0xffffffffull) throw std::runtime_error("Scatter-add: UINT32 indices cannot address an output this large.");
+    const uint64_t blocks = (count + 255) / 256;
+    if (blocks > 0x7fffffffull) throw std::runtime_error("Scatter-add: too many updates for one launch.");
+    std::string offsetsType;
+    uint64_t segments = 0;
+    if (offsets.has_value()) {
+        if (!offsets->isInitialized() || !offsets->isDenseContiguous() || offsets->getTotalNumElements() < 2 ||
+            (offsets->getDataType() != DataType::UINT32 && offsets->getDataType() != DataType::UINT64)) {
+            throw std::runtime_error("Scatter-add requires dense UINT32 or UINT64 offsets [B + 1].");
+        }
+        offsetsType = offsets->getDataType() == DataType::UINT64 ? "thor::u64" : "thor::u32";
+        segments = offsets->getTotalNumElements() - 1;
+    }
+    const std::shared_ptr<CompiledKernel> kernel = compileKernel(addSource(count, outputs, offsetsType, segments), "thor_scatter_add", deviceNum, /*fastContract=*/false);
+    std::ostringstream description;
+    description << "scatter_add(updates=" << count << ",into=" << outputs << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
+    std::vector<Tensor> inputs = {updates, indices};
+    if (offsets.has_value()) inputs.push_back(*offsets);
+    std::vector<size_t> inputArgs;
+    for (size_t i = 0; i < inputs.size(); ++i) inputArgs.push_back(i);
+    return std::make_shared<StampedEquation>(kernel, inputs, std::vector<Tensor>{output}, std::vector<StampedEquation::ScalarArgument>{}, inputArgs,
+                                             std::vector<size_t>{inputs.size()}, inputs.size() + 1, /*passNumel=*/false, count, count > UINT32_MAX,
+                                             static_cast<uint32_t>(blocks), 256, /*flops=*/0, description.str());
+}
+
+}  // namespace ThorImplementation
