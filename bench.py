@@ -314,6 +314,12 @@ def bench_other_configs():
     row_argmax = ex.compile(ex.input("x").scan(ScanOp.arg_max), 0)
     plans = [row_argmax.stamp({"x": t}, stream) for t in xs3]
     timed("scan_c3_row_running_argmax_fp32", [p_.run for p_ in plans], 8 * n, n, plans[0].stage_descriptions()[0])
+    # gradient of the running maximum: reads x and the upstream gradient, writes the gradient (12 B/element)
+    gs3 = [clone(x), clone(x), clone(x)]
+    row_max_scan_backward = ex.compile(ex.input("x").scan(ScanOp.max), 0).compile_backward(["x"], error_input_name="__grad_output")
+    plans = [row_max_scan_backward.stamp({"x": t, "__grad_output": g_}, stream) for t, g_ in zip(xs3, gs3)]
+    timed("backward_scan_c3_row_running_max_fp32", [p_.run for p_ in plans], 12 * n, n, " | ".join(plans[0].stage_descriptions()))
+    del gs3
     flat = ex.compile(ex.input("x").reshape([n]).scan(ScanOp.sum), 0)
     plans = [flat.stamp({"x": t}, stream) for t in xs3]
     timed("scan_flat_cumsum_fp32_2^26", [p_.run for p_ in plans], 8 * n, n, plans[0].stage_descriptions()[0])

@@ -163,6 +163,12 @@ class GraphBuilder {
             // the rotation kernel addresses dense storage; position ids and the effective length are small tensors it reads
             for (uint32_t* operand : {&node.lhs, &node.rhs, &node.aux}) {
                 if (*operand == UINT32_MAX) continue;
+                // a conversion of a bound tensor to the dtype it already has would only copy it: these kernels read the tensor itself
+                const ExprNode& asked = out.nodes[*operand];
+                if (asked.op == ExprOp::CAST && out.nodes[asked.lhs].op == ExprOp::INPUT && out.nodes[asked.lhs].output_dtype == asked.output_dtype &&
+                    out.nodes[asked.lhs].input_tensor_dtype == asked.output_dtype) {
+                    *operand = asked.lhs;
+                }
                 *operand = asTensorOperand(*operand, false);
                 if (isStorageViewOp(out.nodes[*operand].op)) *operand = castOf(*operand, out.nodes[*operand].output_dtype.value());
             }

@@ -11,6 +11,7 @@
 #include "Utilities/Expression/CompiledEquation.h"
 #include "thorhip_numeric_embed.h"
 
+#include <algorithm>
 #include <sstream>
 #include <stdexcept>
 
@@ -30,23 +31,28 @@ std::string clearSource(uint64_t outputs, int clearVec) {
 }
 
 // offsetsType: empty = every update counts; else the updates outside [offsets[0], offsets[segments]) are skipped
-std::string addSource(uint64_t updates, uint64_t outputs, const std::string& offsetsType, uint64_t segments) {
+std::string addSource(uint64_t updates, uint64_t outputs, const std::string& offsetsType, uint64_t segments, uint64_t blocks) {
     std::ostringstream s;
     s << thor_embed::kDevicePrelude;
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scatter_add(const float* __restrict__ updates, const thor::u32* __restrict__ indices,\n";
     s << "                                                                   ";
     if (!offsetsType.empty()) s << "const " << offsetsType << "* __restrict__ offsets, ";
     s << "float* __restrict__ out) {\n";
-    s << "    const thor::u64 i = (thor::u64)blockIdx.x * 256 + threadIdx.x;\n";
-    s << "    thor::u32 key = 0xffffffffu;\n    float v = 0.0f;\n";
-    if (offsetsType.empty()) {
-        s << "    if (i < " << updates << "ull) {\n        key = indices[i];\n        v = updates[i];\n    }\n";
-    } else {
-        s << "    const thor::u64 first = (thor::u64)offsets[0], end = (thor::u64)offsets[" << segments << "];\n";
-        s << "    if (i < " << updates << "ull && i >= first && i < end) {\n        key = indices[i];\n        v = updates[i];\n    }\n";
-    }
-    s << "    if (key >= " << outputs << "ull) key = 0xffffffffu;\n";
     s << "    const int lane = threadIdx.x & 63;\n";
+    if (!offsetsType.empty()) s << "    const thor::u64 first = (thor::u64)offsets[0], end = (thor::u64)offsets[" << segments << "];\n";
+    // a block walks tiles of 256 updates, every lane of it through every step (the shuffles below need whole wavefronts)
+    // (the loads of the next tile are issued before the current one is combined)
+    const std::string live = offsetsType.empty() ? "i < " + std::to_string(updates) + "ull" : "i < " + std::to_string(updates) + "ull && i >= first && i < end";
+    s << "    auto fetch = [&](thor::u64 tile, thor::u32& key, float& v) {\n";
+    s << "        const thor::u64 i = tile * 256 + threadIdx.x;\n";
+    s << "        key = 0xffffffffu;\n        v = 0.0f;\n";
+    s << "        if (" << live << ") {\n            key = __builtin_nontemporal_load(indices + i);\n            v = __builtin_nontemporal_load(updates + i);\n        }\n    };\n";
+    s << "    thor::u32 key, nextKey;\n    float v, nextV;\n";
+    s << "    fetch(blockIdx.x, nextKey, nextV);\n";
+    s << "    for (thor::u64 tile = blockIdx.x; tile < " << (updates + 255) / 256 << "ull; tile += " << blocks << "ull) {\n";
+    s << "    key = nextKey;\n    v = nextV;\n";
+    s << "    fetch(tile + " << blocks << "ull, nextKey, nextV);\n";
+    s << "    if (key >= " << outputs << "ull) key = 0xffffffffu;\n";
     // runs of equal neighbouring destinations inside the wavefront: bit l of `heads` = lane l starts a run
     s << "    const thor::u32 before = __shfl_up(key, 1);\n";
     s << "    const thor::u64 heads = __ballot(lane == 0 || before != key);\n";
@@ -55,7 +61,7 @@ std::string addSource(uint64_t updates, uint64_t outputs, const std::string& off
     s << "        const float other = __shfl_up(v, off);\n";
     s << "        if (lane - off >= start) v += other;\n    }\n";
     s << "    const bool last = lane == 63 || ((heads >> (lane + 1)) & 1ull) != 0;\n";
-    s << "    if (last && key != 0xffffffffu) unsafeAtomicAdd(out + key, v);\n}\n";
+    s << "    if (last && key != 0xffffffffu) unsafeAtomicAdd(out + key, v);\n    }\n}\n";
     return s.str();
 }
 
@@ -95,8 +101,7 @@ std::shared_ptr<StampedEquation> stampScatterAdd(const Tensor& updates, const Te
     const uint64_t count = updates.getTotalNumElements(), outputs = output.getTotalNumElements();
     if (indices.getTotalNumElements() != count) throw std::runtime_error("Scatter-add requires one index per update.");
     if (outputs >= 0xffffffffull) throw std::runtime_error("Scatter-add: UINT32 indices cannot address an output this large.");
-    const uint64_t blocks = (count + 255) / 256;
-    if (blocks > 0x7fffffffull) throw std::runtime_error("Scatter-add: too many updates for one launch.");
+    const uint64_t blocks = std::min<uint64_t>((count + 255) / 256, 8192);
     std::string offsetsType;
     uint64_t segments = 0;
     if (offsets.has_value()) {
@@ -107,7 +112,7 @@ std::shared_ptr<StampedEquation> stampScatterAdd(const Tensor& updates, const Te
         offsetsType = offsets->getDataType() == DataType::UINT64 ? "thor::u64" : "thor::u32";
         segments = offsets->getTotalNumElements() - 1;
     }
-    const std::shared_ptr<CompiledKernel> kernel = compileKernel(addSource(count, outputs, offsetsType, segments), "thor_scatter_add", deviceNum, /*fastContract=*/false);
+    const std::shared_ptr<CompiledKernel> kernel = compileKernel(addSource(count, outputs, offsetsType, segments, blocks), "thor_scatter_add", deviceNum, /*fastContract=*/false);
     std::ostringstream description;
     description << "scatter_add(updates=" << count << ",into=" << outputs << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
     std::vector<Tensor> inputs = {updates, indices};
