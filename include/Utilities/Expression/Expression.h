@@ -132,6 +132,12 @@ inline bool isScanBackwardOp(ExprOp op) {
     return op == ExprOp::SCAN_MIN_BACKWARD || op == ExprOp::SCAN_MAX_BACKWARD || op == ExprOp::SEGMENTED_SCAN_MIN_BACKWARD ||
            op == ExprOp::SEGMENTED_SCAN_MAX_BACKWARD;
 }
+// Gradient of a per-segment min / max (AutoDiff.cpp:5630-5700 there): lhs = the packed values [N, D...], rhs = the FP32 gradient
+// of the reduction's output [B, D...], aux = the offsets.  Each segment's gradient goes to the row that won the column (the
+// lowest row among equals); every other element, and every row outside the partition, gets 0.  FP32, shaped like the values.
+inline bool isSegmentWinnerRoutingOp(ExprOp op) { return op == ExprOp::SEGMENTED_REDUCE_MIN_BACKWARD || op == ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD; }
+// Stages that read up to three dense tensors (lhs, rhs, aux) and scatter gradients into a cleared FP32 tensor.
+inline bool isScatterRoutingOp(ExprOp op) { return isScanBackwardOp(op) || isSegmentWinnerRoutingOp(op); }
 inline bool isRaggedOp(ExprOp op) {
     return isSegmentedReduceOp(op) || op == ExprOp::SEGMENTED_BROADCAST || op == ExprOp::RAGGED_VALUEWISE_EXTENT;
 }

@@ -192,6 +192,7 @@ struct StampedExecutionStage {
     std::shared_ptr<StampedArgMinMax> arg_minmax;
     std::shared_ptr<StampedFusedReduction> fused_reduction;
     std::shared_ptr<StampedSegmentedReductionStage> segmented_reduction;
+    std::shared_ptr<StampedCubSegmentedArgReduction> segmented_arg_reduction;  // SegmentedReduction stages that find winners instead of values
     std::shared_ptr<StampedSegmentedBroadcast> segmented_broadcast;
     std::shared_ptr<StampedScan> scan;
     // Kind::Copy: a named output that is only a view of an input is copied into the caller's tensor

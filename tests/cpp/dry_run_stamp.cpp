@@ -250,6 +250,7 @@ static int runAll() {
                     std::vector<uint64_t> perSegment{200};
                     if (elements > 1) perSegment.push_back(elements);
                     stampBackward(tag + "backward of mean", r.segment_mean(), inputs, Tensor(gpuPlacement, TensorDescriptor(dtype, perSegment)), stream);
+                    stampBackward(tag + "backward of max", r.segment_max(), inputs, Tensor(gpuPlacement, TensorDescriptor(dtype, perSegment)), stream);
                     stampBackward(tag + "backward of exp(sum) spread over rows",
                                   r.getValues().exp() * Expression::segmentedBroadcast(r.segment_sum(), r.getOffsets(), 200, 6000, elements, false), inputs,
                                   Tensor(gpuPlacement, TensorDescriptor(dtype, dims)), stream);

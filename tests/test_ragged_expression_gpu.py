@@ -245,3 +245,52 @@ def test_segmented_reduction_of_an_expression_with_scalars_and_means(stream):
     want = np.stack([((x[lo:hi] - x[lo:hi].mean(axis=0)) ** 2).sum(axis=0) * 0.5 if hi > lo else np.zeros(4)
                      for lo, hi in zip(offsets[:-1].astype(int), offsets[1:].astype(int))])
     np.testing.assert_allclose(copy_gpu_to_numpy(plan.output("scatter"), stream), want, rtol=2e-5, atol=1e-5)
+
+
+# ---- backward of per-segment min / max: the segment's gradient goes to the row that won the column --------------------------------
+def test_segment_min_max_backward_known_answers(stream):
+    """The values and offsets of RaggedExpressionTest.cpp:1795-1824 there; winners read off by hand: min rows 1, -, 3, 5 and max
+    rows 2, -, 4, 6; rows 7 and 8 belong to no segment; the empty segment's gradient goes nowhere."""
+    values = np.array([1, -2, 4, 5, 7, -1, 8, 99, 100], np.float32)
+    offsets = np.array([0, 3, 3, 5, 7], np.uint32)
+    upstream = np.array([10, 20, 30, 40], np.float32)
+    tensors = {"v": copy_numpy_to_gpu(values, stream, DataType.fp32), "o": copy_numpy_to_gpu(offsets, stream, DataType.uint32),
+               "__grad_output": copy_numpy_to_gpu(upstream, stream, DataType.fp32)}
+    expected = {"min": [0, 10, 0, 30, 0, 40, 0, 0, 0], "max": [0, 0, 10, 0, 30, 0, 40, 0, 0]}
+    for kind in ("min", "max"):
+        fwd = ex.compile(getattr(ex.input("v"), "segment_" + kind)(ex.input("o"), 4, 9, 1), device_num=0)
+        plan = fwd.compile_backward(["v"], error_input_name="__grad_output").stamp(tensors, stream)
+        plan.run()
+        assert plan.stage_kind_names().count("SegmentedReduction") == 1 and sum("scatter_add" in d for d in plan.stage_descriptions()) == 1
+        np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("v_grad"), stream), np.array(expected[kind], np.float32))
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16], ids=lambda d: d.name)
+@pytest.mark.parametrize("offsets_dtype", [DataType.uint32, DataType.uint64], ids=lambda d: d.name)
+@pytest.mark.parametrize("kind", ["min", "max"])
+def test_segment_min_max_backward_against_numpy(stream, kind, offsets_dtype, dtype):
+    rng = np.random.default_rng(71)
+    rows, width, segments = 5000, 24, 300
+    cuts = np.sort(rng.integers(0, rows - 100, segments - 1))
+    offsets = np.concatenate([[0], cuts, [rows - 100]])  # empty segments among them, the last 100 rows in no segment
+    values = to_storage(rng.integers(-20, 21, (rows, width)).astype(np.float32) * 0.25, dtype)  # many ties: the lowest row must win
+    upstream = to_storage(rng.integers(-8, 9, (segments, width)).astype(np.float32) * 0.5, dtype)
+    carrier = np.uint32 if offsets_dtype == DataType.uint32 else np.uint64
+    v, o = ex.input("v"), ex.input("o")
+    # through elementwise work on both sides of the reduction
+    loss = getattr(v * 2.0, "segment_" + kind)(o, segments, rows, width) * 3.0
+    plan = ex.compile(loss, device_num=0).compile_backward(["v"], error_input_name="__grad_output").stamp(
+        {"v": copy_numpy_to_gpu(values, stream, dtype), "o": copy_numpy_to_gpu(offsets.astype(carrier), stream, offsets_dtype),
+         "__grad_output": copy_numpy_to_gpu(upstream, stream, dtype)}, stream)
+    plan.run()
+    x = from_storage(values, dtype).astype(np.float64)
+    g = from_storage(upstream, dtype).astype(np.float64)
+    expected = np.zeros((rows, width))
+    for s in range(segments):
+        lo, hi = int(offsets[s]), int(offsets[s + 1])
+        if hi > lo:
+            winner = lo + (np.argmin(x[lo:hi], axis=0) if kind == "min" else np.argmax(x[lo:hi], axis=0))  # first among equals
+            expected[winner, np.arange(width)] = 6.0 * g[s]
+    got = from_storage(copy_gpu_to_numpy(plan.output("v_grad"), stream), dtype).astype(np.float64)
+    assert plan.output("v_grad").get_data_type() == dtype
+    np.testing.assert_array_equal(got, expected)  # 6 * (multiples of 0.5 up to 4) is exact in bf16 too

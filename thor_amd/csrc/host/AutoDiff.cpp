@@ -224,6 +224,19 @@ class BackwardGraph {
         n.ragged_runtime_elements_per_value = like.ragged_runtime_elements_per_value;
         return push(std::move(n), dims[values]);
     }
+    // the gradient of the per-segment min / max `like`: packed values, FP32 gradient of the segments, offsets
+    uint32_t segmentWinnerGradient(uint32_t values, uint32_t gradient, uint32_t offsets, const ExprNode& like) {
+        ExprNode n;
+        n.op = like.op == ExprOp::SEGMENTED_REDUCE_MIN ? ExprOp::SEGMENTED_REDUCE_MIN_BACKWARD : ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD;
+        n.lhs = values;
+        n.rhs = gradient;
+        n.aux = offsets;
+        n.ragged_runtime_batch_size = like.ragged_runtime_batch_size;
+        n.ragged_runtime_max_active_values = like.ragged_runtime_max_active_values;
+        n.ragged_runtime_elements_per_value = like.ragged_runtime_elements_per_value;
+        n.output_dtype = DataType::FP32;
+        return push(std::move(n), dims[values]);
+    }
     // the gradient of the min / max scan `like`: operand, FP32 upstream gradient, offsets of a segmented scan
     uint32_t scanWinnerGradient(uint32_t operand, uint32_t gradient, uint32_t offsets, const ExprNode& like) {
         ExprNode n;
@@ -552,6 +565,11 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
             case ExprOp::SEGMENTED_REDUCE_MEAN:
                 // every row of a segment receives the segment's gradient (divided by the segment's length for a mean)
                 contribute(n.lhs, b.segmentedBroadcast(g, b.value(n.rhs), fdims[n.lhs].at(0), n.op == ExprOp::SEGMENTED_REDUCE_MEAN));
+                break;
+            case ExprOp::SEGMENTED_REDUCE_MIN:
+            case ExprOp::SEGMENTED_REDUCE_MAX:
+                // each segment's gradient goes to the row that won the column (Utilities/Expression/AutoDiff.cpp:5630-5700 there)
+                contribute(n.lhs, b.segmentWinnerGradient(x(), b.cast(g, DataType::FP32), b.value(n.rhs), n));
                 break;
             case ExprOp::SEGMENTED_BROADCAST:
                 contribute(n.lhs, b.segmentedReduce(n.segmented_broadcast_normalize_by_length ? ExprOp::SEGMENTED_REDUCE_MEAN : ExprOp::SEGMENTED_REDUCE_SUM,

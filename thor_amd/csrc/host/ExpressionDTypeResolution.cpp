@@ -29,7 +29,7 @@ bool isBindableInputDType(DataType dtype) {
 }
 
 void rejectUnsupportedOp(ExprOp op) {
-    if (isRaggedOp(op) || isStorageViewOp(op) || isWinnerRoutingOp(op) || op == ExprOp::TAKE_ALONG_AXIS || op == ExprOp::ROPE || isScanBackwardOp(op) || isScanOp(op)) return;
+    if (isRaggedOp(op) || isStorageViewOp(op) || isWinnerRoutingOp(op) || op == ExprOp::TAKE_ALONG_AXIS || op == ExprOp::ROPE || isScatterRoutingOp(op) || isScanOp(op)) return;
     if (Expression::isLeafOp(op) || Expression::isUnaryOp(op) || Expression::isBinaryOp(op) || Expression::isTernaryOp(op)) return;
     throw std::runtime_error("Expression op '" + opName(op) + "' is outside the elementwise / reduction / cast path of this backend.");
 }
@@ -37,7 +37,7 @@ void rejectUnsupportedOp(ExprOp op) {
 std::vector<DataType> tensorParentDTypes(const ExprNode& node, const std::vector<ExprNode>& nodes, const std::vector<DataType>& resolved) {
     std::vector<DataType> out;
     if (isRaggedOp(node.op)) return {resolved.at(node.lhs)};  // the offsets are structure, not a value
-    if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScanBackwardOp(node.op) || isScanOp(node.op)) return {resolved.at(node.lhs)};
+    if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScatterRoutingOp(node.op) || isScanOp(node.op)) return {resolved.at(node.lhs)};
     auto add = [&](uint32_t parent) {
         if (parent >= nodes.size()) throw std::runtime_error("Parent node index out of range during dtype resolution.");
         if (!isScalarLeaf(nodes[parent].op)) out.push_back(resolved[parent]);
@@ -109,6 +109,12 @@ DataType nodeOutputDType(const ExprNode& node, const std::vector<ExprNode>& node
             throw std::runtime_error(std::string("take_along_axis indices must have UINT32 or UINT64 dtype, received: ") + dataTypeName(indexType));
         }
         return node.output_dtype.value_or(resolved[node.lhs]);
+    }
+    if (isSegmentWinnerRoutingOp(node.op)) {
+        if (!isSupportedFusionFloatingType(resolved[node.lhs])) throw std::runtime_error("Segmented min/max backward requires floating-point values.");
+        if (resolved[node.rhs] != DataType::FP32) throw std::runtime_error("Segmented min/max backward requires an FP32 gradient.");
+        if (node.output_dtype.has_value() && node.output_dtype.value() != DataType::FP32) throw std::runtime_error("Segmented min/max backward produces FP32.");
+        return DataType::FP32;
     }
     if (isScanBackwardOp(node.op)) {
         const DataType in = resolved[node.lhs];
@@ -230,7 +236,7 @@ void propagateMaterialisedDTypes(PhysicalExpression& expr, const std::vector<uin
             // an explicit conversion boundary: the source keeps its own compute dtype
         } else if (node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST) {
             toParent(node.lhs);  // never into the offsets
-        } else if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScanBackwardOp(node.op) || isScanOp(node.op)) {
+        } else if (isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScatterRoutingOp(node.op) || isScanOp(node.op)) {
             // the operands are read as stored tensors: nothing to widen
         } else if (isReductionOp(node.op) || node.op == ExprOp::SOFTMAX || isSegmentedReduceOp(node.op)) {
             // the reduction's mandatory fp32 stays inside the reduction; its producer keeps its own policy
@@ -284,7 +290,7 @@ void resolveInPlace(PhysicalExpression& expr, const std::vector<DataType>& rootD
         const DataType logicalIn = nodeLogicalInputDType(node, expr.nodes, resolved);
         DataType requested;
         if (node.op == ExprOp::CAST || isShapeOnly(node.op) || node.op == ExprOp::RAGGED_VALUEWISE_EXTENT || node.op == ExprOp::SEGMENTED_BROADCAST ||
-            isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScanBackwardOp(node.op) || isScanOp(node.op)) {
+            isWinnerRoutingOp(node.op) || node.op == ExprOp::TAKE_ALONG_AXIS || node.op == ExprOp::ROPE || isScatterRoutingOp(node.op) || isScanOp(node.op)) {
             requested = out;  // values pass through unchanged (a normalised broadcast divides in fp32 and rounds once)
         } else if (isSegmentedReduceOp(node.op)) {
             requested = DataType::FP32;
@@ -370,7 +376,7 @@ DataType toSupportedComputeDType(ExprOp op, DataType requested) {
         throw std::runtime_error("Unsupported boolean/comparison/where dtype in toSupportedComputeDType.");
     }
     if (op == ExprOp::CAST || isShapeOnly(op) || op == ExprOp::RAGGED_VALUEWISE_EXTENT || op == ExprOp::SEGMENTED_BROADCAST || isWinnerRoutingOp(op) ||
-        op == ExprOp::TAKE_ALONG_AXIS || op == ExprOp::ROPE || isScanBackwardOp(op) || isScanOp(op)) {
+        op == ExprOp::TAKE_ALONG_AXIS || op == ExprOp::ROPE || isScatterRoutingOp(op) || isScanOp(op)) {
         if (isBindableInputDType(requested)) return requested;
         throw std::runtime_error("Unsupported passthrough dtype in toSupportedComputeDType.");
     }

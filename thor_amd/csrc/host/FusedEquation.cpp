@@ -159,7 +159,7 @@ class GraphBuilder {
             node.lhs = asTensorOperand(node.lhs, false);
             if (isStorageViewOp(out.nodes[node.lhs].op)) node.lhs = castOf(node.lhs, out.nodes[node.lhs].output_dtype.value());
             if (node.op == ExprOp::SEGMENTED_SCAN) node.rhs = asTensorOperand(node.rhs, false);
-        } else if (node.op == ExprOp::ROPE || isScanBackwardOp(node.op)) {
+        } else if (node.op == ExprOp::ROPE || isScatterRoutingOp(node.op)) {
             // the rotation kernel addresses dense storage; position ids and the effective length are small tensors it reads
             for (uint32_t* operand : {&node.lhs, &node.rhs, &node.aux}) {
                 if (*operand == UINT32_MAX) continue;
@@ -244,7 +244,7 @@ uint32_t baseOfView(const PlannedGraph& g, uint32_t node) {
 bool consumesGather(const ExprNode& consumer) {
     if (consumer.op == ExprOp::RAGGED_VALUEWISE_EXTENT || consumer.op == ExprOp::WHERE || consumer.op == ExprOp::CAST) return true;
     if (isReductionOp(consumer.op) || isRaggedOp(consumer.op) || isShapeOnly(consumer.op) || consumer.op == ExprOp::SOFTMAX || isWinnerRoutingOp(consumer.op) ||
-        consumer.op == ExprOp::TAKE_ALONG_AXIS || consumer.op == ExprOp::ROPE || isScanBackwardOp(consumer.op) || isScanOp(consumer.op)) {
+        consumer.op == ExprOp::TAKE_ALONG_AXIS || consumer.op == ExprOp::ROPE || isScatterRoutingOp(consumer.op) || isScanOp(consumer.op)) {
         return false;
     }
     return Expression::isBinaryOp(consumer.op) || Expression::isUnaryOp(consumer.op);
@@ -382,6 +382,18 @@ std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpressio
                     throw std::runtime_error("Segmented scan offsets do not have the ragged descriptor's batch size + 1 entries.");
                 }
                 dims[i] = dims[n.lhs];
+                break;
+            }
+            case ExprOp::SEGMENTED_REDUCE_MIN_BACKWARD:
+            case ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD: {
+                const std::vector<uint64_t>& values = dims[n.lhs];
+                if (n.aux == UINT32_MAX || values.empty() || dims[n.aux].size() != 1 || dims[n.aux][0] < 2) {
+                    throw std::runtime_error("Segmented ragged min/max backward requires values [N,D...], output [B,D...], and offsets [B+1].");
+                }
+                std::vector<uint64_t> segments = values;
+                segments[0] = dims[n.aux][0] - 1;
+                if (dims[n.rhs] != segments) throw std::runtime_error("Segmented ragged min/max backward requires values [N,D...], output [B,D...], and offsets [B+1].");
+                dims[i] = values;
                 break;
             }
             case ExprOp::SCAN_MIN_BACKWARD:
@@ -587,7 +599,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
                 graph->role[i] = Role::Materialized;
                 ensureTensor(n.lhs);
                 ensureTensor(n.rhs);
-            } else if (n.op == ExprOp::ROPE || isScanBackwardOp(n.op)) {
+            } else if (n.op == ExprOp::ROPE || isScatterRoutingOp(n.op)) {
                 graph->role[i] = Role::Materialized;
                 for (uint32_t operand : {n.lhs, n.rhs, n.aux})
                     if (operand != UINT32_MAX) ensureTensor(operand);
@@ -670,7 +682,7 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
                 sources.push_back(graph->expr.nodes[i].lhs);
             } else if (graph->expr.nodes[i].op == ExprOp::SCAN) {
                 sources.push_back(graph->expr.nodes[i].lhs);
-            } else if (graph->expr.nodes[i].op == ExprOp::ROPE || isScanBackwardOp(graph->expr.nodes[i].op)) {
+            } else if (graph->expr.nodes[i].op == ExprOp::ROPE || isScatterRoutingOp(graph->expr.nodes[i].op)) {
                 for (uint32_t operand : {graph->expr.nodes[i].lhs, graph->expr.nodes[i].rhs, graph->expr.nodes[i].aux})
                     if (operand != UINT32_MAX) sources.push_back(operand);
             } else if (isWinnerRoutingOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::TAKE_ALONG_AXIS ||
@@ -853,7 +865,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     auto runsInFusedKernel = [&](uint32_t i) {
         const ExprOp op = expr.nodes[i].op;
         return graph->role[i] == Role::Materialized && !isReductionOp(op) && !isSegmentedReduceOp(op) && op != ExprOp::SEGMENTED_BROADCAST &&
-               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && op != ExprOp::ROPE && !isScanBackwardOp(op) && !isScanOp(op) && op != ExprOp::INPUT;
+               !isWinnerRoutingOp(op) && op != ExprOp::TAKE_ALONG_AXIS && op != ExprOp::ROPE && !isScatterRoutingOp(op) && !isScanOp(op) && op != ExprOp::INPUT;
     };
     std::vector<uint32_t> levelOf = graph->level;
     if (stageFusionEnabled()) {
@@ -865,7 +877,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 sources.push_back(n.lhs);
             } else if (n.op == ExprOp::SCAN) {
                 sources = {n.lhs};
-            } else if (n.op == ExprOp::ROPE || isScanBackwardOp(n.op)) {
+            } else if (n.op == ExprOp::ROPE || isScatterRoutingOp(n.op)) {
                 for (uint32_t operand : {n.lhs, n.rhs, n.aux})
                     if (operand != UINT32_MAX) sources.push_back(operand);
             } else if (isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS || n.op == ExprOp::SEGMENTED_SCAN) {
@@ -1330,6 +1342,50 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 tensorOf[i] = scanned;
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
+                done[i] = 1;
+                continue;
+            }
+            if (isSegmentWinnerRoutingOp(n.op)) {
+                if (fusedKernelsOnly) {
+                    throw std::runtime_error(
+                        "FusedEquation::run() only supports expressions that lower to fused kernels; this expression has a reduction stage. "
+                        "Use stamp() and run the returned plan.");
+                }
+                // the row that won every (segment, column), as a flattened index into the values; then each segment's gradient added
+                // into that element of a cleared FP32 tensor (destinations are distinct, so nothing is actually summed)
+                const Tensor& values = tensorOf[n.lhs];
+                const Tensor& gradient = tensorOf[n.rhs];
+                const Tensor& offsets = tensorOf[n.aux];
+                if (!values.isDenseContiguous() || !gradient.isDenseContiguous() || !offsets.isDenseContiguous()) {
+                    throw std::runtime_error("Segmented min/max backward needs dense operands.");
+                }
+                if (values.getTotalNumElements() >= 0xffffffffull) throw std::runtime_error("Segmented min/max backward: UINT32 winners cannot address this many values.");
+                Tensor winners(gpuPlacement, TensorDescriptor(DataType::UINT32, gradient.getDimensions()));
+                const CubSegmentedArgReduction find(n.op == ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD ? CubArgReductionOp::ArgMax : CubArgReductionOp::ArgMin, DataType::UINT32);
+                StampedExecutionStage findStage;
+                findStage.kind = StampedExecutionStage::Kind::SegmentedReduction;
+                findStage.gpu_num = device_num;
+                findStage.dependency_stage_indices = dependenciesOf({n.lhs, n.aux});
+                findStage.segmented_arg_reduction = find.stampRuntimeOffsets(values, winners, offsets, stream);
+                const uint32_t findIndex = static_cast<uint32_t>(stages.size());
+                stages.push_back(std::move(findStage));
+                Tensor routed = allocateFor(i);
+                StampedExecutionStage clearStage;
+                clearStage.kind = StampedExecutionStage::Kind::FusedKernel;
+                clearStage.gpu_num = device_num;
+                clearStage.kernel = stampScatterClear(routed, device_num);
+                const uint32_t clearIndex = static_cast<uint32_t>(stages.size());
+                stages.push_back(std::move(clearStage));
+                StampedExecutionStage addStage;
+                addStage.kind = StampedExecutionStage::Kind::FusedKernel;
+                addStage.gpu_num = device_num;
+                addStage.dependency_stage_indices = dependenciesOf({n.rhs});
+                addStage.dependency_stage_indices.push_back(findIndex);
+                addStage.dependency_stage_indices.push_back(clearIndex);
+                addStage.kernel = stampScatterAdd(gradient, winners, routed, std::nullopt, device_num);
+                tensorOf[i] = routed;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(addStage));
                 done[i] = 1;
                 continue;
             }

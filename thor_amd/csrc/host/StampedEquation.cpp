@@ -202,6 +202,10 @@ void StampedExecutionStage::runOn(Stream& stream, const std::unordered_map<std::
             fused_reduction->runOn(stream, runtime_scalars);
             return;
         case Kind::SegmentedReduction:
+            if (segmented_arg_reduction) {
+                segmented_arg_reduction->runOn(stream);
+                return;
+            }
             if (!segmented_reduction) throw std::runtime_error("Segmented reduction stage is missing its stamped reduction.");
             segmented_reduction->runOn(stream);
             return;

@@ -349,6 +349,7 @@ int thor_plan_stage_description(thor_plan_t plan, int stage, char* buffer, size_
         if (s.reduction) text = s.reduction->getStamped()->getKernelVariant();
         if (s.fused_reduction) text = s.fused_reduction->getDescription();
         if (s.segmented_reduction) text = s.segmented_reduction->getStamped()->getKernelVariant();
+        if (s.segmented_arg_reduction) text = s.segmented_arg_reduction->getKernelVariant();
         if (s.segmented_broadcast) text = s.segmented_broadcast->getKernelVariant();
         if (s.scan) text = s.scan->getKernelVariant();
         copyOut(text, buffer, capacity, nullptr);)
