@@ -137,7 +137,10 @@ inline bool isScanBackwardOp(ExprOp op) {
 // lowest row among equals); every other element, and every row outside the partition, gets 0.  FP32, shaped like the values.
 inline bool isSegmentWinnerRoutingOp(ExprOp op) { return op == ExprOp::SEGMENTED_REDUCE_MIN_BACKWARD || op == ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD; }
 // Stages that read up to three dense tensors (lhs, rhs, aux) and scatter gradients into a cleared FP32 tensor.
-inline bool isScatterRoutingOp(ExprOp op) { return isScanBackwardOp(op) || isSegmentWinnerRoutingOp(op); }
+// STRIDED_VIEW_BACKWARD (AutoDiff.cpp:2100-2125 there): lhs = the FP32 gradient of a view (shaped like the view); the result has
+// the operand's shape (fill_dims), holds the gradient at the elements the view addresses (view_dims / view_strides /
+// view_element_offset) and 0 everywhere else.  Views that address an element twice are rejected.
+inline bool isScatterRoutingOp(ExprOp op) { return isScanBackwardOp(op) || isSegmentWinnerRoutingOp(op) || op == ExprOp::STRIDED_VIEW_BACKWARD; }
 inline bool isRaggedOp(ExprOp op) {
     return isSegmentedReduceOp(op) || op == ExprOp::SEGMENTED_BROADCAST || op == ExprOp::RAGGED_VALUEWISE_EXTENT;
 }

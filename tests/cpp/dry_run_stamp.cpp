@@ -229,6 +229,11 @@ static int runAll() {
         stampOne(std::string("view ") + dtypeName + " half columns", x.stridedView({4096, 12}, {24, 1}, 12).tanh() * y.stridedView({4096, 12}, {24, 1}, 0),
                  withT, stream, "FusedKernel");
         stampOne(std::string("view ") + dtypeName + " row sums of t^T", z.transpose().reduce_sum({1}), withT, stream);
+        if (dtype != DataType::FP8_E4M3) {
+            Tensor halfUpstream(gpuPlacement, TensorDescriptor(dtype, {4096, 12}));
+            stampBackward(std::string("backward ") + dtypeName + " gated halves of one input", x.stridedView({4096, 12}, {24, 1}, 12).tanh() * x.stridedView({4096, 12}, {24, 1}, 0),
+                          inputs, halfUpstream, stream);
+        }
     }
     // ragged batches: scalar and vector values, both offset dtypes, fused and index-gather paths
     for (const auto& [dtypeName, dtype] : floats) {

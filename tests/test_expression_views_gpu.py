@@ -144,3 +144,42 @@ def test_take_along_axis_validation(stream):
         run({"y": ix.take_along_axis(ii, 2)}, {"x": x, "i": copy_numpy_to_gpu(np.zeros((4, 2), np.uint32), stream, DataType.uint32)}, stream)
     with pytest.raises(ValueError, match="only axis=-1 or an explicit non-negative axis"):
         ix.take_along_axis(ii, -2)
+
+
+# ---- backward of strided views: the gradient lands on the elements the view addresses ---------------------------------------------
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16], ids=lambda d: d.name)
+def test_gradient_through_slices_of_one_input(stream, dtype):
+    rng = np.random.default_rng(41)
+    x = to_storage(rng.uniform(-1, 1, (300, 24)).astype(np.float32), dtype)
+    g = to_storage(rng.uniform(-1, 1, (300, 12)).astype(np.float32), dtype)
+    ix = ex.input("x")
+    gate, value = ix.strided_view([300, 12], [24, 1], 12), ix.strided_view([300, 12], [24, 1], 0)
+    fwd = ex.compile(gate.tanh() * value, device_num=0)
+    plan = fwd.compile_backward(["x"], error_input_name="__grad_output").stamp(
+        {"x": copy_numpy_to_gpu(x, stream, dtype), "__grad_output": copy_numpy_to_gpu(g, stream, dtype)}, stream)
+    plan.run()
+    assert sum("view_scatter" in d for d in plan.stage_descriptions()) == 2 and plan.output("x_grad").get_data_type() == dtype
+    xf, gf = from_storage(x, dtype).astype(np.float64), from_storage(g, dtype).astype(np.float64)
+    expected = np.concatenate([gf * np.tanh(xf[:, 12:]), gf * (1 - np.tanh(xf[:, 12:]) ** 2) * xf[:, :12]], axis=1)
+    tolerance = 2e-6 if dtype == DataType.fp32 else 4e-3
+    np.testing.assert_allclose(from_storage(copy_gpu_to_numpy(plan.output("x_grad"), stream), dtype), expected, rtol=tolerance, atol=tolerance)
+
+
+def test_gradient_of_permuted_and_strided_views(stream):
+    rng = np.random.default_rng(42)
+    x = rng.standard_normal((6, 10, 8)).astype(np.float32)
+    g = rng.standard_normal((8, 5, 3)).astype(np.float32)
+    # every second row of the last three planes, axes reversed: view[c, r, p] = x[3 + p, 2 r, c]
+    view = ex.input("x").strided_view([8, 5, 3], [1, 16, 80], 240)
+    plan = ex.compile(view * 2.0, device_num=0).compile_backward(["x"], error_input_name="__grad_output").stamp(
+        {"x": copy_numpy_to_gpu(x, stream, DataType.fp32), "__grad_output": copy_numpy_to_gpu(g, stream, DataType.fp32)}, stream)
+    plan.run()
+    expected = np.zeros_like(x)
+    expected[3:, ::2, :] = 2.0 * np.transpose(g, (2, 1, 0))
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("x_grad"), stream), expected)
+    # a view that reads an element twice has no gradient here, nor has a view of a view
+    tensors = {"x": copy_numpy_to_gpu(x, stream, DataType.fp32)}
+    with pytest.raises(RuntimeError, match="addresses every element once"):
+        ex.compile(ex.input("x").strided_view([4, 100], [50, 1], 0) * 2.0, device_num=0).compile_backward(["x"]).stamp(tensors, stream)
+    with pytest.raises(RuntimeError, match="operand is itself a view"):
+        ex.compile(ex.input("x").transpose().strided_view([4, 4], [8, 1], 0) * 2.0, device_num=0).compile_backward(["x"]).stamp(tensors, stream)

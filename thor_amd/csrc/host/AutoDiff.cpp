@@ -224,6 +224,18 @@ class BackwardGraph {
         n.ragged_runtime_elements_per_value = like.ragged_runtime_elements_per_value;
         return push(std::move(n), dims[values]);
     }
+    // the gradient of the strided view `like` of an operand shaped `operandDims`
+    uint32_t viewGradient(uint32_t gradient, const ExprNode& like, const Dims& operandDims) {
+        ExprNode n;
+        n.op = ExprOp::STRIDED_VIEW_BACKWARD;
+        n.lhs = gradient;
+        n.view_dims = like.view_dims;
+        n.view_strides = like.view_strides;
+        n.view_element_offset = like.view_element_offset;
+        n.fill_dims = operandDims;
+        n.output_dtype = DataType::FP32;
+        return push(std::move(n), operandDims);
+    }
     // the gradient of the per-segment min / max `like`: packed values, FP32 gradient of the segments, offsets
     uint32_t segmentWinnerGradient(uint32_t values, uint32_t gradient, uint32_t offsets, const ExprNode& like) {
         ExprNode n;
@@ -516,6 +528,12 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
                 break;
             case ExprOp::TRANSPOSE:
                 contribute(n.lhs, b.transpose(g));
+                break;
+            case ExprOp::STRIDED_VIEW:
+                // the gradient lands on the elements the view addresses, 0 elsewhere (Utilities/Expression/AutoDiff.cpp:2100-2125 there);
+                // a view of a view addresses storage that is not the operand's own index space
+                if (isStorageViewOp(forward.nodes[n.lhs].op)) throw std::runtime_error(noRule(n.op) + " The operand is itself a view.");
+                contribute(n.lhs, b.viewGradient(b.cast(g, DataType::FP32), n, fdims[n.lhs]));
                 break;
 
             case ExprOp::REDUCE_SUM:

@@ -854,7 +854,7 @@ std::string opName(ExprOp op) {
         {(uint16_t)ExprOp::LGAMMA, "lgamma"}, {(uint16_t)ExprOp::DIGAMMA, "digamma"}, {(uint16_t)ExprOp::EXP, "exp"},
         {(uint16_t)ExprOp::EXPM1, "expm1"}, {(uint16_t)ExprOp::EXP2, "exp2"}, {(uint16_t)ExprOp::EXP10, "exp10"}, {(uint16_t)ExprOp::LN, "ln"},
         {(uint16_t)ExprOp::LOG1P, "log1p"}, {(uint16_t)ExprOp::LOG2, "log2"}, {(uint16_t)ExprOp::LOG10, "log10"}, {(uint16_t)ExprOp::SQRT, "sqrt"},
-        {(uint16_t)ExprOp::TANH, "tanh"}, {(uint16_t)ExprOp::NORMCDF, "normcdf"}, {(uint16_t)ExprOp::SOFTMAX, "softmax"}, {(uint16_t)ExprOp::ROPE, "rope"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MIN_BACKWARD, "segmented_reduce_min_backward"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD, "segmented_reduce_max_backward"}, {(uint16_t)ExprOp::SCAN_MIN_BACKWARD, "scan_min_backward"}, {(uint16_t)ExprOp::SCAN_MAX_BACKWARD, "scan_max_backward"}, {(uint16_t)ExprOp::SEGMENTED_SCAN_MIN_BACKWARD, "segmented_scan_min_backward"}, {(uint16_t)ExprOp::SEGMENTED_SCAN_MAX_BACKWARD, "segmented_scan_max_backward"}, {(uint16_t)ExprOp::FILL, "fill"},
+        {(uint16_t)ExprOp::TANH, "tanh"}, {(uint16_t)ExprOp::NORMCDF, "normcdf"}, {(uint16_t)ExprOp::SOFTMAX, "softmax"}, {(uint16_t)ExprOp::ROPE, "rope"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MIN_BACKWARD, "segmented_reduce_min_backward"}, {(uint16_t)ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD, "segmented_reduce_max_backward"}, {(uint16_t)ExprOp::STRIDED_VIEW_BACKWARD, "strided_view_backward"}, {(uint16_t)ExprOp::SCAN_MIN_BACKWARD, "scan_min_backward"}, {(uint16_t)ExprOp::SCAN_MAX_BACKWARD, "scan_max_backward"}, {(uint16_t)ExprOp::SEGMENTED_SCAN_MIN_BACKWARD, "segmented_scan_min_backward"}, {(uint16_t)ExprOp::SEGMENTED_SCAN_MAX_BACKWARD, "segmented_scan_max_backward"}, {(uint16_t)ExprOp::FILL, "fill"},
         {(uint16_t)ExprOp::RESHAPE, "reshape"}, {(uint16_t)ExprOp::UNSQUEEZE, "unsqueeze"}, {(uint16_t)ExprOp::SQUEEZE, "squeeze"},
         {(uint16_t)ExprOp::MIN, "min"}, {(uint16_t)ExprOp::MAX, "max"}, {(uint16_t)ExprOp::MIN_GRAD_LEFT, "min_grad_left"},
         {(uint16_t)ExprOp::MIN_GRAD_RIGHT, "min_grad_right"}, {(uint16_t)ExprOp::MAX_GRAD_LEFT, "max_grad_left"},
@@ -938,7 +938,8 @@ std::string canonicalizeNode(const PhysicalExpression& expr, uint32_t nodeIndex,
         if (n.op == ExprOp::RESHAPE) text += ":dims=" + axesText(n.reshape_dims);
         if (n.op == ExprOp::UNSQUEEZE) text += ":axes=" + axesText(n.unsqueeze_axes);
         if (n.op == ExprOp::SQUEEZE) text += ":axes=" + axesText(n.squeeze_axes);
-        if (n.op == ExprOp::STRIDED_VIEW) {
+        if (n.op == ExprOp::STRIDED_VIEW_BACKWARD) text += ":into=" + axesText(n.fill_dims);
+        if (n.op == ExprOp::STRIDED_VIEW || n.op == ExprOp::STRIDED_VIEW_BACKWARD) {
             text += ":dims=" + axesText(n.view_dims) + ":strides=" + axesText(n.view_strides) + ":offset=" + std::to_string(n.view_element_offset);
         }
         if (isRaggedOp(n.op)) {

@@ -110,6 +110,11 @@ DataType nodeOutputDType(const ExprNode& node, const std::vector<ExprNode>& node
         }
         return node.output_dtype.value_or(resolved[node.lhs]);
     }
+    if (node.op == ExprOp::STRIDED_VIEW_BACKWARD) {
+        if (resolved[node.lhs] != DataType::FP32) throw std::runtime_error("Strided view backward requires an FP32 gradient.");
+        if (node.output_dtype.has_value() && node.output_dtype.value() != DataType::FP32) throw std::runtime_error("Strided view backward produces FP32.");
+        return DataType::FP32;
+    }
     if (isSegmentWinnerRoutingOp(node.op)) {
         if (!isSupportedFusionFloatingType(resolved[node.lhs])) throw std::runtime_error("Segmented min/max backward requires floating-point values.");
         if (resolved[node.rhs] != DataType::FP32) throw std::runtime_error("Segmented min/max backward requires an FP32 gradient.");

@@ -384,6 +384,10 @@ std::vector<std::vector<uint64_t>> inferExpressionShapes(const PhysicalExpressio
                 dims[i] = dims[n.lhs];
                 break;
             }
+            case ExprOp::STRIDED_VIEW_BACKWARD:
+                if (dims[n.lhs] != n.view_dims) throw std::runtime_error("Strided view backward requires a gradient shaped like the view.");
+                dims[i] = n.fill_dims;
+                break;
             case ExprOp::SEGMENTED_REDUCE_MIN_BACKWARD:
             case ExprOp::SEGMENTED_REDUCE_MAX_BACKWARD: {
                 const std::vector<uint64_t>& values = dims[n.lhs];
@@ -1342,6 +1346,28 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 tensorOf[i] = scanned;
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
+                done[i] = 1;
+                continue;
+            }
+            if (n.op == ExprOp::STRIDED_VIEW_BACKWARD) {
+                const Tensor& gradient = tensorOf[n.lhs];
+                if (!gradient.isDenseContiguous()) throw std::runtime_error("Strided view backward needs a dense gradient.");
+                Tensor routed = allocateFor(i);
+                StampedExecutionStage clearStage;
+                clearStage.kind = StampedExecutionStage::Kind::FusedKernel;
+                clearStage.gpu_num = device_num;
+                clearStage.kernel = stampScatterClear(routed, device_num);
+                const uint32_t clearIndex = static_cast<uint32_t>(stages.size());
+                stages.push_back(std::move(clearStage));
+                StampedExecutionStage placeStage;
+                placeStage.kind = StampedExecutionStage::Kind::FusedKernel;
+                placeStage.gpu_num = device_num;
+                placeStage.dependency_stage_indices = dependenciesOf({n.lhs});
+                placeStage.dependency_stage_indices.push_back(clearIndex);
+                placeStage.kernel = stampViewScatter(gradient, routed, n.view_dims, n.view_strides, n.view_element_offset, device_num);
+                tensorOf[i] = routed;
+                stageOfNode[i] = static_cast<int>(stages.size());
+                stages.push_back(std::move(placeStage));
                 done[i] = 1;
                 continue;
             }

@@ -13,6 +13,8 @@
 
 #include <algorithm>
 #include <sstream>
+#include <utility>
+#include <vector>
 #include <stdexcept>
 
 namespace ThorImplementation {
@@ -121,6 +123,49 @@ std::shared_ptr<StampedEquation> stampScatterAdd(const Tensor& updates, const Te
     for (size_t i = 0; i < inputs.size(); ++i) inputArgs.push_back(i);
     return std::make_shared<StampedEquation>(kernel, inputs, std::vector<Tensor>{output}, std::vector<StampedEquation::ScalarArgument>{}, inputArgs,
                                              std::vector<size_t>{inputs.size()}, inputs.size() + 1, /*passNumel=*/false, count, count > UINT32_MAX,
+                                             static_cast<uint32_t>(blocks), 256, /*flops=*/0, description.str());
+}
+
+std::shared_ptr<StampedEquation> stampViewScatter(const Tensor& gradient, const Tensor& output, const std::vector<uint64_t>& dims,
+                                                  const std::vector<uint64_t>& strides, uint64_t offset, int deviceNum) {
+    requireDense(gradient, DataType::FP32, "gradient");
+    requireDense(output, DataType::FP32, "output");
+    if (dims.size() != strides.size() || dims.empty()) throw std::runtime_error("Strided view backward needs one stride per dimension.");
+    uint64_t count = 1, last = offset;
+    std::vector<std::pair<uint64_t, uint64_t>> byStride;  // (stride, extent) of the axes that move
+    for (size_t k = 0; k < dims.size(); ++k) {
+        if (dims[k] == 0) throw std::runtime_error("Strided view backward does not support zero-sized dimensions.");
+        count *= dims[k];
+        last += (dims[k] - 1) * strides[k];
+        if (dims[k] > 1) byStride.emplace_back(strides[k], dims[k]);
+    }
+    if (gradient.getTotalNumElements() != count) throw std::runtime_error("Strided view backward requires a gradient shaped like the view.");
+    if (last >= output.getTotalNumElements()) throw std::runtime_error("Strided view backward: the view leaves the operand's storage.");
+    // no element twice: sorted by stride, every axis must step over everything the finer axes span
+    std::sort(byStride.begin(), byStride.end());
+    uint64_t span = 0;
+    for (const auto& [stride, extent] : byStride) {
+        if (stride == 0 || stride <= span) throw std::runtime_error("Strided view backward requires a view that addresses every element once.");
+        span += (extent - 1) * stride;
+    }
+    const uint64_t blocks = (count + 255) / 256;
+    if (blocks > 0x7fffffffull) throw std::runtime_error("Strided view backward: the view is too large for one launch.");
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude;
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_view_scatter(const float* __restrict__ gradient, float* __restrict__ out) {\n";
+    s << "    const thor::u64 e = (thor::u64)blockIdx.x * 256 + threadIdx.x;\n";
+    s << "    if (e >= " << count << "ull) return;\n";
+    s << "    thor::u64 rest = e, at = " << offset << "ull;\n";
+    for (size_t k = dims.size(); k-- > 0;) {
+        if (dims[k] == 1) continue;
+        s << "    at += (rest % " << dims[k] << "ull) * " << strides[k] << "ull;\n    rest /= " << dims[k] << "ull;\n";
+    }
+    s << "    out[at] = __builtin_nontemporal_load(gradient + e);\n}\n";
+    const std::shared_ptr<CompiledKernel> kernel = compileKernel(s.str(), "thor_view_scatter", deviceNum, /*fastContract=*/false);
+    std::ostringstream description;
+    description << "view_scatter(elements=" << count << ",into=" << output.getTotalNumElements() << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
+    return std::make_shared<StampedEquation>(kernel, std::vector<Tensor>{gradient}, std::vector<Tensor>{output}, std::vector<StampedEquation::ScalarArgument>{},
+                                             std::vector<size_t>{0}, std::vector<size_t>{1}, 2, /*passNumel=*/false, count, count > UINT32_MAX,
                                              static_cast<uint32_t>(blocks), 256, /*flops=*/0, description.str());
 }
 

@@ -6,6 +6,7 @@
 #include <cstdint>
 #include <memory>
 #include <optional>
+#include <vector>
 
 namespace ThorImplementation {
 
@@ -16,5 +17,10 @@ std::shared_ptr<StampedEquation> stampScatterClear(const Tensor& output, int dev
 // UINT32, same element count; output FP32.  Kernel arguments: updates, indices, [offsets], output.
 std::shared_ptr<StampedEquation> stampScatterAdd(const Tensor& updates, const Tensor& indices, const Tensor& output, const std::optional<Tensor>& offsets,
                                                  int deviceNum);
+
+// output[offset + sum(c[k] * strides[k])] = gradient[c] for every coordinate c of `dims` (gradient dense FP32 of that shape,
+// output dense FP32).  Throws when two coordinates address one element or any leaves the output.  Kernel arguments: gradient, output.
+std::shared_ptr<StampedEquation> stampViewScatter(const Tensor& gradient, const Tensor& output, const std::vector<uint64_t>& dims,
+                                                  const std::vector<uint64_t>& strides, uint64_t offset, int deviceNum);
 
 }  // namespace ThorImplementation
