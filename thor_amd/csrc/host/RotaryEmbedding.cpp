@@ -172,11 +172,13 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     // Heads between the sequence axis and a last-axis head dimension ([.., S, heads.., D]): everything at one position is one
     // contiguous run, so a block takes a few consecutive positions, leaves their sines and cosines in LDS (one per thread) and
     // streams the run, every head reading the same table.
-    const bool tiled = middleCount > 1 && innerCount == 1 && dimStride == 1 && seqAxis < dimAxis && std::getenv("THOR_ROPE_NO_TILES") == nullptr;
+    const bool tileLayout = middleCount > 1 && innerCount == 1 && dimStride == 1 && seqAxis < dimAxis && std::getenv("THOR_ROPE_NO_TILES") == nullptr;
     uint64_t tilePositions = std::max<uint64_t>(1, threads / half);
     while (tilePositions * middleCount * slots < 2 * threads && tilePositions * 2 * half <= 4096) tilePositions *= 2;
     tilePositions = std::min(tilePositions, seq);
     const uint64_t tiles = (seq + tilePositions - 1) / tilePositions;
+    const bool tileFits = tilePositions * middleCount * slots < (1ull << 31);  // the tiled kernel counts a block's items in 32 bits
+    const bool tiled = tileLayout && tileFits;
     const uint64_t blocks = tiled ? outerCount * tiles : blocksPerChunk * chunks;
     if (blocks > 0x7fffffffull) throw std::runtime_error("RoPE: the tensor is too large for one launch.");
 

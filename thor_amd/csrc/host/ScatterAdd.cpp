@@ -36,34 +36,43 @@ std::string clearSource(uint64_t outputs, int clearVec) {
 std::string addSource(uint64_t updates, uint64_t outputs, const std::string& offsetsType, uint64_t segments, uint64_t blocks) {
     std::ostringstream s;
     s << thor_embed::kDevicePrelude;
+    // x of the lane that CTRL names (a row shift or a row broadcast), 0 where there is no such lane or ROWS leaves the row out
+    s << "template <int CTRL, int ROWS>\n__device__ __forceinline__ float thor_scatter_moved(float x) {\n";
+    s << "    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROWS, 0xf, false));\n}\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scatter_add(const float* __restrict__ updates, const thor::u32* __restrict__ indices,\n";
     s << "                                                                   ";
     if (!offsetsType.empty()) s << "const " << offsetsType << "* __restrict__ offsets, ";
     s << "float* __restrict__ out) {\n";
     s << "    const int lane = threadIdx.x & 63;\n";
     if (!offsetsType.empty()) s << "    const thor::u64 first = (thor::u64)offsets[0], end = (thor::u64)offsets[" << segments << "];\n";
-    // a block walks tiles of 256 updates, every lane of it through every step (the shuffles below need whole wavefronts)
-    // (the loads of the next tile are issued before the current one is combined)
+    // A block walks tiles of 256 updates, four at a time: the loads of all four are issued before the first is combined (with one
+    // tile in flight per wavefront the kernel waits on memory latency: 150 us for 2^26 updates), and every lane of the block goes
+    // through every step, because the moves below need whole wavefronts.
     const std::string live = offsetsType.empty() ? "i < " + std::to_string(updates) + "ull" : "i < " + std::to_string(updates) + "ull && i >= first && i < end";
-    s << "    auto fetch = [&](thor::u64 tile, thor::u32& key, float& v) {\n";
-    s << "        const thor::u64 i = tile * 256 + threadIdx.x;\n";
-    s << "        key = 0xffffffffu;\n        v = 0.0f;\n";
-    s << "        if (" << live << ") {\n            key = __builtin_nontemporal_load(indices + i);\n            v = __builtin_nontemporal_load(updates + i);\n        }\n    };\n";
-    s << "    thor::u32 key, nextKey;\n    float v, nextV;\n";
-    s << "    fetch(blockIdx.x, nextKey, nextV);\n";
-    s << "    for (thor::u64 tile = blockIdx.x; tile < " << (updates + 255) / 256 << "ull; tile += " << blocks << "ull) {\n";
-    s << "    key = nextKey;\n    v = nextV;\n";
-    s << "    fetch(tile + " << blocks << "ull, nextKey, nextV);\n";
-    s << "    if (key >= " << outputs << "ull) key = 0xffffffffu;\n";
+    s << "    constexpr int DEPTH = 4;\n";
+    s << "    for (thor::u64 tile = blockIdx.x; tile < " << (updates + 255) / 256 << "ull; tile += DEPTH * " << blocks << "ull) {\n";
+    s << "        thor::u32 keys[DEPTH];\n        float values[DEPTH];\n";
+    s << "#pragma unroll\n        for (int d = 0; d < DEPTH; ++d) {\n";
+    s << "            const thor::u64 i = (tile + d * " << blocks << "ull) * 256 + threadIdx.x;\n";
+    s << "            keys[d] = 0xffffffffu;\n            values[d] = 0.0f;\n";
+    s << "            if (" << live << ") {\n                keys[d] = __builtin_nontemporal_load(indices + i);\n                values[d] = __builtin_nontemporal_load(updates + i);\n            }\n        }\n";
+    s << "#pragma unroll\n        for (int d = 0; d < DEPTH; ++d) {\n";
+    s << "            thor::u32 key = keys[d] < " << outputs << "ull ? keys[d] : 0xffffffffu;\n            float v = values[d];\n";
     // runs of equal neighbouring destinations inside the wavefront: bit l of `heads` = lane l starts a run
-    s << "    const thor::u32 before = __shfl_up(key, 1);\n";
-    s << "    const thor::u64 heads = __ballot(lane == 0 || before != key);\n";
-    s << "    const int start = 63 - __builtin_clzll(heads & (~0ull >> (63 - lane)));\n";
-    s << "#pragma unroll\n    for (int off = 1; off < 64; off <<= 1) {\n";
-    s << "        const float other = __shfl_up(v, off);\n";
-    s << "        if (lane - off >= start) v += other;\n    }\n";
-    s << "    const bool last = lane == 63 || ((heads >> (lane + 1)) & 1ull) != 0;\n";
-    s << "    if (last && key != 0xffffffffu) unsafeAtomicAdd(out + key, v);\n    }\n}\n";
+    s << "            const thor::u32 before = __shfl_up(key, 1);\n";
+    s << "            const thor::u64 heads = __ballot(lane == 0 || before != key);\n";
+    s << "            const int start = 63 - __builtin_clzll(heads & (~0ull >> (63 - lane)));\n";
+    // inclusive sums within each run, with data-parallel-primitive moves: 1, 2, 4, 8 lanes up inside rows of 16 (a lane without
+    // a source receives 0), then the last lane of row 0 / 2 into row 1 / 3, then lane 31 into the upper half; a lane takes what
+    // arrives only if its run reaches back that far
+    s << "            { const float o = thor_scatter_moved<0x111, 0xf>(v); if (lane - 1 >= start) v += o; }\n";
+    s << "            { const float o = thor_scatter_moved<0x112, 0xf>(v); if (lane - 2 >= start) v += o; }\n";
+    s << "            { const float o = thor_scatter_moved<0x114, 0xf>(v); if (lane - 4 >= start) v += o; }\n";
+    s << "            { const float o = thor_scatter_moved<0x118, 0xf>(v); if (lane - 8 >= start) v += o; }\n";
+    s << "            { const float o = thor_scatter_moved<0x142, 0xa>(v); if ((lane & 16) != 0 && start < (lane & ~15)) v += o; }\n";
+    s << "            { const float o = thor_scatter_moved<0x143, 0xc>(v); if (lane >= 32 && start < 32) v += o; }\n";
+    s << "            const bool last = lane == 63 || ((heads >> (lane + 1)) & 1ull) != 0;\n";
+    s << "            if (last && key != 0xffffffffu) unsafeAtomicAdd(out + key, v);\n        }\n    }\n}\n";
     return s.str();
 }
 
