@@ -33,7 +33,7 @@ std::string clearSource(uint64_t outputs, int clearVec) {
 }
 
 // offsetsType: empty = every update counts; else the updates outside [offsets[0], offsets[segments]) are skipped
-std::string addSource(uint64_t updates, uint64_t outputs, const std::string& offsetsType, uint64_t segments, uint64_t blocks) {
+std::string addSource(uint64_t updates, uint64_t outputs, const std::string& offsetsType, uint64_t segments, uint64_t stretch) {
     std::ostringstream s;
     s << thor_embed::kDevicePrelude;
     // x of the lane that CTRL names (a row shift or a row broadcast), 0 where there is no such lane or ROWS leaves the row out
@@ -45,15 +45,19 @@ std::string addSource(uint64_t updates, uint64_t outputs, const std::string& off
     s << "float* __restrict__ out) {\n";
     s << "    const int lane = threadIdx.x & 63;\n";
     if (!offsetsType.empty()) s << "    const thor::u64 first = (thor::u64)offsets[0], end = (thor::u64)offsets[" << segments << "];\n";
-    // A block walks tiles of 256 updates, four at a time: the loads of all four are issued before the first is combined (with one
-    // tile in flight per wavefront the kernel waits on memory latency: 150 us for 2^26 updates), and every lane of the block goes
-    // through every step, because the moves below need whole wavefronts.
+    // A wavefront owns a stretch of consecutive updates and walks it 64 at a time, the loads of four steps in flight.  The run
+    // that reaches the end of a step is not added yet: its destination and partial sum are carried into the next step (both are
+    // the same in every lane), joined with that step's first run when the destination continues, added otherwise.  A run then
+    // costs one atomic per stretch it touches, however long it is.
     const std::string live = offsetsType.empty() ? "i < " + std::to_string(updates) + "ull" : "i < " + std::to_string(updates) + "ull && i >= first && i < end";
     s << "    constexpr int DEPTH = 4;\n";
-    s << "    for (thor::u64 tile = blockIdx.x; tile < " << (updates + 255) / 256 << "ull; tile += DEPTH * " << blocks << "ull) {\n";
+    s << "    const thor::u64 wave = (thor::u64)blockIdx.x * 4 + (threadIdx.x >> 6);\n";
+    s << "    const thor::u64 base = wave * " << stretch << "ull;\n";
+    s << "    thor::u32 carriedKey = 0xffffffffu;\n    float carried = 0.0f;\n";
+    s << "    for (thor::u64 step = 0; step < " << stretch / 64 << "ull; step += DEPTH) {\n";
     s << "        thor::u32 keys[DEPTH];\n        float values[DEPTH];\n";
     s << "#pragma unroll\n        for (int d = 0; d < DEPTH; ++d) {\n";
-    s << "            const thor::u64 i = (tile + d * " << blocks << "ull) * 256 + threadIdx.x;\n";
+    s << "            const thor::u64 i = base + (step + d) * 64 + lane;\n";
     s << "            keys[d] = 0xffffffffu;\n            values[d] = 0.0f;\n";
     s << "            if (" << live << ") {\n                keys[d] = __builtin_nontemporal_load(indices + i);\n                values[d] = __builtin_nontemporal_load(updates + i);\n            }\n        }\n";
     s << "#pragma unroll\n        for (int d = 0; d < DEPTH; ++d) {\n";
@@ -71,8 +75,15 @@ std::string addSource(uint64_t updates, uint64_t outputs, const std::string& off
     s << "            { const float o = thor_scatter_moved<0x118, 0xf>(v); if (lane - 8 >= start) v += o; }\n";
     s << "            { const float o = thor_scatter_moved<0x142, 0xa>(v); if ((lane & 16) != 0 && start < (lane & ~15)) v += o; }\n";
     s << "            { const float o = thor_scatter_moved<0x143, 0xc>(v); if (lane >= 32 && start < 32) v += o; }\n";
-    s << "            const bool last = lane == 63 || ((heads >> (lane + 1)) & 1ull) != 0;\n";
-    s << "            if (last && key != 0xffffffffu) unsafeAtomicAdd(out + key, v);\n        }\n    }\n}\n";
+    // what the earlier steps carried: into this step's first run, or out to memory
+    s << "            const thor::u32 firstKey = (thor::u32)__builtin_amdgcn_readfirstlane((int)key);\n";
+    s << "            if (firstKey == carriedKey) {\n                if (start == 0) v += carried;\n";
+    s << "            } else if (carriedKey != 0xffffffffu && lane == 0) {\n                unsafeAtomicAdd(out + carriedKey, carried);\n            }\n";
+    s << "            carriedKey = (thor::u32)__builtin_amdgcn_readlane((int)key, 63);\n";
+    s << "            carried = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));\n";
+    s << "            const bool last = lane != 63 && ((heads >> (lane + 1)) & 1ull) != 0;\n";
+    s << "            if (last && key != 0xffffffffu) unsafeAtomicAdd(out + key, v);\n        }\n    }\n";
+    s << "    if (carriedKey != 0xffffffffu && lane == 0) unsafeAtomicAdd(out + carriedKey, carried);\n}\n";
     return s.str();
 }
 
@@ -112,7 +123,11 @@ std::shared_ptr<StampedEquation> stampScatterAdd(const Tensor& updates, const Te
     const uint64_t count = updates.getTotalNumElements(), outputs = output.getTotalNumElements();
     if (indices.getTotalNumElements() != count) throw std::runtime_error("Scatter-add requires one index per update.");
     if (outputs >= 0xffffffffull) throw std::runtime_error("Scatter-add: UINT32 indices cannot address an output this large.");
-    const uint64_t blocks = std::min<uint64_t>((count + 255) / 256, 8192);
+    // a wavefront's stretch: 2048 updates (a multiple of four steps of 64), shorter while that leaves fewer than 4096 blocks
+    uint64_t stretch = 2048;
+    while (stretch > 256 && (count + 4 * stretch - 1) / (4 * stretch) < 4096) stretch /= 2;
+    const uint64_t blocks = (count + 4 * stretch - 1) / (4 * stretch);
+    if (blocks > 0x7fffffffull) throw std::runtime_error("Scatter-add: too many updates for one launch.");
     std::string offsetsType;
     uint64_t segments = 0;
     if (offsets.has_value()) {
@@ -123,9 +138,9 @@ std::shared_ptr<StampedEquation> stampScatterAdd(const Tensor& updates, const Te
         offsetsType = offsets->getDataType() == DataType::UINT64 ? "thor::u64" : "thor::u32";
         segments = offsets->getTotalNumElements() - 1;
     }
-    const std::shared_ptr<CompiledKernel> kernel = compileKernel(addSource(count, outputs, offsetsType, segments, blocks), "thor_scatter_add", deviceNum, /*fastContract=*/false);
+    const std::shared_ptr<CompiledKernel> kernel = compileKernel(addSource(count, outputs, offsetsType, segments, stretch), "thor_scatter_add", deviceNum, /*fastContract=*/false);
     std::ostringstream description;
-    description << "scatter_add(updates=" << count << ",into=" << outputs << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
+    description << "scatter_add(updates=" << count << ",into=" << outputs << ",stretch=" << stretch << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
     std::vector<Tensor> inputs = {updates, indices};
     if (offsets.has_value()) inputs.push_back(*offsets);
     std::vector<size_t> inputArgs;
