@@ -6,9 +6,9 @@
 // Utilities/Expression/Expression.h:32-148 (ops), :231-371 (node), :516-1075 (API), :1077-1115 (stable activations),
 // Utilities/Expression/Expression.cpp:4176-4193,5185-5190 (activation macros).
 //
-// Operations of the reference that sit outside this path (matmul, convolution, attention, RMSNorm, RoPE, embedding, cuDNN
-// softmax, user kernels) keep their ExprOp codes so serialized graphs stay readable, but have no builder here and are
-// rejected by the compiler.
+// Operations of the reference that sit outside this path (matmul, convolution, attention, RMSNorm, embedding, cuDNN softmax,
+// user kernels) keep their ExprOp codes so serialized graphs stay readable, but have no builder here and are rejected by
+// the compiler.
 #pragma once
 
 #include "DeepLearning/Implementation/Tensor/Tensor.h"

@@ -1,4 +1,4 @@
-"""Stamps about 300 expressions and backward equations without a GPU (tests/cpp/dry_run_stamp.cpp): planning, source generation and the run-time
+"""Stamps about 380 expressions and backward equations without a GPU (tests/cpp/dry_run_stamp.cpp): planning, source generation and the run-time
 compilation for gfx950 run as they do on a GPU box, nothing is launched.  Guards against kernels that do not compile; the
 in-process compiler aborts the process on some failures, so the program's output names the case it was working on."""
 from __future__ import annotations
