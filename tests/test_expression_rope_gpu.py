@@ -96,6 +96,11 @@ LAYOUTS = [
     ((3, 5, 70, 36), {"rotary_dim": 20}),                                      # vectors narrower than 16 bytes
     ((3, 5, 70, 30), {"interleaved": True}),
     ((2, 24, 5, 33), {"sequence_axis": 3, "head_dim_axis": 1}),                # the head dimension is not the last axis
+    ((1, 1, 1, 2), {}),                                                        # one pair at position 0: the identity
+    ((2, 3, 1, 6), {"rotary_dim": 2, "position_offset": 9}),
+    ((2, 3, 5, 6), {"rotary_dim": 2, "interleaved": True}),
+    ((7, 2), {"sequence_axis": 0, "head_dim_axis": 1}),                        # rank 2
+    ((3, 4, 2, 5, 16), {"sequence_axis": 1, "head_dim_axis": 4}),              # two axes between sequence and head dimension
     ((6, 40, 16), {"sequence_axis": 1, "head_dim_axis": 2, "scaling_kind": RotaryScalingKind.llama3, "scaling_factor": 8.0,
                    "original_max_position_embeddings": 16, "base": 500000.0}),
     ((2, 4, 200, 64), {"scaling_kind": RotaryScalingKind.yarn, "scaling_factor": 4.0, "original_max_position_embeddings": 64}),
