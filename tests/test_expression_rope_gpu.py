@@ -25,7 +25,7 @@ ORACLE_KIND = {RotaryScalingKind.none: oracle.ROPE_NONE, RotaryScalingKind.linea
                RotaryScalingKind.yarn: oracle.ROPE_YARN, RotaryScalingKind.longrope: oracle.ROPE_LONGROPE, RotaryScalingKind.llama3: oracle.ROPE_LLAMA3}
 EPS32 = float(np.finfo(np.float32).eps)
 # one unit in the last place of the storage type at the magnitudes the tests use (|y| < 8)
-STORAGE_ULP = {DataType.fp32: 0.0, DataType.fp16: 2.0 ** -8, DataType.bf16: 2.0 ** -5}
+STORAGE_ULP = {DataType.fp32: 0.0, DataType.fp16: 2.0 ** -8, DataType.bf16: 2.0 ** -5, DataType.fp8_e4m3: 0.5, DataType.fp8_e5m2: 1.0}
 
 
 @pytest.fixture(scope="module")
@@ -130,6 +130,25 @@ def test_layouts_against_the_oracle(stream, shape, options, dtype):
         tail = [slice(None)] * len(shape)
         tail[options.get("head_dim_axis", 3)] = slice(rotary, None)
         assert np.array_equal(copy_gpu_to_numpy(plan.output("y"), stream)[tuple(tail)], x[tuple(tail)])
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp8_e4m3, DataType.fp8_e5m2], ids=lambda d: d.name)
+@pytest.mark.parametrize("options", [{}, {"rotary_dim": 32, "interleaved": True}, {"sequence_axis": 1, "head_dim_axis": 3}], ids=["split", "interleaved_partial", "bshd"])
+def test_fp8_storage(stream, options, dtype):
+    """8-bit floats are storage only: widened exactly, turned in fp32, rounded once on the way out."""
+    rng = np.random.default_rng(39)
+    shape = (2, 6, 50, 64)
+    x = to_storage(rng.standard_normal(shape).astype(np.float32), dtype)
+    plan = run({"y": ex.input("x").rope(**options), "wide": ex.input("x").rope(output_dtype=DataType.fp32, **options)}, {"x": copy_numpy_to_gpu(x, stream, dtype)}, stream)
+    assert plan.output("y").get_data_type() == dtype and plan.output("wide").get_data_type() == DataType.fp32
+    x32 = from_storage(x, dtype)
+    seq = shape[options.get("sequence_axis", 2)]
+    want = oracle_rope(x, dtype, options, out_dtype=DataType.fp32).astype(np.float64)
+    np.testing.assert_allclose(copy_gpu_to_numpy(plan.output("wide"), stream), want, rtol=0, atol=angle_tolerance(x32, seq, DataType.fp32))
+    got = from_storage(copy_gpu_to_numpy(plan.output("y"), stream), dtype).astype(np.float64)
+    # one rounding to the 8-bit format: within one unit in the last place of the fp32 result's magnitude
+    ulp = np.maximum(2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -9))) - (3 if dtype == DataType.fp8_e4m3 else 2)), 2.0 ** -9)
+    assert np.all(np.abs(got - want) <= ulp + 1e-3)
 
 
 @pytest.mark.parametrize("ids_dtype", [DataType.uint32, DataType.int32, DataType.uint64, DataType.fp32], ids=lambda d: d.name)
