@@ -50,6 +50,32 @@ struct Word<16> {
     typedef u32x4 type;
 };
 
+// Streaming store: written once, never read back by this kernel.  Words of 4 bytes and more are written through every
+// cache level (sc0 sc1 = system scope) with the non-temporal hint; narrower words take the compiler's non-temporal store.
+template <typename W>
+__device__ __forceinline__ void streamStore(W* p, W w) {
+    if constexpr (sizeof(W) == 16) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(w) : "memory");
+    } else if constexpr (sizeof(W) == 8) {
+        asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(w) : "memory");
+    } else if constexpr (sizeof(W) == 4) {
+        asm volatile("global_store_dword %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(w) : "memory");
+    } else {
+        __builtin_nontemporal_store(w, p);
+    }
+}
+
+// The hardware deals consecutive workgroup ids round-robin to the 8 XCDs.  With this renumbering XCD x works on blocks
+// [g*128 + x*16, g*128 + x*16 + 16) of every group g of 128 blocks: a contiguous 16-block run per XCD at any moment.  A
+// bijection on [0, gridDim.x) when gridDim.x is a multiple of 128; the identity otherwise.
+constexpr int kXcds = 8, kXcdRun = 16;
+__device__ __forceinline__ long xcdBlock() {
+    const long b = blockIdx.x;
+    if (gridDim.x % (kXcds * kXcdRun) != 0) return b;
+    const long within = b % (kXcds * kXcdRun);
+    return b - within + (within % kXcds) * kXcdRun + within / kXcds;
+}
+
 // VEC elements of T moved as whole machine words of up to 16 bytes.
 template <typename T, int VEC>
 struct alignas((sizeof(T) * VEC) >= 16 ? 16 : (sizeof(T) * VEC)) Pack {
@@ -69,7 +95,7 @@ struct alignas((sizeof(T) * VEC) >= 16 ? 16 : (sizeof(T) * VEC)) Pack {
         word_t* wp = reinterpret_cast<word_t*>(p);
         const word_t* mine = reinterpret_cast<const word_t*>(v);
 #pragma unroll
-        for (int w = 0; w < kWords; ++w) __builtin_nontemporal_store(mine[w], wp + w);
+        for (int w = 0; w < kWords; ++w) streamStore(wp + w, mine[w]);
     }
 };
 
@@ -90,7 +116,7 @@ template <typename From, typename To, int VEC, int UNROLL>
 __global__ __launch_bounds__(kBlockThreads) void convertSlots(const From* src, To* dst, long begin, long end, long firstSlot,
                                                                long lastSlot) {
     const long stride = (long)gridDim.x * kBlockThreads;
-    for (long s0 = firstSlot + (long)blockIdx.x * kBlockThreads + threadIdx.x; s0 < lastSlot; s0 += stride * UNROLL) {
+    for (long s0 = firstSlot + xcdBlock() * kBlockThreads + threadIdx.x; s0 < lastSlot; s0 += stride * UNROLL) {
         Pack<From, VEC> in[UNROLL];
         bool whole[UNROLL];
 #pragma unroll
@@ -189,6 +215,8 @@ unsigned gridFor(long work_items, int unroll) {
     const long cap = shape.blocks_per_cu > 0 ? (long)shape.compute_units * shape.blocks_per_cu : 0x7fffffffL;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
+    // whole groups of 128 blocks switch the XCD-aware numbering on; the blocks added find no slot and leave
+    if (blocks >= 1024) blocks = (blocks + 127) / 128 * 128;
     return (unsigned)blocks;
 }
 
