@@ -29,6 +29,7 @@ struct LoadedModule {
     ~LoadedModule();
     void* module = nullptr;
     int deviceNum = 0;
+    std::shared_ptr<const std::string> source;  // the compiled text, one copy for every kernel of the module
 };
 
 struct CompiledKernel {
@@ -36,7 +37,11 @@ struct CompiledKernel {
     void* function = nullptr;
     int deviceNum = 0;
     std::string kernelName;
-    std::string source;  // kept for diagnostics and tests
+    // the text the module was compiled from (diagnostics and tests)
+    const std::string& source() const {
+        static const std::string none;
+        return module && module->source ? *module->source : none;
+    }
     int numRegisters = 0;
     int staticLdsBytes = 0;
 
@@ -48,6 +53,9 @@ struct CompiledKernel {
 // keeps the compiler's default contraction (a*b+c inside one expression may fuse, matching the reference's
 // -fmad=true); false compiles with -ffp-contract=off so every operation rounds on its own.
 std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract);
+
+// The cached kernel, or null when `compileKernel` has not built it in this process (nothing is compiled or loaded).
+std::shared_ptr<CompiledKernel> findLoadedKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract);
 
 // Number of run-time compilations performed so far (cache misses); used by tests of the caching behaviour.
 uint64_t compiledKernelCount();

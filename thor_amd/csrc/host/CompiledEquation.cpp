@@ -89,15 +89,47 @@ std::string withTaggedKernelNames(const std::string& source, const std::string& 
 }
 }  // namespace
 
+namespace {
+// The caches are keyed by a 128-bit digest of (device, contraction flag, source) plus the source length, not by the source
+// text: one generated source is 30-70 KB (prelude + reduction or scan templates) and would otherwise be stored once per key.
+struct SourceDigest {
+    uint64_t a = 14695981039346656037ull, b = 0x9e3779b97f4a7c15ull;
+    void absorb(const void* data, size_t bytes) {
+        const unsigned char* p = static_cast<const unsigned char*>(data);
+        for (size_t i = 0; i < bytes; ++i) {
+            a = (a ^ p[i]) * 1099511628211ull;                       // FNV-1a
+            b = (b ^ p[i]) * 0xff51afd7ed558ccdull;                  // a second, independent multiplicative mix
+            b ^= b >> 29;
+        }
+    }
+};
+
+std::string moduleKeyOf(const std::string& source, int deviceNum, bool fastContract) {
+    SourceDigest d;
+    const int header[2] = {deviceNum, fastContract ? 1 : 0};
+    d.absorb(header, sizeof header);
+    d.absorb(source.data(), source.size());
+    char text[80];
+    std::snprintf(text, sizeof text, "%d|%d|%016llx%016llx|%zu", deviceNum, fastContract ? 1 : 0, (unsigned long long)d.a, (unsigned long long)d.b,
+                  source.size());
+    return text;
+}
+}  // namespace
+
+std::shared_ptr<CompiledKernel> findLoadedKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract) {
+    auto hit = kernelCache().get(kernelName + "|" + moduleKeyOf(source, deviceNum, fastContract));
+    return hit ? *hit : nullptr;
+}
+
 std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract) {
-    const std::string moduleKey = std::to_string(deviceNum) + (fastContract ? "|contract|" : "|off|") + source;
+    const std::string moduleKey = moduleKeyOf(source, deviceNum, fastContract);
     const std::string kernelKey = kernelName + "|" + moduleKey;
     return kernelCache().getOrCreate(kernelKey, [&] {
         ScopedGpu scoped(deviceNum);
         const std::string tag = sourceTag(source);
         const std::string taggedName = kernelName + "_" + tag;
-        const std::string taggedSource = withTaggedKernelNames(source, tag);
         std::shared_ptr<LoadedModule> loaded = moduleCache().getOrCreate(moduleKey, [&] {
+            auto taggedSource = std::make_shared<const std::string>(withTaggedKernelNames(source, tag));
             const std::string arch = archOf(deviceNum);
             // "fast" contraction would also rewrite the error-compensated sequences inside the device math library (expf drops
             // from 1 ulp to ~11 ulp), so kernels that may fuse mul+add use the compiler default (fuse within an expression,
@@ -109,15 +141,16 @@ std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const s
             std::vector<char> log(16384, 0);
             if (const char* dump = std::getenv("THOR_DUMP_KERNEL_SOURCE")) {
                 std::ofstream out(std::string(dump) + "/" + taggedName + ".hip");
-                out << taggedSource;
+                out << *taggedSource;
             }
-            const int rc = thorhip_compile(taggedSource.c_str(), (taggedName + ".hip").c_str(), arch.c_str(), options, numOptions, &code, &codeSize,
+            const int rc = thorhip_compile(taggedSource->c_str(), (taggedName + ".hip").c_str(), arch.c_str(), options, numOptions, &code, &codeSize,
                                            log.data(), log.size());
             if (rc != 0) {
                 throw std::runtime_error("Run-time compilation of kernel '" + kernelName + "' failed: " + thorhip_last_error());
             }
             auto module = std::make_shared<LoadedModule>();
             module->deviceNum = deviceNum;
+            module->source = taggedSource;
             const int loadRc = thorhip_module_load(&module->module, code, codeSize);
             (void)thorhip_code_free(code);
             hipCheck(loadRc, "thorhip_module_load");
@@ -128,7 +161,6 @@ std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const s
         kernel->module = loaded;
         kernel->deviceNum = deviceNum;
         kernel->kernelName = taggedName;
-        kernel->source = taggedSource;
         THOR_HIP_CHECK(thorhip_module_get_function(&kernel->function, loaded->module, taggedName.c_str()));
         (void)thorhip_function_get_attributes(kernel->function, &kernel->numRegisters, &kernel->staticLdsBytes, nullptr);
         return kernel;

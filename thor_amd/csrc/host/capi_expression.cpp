@@ -337,8 +337,8 @@ int thor_plan_stage_kind(thor_plan_t plan, int stage, char* buffer, size_t capac
 }
 int thor_plan_stage_source(thor_plan_t plan, int stage, char* buffer, size_t capacity, size_t* needed) {
     THOR_CAPI_TRY_INT(require(plan, "plan"); const StampedExecutionStage& s = plan->plan.stages().at(stage);
-                      copyOut(s.kernel ? s.kernel->getCompiledKernel()->source
-                                       : (s.fused_reduction ? s.fused_reduction->getLaunchPlan().mainKernel->source : std::string()),
+                      copyOut(s.kernel ? s.kernel->getCompiledKernel()->source()
+                                       : (s.fused_reduction ? s.fused_reduction->getLaunchPlan().mainKernel->source() : std::string()),
                               buffer, capacity, needed);)
 }
 int thor_plan_stage_description(thor_plan_t plan, int stage, char* buffer, size_t capacity) {
