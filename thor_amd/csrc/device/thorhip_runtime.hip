@@ -4,11 +4,13 @@
 // (Utilities/Expression/EquationCompiler.cpp:1756-1908).
 #include "thorhip.h"
 #include "thorhip_internal.h"
+#include "thorhip_static_scratch.h"
 
 #include <hip/hiprtc.h>
 
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -20,6 +22,40 @@ std::string& lastError() {
 }  // namespace thorhip
 
 using thorhip::fail;
+
+// ---- scratch memory that exists without any allocation -----------------------------------------------------------------
+// A fixed block of device memory that is part of the library's code object: every GPU the library runs on holds its own
+// copy, at its own address, from the moment the code object is loaded there until the process ends.  Entry points for
+// callers that must not allocate (work under stream capture, serving loops) use it where the ordinary entry points
+// allocate temporary storage.  In host code the array's name is only a handle for hipGetSymbolAddress; the address that
+// kernels, fills and copies use is the one looked up below, once per device, with that device current.
+static __device__ __align__(256) unsigned char scratch[THORHIP_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratchMutex;
+void* scratchAddress[kMaxDevices] = {};
+}  // namespace
+
+namespace thorhip {
+int staticScratch(void** ptr, size_t* capacity_bytes) {
+    THORHIP_REQUIRE(ptr != nullptr, "staticScratch: ptr is NULL");
+    *ptr = nullptr;
+    if (capacity_bytes) *capacity_bytes = THORHIP_STATIC_SCRATCH_BYTES;
+    int device = -1;
+    THORHIP_TRY(hipGetDevice(&device));
+    THORHIP_REQUIRE(device >= 0 && device < kMaxDevices, "staticScratch: device %d is outside the table of %d devices", device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(scratchMutex);
+    if (scratchAddress[device] == nullptr) {
+        void* address = nullptr;
+        THORHIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+        THORHIP_REQUIRE(address != nullptr, "staticScratch: hipGetSymbolAddress returned a null address on device %d", device);
+        scratchAddress[device] = address;
+    }
+    *ptr = scratchAddress[device];
+    return 0;
+}
+}  // namespace thorhip
 
 extern "C" {
 

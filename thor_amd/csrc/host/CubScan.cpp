@@ -44,7 +44,7 @@ Tensor allocateCubTemporaryStorage(const TensorPlacement& placement, size_t byte
     return Tensor(placement, TensorDescriptor(DataType::UINT8, {std::max<uint64_t>(bytes, 1)}));
 }
 
-std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r) {
+std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, bool loadedOnly, size_t tempLimitBytes) {
     if (!isCubScanDTypeSupported(r.dtype)) throw std::invalid_argument(std::string("Unsupported CUB scan dtype ") + dataTypeName(r.dtype) + ".");
     if (r.total == 0) throw std::invalid_argument("CUB scan requires at least one element.");
     if ((r.writeIndex || r.op == 1 || r.op == 2) && r.total > 0xfffffffeull) {
@@ -91,6 +91,10 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r) {
     k.headsBytes = ragged ? roundUp((r.total + 31) / 32 * 4, 256) : 0;
     k.statesBytes = k.carry ? roundUp(3 * k.chunks * 4, 256) : 0;
     k.tempBytes = std::max<size_t>(k.headsBytes + 2 * k.statesBytes, 1);
+    if (k.tempBytes > tempLimitBytes) {
+        throw std::invalid_argument("CUB scan: this request needs " + std::to_string(k.tempBytes) + " bytes of temporary storage, more than the " +
+                                    std::to_string(tempLimitBytes) + " bytes of the fixed scratch block; use the allocating scan.");
+    }
 
     const bool isUnsigned = r.dtype == DataType::UINT32;
     std::ostringstream s;
@@ -120,14 +124,23 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r) {
              "    thor::scanMarkHeads<gen::Cfg>(static_cast<const gen::Cfg::OffsetT*>(offsets), heads);\n}\n";
     }
     const std::string source = s.str();
-    k.mainKernel = compileKernel(source, "thor_scan_main", r.deviceNum, /*fastContract=*/false);
+    auto kernel = [&](const char* name) {
+        if (!loadedOnly) return compileKernel(source, name, r.deviceNum, /*fastContract=*/false);
+        std::shared_ptr<CompiledKernel> loaded = findLoadedKernel(source, name, r.deviceNum, false);
+        if (!loaded) {
+            throw std::runtime_error(std::string("CUB scan: kernel ") + name +
+                                     " of this request is not loaded yet; an ordinary scan of the same dtype, operation, sizes and alignment loads it.");
+        }
+        return loaded;
+    };
+    k.mainKernel = kernel("thor_scan_main");
     if (k.carry) {
-        k.totalsKernel = compileKernel(source, "thor_scan_totals", r.deviceNum, false);
-        k.carriesKernel = compileKernel(source, "thor_scan_carries", r.deviceNum, false);
+        k.totalsKernel = kernel("thor_scan_totals");
+        k.carriesKernel = kernel("thor_scan_carries");
     }
     if (ragged) {
-        k.clearKernel = compileKernel(source, "thor_scan_clear_heads", r.deviceNum, false);
-        k.markKernel = compileKernel(source, "thor_scan_mark_heads", r.deviceNum, false);
+        k.clearKernel = kernel("thor_scan_clear_heads");
+        k.markKernel = kernel("thor_scan_mark_heads");
     }
     std::ostringstream variant;
     variant << (ragged ? "segments" : r.row == r.total ? "flat" : "rows") << "(chunk=" << chunkElems << ",vec=" << vec << ",items=" << items << ",threads=" << threads
@@ -267,6 +280,25 @@ void run(const Plan& plan, const Tensor& temp, const Tensor& input, Tensor& outp
 }
 
 }  // namespace
+
+std::shared_ptr<const CubScanKernels> scanWithLoadedKernels(const Tensor& input, Tensor& output, const Tensor* offsets, uint64_t numItems,
+                                                            uint64_t numSegments, uint64_t segmentSize, int op, bool arg, bool inclusive, bool reverse,
+                                                            void* temp, size_t tempCapacityBytes, Stream& stream) {
+    if (op < 0 || op > 3 || (arg && op != 1 && op != 2)) throw std::invalid_argument("scan op must be 0..3 (1 or 2 for arg scans)");
+    const bool uniform = offsets == nullptr && segmentSize > 0;
+    Checked c = check(input, output, offsets, numItems, uniform ? numItems / segmentSize : numSegments, segmentSize, uniform, arg);
+    const CubScanMode mode = inclusive ? CubScanMode::Inclusive : CubScanMode::Exclusive;
+    const CubScanDirection direction = reverse ? CubScanDirection::Reverse : CubScanDirection::Forward;
+    if (arg) {
+        fill(c.request, op == 1 ? CubArgScanOp::ArgMin : CubArgScanOp::ArgMax, mode, direction);
+    } else {
+        fill(c.request, static_cast<CubScanOp>(op), mode, direction);
+    }
+    std::shared_ptr<const CubScanKernels> kernels = buildScanKernels(c.request, /*loadedOnly=*/true, tempCapacityBytes);
+    launchScan(*kernels, input.getMemPtr(), offsets ? offsets->getMemPtr() : nullptr, temp, tempCapacityBytes, arg ? nullptr : output.getMemPtr(),
+               arg ? output.getMemPtr() : nullptr, stream);
+    return kernels;
+}
 
 #define THOR_SCAN_PLAN_COMMON(plan, checked, opValue, modeValue, directionValue) \
     plan.placement = checked.placement;                                          \

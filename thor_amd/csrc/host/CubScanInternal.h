@@ -33,9 +33,20 @@ struct CubScanKernels {
     std::string variant;
 };
 
-std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& request);
+// loadedOnly: take every kernel from the process-wide cache and throw std::runtime_error when one is missing, so that nothing is
+// compiled or loaded (for callers that must not allocate).  A request whose temporary storage exceeds tempLimitBytes is rejected
+// with std::invalid_argument before any kernel is looked up.
+std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& request, bool loadedOnly = false, size_t tempLimitBytes = ~size_t(0));
 // `temp` holds at least kernels.tempBytes bytes; outValue / outIndex may be null when the request does not write them.
 void launchScan(const CubScanKernels& kernels, const void* input, const void* offsets, void* temp, size_t tempBytes, void* outValue, void* outIndex,
                 Stream& stream);
+
+// One scan (flat: offsets null and segmentSize 0; rows of segmentSize; or the numSegments segments of *offsets) that compiles, loads
+// and allocates nothing: its kernels must be in the process-wide cache already (std::runtime_error otherwise) and its temporary
+// storage is the caller's block `temp` of tempCapacityBytes (std::invalid_argument when the request needs more).  Same validation,
+// kernels and results as the plan / run entry points.
+std::shared_ptr<const CubScanKernels> scanWithLoadedKernels(const Tensor& input, Tensor& output, const Tensor* offsets, uint64_t numItems,
+                                                            uint64_t numSegments, uint64_t segmentSize, int op, bool arg, bool inclusive, bool reverse,
+                                                            void* temp, size_t tempCapacityBytes, Stream& stream);
 
 }  // namespace ThorImplementation

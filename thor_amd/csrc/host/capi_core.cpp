@@ -1,7 +1,10 @@
 // Flat C binding, part 1: errors, Stream, Tensor, TypeConverter, CubReduction, CubArgReduction.
 #include "capi_internal.h"
 
+#include "CubScanInternal.h"
 #include "ReductionPlanner.h"
+#include "../device/thorhip_static_scratch.h"
+#include "Utilities/Common/ScopedGpu.h"
 #include "Utilities/Expression/SegmentedBroadcastKernel.h"
 #include "Utilities/TensorOperations/Cub/CubDevicePrimitives.h"
 #include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
@@ -338,6 +341,23 @@ int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, 
             cubDeviceScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
             kernels = plan.kernels;
         }
+        if (variant) copyOut(cubScanKernelVariant(kernels), variant, variant_capacity, nullptr);)
+}
+
+int thor_scan_no_alloc(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments,
+                       uint64_t segment_size, int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity) {
+    THOR_CAPI_TRY_INT(
+        require(input, "input"); require(output, "output"); require(stream, "stream");
+        if (!input->tensor.isInitialized() || input->tensor.getPlacement().getMemDevice() != TensorPlacement::MemDevices::GPU) {
+            throw std::invalid_argument("CUB scan requires initialized input and output tensors on a GPU.");
+        }
+        // the scratch block of the GPU that holds the tensors: looked up with that GPU current
+        ScopedGpu scoped(static_cast<int>(input->tensor.getPlacement().getDeviceNum()));
+        void* scratch = nullptr;
+        size_t capacity = 0;
+        if (thorhip::staticScratch(&scratch, &capacity) != 0) throw std::runtime_error(thorhip_last_error());
+        const auto kernels = scanWithLoadedKernels(input->tensor, output->tensor, offsets ? &offsets->tensor : nullptr, num_items, num_segments, segment_size,
+                                                   op, arg != 0, inclusive != 0, reverse != 0, scratch, capacity, stream->stream);
         if (variant) copyOut(cubScanKernelVariant(kernels), variant, variant_capacity, nullptr);)
 }
 

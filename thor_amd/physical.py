@@ -62,6 +62,7 @@ PROTOTYPES = {
     "thor_stamped_segmented_reduction_variant": (_i, [_vp, _cp, _sz]),
     "thor_segmented_broadcast": (_i, [_vp, _vp, _vp, _i, _vp]),
     "thor_scan": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
+    "thor_scan_no_alloc": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
     "thor_reduction_generate_source": (_i, [_i, _i, _i, _i, _i, _u64p, _u64p, _i, _u32p, _i, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_arg_reduction_stamp": (_vp, [_i, _u32p, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "thor_stamped_arg_reduction_destroy": (None, [_vp]), "thor_stamped_arg_reduction_run": (_i, [_vp]),
@@ -555,17 +556,20 @@ class ScanOp(enum.IntEnum):
 
 
 def scan(input: PhysicalTensor, output: PhysicalTensor, stream: Stream, op: ScanOp = ScanOp.sum, inclusive: bool = True, reverse: bool = False,
-         segment_size: int = 0, segment_offsets: Optional[PhysicalTensor] = None, num_items: Optional[int] = None) -> str:
+         segment_size: int = 0, segment_offsets: Optional[PhysicalTensor] = None, num_items: Optional[int] = None, no_alloc: bool = False) -> str:
     """Prefix scan of ``input`` into ``output``: flat, over rows of ``segment_size`` elements, or over the segments of an offsets
     tensor; ``ScanOp.arg_min`` / ``arg_max`` write UINT32 flattened indices (cubDeviceScan / cubDeviceSegmentedUniformScan /
-    cubDeviceSegmentedScan and their arg forms, CubDevicePrimitives.h:781-880,951-1012 there).  Returns the kernel variant."""
+    cubDeviceSegmentedScan and their arg forms, CubDevicePrimitives.h:781-880,951-1012 there).  Returns the kernel variant.
+    ``no_alloc`` takes the entry point that allocates, compiles and loads nothing (temporary storage in the library's fixed
+    scratch block; the kernels of the request must have been loaded by an ordinary scan before)."""
     n = int(num_items if num_items is not None else np.prod(input.get_dimensions()))
     arg = op in (ScanOp.arg_min, ScanOp.arg_max)
     code = {ScanOp.arg_min: 1, ScanOp.arg_max: 2}.get(op, int(op))
     segments = (segment_offsets.get_dimensions()[0] - 1) if segment_offsets is not None else (n // segment_size if segment_size else 1)
     text = ctypes.create_string_buffer(512)
-    _check(lib().thor_scan(input._h, output._h, segment_offsets._h if segment_offsets is not None else None, n, segments, segment_size, code, int(arg),
-                           int(inclusive), int(reverse), stream._h, text, 512), "scan")
+    entry = lib().thor_scan_no_alloc if no_alloc else lib().thor_scan
+    _check(entry(input._h, output._h, segment_offsets._h if segment_offsets is not None else None, n, segments, segment_size, code, int(arg),
+                 int(inclusive), int(reverse), stream._h, text, 512), "scan")
     return text.value.decode()
 
 
