@@ -34,7 +34,7 @@ CARRIER = {
 
 def build(force: bool = False) -> str:
     """Compile libthor_oracle.so with gcc when missing (or when force is set)."""
-    sources = [os.path.join(_HERE, name) for name in ("thor_oracle.c", "thor_oracle_expr.c", "thor_oracle.h")]
+    sources = [os.path.join(_HERE, name) for name in ("thor_oracle.c", "thor_oracle_expr.c", "thor_oracle_scan.c", "thor_oracle.h")]
     stale = (not os.path.exists(_LIB_PATH)) or any(os.path.getmtime(_LIB_PATH) < os.path.getmtime(src) for src in sources)
     if force or stale:
         subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"], stdout=subprocess.DEVNULL)
@@ -47,8 +47,7 @@ _lib = None
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
-            build()
+        build()
         L = ctypes.CDLL(_LIB_PATH)
         L.oracle_convert.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_long, ctypes.c_int]
         L.oracle_convert.restype = ctypes.c_int
@@ -69,6 +68,7 @@ def lib() -> ctypes.CDLL:
         L.oracle_relu_scale_bias_f16.argtypes = [vp, vp, vp, vp, lg, lg, lg]
         L.oracle_channel_stats_f16.argtypes = [vp, vp, vp, lg, lg, lg]
         L.oracle_rows_f32.argtypes = [vp, vp, vp, vp, lg, lg]
+        L.oracle_scan.argtypes = [vp, ctypes.c_int, lg, vp, lg, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp]
         _lib = L
     return _lib
 
@@ -241,7 +241,7 @@ def _scan_segment_fast(x, base, integer, dtype):
 
 
 def scan(values: np.ndarray, op: int, inclusive: bool = True, reverse: bool = False, segment_size: int = 0, offsets=None, dtype: int = FP32,
-         fast: bool = True):
+         fast: bool = True, engine: str = None):
     """Sequential restatement of the reference's scans over a flat array of `dtype` carriers
     (Utilities/TensorOperations/Cub/CubScan.cu:47-93 operators, :106-196 identities; CubSegmentedScan.cu for segments).
 
@@ -250,13 +250,34 @@ def scan(values: np.ndarray, op: int, inclusive: bool = True, reverse: bool = Fa
     scans start with 0, 1, the largest / smallest value (+-inf for floats); arg scans return UINT32 flattened indices, with
     0xFFFFFFFF where the prefix is empty.  Segments: `segment_size` > 0 -> consecutive runs of that length; `offsets` -> the
     ranges [offsets[s], offsets[s + 1]); neither -> one scan.  Elements outside every segment keep 0.  `reverse` scans every
-    segment from its end.  Value scans return carriers of `dtype`.  `fast` lets NumPy's sequential accumulate routines stand in
-    for the walk where they do the same operations in the same order (the tests hold the two against each other)."""
+    segment from its end.  Value scans return carriers of `dtype`.
+
+    Three engines perform the same walk and the tests hold them against each other: "c" (thor_oracle_scan.c, the default: fast
+    enough for millions of elements in every dtype), "python" (the loop below; `fast=False` selects it) and "numpy" (NumPy's
+    sequential accumulate routines where they do the same operations in the same order, the loop elsewhere)."""
     flat = np.ascontiguousarray(values).reshape(-1)
     n = flat.size
     arg = op in (SCAN_ARGMIN, SCAN_ARGMAX)
     base = {SCAN_ARGMIN: SCAN_MIN, SCAN_ARGMAX: SCAN_MAX}.get(op, op)
     integer = dtype == UINT32
+    engine = engine or ("c" if fast else "python")
+    if engine == "c":
+        if offsets is not None:
+            pairs = [(int(offsets[s]), int(offsets[s + 1])) for s in range(len(offsets) - 1)]
+        elif segment_size:
+            pairs = [(b, b + segment_size) for b in range(0, n, segment_size)]
+        else:
+            pairs = [(0, n)]
+        table = np.ascontiguousarray(np.array(pairs, np.int64).reshape(-1))
+        carrier = np.ascontiguousarray(flat, dtype=CARRIER[dtype])
+        out_values = np.empty(n, CARRIER[dtype])
+        out_index = np.empty(n, np.uint32)
+        rc = lib().oracle_scan(carrier.ctypes.data, dtype, n, table.ctypes.data, len(pairs), base, int(bool(inclusive)), int(bool(reverse)),
+                               None if arg else out_values.ctypes.data, out_index.ctypes.data if arg else None)
+        if rc != 0:
+            raise ValueError(f"oracle_scan failed with {rc}")
+        return (out_index if arg else out_values).reshape(np.shape(values))
+    fast = engine == "numpy"
     work = flat.astype(np.uint64) if integer else to_f32(flat, dtype).astype(np.float32)
 
     def rounded(x):

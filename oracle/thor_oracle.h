@@ -100,6 +100,12 @@ int oracle_relu_scale_bias_f16(const uint16_t* x, const uint16_t* scale, const u
 int oracle_channel_stats_f16(const uint16_t* x, float* sum, float* sumsq, long n, long c, long hw);
 int oracle_rows_f32(const float* x, float* row_sum, float* row_max, uint32_t* row_argmax, long rows, long cols);
 
+/* Sequential prefix scan (thor_oracle_scan.c) of the `segments` ranges [bounds[2s], bounds[2s+1]) of a flat array of n
+ * UINT32 / FP32 / FP16 / BF16 elements.  op: 0 sum, 1 min, 2 max, 3 product.  out_values (element type) and out_index (flattened
+ * index of the running extreme; min / max only) may be NULL; elements outside every range are set to 0. */
+int oracle_scan(const void* in, int dtype, long n, const int64_t* bounds, long segments, int op, int inclusive, int reverse, void* out_values,
+                uint32_t* out_index);
+
 #ifdef __cplusplus
 }
 #endif

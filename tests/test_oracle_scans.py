@@ -76,7 +76,7 @@ def test_scan_matches_numpy_accumulate(inclusive, reverse):
 
 @pytest.mark.parametrize("dtype", [oracle.UINT32, oracle.FP32, oracle.FP16, oracle.BF16])
 @pytest.mark.parametrize("op", list(OPS.values()))
-def test_fast_paths_equal_the_element_by_element_walk(op, dtype):
+def test_the_three_engines_perform_the_same_walk(op, dtype):
     rng = np.random.default_rng(37)
     n = 700
     offsets = np.concatenate([[0], np.sort(rng.integers(0, n, 12)), [n - 5]])
@@ -88,6 +88,29 @@ def test_fast_paths_equal_the_element_by_element_walk(op, dtype):
     for inclusive in (True, False):
         for reverse in (False, True):
             for kwargs in ({"offsets": offsets}, {"segment_size": 70}, {}):
-                slow = oracle.scan(values, op, inclusive, reverse, dtype=dtype, fast=False, **kwargs)
-                quick = oracle.scan(values, op, inclusive, reverse, dtype=dtype, fast=True, **kwargs)
+                slow = oracle.scan(values, op, inclusive, reverse, dtype=dtype, engine="python", **kwargs)
+                quick = oracle.scan(values, op, inclusive, reverse, dtype=dtype, engine="numpy", **kwargs)
+                compiled = oracle.scan(values, op, inclusive, reverse, dtype=dtype, engine="c", **kwargs)
                 np.testing.assert_array_equal(slow, quick)
+                np.testing.assert_array_equal(slow, compiled)
+
+
+@pytest.mark.parametrize("dtype", [oracle.UINT32, oracle.FP32, oracle.FP16, oracle.BF16])
+def test_products_and_sixteen_bit_sums_round_at_every_step(dtype):
+    """The cases NumPy has no sequential routine for (UINT32 products, bf16 sums and products): the compiled walk against the
+    Python loop on inputs where rounding at every step shows (sums that absorb small addends, products that lose bits)."""
+    rng = np.random.default_rng(39)
+    n = 500
+    if dtype == oracle.UINT32:
+        values = rng.integers(1, 1 << 16, n).astype(np.uint32)
+    else:
+        values = oracle.from_f32(rng.uniform(0.9, 1.1, n).astype(np.float32), dtype)
+    for op in (oracle.SCAN_SUM, oracle.SCAN_PRODUCT):
+        for kwargs in ({"segment_size": 125}, {}):
+            slow = oracle.scan(values, op, True, False, dtype=dtype, engine="python", **kwargs)
+            compiled = oracle.scan(values, op, True, False, dtype=dtype, engine="c", **kwargs)
+            np.testing.assert_array_equal(slow, compiled)
+    if dtype == oracle.BF16:  # 256 + 1 is not a bf16 value: a running bf16 sum of ones stops at 256, an fp32 sum rounded once would not
+        ones = oracle.from_f32(np.ones(400, np.float32), dtype)
+        got = oracle.to_f32(oracle.scan(ones, oracle.SCAN_SUM, True, False, dtype=dtype), dtype)
+        assert got[255] == 256.0 and got[-1] == 256.0

@@ -11,7 +11,7 @@ import os
 import numpy as np
 import pytest
 
-from helpers import copy_gpu_to_numpy, copy_numpy_to_gpu, from_storage, run_staged, to_storage, ulp_distance_f32
+from helpers import from_storage, run_staged, to_storage, ulp_distance_f32
 from thor_amd import physical as ph
 from thor_amd.dtypes import DataType
 from thor_amd.physical import Expression as ex
@@ -33,7 +33,9 @@ def softmax_expr():
     return e / e.reduce_sum(axis=1)
 
 
-TOL = {DataType.fp32: (3e-6, 1e-9), DataType.fp16: (2e-3, 1e-6), DataType.bf16: (1.6e-2, 1e-6)}
+# x - rowmax promotes a 16-bit x against the fp32 maximum to fp32, so every node of the composed softmax computes in fp32 and the
+# result is fp32 whatever the input's dtype: one tolerance, what 2-ulp exp, an fp32 row sum in another order and one division allow
+FP32_RESULT_TOL = (1e-5, 1e-12)
 
 
 @pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)
@@ -51,7 +53,8 @@ def test_softmax_single_pass_matches_staged_and_closed_form(gpu, dtype, shape):
     xf = from_storage(x, dtype).astype(np.float64)
     p = np.exp(xf - xf.max(axis=1, keepdims=True))
     want = p / p.sum(axis=1, keepdims=True)
-    rtol, atol = TOL[dtype]
+    assert got.dtype == np.float32
+    rtol, atol = FP32_RESULT_TOL
     np.testing.assert_allclose(got.astype(np.float64), want, rtol=rtol, atol=atol)
     # against the staged plan: same values up to the order of the fp32 row sum (and, for 16-bit compute, one rounding step)
     np.testing.assert_allclose(got.astype(np.float64), ref.astype(np.float64), rtol=rtol, atol=atol)
@@ -195,42 +198,6 @@ def test_nan_and_inf_rows_behave_like_the_staged_plan(gpu):
     np.testing.assert_array_equal(np.isnan(outs["output"]), np.isnan(outs_s["output"]))
     ok = ~np.isnan(outs_s["output"])
     np.testing.assert_allclose(outs["output"][ok], outs_s["output"][ok], rtol=2e-6, atol=1e-30)
-
-
-def test_config4_full_size_properties(gpu):
-    """softmax over [8192, 4096] bf16 -> fp32 and normalisation over [32768, 1024] fp32 at their full sizes."""
-    rng = np.random.default_rng(1237)
-    stream = ph.Stream(0)
-    x = to_storage((rng.standard_normal((8192, 4096), dtype=np.float32) * 3), DataType.bf16)
-    eq = ex.compile(softmax_expr(), 0)
-    tx = copy_numpy_to_gpu(x, stream, DataType.bf16)
-    plan = eq.stamp({"x": tx}, stream)
-    assert plan.stage_kind_names() == ["FusedRowKernel"]
-    plan.run()
-    got = copy_gpu_to_numpy(plan.output(), stream)
-    assert got.dtype == np.float32 and got.shape == (8192, 4096)
-    xf = from_storage(x, DataType.bf16)
-    assert np.all(got >= 0) and np.all(got <= 1)
-    np.testing.assert_allclose(got.astype(np.float64).sum(axis=1), 1.0, rtol=2e-2)
-    # the maximum of every row stays its maximum (ties allowed), and a sample of rows matches the closed form
-    assert np.all(got[np.arange(8192), xf.argmax(axis=1)] == got.max(axis=1))
-    rows = rng.choice(8192, 64, replace=False)
-    s = xf[rows].astype(np.float64)
-    p = np.exp(s - s.max(axis=1, keepdims=True))
-    np.testing.assert_allclose(got[rows], p / p.sum(axis=1, keepdims=True), rtol=1.6e-2, atol=1e-7)
-
-    y = rng.standard_normal((32768, 1024), dtype=np.float32) * 4 + 1
-    iy = ex.input("y")
-    centered = iy - iy.reduce_mean(axis=1)
-    expr = centered / ((centered * centered).reduce_mean(axis=1) + 1e-5).sqrt()
-    plan, outs = run_staged(expr, {"y": y}, DataType.fp32)
-    assert plan.stage_kind_names() == ["FusedRowKernel"]
-    z = outs["output"].astype(np.float64)
-    np.testing.assert_allclose(z.mean(axis=1), 0.0, atol=2e-6)
-    np.testing.assert_allclose((z * z).mean(axis=1), 1.0, rtol=2e-5)
-    y64 = y[rows].astype(np.float64)
-    mu = y64.mean(axis=1, keepdims=True)
-    np.testing.assert_allclose(z[rows], (y64 - mu) / np.sqrt(((y64 - mu) ** 2).mean(axis=1, keepdims=True) + 1e-5), rtol=2e-5, atol=2e-6)
 
 
 # ---- Expression.softmax() / log_softmax(): the reference lowers these to a cuDNN stage (Expression.cpp:3724-3750); here they

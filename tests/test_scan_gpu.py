@@ -77,8 +77,6 @@ SHAPES = [("rows", (300, 64)), ("rows", (5, 4099)), ("rows", (3, 70000)), ("rows
 @pytest.mark.parametrize("dtype", [DataType.uint32, DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)
 @pytest.mark.parametrize("kind,shape", SHAPES, ids=[f"{k}{s}" for k, s in SHAPES])
 def test_rows_and_flat_scans(stream, kind, shape, dtype, op, inclusive, reverse):
-    if shape[0] * shape[1] > 200000 and (dtype == DataType.bf16 or (op == ScanOp.product and dtype == DataType.uint32)):
-        pytest.skip("the oracle walks these element by element: large cases run for the dtypes NumPy can accumulate")
     rng = np.random.default_rng(41)
     n = shape[0] * shape[1]
     if dtype == DataType.uint32:
