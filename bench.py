@@ -104,7 +104,6 @@ def bench_other_configs():
     from thor_amd.physical import Expression as ex
     from thor_amd.runtime import Event
 
-    import oracle
     stream = ph.Stream(0)
     results = {}
 
@@ -112,10 +111,12 @@ def bench_other_configs():
         handle = stream.handle
 
     def gpu_from(values, dtype):
-        carrier = values if dtype == DataType.fp32 else oracle.convert(np.ascontiguousarray(values, dtype=np.float32), oracle.FP32, int(dtype))
-        shape = list(carrier.shape)
-        cpu = ph.PhysicalTensor(ph.Placement(ph.DeviceType.cpu), ph.PhysicalTensor.Descriptor(dtype, shape))
-        cpu.numpy()[...] = carrier
+        """fp32 host values -> a device tensor of `dtype`: the copy converts on the GPU (Tensor::copyFromAsync), so the GPU legs of the
+        bench need nothing but the product library."""
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        shape = list(values.shape)
+        cpu = ph.PhysicalTensor(ph.Placement(ph.DeviceType.cpu), ph.PhysicalTensor.Descriptor(DataType.fp32, shape))
+        cpu.numpy()[...] = values
         gpu = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(dtype, shape))
         gpu.copy_from_async(cpu, stream)
         stream.synchronize()
@@ -360,8 +361,72 @@ def bench_other_configs():
     return results
 
 
+def _short(name, width=70):
+    import re
+    name = re.sub(r"\(anonymous namespace\)::", "", name)
+    name = re.sub(r"^void ", "", name)
+    return name if len(name) <= width else name[:width]
+
+
+def _bench_lines_by_kernel_tag(bench_json):
+    """kernel-name tag (the 8 hex digits every generated kernel carries) -> the bench lines whose plan names it."""
+    import re
+    if not bench_json:
+        return {}
+    record = json.loads(open(bench_json).read().strip().splitlines()[-1])
+    tags = {}
+    for line, v in record.get("other_configs", {}).items():
+        for tag in re.findall(r"\[[a-z_]+_([0-9a-f]{8})\]", v.get("plan", "")):
+            tags.setdefault(tag, []).append(line)
+    return tags
+
+
+def _line_of(kernel_name, tags):
+    for tag, lines in tags.items():
+        if tag in kernel_name:
+            return ",".join(sorted(set(lines)))
+    return ""
+
+
+def summarize_kernel_trace(db, bench_json=None):
+    """Per-kernel dispatch durations out of the rocpd database a `rocprofv3 --kernel-trace --stats` run of this script wrote."""
+    import sqlite3
+    con = sqlite3.connect(db)
+    tags = _bench_lines_by_kernel_tag(bench_json)
+    rows = list(con.execute("select name, count(*), avg(end-start), min(end-start), max(end-start), sum(end-start) from kernels group by name order by 6 desc"))
+    total = sum(r[5] for r in rows) or 1
+    print(f"{'calls':>6} {'avg_us':>10} {'min_us':>10} {'max_us':>10} {'total_ms':>10} {'pct':>6}  {'kernel':70s} bench line")
+    for name, calls, avg, lo, hi, tot in rows:
+        print(f"{calls:6d} {avg/1e3:10.2f} {lo/1e3:10.2f} {hi/1e3:10.2f} {tot/1e6:10.3f} {100*tot/total:6.2f}  {_short(name):70s} {_line_of(name, tags)}")
+
+
+def summarize_hbm_traffic(fetch_db, write_db, bench_json=None):
+    """HBM bytes per dispatch out of two `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE) of this script with --calibration-copy:
+    each counter is scaled by its own reading for the calibration copy (uint32 -> int32 over 2^28 elements: 1 GiB each way)."""
+    import sqlite3
+    tags = _bench_lines_by_kernel_tag(bench_json)
+
+    def read(db, counter):
+        con = sqlite3.connect(db)
+        return {n: (c, a) for n, c, a in con.execute(
+            "select kernel_name, count(*), avg(value) from counters_collection where counter_name=? group by kernel_name", (counter,))}
+    fetch, write = read(fetch_db, "FETCH_SIZE"), read(write_db, "WRITE_SIZE")
+    calibration = [n for n in fetch if "convertSlots<unsigned int, int" in n][0]
+    kf, kw = 1048576.0 / fetch[calibration][1], 1048576.0 / write[calibration][1]
+    print(f"calibration copy {_short(calibration, 48)}: FETCH_SIZE {fetch[calibration][1]:.1f} KiB, WRITE_SIZE {write[calibration][1]:.1f} KiB "
+          f"per dispatch for 1 048 576 KiB each way -> factors {kf:.5f}, {kw:.5f}")
+    print(f"{'dispatches':>10} {'fetch MiB':>10} {'write MiB':>10} {'total MB':>10}  kernel <- bench line")
+    for name in sorted(fetch, key=lambda n: -(fetch[n][1] * kf + write.get(n, (0, 0))[1] * kw)):
+        fm, wm = fetch[name][1] * kf / 1024, write.get(name, (0, 0))[1] * kw / 1024
+        print(f"{fetch[name][0]:10d} {fm:10.2f} {wm:10.2f} {(fm + wm) * 1.048576:10.2f}  {_short(name)} <- {_line_of(name, tags)}")
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--summarize-kernel-trace", nargs="+", metavar=("DB", "BENCH_JSON"),
+                    help="print the per-kernel duration table of a rocprofv3 --kernel-trace database (optionally tagged with the bench lines of BENCH_JSON) and exit")
+    ap.add_argument("--summarize-hbm-traffic", nargs="+", metavar=("FETCH_DB", "WRITE_DB"),
+                    help="print the HBM-traffic table of two rocprofv3 --pmc databases (FETCH_SIZE run, WRITE_SIZE run[, BENCH_JSON]) and exit")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -372,6 +437,12 @@ def main():
                     help="before the timed region, launch a plain copy kernel of known size (uint32->int32 over the same element count: "
                          "4 B read + 4 B written per element) so that hardware counters of a profiled run can be scaled against it")
     args = ap.parse_args()
+    if args.summarize_kernel_trace:
+        summarize_kernel_trace(*args.summarize_kernel_trace[:2])
+        return
+    if args.summarize_hbm_traffic:
+        summarize_hbm_traffic(*args.summarize_hbm_traffic[:3])
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
@@ -454,6 +525,9 @@ def main():
         b_.free()
     if not args.no_other_configs:
         result["other_configs"] = bench_other_configs()
+        # the fraction of the HBM peak every secondary line reached, next to the headline kernel's (kept compact: drivers keep the parsed line)
+        result["roofline"]["per_config"] = {"c2_convert_fp32_to_fp16": round(achieved / HBM_PEAK_GBPS, 4),
+                                            **{name: round(v["GB/s"] / HBM_PEAK_GBPS, 4) for name, v in result["other_configs"].items()}}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
         if not args.no_other_configs:

@@ -12,6 +12,7 @@
 #pragma once
 
 #include "DeepLearning/Implementation/Tensor/Tensor.h"
+#include "Utilities/Common/Stream.h"
 
 #include <cstdint>
 #include <initializer_list>
@@ -100,8 +101,12 @@ struct RotaryPositionEmbeddingOptions {
     std::vector<double> long_rope_short_factors;
     std::vector<double> long_rope_long_factors;
     std::optional<DataType> output_dtype = std::nullopt;
+    // The arithmetic dtype: FP32 (the default) is the only one the rotation kernels have; anything else is refused with
+    // std::invalid_argument when the node is built.
     std::optional<DataType> compute_dtype = std::nullopt;
-    // Accepted for source compatibility; the rotation always writes a tensor of its own here.
+    // A permission, not a request (the reference's planner MAY rotate a private producer's output in place when it is set;
+    // its default is off because out of place benchmarked faster).  This build never uses the permission: the rotation
+    // always writes a tensor of its own, which is one of the behaviours the flag allows.
     bool allow_in_place_materialization = false;
 };
 
@@ -257,6 +262,11 @@ class Expression {
    public:
     Expression(double value);  // implicit on purpose: `x + 2.0`
 
+    // One of a small pool of helper streams of `gpu_num`, handed out in turn (reference: Expression.h:518, Expression.cpp:48-55).
+    // Stamped plans run their independent branches on them.  The pool holds as many streams as a process has hardware queues
+    // (4): more streams would share queues and overlap nothing more.  Streams are created on first use, at default priority.
+    static Stream& getNextHelperStream(uint32_t gpu_num);
+
     static Expression input(const std::string& name, std::optional<DataType> compute_dtype = std::nullopt,
                             std::optional<DataType> output_dtype = std::nullopt);
     static Expression runtimeScalar(const std::string& name, std::optional<DataType> compute_dtype = std::nullopt,
@@ -408,6 +418,10 @@ class Expression {
     // address the storage of the tensor the operand resolves to, not the logical index space of an earlier view.  Nothing is
     // copied; kernels read through the strides.
     Expression stridedView(const std::vector<uint64_t>& dims, const std::vector<uint64_t>& strides_elements, uint64_t element_offset = 0) const;
+    // The gradient of stridedView(view_dims, view_strides_elements, view_element_offset) of a tensor shaped source_dims: this
+    // expression is the FP32 gradient of the view; the result is FP32, shaped source_dims, zero where the view does not reach.
+    Expression stridedViewBackward(const std::vector<uint64_t>& source_dims, const std::vector<uint64_t>& view_dims,
+                                   const std::vector<uint64_t>& view_strides_elements, uint64_t view_element_offset = 0) const;
     Expression aliasView(const std::vector<uint64_t>& dims, const std::vector<uint64_t>& strides_elements, uint64_t element_offset = 0) const {
         return stridedView(dims, strides_elements, element_offset);
     }
@@ -418,6 +432,11 @@ class Expression {
     // FP32 and keep their dtype; arg scans return UINT32 (Expression.h:640-700, Expression.cpp:3866-3960 there).
     Expression scan(ScanOp op = ScanOp::Sum, int64_t axis = -1, bool inclusive = true) const;
     static Expression scan(const Expression& input, ScanOp op, int64_t axis = -1, bool inclusive = true) { return input.scan(op, axis, inclusive); }
+    Expression exclusiveScanSum(int64_t axis = -1) const { return scan(ScanOp::Sum, axis, false); }
+    Expression inclusiveScanSum(int64_t axis = -1) const { return scan(ScanOp::Sum, axis, true); }
+    static Expression exclusiveScanSum(const Expression& input, int64_t axis = -1) { return input.scan(ScanOp::Sum, axis, false); }
+    static Expression inclusiveScanSum(const Expression& input, int64_t axis = -1) { return input.scan(ScanOp::Sum, axis, true); }
+    static Expression prefixCount(const Expression& mask, bool inclusive = true, int64_t axis = -1) { return mask.prefixCount(inclusive, axis); }
     Expression reverseScan(ScanOp op, int64_t axis = -1, bool inclusive = true) const;
     Expression prefixCount(bool inclusive = true, int64_t axis = -1) const;  // running count of non-zero elements, UINT32
     std::pair<Expression, Expression> scanWithIndices(ScanOp op, int64_t axis = -1, bool inclusive = true) const;  // {values, indices}, Min / Max
@@ -499,6 +518,9 @@ class Expression {
     Expression withDTypes(std::optional<DataType> compute_dtype = std::nullopt, std::optional<DataType> output_dtype = std::nullopt) const;
     Expression withComputeDType(DataType compute_dtype) const { return withDTypes(compute_dtype, std::nullopt); }
     Expression withOutputDType(DataType output_dtype) const { return withDTypes(std::nullopt, output_dtype); }
+
+    // This expression with every use of the tensor input `input_name` reading `replacement` instead.
+    Expression substituteInput(const std::string& input_name, const Expression& replacement) const;
 
     static bool isLeafOp(ExprOp op);
     static bool isUnaryOp(ExprOp op);

@@ -28,12 +28,18 @@ class FusedEquation {
     // Binds tensors and returns a plan whose run() only launches.  Outputs are allocated here unless the caller passes
     // them in `preallocated_outputs` (shape and dtype are validated).
     // `tensor_scalar_inputs` binds the equation's tensorRuntimeScalar inputs to elements of device buffers.
+    // `requestedOutputShapes` (reference: FusedEquation.h:594-599, FusedEquation.cpp:3152-3174): the dimensions the caller wants an
+    // output tensor to carry.  They must be the dimensions the expression gives it up to axes of extent 1 (a row-reduction's
+    // [N, 1] asked for as [N]); anything else throws "Output tensor dimensions are incompatible with the fused equation
+    // result."  A preallocated output of that name is checked against the request and keeps its own dimensions.
     [[nodiscard]] StampedExecutionPlan stamp(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
                                              const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs = {},
-                                             const std::unordered_map<std::string, Tensor>& preallocated_outputs = {}) const;
+                                             const std::unordered_map<std::string, Tensor>& preallocated_outputs = {},
+                                             const std::unordered_map<std::string, std::vector<uint64_t>>& requestedOutputShapes = {}) const;
     [[nodiscard]] StampedExecutionPlan stampSingleOutput(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
                                                          const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs = {},
-                                                         const std::optional<Tensor>& preallocated_output = {}) const;
+                                                         const std::optional<Tensor>& preallocated_output = {},
+                                                         const std::vector<uint64_t>& requestedOutputShape = {}) const;
 
     // Convenience: bind, launch into caller-provided outputs.  Restricted, as in the reference, to expressions that
     // lower to fused kernels only (no reduction stage) -- use stamp() otherwise.
@@ -85,7 +91,8 @@ class FusedEquation {
     std::shared_ptr<PlannedGraph> plannedGraphFor(const std::vector<DataType>& root_dtypes) const;
     std::vector<DataType> rootDTypes(const std::unordered_map<std::string, Tensor>& inputs) const;
     StampedExecutionPlan stampImpl(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
-                                   const std::unordered_map<std::string, Tensor>& preallocated_outputs, bool fusedKernelsOnly) const;
+                                   const std::unordered_map<std::string, Tensor>& preallocated_outputs, bool fusedKernelsOnly,
+                                   const std::unordered_map<std::string, std::vector<uint64_t>>& requestedOutputShapes = {}) const;
 
     struct BackwardRecipe;  // a backward equation before shapes are known: the forward graph and what to differentiate
     FusedEquation(std::shared_ptr<BackwardRecipe> recipe, int device_num);

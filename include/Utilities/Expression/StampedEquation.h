@@ -157,7 +157,10 @@ class StampedScan {
 };
 
 struct StampedExecutionStage {
-    enum class Kind { FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction, SegmentedReduction, SegmentedBroadcast, ReduceMinMaxBackward, Scan };
+    enum class Kind {
+        FusedKernel, Reduction, ArgMinMax, FusedRowKernel, Copy, FusedReduction, SegmentedReduction, SegmentedBroadcast, ReduceMinMaxBackward, Scan,
+        DependencyBarrier,  // launches nothing: a node of the dependency graph only (scheduler tests; reference StampedEquation.h:1461)
+    };
     static std::string kindToString(Kind kind) {
         switch (kind) {
             case Kind::FusedKernel:
@@ -180,8 +183,17 @@ struct StampedExecutionStage {
                 return "ReduceMinMaxBackward";
             case Kind::Scan:
                 return "Scan";
+            case Kind::DependencyBarrier:
+                return "DependencyBarrier";
         }
         return "<unknown>";
+    }
+    static StampedExecutionStage dependencyBarrier(uint32_t gpu_num, std::vector<uint32_t> dependency_stage_indices) {
+        StampedExecutionStage stage;
+        stage.kind = Kind::DependencyBarrier;
+        stage.gpu_num = gpu_num;
+        stage.dependency_stage_indices = std::move(dependency_stage_indices);
+        return stage;
     }
 
     Kind kind = Kind::FusedKernel;
@@ -202,10 +214,31 @@ struct StampedExecutionStage {
     void runOn(Stream& stream, const std::unordered_map<std::string, float>& runtime_scalars) const;
 };
 
+namespace detail {
+
+// Where every stage of a plan runs (reference: StampedEquation.h:1637-1646, StampedEquation.cpp:3958-4047).  Lane 0 is the
+// caller's stream; every other lane is a helper stream, so stages on different lanes may overlap.  A chain never leaves its
+// lane: at a fork the first dependent stage continues on the producer's lane and the others open lanes of their own; a stage
+// inherits the lane of a producer it continues (the caller's lane when it continues several).  A stage whose result is
+// needed on another lane records a completion event; helper lanes that start from nothing wait for the caller-ready event.
+struct StampedExecutionSchedule {
+    std::vector<uint32_t> stage_lane_indices;
+    std::vector<uint32_t> lane_gpu_nums;
+    std::vector<bool> stage_has_downstream_dependency;
+    std::vector<bool> stage_needs_completion_event;
+    bool needs_caller_ready_event = false;
+};
+
+// Throws std::runtime_error when a stage depends on itself or on a later stage.
+StampedExecutionSchedule buildStampedExecutionSchedule(const std::vector<StampedExecutionStage>& steps, uint32_t caller_gpu_num);
+
+}  // namespace detail
+
 class StampedExecutionPlan {
    public:
-    StampedExecutionPlan(std::vector<StampedExecutionStage> steps, std::unordered_map<std::string, Tensor> final_outputs, const Stream& stream)
-        : steps(std::move(steps)), final_outputs(std::move(final_outputs)), stream(stream) {}
+    // Builds the schedule and, when it has helper lanes, takes their streams from Expression's helper-stream pool and creates the
+    // events the joins need: run() itself creates nothing.
+    StampedExecutionPlan(std::vector<StampedExecutionStage> steps, std::unordered_map<std::string, Tensor> final_outputs, const Stream& stream);
 
     void run();
     void run(const std::unordered_map<std::string, float>& runtime_scalars);
@@ -221,15 +254,27 @@ class StampedExecutionPlan {
     std::vector<std::vector<uint32_t>> stageDependencyIndices() const;
     std::vector<CubReductionPath> reductionPaths() const;
     const std::vector<StampedExecutionStage>& stages() const { return steps; }
+    const detail::StampedExecutionSchedule& schedule() const { return execution_schedule; }
 
     Tensor output(const std::string& name) const;
     Tensor output() const;
     const std::unordered_map<std::string, Tensor>& getFinalOutputs() const { return final_outputs; }
 
    private:
+    struct LaneResources {
+        std::vector<Stream> helpers;            // lanes 1 .. of the schedule
+        Event caller_ready;                     // set when the schedule needs it
+        std::vector<Event> stage_completion;    // one slot per stage; initialised where the schedule asks for an event
+    };
+    static LaneResources makeLaneResources(const detail::StampedExecutionSchedule& schedule);
+    void runForked(Stream& run_stream, const detail::StampedExecutionSchedule& schedule, const LaneResources& lanes,
+                   const std::unordered_map<std::string, float>& runtime_scalars) const;
+
     std::vector<StampedExecutionStage> steps;
     std::unordered_map<std::string, Tensor> final_outputs;
     Stream stream;
+    detail::StampedExecutionSchedule execution_schedule;
+    LaneResources lane_resources;
 };
 
 }  // namespace ThorImplementation

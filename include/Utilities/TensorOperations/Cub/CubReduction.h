@@ -213,7 +213,8 @@ struct ReductionLaunchPlan {
     uint32_t prepareGridX = 1, prepareThreads = 256;
     uint32_t mainGridX = 1, mainGridY = 1, mainThreads = 256;
     uint32_t finishGridX = 1, finishThreads = 256;
-    size_t workspaceBytes = 0;  // per-block / per-share partials
+    size_t workspaceBytes = 0;  // per-block / per-share partials, then the ticket words
+    size_t ticketOffset = 0, ticketBytes = 0;  // part of the workspace that must be zero before the first run (0 bytes: none)
     std::string variant;        // human-readable description of the chosen kernel shape
 };
 

@@ -11,7 +11,7 @@
  *   - softmax / normalisation are the composed stage plans       test/Utilities/Expression/CommonInputFusionTest.cpp:281-327
  * Pinning: tests/test_oracle_expressions.py checks every function against numpy float64 closed forms (fp32 results within
  * 2 ulp of the correctly rounded value for elementwise work, 1e-5 relative for sums) and the fp16 paths bit for bit against
- * numpy float16 arithmetic.  Accumulation here is sequential per row / per channel share.
+ * numpy float16 arithmetic.  Row sums of configs 4a / 4b add by halving, the others one after the other.
  */
 #include "thor_oracle.h"
 
@@ -23,6 +23,19 @@ static float sigmoid_f32(float d) {
     const float a = expf(-fmaxf(-d, 0.0f));
     const float b = 1.0f + expf(-fabsf(d));
     return a / b;
+}
+
+/* fp32 sum of v[0..n) (of the squares when `squares` is set) by halving: the reference's reductions are library tree
+ * reductions whose order is not specified (CubReductionOperation.cuh:2908-2956), so any fp32 order is a restatement; this
+ * one keeps the rounding error at log2(n) ulps, where adding 4096 terms one after the other drifts by up to ~1e-5 relative. */
+static float pairwise_sum(const float* v, long n, int squares) {
+    if (n <= 8) {
+        float s = 0.0f;
+        for (long j = 0; j < n; ++j) s += squares ? v[j] * v[j] : v[j];
+        return s;
+    }
+    const long half = n / 2;
+    return pairwise_sum(v, half, squares) + pairwise_sum(v + half, n - half, squares);
 }
 
 /* config 1: out = (a*b + c) * sigmoid(d), fp32 */
@@ -47,12 +60,8 @@ int oracle_softmax_rows_bf16(const uint16_t* x, float* out, long rows, long cols
             const float v = oracle_bf16_bits_to_f32(xr[j]);
             m = (v != v || m != m) ? NAN : fmaxf(m, v);
         }
-        float sum = 0.0f;
-        for (long j = 0; j < cols; ++j) {
-            const float e = expf(oracle_bf16_bits_to_f32(xr[j]) - m);
-            yr[j] = e;
-            sum += e;
-        }
+        for (long j = 0; j < cols; ++j) yr[j] = expf(oracle_bf16_bits_to_f32(xr[j]) - m);
+        const float sum = pairwise_sum(yr, cols, 0);
         for (long j = 0; j < cols; ++j) yr[j] = yr[j] / sum;
     }
     return omp_get_max_threads();
@@ -64,15 +73,9 @@ int oracle_normalize_rows_f32(const float* x, float* out, long rows, long cols, 
     for (long r = 0; r < rows; ++r) {
         const float* xr = x + r * cols;
         float* yr = out + r * cols;
-        float sum = 0.0f;
-        for (long j = 0; j < cols; ++j) sum += xr[j];
-        const float mean = sum / (float)cols;
-        float sq = 0.0f;
-        for (long j = 0; j < cols; ++j) {
-            const float c = xr[j] - mean;
-            yr[j] = c;
-            sq += c * c;
-        }
+        const float mean = pairwise_sum(xr, cols, 0) / (float)cols;
+        for (long j = 0; j < cols; ++j) yr[j] = xr[j] - mean;
+        const float sq = pairwise_sum(yr, cols, 1);
         const float denom = sqrtf(sq / (float)cols + eps);
         for (long j = 0; j < cols; ++j) yr[j] = yr[j] / denom;
     }

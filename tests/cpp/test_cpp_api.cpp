@@ -795,6 +795,192 @@ static void softmaxPlansAndRowKernel(Stream& stream) {
     CHECK(throwsAs<std::invalid_argument>([&] { (void)ix.softmax(SoftmaxAlgorithm::Log); }));
 }
 
+// ---- smaller entry points of the boundary (Expression.h:664,683-684,711-714,1010 and FusedEquation.h:594-599 there) ---------------
+static void boundaryShorthandsAndSubstitution() {
+    Expression x = Expression::input("x");
+    const PhysicalExpression inclusive = x.inclusiveScanSum().expression(), exclusive = Expression::exclusiveScanSum(x, 1).expression();
+    CHECK(inclusive.nodes.back().op == ExprOp::SCAN && inclusive.nodes.back().scan_op == ScanOp::Sum && inclusive.nodes.back().scan_mode == ScanMode::Inclusive);
+    CHECK(exclusive.nodes.back().op == ExprOp::SCAN && exclusive.nodes.back().scan_mode == ScanMode::Exclusive && exclusive.nodes.back().scan_axis == 1);
+    CHECK(Expression::prefixCount(x, false).expression().nodes.back().op == ExprOp::SCAN);
+    // substituteInput: every use of b reads exp(d) instead; b disappears from the inputs, d appears
+    Expression a = Expression::input("a"), b = Expression::input("b"), c = Expression::input("c"), d = Expression::input("d");
+    Expression composed = ((a * b + c) * b).substituteInput("b", d.exp());
+    CHECK((composed.getInputNames() == std::set<std::string>{"a", "c", "d"}));
+    Expression untouched = (a + c).substituteInput("b", d);
+    CHECK((untouched.getInputNames() == std::set<std::string>{"a", "c"}));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)a.substituteInput("", d); }));
+    // stridedViewBackward: validation of the reference, node carries the view and the source shape
+    Expression g = Expression::input("g");
+    const PhysicalExpression routed = g.stridedViewBackward({4, 6}, {2, 3}, {6, 1}, 7).expression();
+    CHECK(routed.nodes.back().op == ExprOp::STRIDED_VIEW_BACKWARD && (routed.nodes.back().fill_dims == std::vector<uint64_t>{4, 6}));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)g.stridedViewBackward({}, {2, 3}, {6, 1}); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)g.stridedViewBackward({4, 6}, {2, 3}, {6}); }));
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)g.stridedViewBackward({4, 6}, {2, 3}, {1, 1}); }));  // overlapping rows
+    // RoPE options that this build does not implement are refused, not ignored
+    RotaryPositionEmbeddingOptions options;
+    options.compute_dtype = DataType::BF16;
+    CHECK(throwsAs<std::invalid_argument>([&] { (void)x.rotaryPositionEmbedding(options); }));
+    options.compute_dtype = DataType::FP32;
+    options.allow_in_place_materialization = true;  // a permission: accepted
+    (void)x.rotaryPositionEmbedding(options);
+}
+
+static void boundaryRequestedShapesAndSubstitutionExecution(Stream& stream) {
+    const uint64_t rows = 6, cols = 50;
+    std::vector<float> xs(rows * cols), ds(rows * cols);
+    for (size_t i = 0; i < xs.size(); ++i) {
+        xs[i] = float(int(i % 9) - 4);
+        ds[i] = 0.01f * float(int(i % 7));
+    }
+    Tensor tx = gpuFrom(xs, {rows, cols}, stream), td = gpuFrom(ds, {rows, cols}, stream);
+    Expression x = Expression::input("x");
+    FusedEquation rowSum = FusedEquation::compile(x.reduce_sum({1}).expression(), 0);
+    StampedExecutionPlan plain = rowSum.stamp({{"x", tx}}, stream);
+    CHECK((plain.output().getDimensions() == std::vector<uint64_t>{rows, 1}));
+    StampedExecutionPlan flat = rowSum.stamp({{"x", tx}}, stream, {}, {}, {{"output", {rows}}});
+    CHECK((flat.output().getDimensions() == std::vector<uint64_t>{rows}));
+    flat.run();
+    const std::vector<float> sums = toHostF32(flat.output(), stream);
+    for (uint64_t r = 0; r < rows; ++r) {
+        double want = 0;
+        for (uint64_t c = 0; c < cols; ++c) want += xs[r * cols + c];
+        CHECK(sums[r] == float(want));
+    }
+    StampedExecutionPlan single = rowSum.stampSingleOutput({{"x", tx}}, stream, {}, std::nullopt, {1, rows, 1});
+    CHECK((single.output().getDimensions() == std::vector<uint64_t>{1, rows, 1}));
+    CHECK(throwsAs<std::runtime_error>([&] { (void)rowSum.stamp({{"x", tx}}, stream, {}, {}, {{"output", {rows + 1}}}); }));
+    CHECK(throwsAs<std::runtime_error>([&] { (void)rowSum.stamp({{"x", tx}}, stream, {}, {}, {{"nonesuch", {rows}}}); }));
+    Tensor own(gpuPlacement, TensorDescriptor(DataType::FP32, {rows, 1}));
+    StampedExecutionPlan kept = rowSum.stamp({{"x", tx}}, stream, {}, {{"output", own}}, {{"output", {rows}}});
+    CHECK((kept.output().getDimensions() == std::vector<uint64_t>{rows, 1}));  // the caller's tensor keeps its dimensions
+
+    // substituteInput runs like the expression written out by hand
+    Expression b = Expression::input("b"), d = Expression::input("d");
+    FusedEquation viaSubstitution = FusedEquation::compile(((x * b + 1.0) * b).substituteInput("b", d.exp()).expression(), 0);
+    FusedEquation byHand = FusedEquation::compile(((x * d.exp() + 1.0) * d.exp()).expression(), 0);
+    StampedExecutionPlan p1 = viaSubstitution.stamp({{"x", tx}, {"d", td}}, stream), p2 = byHand.stamp({{"x", tx}, {"d", td}}, stream);
+    p1.run();
+    p2.run();
+    CHECK(toHostF32(p1.output(), stream) == toHostF32(p2.output(), stream));
+
+    // stridedViewBackward places a gradient shaped like the view into zeros shaped like the source
+    std::vector<float> gs = {1, 2, 3, 4, 5, 6};
+    Tensor tg = gpuFrom(gs, {2, 3}, stream);
+    FusedEquation place = FusedEquation::compile(Expression::input("g").stridedViewBackward({4, 6}, {2, 3}, {6, 1}, 7).expression(), 0);
+    StampedExecutionPlan placed = place.stamp({{"g", tg}}, stream);
+    placed.run();
+    const std::vector<float> routed = toHostF32(placed.output(), stream);
+    CHECK(routed.size() == 24);
+    for (size_t i = 0; i < routed.size(); ++i) {
+        float want = 0;
+        for (int r = 0; r < 2; ++r)
+            for (int c = 0; c < 3; ++c)
+                if (i == size_t(7 + 6 * r + c)) want = gs[r * 3 + c];
+        CHECK(routed[i] == want);
+    }
+}
+
+// ---- stage scheduling: lanes, forks and joins (test/Utilities/Expression/StampedExecutionPlanSchedulerTest.cpp:18-89 there) ----------
+static StampedExecutionStage barrierStage(std::vector<uint32_t> dependencies = {}, uint32_t gpu = 0) {
+    return StampedExecutionStage::dependencyBarrier(gpu, std::move(dependencies));
+}
+
+static void stagePlanScheduler() {
+    typedef std::vector<uint32_t> U;
+    typedef std::vector<bool> B;
+    {  // a linear chain stays on the caller's lane: no events at all
+        std::vector<StampedExecutionStage> stages = {barrierStage(), barrierStage({0}), barrierStage({1}), barrierStage({2})};
+        const detail::StampedExecutionSchedule s = detail::buildStampedExecutionSchedule(stages, 0);
+        CHECK((s.stage_lane_indices == U{0, 0, 0, 0}));
+        CHECK((s.lane_gpu_nums == U{0}));
+        CHECK(!s.needs_caller_ready_event);
+        CHECK((s.stage_needs_completion_event == B{false, false, false, false}));
+    }
+    {  // a fork opens one helper lane, the join comes back to the caller's lane
+        std::vector<StampedExecutionStage> stages = {barrierStage(), barrierStage({0}), barrierStage({0}), barrierStage({1, 2}), barrierStage({3})};
+        const detail::StampedExecutionSchedule s = detail::buildStampedExecutionSchedule(stages, 0);
+        CHECK((s.stage_lane_indices == U{0, 0, 1, 0, 0}));
+        CHECK((s.lane_gpu_nums == U{0, 0}));
+        CHECK(!s.needs_caller_ready_event);
+        CHECK((s.stage_needs_completion_event == B{true, false, true, false, false}));
+    }
+    {  // two independent roots: the helper root waits for the caller-ready event, one event joins it back
+        std::vector<StampedExecutionStage> stages = {barrierStage(), barrierStage(), barrierStage({0, 1}), barrierStage({2})};
+        const detail::StampedExecutionSchedule s = detail::buildStampedExecutionSchedule(stages, 0);
+        CHECK((s.stage_lane_indices == U{0, 1, 0, 0}));
+        CHECK((s.lane_gpu_nums == U{0, 0}));
+        CHECK(s.needs_caller_ready_event);
+        CHECK((s.stage_needs_completion_event == B{false, true, false, false}));
+    }
+    {  // nested forks: only parallel branches get lanes
+        std::vector<StampedExecutionStage> stages = {barrierStage(),    barrierStage({0}), barrierStage({0}),    barrierStage({1}),
+                                                     barrierStage({1}), barrierStage({2}), barrierStage({3, 4}), barrierStage({5, 6})};
+        const detail::StampedExecutionSchedule s = detail::buildStampedExecutionSchedule(stages, 0);
+        CHECK((s.stage_lane_indices == U{0, 0, 1, 0, 2, 1, 0, 0}));
+        CHECK((s.lane_gpu_nums == U{0, 0, 0}));
+    }
+    {  // a helper branch that nothing consumes still gets an event: the run joins it at the end
+        std::vector<StampedExecutionStage> stages = {barrierStage(), barrierStage({0}), barrierStage({0})};
+        const detail::StampedExecutionSchedule s = detail::buildStampedExecutionSchedule(stages, 0);
+        CHECK((s.stage_lane_indices == U{0, 0, 1}));
+        CHECK((s.stage_needs_completion_event == B{true, false, true}));
+    }
+    {  // dependencies must point backwards
+        std::vector<StampedExecutionStage> stages = {barrierStage({1}), barrierStage()};
+        CHECK(throwsAs<std::runtime_error>([&] { (void)detail::buildStampedExecutionSchedule(stages, 0); }));
+    }
+}
+
+static void stagePlanForksAndJoins(Stream& stream) {
+    // barrier-only plan, submitted many times without synchronising in between: events are reused from run to run
+    {
+        std::vector<StampedExecutionStage> stages = {barrierStage(), barrierStage({0}), barrierStage({0}), barrierStage({1, 2})};
+        StampedExecutionPlan plan(std::move(stages), {}, stream);
+        CHECK(plan.schedule().lane_gpu_nums.size() == 2);
+        for (int run = 0; run < 64; ++run) plan.run();
+        stream.synchronize();
+    }
+    // two independent reductions of different inputs, then arithmetic on both: the branches run on two lanes and the result is the
+    // staged one, run after run, with the inputs rewritten on the caller's stream between runs (the helper lane must wait for them)
+    // (rows of different lengths, so that the two reductions cannot share one pass)
+    const uint64_t rows = 300, cols = 1000, colsB = 500;
+    std::vector<float> a(rows * cols), b(rows * colsB);
+    for (size_t i = 0; i < a.size(); ++i) a[i] = float(int(i % 17) - 8);
+    for (size_t i = 0; i < b.size(); ++i) b[i] = float(int(i % 13) - 6);
+    Tensor ta = gpuFrom(a, {rows, cols}, stream), tb = gpuFrom(b, {rows, colsB}, stream);
+    Expression ia = Expression::input("a"), ib = Expression::input("b");
+    Expression combined = ia.reduce_sum({1}) * 2.0 + ib.reduce_max({1});
+    FusedEquation eq = FusedEquation::compile(combined.expression(), 0);
+    StampedExecutionPlan plan = eq.stamp({{"a", ta}, {"b", tb}}, stream);
+    const detail::StampedExecutionSchedule& schedule = plan.schedule();
+    CHECK(schedule.lane_gpu_nums.size() == 2);
+    CHECK(schedule.needs_caller_ready_event);
+    auto expect = [&](const std::vector<float>& av, const std::vector<float>& bv) {
+        const std::vector<float> got = toHostF32(plan.output(), stream);
+        for (uint64_t r = 0; r < rows; ++r) {
+            double sum = 0, top = -1e30;
+            for (uint64_t c = 0; c < cols; ++c) sum += av[r * cols + c];
+            for (uint64_t c = 0; c < colsB; ++c) top = std::max<double>(top, bv[r * colsB + c]);
+            CHECK(got[r] == float(sum * 2.0 + top));  // small integers: exact in any order
+        }
+    };
+    plan.run();
+    expect(a, b);
+    Tensor hostB(cpuPlacement, TensorDescriptor(DataType::FP32, {rows, colsB}));
+    for (int round = 1; round <= 3; ++round) {
+        for (size_t i = 0; i < b.size(); ++i) b[i] = float(int((i + round) % 11) - 5);
+        std::memcpy(hostB.getMemPtr<float>(), b.data(), b.size() * sizeof(float));
+        tb.copyFromAsync(hostB, stream);  // queued on the caller's stream; the helper lane's reduction of b must see it
+        plan.run();
+        expect(a, b);
+    }
+    // the same plan on one lane gives the same values
+    setenv("THOR_DISABLE_STAGE_OVERLAP", "1", 1);
+    plan.run();
+    unsetenv("THOR_DISABLE_STAGE_OVERLAP");
+    expect(a, b);
+}
+
 static void typeConverterOnGpuAndTensorViews(Stream& stream) {
     const uint64_t n = 100003;
     std::vector<float> x(n);
@@ -834,7 +1020,9 @@ int main(int argc, char** argv) {
                                {"raggedExpressionStructure", raggedExpressionStructure},
                                {"autodiffGraphStructure", autodiffGraphStructure},
                                {"scanExpressionStructure", scanExpressionStructure},
-                               {"ropeExpressionStructure", ropeExpressionStructure}};
+                               {"ropeExpressionStructure", ropeExpressionStructure},
+                               {"stagePlanScheduler", stagePlanScheduler},
+                               {"boundaryShorthandsAndSubstitution", boundaryShorthandsAndSubstitution}};
     if (mode == "gpu") {
         auto withStream = [](void (*f)(Stream&)) {
             return [f] {
@@ -851,6 +1039,8 @@ int main(int argc, char** argv) {
         cases.push_back({"autodiffExecution", withStream(autodiffExecution)});
         cases.push_back({"devicePrefixScans", withStream(devicePrefixScans)});
         cases.push_back({"ropeExecution", withStream(ropeExecution)});
+        cases.push_back({"stagePlanForksAndJoins", withStream(stagePlanForksAndJoins)});
+        cases.push_back({"boundaryRequestedShapesAndSubstitutionExecution", withStream(boundaryRequestedShapesAndSubstitutionExecution)});
         cases.push_back({"typeConverterOnGpuAndTensorViews", withStream(typeConverterOnGpuAndTensorViews)});
     }
     for (const Case& c : cases) {

@@ -207,3 +207,29 @@ def test_every_fp32_bit_pattern_narrows_to_bf16_like_the_oracle(gpu):
         assert bad.size == 0, f"chunk {chunk}: {bad.size} mismatches, first input {int(bits[bad[0]]):#010x}: got {got[bad[0]]:#x} want {want[bad[0]]:#x}"
     src.free()
     dst.free()
+
+
+@pytest.mark.parametrize("n", [3500, 1 << 20, (1 << 24) + 5])
+def test_a_kernel_that_follows_sees_the_converted_values(gpu, n):
+    """Chains of launches without host synchronisation in between: a buffer that kernels have read is overwritten by a conversion
+    and read again by the next launch; every reader must see the newest values (no line of the older contents may survive in
+    any cache the streaming stores pass by)."""
+    from thor_amd.runtime import DeviceBuffer, Stream, TypeConverter
+    stream = Stream(0)
+    first, second = c2_like(n, 11), c2_like(n, 12)
+    a, b = DeviceBuffer.from_numpy(first, stream), DeviceBuffer.from_numpy(second, stream)
+    half, back, again = DeviceBuffer(n * 2), DeviceBuffer(n * 4), DeviceBuffer(n * 2)
+    for _ in range(3):
+        TypeConverter.convert_type(a.ptr, half.ptr, DataType.fp32, DataType.fp16, n, stream)      # half <- first
+        TypeConverter.convert_type(half.ptr, back.ptr, DataType.fp16, DataType.fp32, n, stream)   # readers pull half's lines in
+        TypeConverter.convert_type(back.ptr, again.ptr, DataType.fp32, DataType.fp16, n, stream)  # and back's
+        TypeConverter.convert_type(b.ptr, half.ptr, DataType.fp32, DataType.fp16, n, stream)      # half <- second, no sync before
+        TypeConverter.convert_type(half.ptr, back.ptr, DataType.fp16, DataType.fp32, n, stream)   # must read the second contents
+        TypeConverter.convert_type(back.ptr, again.ptr, DataType.fp32, DataType.fp16, n, stream)
+        got_back = back.download(np.float32, n, stream)
+        got_again = again.download(np.float16, n, stream)
+        want_half = oracle.convert(second, oracle.FP32, oracle.FP16)
+        assert_same_bits(got_back, oracle.convert(want_half, oracle.FP16, oracle.FP32), DataType.fp32)
+        assert_same_bits(got_again, want_half, DataType.fp16)
+    for buf in (a, b, half, back, again):
+        buf.free()

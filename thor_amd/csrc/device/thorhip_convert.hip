@@ -52,10 +52,12 @@ struct Word<16> {
 
 // Streaming store: written once, never read back by this kernel.  Words of 4 bytes and more are written through every
 // cache level (sc0 sc1 = system scope) with the non-temporal hint; narrower words take the compiler's non-temporal store.
+// The compiler's hazard checks do not look inside inline assembly: a store of more than 8 bytes still reads its data
+// registers for two cycles after it issues, hence the two wait states (s_nop 1) behind the 16-byte form.
 template <typename W>
 __device__ __forceinline__ void streamStore(W* p, W w) {
     if constexpr (sizeof(W) == 16) {
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(w) : "memory");
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" : : "v"(p), "v"(w) : "memory");
     } else if constexpr (sizeof(W) == 8) {
         asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(w) : "memory");
     } else if constexpr (sizeof(W) == 4) {

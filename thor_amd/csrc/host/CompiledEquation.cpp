@@ -121,7 +121,9 @@ std::shared_ptr<CompiledKernel> findLoadedKernel(const std::string& source, cons
     return hit ? *hit : nullptr;
 }
 
-std::shared_ptr<CompiledKernel> compileKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract) {
+std::shared_ptr<CompiledKernel> compileKernel(const std::string& plainSource, const std::string& kernelName, int deviceNum, bool fastContract) {
+    // diagnostic switch: the compiler's non-temporal stores instead of the write-through ones
+    const std::string source = std::getenv("THOR_PLAIN_STREAM_STORES") ? "#define THOR_PLAIN_STREAM_STORES 1\n" + plainSource : plainSource;
     const std::string moduleKey = moduleKeyOf(source, deviceNum, fastContract);
     const std::string kernelKey = kernelName + "|" + moduleKey;
     return kernelCache().getOrCreate(kernelKey, [&] {

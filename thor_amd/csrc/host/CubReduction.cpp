@@ -263,10 +263,7 @@ std::shared_ptr<StampedCubReduction> CubReduction::stamp(const Tensor& input, co
 
     ScopedGpu scoped(stream.getGpuNum());
     ReductionLaunchPlan plan = buildReductionKernels(request);
-    std::optional<Tensor> workspace;
-    if (plan.workspaceBytes > 0) {
-        workspace = Tensor(input.getPlacement(), TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
-    }
+    std::optional<Tensor> workspace = allocateReductionWorkspace(plan, input.getPlacement(), stream);
     return std::shared_ptr<StampedCubReduction>(
         new StampedCubReduction(op, geometry, input, output, std::move(plan), std::move(workspace), output_scale, stream));
 }
@@ -370,10 +367,7 @@ std::shared_ptr<StampedCubArgReduction> CubArgReduction::stamp(const Tensor& inp
 
     ScopedGpu scoped(stream.getGpuNum());
     ReductionLaunchPlan plan = buildReductionKernels(request);
-    std::optional<Tensor> workspace;
-    if (plan.workspaceBytes > 0) {
-        workspace = Tensor(input.getPlacement(), TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
-    }
+    std::optional<Tensor> workspace = allocateReductionWorkspace(plan, input.getPlacement(), stream);
     return std::shared_ptr<StampedCubArgReduction>(
         new StampedCubArgReduction(op, geometry, input, std::move(value), std::move(index), std::move(plan), std::move(workspace), stream));
 }

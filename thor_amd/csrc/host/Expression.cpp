@@ -4,6 +4,9 @@
 #include "Utilities/Expression/Expression.h"
 
 #include <algorithm>
+#include <array>
+#include <atomic>
+#include <mutex>
 #include <cmath>
 #include <cstdio>
 #include <functional>
@@ -13,6 +16,32 @@
 #include <unordered_set>
 
 namespace ThorImplementation {
+
+namespace {
+struct HelperStreams {
+    static constexpr uint32_t kPerGpu = 4;
+    std::array<Stream, kPerGpu> streams;
+    std::atomic<uint32_t> next{0};
+};
+}  // namespace
+
+Stream& Expression::getNextHelperStream(uint32_t gpu_num) {
+    static std::mutex mutex;
+    // never destroyed: at process exit the device runtime may be gone before static destructors run
+    static std::vector<std::unique_ptr<HelperStreams>>& pools = *new std::vector<std::unique_ptr<HelperStreams>>();
+    HelperStreams* pool = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(mutex);
+        if (pools.size() <= gpu_num) pools.resize(gpu_num + 1);
+        if (!pools[gpu_num]) {
+            pools[gpu_num] = std::make_unique<HelperStreams>();
+            for (Stream& s : pools[gpu_num]->streams) s = Stream(static_cast<int>(gpu_num));
+        }
+        pool = pools[gpu_num].get();
+    }
+    return pool->streams[pool->next.fetch_add(1, std::memory_order_relaxed) % HelperStreams::kPerGpu];
+}
+
 
 uint32_t PhysicalExpression::getOrCreateInputSlot(const std::string& name, NamedInput::Kind kind) {
     for (const NamedInput& in : inputs) {
@@ -50,9 +79,11 @@ class GraphMerger {
         for (const NamedInput& in : dst.inputs) slotByName[in.name] = in.slot;
     }
 
-    uint32_t absorb(const PhysicalExpression& src, uint32_t root) {
+    // `replacedInput` (may be null): tensor inputs of that name are not copied; their consumers read node `replacement` of dst instead
+    uint32_t absorb(const PhysicalExpression& src, uint32_t root, const std::string* replacedInput = nullptr, uint32_t replacement = UINT32_MAX) {
         if (root >= src.nodes.size()) throw std::runtime_error("Expression node index is out of range.");
-        std::unordered_map<uint32_t, uint32_t>& memo = memos[&src];
+        std::unordered_map<uint32_t, uint32_t> substitutionMemo;
+        std::unordered_map<uint32_t, uint32_t>& memo = replacedInput ? substitutionMemo : memos[&src];
         // children precede parents, so an ascending sweep over the reachable set needs no recursion
         std::vector<char> needed(root + 1, 0);
         needed[root] = 1;
@@ -68,6 +99,10 @@ class GraphMerger {
         for (uint32_t i = 0; i <= root; ++i) {
             if (!needed[i] || memo.count(i)) continue;
             ExprNode copy = src.nodes[i];
+            if (replacedInput && copy.op == ExprOp::INPUT && copy.input_slot < src.inputs.size() && src.inputs[copy.input_slot].name == *replacedInput) {
+                memo[i] = replacement;
+                continue;
+            }
             if (copy.lhs != UINT32_MAX) copy.lhs = memo.at(copy.lhs);
             if (copy.rhs != UINT32_MAX) copy.rhs = memo.at(copy.rhs);
             if (copy.aux != UINT32_MAX) copy.aux = memo.at(copy.aux);
@@ -508,6 +543,62 @@ Expression Expression::stridedView(const std::vector<uint64_t>& dims, const std:
     return out;
 }
 
+// The gradient of a strided view as an expression of its own (reference: Expression.cpp:3789-3835 there): `this` is the gradient,
+// shaped like the view; the result is FP32, shaped like the viewed tensor, zero where the view does not reach.
+Expression Expression::stridedViewBackward(const std::vector<uint64_t>& source_dims, const std::vector<uint64_t>& view_dims,
+                                           const std::vector<uint64_t>& view_strides_elements, uint64_t view_element_offset) const {
+    if (!expr) throw std::runtime_error("Cannot create a strided-view backward from an empty expression");
+    if (source_dims.empty()) throw std::invalid_argument("Expression::stridedViewBackward requires non-empty source dimensions.");
+    if (view_dims.empty() || view_dims.size() != view_strides_elements.size()) {
+        throw std::invalid_argument("Expression::stridedViewBackward requires view dimensions and strides with the same non-zero rank.");
+    }
+    uint64_t denseTail = 1;
+    for (size_t axis = view_dims.size(); axis-- > 0;) {
+        if (view_dims[axis] == 0 || view_dims[axis] == std::numeric_limits<uint64_t>::max() || view_strides_elements[axis] < denseTail) {
+            throw std::invalid_argument("Expression::stridedViewBackward requires canonical non-overlapping row-major-like strides.");
+        }
+        if (denseTail > std::numeric_limits<uint64_t>::max() / view_dims[axis]) {
+            throw std::overflow_error("Expression::stridedViewBackward view element count overflows uint64_t.");
+        }
+        denseTail *= view_dims[axis];
+    }
+    uint64_t sourceElements = 1;
+    for (uint64_t d : source_dims) {
+        if (d == 0 || d == std::numeric_limits<uint64_t>::max()) {
+            throw std::invalid_argument("Expression::stridedViewBackward requires concrete non-zero source dimensions.");
+        }
+        if (sourceElements > std::numeric_limits<uint64_t>::max() / d) throw std::overflow_error("Expression::stridedViewBackward source element count overflows uint64_t.");
+        sourceElements *= d;
+    }
+    uint64_t last = view_element_offset;
+    for (size_t axis = 0; axis < view_dims.size(); ++axis) last += (view_dims[axis] - 1) * view_strides_elements[axis];
+    if (last >= sourceElements) throw std::invalid_argument("Expression::stridedViewBackward view reaches past the source tensor.");
+    Expression out = unaryOp(*this, ExprOp::STRIDED_VIEW_BACKWARD);
+    ExprNode& node = out.expr->nodes[out.nodeIndex];
+    node.view_dims = view_dims;
+    node.view_strides = view_strides_elements;
+    node.view_element_offset = view_element_offset;
+    node.fill_dims = source_dims;
+    node.output_dtype = DataType::FP32;
+    return out;
+}
+
+// Every use of the tensor input `input_name` reads `replacement` instead (reference: Expression.cpp:3173-3198 there).  The result's
+// inputs are those of the replacement and the remaining ones of this expression, merged by name.
+Expression Expression::substituteInput(const std::string& input_name, const Expression& replacement) const {
+    if (input_name.empty()) throw std::invalid_argument("Expression::substituteInput requires a non-empty input name.");
+    if (!expr) throw std::runtime_error("Expression::substituteInput called on an expression with no underlying graph.");
+    if (!replacement.expr) throw std::runtime_error("Expression::substituteInput replacement has no underlying graph.");
+    if (replacement.nodeIndex >= replacement.expr->nodes.size()) throw std::runtime_error("Expression::substituteInput replacement node index is out of range.");
+    if (nodeIndex >= expr->nodes.size()) throw std::runtime_error("Expression::substituteInput source node index is out of range.");
+    auto out = std::make_shared<PhysicalExpression>();
+    GraphMerger merger(*out);
+    const uint32_t replacementRoot = merger.absorb(*replacement.expr, replacement.nodeIndex);
+    const uint32_t root = merger.absorb(*expr, nodeIndex, &input_name, replacementRoot);
+    out->output_node = root;
+    return Expression(out, root);
+}
+
 // ---- scans -----------------------------------------------------------------------------------------------------------------
 namespace {
 void validateScanOp(ScanOp op, const char* api) {
@@ -585,6 +676,10 @@ Expression Expression::takeAlongAxis(const Expression& indices, int64_t axis) co
 // ---- rotary position embedding (Expression.cpp:4334-4507 there) -----------------------------------------------------------
 namespace {
 ExprNode ropeNodeFrom(const RotaryPositionEmbeddingOptions& options) {
+    if (options.compute_dtype.has_value() && options.compute_dtype.value() != DataType::FP32) {
+        // the rotation kernels work in FP32 whatever the storage dtype; another arithmetic dtype is refused rather than ignored
+        throw std::invalid_argument(std::string("RoPE rotates in FP32: compute_dtype ") + dataTypeName(options.compute_dtype.value()) + " is not supported.");
+    }
     if (options.base <= 0.0) throw std::runtime_error("RoPE base must be positive.");
     if (options.scaling_factor <= 0.0) throw std::runtime_error("RoPE scaling factor must be positive.");
     if (options.attention_factor.has_value() && options.attention_factor.value() <= 0.0) throw std::runtime_error("RoPE attention_factor must be positive.");

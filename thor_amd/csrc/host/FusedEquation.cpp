@@ -754,27 +754,44 @@ std::unordered_map<std::string, Tensor> FusedEquation::withTensorScalars(const s
 
 StampedExecutionPlan FusedEquation::stamp(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
                                           const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs,
-                                          const std::unordered_map<std::string, Tensor>& preallocated_outputs) const {
-    return stampImpl(withTensorScalars(inputs, tensor_scalar_inputs), stream, preallocated_outputs, false);
+                                          const std::unordered_map<std::string, Tensor>& preallocated_outputs,
+                                          const std::unordered_map<std::string, std::vector<uint64_t>>& requestedOutputShapes) const {
+    return stampImpl(withTensorScalars(inputs, tensor_scalar_inputs), stream, preallocated_outputs, false, requestedOutputShapes);
 }
 
 StampedExecutionPlan FusedEquation::stampSingleOutput(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
                                                       const std::unordered_map<std::string, TensorScalarBinding>& tensor_scalar_inputs,
-                                                      const std::optional<Tensor>& preallocated_output) const {
+                                                      const std::optional<Tensor>& preallocated_output,
+                                                      const std::vector<uint64_t>& requestedOutputShape) const {
     if (outputs_template.outputs.size() != 1) throw std::runtime_error("stampSingleOutput requires an equation with exactly one output.");
     std::unordered_map<std::string, Tensor> pre;
     if (preallocated_output.has_value()) pre.emplace(outputs_template.outputs[0].name, preallocated_output.value());
-    return stampImpl(withTensorScalars(inputs, tensor_scalar_inputs), stream, pre, false);
+    std::unordered_map<std::string, std::vector<uint64_t>> requested;
+    if (!requestedOutputShape.empty()) requested.emplace(outputs_template.outputs[0].name, requestedOutputShape);
+    return stampImpl(withTensorScalars(inputs, tensor_scalar_inputs), stream, pre, false, requested);
 }
 
+namespace {
+// equal once axes of extent 1 are dropped (reference: outputDimensionsMatchIgnoringSingletons, FusedEquation.cpp:3170-3174)
+bool sameDimensionsIgnoringSingletons(const std::vector<uint64_t>& a, const std::vector<uint64_t>& b) {
+    std::vector<uint64_t> x, y;
+    for (uint64_t d : a)
+        if (d != 1) x.push_back(d);
+    for (uint64_t d : b)
+        if (d != 1) y.push_back(d);
+    return x == y;
+}
+}  // namespace
+
 StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::string, Tensor>& inputs, const Stream& stream,
-                                              const std::unordered_map<std::string, Tensor>& preallocated, bool fusedKernelsOnly) const {
+                                              const std::unordered_map<std::string, Tensor>& preallocated, bool fusedKernelsOnly,
+                                              const std::unordered_map<std::string, std::vector<uint64_t>>& requestedOutputShapes) const {
     if (!stream.isInitialized()) throw std::runtime_error("FusedEquation::stamp requires an initialized stream.");
     if (stream.getGpuNum() != device_num) throw std::runtime_error("FusedEquation::stamp: the stream belongs to another GPU than the equation.");
     if (backward) {
         std::unordered_map<std::string, Tensor> used;
         const std::shared_ptr<const FusedEquation> equation = backwardFor(inputs, used);
-        return equation->stampImpl(used, stream, preallocated, fusedKernelsOnly);
+        return equation->stampImpl(used, stream, preallocated, fusedKernelsOnly, requestedOutputShapes);
     }
     const std::vector<DataType> dtypes = rootDTypes(inputs);
     const std::shared_ptr<PlannedGraph> graph = plannedGraphFor(dtypes);
@@ -941,7 +958,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
     const bool stageFusion = stageFusionEnabled() && !fusedKernelsOnly;
     std::vector<uint8_t> roles(graph->role.size());
     for (size_t i = 0; i < roles.size(); ++i) roles[i] = static_cast<uint8_t>(graph->role[i]);
-    RowFusionContext context{expr, graph->outputs, root_inputs, roles, dims, tensorOf, done, stages, stageOfNode, allocateFor, device_num};
+    RowFusionContext context{expr, graph->outputs, root_inputs, roles, dims, tensorOf, done, stages, stageOfNode, allocateFor, device_num, stream};
     if (stageFusion) {
         // Recognise chains of last-axis reductions and row-wise elementwise work over one [rows, R] input and emit them
         // as one kernel that keeps each row in registers.
@@ -1211,8 +1228,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
         request.inputDType = inputs.front().getDataType();
 
         ReductionLaunchPlan plan = buildReductionKernels(request);
-        std::optional<Tensor> workspace;
-        if (plan.workspaceBytes > 0) workspace = Tensor(gpuPlacement, TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
+        std::optional<Tensor> workspace = allocateReductionWorkspace(plan, gpuPlacement, stream);
         Tensor output = allocateFor(node);
         std::vector<std::string> scalarNames;
         for (uint32_t slot : scalarSlots) scalarNames.push_back(root_inputs.at(slot).name);
@@ -1613,7 +1629,18 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             stages.push_back(std::move(copy));
             produced = pre->second;
         }
+        auto requested = requestedOutputShapes.find(o.name);
+        if (requested != requestedOutputShapes.end() && !requested->second.empty()) {
+            if (!sameDimensionsIgnoringSingletons(produced.getDimensions(), requested->second)) {
+                throw std::runtime_error("Output tensor dimensions are incompatible with the fused equation result.");
+            }
+            // a caller's own tensor keeps its dimensions; a tensor allocated here is handed out with the requested ones
+            if (pre == preallocated.end() && produced.isDenseContiguous() && produced.getDimensions() != requested->second) produced.reshape(requested->second);
+        }
         finalOutputs.emplace(o.name, produced);
+    }
+    for (const auto& [name, shape] : requestedOutputShapes) {
+        if (!shape.empty() && finalOutputs.find(name) == finalOutputs.end()) throw std::runtime_error("Requested output shape names '" + name + "', which is not an output of this equation.");
     }
     return StampedExecutionPlan(std::move(stages), std::move(finalOutputs), stream);
 }

@@ -313,8 +313,7 @@ void tryReductionFusion(RowFusionContext& ctx) {
         request.inputDType = inputs.front().getDataType();
 
         ReductionLaunchPlan plan = buildReductionKernels(request);
-        std::optional<Tensor> workspace;
-        if (plan.workspaceBytes > 0) workspace = Tensor(gpuPlacement, TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
+        std::optional<Tensor> workspace = allocateReductionWorkspace(plan, gpuPlacement, ctx.stream);
         std::vector<Tensor> outputs, elementwiseOutputs;
         for (uint32_t r : reductions) {
             Tensor out = ctx.allocateFor(r);

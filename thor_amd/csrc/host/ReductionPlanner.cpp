@@ -1,9 +1,12 @@
 #include "ReductionPlanner.h"
 
+#include "Utilities/Common/ScopedGpu.h"
+#include "Utilities/Common/Stream.h"
 #include "Utilities/Expression/CompiledEquation.h"
 #include "thorhip_numeric_embed.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <sstream>
 #include <stdexcept>
 
@@ -108,6 +111,14 @@ std::string offsetFunction(const char* name, const std::vector<uint64_t>& dims, 
 
 }  // namespace
 
+int xcdRunLength(int preferred) {
+    if (const char* env = std::getenv("THOR_XCD_RUN")) {
+        const long v = std::atol(env);
+        if (v >= 1 && v <= 1024) return static_cast<int>(v);
+    }
+    return preferred;
+}
+
 uint64_t pointerAlignment(const void* p) {
     const uint64_t address = reinterpret_cast<uint64_t>(p);
     uint64_t alignment = 256;
@@ -156,11 +167,44 @@ std::string ReductionShape::describe() const {
             out << "strided(kept_rank=" << keptDims.size() << ",reduced_rank=" << reducedDims.size() << ",split=" << split;
             break;
     }
-    out << ",vec=" << vec << ",threads=" << threads << ",grid=" << gridX << "x" << gridY << ")";
+    out << ",vec=" << vec << ",threads=" << threads << ",grid=" << gridX << "x" << gridY << (tickets ? ",last_share_folds" : "") << ")";
     return out.str();
 }
 
+namespace {
+ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request);
+}
+
 ReductionShape planReductionShape(const ReductionKernelRequest& request) {
+    ReductionShape shape = planShapeWithoutTickets(request);
+    // Finishing inside the main launch: whole-tensor reductions over several blocks, and split reductions whose shares of one
+    // output group are whole blocks.  THOR_REDUCE_TICKETS=0 keeps the finishing launch (tuning switch).
+    // Measured on MI355X, finishing launch against last share: per-channel sums of an NCHW tensor (strided, 256 x 16 blocks) 21.0 /
+    // 21.2 us, 16 rows of 2^22 (rows, 16 x 8 blocks) 49.5 / 48.9 us: as fast with one launch fewer, so these two kinds take
+    // tickets.  Whole-tensor sums (1024 arrivals on one word: 42 / 47 us) and column sums (256 device-wide partial stores per
+    // block: 53 / 84 us) keep the finishing launch unless THOR_REDUCE_TICKETS=2 forces tickets everywhere.
+    const char* env = std::getenv("THOR_REDUCE_TICKETS");
+    const bool wanted = env == nullptr || std::atoi(env) != 0;
+    const bool forced = env != nullptr && std::atoi(env) == 2;
+    uint64_t count = 0;
+    switch (shape.kernel) {
+        case ReductionShape::Kernel::All: count = forced && shape.blocks > 1 ? 1 : 0; break;
+        case ReductionShape::Kernel::Rows: count = shape.split > 1 && shape.threadsPerRow > 64 ? request.geometry.outer_size : 0; break;
+        case ReductionShape::Kernel::Columns: count = forced && shape.split > 1 ? shape.gridX : 0; break;
+        case ReductionShape::Kernel::Strided: count = shape.split > 1 ? request.geometry.output_elements : 0; break;
+        case ReductionShape::Kernel::Segments: break;
+    }
+    if (wanted && count > 0 && shape.workspaceBytes > 0) {
+        shape.tickets = true;
+        shape.ticketCount = count;
+        shape.ticketOffset = (shape.workspaceBytes + 255) / 256 * 256;
+        shape.workspaceBytes = shape.ticketOffset + count * 4;
+    }
+    return shape;
+}
+
+namespace {
+ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
     const CubReductionGeometry& g = request.geometry;
     uint32_t elementBytes = dataTypeSizeInBytes(request.inputDType);
     if (!request.values.empty()) {
@@ -340,14 +384,19 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
     const uint64_t reductionVectors = g.reduction_size / shape.vec;
     const uint64_t outputs = g.output_elements;
     if (outputs < 2048 && reductionVectors > 256ull * 8) {
-        shape.split = std::min<uint64_t>({ceilDiv(4096, outputs), reductionVectors / (256ull * 4), kMaxGridY});
+        uint64_t wantedBlocks = 4096;
+        if (const char* env = std::getenv("THOR_STRIDED_BLOCKS")) wantedBlocks = std::max<long>(std::atol(env), 1);  // tuning switch
+        shape.split = std::min<uint64_t>({ceilDiv(wantedBlocks, outputs), reductionVectors / (256ull * 4), kMaxGridY});
         if (shape.split < 2) shape.split = 1;
     }
+    shape.unroll = 4;
+    if (const char* env = std::getenv("THOR_STRIDED_BATCH")) shape.unroll = std::min<long>(std::max<long>(std::atol(env), 1), 16);  // tuning switch
     shape.gridX = static_cast<uint32_t>(outputs);
     shape.gridY = static_cast<uint32_t>(shape.split);
     finishSplit(outputs);
     return shape;
 }
+}  // namespace
 
 std::string generateReductionSource(const ReductionKernelRequest& request, const ReductionShape& shape) {
     const CubReductionGeometry& g = request.geometry;
@@ -370,6 +419,11 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     s << "    typedef " << indexType << " IndexT;\n";
     s << "    static constexpr int kVec = " << shape.vec << ";\n";
     s << "    static constexpr int kThreads = " << shape.threads << ";\n";
+    s << "    static constexpr bool kTickets = " << (shape.tickets ? "true" : "false") << ";\n";
+    s << "    static constexpr u64 kTicketOffset = " << shape.ticketOffset << "ull;\n";
+    // one block per row of 8192 fp32: runs of 4 rows (128 KiB) per XCD measured +1.5 % (6.57 -> 6.67 TB/s), runs of 2 -3 %; rows
+    // that share a block and whole-tensor sums gain nothing from any run length
+    s << "    static constexpr int kXcdRun = " << xcdRunLength(shape.kernel == ReductionShape::Kernel::Rows && shape.threadsPerRow > 64 ? 4 : 1) << ";\n";
     s << "    static constexpr u64 kSplit = " << shape.split << "ull;\n";
     s << "    static constexpr u64 kOutputs = " << g.output_elements << "ull;\n";
     s << "    static constexpr float kDivisor = (float)" << g.reduction_size << "ull;\n";
@@ -543,6 +597,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
                 rs.back() = shape.vec;  // one step of the innermost axis = one vector
             }
             s << "    static constexpr u64 kReduction = " << (g.reduction_size / shape.vec) << "ull;\n";
+            s << "    static constexpr int kBatch = " << shape.unroll << ";\n";
             s << offsetFunction("keptOffset", shape.keptDims, shape.keptStrides);
             s << offsetFunction("reducedOffset", rd, rs);
             body = "thor::reduceStrided<gen::Cfg>(src, out, partials, scale);";
@@ -591,7 +646,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
           << "};\n    thor::finishSegments<gen::Cfg>(partials, out, scale, static_cast<const gen::Cfg::OffsetT*>(offsets));\n}\n";
         s << "extern \"C\" __global__ __launch_bounds__(256) void thor_reduce_prepare(void* partials, const void* offsets) {\n"
              "    thor::prepareSegments<gen::Cfg>(partials, static_cast<const gen::Cfg::OffsetT*>(offsets));\n}\n";
-    } else if (twoStageAll || shape.split > 1) {
+    } else if ((twoStageAll || shape.split > 1) && !shape.tickets) {
         s << "extern \"C\" __global__ __launch_bounds__(" << (twoStageAll ? 1024 : 256) << ") void thor_reduce_finish(const void* partials, "
           << finishParams.str() << ", float scale) {\n    const gen::Cfg::Outputs out{" << finishInit.str() << "};\n    thor::"
           << (twoStageAll ? "finishAll" : "finishPartials") << "<gen::Cfg>(partials, out, scale);\n}\n";
@@ -605,7 +660,10 @@ ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request)
     ReductionLaunchPlan plan;
     // fp32 accumulation order is part of the result: never let the compiler fuse or reassociate across elements
     plan.mainKernel = compileKernel(source, "thor_reduce_main", request.deviceNum, /*fastContract=*/false);
-    if (shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1) {
+    if (shape.tickets) {
+        plan.ticketOffset = shape.ticketOffset;
+        plan.ticketBytes = shape.ticketCount * 4;
+    } else if (shape.kernel == ReductionShape::Kernel::All && shape.blocks > 1) {
         plan.finishKernel = compileKernel(source, "thor_reduce_finish", request.deviceNum, false);
         plan.finishThreads = 1024;
         plan.finishGridX = 1;
@@ -630,6 +688,18 @@ ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request)
     plan.workspaceBytes = shape.workspaceBytes;
     plan.variant = shape.describe() + " [" + plan.mainKernel->kernelName + "]";
     return plan;
+}
+
+std::optional<Tensor> allocateReductionWorkspace(const ReductionLaunchPlan& plan, const TensorPlacement& placement, const Stream& stampStream) {
+    if (plan.workspaceBytes == 0) return std::nullopt;
+    Tensor workspace(placement, TensorDescriptor(DataType::UINT8, {plan.workspaceBytes}));
+    if (plan.ticketBytes > 0) {
+        Stream stream = stampStream;
+        ScopedGpu scoped(stream.getGpuNum());
+        THOR_HIP_CHECK(thorhip_memset_async(workspace.getMemPtr<char>() + plan.ticketOffset, 0, plan.ticketBytes, stream.getStream()));
+        stream.synchronize();
+    }
+    return workspace;
 }
 
 }  // namespace ThorImplementation

@@ -5,6 +5,7 @@
 #include "Utilities/TensorOperations/Cub/CubReduction.h"
 
 #include <cstdint>
+#include <optional>
 #include <string>
 #include <vector>
 
@@ -71,6 +72,11 @@ struct ReductionShape {
     bool indexIs64 = false;
     uint32_t gridX = 1, gridY = 1;
     size_t workspaceBytes = 0;
+    // Blocks that share an output count in on ticket words and the last one folds the partials (no finishing launch): the
+    // words live in the workspace at ticketOffset and must be zero before the first run.
+    bool tickets = false;
+    uint64_t ticketCount = 0;
+    size_t ticketOffset = 0;
     // collapsed axes of the strided kernel
     std::vector<uint64_t> keptDims, keptStrides, reducedDims, reducedStrides;
     // Columns kernel over a view: index (into keptDims) of the kept axis that is contiguous in memory, or -1 for the
@@ -84,9 +90,15 @@ struct ReductionShape {
 };
 
 uint64_t pointerAlignment(const void* p);
+
+// Length of the runs of adjacent blocks that the row kernels give to one XCD (thor::xcdBlock in the device prelude); 1 = the
+// hardware's round-robin order.  THOR_XCD_RUN overrides the kernel's preferred length (tuning switch).
+int xcdRunLength(int preferred);
 ReductionShape planReductionShape(const ReductionKernelRequest& request);
 std::string generateReductionSource(const ReductionKernelRequest& request, const ReductionShape& shape);
 ReductionLaunchPlan buildReductionKernels(const ReductionKernelRequest& request);
+// The workspace a launch plan needs (nothing when it needs none), with its ticket words cleared; `stream` is synchronised.
+std::optional<Tensor> allocateReductionWorkspace(const ReductionLaunchPlan& plan, const TensorPlacement& placement, const Stream& stream);
 
 const char* deviceTypeName(DataType dtype);  // "thor::f16", "float", ...
 

@@ -408,10 +408,11 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     s << "    constexpr int T = " << T << ", V = " << vec << ", ITEMS = " << items << ";\n";
     s << "    constexpr unsigned long long R = " << rg.R << "ull, ROWS = " << rg.rows << "ull, VECTORS = " << vectors << "ull;\n";
     if (subWave) {
-        s << "    const unsigned long long row = (unsigned long long)blockIdx.x * " << rowsPerBlock << "ull + threadIdx.x / T;\n";
+        s << "    const unsigned long long row = (unsigned long long)thor::xcdBlock<" << xcdRunLength(1) << ">(blockIdx.x, gridDim.x) * " << rowsPerBlock
+          << "ull + threadIdx.x / T;\n";
         s << "    const int lane = threadIdx.x % T;\n";
     } else {
-        s << "    const unsigned long long row = blockIdx.x;\n    const int lane = threadIdx.x;\n";
+        s << "    const unsigned long long row = thor::xcdBlock<" << xcdRunLength(1) << ">(blockIdx.x, gridDim.x);\n    const int lane = threadIdx.x;\n";
     }
     s << "    const bool rowLive = row < ROWS;\n";
     s << "    const unsigned long long rowIndex = rowLive ? row : 0ull;\n";

@@ -25,6 +25,7 @@ struct RowFusionContext {
     std::vector<int>& stageOfNode;
     std::function<Tensor(uint32_t)> allocateFor;
     int deviceNum;
+    Stream stream;  // the stream of the stamp call (workspaces are prepared on it)
 };
 
 // Appends FusedRowKernel stages for every group it recognises and marks the nodes they produce as done.

@@ -2,7 +2,10 @@
 
 #include "Utilities/Common/ScopedGpu.h"
 
+#include "Utilities/Expression/Expression.h"
+
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
 #include <stdexcept>
 
@@ -217,16 +220,139 @@ void StampedExecutionStage::runOn(Stream& stream, const std::unordered_map<std::
             if (!scan) throw std::runtime_error("Scan stage is missing its stamped scan.");
             scan->runOn(stream);
             return;
+        case Kind::DependencyBarrier:
+            return;
     }
 }
+
+detail::StampedExecutionSchedule detail::buildStampedExecutionSchedule(const std::vector<StampedExecutionStage>& steps, uint32_t caller_gpu_num) {
+    StampedExecutionSchedule schedule;
+    const uint32_t count = static_cast<uint32_t>(steps.size());
+    schedule.stage_lane_indices.assign(count, 0);
+    schedule.stage_has_downstream_dependency.assign(count, false);
+    schedule.stage_needs_completion_event.assign(count, false);
+    schedule.lane_gpu_nums.push_back(caller_gpu_num);
+    if (count == 0) return schedule;
+
+    // heir[p]: the dependent stage that stays on p's lane = the first stage on p's GPU that consumes p
+    constexpr uint32_t kNone = 0xffffffffu;
+    std::vector<uint32_t> heir(count, kNone);
+    for (uint32_t stage = 0; stage < count; ++stage) {
+        for (uint32_t producer : steps[stage].dependency_stage_indices) {
+            if (producer >= stage) throw std::runtime_error("StampedExecutionPlan::runOn requires dependency_stage_indices to be topologically ordered.");
+            if (heir[producer] == kNone && steps[producer].gpu_num == steps[stage].gpu_num) heir[producer] = stage;
+        }
+    }
+    bool callerLaneHasRoot = false;
+    for (uint32_t stage = 0; stage < count; ++stage) {
+        uint32_t lane = kNone;
+        for (uint32_t producer : steps[stage].dependency_stage_indices) {
+            if (heir[producer] != stage) continue;
+            const uint32_t candidate = schedule.stage_lane_indices[producer];
+            if (lane == kNone || candidate == 0) lane = candidate;  // heir of several producers: the caller's lane wins, else the first
+            if (lane == 0) break;
+        }
+        if (lane == kNone && steps[stage].dependency_stage_indices.empty() && !callerLaneHasRoot && steps[stage].gpu_num == caller_gpu_num) {
+            lane = 0;
+            callerLaneHasRoot = true;
+        }
+        if (lane == kNone) {
+            lane = static_cast<uint32_t>(schedule.lane_gpu_nums.size());
+            schedule.lane_gpu_nums.push_back(steps[stage].gpu_num);
+        }
+        schedule.stage_lane_indices[stage] = lane;
+    }
+    for (uint32_t stage = 0; stage < count; ++stage) {
+        const uint32_t lane = schedule.stage_lane_indices[stage];
+        if (steps[stage].dependency_stage_indices.empty() && lane != 0) schedule.needs_caller_ready_event = true;
+        for (uint32_t producer : steps[stage].dependency_stage_indices) {
+            schedule.stage_has_downstream_dependency[producer] = true;
+            if (schedule.stage_lane_indices[producer] != lane) schedule.stage_needs_completion_event[producer] = true;
+        }
+    }
+    // the last stage of a helper lane that nothing consumes is joined back into the caller's stream at the end of the run
+    for (uint32_t stage = 0; stage < count; ++stage) {
+        if (!schedule.stage_has_downstream_dependency[stage] && schedule.stage_lane_indices[stage] != 0) schedule.stage_needs_completion_event[stage] = true;
+    }
+    return schedule;
+}
+
+StampedExecutionPlan::LaneResources StampedExecutionPlan::makeLaneResources(const detail::StampedExecutionSchedule& schedule) {
+    LaneResources lanes;
+    if (schedule.lane_gpu_nums.size() <= 1) return lanes;
+    for (size_t lane = 1; lane < schedule.lane_gpu_nums.size(); ++lane) lanes.helpers.push_back(Expression::getNextHelperStream(schedule.lane_gpu_nums[lane]));
+    if (schedule.needs_caller_ready_event) lanes.caller_ready = Event(static_cast<int>(schedule.lane_gpu_nums[0]));
+    lanes.stage_completion.resize(schedule.stage_lane_indices.size());
+    for (size_t stage = 0; stage < schedule.stage_lane_indices.size(); ++stage) {
+        if (schedule.stage_needs_completion_event[stage]) {
+            lanes.stage_completion[stage] = Event(static_cast<int>(schedule.lane_gpu_nums[schedule.stage_lane_indices[stage]]));
+        }
+    }
+    return lanes;
+}
+
+StampedExecutionPlan::StampedExecutionPlan(std::vector<StampedExecutionStage> plan_steps, std::unordered_map<std::string, Tensor> outputs,
+                                           const Stream& plan_stream)
+    : steps(std::move(plan_steps)), final_outputs(std::move(outputs)), stream(plan_stream),
+      execution_schedule(detail::buildStampedExecutionSchedule(steps, plan_stream.isInitialized() ? static_cast<uint32_t>(plan_stream.getGpuNum()) : 0u)),
+      lane_resources(makeLaneResources(execution_schedule)) {}
 
 void StampedExecutionPlan::run() { runOn(stream, {}); }
 void StampedExecutionPlan::run(const std::unordered_map<std::string, float>& runtime_scalars) { runOn(stream, runtime_scalars); }
 void StampedExecutionPlan::runOn(Stream& run_stream) const { runOn(run_stream, {}); }
 
 void StampedExecutionPlan::runOn(Stream& run_stream, const std::unordered_map<std::string, float>& runtime_scalars) const {
-    // Stages are stored in dependency order and issued on one stream: stream order is the synchronisation.
-    for (const StampedExecutionStage& step : steps) step.runOn(run_stream, runtime_scalars);
+    // Single stages and plans without a branch (every stage on the caller's lane) need no scheduler: stages are stored in
+    // dependency order and stream order is the synchronisation (reference: StampedEquation.cpp:4065-4113).
+    if (execution_schedule.lane_gpu_nums.size() <= 1 || std::getenv("THOR_DISABLE_STAGE_OVERLAP") != nullptr) {
+        for (const StampedExecutionStage& step : steps) step.runOn(run_stream, runtime_scalars);
+        return;
+    }
+    if (run_stream.getGpuNum() == stream.getGpuNum()) {
+        runForked(run_stream, execution_schedule, lane_resources, runtime_scalars);
+        return;
+    }
+    // a run on another GPU's stream than the plan was stamped for: its own schedule and lanes, made for this run
+    const detail::StampedExecutionSchedule other = detail::buildStampedExecutionSchedule(steps, static_cast<uint32_t>(run_stream.getGpuNum()));
+    const LaneResources lanes = makeLaneResources(other);
+    runForked(run_stream, other, lanes, runtime_scalars);
+}
+
+// Independent branches on helper streams, joined with events (reference: StampedEquation.cpp:4115-4207).  Events are the plan's
+// own, created when it was stamped; a wait captures the event's latest record at the time of the call, so the next run may
+// record the same events again without waiting for this one.
+void StampedExecutionPlan::runForked(Stream& run_stream, const detail::StampedExecutionSchedule& schedule, const LaneResources& lanes,
+                                     const std::unordered_map<std::string, float>& runtime_scalars) const {
+    auto laneStream = [&](uint32_t lane) -> const Stream& { return lane == 0 ? run_stream : lanes.helpers[lane - 1]; };
+    if (schedule.needs_caller_ready_event) {
+        Event ready = lanes.caller_ready;
+        run_stream.putEvent(ready);
+    }
+    for (uint32_t index = 0; index < steps.size(); ++index) {
+        const StampedExecutionStage& stage = steps[index];
+        const uint32_t lane = schedule.stage_lane_indices[index];
+        Stream launch = laneStream(lane);
+        if (stage.dependency_stage_indices.empty() && lane != 0) launch.waitEvent(lanes.caller_ready);  // work queued on the caller's stream comes first
+        for (uint32_t producer : stage.dependency_stage_indices) {
+            const Stream& producerStream = laneStream(schedule.stage_lane_indices[producer]);
+            if (launch == producerStream) continue;
+            if (!lanes.stage_completion[producer].isInitialized()) {
+                throw std::runtime_error("StampedExecutionPlan::runOn missing completion event for cross-stream dependency stage.");
+            }
+            launch.waitEvent(lanes.stage_completion[producer]);
+        }
+        stage.runOn(launch, runtime_scalars);
+        if (schedule.stage_needs_completion_event[index]) {
+            Event done = lanes.stage_completion[index];
+            launch.putEvent(done);
+        }
+    }
+    // helper work that nothing consumed joins the caller's stream; branches that fed a stage on it are joined already
+    for (uint32_t index = 0; index < steps.size(); ++index) {
+        const uint32_t lane = schedule.stage_lane_indices[index];
+        if (schedule.stage_has_downstream_dependency[index] || lane == 0 || laneStream(lane) == run_stream) continue;
+        run_stream.waitEvent(lanes.stage_completion[index]);
+    }
 }
 
 std::unordered_set<std::string> StampedExecutionPlan::runtimeScalarNames() const {
