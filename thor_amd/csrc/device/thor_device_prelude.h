@@ -216,9 +216,9 @@ struct MaxOp {
     __device__ __forceinline__ static float combine(float a, float b) { return ((b > a) | (b != b)) ? b : a; }
 };
 
-// Partials travel between blocks (of one launch, or of a launch and its finishing launch) through memory words that are
-// written and read at device scope: relaxed atomic stores and loads of agent scope, which go past the per-XCD L2 instead
-// of leaving a dirty or stale line in it.  A block that has waited for its own stores (partialsWritten) may then announce
+// Partials that travel between blocks of one launch (ticket protocol of the reduction kernels) go through memory words that
+// are written and read at device scope: relaxed atomic stores and loads of agent scope, which go past the per-XCD L2 instead
+// of leaving a dirty or stale line in it.  (Partials for a finishing launch are plain stores: the launch boundary publishes them.)  A block that has waited for its own stores (partialsWritten) may then announce
 // them with an atomic counter, and a reader that has seen the count needs no cache invalidation.
 template <typename W>
 __device__ __forceinline__ void storeDeviceWide(W* p, W w) {
@@ -249,8 +249,16 @@ struct ValueAcc {
     }
     // A partial of `slots` accumulators is one float array of that length.
     __device__ __forceinline__ static u64 partialBytes(u64 slots) { return ((slots * 4 + 7) / 8) * 8; }
-    __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64) const { storeDeviceWide(static_cast<float*>(partials) + slot, v); }
-    __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64) { v = loadDeviceWide(static_cast<const float*>(partials) + slot); }
+    // DEVICE_WIDE: the partial is read by another block of the same launch (ticket protocol); otherwise by a later launch
+    template <bool DEVICE_WIDE = false>
+    __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64) const {
+        if (DEVICE_WIDE) storeDeviceWide(static_cast<float*>(partials) + slot, v);
+        else static_cast<float*>(partials)[slot] = v;
+    }
+    template <bool DEVICE_WIDE = false>
+    __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64) {
+        v = DEVICE_WIDE ? loadDeviceWide(static_cast<const float*>(partials) + slot) : static_cast<const float*>(partials)[slot];
+    }
 };
 
 // Candidate {value, index}: NaN beats every number, equal values (and two NaNs) keep the lower index.  The empty
@@ -299,13 +307,24 @@ struct ArgAcc {
     }
     // A partial of `slots` candidates is a float array followed by an IndexT array of the same length.
     __device__ __forceinline__ static u64 partialBytes(u64 slots) { return ((slots * 4 + 7) / 8) * 8 + slots * sizeof(IndexT); }
+    template <bool DEVICE_WIDE = false>
     __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64 slots) const {
-        storeDeviceWide(static_cast<float*>(partials) + slot, v);
-        storeDeviceWide(reinterpret_cast<IndexT*>(static_cast<char*>(partials) + ((slots * 4 + 7) / 8) * 8) + slot, i);
+        float* values = static_cast<float*>(partials);
+        IndexT* indices = reinterpret_cast<IndexT*>(static_cast<char*>(partials) + ((slots * 4 + 7) / 8) * 8);
+        if (DEVICE_WIDE) {
+            storeDeviceWide(values + slot, v);
+            storeDeviceWide(indices + slot, i);
+        } else {
+            values[slot] = v;
+            indices[slot] = i;
+        }
     }
+    template <bool DEVICE_WIDE = false>
     __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64 slots) {
-        v = loadDeviceWide(static_cast<const float*>(partials) + slot);
-        i = loadDeviceWide(reinterpret_cast<const IndexT*>(static_cast<const char*>(partials) + ((slots * 4 + 7) / 8) * 8) + slot);
+        const float* values = static_cast<const float*>(partials);
+        const IndexT* indices = reinterpret_cast<const IndexT*>(static_cast<const char*>(partials) + ((slots * 4 + 7) / 8) * 8);
+        v = DEVICE_WIDE ? loadDeviceWide(values + slot) : values[slot];
+        i = DEVICE_WIDE ? loadDeviceWide(indices + slot) : indices[slot];
     }
 };
 

@@ -56,7 +56,7 @@ __device__ __forceinline__ void foldShares(const void* partials, u64 output, con
     acc.reset();
     for (u64 s = lane; s < Cfg::kSplit; s += kWave) {
         Acc part;
-        part.loadPartial(partials, output * Cfg::kSplit + s, Cfg::kOutputs * Cfg::kSplit);
+        part.template loadPartial<Cfg::kTickets>(partials, output * Cfg::kSplit + s, Cfg::kOutputs * Cfg::kSplit);
         acc.merge(part);
     }
     groupReduce<kWave>(acc);
@@ -109,7 +109,7 @@ __device__ __forceinline__ void reduceAll(const typename Cfg::Sources& src, cons
         if (Cfg::kBlocks == 1) {
             Cfg::store(acc, 0, out, scale);
         } else {
-            acc.storePartial(partials, block, Cfg::kBlocks);
+            acc.template storePartial<Cfg::kTickets>(partials, block, Cfg::kBlocks);
             if (Cfg::kTickets) partialsWritten();
         }
     }
@@ -120,7 +120,7 @@ __device__ __forceinline__ void reduceAll(const typename Cfg::Sources& src, cons
         total.reset();
         for (u32 b = threadIdx.x; b < (u32)Cfg::kBlocks; b += Cfg::kThreads) {
             Acc part;
-            part.loadPartial(partials, b, Cfg::kBlocks);
+            part.template loadPartial<true>(partials, b, Cfg::kBlocks);
             total.merge(part);
         }
         blockReduce<Cfg::kThreads, false>(total, finishScratch);
@@ -207,7 +207,7 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
     }
     if (lane == 0 && rowLive) {
         if (Cfg::kSplit > 1) {
-            acc.storePartial(partials, row * Cfg::kSplit + segment, Cfg::kOuter * Cfg::kSplit);
+            acc.template storePartial<Cfg::kTickets>(partials, row * Cfg::kSplit + segment, Cfg::kOuter * Cfg::kSplit);
             if (Cfg::kTickets) partialsWritten();
         } else {
             Cfg::store(acc, row, out, scale);
@@ -287,7 +287,7 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
 #pragma unroll
         for (int k = 0; k < Cfg::kVec; ++k) {
             if (Cfg::kSplit > 1) {
-                acc[k].storePartial(partials, Cfg::partialSlot(column, k) * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
+                acc[k].template storePartial<Cfg::kTickets>(partials, Cfg::partialSlot(column, k) * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
             } else {
                 Cfg::store(acc[k], Cfg::outputIndex(column, k), out, scale);
             }
@@ -349,7 +349,7 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::Sources& src, 
     blockReduce<Cfg::kThreads, false>(acc, scratch);
     if (threadIdx.x == 0) {
         if (Cfg::kSplit > 1) {
-            acc.storePartial(partials, output * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
+            acc.template storePartial<Cfg::kTickets>(partials, output * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
             if (Cfg::kTickets) partialsWritten();
         } else {
             Cfg::store(acc, output, out, scale);

@@ -471,12 +471,12 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
         for (size_t j = 0; j < values.size(); ++j) s << "            r.a" << j << " = a" << j << ".shuffleXor(mask);\n";
         s << "            return r;\n        }\n";
         // partials: one float array per member, back to back
-        s << "        __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64 slots) const {\n"
+        s << "        template <bool DEVICE_WIDE = false>\n        __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64 slots) const {\n"
              "            char* base = static_cast<char*>(partials);\n            const u64 stride = ((slots * 4 + 7) / 8) * 8;\n";
-        for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".storePartial(base + " << j << " * stride, slot, slots);\n";
-        s << "        }\n        __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64 slots) {\n"
+        for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".template storePartial<DEVICE_WIDE>(base + " << j << " * stride, slot, slots);\n";
+        s << "        }\n        template <bool DEVICE_WIDE = false>\n        __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64 slots) {\n"
              "            const char* base = static_cast<const char*>(partials);\n            const u64 stride = ((slots * 4 + 7) / 8) * 8;\n";
-        for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".loadPartial(base + " << j << " * stride, slot, slots);\n";
+        for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".template loadPartial<DEVICE_WIDE>(base + " << j << " * stride, slot, slots);\n";
         s << "        }\n    };\n";
     }
     s << "    static __device__ __forceinline__ void accumulateOne(Acc& acc, const Loaded& l, const Sources& s, const Kept& kk, int k, IndexT index) {\n";
