@@ -104,6 +104,13 @@ int thorhip_event_elapsed_ms(float* ms, void* start, void* stop);
 int thorhip_compile(const char* source, const char* program_name, const char* arch, const char* const* options,
                     int num_options, void** code, size_t* code_size, char* log, size_t log_capacity);
 int thorhip_code_free(void* code);
+/* Compile isolation.  With it on, thorhip_compile runs the compiler in a child process of its own (the worker program next to
+ * the library, started with posix_spawn; it links the run-time compiler only and never touches a GPU) and gets the code object
+ * or the log back over a pipe, so that a compiler that aborts - an internal compiler error ends in abort() - fails that one
+ * compilation with an error instead of ending the calling process.  Costs a process start per compilation (compiled kernels
+ * are cached by the host layer).  Off by default; THORHIP_COMPILE_ISOLATION=1 in the environment turns it on.  Returns the
+ * previous setting.  No counterpart in the reference, whose NVRTC calls are in-process (EquationCompiler.cpp:1864-1908). */
+int thorhip_set_compile_isolation(int enabled);
 int thorhip_module_load(void** module, const void* code, size_t code_size);
 int thorhip_module_unload(void* module);
 int thorhip_module_get_function(void** function, void* module, const char* kernel_name);

@@ -63,6 +63,7 @@ THORHIP_PROTOTYPES = {
     "thorhip_event_record": (_i, [_vp, _vp]),
     "thorhip_event_synchronize": (_i, [_vp]),
     "thorhip_event_elapsed_ms": (_i, [ctypes.POINTER(ctypes.c_float), _vp, _vp]),
+    "thorhip_set_compile_isolation": (_i, [_i]),
     "thorhip_compile": (_i, [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_char_p), _i, _vpp, _szp,
                              ctypes.c_char_p, _sz]),
     "thorhip_code_free": (_i, [_vp]),

@@ -8,11 +8,23 @@
 
 #include <hip/hiprtc.h>
 
+#include <atomic>
+#include <cerrno>
+#include <csignal>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
 #include <vector>
+
+#include <dlfcn.h>
+#include <poll.h>
+#include <spawn.h>
+#include <sys/socket.h>
+#include <sys/wait.h>
+#include <unistd.h>
+
+extern char** environ;
 
 namespace thorhip {
 std::string& lastError() {
@@ -260,6 +272,145 @@ static void copyLog(hiprtcProgram prog, char* log, size_t cap) {
     std::snprintf(log, cap, "%s", text.c_str());
 }
 
+// ---- compilation in a process of its own ------------------------------------------------------------------------------
+// -1: not decided yet (THORHIP_COMPILE_ISOLATION in the environment decides at the first compile), 0 off, 1 on
+static std::atomic<int> compileIsolation{-1};
+
+static bool isolationEnabled() {
+    int mode = compileIsolation.load();
+    if (mode < 0) {
+        const char* env = std::getenv("THORHIP_COMPILE_ISOLATION");
+        mode = (env != nullptr && std::atoi(env) != 0) ? 1 : 0;
+        compileIsolation.store(mode);
+    }
+    return mode == 1;
+}
+
+// The worker sits next to this library (built by the same Makefile); THORHIP_RTC_WORKER names another one.
+static std::string workerPath() {
+    if (const char* env = std::getenv("THORHIP_RTC_WORKER")) return env;
+    Dl_info info;
+    if (dladdr(reinterpret_cast<const void*>(&thorhip_abi_version), &info) != 0 && info.dli_fname != nullptr) {
+        std::string path = info.dli_fname;
+        const size_t slash = path.rfind('/');
+        return (slash == std::string::npos ? std::string(".") : path.substr(0, slash)) + "/thorhip_rtc_worker";
+    }
+    return "thorhip_rtc_worker";
+}
+
+static bool sendAll(int fd, const void* data, size_t bytes) {
+    const char* p = static_cast<const char*>(data);
+    while (bytes > 0) {
+        const ssize_t n = ::send(fd, p, bytes, MSG_NOSIGNAL);  // a worker that died must not raise SIGPIPE here
+        if (n < 0 && errno == EINTR) continue;
+        if (n <= 0) return false;
+        p += n;
+        bytes -= static_cast<size_t>(n);
+    }
+    return true;
+}
+static bool sendString(int fd, const std::string& s) {
+    const uint64_t n = s.size();
+    return sendAll(fd, &n, sizeof n) && (n == 0 || sendAll(fd, s.data(), n));
+}
+
+// Runs one compilation in the worker program.  The worker gets the request on its standard input and answers on its standard
+// output; what it (or the compiler inside it) prints to standard error is kept for the error text.  A worker that ends on a
+// signal - the compiler called abort() - is reported as a failed compilation; the calling process is never replaced or harmed.
+static int compileInWorker(const std::string& source, const std::string& name, const std::string& arch, const std::vector<std::string>& flags,
+                           void** code, size_t* code_size, char* log, size_t log_capacity) {
+    const std::string path = workerPath();
+    int toWorker[2], fromWorker[2], errWorker[2];
+    if (socketpair(AF_UNIX, SOCK_STREAM, 0, toWorker) != 0) return fail(-7, "thorhip_compile: socketpair failed: %s", std::strerror(errno));
+    if (pipe(fromWorker) != 0 || pipe(errWorker) != 0) return fail(-7, "thorhip_compile: pipe failed: %s", std::strerror(errno));
+    posix_spawn_file_actions_t actions;
+    posix_spawn_file_actions_init(&actions);
+    posix_spawn_file_actions_adddup2(&actions, toWorker[0], STDIN_FILENO);
+    posix_spawn_file_actions_adddup2(&actions, fromWorker[1], STDOUT_FILENO);
+    posix_spawn_file_actions_adddup2(&actions, errWorker[1], STDERR_FILENO);
+    for (int fd : {toWorker[0], toWorker[1], fromWorker[0], fromWorker[1], errWorker[0], errWorker[1]}) posix_spawn_file_actions_addclose(&actions, fd);
+    char* const argv[] = {const_cast<char*>(path.c_str()), nullptr};
+    pid_t pid = -1;
+    const int spawned = posix_spawn(&pid, path.c_str(), &actions, nullptr, argv, environ);
+    posix_spawn_file_actions_destroy(&actions);
+    ::close(toWorker[0]);
+    ::close(fromWorker[1]);
+    ::close(errWorker[1]);
+    if (spawned != 0) {
+        for (int fd : {toWorker[1], fromWorker[0], errWorker[0]}) ::close(fd);
+        return fail(-7, "thorhip_compile: cannot start the compiler worker '%s': %s", path.c_str(), std::strerror(spawned));
+    }
+    bool sent = sendString(toWorker[1], name) && sendString(toWorker[1], arch) && sendString(toWorker[1], source);
+    const uint64_t optionCount = flags.size();
+    sent = sent && sendAll(toWorker[1], &optionCount, sizeof optionCount);
+    for (const std::string& f : flags) sent = sent && sendString(toWorker[1], f);
+    ::close(toWorker[1]);
+
+    std::string answer, errors;
+    pollfd fds[2] = {{fromWorker[0], POLLIN, 0}, {errWorker[0], POLLIN, 0}};
+    int open = 2;
+    while (open > 0) {
+        if (poll(fds, 2, -1) < 0) {
+            if (errno == EINTR) continue;
+            break;
+        }
+        for (int i = 0; i < 2; ++i) {
+            if (fds[i].fd < 0 || (fds[i].revents & (POLLIN | POLLHUP | POLLERR)) == 0) continue;
+            char buffer[65536];
+            const ssize_t n = ::read(fds[i].fd, buffer, sizeof buffer);
+            if (n > 0) {
+                (i == 0 ? answer : errors).append(buffer, static_cast<size_t>(n));
+            } else if (n == 0 || errno != EINTR) {
+                ::close(fds[i].fd);
+                fds[i].fd = -1;
+                --open;
+            }
+        }
+    }
+    for (pollfd& f : fds)
+        if (f.fd >= 0) ::close(f.fd);
+    int status = 0;
+    while (waitpid(pid, &status, 0) < 0 && errno == EINTR) {
+    }
+    if (errors.size() > 1500) errors = errors.substr(0, 700) + "\n...\n" + errors.substr(errors.size() - 700);
+    if (WIFSIGNALED(status)) {
+        return fail(-8, "thorhip_compile: the compiler ended on signal %d (%s) while compiling '%s' for %s; the calling process is unharmed.\n%s",
+                    WTERMSIG(status), strsignal(WTERMSIG(status)), name.c_str(), arch.c_str(), errors.c_str());
+    }
+    if (!sent) return fail(-8, "thorhip_compile: the compiler worker closed its input early (exit status %d).\n%s", WEXITSTATUS(status), errors.c_str());
+    // answer: status, code (length, bytes), log (length, bytes)
+    auto take = [&](size_t& at, void* into, size_t bytes) {
+        if (answer.size() < at + bytes) return false;
+        std::memcpy(into, answer.data() + at, bytes);
+        at += bytes;
+        return true;
+    };
+    size_t at = 0;
+    int64_t workerStatus = 0;
+    uint64_t codeBytes = 0, logBytes = 0;
+    if (!take(at, &workerStatus, sizeof workerStatus) || !take(at, &codeBytes, sizeof codeBytes) || answer.size() < at + codeBytes) {
+        return fail(-8, "thorhip_compile: the compiler worker gave no complete answer (exit status %d).\n%s", WEXITSTATUS(status), errors.c_str());
+    }
+    const size_t codeAt = at;
+    at += codeBytes;
+    std::string workerLog;
+    if (take(at, &logBytes, sizeof logBytes) && answer.size() >= at + logBytes) workerLog.assign(answer, at, logBytes);
+    if (log != nullptr && log_capacity > 0) std::snprintf(log, log_capacity, "%s", workerLog.c_str());
+    if (workerStatus != 0 || codeBytes == 0) return fail(-3, "hiprtcCompileProgram(%s) failed in the compiler worker: %s", arch.c_str(), workerLog.c_str());
+    void* blob = std::malloc(codeBytes);
+    if (blob == nullptr) return fail(-5, "thorhip_compile: out of host memory for a %zu byte code object", (size_t)codeBytes);
+    std::memcpy(blob, answer.data() + codeAt, codeBytes);
+    *code = blob;
+    *code_size = codeBytes;
+    return 0;
+}
+
+int thorhip_set_compile_isolation(int enabled) {
+    const int before = isolationEnabled() ? 1 : 0;
+    compileIsolation.store(enabled != 0 ? 1 : 0);
+    return before;
+}
+
 int thorhip_compile(const char* source, const char* program_name, const char* arch, const char* const* options,
                     int num_options, void** code, size_t* code_size, char* log, size_t log_capacity) {
     THORHIP_REQUIRE(source != nullptr && code != nullptr && code_size != nullptr, "thorhip_compile: NULL argument");
@@ -281,6 +432,12 @@ int thorhip_compile(const char* source, const char* program_name, const char* ar
         }
     }
     const std::string arch_flag = "--offload-arch=" + arch_name;
+
+    if (isolationEnabled()) {
+        std::vector<std::string> workerFlags = {arch_flag, "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+        for (int i = 0; i < num_options; ++i) workerFlags.push_back(options[i]);
+        return compileInWorker(source, program_name ? program_name : "thor_fused.hip", arch_name, workerFlags, code, code_size, log, log_capacity);
+    }
 
     hiprtcProgram prog = nullptr;
     hiprtcResult rc = hiprtcCreateProgram(&prog, source, program_name ? program_name : "thor_fused.hip", 0, nullptr, nullptr);
