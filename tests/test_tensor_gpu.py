@@ -52,3 +52,31 @@ def test_device_to_device_and_host_to_host_conversion(gpu):
     np.testing.assert_array_equal(hh.numpy().view(np.uint16), oracle.convert(x, oracle.FP32, oracle.FP16).view(np.uint16))
     with pytest.raises(ValueError, match="element counts"):
         gpu_tensor([5], DataType.fp32).copy_from_async(host, stream)
+
+
+def test_alias_view_rejects_strides_that_wrap_around(gpu):
+    """A stride large enough for (dim - 1) * stride to wrap past 2^64 must not pass the bounds check of aliasView."""
+    t = gpu_tensor([4, 6], DataType.fp32)
+    ok = t.alias_view([6, 4], [1, 6])
+    assert ok.get_dimensions() == [6, 4]
+    huge = (1 << 63) + 3  # 2 * huge wraps to 6
+    with pytest.raises(Exception, match="outside the backing allocation"):
+        t.alias_view([3, 2], [huge, 1])
+    with pytest.raises(Exception, match="outside the backing allocation"):
+        t.alias_view([2], [1], (1 << 64) - 1)
+    with pytest.raises(Exception, match="outside the backing allocation"):
+        t.alias_view([4, 7], [6, 1])
+
+
+def test_numpy_view_keeps_its_tensor_alive(gpu):
+    """The array returned by numpy() must hold the pinned allocation: dropping the tensor first may not free the memory."""
+    import gc
+    host = cpu_tensor([1024], DataType.fp32)
+    view = host.numpy()
+    view[...] = np.arange(1024, dtype=np.float32)
+    del host
+    gc.collect()
+    filler = [cpu_tensor([1024], DataType.fp32) for _ in range(8)]  # would reuse the freed block
+    for f in filler:
+        f.numpy()[...] = -1.0
+    np.testing.assert_array_equal(view, np.arange(1024, dtype=np.float32))

@@ -99,13 +99,21 @@ Tensor Tensor::aliasView(std::vector<uint64_t> dimensions, std::vector<uint64_t>
     if (dimensions.empty() || dimensions.size() != strides_elements.size()) {
         throw std::invalid_argument("Tensor::aliasView requires one stride per dimension.");
     }
+    // the last element the view reaches, every product and sum checked: strides that wrap around 2^64 must not slip past the
+    // bounds test
+    const char* outside = "Tensor::aliasView addresses elements outside the backing allocation.";
     uint64_t last = element_offset;
     for (size_t i = 0; i < dimensions.size(); ++i) {
         if (dimensions[i] == 0) throw std::invalid_argument("Tensor::aliasView does not support zero-sized dimensions.");
-        last += (dimensions[i] - 1) * strides_elements[i];
+        uint64_t reach = 0;
+        if (__builtin_mul_overflow(dimensions[i] - 1, strides_elements[i], &reach) || __builtin_add_overflow(last, reach, &last)) {
+            throw std::invalid_argument(outside);
+        }
     }
+    uint64_t lastInStorage = 0;
+    if (__builtin_add_overflow(storageElementOffset, last, &lastInStorage)) throw std::invalid_argument(outside);
     // storageNumElements is the element count of the whole allocation; views inherit it unchanged
-    if (storageElementOffset + last >= storageNumElements) {
+    if (lastInStorage >= storageNumElements) {
         throw std::invalid_argument("Tensor::aliasView addresses elements outside the backing allocation.");
     }
     Tensor view = *this;
@@ -133,6 +141,7 @@ void Tensor::memsetAsync(Stream stream, int8_t value, uint64_t numElements) {
 void Tensor::memset(int8_t value, uint64_t numElements) {
     THOR_THROW_IF_FALSE(isInitialized() && isDenseContiguous());
     const uint64_t n = numElements == 0 ? getTotalNumElements() : numElements;
+    THOR_THROW_IF_FALSE(n <= getTotalNumElements());
     const size_t bytes = n * dataTypeSizeInBytes(getDataType());
     if (placement.getMemDevice() == TensorPlacement::MemDevices::GPU) {
         ScopedGpu scoped(placement.getDeviceNum());
