@@ -143,6 +143,19 @@ int thor_segmented_broadcast(thor_tensor_t per_segment_values, thor_tensor_t seg
 int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments, uint64_t segment_size,
               int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity);
 
+/* Select-flagged (Utilities/TensorOperations/Cub/CubDevicePrimitives.h:87-93,490-516 there): output receives the elements of input
+ * whose flag (BOOLEAN or UINT8) is nonzero, in input order, and *num_selected_out (UINT32) their number; prepare, allocate the
+ * temporary storage and run in one call.  num_items == 0 writes a zero count. */
+int thor_select_flagged(thor_tensor_t input, thor_tensor_t flags, thor_tensor_t output, thor_tensor_t num_selected_out, uint64_t num_items,
+                        thor_stream_t stream, char* variant, size_t variant_capacity);
+
+/* Top-k (CubDevicePrimitives.h:47-85,357-488 there): the k largest (largest != 0) or smallest keys, unordered; values_in /
+ * values_out (UINT32, both or neither) travel with their keys.  segmented == 0: one selection over the first segment_size keys
+ * (num_segments is ignored), k capped at that count.  segmented != 0: num_segments rows of segment_size <= 8192 keys each,
+ * k < segment_size keys of every row written row after row. */
+int thor_topk(thor_tensor_t keys_in, thor_tensor_t keys_out, thor_tensor_t values_in, thor_tensor_t values_out, uint64_t num_segments,
+              uint64_t segment_size, uint64_t k, int largest, int segmented, thor_stream_t stream, char* variant, size_t variant_capacity);
+
 /* thor_scan for callers that cannot allocate (work recorded under stream capture, serving loops, harnesses that forbid
  * hipMalloc).  It has no counterpart in the reference.  Same arguments, kernels and results as thor_scan, but the temporary
  * storage (segment-head bitmap, chunk totals and carries) is a fixed 4 MiB block of device memory that is part of the library's

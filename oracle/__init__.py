@@ -338,6 +338,49 @@ def scan(values: np.ndarray, op: int, inclusive: bool = True, reverse: bool = Fa
 ROPE_NONE, ROPE_LINEAR, ROPE_DYNAMIC_NTK, ROPE_YARN, ROPE_LONGROPE, ROPE_LLAMA3 = 0, 1, 2, 3, 4, 5
 
 
+def select_flagged(values: np.ndarray, flags: np.ndarray):
+    """The elements of `values` whose flag is nonzero, in input order, and their number: what cub::DeviceSelect::Flagged
+    documents and the reference relies on (Utilities/TensorOperations/Cub/CubSelect.cu:43-50; CUB is a third-party library
+    that is not part of the reference tree).  Carriers pass through untouched."""
+    flat = np.ascontiguousarray(values).reshape(-1)
+    raised = np.ascontiguousarray(flags).reshape(-1) != 0
+    kept = flat[raised[:flat.size]] if flat.size else flat[:0]
+    return kept, int(kept.size)
+
+
+def key_order_image(keys: np.ndarray, dtype: int) -> np.ndarray:
+    """An int64 per key that sorts like the key does for the reference's selection library: integers by value, floats by sign
+    and magnitude of their bits, so -0 sorts below +0 and NaNs beyond the infinities (the radix order cub documents for
+    floating-point keys)."""
+    flat = np.ascontiguousarray(keys).reshape(-1)
+    if dtype in (UINT8, UINT16, UINT32, INT8, INT16, INT32):
+        return flat.astype(np.int64)
+    width = {FP16: 16, BF16: 16, FP32: 32}[dtype]
+    bits = flat.view({16: np.uint16, 32: np.uint32}[width]).astype(np.int64)
+    sign = 1 << (width - 1)
+    magnitude = bits & (sign - 1)
+    return np.where(bits & sign, -magnitude - 1, magnitude)
+
+
+def top_k(keys: np.ndarray, k: int, largest: bool = True, dtype: int = FP32, segment_size: int = 0):
+    """The k largest (or smallest) keys of the flat array, or of every run of `segment_size` keys, best first; k is capped at
+    the run length (Utilities/TensorOperations/Cub/CubTopK.cu:27-60,333-420 device-wide, :120-330,520-735 fixed-size segments;
+    the selection itself is cub's).  The reference's output is unordered and which of several equal keys is taken is not
+    fixed, so callers compare sorted keys; returns (keys [segments, k] as carriers, positions [segments, k] of one valid
+    choice, and the order image of the k-th key per segment, which decides whether a candidate answer is admissible)."""
+    flat = np.ascontiguousarray(keys).reshape(-1)
+    run = segment_size if segment_size else flat.size
+    if run == 0:
+        return flat[:0].reshape(0, 0), np.zeros((0, 0), np.int64), np.zeros((0,), np.int64)
+    image = key_order_image(flat, dtype).reshape(-1, run)
+    take = min(k, run)
+    ranked = np.argsort(-image if largest else image, axis=1, kind="stable")[:, :take]
+    positions = ranked + np.arange(image.shape[0])[:, None] * run
+    chosen = flat[positions.reshape(-1)].reshape(image.shape[0], take)
+    threshold = np.take_along_axis(image, ranked[:, take - 1:take], axis=1)[:, 0] if take else np.zeros((image.shape[0],), np.int64)
+    return chosen, positions, threshold
+
+
 def rope_attention_factor(scaling_kind=ROPE_NONE, scaling_factor=1.0, original_max_position_embeddings=0, attention_factor=None):
     """The magnitude correction a ROPE node carries (Utilities/Expression/Expression.cpp:4398-4413): the caller's, else
     0.1 ln(s) + 1 for YaRN and sqrt(1 + ln(s) / ln(original_max)) for LongRoPE when s > 1, else 1."""

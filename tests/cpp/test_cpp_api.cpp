@@ -14,6 +14,7 @@
 #include "Utilities/TensorOperations/Cub/CubReduction.h"
 #include "Utilities/TensorOperations/DataTypeConversions/TypeConverter.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -25,6 +26,7 @@
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 using namespace ThorImplementation;
@@ -753,6 +755,146 @@ static void devicePrefixScans(Stream& stream) {
     CHECK((toHostRaw<uint32_t>(plan.output("y"), stream) == std::vector<uint32_t>{2, 3, 3, 4, 5, 5, 5, 5}));
 }
 
+static void deviceSelectAndTopK(Stream& stream) {
+    // plan / shared temporary storage / run of select-flagged and the four top-k families, on the reference's literal vectors
+    // (CubDevicePrimitivesTest.cpp:664-1030 there: TopKKeysLargestAndSmallestUseCubDeviceTopK, TopKPairsCarriesUint32IndexValues,
+    // TopKCapsKToNumItems, SelectFlagged*, SegmentedTopK*, the *Rejects* cases)
+    auto upload = [&](const std::vector<uint32_t>& v) {
+        Tensor host(cpuPlacement, TensorDescriptor(DataType::UINT32, {v.size()}));
+        std::memcpy(host.getMemPtr<uint32_t>(), v.data(), v.size() * 4);
+        Tensor device(gpuPlacement, TensorDescriptor(DataType::UINT32, {v.size()}));
+        device.copyFromAsync(host, stream);
+        stream.synchronize();
+        return device;
+    };
+    auto uploadBytes = [&](const std::vector<uint8_t>& v, DataType dtype) {
+        Tensor host(cpuPlacement, TensorDescriptor(dtype, {v.size()}));
+        std::memcpy(host.getMemPtr(), v.data(), v.size());
+        Tensor device(gpuPlacement, TensorDescriptor(dtype, {v.size()}));
+        device.copyFromAsync(host, stream);
+        stream.synchronize();
+        return device;
+    };
+    {
+        const Tensor keys = upload({5, 3, 1, 7, 8, 2, 4, 6});
+        Tensor largestOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {3})), smallestOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {4}));
+        const CubDeviceTopKKeysPlan largest = prepareCubDeviceTopKKeys(keys, largestOut, 8, 3, CubTopKOrder::Largest);
+        const CubDeviceTopKKeysPlan smallest = prepareCubDeviceTopKKeys(keys, smallestOut, 8, 4, CubTopKOrder::Smallest);
+        CHECK(largest.key_dtype == DataType::UINT32 && largest.num_items == 8 && largest.k == 3 && largest.order == CubTopKOrder::Largest);
+        CHECK(cubDeviceTopKKeysTempBytes(keys, largestOut, 8, 3, CubTopKOrder::Largest) == largest.temp_storage_bytes);
+        const CubTemporaryStoragePlan shared = cubMaxTemporaryStoragePlan(
+            {cubTemporaryStoragePlan(gpuPlacement, largest.temp_storage_bytes), cubTemporaryStoragePlan(gpuPlacement, smallest.temp_storage_bytes)});
+        CHECK(shared.bytes >= largest.temp_storage_bytes && shared.bytes >= smallest.temp_storage_bytes);
+        const Tensor temp = allocateCubTemporaryStorage(shared);
+        cubDeviceTopKKeys(largest, temp, keys, largestOut, stream);
+        cubDeviceTopKKeys(smallest, temp, keys, smallestOut, stream);
+        std::vector<uint32_t> l = toHostRaw<uint32_t>(largestOut, stream), sm = toHostRaw<uint32_t>(smallestOut, stream);
+        std::sort(l.begin(), l.end(), std::greater<uint32_t>());
+        std::sort(sm.begin(), sm.end());
+        CHECK((l == std::vector<uint32_t>{8, 7, 6}));
+        CHECK((sm == std::vector<uint32_t>{1, 2, 3, 4}));
+        // k beyond the input is capped; the one-call form takes the byte count
+        const Tensor three = upload({5, 3, 7});
+        Tensor capped(gpuPlacement, TensorDescriptor(DataType::UINT32, {3}));
+        cubDeviceTopKKeys(temp, shared.bytes, three, capped, 3, 99, stream);
+        std::vector<uint32_t> c = toHostRaw<uint32_t>(capped, stream);
+        std::sort(c.begin(), c.end(), std::greater<uint32_t>());
+        CHECK((c == std::vector<uint32_t>{7, 5, 3}));
+        CHECK(throwsAs<std::invalid_argument>([&] { cubDeviceTopKKeys(temp, 1, three, capped, 3, 2, stream); }));
+        CHECK(throwsAs<std::invalid_argument>([&] { cubDeviceTopKKeys(largest, allocateCubTemporaryStorage(gpuPlacement, 1), keys, largestOut, stream); }));
+        Tensor fpOut(gpuPlacement, TensorDescriptor(DataType::FP32, {2})), smallOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {1}));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceTopKKeys(three, fpOut, 3, 2); }));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceTopKKeys(three, smallOut, 3, 2); }));
+        const Tensor fp8In(gpuPlacement, TensorDescriptor(DataType::FP8_E4M3, {2}));
+        Tensor fp8Out(gpuPlacement, TensorDescriptor(DataType::FP8_E4M3, {1}));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceTopKKeys(fp8In, fp8Out, 2, 1); }));
+        CHECK(isCubTopKKeyDTypeSupported(DataType::BF16) && !isCubTopKKeyDTypeSupported(DataType::FP8_E4M3) && !isCubTopKKeyDTypeSupported(DataType::UINT64));
+        CHECK(isCubTopKValueDTypeSupported(DataType::UINT32) && !isCubTopKValueDTypeSupported(DataType::FP32));
+    }
+    {
+        const Tensor keys = gpuFrom({5.0f, -3.0f, 1.0f, 7.0f, 8.0f, 2.0f, 4.0f, 6.0f}, {8}, stream);
+        const Tensor values = upload({0, 1, 2, 3, 4, 5, 6, 7});
+        Tensor keysOut(gpuPlacement, TensorDescriptor(DataType::FP32, {4})), valuesOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {4}));
+        const CubDeviceTopKPairsPlan plan = prepareCubDeviceTopKPairs(keys, keysOut, values, valuesOut, 8, 4, CubTopKOrder::Largest);
+        CHECK(plan.value_dtype == DataType::UINT32);
+        cubDeviceTopKPairs(plan, allocateCubTemporaryStorage(cubTemporaryStoragePlan(gpuPlacement, plan.temp_storage_bytes)), keys, keysOut, values, valuesOut,
+                           stream);
+        const std::vector<float> k = toHostF32(keysOut, stream);
+        const std::vector<uint32_t> v = toHostRaw<uint32_t>(valuesOut, stream);
+        std::vector<std::pair<float, uint32_t>> pairs;
+        for (size_t i = 0; i < k.size(); ++i) pairs.emplace_back(k[i], v[i]);
+        std::sort(pairs.begin(), pairs.end(), [](const auto& a, const auto& b) { return a.first > b.first; });
+        CHECK((pairs == std::vector<std::pair<float, uint32_t>>{{8.0f, 4u}, {7.0f, 3u}, {6.0f, 7u}, {5.0f, 0u}}));
+        const Tensor fpValues = gpuFrom({10.0f, 20.0f, 30.0f}, {3}, stream);
+        Tensor fpValuesOut(gpuPlacement, TensorDescriptor(DataType::FP32, {2}));
+        const Tensor three = upload({1, 2, 3});
+        Tensor twoOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {2}));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceTopKPairs(three, twoOut, fpValues, fpValuesOut, 3, 2); }));
+    }
+    {
+        const Tensor input = upload({10, 20, 30, 40, 50, 60});
+        const Tensor flags = uploadBytes({1, 0, 1, 0, 0, 1}, DataType::BOOLEAN);
+        Tensor output(gpuPlacement, TensorDescriptor(DataType::UINT32, {6})), count(gpuPlacement, TensorDescriptor(DataType::UINT32, {1}));
+        const CubDeviceSelectFlaggedPlan plan = prepareCubDeviceSelectFlagged(input, flags, output, count, 6);
+        CHECK(plan.input_dtype == DataType::UINT32 && plan.flag_dtype == DataType::BOOLEAN && plan.num_items == 6);
+        CHECK(cubDeviceSelectFlaggedTempBytes(input, flags, output, count, 6) == plan.temp_storage_bytes);
+        const Tensor temp = allocateCubTemporaryStorage(cubTemporaryStoragePlan(gpuPlacement, plan.temp_storage_bytes));
+        cubDeviceSelectFlagged(plan, temp, input, flags, output, count, stream);
+        CHECK((toHostRaw<uint32_t>(count, stream) == std::vector<uint32_t>{3}));
+        const std::vector<uint32_t> selected = toHostRaw<uint32_t>(output, stream);
+        CHECK((std::vector<uint32_t>(selected.begin(), selected.begin() + 3) == std::vector<uint32_t>{10, 30, 60}));
+        // no items: only the count is written
+        Tensor dirty = upload({77});
+        const Tensor byteFlags = uploadBytes({1}, DataType::UINT8);
+        Tensor one(gpuPlacement, TensorDescriptor(DataType::UINT32, {1}));
+        const CubDeviceSelectFlaggedPlan none = prepareCubDeviceSelectFlagged(upload({123}), byteFlags, one, dirty, 0);
+        cubDeviceSelectFlagged(none, allocateCubTemporaryStorage(gpuPlacement, none.temp_storage_bytes), upload({123}), byteFlags, one, dirty, stream);
+        CHECK((toHostRaw<uint32_t>(dirty, stream) == std::vector<uint32_t>{0}));
+        const Tensor fpFlags(gpuPlacement, TensorDescriptor(DataType::FP32, {6}));
+        Tensor fpOut(gpuPlacement, TensorDescriptor(DataType::FP32, {6})), fpCount(gpuPlacement, TensorDescriptor(DataType::FP32, {1}));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceSelectFlagged(input, fpFlags, output, count, 6); }));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceSelectFlagged(input, flags, fpOut, count, 6); }));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceSelectFlagged(input, flags, output, fpCount, 6); }));
+        CHECK(throwsAs<std::invalid_argument>([&] { cubDeviceSelectFlagged(temp, 0, input, flags, output, count, 6, stream); }));
+        CHECK(isCubSelectFlagDTypeSupported(DataType::BOOLEAN) && isCubSelectFlagDTypeSupported(DataType::UINT8) && !isCubSelectFlagDTypeSupported(DataType::UINT32));
+        CHECK(isCubSelectValueDTypeSupported(DataType::FP16) && !isCubSelectValueDTypeSupported(DataType::FP8_E5M2));
+    }
+    {
+        const Tensor keys = upload({1, 5, 3, 9, 2, 10, 4, 8, 6, 7, 11, 15, 12, 14, 13});
+        Tensor largestOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {6})), smallestOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {6}));
+        const CubDeviceSegmentedTopKKeysPlan largest = prepareCubDeviceSegmentedTopKKeys(keys, largestOut, 3, 5, 2, CubTopKOrder::Largest);
+        const CubDeviceSegmentedTopKKeysPlan smallest = prepareCubDeviceSegmentedTopKKeys(keys, smallestOut, 3, 5, 2, CubTopKOrder::Smallest);
+        CHECK(largest.num_segments == 3 && largest.segment_size == 5 && largest.k == 2);
+        const Tensor temp = allocateCubTemporaryStorage(cubMaxTemporaryStoragePlan(
+            {cubTemporaryStoragePlan(gpuPlacement, largest.temp_storage_bytes), cubTemporaryStoragePlan(gpuPlacement, smallest.temp_storage_bytes)}));
+        cubDeviceSegmentedTopKKeys(largest, temp, keys, largestOut, stream);
+        cubDeviceSegmentedTopKKeys(smallest, temp, keys, smallestOut, stream);
+        std::vector<uint32_t> l = toHostRaw<uint32_t>(largestOut, stream), sm = toHostRaw<uint32_t>(smallestOut, stream);
+        for (size_t at = 0; at < 6; at += 2) {
+            std::sort(l.begin() + at, l.begin() + at + 2, std::greater<uint32_t>());
+            std::sort(sm.begin() + at, sm.begin() + at + 2);
+        }
+        CHECK((l == std::vector<uint32_t>{9, 5, 10, 8, 15, 14}));
+        CHECK((sm == std::vector<uint32_t>{1, 2, 4, 6, 11, 12}));
+        const Tensor floatKeys = gpuFrom({1, 5, 3, 9, 2, 10, 4, 8, 6, 7, 11, 15, 12, 14, 13}, {15}, stream);
+        const Tensor values = upload({100, 101, 102, 103, 104, 200, 201, 202, 203, 204, 300, 301, 302, 303, 304});
+        Tensor keysOut(gpuPlacement, TensorDescriptor(DataType::FP32, {6})), valuesOut(gpuPlacement, TensorDescriptor(DataType::UINT32, {6}));
+        const CubDeviceSegmentedTopKPairsPlan pairsPlan = prepareCubDeviceSegmentedTopKPairs(floatKeys, keysOut, values, valuesOut, 3, 5, 2, CubTopKOrder::Largest);
+        cubDeviceSegmentedTopKPairs(pairsPlan, temp, floatKeys, keysOut, values, valuesOut, stream);
+        const std::vector<float> k = toHostF32(keysOut, stream);
+        const std::vector<uint32_t> v = toHostRaw<uint32_t>(valuesOut, stream);
+        std::vector<std::pair<float, uint32_t>> pairs;
+        for (size_t i = 0; i < k.size(); ++i) pairs.emplace_back(k[i], v[i]);
+        for (size_t at = 0; at < 6; at += 2) std::sort(pairs.begin() + at, pairs.begin() + at + 2, [](const auto& a, const auto& b) { return a.first > b.first; });
+        CHECK((pairs == std::vector<std::pair<float, uint32_t>>{{9.0f, 103u}, {5.0f, 101u}, {10.0f, 200u}, {8.0f, 202u}, {15.0f, 301u}, {14.0f, 303u}}));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceSegmentedTopKKeys(keys, largestOut, 3, 5, 5); }));  // k must stay below the segment
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceSegmentedTopKKeys(keys, largestOut, 3, 0, 1); }));
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)prepareCubDeviceSegmentedTopKKeys(keys, largestOut, 4, 5, 1); }));  // keys_in too small
+        const CubDeviceSegmentedTopKKeysPlan nothing = prepareCubDeviceSegmentedTopKKeys(keys, largestOut, 3, 5, 0);
+        cubDeviceSegmentedTopKKeys(nothing, temp, keys, largestOut, stream);  // k == 0: nothing to do, nothing thrown
+    }
+}
+
 static void softmaxPlansAndRowKernel(Stream& stream) {
     const uint64_t rows = 7, cols = 130;
     std::vector<float> x(rows * cols);
@@ -1040,6 +1182,7 @@ int main(int argc, char** argv) {
         cases.push_back({"softmaxPlansAndRowKernel", withStream(softmaxPlansAndRowKernel)});
         cases.push_back({"autodiffExecution", withStream(autodiffExecution)});
         cases.push_back({"devicePrefixScans", withStream(devicePrefixScans)});
+        cases.push_back({"deviceSelectAndTopK", withStream(deviceSelectAndTopK)});
         cases.push_back({"ropeExecution", withStream(ropeExecution)});
         cases.push_back({"stagePlanForksAndJoins", withStream(stagePlanForksAndJoins)});
         cases.push_back({"boundaryRequestedShapesAndSubstitutionExecution", withStream(boundaryRequestedShapesAndSubstitutionExecution)});

@@ -1,0 +1,297 @@
+"""Select-flagged and top-k through the C-ABI (thor_select_flagged / thor_topk over cubDeviceSelectFlagged, cubDeviceTopKKeys / Pairs
+and cubDeviceSegmentedTopKKeys / Pairs) against the oracle.  The compaction is compared bit for bit, in order.  Top-k output is
+unordered in the reference and which of several equal keys is taken is not fixed, so the keys are compared bit for bit after
+sorting, and the values of pairs by what they point at: every returned (key, value) pair must be a pair of the input and no input
+position may be returned twice."""
+from __future__ import annotations
+
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import copy_gpu_to_numpy, copy_numpy_to_gpu, gpu_tensor, to_storage
+from thor_amd import physical as ph
+from thor_amd.dtypes import DataType, numpy_carrier
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "selection_kats.json")) as f:
+    KATS = json.load(f)
+KEY_DTYPES = [DataType.uint8, DataType.int8, DataType.uint16, DataType.int16, DataType.uint32, DataType.int32, DataType.fp16, DataType.bf16,
+              DataType.fp32]
+FLOATS = (DataType.fp16, DataType.bf16, DataType.fp32)
+
+
+@pytest.fixture(scope="module")
+def stream(gpu):
+    return ph.Stream(0)
+
+
+def carriers(values, dtype):
+    if dtype in FLOATS:
+        return to_storage(np.array(values, np.float32), dtype)
+    return np.array(values, numpy_carrier(dtype))
+
+
+def random_keys(rng, n, dtype, distinct_levels=None):
+    if dtype in FLOATS:
+        values = rng.standard_normal(n).astype(np.float32) * 100
+        if distinct_levels:
+            values = np.round(values / 100 * distinct_levels)
+        return to_storage(values, dtype)
+    info = np.iinfo(numpy_carrier(dtype))
+    low, high = (info.min, int(info.max) + 1) if not distinct_levels else (max(info.min, -distinct_levels), min(int(info.max) + 1, distinct_levels))
+    return rng.integers(low, high, n).astype(numpy_carrier(dtype))
+
+
+def bits_of(carrier):
+    return np.ascontiguousarray(carrier).view({1: np.uint8, 2: np.uint16, 4: np.uint32}[carrier.dtype.itemsize])
+
+
+def sorted_by_order(carrier, dtype, largest):
+    image = oracle.key_order_image(carrier, int(dtype))
+    order = np.argsort(-image if largest else image, kind="stable")
+    return bits_of(carrier.reshape(-1))[order]
+
+
+# ---- select-flagged ----------------------------------------------------------------------------------------------------------------
+def run_select(values, flags, dtype, flag_dtype, stream, num_items=None, count_before=77):
+    n = values.size if num_items is None else num_items
+    x = copy_numpy_to_gpu(values, stream, dtype)
+    f = copy_numpy_to_gpu(flags, stream, flag_dtype)
+    out = copy_numpy_to_gpu(np.zeros(max(values.size, 1), numpy_carrier(dtype)), stream, dtype)
+    count = copy_numpy_to_gpu(np.array([count_before], np.uint32), stream, DataType.uint32)
+    variant = ph.select_flagged(x, f, out, count, stream, num_items=n)
+    return copy_gpu_to_numpy(out, stream), int(copy_gpu_to_numpy(count, stream)[0]), variant
+
+
+@pytest.mark.parametrize("case", KATS["select"], ids=lambda c: f"{c['dtype']}-{c['num_items']}")
+def test_select_reference_vectors(stream, case):
+    dtype, flag_dtype = DataType[case["dtype"]], DataType[case["flag_dtype"]]
+    values = carriers(case["values"], dtype)
+    got, count, _ = run_select(values, np.array(case["flags"], np.uint8), dtype, flag_dtype, stream, case["num_items"])
+    assert count == len(case["expected"])
+    np.testing.assert_array_equal(bits_of(got[:count]), bits_of(carriers(case["expected"], dtype)))
+
+
+@pytest.mark.parametrize("dtype", KEY_DTYPES, ids=lambda d: d.name)
+@pytest.mark.parametrize("n", [1, 63, 4095, 4096, 4097, 1_000_003])
+def test_select_keeps_the_flagged_elements_in_order(stream, dtype, n):
+    rng = np.random.default_rng(n * 31 + int(dtype))
+    values = random_keys(rng, n, dtype)
+    flags = ((rng.random(n) < 0.37) * rng.integers(1, 256, n)).astype(np.uint8)
+    got, count, variant = run_select(values, flags, dtype, DataType.uint8, stream)
+    expected, expected_count = oracle.select_flagged(values, flags)
+    assert count == expected_count and "select-flagged" in variant
+    np.testing.assert_array_equal(bits_of(got[:count]), bits_of(expected))
+    np.testing.assert_array_equal(bits_of(got[count:]), 0)  # nothing is written past the selected elements
+
+
+@pytest.mark.parametrize("density", [0.0, 1.0, 0.001, 0.999])
+def test_select_at_extreme_densities_with_boolean_flags(stream, density):
+    n = 300_000
+    rng = np.random.default_rng(int(density * 1000) + 1)
+    values = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    flags = (rng.random(n) < density).astype(np.uint8)
+    got, count, _ = run_select(values, flags, DataType.uint32, DataType.boolean, stream)
+    expected, expected_count = oracle.select_flagged(values, flags)
+    assert count == expected_count
+    np.testing.assert_array_equal(got[:count], expected)
+
+
+def test_select_over_a_prefix_of_larger_tensors(stream):
+    rng = np.random.default_rng(8)
+    values = rng.standard_normal(10_000).astype(np.float32)
+    flags = (rng.random(10_000) < 0.5).astype(np.uint8)
+    got, count, _ = run_select(values, flags, DataType.fp32, DataType.uint8, stream, num_items=6_001)
+    expected, expected_count = oracle.select_flagged(values[:6_001], flags[:6_001])
+    assert count == expected_count
+    np.testing.assert_array_equal(got[:count], expected)
+
+
+def test_select_full_size_partition_round_trip(stream):
+    """2^26 elements: the flagged elements and the unflagged ones together are the input, each part in input order."""
+    n = 1 << 26
+    rng = np.random.default_rng(26)
+    values = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    flags = (rng.random(n) < 0.5).astype(np.uint8)
+    kept, kept_count, _ = run_select(values, flags, DataType.uint32, DataType.uint8, stream)
+    dropped, dropped_count, _ = run_select(values, 1 - flags, DataType.uint32, DataType.uint8, stream)
+    assert kept_count == int(flags.sum()) and kept_count + dropped_count == n
+    merged = np.empty(n, np.uint32)
+    merged[flags != 0] = kept[:kept_count]
+    merged[flags == 0] = dropped[:dropped_count]
+    np.testing.assert_array_equal(merged, values)
+
+
+def test_select_rejects_what_the_reference_rejects(stream):
+    x = gpu_tensor([4], DataType.uint32)
+    flags = gpu_tensor([4], DataType.uint8)
+    count = gpu_tensor([1], DataType.uint32)
+    with pytest.raises(ValueError, match="input/output dtypes must match"):
+        ph.select_flagged(x, flags, gpu_tensor([4], DataType.fp32), count, stream)
+    with pytest.raises(ValueError, match="Unsupported CUB select flag dtype"):
+        ph.select_flagged(x, gpu_tensor([4], DataType.fp32), gpu_tensor([4], DataType.uint32), count, stream)
+    with pytest.raises(ValueError, match="num_selected_out must have dtype uint32"):
+        ph.select_flagged(x, flags, gpu_tensor([4], DataType.uint32), gpu_tensor([1], DataType.fp32), stream)
+    with pytest.raises(ValueError, match="output has fewer elements than num_items"):
+        ph.select_flagged(x, flags, gpu_tensor([3], DataType.uint32), count, stream)
+    with pytest.raises(ValueError, match="Unsupported CUB select value dtype"):
+        ph.select_flagged(gpu_tensor([4], DataType.fp8_e4m3), flags, gpu_tensor([4], DataType.fp8_e4m3), count, stream)
+
+
+# ---- top-k -------------------------------------------------------------------------------------------------------------------------
+def run_top_k(keys, dtype, k, largest, stream, pairs=False, segment_size=None, values=None):
+    flat = keys.reshape(-1)
+    run = segment_size if segment_size else flat.size
+    segments = flat.size // run if run else 0
+    take = min(k, run)
+    x = copy_numpy_to_gpu(flat, stream, dtype)
+    out = copy_numpy_to_gpu(np.zeros(max(segments * take, 1), numpy_carrier(dtype)), stream, dtype)
+    values_in = values_out = None
+    if pairs:
+        values = np.arange(flat.size, dtype=np.uint32) if values is None else np.asarray(values, np.uint32)
+        values_in = copy_numpy_to_gpu(values, stream, DataType.uint32)
+        values_out = copy_numpy_to_gpu(np.full(max(segments * take, 1), 0xffffffff, np.uint32), stream, DataType.uint32)
+    variant = ph.top_k(x, out, k, stream, largest=largest, values_in=values_in, values_out=values_out,
+                       **({"segment_size": segment_size, "num_segments": segments} if segment_size else {"num_items": flat.size}))
+    got = copy_gpu_to_numpy(out, stream)[:segments * take].reshape(segments, take)
+    got_values = copy_gpu_to_numpy(values_out, stream)[:segments * take].reshape(segments, take) if pairs else None
+    return got, got_values, variant
+
+
+def check_top_k(keys, dtype, k, largest, got, got_values, segment_size=None):
+    flat = keys.reshape(-1)
+    expected, _, _ = oracle.top_k(flat, k, largest, int(dtype), segment_size or 0)
+    assert got.shape == expected.shape
+    for row in range(expected.shape[0]):
+        np.testing.assert_array_equal(sorted_by_order(got[row], dtype, largest), bits_of(expected[row]))
+    if got_values is not None:
+        run = segment_size or flat.size
+        for row in range(expected.shape[0]):
+            positions = got_values[row].astype(np.int64)
+            assert len(np.unique(positions)) == positions.size
+            assert positions.min() >= row * run and positions.max() < (row + 1) * run
+            np.testing.assert_array_equal(bits_of(flat[positions]), bits_of(got[row]))
+
+
+@pytest.mark.parametrize("case", KATS["topk"] + KATS["segmented_topk"],
+                         ids=lambda c: f"{c['dtype']}-k{c['k']}-{'largest' if c['largest'] else 'smallest'}-{c.get('segments', 0)}")
+def test_top_k_reference_vectors(stream, case):
+    dtype = DataType[case["dtype"]]
+    keys = carriers(case["keys"], dtype)
+    segment_size = case.get("segment_size")
+    got, got_values, _ = run_top_k(keys, dtype, case["k"], case["largest"], stream, pairs="values" in case, segment_size=segment_size,
+                                   values=case.get("values"))
+    expected = carriers(case["expected"], dtype).reshape(got.shape)
+    for row in range(got.shape[0]):
+        np.testing.assert_array_equal(sorted_by_order(got[row], dtype, case["largest"]), bits_of(expected[row]))
+    if "values" in case:
+        pairs = sorted(zip(bits_of(got.reshape(-1)).tolist(), got_values.reshape(-1).tolist()))
+        assert pairs == sorted(zip(bits_of(expected.reshape(-1)).tolist(), case["expected_values"]))
+
+
+@pytest.mark.parametrize("dtype", KEY_DTYPES, ids=lambda d: d.name)
+@pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
+@pytest.mark.parametrize("n,k", [(1, 1), (257, 256), (2049, 2049), (100_003, 1), (100_003, 1000), (1_000_000, 65_537)])
+def test_top_k_keys(stream, dtype, largest, n, k):
+    rng = np.random.default_rng(n * 7 + k + int(dtype))
+    keys = random_keys(rng, n, dtype)
+    got, _, variant = run_top_k(keys, dtype, k, largest, stream)
+    assert "radix-select" in variant
+    check_top_k(keys, dtype, k, largest, got, None)
+
+
+@pytest.mark.parametrize("dtype", [DataType.uint8, DataType.int16, DataType.fp16, DataType.fp32, DataType.uint32], ids=lambda d: d.name)
+@pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
+def test_top_k_pairs_with_many_equal_keys(stream, dtype, largest):
+    rng = np.random.default_rng(int(dtype) + 100)
+    keys = random_keys(rng, 200_000, dtype, distinct_levels=20)
+    for k in (1, 4_000, 150_000):
+        got, got_values, _ = run_top_k(keys, dtype, k, largest, stream, pairs=True)
+        check_top_k(keys, dtype, k, largest, got, got_values)
+
+
+def test_top_k_of_equal_keys_and_k_beyond_the_input(stream):
+    keys = np.full(10_000, 7, np.uint32)
+    got, got_values, _ = run_top_k(keys, DataType.uint32, 99_999, True, stream, pairs=True)
+    check_top_k(keys, DataType.uint32, 99_999, True, got, got_values)
+    assert got.shape == (1, 10_000)
+
+
+def test_top_k_float_specials(stream):
+    """-0 below +0, infinities at the ends, NaNs beyond them by sign: the order of the key bits."""
+    specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 1e-45, -1e-45], np.float32)
+    negative_nan = np.frombuffer(np.uint32(0xffc00001).tobytes(), np.float32)
+    rng = np.random.default_rng(4)
+    keys = np.concatenate([specials, negative_nan, rng.standard_normal(5_000).astype(np.float32)])
+    rng.shuffle(keys)
+    for largest in (True, False):
+        for k in (1, 2, 3, 5, 2_505):
+            got, _, _ = run_top_k(keys, DataType.fp32, k, largest, stream)
+            check_top_k(keys, DataType.fp32, k, largest, got, None)
+
+
+def test_top_k_zero_k_leaves_the_output_alone(stream):
+    keys = copy_numpy_to_gpu(np.arange(8, dtype=np.uint32), stream, DataType.uint32)
+    out = copy_numpy_to_gpu(np.full(4, 99, np.uint32), stream, DataType.uint32)
+    assert ph.top_k(keys, out, 0, stream) == ""
+    np.testing.assert_array_equal(copy_gpu_to_numpy(out, stream), 99)
+
+
+@pytest.mark.parametrize("dtype", KEY_DTYPES, ids=lambda d: d.name)
+@pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
+@pytest.mark.parametrize("segments,segment_size,k", [(1, 2, 1), (33, 257, 256), (100, 1000, 10), (16, 8192, 8191), (3000, 64, 8)])
+def test_top_k_of_rows(stream, dtype, largest, segments, segment_size, k):
+    rng = np.random.default_rng(segments * 13 + segment_size + k + int(dtype))
+    keys = random_keys(rng, segments * segment_size, dtype)
+    got, got_values, variant = run_top_k(keys, dtype, k, largest, stream, pairs=True, segment_size=segment_size)
+    assert "row top-k" in variant
+    check_top_k(keys, dtype, k, largest, got, got_values, segment_size=segment_size)
+
+
+def test_top_k_of_rows_keys_only_with_ties(stream):
+    rng = np.random.default_rng(77)
+    keys = random_keys(rng, 512 * 300, DataType.bf16, distinct_levels=6)
+    got, _, _ = run_top_k(keys, DataType.bf16, 100, True, stream, segment_size=300)
+    check_top_k(keys, DataType.bf16, 100, True, got, None, segment_size=300)
+
+
+def test_top_k_full_size_against_a_host_partition(stream):
+    """2^26 fp32 keys, k = 2^16: the answer's smallest key is the k-th largest of the input and every key above it is present
+    (checked with NumPy's partition, which shares nothing with the radix selection)."""
+    n, k = 1 << 26, 1 << 16
+    rng = np.random.default_rng(2026)
+    keys = rng.standard_normal(n).astype(np.float32)
+    got, got_values, _ = run_top_k(keys, DataType.fp32, k, True, stream, pairs=True)
+    kth = np.partition(keys, n - k)[n - k]
+    assert got.min() == kth
+    assert int((keys > kth).sum()) == int((got > kth).sum())
+    positions = got_values.reshape(-1).astype(np.int64)
+    assert len(np.unique(positions)) == k
+    np.testing.assert_array_equal(keys[positions], got.reshape(-1))
+    np.testing.assert_array_equal(np.sort(got.reshape(-1)), np.sort(np.partition(keys, n - k)[n - k:]))
+
+
+def test_top_k_rejects_what_the_reference_rejects(stream):
+    keys = gpu_tensor([15], DataType.uint32)
+    with pytest.raises(ValueError, match="key input/output dtypes must match"):
+        ph.top_k(keys, gpu_tensor([2], DataType.fp32), 2, stream)
+    with pytest.raises(ValueError, match="Unsupported CUB top-k key dtype"):
+        ph.top_k(gpu_tensor([2], DataType.fp8_e4m3), gpu_tensor([1], DataType.fp8_e4m3), 1, stream)
+    with pytest.raises(ValueError, match="Unsupported CUB top-k index value dtype"):
+        ph.top_k(keys, gpu_tensor([2], DataType.uint32), 2, stream, values_in=gpu_tensor([15], DataType.fp32), values_out=gpu_tensor([2], DataType.fp32))
+    with pytest.raises(ValueError, match="keys_out has fewer elements than num_items"):
+        ph.top_k(keys, gpu_tensor([1], DataType.uint32), 2, stream)
+    with pytest.raises(ValueError, match="requires k to be smaller than the fixed segment size"):
+        ph.top_k(keys, gpu_tensor([15], DataType.uint32), 5, stream, segment_size=5, num_segments=3)
+    with pytest.raises(ValueError, match="segment_size exceeds"):
+        ph.top_k(gpu_tensor([8193 * 2], DataType.uint32), gpu_tensor([2], DataType.uint32), 1, stream, segment_size=8193, num_segments=2)
+    with pytest.raises(ValueError, match="segment_size must be nonzero"):
+        ph.top_k(keys, gpu_tensor([3], DataType.uint32), 1, stream, segment_size=0, num_segments=3)
+    with pytest.raises(ValueError, match="Unsupported CUB segmented top-k key dtype"):
+        ph.top_k(gpu_tensor([4], DataType.fp64), gpu_tensor([2], DataType.fp64), 1, stream, segment_size=2, num_segments=2)

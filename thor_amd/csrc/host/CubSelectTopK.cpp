@@ -1,0 +1,573 @@
+// Select-flagged and top-k: validation, kernel specialisation and launch (kernels: device/thor_device_select.h; reference
+// behaviour: Utilities/TensorOperations/Cub/CubSelect.cu:54-136 plan / run protocol, CubTopK.cu:333-735 the four top-k families,
+// CubDevicePrimitiveSupport.cpp:116-182,225-330 argument checks and the fixed-size limits of the row form).
+#include "Utilities/TensorOperations/Cub/CubDevicePrimitives.h"
+
+#include "Utilities/Common/ScopedGpu.h"
+#include "Utilities/Expression/CompiledEquation.h"
+#include "thorhip_numeric_embed.h"
+
+#include <algorithm>
+#include <limits>
+#include <sstream>
+#include <stdexcept>
+#include <vector>
+
+namespace ThorImplementation {
+
+// What one plan launches.  kind 0: select-flagged (count, offsets, scatter); 1: device-wide top-k (init, then histogram + pick per
+// digit, gather); 2: top-k of rows (one launch).  A plan with nothing to do (no items, k == 0) holds no kernels.
+struct CubSelectionKernels {
+    int kind = 0;
+    int deviceNum = 0;
+    std::shared_ptr<CompiledKernel> first, second, third, fourth;
+    uint64_t chunks = 0;          // blocks of the counting / scattering / gathering launches; rows for kind 2
+    uint32_t histogramBlocks = 0;
+    uint32_t threads = 256;
+    int digits = 0;
+    size_t countsBytes = 0;  // select: chunk counts, then as many chunk bases
+    size_t tempBytes = 1;
+    std::string variant;
+};
+
+namespace {
+
+constexpr uint64_t kRowTopKMaxSegment = 8192, kRowTopKMaxK = 8192;
+constexpr uint32_t kSelectThreads = 256, kSelectItems = 16;
+constexpr uint32_t kGatherThreads = 256, kGatherItems = 8;
+
+size_t roundUp(size_t v, size_t to) { return (v + to - 1) / to * to; }
+
+void requireDenseGpu(const Tensor& tensor, const char* name) {
+    if (!tensor.isInitialized()) throw std::invalid_argument(std::string(name) + " must be initialized.");
+    if (tensor.getPlacement().getMemDevice() != TensorPlacement::MemDevices::GPU) throw std::invalid_argument(std::string(name) + " must be a GPU tensor.");
+    if (!tensor.isDenseContiguous()) throw std::invalid_argument(std::string(name) + " must be dense contiguous.");
+}
+void requireSamePlacement(const Tensor& a, const Tensor& b, const char* aName, const char* bName) {
+    if (a.getPlacement() != b.getPlacement()) throw std::invalid_argument(std::string(aName) + " and " + bName + " must live on the same GPU placement.");
+}
+void requireStorage(const Tensor& tensor, const char* name, uint64_t items) {
+    if (tensor.getTotalNumElements() < items) throw std::invalid_argument(std::string(name) + " has fewer elements than num_items.");
+}
+void requireCount(uint64_t value, const char* name) {
+    if (value > static_cast<uint64_t>(std::numeric_limits<int64_t>::max())) throw std::invalid_argument(std::string(name) + " exceeds CUB's int64 count limit.");
+}
+void requireTemp(const Tensor& temp, const TensorPlacement& placement, size_t bytes) {
+    requireDenseGpu(temp, "temp_storage");
+    if (temp.getPlacement() != placement) throw std::invalid_argument("temp_storage must live on the same GPU placement as the operation tensors.");
+    if (temp.getDataType() != DataType::UINT8) throw std::invalid_argument("temp_storage must have dtype uint8.");
+    if (temp.getTotalNumElements() < bytes) throw std::invalid_argument("temp_storage has fewer bytes than temp_storage_bytes.");
+}
+void requireStream(const Stream& stream, const TensorPlacement& placement) {
+    if (!stream.isInitialized() || stream.getGpuNum() != static_cast<int>(placement.getDeviceNum())) {
+        throw std::invalid_argument("The stream must live on the GPU of the operation tensors.");
+    }
+}
+
+const char* rawWordName(DataType dtype) {
+    switch (dataTypeSizeInBytes(dtype)) {
+        case 1: return "thor::u8";
+        case 2: return "thor::u16";
+        default: return "thor::u32";
+    }
+}
+int keyKind(DataType dtype) {  // 0 unsigned, 1 signed, 2 float
+    switch (dtype) {
+        case DataType::INT8:
+        case DataType::INT16:
+        case DataType::INT32: return 1;
+        case DataType::FP16:
+        case DataType::BF16:
+        case DataType::FP32: return 2;
+        default: return 0;
+    }
+}
+
+// ---- select-flagged --------------------------------------------------------------------------------------------------------------
+void validateSelect(const Tensor& input, const Tensor& flags, const Tensor& output, const Tensor& numSelected, uint64_t numItems) {
+    requireDenseGpu(input, "input");
+    requireDenseGpu(flags, "flags");
+    requireDenseGpu(output, "output");
+    requireDenseGpu(numSelected, "num_selected_out");
+    requireSamePlacement(input, flags, "input", "flags");
+    requireSamePlacement(input, output, "input", "output");
+    requireSamePlacement(input, numSelected, "input", "num_selected_out");
+    requireStorage(input, "input", numItems);
+    requireStorage(flags, "flags", numItems);
+    requireStorage(output, "output", numItems);
+    requireStorage(numSelected, "num_selected_out", 1);
+    if (input.getDataType() != output.getDataType()) throw std::invalid_argument("CUB select input/output dtypes must match.");
+    if (!isCubSelectValueDTypeSupported(input.getDataType())) {
+        throw std::invalid_argument(std::string("Unsupported CUB select value dtype ") + dataTypeName(input.getDataType()) + ".");
+    }
+    if (!isCubSelectFlagDTypeSupported(flags.getDataType())) {
+        throw std::invalid_argument(std::string("Unsupported CUB select flag dtype ") + dataTypeName(flags.getDataType()) + ".");
+    }
+    if (numSelected.getDataType() != DataType::UINT32) throw std::invalid_argument("CUB select num_selected_out must have dtype uint32.");
+    if (numItems > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) {
+        throw std::invalid_argument("CUB device primitive num_items exceeds CUB's int item-count limit.");
+    }
+}
+
+std::shared_ptr<const CubSelectionKernels> buildSelectKernels(DataType dtype, uint64_t numItems, int deviceNum) {
+    auto kernels = std::make_shared<CubSelectionKernels>();
+    CubSelectionKernels& k = *kernels;
+    k.kind = 0;
+    k.deviceNum = deviceNum;
+    k.threads = kSelectThreads;
+    const uint64_t chunkElems = uint64_t(kSelectThreads) * kSelectItems;
+    k.chunks = std::max<uint64_t>((numItems + chunkElems - 1) / chunkElems, 1);
+    k.countsBytes = roundUp(k.chunks * 4, 256);
+    k.tempBytes = 2 * k.countsBytes;
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
+    s << "namespace gen {\nstruct Cfg {\n    typedef " << rawWordName(dtype) << " Word;\n    static constexpr thor::u64 kTotal = " << numItems
+      << "ull;\n    static constexpr int kThreads = " << kSelectThreads << ";\n    static constexpr int kItems = " << kSelectItems
+      << ";\n    static constexpr thor::u64 kChunks = " << k.chunks << "ull;\n};\n}  // namespace gen\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << kSelectThreads
+      << ") void thor_select_count(const thor::u8* flags, thor::u32* counts) { thor::selectCount<gen::Cfg>(flags, counts); }\n";
+    s << "extern \"C\" __global__ __launch_bounds__(1024) void thor_select_offsets(const thor::u32* counts, thor::u32* bases, thor::u32* numSelected) {\n"
+         "    thor::selectOffsets<gen::Cfg>(counts, bases, numSelected);\n}\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << kSelectThreads
+      << ") void thor_select_scatter(const gen::Cfg::Word* in, const thor::u8* flags, const thor::u32* bases, gen::Cfg::Word* out) {\n"
+         "    thor::selectScatter<gen::Cfg>(in, flags, bases, out);\n}\n";
+    const std::string source = s.str();
+    k.first = compileKernel(source, "thor_select_count", deviceNum, /*fastContract=*/false);
+    k.second = compileKernel(source, "thor_select_offsets", deviceNum, false);
+    k.third = compileKernel(source, "thor_select_scatter", deviceNum, false);
+    std::ostringstream v;
+    v << "select-flagged word" << dataTypeSizeInBytes(dtype) * 8 << " chunks" << k.chunks << "x" << chunkElems << " launches3";
+    k.variant = v.str();
+    return kernels;
+}
+
+// ---- top-k -----------------------------------------------------------------------------------------------------------------------
+void validateTopKKeys(const Tensor& keysIn, const Tensor& keysOut, uint64_t numItems, uint64_t k) {
+    requireDenseGpu(keysIn, "keys_in");
+    requireDenseGpu(keysOut, "keys_out");
+    requireSamePlacement(keysIn, keysOut, "keys_in", "keys_out");
+    requireStorage(keysIn, "keys_in", numItems);
+    requireStorage(keysOut, "keys_out", std::min(numItems, k));
+    if (keysIn.getDataType() != keysOut.getDataType()) throw std::invalid_argument("CUB top-k key input/output dtypes must match.");
+    if (!isCubTopKKeyDTypeSupported(keysIn.getDataType())) {
+        throw std::invalid_argument(std::string("Unsupported CUB top-k key dtype ") + dataTypeName(keysIn.getDataType()) + ".");
+    }
+    requireCount(numItems, "num_items");
+    requireCount(k, "k");
+    // the kernels count keys in 32-bit words
+    if (numItems > 0xffffffffull) throw std::invalid_argument("CUB top-k num_items exceeds the 32-bit counters of this implementation.");
+}
+void validateTopKPairs(const Tensor& keysIn, const Tensor& keysOut, const Tensor& valuesIn, const Tensor& valuesOut, uint64_t numItems, uint64_t k) {
+    validateTopKKeys(keysIn, keysOut, numItems, k);
+    requireDenseGpu(valuesIn, "values_in");
+    requireDenseGpu(valuesOut, "values_out");
+    requireSamePlacement(keysIn, valuesIn, "keys_in", "values_in");
+    requireSamePlacement(keysIn, valuesOut, "keys_in", "values_out");
+    requireStorage(valuesIn, "values_in", numItems);
+    requireStorage(valuesOut, "values_out", std::min(numItems, k));
+    if (valuesIn.getDataType() != valuesOut.getDataType()) throw std::invalid_argument("CUB top-k value input/output dtypes must match.");
+    if (!isCubTopKValueDTypeSupported(valuesIn.getDataType())) {
+        throw std::invalid_argument(std::string("Unsupported CUB top-k index value dtype ") + dataTypeName(valuesIn.getDataType()) + ".");
+    }
+}
+
+uint64_t rowTopKTotalItems(uint64_t numSegments, uint64_t segmentSize) {
+    if (segmentSize != 0 && numSegments > std::numeric_limits<uint64_t>::max() / segmentSize) {
+        throw std::invalid_argument("CUB segmented top-k num_segments * segment_size overflows uint64_t.");
+    }
+    const uint64_t total = numSegments * segmentSize;
+    if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) {
+        throw std::invalid_argument("CUB segmented top-k total item count exceeds the current CUB fixed-size implementation limit.");
+    }
+    return total;
+}
+uint64_t rowTopKOutputItems(uint64_t numSegments, uint64_t segmentSize, uint64_t k) {
+    const uint64_t perSegment = std::min(segmentSize, k);
+    if (perSegment != 0 && numSegments > std::numeric_limits<uint64_t>::max() / perSegment) {
+        throw std::invalid_argument("CUB segmented top-k num_segments * k overflows uint64_t.");
+    }
+    requireCount(numSegments * perSegment, "num_segments * k");
+    return numSegments * perSegment;
+}
+void validateRowTopKKeys(const Tensor& keysIn, const Tensor& keysOut, uint64_t numSegments, uint64_t segmentSize, uint64_t k) {
+    requireDenseGpu(keysIn, "keys_in");
+    requireDenseGpu(keysOut, "keys_out");
+    requireSamePlacement(keysIn, keysOut, "keys_in", "keys_out");
+    requireStorage(keysIn, "keys_in", rowTopKTotalItems(numSegments, segmentSize));
+    requireStorage(keysOut, "keys_out", rowTopKOutputItems(numSegments, segmentSize, k));
+    if (keysIn.getDataType() != keysOut.getDataType()) throw std::invalid_argument("CUB segmented top-k key input/output dtypes must match.");
+    if (!isCubTopKKeyDTypeSupported(keysIn.getDataType())) {
+        throw std::invalid_argument(std::string("Unsupported CUB segmented top-k key dtype ") + dataTypeName(keysIn.getDataType()) + ".");
+    }
+    requireCount(numSegments, "num_segments");
+    requireCount(segmentSize, "segment_size");
+    requireCount(k, "k");
+    if (numSegments == 0 || k == 0) return;
+    if (segmentSize == 0) throw std::invalid_argument("CUB segmented top-k segment_size must be nonzero when num_segments and k are nonzero.");
+    if (segmentSize > kRowTopKMaxSegment) throw std::invalid_argument("CUB segmented top-k segment_size exceeds CUB's current fixed-size support limit.");
+    if (k > kRowTopKMaxK) throw std::invalid_argument("CUB segmented top-k k exceeds CUB's current fixed-size support limit.");
+    if (k >= segmentSize) throw std::invalid_argument("CUB segmented top-k currently requires k to be smaller than the fixed segment size.");
+}
+void validateRowTopKPairs(const Tensor& keysIn, const Tensor& keysOut, const Tensor& valuesIn, const Tensor& valuesOut, uint64_t numSegments,
+                          uint64_t segmentSize, uint64_t k) {
+    validateRowTopKKeys(keysIn, keysOut, numSegments, segmentSize, k);
+    requireDenseGpu(valuesIn, "values_in");
+    requireDenseGpu(valuesOut, "values_out");
+    requireSamePlacement(keysIn, valuesIn, "keys_in", "values_in");
+    requireSamePlacement(keysIn, valuesOut, "keys_in", "values_out");
+    requireStorage(valuesIn, "values_in", rowTopKTotalItems(numSegments, segmentSize));
+    requireStorage(valuesOut, "values_out", rowTopKOutputItems(numSegments, segmentSize, k));
+    if (valuesIn.getDataType() != valuesOut.getDataType()) throw std::invalid_argument("CUB segmented top-k value input/output dtypes must match.");
+    if (!isCubTopKValueDTypeSupported(valuesIn.getDataType())) {
+        throw std::invalid_argument(std::string("Unsupported CUB segmented top-k index value dtype ") + dataTypeName(valuesIn.getDataType()) + ".");
+    }
+}
+
+void writeKeyTraits(std::ostringstream& s, DataType dtype, bool largest, bool pairs) {
+    s << "    typedef " << rawWordName(dtype) << " Raw;\n    static constexpr int kKind = " << keyKind(dtype)
+      << ";\n    static constexpr int kBits = " << dataTypeSizeInBytes(dtype) * 8 << ";\n    static constexpr bool kLargest = " << (largest ? "true" : "false")
+      << ";\n    static constexpr bool kPairs = " << (pairs ? "true" : "false") << ";\n";
+}
+
+// numItems > 0 and 0 < k (already capped at numItems)
+std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint64_t numItems, uint64_t k, bool largest, bool pairs, int deviceNum) {
+    auto kernels = std::make_shared<CubSelectionKernels>();
+    CubSelectionKernels& sel = *kernels;
+    sel.kind = 1;
+    sel.deviceNum = deviceNum;
+    sel.threads = kGatherThreads;
+    sel.digits = static_cast<int>(dataTypeSizeInBytes(dtype));
+    const uint64_t chunkElems = uint64_t(kGatherThreads) * kGatherItems;
+    sel.chunks = (numItems + chunkElems - 1) / chunkElems;
+    // enough striding blocks to keep every compute unit busy, few enough that the global histogram sees little contention
+    sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((numItems + 255) / 256, 2048));
+    sel.tempBytes = (256 + 4) * 4;
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
+    s << "namespace gen {\nstruct Cfg {\n";
+    writeKeyTraits(s, dtype, largest, pairs);
+    s << "    static constexpr thor::u64 kTotal = " << numItems << "ull;\n    static constexpr thor::u64 kK = " << k
+      << "ull;\n    static constexpr int kThreads = " << kGatherThreads << ";\n    static constexpr int kItems = " << kGatherItems
+      << ";\n};\n}  // namespace gen\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_init(thor::u32* temp) { thor::topkInit<gen::Cfg>(temp); }\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift) {\n"
+         "    thor::topkHistogram<gen::Cfg>(keys, temp, shift);\n}\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_pick(thor::u32* temp, thor::u32 shift) { thor::topkPick<gen::Cfg>(temp, shift); }\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << kGatherThreads
+      << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n"
+         "    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
+    const std::string source = s.str();
+    sel.first = compileKernel(source, "thor_topk_init", deviceNum, false);
+    sel.second = compileKernel(source, "thor_topk_histogram", deviceNum, false);
+    sel.third = compileKernel(source, "thor_topk_pick", deviceNum, false);
+    sel.fourth = compileKernel(source, "thor_topk_gather", deviceNum, false);
+    std::ostringstream v;
+    v << "top-k radix-select bits" << sel.digits * 8 << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of " << numItems
+      << " launches" << 2 + 2 * sel.digits;
+    sel.variant = v.str();
+    return kernels;
+}
+
+// numSegments > 0, 0 < k < segmentSize <= 8192
+std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, uint64_t numSegments, uint64_t segmentSize, uint64_t k, bool largest,
+                                                               bool pairs, int deviceNum) {
+    auto kernels = std::make_shared<CubSelectionKernels>();
+    CubSelectionKernels& sel = *kernels;
+    sel.kind = 2;
+    sel.deviceNum = deviceNum;
+    sel.threads = 256;
+    sel.digits = static_cast<int>(dataTypeSizeInBytes(dtype));
+    sel.chunks = numSegments;
+    const uint64_t items = (segmentSize + 255) / 256;
+    std::ostringstream s;
+    s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
+    s << "namespace gen {\nstruct Cfg {\n";
+    writeKeyTraits(s, dtype, largest, pairs);
+    s << "    static constexpr thor::u32 kSegment = " << segmentSize << "u;\n    static constexpr thor::u64 kK = " << k
+      << "ull;\n    static constexpr int kThreads = 256;\n    static constexpr int kItems = " << items << ";\n};\n}  // namespace gen\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_rows(const gen::Cfg::Raw* keys, const thor::u32* values, gen::Cfg::Raw* outKeys, "
+         "thor::u32* outValues) {\n    thor::topkRows<gen::Cfg>(keys, values, outKeys, outValues);\n}\n";
+    sel.first = compileKernel(s.str(), "thor_topk_rows", deviceNum, false);
+    std::ostringstream v;
+    v << "row top-k radix-select bits" << sel.digits * 8 << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of "
+      << segmentSize << " rows" << numSegments << " launches1";
+    sel.variant = v.str();
+    return kernels;
+}
+
+void launchTopK(const CubSelectionKernels& sel, const void* keysIn, const void* valuesIn, void* temp, void* keysOut, void* valuesOut, Stream& stream) {
+    ScopedGpu scoped(sel.deviceNum);
+    void* raw = stream.getStream();
+    if (sel.kind == 2) {
+        std::vector<void*> args = {&keysIn, &valuesIn, &keysOut, &valuesOut};
+        sel.first->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, args);
+        return;
+    }
+    std::vector<void*> initArgs = {&temp};
+    sel.first->launch(1, 1, 1, 256, raw, initArgs);
+    for (int digit = sel.digits - 1; digit >= 0; --digit) {
+        uint32_t shift = static_cast<uint32_t>(digit) * 8;
+        std::vector<void*> histogramArgs = {&keysIn, &temp, &shift};
+        sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, histogramArgs);
+        std::vector<void*> pickArgs = {&temp, &shift};
+        sel.third->launch(1, 1, 1, 256, raw, pickArgs);
+    }
+    std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut};
+    sel.fourth->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, gatherArgs);
+}
+
+void* tempPointer(const Tensor& temp) { return const_cast<Tensor&>(temp).getMemPtr(); }
+
+}  // namespace
+
+bool isCubTopKKeyDTypeSupported(DataType dtype) {
+    switch (dtype) {
+        case DataType::UINT8:
+        case DataType::INT8:
+        case DataType::UINT16:
+        case DataType::INT16:
+        case DataType::UINT32:
+        case DataType::INT32:
+        case DataType::FP16:
+        case DataType::BF16:
+        case DataType::FP32: return true;
+        default: return false;
+    }
+}
+bool isCubTopKValueDTypeSupported(DataType dtype) { return dtype == DataType::UINT32; }
+bool isCubSelectValueDTypeSupported(DataType dtype) { return isCubTopKKeyDTypeSupported(dtype); }
+bool isCubSelectFlagDTypeSupported(DataType dtype) { return dtype == DataType::BOOLEAN || dtype == DataType::UINT8; }
+
+CubTemporaryStoragePlan cubTemporaryStoragePlan(const TensorPlacement& placement, size_t bytes) {
+    if (placement.getMemDevice() != TensorPlacement::MemDevices::GPU) throw std::invalid_argument("CUB temporary storage must be planned on GPU placement.");
+    CubTemporaryStoragePlan plan;
+    plan.placement = placement;
+    plan.bytes = std::max<size_t>(bytes, 1);
+    return plan;
+}
+CubTemporaryStoragePlan cubMaxTemporaryStoragePlan(std::initializer_list<CubTemporaryStoragePlan> plans) {
+    if (plans.size() == 0) throw std::invalid_argument("At least one CUB temporary-storage plan is required.");
+    auto it = plans.begin();
+    CubTemporaryStoragePlan combined = cubTemporaryStoragePlan(it->placement, it->bytes);
+    for (++it; it != plans.end(); ++it) {
+        if (it->placement != combined.placement) throw std::invalid_argument("All CUB temporary-storage plans must use the same GPU placement.");
+        combined.bytes = std::max(combined.bytes, std::max<size_t>(it->bytes, 1));
+    }
+    return combined;
+}
+Tensor allocateCubTemporaryStorage(const CubTemporaryStoragePlan& plan) { return allocateCubTemporaryStorage(plan.placement, plan.bytes); }
+
+std::string cubSelectionKernelVariant(const std::shared_ptr<const CubSelectionKernels>& kernels) { return kernels ? kernels->variant : std::string(); }
+
+// ---- select-flagged --------------------------------------------------------------------------------------------------------------
+CubDeviceSelectFlaggedPlan prepareCubDeviceSelectFlagged(const Tensor& input, const Tensor& flags, const Tensor& output, const Tensor& numSelected,
+                                                         uint64_t numItems) {
+    validateSelect(input, flags, output, numSelected, numItems);
+    CubDeviceSelectFlaggedPlan plan;
+    plan.placement = input.getPlacement();
+    plan.input_dtype = input.getDataType();
+    plan.flag_dtype = flags.getDataType();
+    plan.num_items = numItems;
+    // no items: the run only writes the zero count, with the offsets kernel of a one-chunk plan over no elements
+    plan.kernels = buildSelectKernels(plan.input_dtype, numItems, static_cast<int>(plan.placement.getDeviceNum()));
+    plan.temp_storage_bytes = std::max<size_t>(plan.kernels->tempBytes, 1);
+    return plan;
+}
+size_t cubDeviceSelectFlaggedTempBytes(const Tensor& input, const Tensor& flags, const Tensor& output, const Tensor& numSelected, uint64_t numItems) {
+    return prepareCubDeviceSelectFlagged(input, flags, output, numSelected, numItems).temp_storage_bytes;
+}
+void cubDeviceSelectFlagged(const CubDeviceSelectFlaggedPlan& plan, const Tensor& temp, const Tensor& input, const Tensor& flags, Tensor& output,
+                            Tensor& numSelected, Stream& stream) {
+    validateSelect(input, flags, output, numSelected, plan.num_items);
+    if (input.getPlacement() != plan.placement || input.getDataType() != plan.input_dtype || flags.getDataType() != plan.flag_dtype || !plan.kernels) {
+        throw std::invalid_argument("CUB select-flagged plan is not compatible with the provided tensors.");
+    }
+    requireTemp(temp, plan.placement, plan.temp_storage_bytes);
+    requireStream(stream, plan.placement);
+    const CubSelectionKernels& k = *plan.kernels;
+    ScopedGpu scoped(k.deviceNum);
+    void* raw = stream.getStream();
+    char* base = static_cast<char*>(tempPointer(temp));
+    void* counts = base;
+    void* bases = base + k.countsBytes;
+    const void* in = const_cast<Tensor&>(input).getMemPtr();
+    const void* flagBytes = const_cast<Tensor&>(flags).getMemPtr();
+    void* out = output.getMemPtr();
+    void* total = numSelected.getMemPtr();
+    std::vector<void*> countArgs = {&flagBytes, &counts};
+    k.first->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, countArgs);
+    std::vector<void*> offsetArgs = {&counts, &bases, &total};
+    k.second->launch(1, 1, 1, 1024, raw, offsetArgs);
+    if (plan.num_items == 0) return;
+    std::vector<void*> scatterArgs = {&in, &flagBytes, &bases, &out};
+    k.third->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, scatterArgs);
+}
+void cubDeviceSelectFlagged(const Tensor& temp, size_t tempBytes, const Tensor& input, const Tensor& flags, Tensor& output, Tensor& numSelected,
+                            uint64_t numItems, Stream& stream) {
+    CubDeviceSelectFlaggedPlan plan = prepareCubDeviceSelectFlagged(input, flags, output, numSelected, numItems);
+    if (tempBytes < plan.temp_storage_bytes) throw std::invalid_argument("temp_storage_bytes is smaller than the prepared CUB select-flagged requirement.");
+    plan.temp_storage_bytes = tempBytes;
+    cubDeviceSelectFlagged(plan, temp, input, flags, output, numSelected, stream);
+}
+
+// ---- device-wide top-k -------------------------------------------------------------------------------------------------------------
+namespace {
+
+template <typename Plan>
+void fillTopKPlan(Plan& plan, const Tensor& keysIn, uint64_t numItems, uint64_t k, CubTopKOrder order, bool pairs) {
+    plan.placement = keysIn.getPlacement();
+    plan.key_dtype = keysIn.getDataType();
+    plan.num_items = numItems;
+    plan.k = k;
+    plan.order = order;
+    const uint64_t selected = std::min(numItems, k);
+    if (selected != 0) {
+        plan.kernels = buildTopKKernels(plan.key_dtype, numItems, selected, order == CubTopKOrder::Largest, pairs, static_cast<int>(plan.placement.getDeviceNum()));
+    }
+    plan.temp_storage_bytes = plan.kernels ? plan.kernels->tempBytes : 1;
+}
+
+template <typename Plan>
+void fillRowTopKPlan(Plan& plan, const Tensor& keysIn, uint64_t numSegments, uint64_t segmentSize, uint64_t k, CubTopKOrder order, bool pairs) {
+    plan.placement = keysIn.getPlacement();
+    plan.key_dtype = keysIn.getDataType();
+    plan.num_segments = numSegments;
+    plan.segment_size = segmentSize;
+    plan.k = k;
+    plan.order = order;
+    if (numSegments != 0 && k != 0) {
+        plan.kernels = buildRowTopKKernels(plan.key_dtype, numSegments, segmentSize, k, order == CubTopKOrder::Largest, pairs,
+                                           static_cast<int>(plan.placement.getDeviceNum()));
+    }
+    plan.temp_storage_bytes = 1;
+}
+
+}  // namespace
+
+CubDeviceTopKKeysPlan prepareCubDeviceTopKKeys(const Tensor& keysIn, const Tensor& keysOut, uint64_t numItems, uint64_t k, CubTopKOrder order) {
+    validateTopKKeys(keysIn, keysOut, numItems, k);
+    CubDeviceTopKKeysPlan plan;
+    fillTopKPlan(plan, keysIn, numItems, k, order, false);
+    return plan;
+}
+size_t cubDeviceTopKKeysTempBytes(const Tensor& keysIn, const Tensor& keysOut, uint64_t numItems, uint64_t k, CubTopKOrder order) {
+    return prepareCubDeviceTopKKeys(keysIn, keysOut, numItems, k, order).temp_storage_bytes;
+}
+void cubDeviceTopKKeys(const CubDeviceTopKKeysPlan& plan, const Tensor& temp, const Tensor& keysIn, Tensor& keysOut, Stream& stream) {
+    validateTopKKeys(keysIn, keysOut, plan.num_items, plan.k);
+    if (keysIn.getPlacement() != plan.placement || keysIn.getDataType() != plan.key_dtype) {
+        throw std::invalid_argument("CUB top-k-keys plan is not compatible with the provided tensors.");
+    }
+    requireTemp(temp, plan.placement, plan.temp_storage_bytes);
+    requireStream(stream, plan.placement);
+    if (!plan.kernels) return;
+    launchTopK(*plan.kernels, const_cast<Tensor&>(keysIn).getMemPtr(), nullptr, tempPointer(temp), keysOut.getMemPtr(), nullptr, stream);
+}
+void cubDeviceTopKKeys(const Tensor& temp, size_t tempBytes, const Tensor& keysIn, Tensor& keysOut, uint64_t numItems, uint64_t k, Stream& stream,
+                       CubTopKOrder order) {
+    CubDeviceTopKKeysPlan plan = prepareCubDeviceTopKKeys(keysIn, keysOut, numItems, k, order);
+    if (tempBytes < plan.temp_storage_bytes) throw std::invalid_argument("temp_storage_bytes is smaller than the prepared CUB top-k-keys requirement.");
+    plan.temp_storage_bytes = tempBytes;
+    cubDeviceTopKKeys(plan, temp, keysIn, keysOut, stream);
+}
+
+CubDeviceTopKPairsPlan prepareCubDeviceTopKPairs(const Tensor& keysIn, const Tensor& keysOut, const Tensor& valuesIn, const Tensor& valuesOut,
+                                                 uint64_t numItems, uint64_t k, CubTopKOrder order) {
+    validateTopKPairs(keysIn, keysOut, valuesIn, valuesOut, numItems, k);
+    CubDeviceTopKPairsPlan plan;
+    plan.value_dtype = valuesIn.getDataType();
+    fillTopKPlan(plan, keysIn, numItems, k, order, true);
+    return plan;
+}
+size_t cubDeviceTopKPairsTempBytes(const Tensor& keysIn, const Tensor& keysOut, const Tensor& valuesIn, const Tensor& valuesOut, uint64_t numItems,
+                                   uint64_t k, CubTopKOrder order) {
+    return prepareCubDeviceTopKPairs(keysIn, keysOut, valuesIn, valuesOut, numItems, k, order).temp_storage_bytes;
+}
+void cubDeviceTopKPairs(const CubDeviceTopKPairsPlan& plan, const Tensor& temp, const Tensor& keysIn, Tensor& keysOut, const Tensor& valuesIn,
+                        Tensor& valuesOut, Stream& stream) {
+    validateTopKPairs(keysIn, keysOut, valuesIn, valuesOut, plan.num_items, plan.k);
+    if (keysIn.getPlacement() != plan.placement || keysIn.getDataType() != plan.key_dtype || valuesIn.getDataType() != plan.value_dtype) {
+        throw std::invalid_argument("CUB top-k-pairs plan is not compatible with the provided tensors.");
+    }
+    requireTemp(temp, plan.placement, plan.temp_storage_bytes);
+    requireStream(stream, plan.placement);
+    if (!plan.kernels) return;
+    launchTopK(*plan.kernels, const_cast<Tensor&>(keysIn).getMemPtr(), const_cast<Tensor&>(valuesIn).getMemPtr(), tempPointer(temp), keysOut.getMemPtr(),
+               valuesOut.getMemPtr(), stream);
+}
+void cubDeviceTopKPairs(const Tensor& temp, size_t tempBytes, const Tensor& keysIn, Tensor& keysOut, const Tensor& valuesIn, Tensor& valuesOut,
+                        uint64_t numItems, uint64_t k, Stream& stream, CubTopKOrder order) {
+    CubDeviceTopKPairsPlan plan = prepareCubDeviceTopKPairs(keysIn, keysOut, valuesIn, valuesOut, numItems, k, order);
+    if (tempBytes < plan.temp_storage_bytes) throw std::invalid_argument("temp_storage_bytes is smaller than the prepared CUB top-k-pairs requirement.");
+    plan.temp_storage_bytes = tempBytes;
+    cubDeviceTopKPairs(plan, temp, keysIn, keysOut, valuesIn, valuesOut, stream);
+}
+
+// ---- top-k of rows ---------------------------------------------------------------------------------------------------------------
+CubDeviceSegmentedTopKKeysPlan prepareCubDeviceSegmentedTopKKeys(const Tensor& keysIn, const Tensor& keysOut, uint64_t numSegments, uint64_t segmentSize,
+                                                                 uint64_t k, CubTopKOrder order) {
+    validateRowTopKKeys(keysIn, keysOut, numSegments, segmentSize, k);
+    CubDeviceSegmentedTopKKeysPlan plan;
+    fillRowTopKPlan(plan, keysIn, numSegments, segmentSize, k, order, false);
+    return plan;
+}
+size_t cubDeviceSegmentedTopKKeysTempBytes(const Tensor& keysIn, const Tensor& keysOut, uint64_t numSegments, uint64_t segmentSize, uint64_t k,
+                                           CubTopKOrder order) {
+    return prepareCubDeviceSegmentedTopKKeys(keysIn, keysOut, numSegments, segmentSize, k, order).temp_storage_bytes;
+}
+void cubDeviceSegmentedTopKKeys(const CubDeviceSegmentedTopKKeysPlan& plan, const Tensor& temp, const Tensor& keysIn, Tensor& keysOut, Stream& stream) {
+    validateRowTopKKeys(keysIn, keysOut, plan.num_segments, plan.segment_size, plan.k);
+    if (keysIn.getPlacement() != plan.placement || keysIn.getDataType() != plan.key_dtype) {
+        throw std::invalid_argument("CUB segmented top-k-keys plan is not compatible with the provided tensors.");
+    }
+    requireTemp(temp, plan.placement, plan.temp_storage_bytes);
+    requireStream(stream, plan.placement);
+    if (!plan.kernels) return;
+    launchTopK(*plan.kernels, const_cast<Tensor&>(keysIn).getMemPtr(), nullptr, nullptr, keysOut.getMemPtr(), nullptr, stream);
+}
+void cubDeviceSegmentedTopKKeys(const Tensor& temp, size_t tempBytes, const Tensor& keysIn, Tensor& keysOut, uint64_t numSegments, uint64_t segmentSize,
+                                uint64_t k, Stream& stream, CubTopKOrder order) {
+    CubDeviceSegmentedTopKKeysPlan plan = prepareCubDeviceSegmentedTopKKeys(keysIn, keysOut, numSegments, segmentSize, k, order);
+    if (tempBytes < plan.temp_storage_bytes) {
+        throw std::invalid_argument("temp_storage_bytes is smaller than the prepared CUB segmented top-k-keys requirement.");
+    }
+    plan.temp_storage_bytes = tempBytes;
+    cubDeviceSegmentedTopKKeys(plan, temp, keysIn, keysOut, stream);
+}
+
+CubDeviceSegmentedTopKPairsPlan prepareCubDeviceSegmentedTopKPairs(const Tensor& keysIn, const Tensor& keysOut, const Tensor& valuesIn,
+                                                                   const Tensor& valuesOut, uint64_t numSegments, uint64_t segmentSize, uint64_t k,
+                                                                   CubTopKOrder order) {
+    validateRowTopKPairs(keysIn, keysOut, valuesIn, valuesOut, numSegments, segmentSize, k);
+    CubDeviceSegmentedTopKPairsPlan plan;
+    plan.value_dtype = valuesIn.getDataType();
+    fillRowTopKPlan(plan, keysIn, numSegments, segmentSize, k, order, true);
+    return plan;
+}
+size_t cubDeviceSegmentedTopKPairsTempBytes(const Tensor& keysIn, const Tensor& keysOut, const Tensor& valuesIn, const Tensor& valuesOut,
+                                            uint64_t numSegments, uint64_t segmentSize, uint64_t k, CubTopKOrder order) {
+    return prepareCubDeviceSegmentedTopKPairs(keysIn, keysOut, valuesIn, valuesOut, numSegments, segmentSize, k, order).temp_storage_bytes;
+}
+void cubDeviceSegmentedTopKPairs(const CubDeviceSegmentedTopKPairsPlan& plan, const Tensor& temp, const Tensor& keysIn, Tensor& keysOut,
+                                 const Tensor& valuesIn, Tensor& valuesOut, Stream& stream) {
+    validateRowTopKPairs(keysIn, keysOut, valuesIn, valuesOut, plan.num_segments, plan.segment_size, plan.k);
+    if (keysIn.getPlacement() != plan.placement || keysIn.getDataType() != plan.key_dtype || valuesIn.getDataType() != plan.value_dtype) {
+        throw std::invalid_argument("CUB segmented top-k-pairs plan is not compatible with the provided tensors.");
+    }
+    requireTemp(temp, plan.placement, plan.temp_storage_bytes);
+    requireStream(stream, plan.placement);
+    if (!plan.kernels) return;
+    launchTopK(*plan.kernels, const_cast<Tensor&>(keysIn).getMemPtr(), const_cast<Tensor&>(valuesIn).getMemPtr(), nullptr, keysOut.getMemPtr(),
+               valuesOut.getMemPtr(), stream);
+}
+void cubDeviceSegmentedTopKPairs(const Tensor& temp, size_t tempBytes, const Tensor& keysIn, Tensor& keysOut, const Tensor& valuesIn, Tensor& valuesOut,
+                                 uint64_t numSegments, uint64_t segmentSize, uint64_t k, Stream& stream, CubTopKOrder order) {
+    CubDeviceSegmentedTopKPairsPlan plan = prepareCubDeviceSegmentedTopKPairs(keysIn, keysOut, valuesIn, valuesOut, numSegments, segmentSize, k, order);
+    if (tempBytes < plan.temp_storage_bytes) {
+        throw std::invalid_argument("temp_storage_bytes is smaller than the prepared CUB segmented top-k-pairs requirement.");
+    }
+    plan.temp_storage_bytes = tempBytes;
+    cubDeviceSegmentedTopKPairs(plan, temp, keysIn, keysOut, valuesIn, valuesOut, stream);
+}
+
+}  // namespace ThorImplementation

@@ -174,6 +174,7 @@ uint64_t StampedExecutionStage::flopCount() const {
             return segmented_reduction ? segmented_reduction->flopCount() : 0;
         case Kind::SegmentedBroadcast:
         case Kind::Scan:
+        case Kind::DependencyBarrier:
             return 0;
     }
     return 0;

@@ -300,6 +300,49 @@ int thor_segmented_broadcast(thor_tensor_t per_segment_values, thor_tensor_t seg
                                                stream->stream);)
 }
 
+int thor_select_flagged(thor_tensor_t input, thor_tensor_t flags, thor_tensor_t output, thor_tensor_t num_selected_out, uint64_t num_items,
+                        thor_stream_t stream, char* variant, size_t variant_capacity) {
+    THOR_CAPI_TRY_INT(require(input, "input"); require(flags, "flags"); require(output, "output"); require(num_selected_out, "num_selected_out");
+                      require(stream, "stream");
+                      const auto plan = prepareCubDeviceSelectFlagged(input->tensor, flags->tensor, output->tensor, num_selected_out->tensor, num_items);
+                      cubDeviceSelectFlagged(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), input->tensor, flags->tensor,
+                                             output->tensor, num_selected_out->tensor, stream->stream);
+                      if (variant) copyOut(cubSelectionKernelVariant(plan.kernels), variant, variant_capacity, nullptr);)
+}
+
+int thor_topk(thor_tensor_t keys_in, thor_tensor_t keys_out, thor_tensor_t values_in, thor_tensor_t values_out, uint64_t num_segments,
+              uint64_t segment_size, uint64_t k, int largest, int segmented, thor_stream_t stream, char* variant, size_t variant_capacity) {
+    THOR_CAPI_TRY_INT(
+        require(keys_in, "keys_in"); require(keys_out, "keys_out"); require(stream, "stream");
+        if ((values_in == nullptr) != (values_out == nullptr)) throw std::invalid_argument("top-k takes values_in and values_out together or neither");
+        const CubTopKOrder order = largest ? CubTopKOrder::Largest : CubTopKOrder::Smallest;
+        std::shared_ptr<const CubSelectionKernels> kernels;
+        if (segmented) {
+            if (values_in) {
+                const auto plan = prepareCubDeviceSegmentedTopKPairs(keys_in->tensor, keys_out->tensor, values_in->tensor, values_out->tensor,
+                                                                     num_segments, segment_size, k, order);
+                cubDeviceSegmentedTopKPairs(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), keys_in->tensor, keys_out->tensor,
+                                            values_in->tensor, values_out->tensor, stream->stream);
+                kernels = plan.kernels;
+            } else {
+                const auto plan = prepareCubDeviceSegmentedTopKKeys(keys_in->tensor, keys_out->tensor, num_segments, segment_size, k, order);
+                cubDeviceSegmentedTopKKeys(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), keys_in->tensor, keys_out->tensor,
+                                           stream->stream);
+                kernels = plan.kernels;
+            }
+        } else if (values_in) {
+            const auto plan = prepareCubDeviceTopKPairs(keys_in->tensor, keys_out->tensor, values_in->tensor, values_out->tensor, segment_size, k, order);
+            cubDeviceTopKPairs(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), keys_in->tensor, keys_out->tensor,
+                               values_in->tensor, values_out->tensor, stream->stream);
+            kernels = plan.kernels;
+        } else {
+            const auto plan = prepareCubDeviceTopKKeys(keys_in->tensor, keys_out->tensor, segment_size, k, order);
+            cubDeviceTopKKeys(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), keys_in->tensor, keys_out->tensor, stream->stream);
+            kernels = plan.kernels;
+        }
+        if (variant) copyOut(cubSelectionKernelVariant(kernels), variant, variant_capacity, nullptr);)
+}
+
 int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments, uint64_t segment_size,
               int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity) {
     THOR_CAPI_TRY_INT(

@@ -63,6 +63,8 @@ PROTOTYPES = {
     "thor_segmented_broadcast": (_i, [_vp, _vp, _vp, _i, _vp]),
     "thor_scan": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
     "thor_scan_no_alloc": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
+    "thor_select_flagged": (_i, [_vp, _vp, _vp, _vp, ctypes.c_uint64, _vp, _cp, _sz]),
+    "thor_topk": (_i, [_vp, _vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _vp, _cp, _sz]),
     "thor_reduction_generate_source": (_i, [_i, _i, _i, _i, _i, _u64p, _u64p, _i, _u32p, _i, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_arg_reduction_stamp": (_vp, [_i, _u32p, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "thor_stamped_arg_reduction_destroy": (None, [_vp]), "thor_stamped_arg_reduction_run": (_i, [_vp]),
@@ -258,7 +260,7 @@ class PhysicalTensor:
         buf = (ctypes.c_char * (n * carrier.itemsize)).from_address(self.mem_ptr())
         arr = np.frombuffer(buf, dtype=carrier, count=n).reshape(self.get_dimensions())
         arr.flags.writeable = True
-        self._keepalive = buf
+        buf._tensor = self  # the array's base is `buf`: it keeps this tensor, and with it the pinned memory, alive as long as the array lives
         return arr
 
     def copy_from_async(self, source: "PhysicalTensor", stream: Stream):
@@ -570,6 +572,35 @@ def scan(input: PhysicalTensor, output: PhysicalTensor, stream: Stream, op: Scan
     entry = lib().thor_scan_no_alloc if no_alloc else lib().thor_scan
     _check(entry(input._h, output._h, segment_offsets._h if segment_offsets is not None else None, n, segments, segment_size, code, int(arg),
                  int(inclusive), int(reverse), stream._h, text, 512), "scan")
+    return text.value.decode()
+
+
+def select_flagged(input: PhysicalTensor, flags: PhysicalTensor, output: PhysicalTensor, num_selected_out: PhysicalTensor, stream: Stream,
+                   num_items: Optional[int] = None) -> str:
+    """``output`` receives the elements of ``input`` whose flag (BOOLEAN / UINT8) is nonzero, in input order, ``num_selected_out``
+    (UINT32, one element) their number (cubDeviceSelectFlagged, CubDevicePrimitives.h:490-516 there).  Returns the kernel variant."""
+    n = int(num_items if num_items is not None else np.prod(input.get_dimensions()))
+    text = ctypes.create_string_buffer(512)
+    _check(lib().thor_select_flagged(input._h, flags._h, output._h, num_selected_out._h, n, stream._h, text, 512), "select_flagged")
+    return text.value.decode()
+
+
+def top_k(keys_in: PhysicalTensor, keys_out: PhysicalTensor, k: int, stream: Stream, largest: bool = True,
+          values_in: Optional[PhysicalTensor] = None, values_out: Optional[PhysicalTensor] = None, num_items: Optional[int] = None,
+          num_segments: Optional[int] = None, segment_size: Optional[int] = None) -> str:
+    """The ``k`` largest (or smallest) keys, unordered, with their UINT32 values when both value tensors are given
+    (cubDeviceTopKKeys / cubDeviceTopKPairs, CubDevicePrimitives.h:357-420 there).  With ``segment_size`` the selection runs in
+    every row of that many keys (at most 8192, ``k`` below it) and writes ``k`` keys per row (cubDeviceSegmentedTopKKeys / Pairs,
+    :422-488 there).  Returns the kernel variant (empty when there is nothing to select)."""
+    text = ctypes.create_string_buffer(512)
+    values = (values_in._h if values_in is not None else None, values_out._h if values_out is not None else None)
+    if segment_size is not None:
+        segments = int(num_segments if num_segments is not None else np.prod(keys_in.get_dimensions()) // max(int(segment_size), 1))
+        _check(lib().thor_topk(keys_in._h, keys_out._h, values[0], values[1], segments, int(segment_size), int(k), int(largest), 1, stream._h, text, 512),
+               "top_k")
+    else:
+        n = int(num_items if num_items is not None else np.prod(keys_in.get_dimensions()))
+        _check(lib().thor_topk(keys_in._h, keys_out._h, values[0], values[1], 0, n, int(k), int(largest), 0, stream._h, text, 512), "top_k")
     return text.value.decode()
 
 
