@@ -145,6 +145,12 @@ class StampedScan {
     StampedScan(std::shared_ptr<const CubScanKernels> kernels, Tensor input, std::optional<Tensor> offsets, Tensor temp, Tensor values, Tensor indices)
         : kernels(std::move(kernels)), input(std::move(input)), offsets(std::move(offsets)), temp(std::move(temp)), values(std::move(values)),
           indices(std::move(indices)) {}
+    // the gradient of a min / max scan over rows in one launch: reads the operand and the FP32 upstream gradient, writes `routed`
+    static StampedScan routing(std::shared_ptr<const CubScanKernels> kernels, Tensor input, Tensor gradient, Tensor routed) {
+        StampedScan scan(std::move(kernels), std::move(input), std::nullopt, Tensor(), std::move(routed), /*indexOutput=*/false);
+        scan.gradient = std::move(gradient);
+        return scan;
+    }
     void runOn(Stream& stream) const;
     Tensor getOutputTensor() const { return values.isInitialized() ? values : indices; }
     std::string getKernelVariant() const;
@@ -153,7 +159,7 @@ class StampedScan {
     std::shared_ptr<const CubScanKernels> kernels;
     Tensor input;
     std::optional<Tensor> offsets;
-    Tensor temp, values, indices;
+    Tensor temp, values, indices, gradient;
 };
 
 struct StampedExecutionStage {

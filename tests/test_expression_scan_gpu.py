@@ -223,9 +223,9 @@ def winners_gradient(values, grad, op, inclusive, reverse=False, segment_size=0,
 
 
 @pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16], ids=lambda d: d.name)
-@pytest.mark.parametrize("inclusive,reverse", [(True, False), (False, False), (True, True)])
+@pytest.mark.parametrize("inclusive,reverse", [(True, False), (False, False), (True, True), (False, True)])
 @pytest.mark.parametrize("name", ["min", "max"])
-@pytest.mark.parametrize("shape", [(64, 1000), (3, 20000), (1, 7)], ids=str)
+@pytest.mark.parametrize("shape", [(64, 1000), (3, 20000), (1, 7), (16, 8192), (300, 256), (37, 33), (9, 4100)], ids=str)
 def test_row_minmax_scan_backward(stream, shape, name, inclusive, reverse, dtype):
     rng = np.random.default_rng(61)
     # few distinct values: long runs of one winner, and ties that the first occurrence must win
@@ -236,12 +236,35 @@ def test_row_minmax_scan_backward(stream, shape, name, inclusive, reverse, dtype
     bwd = ex.compile(scanned, device_num=0).compile_backward(["x"], error_input_name="__grad_output")
     plan = bwd.stamp({"x": copy_numpy_to_gpu(values, stream, dtype), "__grad_output": copy_numpy_to_gpu(grad, stream, dtype)}, stream)
     plan.run()
+    # rows that fit one block's chunk (8192 positions) take one launch: winners, run sums and the routed gradient together
+    descriptions = " | ".join(plan.stage_descriptions())
+    assert ("scan-route" in descriptions) == (shape[-1] <= 8192) and ("scatter_add" in descriptions) == (shape[-1] > 8192), descriptions
     expected = winners_gradient(values, from_storage(grad, dtype), ORACLE_OP[ScanOp["arg_" + name]], inclusive, reverse, segment_size=shape[-1], dtype=int(dtype))
     got = from_storage(copy_gpu_to_numpy(plan.output("x_grad"), stream), dtype).astype(np.float64)
     if dtype == DataType.fp32:
         np.testing.assert_array_equal(got, expected)  # exact sums: the order of the additions cannot show
     else:
         np.testing.assert_allclose(got, from_storage(to_storage(expected.astype(np.float32), dtype), dtype), rtol=0, atol=0)
+
+
+def test_row_running_max_backward_with_real_gradients(stream):
+    """Random fp32 gradients: the run sums are compared with float64 sums within the rounding of a tree of fp32 additions, and
+    every element that never held the running maximum gets exactly zero."""
+    rng = np.random.default_rng(63)
+    values = rng.standard_normal((256, 8192)).astype(np.float32)
+    grad = rng.standard_normal((256, 8192)).astype(np.float32)
+    bwd = ex.compile(ex.input("x").scan(ScanOp.max), device_num=0).compile_backward(["x"], error_input_name="__grad_output")
+    plan = bwd.stamp({"x": copy_numpy_to_gpu(values, stream, DataType.fp32), "__grad_output": copy_numpy_to_gpu(grad, stream, DataType.fp32)}, stream)
+    assert plan.stage_kind_names() == ["Scan"]
+    for _ in range(2):  # the LDS copy is cleared by every launch
+        plan.run()
+        got = copy_gpu_to_numpy(plan.output("x_grad"), stream).astype(np.float64)
+        expected = winners_gradient(values, grad, oracle.SCAN_ARGMAX, True, segment_size=8192)
+        scale = np.zeros_like(expected)
+        winners = oracle.scan(values, oracle.SCAN_ARGMAX, True, segment_size=8192, dtype=oracle.FP32).reshape(-1).astype(np.int64)
+        np.add.at(scale.reshape(-1), winners, np.abs(grad.reshape(-1)).astype(np.float64))
+        assert np.all(np.abs(got - expected) <= 2e-6 * scale)
+        assert np.all(got[scale == 0] == 0)
 
 
 def test_ragged_minmax_scan_backward_and_chain_rule(stream):

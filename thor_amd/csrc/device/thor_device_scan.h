@@ -149,6 +149,14 @@ __device__ __forceinline__ void scanStoreState(void* buffer, u64 slot, const Sca
     words[2 * Cfg::kChunks + slot] = s.head;
 }
 
+// the traits of the sum over runs that routes a min / max scan's gradient (only what the combining code looks at)
+struct ScanRunSum {
+    typedef float T;
+    typedef float Acc;
+    static constexpr bool kUnsigned = false;
+    static constexpr int kOp = 0;
+};
+
 // bit k set: logical position p + k starts a segment (p is a multiple of kVec)
 template <typename Cfg>
 __device__ __forceinline__ u32 scanHeadBits(const u32* heads, u64 p) {
@@ -163,9 +171,15 @@ __device__ __forceinline__ u32 scanHeadBits(const u32* heads, u64 p) {
 
 // AGGREGATE_ONLY: write the chunk's total to `aggregates` and nothing else.  Otherwise: take the chunk's carry from
 // `carries` (when Cfg::kCarry) and write the scanned values and / or indices.
-template <typename Cfg, bool AGGREGATE_ONLY>
-__device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* heads, const void* carries, void* aggregates,
-                                          typename Cfg::T* outValue, u32* outIndex) {
+//
+// ROUTE (the gradient of a min / max scan; chunks hold whole rows, nothing is carried): the winners stay in registers.  Position
+// p's gradient belongs to the element that won p's prefix, and the positions one element wins are consecutive: they begin at
+// the element itself (after it, for an exclusive scan) and end before the next element that beats it.  So a second scan over
+// the same chunk sums `gradient` over those runs, the last position of each run puts the run's sum where the winner lies in a
+// zeroed copy of the chunk in LDS, and the copy is written out with full vectors: every element of `routed` is written once.
+template <typename Cfg, bool AGGREGATE_ONLY, bool ROUTE>
+__device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u32* heads, const void* carries, void* aggregates,
+                                              typename Cfg::T* outValue, u32* outIndex, const float* gradient, float* routed) {
     typedef typename Cfg::T T;
     typedef typename Cfg::Acc Acc;
     typedef ScanState<Cfg> S;
@@ -184,6 +198,9 @@ __device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* 
     bool live[ITEMS];
     u64 physical[ITEMS];  // first element of the vector in memory
     S laneExclusive[ITEMS];
+    __shared__ float routeTile[ROUTE ? ITEMS * THREADS * V : 1];  // indexed by the position inside the chunk
+    Pack<float, V> upstream[ROUTE ? ITEMS : 1];
+    u32 rowHeads[ROUTE ? ITEMS : 1];
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         const u64 local = ((u64)it * THREADS + threadIdx.x) * V;
@@ -195,6 +212,12 @@ __device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* 
         if (live[it]) {
             x.loadStream(in + physical[it]);
             headBits = scanHeadBits<Cfg>(heads, p);
+        }
+        if constexpr (ROUTE) {
+            if (live[it]) upstream[it].loadStream(gradient + physical[it]);
+            rowHeads[it] = headBits;
+#pragma unroll
+            for (int k = 0; k < V; ++k) routeTile[local + k] = 0.0f;
         }
         S run = scanEmpty<Cfg>();
         sealed[it] = 0;
@@ -257,6 +280,7 @@ __device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* 
     }
     if (AGGREGATE_ONLY) return;
     __syncthreads();
+    u32 winners[ROUTE ? ITEMS : 1][V];  // in scan order
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         if (!live[it]) continue;
@@ -277,10 +301,112 @@ __device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* 
             i = own ? preIndex[it][k] : i;
             values.v[Cfg::kReverse ? V - 1 - k : k] = scanStore<T>(v);
             indices.v[Cfg::kReverse ? V - 1 - k : k] = i;
+            if constexpr (ROUTE) winners[it][k] = i;
         }
-        if (Cfg::kWriteValue) values.storeStream(outValue + physical[it]);
-        if (Cfg::kWriteIndex) indices.storeStream(outIndex + physical[it]);
+        if constexpr (!ROUTE) {
+            if (Cfg::kWriteValue) values.storeStream(outValue + physical[it]);
+            if (Cfg::kWriteIndex) indices.storeStream(outIndex + physical[it]);
+        }
     }
+    if constexpr (ROUTE) {
+        typedef ScanRunSum R;
+        typedef ScanState<R> RS;
+        // a run begins where a position is won by itself (inclusive) or by the position just before it (exclusive), and at
+        // every row head; positions outside the chunk's data count as heads so that the last run ends before them
+        float sums[ITEMS][V];
+        u32 runHeads[ITEMS], runSealed[ITEMS];
+        RS runExclusive[ITEMS];
+        __syncthreads();  // the totals of the first scan have been read
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+            RS run = scanEmpty<R>();
+            runHeads[it] = 0;
+            runSealed[it] = 0;
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                const u32 own = (u32)(physical[it] + (Cfg::kReverse ? V - 1 - k : k));
+                const u32 opener = Cfg::kInclusive ? own : (Cfg::kReverse ? own + 1u : own - 1u);
+                RS e;
+                e.v = live[it] ? upstream[it].v[Cfg::kReverse ? V - 1 - k : k] : 0.0f;
+                e.i = kNoIndex;
+                e.head = !live[it] || winners[it][k] == opener || winners[it][k] == kNoIndex || ((rowHeads[it] >> k) & 1u) ? 1u : 0u;
+                runHeads[it] |= e.head << k;
+                run = scanCombine<R>(run, e);
+                sums[it][k] = run.v;
+                runSealed[it] |= run.head << k;
+            }
+            const RS inclusive = scanWave<R, true>(run);
+            runExclusive[it] = scanShuffleUp<R>(inclusive, 1);
+            if (lane == 0) runExclusive[it] = scanEmpty<R>();
+            if (lane == kWave - 1) {
+                totalValue[it * WAVES + wave] = __builtin_bit_cast(u32, inclusive.v);
+                totalHead[it * WAVES + wave] = inclusive.head;
+            }
+            if (lane == 0) totalIndex[it * WAVES + wave] = runHeads[it] & 1u;  // does this wavefront's round begin with a head
+        }
+        __syncthreads();
+        u32 nextWaveBegins[ITEMS];  // the head bit of the position after this wavefront's round
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) nextWaveBegins[it] = it * WAVES + wave + 1 < ITEMS * WAVES ? totalIndex[it * WAVES + wave + 1] : 1u;
+        __syncthreads();
+        if (wave == 0) {
+            RS mine = scanEmpty<R>();
+            if (lane < ITEMS * WAVES) {
+                mine.v = __builtin_bit_cast(float, totalValue[lane]);
+                mine.head = totalHead[lane];
+            }
+            const RS inclusive = scanWave<R>(mine);
+            RS before = scanShuffleUp<R>(inclusive, 1);
+            if (lane == 0) before = scanEmpty<R>();
+            if (lane < ITEMS * WAVES) {
+                totalValue[lane] = __builtin_bit_cast(u32, before.v);
+                totalHead[lane] = before.head;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+            RS base;
+            base.v = __builtin_bit_cast(float, totalValue[it * WAVES + wave]);
+            base.i = kNoIndex;
+            base.head = totalHead[it * WAVES + wave];
+            base = scanCombine<R>(base, runExclusive[it]);
+            // the head bit of the position after this vector: the next lane's first, or the next wavefront's
+            u32 following = __shfl_down(runHeads[it] & 1u, 1, kWave);
+            if (lane == kWave - 1) following = nextWaveBegins[it];
+            if (!live[it]) continue;
+            const u32 ends = (runHeads[it] >> 1) | (following << (V - 1));  // bit k: position k closes its run
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                const float sum = ((runSealed[it] >> k) & 1u) ? sums[it][k] : base.v + sums[it][k];
+                const u32 winner = winners[it][k];
+                if (((ends >> k) & 1u) && winner != kNoIndex) {
+                    const u64 position = Cfg::kReverse ? Cfg::kTotal - 1 - winner : (u64)winner;
+                    routeTile[position - chunkBase] = sum;
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+            if (!live[it]) continue;
+            const u64 local = ((u64)it * THREADS + threadIdx.x) * V;
+            Pack<float, V> out;
+#pragma unroll
+            for (int k = 0; k < V; ++k) out.v[Cfg::kReverse ? V - 1 - k : k] = routeTile[local + k];
+            out.storeStream(routed + physical[it]);
+        }
+    }
+}
+
+template <typename Cfg, bool AGGREGATE_ONLY>
+__device__ __forceinline__ void scanChunk(const typename Cfg::T* in, const u32* heads, const void* carries, void* aggregates,
+                                          typename Cfg::T* outValue, u32* outIndex) {
+    scanChunkCore<Cfg, AGGREGATE_ONLY, false>(in, heads, carries, aggregates, outValue, outIndex, nullptr, nullptr);
+}
+template <typename Cfg>
+__device__ __forceinline__ void scanRoute(const typename Cfg::T* in, const float* gradient, float* routed) {
+    scanChunkCore<Cfg, false, true>(in, nullptr, nullptr, nullptr, nullptr, nullptr, gradient, routed);
 }
 
 // One block: the totals of kChunks chunks -> the state that precedes each chunk.  A thread owns a run of consecutive chunks.

@@ -32,6 +32,76 @@ const char* scanStorageName(DataType dtype) {
     throw std::invalid_argument(std::string("Unsupported CUB scan dtype ") + dataTypeName(dtype) + ".");
 }
 
+struct ScanChunking {
+    uint64_t vec = 1, threads = 256, items = 4, chunkElems = 0;
+    bool carry = true;
+    bool routable = false;  // a request with route set can run as it is
+};
+
+ScanChunking chooseScanChunking(const ScanRequest& r) {
+    ScanChunking c;
+    const bool ragged = r.row == 0;
+    const uint32_t elementBytes = dataTypeSizeInBytes(r.dtype);
+    c.vec = 16 / elementBytes;
+    while (c.vec > 1 && (r.total % c.vec != 0 || r.alignmentBytes % (c.vec * std::max<uint32_t>(elementBytes, r.writeIndex || r.route ? 4 : elementBytes)) != 0)) {
+        c.vec /= 2;
+    }
+    bool threadsForced = false;
+    if (const char* env = std::getenv("THOR_SCAN_THREADS")) {  // tuning switch: 256, 512 or 1024 threads per block
+        const long requested = std::atol(env);
+        if (requested == 256 || requested == 512 || requested == 1024) {
+            c.threads = static_cast<uint64_t>(requested);
+            threadsForced = true;
+        }
+    }
+    const uint64_t lanesWorth = c.threads * c.vec;
+    uint64_t maxItems = 64 / (c.threads / 64) < 16 ? 64 / (c.threads / 64) : 16;
+    // routing a gradient keeps an fp32 copy of the chunk in LDS: at most 32 KiB of it
+    if (r.route) maxItems = std::min<uint64_t>(maxItems, kScanRouteMaxChunkElems / lanesWorth);
+    c.chunkElems = lanesWorth * c.items;
+    if (!ragged && maxItems > 0 && r.row <= lanesWorth * maxItems) {
+        // chunks of whole rows: every chunk starts at a head and needs nothing from its predecessors
+        const uint64_t step = c.vec / std::gcd(r.row, c.vec);  // rows per chunk must keep chunk starts on vector boundaries
+        const uint64_t rowsPerChunk = std::max<uint64_t>(lanesWorth * std::min<uint64_t>(4, maxItems) / r.row / step * step, step);
+        if (rowsPerChunk * r.row <= lanesWorth * maxItems) {
+            c.chunkElems = rowsPerChunk * r.row;
+            c.items = (c.chunkElems + lanesWorth - 1) / lanesWorth;
+            c.carry = false;
+        }
+    }
+    if (!c.carry && !threadsForced) {
+        // A chunk of whole rows keeps its size; more threads hold fewer vectors each.  Measured on [8192, 8192] fp32 (256 / 512 /
+        // 1024 threads): running sum 96 / 91 / 95 us, running arg-max 106 / 88 / 93 us, routed gradient 239 / 162 / 139 us - the
+        // register arrays of the longer per-thread walks cost more residency than the extra wavefront totals.
+        const uint64_t wanted = r.route ? 2 : 4;
+        while (c.items > wanted && c.threads < 1024) {
+            c.threads *= 2;
+            c.items = (c.chunkElems + c.threads * c.vec - 1) / (c.threads * c.vec);
+        }
+    }
+    c.routable = !c.carry && !ragged && (r.op == 1 || r.op == 2);
+    if (c.carry) {
+        c.items = std::min<uint64_t>(8, std::max<uint64_t>(maxItems, 1));
+        c.chunkElems = lanesWorth * c.items;
+    }
+    return c;
+}
+
+void writeScanTraits(std::ostringstream& s, const ScanRequest& r, bool isUnsigned, uint64_t threads, uint64_t vec, uint64_t items, uint64_t chunkElems,
+                     const CubScanKernels& k) {
+    s << "namespace gen {\nstruct Cfg {\n    typedef " << scanStorageName(r.dtype) << " T;\n    typedef " << (isUnsigned ? "thor::u32" : "float")
+      << " Acc;\n    typedef " << (r.offsets64 ? "thor::u64" : "thor::u32") << " OffsetT;\n"
+      << "    static constexpr bool kUnsigned = " << (isUnsigned ? "true" : "false") << ";\n    static constexpr int kOp = " << r.op
+      << ";\n    static constexpr bool kArg = " << (r.writeIndex ? "true" : "false") << ";\n    static constexpr bool kInclusive = "
+      << (r.inclusive ? "true" : "false") << ";\n    static constexpr bool kReverse = " << (r.reverse ? "true" : "false")
+      << ";\n    static constexpr thor::u64 kTotal = " << r.total << "ull;\n    static constexpr thor::u64 kRow = " << r.row
+      << "ull;\n    static constexpr thor::u64 kSegments = " << r.segments << "ull;\n    static constexpr int kThreads = " << threads
+      << ";\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kItems = " << items
+      << ";\n    static constexpr thor::u64 kChunkElems = " << chunkElems << "ull;\n    static constexpr thor::u64 kChunks = " << k.chunks
+      << "ull;\n    static constexpr bool kCarry = " << (k.carry ? "true" : "false") << ";\n    static constexpr bool kWriteValue = "
+      << (r.writeValue ? "true" : "false") << ";\n    static constexpr bool kWriteIndex = " << (r.writeIndex ? "true" : "false") << ";\n};\n}  // namespace gen\n";
+}
+
 }  // namespace
 
 bool isCubScanDTypeSupported(DataType dtype) {
@@ -56,32 +126,12 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
     auto kernels = std::make_shared<CubScanKernels>();
     CubScanKernels& k = *kernels;
     k.request = r;
-    const uint32_t elementBytes = dataTypeSizeInBytes(r.dtype);
-    uint64_t vec = 16 / elementBytes;
-    while (vec > 1 && (r.total % vec != 0 || r.alignmentBytes % (vec * std::max<uint32_t>(elementBytes, r.writeIndex ? 4 : elementBytes)) != 0)) vec /= 2;
-    uint64_t threads = 256;
-    if (const char* env = std::getenv("THOR_SCAN_THREADS")) {  // tuning switch: 256, 512 or 1024 threads per block
-        const long requested = std::atol(env);
-        if (requested == 256 || requested == 512 || requested == 1024) threads = static_cast<uint64_t>(requested);
+    const ScanChunking chunking = chooseScanChunking(r);
+    if (r.route && !chunking.routable) {
+        throw std::invalid_argument("CUB scan: the one-pass gradient routing needs a min / max scan over rows that fit one block's chunk.");
     }
-    const uint64_t lanesWorth = threads * vec, maxItems = 64 / (threads / 64) < 16 ? 64 / (threads / 64) : 16;
-    uint64_t items = 4;
-    uint64_t chunkElems = lanesWorth * items;
-    k.carry = true;
-    if (!ragged && r.row <= lanesWorth * maxItems) {
-        // chunks of whole rows: every chunk starts at a head and needs nothing from its predecessors
-        const uint64_t step = vec / std::gcd(r.row, vec);  // rows per chunk must keep chunk starts on vector boundaries
-        uint64_t rowsPerChunk = std::max<uint64_t>(lanesWorth * 4 / r.row / step * step, step);
-        if (rowsPerChunk * r.row <= lanesWorth * maxItems) {
-            chunkElems = rowsPerChunk * r.row;
-            items = (chunkElems + lanesWorth - 1) / lanesWorth;
-            k.carry = false;
-        }
-    }
-    if (k.carry) {
-        items = std::min<uint64_t>(8, maxItems);
-        chunkElems = lanesWorth * items;
-    }
+    const uint64_t vec = chunking.vec, threads = chunking.threads, items = chunking.items, chunkElems = chunking.chunkElems;
+    k.carry = chunking.carry;
     k.threads = static_cast<uint32_t>(threads);
     k.chunks = (r.total + chunkElems - 1) / chunkElems;
     if (k.chunks == 1) k.carry = false;
@@ -97,19 +147,23 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
     }
 
     const bool isUnsigned = r.dtype == DataType::UINT32;
+    if (r.route) {
+        std::ostringstream s;
+        s << thor_embed::kDevicePrelude << thor_embed::kScanKernels;
+        writeScanTraits(s, r, isUnsigned, threads, vec, items, chunkElems, k);
+        s << "extern \"C\" __global__ __launch_bounds__(" << threads
+          << ") void thor_scan_route(const gen::Cfg::T* in, const float* gradient, float* routed) {\n    thor::scanRoute<gen::Cfg>(in, gradient, routed);\n}\n";
+        k.mainKernel = compileKernel(s.str(), "thor_scan_route", r.deviceNum, /*fastContract=*/false);
+        std::ostringstream v;
+        v << "scan-route " << (r.op == 1 ? "min" : "max") << (r.inclusive ? " inclusive" : " exclusive") << (r.reverse ? " reverse" : "") << " rows" << r.row
+          << " chunk" << chunkElems << " vec" << vec << " threads" << threads << " launches1";
+        k.variant = v.str();
+        return kernels;
+    }
     std::ostringstream s;
     s << thor_embed::kDevicePrelude << thor_embed::kScanKernels;
-    s << "namespace gen {\nstruct Cfg {\n    typedef " << scanStorageName(r.dtype) << " T;\n    typedef " << (isUnsigned ? "thor::u32" : "float")
-      << " Acc;\n    typedef " << (r.offsets64 ? "thor::u64" : "thor::u32") << " OffsetT;\n"
-      << "    static constexpr bool kUnsigned = " << (isUnsigned ? "true" : "false") << ";\n    static constexpr int kOp = " << r.op
-      << ";\n    static constexpr bool kArg = " << (r.writeIndex ? "true" : "false") << ";\n    static constexpr bool kInclusive = "
-      << (r.inclusive ? "true" : "false") << ";\n    static constexpr bool kReverse = " << (r.reverse ? "true" : "false")
-      << ";\n    static constexpr thor::u64 kTotal = " << r.total << "ull;\n    static constexpr thor::u64 kRow = " << r.row
-      << "ull;\n    static constexpr thor::u64 kSegments = " << r.segments << "ull;\n    static constexpr int kThreads = " << threads
-      << ";\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kItems = " << items
-      << ";\n    static constexpr thor::u64 kChunkElems = " << chunkElems << "ull;\n    static constexpr thor::u64 kChunks = " << k.chunks
-      << "ull;\n    static constexpr bool kCarry = " << (k.carry ? "true" : "false") << ";\n    static constexpr bool kWriteValue = "
-      << (r.writeValue ? "true" : "false") << ";\n    static constexpr bool kWriteIndex = " << (r.writeIndex ? "true" : "false") << ";\n};\n}  // namespace gen\n";
+    writeScanTraits(s, r, isUnsigned, threads, vec, items, chunkElems, k);
+
     s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void thor_scan_main(const gen::Cfg::T* in, const thor::u32* heads, const void* carries, "
          "gen::Cfg::T* outValue, thor::u32* outIndex) {\n    thor::scanChunk<gen::Cfg, false>(in, heads, carries, nullptr, outValue, outIndex);\n}\n";
     if (k.carry) {
@@ -178,7 +232,26 @@ void launchScan(const CubScanKernels& k, const void* input, const void* offsets,
     k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, mainArgs);
 }
 
+bool scanRouteFits(const ScanRequest& request) {
+    ScanRequest routed = request;
+    routed.route = true;
+    return request.total != 0 && request.row != 0 && request.total % request.row == 0 && isCubScanDTypeSupported(request.dtype) &&
+           chooseScanChunking(routed).routable;
+}
+
+void launchScanRoute(const CubScanKernels& k, const void* input, const void* gradient, void* routed, Stream& stream) {
+    if (!k.request.route) throw std::invalid_argument("CUB scan: these kernels do not route a gradient.");
+    if (!stream.isInitialized() || stream.getGpuNum() != k.request.deviceNum) throw std::invalid_argument("CUB scan stream must live on the plan's GPU.");
+    ScopedGpu scoped(k.request.deviceNum);
+    std::vector<void*> args = {&input, &gradient, &routed};
+    k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, stream.getStream(), args);
+}
+
 void StampedScan::runOn(Stream& stream) const {
+    if (gradient.isInitialized()) {
+        launchScanRoute(*kernels, input.getMemPtr(), gradient.getMemPtr(), const_cast<Tensor&>(values).getMemPtr(), stream);
+        return;
+    }
     launchScan(*kernels, input.getMemPtr(), offsets.has_value() ? offsets->getMemPtr() : nullptr, const_cast<Tensor&>(temp).getMemPtr(),
                temp.getTotalNumElements(), values.isInitialized() ? const_cast<Tensor&>(values).getMemPtr() : nullptr,
                indices.isInitialized() ? const_cast<Tensor&>(indices).getMemPtr() : nullptr, stream);

@@ -20,6 +20,10 @@ struct ScanRequest {
     bool writeValue = true, writeIndex = false;
     bool inclusive = true, reverse = false;
     uint64_t alignmentBytes = 256;  // largest power of two (capped at 256) dividing the input and output addresses
+    // Not a scan of its own: the gradient of the min / max scan described above, in one launch (reads the operand and an FP32
+    // upstream gradient, writes the FP32 gradient of the operand).  Only for rows (row != 0) that fit a block's chunk; see
+    // scanRouteFits.
+    bool route = false;
     int deviceNum = 0;
 };
 
@@ -32,6 +36,12 @@ struct CubScanKernels {
     size_t headsBytes = 0, statesBytes = 0, tempBytes = 1;
     std::string variant;
 };
+
+constexpr uint64_t kScanRouteMaxChunkElems = 8192;
+// Whether buildScanKernels accepts `request` with route set (otherwise the gradient takes an arg scan and a scatter).
+bool scanRouteFits(const ScanRequest& request);
+// Launches the routing kernel of a request built with route set.
+void launchScanRoute(const CubScanKernels& kernels, const void* input, const void* gradient, void* routed, Stream& stream);
 
 // loadedOnly: take every kernel from the process-wide cache and throw std::runtime_error when one is missing, so that nothing is
 // compiled or loaded (for callers that must not allocate).  A request whose temporary storage exceeds tempLimitBytes is rejected

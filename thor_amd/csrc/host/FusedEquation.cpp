@@ -1467,6 +1467,26 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                     request.row = dims[n.lhs].back();
                     request.segments = request.total / request.row;
                 }
+                if (!segmented && gradient.getDataType() == DataType::FP32 && n.output_dtype.value() == DataType::FP32) {
+                    // rows that fit one block: winners, the sums of the gradient over the positions each of them won, and the
+                    // gradient of the operand in one launch (every element is written, so nothing is cleared first)
+                    Tensor routed = allocateFor(i);
+                    ScanRequest oneLaunch = request;
+                    oneLaunch.route = true;
+                    oneLaunch.alignmentBytes = std::min({pointerAlignment(values.getMemPtr()), pointerAlignment(gradient.getMemPtr()), pointerAlignment(routed.getMemPtr())});
+                    if (scanRouteFits(oneLaunch)) {
+                        StampedExecutionStage routeStage;
+                        routeStage.kind = StampedExecutionStage::Kind::Scan;
+                        routeStage.gpu_num = device_num;
+                        routeStage.dependency_stage_indices = dependenciesOf({n.lhs, n.rhs});
+                        routeStage.scan = std::make_shared<StampedScan>(StampedScan::routing(buildScanKernels(oneLaunch), values, gradient, routed));
+                        tensorOf[i] = routed;
+                        stageOfNode[i] = static_cast<int>(stages.size());
+                        stages.push_back(std::move(routeStage));
+                        done[i] = 1;
+                        continue;
+                    }
+                }
                 const std::shared_ptr<const CubScanKernels> kernels = buildScanKernels(request);
                 Tensor temp(gpuPlacement, TensorDescriptor(DataType::UINT8, {std::max<uint64_t>(kernels->tempBytes, 1)}));
                 StampedExecutionStage scanStage;
