@@ -283,8 +283,9 @@ struct ArgAcc {
     // equal value never replaces the candidate: only a strictly better value, the first NaN, or the first element at all.
     template <typename I>
     __device__ __forceinline__ void add(float x, I index) {
-        const bool strictlyBetter = IS_MAX ? (x > v) : (x < v);
-        const bool take = strictlyBetter | ((x != x) & (v == v)) | (i == ~(IndexT)0);
+        // strictly better, or the first NaN: "not (x no better than v)" holds for both, and a NaN that is held stays
+        const bool noBetter = IS_MAX ? (x <= v) : (x >= v);
+        const bool take = (!noBetter & (v == v)) | (i == ~(IndexT)0);
         v = take ? x : v;  // selects, not branches: lanes of a wavefront rarely agree
         i = take ? (IndexT)index : i;
     }

@@ -374,8 +374,9 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::Sources& src, 
 //                    chunk's `head` partial, a piece of a segment that continues into the next chunk to its `tail` partial
 //   finishSegments   folds tail[c] with head[c + 1 .. c1] for every segment that spans chunks
 // Offsets are clamped to the row count, so an invalid partition gives meaningless results but never reads outside the
-// values tensor.  An element's index (arg reductions) is its packed position row * kD + d; empty segments keep the
-// accumulator's identity (sum 0, min +inf, max -inf, index all-ones) and a mean over zero rows is 0.
+// values tensor.  An element's index (arg reductions) is its packed position row * kD + d; the candidates carry the row alone
+// (every thread, team and partial belongs to one trailing element d, so rows order like positions) and Cfg::store packs it.
+// Empty segments keep the accumulator's identity (sum 0, min +inf, max -inf, index all-ones) and a mean over zero rows is 0.
 // Workspace: accumulators [kChunks][2][kD]; u64 tails[kChunks] (the segment whose tail the chunk holds, or all-ones);
 // u64 firstSegment[kChunks].
 // Cfg: kD, kRows, kSegments, kColumnTiles, kLanesX, kBatch, kChunkRows, kChunks, kMinTeam, kFinishLanes, kFinishThreads,
@@ -546,9 +547,9 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
                 for (int u = 0; u < kBatch; ++u) Cfg::load(src, (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset, x[u]);
 #pragma unroll
                 for (int u = 0; u < kBatch; ++u) {
-                    const u64 base = (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset;
+                    const IndexT row = (IndexT)(r0 + (u64)u * rowLanes);
 #pragma unroll
-                    for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, (IndexT)(base + k));
+                    for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, row);
                 }
             } else {
                 bool live[kBatch];
@@ -562,9 +563,9 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
 #pragma unroll
                 for (int u = 0; u < kBatch; ++u) {
                     if (live[u]) {
-                        const u64 base = (r0 + (u64)u * rowLanes) * Cfg::kD + columnOffset;
+                        const IndexT row = (IndexT)(r0 + (u64)u * rowLanes);
 #pragma unroll
-                        for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, (IndexT)(base + k));
+                        for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, row);
                     }
                 }
             }

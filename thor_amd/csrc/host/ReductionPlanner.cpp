@@ -223,10 +223,16 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
 
     if (request.segmented) {
         shape.kernel = ReductionShape::Kernel::Segments;
-        shape.indexIs64 = true;  // packed global indices; the all-ones sentinel must survive the conversion to a 64-bit output
+        // candidates carry the row of the element (32 bits while rows fit: half the registers, shuffles and partial bytes); the
+        // store packs row * trailing + element into the output's index type and keeps the all-ones mark of an empty segment
+        shape.indexIs64 = request.segmentedRows >= 0xffffffffull;
         shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {request.trailing});
         shape.threads = 256;
         shape.unroll = 8;
+        if (const char* env = std::getenv("THOR_SEGMENT_BATCH")) {  // tuning switch: rows in flight per lane
+            const long requested = std::atol(env);
+            if (requested == 1 || requested == 2 || requested == 4 || requested == 8 || requested == 16) shape.unroll = static_cast<int>(requested);
+        }
         const uint64_t columnsPerRow = request.trailing / shape.vec;
         shape.threadsPerRow = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(columnsPerRow)));
         const uint64_t lanesX = static_cast<uint64_t>(shape.threadsPerRow);
@@ -243,7 +249,13 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         shape.chunks = std::max<uint64_t>(ceilDiv(request.segmentedRows, shape.chunkRows), 1);
         // the smallest team that shares one segment: eight rows in flight per lane should cover an average segment
         const uint64_t rowLanes = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(averageRows) / shape.unroll, 1), 8);
-        shape.minTeam = static_cast<int>(std::min<uint64_t>(lanesX * rowLanes, 256));
+        // ... and a team no wider than a wavefront folds with shuffles alone (no LDS round, no barriers): log-normal segments
+        // of 64 rows x 64 fp32 on average, teams of 128 -> 64 threads: sum 209 -> 193 us, arg-max 340 -> 282 us
+        shape.minTeam = static_cast<int>(std::min<uint64_t>(lanesX * rowLanes, std::max<uint64_t>(lanesX, 64)));
+        if (const char* env = std::getenv("THOR_SEGMENT_MIN_TEAM")) {  // tuning switch: threads of the smallest team
+            const uint64_t requested = static_cast<uint64_t>(std::atol(env));
+            if (requested >= lanesX && requested <= 256 && (requested & (requested - 1)) == 0) shape.minTeam = static_cast<int>(requested);
+        }
         shape.finishLanes = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(request.trailing)));
         // a segment of average length runs over averageRows / chunkRows chunks, folded by finishThreads / finishLanes row
         // lanes: one wavefront while that leaves each lane a handful of partials, else a block
@@ -251,7 +263,7 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         shape.blocks = tiles;
         shape.gridX = static_cast<uint32_t>(shape.chunks * tiles);
         shape.gridY = 1;
-        if (shape.chunks > 1) shape.workspaceBytes = partialBytes(shape.chunks * 2 * request.trailing, request.isArg, true) + shape.chunks * 16;
+        if (shape.chunks > 1) shape.workspaceBytes = partialBytes(shape.chunks * 2 * request.trailing, request.isArg, shape.indexIs64) + shape.chunks * 16;
         return shape;
     }
 
@@ -508,7 +520,16 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     s << "    static __device__ __forceinline__ void store(const Acc& acc, u64 outIndex, const Outputs& o, float scale, float divisor = kDivisor) {\n";
     if (request.isArg) {
         if (request.writeValue) s << "        o.out0[outIndex] = fromFloat<" << deviceTypeName(values[0].outputDType) << ">(acc.v);\n";
-        if (request.writeIndex) s << "        o.indexOut[outIndex] = (" << (request.indexOutputDType == DataType::UINT64 ? "u64" : "u32") << ")acc.i;\n";
+        if (request.writeIndex) {
+            const char* stored = request.indexOutputDType == DataType::UINT64 ? "u64" : "u32";
+            if (request.segmented) {
+                // the candidate holds a row; the packed position adds the trailing element this output belongs to
+                s << "        o.indexOut[outIndex] = acc.i == ~(IndexT)0 ? ~(" << stored << ")0 : (" << stored << ")((u64)acc.i * " << request.trailing
+                  << "ull + outIndex % " << request.trailing << "ull);\n";
+            } else {
+                s << "        o.indexOut[outIndex] = acc.i == ~(IndexT)0 ? ~(" << stored << ")0 : (" << stored << ")acc.i;\n";
+            }
+        }
         s << "        (void)scale;\n";
     } else {
         for (size_t j = 0; j < values.size(); ++j) {
@@ -632,7 +653,12 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     finishParams << "void* indexOut";
     outputInit << "static_cast<decltype(gen::Cfg::Outputs::indexOut)>(indexOut)";
     finishInit << "static_cast<decltype(gen::Cfg::Outputs::indexOut)>(indexOut)";
-    s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads << ") void thor_reduce_main(";
+    s << "extern \"C\" __global__ __launch_bounds__(" << shape.threads << ") ";
+    if (const char* env = std::getenv("THOR_REDUCE_WAVES_PER_SIMD")) {  // tuning switch: register budget for N resident wavefronts per SIMD
+        const long requested = std::atol(env);
+        if (requested >= 1 && requested <= 8) s << "__attribute__((amdgpu_waves_per_eu(" << requested << "))) ";
+    }
+    s << "void thor_reduce_main(";
     for (size_t i = 0; i < sources.size(); ++i) s << "const " << deviceTypeName(sources[i].storage) << "* in" << i << ", ";
     for (uint32_t slot : request.scalarSlots) s << "float s" << slot << ", ";
     s << outputParams.str() << ", void* partials, float scale" << (request.segmented ? ", const void* offsets" : "") << ") {\n    const gen::Cfg::Sources src{";
