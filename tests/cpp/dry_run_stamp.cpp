@@ -182,7 +182,9 @@ static int runAll() {
             const std::unordered_map<std::string, Tensor> ropeInputs{{"q", q}, {"odd", odd}, {"positions", positions}, {"length", length}};
             const Expression iq = Expression::input("q"), iodd = Expression::input("odd");
             RotaryPositionEmbeddingOptions o;
-            stampOne(std::string("rope ") + dtypeName + " plain", iq.rope(o) * 2.0, ropeInputs, stream);
+            stampOne(std::string("rope ") + dtypeName + " plain", iq.rope(o) * 2.0, ropeInputs, stream, "FusedKernel");
+            stampOne(std::string("rope ") + dtypeName + " between products and sums", (iq * iq + iq.tanh()).rope(o) * iq + iq * 0.5, ropeInputs, stream,
+                     "FusedKernel");
             o.interleaved = true;
             o.rotary_dim = 32;
             stampOne(std::string("rope ") + dtypeName + " interleaved partial", (iq + 1.0).rope(o), ropeInputs, stream);

@@ -266,6 +266,70 @@ def test_rotation_inside_a_larger_graph(stream):
                                oracle_rope(swapped, DataType.fp32, {"sequence_axis": 3, "head_dim_axis": 2}), rtol=0, atol=tol)
 
 
+def _neighbour_graphs():
+    x, y, z, a = ex.input("x"), ex.input("y"), ex.input("z"), ex.runtime_scalar("a")
+    return [
+        ("affine_before_scale_after", lambda: (x * 2.0 + 1.0).rope() * 0.5, (2, 3, 40, 32), DataType.fp32, "x"),
+        ("products_and_sums_of_three_tensors", lambda: (x * y + z).rope(rotary_dim=16) * y + z * x, (2, 3, 40, 32), DataType.fp32, "xyz"),
+        ("transcendental_neighbours", lambda: (x.tanh() * y).rope(interleaved=True).exp() / (z * z + 1.0), (2, 3, 40, 32), DataType.fp32, "xyz"),
+        ("runtime_scalar_both_sides", lambda: (x * a + y).rope() * a + 1.0, (2, 3, 40, 32), DataType.fp32, "xya"),
+        ("heads_after_sequence", lambda: (x - y).rope(sequence_axis=1, head_dim_axis=3) + z, (2, 40, 3, 32), DataType.fp32, "xyz"),
+        ("bf16_every_step_rounded", lambda: (x * y + z).rope() * y - x, (2, 3, 40, 32), DataType.bf16, "xyz"),
+        ("fp16_partial_interleaved", lambda: (x + y).rope(rotary_dim=16, interleaved=True) * z, (2, 3, 40, 32), DataType.fp16, "xyz"),
+        ("only_after", lambda: x.rope() * y + 0.25, (2, 3, 40, 32), DataType.fp32, "xy"),
+        ("only_before", lambda: (x * y).rope(), (2, 3, 40, 32), DataType.fp32, "xy"),
+        ("llama3_long_head", lambda: (x * 0.5 + y).rope(scaling_kind=RotaryScalingKind.llama3, scaling_factor=8.0, original_max_position_embeddings=16) - z,
+         (1, 2, 64, 128), DataType.bf16, "xyz"),
+    ]
+
+
+@pytest.mark.parametrize("name", [g[0] for g in _neighbour_graphs()])
+def test_elementwise_neighbours_run_inside_the_rotation(stream, monkeypatch, name):
+    """(x * 2 + 1).rope() * 0.5 is one kernel (one FusedKernel stage there too: RoPE is an operation of the reference's fused kernels)
+    and gives, bit for bit, what the plan of separate elementwise and rotation kernels gives."""
+    _, build, shape, dtype, used = next(g for g in _neighbour_graphs() if g[0] == name)
+    rng = np.random.default_rng(abs(hash(name)) % 1000)
+    tensors = {k: copy_numpy_to_gpu(to_storage(rng.standard_normal(shape).astype(np.float32), dtype), stream, dtype) for k in "xyz"}
+    results = {}
+    for fused in (True, False):
+        if fused:
+            monkeypatch.delenv("THOR_DISABLE_STAGE_FUSION", raising=False)
+        else:
+            monkeypatch.setenv("THOR_DISABLE_STAGE_FUSION", "1")
+        equation = ex.compile(ex.outputs({"y": build()}), device_num=0)
+        plan = equation.stamp({k: t for k, t in tensors.items() if k in used}, stream)
+        plan.run({"a": 1.75} if "a" in used else None)
+        results[fused] = (plan.stage_kind_names(), plan.stage_descriptions(), copy_gpu_to_numpy(plan.output("y"), stream))
+    kinds, descriptions, fused_values = results[True]
+    assert kinds == ["FusedKernel"] and descriptions[0].startswith("fused "), descriptions
+    assert ("prologue+" in descriptions[0]) == (name != "only_after") and ("+epilogue" in descriptions[0]) == (name != "only_before")
+    assert len(results[False][0]) == 1 + (name != "only_after") + (name != "only_before")
+    if name == "products_and_sums_of_three_tensors":
+        # r * y + z * x: which of the two products joins the addition in one fused multiply-add is the compiler's choice in each
+        # kernel; the two results differ by at most the rounding of the product that was rounded on its own
+        staged = results[False][2].astype(np.float64)
+        zx = np.abs(copy_gpu_to_numpy(tensors["z"], stream).astype(np.float64) * copy_gpu_to_numpy(tensors["x"], stream).astype(np.float64))
+        assert np.all(np.abs(fused_values.astype(np.float64) - staged) <= 2.0 ** -23 * (np.abs(staged) + 2 * zx))
+    else:
+        np.testing.assert_array_equal(fused_values.view(np.uint8), results[False][2].view(np.uint8))
+
+
+def test_a_rotation_read_twice_or_named_keeps_its_own_tensor(stream):
+    rng = np.random.default_rng(39)
+    x32 = rng.standard_normal((2, 3, 40, 32)).astype(np.float32)
+    ix = ex.input("x")
+    turned = (ix * 2.0).rope()
+    plan = run({"turned": turned, "half": turned * 0.5, "squared": turned * turned}, {"x": copy_numpy_to_gpu(x32, stream, DataType.fp32)}, stream)
+    # the operand is still computed inside the rotation; its two readers share one elementwise kernel
+    assert len(plan.stage_kind_names()) == 2 and "prologue+" in plan.stage_descriptions()[0] and "+epilogue" not in plan.stage_descriptions()[0]
+    expected = oracle_rope(x32 * np.float32(2), DataType.fp32, {})
+    tol = angle_tolerance(2 * x32, 40.0, DataType.fp32)
+    got = copy_gpu_to_numpy(plan.output("turned"), stream)
+    np.testing.assert_allclose(got, expected, rtol=0, atol=tol)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("half"), stream), got * np.float32(0.5))
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("squared"), stream), got * got)
+
+
 def test_output_dtype_and_equal_parameters_share_kernels(stream):
     rng = np.random.default_rng(36)
     x = to_storage(rng.standard_normal((1, 2, 33, 64)).astype(np.float32), DataType.fp16)

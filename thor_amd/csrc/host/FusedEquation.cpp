@@ -635,6 +635,23 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             for (uint32_t i = 0; i < count; ++i) {
                 if (graph->expr.nodes[i].op == ExprOp::SEGMENTED_BROADCAST && used[i] && fusable[i] && !named[i]) graph->role[i] = Role::Gather;
             }
+            // An elementwise value that only one rotation reads is computed inside the rotation's kernel, element by element.
+            for (uint32_t r = 0; r < count; ++r) {
+                const ExprNode& rope = graph->expr.nodes[r];
+                if (rope.op != ExprOp::ROPE) continue;
+                const uint32_t m = rope.lhs;
+                const ExprNode& operand = graph->expr.nodes[m];
+                const bool elementwise = Expression::isBinaryOp(operand.op) || operand.op == ExprOp::WHERE || operand.op == ExprOp::CAST ||
+                                         (Expression::isUnaryOp(operand.op) && !isReductionOp(operand.op) && !isShapeOnly(operand.op) && operand.op != ExprOp::SOFTMAX);
+                if (graph->role[m] != Role::Materialized || named[m] || !elementwise) continue;
+                bool ok = true;
+                for (uint32_t j = 0; j < count && ok; ++j) {
+                    const ExprNode& consumer = graph->expr.nodes[j];
+                    if (j != r && (consumer.lhs == m || consumer.rhs == m || consumer.aux == m)) ok = false;
+                }
+                if (rope.rhs == m || rope.aux == m) ok = false;
+                if (ok) graph->role[m] = Role::Inline;
+            }
             // An elementwise value that only segmented reductions over one partition need as a tensor is never stored: the
             // reduction evaluates it in registers (per-segment values of the same partition are read once per segment), and
             // elementwise consumers recompute it.
@@ -687,8 +704,14 @@ std::shared_ptr<PlannedGraph> FusedEquation::plannedGraphFor(const std::vector<D
             } else if (graph->expr.nodes[i].op == ExprOp::SCAN) {
                 sources.push_back(graph->expr.nodes[i].lhs);
             } else if (graph->expr.nodes[i].op == ExprOp::ROPE || isScatterRoutingOp(graph->expr.nodes[i].op)) {
-                for (uint32_t operand : {graph->expr.nodes[i].lhs, graph->expr.nodes[i].rhs, graph->expr.nodes[i].aux})
-                    if (operand != UINT32_MAX) sources.push_back(operand);
+                for (uint32_t operand : {graph->expr.nodes[i].lhs, graph->expr.nodes[i].rhs, graph->expr.nodes[i].aux}) {
+                    if (operand == UINT32_MAX) continue;
+                    if (graph->role[operand] == Role::Inline) {
+                        collectSources(*graph, operand, sources, scalars);  // evaluated inside the rotation
+                    } else {
+                        sources.push_back(operand);
+                    }
+                }
             } else if (isWinnerRoutingOp(graph->expr.nodes[i].op) || graph->expr.nodes[i].op == ExprOp::TAKE_ALONG_AXIS ||
                        graph->expr.nodes[i].op == ExprOp::SEGMENTED_SCAN) {
                 sources.push_back(graph->expr.nodes[i].lhs);
@@ -899,8 +922,14 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
             } else if (n.op == ExprOp::SCAN) {
                 sources = {n.lhs};
             } else if (n.op == ExprOp::ROPE || isScatterRoutingOp(n.op)) {
-                for (uint32_t operand : {n.lhs, n.rhs, n.aux})
-                    if (operand != UINT32_MAX) sources.push_back(operand);
+                for (uint32_t operand : {n.lhs, n.rhs, n.aux}) {
+                    if (operand == UINT32_MAX) continue;
+                    if (graph->role[operand] == Role::Inline) {
+                        collectSources(*graph, operand, sources, scalars);
+                    } else {
+                        sources.push_back(operand);
+                    }
+                }
             } else if (isWinnerRoutingOp(n.op) || n.op == ExprOp::TAKE_ALONG_AXIS || n.op == ExprOp::SEGMENTED_SCAN) {
                 sources = {n.lhs, n.rhs};
             } else if (isSegmentedReduceOp(n.op) || n.op == ExprOp::SEGMENTED_BROADCAST) {
@@ -1517,20 +1546,135 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                 continue;
             }
             if (n.op == ExprOp::ROPE) {
-                Tensor rotated = allocateFor(i);
+                const std::vector<uint64_t> shape = orScalarShape(dims[i]);
+                RopeFusion fusion;
+                std::vector<uint32_t> operands;
+                // Elementwise statements for `root` over tensors of the rotated shape (placeholders "@<tag><index>@" stand for their
+                // loaded elements), runtime scalars and, in an epilogue, the rotated value.  False: something else is involved.
+                auto buildPiece = [&](uint32_t root, bool epilogue, RopeFusion::Piece& piece, std::vector<uint32_t>& pieceSources) -> bool {
+                    std::vector<uint32_t> sources, scalarSlots;
+                    collectSources(*graph, root, sources, scalarSlots);
+                    BodyEmitter body(expr);
+                    std::string text;
+                    bool readsRotation = false;
+                    for (uint32_t source : sources) {
+                        if (epilogue && source == i) {
+                            body.defineSource(i, n.output_dtype.value(), "@R@");
+                            readsRotation = true;
+                            continue;
+                        }
+                        const Tensor& t = tensorOf[source];
+                        if (!done[source] && expr.nodes[source].op != ExprOp::INPUT && graph->role[source] != Role::InputSource) return false;
+                        if (!t.isInitialized() || !t.isDenseContiguous() || t.getDimensions() != shape) return false;
+                        const DataType valueDType = expr.nodes[source].output_dtype.value();
+                        const std::string raw = std::string("@") + (epilogue ? "E" : "P") + std::to_string(piece.tensors.size()) + "@";
+                        text += "const " + std::string(valueCType(valueDType)) + " t" + std::to_string(source) + " = " +
+                                castValueExpr(storageToValueExpr(raw, t.getDataType()), t.getDataType(), valueDType) + ";\n";
+                        body.defineSource(source, valueDType);
+                        piece.tensors.push_back(t);
+                        pieceSources.push_back(source);
+                    }
+                    if (epilogue && !readsRotation) return false;
+                    if (piece.tensors.empty() && !epilogue) return false;
+                    piece.contract = true;
+                    for (uint32_t v : body.collect({root})) {
+                        const ExprNode& node = expr.nodes[v];
+                        const bool elementwise = Expression::isBinaryOp(node.op) || node.op == ExprOp::WHERE || node.op == ExprOp::CAST ||
+                                                 node.op == ExprOp::RUNTIME_SCALAR || node.op == ExprOp::SCALAR_FP ||
+                                                 (Expression::isUnaryOp(node.op) && !isReductionOp(node.op) && !isShapeOnly(node.op) && node.op != ExprOp::SOFTMAX);
+                        if (!elementwise) return false;
+                        const DataType c = emittedValueDType(node);
+                        if (c == DataType::FP16 || c == DataType::BF16) piece.contract = false;
+                        fusion.extraFlopsPerElement += body.emit(text, v, "");
+                    }
+                    piece.statements = text;
+                    const DataType stored = expr.nodes[root].output_dtype.value();
+                    piece.value = epilogue ? valueToStorageExpr(body.ref(root, stored), stored) : castValueExpr(body.ref(root, stored), stored, DataType::FP32);
+                    for (uint32_t slot : scalarSlots) {
+                        if (std::find(fusion.scalarSlots.begin(), fusion.scalarSlots.end(), slot) == fusion.scalarSlots.end()) {
+                            fusion.scalarSlots.push_back(slot);
+                            fusion.scalarNames.push_back(root_inputs.at(slot).name);
+                        }
+                    }
+                    return true;
+                };
+                // the operand: a tensor, or elementwise work the planner left to this kernel
+                Tensor shapeCarrier;
+                if (graph->role[n.lhs] == Role::Inline) {
+                    RopeFusion saved = fusion;
+                    RopeFusion::Piece piece;
+                    std::vector<uint32_t> pieceSources;
+                    if (stageFusion && buildPiece(n.lhs, false, piece, pieceSources)) {
+                        fusion.operandDType = expr.nodes[n.lhs].output_dtype.value();
+                        shapeCarrier = piece.tensors.front();
+                        fusion.prologue = std::move(piece);
+                        operands = pieceSources;
+                    } else {
+                        fusion = saved;
+                        emitFusedGroup({n.lhs});  // store the operand first
+                    }
+                }
+                if (!fusion.prologue.has_value()) {
+                    operands = {n.lhs};
+                    shapeCarrier = tensorOf[n.lhs];
+                }
+                if (n.rhs != UINT32_MAX) operands.push_back(n.rhs);
+                if (n.aux != UINT32_MAX) operands.push_back(n.aux);
+                // the consumer: when one elementwise value (of this shape, nothing else unfinished under it) is all that reads the
+                // rotation, this kernel computes and stores that value instead
+                uint32_t stored = i;
+                if (stageFusion && outputNameOfNode.find(i) == outputNameOfNode.end()) {
+                    uint32_t reader = UINT32_MAX;
+                    bool single = true;
+                    for (uint32_t j = 0; j < expr.nodes.size() && single; ++j) {
+                        if (j == i || !isTensorRole(graph->role[j]) || done[j]) continue;
+                        const ExprNode& candidate = expr.nodes[j];
+                        std::vector<uint32_t> sources, scalars;
+                        if (runsInFusedKernel(j)) {
+                            collectSources(*graph, j, sources, scalars);
+                        } else {
+                            for (uint32_t c : {candidate.lhs, candidate.rhs, candidate.aux})
+                                if (c != UINT32_MAX) sources.push_back(c);
+                            // (a value an inline operand of another stage reads also counts as read by that stage)
+                            std::vector<uint32_t> deeper;
+                            for (uint32_t c : sources)
+                                if (graph->role[c] == Role::Inline) collectSources(*graph, c, deeper, scalars);
+                            sources.insert(sources.end(), deeper.begin(), deeper.end());
+                        }
+                        if (std::find(sources.begin(), sources.end(), i) == sources.end()) continue;
+                        if (reader != UINT32_MAX || !runsInFusedKernel(j) || candidate.op == ExprOp::RAGGED_VALUEWISE_EXTENT || orScalarShape(dims[j]) != shape) {
+                            single = false;
+                        } else {
+                            reader = j;
+                        }
+                    }
+                    if (single && reader != UINT32_MAX) {
+                        RopeFusion saved = fusion;
+                        RopeFusion::Piece piece;
+                        std::vector<uint32_t> pieceSources;
+                        if (buildPiece(reader, true, piece, pieceSources)) {
+                            fusion.rotatedDType = n.output_dtype.value();
+                            fusion.epilogue = std::move(piece);
+                            operands.insert(operands.end(), pieceSources.begin(), pieceSources.end());
+                            stored = reader;
+                        } else {
+                            fusion = saved;
+                        }
+                    }
+                }
+                Tensor result = allocateFor(stored);
                 StampedExecutionStage stage;
                 stage.kind = StampedExecutionStage::Kind::FusedKernel;
                 stage.gpu_num = device_num;
-                std::vector<uint32_t> operands = {n.lhs};
-                if (n.rhs != UINT32_MAX) operands.push_back(n.rhs);
-                if (n.aux != UINT32_MAX) operands.push_back(n.aux);
                 stage.dependency_stage_indices = dependenciesOf(operands);
-                stage.kernel = stampRotaryEmbedding(tensorOf[n.lhs], n.rhs != UINT32_MAX ? std::optional<Tensor>(tensorOf[n.rhs]) : std::nullopt,
-                                                    n.aux != UINT32_MAX ? std::optional<Tensor>(tensorOf[n.aux]) : std::nullopt, rotated, n, device_num);
-                tensorOf[i] = rotated;
+                stage.kernel = stampRotaryEmbedding(shapeCarrier, n.rhs != UINT32_MAX ? std::optional<Tensor>(tensorOf[n.rhs]) : std::nullopt,
+                                                    n.aux != UINT32_MAX ? std::optional<Tensor>(tensorOf[n.aux]) : std::nullopt, result, n, device_num, fusion);
+                tensorOf[stored] = result;
+                stageOfNode[stored] = static_cast<int>(stages.size());
                 stageOfNode[i] = static_cast<int>(stages.size());
                 stages.push_back(std::move(stage));
                 done[i] = 1;
+                done[stored] = 1;
                 continue;
             }
             if (n.op == ExprOp::TAKE_ALONG_AXIS) {

@@ -93,6 +93,12 @@ std::string frequencyStatements(const ExprNode& n, uint64_t rotary, const std::s
 std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, const std::optional<Tensor>& positionIds,
                                                       const std::optional<Tensor>& effectiveLength, const Tensor& output, const ExprNode& n,
                                                       int deviceNum) {
+    return stampRotaryEmbedding(values, positionIds, effectiveLength, output, n, deviceNum, RopeFusion{});
+}
+
+std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, const std::optional<Tensor>& positionIds,
+                                                      const std::optional<Tensor>& effectiveLength, const Tensor& output, const ExprNode& n,
+                                                      int deviceNum, const RopeFusion& fusion) {
     if (!values.isInitialized() || !output.isInitialized()) throw std::runtime_error("RoPE requires initialized tensors.");
     const std::vector<uint64_t>& dims = values.getDimensions();
     const uint32_t seqAxis = n.rope_sequence_axis, dimAxis = n.rope_head_dim_axis;
@@ -141,15 +147,29 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     const uint64_t walk = outerCount * middleCount * innerCount;  // coordinates a thread visits with one set of angles
     const uint64_t total = walk * seq * headDim;
 
-    const uint32_t inBytes = dataTypeSizeInBytes(values.getDataType()), outBytes = dataTypeSizeInBytes(output.getDataType());
+    // every tensor the kernel streams: the operand (or what the prologue computes it from), what the epilogue reads, the output
+    std::vector<Tensor> streamed;
+    if (fusion.prologue.has_value()) {
+        streamed = fusion.prologue->tensors;
+    } else {
+        streamed.push_back(values);
+    }
+    if (fusion.epilogue.has_value()) streamed.insert(streamed.end(), fusion.epilogue->tensors.begin(), fusion.epilogue->tensors.end());
+    streamed.push_back(output);
+    uint32_t widest = 1;
+    for (const Tensor& t : streamed) {
+        if (!t.isInitialized() || !t.isDenseContiguous() || t.getDimensions() != dims) throw std::runtime_error("RoPE streams dense tensors of the rotated shape.");
+        widest = std::max<uint32_t>(widest, dataTypeSizeInBytes(t.getDataType()));
+    }
     const uint64_t tail = headDim - rotary;
-    int vec = dimStride == 1 ? static_cast<int>(16 / std::max(inBytes, outBytes)) : 1;
+    int vec = dimStride == 1 ? static_cast<int>(16 / widest) : 1;
     auto fits = [&](int v) {
         if (v == 1) return true;
         if (tail % v != 0) return false;
         if (n.rope_interleaved ? rotary % v != 0 : half % v != 0) return false;
-        return pointerAlignment(values.getMemPtr()) % (static_cast<uint64_t>(v) * inBytes) == 0 &&
-               pointerAlignment(output.getMemPtr()) % (static_cast<uint64_t>(v) * outBytes) == 0;
+        for (const Tensor& t : streamed)
+            if (pointerAlignment(t.getMemPtr()) % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(t.getDataType())) != 0) return false;
+        return true;
     };
     while (!fits(vec)) vec /= 2;
     const bool pairsInsideVector = n.rope_interleaved && vec > 1;
@@ -186,6 +206,113 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     const bool needsLength = n.rope_scaling_kind == RotaryScalingKind::DynamicNTK || n.rope_scaling_kind == RotaryScalingKind::LongRope;
     // a block shares the table of frequencies when that saves work: more than one thread of the block per pair
     const bool sharedFrequencies = half <= 8192 && items >= 2 * half;
+    const bool hasPrologue = fusion.prologue.has_value(), hasEpilogue = fusion.epilogue.has_value();
+
+    // ---- the three things a site (one vector of elements at one offset) does, with or without fused elementwise work ----
+    auto replaceAll = [](std::string text, const std::string& what, const std::string& with) {
+        for (size_t at = text.find(what); at != std::string::npos; at = text.find(what, at + with.size())) text.replace(at, what.size(), with);
+        return text;
+    };
+    auto indented = [](const std::string& statements, const std::string& ind) {
+        std::string out;
+        size_t at = 0;
+        while (at < statements.size()) {
+            const size_t eol = statements.find('\n', at);
+            const std::string line = statements.substr(at, eol == std::string::npos ? std::string::npos : eol - at);
+            const size_t firstText = line.find_first_not_of(' ');
+            if (firstText != std::string::npos) out += ind + line.substr(firstText) + "\n";
+            if (eol == std::string::npos) break;
+            at = eol + 1;
+        }
+        return out;
+    };
+    const char* contractOn = "#pragma clang fp contract(fast)\n";
+    // loads of one site: the operand's sources and what the epilogue reads, all at `offset`
+    auto loadSite = [&](const std::string& ind, const std::string& site, const std::string& offset) {
+        std::string out;
+        if (hasPrologue) {
+            for (size_t i = 0; i < fusion.prologue->tensors.size(); ++i) {
+                const std::string name = site + "_" + std::to_string(i);
+                out += ind + "thor::Pack<" + deviceTypeName(fusion.prologue->tensors[i].getDataType()) + ", V> " + name + ";\n";
+                out += ind + name + ".loadStream(p" + std::to_string(i) + " + " + offset + ");\n";
+            }
+        } else {
+            out += ind + "thor::Pack<" + inType + ", V> " + site + ";\n" + ind + site + ".loadStream(x + " + offset + ");\n";
+        }
+        if (hasEpilogue) {
+            for (size_t i = 0; i < fusion.epilogue->tensors.size(); ++i) {
+                const std::string name = site + "_e" + std::to_string(i);
+                out += ind + "thor::Pack<" + deviceTypeName(fusion.epilogue->tensors[i].getDataType()) + ", V> " + name + ";\n";
+                out += ind + name + ".loadStream(e" + std::to_string(i) + " + " + offset + ");\n";
+            }
+        }
+        return out;
+    };
+    // `float var` = element k of the site as the rotation reads it
+    auto operandOf = [&](const std::string& ind, const std::string& var, const std::string& site, const std::string& k) {
+        if (!hasPrologue) return ind + "const float " + var + " = thor::toFloat(" + site + ".v[" + k + "]);\n";
+        std::string text = fusion.prologue->statements;
+        for (size_t i = 0; i < fusion.prologue->tensors.size(); ++i) {
+            text = replaceAll(text, "@P" + std::to_string(i) + "@", site + "_" + std::to_string(i) + ".v[" + k + "]");
+        }
+        std::string out = ind + "float " + var + ";\n" + ind + "{\n";
+        if (fusion.prologue->contract) out += contractOn;
+        out += indented(text, ind + "    ");
+        out += ind + "    " + var + " = " + fusion.prologue->value + ";\n" + ind + "}\n";
+        return out;
+    };
+    // element k of the output site from the rotated (or, beyond the rotary part, untouched) fp32 value
+    auto resultTo = [&](const std::string& ind, const std::string& outSite, const std::string& site, const std::string& k, const std::string& rotated) {
+        if (!hasEpilogue) return ind + outSite + ".v[" + k + "] = thor::fromFloat<" + outType + ">(" + rotated + ");\n";
+        std::string text = fusion.epilogue->statements;
+        for (size_t i = 0; i < fusion.epilogue->tensors.size(); ++i) {
+            text = replaceAll(text, "@E" + std::to_string(i) + "@", site + "_e" + std::to_string(i) + ".v[" + k + "]");
+        }
+        std::string out = ind + "{\n";
+        out += ind + "    const float turned = " + rotated + ";\n";
+        out += ind + "    const " + std::string(valueCType(fusion.rotatedDType)) + " rotatedValue = " + castValueExpr("turned", DataType::FP32, fusion.rotatedDType) +
+               ";\n";
+        out += ind + "    {\n";
+        if (fusion.epilogue->contract) out += contractOn;
+        out += indented(replaceAll(text, "@R@", "rotatedValue"), ind + "        ");
+        out += ind + "        " + outSite + ".v[" + k + "] = " + fusion.epilogue->value + ";\n";
+        out += ind + "    }\n" + ind + "}\n";
+        return out;
+    };
+    // a vector of the part of the head dimension that is not rotated: through the same elementwise work, unturned
+    auto copySite = [&](const std::string& ind, const std::string& offset) {
+        std::string out = loadSite(ind, "p", offset);
+        out += ind + "thor::Pack<" + outType + ", V> q;\n";
+        out += "#pragma unroll\n" + ind + "for (int k = 0; k < V; ++k) {\n";
+        out += operandOf(ind + "    ", "a", "p", "k");
+        out += resultTo(ind + "    ", "q", "p", "k", "a");
+        out += ind + "}\n" + ind + "q.storeStream(out + " + offset + ");\n";
+        return out;
+    };
+    // pairs that lie inside one vector (interleaved layout)
+    auto turnInsideVector = [&](const std::string& ind, const std::string& offset) {
+        std::string out = loadSite(ind, "p", offset);
+        out += ind + "thor::Pack<" + outType + ", V> q;\n";
+        out += "#pragma unroll\n" + ind + "for (int k = 0; k < P; ++k) {\n";
+        out += operandOf(ind + "    ", "a", "p", "2 * k");
+        out += operandOf(ind + "    ", "b", "p", "2 * k + 1");
+        out += resultTo(ind + "    ", "q", "p", "2 * k", "a * cs[k] - b * sn[k]");
+        out += resultTo(ind + "    ", "q", "p", "2 * k + 1", "a * sn[k] + b * cs[k]");
+        out += ind + "}\n" + ind + "q.storeStream(out + " + offset + ");\n";
+        return out;
+    };
+    // the two elements of a pair in two vectors `apart` coordinates from each other
+    auto turnAcrossVectors = [&](const std::string& ind, const std::string& offsetA, const std::string& offsetB) {
+        std::string out = loadSite(ind, "pa", offsetA) + loadSite(ind, "pb", offsetB);
+        out += ind + "thor::Pack<" + outType + ", V> qa, qb;\n";
+        out += "#pragma unroll\n" + ind + "for (int k = 0; k < V; ++k) {\n";
+        out += operandOf(ind + "    ", "a", "pa", "k");
+        out += operandOf(ind + "    ", "b", "pb", "k");
+        out += resultTo(ind + "    ", "qa", "pa", "k", "a * cs[k] - b * sn[k]");
+        out += resultTo(ind + "    ", "qb", "pb", "k", "a * sn[k] + b * cs[k]");
+        out += ind + "}\n" + ind + "qa.storeStream(out + " + offsetA + ");\n" + ind + "qb.storeStream(out + " + offsetB + ");\n";
+        return out;
+    };
 
     std::ostringstream s;
     s << thor_embed::kDevicePrelude;
@@ -193,9 +320,22 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "__device__ const float thor_rope_short_factors[" << half << "] = " << floatArray(n.rope_long_rope_short_factors) << ";\n";
         s << "__device__ const float thor_rope_long_factors[" << half << "] = " << floatArray(n.rope_long_rope_long_factors) << ";\n";
     }
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_rope(const " << inType << "* __restrict__ x";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_rope(";
+    if (hasPrologue) {
+        for (size_t i = 0; i < fusion.prologue->tensors.size(); ++i) {
+            s << (i ? ", " : "") << "const " << deviceTypeName(fusion.prologue->tensors[i].getDataType()) << "* __restrict__ p" << i;
+        }
+    } else {
+        s << "const " << inType << "* __restrict__ x";
+    }
     if (positionIds.has_value()) s << ", const " << deviceTypeName(positionIds->getDataType()) << "* __restrict__ ids";
     if (effectiveLength.has_value()) s << ", const " << deviceTypeName(effectiveLength->getDataType()) << "* __restrict__ length";
+    if (hasEpilogue) {
+        for (size_t i = 0; i < fusion.epilogue->tensors.size(); ++i) {
+            s << ", const " << deviceTypeName(fusion.epilogue->tensors[i].getDataType()) << "* __restrict__ e" << i;
+        }
+    }
+    for (uint32_t slot : fusion.scalarSlots) s << ", float s" << slot;
     s << ", " << outType << "* __restrict__ out) {\n";
     s << "    constexpr int V = " << vec << ", P = " << pairsPerThread << ";\n";
     if (needsLength) {
@@ -238,32 +378,18 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         if (tail != 0) {
             s << "        if (slot >= " << pairSlots << "u) {\n";
             s << "            const thor::u64 e = rowBase + " << rotary << "ull + (slot - " << pairSlots << "u) * V;\n";
-            s << "            thor::Pack<" << inType << ", V> p;\n            p.loadStream(x + e);\n";
-            s << "            thor::Pack<" << outType << ", V> q;\n";
-            s << "#pragma unroll\n            for (int k = 0; k < V; ++k) q.v[k] = thor::fromFloat<" << outType << ">(thor::toFloat(p.v[k]));\n";
-            s << "            q.storeStream(out + e);\n            continue;\n        }\n";
+            s << copySite("            ", "e");
+            s << "            continue;\n        }\n";
         }
         s << "        const thor::u32 firstPair = slot * P;\n";
         s << "        const float* sn = sines + (row / " << middleCount << "u) * " << half << "u + firstPair;\n";
         s << "        const float* cs = cosines + (row / " << middleCount << "u) * " << half << "u + firstPair;\n";
         if (pairsInsideVector) {
             s << "        const thor::u64 e = rowBase + firstPair * 2;\n";
-            s << "        thor::Pack<" << inType << ", V> p;\n        p.loadStream(x + e);\n";
-            s << "        thor::Pack<" << outType << ", V> q;\n";
-            s << "#pragma unroll\n        for (int k = 0; k < P; ++k) {\n";
-            s << "            const float a = thor::toFloat(p.v[2 * k]), b = thor::toFloat(p.v[2 * k + 1]);\n";
-            s << "            q.v[2 * k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
-            s << "            q.v[2 * k + 1] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
-            s << "        }\n        q.storeStream(out + e);\n";
+            s << turnInsideVector("        ", "e");
         } else {
             s << "        const thor::u64 ea = rowBase + " << (n.rope_interleaved ? "firstPair * 2" : "firstPair") << ", eb = ea + " << apart << "ull;\n";
-            s << "        thor::Pack<" << inType << ", V> pa, pb;\n        pa.loadStream(x + ea);\n        pb.loadStream(x + eb);\n";
-            s << "        thor::Pack<" << outType << ", V> qa, qb;\n";
-            s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
-            s << "            const float a = thor::toFloat(pa.v[k]), b = thor::toFloat(pb.v[k]);\n";
-            s << "            qa.v[k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
-            s << "            qb.v[k] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
-            s << "        }\n        qa.storeStream(out + ea);\n        qb.storeStream(out + eb);\n";
+            s << turnAcrossVectors("        ", "ea", "eb");
         }
         s << "    }\n}\n";
     } else {
@@ -293,10 +419,9 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "        // beyond the rotary part: a copy\n";
         s << "        const thor::u64 d = " << rotary << "ull + (slot - " << pairSlots << "ull) * V;\n";
         s << "        for (thor::u64 w = walkFirst; w < walkLast; ++w) {\n";
-        s << "            thor::Pack<" << inType << ", V> p;\n            p.loadStream(x + at(w, d));\n";
-        s << "            thor::Pack<" << outType << ", V> q;\n";
-        s << "#pragma unroll\n            for (int k = 0; k < V; ++k) q.v[k] = thor::fromFloat<" << outType << ">(thor::toFloat(p.v[k]));\n";
-        s << "            q.storeStream(out + at(w, d));\n        }\n        return;\n    }\n";
+        s << "            const thor::u64 e = at(w, d);\n";
+        s << copySite("            ", "e");
+        s << "        }\n        return;\n    }\n";
     }
     s << "    const thor::u64 firstPair = slot * P;\n";
     if (positionIds.has_value()) {
@@ -325,23 +450,11 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     s << "    for (thor::u64 w = walkFirst; w < walkLast; ++w) {\n";
     if (pairsInsideVector) {
         s << "        const thor::u64 e = at(w, firstPair * 2);\n";
-        s << "        thor::Pack<" << inType << ", V> p;\n        p.loadStream(x + e);\n";
-        s << "        thor::Pack<" << outType << ", V> q;\n";
-        s << "#pragma unroll\n        for (int k = 0; k < P; ++k) {\n";
-        s << "            const float a = thor::toFloat(p.v[2 * k]), b = thor::toFloat(p.v[2 * k + 1]);\n";
-        s << "            q.v[2 * k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
-        s << "            q.v[2 * k + 1] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
-        s << "        }\n        q.storeStream(out + e);\n";
+        s << turnInsideVector("        ", "e");
     } else {
         const std::string firstCoordinate = n.rope_interleaved ? "firstPair * 2" : "firstPair";
         s << "        const thor::u64 ea = at(w, " << firstCoordinate << "), eb = at(w, " << firstCoordinate << " + " << apart << "ull);\n";
-        s << "        thor::Pack<" << inType << ", V> pa, pb;\n        pa.loadStream(x + ea);\n        pb.loadStream(x + eb);\n";
-        s << "        thor::Pack<" << outType << ", V> qa, qb;\n";
-        s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
-        s << "            const float a = thor::toFloat(pa.v[k]), b = thor::toFloat(pb.v[k]);\n";
-        s << "            qa.v[k] = thor::fromFloat<" << outType << ">(a * cs[k] - b * sn[k]);\n";
-        s << "            qb.v[k] = thor::fromFloat<" << outType << ">(a * sn[k] + b * cs[k]);\n";
-        s << "        }\n        qa.storeStream(out + ea);\n        qb.storeStream(out + eb);\n";
+        s << turnAcrossVectors("        ", "ea", "eb");
     }
     s << "    }\n}\n";
     }
@@ -356,14 +469,27 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         description << ",walk=" << walk << "/" << chunks;
     }
     description << ",vec=" << vec << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
-    std::vector<Tensor> inputs = {values};
+    std::vector<Tensor> inputs;
+    if (hasPrologue) {
+        inputs = fusion.prologue->tensors;
+    } else {
+        inputs.push_back(values);
+    }
     if (positionIds.has_value()) inputs.push_back(*positionIds);
     if (effectiveLength.has_value()) inputs.push_back(*effectiveLength);
+    if (hasEpilogue) inputs.insert(inputs.end(), fusion.epilogue->tensors.begin(), fusion.epilogue->tensors.end());
     std::vector<size_t> inputArgs;
     for (size_t i = 0; i < inputs.size(); ++i) inputArgs.push_back(i);
-    return std::make_shared<StampedEquation>(kernel, inputs, std::vector<Tensor>{output}, std::vector<StampedEquation::ScalarArgument>{}, inputArgs,
-                                             std::vector<size_t>{inputs.size()}, inputs.size() + 1, /*passNumel=*/false, total, total > UINT32_MAX,
-                                             static_cast<uint32_t>(blocks), threads, /*flops=*/0, description.str());
+    std::vector<StampedEquation::ScalarArgument> scalarArgs;
+    size_t next = inputs.size();
+    for (const std::string& name : fusion.scalarNames) scalarArgs.push_back({name, next++});
+    std::string text = description.str();
+    if (hasPrologue || hasEpilogue) {
+        text = std::string("fused ") + (hasPrologue ? "prologue+" : "") + text.substr(0, text.find(" [")) + (hasEpilogue ? "+epilogue" : "") + text.substr(text.find(" ["));
+    }
+    return std::make_shared<StampedEquation>(kernel, inputs, std::vector<Tensor>{output}, scalarArgs, inputArgs, std::vector<size_t>{next}, next + 1,
+                                             /*passNumel=*/false, total, total > UINT32_MAX, static_cast<uint32_t>(blocks), threads,
+                                             /*flops=*/fusion.extraFlopsPerElement * total, text);
 }
 
 }  // namespace ThorImplementation
