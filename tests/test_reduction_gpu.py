@@ -195,7 +195,14 @@ PERMUTED = [
     ((40, 33, 64), (2, 0, 1), [1, 2]),   # ... and both other axes
     ((12, 16, 48), (0, 2, 1), [2]),      # batch kept, inner two swapped
     ((7, 130), (1, 0), [1]),             # lane axis not a multiple of the vector width
+    # outputs whose fastest axis is not the lane axis: written through the LDS transpose
+    ((37, 5, 132), (2, 1, 0), [1]),      # ragged tiles in both directions
+    ((64, 8, 256), (2, 1, 0), [1]),
+    ((20, 3, 17, 64), (3, 1, 0, 2), [1]),  # two kept axes after the lane axis
+    ((300, 2, 16), (2, 1, 0), [1]),      # one vector-wide lane axis
 ]
+TRANSPOSED_STORE = {((40, 33, 64), (2, 0, 1), (1,)), ((37, 5, 132), (2, 1, 0), (1,)), ((64, 8, 256), (2, 1, 0), (1,)), ((20, 3, 17, 64), (3, 1, 0, 2), (1,)),
+                    ((300, 2, 16), (2, 1, 0), (1,))}
 
 
 @pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16], ids=lambda d: d.name)
@@ -216,6 +223,7 @@ def test_permuted_views_reduce_with_lanes_on_the_contiguous_kept_axis(stream, sh
         want = oracle.reduce(OPS[name][1], logical, oracle.FP32, axes)
         np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream).reshape(want.shape), want, err_msg=f"{name} {stamped.get_kernel_variant()}")
     assert "view_columns" in stamped.get_kernel_variant()
+    assert ("transposed_store" in stamped.get_kernel_variant()) == ((shape, perm, tuple(axes)) in TRANSPOSED_STORE), stamped.get_kernel_variant()
     for op, oracle_op in ((ph.CubArgReductionOp.ArgMax, oracle.ARGMAX), (ph.CubArgReductionOp.ArgMin, oracle.ARGMIN)):
         arg = ph.CubArgReduction(op, axes, value_output_dtype=DataType.fp32).stamp(view, stream)
         arg.run()

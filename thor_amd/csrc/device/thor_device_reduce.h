@@ -360,6 +360,63 @@ __device__ __forceinline__ void reduceStrided(const typename Cfg::Sources& src, 
     }
 }
 
+// reduceColumns for outputs whose fastest axis is not the one the lanes lie on (a transposed matrix reduced along its rows,
+// the [inner, outer] outputs of the reference's tiled kernels: Utilities/TensorOperations/Cub/CubReductionOperation.cuh:
+// 2165-2534 there): lanes along the input's contiguous kept axis would scatter single elements over the output.  Here a
+// block owns kLanesX * kVec lane positions times kTransposeRows consecutive values of the next kept coordinate q (the
+// output's fastest axis); every row group reduces whole columns of its own q values (nothing is folded between threads),
+// the results meet in LDS and leave along q: the writes of a block are runs of kTransposeRows adjacent elements.
+// Cfg additionally: kTransposeRows, kLaneVectors (vectors along the lane axis), kQ (= kColumns / kLaneVectors); column
+// c = q * kLaneVectors + vector.  Only without a split of R.
+template <typename Cfg>
+__device__ __forceinline__ void reduceColumnsTransposed(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, float scale) {
+    typedef typename Cfg::IndexT IndexT;
+    typedef typename Cfg::Acc Acc;
+    constexpr int kGroups = Cfg::kThreads / Cfg::kLanesX;
+    constexpr int kBatch = Cfg::kBatch;
+    constexpr int kRows = Cfg::kTransposeRows, kWidth = Cfg::kLanesX * Cfg::kVec;
+    constexpr u64 kTilesPerRow = (Cfg::kLaneVectors + Cfg::kLanesX - 1) / Cfg::kLanesX;
+    __shared__ Acc tile[kRows][kWidth + 1];
+    const int lx = threadIdx.x % Cfg::kLanesX, group = threadIdx.x / Cfg::kLanesX;
+    const u64 firstVector = (blockIdx.x % kTilesPerRow) * Cfg::kLanesX, firstQ = (blockIdx.x / kTilesPerRow) * kRows;
+    const bool vectorLive = firstVector + lx < Cfg::kLaneVectors;
+    for (int j = group; j < kRows; j += kGroups) {
+        const u64 q = firstQ + j;
+        if (!vectorLive || q >= Cfg::kQ) continue;
+        const u64 column = q * Cfg::kLaneVectors + firstVector + lx;
+        const u64 base = Cfg::columnBase(column);
+        Acc acc[Cfg::kVec];
+        typename Cfg::Kept kept[Cfg::kVec];
+#pragma unroll
+        for (int k = 0; k < Cfg::kVec; ++k) {
+            acc[k].reset();
+            Cfg::loadKept(src, Cfg::partialSlot(column, k), kept[k]);
+        }
+        for (u64 r0 = 0; r0 < Cfg::kR; r0 += kBatch) {
+            typename Cfg::Loaded x[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u)
+                if (r0 + u < Cfg::kR) Cfg::load(src, base + Cfg::rowOffset(r0 + u), x[u]);
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                if (r0 + u < Cfg::kR) {
+#pragma unroll
+                    for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, (IndexT)(r0 + u));
+                    Cfg::template elementwise<1>(src, out, base + Cfg::rowOffset(r0 + u), x[u], kept);
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < Cfg::kVec; ++k) tile[j][lx * Cfg::kVec + k] = acc[k];
+    }
+    __syncthreads();
+    for (int slot = threadIdx.x; slot < kRows * kWidth; slot += Cfg::kThreads) {
+        const int j = slot % kRows, i = slot / kRows;
+        const u64 q = firstQ + j, vector = firstVector + i / Cfg::kVec;
+        if (q < Cfg::kQ && vector < Cfg::kLaneVectors) Cfg::store(tile[j][i], Cfg::outputIndex(q * Cfg::kLaneVectors + vector, i % Cfg::kVec), out, scale);
+    }
+}
+
 // ---- offset-segmented rows: values [N, D] and offsets [B + 1] -> [B, D] ---------------------------------------------------------
 // Segment b is the row range [offsets[b], offsets[b + 1]); the offsets are read when the kernels run, so a stamped
 // reduction follows whatever partition is in the tensor at that moment (replaces cub::DeviceSegmentedReduce and the

@@ -43,6 +43,17 @@ size_t partialBytes(uint64_t slots, bool isArg, bool indexIs64) {
     return bytes;
 }
 
+// Outputs that lanes would scatter (the lane axis is not the output's fastest one) leave through an LDS transpose when the
+// writes are a visible share of the traffic and one block can own whole columns: no split of R, R at most 512, at least 16
+// coordinates along the output's fastest axis.  Measured on fp32 [512, 8, 16384] seen as [16384, 8, 512], sum over the middle
+// axis: 84 us with scattered stores.
+int transposeRowsFor(uint64_t split, uint64_t reductionSize, uint64_t fastestOutputExtent, uint64_t laneOutputStride, uint64_t rowBytes) {
+    if (std::getenv("THOR_REDUCE_NO_TRANSPOSE") != nullptr) return 0;
+    if (split != 1 || laneOutputStride == 1 || reductionSize > 512 || fastestOutputExtent < 16) return 0;
+    if (16 * rowBytes > 65536) return 0;  // the block's results wait in LDS: 16 rows of lanes x vector + 1 accumulators
+    return 16;
+}
+
 // Merges adjacent axes that address memory as one longer axis (outer stride == inner dim * inner stride) and drops
 // singleton axes.  Order is preserved, so row-major positions inside the collapsed domain are unchanged.
 void collapseAxes(std::vector<uint64_t>& dims, std::vector<uint64_t>& strides) {
@@ -159,6 +170,7 @@ std::string ReductionShape::describe() const {
             break;
         case Kernel::Columns:
             out << (laneAxis < 0 ? "columns(lanes_x=" : "view_columns(lanes_x=") << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
+            if (transposeRows > 0) out << ",transposed_store=" << transposeRows;
             break;
         case Kernel::Segments:
             out << "segments(lanes_x=" << threadsPerRow << ",rows_in_flight=" << unroll << ",chunk_rows=" << chunkRows << ",min_team=" << minTeam;
@@ -216,6 +228,7 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
     const uint64_t accumulators = request.values.empty() ? 1 : request.values.size();
     ReductionShape shape;
     shape.indexIs64 = g.input_elements >= (1ull << 31) || g.reduction_size >= (1ull << 31);
+    const uint64_t accumulatorBytes = request.isArg ? (shape.indexIs64 ? 16 : 8) : 4 * accumulators;
 
     auto finishSplit = [&](uint64_t outputs) {
         if (shape.split > 1) shape.workspaceBytes = accumulators * partialBytes(outputs * shape.split, request.isArg, shape.indexIs64);
@@ -320,6 +333,14 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         const uint64_t columnsNow = g.outer_size * (g.inner_size / shape.vec);
         shape.gridX = static_cast<uint32_t>(ceilDiv(columnsNow, shape.threadsPerRow));
         shape.gridY = static_cast<uint32_t>(shape.split);
+        if (g.tiled_output_outer_stride == 1) {
+            // [inner, outer] output: consecutive outer coordinates are adjacent in the output
+            shape.transposeRows = transposeRowsFor(shape.split, g.reduction_size, g.outer_size, g.tiled_output_inner_stride,
+                                                    (static_cast<uint64_t>(shape.threadsPerRow) * shape.vec + 1) * accumulatorBytes);
+            if (shape.transposeRows > 0) {
+                shape.gridX = static_cast<uint32_t>(ceilDiv(g.inner_size / shape.vec, shape.threadsPerRow) * ceilDiv(g.outer_size, shape.transposeRows));
+            }
+        }
         finishSplit(g.output_elements);
         return shape;
     }
@@ -378,6 +399,17 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         }
         shape.gridX = static_cast<uint32_t>(ceilDiv(columns, shape.threadsPerRow));
         shape.gridY = static_cast<uint32_t>(shape.split);
+        if (static_cast<size_t>(laneAxis) + 1 != shape.keptDims.size()) {
+            // the columns after the lane axis run along the last kept axis, the output's fastest one
+            uint64_t laneOutputStride = 1;
+            for (size_t a = static_cast<size_t>(laneAxis) + 1; a < shape.keptDims.size(); ++a) laneOutputStride *= shape.keptDims[a];
+            shape.transposeRows = transposeRowsFor(shape.split, g.reduction_size, shape.keptDims.back(), laneOutputStride,
+                                                    (static_cast<uint64_t>(shape.threadsPerRow) * vec + 1) * accumulatorBytes);
+            if (shape.transposeRows > 0) {
+                const uint64_t laneVectors = shape.keptDims[laneAxis] / vec;
+                shape.gridX = static_cast<uint32_t>(ceilDiv(laneVectors, shape.threadsPerRow) * ceilDiv(columns / laneVectors, shape.transposeRows));
+            }
+        }
         finishSplit(g.output_elements);
         return shape;
     }
@@ -595,6 +627,13 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
                 s << offsetFunction("rowOffset", shape.reducedDims, shape.reducedStrides);
             }
             body = "thor::reduceColumns<gen::Cfg>(src, out, partials, scale);";
+            if (shape.transposeRows > 0) {
+                const uint64_t laneVectors = (shape.laneAxis < 0 ? g.inner_size : shape.keptDims[static_cast<size_t>(shape.laneAxis)]) / shape.vec;
+                s << "    static constexpr int kTransposeRows = " << shape.transposeRows << ";\n";
+                s << "    static constexpr u64 kLaneVectors = " << laneVectors << "ull;\n";
+                s << "    static constexpr u64 kQ = " << (g.output_elements / shape.vec / laneVectors) << "ull;\n";
+                body = "thor::reduceColumnsTransposed<gen::Cfg>(src, out, scale);";
+            }
             break;
         case ReductionShape::Kernel::Segments:
             s << "    typedef " << (request.offsetsAre64 ? "u64" : "u32") << " OffsetT;\n";

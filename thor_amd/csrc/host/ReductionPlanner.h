@@ -82,6 +82,9 @@ struct ReductionShape {
     // Columns kernel over a view: index (into keptDims) of the kept axis that is contiguous in memory, or -1 for the
     // dense [outer, R, inner] layout
     int laneAxis = -1;
+    // Columns whose lanes do not lie on the output's fastest axis: a block reduces this many consecutive coordinates of that axis
+    // and writes them out together through LDS (0: every lane stores its own outputs)
+    int transposeRows = 0;
     // Segments kernel: rows per block, number of such chunks, smallest team of threads that shares a segment, columns per
     // block of the finishing launch
     uint64_t chunkRows = 0, chunks = 1;
