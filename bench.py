@@ -358,6 +358,46 @@ def bench_other_configs():
         plans = [rope.stamp({"q": t}, stream) for t in (q, clone(q))]
         timed(label, [p_.run for p_ in plans], 2 * size_of(dtype) * count, count, plans[0].stage_descriptions()[0])
         del plans, q
+
+    # ---- select-flagged and top-k (the selection primitives next to the scans): bytes counted are the keys / values and flags read
+    # once and the selected elements written once
+    n = 1 << 26
+    keys = gpu_from(np.resize(rng.standard_normal(1 << 22).astype(np.float32), n), DataType.fp32)
+    flag_block = (rng.random(1 << 22) < 0.5).astype(np.uint8)
+    flags = gpu_from(np.resize(flag_block, n), DataType.uint8)
+    kept = int(np.resize(flag_block, n).sum())
+    selected = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [n]))
+    count = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.uint32, [1]))
+    plan = ph.SelectionPlan.select_flagged(keys, flags, selected, count)
+    temp = plan.allocate_temp_storage()
+    timed("select_flagged_fp32_2^26_half_kept", lambda: plan.run(temp, keys, flags, selected, count, stream=stream), 5 * n + 4 * kept, n, plan.variant())
+    del flags, selected, plan, temp
+    for k in (64, 65536):
+        best = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [k]))
+        plan = ph.SelectionPlan.top_k(keys, best, k)
+        temp = plan.allocate_temp_storage()
+        timed(f"topk_fp32_2^26_k{k}", lambda: plan.run(temp, keys, best, stream=stream), 4 * n + 4 * k, n, plan.variant())
+        del plan, temp, best
+    del keys
+    rows_k = gpu_from(np.resize(rng.standard_normal(1 << 22).astype(np.float32), (16384, 4096)), DataType.bf16)
+    best = ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.bf16, [16384, 64]))
+    plan = ph.SelectionPlan.top_k(rows_k, best, 64, segment_size=4096, num_segments=16384)
+    temp = plan.allocate_temp_storage()
+    timed("topk_rows_bf16_16384x4096_k64", lambda: plan.run(temp, rows_k, best, stream=stream), 2 * 16384 * 4096 + 2 * 16384 * 64, 16384 * 4096,
+          plan.variant())
+    del rows_k, best, plan, temp
+
+    # ---- a reduction whose output's fastest axis is not the input's: fp32 storage [512, 8, 16384] seen as [16384, 8, 512], summed over
+    # the middle axis into a dense [16384, 512] (written through an LDS transpose)
+    storage = [ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp32, [512, 8, 16384])) for _ in range(3)]
+    for t in storage:
+        t.memset_async(0, stream)
+    stream.synchronize()
+    views = [t.alias_view([16384, 8, 512], [1, 16384, 8 * 16384]) for t in storage]
+    permuted = [ph.CubReduction(ph.CubReductionOp.Sum, [1], DataType.fp32).stamp(v, stream) for v in views]
+    timed("permuted_output_sum_fp32_16384x8x512_view", [p_.run for p_ in permuted], 4 * 512 * 8 * 16384 + 4 * 512 * 16384, 512 * 8 * 16384,
+          permuted[0].get_kernel_variant())
+    del storage, views, permuted
     return results
 
 

@@ -114,6 +114,7 @@ struct CubDeviceTopKKeysPlan {
     uint64_t k = 0;
     CubTopKOrder order = CubTopKOrder::Largest;
     size_t temp_storage_bytes = 0;
+    uint64_t key_alignment_bytes = 1;  // what the kernels assume of keys_in (not in the reference's struct)
     std::shared_ptr<const CubSelectionKernels> kernels;
 };
 struct CubDeviceTopKPairsPlan {
@@ -124,6 +125,7 @@ struct CubDeviceTopKPairsPlan {
     uint64_t k = 0;
     CubTopKOrder order = CubTopKOrder::Largest;
     size_t temp_storage_bytes = 0;
+    uint64_t key_alignment_bytes = 1;
     std::shared_ptr<const CubSelectionKernels> kernels;
 };
 struct CubDeviceSegmentedTopKKeysPlan {
@@ -153,6 +155,7 @@ struct CubDeviceSelectFlaggedPlan {
     DataType flag_dtype = DataType::BOOLEAN;
     uint64_t num_items = 0;
     size_t temp_storage_bytes = 0;
+    uint64_t vector_elements = 1;  // 4: the kernels read input, flags and output in groups of four elements (not in the reference's struct)
     std::shared_ptr<const CubSelectionKernels> kernels;
 };
 

@@ -27,6 +27,7 @@ typedef struct thor_stream* thor_stream_t;
 typedef struct thor_stamped_reduction* thor_stamped_reduction_t;
 typedef struct thor_stamped_arg_reduction* thor_stamped_arg_reduction_t;
 typedef struct thor_stamped_segmented_reduction* thor_stamped_segmented_reduction_t;
+typedef struct thor_selection_plan* thor_selection_plan_t;
 typedef struct thor_expr* thor_expr_t;
 typedef struct thor_outputs* thor_outputs_t;
 typedef struct thor_fused_equation* thor_fused_equation_t;
@@ -155,6 +156,21 @@ int thor_select_flagged(thor_tensor_t input, thor_tensor_t flags, thor_tensor_t 
  * k < segment_size keys of every row written row after row. */
 int thor_topk(thor_tensor_t keys_in, thor_tensor_t keys_out, thor_tensor_t values_in, thor_tensor_t values_out, uint64_t num_segments,
               uint64_t segment_size, uint64_t k, int largest, int segmented, thor_stream_t stream, char* variant, size_t variant_capacity);
+
+/* The plan / temporary-storage / run protocol of the same primitives (prepareCubDevice..., ...TempBytes and the run functions that take
+ * a plan, CubDevicePrimitives.h:357-516 there): prepare once, keep a UINT8 temporary-storage tensor of at least
+ * thor_selection_plan_temp_bytes bytes (several plans may share the largest), run any number of times with nothing allocated.
+ * thor_selection_plan_run takes the tensors in the order of the prepare call that made the plan: (input, flags, output,
+ * num_selected_out) or (keys_in, keys_out, values_in, values_out; the values NULL for key-only plans). */
+thor_selection_plan_t thor_select_flagged_prepare(thor_tensor_t input, thor_tensor_t flags, thor_tensor_t output, thor_tensor_t num_selected_out,
+                                                  uint64_t num_items);
+thor_selection_plan_t thor_topk_prepare(thor_tensor_t keys_in, thor_tensor_t keys_out, thor_tensor_t values_in, thor_tensor_t values_out,
+                                        uint64_t num_segments, uint64_t segment_size, uint64_t k, int largest, int segmented);
+size_t thor_selection_plan_temp_bytes(thor_selection_plan_t plan);
+int thor_selection_plan_run(thor_selection_plan_t plan, thor_tensor_t temp_storage, thor_tensor_t a, thor_tensor_t b, thor_tensor_t c, thor_tensor_t d,
+                            thor_stream_t stream);
+int thor_selection_plan_variant(thor_selection_plan_t plan, char* buffer, size_t capacity);
+void thor_selection_plan_destroy(thor_selection_plan_t plan);
 
 /* thor_scan for callers that cannot allocate (work recorded under stream capture, serving loops, harnesses that forbid
  * hipMalloc).  It has no counterpart in the reference.  Same arguments, kernels and results as thor_scan, but the temporary

@@ -295,3 +295,32 @@ def test_top_k_rejects_what_the_reference_rejects(stream):
         ph.top_k(keys, gpu_tensor([3], DataType.uint32), 1, stream, segment_size=0, num_segments=3)
     with pytest.raises(ValueError, match="Unsupported CUB segmented top-k key dtype"):
         ph.top_k(gpu_tensor([4], DataType.fp64), gpu_tensor([2], DataType.fp64), 1, stream, segment_size=2, num_segments=2)
+
+
+def test_prepared_plans_share_one_temporary_storage_and_run_repeatedly(stream):
+    """PreparedPlansCanShareOnePreallocatedWorkspace / PreparedPlanRejectsUndersizedWorkspace of the reference's tests
+    (CubDevicePrimitivesTest.cpp:1787-1930), for the plans built here."""
+    rng = np.random.default_rng(90)
+    n = 300_000
+    keys = rng.standard_normal(n).astype(np.float32)
+    flags = (rng.random(n) < 0.25).astype(np.uint8)
+    x = copy_numpy_to_gpu(keys, stream, DataType.fp32)
+    f = copy_numpy_to_gpu(flags, stream, DataType.uint8)
+    picked, count = gpu_tensor([n], DataType.fp32), gpu_tensor([1], DataType.uint32)
+    best, best_at = gpu_tensor([1000], DataType.fp32), gpu_tensor([1000], DataType.uint32)
+    positions = copy_numpy_to_gpu(np.arange(n, dtype=np.uint32), stream, DataType.uint32)
+    select = ph.SelectionPlan.select_flagged(x, f, picked, count)
+    top = ph.SelectionPlan.top_k(x, best, 1000, largest=False, values_in=positions, values_out=best_at)
+    assert "select-flagged" in select.variant() and "smallest pairs" in top.variant()
+    temp = gpu_tensor([max(select.temp_storage_bytes, top.temp_storage_bytes)], DataType.uint8)
+    for _ in range(3):
+        select.run(temp, x, f, picked, count, stream=stream)
+        top.run(temp, x, best, positions, best_at, stream=stream)
+        expected, expected_count = oracle.select_flagged(keys, flags)
+        assert int(copy_gpu_to_numpy(count, stream)[0]) == expected_count
+        np.testing.assert_array_equal(copy_gpu_to_numpy(picked, stream)[:expected_count], expected)
+        check_top_k(keys, DataType.fp32, 1000, False, copy_gpu_to_numpy(best, stream).reshape(1, -1), copy_gpu_to_numpy(best_at, stream).reshape(1, -1))
+    with pytest.raises(ValueError, match="temp_storage has fewer bytes"):
+        select.run(gpu_tensor([16], DataType.uint8), x, f, picked, count, stream=stream)
+    with pytest.raises(ValueError, match="plan is not compatible"):
+        top.run(temp, copy_numpy_to_gpu(keys.astype(np.float16), stream, DataType.fp16), gpu_tensor([1000], DataType.fp16), positions, best_at, stream=stream)

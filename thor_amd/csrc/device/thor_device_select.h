@@ -2,15 +2,15 @@
 // generated traits structs (placed after thor_device_prelude.h).  Replaces cub::DeviceSelect::Flagged and cub::DeviceTopK /
 // the batched fixed-size top-k the reference calls (Utilities/TensorOperations/Cub/CubSelect.cu:26-50, CubTopK.cu:27-330).
 //
-// Select-flagged keeps the input's order.  A block owns a chunk of consecutive positions, 16 per thread: one launch counts the
-// raised flags of every chunk, one block turns the counts into output offsets (and writes the total), and the last launch
-// reads the flags again, ranks them inside the block with wavefront shuffles and copies the flagged elements to their places.
-// No block waits for another one.
+// Select-flagged keeps the input's order.  A block owns a chunk of consecutive positions: one launch counts the raised flags
+// of every chunk, one block turns the counts into output offsets (and writes the total), and the last launch reads the flags
+// and the elements with lane-interleaved vector loads, ranks the flagged ones in position order, gathers them in LDS and
+// writes the chunk's run of the output with adjacent lanes on adjacent elements.  No block waits for another one.
 //
 // Top-k is a radix selection on an order-preserving unsigned image of the key (sign handling for floats and signed integers;
 // for "smallest" the image is complemented, so the code always looks for the largest images).  From the most significant
-// 8-bit digit down: a histogram of the digit over the keys that still match the digits fixed so far, then the bucket that
-// holds the k-th largest image is fixed.  After the last digit the image T of the k-th key and the number of keys equal to T
+// digit down (11, 11 and 10 bits of a 32-bit key; 8-bit digits of narrower ones): a histogram of the digit over the keys
+// that still match the digits fixed so far, then the bucket that holds the k-th largest image is fixed.  After the last digit the image T of the k-th key and the number of keys equal to T
 // that belong to the answer are known; one more pass writes every key above T and that many keys equal to T.  The answer is
 // the k best keys (with their values, for pairs) in no particular order, like the reference's (its library calls ask for
 // unsorted, not run-to-run deterministic output); which of several equal keys at the threshold are taken is not fixed either.
@@ -45,16 +45,26 @@ __device__ __forceinline__ u32 blockExclusiveSum(u32 x, u32* lds, u32& total) {
 }
 
 // ---- select-flagged ----------------------------------------------------------------------------------------------------------
-// Cfg: Word (u8 / u16 / u32: elements are copied as raw words), kTotal, kThreads (256), kItems (16), kChunks.
+// Cfg: Word (u8 / u16 / u32: elements are copied as raw words), kTotal, kThreads (256), kVec (4 when the tensors are aligned to
+// four elements, else 1), kRounds (4), kChunks.  A block owns kThreads * kVec * kRounds consecutive positions, read in rounds of
+// lane-interleaved vectors: vector v = round * kThreads + thread holds positions [v * kVec, v * kVec + kVec) of the chunk.
+template <typename Cfg>
+struct SelectChunk {
+    static constexpr u64 kElems = (u64)Cfg::kThreads * Cfg::kVec * Cfg::kRounds;
+};
+
+// bit k set: the flag of position `first + k` is raised (k < kVec; positions at or past kTotal count as not raised)
 template <typename Cfg>
 __device__ __forceinline__ u32 selectFlagBits(const u8* flags, u64 first) {
-    // bit k set: the flag of position first + k is raised
     u32 bits = 0;
-    if (first + Cfg::kItems <= Cfg::kTotal) {
-#pragma unroll
-        for (int k = 0; k < Cfg::kItems; ++k) bits |= (flags[first + k] != 0 ? 1u : 0u) << k;
+    if (Cfg::kVec == 4 && first + 4 <= Cfg::kTotal) {
+        const u32 w = *reinterpret_cast<const u32*>(flags + first);
+        // the top bit of every byte that is not zero
+        const u32 raised = (((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) & 0x80808080u;
+        bits = ((raised >> 7) & 1u) | ((raised >> 14) & 2u) | ((raised >> 21) & 4u) | ((raised >> 28) & 8u);
     } else {
-        for (int k = 0; k < Cfg::kItems; ++k)
+#pragma unroll
+        for (int k = 0; k < Cfg::kVec; ++k)
             if (first + k < Cfg::kTotal) bits |= (flags[first + k] != 0 ? 1u : 0u) << k;
     }
     return bits;
@@ -63,40 +73,98 @@ __device__ __forceinline__ u32 selectFlagBits(const u8* flags, u64 first) {
 template <typename Cfg>
 __device__ __forceinline__ void selectCount(const u8* flags, u32* counts) {
     __shared__ u32 lds[Cfg::kThreads / kWave];
-    const u64 first = ((u64)blockIdx.x * Cfg::kThreads + threadIdx.x) * Cfg::kItems;
-    const u32 mine = first < Cfg::kTotal ? (u32)__builtin_popcount(selectFlagBits<Cfg>(flags, first)) : 0u;
+    const u64 chunkBase = (u64)blockIdx.x * SelectChunk<Cfg>::kElems;
+    u32 mine = 0;
+#pragma unroll
+    for (int round = 0; round < Cfg::kRounds; ++round) {
+        const u64 first = chunkBase + ((u64)round * Cfg::kThreads + threadIdx.x) * Cfg::kVec;
+        if (first < Cfg::kTotal) mine += (u32)__builtin_popcount(selectFlagBits<Cfg>(flags, first));
+    }
     u32 total;
     (void)blockExclusiveSum<Cfg::kThreads>(mine, lds, total);
     if (threadIdx.x == 0) counts[blockIdx.x] = total;
 }
 
-// One block of 1024 threads: counts[kChunks] -> bases[kChunks] (exclusive), the grand total -> *numSelected.
+// One block of 1024 threads: counts[kChunks] -> bases[kChunks] (exclusive), the grand total -> *numSelected.  A thread owns a
+// run of consecutive chunks, so one block-wide scan serves any number of them.
 template <typename Cfg>
 __device__ __forceinline__ void selectOffsets(const u32* counts, u32* bases, u32* numSelected) {
     __shared__ u32 lds[1024 / kWave];
-    u32 carry = 0;
-    for (u64 c0 = 0; c0 < Cfg::kChunks; c0 += 1024) {
-        const u64 c = c0 + threadIdx.x;
-        const u32 mine = c < Cfg::kChunks ? counts[c] : 0u;
-        u32 total;
-        const u32 before = blockExclusiveSum<1024>(mine, lds, total);
-        if (c < Cfg::kChunks) bases[c] = carry + before;
-        carry += total;
+    constexpr u64 kPer = (Cfg::kChunks + 1023) / 1024;
+    constexpr bool kHeld = kPer <= 64;  // a thread's counts are loaded at once (independent loads) and kept
+    const u64 first = (u64)threadIdx.x * kPer;
+    u32 held[kHeld ? kPer : 1];
+    u32 mine = 0;
+    if (kHeld) {
+#pragma unroll
+        for (u64 j = 0; j < kPer; ++j) held[j] = first + j < Cfg::kChunks ? counts[first + j] : 0u;
+#pragma unroll
+        for (u64 j = 0; j < kPer; ++j) mine += held[j];
+    } else {
+        for (u64 c = first; c < first + kPer && c < Cfg::kChunks; ++c) mine += counts[c];
     }
-    if (threadIdx.x == 0) *numSelected = carry;
+    u32 total;
+    u32 running = blockExclusiveSum<1024>(mine, lds, total);
+    if (kHeld) {
+#pragma unroll
+        for (u64 j = 0; j < kPer; ++j) {
+            if (first + j < Cfg::kChunks) bases[first + j] = running;
+            running += held[j];
+        }
+    } else {
+        for (u64 c = first; c < first + kPer && c < Cfg::kChunks; ++c) {
+            bases[c] = running;
+            running += counts[c];
+        }
+    }
+    if (threadIdx.x == 0) *numSelected = total;
 }
 
+// The flagged elements of the chunk are ranked in position order, gathered in LDS and written out as one contiguous run.
 template <typename Cfg>
 __device__ __forceinline__ void selectScatter(const typename Cfg::Word* in, const u8* flags, const u32* bases, typename Cfg::Word* out) {
-    __shared__ u32 lds[Cfg::kThreads / kWave];
-    const u64 first = ((u64)blockIdx.x * Cfg::kThreads + threadIdx.x) * Cfg::kItems;
-    const u32 bits = first < Cfg::kTotal ? selectFlagBits<Cfg>(flags, first) : 0u;
-    u32 total;
-    u32 at = bases[blockIdx.x] + blockExclusiveSum<Cfg::kThreads>((u32)__builtin_popcount(bits), lds, total);
+    typedef typename Cfg::Word Word;
+    static_assert(Cfg::kRounds == 4, "the ranks of four rounds travel in the four 16-bit fields of one 64-bit sum");
+    __shared__ u32 lds[2 * (Cfg::kThreads / kWave)];
+    __shared__ Word kept[SelectChunk<Cfg>::kElems];
+    const u64 chunkBase = (u64)blockIdx.x * SelectChunk<Cfg>::kElems;
+    u32 bits[Cfg::kRounds];
+    Pack<Word, Cfg::kVec> values[Cfg::kRounds];
+    u64 packed = 0;  // field r: flagged elements this thread holds in round r
 #pragma unroll
-    for (int k = 0; k < Cfg::kItems; ++k) {
-        if (bits & (1u << k)) out[at++] = in[first + k];
+    for (int round = 0; round < Cfg::kRounds; ++round) {
+        const u64 first = chunkBase + ((u64)round * Cfg::kThreads + threadIdx.x) * Cfg::kVec;
+        bits[round] = 0;
+        if (first < Cfg::kTotal) {
+            bits[round] = selectFlagBits<Cfg>(flags, first);
+            if (first + Cfg::kVec <= Cfg::kTotal) {
+                values[round].loadStream(in + first);
+            } else {
+#pragma unroll
+                for (int k = 0; k < Cfg::kVec; ++k)
+                    if (first + k < Cfg::kTotal) values[round].v[k] = in[first + k];
+            }
+        }
+        packed |= (u64)__builtin_popcount(bits[round]) << (16 * round);
     }
+    // exclusive sums over the threads of every field at once (a field stays below 2^16: at most kThreads * kVec per round)
+    u32 totalLo, totalHi;
+    const u32 beforeLo = blockExclusiveSum<Cfg::kThreads>((u32)packed, lds, totalLo);
+    const u32 beforeHi = blockExclusiveSum<Cfg::kThreads>((u32)(packed >> 32), lds + Cfg::kThreads / kWave, totalHi);
+    const u32 roundTotal[4] = {totalLo & 0xffffu, totalLo >> 16, totalHi & 0xffffu, totalHi >> 16};
+    const u32 before[4] = {beforeLo & 0xffffu, beforeLo >> 16, beforeHi & 0xffffu, beforeHi >> 16};
+    u32 roundBase = 0;
+#pragma unroll
+    for (int round = 0; round < Cfg::kRounds; ++round) {
+        u32 at = roundBase + before[round];
+#pragma unroll
+        for (int k = 0; k < Cfg::kVec; ++k)
+            if (bits[round] & (1u << k)) kept[at++] = values[round].v[k];
+        roundBase += roundTotal[round];
+    }
+    __syncthreads();
+    Word* run = out + bases[blockIdx.x];
+    for (u32 i = threadIdx.x; i < roundBase; i += Cfg::kThreads) run[i] = kept[i];
 }
 
 // ---- key images ----------------------------------------------------------------------------------------------------------------
@@ -112,15 +180,34 @@ __device__ __forceinline__ u32 topkImage(typename Cfg::Raw raw) {
     return Cfg::kLargest ? u : (~u & kMask);
 }
 
-// The bucket of a 256-bin histogram that holds the `wanted`-th largest digit (1-based, wanted <= the histogram's total), found
-// by the 256 threads of a block: thread t looks at bin 255 - t.  Returns the bucket in every thread; `above` receives the
-// number of entries in larger buckets.  `lds`: 4 + 2 words.
-__device__ __forceinline__ u32 topkPickBucket(u32 binCount, u32 wanted, u32* lds, u32& above) {
+// Digits are taken from the most significant end: 11, 11 and 10 bits of a 32-bit image, 8 and 8 of a 16-bit one, 8 of an 8-bit one.
+constexpr int kTopkMaxBins = 2048;
+constexpr int kTopkBinsPerThread = kTopkMaxBins / 256;
+
+// The bucket of a histogram of `numBins` bins (a power of two, at most 2048) that holds the `wanted`-th largest digit (1-based,
+// wanted <= the histogram's total), found by the 256 threads of a block: thread t looks at the 8 bins of descending ranks
+// [8 t, 8 t + 8).  Returns the bucket in every thread; `above` receives the number of entries in larger buckets.  `lds`: 6 words.
+template <typename Bins>
+__device__ __forceinline__ u32 topkPickBucket(const Bins& bins, u32 numBins, u32 wanted, u32* lds, u32& above) {
+    u32 counts[kTopkBinsPerThread];
+    u32 mine = 0;
+#pragma unroll
+    for (int i = 0; i < kTopkBinsPerThread; ++i) {
+        const u32 rank = threadIdx.x * kTopkBinsPerThread + i;
+        counts[i] = rank < numBins ? bins(numBins - 1u - rank) : 0u;
+        mine += counts[i];
+    }
     u32 total;
-    const u32 before = blockExclusiveSum<256>(binCount, lds, total);  // entries in larger bins
-    if (before < wanted && wanted <= before + binCount) {
-        lds[4] = 255u - threadIdx.x;
-        lds[5] = before;
+    u32 before = blockExclusiveSum<256>(mine, lds, total);  // entries in the bins of the threads before this one: all larger
+    if (before < wanted && wanted <= before + mine) {
+#pragma unroll
+        for (int i = 0; i < kTopkBinsPerThread; ++i) {
+            if (before < wanted && wanted <= before + counts[i]) {
+                lds[4] = numBins - 1u - (threadIdx.x * kTopkBinsPerThread + i);
+                lds[5] = before;
+            }
+            before += counts[i];
+        }
     }
     __syncthreads();
     const u32 bucket = lds[4];
@@ -130,8 +217,9 @@ __device__ __forceinline__ u32 topkPickBucket(u32 binCount, u32 wanted, u32* lds
 }
 
 // ---- device-wide top-k -----------------------------------------------------------------------------------------------------------
-// Cfg: Raw (u8 / u16 / u32 word of the key), kKind, kBits, kLargest, kTotal, kK (already capped at kTotal, > 0), kPairs, kItems
-// (keys per thread of the gathering pass).  Temporary storage: 256 histogram words, then the state words below.
+// Cfg: Raw (u8 / u16 / u32 word of the key), kKind, kBits, kLargest, kTotal, kK (already capped at kTotal, > 0), kPairs, kVec (keys
+// per vector load: 16 bytes' worth when the key tensor is aligned and kTotal divides, else 1), kItems (vectors per thread of the
+// gathering pass).  Temporary storage: 2048 histogram words, then the state words below.
 struct TopkState {
     u32 prefix;     // the digits fixed so far, in place
     u32 remaining;  // the rank (1-based) of the wanted key among the keys that match the prefix
@@ -141,9 +229,9 @@ struct TopkState {
 
 template <typename Cfg>
 __device__ __forceinline__ void topkInit(u32* temp) {
-    temp[threadIdx.x] = 0;
+    for (int b = threadIdx.x; b < kTopkMaxBins; b += 256) temp[b] = 0;
     if (threadIdx.x == 0) {
-        TopkState* state = reinterpret_cast<TopkState*>(temp + 256);
+        TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
         state->prefix = 0;
         state->remaining = (u32)Cfg::kK;
         state->taken = 0;
@@ -151,57 +239,106 @@ __device__ __forceinline__ void topkInit(u32* temp) {
     }
 }
 
-// Histogram of the digit at `shift` over the keys whose higher digits equal the prefix.  Blocks stride over the keys.
+// Histogram of the `bits`-wide digit at `shift` over the keys whose higher digits equal the prefix.  Blocks stride over the keys
+// in vectors, four vectors of a thread in flight.
 template <typename Cfg>
-__device__ __forceinline__ void topkHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift) {
-    __shared__ u32 bins[256];
-    bins[threadIdx.x] = 0;
+__device__ __forceinline__ void topkHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
+    typedef typename Cfg::Raw Raw;
+    constexpr int V = Cfg::kVec, kUnroll = 4;
+    __shared__ u32 bins[kTopkMaxBins];
+    const u32 numBins = 1u << bits;
+    for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
     __syncthreads();
-    const u32 prefix = reinterpret_cast<const TopkState*>(temp + 256)->prefix;
-    const u32 fixedBits = shift + 8 >= 32 ? 0u : (0xffffffffu << (shift + 8));
-    for (u64 i = (u64)blockIdx.x * 256 + threadIdx.x; i < Cfg::kTotal; i += (u64)gridDim.x * 256) {
-        const u32 image = topkImage<Cfg>(keys[i]);
-        if ((image & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image >> shift) & 255u], 1u);
+    const u32 prefix = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins)->prefix;
+    const u32 fixedBits = shift + bits >= 32 ? 0u : (0xffffffffu << (shift + bits));
+    const u32 digitMask = numBins - 1u;
+    constexpr u64 kVectors = Cfg::kTotal / V;  // kTotal is a multiple of V
+    const u64 stride = (u64)gridDim.x * 256;
+    for (u64 v0 = (u64)blockIdx.x * 256 + threadIdx.x; v0 < kVectors; v0 += stride * kUnroll) {
+        Pack<Raw, V> x[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            if (v0 + u * stride < kVectors) x[u].loadStream(keys + (v0 + u * stride) * V);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (v0 + u * stride < kVectors) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) {
+                    const u32 image = topkImage<Cfg>(x[u].v[k]);
+                    if ((image & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
+                }
+            }
+        }
     }
     __syncthreads();
-    const u32 mine = bins[threadIdx.x];
-    if (mine != 0) atomicAdd(&temp[threadIdx.x], mine);
+    for (u32 b = threadIdx.x; b < numBins; b += 256) {
+        const u32 mine = bins[b];
+        if (mine != 0) atomicAdd(&temp[b], mine);
+    }
 }
 
 // One block of 256 threads: fixes the digit at `shift` and clears the histogram for the next pass.
 template <typename Cfg>
-__device__ __forceinline__ void topkPick(u32* temp, u32 shift) {
+__device__ __forceinline__ void topkPick(u32* temp, u32 shift, u32 bits) {
     __shared__ u32 lds[8];
-    TopkState* state = reinterpret_cast<TopkState*>(temp + 256);
+    TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
     const u32 wanted = state->remaining, prefix = state->prefix;
     u32 above;
-    const u32 bucket = topkPickBucket(temp[255 - threadIdx.x], wanted, lds, above);
-    temp[threadIdx.x] = 0;
+    const u32 bucket = topkPickBucket([&](u32 b) { return temp[b]; }, 1u << bits, wanted, lds, above);
+    for (int b = threadIdx.x; b < kTopkMaxBins; b += 256) temp[b] = 0;
     if (threadIdx.x == 0) {
         state->prefix = prefix | (bucket << shift);
         state->remaining = wanted - above;
     }
 }
 
-// Writes the keys above the threshold image (kK - remaining of them) and `remaining` of the keys equal to it.
+// Writes the keys above the threshold image (kK - remaining of them) and `remaining` of the keys equal to it.  Every
+// wavefront counts its qualifying keys with votes, the block adds the counts up and asks once for that many output slots
+// (requests for slots from all over the grid meet at one address, and the memory system serves those one after the other:
+// one request per wavefront vote cost 0.7 ms at k = 65 536); a block without qualifying keys, the usual case when k is
+// small next to the input, leaves after the count.
 template <typename Cfg>
 __device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
-    __shared__ u32 lds[Cfg::kThreads / kWave];
-    __shared__ u32 bases[2];
-    TopkState* state = reinterpret_cast<TopkState*>(temp + 256);
+    typedef typename Cfg::Raw Raw;
+    constexpr int V = Cfg::kVec, kWaves = Cfg::kThreads / kWave;
+    __shared__ u32 waveAbove[kWaves], waveTies[kWaves], bases[2];
+    TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
     const u32 threshold = state->prefix, wantedTies = state->remaining, firstTieSlot = (u32)Cfg::kK - wantedTies;
-    const u64 first = ((u64)blockIdx.x * Cfg::kThreads + threadIdx.x) * Cfg::kItems;
-    u32 aboveBits = 0, tieBits = 0;
-    for (int k = 0; k < Cfg::kItems; ++k) {
-        if (first + k < Cfg::kTotal) {
-            const u32 image = topkImage<Cfg>(keys[first + k]);
-            aboveBits |= (image > threshold ? 1u : 0u) << k;
-            tieBits |= (image == threshold ? 1u : 0u) << k;
+    constexpr u64 kVectors = Cfg::kTotal / V;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const u64 lowerLanes = ((u64)1 << lane) - 1;
+    const u64 blockFirst = (u64)blockIdx.x * Cfg::kThreads * Cfg::kItems;
+    Pack<Raw, V> x[Cfg::kItems];
+#pragma unroll
+    for (int it = 0; it < Cfg::kItems; ++it) {
+        const u64 v = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x;
+        if (v < kVectors) x[it].loadStream(keys + v * V);
+    }
+    u32 above = 0, ties = 0;  // of this wavefront
+#pragma unroll
+    for (int it = 0; it < Cfg::kItems; ++it) {
+        const bool live = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x < kVectors;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const u32 image = live ? topkImage<Cfg>(x[it].v[k]) : 0u;
+            above += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(live && image > threshold));
+            ties += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(live && image == threshold));
         }
     }
-    u32 blockAbove, blockTies;
-    u32 aboveAt = blockExclusiveSum<Cfg::kThreads>((u32)__builtin_popcount(aboveBits), lds, blockAbove);
-    u32 tieAt = blockExclusiveSum<Cfg::kThreads>((u32)__builtin_popcount(tieBits), lds, blockTies);
+    if (lane == 0) {
+        waveAbove[wave] = above;
+        waveTies[wave] = ties;
+    }
+    __syncthreads();
+    u32 aboveAt = 0, tieAt = 0, blockAbove = 0, blockTies = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        aboveAt += w < wave ? waveAbove[w] : 0u;
+        tieAt += w < wave ? waveTies[w] : 0u;
+        blockAbove += waveAbove[w];
+        blockTies += waveTies[w];
+    }
+    if (blockAbove + blockTies == 0) return;
     if (threadIdx.x == 0) {
         bases[0] = blockAbove ? atomicAdd(&state->taken, blockAbove) : 0u;
         bases[1] = blockTies ? atomicAdd(&state->ties, blockTies) : 0u;
@@ -209,25 +346,38 @@ __device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const 
     __syncthreads();
     aboveAt += bases[0];
     tieAt += bases[1];
-    for (int k = 0; k < Cfg::kItems; ++k) {
-        u32 slot = 0xffffffffu;
-        if (aboveBits & (1u << k)) slot = aboveAt++;
-        if (tieBits & (1u << k)) {
-            if (tieAt < wantedTies) slot = firstTieSlot + tieAt;
-            ++tieAt;
-        }
-        if (slot != 0xffffffffu) {
-            outKeys[slot] = keys[first + k];
-            if (Cfg::kPairs) outValues[slot] = values[first + k];
+    if (above + ties == 0) return;  // nothing in this wavefront
+#pragma unroll
+    for (int it = 0; it < Cfg::kItems; ++it) {
+        const u64 v = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x;
+        const bool live = v < kVectors;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const u32 image = live ? topkImage<Cfg>(x[it].v[k]) : 0u;
+            const bool isAbove = live && image > threshold, isTie = live && image == threshold;
+            const u64 aboveVotes = __builtin_amdgcn_ballot_w64(isAbove), tieVotes = __builtin_amdgcn_ballot_w64(isTie);
+            u32 slot = 0xffffffffu;
+            if (isAbove) slot = aboveAt + (u32)__builtin_popcountll(aboveVotes & lowerLanes);
+            if (isTie) {
+                const u32 rank = tieAt + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+                if (rank < wantedTies) slot = firstTieSlot + rank;
+            }
+            aboveAt += (u32)__builtin_popcountll(aboveVotes);
+            tieAt += (u32)__builtin_popcountll(tieVotes);
+            if (slot != 0xffffffffu) {
+                outKeys[slot] = x[it].v[k];
+                if (Cfg::kPairs) outValues[slot] = values[v * V + k];
+            }
         }
     }
 }
 
 // ---- top-k of every row: one block per row ------------------------------------------------------------------------------------------
-// Cfg additionally: kSegment (row length, <= kThreads * kItems), kK < kSegment.  Output row r holds kK keys at outKeys + r * kK.
+// Cfg additionally: kSegment (row length, <= kThreads * kItems), kK < kSegment; kItems counts single keys here.  Output row r
+// holds kK keys at outKeys + r * kK.
 template <typename Cfg>
 __device__ __forceinline__ void topkRows(const typename Cfg::Raw* keys, const u32* values, typename Cfg::Raw* outKeys, u32* outValues) {
-    __shared__ u32 bins[256];
+    __shared__ u32 bins[kTopkMaxBins];
     __shared__ u32 lds[8];
     __shared__ u32 counters[2];
     const u64 rowBase = (u64)blockIdx.x * Cfg::kSegment;
@@ -238,20 +388,25 @@ __device__ __forceinline__ void topkRows(const typename Cfg::Raw* keys, const u3
         image[k] = p < Cfg::kSegment ? topkImage<Cfg>(keys[rowBase + p]) : 0u;
     }
     u32 prefix = 0, remaining = (u32)Cfg::kK;
-    for (int shift = Cfg::kBits - 8; shift >= 0; shift -= 8) {
-        bins[threadIdx.x] = 0;
+    int high = Cfg::kBits;  // digits below `high` are still open
+    while (high > 0) {
+        const int bits = Cfg::kBits == 32 ? (high > 10 ? 11 : 10) : 8;
+        const int shift = high - bits;
+        const u32 numBins = 1u << bits;
+        for (u32 b = threadIdx.x; b < numBins; b += Cfg::kThreads) bins[b] = 0;
         __syncthreads();
-        const u32 fixedBits = shift + 8 >= 32 ? 0u : (0xffffffffu << (shift + 8));
+        const u32 fixedBits = high >= 32 ? 0u : (0xffffffffu << high);
 #pragma unroll
         for (int k = 0; k < Cfg::kItems; ++k) {
             const u32 p = (u32)k * Cfg::kThreads + threadIdx.x;
-            if (p < Cfg::kSegment && (image[k] & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image[k] >> shift) & 255u], 1u);
+            if (p < Cfg::kSegment && (image[k] & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image[k] >> shift) & (numBins - 1u)], 1u);
         }
         __syncthreads();
         u32 above;
-        const u32 bucket = topkPickBucket(bins[255 - threadIdx.x], remaining, lds, above);
+        const u32 bucket = topkPickBucket([&](u32 b) { return bins[b]; }, numBins, remaining, lds, above);
         prefix |= bucket << shift;
         remaining -= above;
+        high = shift;
     }
     if (threadIdx.x < 2) counters[threadIdx.x] = 0;
     __syncthreads();

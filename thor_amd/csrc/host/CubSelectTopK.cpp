@@ -3,6 +3,7 @@
 // CubDevicePrimitiveSupport.cpp:116-182,225-330 argument checks and the fixed-size limits of the row form).
 #include "Utilities/TensorOperations/Cub/CubDevicePrimitives.h"
 
+#include "ReductionPlanner.h"
 #include "Utilities/Common/ScopedGpu.h"
 #include "Utilities/Expression/CompiledEquation.h"
 #include "thorhip_numeric_embed.h"
@@ -24,7 +25,8 @@ struct CubSelectionKernels {
     uint64_t chunks = 0;          // blocks of the counting / scattering / gathering launches; rows for kind 2
     uint32_t histogramBlocks = 0;
     uint32_t threads = 256;
-    int digits = 0;
+    int digits = 0;                                // passes of the device-wide selection
+    std::vector<std::pair<uint32_t, uint32_t>> digitPlan;  // (shift, bits) from the most significant digit down
     size_t countsBytes = 0;  // select: chunk counts, then as many chunk bases
     size_t tempBytes = 1;
     std::string variant;
@@ -33,8 +35,9 @@ struct CubSelectionKernels {
 namespace {
 
 constexpr uint64_t kRowTopKMaxSegment = 8192, kRowTopKMaxK = 8192;
-constexpr uint32_t kSelectThreads = 256, kSelectItems = 16;
-constexpr uint32_t kGatherThreads = 256, kGatherItems = 8;
+constexpr uint32_t kSelectThreads = 256, kSelectRounds = 4;
+constexpr uint32_t kGatherThreads = 256, kGatherItems = 8;  // vectors per thread
+constexpr uint32_t kTopKBins = 2048;
 
 size_t roundUp(size_t v, size_t to) { return (v + to - 1) / to * to; }
 
@@ -109,21 +112,21 @@ void validateSelect(const Tensor& input, const Tensor& flags, const Tensor& outp
     }
 }
 
-std::shared_ptr<const CubSelectionKernels> buildSelectKernels(DataType dtype, uint64_t numItems, int deviceNum) {
+std::shared_ptr<const CubSelectionKernels> buildSelectKernels(DataType dtype, uint64_t numItems, int deviceNum, uint32_t vec) {
     auto kernels = std::make_shared<CubSelectionKernels>();
     CubSelectionKernels& k = *kernels;
     k.kind = 0;
     k.deviceNum = deviceNum;
     k.threads = kSelectThreads;
-    const uint64_t chunkElems = uint64_t(kSelectThreads) * kSelectItems;
+    const uint64_t chunkElems = uint64_t(kSelectThreads) * vec * kSelectRounds;
     k.chunks = std::max<uint64_t>((numItems + chunkElems - 1) / chunkElems, 1);
     k.countsBytes = roundUp(k.chunks * 4, 256);
     k.tempBytes = 2 * k.countsBytes;
     std::ostringstream s;
     s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
     s << "namespace gen {\nstruct Cfg {\n    typedef " << rawWordName(dtype) << " Word;\n    static constexpr thor::u64 kTotal = " << numItems
-      << "ull;\n    static constexpr int kThreads = " << kSelectThreads << ";\n    static constexpr int kItems = " << kSelectItems
-      << ";\n    static constexpr thor::u64 kChunks = " << k.chunks << "ull;\n};\n}  // namespace gen\n";
+      << "ull;\n    static constexpr int kThreads = " << kSelectThreads << ";\n    static constexpr int kVec = " << vec
+      << ";\n    static constexpr int kRounds = " << kSelectRounds << ";\n    static constexpr thor::u64 kChunks = " << k.chunks << "ull;\n};\n}  // namespace gen\n";
     s << "extern \"C\" __global__ __launch_bounds__(" << kSelectThreads
       << ") void thor_select_count(const thor::u8* flags, thor::u32* counts) { thor::selectCount<gen::Cfg>(flags, counts); }\n";
     s << "extern \"C\" __global__ __launch_bounds__(1024) void thor_select_offsets(const thor::u32* counts, thor::u32* bases, thor::u32* numSelected) {\n"
@@ -136,7 +139,7 @@ std::shared_ptr<const CubSelectionKernels> buildSelectKernels(DataType dtype, ui
     k.second = compileKernel(source, "thor_select_offsets", deviceNum, false);
     k.third = compileKernel(source, "thor_select_scatter", deviceNum, false);
     std::ostringstream v;
-    v << "select-flagged word" << dataTypeSizeInBytes(dtype) * 8 << " chunks" << k.chunks << "x" << chunkElems << " launches3";
+    v << "select-flagged word" << dataTypeSizeInBytes(dtype) * 8 << " vec" << vec << " chunks" << k.chunks << "x" << chunkElems << " launches3";
     k.variant = v.str();
     return kernels;
 }
@@ -229,30 +232,43 @@ void writeKeyTraits(std::ostringstream& s, DataType dtype, bool largest, bool pa
       << ";\n    static constexpr bool kPairs = " << (pairs ? "true" : "false") << ";\n";
 }
 
+std::vector<std::pair<uint32_t, uint32_t>> digitPlanFor(uint32_t keyBits) {
+    if (keyBits == 32) return {{21, 11}, {10, 11}, {0, 10}};
+    if (keyBits == 16) return {{8, 8}, {0, 8}};
+    return {{0, 8}};
+}
+
 // numItems > 0 and 0 < k (already capped at numItems)
-std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint64_t numItems, uint64_t k, bool largest, bool pairs, int deviceNum) {
+std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint64_t numItems, uint64_t k, bool largest, bool pairs, int deviceNum,
+                                                            uint64_t keyAlignmentBytes) {
     auto kernels = std::make_shared<CubSelectionKernels>();
     CubSelectionKernels& sel = *kernels;
     sel.kind = 1;
     sel.deviceNum = deviceNum;
     sel.threads = kGatherThreads;
-    sel.digits = static_cast<int>(dataTypeSizeInBytes(dtype));
-    const uint64_t chunkElems = uint64_t(kGatherThreads) * kGatherItems;
-    sel.chunks = (numItems + chunkElems - 1) / chunkElems;
+    const uint32_t keyBytes = dataTypeSizeInBytes(dtype);
+    sel.digitPlan = digitPlanFor(keyBytes * 8);
+    sel.digits = static_cast<int>(sel.digitPlan.size());
+    uint64_t vec = 16 / keyBytes;
+    while (vec > 1 && (numItems % vec != 0 || keyAlignmentBytes % (vec * keyBytes) != 0)) vec /= 2;
+    const uint64_t vectors = numItems / vec;
+    const uint64_t chunkVectors = uint64_t(kGatherThreads) * kGatherItems;
+    sel.chunks = (vectors + chunkVectors - 1) / chunkVectors;
     // enough striding blocks to keep every compute unit busy, few enough that the global histogram sees little contention
-    sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((numItems + 255) / 256, 2048));
-    sel.tempBytes = (256 + 4) * 4;
+    sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, 2048));
+    sel.tempBytes = (kTopKBins + 4) * 4;
     std::ostringstream s;
     s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
     s << "namespace gen {\nstruct Cfg {\n";
     writeKeyTraits(s, dtype, largest, pairs);
     s << "    static constexpr thor::u64 kTotal = " << numItems << "ull;\n    static constexpr thor::u64 kK = " << k
-      << "ull;\n    static constexpr int kThreads = " << kGatherThreads << ";\n    static constexpr int kItems = " << kGatherItems
-      << ";\n};\n}  // namespace gen\n";
+      << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = " << kGatherThreads
+      << ";\n    static constexpr int kItems = " << kGatherItems << ";\n};\n}  // namespace gen\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_init(thor::u32* temp) { thor::topkInit<gen::Cfg>(temp); }\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift) {\n"
-         "    thor::topkHistogram<gen::Cfg>(keys, temp, shift);\n}\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_pick(thor::u32* temp, thor::u32 shift) { thor::topkPick<gen::Cfg>(temp, shift); }\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
+         "    thor::topkHistogram<gen::Cfg>(keys, temp, shift, bits);\n}\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_pick(thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
+         "    thor::topkPick<gen::Cfg>(temp, shift, bits);\n}\n";
     s << "extern \"C\" __global__ __launch_bounds__(" << kGatherThreads
       << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n"
          "    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
@@ -262,8 +278,8 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     sel.third = compileKernel(source, "thor_topk_pick", deviceNum, false);
     sel.fourth = compileKernel(source, "thor_topk_gather", deviceNum, false);
     std::ostringstream v;
-    v << "top-k radix-select bits" << sel.digits * 8 << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of " << numItems
-      << " launches" << 2 + 2 * sel.digits;
+    v << "top-k radix-select bits" << keyBytes * 8 << " digits" << sel.digits << " vec" << vec << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys")
+      << " k" << k << " of " << numItems << " launches" << 2 + 2 * sel.digits;
     sel.variant = v.str();
     return kernels;
 }
@@ -276,7 +292,7 @@ std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, u
     sel.kind = 2;
     sel.deviceNum = deviceNum;
     sel.threads = 256;
-    sel.digits = static_cast<int>(dataTypeSizeInBytes(dtype));
+    sel.digits = static_cast<int>(digitPlanFor(dataTypeSizeInBytes(dtype) * 8).size());
     sel.chunks = numSegments;
     const uint64_t items = (segmentSize + 255) / 256;
     std::ostringstream s;
@@ -289,7 +305,7 @@ std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, u
          "thor::u32* outValues) {\n    thor::topkRows<gen::Cfg>(keys, values, outKeys, outValues);\n}\n";
     sel.first = compileKernel(s.str(), "thor_topk_rows", deviceNum, false);
     std::ostringstream v;
-    v << "row top-k radix-select bits" << sel.digits * 8 << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of "
+    v << "row top-k radix-select bits" << dataTypeSizeInBytes(dtype) * 8 << " digits" << sel.digits << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of "
       << segmentSize << " rows" << numSegments << " launches1";
     sel.variant = v.str();
     return kernels;
@@ -305,11 +321,11 @@ void launchTopK(const CubSelectionKernels& sel, const void* keysIn, const void* 
     }
     std::vector<void*> initArgs = {&temp};
     sel.first->launch(1, 1, 1, 256, raw, initArgs);
-    for (int digit = sel.digits - 1; digit >= 0; --digit) {
-        uint32_t shift = static_cast<uint32_t>(digit) * 8;
-        std::vector<void*> histogramArgs = {&keysIn, &temp, &shift};
+    for (const std::pair<uint32_t, uint32_t>& digit : sel.digitPlan) {
+        uint32_t shift = digit.first, bits = digit.second;
+        std::vector<void*> histogramArgs = {&keysIn, &temp, &shift, &bits};
         sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, histogramArgs);
-        std::vector<void*> pickArgs = {&temp, &shift};
+        std::vector<void*> pickArgs = {&temp, &shift, &bits};
         sel.third->launch(1, 1, 1, 256, raw, pickArgs);
     }
     std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut};
@@ -369,7 +385,13 @@ CubDeviceSelectFlaggedPlan prepareCubDeviceSelectFlagged(const Tensor& input, co
     plan.flag_dtype = flags.getDataType();
     plan.num_items = numItems;
     // no items: the run only writes the zero count, with the offsets kernel of a one-chunk plan over no elements
-    plan.kernels = buildSelectKernels(plan.input_dtype, numItems, static_cast<int>(plan.placement.getDeviceNum()));
+    // the kernels are specialised for how the three streams are aligned: groups of four elements (four flag bytes) or single ones
+    const uint64_t groupBytes = 4 * dataTypeSizeInBytes(plan.input_dtype);
+    plan.vector_elements = pointerAlignment(input.getMemPtr()) % groupBytes == 0 && pointerAlignment(output.getMemPtr()) % groupBytes == 0 &&
+                                   pointerAlignment(flags.getMemPtr()) % 4 == 0
+                               ? 4
+                               : 1;
+    plan.kernels = buildSelectKernels(plan.input_dtype, numItems, static_cast<int>(plan.placement.getDeviceNum()), static_cast<uint32_t>(plan.vector_elements));
     plan.temp_storage_bytes = std::max<size_t>(plan.kernels->tempBytes, 1);
     return plan;
 }
@@ -381,6 +403,13 @@ void cubDeviceSelectFlagged(const CubDeviceSelectFlaggedPlan& plan, const Tensor
     validateSelect(input, flags, output, numSelected, plan.num_items);
     if (input.getPlacement() != plan.placement || input.getDataType() != plan.input_dtype || flags.getDataType() != plan.flag_dtype || !plan.kernels) {
         throw std::invalid_argument("CUB select-flagged plan is not compatible with the provided tensors.");
+    }
+    if (plan.vector_elements > 1) {
+        const uint64_t bytes = plan.vector_elements * dataTypeSizeInBytes(plan.input_dtype);
+        if (pointerAlignment(input.getMemPtr()) % bytes != 0 || pointerAlignment(output.getMemPtr()) % bytes != 0 ||
+            pointerAlignment(flags.getMemPtr()) % plan.vector_elements != 0) {
+            throw std::invalid_argument("CUB select-flagged plan was prepared for tensors aligned to four elements; these are not.");
+        }
     }
     requireTemp(temp, plan.placement, plan.temp_storage_bytes);
     requireStream(stream, plan.placement);
@@ -422,7 +451,9 @@ void fillTopKPlan(Plan& plan, const Tensor& keysIn, uint64_t numItems, uint64_t 
     plan.order = order;
     const uint64_t selected = std::min(numItems, k);
     if (selected != 0) {
-        plan.kernels = buildTopKKernels(plan.key_dtype, numItems, selected, order == CubTopKOrder::Largest, pairs, static_cast<int>(plan.placement.getDeviceNum()));
+        plan.key_alignment_bytes = std::min<uint64_t>(pointerAlignment(keysIn.getMemPtr()), 16);
+        plan.kernels = buildTopKKernels(plan.key_dtype, numItems, selected, order == CubTopKOrder::Largest, pairs, static_cast<int>(plan.placement.getDeviceNum()),
+                                        plan.key_alignment_bytes);
     }
     plan.temp_storage_bytes = plan.kernels ? plan.kernels->tempBytes : 1;
 }
@@ -458,6 +489,9 @@ void cubDeviceTopKKeys(const CubDeviceTopKKeysPlan& plan, const Tensor& temp, co
     if (keysIn.getPlacement() != plan.placement || keysIn.getDataType() != plan.key_dtype) {
         throw std::invalid_argument("CUB top-k-keys plan is not compatible with the provided tensors.");
     }
+    if (pointerAlignment(keysIn.getMemPtr()) % plan.key_alignment_bytes != 0) {
+        throw std::invalid_argument("CUB top-k-keys plan was prepared for keys with a stricter alignment than these have.");
+    }
     requireTemp(temp, plan.placement, plan.temp_storage_bytes);
     requireStream(stream, plan.placement);
     if (!plan.kernels) return;
@@ -488,6 +522,9 @@ void cubDeviceTopKPairs(const CubDeviceTopKPairsPlan& plan, const Tensor& temp, 
     validateTopKPairs(keysIn, keysOut, valuesIn, valuesOut, plan.num_items, plan.k);
     if (keysIn.getPlacement() != plan.placement || keysIn.getDataType() != plan.key_dtype || valuesIn.getDataType() != plan.value_dtype) {
         throw std::invalid_argument("CUB top-k-pairs plan is not compatible with the provided tensors.");
+    }
+    if (pointerAlignment(keysIn.getMemPtr()) % plan.key_alignment_bytes != 0) {
+        throw std::invalid_argument("CUB top-k-pairs plan was prepared for keys with a stricter alignment than these have.");
     }
     requireTemp(temp, plan.placement, plan.temp_storage_bytes);
     requireStream(stream, plan.placement);

@@ -343,6 +343,84 @@ int thor_topk(thor_tensor_t keys_in, thor_tensor_t keys_out, thor_tensor_t value
         if (variant) copyOut(cubSelectionKernelVariant(kernels), variant, variant_capacity, nullptr);)
 }
 
+struct thor_selection_plan {
+    int kind = 0;  // 0 select-flagged, 1 top-k keys, 2 top-k pairs, 3 row top-k keys, 4 row top-k pairs
+    CubDeviceSelectFlaggedPlan select;
+    CubDeviceTopKKeysPlan keys;
+    CubDeviceTopKPairsPlan pairs;
+    CubDeviceSegmentedTopKKeysPlan rowKeys;
+    CubDeviceSegmentedTopKPairsPlan rowPairs;
+    size_t tempBytes = 1;
+    std::shared_ptr<const CubSelectionKernels> kernels;
+};
+
+thor_selection_plan_t thor_select_flagged_prepare(thor_tensor_t input, thor_tensor_t flags, thor_tensor_t output, thor_tensor_t num_selected_out,
+                                                  uint64_t num_items) {
+    THOR_CAPI_TRY_PTR(require(input, "input"); require(flags, "flags"); require(output, "output"); require(num_selected_out, "num_selected_out");
+                      auto handle = std::make_unique<thor_selection_plan>();
+                      handle->select = prepareCubDeviceSelectFlagged(input->tensor, flags->tensor, output->tensor, num_selected_out->tensor, num_items);
+                      handle->tempBytes = handle->select.temp_storage_bytes; handle->kernels = handle->select.kernels; return handle.release();)
+}
+
+thor_selection_plan_t thor_topk_prepare(thor_tensor_t keys_in, thor_tensor_t keys_out, thor_tensor_t values_in, thor_tensor_t values_out,
+                                        uint64_t num_segments, uint64_t segment_size, uint64_t k, int largest, int segmented) {
+    THOR_CAPI_TRY_PTR(
+        require(keys_in, "keys_in"); require(keys_out, "keys_out");
+        if ((values_in == nullptr) != (values_out == nullptr)) throw std::invalid_argument("top-k takes values_in and values_out together or neither");
+        const CubTopKOrder order = largest ? CubTopKOrder::Largest : CubTopKOrder::Smallest;
+        auto handle = std::make_unique<thor_selection_plan>();
+        if (segmented && values_in) {
+            handle->kind = 4;
+            handle->rowPairs = prepareCubDeviceSegmentedTopKPairs(keys_in->tensor, keys_out->tensor, values_in->tensor, values_out->tensor, num_segments,
+                                                                  segment_size, k, order);
+            handle->tempBytes = handle->rowPairs.temp_storage_bytes;
+            handle->kernels = handle->rowPairs.kernels;
+        } else if (segmented) {
+            handle->kind = 3;
+            handle->rowKeys = prepareCubDeviceSegmentedTopKKeys(keys_in->tensor, keys_out->tensor, num_segments, segment_size, k, order);
+            handle->tempBytes = handle->rowKeys.temp_storage_bytes;
+            handle->kernels = handle->rowKeys.kernels;
+        } else if (values_in) {
+            handle->kind = 2;
+            handle->pairs = prepareCubDeviceTopKPairs(keys_in->tensor, keys_out->tensor, values_in->tensor, values_out->tensor, segment_size, k, order);
+            handle->tempBytes = handle->pairs.temp_storage_bytes;
+            handle->kernels = handle->pairs.kernels;
+        } else {
+            handle->kind = 1;
+            handle->keys = prepareCubDeviceTopKKeys(keys_in->tensor, keys_out->tensor, segment_size, k, order);
+            handle->tempBytes = handle->keys.temp_storage_bytes;
+            handle->kernels = handle->keys.kernels;
+        }
+        return handle.release();)
+}
+
+size_t thor_selection_plan_temp_bytes(thor_selection_plan_t plan) { return plan ? plan->tempBytes : 0; }
+
+int thor_selection_plan_run(thor_selection_plan_t plan, thor_tensor_t temp_storage, thor_tensor_t a, thor_tensor_t b, thor_tensor_t c, thor_tensor_t d,
+                            thor_stream_t stream) {
+    THOR_CAPI_TRY_INT(
+        require(plan, "selection plan"); require(temp_storage, "temp_storage"); require(a, "first tensor"); require(b, "second tensor");
+        require(stream, "stream");
+        const bool four = plan->kind == 0 || plan->kind == 2 || plan->kind == 4;
+        if (four) {
+            require(c, "third tensor");
+            require(d, "fourth tensor");
+        }
+        switch (plan->kind) {
+            case 0: cubDeviceSelectFlagged(plan->select, temp_storage->tensor, a->tensor, b->tensor, c->tensor, d->tensor, stream->stream); break;
+            case 1: cubDeviceTopKKeys(plan->keys, temp_storage->tensor, a->tensor, b->tensor, stream->stream); break;
+            case 2: cubDeviceTopKPairs(plan->pairs, temp_storage->tensor, a->tensor, b->tensor, c->tensor, d->tensor, stream->stream); break;
+            case 3: cubDeviceSegmentedTopKKeys(plan->rowKeys, temp_storage->tensor, a->tensor, b->tensor, stream->stream); break;
+            default: cubDeviceSegmentedTopKPairs(plan->rowPairs, temp_storage->tensor, a->tensor, b->tensor, c->tensor, d->tensor, stream->stream); break;
+        })
+}
+
+int thor_selection_plan_variant(thor_selection_plan_t plan, char* buffer, size_t capacity) {
+    THOR_CAPI_TRY_INT(require(plan, "selection plan"); copyOut(cubSelectionKernelVariant(plan->kernels), buffer, capacity, nullptr);)
+}
+
+void thor_selection_plan_destroy(thor_selection_plan_t plan) { delete plan; }
+
 int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments, uint64_t segment_size,
               int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity) {
     THOR_CAPI_TRY_INT(

@@ -64,6 +64,10 @@ PROTOTYPES = {
     "thor_scan": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
     "thor_scan_no_alloc": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
     "thor_select_flagged": (_i, [_vp, _vp, _vp, _vp, ctypes.c_uint64, _vp, _cp, _sz]),
+    "thor_select_flagged_prepare": (_vp, [_vp, _vp, _vp, _vp, ctypes.c_uint64]),
+    "thor_topk_prepare": (_vp, [_vp, _vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i]),
+    "thor_selection_plan_temp_bytes": (_sz, [_vp]), "thor_selection_plan_run": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "thor_selection_plan_variant": (_i, [_vp, _cp, _sz]), "thor_selection_plan_destroy": (None, [_vp]),
     "thor_topk": (_i, [_vp, _vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _vp, _cp, _sz]),
     "thor_reduction_generate_source": (_i, [_i, _i, _i, _i, _i, _u64p, _u64p, _i, _u32p, _i, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_arg_reduction_stamp": (_vp, [_i, _u32p, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
@@ -573,6 +577,58 @@ def scan(input: PhysicalTensor, output: PhysicalTensor, stream: Stream, op: Scan
     _check(entry(input._h, output._h, segment_offsets._h if segment_offsets is not None else None, n, segments, segment_size, code, int(arg),
                  int(inclusive), int(reverse), stream._h, text, 512), "scan")
     return text.value.decode()
+
+
+class SelectionPlan:
+    """A prepared select-flagged or top-k (prepareCubDeviceSelectFlagged / prepareCubDeviceTopKKeys / ...Pairs / Segmented..., the plan
+    structs of CubDevicePrimitives.h:47-93 there): ``temp_storage_bytes`` of UINT8 temporary storage, ``run`` with the tensors in the
+    order the plan was prepared with.  Nothing is allocated by ``run``."""
+
+    def __init__(self, ptr, what):
+        self._h = _handle(ptr, what)
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                lib().thor_selection_plan_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    @staticmethod
+    def select_flagged(input: PhysicalTensor, flags: PhysicalTensor, output: PhysicalTensor, num_selected_out: PhysicalTensor,
+                       num_items: Optional[int] = None) -> "SelectionPlan":
+        n = int(num_items if num_items is not None else np.prod(input.get_dimensions()))
+        return SelectionPlan(lib().thor_select_flagged_prepare(input._h, flags._h, output._h, num_selected_out._h, n), "prepare select_flagged")
+
+    @staticmethod
+    def top_k(keys_in: PhysicalTensor, keys_out: PhysicalTensor, k: int, largest: bool = True, values_in: Optional[PhysicalTensor] = None,
+              values_out: Optional[PhysicalTensor] = None, num_items: Optional[int] = None, num_segments: Optional[int] = None,
+              segment_size: Optional[int] = None) -> "SelectionPlan":
+        values = (values_in._h if values_in is not None else None, values_out._h if values_out is not None else None)
+        if segment_size is not None:
+            segments = int(num_segments if num_segments is not None else np.prod(keys_in.get_dimensions()) // max(int(segment_size), 1))
+            return SelectionPlan(lib().thor_topk_prepare(keys_in._h, keys_out._h, values[0], values[1], segments, int(segment_size), int(k), int(largest), 1),
+                                 "prepare top_k")
+        n = int(num_items if num_items is not None else np.prod(keys_in.get_dimensions()))
+        return SelectionPlan(lib().thor_topk_prepare(keys_in._h, keys_out._h, values[0], values[1], 0, n, int(k), int(largest), 0), "prepare top_k")
+
+    @property
+    def temp_storage_bytes(self) -> int:
+        return int(lib().thor_selection_plan_temp_bytes(self._h))
+
+    def allocate_temp_storage(self, gpu_num: int = 0) -> PhysicalTensor:
+        return PhysicalTensor(Placement(DeviceType.gpu, gpu_num), PhysicalTensor.Descriptor(DataType.uint8, [max(self.temp_storage_bytes, 1)]))
+
+    def run(self, temp_storage: PhysicalTensor, a: PhysicalTensor, b: PhysicalTensor, c: Optional[PhysicalTensor] = None,
+            d: Optional[PhysicalTensor] = None, *, stream: Stream):
+        _check(lib().thor_selection_plan_run(self._h, temp_storage._h, a._h, b._h, c._h if c is not None else None, d._h if d is not None else None,
+                                             stream._h), "SelectionPlan.run")
+
+    def variant(self) -> str:
+        text = ctypes.create_string_buffer(512)
+        _check(lib().thor_selection_plan_variant(self._h, text, 512), "SelectionPlan.variant")
+        return text.value.decode()
 
 
 def select_flagged(input: PhysicalTensor, flags: PhysicalTensor, output: PhysicalTensor, num_selected_out: PhysicalTensor, stream: Stream,
