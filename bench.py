@@ -97,8 +97,9 @@ def cpu_baseline_other_configs(seconds_each: float = 1.5):
     return out
 
 
-def bench_other_configs():
-    """BASELINE configs 1, 3, 4, 5 through the Expression / reduction API: GB/s on algorithmic bytes, HIP-event timed."""
+def bench_other_configs(only=None):
+    """BASELINE configs 1, 3, 4, 5 through the Expression / reduction API: GB/s on algorithmic bytes, HIP-event timed.  `only`: substrings;
+    a line whose name holds none of them is set up but not launched (for short profiler runs)."""
     from thor_amd import physical as ph
     from thor_amd.dtypes import DataType
     from thor_amd.physical import Expression as ex
@@ -131,6 +132,8 @@ def bench_other_configs():
     def timed(name, runs, nbytes, elements, note=""):
         """Median of 5 samples; a sample is one pass over every rotating buffer (at least 8 launches), bracketed by events on
         the launch stream (the reference's protocol: warm-up, >= 5 samples x >= 4 iterations, median)."""
+        if only and not any(part in name for part in only):
+            return
         if callable(runs):
             runs = [runs]
         reps = max(8, len(runs))
@@ -442,23 +445,50 @@ def summarize_kernel_trace(db, bench_json=None):
 
 def summarize_hbm_traffic(fetch_db, write_db, bench_json=None):
     """HBM bytes per dispatch out of two `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE) of this script with --calibration-copy:
-    each counter is scaled by its own reading for the calibration copy (uint32 -> int32 over 2^28 elements: 1 GiB each way)."""
+    each counter is scaled by its own reading for the calibration copy (uint32 -> int32 over 2^28 elements: 1 GiB each way).  Dispatches
+    of one kernel with different grids (the same conversion kernel also prepares smaller inputs) are listed apart."""
     import sqlite3
     tags = _bench_lines_by_kernel_tag(bench_json)
 
     def read(db, counter):
         con = sqlite3.connect(db)
-        return {n: (c, a) for n, c, a in con.execute(
-            "select kernel_name, count(*), avg(value) from counters_collection where counter_name=? group by kernel_name", (counter,))}
+        return {(n, g): (c, a) for n, g, c, a in con.execute(
+            "select kernel_name, grid_size, count(*), avg(value) from counters_collection where counter_name=? group by kernel_name, grid_size", (counter,))}
     fetch, write = read(fetch_db, "FETCH_SIZE"), read(write_db, "WRITE_SIZE")
-    calibration = [n for n in fetch if "convertSlots<unsigned int, int" in n][0]
+    calibration = max((key for key in fetch if "convertSlots<unsigned int, int" in key[0]), key=lambda key: key[1])
     kf, kw = 1048576.0 / fetch[calibration][1], 1048576.0 / write[calibration][1]
-    print(f"calibration copy {_short(calibration, 48)}: FETCH_SIZE {fetch[calibration][1]:.1f} KiB, WRITE_SIZE {write[calibration][1]:.1f} KiB "
+    print(f"calibration copy {_short(calibration[0], 48)}: FETCH_SIZE {fetch[calibration][1]:.1f} KiB, WRITE_SIZE {write[calibration][1]:.1f} KiB "
           f"per dispatch for 1 048 576 KiB each way -> factors {kf:.5f}, {kw:.5f}")
-    print(f"{'dispatches':>10} {'fetch MiB':>10} {'write MiB':>10} {'total MB':>10}  kernel <- bench line")
-    for name in sorted(fetch, key=lambda n: -(fetch[n][1] * kf + write.get(n, (0, 0))[1] * kw)):
-        fm, wm = fetch[name][1] * kf / 1024, write.get(name, (0, 0))[1] * kw / 1024
-        print(f"{fetch[name][0]:10d} {fm:10.2f} {wm:10.2f} {(fm + wm) * 1.048576:10.2f}  {_short(name)} <- {_line_of(name, tags)}")
+    print(f"{'dispatches':>10} {'grid':>11} {'fetch MiB':>10} {'write MiB':>10} {'total MB':>10}  kernel <- bench line")
+    for key in sorted(fetch, key=lambda k: -(fetch[k][1] * kf + write.get(k, (0, 0))[1] * kw)):
+        fm, wm = fetch[key][1] * kf / 1024, write.get(key, (0, 0))[1] * kw / 1024
+        print(f"{fetch[key][0]:10d} {key[1]:11d} {fm:10.2f} {wm:10.2f} {(fm + wm) * 1.048576:10.2f}  {_short(key[0])} <- {_line_of(key[0], tags)}")
+
+
+def summarize_counters(dbs, bench_json=None):
+    """Average per dispatch of every counter in one or more `rocprofv3 --pmc` databases of this script: one row per kernel and grid
+    size, one column per counter, plus the average dispatch duration of the first database that saw the kernel."""
+    import sqlite3
+    tags = _bench_lines_by_kernel_tag(bench_json)
+    table, names = {}, []
+    for db in dbs:
+        con = sqlite3.connect(db)
+        for kernel, grid, counter, count, avg, duration in con.execute(
+                "select kernel_name, grid_size, counter_name, count(*), avg(value), avg(duration) from counters_collection "
+                "group by kernel_name, grid_size, counter_name"):
+            row = table.setdefault((kernel, grid), {"dispatches": count, "us": duration / 1e3})
+            row[counter] = avg
+            if counter not in names:
+                names.append(counter)
+    for at in range(0, len(names), 4):
+        group = names[at:at + 4]
+        print(f"{'dispatches':>10} {'grid':>11} {'avg_us':>9} " + " ".join(f"{n:>36s}" for n in group) + "  kernel <- bench line")
+        for (kernel, grid), row in sorted(table.items(), key=lambda item: -item[1]["us"]):
+            if not any(n in row for n in group) or row["us"] < 15.0:
+                continue
+            print(f"{row['dispatches']:10d} {grid:11d} {row['us']:9.1f} " + " ".join(f"{row.get(n, float('nan')):36.1f}" for n in group) +
+                  f"  {_short(kernel, 44)} <- {_line_of(kernel, tags)}")
+        print()
 
 
 def main():
@@ -467,6 +497,10 @@ def main():
                     help="print the per-kernel duration table of a rocprofv3 --kernel-trace database (optionally tagged with the bench lines of BENCH_JSON) and exit")
     ap.add_argument("--summarize-hbm-traffic", nargs="+", metavar=("FETCH_DB", "WRITE_DB"),
                     help="print the HBM-traffic table of two rocprofv3 --pmc databases (FETCH_SIZE run, WRITE_SIZE run[, BENCH_JSON]) and exit")
+    ap.add_argument("--summarize-counters", nargs="+", metavar="DB",
+                    help="print the average reading per dispatch of every counter in the given rocprofv3 --pmc databases, kernel by kernel "
+                         "(a last argument ending in .json is taken as BENCH_JSON), and exit")
+    ap.add_argument("--lines", default="", help="comma-separated substrings: launch only the secondary lines whose name holds one of them")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -482,6 +516,11 @@ def main():
         return
     if args.summarize_hbm_traffic:
         summarize_hbm_traffic(*args.summarize_hbm_traffic[:3])
+        return
+    if args.summarize_counters:
+        given = list(args.summarize_counters)
+        bench_json = given.pop() if given[-1].endswith(".json") else None
+        summarize_counters(given, bench_json)
         return
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -564,7 +603,7 @@ def main():
     for b_ in (src, f16, b16, w16, wb16):
         b_.free()
     if not args.no_other_configs:
-        result["other_configs"] = bench_other_configs()
+        result["other_configs"] = bench_other_configs([part for part in args.lines.split(",") if part] or None)
         # the fraction of the HBM peak every secondary line reached, next to the headline kernel's (kept compact: drivers keep the parsed line)
         result["roofline"]["per_config"] = {"c2_convert_fp32_to_fp16": round(achieved / HBM_PEAK_GBPS, 4),
                                             **{name: round(v["GB/s"] / HBM_PEAK_GBPS, 4) for name, v in result["other_configs"].items()}}

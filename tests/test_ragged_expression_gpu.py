@@ -198,7 +198,9 @@ def test_fused_and_staged_softmax_plans_agree(stream, dtype):
         return out
 
     fused, reference = both(), staged(both)
-    assert fused["softmax"][0] == ["SegmentedReduction", "FusedReduction", "SegmentedBroadcast", "FusedKernel"]
+    # the segment maximum and the sum of exponentials come out of one pass over the values when the arithmetic is fp32
+    one_pass = ["FusedReduction", "SegmentedBroadcast", "FusedKernel"]
+    assert fused["softmax"][0] == (one_pass if dtype == DataType.fp32 else ["SegmentedReduction"] + one_pass), fused["softmax"][0]
     assert reference["softmax"][0] == ["SegmentedReduction", "SegmentedBroadcast", "FusedKernel", "SegmentedReduction", "SegmentedBroadcast", "FusedKernel"]
     tolerance = 1e-6 if dtype == DataType.fp32 else 2e-3
     for name in ("softmax", "log_softmax"):

@@ -261,6 +261,61 @@ struct ValueAcc {
     }
 };
 
+// The two statistics of a softmax in one pass: m = the maximum of the elements seen (NaN wins, like MaxOp) and
+// s = the sum of exp(x - m) over them.  A new maximum rescales the sum gathered so far; merging rescales the side with the
+// smaller maximum.  One exponential per element: with d = x - m, exp(-|d|) is the factor of the old sum (d > 0) or the new
+// term (d <= 0).  Elements equal to -inf add nothing, so an empty accumulator is {-inf, 0}.  (The library's expf on purpose: a
+// base-2 hardware exponential with a compensated argument is as accurate and a sixth of the instructions, but measured
+// slower in the segment kernel, 574 against 340 us: the compiler overlaps more of them and residency drops to two wavefronts.)
+struct OnlineSoftmaxAcc {
+    float m, s;
+    __device__ __forceinline__ void reset() {
+        m = -__builtin_inff();
+        s = 0.0f;
+    }
+    template <typename I>
+    __device__ __forceinline__ void add(float x, I) {
+        const float d = x - m;
+        const float e = x == -__builtin_inff() ? 0.0f : expf(-fabsf(d));  // m == -inf, x finite: d = +inf, e = 0
+        const bool rises = (d > 0.0f) | (x != x);
+        s = rises ? s * e + 1.0f : s + e;
+        m = MaxOp::combine(m, x);
+    }
+    __device__ __forceinline__ static float scaleTo(float from, float to) { return from == -__builtin_inff() ? 0.0f : expf(from - to); }
+    __device__ __forceinline__ void merge(const OnlineSoftmaxAcc& o) {
+        const float top = MaxOp::combine(m, o.m);
+        s = s * scaleTo(m, top) + o.s * scaleTo(o.m, top);
+        m = top;
+    }
+    __device__ __forceinline__ OnlineSoftmaxAcc shuffleXor(int mask) const {
+        OnlineSoftmaxAcc r;
+        r.m = __shfl_xor(m, mask, kWave);
+        r.s = __shfl_xor(s, mask, kWave);
+        return r;
+    }
+    // A partial of `slots` accumulators is two float arrays of that length, maxima first.
+    __device__ __forceinline__ static u64 partialBytes(u64 slots) { return 2 * (((slots * 4 + 7) / 8) * 8); }
+    template <bool DEVICE_WIDE = false>
+    __device__ __forceinline__ void storePartial(void* partials, u64 slot, u64 slots) const {
+        float* maxima = static_cast<float*>(partials);
+        float* sums = reinterpret_cast<float*>(static_cast<char*>(partials) + ((slots * 4 + 7) / 8) * 8);
+        if (DEVICE_WIDE) {
+            storeDeviceWide(maxima + slot, m);
+            storeDeviceWide(sums + slot, s);
+        } else {
+            maxima[slot] = m;
+            sums[slot] = s;
+        }
+    }
+    template <bool DEVICE_WIDE = false>
+    __device__ __forceinline__ void loadPartial(const void* partials, u64 slot, u64 slots) {
+        const float* maxima = static_cast<const float*>(partials);
+        const float* sums = reinterpret_cast<const float*>(static_cast<const char*>(partials) + ((slots * 4 + 7) / 8) * 8);
+        m = DEVICE_WIDE ? loadDeviceWide(maxima + slot) : maxima[slot];
+        s = DEVICE_WIDE ? loadDeviceWide(sums + slot) : sums[slot];
+    }
+};
+
 // Candidate {value, index}: NaN beats every number, equal values (and two NaNs) keep the lower index.  The empty
 // candidate carries the all-ones index, so any real element wins against it.
 template <bool IS_MAX, typename IndexT>

@@ -1276,6 +1276,85 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
         return true;
     };
 
+    // The two statistics of a segment softmax in one pass over the values: `node` is the segment maximum of a tensor x, and a
+    // segment sum over the same partition of exp(x - broadcast(maximum)) (fp32 arithmetic, nothing else in between) is waiting
+    // further up.  One segment kernel with a {maximum, sum of exponentials} accumulator writes both.  False = not that pattern.
+    auto stampSegmentSoftmaxStatistics = [&](uint32_t node) -> bool {
+        const ExprNode& n = expr.nodes[node];
+        if (n.op != ExprOp::SEGMENTED_REDUCE_MAX || graph->role[n.lhs] == Role::Inline) return false;
+        uint32_t sumNode = UINT32_MAX;
+        for (uint32_t j = node + 1; j < expr.nodes.size() && sumNode == UINT32_MAX; ++j) {
+            const ExprNode& sum = expr.nodes[j];
+            if (done[j] || sum.op != ExprOp::SEGMENTED_REDUCE_SUM || graph->role[j] != Role::Materialized || sum.rhs != n.rhs) continue;
+            if (sum.lhs == UINT32_MAX || graph->role[sum.lhs] != Role::Inline) continue;
+            const ExprNode& e = expr.nodes[sum.lhs];
+            if (e.op != ExprOp::EXP || emittedValueDType(e) != DataType::FP32 || e.output_dtype != DataType::FP32 || graph->role[e.lhs] != Role::Inline) continue;
+            const ExprNode& d = expr.nodes[e.lhs];
+            if (d.op != ExprOp::SUB || emittedValueDType(d) != DataType::FP32 || d.lhs != n.lhs || d.rhs == UINT32_MAX) continue;
+            const ExprNode& g = expr.nodes[d.rhs];
+            if (g.op != ExprOp::SEGMENTED_BROADCAST || graph->role[d.rhs] != Role::Gather || g.lhs != node || g.rhs != n.rhs ||
+                g.segmented_broadcast_normalize_by_length) {
+                continue;
+            }
+            sumNode = j;
+        }
+        if (sumNode == UINT32_MAX) return false;
+        const Tensor& values = tensorOf[n.lhs];
+        const Tensor& offsets = tensorOf[n.rhs];
+        if (!values.isInitialized() || !values.isDenseContiguous() || !offsets.isInitialized() || !offsets.isDenseContiguous()) return false;
+        const std::vector<uint64_t> valueShape = orScalarShape(dims[n.lhs]);
+        if (valueShape.empty()) return false;
+        uint64_t trailing = 1;
+        for (size_t a = 1; a < valueShape.size(); ++a) trailing *= valueShape[a];
+        const uint64_t rows = valueShape[0], segments = offsets.getTotalNumElements() - 1;
+        ReductionKernelRequest request;
+        request.segmented = true;
+        request.segments = segments;
+        request.segmentedRows = rows;
+        request.trailing = trailing;
+        request.offsetsAre64 = offsets.getDataType() == DataType::UINT64;
+        request.deviceNum = device_num;
+        request.inputAlignmentBytes = pointerAlignment(values.getMemPtr());
+        request.geometry.path = CubReductionPath::OffsetSegmented;
+        request.geometry.rank = static_cast<uint32_t>(valueShape.size());
+        request.geometry.input_elements = rows * trailing;
+        request.geometry.output_elements = segments * trailing;
+        request.geometry.reduction_size = rows;
+        request.geometry.output_dimensions = orScalarShape(dims[node]);
+        request.geometry.squeezed_output_dimensions = request.geometry.output_dimensions;
+        ReductionKernelRequest::Source source;
+        source.storage = values.getDataType();
+        source.kind = ReductionKernelRequest::Source::Kind::Vector;
+        request.sources.push_back(source);
+        const DataType valueDType = expr.nodes[n.lhs].output_dtype.value();
+        request.prologue = "        const float x0 = " +
+                           castValueExpr(castValueExpr(storageToValueExpr("l.p0.v[k]", values.getDataType()), values.getDataType(), valueDType), valueDType,
+                                         DataType::FP32) +
+                           ";\n";
+        request.values.push_back({CubReductionOp::Max, n.output_dtype.value(), "x0"});
+        request.values.push_back({CubReductionOp::Sum, expr.nodes[sumNode].output_dtype.value(), "x0"});
+        request.onlineSoftmax = true;
+        request.inputDType = values.getDataType();
+
+        ReductionLaunchPlan plan = buildReductionKernels(request);
+        std::optional<Tensor> workspace = allocateReductionWorkspace(plan, gpuPlacement, stream);
+        Tensor maxima = allocateFor(node), sums = allocateFor(sumNode);
+        StampedExecutionStage stage;
+        stage.kind = StampedExecutionStage::Kind::FusedReduction;
+        stage.gpu_num = device_num;
+        stage.dependency_stage_indices = dependenciesOf({n.lhs, n.rhs});
+        plan.variant = "segment_softmax_statistics(max, sum of exp in one pass) " + plan.variant;
+        stage.fused_reduction = std::make_shared<StampedFusedReduction>(std::move(plan), std::vector<Tensor>{values}, std::vector<std::string>{},
+                                                                        std::vector<Tensor>{maxima, sums}, std::vector<Tensor>{}, workspace,
+                                                                        4 * rows * trailing, offsets);
+        tensorOf[node] = maxima;
+        tensorOf[sumNode] = sums;
+        stageOfNode[node] = stageOfNode[sumNode] = static_cast<int>(stages.size());
+        stages.push_back(std::move(stage));
+        done[node] = done[sumNode] = 1;
+        return true;
+    };
+
     for (uint32_t level = 0; level <= maxLevel; ++level) {
         if (stageFusion) {
             // Reductions over one shape and axes whose inputs exist by now (or are elementwise functions of such tensors
@@ -1298,6 +1377,7 @@ StampedExecutionPlan FusedEquation::stampImpl(const std::unordered_map<std::stri
                     if (stampSegmentedReductionOfExpression(i)) continue;
                     emitFusedGroup({n.lhs});  // operands the reduction cannot evaluate by itself: store the values first
                 }
+                if (stageFusion && stampSegmentSoftmaxStatistics(i)) continue;
                 const Tensor& values = tensorOf[n.lhs];
                 const Tensor& offsets = tensorOf[n.rhs];
                 Tensor output = allocateFor(i);

@@ -276,7 +276,9 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         shape.blocks = tiles;
         shape.gridX = static_cast<uint32_t>(shape.chunks * tiles);
         shape.gridY = 1;
-        if (shape.chunks > 1) shape.workspaceBytes = partialBytes(shape.chunks * 2 * request.trailing, request.isArg, shape.indexIs64) + shape.chunks * 16;
+        if (shape.chunks > 1) {
+            shape.workspaceBytes = accumulators * partialBytes(shape.chunks * 2 * request.trailing, request.isArg, shape.indexIs64) + shape.chunks * 16;
+        }
         return shape;
     }
 
@@ -502,6 +504,9 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     if (request.isArg) {
         int f = 0;
         s << "    typedef " << accumulatorType(request, shape.indexIs64, f) << " Acc;\n";
+    } else if (request.onlineSoftmax) {
+        if (values.size() != 2) throw std::invalid_argument("The one-pass softmax statistics are two values: the maximum and the sum of exponentials.");
+        s << "    typedef OnlineSoftmaxAcc Acc;\n";
     } else if (values.size() == 1) {
         s << "    typedef " << valueAccumulatorType(values[0].op, finalize[0]) << " Acc;\n";
     } else {
@@ -525,7 +530,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     }
     s << "    static __device__ __forceinline__ void accumulateOne(Acc& acc, const Loaded& l, const Sources& s, const Kept& kk, int k, IndexT index) {\n";
     s << prologue;
-    if (request.isArg || values.size() == 1) {
+    if (request.isArg || values.size() == 1 || request.onlineSoftmax) {
         s << "        acc.add(" << values[0].expression << ", index);\n";
     } else {
         for (size_t j = 0; j < values.size(); ++j) s << "        acc.a" << j << ".add(" << values[j].expression << ", index);\n";
@@ -562,6 +567,10 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
                 s << "        o.indexOut[outIndex] = acc.i == ~(IndexT)0 ? ~(" << stored << ")0 : (" << stored << ")acc.i;\n";
             }
         }
+        s << "        (void)scale;\n";
+    } else if (request.onlineSoftmax) {
+        s << "        o.out0[outIndex] = fromFloat<" << deviceTypeName(values[0].outputDType) << ">(acc.m);\n";
+        s << "        o.out1[outIndex] = fromFloat<" << deviceTypeName(values[1].outputDType) << ">(acc.s);\n";
         s << "        (void)scale;\n";
     } else {
         for (size_t j = 0; j < values.size(); ++j) {

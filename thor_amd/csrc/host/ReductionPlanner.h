@@ -47,6 +47,9 @@ struct ReductionKernelRequest {
         DataType outputDType = DataType::FP32;
         std::string expression;  // fp32 C expression of the value to accumulate, in terms of the prologue's names
     };
+    // Two values that are the statistics of a softmax over the same elements: values[0] = their maximum, values[1] = the sum of
+    // exp(element - maximum); values[0].expression is the element, one accumulator ({max, sum}) gathers both in one pass.
+    bool onlineSoftmax = false;
     struct Elementwise {
         DataType outputDType = DataType::FP32;
         std::string expression;  // storage-typed C expression of the element to store, in terms of the prologue's names
