@@ -251,6 +251,21 @@ class Outputs {
     PhysicalOutputs physicalOutputs() const;
     static Outputs fromPhysicalOutputs(PhysicalOutputs physicalOutputs);
 
+    // Outputs that take, name by name, the then-branch's value where `predicate` (a single element, read on the device at every
+    // run) is nonzero and the else-branch's value otherwise (reference: Expression.h:474-483, Expression.cpp:5342-5390 there).
+    // The reference runs one branch through a conditional graph node; this build evaluates both branches and selects element
+    // by element (`where(predicate != 0, then, else)`), which gives the same outputs for these side-effect-free expressions -
+    // values of the branch not taken, NaNs included, never reach an output - usually inside one fused kernel, and the same
+    // gradients (a gradient flows into the branch that was taken).  The result is an ordinary Outputs: isConditional() is false
+    // and a stamped plan shows the stages of the selection, not a Conditional stage.
+    static Outputs conditional(const Expression& predicate, const Outputs& then_outputs, const Outputs& else_outputs);
+    static Outputs ifElse(const Expression& predicate, const Outputs& then_outputs, const Outputs& else_outputs) {
+        return conditional(predicate, then_outputs, else_outputs);
+    }
+    static Outputs ifElifElse(const Expression& predicate, const Outputs& then_outputs, const std::vector<std::pair<Expression, Outputs>>& elif_branches,
+                              const Outputs& else_outputs);
+    bool isConditional() const { return false; }
+
    private:
     Outputs(std::shared_ptr<PhysicalExpression> expr, std::vector<NamedOutput> outputs) : expr(std::move(expr)), outputs(std::move(outputs)) {}
     std::shared_ptr<PhysicalExpression> expr;
@@ -528,6 +543,7 @@ class Expression {
     static bool isTernaryOp(ExprOp op);
 
    private:
+    friend class Outputs;
     Expression(std::shared_ptr<PhysicalExpression> expr, uint32_t nodeIndex) : expr(std::move(expr)), nodeIndex(nodeIndex) {}
     static Expression unaryOp(const Expression& input, ExprOp op);
     static Expression binaryOp(const Expression& lhs, const Expression& rhs, ExprOp op);

@@ -258,6 +258,10 @@ int thor_expr_canonical(thor_expr_t expr, char* buffer, size_t capacity, size_t*
 /* Expression::outputs({{name, expr}, ...}) */
 thor_outputs_t thor_outputs_create(const char* const* names, const thor_expr_t* exprs, int count);
 void thor_outputs_destroy(thor_outputs_t outputs);
+/* Outputs::ifElse / ifElifElse (Expression.h:474-483 there): name by name the then-branch's value where the single-element predicate is
+ * nonzero, else the next branch whose predicate is nonzero, else the else-branch.  num_elif may be 0 (plain if / else). */
+thor_outputs_t thor_outputs_conditional(thor_expr_t predicate, thor_outputs_t then_outputs, const thor_expr_t* elif_predicates,
+                                        const thor_outputs_t* elif_outputs, int num_elif, thor_outputs_t else_outputs);
 
 /* ---- FusedEquation (Utilities/Expression/FusedEquation.h:574-632) --------------------------------------------------------- */
 thor_fused_equation_t thor_fused_equation_compile(thor_outputs_t outputs, int device_num);

@@ -965,6 +965,18 @@ static void boundaryShorthandsAndSubstitution() {
     options.compute_dtype = DataType::FP32;
     options.allow_in_place_materialization = true;  // a permission: accepted
     (void)x.rotaryPositionEmbedding(options);
+    // conditional outputs: same branch names in the same order, at least one elif for ifElifElse (Expression.cpp:5342-5390 there)
+    const Expression selector = Expression::input("selector");
+    const Outputs thenOutputs = Expression::outputs({{"y", x + 10.0}}), elseOutputs = Expression::outputs({{"y", x + 40.0}});
+    const Outputs chosen = Outputs::ifElse(selector > 0.0, thenOutputs, elseOutputs);
+    CHECK(!chosen.isConditional() && chosen.namedOutputs().size() == 1 && chosen.namedOutputs()[0].name == "y");
+    CHECK(chosen.expression()->nodes[chosen.namedOutputs()[0].node_idx].op == ExprOp::WHERE);
+    CHECK(throwsAs<std::runtime_error>([&] { (void)Outputs::ifElse(selector > 0.0, thenOutputs, Expression::outputs({{"z", x}})); }));
+    CHECK(throwsAs<std::runtime_error>([&] { (void)Outputs::ifElifElse(selector > 2.0, thenOutputs, {}, elseOutputs); }));
+    const Outputs ladder = Outputs::ifElifElse(selector > 2.0, thenOutputs, {{selector > 1.0, Expression::outputs({{"y", x + 20.0}})}}, elseOutputs);
+    CHECK(FusedEquation::compile(ladder.physicalOutputs(), 0).getOutputShapes({{"x", Tensor(cpuPlacement, TensorDescriptor(DataType::FP32, {4, 5}))},
+                                                                               {"selector", Tensor(cpuPlacement, TensorDescriptor(DataType::FP32, {1}))}})
+              .at("y") == std::vector<uint64_t>({4, 5}));
 }
 
 static void boundaryRequestedShapesAndSubstitutionExecution(Stream& stream) {

@@ -374,3 +374,60 @@ def test_kernels_are_cached_across_stamps_and_sizes(gpu):
     a = copy_numpy_to_gpu(np.ones(8, np.float32), stream, DataType.fp32)
     eq2.stamp({"p": a, "q": a}, stream).run()
     assert ph.compiled_kernel_count() - before <= 1
+
+
+# ---- conditional outputs (Outputs::ifElse / ifElifElse): the reference's cases, test_expression_outputs.py:625-760 there ---------------
+@pytest.fixture(scope="module")
+def stream(gpu):
+    return ph.Stream(0)
+
+
+def _scalar(value, stream):
+    return copy_numpy_to_gpu(np.array([value], np.float32), stream, DataType.fp32)
+
+
+def test_if_elif_else_takes_the_first_matching_branch(stream):
+    x, selector = ex.input("x"), ex.input("selector")
+    conditional = ex.if_elif_else(selector > 2.0, ex.outputs({"y": x * 10.0}),
+                                  [(selector > 1.0, ex.outputs({"y": x * 20.0})), (selector > 0.0, ex.outputs({"y": x * 30.0}))],
+                                  ex.outputs({"y": x * 40.0}))
+    equation = conditional.compile(device_num=0)
+    x_gpu = copy_numpy_to_gpu(np.array([1.0, 2.0], np.float32), stream, DataType.fp32)
+    selector_gpu = _scalar(0.0, stream)
+    plan = equation.stamp({"x": x_gpu, "selector": selector_gpu}, stream)
+    assert plan.stage_kind_names() == ["FusedKernel"]  # every branch and the selection in one kernel
+    for value, expected in [(3.0, [10.0, 20.0]), (2.0, [20.0, 40.0]), (1.0, [30.0, 60.0]), (-1.0, [40.0, 80.0])]:
+        selector_gpu.copy_from_async(_scalar(value, stream), stream)  # the predicate is read on the device at every run
+        plan.run()
+        np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output("y"), stream), np.array(expected, np.float32))
+
+
+def test_if_else_with_a_device_predicate_several_outputs_and_a_poisoned_branch(stream):
+    """Values of the branch that is not taken never reach an output, NaN and infinity included; reductions and several outputs
+    are allowed inside the branches."""
+    x = ex.input("x")
+    predicate = ex.input("predicate_value") > 0.0
+    conditional = ex.if_else(predicate, ex.outputs({"y": x + 10.0, "total": x.reduce_sum(axis=0)}),
+                             ex.outputs({"y": (x - x) / (x - x), "total": x.reduce_max(axis=0) * float("inf")}))
+    equation = conditional.compile(device_num=0)
+    x_gpu = copy_numpy_to_gpu(np.array([1.0, 2.0, 3.0, 4.0], np.float32), stream, DataType.fp32)
+    taken = equation.stamp({"x": x_gpu, "predicate_value": _scalar(1.0, stream)}, stream)
+    taken.run()
+    np.testing.assert_array_equal(copy_gpu_to_numpy(taken.output("y"), stream), np.array([11.0, 12.0, 13.0, 14.0], np.float32))
+    np.testing.assert_array_equal(copy_gpu_to_numpy(taken.output("total"), stream).reshape(-1), np.array([10.0], np.float32))
+    other = equation.stamp({"x": x_gpu, "predicate_value": _scalar(-1.0, stream)}, stream)
+    other.run()
+    assert np.all(np.isnan(copy_gpu_to_numpy(other.output("y"), stream)))
+    assert np.all(np.isinf(copy_gpu_to_numpy(other.output("total"), stream)))
+
+
+def test_the_gradient_of_a_conditional_flows_into_the_branch_that_was_taken(stream):
+    x, predicate_value = ex.input("x"), ex.input("predicate_value")
+    conditional = ex.if_else(predicate_value > 0.0, ex.outputs({"y": x * x}), ex.outputs({"y": x * 3.0}))
+    backward = conditional.compile(device_num=0).compile_backward(["x"], error_input_name="dy")
+    x_gpu = copy_numpy_to_gpu(np.array([-2.0, -1.0, 2.0, 4.0], np.float32), stream, DataType.fp32)
+    dy_gpu = copy_numpy_to_gpu(np.array([1.0, 2.0, 3.0, 4.0], np.float32), stream, DataType.fp32)
+    for value, expected in [(1.0, [-4.0, -4.0, 12.0, 32.0]), (-1.0, [3.0, 6.0, 9.0, 12.0])]:
+        plan = backward.stamp({"x": x_gpu, "predicate_value": _scalar(value, stream), "dy": dy_gpu}, stream)
+        plan.run()
+        np.testing.assert_allclose(copy_gpu_to_numpy(plan.output("x_grad"), stream), np.array(expected, np.float32), rtol=1e-6, atol=1e-6)

@@ -169,3 +169,19 @@ def test_cpu_type_converter_large_buffer_uses_the_thread_partition_and_stays_exa
         np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
         back = ph.convert_type_cpu(got, dst, D.fp32)
         np.testing.assert_array_equal(back.view(np.uint32), oracle.convert(want, int(dst), oracle.FP32).view(np.uint32))
+
+
+def test_conditional_outputs_validate_their_branches_like_the_reference():
+    """Outputs::conditional / ifElifElse argument checks (Expression.cpp:5342-5390 there; test_expression_outputs.py:597-622)."""
+    x, selector = ex.input("x"), ex.input("selector")
+    then_outputs, else_outputs = ex.outputs({"y": x + 10.0}), ex.outputs({"y": x + 40.0})
+    with pytest.raises(RuntimeError, match="requires at least one elif branch"):
+        ex.if_elif_else(selector > 2.0, then_outputs, [], else_outputs)
+    with pytest.raises(RuntimeError, match="same output names in the same order"):
+        ex.if_else(selector > 0.0, then_outputs, ex.outputs({"z": x}))
+    with pytest.raises(RuntimeError, match="same output names in the same order"):
+        ex.if_else(selector > 0.0, ex.outputs({"a": x, "b": x * 2.0}), ex.outputs({"b": x, "a": x}))
+    chained = ex.if_elif_else(selector > 2.0, then_outputs, [(selector > 1.0, ex.outputs({"y": x + 20.0})), (selector > 0.0, ex.outputs({"y": x + 30.0}))],
+                              else_outputs)
+    shape, dtype = chained.compile(0).get_output_shape({"x": cpu([4, 5], D.fp32), "selector": cpu([1], D.fp32)}, "y")
+    assert shape == [4, 5] and dtype == D.fp32

@@ -281,6 +281,30 @@ Outputs Expression::outputs(const std::vector<std::pair<std::string, Expression>
     return Outputs(std::move(merged), std::move(outs));
 }
 
+Outputs Outputs::conditional(const Expression& predicate, const Outputs& then_outputs, const Outputs& else_outputs) {
+    if (then_outputs.outputs.empty() || else_outputs.outputs.empty()) {
+        throw std::runtime_error("Outputs::conditional requires non-empty then and else branches.");
+    }
+    bool sameNames = then_outputs.outputs.size() == else_outputs.outputs.size();
+    for (size_t i = 0; sameNames && i < then_outputs.outputs.size(); ++i) sameNames = then_outputs.outputs[i].name == else_outputs.outputs[i].name;
+    if (!sameNames) throw std::runtime_error("Outputs::conditional requires then/else branches to expose the same output names in the same order.");
+    const Expression taken = predicate.notEqual(Expression(0.0));
+    std::vector<std::pair<std::string, Expression>> selected;
+    for (size_t i = 0; i < then_outputs.outputs.size(); ++i) {
+        const Expression whenTrue(then_outputs.expr, then_outputs.outputs[i].node_idx), whenFalse(else_outputs.expr, else_outputs.outputs[i].node_idx);
+        selected.emplace_back(then_outputs.outputs[i].name, Expression::where(taken, whenTrue, whenFalse));
+    }
+    return Expression::outputs(selected);
+}
+
+Outputs Outputs::ifElifElse(const Expression& predicate, const Outputs& then_outputs, const std::vector<std::pair<Expression, Outputs>>& elif_branches,
+                            const Outputs& else_outputs) {
+    if (elif_branches.empty()) throw std::runtime_error("Outputs::ifElifElse requires at least one elif branch.");
+    Outputs chained = else_outputs;
+    for (auto it = elif_branches.rbegin(); it != elif_branches.rend(); ++it) chained = conditional(it->first, it->second, chained);
+    return conditional(predicate, then_outputs, chained);
+}
+
 Outputs Expression::outputs(std::initializer_list<std::pair<std::string, Expression>> named_exprs) {
     return outputs(std::vector<std::pair<std::string, Expression>>(named_exprs));
 }

@@ -249,6 +249,18 @@ thor_outputs_t thor_outputs_create(const char* const* names, const thor_expr_t* 
         return new thor_outputs{Expression::outputs(named)};)
 }
 void thor_outputs_destroy(thor_outputs_t outputs) { delete outputs; }
+thor_outputs_t thor_outputs_conditional(thor_expr_t predicate, thor_outputs_t then_outputs, const thor_expr_t* elif_predicates,
+                                        const thor_outputs_t* elif_outputs, int num_elif, thor_outputs_t else_outputs) {
+    THOR_CAPI_TRY_PTR(
+        require(predicate, "predicate"); require(then_outputs, "then outputs"); require(else_outputs, "else outputs");
+        if (num_elif <= 0) return new thor_outputs{Outputs::ifElse(predicate->expr, then_outputs->outputs, else_outputs->outputs)};
+        std::vector<std::pair<Expression, Outputs>> branches;
+        for (int i = 0; i < num_elif; ++i) {
+            if (elif_predicates[i] == nullptr || elif_outputs[i] == nullptr) throw std::invalid_argument("NULL elif predicate or outputs");
+            branches.emplace_back(elif_predicates[i]->expr, elif_outputs[i]->outputs);
+        }
+        return new thor_outputs{Outputs::ifElifElse(predicate->expr, then_outputs->outputs, branches, else_outputs->outputs)};)
+}
 
 // ---- FusedEquation ------------------------------------------------------------------------------------------------------------
 thor_fused_equation_t thor_fused_equation_compile(thor_outputs_t outputs, int device_num) {

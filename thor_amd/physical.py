@@ -87,6 +87,7 @@ PROTOTYPES = {
     "thor_expr_unsqueeze": (_vp, [_vp, _u64p, _i]), "thor_expr_squeeze": (_vp, [_vp, _u64p, _i]), "thor_expr_destroy": (None, [_vp]),
     "thor_expr_num_nodes": (_i, [_vp]), "thor_expr_canonical": (_i, [_vp, _cp, _sz, ctypes.POINTER(_sz)]),
     "thor_outputs_create": (_vp, [_cpp, _vpp, _i]), "thor_outputs_destroy": (None, [_vp]),
+    "thor_outputs_conditional": (_vp, [_vp, _vp, _vpp, _vpp, _i, _vp]),
     "thor_fused_equation_compile": (_vp, [_vp, _i]), "thor_fused_equation_destroy": (None, [_vp]),
     "thor_fused_equation_compile_backward": (_vp, [_vp, _cpp, _i, _cpp, _cpp, _i, _i]),
     "thor_fused_equation_num_outputs": (_i, [_vp]), "thor_fused_equation_output_name": (_i, [_vp, _i, _cp, _sz]),
@@ -924,6 +925,20 @@ class Expression:
         return Outputs(named)
 
     @staticmethod
+    def if_else(predicate: "Expression", then_outputs: "Outputs", else_outputs: "Outputs") -> "Outputs":
+        """Outputs that take the then-branch's values where the single-element ``predicate`` is nonzero at run time, the
+        else-branch's otherwise (thor.physical.Expression.if_else; both branches are evaluated here and selected element by element)."""
+        return Outputs._conditional(predicate, then_outputs, [], else_outputs)
+
+    conditional = if_else
+
+    @staticmethod
+    def if_elif_else(predicate: "Expression", then_outputs: "Outputs", elif_branches, else_outputs: "Outputs") -> "Outputs":
+        if not elif_branches:
+            raise RuntimeError("Outputs::ifElifElse requires at least one elif branch.")
+        return Outputs._conditional(predicate, then_outputs, list(elif_branches), else_outputs)
+
+    @staticmethod
     def compile(expr_or_outputs, device_num: int = 0) -> "FusedEquation":
         outputs = expr_or_outputs if isinstance(expr_or_outputs, Outputs) else Outputs({"output": _as_expr(expr_or_outputs)})
         return FusedEquation(_handle(lib().thor_fused_equation_compile(outputs._h, device_num), "Expression.compile"))
@@ -950,6 +965,16 @@ class Outputs:
     def __init__(self, named: Dict[str, Expression]):
         names = list(named.keys())
         self._h = _handle(lib().thor_outputs_create(_names(names), _ptrs([named[n]._h for n in names]), len(names)), "Expression.outputs")
+
+    @staticmethod
+    def _conditional(predicate: Expression, then_outputs: "Outputs", elif_branches, else_outputs: "Outputs") -> "Outputs":
+        out = Outputs.__new__(Outputs)
+        out._h = _handle(lib().thor_outputs_conditional(_as_expr(predicate)._h, then_outputs._h, _ptrs([_as_expr(p)._h for p, _ in elif_branches]),
+                                                        _ptrs([o._h for _, o in elif_branches]), len(elif_branches), else_outputs._h), "Outputs.conditional")
+        return out
+
+    def compile(self, device_num: int = 0) -> "FusedEquation":
+        return Expression.compile(self, device_num)
 
     def __del__(self):
         try:
