@@ -21,7 +21,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E published peak
 # HBM bytes one fp32->fp16 launch over 2^28 elements moves, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs scaled by the
 # same counters' readings for a plain copy kernel of known size (profiles/convert_round_trip_2p28_hbm_traffic.txt).
-MEASURED_TRAFFIC_BYTES_2P28 = 1572374 * 1024
+MEASURED_TRAFFIC_BYTES_2P28 = 1_610_591_764  # 1023.98 MiB fetched + 512.00 MiB written
 BYTES_PER_ELEMENT = 6   # fp32 <-> 16-bit: 4 + 2
 
 

@@ -156,7 +156,7 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
         k.mainKernel = compileKernel(s.str(), "thor_scan_route", r.deviceNum, /*fastContract=*/false);
         std::ostringstream v;
         v << "scan-route " << (r.op == 1 ? "min" : "max") << (r.inclusive ? " inclusive" : " exclusive") << (r.reverse ? " reverse" : "") << " rows" << r.row
-          << " chunk" << chunkElems << " vec" << vec << " threads" << threads << " launches1";
+          << " chunk" << chunkElems << " vec" << vec << " threads" << threads << " launches1 [" << k.mainKernel->kernelName << "]";
         k.variant = v.str();
         return kernels;
     }

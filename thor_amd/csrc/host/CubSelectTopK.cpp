@@ -139,7 +139,8 @@ std::shared_ptr<const CubSelectionKernels> buildSelectKernels(DataType dtype, ui
     k.second = compileKernel(source, "thor_select_offsets", deviceNum, false);
     k.third = compileKernel(source, "thor_select_scatter", deviceNum, false);
     std::ostringstream v;
-    v << "select-flagged word" << dataTypeSizeInBytes(dtype) * 8 << " vec" << vec << " chunks" << k.chunks << "x" << chunkElems << " launches3";
+    v << "select-flagged word" << dataTypeSizeInBytes(dtype) * 8 << " vec" << vec << " chunks" << k.chunks << "x" << chunkElems << " launches3 ["
+      << k.third->kernelName << "]";
     k.variant = v.str();
     return kernels;
 }
@@ -279,7 +280,7 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     sel.fourth = compileKernel(source, "thor_topk_gather", deviceNum, false);
     std::ostringstream v;
     v << "top-k radix-select bits" << keyBytes * 8 << " digits" << sel.digits << " vec" << vec << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys")
-      << " k" << k << " of " << numItems << " launches" << 2 + 2 * sel.digits;
+      << " k" << k << " of " << numItems << " launches" << 2 + 2 * sel.digits << " [" << sel.second->kernelName << "]";
     sel.variant = v.str();
     return kernels;
 }
@@ -306,7 +307,7 @@ std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, u
     sel.first = compileKernel(s.str(), "thor_topk_rows", deviceNum, false);
     std::ostringstream v;
     v << "row top-k radix-select bits" << dataTypeSizeInBytes(dtype) * 8 << " digits" << sel.digits << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of "
-      << segmentSize << " rows" << numSegments << " launches1";
+      << segmentSize << " rows" << numSegments << " launches1 [" << sel.first->kernelName << "]";
     sel.variant = v.str();
     return kernels;
 }
