@@ -489,6 +489,44 @@ def summarize_counters(dbs, bench_json=None):
             print(f"{row['dispatches']:10d} {grid:11d} {row['us']:9.1f} " + " ".join(f"{row.get(n, float('nan')):36.1f}" for n in group) +
                   f"  {_short(kernel, 44)} <- {_line_of(kernel, tags)}")
         print()
+    # Ratios that say where a memory-bound kernel waits.  The *_sum counters add up the L2 channel instances (16 per XCD, 8 XCDs),
+    # so a ratio of two of them is per instance; a level counter divided by its request counter is the mean time a request was
+    # outstanding (Little's law), in L2 clocks.
+    instances = 128.0
+    derived = [
+        ("L2 busy %", lambda r: 100 * r["TCC_BUSY_sum"] / r["TCC_CYCLE_sum"]),
+        ("L2 miss %", lambda r: 100 * r["TCC_MISS_sum"] / (r["TCC_HIT_sum"] + r["TCC_MISS_sum"])),
+        ("rd req", lambda r: r["TCC_EA0_RDREQ_sum"]),
+        ("wr req", lambda r: r["TCC_EA0_WRREQ_sum"]),
+        ("rd latency clk", lambda r: r["TCC_EA0_RDREQ_LEVEL_sum"] / r["TCC_EA0_RDREQ_sum"]),
+        ("rd in flight", lambda r: r["TCC_EA0_RDREQ_LEVEL_sum"] / (r["TCC_CYCLE_sum"] / instances)),
+        ("L2 MHz", lambda r: r["TCC_CYCLE_sum"] / instances / r["us"]),
+        ("rd credit stall %", lambda r: 100 * r["TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum"] / r["TCC_CYCLE_sum"]),
+        ("wr credit stall %", lambda r: 100 * r["TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum"] / r["TCC_CYCLE_sum"]),
+        ("wr req stall %", lambda r: 100 * r["TCC_EA0_WRREQ_STALL_sum"] / r["TCC_CYCLE_sum"]),
+        ("tag stall %", lambda r: 100 * r["TCC_TAG_STALL_sum"] / r["TCC_CYCLE_sum"]),
+        ("wave wait %", lambda r: 100 * r["SQ_WAIT_INST_ANY"] / r["SQ_WAVE_CYCLES"]),
+    ]
+    usable = []
+    for title, ratio in derived:
+        try:
+            ratio(max(table.values(), key=lambda r: r["us"]))
+            usable.append((title, ratio))
+        except (KeyError, ZeroDivisionError):
+            pass
+    if usable:
+        print("derived per dispatch (sums over the 128 L2 channel instances; latency and in-flight counts by Little's law):")
+        print(f"{'grid':>11} {'avg_us':>9} " + " ".join(f"{title:>17s}" for title, _ in usable) + "  kernel <- bench line")
+        for (kernel, grid), row in sorted(table.items(), key=lambda item: -item[1]["us"]):
+            if row["us"] < 15.0:
+                continue
+            cells = []
+            for _, ratio in usable:
+                try:
+                    cells.append(f"{ratio(row):17.1f}")
+                except (KeyError, ZeroDivisionError):
+                    cells.append(f"{'-':>17s}")
+            print(f"{grid:11d} {row['us']:9.1f} " + " ".join(cells) + f"  {_short(kernel, 44)} <- {_line_of(kernel, tags)}")
 
 
 def main():
