@@ -249,9 +249,11 @@ static int runAll() {
                 const std::unordered_map<std::string, Tensor> inputs{{"x.values", Tensor(gpuPlacement, TensorDescriptor(dtype, dims))},
                                                                     {"x.offsets", Tensor(gpuPlacement, TensorDescriptor(offsetsType, {201}))}};
                 const std::string tag = std::string("ragged ") + dtypeName + " E=" + std::to_string(elements) + (offsetsType == DataType::UINT64 ? " u64 " : " u32 ");
-                stampOne(tag + "softmax", r.segment_softmax().getValues(), inputs, stream, "SegmentedReduction,FusedReduction,SegmentedBroadcast,FusedKernel");
-                stampOne(tag + "log softmax", r.segment_log_softmax().getValues(), inputs, stream,
-                         "SegmentedReduction,FusedReduction,SegmentedBroadcast,FusedKernel");
+                // fp32 values: maximum and sum of exponentials come out of one pass over the values
+                const char* softmaxStages = dtype == DataType::FP32 ? "FusedReduction,SegmentedBroadcast,FusedKernel"
+                                                                    : "SegmentedReduction,FusedReduction,SegmentedBroadcast,FusedKernel";
+                stampOne(tag + "softmax", r.segment_softmax().getValues(), inputs, stream, softmaxStages);
+                stampOne(tag + "log softmax", r.segment_log_softmax().getValues(), inputs, stream, softmaxStages);
                 stampOne(tag + "mean", r.segment_mean(), inputs, stream, "SegmentedReduction");
                 {
                     std::vector<uint64_t> perSegment{200};

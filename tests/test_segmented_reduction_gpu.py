@@ -129,6 +129,62 @@ def test_random_ragged_partitions_against_numpy(stream, shape, segments, dtype):
                 np.testing.assert_array_equal(got[b], (offsets[b] + winner) * trailing + np.arange(trailing), err_msg=f"{name} segment {b}")
 
 
+def awkward_offsets(rows):
+    """Partitions that put every case of the segment kernels side by side: empty segments at position 0, at multiples of the
+    lane ranges and chunks (16, 64, 256 rows), runs of one-row segments, a segment that spans many chunks, rows after the
+    last segment."""
+    cuts = [0, 0, 0, 1, 2, 3, 3, 16, 16, 40, 64, 64, 64, 100, 256, 256, 300, 301, 302, 303, 512, 1800, 1800, 2047, 2048, 2048, 2600]
+    cuts = [c for c in cuts if c <= rows]
+    return np.array(cuts + [min(rows, 2900)] * 3, dtype=np.int64)
+
+
+SEGMENT_KERNELS = [("teams", {}), ("rows", {}), ("rows", {"THOR_SEGMENT_THREADS": "64"}),
+                   ("rows", {"THOR_SEGMENT_GROUP": "16", "THOR_SEGMENT_BATCH": "8"}), ("rows", {"THOR_SEGMENT_GROUP": "2", "THOR_SEGMENT_THREADS": "128"})]
+
+
+@pytest.mark.parametrize("kernel,switches", SEGMENT_KERNELS, ids=[k + "".join(f"-{n[13:].lower()}{v}" for n, v in e.items()) for k, e in SEGMENT_KERNELS])
+@pytest.mark.parametrize("shape,dtype", [((3000, 64), DataType.fp32), ((3000, 200), DataType.fp16), ((2100, 3), DataType.fp32), ((3000, 512), DataType.bf16)],
+                         ids=["3000x64-fp32", "3000x200-fp16", "2100x3-fp32", "3000x512-bf16"])
+def test_both_segment_kernels_on_awkward_partitions(stream, monkeypatch, kernel, switches, shape, dtype):
+    """The planner picks between two kernels (segments dealt out to teams of lanes, rows dealt out to lanes) by the shape; the
+    tuning switches force each of them, and other block sizes and walking groups, on the same partitions."""
+    monkeypatch.setenv("THOR_SEGMENT_KERNEL", kernel)
+    for name, value in switches.items():
+        monkeypatch.setenv(name, value)
+    rng = np.random.default_rng(shape[1])
+    x = to_storage(rng.standard_normal(shape).astype(np.float32), dtype)
+    x[5, 0] = x[1900, 1] = to_storage(np.array([np.nan], np.float32), dtype)[0]
+    xf = from_storage(x, dtype).astype(np.float64)
+    offsets = awkward_offsets(shape[0])
+    tx = copy_numpy_to_gpu(x, stream, dtype)
+    for offsets_dtype in (DataType.uint32, DataType.uint64):
+        toff = upload_offsets(offsets, stream, offsets_dtype)
+        lengths = np.diff(offsets).reshape(-1, 1)
+        for name, op in VALUE_OPS.items():
+            stamped = ph.CubSegmentedReduction(op, DataType.fp32).stamp(tx, toff, stream)
+            assert ("by_rows" if kernel == "rows" else "by_teams") in stamped.get_kernel_variant()
+            stamped.run()
+            got = gpu_to_f32(stamped.get_output_tensor(), stream).astype(np.float64)
+            want = segment_reference(xf, offsets, name)
+            if name in ("Min", "Max"):
+                np.testing.assert_array_equal(got, want, err_msg=f"{name} {stamped.get_kernel_variant()}")
+            else:
+                absolute = segment_reference(np.abs(np.nan_to_num(xf)), offsets, "Sum") / (np.maximum(lengths, 1) if name == "Mean" else 1)
+                assert np.array_equal(np.isnan(got), np.isnan(want)), f"{name} {stamped.get_kernel_variant()}"
+                assert np.all(np.isnan(want) | (np.abs(got - want) <= 1e-5 * absolute + 1e-30)), f"{name} {stamped.get_kernel_variant()}"
+        for name, op in ARG_OPS.items():
+            stamped = ph.CubSegmentedArgReduction(op).stamp(tx, toff, stream)
+            stamped.run()
+            got = copy_gpu_to_numpy(stamped.get_index_output_tensor(), stream).reshape(len(offsets) - 1, shape[1])
+            for b in range(len(offsets) - 1):
+                rows = xf[offsets[b]:offsets[b + 1]]
+                if rows.shape[0] == 0:
+                    assert np.all(got[b] == np.iinfo(np.uint64).max), f"{name} empty segment {b}"
+                else:
+                    winner = rows.argmin(axis=0) if name == "ArgMin" else rows.argmax(axis=0)  # numpy: the first NaN wins, else the first best
+                    np.testing.assert_array_equal(got[b], (offsets[b] + winner) * shape[1] + np.arange(shape[1]), err_msg=f"{name} segment {b} {stamped.get_kernel_variant()}")
+
+
 def test_offsets_are_read_at_run_time_and_outputs_are_reused(stream):
     """CubOffsetSegmentedReductionTest.cpp:239-295: runtime offsets are not inspected by the stamp; a stamped reduction follows the
     partition that is in the offsets tensor when it runs."""

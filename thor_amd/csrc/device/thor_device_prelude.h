@@ -281,6 +281,28 @@ struct OnlineSoftmaxAcc {
         s = rises ? s * e + 1.0f : s + e;
         m = MaxOp::combine(m, x);
     }
+    // N elements at once (-inf marks "no element"): their maximum, then N independent base-2 hardware exponentials of
+    // (x - maximum) * log2(e), then one merge.  The difference is formed before the scaling, so an exponent t carries a
+    // relative error of 2^-24 and the term 2^t one of |t| * 4e-8 plus the instruction's own ulp: terms far below the
+    // maximum are the inexact ones, and x * e^-x <= 1 / e bounds what they add to the sum's error at 2.2e-8 each.
+    template <int N>
+    __device__ __forceinline__ void addMany(const float (&x)[N]) {
+        constexpr float kLog2e = 1.44269504f;
+        float top = x[0];
+#pragma unroll
+        for (int u = 1; u < N; ++u) top = __builtin_fmaxf(top, x[u]);  // ignores NaNs: they come back through the sum
+        const float base = top == -__builtin_inff() ? 0.0f : top;      // all -inf: every term is 2^-inf = 0
+        float sum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < N; ++u) sum += __builtin_amdgcn_exp2f((x[u] - base) * kLog2e);
+        // a NaN sum: some x was NaN (then the maximum is NaN as well), or the maximum is +inf (inf - inf)
+        if (sum != sum && top != __builtin_inff()) top = __builtin_nanf("");
+        // merge {top, sum}: both sides rescaled to the common maximum the same way
+        const float joint = MaxOp::combine(m, top);
+        const float anchor = joint == -__builtin_inff() ? 0.0f : joint;
+        s = s * __builtin_amdgcn_exp2f((m - anchor) * kLog2e) + sum * __builtin_amdgcn_exp2f((top - anchor) * kLog2e);
+        m = joint;
+    }
     __device__ __forceinline__ static float scaleTo(float from, float to) { return from == -__builtin_inff() ? 0.0f : expf(from - to); }
     __device__ __forceinline__ void merge(const OnlineSoftmaxAcc& o) {
         const float top = MaxOp::combine(m, o.m);

@@ -652,6 +652,243 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
     }
 }
 
+// The same chunks, partials and finishing launch with the work dealt out by rows instead of by segments: thread
+// (row lane, column) owns kBatch consecutive rows of the chunk and issues all of their loads before it knows where the
+// segments lie, so the data in flight depends on neither the partition nor the offsets' latency, and every thread does the same
+// amount of work whatever the lengths are.  The chunk's offsets are staged in LDS meanwhile.  A thread then walks its
+// rows run by run (a run = the rows of one segment inside the thread's range):
+//   * a segment that begins and ends inside the range is finalised and stored by the thread itself;
+//   * the first run, when its segment began before the range, is parked as the thread's `head`; the last run, when its
+//     segment goes on after the range, as its `tail` (a range in the middle of a long segment has only a tail);
+//   * one row of threads then goes over the row lanes in order, folding tails into heads: segments that end here are stored
+//     (or go to the chunk's head partial when they began in an earlier chunk), what is left is the chunk's tail partial.
+// Empty segments are stored (identity) by the thread that owns the row before their position; those at position 0 by the
+// first thread of the first chunk.  Rows outside every segment are skipped.  Meant for segments of kBatch rows or more on
+// average: the rows are walked kWalkGroup at a time, and a group is walked once per segment that touches it.  (Resident
+// blocks that stride over the chunks measured slower than one block per chunk: a block's loads, walk and fold do not overlap.)
+// Cfg as for reduceSegments; kChunkRows == kThreads / kLanesX * kBatch.
+template <typename Cfg>
+__device__ __forceinline__ void reduceSegmentsByRows(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* workspace, float scale,
+                                                     const typename Cfg::OffsetT* offsets) {
+    typedef typename Cfg::IndexT IndexT;
+    typedef typename Cfg::Acc Acc;
+    typedef SegmentWorkspace<Cfg> Workspace;
+    constexpr u64 kColumnsPerRow = Cfg::kD / Cfg::kVec;
+    constexpr int kBatch = Cfg::kBatch;
+    constexpr int kGroup = kBatch < Cfg::kWalkGroup ? kBatch : Cfg::kWalkGroup;  // rows walked together: a run costs a pass over the groups it touches
+    constexpr int kRowLanes = Cfg::kThreads / Cfg::kLanesX;
+    constexpr int kWindow = Cfg::kThreads;  // offsets staged per chunk: kWindow + 1
+    constexpr u64 kNone = ~(u64)0;
+    static_assert(Cfg::kChunkRows == (u64)kRowLanes * kBatch, "a chunk is one range of rows per row lane");
+    __shared__ u64 bounds[kWindow + 1];
+    __shared__ Acc heads[kRowLanes * Cfg::kLanesX * Cfg::kVec];
+    __shared__ Acc tails[kRowLanes * Cfg::kLanesX * Cfg::kVec];
+    __shared__ u64 headSegment[kRowLanes];
+    __shared__ u64 tailSegment[kRowLanes];
+
+    const int lx = threadIdx.x % Cfg::kLanesX;
+    const int rowLane = threadIdx.x / Cfg::kLanesX;
+    const int slot = (rowLane * Cfg::kLanesX + lx) * Cfg::kVec;
+
+    {
+        const u64 chunk = blockIdx.x / Cfg::kColumnTiles, tile = blockIdx.x % Cfg::kColumnTiles;
+        const u64 cBegin = chunk * Cfg::kChunkRows;
+        const u64 cEnd = cBegin + Cfg::kChunkRows < Cfg::kRows ? cBegin + Cfg::kChunkRows : Cfg::kRows;
+        const u64 column = tile * Cfg::kLanesX + lx;
+        const bool columnLive = column < kColumnsPerRow;
+        const u64 columnOffset = (columnLive ? column : 0) * Cfg::kVec;  // dead lanes read column 0 and store nothing
+        const u64 rowBegin = cBegin + (u64)rowLane * kBatch;
+        const u64 rowEnd = rowBegin + kBatch < cEnd ? rowBegin + kBatch : cEnd;
+        const int liveRows = rowEnd > rowBegin ? (int)(rowEnd - rowBegin) : 0;
+
+        // every load of the thread, before anything that depends on the offsets
+        typename Cfg::Loaded x[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            if (u < liveRows) Cfg::load(src, (rowBegin + (u64)u) * Cfg::kD + columnOffset, x[u]);
+        }
+
+        u64 sLo = 0, sEnd = Cfg::kSegments;
+        if (Cfg::kChunks > 1) {
+            constexpr u64 kStraddles = (u64)1 << 63;
+            sLo = Workspace::firstSegment(workspace)[chunk] & ~kStraddles;
+            if (sLo > Cfg::kSegments) sLo = Cfg::kSegments;
+            if (chunk + 1 < Cfg::kChunks) {
+                const u64 entry = Workspace::firstSegment(workspace)[chunk + 1];
+                sEnd = (entry & ~kStraddles) + (entry >> 63);
+                if (sEnd > Cfg::kSegments) sEnd = Cfg::kSegments;
+            }
+        }
+        for (int i = threadIdx.x; i <= kWindow; i += Cfg::kThreads) {
+            const u64 at = sLo + (u64)i;
+            bounds[i] = segmentOffset<Cfg>(offsets, at < Cfg::kSegments ? at : Cfg::kSegments);
+        }
+        __syncthreads();
+        auto bound = [&](u64 at) -> u64 {  // offsets[at], clamped; at <= kSegments
+            return at - sLo <= (u64)kWindow ? bounds[at - sLo] : segmentOffset<Cfg>(offsets, at);
+        };
+
+        // the first segment that ends after the range's first row (kSegments when none does)
+        u64 s = sLo;
+        {
+            u64 hi = sEnd;
+            while (s < hi) {
+                const u64 mid = (s + hi) / 2;
+                if (bound(mid + 1) > rowBegin) hi = mid; else s = mid + 1;
+            }
+        }
+        auto storeEmpty = [&](u64 segment) {
+            if (!columnLive) return;
+#pragma unroll
+            for (int k = 0; k < Cfg::kVec; ++k) {
+                Acc identity;
+                identity.reset();
+                Cfg::store(identity, segment * Cfg::kD + column * Cfg::kVec + k, out, scale, 0.0f);
+            }
+        };
+        if (liveRows > 0 && rowBegin == 0) {
+            for (u64 e = 0; e < s; ++e) storeEmpty(e);  // empty segments at position 0 have no row before them
+        }
+
+        u64 myHead = kNone, myTail = kNone;
+        if (liveRows > 0) {
+            Acc acc[Cfg::kVec];
+            typename Cfg::Kept kept[Cfg::kVec];
+            u64 first = 0, last = 0;  // rows of segment s
+            auto enter = [&]() {
+                first = bound(s);
+                last = bound(s + 1);
+#pragma unroll
+                for (int k = 0; k < Cfg::kVec; ++k) {
+                    Cfg::loadKept(src, s * Cfg::kD + columnOffset + k, kept[k]);
+                    acc[k].reset();
+                }
+            };
+            if (s < Cfg::kSegments) enter();
+#pragma unroll
+            for (int g = 0; g < kBatch; g += kGroup) {
+                if (g < liveRows) {
+                    const u64 groupEnd = rowBegin + g + kGroup < rowEnd ? rowBegin + g + kGroup : rowEnd;
+                    while (s < Cfg::kSegments && first < groupEnd) {
+                        const int lo = first > rowBegin ? (int)(first - rowBegin) : 0;
+                        const int hi = last < groupEnd ? (last > rowBegin ? (int)(last - rowBegin) : 0) : (int)(groupEnd - rowBegin);
+                        if constexpr (Cfg::kOnlineSoftmax) {
+                            // the rows of the run at once: their maximum first, then independent exponentials (rows outside
+                            // the run count as -inf and add nothing), one merge into the running pair
+                            float v[kGroup][Cfg::kVec];
+#pragma unroll
+                            for (int u = g; u < g + kGroup; ++u) {
+                                const bool inRun = u >= lo && u < hi;
+#pragma unroll
+                                for (int k = 0; k < Cfg::kVec; ++k) v[u - g][k] = inRun ? Cfg::valueOne(x[u], src, kept[k], k) : -__builtin_inff();
+                            }
+#pragma unroll
+                            for (int k = 0; k < Cfg::kVec; ++k) {
+                                float values[kGroup];
+#pragma unroll
+                                for (int u = 0; u < kGroup; ++u) values[u] = v[u][k];
+                                acc[k].template addMany<kGroup>(values);
+                            }
+                        } else {
+#pragma unroll
+                            for (int u = g; u < g + kGroup; ++u) {
+                                if (u >= lo && u < hi) {
+                                    const IndexT row = (IndexT)(rowBegin + (u64)u);
+#pragma unroll
+                                    for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k], x[u], src, kept[k], k, row);
+                                }
+                            }
+                        }
+                        if (last > groupEnd) break;  // goes on after these rows
+                        if (first < rowBegin) {      // began before the range and ends in it
+                            myHead = s;
+#pragma unroll
+                            for (int k = 0; k < Cfg::kVec; ++k) heads[slot + k] = acc[k];
+                        } else if (columnLive) {
+#pragma unroll
+                            for (int k = 0; k < Cfg::kVec; ++k)
+                                Cfg::store(acc[k], s * Cfg::kD + column * Cfg::kVec + k, out, scale, (float)(last > first ? last - first : 0));
+                        }
+                        ++s;
+                        if (s < Cfg::kSegments) enter();
+                    }
+                }
+            }
+            if (s < Cfg::kSegments && first < rowEnd && last > rowEnd) {
+                myTail = s;  // goes on after the range
+#pragma unroll
+                for (int k = 0; k < Cfg::kVec; ++k) tails[slot + k] = acc[k];
+            } else {
+                // nothing goes on past the range: the empty segments at the position after its last row belong to this thread
+                while (s < Cfg::kSegments && bound(s) == rowEnd && bound(s + 1) == rowEnd) {
+                    storeEmpty(s);
+                    ++s;
+                }
+            }
+        }
+        if (lx == 0) {
+            headSegment[rowLane] = myHead;
+            tailSegment[rowLane] = myTail;
+        }
+        __syncthreads();
+
+        // one row of threads folds the parked runs in row order
+        if (rowLane == 0) {
+            Acc running[Cfg::kVec];
+            u64 runningSegment = kNone;
+#pragma unroll
+            for (int k = 0; k < Cfg::kVec; ++k) running[k].reset();
+            for (int j = 0; j < kRowLanes; ++j) {
+                const int parked = (j * Cfg::kLanesX + lx) * Cfg::kVec;
+                const u64 ended = headSegment[j];
+                if (ended != kNone) {
+                    const u64 first = bound(ended), last = bound(ended + 1);
+#pragma unroll
+                    for (int k = 0; k < Cfg::kVec; ++k) {
+                        Acc total = heads[parked + k];
+                        if (runningSegment == ended) {
+                            total = running[k];
+                            total.merge(heads[parked + k]);
+                        }
+                        if (columnLive) {
+                            const u64 d = column * Cfg::kVec + k;
+                            if (first < cBegin) {
+                                total.storePartial(workspace, (chunk * 2 + 0) * Cfg::kD + d, Workspace::kPartialSlots);
+                            } else {
+                                Cfg::store(total, ended * Cfg::kD + d, out, scale, (float)(last > first ? last - first : 0));
+                            }
+                        }
+                        running[k].reset();
+                    }
+                    runningSegment = kNone;
+                }
+                const u64 open = tailSegment[j];
+                if (open != kNone) {
+#pragma unroll
+                    for (int k = 0; k < Cfg::kVec; ++k) {
+                        if (runningSegment == open) {
+                            running[k].merge(tails[parked + k]);
+                        } else {
+                            running[k] = tails[parked + k];
+                        }
+                    }
+                    runningSegment = open;
+                }
+            }
+            bool holdsTail = false;
+            if (runningSegment != kNone) {
+                holdsTail = bound(runningSegment) >= cBegin;
+                if (columnLive) {
+#pragma unroll
+                    for (int k = 0; k < Cfg::kVec; ++k)
+                        running[k].storePartial(workspace, (chunk * 2 + (holdsTail ? 1 : 0)) * Cfg::kD + column * Cfg::kVec + k, Workspace::kPartialSlots);
+                }
+            }
+            if (Cfg::kChunks > 1 && tile == 0 && lx == 0) Workspace::tails(workspace)[chunk] = holdsTail ? runningSegment : kNone;
+        }
+    }
+}
+
 // Last launch: block (c, column tile) finishes the segment whose tail chunk c holds, if any: tail[c] and the heads of the
 // chunks the segment runs on into, spread over the block's kFinishThreads / kFinishLanes row lanes.  The mean's divisor is
 // the row count the offsets hold now.  kFinishLanes = columns (single trailing elements) per block, a power of two <= 64.

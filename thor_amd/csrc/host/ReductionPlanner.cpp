@@ -173,7 +173,8 @@ std::string ReductionShape::describe() const {
             if (transposeRows > 0) out << ",transposed_store=" << transposeRows;
             break;
         case Kernel::Segments:
-            out << "segments(lanes_x=" << threadsPerRow << ",rows_in_flight=" << unroll << ",chunk_rows=" << chunkRows << ",min_team=" << minTeam;
+            out << "segments(" << (segmentsByRows ? "by_rows," : "by_teams,") << "lanes_x=" << threadsPerRow << ",rows_in_flight=" << unroll << ",chunk_rows=" << chunkRows;
+            if (!segmentsByRows) out << ",min_team=" << minTeam;
             break;
         case Kernel::Strided:
             out << "strided(kept_rank=" << keptDims.size() << ",reduced_rank=" << reducedDims.size() << ",split=" << split;
@@ -268,6 +269,41 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         if (const char* env = std::getenv("THOR_SEGMENT_MIN_TEAM")) {  // tuning switch: threads of the smallest team
             const uint64_t requested = static_cast<uint64_t>(std::atol(env));
             if (requested >= lanesX && requested <= 256 && (requested & (requested - 1)) == 0) shape.minTeam = static_cast<int>(requested);
+        }
+        // Work dealt out by rows (every lane owns `unroll` consecutive rows and loads them before it looks at the offsets)
+        // when a row lane reads whole cache lines and segments are long enough that most ranges hold one or two of them:
+        // log-normal segments of 64 rows x 64 fp32 on average: see the measurements beside the kernel's bench lines.
+        const bool wholeLines = lanesX * shape.vec * elementBytes >= 128;
+        uint64_t vectorSources = 0;
+        for (const ReductionKernelRequest::Source& source : request.sources) vectorSources += source.kind == ReductionKernelRequest::Source::Kind::Vector;
+        vectorSources = std::max<uint64_t>(vectorSources, 1);
+        shape.segmentsByRows = wholeLines && averageRows >= 8;
+        if (const char* env = std::getenv("THOR_SEGMENT_KERNEL")) {  // tuning / test switch: "teams" or "rows"
+            if (std::string(env) == "teams") shape.segmentsByRows = false;
+            if (std::string(env) == "rows") shape.segmentsByRows = true;
+        }
+        if (shape.segmentsByRows) {
+            if (std::getenv("THOR_SEGMENT_BATCH") == nullptr) shape.unroll = averageRows >= 32 ? 16 : 8;
+            // at most 64 registers of rows, and 64 elements per lane in the unrolled walk (fp8 vectors of 16 x 16 rows compile for minutes)
+            while (shape.unroll > 1 && (static_cast<uint64_t>(shape.unroll) * shape.vec * elementBytes * vectorSources > 256 ||
+                                        static_cast<uint64_t>(shape.unroll) * shape.vec > 64))
+                shape.unroll /= 2;
+            // Smaller blocks when the accumulation is longer: the wavefronts of a block meet at two barriers and their walks
+            // differ with the partition.  Log-normal segments of 64 rows x 64 fp32 on average, 256 / 128 / 64 threads:
+            // arg-max 227 / 208 / 250 us, the pair of a one-pass softmax 290 / 265 / 255 us, sums 190 / 195 / 202 us.
+            if (request.onlineSoftmax) shape.threads = 64;
+            else if (request.isArg) shape.threads = 128;
+            shape.threads = std::max<int>(shape.threads, static_cast<int>(lanesX));
+            if (const char* env = std::getenv("THOR_SEGMENT_THREADS")) {  // tuning switch: threads per block
+                const uint64_t requested = static_cast<uint64_t>(std::atol(env));
+                if ((requested == 64 || requested == 128 || requested == 256) && requested >= lanesX) shape.threads = static_cast<int>(requested);
+            }
+            shape.chunkRows = (static_cast<uint64_t>(shape.threads) / lanesX) * static_cast<uint64_t>(shape.unroll);
+            shape.chunks = std::max<uint64_t>(ceilDiv(request.segmentedRows, shape.chunkRows), 1);
+            if (const char* env = std::getenv("THOR_SEGMENT_GROUP")) {  // tuning switch: rows walked together
+                const long requested = std::atol(env);
+                if (requested == 1 || requested == 2 || requested == 4 || requested == 8 || requested == 16) shape.walkGroup = static_cast<int>(requested);
+            }
         }
         shape.finishLanes = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(request.trailing)));
         // a segment of average length runs over averageRows / chunkRows chunks, folded by finishThreads / finishLanes row
@@ -528,6 +564,9 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
         for (size_t j = 0; j < values.size(); ++j) s << "            a" << j << ".template loadPartial<DEVICE_WIDE>(base + " << j << " * stride, slot, slots);\n";
         s << "        }\n    };\n";
     }
+    s << "    static constexpr bool kOnlineSoftmax = " << (request.onlineSoftmax ? "true" : "false") << ";\n";
+    s << "    static __device__ __forceinline__ float valueOne(const Loaded& l, const Sources& s, const Kept& kk, int k) {\n" << prologue;
+    s << "        (void)l; (void)s; (void)kk; (void)k;\n        return " << values[0].expression << ";\n    }\n";
     s << "    static __device__ __forceinline__ void accumulateOne(Acc& acc, const Loaded& l, const Sources& s, const Kept& kk, int k, IndexT index) {\n";
     s << prologue;
     if (request.isArg || values.size() == 1 || request.onlineSoftmax) {
@@ -655,9 +694,11 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             s << "    static constexpr u64 kChunkRows = " << shape.chunkRows << "ull;\n";
             s << "    static constexpr u64 kChunks = " << shape.chunks << "ull;\n";
             s << "    static constexpr int kMinTeam = " << shape.minTeam << ";\n";
+            s << "    static constexpr int kWalkGroup = " << shape.walkGroup << ";\n";
             s << "    static constexpr int kFinishLanes = " << shape.finishLanes << ";\n";
             s << "    static constexpr int kFinishThreads = " << shape.finishThreads << ";\n";
-            body = "thor::reduceSegments<gen::Cfg>(src, out, partials, scale, static_cast<const gen::Cfg::OffsetT*>(offsets));";
+            body = shape.segmentsByRows ? "thor::reduceSegmentsByRows<gen::Cfg>(src, out, partials, scale, static_cast<const gen::Cfg::OffsetT*>(offsets));"
+                                        : "thor::reduceSegments<gen::Cfg>(src, out, partials, scale, static_cast<const gen::Cfg::OffsetT*>(offsets));";
             break;
         case ReductionShape::Kernel::Strided: {
             std::vector<uint64_t> rd = shape.reducedDims, rs = shape.reducedStrides;

@@ -92,6 +92,9 @@ struct ReductionShape {
     // block of the finishing launch
     uint64_t chunkRows = 0, chunks = 1;
     int minTeam = 1, finishLanes = 1, finishThreads = 256;
+    // Segments kernel: rows dealt out to lanes (reduceSegmentsByRows) instead of segments dealt out to teams (reduceSegments)
+    bool segmentsByRows = false;
+    int walkGroup = 4;  // reduceSegmentsByRows: rows of a lane's range that are walked together
     std::string describe() const;
 };
 
