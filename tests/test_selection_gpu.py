@@ -216,6 +216,40 @@ def test_top_k_pairs_with_many_equal_keys(stream, dtype, largest):
         check_top_k(keys, dtype, k, largest, got, got_values)
 
 
+@pytest.mark.parametrize("dtype", [d for d in KEY_DTYPES if d not in (DataType.uint8, DataType.int8)], ids=lambda d: d.name)
+@pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
+@pytest.mark.parametrize("region", [None, "1"], ids=["roomy", "overflowing"])
+def test_top_k_over_candidates(stream, monkeypatch, dtype, largest, region):
+    """Long inputs copy the keys that can still be part of the answer during the second pass and finish on those candidates; the
+    switch asks for that on short inputs too.  With one entry per wavefront the candidate regions overflow and the passes over
+    the whole input take over: both ways must give the same answer."""
+    monkeypatch.setenv("THOR_TOPK_CANDIDATES", "1")
+    if region:
+        monkeypatch.setenv("THOR_TOPK_REGION", region)
+    rng = np.random.default_rng(int(dtype) * 3 + largest)
+    for n, k, levels in ((100_003, 1, None), (100_003, 1000, None), (300_001, 4_000, 20), (300_001, 250_000, 20), (65_536, 65_536, None)):
+        keys = random_keys(rng, n, dtype, distinct_levels=levels)
+        got, got_values, variant = run_top_k(keys, dtype, k, largest, stream, pairs=True)
+        assert "candidates(" in variant
+        check_top_k(keys, dtype, k, largest, got, got_values)
+        got, _, _ = run_top_k(keys, dtype, k, largest, stream)
+        check_top_k(keys, dtype, k, largest, got, None)
+
+
+def test_top_k_long_inputs_use_candidates_by_default(stream):
+    rng = np.random.default_rng(77)
+    keys = rng.standard_normal((1 << 21) + 12).astype(np.float32)
+    keys[rng.integers(0, keys.size, 50)] = np.float32(9.5)  # ties at the top
+    for k in (1, 40, 64, 70_000):
+        got, got_values, variant = run_top_k(keys, DataType.fp32, k, True, stream, pairs=True)
+        assert "candidates(" in variant
+        check_top_k(keys, DataType.fp32, k, True, got, got_values)
+    sorted_keys = np.sort(keys)  # every candidate in one stretch of the input
+    for largest in (True, False):
+        got, got_values, _ = run_top_k(sorted_keys, DataType.fp32, 3_000, largest, stream, pairs=True)
+        check_top_k(sorted_keys, DataType.fp32, 3_000, largest, got, got_values)
+
+
 def test_top_k_of_equal_keys_and_k_beyond_the_input(stream):
     keys = np.full(10_000, 7, np.uint32)
     got, got_values, _ = run_top_k(keys, DataType.uint32, 99_999, True, stream, pairs=True)

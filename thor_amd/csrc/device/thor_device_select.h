@@ -219,13 +219,16 @@ __device__ __forceinline__ u32 topkPickBucket(const Bins& bins, u32 numBins, u32
 // ---- device-wide top-k -----------------------------------------------------------------------------------------------------------
 // Cfg: Raw (u8 / u16 / u32 word of the key), kKind, kBits, kLargest, kTotal, kK (already capped at kTotal, > 0), kPairs, kVec (keys
 // per vector load: 16 bytes' worth when the key tensor is aligned and kTotal divides, else 1), kItems (vectors per thread of the
-// gathering pass).  Temporary storage: 2048 histogram words, then the state words below.
+// gathering pass).  Temporary storage: 2048 histogram words, then the eight state words below (then the candidates, see there).
 struct TopkState {
     u32 prefix;     // the digits fixed so far, in place
     u32 remaining;  // the rank (1-based) of the wanted key among the keys that match the prefix
     u32 taken;      // output slots handed out to keys above the threshold
     u32 ties;       // keys equal to the threshold seen so far by the gathering pass
+    u32 overflow;   // candidate regions (below) were too small for this input: the passes over the whole input take over
+    u32 unused[3];
 };
+constexpr int kTopkStateWords = 8;
 
 template <typename Cfg>
 __device__ __forceinline__ void topkInit(u32* temp) {
@@ -236,16 +239,18 @@ __device__ __forceinline__ void topkInit(u32* temp) {
         state->remaining = (u32)Cfg::kK;
         state->taken = 0;
         state->ties = 0;
+        state->overflow = 0;
     }
 }
 
 // Histogram of the `bits`-wide digit at `shift` over the keys whose higher digits equal the prefix.  Blocks stride over the keys
 // in vectors, four vectors of a thread in flight.
 template <typename Cfg>
-__device__ __forceinline__ void topkHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
+__device__ __forceinline__ void topkHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits, u32 fallbackOnly) {
     typedef typename Cfg::Raw Raw;
     constexpr int V = Cfg::kVec, kUnroll = 4;
     __shared__ u32 bins[kTopkMaxBins];
+    if (fallbackOnly && reinterpret_cast<const TopkState*>(temp + kTopkMaxBins)->overflow == 0) return;  // the candidates were counted instead
     const u32 numBins = 1u << bits;
     for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
     __syncthreads();
@@ -298,46 +303,229 @@ __device__ __forceinline__ void topkPick(u32* temp, u32 shift, u32 bits) {
 // one request per wavefront vote cost 0.7 ms at k = 65 536); a block without qualifying keys, the usual case when k is
 // small next to the input, leaves after the count.
 template <typename Cfg>
-__device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
+__device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues,
+                                           u32 fallbackOnly) {
     typedef typename Cfg::Raw Raw;
     constexpr int V = Cfg::kVec, kWaves = Cfg::kThreads / kWave;
     __shared__ u32 waveAbove[kWaves], waveTies[kWaves], bases[2];
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
+    if (fallbackOnly && state->overflow == 0) return;  // the candidates were gathered instead
     const u32 threshold = state->prefix, wantedTies = state->remaining, firstTieSlot = (u32)Cfg::kK - wantedTies;
     constexpr u64 kVectors = Cfg::kTotal / V;
+    constexpr u64 kChunkVectors = (u64)Cfg::kThreads * Cfg::kItems;
+    constexpr u64 kChunks = (kVectors + kChunkVectors - 1) / kChunkVectors;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const u64 lowerLanes = ((u64)1 << lane) - 1;
-    const u64 blockFirst = (u64)blockIdx.x * Cfg::kThreads * Cfg::kItems;
-    Pack<Raw, V> x[Cfg::kItems];
+    for (u64 chunk = blockIdx.x; chunk < kChunks; chunk += gridDim.x) {
+        if (chunk != blockIdx.x) __syncthreads();  // the previous chunk's counts and bases have been read
+        const u64 blockFirst = chunk * kChunkVectors;
+        Pack<Raw, V> x[Cfg::kItems];
 #pragma unroll
-    for (int it = 0; it < Cfg::kItems; ++it) {
-        const u64 v = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x;
-        if (v < kVectors) x[it].loadStream(keys + v * V);
+        for (int it = 0; it < Cfg::kItems; ++it) {
+            const u64 v = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x;
+            if (v < kVectors) x[it].loadStream(keys + v * V);
+        }
+        u32 above = 0, ties = 0;  // of this wavefront
+#pragma unroll
+        for (int it = 0; it < Cfg::kItems; ++it) {
+            const bool live = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x < kVectors;
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                const u32 image = live ? topkImage<Cfg>(x[it].v[k]) : 0u;
+                above += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(live && image > threshold));
+                ties += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(live && image == threshold));
+            }
+        }
+        if (lane == 0) {
+            waveAbove[wave] = above;
+            waveTies[wave] = ties;
+        }
+        __syncthreads();
+        u32 aboveAt = 0, tieAt = 0, blockAbove = 0, blockTies = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            aboveAt += w < wave ? waveAbove[w] : 0u;
+            tieAt += w < wave ? waveTies[w] : 0u;
+            blockAbove += waveAbove[w];
+            blockTies += waveTies[w];
+        }
+        if (blockAbove + blockTies == 0) continue;
+        if (threadIdx.x == 0) {
+            bases[0] = blockAbove ? atomicAdd(&state->taken, blockAbove) : 0u;
+            bases[1] = blockTies ? atomicAdd(&state->ties, blockTies) : 0u;
+        }
+        __syncthreads();
+        aboveAt += bases[0];
+        tieAt += bases[1];
+        if (above + ties == 0) continue;  // nothing in this wavefront
+#pragma unroll
+        for (int it = 0; it < Cfg::kItems; ++it) {
+            const u64 v = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x;
+            const bool live = v < kVectors;
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                const u32 image = live ? topkImage<Cfg>(x[it].v[k]) : 0u;
+                const bool isAbove = live && image > threshold, isTie = live && image == threshold;
+                const u64 aboveVotes = __builtin_amdgcn_ballot_w64(isAbove), tieVotes = __builtin_amdgcn_ballot_w64(isTie);
+                u32 slot = 0xffffffffu;
+                if (isAbove) slot = aboveAt + (u32)__builtin_popcountll(aboveVotes & lowerLanes);
+                if (isTie) {
+                    const u32 rank = tieAt + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+                    if (rank < wantedTies) slot = firstTieSlot + rank;
+                }
+                aboveAt += (u32)__builtin_popcountll(aboveVotes);
+                tieAt += (u32)__builtin_popcountll(tieVotes);
+                if (slot != 0xffffffffu) {
+                    outKeys[slot] = x[it].v[k];
+                    if (Cfg::kPairs) outValues[slot] = values[v * V + k];
+                }
+            }
+        }
     }
-    u32 above = 0, ties = 0;  // of this wavefront
+}
+
+// ---- candidates ------------------------------------------------------------------------------------------------------------------
+// Long inputs are read in full twice instead of once per digit and once more for the output: after the first digit is fixed,
+// the pass that counts the second digit also copies every key whose first digit is at or above the fixed one (the keys that
+// can still be part of the answer: fewer than kK above the bucket plus the bucket itself) into the temporary storage, and the
+// later digits and the output are taken from those candidates.  Every wavefront of the copying pass owns a region of
+// kRegion entries (keys as 32-bit words; for pairs the key's position as well) and counts what it wrote: no wavefront asks
+// another for room.  A region that would overflow (a bucket that holds a large part of the input: many equal keys, k close to
+// kTotal) raises `overflow`; the passes over the candidates then leave at once and the passes over the whole input, launched
+// after them, do the work.
+// Cfg additionally: kCompact, kFirstShift (the shift of the first digit), kRegion, kRegions (wavefronts of the copying
+// pass), kCandidateBlocks.  Temporary storage after the state: kRegions counts, kRegions * kRegion keys, the same number of
+// positions (pairs).
+template <typename Cfg>
+struct TopkCandidates {
+    __device__ __forceinline__ static u32* counts(u32* temp) { return temp + kTopkMaxBins + kTopkStateWords; }
+    __device__ __forceinline__ static u32* keys(u32* temp) { return counts(temp) + Cfg::kRegions; }
+    __device__ __forceinline__ static u32* positions(u32* temp) { return keys(temp) + (u64)Cfg::kRegions * Cfg::kRegion; }
+};
+
+// Launched with kRegions / 4 blocks of 256 threads, after the first digit has been fixed: histogram of the digit at `shift`
+// over the keys that match the first digit, and the candidates of every wavefront into its region.
+template <typename Cfg>
+__device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
+    typedef typename Cfg::Raw Raw;
+    constexpr int V = Cfg::kVec, kUnroll = 4;
+    __shared__ u32 bins[kTopkMaxBins];
+    const u32 numBins = 1u << bits;
+    for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
+    __syncthreads();
+    TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
+    constexpr u32 kFirstDigit = 0xffffffffu << Cfg::kFirstShift;
+    const u32 floorImage = state->prefix & kFirstDigit;  // images at or above it are candidates, images that match it are counted
+    const u32 digitMask = numBins - 1u;
+    const int lane = threadIdx.x % kWave;
+    const u64 lowerLanes = ((u64)1 << lane) - 1;
+    const u32 region = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+    u32* regionKeys = TopkCandidates<Cfg>::keys(temp) + (u64)region * Cfg::kRegion;
+    u32* regionPositions = TopkCandidates<Cfg>::positions(temp) + (u64)region * Cfg::kRegion;
+    u32 cursor = 0;  // candidates of this wavefront so far: the same in every lane that is still in the loop (lane 0 leaves last)
+    constexpr u64 kVectors = Cfg::kTotal / V;
+    const u64 stride = (u64)gridDim.x * 256;
+    for (u64 v0 = (u64)blockIdx.x * 256 + threadIdx.x; v0 < kVectors; v0 += stride * kUnroll) {
+        Pack<Raw, V> x[kUnroll];
 #pragma unroll
-    for (int it = 0; it < Cfg::kItems; ++it) {
-        const bool live = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x < kVectors;
+        for (int u = 0; u < kUnroll; ++u)
+            if (v0 + u * stride < kVectors) x[u].loadStream(keys + (v0 + u * stride) * V);
 #pragma unroll
-        for (int k = 0; k < V; ++k) {
-            const u32 image = live ? topkImage<Cfg>(x[it].v[k]) : 0u;
-            above += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(live && image > threshold));
-            ties += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(live && image == threshold));
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool live = v0 + u * stride < kVectors;
+            u32 image[V];
+            bool any = false;
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                image[k] = live ? topkImage<Cfg>(x[u].v[k]) : 0u;
+                any |= live && image[k] >= floorImage;
+            }
+            if (__builtin_amdgcn_ballot_w64(any) == 0) continue;  // the usual case when k is small next to the input
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                const bool candidate = live && image[k] >= floorImage;
+                const u64 votes = __builtin_amdgcn_ballot_w64(candidate);
+                if (candidate) {
+                    const u32 slot = cursor + (u32)__builtin_popcountll(votes & lowerLanes);
+                    if (slot < Cfg::kRegion) {
+                        regionKeys[slot] = (u32)x[u].v[k];
+                        if (Cfg::kPairs) regionPositions[slot] = (u32)((v0 + u * stride) * V + k);
+                    }
+                    if ((image[k] & kFirstDigit) == floorImage) atomicAdd(&bins[(image[k] >> shift) & digitMask], 1u);
+                }
+                cursor += (u32)__builtin_popcountll(votes);
+            }
         }
     }
     if (lane == 0) {
-        waveAbove[wave] = above;
-        waveTies[wave] = ties;
+        TopkCandidates<Cfg>::counts(temp)[region] = cursor < Cfg::kRegion ? cursor : Cfg::kRegion;
+        if (cursor > Cfg::kRegion) atomicOr(&state->overflow, 1u);
     }
     __syncthreads();
-    u32 aboveAt = 0, tieAt = 0, blockAbove = 0, blockTies = 0;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-        aboveAt += w < wave ? waveAbove[w] : 0u;
-        tieAt += w < wave ? waveTies[w] : 0u;
-        blockAbove += waveAbove[w];
-        blockTies += waveTies[w];
+    for (u32 b = threadIdx.x; b < numBins; b += 256) {
+        const u32 mine = bins[b];
+        if (mine != 0) atomicAdd(&temp[b], mine);
     }
+}
+
+// kCandidateBlocks blocks of 256 threads: histogram of the digit at `shift` over the candidates that match the digits fixed so far.
+template <typename Cfg>
+__device__ __forceinline__ void topkCandidateHistogram(u32* temp, u32 shift, u32 bits) {
+    typedef typename Cfg::Raw Raw;
+    __shared__ u32 bins[kTopkMaxBins];
+    const TopkState* state = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins);
+    if (state->overflow != 0) return;
+    const u32 numBins = 1u << bits;
+    for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
+    __syncthreads();
+    const u32 prefix = state->prefix;
+    const u32 fixedBits = shift + bits >= 32 ? 0u : (0xffffffffu << (shift + bits));
+    const u32 digitMask = numBins - 1u;
+    const int lane = threadIdx.x % kWave;
+    const u32* counts = TopkCandidates<Cfg>::counts(temp);
+    const u32* candidateKeys = TopkCandidates<Cfg>::keys(temp);
+    for (u32 region = blockIdx.x * (256 / kWave) + threadIdx.x / kWave; region < Cfg::kRegions; region += gridDim.x * (256 / kWave)) {
+        const u32 count = counts[region];
+        for (u32 i = lane; i < count; i += kWave) {
+            const u32 image = topkImage<Cfg>((Raw)candidateKeys[(u64)region * Cfg::kRegion + i]);
+            if ((image & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
+        }
+    }
+    __syncthreads();
+    for (u32 b = threadIdx.x; b < numBins; b += 256) {
+        const u32 mine = bins[b];
+        if (mine != 0) atomicAdd(&temp[b], mine);
+    }
+}
+
+// kCandidateBlocks blocks of 256 threads: the output out of the candidates.  Every thread counts the candidates it will write
+// (above the threshold; equal to it), a block scan turns the counts into ranks inside the block, one thread asks for the
+// block's output slots, and a second walk over the same candidates writes them.
+template <typename Cfg>
+__device__ __forceinline__ void topkCandidateGather(const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
+    typedef typename Cfg::Raw Raw;
+    __shared__ u32 lds[8];
+    __shared__ u32 bases[2];
+    TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
+    if (state->overflow != 0) return;
+    const u32 threshold = state->prefix, wantedTies = state->remaining, firstTieSlot = (u32)Cfg::kK - wantedTies;
+    const int lane = threadIdx.x % kWave;
+    const u32* counts = TopkCandidates<Cfg>::counts(temp);
+    const u32* candidateKeys = TopkCandidates<Cfg>::keys(temp);
+    const u32* candidatePositions = TopkCandidates<Cfg>::positions(temp);
+    const u32 firstRegion = blockIdx.x * (256 / kWave) + threadIdx.x / kWave, regionStep = gridDim.x * (256 / kWave);
+    u32 above = 0, ties = 0;
+    for (u32 region = firstRegion; region < Cfg::kRegions; region += regionStep) {
+        const u32 count = counts[region];
+        for (u32 i = lane; i < count; i += kWave) {
+            const u32 image = topkImage<Cfg>((Raw)candidateKeys[(u64)region * Cfg::kRegion + i]);
+            above += image > threshold;
+            ties += image == threshold;
+        }
+    }
+    u32 blockAbove, blockTies;
+    u32 aboveAt = blockExclusiveSum<256>(above, lds, blockAbove);
+    u32 tieAt = blockExclusiveSum<256>(ties, lds, blockTies);
     if (blockAbove + blockTies == 0) return;
     if (threadIdx.x == 0) {
         bases[0] = blockAbove ? atomicAdd(&state->taken, blockAbove) : 0u;
@@ -346,27 +534,21 @@ __device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const 
     __syncthreads();
     aboveAt += bases[0];
     tieAt += bases[1];
-    if (above + ties == 0) return;  // nothing in this wavefront
-#pragma unroll
-    for (int it = 0; it < Cfg::kItems; ++it) {
-        const u64 v = blockFirst + (u64)it * Cfg::kThreads + threadIdx.x;
-        const bool live = v < kVectors;
-#pragma unroll
-        for (int k = 0; k < V; ++k) {
-            const u32 image = live ? topkImage<Cfg>(x[it].v[k]) : 0u;
-            const bool isAbove = live && image > threshold, isTie = live && image == threshold;
-            const u64 aboveVotes = __builtin_amdgcn_ballot_w64(isAbove), tieVotes = __builtin_amdgcn_ballot_w64(isTie);
+    for (u32 region = firstRegion; region < Cfg::kRegions; region += regionStep) {
+        const u32 count = counts[region];
+        for (u32 i = lane; i < count; i += kWave) {
+            const u64 at = (u64)region * Cfg::kRegion + i;
+            const u32 word = candidateKeys[at];
+            const u32 image = topkImage<Cfg>((Raw)word);
             u32 slot = 0xffffffffu;
-            if (isAbove) slot = aboveAt + (u32)__builtin_popcountll(aboveVotes & lowerLanes);
-            if (isTie) {
-                const u32 rank = tieAt + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+            if (image > threshold) slot = aboveAt++;
+            if (image == threshold) {
+                const u32 rank = tieAt++;
                 if (rank < wantedTies) slot = firstTieSlot + rank;
             }
-            aboveAt += (u32)__builtin_popcountll(aboveVotes);
-            tieAt += (u32)__builtin_popcountll(tieVotes);
             if (slot != 0xffffffffu) {
-                outKeys[slot] = x[it].v[k];
-                if (Cfg::kPairs) outValues[slot] = values[v * V + k];
+                outKeys[slot] = (Raw)word;
+                if (Cfg::kPairs) outValues[slot] = values[candidatePositions[at]];
             }
         }
     }

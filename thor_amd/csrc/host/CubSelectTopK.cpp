@@ -9,8 +9,10 @@
 #include "thorhip_numeric_embed.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
 #include <sstream>
+#include <string>
 #include <stdexcept>
 #include <vector>
 
@@ -22,6 +24,9 @@ struct CubSelectionKernels {
     int kind = 0;
     int deviceNum = 0;
     std::shared_ptr<CompiledKernel> first, second, third, fourth;
+    // device-wide top-k over candidates: the copying pass, the histogram and the gathering pass over the candidates
+    std::shared_ptr<CompiledKernel> compact, candidateHistogram, candidateGather;
+    uint32_t candidateBlocks = 0, fallbackGatherBlocks = 0;
     uint64_t chunks = 0;          // blocks of the counting / scattering / gathering launches; rows for kind 2
     uint32_t histogramBlocks = 0;
     uint32_t threads = 256;
@@ -37,7 +42,8 @@ namespace {
 constexpr uint64_t kRowTopKMaxSegment = 8192, kRowTopKMaxK = 8192;
 constexpr uint32_t kSelectThreads = 256, kSelectRounds = 4;
 constexpr uint32_t kGatherThreads = 256, kGatherItems = 8;  // vectors per thread
-constexpr uint32_t kTopKBins = 2048;
+constexpr uint32_t kTopKBins = 2048, kTopKStateWords = 8;
+constexpr uint64_t kTopKCompactMinItems = 1ull << 20;
 
 size_t roundUp(size_t v, size_t to) { return (v + to - 1) / to * to; }
 
@@ -257,30 +263,62 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     sel.chunks = (vectors + chunkVectors - 1) / chunkVectors;
     // enough striding blocks to keep every compute unit busy, few enough that the global histogram sees little contention
     sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, 2048));
-    sel.tempBytes = (kTopKBins + 4) * 4;
+    // Long inputs with more than one digit: the second pass over the input also copies the keys that can still be part of the
+    // answer, and the later digits and the output are taken from those candidates (two reads of the input instead of one per
+    // digit plus one).  Every wavefront of that pass owns room for its share of a 32nd of the input, at least 64 entries.
+    bool compact = sel.digits >= 2 && numItems >= kTopKCompactMinItems && numItems < (1ull << 32);
+    if (const char* env = std::getenv("THOR_TOPK_CANDIDATES")) {  // tuning / test switch: "0" reads the whole input in every pass
+        if (std::string(env) == "0") compact = false;
+        if (std::string(env) == "1") compact = sel.digits >= 2 && numItems < (1ull << 32);
+    }
+    const uint64_t regions = uint64_t(sel.histogramBlocks) * (256 / 64);
+    uint64_t regionEntries = std::max<uint64_t>((numItems / 32 + regions - 1) / regions, 64);
+    if (const char* env = std::getenv("THOR_TOPK_REGION")) regionEntries = std::max<long>(std::atol(env), 1);  // test switch: entries per wavefront
+    sel.candidateBlocks = static_cast<uint32_t>(std::min<uint64_t>((regions + 3) / 4, 128));
+    sel.fallbackGatherBlocks = static_cast<uint32_t>(std::min<uint64_t>(sel.chunks, 2048));
+    sel.tempBytes = (kTopKBins + kTopKStateWords) * 4;
+    if (compact) sel.tempBytes += (regions + regions * regionEntries * (pairs ? 2 : 1)) * 4;
     std::ostringstream s;
     s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
     s << "namespace gen {\nstruct Cfg {\n";
     writeKeyTraits(s, dtype, largest, pairs);
     s << "    static constexpr thor::u64 kTotal = " << numItems << "ull;\n    static constexpr thor::u64 kK = " << k
       << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = " << kGatherThreads
-      << ";\n    static constexpr int kItems = " << kGatherItems << ";\n};\n}  // namespace gen\n";
+      << ";\n    static constexpr int kItems = " << kGatherItems << ";\n    static constexpr bool kCompact = " << (compact ? "true" : "false")
+      << ";\n    static constexpr thor::u32 kFirstShift = " << sel.digitPlan.front().first << "u;\n    static constexpr thor::u32 kRegion = " << regionEntries
+      << "u;\n    static constexpr thor::u32 kRegions = " << regions << "u;\n};\n}  // namespace gen\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_init(thor::u32* temp) { thor::topkInit<gen::Cfg>(temp); }\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
-         "    thor::topkHistogram<gen::Cfg>(keys, temp, shift, bits);\n}\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits, "
+         "thor::u32 fallbackOnly) {\n    thor::topkHistogram<gen::Cfg>(keys, temp, shift, bits, fallbackOnly);\n}\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_pick(thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
          "    thor::topkPick<gen::Cfg>(temp, shift, bits);\n}\n";
     s << "extern \"C\" __global__ __launch_bounds__(" << kGatherThreads
-      << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n"
-         "    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
+      << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues, "
+         "thor::u32 fallbackOnly) {\n    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues, fallbackOnly);\n}\n";
+    if (compact) {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_compact(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
+             "    thor::topkCompact<gen::Cfg>(keys, temp, shift, bits);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_histogram(thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
+             "    thor::topkCandidateHistogram<gen::Cfg>(temp, shift, bits);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_gather(const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, "
+             "thor::u32* outValues) {\n    thor::topkCandidateGather<gen::Cfg>(values, temp, outKeys, outValues);\n}\n";
+    }
     const std::string source = s.str();
     sel.first = compileKernel(source, "thor_topk_init", deviceNum, false);
     sel.second = compileKernel(source, "thor_topk_histogram", deviceNum, false);
     sel.third = compileKernel(source, "thor_topk_pick", deviceNum, false);
     sel.fourth = compileKernel(source, "thor_topk_gather", deviceNum, false);
+    int launches = 2 + 2 * sel.digits;
+    if (compact) {
+        sel.compact = compileKernel(source, "thor_topk_compact", deviceNum, false);
+        sel.candidateHistogram = compileKernel(source, "thor_topk_candidate_histogram", deviceNum, false);
+        sel.candidateGather = compileKernel(source, "thor_topk_candidate_gather", deviceNum, false);
+        launches = 2 + 2 * sel.digits + (sel.digits - 2) + 1;
+    }
     std::ostringstream v;
     v << "top-k radix-select bits" << keyBytes * 8 << " digits" << sel.digits << " vec" << vec << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys")
-      << " k" << k << " of " << numItems << " launches" << 2 + 2 * sel.digits << " [" << sel.second->kernelName << "]";
+      << " k" << k << " of " << numItems << (compact ? " candidates(regions=" + std::to_string(regions) + "x" + std::to_string(regionEntries) + ")" : std::string())
+      << " launches" << launches << " [" << sel.second->kernelName << "]";
     sel.variant = v.str();
     return kernels;
 }
@@ -322,15 +360,33 @@ void launchTopK(const CubSelectionKernels& sel, const void* keysIn, const void* 
     }
     std::vector<void*> initArgs = {&temp};
     sel.first->launch(1, 1, 1, 256, raw, initArgs);
-    for (const std::pair<uint32_t, uint32_t>& digit : sel.digitPlan) {
-        uint32_t shift = digit.first, bits = digit.second;
-        std::vector<void*> histogramArgs = {&keysIn, &temp, &shift, &bits};
-        sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, histogramArgs);
+    uint32_t everyInput = 0, fallbackOnly = 1;
+    for (size_t d = 0; d < sel.digitPlan.size(); ++d) {
+        uint32_t shift = sel.digitPlan[d].first, bits = sel.digitPlan[d].second;
+        if (sel.compact && d == 1) {
+            std::vector<void*> compactArgs = {&keysIn, &temp, &shift, &bits};
+            sel.compact->launch(sel.histogramBlocks, 1, 1, 256, raw, compactArgs);
+        } else if (sel.compact && d > 1) {
+            std::vector<void*> candidateArgs = {&temp, &shift, &bits};
+            sel.candidateHistogram->launch(sel.candidateBlocks, 1, 1, 256, raw, candidateArgs);
+            std::vector<void*> histogramArgs = {&keysIn, &temp, &shift, &bits, &fallbackOnly};
+            sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, histogramArgs);
+        } else {
+            std::vector<void*> histogramArgs = {&keysIn, &temp, &shift, &bits, &everyInput};
+            sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, histogramArgs);
+        }
         std::vector<void*> pickArgs = {&temp, &shift, &bits};
         sel.third->launch(1, 1, 1, 256, raw, pickArgs);
     }
-    std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut};
-    sel.fourth->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, gatherArgs);
+    if (sel.compact) {
+        std::vector<void*> candidateArgs = {&valuesIn, &temp, &keysOut, &valuesOut};
+        sel.candidateGather->launch(sel.candidateBlocks, 1, 1, 256, raw, candidateArgs);
+        std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut, &fallbackOnly};
+        sel.fourth->launch(sel.fallbackGatherBlocks, 1, 1, sel.threads, raw, gatherArgs);
+    } else {
+        std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut, &everyInput};
+        sel.fourth->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, gatherArgs);
+    }
 }
 
 void* tempPointer(const Tensor& temp) { return const_cast<Tensor&>(temp).getMemPtr(); }
