@@ -242,6 +242,29 @@ def test_numpy_broadcasting_semantics(gpu, sa, sb, dtype):
         np.testing.assert_array_equal(got, want)
 
 
+ODD_BROADCASTS = [
+    ((129, 1001), (1001,), (129, 1)), ((7, 33, 125), (33, 1), (125,)), ((3, 1367), (1, 1367), (3, 1)), ((4099, 3), (3,), (4099, 1)),
+    ((5, 1, 821), (1, 9, 821), (9, 1)), ((64, 65), (64, 65), (65,)),
+]
+
+
+@pytest.mark.parametrize("sa,sb,sc", ODD_BROADCASTS, ids=lambda s: str(s))
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)
+def test_broadcasts_whose_innermost_extent_no_vector_divides(gpu, sa, sb, sc, dtype):
+    """Rows of 1001, 125, 3 ... elements: lanes own vectors of the dense output that straddle rows, and the broadcast operands are
+    read at coordinates carried along the vector.  Same results as the element-by-element form, bit for bit in 16-bit arithmetic."""
+    rng = np.random.default_rng(11)
+    a, b, c = (to_storage(rng.standard_normal(shape).astype(np.float32), dtype) for shape in (sa, sb, sc))
+    plan, outs = run_staged((ex.input("a") + ex.input("b")) * ex.input("c"), {"a": a, "b": b, "c": c}, dtype)
+    af, bf, cf = (from_storage(v, dtype) for v in (a, b, c))
+    want = rnd(rnd(af + bf, dtype) * cf, dtype)
+    got = from_storage(outs["output"], dtype)
+    assert got.shape == want.shape
+    np.testing.assert_array_equal(got, want)
+    if want.size >= 4096:
+        assert "vectors_straddle_rows" in plan.stage_descriptions()[0], plan.stage_descriptions()
+
+
 def test_strided_view_inputs(gpu):
     stream = ph.Stream(0)
     x = np.arange(30, dtype=np.float32).reshape(5, 6)

@@ -552,6 +552,33 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
     }
     const bool tiled = tileAxis >= 0;
     if (tiled) vec = 1;
+    // An innermost extent (or an operand's stride) that no vector length divides: the lanes still own vectors of the dense
+    // output, which may straddle rows; operands laid out like the output are read as vectors too, the others element by
+    // element at coordinates that are carried along the vector.
+    bool straddling = false;
+    std::vector<char> likeOutput(r.operands.size(), 0);
+    if (!k.flat && !tiled && vec == 1 && !r.extent.has_value() && r.gathers.empty() && k.numel >= 4096) {
+        int wide = static_cast<int>(16 / widest);
+        std::vector<uint64_t> dense(layout.dims.size(), 1);
+        for (size_t a = layout.dims.size(); a-- > 1;) dense[a - 1] = dense[a] * layout.dims[a];
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            likeOutput[o] = !single[o];
+            for (size_t a = 0; a < layout.dims.size(); ++a)
+                if (layout.dims[a] > 1 && layout.operandStride[o][a] != dense[a]) likeOutput[o] = 0;
+        }
+        auto aligned = [&](int v) {
+            for (const KernelOutput& out : r.outputs)
+                if (out.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(out.storageDType)) != 0) return false;
+            for (size_t o = 0; o < r.operands.size(); ++o)
+                if (likeOutput[o] && r.operands[o].alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(r.operands[o].storageDType)) != 0) return false;
+            return true;
+        };
+        while (wide > 1 && !aligned(wide)) wide /= 2;
+        if (wide > 1) {
+            straddling = true;
+            vec = wide;
+        }
+    }
     k.vec = vec;
     k.passNumel = k.flat;
 
@@ -794,6 +821,62 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         k.gridX = static_cast<uint32_t>(blocks);
         k.vec = vb;
         k.description = "tiled(axis=" + std::to_string(tileAxis) + "/" + std::to_string(rank) + ",tile=64x" + std::to_string(tileB) + ")";
+    } else if (straddling) {
+        const std::vector<uint64_t>& dims = layout.dims;
+        const size_t rank = dims.size();
+        s << "    const index_t base = ((index_t)blockIdx.x * " << threads << "u + threadIdx.x) * V;\n";
+        s << "    if (base >= " << k.numel << "ull) return;\n";
+        // coordinates of element `base`; element base + k is reached by adding one k times, with carries
+        s << "    index_t rest = base;\n";
+        for (size_t a = rank; a-- > 0;) {
+            if (a == 0) {
+                s << "    index_t c0 = rest;\n";
+            } else {
+                s << "    index_t c" << a << " = rest % " << dims[a] << "u;\n    rest /= " << dims[a] << "u;\n";
+            }
+        }
+        auto offsetOf = [&](size_t o) {
+            std::string text = "0ull";
+            for (size_t a = 0; a < rank; ++a)
+                if (layout.operandStride[o][a] != 0 && dims[a] > 1) text += " + (unsigned long long)c" + std::to_string(a) + " * " + std::to_string(layout.operandStride[o][a]) + "ull";
+            return text;
+        };
+        std::string advance = "        ++c" + std::to_string(rank - 1) + ";\n";
+        for (size_t a = rank; a-- > 1;)
+            advance += "        if (c" + std::to_string(a) + " == " + std::to_string(dims[a]) + "u) { c" + std::to_string(a) + " = 0; ++c" + std::to_string(a - 1) + "; }\n";
+        s << "    if (base + V <= " << k.numel << "ull) {\n";
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            if (!likeOutput[o]) continue;
+            s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n        p" << o << ".loadStream(in" << o << " + base);\n";
+        }
+        for (size_t o = 0; o < r.outputs.size(); ++o) s << "        thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", V> q" << o << ";\n";
+        s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
+        s << emitBody(
+            "            ",
+            [&](size_t o) {
+                if (single[o]) return "in" + std::to_string(o) + "[0]";
+                if (likeOutput[o]) return "p" + std::to_string(o) + ".v[k]";
+                return "in" + std::to_string(o) + "[" + offsetOf(o) + "]";
+            },
+            [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; }, noGather);
+        s << advance;
+        s << "        }\n";
+        for (size_t o = 0; o < r.outputs.size(); ++o) s << "        q" << o << ".storeStream(out" << o << " + base);\n";
+        s << "        return;\n    }\n";
+        s << "    for (index_t e = base; e < " << k.numel << "ull; ++e) {\n";
+        s << emitBody(
+            "        ",
+            [&](size_t o) {
+                if (single[o]) return "in" + std::to_string(o) + "[0]";
+                if (likeOutput[o]) return "in" + std::to_string(o) + "[e]";
+                return "in" + std::to_string(o) + "[" + offsetOf(o) + "]";
+            },
+            [](size_t o, const std::string& v) { return "out" + std::to_string(o) + "[e] = " + v + ";"; }, noGather);
+        s << advance;
+        s << "    }\n";
+        const uint64_t lanes = (k.numel + vec - 1) / vec;
+        k.gridX = static_cast<uint32_t>(std::max<uint64_t>((lanes + threads - 1) / threads, 1));
+        k.description = "broadcast(axes=" + std::to_string(rank) + ",vec=" + std::to_string(vec) + ",vectors_straddle_rows)";
     } else {
         std::vector<uint64_t> dims = layout.dims;
         dims.back() /= vec;  // the innermost axis is walked in vectors
