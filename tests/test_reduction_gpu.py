@@ -65,6 +65,8 @@ SHAPES = [
     ([3, 5], [1]), ([64, 1], [1]), ([33, 17], [1]), ([128, 64], [1]), ([100, 1000], [1]), ([7, 4096], [1]), ([5, 8191], [1]), ([3, 70000], [1]),
     ([2, 1 << 19], [1]), ([1000, 3], [0]), ([64, 64], [0]), ([4097, 8], [0]), ([2, 300, 40], [1]), ([5, 6, 7, 8], [1, 2]), ([5, 6, 7, 8], [0, 1]),
     ([4, 6, 10, 12], [0, 2, 3]), ([3, 4, 5, 6], [1, 3]), ([2, 3, 4, 5, 2], [0, 2, 4]), ([8, 16, 32], [0, 2]),
+    # rows no vector divides: vectors at addresses aligned to the element only, the rest of the row one by one
+    ([100, 1001], [1]), ([37, 50257], [1]), ([5000, 63], [1]), ([3, 70001], [1]), ([9, 131], [1]),
 ]
 
 
@@ -112,6 +114,28 @@ def test_arg_ops_against_oracle_with_ties_and_nans(stream, dims, axes):
             want_idx, want_val = oracle.arg_reduce(oop, x, oracle.FP32, axes)
             np.testing.assert_array_equal(idx.astype(np.uint64), want_idx)
             np.testing.assert_array_equal(val, want_val)
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16], ids=lambda d: d.name)
+def test_rows_no_vector_divides_and_rows_that_begin_off_a_vector(stream, dtype):
+    rng = np.random.default_rng(3)
+    x = to_storage(rng.standard_normal((64, 1003)).astype(np.float32), dtype)
+    t = copy_numpy_to_gpu(x, stream, dtype)
+    stamped = ph.CubReduction(ph.CubReductionOp.Sum, [1], DataType.fp32).stamp(t, stream)
+    assert "unaligned_vectors" in stamped.get_kernel_variant()
+    stamped.run()
+    exact = oracle.reduce_f64(oracle.SUM, x, int(dtype), [1])
+    magnitude = oracle.reduce_f64(oracle.L1NORM, x, int(dtype), [1])
+    assert np.all(np.abs(gpu_to_f32(stamped.get_output_tensor(), stream).astype(np.float64) - exact) <= 1e-5 * magnitude + 1e-30)
+    # a view whose rows have a vector's length but begin one element into the storage
+    for rows_in_view, row_stride in ((60, 1003), (64000 // 1000, 1000)):
+        view = t.alias_view([rows_in_view, 1000], [row_stride, 1], element_offset=1)
+        stamped = ph.CubReduction(ph.CubReductionOp.Max, [1], DataType.fp32).stamp(view, stream)
+        stamped.run()
+        carrier = x.reshape(-1)[1:]
+        rows = np.stack([carrier[r * row_stride:r * row_stride + 1000] for r in range(rows_in_view)])
+        np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream), oracle.reduce_f64(oracle.MAX, rows, int(dtype), [1]).astype(np.float32),
+                                      err_msg=stamped.get_kernel_variant())
 
 
 def test_output_dtypes_scale_and_fp8_saturation(stream):

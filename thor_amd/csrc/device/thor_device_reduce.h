@@ -199,6 +199,18 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
             }
         }
     }
+    if constexpr (Cfg::kR % Cfg::kVec != 0) {
+        // a row length no vector divides (the vectors above were read at unaligned addresses): the rest of the row, one
+        // element per lane, by the block that holds the row's last segment
+        constexpr u64 kTail = Cfg::kR % Cfg::kVec;
+        if (rowLive && segment == (u64)Cfg::kSplit - 1) {
+            for (u64 t = (u64)lane; t < kTail; t += TPR) {
+                typename Cfg::Loaded x;
+                Cfg::loadFirstOnly(src, rowBase + kVectorsPerRow * Cfg::kVec + t, x);
+                Cfg::accumulateOne(acc, x, src, kept, 0, (IndexT)(kVectorsPerRow * Cfg::kVec + t));
+            }
+        }
+    }
     if (kSubWave) {
         groupReduce<TPR>(acc);
     } else {

@@ -167,6 +167,7 @@ std::string ReductionShape::describe() const {
             break;
         case Kernel::Rows:
             out << "rows(lanes_per_row=" << threadsPerRow << ",split=" << split;
+            if (unalignedVectors) out << ",unaligned_vectors";
             break;
         case Kernel::Columns:
             out << (laneAxis < 0 ? "columns(lanes_x=" : "view_columns(lanes_x=") << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
@@ -335,7 +336,14 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
     if (g.path == CubReductionPath::ContiguousFixedSegment) {
         shape.kernel = ReductionShape::Kernel::Rows;
         shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.reduction_size});
-        const uint64_t vectorsPerRow = g.reduction_size / shape.vec;
+        // A row length (or a pointer) that no vector fits: the lanes still read 16-byte vectors, at addresses that are only
+        // aligned to the element, and the last row_length % vec elements of a row one by one.
+        const int wide = static_cast<int>(16 / elementBytes);
+        if (shape.vec < wide && request.elementwise.empty() && g.reduction_size >= 4ull * wide && request.inputAlignmentBytes % elementBytes == 0) {
+            shape.vec = wide;
+            shape.unalignedVectors = true;
+        }
+        const uint64_t vectorsPerRow = std::max<uint64_t>(g.reduction_size / shape.vec, 1);
         // aim at about 8 vector loads in flight per lane
         uint64_t lanes = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(ceilDiv(vectorsPerRow, 8)), 1), 1024);
         // ... but never fewer than 8 lanes on a row that has the vectors for them: the lanes of a row read adjacent vectors, and
@@ -524,7 +532,12 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     s << "    };\n";
     s << "    static __device__ __forceinline__ void load(const Sources& s, u64 offset, Loaded& l) {\n";
     for (size_t i = 0; i < sources.size(); ++i)
-        if (sources[i].kind == SourceKind::Vector) s << "        l.p" << i << ".loadStream(s.in" << i << " + offset);\n";
+        if (sources[i].kind == SourceKind::Vector)
+            s << "        l.p" << i << (shape.unalignedVectors ? ".loadStreamUnaligned(s.in" : ".loadStream(s.in") << i << " + offset);\n";
+    s << "        (void)s; (void)offset; (void)l;\n    }\n";
+    s << "    static __device__ __forceinline__ void loadFirstOnly(const Sources& s, u64 offset, Loaded& l) {\n";  // element 0 of every vector source
+    for (size_t i = 0; i < sources.size(); ++i)
+        if (sources[i].kind == SourceKind::Vector) s << "        l.p" << i << ".v[0] = s.in" << i << "[offset];\n";
     s << "        (void)s; (void)offset; (void)l;\n    }\n";
     // values that depend only on the output
     s << "    struct Kept {\n";

@@ -94,6 +94,8 @@ struct ReductionShape {
     int minTeam = 1, finishLanes = 1, finishThreads = 256;
     // Segments kernel: rows dealt out to lanes (reduceSegmentsByRows) instead of segments dealt out to teams (reduceSegments)
     bool segmentsByRows = false;
+    // Rows kernel: vectors at addresses that are only aligned to the element; the last reduction_size % vec elements of a row go one by one
+    bool unalignedVectors = false;
     int walkGroup = 4;  // reduceSegmentsByRows: rows of a lane's range that are walked together
     std::string describe() const;
 };
