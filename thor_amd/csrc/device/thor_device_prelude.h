@@ -97,6 +97,13 @@ struct alignas((sizeof(T) * VEC) >= 16 ? 16 : (sizeof(T) * VEC)) Pack {
 #pragma unroll
         for (int w = 0; w < kWords; ++w) mine[w] = __builtin_nontemporal_load(wp + w);
     }
+    __device__ __forceinline__ void loadUnaligned(const T* p) {
+        typedef word_t __attribute__((aligned(alignof(T)))) unaligned_word_t;
+        const unaligned_word_t* wp = reinterpret_cast<const unaligned_word_t*>(p);
+        word_t* mine = reinterpret_cast<word_t*>(v);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) mine[w] = wp[w];
+    }
     __device__ __forceinline__ void load(const T* p) {
         const word_t* wp = reinterpret_cast<const word_t*>(p);
         word_t* mine = reinterpret_cast<word_t*>(v);

@@ -321,6 +321,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         if (isElem(rg.cls[m])) consider(expr.nodes[m].output_dtype.value());
     if (narrow > wide) return false;  // nothing streamed per element: not worth a row kernel
     int vec = static_cast<int>(std::max<uint32_t>(16 / wide, std::min<uint32_t>(4, 16 / narrow)));
+    const int wantedVec = vec;
     while (vec > 1 && rg.R % vec != 0) vec /= 2;
     // pointers of existing tensors must allow the vector accesses (fresh allocations are 256-byte aligned)
     for (uint32_t s : em.sourceNodes) {
@@ -328,6 +329,14 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         const uint64_t align = pointerAlignment(ctx.tensorOf[s].getMemPtr());
         while (vec > 1 && align % std::min<uint64_t>(16, static_cast<uint64_t>(vec) * dataTypeSizeInBytes(ctx.tensorOf[s].getDataType())) != 0) vec /= 2;
     }
+    // A row length (or a pointer) that the vector does not fit: the lanes keep the full vector, read and written at addresses
+    // that are only aligned to the element; the row's last vector overlaps the one before it (rows of 1001 or 50257).
+    bool unaligned = false;
+    if (vec < wantedVec && rg.R >= 4ull * static_cast<uint64_t>(wantedVec)) {
+        vec = wantedVec;
+        unaligned = true;
+    }
+    const uint64_t tail = rg.R % static_cast<uint64_t>(vec);
     // ---- phases ---------------------------------------------------------------------------------------------------------
     // elem nodes get the loop they are computed in; uniform nodes get the number of folds that must have happened
     std::vector<int> phase(count, 0);
@@ -370,7 +379,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         const DataType dt = ctx.role[m] == Role::Materialized ? expr.nodes[m].output_dtype.value() : emittedValueDType(expr.nodes[m]);
         registersPerElement += std::max(1.0, dataTypeSizeInBytes(dt) / 4.0);  // 16-bit values sit in registers of their own
     }
-    const uint64_t vectors = rg.R / vec;
+    const uint64_t vectors = (rg.R + vec - 1) / vec;  // the last one is partial when tail != 0
     auto budget = [](uint64_t lanes) { return lanes <= 512 ? 160.0 : 96.0; };
     // Measured on MI355X (softmax and normalisation, rows of 128 to 8192 elements): two 16-byte vectors per lane up to one
     // 256-thread block per row is fastest; longer rows then take more vectors per lane until the row data reaches about
@@ -418,11 +427,25 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     s << "    const unsigned long long rowIndex = rowLive ? row : 0ull;\n";
     s << "    const unsigned long long rowBase = rowIndex * R;\n";
     // when every lane of every block has a whole vector of a real row, the bounds checks vanish at compile time
-    const bool allLive = vectors % T == 0 && rg.rows % rowsPerBlock == 0;
+    const bool allLive = vectors % T == 0 && rg.rows % rowsPerBlock == 0 && tail == 0;
     const std::string liveIf = allLive ? "" : "if (live[it]) ";
     s << "    bool live[ITEMS];\n    unsigned long long column[ITEMS];\n";
     s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        const unsigned long long v = (unsigned long long)it * T + lane;\n"
          "        live[it] = rowLive && v < VECTORS;\n        column[it] = (v < VECTORS ? v : 0ull) * V;\n    }\n";
+    if (tail != 0) {
+        // The row's last vector is read (and written) V - tail elements early, so that it ends with the row: it overlaps the
+        // vector before it, folds skip the elements it shares with that one, and the stores write those twice with the same bits.
+        s << "    int skip[ITEMS];\n#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n"
+             "        const unsigned long long v = (unsigned long long)it * T + lane;\n"
+             "        skip[it] = v + 1 == VECTORS ? " << (vec - tail) << " : 0;\n"
+             "        if (v + 1 == VECTORS) column[it] = R - V;\n    }\n";
+    }
+    auto loadItem = [&](const std::string& pack, const std::string& address, bool stream) {
+        return "        " + liveIf + pack + (unaligned ? (stream ? ".loadStreamUnaligned(" : ".loadUnaligned(") : (stream ? ".loadStream(" : ".load(")) + address + ");\n";
+    };
+    auto storeItem = [&](const std::string& pack, const std::string& address) {
+        return "        " + liveIf + pack + ".storeStream(" + address + ");\n";  // the store instruction takes any alignment
+    };
 
     // sources
     std::map<uint32_t, size_t> sourceIndex;
@@ -437,9 +460,9 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
             s << "    thor::Pack<" << type << ", V> p" << o << "[ITEMS];\n";
             s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        p" << o << "[it] = {};\n";
             if (rg.cls[node] == Cls::RowVec) {
-                s << "        " << liveIf << "p" << o << "[it].loadStream(in" << o << " + rowBase + column[it]);\n";
+                s << loadItem("p" + std::to_string(o) + "[it]", "in" + std::to_string(o) + " + rowBase + column[it]", true);
             } else {
-                s << "        " << liveIf << "p" << o << "[it].load(in" << o << " + column[it]);\n";
+                s << loadItem("p" + std::to_string(o) + "[it]", "in" + std::to_string(o) + " + column[it]", false);
             }
             s << "    }\n";
         } else {
@@ -587,14 +610,19 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         s << "        }\n";
         if (!folding.empty()) {
             // one bounds decision per vector, not per element
-            s << "        " << liveIf << "{\n#pragma unroll\n            for (int k = 0; k < V; ++k) {\n";
-            for (uint32_t r : folding) s << "                acc" << r << ".add(a" << r << "[k], 0u);\n";
-            s << "            }\n        }\n";
+            if (tail == 0) {
+                s << "        " << liveIf << "{\n#pragma unroll\n            for (int k = 0; k < V; ++k) {\n";
+                for (uint32_t r : folding) s << "                acc" << r << ".add(a" << r << "[k], 0u);\n";
+                s << "            }\n        }\n";
+            } else {
+                s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n            if (live[it] && k >= skip[it]) {\n";
+                for (uint32_t r : folding) s << "                acc" << r << ".add(a" << r << "[k], 0u);\n";
+                s << "            }\n        }\n";
+            }
         }
         for (uint32_t m : storedHere) {
             const Cls c = rg.cls[m];
-            s << "        " << liveIf << "q" << outputIndex[m] << ".storeStream(out" << outputIndex[m] << " + " << (c == Cls::RowVec ? "rowBase + " : "")
-              << "column[it]);\n";
+            s << storeItem("q" + std::to_string(outputIndex[m]), "out" + std::to_string(outputIndex[m]) + " + " + (c == Cls::RowVec ? "rowBase + " : "") + "column[it]");
         }
         s << "    }\n";
         // fold the lanes that share the row, then the values that depend on the results
@@ -629,7 +657,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     em.source = s.str();
     em.flops *= rg.rows;
     em.description = "row_fused(rows=" + std::to_string(rg.rows) + ",R=" + std::to_string(rg.R) + ",lanes_per_row=" + std::to_string(T) +
-                     ",items=" + std::to_string(items) + ",vec=" + std::to_string(vec) + ",loops=" + std::to_string(numLoops) + ")";
+                     ",items=" + std::to_string(items) + ",vec=" + std::to_string(vec) + (unaligned ? ",unaligned_vectors" : "") + ",loops=" + std::to_string(numLoops) + ")";
     return true;
 }
 
