@@ -151,6 +151,31 @@ def test_no_access_outside_the_range_and_unaligned_views(gpu):
     assert raw[0] == 0x5A5A and np.all(raw[1 + n:] == 0x5A5A)
 
 
+@pytest.mark.parametrize("src_off,dst_off", [(1, 1), (3, 3), (2, 1), (0, 3), (1, 0), (5, 5), (7, 2)])
+@pytest.mark.parametrize("pair", [("fp32", "fp16"), ("fp16", "fp32"), ("fp32", "bf16"), ("bf16", "fp16"), ("fp16", "fp8_e4m3")], ids=lambda p: "-".join(p))
+def test_views_that_begin_inside_a_word(gpu, src_off, dst_off, pair):
+    """Source and destination a few elements past a word boundary, by the same count (both become aligned once the slots are
+    counted from the boundary below the destination) and by different counts (source words are read where they lie): bit-exact
+    against the oracle, guard bytes on both sides of the destination untouched."""
+    from thor_amd.runtime import DeviceBuffer, TypeConverter
+    src_dtype, dst_dtype = DataType[pair[0]], DataType[pair[1]]
+    codes = {"fp32": oracle.FP32, "fp16": oracle.FP16, "bf16": oracle.BF16, "fp8_e4m3": oracle.FP8_E4M3}
+    src_code, dst_code = codes[pair[0]], codes[pair[1]]
+    dst_carrier = np.dtype(oracle.CARRIER[dst_code])
+    n = 70_001
+    x32 = c2_like(n + 16, 9)
+    x = x32 if pair[0] == "fp32" else oracle.convert(x32, oracle.FP32, src_code)
+    src = DeviceBuffer.from_numpy(x)
+    dst = DeviceBuffer((n + 64) * dst_carrier.itemsize)
+    dst.memset(0x5A)
+    gpu.device_synchronize()
+    TypeConverter.convert_type(src.ptr + src_off * x.itemsize, dst.ptr + dst_off * dst_carrier.itemsize, src_dtype, dst_dtype, n)
+    raw = dst.download(dst_carrier, n + 64)
+    want = oracle.convert(x[src_off:src_off + n], src_code, dst_code)
+    assert raw[dst_off:dst_off + n].tobytes() == want.tobytes()
+    assert np.all(np.frombuffer(raw[:dst_off].tobytes(), np.uint8) == 0x5A) and np.all(np.frombuffer(raw[dst_off + n:].tobytes(), np.uint8) == 0x5A)
+
+
 def test_overlap_and_argument_errors(gpu):
     from thor_amd._lib import ThorHipError
     from thor_amd.runtime import DeviceBuffer, TypeConverter

@@ -368,9 +368,14 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.inner_size});
         shape.threads = 256;
         shape.unroll = 8;  // rows in flight per thread
+        if (const char* env = std::getenv("THOR_COLUMNS_BATCH")) shape.unroll = std::min<long>(std::max<long>(std::atol(env), 1), 16);  // tuning switch
         const uint64_t columns = g.outer_size * (g.inner_size / shape.vec);
         // a block is up to one wavefront of columns wide; the rest of its threads are row groups folded through LDS
         shape.threadsPerRow = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(columns)));
+        if (const char* env = std::getenv("THOR_COLUMNS_LANES")) {  // tuning switch: lanes across the columns of a block
+            const long requested = std::atol(env);
+            if ((requested == 64 || requested == 128 || requested == 256) && static_cast<uint64_t>(requested) <= pow2Ceil(columns)) shape.threadsPerRow = static_cast<int>(requested);
+        }
         const uint64_t groups = 256 / shape.threadsPerRow;
         // enough threads to keep loads in flight on every CU, but at least 16 rows per thread and partials that stay small
         // next to the input (measured on 8192 x 8192 fp32: 512 Ki threads reach 5.3 TB/s, 128 Ki threads 3.8 TB/s)
@@ -378,6 +383,9 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         if (columns * groups < wantedThreads && g.reduction_size >= groups * 32) {
             shape.split = std::min<uint64_t>({ceilDiv(wantedThreads, columns * groups), g.reduction_size / (groups * 16), kMaxGridY});
             if (shape.split < 2) shape.split = 1;
+        }
+        if (const char* env = std::getenv("THOR_COLUMNS_SPLIT")) {  // tuning switch
+            shape.split = std::min<uint64_t>({static_cast<uint64_t>(std::max<long>(std::atol(env), 1)), std::max<uint64_t>(g.reduction_size / groups, 1), kMaxGridY});
         }
         const uint64_t columnsNow = g.outer_size * (g.inner_size / shape.vec);
         shape.gridX = static_cast<uint32_t>(ceilDiv(columnsNow, shape.threadsPerRow));
