@@ -64,6 +64,36 @@ def test_strided_views_address_the_operands_storage(stream):
         run({"y": ex.input("v").transpose() + 1.0}, {"v": copy_numpy_to_gpu(x[0], stream, DataType.fp32)}, stream)
 
 
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)
+@pytest.mark.parametrize("offset", [1, 3, 5])
+def test_operands_that_begin_inside_a_word_keep_vector_loads(stream, dtype, offset):
+    """Views a few elements into their storage, and rows whose pitch no vector divides: the kernels keep their vector length
+    and read those operands where they lie; the dense output is written in aligned vectors."""
+    rng = np.random.default_rng(offset)
+    n = 50_000
+    a = to_storage(rng.standard_normal(n + 8).astype(np.float32), dtype)
+    b = to_storage(rng.standard_normal(n + 8).astype(np.float32), dtype)
+    ta, tb = copy_numpy_to_gpu(a, stream, dtype), copy_numpy_to_gpu(b, stream, dtype)
+    va, vb = ta.alias_view([n], [1], element_offset=offset), tb.alias_view([n], [1], element_offset=offset + 1)
+    plan = ex.compile(ex.input("a") + ex.input("b"), 0).stamp({"a": va, "b": vb}, stream)
+    plan.run()
+    assert "vec=1" not in plan.stage_descriptions()[0], plan.stage_descriptions()
+    want = to_storage(from_storage(a[offset:offset + n], dtype) + from_storage(b[offset + 1:offset + 1 + n], dtype), dtype)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output(), stream), want)
+    # rows of 256 elements cut out of rows of 259: every row begins at another offset inside a word
+    m = to_storage(rng.standard_normal((300, 259)).astype(np.float32), dtype)
+    c = to_storage(rng.standard_normal(256).astype(np.float32), dtype)
+    tm, tc = copy_numpy_to_gpu(m, stream, dtype), copy_numpy_to_gpu(c, stream, dtype)
+    vm = tm.alias_view([300, 256], [259, 1], element_offset=offset % 3)
+    plan = ex.compile(ex.input("m") * ex.input("c"), 0).stamp({"m": vm, "c": tc}, stream)
+    plan.run()
+    assert "vec=1" not in plan.stage_descriptions()[0], plan.stage_descriptions()
+    rows = m.reshape(-1)[offset % 3:][:299 * 259 + 256]
+    window = np.stack([rows[r * 259:r * 259 + 256] for r in range(300)])
+    want = to_storage(from_storage(window, dtype) * from_storage(c, dtype), dtype)
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output(), stream), want)
+
+
 @pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16], ids=lambda d: d.name)
 def test_ragged_kernel_over_a_slice_of_the_packed_values(stream, dtype):
     """A trailing slice [capacity, H] of packed values [capacity, 2H] is a strided view: the kernel is not a flat one, and it

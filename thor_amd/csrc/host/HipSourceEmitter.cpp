@@ -509,27 +509,27 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
     auto fits = [&](int v) {
         for (const KernelOutput& out : r.outputs)
             if (out.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(out.storageDType)) != 0) return false;
-        if (k.flat) {
-            for (size_t o = 0; o < r.operands.size(); ++o) {
-                const KernelOperand& op = r.operands[o];
-                if (!single[o] && op.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(op.storageDType)) != 0) return false;
-            }
-            return true;
-        }
+        // operands only have to be aligned to their element: a vector of an operand that begins inside a word (a view a few
+        // elements into its storage, rows whose pitch no vector divides) is read where it lies, at the rate of aligned loads
+        for (size_t o = 0; o < r.operands.size(); ++o)
+            if (!single[o] && r.operands[o].alignmentBytes % dataTypeSizeInBytes(r.operands[o].storageDType) != 0) return false;
+        if (k.flat) return true;
         if (layout.dims.back() % v != 0) return false;
         if (r.extent.has_value() && r.extent->elementsPerValue % v != 0) return false;  // a vector never straddles the last active row
-        for (size_t o = 0; o < r.operands.size(); ++o) {
-            const std::vector<uint64_t>& s = layout.operandStride[o];
-            if (s.back() > 1) return false;  // neither contiguous nor broadcast along the innermost axis
-            if (s.back() == 1) {
-                if (r.operands[o].alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(r.operands[o].storageDType)) != 0) return false;
-                for (size_t a = 0; a + 1 < s.size(); ++a)
-                    if (s[a] % v != 0) return false;
-            }
-        }
+        for (size_t o = 0; o < r.operands.size(); ++o)
+            if (layout.operandStride[o].back() > 1) return false;  // neither contiguous nor broadcast along the innermost axis
         return true;
     };
     while (vec > 1 && !fits(vec)) vec /= 2;
+    // which operands are read with aligned vector loads at the chosen length
+    auto operandAligned = [&](size_t o, int v) {
+        if (r.operands[o].alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(r.operands[o].storageDType)) != 0) return false;
+        if (!k.flat)
+            for (size_t a = 0; a + 1 < layout.operandStride[o].size(); ++a)
+                if (layout.operandStride[o][a] % v != 0) return false;
+        return true;
+    };
+    auto vectorLoad = [&](size_t o, int v) { return operandAligned(o, v) ? ".loadStream(" : ".loadStreamUnaligned("; };
 
     // Operands whose contiguous axis is another axis of the output than the innermost one (transposes, permuted views): read
     // through LDS tiles, so that both the operand and the output are addressed along their own contiguous axis.
@@ -569,9 +569,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         auto aligned = [&](int v) {
             for (const KernelOutput& out : r.outputs)
                 if (out.alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(out.storageDType)) != 0) return false;
-            for (size_t o = 0; o < r.operands.size(); ++o)
-                if (likeOutput[o] && r.operands[o].alignmentBytes % (static_cast<uint64_t>(v) * dataTypeSizeInBytes(r.operands[o].storageDType)) != 0) return false;
-            return true;
+            return true;  // (operands are read where they lie)
         };
         while (wide > 1 && !aligned(wide)) wide /= 2;
         if (wide > 1) {
@@ -710,7 +708,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
             for (size_t o = 0; o < r.operands.size(); ++o) {
                 if (single[o]) continue;
                 s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n";
-                s << "        p" << o << ".loadStream(in" << o << " + base);\n";
+                s << "        p" << o << vectorLoad(o, vec) << "in" << o << " + base);\n";
             }
             for (size_t o = 0; o < r.outputs.size(); ++o) s << "        thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", V> q" << o << ";\n";
             s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
@@ -847,7 +845,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
         s << "    if (base + V <= " << k.numel << "ull) {\n";
         for (size_t o = 0; o < r.operands.size(); ++o) {
             if (!likeOutput[o]) continue;
-            s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n        p" << o << ".loadStream(in" << o << " + base);\n";
+            s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n        p" << o << vectorLoad(o, vec) << "in" << o << " + base);\n";
         }
         for (size_t o = 0; o < r.outputs.size(); ++o) s << "        thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", V> q" << o << ";\n";
         s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
@@ -908,7 +906,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
             const bool contiguous = layout.operandStride[o].back() == 1;
             const char* type = deviceTypeName(r.operands[o].storageDType);
             if (contiguous && vec > 1) {
-                s << "    thor::Pack<" << type << ", V> p" << o << ";\n    p" << o << ".loadStream(in" << o << " + off" << o << ");\n";
+                s << "    thor::Pack<" << type << ", V> p" << o << ";\n    p" << o << vectorLoad(o, vec) << "in" << o << " + off" << o << ");\n";
             } else {
                 s << "    const " << type << " b" << o << " = in" << o << "[off" << o << "];\n";
             }
