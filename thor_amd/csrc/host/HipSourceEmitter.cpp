@@ -847,6 +847,16 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
             if (!likeOutput[o]) continue;
             s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> p" << o << ";\n        p" << o << vectorLoad(o, vec) << "in" << o << " + base);\n";
         }
+        // broadcast operands that are contiguous along the innermost axis: one vector when the lane's elements stay inside
+        // a row of theirs, element by element (at the carried coordinates) in the lanes whose vector wraps
+        std::vector<char> rowVector(r.operands.size(), 0);
+        for (size_t o = 0; o < r.operands.size(); ++o) {
+            if (single[o] || likeOutput[o] || layout.operandStride[o][rank - 1] != 1 || dims[rank - 1] < static_cast<uint64_t>(vec)) continue;
+            rowVector[o] = 1;
+            s << "        const bool inRow" << o << " = c" << (rank - 1) << " + V <= " << dims[rank - 1] << "u;\n";
+            s << "        thor::Pack<" << deviceTypeName(r.operands[o].storageDType) << ", V> pb" << o << ";\n";
+            s << "        if (inRow" << o << ") pb" << o << ".loadUnaligned(in" << o << " + " << offsetOf(o) << ");\n";
+        }
         for (size_t o = 0; o < r.outputs.size(); ++o) s << "        thor::Pack<" << deviceTypeName(r.outputs[o].storageDType) << ", V> q" << o << ";\n";
         s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
         s << emitBody(
@@ -854,6 +864,7 @@ EmittedKernel emitFusedKernel(const FusedKernelRequest& r) {
             [&](size_t o) {
                 if (single[o]) return "in" + std::to_string(o) + "[0]";
                 if (likeOutput[o]) return "p" + std::to_string(o) + ".v[k]";
+                if (rowVector[o]) return "(inRow" + std::to_string(o) + " ? pb" + std::to_string(o) + ".v[k] : in" + std::to_string(o) + "[" + offsetOf(o) + "])";
                 return "in" + std::to_string(o) + "[" + offsetOf(o) + "]";
             },
             [](size_t o, const std::string& v) { return "q" + std::to_string(o) + ".v[k] = " + v + ";"; }, noGather);
