@@ -76,6 +76,33 @@ def test_row_longer_than_the_register_budget_uses_streaming_stages(gpu):
     np.testing.assert_allclose(outs["output"], p / p.sum(axis=1, keepdims=True), rtol=3e-6, atol=1e-12)
 
 
+def test_rows_that_fit_only_without_kept_values_recompute_them(gpu):
+    """A row of 50 257 fp32 plus its exponentials is more than a block's registers hold; the row alone fits, and the last loop
+    computes the exponentials again from it."""
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal((6, 50257)) * 3).astype(np.float32)
+    plan, outs = run_staged(softmax_expr(), {"x": x}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedRowKernel"] and "values_recomputed" in plan.stage_descriptions()[0], plan.stage_descriptions()
+    x64 = x.astype(np.float64)
+    p = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(outs["output"], p / p.sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-12)
+    _, outs_s = staged(softmax_expr(), {"x": x}, DataType.fp32)
+    np.testing.assert_allclose(outs["output"], outs_s["output"], rtol=1e-5, atol=1e-12)
+    # mean / variance normalisation with scale and shift: two kept values (the centred row and its square) are recomputed
+    R = 28001
+    xn = (rng.standard_normal((5, R)) * 2 + 0.5).astype(np.float32)
+    gamma, beta = rng.uniform(0.5, 1.5, R).astype(np.float32), rng.uniform(-1, 1, R).astype(np.float32)
+    ix, ig, ib = ex.input("x"), ex.input("gamma"), ex.input("beta")
+    centered = ix - ix.reduce_mean(axis=1)
+    expr = centered / ((centered * centered).reduce_mean(axis=1) + 1e-5).sqrt() * ig + ib
+    plan, outs = run_staged(expr, {"x": xn, "gamma": gamma, "beta": beta}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedRowKernel"] and "values_recomputed" in plan.stage_descriptions()[0], plan.stage_descriptions()
+    x64 = xn.astype(np.float64)
+    mu = x64.mean(axis=1, keepdims=True)
+    var = ((x64 - mu) ** 2).mean(axis=1, keepdims=True)
+    np.testing.assert_allclose(outs["output"], (x64 - mu) / np.sqrt(var + 1e-5) * gamma + beta, rtol=2e-5, atol=2e-5)
+
+
 def test_order_independent_parts_are_bit_identical_to_the_staged_plan(gpu):
     """x - rowmax, rowmax and rowmax - rowmin involve no accumulation order: both plans must agree bit for bit.  Division by a
     per-row value uses one reciprocal per row plus a fused correction step in the row kernel: within 1 ulp of the IEEE

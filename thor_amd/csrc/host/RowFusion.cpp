@@ -7,6 +7,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <functional>
 #include <map>
 #include <numeric>
 #include <set>
@@ -371,14 +372,6 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     // ---- lanes per row ---------------------------------------------------------------------------------------------------
     // about eight vectors per lane, more lanes when the row's registers (the loaded row plus every per-element value
     // that has to survive a fold) would not fit the budget a block of that size leaves per lane
-    double registersPerElement = 0.0;
-    for (uint32_t sNode : em.sourceNodes)
-        if (isElem(rg.cls[sNode])) registersPerElement += dataTypeSizeInBytes(ctx.tensorOf[sNode].getDataType()) / 4.0;
-    for (uint32_t m : members) {
-        if (!needsArray[m]) continue;
-        const DataType dt = ctx.role[m] == Role::Materialized ? expr.nodes[m].output_dtype.value() : emittedValueDType(expr.nodes[m]);
-        registersPerElement += std::max(1.0, dataTypeSizeInBytes(dt) / 4.0);  // 16-bit values sit in registers of their own
-    }
     const uint64_t vectors = (rg.R + vec - 1) / vec;  // the last one is partial when tail != 0
     auto budget = [](uint64_t lanes) { return lanes <= 512 ? 160.0 : 96.0; };
     // Measured on MI355X (softmax and normalisation, rows of 128 to 8192 elements): two 16-byte vectors per lane up to one
@@ -386,12 +379,32 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     // 64 registers, and only after that more lanes.
     const double softTarget = 64.0;
     const uint64_t vectorsPerLane = narrow < wide ? 4 : 2;  // narrow-side words are half words: take twice as many
-    uint64_t T = 1;
-    while (T < 256 && T * vectorsPerLane < vectors) T <<= 1;
-    while (T < 1024 && T < vectors && (vectors + T - 1) / T * vec * registersPerElement > softTarget) T <<= 1;
-    while (T < 1024 && ((vectors + T - 1) / T * vec > 64 || (vectors + T - 1) / T * vec * registersPerElement > budget(T))) T <<= 1;
-    const uint64_t items = (vectors + T - 1) / T;
-    if (items * vec > 64 || items * vec * registersPerElement > budget(T)) return false;  // the row does not fit one block's registers
+    uint64_t T = 1, items = 0;
+    auto sizeBlock = [&](bool withArrays) {
+        double registersPerElement = 0.0;
+        for (uint32_t sNode : em.sourceNodes)
+            if (isElem(rg.cls[sNode])) registersPerElement += dataTypeSizeInBytes(ctx.tensorOf[sNode].getDataType()) / 4.0;
+        for (uint32_t m : members) {
+            if (!withArrays || !needsArray[m]) continue;
+            const DataType dt = ctx.role[m] == Role::Materialized ? expr.nodes[m].output_dtype.value() : emittedValueDType(expr.nodes[m]);
+            registersPerElement += std::max(1.0, dataTypeSizeInBytes(dt) / 4.0);  // 16-bit values sit in registers of their own
+        }
+        T = 1;
+        while (T < 256 && T * vectorsPerLane < vectors) T <<= 1;
+        while (T < 1024 && T < vectors && (vectors + T - 1) / T * vec * registersPerElement > softTarget) T <<= 1;
+        while (T < 1024 && ((vectors + T - 1) / T * vec > 64 || (vectors + T - 1) / T * vec * registersPerElement > budget(T))) T <<= 1;
+        items = (vectors + T - 1) / T;
+        return !(items * vec > 64 || items * vec * registersPerElement > budget(T));
+    };
+    // A row whose values would not fit next to it keeps only the row itself in registers: values that a later loop needs are
+    // computed again there from the row (every per-element value is a function of the sources and of per-row values) -- for
+    // softmax a second exponential per element instead of a register per element.
+    bool recompute = false;
+    if (!sizeBlock(true)) {
+        if (!sizeBlock(false)) return false;  // the row does not fit one block's registers
+        recompute = true;
+        std::fill(needsArray.begin(), needsArray.end(), 0);
+    }
     const bool subWave = T <= 64;
     const uint64_t threads = subWave ? 256 : T;
     const uint64_t rowsPerBlock = subWave ? 256 / T : 1;
@@ -556,6 +569,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         for (const auto& [node, name] : rowDivisorOf) body.defineRowDivisor(node, name);
         std::string text;
         std::set<uint32_t> extracted;
+        std::function<void(uint32_t)> extractRef;
         auto extract = [&](uint32_t c) {
             if (c == UINT32_MAX || body.defined(c) || extracted.count(c)) return;
             if (rg.isSource[c] && isElem(rg.cls[c])) {
@@ -566,13 +580,34 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
                 text += "            const " + std::string(valueCType(valueDType)) + " t" + std::to_string(c) + " = " + value + ";\n";
                 body.defineSource(c, valueDType);
                 extracted.insert(c);
-            } else if (rg.member[c] && isElem(rg.cls[c]) && phase[c] < loop) {
+            } else if (rg.member[c] && isElem(rg.cls[c]) && phase[c] < loop && !recompute) {
                 const DataType dt = ctx.role[c] == Role::Materialized ? expr.nodes[c].output_dtype.value() : emittedValueDType(expr.nodes[c]);
                 text += "            const " + std::string(valueCType(dt)) + " t" + std::to_string(c) + " = v" + std::to_string(c) + "[it][k];\n";
                 body.defineSource(c, dt);
                 extracted.insert(c);
+            } else if (rg.member[c] && isElem(rg.cls[c]) && phase[c] < loop) {
+                // computed again from the row: the same statements as in its own loop (and the same rounding where it is stored)
+                const ExprNode& n = expr.nodes[c];
+                for (uint32_t child : {n.lhs, n.rhs, n.aux}) extractRef(child);
+                double folded;
+                if (tryFoldConstant(expr, c, folded)) {
+                    const DataType dt = emittedValueDType(n);
+                    text += "            const " + std::string(valueCType(dt)) + " t" + std::to_string(c) + " = " + castValueExpr(floatLiteral(folded), DataType::FP32, dt) + ";\n";
+                    body.defineSource(c, dt);
+                } else {
+                    em.flops += body.emit(text, c, "            ") * rg.R;
+                }
+                if (ctx.role[c] == Role::Materialized) {
+                    const DataType outDType = n.output_dtype.value();
+                    if (body.dtypeOf(c) != outDType) {
+                        text += "            const " + std::string(valueCType(outDType)) + " m" + std::to_string(c) + " = " + body.ref(c, outDType) + ";\n";
+                        body.defineSource(c, outDType, "m" + std::to_string(c));
+                    }
+                }
+                extracted.insert(c);
             }
         };
+        extractRef = extract;
         for (uint32_t m : elemNodes) {
             const ExprNode& n = expr.nodes[m];
             for (uint32_t c : {n.lhs, n.rhs, n.aux}) extract(c);
@@ -657,7 +692,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     em.source = s.str();
     em.flops *= rg.rows;
     em.description = "row_fused(rows=" + std::to_string(rg.rows) + ",R=" + std::to_string(rg.R) + ",lanes_per_row=" + std::to_string(T) +
-                     ",items=" + std::to_string(items) + ",vec=" + std::to_string(vec) + (unaligned ? ",unaligned_vectors" : "") + ",loops=" + std::to_string(numLoops) + ")";
+                     ",items=" + std::to_string(items) + ",vec=" + std::to_string(vec) + (unaligned ? ",unaligned_vectors" : "") + (recompute ? ",values_recomputed" : "") + ",loops=" + std::to_string(numLoops) + ")";
     return true;
 }
 
