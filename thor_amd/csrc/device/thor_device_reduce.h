@@ -1004,7 +1004,45 @@ __device__ __forceinline__ void broadcastSegments(const typename Cfg::T* values,
         const u64 rHi = bounds[kWindow] < cEnd ? bounds[kWindow] : cEnd;
         if (rLo < rHi) {
             const u64 vLo = rLo * kE / kVec, vHi = (rHi * kE + kVec - 1) / kVec;
-            for (u64 v = vLo + threadIdx.x; v < vHi; v += Cfg::kThreads) {
+            u64 vFirst = vLo + threadIdx.x;
+            if constexpr (kRowVectors && !Cfg::kIds) {
+                // four vectors of a thread at a time: their searches interleave and their four loads of per-segment values
+                // are in flight together (one vector per round leaves the chain search -> load -> store to wait alone:
+                // 1 GiB written in 223 us; four: see the bench line)
+                constexpr int kRound = 4;
+                for (; vFirst + (u64)(kRound - 1) * Cfg::kThreads < vHi; vFirst += (u64)kRound * Cfg::kThreads) {
+                    int j[kRound];
+                    u64 component[kRound];
+                    bool live[kRound];
+#pragma unroll
+                    for (int u = 0; u < kRound; ++u) {
+                        const u64 e0 = (vFirst + (u64)u * Cfg::kThreads) * kVec;
+                        const u64 row = e0 / kE;
+                        component[u] = e0 % kE;
+                        live[u] = row >= rLo && row < rHi;
+                        const u64 searched = row > rLo ? row : rLo;
+                        j[u] = 0;
+#pragma unroll
+                        for (int step = kWindow / 2; step >= 1; step /= 2) {
+                            if (bounds[j[u] + step] <= searched) j[u] += step;
+                        }
+                    }
+                    Pack<T, kVec> x[kRound];
+#pragma unroll
+                    for (int u = 0; u < kRound; ++u)
+                        if (live[u]) x[u].load(values + (window + j[u]) * kE + component[u]);
+#pragma unroll
+                    for (int u = 0; u < kRound; ++u) {
+                        if (live[u]) {
+                            const u64 length = bounds[j[u] + 1] - bounds[j[u]];
+#pragma unroll
+                            for (int k = 0; k < kVec; ++k) x[u].v[k] = broadcastValue<Cfg>(x[u].v[k], length);
+                            x[u].storeStream(out + (vFirst + (u64)u * Cfg::kThreads) * kVec);
+                        }
+                    }
+                }
+            }
+            for (u64 v = vFirst; v < vHi; v += Cfg::kThreads) {
                 const u64 e0 = v * kVec;
                 u64 row = e0 / kE;
                 u64 component = e0 % kE;
