@@ -185,6 +185,56 @@ def test_both_segment_kernels_on_awkward_partitions(stream, monkeypatch, kernel,
                     np.testing.assert_array_equal(got[b], (offsets[b] + winner) * shape[1] + np.arange(shape[1]), err_msg=f"{name} segment {b} {stamped.get_kernel_variant()}")
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_partitions_give_the_same_answer_through_both_kernels(stream, monkeypatch, seed):
+    """Random partitions with many empty and one-row segments, rows of 1 to 260 elements: maxima and winners must agree bit for
+    bit between the two segment kernels and with numpy, sums within the accumulation-order tolerance."""
+    rng = np.random.default_rng(1000 + seed)
+    rows = int(rng.integers(1, 6000))
+    width = int(rng.choice([1, 2, 3, 16, 48, 64, 130, 260]))
+    segments = int(rng.integers(1, 400))
+    style = seed % 3
+    if style == 0:
+        cuts = np.sort(rng.integers(0, rows + 1, segments - 1)) if segments > 1 else np.array([], np.int64)
+    elif style == 1:  # geometric lengths: mostly tiny segments, a few long ones
+        lengths = rng.geometric(0.3, segments) - 1
+        cuts = np.minimum(np.cumsum(lengths)[:-1], rows) if segments > 1 else np.array([], np.int64)
+    else:  # one long segment among empties
+        cuts = np.sort(rng.choice([0, rows // 3, rows], segments - 1)) if segments > 1 else np.array([], np.int64)
+    last = int(rng.integers(cuts[-1] if len(cuts) else 0, rows + 1))
+    offsets = np.concatenate([[0], cuts, [last]]).astype(np.int64)
+    dtype = [DataType.fp32, DataType.fp16, DataType.bf16][seed % 3]
+    x = to_storage(rng.integers(-6, 7, (rows, width)).astype(np.float32) / 4, dtype)  # few distinct values: ties everywhere
+    xf = from_storage(x, dtype).astype(np.float64)
+    tx = copy_numpy_to_gpu(x, stream, dtype)
+    toff = upload_offsets(offsets, stream)
+    results = {}
+    for kernel in ("teams", "rows"):
+        monkeypatch.setenv("THOR_SEGMENT_KERNEL", kernel)
+        stamped = ph.CubSegmentedReduction(ph.CubReductionOp.Max, DataType.fp32).stamp(tx, toff, stream)
+        stamped.run()
+        maxima = gpu_to_f32(stamped.get_output_tensor(), stream)
+        stamped = ph.CubSegmentedReduction(ph.CubReductionOp.Sum, DataType.fp32).stamp(tx, toff, stream)
+        stamped.run()
+        sums = gpu_to_f32(stamped.get_output_tensor(), stream)
+        stamped = ph.CubSegmentedArgReduction(ph.CubArgReductionOp.ArgMin, DataType.uint32).stamp(tx, toff, stream)
+        stamped.run()
+        winners = copy_gpu_to_numpy(stamped.get_index_output_tensor(), stream)
+        results[kernel] = (maxima, sums, winners)
+    np.testing.assert_array_equal(results["teams"][0], results["rows"][0])
+    np.testing.assert_array_equal(results["teams"][2], results["rows"][2])
+    np.testing.assert_array_equal(results["rows"][0].reshape(segments, width), segment_reference(xf, offsets, "Max").astype(np.float32))
+    np.testing.assert_array_equal(results["rows"][1].reshape(segments, width), segment_reference(xf, offsets, "Sum").astype(np.float32))  # quarters: exact
+    flat = xf.reshape(rows, width)
+    got = results["rows"][2].reshape(segments, width)
+    for b in range(segments):
+        piece = flat[offsets[b]:offsets[b + 1]]
+        if piece.shape[0] == 0:
+            assert np.all(got[b] == np.iinfo(np.uint32).max)
+        else:
+            np.testing.assert_array_equal(got[b], (offsets[b] + piece.argmin(axis=0)) * width + np.arange(width))
+
+
 def test_offsets_are_read_at_run_time_and_outputs_are_reused(stream):
     """CubOffsetSegmentedReductionTest.cpp:239-295: runtime offsets are not inspected by the stamp; a stamped reduction follows the
     partition that is in the offsets tensor when it runs."""
