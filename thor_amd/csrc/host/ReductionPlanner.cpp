@@ -405,6 +405,10 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
     // Strided: arbitrary kept / reduced axes, including views and the affine rank-1 whole-tensor case.
     shape.kernel = ReductionShape::Kernel::Strided;
     shape.threads = 256;
+    if (const char* env = std::getenv("THOR_STRIDED_THREADS")) {  // tuning switch: threads per block
+        const long requested = std::atol(env);
+        if (requested == 256 || requested == 512 || requested == 1024) shape.threads = static_cast<int>(requested);
+    }
     for (size_t a = 0; a < g.indexing.retained_axes.size(); ++a) {
         shape.keptDims.push_back(g.indexing.retained_dimensions[a]);
         shape.keptStrides.push_back(g.indexing.input_strides[g.indexing.retained_axes[a]]);
@@ -484,7 +488,15 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
     }
     const uint64_t reductionVectors = g.reduction_size / shape.vec;
     const uint64_t outputs = g.output_elements;
-    if (outputs < 2048 && reductionVectors > 256ull * 8) {
+    // About one output per compute unit or more, each over a long reduction: one 1024-thread block per output reads it whole.
+    // Nothing is split, so no share waits to fold the others (per-channel sums of [64, 256, 56, 56] fp16, 98 MiB: 20.5 us as
+    // 16 shares of 256 threads per channel with the last share folding, 18.1 us this way).
+    // (Not with an elementwise output: twice the bytes per launch make the fold a smaller share, 38.3 against 39.5 us.)
+    const bool wholeOutputs = outputs >= 192 && outputs < 2048 && reductionVectors >= 1024ull * 16 && request.elementwise.empty() && std::getenv("THOR_STRIDED_BLOCKS") == nullptr &&
+                              std::getenv("THOR_STRIDED_THREADS") == nullptr;
+    if (wholeOutputs) {
+        shape.threads = 1024;
+    } else if (outputs < 2048 && reductionVectors > 256ull * 8) {
         uint64_t wantedBlocks = 4096;
         if (const char* env = std::getenv("THOR_STRIDED_BLOCKS")) wantedBlocks = std::max<long>(std::atol(env), 1);  // tuning switch
         shape.split = std::min<uint64_t>({ceilDiv(wantedBlocks, outputs), reductionVectors / (256ull * 4), kMaxGridY});
