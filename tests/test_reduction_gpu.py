@@ -67,6 +67,8 @@ SHAPES = [
     ([4, 6, 10, 12], [0, 2, 3]), ([3, 4, 5, 6], [1, 3]), ([2, 3, 4, 5, 2], [0, 2, 4]), ([8, 16, 32], [0, 2]),
     # rows no vector divides: vectors at addresses aligned to the element only, the rest of the row one by one
     ([100, 1001], [1]), ([37, 50257], [1]), ([5000, 63], [1]), ([3, 70001], [1]), ([9, 131], [1]),
+    # a middle axis over an inner extent of a few elements: the rows kernel with one accumulator per inner element
+    ([64, 300, 4], [1]), ([4096, 50, 2], [1]), ([33, 1000, 4], [1]), ([7, 5, 2, 2], [1]), ([2000, 6, 4], [1]),
 ]
 
 
@@ -136,6 +138,20 @@ def test_rows_no_vector_divides_and_rows_that_begin_off_a_vector(stream, dtype):
         rows = np.stack([carrier[r * row_stride:r * row_stride + 1000] for r in range(rows_in_view)])
         np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream), oracle.reduce_f64(oracle.MAX, rows, int(dtype), [1]).astype(np.float32),
                                       err_msg=stamped.get_kernel_variant())
+
+
+def test_small_inner_extents_take_the_rows_kernel_with_interleaved_outputs(stream):
+    x = np.arange(64 * 300 * 4, dtype=np.float32).reshape(64, 300, 4) % 17
+    t = copy_numpy_to_gpu(x, stream, DataType.fp32)
+    stamped = ph.CubReduction(ph.CubReductionOp.Sum, [1], DataType.fp32).stamp(t, stream)
+    assert "outputs_per_row=4" in stamped.get_kernel_variant(), stamped.get_kernel_variant()
+    stamped.run()
+    np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream).reshape(64, 4), x.sum(axis=1))  # small integers: exact
+    arg = ph.CubArgReduction(ph.CubArgReductionOp.ArgMax, [1], value_output_dtype=DataType.fp32, index_output_dtype=DataType.uint32).stamp(t, stream)
+    assert "outputs_per_row=4" in arg.get_kernel_variant(), arg.get_kernel_variant()
+    arg.run()
+    np.testing.assert_array_equal(copy_gpu_to_numpy(arg.get_index_output_tensor(), stream).reshape(64, 4), x.argmax(axis=1).astype(np.uint32))
+    np.testing.assert_array_equal(gpu_to_f32(arg.get_value_output_tensor(), stream).reshape(64, 4), x.max(axis=1))
 
 
 def test_output_dtypes_scale_and_fp8_saturation(stream):

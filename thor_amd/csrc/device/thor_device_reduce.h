@@ -175,8 +175,13 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
     const bool rowLive = row < Cfg::kOuter;
     const u64 rowBase = (rowLive ? row : 0) * Cfg::kR;
 
-    Acc acc;
-    acc.reset();
+    // kInterleave > 1: the row holds kInterleave outputs element by element ([outer, R, inner] with an inner extent that
+    // divides the vector): element e of the row belongs to output e % kInterleave and to reduction position e / kInterleave
+    constexpr int J = Cfg::kInterleave;
+    static_assert(Cfg::kVec % J == 0 && (J == 1 || Cfg::kSplit == 1), "interleaved outputs: whole groups per vector, rows not split");
+    Acc acc[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) acc[j].reset();
     typename Cfg::Kept kept;
     Cfg::loadKept(src, rowLive ? row : 0, kept);
     constexpr int kBatch = kIters >= 8 ? 8 : (int)(kIters > 0 ? kIters : 1);
@@ -194,7 +199,7 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
             if (live[u]) {
                 const u64 v = vBegin + (it + u) * TPR + lane;
 #pragma unroll
-                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc, x[u], src, kept, k, (IndexT)(v * Cfg::kVec + k));
+                for (int k = 0; k < Cfg::kVec; ++k) Cfg::accumulateOne(acc[k % J], x[u], src, kept, k, (IndexT)((v * Cfg::kVec + k) / J));
                 Cfg::template elementwise<0>(src, out, rowBase + v * Cfg::kVec, x[u], &kept);
             }
         }
@@ -207,22 +212,25 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
             for (u64 t = (u64)lane; t < kTail; t += TPR) {
                 typename Cfg::Loaded x;
                 Cfg::loadFirstOnly(src, rowBase + kVectorsPerRow * Cfg::kVec + t, x);
-                Cfg::accumulateOne(acc, x, src, kept, 0, (IndexT)(kVectorsPerRow * Cfg::kVec + t));
+                Cfg::accumulateOne(acc[0], x, src, kept, 0, (IndexT)(kVectorsPerRow * Cfg::kVec + t));
             }
         }
     }
     if (kSubWave) {
-        groupReduce<TPR>(acc);
+#pragma unroll
+        for (int j = 0; j < J; ++j) groupReduce<TPR>(acc[j]);
     } else {
-        __shared__ Acc scratch[Cfg::kThreads / kWave];
-        blockReduce<Cfg::kThreads, false>(acc, scratch);
+        __shared__ Acc scratch[J][Cfg::kThreads / kWave];
+#pragma unroll
+        for (int j = 0; j < J; ++j) blockReduce<Cfg::kThreads, false>(acc[j], scratch[j]);
     }
     if (lane == 0 && rowLive) {
         if (Cfg::kSplit > 1) {
-            acc.template storePartial<Cfg::kTickets>(partials, row * Cfg::kSplit + segment, Cfg::kOuter * Cfg::kSplit);
+            acc[0].template storePartial<Cfg::kTickets>(partials, row * Cfg::kSplit + segment, Cfg::kOuter * Cfg::kSplit);
             if (Cfg::kTickets) partialsWritten();
         } else {
-            Cfg::store(acc, row, out, scale);
+#pragma unroll
+            for (int j = 0; j < J; ++j) Cfg::store(acc[j], row * J + j, out, scale);
         }
     }
     if (Cfg::kTickets && Cfg::kSplit > 1 && !kSubWave && rowLive) {  // one row per block: the row's last share folds

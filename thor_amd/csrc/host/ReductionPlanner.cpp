@@ -168,6 +168,7 @@ std::string ReductionShape::describe() const {
         case Kernel::Rows:
             out << "rows(lanes_per_row=" << threadsPerRow << ",split=" << split;
             if (unalignedVectors) out << ",unaligned_vectors";
+            if (interleave > 1) out << ",outputs_per_row=" << interleave;
             break;
         case Kernel::Columns:
             out << (laneAxis < 0 ? "columns(lanes_x=" : "view_columns(lanes_x=") << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
@@ -364,6 +365,35 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
     }
 
     if (g.path == CubReductionPath::TiledFixedSegment) {
+        // [outer, R, inner] with an inner extent of a few elements (a 16-byte vector holds a whole number of inner rows): lanes
+        // across the outputs would each walk a stream of their own, 16 bytes at a time.  The rows kernel reads the
+        // contiguous row of R * inner elements instead and keeps one accumulator per inner element
+        // ([4096, 4096, 4] fp32 over the middle axis: 178 us with lanes across outputs).
+        {
+            const uint64_t innerBytes = g.inner_size * elementBytes;
+            bool keptSources = false;
+            for (const ReductionKernelRequest::Source& source : request.sources) keptSources = keptSources || source.kind != ReductionKernelRequest::Source::Kind::Vector;
+            const int vec = static_cast<int>(16 / elementBytes);
+            const uint64_t rowElements = g.reduction_size * g.inner_size;
+            const bool denseOutput = g.tiled_output_inner_stride == 1 && g.tiled_output_outer_stride == g.inner_size;
+            if (g.inner_size > 1 && innerBytes <= 16 && 16 % innerBytes == 0 && !keptSources && request.elementwise.empty() && denseOutput &&
+                rowElements % vec == 0 && request.inputAlignmentBytes % 16 == 0 && std::getenv("THOR_REDUCE_NO_INTERLEAVE") == nullptr) {
+                const uint64_t vectorsPerRow = rowElements / vec;
+                uint64_t lanes = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(ceilDiv(vectorsPerRow, 8)), 1), 1024);
+                lanes = std::max<uint64_t>(lanes, std::min<uint64_t>(8, pow2Ceil(vectorsPerRow)));
+                if (g.outer_size * lanes >= kTargetThreads || vectorsPerRow <= lanes * 16) {  // enough rows that none has to be split
+                    shape.kernel = ReductionShape::Kernel::Rows;
+                    shape.vec = vec;
+                    shape.interleave = static_cast<int>(g.inner_size);
+                    shape.threadsPerRow = static_cast<int>(lanes);
+                    shape.threads = lanes <= 64 ? 256 : static_cast<int>(lanes);
+                    const uint64_t rowsPerBlock = lanes <= 64 ? 256 / lanes : 1;
+                    shape.gridX = static_cast<uint32_t>(ceilDiv(g.outer_size, rowsPerBlock));
+                    shape.gridY = 1;
+                    return shape;
+                }
+            }
+        }
         shape.kernel = ReductionShape::Kernel::Columns;
         shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.inner_size});
         shape.threads = 256;
@@ -667,7 +697,8 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             break;
         case ReductionShape::Kernel::Rows:
             s << "    static constexpr u64 kOuter = " << g.outer_size << "ull;\n";
-            s << "    static constexpr u64 kR = " << g.reduction_size << "ull;\n";
+            s << "    static constexpr u64 kR = " << g.reduction_size * static_cast<uint64_t>(shape.interleave) << "ull;\n";  // elements of a row
+            s << "    static constexpr int kInterleave = " << shape.interleave << ";\n";
             s << "    static constexpr int kThreadsPerRow = " << shape.threadsPerRow << ";\n";
             body = "thor::reduceRows<gen::Cfg>(src, out, partials, scale);";
             break;

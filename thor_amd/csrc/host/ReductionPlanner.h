@@ -96,6 +96,8 @@ struct ReductionShape {
     bool segmentsByRows = false;
     // Rows kernel: vectors at addresses that are only aligned to the element; the last reduction_size % vec elements of a row go one by one
     bool unalignedVectors = false;
+    // Rows kernel over [outer, R, inner] with a small inner extent: outputs per row, their elements interleaved along the row
+    int interleave = 1;
     int walkGroup = 4;  // reduceSegmentsByRows: rows of a lane's range that are walked together
     std::string describe() const;
 };
