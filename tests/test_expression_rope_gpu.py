@@ -106,6 +106,8 @@ LAYOUTS = [
     ((2, 4, 200, 64), {"scaling_kind": RotaryScalingKind.yarn, "scaling_factor": 4.0, "original_max_position_embeddings": 64}),
     ((2, 4, 200, 64), {"scaling_kind": RotaryScalingKind.dynamic_ntk, "scaling_factor": 2.0, "original_max_position_embeddings": 64}),
     ((2, 4, 200, 64), {"scaling_kind": RotaryScalingKind.linear, "scaling_factor": 4.0}),
+    # halves that are not whole 64-byte sectors: two adjacent lanes share the pairs
+    ((2, 3, 50, 80), {}), ((2, 3, 33, 96), {"position_offset": 4}), ((3, 2, 40, 128), {"rotary_dim": 80}), ((2, 2, 17, 48), {"inverse": True}),
 ]
 
 
@@ -248,6 +250,28 @@ def test_walking_and_tiled_kernels_agree(stream, monkeypatch):
         results.append((plan.stage_descriptions()[-1], copy_gpu_to_numpy(plan.output("y"), stream)))
     assert "tile=" in results[0][0] and "walk=" in results[1][0] and "walk=15/1," in results[2][0]
     assert np.array_equal(results[0][1], results[1][1]) and np.array_equal(results[1][1], results[2][1])
+
+
+@pytest.mark.parametrize("dtype", [DataType.bf16, DataType.fp32], ids=lambda d: d.name)
+def test_lanes_that_share_pairs_give_the_bits_of_lanes_that_own_them(stream, monkeypatch, dtype):
+    """Head dimensions whose halves are not whole 64-byte sectors (80, 96; a partly rotated 128) pair adjacent lanes: each reads,
+    turns and writes one of the two vectors of a pair.  Switched off, one lane owns both; the results must be the same bits,
+    with a fused elementwise neighbour as well."""
+    rng = np.random.default_rng(80)
+    for shape, options in (((2, 5, 70, 80), {}), ((1, 3, 129, 96), {"position_offset": 11}), ((2, 2, 64, 128), {"rotary_dim": 80})):
+        x = to_storage(rng.standard_normal(shape).astype(np.float32), dtype)
+        t = copy_numpy_to_gpu(x, stream, dtype)
+        for build in (lambda v: v.rope(**options), lambda v: (v * 2.0 + 1.0).rope(**options) * 0.5):
+            results = []
+            for off in (False, True):
+                monkeypatch.delenv("THOR_ROPE_NO_PAIRED_LANES", raising=False)
+                if off:
+                    monkeypatch.setenv("THOR_ROPE_NO_PAIRED_LANES", "1")
+                plan = run({"y": build(ex.input("x"))}, {"x": t}, stream)
+                results.append((plan.stage_descriptions()[-1], copy_gpu_to_numpy(plan.output("y"), stream)))
+            half_bytes = options.get("rotary_dim", shape[3]) // 2 * (2 if dtype == DataType.bf16 else 4)
+            assert ("paired_lanes" in results[0][0]) == (half_bytes % 64 != 0) and "paired_lanes" not in results[1][0], results[0][0]
+            assert np.array_equal(results[0][1], results[1][1])
 
 
 def test_rotation_inside_a_larger_graph(stream):

@@ -176,7 +176,15 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     const uint64_t pairSlots = n.rope_interleaved ? (vec > 1 ? rotary / vec : half) : half / vec;
     const int pairsPerThread = n.rope_interleaved ? (vec > 1 ? vec / 2 : 1) : vec;
     const uint64_t slots = pairSlots + tail / vec;
-    const uint64_t items = seq * slots;
+    // Half-rotated layout whose halves are not whole 64-byte sectors (head dimensions of 80 or 96 halves, 80 floats): a lane
+    // that reads both vectors of its pairs touches every sector of the row in each of its two loads and uses part of it.  Two
+    // adjacent lanes then share the pairs: each reads, turns and writes one of the two vectors and gets the other operand from
+    // its neighbour, so one load of the wavefront covers the rows whole ([8, 32, 4096, 80] bf16: 137 us the other way).
+    uint32_t narrowest = 8;
+    for (const Tensor& t : streamed) narrowest = std::min<uint32_t>(narrowest, dataTypeSizeInBytes(t.getDataType()));
+    const bool pairedLanes = !n.rope_interleaved && vec > 1 && (half * narrowest) % 64 != 0 && std::getenv("THOR_ROPE_NO_PAIRED_LANES") == nullptr;
+    const uint64_t walkSlots = pairedLanes ? (2 * pairSlots + tail / vec + 1) / 2 * 2 : slots;  // an even count keeps the two lanes of a pair adjacent
+    const uint64_t items = seq * walkSlots;
     const uint32_t threads = 256;
     const uint64_t blocksPerChunk = (items + threads - 1) / threads;
     // Many blocks, each thread walking at least two coordinates with its angles (measured on [8, 32, 4096, 128] bf16: 88 us
@@ -405,7 +413,7 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     s << "    const thor::u64 chunk = blockIdx.x / " << blocksPerChunk << "u;\n";
     s << "    const thor::u64 item = (thor::u64)(blockIdx.x % " << blocksPerChunk << "u) * " << threads << " + threadIdx.x;\n";
     s << "    if (item >= " << items << "ull) return;\n";
-    s << "    const thor::u64 position = item / " << slots << "ull, slot = item % " << slots << "ull;\n";
+    s << "    const thor::u64 position = item / " << walkSlots << "ull, slot = item % " << walkSlots << "ull;\n";
     s << "    const thor::u64 walkFirst = chunk * " << walkPerChunk << "ull;\n";
     s << "    const thor::u64 walkLast = walkFirst + " << walkPerChunk << "ull < " << walk << "ull ? walkFirst + " << walkPerChunk << "ull : " << walk << "ull;\n";
     // address of (walk coordinate w, this position, head-dimension coordinate d)
@@ -414,16 +422,22 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
       << "ull;\n";
     s << "        return o * " << outerStride << "ull + m * " << middleStride << "ull + i + position * " << seqStride << "ull + d * " << dimStride << "ull;\n";
     s << "    };\n";
-    if (tail != 0) {
-        s << "    if (slot >= " << pairSlots << "ull) {\n";
+    const uint64_t turningSlots = pairedLanes ? 2 * pairSlots : pairSlots;
+    if (tail != 0 || walkSlots != turningSlots) {
+        s << "    if (slot >= " << turningSlots << "ull) {\n";
+        if (walkSlots != turningSlots + tail / vec) s << "        if (slot >= " << turningSlots + tail / vec << "ull) return;  // the slot that makes the count even\n";
         s << "        // beyond the rotary part: a copy\n";
-        s << "        const thor::u64 d = " << rotary << "ull + (slot - " << pairSlots << "ull) * V;\n";
+        s << "        const thor::u64 d = " << rotary << "ull + (slot - " << turningSlots << "ull) * V;\n";
         s << "        for (thor::u64 w = walkFirst; w < walkLast; ++w) {\n";
         s << "            const thor::u64 e = at(w, d);\n";
         s << copySite("            ", "e");
         s << "        }\n        return;\n    }\n";
     }
-    s << "    const thor::u64 firstPair = slot * P;\n";
+    if (pairedLanes) {
+        s << "    const thor::u64 firstPair = (slot / 2) * P;\n    const bool second = (slot & 1ull) != 0;\n";
+    } else {
+        s << "    const thor::u64 firstPair = slot * P;\n";
+    }
     if (positionIds.has_value()) {
         s << "    float angleBase = thor::toFloat(ids[position]);\n";
     } else {
@@ -446,9 +460,22 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     }
     if (n.rope_inverse) s << "        sn[k] = -sn[k];\n";
     s << "    }\n";
+    if (pairedLanes) {
+        // own * cos + other * (+-sin): the first lane of a pair holds a (a cos - b sin), the second b (b cos + a sin)
+        s << "    float turn[P];\n#pragma unroll\n    for (int k = 0; k < P; ++k) turn[k] = second ? sn[k] : -sn[k];\n";
+    }
     s << "#pragma unroll 1\n";
     s << "    for (thor::u64 w = walkFirst; w < walkLast; ++w) {\n";
-    if (pairsInsideVector) {
+    if (pairedLanes) {
+        s << "        const thor::u64 e = at(w, firstPair + (second ? " << apart << "ull : 0ull));\n";
+        s << loadSite("        ", "p", "e");
+        s << "        thor::Pack<" << outType << ", V> q;\n";
+        s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
+        s << operandOf("            ", "a", "p", "k");
+        s << "            const float b = __shfl_xor(a, 1);\n";
+        s << resultTo("            ", "q", "p", "k", "a * cs[k] + b * turn[k]");
+        s << "        }\n        q.storeStream(out + e);\n";
+    } else if (pairsInsideVector) {
         s << "        const thor::u64 e = at(w, firstPair * 2);\n";
         s << turnInsideVector("        ", "e");
     } else {
@@ -466,7 +493,7 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     if (tiled) {
         description << ",tile=" << tilePositions << "x" << middleCount;
     } else {
-        description << ",walk=" << walk << "/" << chunks;
+        description << ",walk=" << walk << "/" << chunks << (pairedLanes ? ",paired_lanes" : "");
     }
     description << ",vec=" << vec << ",grid=" << blocks << ") [" << kernel->kernelName << "]";
     std::vector<Tensor> inputs;
