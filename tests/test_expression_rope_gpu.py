@@ -108,6 +108,7 @@ LAYOUTS = [
     ((2, 4, 200, 64), {"scaling_kind": RotaryScalingKind.linear, "scaling_factor": 4.0}),
     # halves that are not whole 64-byte sectors: two adjacent lanes share the pairs
     ((2, 3, 50, 80), {}), ((2, 3, 33, 96), {"position_offset": 4}), ((3, 2, 40, 128), {"rotary_dim": 80}), ((2, 2, 17, 48), {"inverse": True}),
+    ((2, 50, 3, 80), {"sequence_axis": 1, "head_dim_axis": 3}), ((2, 19, 6, 96), {"sequence_axis": 1, "head_dim_axis": 3, "rotary_dim": 80}),
 ]
 
 
@@ -258,7 +259,8 @@ def test_lanes_that_share_pairs_give_the_bits_of_lanes_that_own_them(stream, mon
     turns and writes one of the two vectors of a pair.  Switched off, one lane owns both; the results must be the same bits,
     with a fused elementwise neighbour as well."""
     rng = np.random.default_rng(80)
-    for shape, options in (((2, 5, 70, 80), {}), ((1, 3, 129, 96), {"position_offset": 11}), ((2, 2, 64, 128), {"rotary_dim": 80})):
+    for shape, options in (((2, 5, 70, 80), {}), ((1, 3, 129, 96), {"position_offset": 11}), ((2, 2, 64, 128), {"rotary_dim": 80}),
+                           ((2, 70, 5, 80), {"sequence_axis": 1, "head_dim_axis": 3}), ((3, 33, 4, 128), {"sequence_axis": 1, "head_dim_axis": 3, "rotary_dim": 48})):
         x = to_storage(rng.standard_normal(shape).astype(np.float32), dtype)
         t = copy_numpy_to_gpu(x, stream, dtype)
         for build in (lambda v: v.rope(**options), lambda v: (v * 2.0 + 1.0).rope(**options) * 0.5):

@@ -202,10 +202,10 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     // streams the run, every head reading the same table.
     const bool tileLayout = middleCount > 1 && innerCount == 1 && dimStride == 1 && seqAxis < dimAxis && std::getenv("THOR_ROPE_NO_TILES") == nullptr;
     uint64_t tilePositions = std::max<uint64_t>(1, threads / half);
-    while (tilePositions * middleCount * slots < 2 * threads && tilePositions * 2 * half <= 4096) tilePositions *= 2;
+    while (tilePositions * middleCount * walkSlots < 2 * threads && tilePositions * 2 * half <= 4096) tilePositions *= 2;
     tilePositions = std::min(tilePositions, seq);
     const uint64_t tiles = (seq + tilePositions - 1) / tilePositions;
-    const bool tileFits = tilePositions * middleCount * slots < (1ull << 31);  // the tiled kernel counts a block's items in 32 bits
+    const bool tileFits = tilePositions * middleCount * walkSlots < (1ull << 31);  // the tiled kernel counts a block's items in 32 bits
     const bool tiled = tileLayout && tileFits;
     const uint64_t blocks = tiled ? outerCount * tiles : blocksPerChunk * chunks;
     if (blocks > 0x7fffffffull) throw std::runtime_error("RoPE: the tensor is too large for one launch.");
@@ -379,20 +379,35 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "    __syncthreads();\n";
         s << "    const thor::u64 base = outer * " << outerStride << "ull + firstPosition * " << seqStride << "ull;\n";
         s << "    const thor::u64 left = " << seq << "ull - firstPosition;\n";
-        s << "    const thor::u32 liveItems = (thor::u32)(left < " << tilePositions << "ull ? left : " << tilePositions << "ull) * " << middleCount * slots << "u;\n";
+        const uint64_t tileTurningSlots = pairedLanes ? 2 * pairSlots : pairSlots;
+        s << "    const thor::u32 liveItems = (thor::u32)(left < " << tilePositions << "ull ? left : " << tilePositions << "ull) * " << middleCount * walkSlots << "u;\n";
         s << "    for (thor::u32 item = threadIdx.x; item < liveItems; item += " << threads << "u) {\n";
-        s << "        const thor::u32 row = item / " << slots << "u, slot = item % " << slots << "u;\n";
+        s << "        const thor::u32 row = item / " << walkSlots << "u, slot = item % " << walkSlots << "u;\n";
         s << "        const thor::u64 rowBase = base + (thor::u64)row * " << headDim << "ull;\n";
-        if (tail != 0) {
-            s << "        if (slot >= " << pairSlots << "u) {\n";
-            s << "            const thor::u64 e = rowBase + " << rotary << "ull + (slot - " << pairSlots << "u) * V;\n";
+        if (tail != 0 || walkSlots != tileTurningSlots) {
+            s << "        if (slot >= " << tileTurningSlots << "u) {\n";
+            if (walkSlots != tileTurningSlots + tail / vec) s << "            if (slot >= " << tileTurningSlots + tail / vec << "u) continue;  // the slot that makes the count even\n";
+            s << "            const thor::u64 e = rowBase + " << rotary << "ull + (slot - " << tileTurningSlots << "u) * V;\n";
             s << copySite("            ", "e");
             s << "            continue;\n        }\n";
         }
-        s << "        const thor::u32 firstPair = slot * P;\n";
+        if (pairedLanes) {
+            s << "        const thor::u32 firstPair = (slot / 2u) * P;\n        const bool second = (slot & 1u) != 0;\n";
+        } else {
+            s << "        const thor::u32 firstPair = slot * P;\n";
+        }
         s << "        const float* sn = sines + (row / " << middleCount << "u) * " << half << "u + firstPair;\n";
         s << "        const float* cs = cosines + (row / " << middleCount << "u) * " << half << "u + firstPair;\n";
-        if (pairsInsideVector) {
+        if (pairedLanes) {
+            s << "        const thor::u64 e = rowBase + firstPair + (second ? " << apart << "u : 0u);\n";
+            s << loadSite("        ", "p", "e");
+            s << "        thor::Pack<" << outType << ", V> q;\n";
+            s << "#pragma unroll\n        for (int k = 0; k < V; ++k) {\n";
+            s << operandOf("            ", "a", "p", "k");
+            s << "            const float b = __shfl_xor(a, 1);\n";
+            s << resultTo("            ", "q", "p", "k", "a * cs[k] + b * (second ? sn[k] : -sn[k])");
+            s << "        }\n        q.storeStream(out + e);\n";
+        } else if (pairsInsideVector) {
             s << "        const thor::u64 e = rowBase + firstPair * 2;\n";
             s << turnInsideVector("        ", "e");
         } else {
@@ -491,7 +506,7 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     description << "rope(seq=" << seq << ",head_dim=" << headDim << ",rotary=" << rotary << (n.rope_interleaved ? ",interleaved" : "")
                 << (n.rope_inverse ? ",inverse" : "");
     if (tiled) {
-        description << ",tile=" << tilePositions << "x" << middleCount;
+        description << ",tile=" << tilePositions << "x" << middleCount << (pairedLanes ? ",paired_lanes" : "");
     } else {
         description << ",walk=" << walk << "/" << chunks << (pairedLanes ? ",paired_lanes" : "");
     }
