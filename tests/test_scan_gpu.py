@@ -120,7 +120,7 @@ def test_offset_segmented_scans(stream, dtype, op, inclusive, reverse, offsets_d
         np.testing.assert_array_equal(got[:active], expected[:active])
     else:
         check(got[:active], carrier[:active], dtype, op, inclusive, reverse, offsets=offsets)
-    assert "segments(" in variant and "totals+carries+scan" in variant
+    assert "segments(" in variant and "published_totals" in variant
 
 
 def test_full_size_properties(stream):
@@ -160,3 +160,40 @@ def test_validation(stream):
         ph.scan(x, gpu_tensor([64], DataType.fp32), stream, segment_size=7)
     with pytest.raises(ValueError, match="offsets must be UINT32 or UINT64"):
         ph.scan(x, gpu_tensor([64], DataType.fp32), stream, segment_offsets=copy_numpy_to_gpu(np.zeros(3, np.float32), stream, DataType.fp32))
+
+
+@pytest.mark.parametrize("reverse", [False, True], ids=["forward", "reverse"])
+@pytest.mark.parametrize("dtype,op", [(DataType.uint32, ScanOp.sum), (DataType.fp32, ScanOp.min), (DataType.bf16, ScanOp.arg_max),
+                                      (DataType.fp32, ScanOp.sum)], ids=["u32-sum", "fp32-min", "bf16-argmax", "fp32-sum"])
+@pytest.mark.parametrize("n,segments", [(16_800_001, 0), (16_800_001, 3), (1_000_000, 2000)], ids=["flat-4102-chunks", "3-segments", "2000-segments"])
+def test_published_totals_agree_with_separate_passes(stream, monkeypatch, n, segments, dtype, op, reverse):
+    """Chunks that read what precedes them from the totals other blocks publish (one launch over the data) against the same
+    scan with totals and carries computed by launches of their own: the same bits for exact operations; float sums agree with
+    the oracle within the bound of another order of additions and are the same bits from run to run.  The odd length keeps
+    one element per lane and round, so 16.8 million elements are 4102 chunks: all three levels of published totals are read."""
+    rng = np.random.default_rng(47)
+    if dtype == DataType.uint32:
+        carrier = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    else:
+        carrier = to_storage((np.round(rng.standard_normal(n) * 8) / 8).astype(np.float32), dtype)
+    offsets = None
+    if segments:
+        cuts = np.sort(rng.integers(0, n, segments - 1))
+        offsets = np.concatenate([[0], cuts, [n]])
+    got, variant = run_scan(carrier, dtype, stream, op, True, reverse, offsets=offsets)
+    assert "published_totals" in variant, variant
+    again, _ = run_scan(carrier, dtype, stream, op, True, reverse, offsets=offsets)
+    np.testing.assert_array_equal(again.view(np.uint8), got.view(np.uint8))
+    monkeypatch.setenv("THOR_SCAN_PASSES", "3")
+    separate, variant = run_scan(carrier, dtype, stream, op, True, reverse, offsets=offsets)
+    assert "totals+carries+scan" in variant, variant
+    if dtype == DataType.uint32 or op != ScanOp.sum:
+        np.testing.assert_array_equal(got, separate)
+        kwargs = {"offsets": offsets} if segments else {}
+        np.testing.assert_array_equal(got, oracle.scan(carrier, ORACLE_OP[op], True, reverse, dtype=int(dtype), **kwargs))
+    elif segments:
+        check(got, carrier, dtype, op, True, reverse, offsets=offsets)
+        check(separate, carrier, dtype, op, True, reverse, offsets=offsets)
+    else:
+        check(got, carrier, dtype, op, True, reverse)
+        check(separate, carrier, dtype, op, True, reverse)

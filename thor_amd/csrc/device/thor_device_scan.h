@@ -9,15 +9,22 @@
 // state that flows is {value, index of the value (arg scans), "a head lies in the summarised range"}; combining an earlier
 // state with a later one keeps the later one alone when it holds a head.
 //
-// Chunks that start inside a segment need the state of what precedes them.  That takes three launches, none of which
-// waits on another block: the same kernel without stores writes each chunk's total, one block turns the totals into
-// carries, the full kernel applies them.  When segments are rows that chunks hold whole, the single launch is enough.
+// Chunks that start inside a segment need the state of what precedes them.  When segments are rows that chunks hold whole,
+// there is nothing to carry.  Otherwise (Cfg::kLookback) a block takes its chunk by ticket, publishes the chunk's total as
+// soon as it has it, and folds the totals of what precedes it from a fixed tree of base 64: the totals of the earlier chunks
+// of its group of 64, of the earlier groups of its super-group of 64 groups, and of the earlier super-groups (the last chunk
+// of a group publishes the group's total, the last of a super-group that one's).  A block only ever waits for chunks with
+// smaller tickets, which are running or done, and the shape of the fold does not depend on who arrived when: results are
+// the same from run to run.  Every element is read once and written once.  Beyond 64^3 chunks three launches, none of which
+// waits on another block, do the same: the kernel without stores writes each chunk's total, one block turns the totals into
+// carries, the full kernel applies them.
 //
 // A reverse scan walks the same code over mirrored positions (logical p = total - 1 - physical q).
 //
 // Cfg: T (storage), Acc (u32 for UINT32, float otherwise), kUnsigned, kOp (0 sum, 1 min, 2 max, 3 product), kArg, kInclusive, kReverse,
 // kTotal, kRow (row length; 0 = heads come from a bitmap), kThreads, kVec, kItems, kChunkElems (positions per block, a
-// multiple of kVec, at most kThreads * kVec * kItems), kChunks, kCarry, kWriteValue, kWriteIndex.
+// multiple of kVec, at most kThreads * kVec * kItems), kChunks, kCarry, kLookback (with kCarry: what precedes a chunk comes
+// from the published totals, not from a carries array), kClearWords, kWriteValue, kWriteIndex.
 #pragma once
 
 namespace thor {
@@ -157,6 +164,130 @@ struct ScanRunSum {
     static constexpr int kOp = 0;
 };
 
+// ---- published totals (Cfg::kLookback) ----------------------------------------------------------------------------------------
+// The block of memory a scan with published totals works in: 32 control words of 8 bytes (word 0: the ticket counter, word 1:
+// the number of waits that gave up), then one entry of two 8-byte words per chunk, per group and per super-group.  A word
+// holds 32 bits of state above a tag (bit 0: written, bit 1: a head lies in the summarised range); the first word carries
+// the value, the second (min / max only) the index.  Every word is written once per run, whole, after the block was
+// cleared, so a reader that sees the tag sees the state: no fences.
+constexpr u32 kScanControlWords = 32;
+constexpr u32 kScanWaitLimit = 1u << 22;  // polls before a wait gives up (seconds); never reached while earlier tickets run
+
+template <typename Cfg>
+__device__ __forceinline__ void scanPublish(u64* entries, u64 entry, const ScanState<Cfg>& s) {
+    const u64 tag = 1u | (s.head ? 2u : 0u);
+    __hip_atomic_store(entries + 2 * entry, ((u64)__builtin_bit_cast(u32, s.v) << 32) | tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (Cfg::kOp == 1 || Cfg::kOp == 2) {
+        __hip_atomic_store(entries + 2 * entry + 1, ((u64)s.i << 32) | tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// One look at entries [first, first + count), count <= 64, by a whole wavefront: lane l reads entry first + l.
+struct ScanGlimpse {
+    u64 w0, w1;
+};
+template <typename Cfg>
+__device__ __forceinline__ ScanGlimpse scanGlimpse(u64* entries, u64 first, u32 count) {
+    const u32 lane = threadIdx.x % kWave;
+    ScanGlimpse g = {0, 0};
+    if (lane < count) {
+        u64* slot = entries + 2 * (first + lane);
+        g.w0 = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (Cfg::kOp == 1 || Cfg::kOp == 2) g.w1 = __hip_atomic_load(slot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return g;
+}
+
+// The combination, in order, of entries [first, first + count), count <= 64: called by one whole wavefront, lane l waits for
+// entry first + l (`seen`: an earlier look at the same entries, or zeros); every lane returns the result.
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanAwait(u64* entries, u64 first, u32 count, u64* control, ScanGlimpse seen) {
+    typedef ScanState<Cfg> S;
+    constexpr bool kIndexed = Cfg::kOp == 1 || Cfg::kOp == 2;
+    const u32 lane = threadIdx.x % kWave;
+    const bool mine = lane < count;
+    for (u32 polls = 0;; ++polls) {
+        const bool ready = !mine || ((seen.w0 & 1u) != 0 && (!kIndexed || (seen.w1 & 1u) != 0));
+        if (__ballot(!ready) == 0) break;
+        if (polls >= kScanWaitLimit) {
+            if (lane == 0) atomicAdd(reinterpret_cast<u32*>(control + 1), 1u);
+            break;
+        }
+        if (polls) __builtin_amdgcn_s_sleep(1);
+        if (!ready) seen = scanGlimpse<Cfg>(entries, first, count);
+    }
+    S s = scanEmpty<Cfg>();
+    if (mine && (seen.w0 & 1u) != 0 && (!kIndexed || (seen.w1 & 1u) != 0)) {
+        s.v = __builtin_bit_cast(typename Cfg::Acc, (u32)(seen.w0 >> 32));
+        s.i = kIndexed ? (u32)(seen.w1 >> 32) : kNoIndex;
+        s.head = (u32)(seen.w0 >> 1) & 1u;
+    }
+    s = scanWave<Cfg>(s);
+    S all;
+    all.v = __shfl(s.v, kWave - 1, kWave);
+    all.i = kIndexed ? __shfl(s.i, kWave - 1, kWave) : kNoIndex;
+    all.head = __shfl(s.head, kWave - 1, kWave);
+    return all;
+}
+
+// Where chunk `chunk` sits in the tree of totals, and the arrays of the tree inside the block of memory.
+template <typename Cfg>
+struct ScanPlace {
+    u64 *control, *chunkTotals, *groupTotals, *superTotals;
+    u64 group, super;
+    u32 inGroup, inSuper;
+    __device__ __forceinline__ ScanPlace(void* block, u64 chunk) {
+        constexpr u64 kGroups = (Cfg::kChunks + 63) / 64;
+        control = static_cast<u64*>(block);
+        chunkTotals = control + kScanControlWords;
+        groupTotals = chunkTotals + 2 * Cfg::kChunks;
+        superTotals = groupTotals + 2 * kGroups;
+        inGroup = (u32)(chunk % 64);
+        group = chunk / 64;
+        inSuper = (u32)(group % 64);
+        super = group / 64;
+    }
+};
+
+// The totals of earlier groups and super-groups are old news by the time a chunk starts: a first look at them, taken before
+// the chunk's own data is loaded, is usually all it takes.
+template <typename Cfg>
+struct ScanEarlyLook {
+    ScanGlimpse groups, supers;
+};
+template <typename Cfg>
+__device__ __forceinline__ ScanEarlyLook<Cfg> scanLookEarly(void* block, u64 chunk) {
+    const ScanPlace<Cfg> at(block, chunk);
+    ScanEarlyLook<Cfg> early;
+    early.groups = scanGlimpse<Cfg>(at.groupTotals, at.group - at.inSuper, at.inSuper);
+    early.supers = scanGlimpse<Cfg>(at.superTotals, 0, (u32)at.super);
+    return early;
+}
+
+// What precedes chunk `chunk`, given its own total (the same in every lane of the calling wavefront); publishes the totals
+// this chunk owes to later ones.
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanLookBack(void* block, u64 chunk, const ScanState<Cfg>& total, const ScanEarlyLook<Cfg>& early) {
+    typedef ScanState<Cfg> S;
+    const ScanPlace<Cfg> at(block, chunk);
+    const u32 lane = threadIdx.x % kWave;
+    const bool closesGroup = at.inGroup == 63, closesSuper = closesGroup && at.inSuper == 63;
+    if (lane == 0 && !closesGroup) scanPublish<Cfg>(at.chunkTotals, chunk, total);  // the closing chunk's own total has no reader
+    S chunksBefore = scanEmpty<Cfg>(), groupsBefore = scanEmpty<Cfg>(), supersBefore = scanEmpty<Cfg>();
+    const ScanGlimpse nothing = {0, 0};
+    if (at.inGroup > 0) chunksBefore = scanAwait<Cfg>(at.chunkTotals, chunk - at.inGroup, at.inGroup, at.control, nothing);
+    const S groupTotal = scanCombine<Cfg>(chunksBefore, total);
+    if (closesGroup && lane == 0) scanPublish<Cfg>(at.groupTotals, at.group, groupTotal);
+    // a head in what was folded so far cuts off everything earlier: no need to wait for it
+    if (at.inSuper > 0 && (!chunksBefore.head || closesSuper)) {
+        groupsBefore = scanAwait<Cfg>(at.groupTotals, at.group - at.inSuper, at.inSuper, at.control, early.groups);
+    }
+    if (closesSuper && lane == 0) scanPublish<Cfg>(at.superTotals, at.super, scanCombine<Cfg>(groupsBefore, groupTotal));
+    const S lower = scanCombine<Cfg>(groupsBefore, chunksBefore);
+    if (at.super > 0 && !lower.head) supersBefore = scanAwait<Cfg>(at.superTotals, 0, (u32)at.super, at.control, early.supers);
+    return scanCombine<Cfg>(supersBefore, lower);
+}
+
 // bit k set: logical position p + k starts a segment (p is a multiple of kVec)
 template <typename Cfg>
 __device__ __forceinline__ u32 scanHeadBits(const u32* heads, u64 p) {
@@ -188,7 +319,20 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
     // rows that start only where a round of the block starts (or one flat scan): heads need not travel between lanes
     constexpr bool kPlain = Cfg::kRow != 0 && (Cfg::kRow % ((u64)THREADS * V) == 0 || Cfg::kRow == Cfg::kTotal);
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const u64 chunkBase = (u64)blockIdx.x * Cfg::kChunkElems;
+    constexpr bool kLook = Cfg::kLookback && Cfg::kCarry && !AGGREGATE_ONLY && !ROUTE;
+    u64 chunk = blockIdx.x;
+    if constexpr (kLook) {
+        // chunks in the order blocks start: whoever a block waits for has started before it
+        __shared__ u32 ticket;
+        if (threadIdx.x == 0) ticket = atomicAdd(static_cast<u32*>(const_cast<void*>(carries)), 1u);
+        __syncthreads();
+        chunk = ticket;
+    }
+    ScanEarlyLook<Cfg> early = {};
+    if constexpr (kLook) {
+        if (wave == 0) early = scanLookEarly<Cfg>(const_cast<void*>(carries), chunk);
+    }
+    const u64 chunkBase = chunk * Cfg::kChunkElems;
 
     __shared__ u32 totalValue[ITEMS * WAVES], totalIndex[ITEMS * WAVES], totalHead[ITEMS * WAVES];
 
@@ -266,11 +410,19 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
         }
         const S inclusive = scanWave<Cfg>(mine);
         if (AGGREGATE_ONLY) {
-            if (lane == kWave - 1) scanStoreState<Cfg>(aggregates, blockIdx.x, inclusive);
+            if (lane == kWave - 1) scanStoreState<Cfg>(aggregates, chunk, inclusive);
         } else {
             S before = scanShuffleUp<Cfg>(inclusive, 1);
             if (lane == 0) before = scanEmpty<Cfg>();
-            if (Cfg::kCarry) before = scanCombine<Cfg>(scanLoadState<Cfg>(carries, blockIdx.x), before);
+            if constexpr (kLook) {
+                S total;
+                total.v = __shfl(inclusive.v, kWave - 1, kWave);
+                total.i = (Cfg::kOp == 1 || Cfg::kOp == 2) ? __shfl(inclusive.i, kWave - 1, kWave) : kNoIndex;
+                total.head = __shfl(inclusive.head, kWave - 1, kWave);
+                before = scanCombine<Cfg>(scanLookBack<Cfg>(const_cast<void*>(carries), chunk, total, early), before);
+            } else if (Cfg::kCarry) {
+                before = scanCombine<Cfg>(scanLoadState<Cfg>(carries, chunk), before);
+            }
             if (lane < ITEMS * WAVES) {
                 totalValue[lane] = __builtin_bit_cast(u32, before.v);
                 totalIndex[lane] = before.i;
@@ -464,12 +616,13 @@ __device__ __forceinline__ void scanCarries(const void* aggregates, void* carrie
     }
 }
 
-// Segment heads of a row partition as one bit per logical position.  The bitmap is cleared by scanClearHeads first.
+// Segment heads of a row partition as one bit per logical position.  scanClear zeroes the bitmap, and the block of the
+// published totals behind it, first: Cfg::kClearWords words from the start of the temporary storage.
 // Cfg: OffsetT, kSegments, kTotal, kReverse.
 template <typename Cfg>
-__device__ __forceinline__ void scanClearHeads(u32* heads) {
+__device__ __forceinline__ void scanClear(u32* words) {
     const u64 word = (u64)blockIdx.x * blockDim.x + threadIdx.x;
-    if (word < (Cfg::kTotal + 31) / 32) heads[word] = 0;
+    if (word < Cfg::kClearWords) words[word] = 0;
 }
 template <typename Cfg>
 __device__ __forceinline__ void scanMarkHeads(const typename Cfg::OffsetT* offsets, u32* heads) {

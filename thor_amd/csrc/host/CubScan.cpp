@@ -81,8 +81,14 @@ ScanChunking chooseScanChunking(const ScanRequest& r) {
     }
     c.routable = !c.carry && !ragged && (r.op == 1 || r.op == 2);
     if (c.carry) {
-        c.items = std::min<uint64_t>(8, std::max<uint64_t>(maxItems, 1));
-        c.chunkElems = lanesWorth * c.items;
+        // Chunks that wait for each other's totals: the fewer and larger, the fewer tickets and waits.  2^26 fp32 elements, flat:
+        // 256 threads x 8 vectors 162 us, 512 x 8 127 us, 1024 x 4 117 us.  Shorter inputs keep the small chunks that fill the device.
+        uint64_t threads = c.threads;
+        if (!threadsForced && r.total >= 1024ull * 1024 * c.vec * 4) threads = 1024;
+        const uint64_t wavesWorth = 64 / (threads / 64);
+        c.threads = threads;
+        c.items = std::min<uint64_t>(8, std::max<uint64_t>(std::min<uint64_t>(wavesWorth, 16), 1));
+        c.chunkElems = c.threads * c.vec * c.items;
     }
     return c;
 }
@@ -98,7 +104,9 @@ void writeScanTraits(std::ostringstream& s, const ScanRequest& r, bool isUnsigne
       << "ull;\n    static constexpr thor::u64 kSegments = " << r.segments << "ull;\n    static constexpr int kThreads = " << threads
       << ";\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kItems = " << items
       << ";\n    static constexpr thor::u64 kChunkElems = " << chunkElems << "ull;\n    static constexpr thor::u64 kChunks = " << k.chunks
-      << "ull;\n    static constexpr bool kCarry = " << (k.carry ? "true" : "false") << ";\n    static constexpr bool kWriteValue = "
+      << "ull;\n    static constexpr bool kCarry = " << (k.carry ? "true" : "false") << ";\n    static constexpr bool kLookback = "
+      << (k.lookback ? "true" : "false") << ";\n    static constexpr thor::u64 kClearWords = " << k.clearWords
+      << "ull;\n    static constexpr bool kWriteValue = "
       << (r.writeValue ? "true" : "false") << ";\n    static constexpr bool kWriteIndex = " << (r.writeIndex ? "true" : "false") << ";\n};\n}  // namespace gen\n";
 }
 
@@ -137,10 +145,25 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
     if (k.chunks == 1) k.carry = false;
     if (k.chunks > 0x7fffffffull) throw std::invalid_argument("CUB scan: too many elements for one launch.");
 
-    // temporary storage: head bitmap (ragged), chunk totals, chunk carries
+    // Chunks that need what precedes them read it from totals that the blocks publish to each other (one pass over the data);
+    // the fixed tree of those totals is three levels of 64, beyond which (or with THOR_SCAN_PASSES=3) separate launches
+    // compute totals and carries first.
+    const char* passes = std::getenv("THOR_SCAN_PASSES");
+    k.lookback = k.carry && k.chunks <= 64ull * 64 * 64 && !(passes && std::atoi(passes) == 3);
+
+    // temporary storage: head bitmap (ragged), then either the block of published totals (32 control words and two words per
+    // chunk, group and super-group, 8 bytes each) or chunk totals and chunk carries
     k.headsBytes = ragged ? roundUp((r.total + 31) / 32 * 4, 256) : 0;
-    k.statesBytes = k.carry ? roundUp(3 * k.chunks * 4, 256) : 0;
-    k.tempBytes = std::max<size_t>(k.headsBytes + 2 * k.statesBytes, 1);
+    if (k.lookback) {
+        const uint64_t groups = (k.chunks + 63) / 64, supers = (groups + 63) / 64;
+        k.statesBytes = roundUp(8 * (32 + 2 * (k.chunks + groups + supers)), 256);
+        k.tempBytes = k.headsBytes + k.statesBytes;
+        k.clearWords = k.tempBytes / 4;
+    } else {
+        k.statesBytes = k.carry ? roundUp(3 * k.chunks * 4, 256) : 0;
+        k.tempBytes = std::max<size_t>(k.headsBytes + 2 * k.statesBytes, 1);
+        k.clearWords = k.headsBytes / 4;
+    }
     if (k.tempBytes > tempLimitBytes) {
         throw std::invalid_argument("CUB scan: this request needs " + std::to_string(k.tempBytes) + " bytes of temporary storage, more than the " +
                                     std::to_string(tempLimitBytes) + " bytes of the fixed scratch block; use the allocating scan.");
@@ -166,14 +189,14 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
 
     s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void thor_scan_main(const gen::Cfg::T* in, const thor::u32* heads, const void* carries, "
          "gen::Cfg::T* outValue, thor::u32* outIndex) {\n    thor::scanChunk<gen::Cfg, false>(in, heads, carries, nullptr, outValue, outIndex);\n}\n";
-    if (k.carry) {
+    if (k.carry && !k.lookback) {
         s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void thor_scan_totals(const gen::Cfg::T* in, const thor::u32* heads, void* totals) {\n"
              "    thor::scanChunk<gen::Cfg, true>(in, heads, nullptr, totals, nullptr, nullptr);\n}\n";
         s << "extern \"C\" __global__ __launch_bounds__(1024) void thor_scan_carries(const void* totals, void* carries) {\n"
              "    thor::scanCarries<gen::Cfg>(totals, carries);\n}\n";
     }
+    if (k.clearWords) s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_clear(thor::u32* words) { thor::scanClear<gen::Cfg>(words); }\n";
     if (ragged) {
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_clear_heads(thor::u32* heads) { thor::scanClearHeads<gen::Cfg>(heads); }\n";
         s << "extern \"C\" __global__ __launch_bounds__(256) void thor_scan_mark_heads(const void* offsets, thor::u32* heads) {\n"
              "    thor::scanMarkHeads<gen::Cfg>(static_cast<const gen::Cfg::OffsetT*>(offsets), heads);\n}\n";
     }
@@ -188,17 +211,15 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
         return loaded;
     };
     k.mainKernel = kernel("thor_scan_main");
-    if (k.carry) {
+    if (k.carry && !k.lookback) {
         k.totalsKernel = kernel("thor_scan_totals");
         k.carriesKernel = kernel("thor_scan_carries");
     }
-    if (ragged) {
-        k.clearKernel = kernel("thor_scan_clear_heads");
-        k.markKernel = kernel("thor_scan_mark_heads");
-    }
+    if (k.clearWords) k.clearKernel = kernel("thor_scan_clear");
+    if (ragged) k.markKernel = kernel("thor_scan_mark_heads");
     std::ostringstream variant;
     variant << (ragged ? "segments" : r.row == r.total ? "flat" : "rows") << "(chunk=" << chunkElems << ",vec=" << vec << ",items=" << items << ",threads=" << threads
-            << ",grid=" << k.chunks << (k.carry ? ",passes=totals+carries+scan" : ",passes=scan") << (r.reverse ? ",reverse" : "") << ") ["
+            << ",grid=" << k.chunks << (k.lookback ? ",passes=scan,published_totals" : k.carry ? ",passes=totals+carries+scan" : ",passes=scan") << (r.reverse ? ",reverse" : "") << ") ["
             << k.mainKernel->kernelName << "]";
     k.variant = variant.str();
     return kernels;
@@ -212,17 +233,20 @@ void launchScan(const CubScanKernels& k, const void* input, const void* offsets,
     char* base = static_cast<char*>(temp);
     void* heads = k.headsBytes ? base : nullptr;
     void* totals = k.statesBytes ? base + k.headsBytes : nullptr;
-    void* carries = k.statesBytes ? base + k.headsBytes + k.statesBytes : nullptr;
+    // with published totals the scan kernel's `carries` argument is the block they live in
+    void* carries = k.lookback ? totals : k.statesBytes ? base + k.headsBytes + k.statesBytes : nullptr;
     void* raw = stream.getStream();
+    if (k.markKernel && offsets == nullptr) throw std::invalid_argument("CUB segmented scan requires segment offsets.");
     if (k.clearKernel) {
-        if (offsets == nullptr) throw std::invalid_argument("CUB segmented scan requires segment offsets.");
-        const uint64_t words = (k.request.total + 31) / 32;
-        std::vector<void*> clearArgs = {&heads};
-        k.clearKernel->launch(static_cast<uint32_t>((words + 255) / 256), 1, 1, 256, raw, clearArgs);
+        void* words = base;
+        std::vector<void*> clearArgs = {&words};
+        k.clearKernel->launch(static_cast<uint32_t>((k.clearWords + 255) / 256), 1, 1, 256, raw, clearArgs);
+    }
+    if (k.markKernel) {
         std::vector<void*> markArgs = {&offsets, &heads};
         k.markKernel->launch(static_cast<uint32_t>((k.request.segments + 1 + 255) / 256), 1, 1, 256, raw, markArgs);
     }
-    if (k.carry) {
+    if (k.totalsKernel) {
         std::vector<void*> totalsArgs = {&input, &heads, &totals};
         k.totalsKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, totalsArgs);
         std::vector<void*> carriesArgs = {&totals, &carries};

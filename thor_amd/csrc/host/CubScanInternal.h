@@ -33,6 +33,8 @@ struct CubScanKernels {
     uint64_t chunks = 1;
     uint32_t threads = 256;
     bool carry = false;
+    bool lookback = false;    // chunks read what precedes them from totals the blocks publish to each other (one launch over the data)
+    uint64_t clearWords = 0;  // 4-byte words at the start of the temporary storage that every run zeroes first
     size_t headsBytes = 0, statesBytes = 0, tempBytes = 1;
     std::string variant;
 };
