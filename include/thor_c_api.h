@@ -174,15 +174,15 @@ void thor_selection_plan_destroy(thor_selection_plan_t plan);
 
 /* thor_scan for callers that cannot allocate (work recorded under stream capture, serving loops, harnesses that forbid
  * hipMalloc).  It has no counterpart in the reference.  Same arguments, kernels and results as thor_scan, but the temporary
- * storage (segment-head bitmap, chunk totals and carries) is a fixed 4 MiB block of device memory that is part of the library's
+ * storage (segment-head bitmap, the totals that chunks publish to each other) is a fixed 4 MiB block of device memory that is part of the library's
  * code object, and nothing is compiled or loaded: no hipMalloc, hipFree, hipRTC or module load happens in this call.
  *   - The kernels of the request (dtype, operation, mode, direction, sizes, pointer alignment) must have been loaded by an earlier
  *     thor_scan (or a stamped Expression scan) with the same request in this process; otherwise the call fails and says so.
  *   - Requests that need more than 4 MiB of temporary storage fail with a message that gives both sizes.  Flat and row scans
- *     need 24 bytes per 8 192-element chunk (fp32: up to ~2^30 elements); offset-segmented scans add one bit per element
- *     (up to ~2^24 elements).
- *   - Every call on one GPU uses that GPU's block.  A call leaves nothing behind that a later call depends on (the bitmap is
- *     cleared by the call's own first kernel, totals and carries are written before they are read), but two calls that overlap
+ *     need about 16 bytes per chunk of 4 096 to 32 768 elements (fp32: up to ~2^31 elements); offset-segmented scans add one
+ *     bit per element (up to ~2^24 elements).
+ *   - Every call on one GPU uses that GPU's block.  A call leaves nothing behind that a later call depends on (the bitmap
+ *     and the block of totals are cleared by the call's own first kernel), but two calls that overlap
  *     in time on one GPU - different streams, different threads - race on the block. */
 int thor_scan_no_alloc(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments,
                        uint64_t segment_size, int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant,
