@@ -69,6 +69,8 @@ SHAPES = [
     ([100, 1001], [1]), ([37, 50257], [1]), ([5000, 63], [1]), ([3, 70001], [1]), ([9, 131], [1]),
     # a middle axis over an inner extent of a few elements: the rows kernel with one accumulator per inner element
     ([64, 300, 4], [1]), ([4096, 50, 2], [1]), ([33, 1000, 4], [1]), ([7, 5, 2, 2], [1]), ([2000, 6, 4], [1]),
+    # columns over an inner extent no vector divides: the last vector ends with the extent and overlaps the one before it
+    ([300, 1001], [0]), ([5000, 63], [0]), ([17, 50257], [0]), ([3, 200, 77], [1]), ([40, 9, 131], [0, 1]), ([2, 1000, 17], [1]), ([600, 9], [0]),
 ]
 
 
@@ -138,6 +140,36 @@ def test_rows_no_vector_divides_and_rows_that_begin_off_a_vector(stream, dtype):
         rows = np.stack([carrier[r * row_stride:r * row_stride + 1000] for r in range(rows_in_view)])
         np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream), oracle.reduce_f64(oracle.MAX, rows, int(dtype), [1]).astype(np.float32),
                                       err_msg=stamped.get_kernel_variant())
+
+
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16], ids=lambda d: d.name)
+def test_columns_over_inner_extents_no_vector_divides(stream, dtype):
+    """Lanes own whole vectors of outputs although the inner extent is odd; every output is stored once, by one owner: small
+    integers make the sums exact, so an output summed twice or taken from a neighbour shows.  Split and unsplit shapes, an
+    outer axis, the arg form, and a view that begins one element into the storage."""
+    rng = np.random.default_rng(11)
+    for dims, axes in (([3000, 1001], [0]), ([40, 50257], [0]), ([5, 700, 77], [1]), ([100000, 19], [0])):
+        x = to_storage(rng.integers(-4, 5, size=dims).astype(np.float32), dtype)
+        t = copy_numpy_to_gpu(x, stream, dtype)
+        stamped = ph.CubReduction(ph.CubReductionOp.Sum, axes, DataType.fp32).stamp(t, stream)
+        assert "columns(" in stamped.get_kernel_variant() and "unaligned_vectors" in stamped.get_kernel_variant(), stamped.get_kernel_variant()
+        stamped.run()
+        want = oracle.reduce_f64(oracle.SUM, x, int(dtype), axes).astype(np.float32)
+        np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream).reshape(want.shape), want, err_msg=stamped.get_kernel_variant())
+        arg = ph.CubArgReduction(ph.CubArgReductionOp.ArgMax, axes, value_output_dtype=DataType.fp32, index_output_dtype=DataType.uint32).stamp(t, stream)
+        arg.run()
+        want_idx, want_val = oracle.arg_reduce(oracle.ARGMAX, x, int(dtype), axes)
+        np.testing.assert_array_equal(copy_gpu_to_numpy(arg.get_index_output_tensor(), stream).astype(np.uint64).reshape(want_idx.shape), want_idx,
+                                      err_msg=arg.get_kernel_variant())
+        np.testing.assert_array_equal(gpu_to_f32(arg.get_value_output_tensor(), stream).reshape(want_val.shape), want_val)
+    # an even inner extent read from one element into the storage: no address is a multiple of the vector
+    x = to_storage(rng.integers(-4, 5, size=(500 * 1000 + 8,)).astype(np.float32), dtype)
+    t = copy_numpy_to_gpu(x, stream, dtype)
+    view = t.alias_view([500, 1000], [1000, 1], element_offset=1)
+    stamped = ph.CubReduction(ph.CubReductionOp.Sum, [0], DataType.fp32).stamp(view, stream)
+    stamped.run()
+    want = oracle.reduce_f64(oracle.SUM, x[1:1 + 500 * 1000].reshape(500, 1000), int(dtype), [0]).astype(np.float32)
+    np.testing.assert_array_equal(gpu_to_f32(stamped.get_output_tensor(), stream).reshape(want.shape), want, err_msg=stamped.get_kernel_variant())
 
 
 def test_small_inner_extents_take_the_rows_kernel_with_interleaved_outputs(stream):

@@ -243,9 +243,11 @@ __device__ __forceinline__ void reduceRows(const typename Cfg::Sources& src, con
 // 1 KiB of contiguous memory per step of the reduction.  A block is kLanesX columns wide and kThreads / kLanesX row
 // groups deep: row group g of share s walks reduction positions rBegin + g, rBegin + g + groups, ...; the groups are
 // then folded through LDS, so the depth adds parallelism without adding partials.
-// Cfg: kColumns, kR (reduction positions), kLanesX (power of two <= 64), kBatch (positions in flight per thread), kSplit
+// Cfg: kColumns, kR (reduction positions), kLanesX (<= 64, any width; a power of two for the transposed form), kBatch (positions in flight per thread), kSplit
 // (shares of kR, grid y), and the generated address functions columnBase(column), rowOffset(r), outputIndex(column, k)
-// (where element k of the column is stored) and partialSlot(column, k) (its row-major output number).
+// (where element k of the column is stored), partialSlot(column, k) (its row-major output number) and ownsElement(column, k)
+// (false for the outputs that the last column of an inner extent shares with the one before it, when the vector width does
+// not divide the extent: that column is moved back to end with the extent).
 template <typename Cfg>
 __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, const typename Cfg::Outputs& out, void* partials, float scale) {
     typedef typename Cfg::IndexT IndexT;
@@ -255,7 +257,8 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
     constexpr int kBatch = Cfg::kBatch;
     const int lx = threadIdx.x % Cfg::kLanesX, group = threadIdx.x / Cfg::kLanesX;
     const u64 column = (u64)blockIdx.x * Cfg::kLanesX + lx;
-    const bool columnLive = column < Cfg::kColumns;
+    // a width that does not divide the block leaves its last threads without a row group
+    const bool columnLive = column < Cfg::kColumns && group < kGroups;
     const u64 safeColumn = columnLive ? column : 0;
     const u64 share = Cfg::kSplit > 1 ? blockIdx.y : 0;
     const u64 rBegin = share * kRowsPerShare;
@@ -291,7 +294,7 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
     if (kGroups > 1) {
         // fold the row groups: group g > 0 parks its accumulators, group 0 merges them in group order
         __shared__ Acc parked[(kGroups > 1 ? kGroups - 1 : 1) * Cfg::kLanesX * Cfg::kVec];
-        if (group > 0) {
+        if (group > 0 && group < kGroups) {
 #pragma unroll
             for (int k = 0; k < Cfg::kVec; ++k) parked[((group - 1) * Cfg::kLanesX + lx) * Cfg::kVec + k] = acc[k];
         }
@@ -306,6 +309,7 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
     if (group == 0 && columnLive) {
 #pragma unroll
         for (int k = 0; k < Cfg::kVec; ++k) {
+            if (!Cfg::ownsElement(column, k)) continue;  // an output that the column before this one holds as well
             if (Cfg::kSplit > 1) {
                 acc[k].template storePartial<Cfg::kTickets>(partials, Cfg::partialSlot(column, k) * Cfg::kSplit + share, Cfg::kOutputs * Cfg::kSplit);
             } else {
@@ -321,7 +325,7 @@ __device__ __forceinline__ void reduceColumns(const typename Cfg::Sources& src, 
         const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
         for (int o = wave; o < Cfg::kLanesX * Cfg::kVec; o += kWaves) {
             const u64 c = (u64)blockIdx.x * Cfg::kLanesX + o / Cfg::kVec;
-            if (c < Cfg::kColumns) foldShares<Cfg>(partials, Cfg::partialSlot(c, o % Cfg::kVec), out, scale, lane);
+            if (c < Cfg::kColumns && Cfg::ownsElement(c, o % Cfg::kVec)) foldShares<Cfg>(partials, Cfg::partialSlot(c, o % Cfg::kVec), out, scale, lane);
         }
     }
 }

@@ -172,6 +172,7 @@ std::string ReductionShape::describe() const {
             break;
         case Kernel::Columns:
             out << (laneAxis < 0 ? "columns(lanes_x=" : "view_columns(lanes_x=") << threadsPerRow << ",rows_in_flight=" << unroll << ",split=" << split;
+            if (unalignedVectors) out << ",unaligned_vectors";
             if (transposeRows > 0) out << ",transposed_store=" << transposeRows;
             break;
         case Kernel::Segments:
@@ -396,12 +397,27 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         }
         shape.kernel = ReductionShape::Kernel::Columns;
         shape.vec = chooseVector(elementBytes, request.inputAlignmentBytes, {g.inner_size});
+        // An inner extent (or a pointer) that no vector fits: the lanes still own 16-byte vectors of outputs and read them at
+        // addresses that are only aligned to the element; the last vector of the inner extent is moved back to end with it, and
+        // the outputs it shares with the vector before it are stored by that one.
+        const int wideColumns = static_cast<int>(16 / elementBytes);
+        if (shape.vec < wideColumns && request.elementwise.empty() && g.inner_size >= 2ull * wideColumns && g.tiled_output_outer_stride != 1 &&
+            request.inputAlignmentBytes % elementBytes == 0 && std::getenv("THOR_COLUMNS_NO_UNALIGNED") == nullptr) {
+            shape.vec = wideColumns;
+            shape.unalignedVectors = true;
+        }
+        const uint64_t innerColumns = ceilDiv(g.inner_size, shape.vec);
         shape.threads = 256;
         shape.unroll = 8;  // rows in flight per thread
         if (const char* env = std::getenv("THOR_COLUMNS_BATCH")) shape.unroll = std::min<long>(std::max<long>(std::atol(env), 1), 16);  // tuning switch
-        const uint64_t columns = g.outer_size * (g.inner_size / shape.vec);
+        const uint64_t columns = g.outer_size * innerColumns;
         // a block is up to one wavefront of columns wide; the rest of its threads are row groups folded through LDS
         shape.threadsPerRow = static_cast<int>(std::min<uint64_t>(64, pow2Ceil(columns)));
+        if (g.tiled_output_outer_stride != 1 && std::getenv("THOR_COLUMNS_POW2_LANES") == nullptr) {
+            // as many blocks across the columns as 64-lane blocks would take, each as wide as its share of the columns: 20
+            // columns are 20 lanes and 12 row groups (not 32 lanes of which 12 idle), 77 columns two blocks of 39 (not 64 + 13)
+            shape.threadsPerRow = static_cast<int>(ceilDiv(columns, ceilDiv(columns, 64)));
+        }
         if (const char* env = std::getenv("THOR_COLUMNS_LANES")) {  // tuning switch: lanes across the columns of a block
             const long requested = std::atol(env);
             if ((requested == 64 || requested == 128 || requested == 256) && static_cast<uint64_t>(requested) <= pow2Ceil(columns)) shape.threadsPerRow = static_cast<int>(requested);
@@ -417,15 +433,14 @@ ReductionShape planShapeWithoutTickets(const ReductionKernelRequest& request) {
         if (const char* env = std::getenv("THOR_COLUMNS_SPLIT")) {  // tuning switch
             shape.split = std::min<uint64_t>({static_cast<uint64_t>(std::max<long>(std::atol(env), 1)), std::max<uint64_t>(g.reduction_size / groups, 1), kMaxGridY});
         }
-        const uint64_t columnsNow = g.outer_size * (g.inner_size / shape.vec);
-        shape.gridX = static_cast<uint32_t>(ceilDiv(columnsNow, shape.threadsPerRow));
+        shape.gridX = static_cast<uint32_t>(ceilDiv(columns, shape.threadsPerRow));
         shape.gridY = static_cast<uint32_t>(shape.split);
         if (g.tiled_output_outer_stride == 1) {
             // [inner, outer] output: consecutive outer coordinates are adjacent in the output
             shape.transposeRows = transposeRowsFor(shape.split, g.reduction_size, g.outer_size, g.tiled_output_inner_stride,
                                                     (static_cast<uint64_t>(shape.threadsPerRow) * shape.vec + 1) * accumulatorBytes);
             if (shape.transposeRows > 0) {
-                shape.gridX = static_cast<uint32_t>(ceilDiv(g.inner_size / shape.vec, shape.threadsPerRow) * ceilDiv(g.outer_size, shape.transposeRows));
+                shape.gridX = static_cast<uint32_t>(ceilDiv(innerColumns, shape.threadsPerRow) * ceilDiv(g.outer_size, shape.transposeRows));
             }
         }
         finishSplit(g.output_elements);
@@ -706,19 +721,28 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
             s << "    static constexpr u64 kR = " << g.reduction_size << "ull;\n";
             s << "    static constexpr int kBatch = " << shape.unroll << ";\n";
             s << "    static constexpr int kLanesX = " << shape.threadsPerRow << ";\n";
-            s << "    static constexpr u64 kColumns = " << (g.output_elements / shape.vec) << "ull;\n";
             if (shape.laneAxis < 0) {
-                // dense [outer, R, inner]
-                const uint64_t innerVectors = g.inner_size / shape.vec;
+                // dense [outer, R, inner]: a column begins at a multiple of the vector width, except the last one of an inner
+                // extent that the width does not divide, which ends with the extent and owns only what the one before does not
+                const uint64_t innerVectors = ceilDiv(g.inner_size, static_cast<uint64_t>(shape.vec));
+                const uint64_t lastFirst = g.inner_size - static_cast<uint64_t>(shape.vec);
+                const uint64_t shared = innerVectors * shape.vec - g.inner_size;  // leading elements of the last column that the one before owns
+                s << "    static constexpr u64 kColumns = " << (g.outer_size * innerVectors) << "ull;\n";
+                s << "    static __device__ __forceinline__ u64 columnFirst(u64 c) { const u64 first = (c % " << innerVectors << "ull) * " << shape.vec
+                  << "ull; return first < " << lastFirst << "ull ? first : " << lastFirst << "ull; }\n";
+                s << "    static __device__ __forceinline__ bool ownsElement(u64 c, int k) { return " << (shared == 0 ? "true" : "") ;
+                if (shared != 0) s << "c % " << innerVectors << "ull != " << (innerVectors - 1) << "ull || k >= " << shared;
+                s << "; }\n";
                 s << "    static __device__ __forceinline__ u64 columnBase(u64 c) { return (c / " << innerVectors << "ull) * " << (g.reduction_size * g.inner_size)
-                  << "ull + (c % " << innerVectors << "ull) * " << shape.vec << "ull; }\n";
+                  << "ull + columnFirst(c); }\n";
                 s << "    static __device__ __forceinline__ u64 rowOffset(u64 r) { return r * " << g.inner_size << "ull; }\n";
                 s << "    static __device__ __forceinline__ u64 partialSlot(u64 c, int k) { return (c / " << innerVectors << "ull) * " << g.inner_size
-                  << "ull + (c % " << innerVectors << "ull) * " << shape.vec << "ull + k; }\n";
+                  << "ull + columnFirst(c) + k; }\n";
                 s << "    static __device__ __forceinline__ u64 outputIndex(u64 c, int k) { return (c / " << innerVectors << "ull) * "
-                  << g.tiled_output_outer_stride << "ull + ((c % " << innerVectors << "ull) * " << shape.vec << "ull + k) * " << g.tiled_output_inner_stride
-                  << "ull; }\n";
+                  << g.tiled_output_outer_stride << "ull + (columnFirst(c) + k) * " << g.tiled_output_inner_stride << "ull; }\n";
             } else {
+                s << "    static constexpr u64 kColumns = " << (g.output_elements / shape.vec) << "ull;\n";
+                s << "    static __device__ __forceinline__ bool ownsElement(u64, int) { return true; }\n";
                 // a view: columns enumerate the kept coordinates with the contiguous axis fastest (in vectors); outputs are
                 // numbered row-major over the kept axes in their logical order
                 const size_t lane = static_cast<size_t>(shape.laneAxis);
