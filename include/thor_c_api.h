@@ -140,7 +140,10 @@ int thor_segmented_broadcast(thor_tensor_t per_segment_values, thor_tensor_t seg
 /* Prefix scans (Utilities/TensorOperations/Cub/CubDevicePrimitives.h:781-880,951-1012 there): prepare, allocate the temporary
  * storage and run in one call.  op: 0 sum, 1 min, 2 max, 3 product; arg != 0 (op 1 or 2): output holds UINT32 flattened indices
  * of the winning prefix element.  Segments: offsets != NULL -> the num_segments segments of an offsets tensor; else
- * segment_size > 0 -> num_items / segment_size rows; else one scan.  `variant` (may be NULL) receives how the plan runs. */
+ * segment_size > 0 -> num_items / segment_size rows; else one scan.  `variant` (may be NULL) receives how the plan runs.
+ * The call returns when the scan has run (it owns the temporary storage and frees it), and fails if a block of a scan whose
+ * chunks read each other's totals gave up a wait (bounded so that every wavefront has an exit; not reachable while the blocks
+ * of earlier chunks run). */
 int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments, uint64_t segment_size,
               int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity);
 

@@ -220,8 +220,8 @@ def test_top_k_pairs_with_many_equal_keys(stream, dtype, largest):
 @pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
 @pytest.mark.parametrize("region", [None, "1"], ids=["roomy", "overflowing"])
 def test_top_k_over_candidates(stream, monkeypatch, dtype, largest, region):
-    """Long inputs copy the keys that can still be part of the answer during the second pass and finish on those candidates; the
-    switch asks for that on short inputs too.  With one entry per wavefront the candidate regions overflow and the passes over
+    """Long inputs copy the keys at or above a floor taken from a sample (the keys that can still be part of the answer) during
+    the one pass over the input and finish on those candidates; the switch asks for that on short inputs and large k too.  With one entry per wavefront the candidate regions overflow and the passes over
     the whole input take over: both ways must give the same answer."""
     monkeypatch.setenv("THOR_TOPK_CANDIDATES", "1")
     if region:
@@ -240,9 +240,9 @@ def test_top_k_long_inputs_use_candidates_by_default(stream):
     rng = np.random.default_rng(77)
     keys = rng.standard_normal((1 << 21) + 12).astype(np.float32)
     keys[rng.integers(0, keys.size, 50)] = np.float32(9.5)  # ties at the top
-    for k in (1, 40, 64, 70_000):
+    for k in (1, 40, 64, 8_000, 70_000):
         got, got_values, variant = run_top_k(keys, DataType.fp32, k, True, stream, pairs=True)
-        assert "candidates(" in variant
+        assert ("candidates(" in variant) == (k * 256 <= keys.size)  # a k beyond a 256th of the input reads it once per digit
         check_top_k(keys, DataType.fp32, k, True, got, got_values)
     sorted_keys = np.sort(keys)  # every candidate in one stretch of the input
     for largest in (True, False):

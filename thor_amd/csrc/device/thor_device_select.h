@@ -226,7 +226,9 @@ struct TopkState {
     u32 taken;      // output slots handed out to keys above the threshold
     u32 ties;       // keys equal to the threshold seen so far by the gathering pass
     u32 overflow;   // candidate regions (below) were too small for this input: the passes over the whole input take over
-    u32 unused[3];
+    u32 arrived;    // blocks of the running counting pass that have added their histogram (zero between passes)
+    u32 floor;      // candidates (below): keys whose image is at least this can still be part of the answer
+    u32 floorRemaining;  // while the floor is being fixed digit by digit over the sample: what `remaining` is for the prefix
 };
 constexpr int kTopkStateWords = 8;
 
@@ -240,17 +242,60 @@ __device__ __forceinline__ void topkInit(u32* temp) {
         state->taken = 0;
         state->ties = 0;
         state->overflow = 0;
+        state->arrived = 0;
+        state->floor = 0;
+        state->floorRemaining = (u32)Cfg::kK;
     }
+}
+
+// One block of 256 threads: fixes the digit at `shift` and clears the histogram for the next pass.  The histogram words were
+// added to by blocks all over the device: they are read at device scope.
+// FLOOR: the histogram is that of a sample of the input, and the digits of the sample's kK-th largest key are fixed in
+// `floor` / `floorRemaining` instead (at least kK keys of the input lie at or above that key's digits: those of the sample).
+template <typename Cfg, bool FLOOR = false>
+__device__ __forceinline__ void topkPick(u32* temp, u32 shift, u32 bits) {
+    __shared__ u32 lds[8];
+    TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
+    const u32 wanted = FLOOR ? state->floorRemaining : state->remaining, prefix = FLOOR ? state->floor : state->prefix;
+    u32 above;
+    const u32 bucket = topkPickBucket([&](u32 b) { return loadDeviceWide(&temp[b]); }, 1u << bits, wanted, lds, above);
+    for (int b = threadIdx.x; b < kTopkMaxBins; b += 256) temp[b] = 0;
+    if (threadIdx.x == 0) {
+        if (FLOOR) {
+            state->floor = prefix | (bucket << shift);
+            state->floorRemaining = wanted - above;
+        } else {
+            state->prefix = prefix | (bucket << shift);
+            state->remaining = wanted - above;
+        }
+    }
+}
+
+// The end of a counting pass, called by every block (256 threads) once it has added its histogram to the shared one: the
+// block waits until those additions are acknowledged and counts itself in; the block that counts in last fixes the digit,
+// so the pass needs no launch of its own for that.
+template <typename Cfg, bool FLOOR = false>
+__device__ __forceinline__ void topkPickWhenLast(u32* temp, u32 shift, u32 bits) {
+    __shared__ u32 last;
+    partialsWritten();
+    __syncthreads();
+    TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
+    if (threadIdx.x == 0) {
+        const u32 before = __hip_atomic_fetch_add(&state->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last = before + 1u == gridDim.x ? 1u : 0u;
+        if (last) storeDeviceWide(&state->arrived, 0u);
+    }
+    __syncthreads();
+    if (last) topkPick<Cfg, FLOOR>(temp, shift, bits);
 }
 
 // Histogram of the `bits`-wide digit at `shift` over the keys whose higher digits equal the prefix.  Blocks stride over the keys
 // in vectors, four vectors of a thread in flight.
 template <typename Cfg>
-__device__ __forceinline__ void topkHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits, u32 fallbackOnly) {
+__device__ __forceinline__ void topkHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
     typedef typename Cfg::Raw Raw;
     constexpr int V = Cfg::kVec, kUnroll = 4;
     __shared__ u32 bins[kTopkMaxBins];
-    if (fallbackOnly && reinterpret_cast<const TopkState*>(temp + kTopkMaxBins)->overflow == 0) return;  // the candidates were counted instead
     const u32 numBins = 1u << bits;
     for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
     __syncthreads();
@@ -280,21 +325,7 @@ __device__ __forceinline__ void topkHistogram(const typename Cfg::Raw* keys, u32
         const u32 mine = bins[b];
         if (mine != 0) atomicAdd(&temp[b], mine);
     }
-}
-
-// One block of 256 threads: fixes the digit at `shift` and clears the histogram for the next pass.
-template <typename Cfg>
-__device__ __forceinline__ void topkPick(u32* temp, u32 shift, u32 bits) {
-    __shared__ u32 lds[8];
-    TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-    const u32 wanted = state->remaining, prefix = state->prefix;
-    u32 above;
-    const u32 bucket = topkPickBucket([&](u32 b) { return temp[b]; }, 1u << bits, wanted, lds, above);
-    for (int b = threadIdx.x; b < kTopkMaxBins; b += 256) temp[b] = 0;
-    if (threadIdx.x == 0) {
-        state->prefix = prefix | (bucket << shift);
-        state->remaining = wanted - above;
-    }
+    topkPickWhenLast<Cfg>(temp, shift, bits);
 }
 
 // Writes the keys above the threshold image (kK - remaining of them) and `remaining` of the keys equal to it.  Every
@@ -303,13 +334,11 @@ __device__ __forceinline__ void topkPick(u32* temp, u32 shift, u32 bits) {
 // one request per wavefront vote cost 0.7 ms at k = 65 536); a block without qualifying keys, the usual case when k is
 // small next to the input, leaves after the count.
 template <typename Cfg>
-__device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues,
-                                           u32 fallbackOnly) {
+__device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
     typedef typename Cfg::Raw Raw;
     constexpr int V = Cfg::kVec, kWaves = Cfg::kThreads / kWave;
     __shared__ u32 waveAbove[kWaves], waveTies[kWaves], bases[2];
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-    if (fallbackOnly && state->overflow == 0) return;  // the candidates were gathered instead
     const u32 threshold = state->prefix, wantedTies = state->remaining, firstTieSlot = (u32)Cfg::kK - wantedTies;
     constexpr u64 kVectors = Cfg::kTotal / V;
     constexpr u64 kChunkVectors = (u64)Cfg::kThreads * Cfg::kItems;
@@ -385,17 +414,19 @@ __device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const 
 }
 
 // ---- candidates ------------------------------------------------------------------------------------------------------------------
-// Long inputs are read in full twice instead of once per digit and once more for the output: after the first digit is fixed,
-// the pass that counts the second digit also copies every key whose first digit is at or above the fixed one (the keys that
-// can still be part of the answer: fewer than kK above the bucket plus the bucket itself) into the temporary storage, and the
-// later digits and the output are taken from those candidates.  Every wavefront of the copying pass owns a region of
+// Long inputs are read in full once instead of once per digit and once more for the output.  A first small launch counts the
+// first digit over a sample of the input (runs of 256 vectors spread evenly, max(2^16, 128 kK) keys), a second one the second
+// digit, and the two leading digits of the sample's kK-th largest key become the floor: at least kK keys of the input lie at or
+// above it, so the answer does too, whatever the sample missed.  The pass over the whole input then counts the first digit of the keys at or above the floor only (the
+// others cannot change which bucket holds the kK-th largest key, nor how many keys lie above it) and copies those keys, the
+// candidates, into the temporary storage; the later digits and the output are taken from the candidates.  With a floor most
+// keys fail one comparison and touch no histogram: the pass streams.  Every wavefront of the copying pass owns a region of
 // kRegion entries (keys as 32-bit words; for pairs the key's position as well) and counts what it wrote: no wavefront asks
 // another for room.  A region that would overflow (a bucket that holds a large part of the input: many equal keys, k close to
-// kTotal) raises `overflow`; the passes over the candidates then leave at once and the passes over the whole input, launched
-// after them, do the work.
-// Cfg additionally: kCompact, kFirstShift (the shift of the first digit), kRegion, kRegions (wavefronts of the copying
-// pass), kCandidateBlocks.  Temporary storage after the state: kRegions counts, kRegions * kRegion keys, the same number of
-// positions (pairs).
+// kTotal) raises `overflow`; the launches over the candidates then walk the whole input instead, with the blocks they have.
+// Cfg additionally: kCompact, kRegion, kRegions (wavefronts of the copying pass), kSampleVectors (a multiple of 256; 0: no
+// sample, the floor stays 0), kSampleRunStride (vectors from one run of the sample to the next).  Temporary storage after the
+// state: kRegions counts, kRegions * kRegion keys, the same number of positions (pairs).
 template <typename Cfg>
 struct TopkCandidates {
     __device__ __forceinline__ static u32* counts(u32* temp) { return temp + kTopkMaxBins + kTopkStateWords; }
@@ -403,8 +434,39 @@ struct TopkCandidates {
     __device__ __forceinline__ static u32* positions(u32* temp) { return keys(temp) + (u64)Cfg::kRegions * Cfg::kRegion; }
 };
 
-// Launched with kRegions / 4 blocks of 256 threads, after the first digit has been fixed: histogram of the digit at `shift`
-// over the keys that match the first digit, and the candidates of every wavefront into its region.
+// The digit at `shift` over the keys of the sample whose higher digits equal the floor's; the block that finishes last fixes
+// that digit of the floor.  Launched for the first digit and then for the second: a floor of one digit would make candidates of
+// the whole bucket of that digit, which for keys that crowd a few leading digits is a large part of the input.
+template <typename Cfg>
+__device__ __forceinline__ void topkSample(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
+    typedef typename Cfg::Raw Raw;
+    constexpr int V = Cfg::kVec;
+    __shared__ u32 bins[kTopkMaxBins];
+    const u32 numBins = 1u << bits;
+    for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
+    __syncthreads();
+    const u32 floorSoFar = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins)->floor;
+    const u32 fixedBits = shift + bits >= 32 ? 0u : (0xffffffffu << (shift + bits));
+    const u32 digitMask = numBins - 1u;
+    for (u64 j = (u64)blockIdx.x * 256 + threadIdx.x; j < Cfg::kSampleVectors; j += (u64)gridDim.x * 256) {
+        Pack<Raw, V> x;
+        x.load(keys + ((j / 256) * Cfg::kSampleRunStride + j % 256) * V);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const u32 image = topkImage<Cfg>(x.v[k]);
+            if ((image & fixedBits) == (floorSoFar & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
+        }
+    }
+    __syncthreads();
+    for (u32 b = threadIdx.x; b < numBins; b += 256) {
+        const u32 mine = bins[b];
+        if (mine != 0) atomicAdd(&temp[b], mine);
+    }
+    topkPickWhenLast<Cfg, true>(temp, shift, bits);
+}
+
+// Launched with kRegions / 4 blocks of 256 threads: histogram of the first digit (at `shift`) over the keys at or above the
+// floor, and those keys, the candidates of every wavefront, into its region; the block that finishes last fixes the digit.
 template <typename Cfg>
 __device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
     typedef typename Cfg::Raw Raw;
@@ -414,8 +476,7 @@ __device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* 
     for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
     __syncthreads();
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-    constexpr u32 kFirstDigit = 0xffffffffu << Cfg::kFirstShift;
-    const u32 floorImage = state->prefix & kFirstDigit;  // images at or above it are candidates, images that match it are counted
+    const u32 floorImage = state->floor;  // images at or above it are candidates
     const u32 digitMask = numBins - 1u;
     const int lane = threadIdx.x % kWave;
     const u64 lowerLanes = ((u64)1 << lane) - 1;
@@ -451,7 +512,7 @@ __device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* 
                         regionKeys[slot] = (u32)x[u].v[k];
                         if (Cfg::kPairs) regionPositions[slot] = (u32)((v0 + u * stride) * V + k);
                     }
-                    if ((image[k] & kFirstDigit) == floorImage) atomicAdd(&bins[(image[k] >> shift) & digitMask], 1u);
+                    atomicAdd(&bins[(image[k] >> shift) & digitMask], 1u);
                 }
                 cursor += (u32)__builtin_popcountll(votes);
             }
@@ -466,15 +527,19 @@ __device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* 
         const u32 mine = bins[b];
         if (mine != 0) atomicAdd(&temp[b], mine);
     }
+    topkPickWhenLast<Cfg>(temp, shift, bits);
 }
 
 // kCandidateBlocks blocks of 256 threads: histogram of the digit at `shift` over the candidates that match the digits fixed so far.
 template <typename Cfg>
-__device__ __forceinline__ void topkCandidateHistogram(u32* temp, u32 shift, u32 bits) {
+__device__ __forceinline__ void topkCandidateHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
     typedef typename Cfg::Raw Raw;
     __shared__ u32 bins[kTopkMaxBins];
     const TopkState* state = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins);
-    if (state->overflow != 0) return;
+    if (state->overflow != 0) {  // the regions were too small: count over the whole input, with the blocks of this launch
+        topkHistogram<Cfg>(keys, temp, shift, bits);
+        return;
+    }
     const u32 numBins = 1u << bits;
     for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
     __syncthreads();
@@ -496,18 +561,22 @@ __device__ __forceinline__ void topkCandidateHistogram(u32* temp, u32 shift, u32
         const u32 mine = bins[b];
         if (mine != 0) atomicAdd(&temp[b], mine);
     }
+    topkPickWhenLast<Cfg>(temp, shift, bits);
 }
 
 // kCandidateBlocks blocks of 256 threads: the output out of the candidates.  Every thread counts the candidates it will write
 // (above the threshold; equal to it), a block scan turns the counts into ranks inside the block, one thread asks for the
 // block's output slots, and a second walk over the same candidates writes them.
 template <typename Cfg>
-__device__ __forceinline__ void topkCandidateGather(const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
+__device__ __forceinline__ void topkCandidateGather(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
     typedef typename Cfg::Raw Raw;
     __shared__ u32 lds[8];
     __shared__ u32 bases[2];
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-    if (state->overflow != 0) return;
+    if (state->overflow != 0) {  // the regions were too small: gather from the whole input, with the blocks of this launch
+        topkGather<Cfg>(keys, values, temp, outKeys, outValues);
+        return;
+    }
     const u32 threshold = state->prefix, wantedTies = state->remaining, firstTieSlot = (u32)Cfg::kK - wantedTies;
     const int lane = threadIdx.x % kWave;
     const u32* counts = TopkCandidates<Cfg>::counts(temp);

@@ -256,6 +256,18 @@ void launchScan(const CubScanKernels& k, const void* input, const void* offsets,
     k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, mainArgs);
 }
 
+uint32_t scanWaitsGivenUp(const CubScanKernels& k, const void* temp, Stream& stream) {
+    if (!k.lookback || temp == nullptr) return 0;
+    ScopedGpu scoped(k.request.deviceNum);
+    uint32_t count = 0;
+    // the second control word of the block of published totals, which follows the head bitmap
+    const char* word = static_cast<const char*>(temp) + k.headsBytes + 8;
+    if (thorhip_memcpy_async(&count, word, sizeof count, THORHIP_D2H, stream.getStream()) != 0 || thorhip_stream_synchronize(stream.getStream()) != 0) {
+        throw std::runtime_error(std::string("CUB scan: reading the wait counter failed: ") + thorhip_last_error());
+    }
+    return count;
+}
+
 bool scanRouteFits(const ScanRequest& request) {
     ScanRequest routed = request;
     routed.route = true;

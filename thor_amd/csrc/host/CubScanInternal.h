@@ -53,6 +53,11 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& reques
 void launchScan(const CubScanKernels& kernels, const void* input, const void* offsets, void* temp, size_t tempBytes, void* outValue, void* outIndex,
                 Stream& stream);
 
+// How many waits of the last launch on `temp` gave up (scans that publish totals between blocks bound every wait so that
+// each wavefront has an exit; a wait that gives up leaves wrong results behind).  Waits for the stream, then reads one word
+// of `temp`: for callers that synchronise anyway.  Always 0 for kernels that do not wait on each other.
+uint32_t scanWaitsGivenUp(const CubScanKernels& kernels, const void* temp, Stream& stream);
+
 // One scan (flat: offsets null and segmentSize 0; rows of segmentSize; or the numSegments segments of *offsets) that compiles, loads
 // and allocates nothing: its kernels must be in the process-wide cache already (std::runtime_error otherwise) and its temporary
 // storage is the caller's block `temp` of tempCapacityBytes (std::invalid_argument when the request needs more).  Same validation,

@@ -18,15 +18,17 @@
 
 namespace ThorImplementation {
 
-// What one plan launches.  kind 0: select-flagged (count, offsets, scatter); 1: device-wide top-k (init, then histogram + pick per
-// digit, gather); 2: top-k of rows (one launch).  A plan with nothing to do (no items, k == 0) holds no kernels.
+// What one plan launches.  kind 0: select-flagged (count, offsets, scatter); 1: device-wide top-k (init, then one counting pass
+// per digit whose last block picks the digit, gather; `third` is not used); 2: top-k of rows (one launch).  A plan with nothing to do (no items, k == 0) holds no kernels.
 struct CubSelectionKernels {
     int kind = 0;
     int deviceNum = 0;
     std::shared_ptr<CompiledKernel> first, second, third, fourth;
-    // device-wide top-k over candidates: the copying pass, the histogram and the gathering pass over the candidates
-    std::shared_ptr<CompiledKernel> compact, candidateHistogram, candidateGather;
-    uint32_t candidateBlocks = 0, fallbackGatherBlocks = 0;
+    // device-wide top-k over candidates: the sample that sets their floor, the copying pass, the histogram and the gathering
+    // pass over the candidates
+    std::shared_ptr<CompiledKernel> sample, compact, candidateHistogram, candidateGather;
+    uint32_t candidateBlocks = 0, sampleBlocks = 0;
+    uint64_t sampleVectors = 0;
     uint64_t chunks = 0;          // blocks of the counting / scattering / gathering launches; rows for kind 2
     uint32_t histogramBlocks = 0;
     uint32_t threads = 256;
@@ -263,19 +265,27 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     sel.chunks = (vectors + chunkVectors - 1) / chunkVectors;
     // enough striding blocks to keep every compute unit busy, few enough that the global histogram sees little contention
     sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, 2048));
-    // Long inputs with more than one digit: the second pass over the input also copies the keys that can still be part of the
-    // answer, and the later digits and the output are taken from those candidates (two reads of the input instead of one per
-    // digit plus one).  Every wavefront of that pass owns room for its share of a 32nd of the input, at least 64 entries.
-    bool compact = sel.digits >= 2 && numItems >= kTopKCompactMinItems && numItems < (1ull << 32);
+    // Long inputs with more than one digit: the pass over the input that counts the first digit also copies the keys that can
+    // still be part of the answer, and the later digits and the output are taken from those candidates (one read of the input
+    // instead of one per digit plus one).  Every wavefront of that pass owns room for its share of a 32nd of the input, at
+    // least 64 entries.
+    // The floor of the candidates comes from a sample of max(2^16, 128 k) keys, in runs of 256 vectors: about k / sample of the
+    // input, and what shares the floor's bucket with it, becomes candidates.  When k is more than a 256th of the input the
+    // candidates would not fit their regions: every digit then reads the whole input.
+    bool compact = sel.digits >= 2 && numItems >= kTopKCompactMinItems && numItems < (1ull << 32) && k * 256 <= numItems;
     if (const char* env = std::getenv("THOR_TOPK_CANDIDATES")) {  // tuning / test switch: "0" reads the whole input in every pass
         if (std::string(env) == "0") compact = false;
         if (std::string(env) == "1") compact = sel.digits >= 2 && numItems < (1ull << 32);
     }
+    const uint64_t sampleRuns = std::min<uint64_t>(std::max<uint64_t>(uint64_t(1) << 16, 128 * k) / vec, vectors) / 256;
+    sel.sampleVectors = sampleRuns * 256 * vec >= k ? sampleRuns * 256 : 0;  // a sample that holds fewer than k keys gives no floor
+    const uint64_t sampleRunStride = sel.sampleVectors ? vectors / sampleRuns : 0;
+    sel.sampleBlocks = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(sel.sampleVectors / 1024, 1), 256));
     const uint64_t regions = uint64_t(sel.histogramBlocks) * (256 / 64);
     uint64_t regionEntries = std::max<uint64_t>((numItems / 32 + regions - 1) / regions, 64);
     if (const char* env = std::getenv("THOR_TOPK_REGION")) regionEntries = std::max<long>(std::atol(env), 1);  // test switch: entries per wavefront
-    sel.candidateBlocks = static_cast<uint32_t>(std::min<uint64_t>((regions + 3) / 4, 128));
-    sel.fallbackGatherBlocks = static_cast<uint32_t>(std::min<uint64_t>(sel.chunks, 2048));
+    // few blocks walk the candidates; the same launches walk the whole input when the regions overflowed, so not too few
+    sel.candidateBlocks = static_cast<uint32_t>(std::min<uint64_t>((regions + 3) / 4, 256));
     sel.tempBytes = (kTopKBins + kTopKStateWords) * 4;
     if (compact) sel.tempBytes += (regions + regions * regionEntries * (pairs ? 2 : 1)) * 4;
     std::ostringstream s;
@@ -285,35 +295,39 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     s << "    static constexpr thor::u64 kTotal = " << numItems << "ull;\n    static constexpr thor::u64 kK = " << k
       << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = " << kGatherThreads
       << ";\n    static constexpr int kItems = " << kGatherItems << ";\n    static constexpr bool kCompact = " << (compact ? "true" : "false")
-      << ";\n    static constexpr thor::u32 kFirstShift = " << sel.digitPlan.front().first << "u;\n    static constexpr thor::u32 kRegion = " << regionEntries
-      << "u;\n    static constexpr thor::u32 kRegions = " << regions << "u;\n};\n}  // namespace gen\n";
+      << ";\n    static constexpr thor::u32 kRegion = " << regionEntries << "u;\n    static constexpr thor::u32 kRegions = " << regions
+      << "u;\n    static constexpr thor::u64 kSampleVectors = " << sel.sampleVectors << "ull;\n    static constexpr thor::u64 kSampleRunStride = "
+      << sampleRunStride << "ull;\n};\n}  // namespace gen\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_init(thor::u32* temp) { thor::topkInit<gen::Cfg>(temp); }\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits, "
-         "thor::u32 fallbackOnly) {\n    thor::topkHistogram<gen::Cfg>(keys, temp, shift, bits, fallbackOnly);\n}\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_pick(thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
-         "    thor::topkPick<gen::Cfg>(temp, shift, bits);\n}\n";
+    // every counting pass ends with the pick of its digit, by the block that finishes last
+    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
+         "    thor::topkHistogram<gen::Cfg>(keys, temp, shift, bits);\n}\n";
     s << "extern \"C\" __global__ __launch_bounds__(" << kGatherThreads
-      << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues, "
-         "thor::u32 fallbackOnly) {\n    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues, fallbackOnly);\n}\n";
+      << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n"
+         "    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
     if (compact) {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_sample(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
+             "    thor::topkSample<gen::Cfg>(keys, temp, shift, bits);\n}\n";
         s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_compact(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
              "    thor::topkCompact<gen::Cfg>(keys, temp, shift, bits);\n}\n";
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_histogram(thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
-             "    thor::topkCandidateHistogram<gen::Cfg>(temp, shift, bits);\n}\n";
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_gather(const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, "
-             "thor::u32* outValues) {\n    thor::topkCandidateGather<gen::Cfg>(values, temp, outKeys, outValues);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, "
+             "thor::u32 bits) {\n    thor::topkCandidateHistogram<gen::Cfg>(keys, temp, shift, bits);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, "
+             "gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n    thor::topkCandidateGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
     }
     const std::string source = s.str();
     sel.first = compileKernel(source, "thor_topk_init", deviceNum, false);
     sel.second = compileKernel(source, "thor_topk_histogram", deviceNum, false);
-    sel.third = compileKernel(source, "thor_topk_pick", deviceNum, false);
     sel.fourth = compileKernel(source, "thor_topk_gather", deviceNum, false);
-    int launches = 2 + 2 * sel.digits;
+    int launches = 2 + sel.digits;  // init, one counting pass per digit, the gathering pass
     if (compact) {
+        if (sel.sampleVectors) {
+            sel.sample = compileKernel(source, "thor_topk_sample", deviceNum, false);
+            launches += 2;
+        }
         sel.compact = compileKernel(source, "thor_topk_compact", deviceNum, false);
         sel.candidateHistogram = compileKernel(source, "thor_topk_candidate_histogram", deviceNum, false);
         sel.candidateGather = compileKernel(source, "thor_topk_candidate_gather", deviceNum, false);
-        launches = 2 + 2 * sel.digits + (sel.digits - 2) + 1;
     }
     std::ostringstream v;
     v << "top-k radix-select bits" << keyBytes * 8 << " digits" << sel.digits << " vec" << vec << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys")
@@ -360,31 +374,28 @@ void launchTopK(const CubSelectionKernels& sel, const void* keysIn, const void* 
     }
     std::vector<void*> initArgs = {&temp};
     sel.first->launch(1, 1, 1, 256, raw, initArgs);
-    uint32_t everyInput = 0, fallbackOnly = 1;
     for (size_t d = 0; d < sel.digitPlan.size(); ++d) {
         uint32_t shift = sel.digitPlan[d].first, bits = sel.digitPlan[d].second;
-        if (sel.compact && d == 1) {
-            std::vector<void*> compactArgs = {&keysIn, &temp, &shift, &bits};
-            sel.compact->launch(sel.histogramBlocks, 1, 1, 256, raw, compactArgs);
-        } else if (sel.compact && d > 1) {
-            std::vector<void*> candidateArgs = {&temp, &shift, &bits};
-            sel.candidateHistogram->launch(sel.candidateBlocks, 1, 1, 256, raw, candidateArgs);
-            std::vector<void*> histogramArgs = {&keysIn, &temp, &shift, &bits, &fallbackOnly};
-            sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, histogramArgs);
+        std::vector<void*> countArgs = {&keysIn, &temp, &shift, &bits};
+        if (sel.compact && d == 0) {
+            if (sel.sample) {
+                // the floor of the candidates: the two leading digits of the sample's k-th largest key
+                sel.sample->launch(sel.sampleBlocks, 1, 1, 256, raw, countArgs);
+                uint32_t secondShift = sel.digitPlan[1].first, secondBits = sel.digitPlan[1].second;
+                std::vector<void*> secondArgs = {&keysIn, &temp, &secondShift, &secondBits};
+                sel.sample->launch(sel.sampleBlocks, 1, 1, 256, raw, secondArgs);
+            }
+            sel.compact->launch(sel.histogramBlocks, 1, 1, 256, raw, countArgs);
+        } else if (sel.compact) {
+            sel.candidateHistogram->launch(sel.candidateBlocks, 1, 1, 256, raw, countArgs);
         } else {
-            std::vector<void*> histogramArgs = {&keysIn, &temp, &shift, &bits, &everyInput};
-            sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, histogramArgs);
+            sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, countArgs);
         }
-        std::vector<void*> pickArgs = {&temp, &shift, &bits};
-        sel.third->launch(1, 1, 1, 256, raw, pickArgs);
     }
+    std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut};
     if (sel.compact) {
-        std::vector<void*> candidateArgs = {&valuesIn, &temp, &keysOut, &valuesOut};
-        sel.candidateGather->launch(sel.candidateBlocks, 1, 1, 256, raw, candidateArgs);
-        std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut, &fallbackOnly};
-        sel.fourth->launch(sel.fallbackGatherBlocks, 1, 1, sel.threads, raw, gatherArgs);
+        sel.candidateGather->launch(sel.candidateBlocks, 1, 1, 256, raw, gatherArgs);
     } else {
-        std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut, &everyInput};
         sel.fourth->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, gatherArgs);
     }
 }

@@ -433,34 +433,46 @@ int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, 
         const Tensor& in = input->tensor;
         Tensor& out = output->tensor;
         std::shared_ptr<const CubScanKernels> kernels;
+        Tensor temp;
         if (offsets) {
             if (arg) {
                 const auto plan = prepareCubDeviceSegmentedArgScan(in, out, offsets->tensor, num_items, num_segments, argOp, mode, direction);
-                cubDeviceSegmentedArgScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, offsets->tensor, stream->stream);
+                temp = allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes);
+                cubDeviceSegmentedArgScan(plan, temp, in, out, offsets->tensor, stream->stream);
                 kernels = plan.kernels;
             } else {
                 const auto plan = prepareCubDeviceSegmentedScan(in, out, offsets->tensor, num_items, num_segments, valueOp, mode, direction);
-                cubDeviceSegmentedScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, offsets->tensor, stream->stream);
+                temp = allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes);
+                cubDeviceSegmentedScan(plan, temp, in, out, offsets->tensor, stream->stream);
                 kernels = plan.kernels;
             }
         } else if (segment_size > 0) {
             if (arg) {
                 const auto plan = prepareCubDeviceSegmentedUniformArgScan(in, out, num_items, num_items / segment_size, segment_size, argOp, mode, direction);
-                cubDeviceSegmentedUniformArgScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+                temp = allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes);
+                cubDeviceSegmentedUniformArgScan(plan, temp, in, out, stream->stream);
                 kernels = plan.kernels;
             } else {
                 const auto plan = prepareCubDeviceSegmentedUniformScan(in, out, num_items, num_items / segment_size, segment_size, valueOp, mode, direction);
-                cubDeviceSegmentedUniformScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+                temp = allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes);
+                cubDeviceSegmentedUniformScan(plan, temp, in, out, stream->stream);
                 kernels = plan.kernels;
             }
         } else if (arg) {
             const auto plan = prepareCubDeviceArgScan(in, out, num_items, argOp, mode, direction);
-            cubDeviceArgScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+            temp = allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes);
+            cubDeviceArgScan(plan, temp, in, out, stream->stream);
             kernels = plan.kernels;
         } else {
             const auto plan = prepareCubDeviceScan(in, out, num_items, valueOp, mode, direction);
-            cubDeviceScan(plan, allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes), in, out, stream->stream);
+            temp = allocateCubTemporaryStorage(plan.placement, plan.temp_storage_bytes);
+            cubDeviceScan(plan, temp, in, out, stream->stream);
             kernels = plan.kernels;
+        }
+        // this entry point frees its temporary storage on return, which waits for the device anyway: a wait between blocks that
+        // gave up is reported here
+        if (const uint32_t gaveUp = scanWaitsGivenUp(*kernels, temp.getMemPtr(), stream->stream)) {
+            throw std::runtime_error("CUB scan: " + std::to_string(gaveUp) + " wait(s) for the totals of earlier chunks gave up; the results are incomplete.");
         }
         if (variant) copyOut(cubScanKernelVariant(kernels), variant, variant_capacity, nullptr);)
 }
