@@ -448,13 +448,24 @@ __device__ __forceinline__ void topkSample(const typename Cfg::Raw* keys, u32* t
     const u32 floorSoFar = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins)->floor;
     const u32 fixedBits = shift + bits >= 32 ? 0u : (0xffffffffu << (shift + bits));
     const u32 digitMask = numBins - 1u;
-    for (u64 j = (u64)blockIdx.x * 256 + threadIdx.x; j < Cfg::kSampleVectors; j += (u64)gridDim.x * 256) {
-        Pack<Raw, V> x;
-        x.load(keys + ((j / 256) * Cfg::kSampleRunStride + j % 256) * V);
+    constexpr int kUnroll = 4;
+    const u64 stride = (u64)gridDim.x * 256;
+    for (u64 j0 = (u64)blockIdx.x * 256 + threadIdx.x; j0 < Cfg::kSampleVectors; j0 += stride * kUnroll) {
+        Pack<Raw, V> x[kUnroll];
 #pragma unroll
-        for (int k = 0; k < V; ++k) {
-            const u32 image = topkImage<Cfg>(x.v[k]);
-            if ((image & fixedBits) == (floorSoFar & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
+        for (int u = 0; u < kUnroll; ++u) {
+            const u64 j = j0 + u * stride;
+            if (j < Cfg::kSampleVectors) x[u].load(keys + ((j / 256) * Cfg::kSampleRunStride + j % 256) * V);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (j0 + u * stride < Cfg::kSampleVectors) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) {
+                    const u32 image = topkImage<Cfg>(x[u].v[k]);
+                    if ((image & fixedBits) == (floorSoFar & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
+                }
+            }
         }
     }
     __syncthreads();
@@ -470,7 +481,7 @@ __device__ __forceinline__ void topkSample(const typename Cfg::Raw* keys, u32* t
 template <typename Cfg>
 __device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
     typedef typename Cfg::Raw Raw;
-    constexpr int V = Cfg::kVec, kUnroll = 4;
+    constexpr int V = Cfg::kVec, kUnroll = Cfg::kCompactUnroll;
     __shared__ u32 bins[kTopkMaxBins];
     const u32 numBins = 1u << bits;
     for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;

@@ -271,7 +271,9 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     // least 64 entries.
     // The floor of the candidates comes from a sample of max(2^16, 128 k) keys, in runs of 256 vectors: about k / sample of the
     // input, and what shares the floor's bucket with it, becomes candidates.  When k is more than a 256th of the input the
-    // candidates would not fit their regions: every digit then reads the whole input.
+    // candidates would not fit their regions: every digit then reads the whole input.  (Half the sample, twice the candidates,
+    // still fits on average, but not when the input repeats itself: a 2^22-key block tiled to 2^26 keys shows every wavefront
+    // the same few hundred keys sixteen times, and some regions overflowed.)
     bool compact = sel.digits >= 2 && numItems >= kTopKCompactMinItems && numItems < (1ull << 32) && k * 256 <= numItems;
     if (const char* env = std::getenv("THOR_TOPK_CANDIDATES")) {  // tuning / test switch: "0" reads the whole input in every pass
         if (std::string(env) == "0") compact = false;
@@ -280,12 +282,14 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     const uint64_t sampleRuns = std::min<uint64_t>(std::max<uint64_t>(uint64_t(1) << 16, 128 * k) / vec, vectors) / 256;
     sel.sampleVectors = sampleRuns * 256 * vec >= k ? sampleRuns * 256 : 0;  // a sample that holds fewer than k keys gives no floor
     const uint64_t sampleRunStride = sel.sampleVectors ? vectors / sampleRuns : 0;
-    sel.sampleBlocks = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(sel.sampleVectors / 1024, 1), 256));
+    sel.sampleBlocks = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(sel.sampleVectors / 1024, 1), 1024));
     const uint64_t regions = uint64_t(sel.histogramBlocks) * (256 / 64);
     uint64_t regionEntries = std::max<uint64_t>((numItems / 32 + regions - 1) / regions, 64);
     if (const char* env = std::getenv("THOR_TOPK_REGION")) regionEntries = std::max<long>(std::atol(env), 1);  // test switch: entries per wavefront
     // few blocks walk the candidates; the same launches walk the whole input when the regions overflowed, so not too few
-    sel.candidateBlocks = static_cast<uint32_t>(std::min<uint64_t>((regions + 3) / 4, 256));
+    long candidateBlockLimit = 256;
+    if (const char* env = std::getenv("THOR_TOPK_CANDIDATE_BLOCKS")) candidateBlockLimit = std::max<long>(std::atol(env), 1);  // tuning switch
+    sel.candidateBlocks = static_cast<uint32_t>(std::min<uint64_t>((regions + 3) / 4, static_cast<uint64_t>(candidateBlockLimit)));
     sel.tempBytes = (kTopKBins + kTopKStateWords) * 4;
     if (compact) sel.tempBytes += (regions + regions * regionEntries * (pairs ? 2 : 1)) * 4;
     std::ostringstream s;
@@ -295,6 +299,7 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     s << "    static constexpr thor::u64 kTotal = " << numItems << "ull;\n    static constexpr thor::u64 kK = " << k
       << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = " << kGatherThreads
       << ";\n    static constexpr int kItems = " << kGatherItems << ";\n    static constexpr bool kCompact = " << (compact ? "true" : "false")
+      << ";\n    static constexpr int kCompactUnroll = " << (std::getenv("THOR_TOPK_COMPACT_UNROLL") ? std::max(std::atoi(std::getenv("THOR_TOPK_COMPACT_UNROLL")), 1) : 4)
       << ";\n    static constexpr thor::u32 kRegion = " << regionEntries << "u;\n    static constexpr thor::u32 kRegions = " << regions
       << "u;\n    static constexpr thor::u64 kSampleVectors = " << sel.sampleVectors << "ull;\n    static constexpr thor::u64 kSampleRunStride = "
       << sampleRunStride << "ull;\n};\n}  // namespace gen\n";
