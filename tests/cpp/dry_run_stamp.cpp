@@ -152,6 +152,10 @@ static int runAll() {
             stampOne(std::string("scan ") + dtypeName + " exclusive sum - argmin", x.scan(ScanOp::Sum, -1, false), inputs, stream, "Scan");
             stampOne(std::string("scan ") + dtypeName + " argmin", x.scan(ScanOp::ArgMin), inputs, stream, "Scan");
             stampBackward(std::string("backward ") + dtypeName + " sum scan", x.scan(ScanOp::Sum), inputs, fullGradient, stream, "Scan");
+            // one flat scan over several chunks: the kernels whose blocks publish their totals to each other
+            stampOne(std::string("scan ") + dtypeName + " flat sum over 12 chunks", x.reshape({4096 * 24}).scan(ScanOp::Sum), inputs, stream, "Scan");
+            stampOne(std::string("scan ") + dtypeName + " flat exclusive argmax over 12 chunks", x.reshape({4096 * 24}).scan(ScanOp::ArgMax, -1, false), inputs,
+                     stream, "Scan");
         }
         // a scalar kept in device memory next to flat operands
         {
