@@ -10,8 +10,10 @@
 // Top-k is a radix selection on an order-preserving unsigned image of the key (sign handling for floats and signed integers;
 // for "smallest" the image is complemented, so the code always looks for the largest images).  From the most significant
 // digit down (11, 11 and 10 bits of a 32-bit key; 8-bit digits of narrower ones): a histogram of the digit over the keys
-// that still match the digits fixed so far, then the bucket that holds the k-th largest image is fixed.  After the last digit the image T of the k-th key and the number of keys equal to T
-// that belong to the answer are known; one more pass writes every key above T and that many keys equal to T.  The answer is
+// that still match the digits fixed so far, then the bucket that holds the k-th largest image is fixed (by the block of the
+// counting pass that finishes last).  After the last digit the image T of the k-th key and the number of keys equal to T
+// that belong to the answer are known; one more pass writes every key above T and that many keys equal to T.  Long inputs
+// are read once: see "candidates" below.  The answer is
 // the k best keys (with their values, for pairs) in no particular order, like the reference's (its library calls ask for
 // unsorted, not run-to-run deterministic output); which of several equal keys at the threshold are taken is not fixed either.
 // Rows (fixed-size segments of at most 8192 keys) run the same selection inside one block, keys in registers, histogram in LDS.

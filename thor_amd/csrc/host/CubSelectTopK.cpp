@@ -264,7 +264,9 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     const uint64_t chunkVectors = uint64_t(kGatherThreads) * kGatherItems;
     sel.chunks = (vectors + chunkVectors - 1) / chunkVectors;
     // enough striding blocks to keep every compute unit busy, few enough that the global histogram sees little contention
-    sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, 2048));
+    uint64_t histogramBlockLimit = 2048;
+    if (const char* env = std::getenv("THOR_TOPK_BLOCKS")) histogramBlockLimit = std::max<long>(std::atol(env), 1);  // tuning switch
+    sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, histogramBlockLimit));
     // Long inputs with more than one digit: the pass over the input that counts the first digit also copies the keys that can
     // still be part of the answer, and the later digits and the output are taken from those candidates (one read of the input
     // instead of one per digit plus one).  Every wavefront of that pass owns room for its share of a 32nd of the input, at
@@ -282,7 +284,9 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     const uint64_t sampleRuns = std::min<uint64_t>(std::max<uint64_t>(uint64_t(1) << 16, 128 * k) / vec, vectors) / 256;
     sel.sampleVectors = sampleRuns * 256 * vec >= k ? sampleRuns * 256 : 0;  // a sample that holds fewer than k keys gives no floor
     const uint64_t sampleRunStride = sel.sampleVectors ? vectors / sampleRuns : 0;
-    sel.sampleBlocks = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(sel.sampleVectors / 1024, 1), 1024));
+    uint64_t sampleBlockLimit = 1024;
+    if (const char* env = std::getenv("THOR_TOPK_SAMPLE_BLOCKS")) sampleBlockLimit = std::max<long>(std::atol(env), 1);  // tuning switch
+    sel.sampleBlocks = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(sel.sampleVectors / 1024, 1), sampleBlockLimit));
     const uint64_t regions = uint64_t(sel.histogramBlocks) * (256 / 64);
     uint64_t regionEntries = std::max<uint64_t>((numItems / 32 + regions - 1) / regions, 64);
     if (const char* env = std::getenv("THOR_TOPK_REGION")) regionEntries = std::max<long>(std::atol(env), 1);  // test switch: entries per wavefront
