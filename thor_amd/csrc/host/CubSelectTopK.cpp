@@ -264,9 +264,7 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     const uint64_t chunkVectors = uint64_t(kGatherThreads) * kGatherItems;
     sel.chunks = (vectors + chunkVectors - 1) / chunkVectors;
     // enough striding blocks to keep every compute unit busy, few enough that the global histogram sees little contention
-    uint64_t histogramBlockLimit = 2048;
-    if (const char* env = std::getenv("THOR_TOPK_BLOCKS")) histogramBlockLimit = std::max<long>(std::atol(env), 1);  // tuning switch
-    sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, histogramBlockLimit));
+    sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, 2048));
     // Long inputs with more than one digit: the pass over the input that counts the first digit also copies the keys that can
     // still be part of the answer, and the later digits and the output are taken from those candidates (one read of the input
     // instead of one per digit plus one).  Every wavefront of that pass owns room for its share of a 32nd of the input, at
@@ -281,10 +279,18 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
         if (std::string(env) == "0") compact = false;
         if (std::string(env) == "1") compact = sel.digits >= 2 && numItems < (1ull << 32);
     }
+    if (compact) {
+        // Every block of a counting pass ends with additions to the same few words of the shared histogram and a ticket, and those
+        // are served one after the other: 2^26 fp32 keys, k = 64 / 65 536, with 512 / 1024 / 2048 blocks in the pass over the input
+        // 95 / 87 / 97 us and 158 / 133 / 147 us (4096 blocks: regions too small, overflow).
+        uint64_t limit = 1024;
+        if (const char* env = std::getenv("THOR_TOPK_BLOCKS")) limit = std::max<long>(std::atol(env), 1);  // tuning switch
+        sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, limit));
+    }
     const uint64_t sampleRuns = std::min<uint64_t>(std::max<uint64_t>(uint64_t(1) << 16, 128 * k) / vec, vectors) / 256;
     sel.sampleVectors = sampleRuns * 256 * vec >= k ? sampleRuns * 256 : 0;  // a sample that holds fewer than k keys gives no floor
     const uint64_t sampleRunStride = sel.sampleVectors ? vectors / sampleRuns : 0;
-    uint64_t sampleBlockLimit = 1024;
+    uint64_t sampleBlockLimit = 256;  // 8.4 M sampled keys: 147 us for the whole top-k with 1024 blocks, 133 us with 256
     if (const char* env = std::getenv("THOR_TOPK_SAMPLE_BLOCKS")) sampleBlockLimit = std::max<long>(std::atol(env), 1);  // tuning switch
     sel.sampleBlocks = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(sel.sampleVectors / 1024, 1), sampleBlockLimit));
     const uint64_t regions = uint64_t(sel.histogramBlocks) * (256 / 64);
