@@ -72,19 +72,38 @@ __device__ __forceinline__ u32 selectFlagBits(const u8* flags, u64 first) {
     return bits;
 }
 
+// The raised flags of every chunk.  A wavefront counts one chunk (the count does not care in which order the scattering pass
+// will read the chunk): sixteen flag bytes per lane and load, all loads of the chunk in flight, no LDS and no barrier.  Launched
+// with kChunks / (kThreads / 64) blocks, rounded up.
 template <typename Cfg>
 __device__ __forceinline__ void selectCount(const u8* flags, u32* counts) {
-    __shared__ u32 lds[Cfg::kThreads / kWave];
-    const u64 chunkBase = (u64)blockIdx.x * SelectChunk<Cfg>::kElems;
+    constexpr u64 kElems = SelectChunk<Cfg>::kElems;
+    const int lane = threadIdx.x % kWave;
+    const u64 chunk = (u64)blockIdx.x * (Cfg::kThreads / kWave) + threadIdx.x / kWave;
+    if (chunk >= Cfg::kChunks) return;
+    const u64 chunkBase = chunk * kElems;
     u32 mine = 0;
+    if (Cfg::kVec == 4 && kElems % (kWave * 16) == 0 && chunkBase + kElems <= Cfg::kTotal) {
+        constexpr int kLoads = (int)(kElems / (kWave * 16));
+        Pack<u32, 4> words[kLoads];
 #pragma unroll
-    for (int round = 0; round < Cfg::kRounds; ++round) {
-        const u64 first = chunkBase + ((u64)round * Cfg::kThreads + threadIdx.x) * Cfg::kVec;
-        if (first < Cfg::kTotal) mine += (u32)__builtin_popcount(selectFlagBits<Cfg>(flags, first));
+        for (int j = 0; j < kLoads; ++j) words[j].loadStream(reinterpret_cast<const u32*>(flags + chunkBase) + ((u64)j * kWave + lane) * 4);
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const u32 w = words[j].v[k];
+                mine += (u32)__builtin_popcount((((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) & 0x80808080u);  // bytes that are not zero
+            }
+        }
+    } else {
+        for (u64 first = chunkBase + (u64)lane * Cfg::kVec; first < chunkBase + kElems && first < Cfg::kTotal; first += (u64)kWave * Cfg::kVec) {
+            mine += (u32)__builtin_popcount(selectFlagBits<Cfg>(flags, first));
+        }
     }
-    u32 total;
-    (void)blockExclusiveSum<Cfg::kThreads>(mine, lds, total);
-    if (threadIdx.x == 0) counts[blockIdx.x] = total;
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_xor(mine, d, kWave);
+    if (lane == 0) counts[chunk] = mine;
 }
 
 // One block of 1024 threads: counts[kChunks] -> bases[kChunks] (exclusive), the grand total -> *numSelected.  A thread owns a

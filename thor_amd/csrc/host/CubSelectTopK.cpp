@@ -507,7 +507,8 @@ void cubDeviceSelectFlagged(const CubDeviceSelectFlaggedPlan& plan, const Tensor
     void* out = output.getMemPtr();
     void* total = numSelected.getMemPtr();
     std::vector<void*> countArgs = {&flagBytes, &counts};
-    k.first->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, countArgs);
+    const uint64_t chunksPerBlock = k.threads / 64;  // a wavefront counts a chunk
+    k.first->launch(static_cast<uint32_t>((k.chunks + chunksPerBlock - 1) / chunksPerBlock), 1, 1, k.threads, raw, countArgs);
     std::vector<void*> offsetArgs = {&counts, &bases, &total};
     k.second->launch(1, 1, 1, 1024, raw, offsetArgs);
     if (plan.num_items == 0) return;
