@@ -562,6 +562,28 @@ __device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* 
     topkPickWhenLast<Cfg>(temp, shift, bits);
 }
 
+// A wavefront's walk over its candidate regions (region = first, first + step, ...): the counts of kTopkRegionBatch regions
+// are loaded together, then the first 64 entries of each (most regions hold fewer), so a region costs no round trip of its
+// own; `visit(word, region, index)` sees every entry once.
+constexpr int kTopkRegionBatch = 4;
+template <typename Cfg, typename Visit>
+__device__ __forceinline__ void topkWalkRegions(const u32* counts, const u32* entries, u32 first, u32 step, const Visit& visit) {
+    const u32 lane = threadIdx.x % kWave;
+    for (u32 r0 = first; r0 < Cfg::kRegions; r0 += step * kTopkRegionBatch) {
+        u32 count[kTopkRegionBatch], word[kTopkRegionBatch];
+#pragma unroll
+        for (int j = 0; j < kTopkRegionBatch; ++j) count[j] = r0 + j * step < Cfg::kRegions ? counts[r0 + j * step] : 0u;
+#pragma unroll
+        for (int j = 0; j < kTopkRegionBatch; ++j)
+            if (lane < count[j]) word[j] = entries[(u64)(r0 + j * step) * Cfg::kRegion + lane];
+#pragma unroll
+        for (int j = 0; j < kTopkRegionBatch; ++j) {
+            if (lane < count[j]) visit(word[j], r0 + j * step, lane);
+            for (u32 i = lane + kWave; i < count[j]; i += kWave) visit(entries[(u64)(r0 + j * step) * Cfg::kRegion + i], r0 + j * step, i);
+        }
+    }
+}
+
 // kCandidateBlocks blocks of 256 threads: histogram of the digit at `shift` over the candidates that match the digits fixed so far.
 template <typename Cfg>
 __device__ __forceinline__ void topkCandidateHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
@@ -581,13 +603,10 @@ __device__ __forceinline__ void topkCandidateHistogram(const typename Cfg::Raw* 
     const int lane = threadIdx.x % kWave;
     const u32* counts = TopkCandidates<Cfg>::counts(temp);
     const u32* candidateKeys = TopkCandidates<Cfg>::keys(temp);
-    for (u32 region = blockIdx.x * (256 / kWave) + threadIdx.x / kWave; region < Cfg::kRegions; region += gridDim.x * (256 / kWave)) {
-        const u32 count = counts[region];
-        for (u32 i = lane; i < count; i += kWave) {
-            const u32 image = topkImage<Cfg>((Raw)candidateKeys[(u64)region * Cfg::kRegion + i]);
-            if ((image & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
-        }
-    }
+    topkWalkRegions<Cfg>(counts, candidateKeys, blockIdx.x * (256 / kWave) + threadIdx.x / kWave, gridDim.x * (256 / kWave), [&](u32 word, u32, u32) {
+        const u32 image = topkImage<Cfg>((Raw)word);
+        if ((image & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
+    });
     __syncthreads();
     for (u32 b = threadIdx.x; b < numBins; b += 256) {
         const u32 mine = bins[b];
@@ -616,14 +635,11 @@ __device__ __forceinline__ void topkCandidateGather(const typename Cfg::Raw* key
     const u32* candidatePositions = TopkCandidates<Cfg>::positions(temp);
     const u32 firstRegion = blockIdx.x * (256 / kWave) + threadIdx.x / kWave, regionStep = gridDim.x * (256 / kWave);
     u32 above = 0, ties = 0;
-    for (u32 region = firstRegion; region < Cfg::kRegions; region += regionStep) {
-        const u32 count = counts[region];
-        for (u32 i = lane; i < count; i += kWave) {
-            const u32 image = topkImage<Cfg>((Raw)candidateKeys[(u64)region * Cfg::kRegion + i]);
-            above += image > threshold;
-            ties += image == threshold;
-        }
-    }
+    topkWalkRegions<Cfg>(counts, candidateKeys, firstRegion, regionStep, [&](u32 word, u32, u32) {
+        const u32 image = topkImage<Cfg>((Raw)word);
+        above += image > threshold;
+        ties += image == threshold;
+    });
     u32 blockAbove, blockTies;
     u32 aboveAt = blockExclusiveSum<256>(above, lds, blockAbove);
     u32 tieAt = blockExclusiveSum<256>(ties, lds, blockTies);
@@ -635,24 +651,20 @@ __device__ __forceinline__ void topkCandidateGather(const typename Cfg::Raw* key
     __syncthreads();
     aboveAt += bases[0];
     tieAt += bases[1];
-    for (u32 region = firstRegion; region < Cfg::kRegions; region += regionStep) {
-        const u32 count = counts[region];
-        for (u32 i = lane; i < count; i += kWave) {
-            const u64 at = (u64)region * Cfg::kRegion + i;
-            const u32 word = candidateKeys[at];
-            const u32 image = topkImage<Cfg>((Raw)word);
-            u32 slot = 0xffffffffu;
-            if (image > threshold) slot = aboveAt++;
-            if (image == threshold) {
-                const u32 rank = tieAt++;
-                if (rank < wantedTies) slot = firstTieSlot + rank;
-            }
-            if (slot != 0xffffffffu) {
-                outKeys[slot] = (Raw)word;
-                if (Cfg::kPairs) outValues[slot] = values[candidatePositions[at]];
-            }
+    // the same entries per thread as in the count above: every thread hands out the ranks it counted
+    topkWalkRegions<Cfg>(counts, candidateKeys, firstRegion, regionStep, [&](u32 word, u32 region, u32 index) {
+        const u32 image = topkImage<Cfg>((Raw)word);
+        u32 slot = 0xffffffffu;
+        if (image > threshold) slot = aboveAt++;
+        if (image == threshold) {
+            const u32 rank = tieAt++;
+            if (rank < wantedTies) slot = firstTieSlot + rank;
         }
-    }
+        if (slot != 0xffffffffu) {
+            outKeys[slot] = (Raw)word;
+            if (Cfg::kPairs) outValues[slot] = values[candidatePositions[(u64)region * Cfg::kRegion + index]];
+        }
+    });
 }
 
 // ---- top-k of every row: one block per row ------------------------------------------------------------------------------------------
