@@ -600,7 +600,6 @@ __device__ __forceinline__ void topkCandidateHistogram(const typename Cfg::Raw* 
     const u32 prefix = state->prefix;
     const u32 fixedBits = shift + bits >= 32 ? 0u : (0xffffffffu << (shift + bits));
     const u32 digitMask = numBins - 1u;
-    const int lane = threadIdx.x % kWave;
     const u32* counts = TopkCandidates<Cfg>::counts(temp);
     const u32* candidateKeys = TopkCandidates<Cfg>::keys(temp);
     topkWalkRegions<Cfg>(counts, candidateKeys, blockIdx.x * (256 / kWave) + threadIdx.x / kWave, gridDim.x * (256 / kWave), [&](u32 word, u32, u32) {
@@ -629,7 +628,6 @@ __device__ __forceinline__ void topkCandidateGather(const typename Cfg::Raw* key
         return;
     }
     const u32 threshold = state->prefix, wantedTies = state->remaining, firstTieSlot = (u32)Cfg::kK - wantedTies;
-    const int lane = threadIdx.x % kWave;
     const u32* counts = TopkCandidates<Cfg>::counts(temp);
     const u32* candidateKeys = TopkCandidates<Cfg>::keys(temp);
     const u32* candidatePositions = TopkCandidates<Cfg>::positions(temp);
