@@ -197,3 +197,20 @@ def test_published_totals_agree_with_separate_passes(stream, monkeypatch, n, seg
     else:
         check(got, carrier, dtype, op, True, reverse)
         check(separate, carrier, dtype, op, True, reverse)
+
+
+@pytest.mark.parametrize("dtype,op,inclusive,reverse", [(DataType.uint32, ScanOp.sum, True, False), (DataType.fp32, ScanOp.max, False, True),
+                                                        (DataType.bf16, ScanOp.arg_min, True, False)], ids=["u32-sum", "fp32-max-excl-rev", "bf16-argmin"])
+def test_rows_longer_than_a_chunk_at_a_size_that_takes_the_large_blocks(stream, dtype, op, inclusive, reverse):
+    """672 rows of 50 257 elements (33.8 million): every row spans several chunks of the 1 024-thread blocks, heads fall inside
+    vectors, and a chunk reads what precedes it in its row from totals published by other blocks, two levels deep."""
+    rng = np.random.default_rng(53)
+    rows, length = 672, 50257
+    if dtype == DataType.uint32:
+        carrier = rng.integers(0, 1 << 32, rows * length, dtype=np.uint64).astype(np.uint32)
+    else:
+        carrier = to_storage((np.round(rng.standard_normal(rows * length) * 8) / 8).astype(np.float32), dtype)
+    carrier = carrier.reshape(rows, length)
+    got, variant = run_scan(carrier, dtype, stream, op, inclusive, reverse, segment_size=length)
+    assert "threads=1024" in variant and "published_totals" in variant, variant
+    check(got, carrier, dtype, op, inclusive, reverse, segment_size=length)
