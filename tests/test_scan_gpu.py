@@ -214,3 +214,17 @@ def test_rows_longer_than_a_chunk_at_a_size_that_takes_the_large_blocks(stream, 
     got, variant = run_scan(carrier, dtype, stream, op, inclusive, reverse, segment_size=length)
     assert "threads=1024" in variant and "published_totals" in variant, variant
     check(got, carrier, dtype, op, inclusive, reverse, segment_size=length)
+
+
+def test_a_wait_that_gives_up_is_reported(stream, monkeypatch):
+    """Waits between blocks are bounded so that every wavefront has an exit.  With the bound forced to zero polls a chunk that
+    needs a total gives up at once (every kernel still runs to its end), and thor_scan reports that instead of handing back
+    incomplete results; the same scan with the ordinary bound is exact."""
+    x = np.ones(1 << 22, np.uint32)
+    monkeypatch.setenv("THOR_SCAN_WAIT_LIMIT", "0")
+    with pytest.raises(RuntimeError, match="gave up"):
+        run_scan(x, DataType.uint32, stream, ScanOp.sum, True, False)
+    monkeypatch.delenv("THOR_SCAN_WAIT_LIMIT")
+    got, variant = run_scan(x, DataType.uint32, stream, ScanOp.sum, True, False)
+    assert "published_totals" in variant, variant
+    np.testing.assert_array_equal(got, np.arange(1, x.size + 1, dtype=np.uint32))

@@ -24,7 +24,7 @@
 // Cfg: T (storage), Acc (u32 for UINT32, float otherwise), kUnsigned, kOp (0 sum, 1 min, 2 max, 3 product), kArg, kInclusive, kReverse,
 // kTotal, kRow (row length; 0 = heads come from a bitmap), kThreads, kVec, kItems, kChunkElems (positions per block, a
 // multiple of kVec, at most kThreads * kVec * kItems), kChunks, kCarry, kLookback (with kCarry: what precedes a chunk comes
-// from the published totals, not from a carries array), kClearWords, kWriteValue, kWriteIndex.
+// from the published totals, not from a carries array; kWaitLimit polls bound every wait), kClearWords, kWriteValue, kWriteIndex.
 #pragma once
 
 namespace thor {
@@ -171,7 +171,6 @@ struct ScanRunSum {
 // the value, the second (min / max only) the index.  Every word is written once per run, whole, after the block was
 // cleared, so a reader that sees the tag sees the state: no fences.
 constexpr u32 kScanControlWords = 32;
-constexpr u32 kScanWaitLimit = 1u << 22;  // polls before a wait gives up (seconds); never reached while earlier tickets run
 
 template <typename Cfg>
 __device__ __forceinline__ void scanPublish(u64* entries, u64 entry, const ScanState<Cfg>& s) {
@@ -209,7 +208,7 @@ __device__ __forceinline__ ScanState<Cfg> scanAwait(u64* entries, u64 first, u32
     for (u32 polls = 0;; ++polls) {
         const bool ready = !mine || ((seen.w0 & 1u) != 0 && (!kIndexed || (seen.w1 & 1u) != 0));
         if (__ballot(!ready) == 0) break;
-        if (polls >= kScanWaitLimit) {
+        if (polls >= Cfg::kWaitLimit) {  // polls before a wait gives up: seconds' worth, never reached while earlier tickets run
             if (lane == 0) atomicAdd(reinterpret_cast<u32*>(control + 1), 1u);
             break;
         }

@@ -95,6 +95,10 @@ ScanChunking chooseScanChunking(const ScanRequest& r) {
 
 void writeScanTraits(std::ostringstream& s, const ScanRequest& r, bool isUnsigned, uint64_t threads, uint64_t vec, uint64_t items, uint64_t chunkElems,
                      const CubScanKernels& k) {
+    // Waits between blocks are bounded so that every wavefront has an exit: 2^22 polls are seconds.  The test switch makes the
+    // bound so small that waits give up, to exercise how that is reported (the kernels still run to their end).
+    unsigned long waitLimit = 1ul << 22;
+    if (const char* env = std::getenv("THOR_SCAN_WAIT_LIMIT")) waitLimit = std::min<unsigned long>(std::strtoul(env, nullptr, 10), 1ul << 30);
     s << "namespace gen {\nstruct Cfg {\n    typedef " << scanStorageName(r.dtype) << " T;\n    typedef " << (isUnsigned ? "thor::u32" : "float")
       << " Acc;\n    typedef " << (r.offsets64 ? "thor::u64" : "thor::u32") << " OffsetT;\n"
       << "    static constexpr bool kUnsigned = " << (isUnsigned ? "true" : "false") << ";\n    static constexpr int kOp = " << r.op
@@ -105,7 +109,7 @@ void writeScanTraits(std::ostringstream& s, const ScanRequest& r, bool isUnsigne
       << ";\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kItems = " << items
       << ";\n    static constexpr thor::u64 kChunkElems = " << chunkElems << "ull;\n    static constexpr thor::u64 kChunks = " << k.chunks
       << "ull;\n    static constexpr bool kCarry = " << (k.carry ? "true" : "false") << ";\n    static constexpr bool kLookback = "
-      << (k.lookback ? "true" : "false") << ";\n    static constexpr thor::u64 kClearWords = " << k.clearWords
+      << (k.lookback ? "true" : "false") << ";\n    static constexpr thor::u32 kWaitLimit = " << waitLimit << "u;\n    static constexpr thor::u64 kClearWords = " << k.clearWords
       << "ull;\n    static constexpr bool kWriteValue = "
       << (r.writeValue ? "true" : "false") << ";\n    static constexpr bool kWriteIndex = " << (r.writeIndex ? "true" : "false") << ";\n};\n}  // namespace gen\n";
 }
