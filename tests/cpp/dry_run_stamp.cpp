@@ -7,6 +7,8 @@
 
 #include "Utilities/Expression/FusedEquation.h"
 #include "Utilities/Expression/RaggedExpression.h"
+#include "Utilities/TensorOperations/Cub/CubDevicePrimitives.h"
+#include "Utilities/TensorOperations/Cub/CubReduction.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -275,6 +277,39 @@ static int runAll() {
                 }
             }
         }
+    }
+    // The primitives next to the expressions: their kernels are generated and compiled when a plan is prepared.  Top-k with and
+    // without candidates (long and short inputs, keys and pairs, 32- and 16-bit keys), rows, select-flagged, scans over the
+    // segments of an offsets tensor and over rows longer than a chunk, column reductions over an inner extent no vector divides.
+    auto primitive = [&](const std::string& name, const std::function<void()>& prepare) {
+        std::printf("[ RUN  ] %s\n", name.c_str());
+        std::fflush(stdout);
+        prepare();
+        ++stamped;
+    };
+    for (const auto& [dtypeName, dtype] : std::vector<std::pair<const char*, DataType>>{{"fp32", DataType::FP32}, {"bf16", DataType::BF16}}) {
+        for (const uint64_t n : {uint64_t(5000), uint64_t(1) << 21}) {
+            Tensor keys(gpuPlacement, TensorDescriptor(dtype, {n})), best(gpuPlacement, TensorDescriptor(dtype, {64}));
+            Tensor values(gpuPlacement, TensorDescriptor(DataType::UINT32, {n})), bestValues(gpuPlacement, TensorDescriptor(DataType::UINT32, {64}));
+            primitive(std::string("top-k keys ") + dtypeName + " of " + std::to_string(n), [&] { (void)prepareCubDeviceTopKKeys(keys, best, n, 64, CubTopKOrder::Largest); });
+            primitive(std::string("top-k pairs ") + dtypeName + " of " + std::to_string(n),
+                      [&] { (void)prepareCubDeviceTopKPairs(keys, best, values, bestValues, n, 64, CubTopKOrder::Smallest); });
+        }
+        Tensor rows(gpuPlacement, TensorDescriptor(dtype, {256, 4096})), rowBest(gpuPlacement, TensorDescriptor(dtype, {256, 64}));
+        primitive(std::string("top-k of rows ") + dtypeName, [&] { (void)prepareCubDeviceSegmentedTopKKeys(rows, rowBest, 256, 4096, 64, CubTopKOrder::Largest); });
+        Tensor x(gpuPlacement, TensorDescriptor(dtype, {uint64_t(1) << 20})), y(gpuPlacement, TensorDescriptor(dtype, {uint64_t(1) << 20}));
+        Tensor flags(gpuPlacement, TensorDescriptor(DataType::UINT8, {uint64_t(1) << 20})), count(gpuPlacement, TensorDescriptor(DataType::UINT32, {1}));
+        primitive(std::string("select-flagged ") + dtypeName, [&] { (void)prepareCubDeviceSelectFlagged(x, flags, y, count, uint64_t(1) << 20); });
+        Tensor offsets(gpuPlacement, TensorDescriptor(DataType::UINT32, {101}));
+        for (uint32_t i = 0; i <= 100; ++i) static_cast<uint32_t*>(offsets.getMemPtr())[i] = i * 10000u;
+        primitive(std::string("scan over offset segments ") + dtypeName,
+                  [&] { (void)prepareCubDeviceSegmentedScan(x, y, offsets, 1000000, 100, CubScanOp::Max, CubScanMode::Exclusive, CubScanDirection::Reverse); });
+        primitive(std::string("scan over rows longer than a chunk ") + dtypeName, [&] {
+            (void)prepareCubDeviceSegmentedUniformScan(x, y, uint64_t(1) << 20, 16, uint64_t(1) << 16, CubScanOp::Sum, CubScanMode::Inclusive, CubScanDirection::Forward);
+        });
+        Tensor odd(gpuPlacement, TensorDescriptor(dtype, {300, 1001}));
+        primitive(std::string("column sum over an inner extent of 1001 ") + dtypeName, [&] { (void)CubReduction(CubReductionOp::Sum, {0}, DataType::FP32).stamp(odd, stream); });
+        primitive(std::string("column arg-max over an inner extent of 1001 ") + dtypeName, [&] { (void)CubArgReduction(CubArgReductionOp::ArgMax, {0}).stamp(odd, stream); });
     }
     std::printf("%d expressions stamped, 0 failures\n", stamped);
     return 0;
