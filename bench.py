@@ -642,13 +642,18 @@ def main():
         b_.free()
     if not args.no_other_configs:
         result["other_configs"] = bench_other_configs([part for part in args.lines.split(",") if part] or None)
-        # the fraction of the HBM peak every secondary line reached, next to the headline kernel's (kept compact: drivers keep the parsed line)
-        result["roofline"]["per_config"] = {"c2_convert_fp32_to_fp16": round(achieved / HBM_PEAK_GBPS, 4),
-                                            **{name: round(v["GB/s"] / HBM_PEAK_GBPS, 4) for name, v in result["other_configs"].items()}}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
         if not args.no_other_configs:
             result["cpu_baseline_other_configs"] = cpu_baseline_other_configs()
+    if not args.no_other_configs:
+        # The fraction of the HBM peak of every line, as the last key of the JSON line so that it survives in a record that keeps
+        # only the end of the output: the BASELINE configurations first (C2's four directions together, then C1, C3, C4, C5 in
+        # the order bench_other_configs runs them), the lines next to the path after them.
+        fractions = {"c2_convert_round_trip_2^%d" % args.log2_elements: round(value / HBM_PEAK_GBPS, 4),
+                     "c2_convert_fp32_to_fp16": round(achieved / HBM_PEAK_GBPS, 4)}
+        fractions.update({name: round(v["GB/s"] / HBM_PEAK_GBPS, 4) for name, v in result["other_configs"].items()})
+        result["per_config_frac"] = fractions
     print(json.dumps(result))
 
 

@@ -224,6 +224,10 @@ void cubDeviceSegmentedArgScan(const CubDeviceSegmentedArgScanPlan& plan, const 
 
 // How a plan runs: chunk size, vector width, grid, number of launches (diagnostics and tests).
 [[nodiscard]] std::string cubScanKernelVariant(const std::shared_ptr<const CubScanKernels>& kernels);
+// Diagnostic: how many bounded waits between the blocks of the last run on `temp_storage` gave up.  Such a wait computes the
+// totals it lacks from the input, in the order their owners would have, so a run's results are complete and the same bits either
+// way; the count is 0 in normal operation (a block only waits for blocks that started before it).  Synchronises `stream`.
+[[nodiscard]] uint32_t cubScanWaitsRecovered(const std::shared_ptr<const CubScanKernels>& kernels, const Tensor& temp_storage, Stream& stream);
 
 // ---- top-k: the k largest (or smallest) keys, in no particular order; which of several equal keys at the boundary are taken is ----
 // ---- not fixed (the reference asks its library for unsorted, not run-to-run deterministic output: CubTopK.cu:34-36 there) -----------

@@ -141,11 +141,17 @@ int thor_segmented_broadcast(thor_tensor_t per_segment_values, thor_tensor_t seg
  * storage and run in one call.  op: 0 sum, 1 min, 2 max, 3 product; arg != 0 (op 1 or 2): output holds UINT32 flattened indices
  * of the winning prefix element.  Segments: offsets != NULL -> the num_segments segments of an offsets tensor; else
  * segment_size > 0 -> num_items / segment_size rows; else one scan.  `variant` (may be NULL) receives how the plan runs.
- * The call returns when the scan has run (it owns the temporary storage and frees it), and fails if a block of a scan whose
- * chunks read each other's totals gave up a wait (bounded so that every wavefront has an exit; not reachable while the blocks
- * of earlier chunks run). */
+ * The call returns when the scan has run (it owns the temporary storage and frees it). */
 int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments, uint64_t segment_size,
               int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity);
+
+/* Diagnostic (no counterpart in the reference, whose scans never return a partial result either): blocks of a one-launch scan
+ * read the totals of earlier chunks from each other, and every such wait is bounded so that each wavefront has an exit.  A wait
+ * that gives up computes the totals it lacks from the input in the order their owners would have, so every scan entry point -
+ * thor_scan, thor_scan_no_alloc, the plan / run functions of CubDevicePrimitives.h, the Scan stage of a stamped Expression -
+ * returns complete results, the same bits, whether or not a wait gave up.  This returns how many waits did so over all
+ * thor_scan calls of the process so far (0 in normal operation: a block only waits for blocks that started before it). */
+uint64_t thor_scan_waits_recovered(void);
 
 /* Select-flagged (Utilities/TensorOperations/Cub/CubDevicePrimitives.h:87-93,490-516 there): output receives the elements of input
  * whose flag (BOOLEAN or UINT8) is nonzero, in input order, and *num_selected_out (UINT32) their number; prepare, allocate the

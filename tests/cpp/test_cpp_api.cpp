@@ -747,6 +747,28 @@ static void devicePrefixScans(Stream& stream) {
         cubDeviceScan(carried, allocateCubTemporaryStorage(gpuPlacement, 1), big, bigOut, stream);  // too little temporary storage
     }));
     CHECK(isCubScanDTypeSupported(DataType::BF16) && !isCubScanDTypeSupported(DataType::INT32) && isCubSegmentOffsetDTypeSupported(DataType::UINT64));
+    {
+        // A bounded wait between blocks that gives up (forced: a bound of zero polls) works the totals it lacks out of the input:
+        // the plan / run entry point hands back complete results (CubScan.cu there never returns a partial result either), and
+        // the diagnostic says that waits took the way out.
+        setenv("THOR_SCAN_WAIT_LIMIT", "0", 1);
+        const uint64_t n = 1 << 20;
+        const Tensor ones = upload(std::vector<uint32_t>(n, 1u), {n});
+        Tensor counted(gpuPlacement, TensorDescriptor(DataType::UINT32, {n}));
+        const CubDeviceScanPlan impatient = prepareCubDeviceScan(ones, counted, n, CubScanOp::Sum, CubScanMode::Inclusive);
+        unsetenv("THOR_SCAN_WAIT_LIMIT");
+        CHECK(cubScanKernelVariant(impatient.kernels).find("published_totals") != std::string::npos);
+        const Tensor temp = allocateCubTemporaryStorage(gpuPlacement, impatient.temp_storage_bytes);
+        cubDeviceScan(impatient, temp, ones, counted, stream);
+        const std::vector<uint32_t> got = toHostRaw<uint32_t>(counted, stream);
+        bool counts = got.size() == n;
+        for (uint64_t i = 0; counts && i < n; ++i) counts = got[i] == i + 1;
+        CHECK(counts);
+        CHECK(cubScanWaitsRecovered(impatient.kernels, temp, stream) > 0);
+        const CubDeviceScanPlan patient = prepareCubDeviceScan(ones, counted, n, CubScanOp::Sum, CubScanMode::Inclusive);
+        cubDeviceScan(patient, temp, ones, counted, stream);
+        CHECK(cubScanWaitsRecovered(patient.kernels, temp, stream) == 0);
+    }
     // through the Expression: one Scan stage
     const FusedEquation running = FusedEquation::compile(Expression::outputs({{"y", Expression::input("x").scan(ScanOp::Max)}}).physicalOutputs(), 0);
     StampedExecutionPlan plan = running.stamp({{"x", rows}}, stream);

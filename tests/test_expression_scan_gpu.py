@@ -222,10 +222,16 @@ def winners_gradient(values, grad, op, inclusive, reverse=False, segment_size=0,
     return expected.reshape(values.shape)
 
 
-@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16], ids=lambda d: d.name)
-@pytest.mark.parametrize("inclusive,reverse", [(True, False), (False, False), (True, True), (False, True)])
-@pytest.mark.parametrize("name", ["min", "max"])
-@pytest.mark.parametrize("shape", [(64, 1000), (3, 20000), (1, 7), (16, 8192), (300, 256), (37, 33), (9, 4100)], ids=str)
+# Every shape meets every (inclusive, reverse) pair in fp32, min and max taking turns; bf16 meets every shape once, with the
+# other operation, and every pair at least once.
+ROUTE_SHAPES = [(64, 1000), (3, 20000), (1, 7), (16, 8192), (300, 256), (37, 33), (9, 4100)]
+ROUTE_MODES = [(True, False), (False, False), (True, True), (False, True)]
+ROUTE_CASES = [(s, ("min", "max")[(i + j) % 2], m[0], m[1], DataType.fp32) for i, s in enumerate(ROUTE_SHAPES) for j, m in enumerate(ROUTE_MODES)]
+ROUTE_CASES += [(s, ("max", "min")[i % 2], *ROUTE_MODES[i % 4], DataType.bf16) for i, s in enumerate(ROUTE_SHAPES)]
+
+
+@pytest.mark.parametrize("shape,name,inclusive,reverse,dtype", ROUTE_CASES,
+                         ids=[f"{s}-{n}-{'incl' if i else 'excl'}{'-rev' if r else ''}-{d.name}" for s, n, i, r, d in ROUTE_CASES])
 def test_row_minmax_scan_backward(stream, shape, name, inclusive, reverse, dtype):
     rng = np.random.default_rng(61)
     # few distinct values: long runs of one winner, and ties that the first occurrence must win

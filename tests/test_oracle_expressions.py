@@ -43,6 +43,33 @@ def test_softmax_rows_bf16_and_normalize_rows():
     np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
 
 
+def test_softmax_and_normalize_at_the_row_lengths_of_the_baseline_config():
+    """Rows of 4 096 bf16 (softmax) and 1 024 fp32 (normalise), the lengths the full-size GPU comparison runs on: the fp32
+    row sums of the restatement (pairwise) stay within 3e-6 of the float64 closed form there, and every softmax row sums
+    to one."""
+    rng = np.random.default_rng(1239)
+    x = (rng.standard_normal((48, 4096)) * 3).astype(np.float32)
+    x[0] = 0.0  # a flat row: every probability is 1/4096 exactly
+    x[1, :] = -30.0
+    x[1, 77] = 30.0  # one dominant element: the others underflow towards 0 without disturbing the sum
+    bits = oracle.convert(x, oracle.FP32, oracle.BF16)
+    got, _ = oracle.softmax_rows_bf16(bits)
+    xb = oracle.convert(bits, oracle.BF16, oracle.FP32).astype(np.float64)
+    p = np.exp(xb - xb.max(axis=1, keepdims=True))
+    want = p / p.sum(axis=1, keepdims=True)
+    np.testing.assert_allclose(got, want, rtol=3e-6, atol=1e-30)
+    np.testing.assert_array_equal(got[0], np.full(4096, 1.0 / 4096, np.float32))
+    assert got[1, 77] == 1.0
+    np.testing.assert_allclose(got.astype(np.float64).sum(axis=1), 1.0, rtol=2e-6)
+    y = (rng.standard_normal((96, 1024)) * 4 + 1).astype(np.float32)
+    got, _ = oracle.normalize_rows_f32(y, 1e-5)
+    y64 = y.astype(np.float64)
+    mu = y64.mean(axis=1, keepdims=True)
+    want = (y64 - mu) / np.sqrt(((y64 - mu) ** 2).mean(axis=1, keepdims=True) + 1e-5)
+    # x - mean cancels near the mean: the absolute term is a few fp32 roundings of |x| ~ 16 divided by sigma ~ 4
+    np.testing.assert_allclose(got, want, rtol=3e-6, atol=3e-6)
+
+
 def test_fp16_relu_scale_bias_is_bit_exact_with_ieee_half_arithmetic_and_stats_accumulate_in_fp32():
     rng = np.random.default_rng(1238)
     x = rng.standard_normal((3, 8, 5, 7)).astype(np.float16)

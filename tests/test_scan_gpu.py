@@ -71,11 +71,17 @@ def check(got, carrier, dtype, op, inclusive, reverse, **segments):
 SHAPES = [("rows", (300, 64)), ("rows", (5, 4099)), ("rows", (3, 70000)), ("rows", (2048, 3)), ("flat", (1, 1 << 20))]
 
 
-@pytest.mark.parametrize("reverse", [False, True], ids=["forward", "reverse"])
-@pytest.mark.parametrize("inclusive", [True, False], ids=["inclusive", "exclusive"])
-@pytest.mark.parametrize("op", [ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.product, ScanOp.arg_min, ScanOp.arg_max], ids=lambda o: o.name)
-@pytest.mark.parametrize("dtype", [DataType.uint32, DataType.fp32, DataType.fp16, DataType.bf16], ids=lambda d: d.name)
-@pytest.mark.parametrize("kind,shape", SHAPES, ids=[f"{k}{s}" for k, s in SHAPES])
+SCAN_OPS = [ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.product, ScanOp.arg_min, ScanOp.arg_max]
+SCAN_DTYPES = [DataType.uint32, DataType.fp32, DataType.fp16, DataType.bf16]
+SCAN_MODES = [(True, False), (False, False), (True, True), (False, True)]  # (inclusive, reverse)
+# Shape (which chunking the planner picks), dtype and operation (the arithmetic) in full; mode and direction are switches of the
+# same code, so each (shape, dtype, operation) takes one of their four combinations, turning so that every (shape, dtype),
+# (shape, operation) and (dtype, operation) pair meets all four (or, for the six operations, at least three of them).
+ROWS_AND_FLAT = [(k, s, d, o, *SCAN_MODES[(i + j + m) % 4]) for i, (k, s) in enumerate(SHAPES) for j, d in enumerate(SCAN_DTYPES) for m, o in enumerate(SCAN_OPS)]
+
+
+@pytest.mark.parametrize("kind,shape,dtype,op,inclusive,reverse", ROWS_AND_FLAT,
+                         ids=[f"{k}{s}-{d.name}-{o.name}-{'incl' if i else 'excl'}{'-rev' if r else ''}" for k, s, d, o, i, r in ROWS_AND_FLAT])
 def test_rows_and_flat_scans(stream, kind, shape, dtype, op, inclusive, reverse):
     rng = np.random.default_rng(41)
     n = shape[0] * shape[1]
@@ -97,11 +103,14 @@ def test_rows_and_flat_scans(stream, kind, shape, dtype, op, inclusive, reverse)
         assert "passes=scan)" in variant or "passes=scan," in variant  # rows that fit a block need no carries
 
 
-@pytest.mark.parametrize("offsets_dtype", [DataType.uint32, DataType.uint64], ids=lambda d: d.name)
-@pytest.mark.parametrize("reverse", [False, True], ids=["forward", "reverse"])
-@pytest.mark.parametrize("inclusive", [True, False], ids=["inclusive", "exclusive"])
-@pytest.mark.parametrize("op", [ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.arg_min, ScanOp.arg_max], ids=lambda o: o.name)
-@pytest.mark.parametrize("dtype", [DataType.uint32, DataType.fp32, DataType.bf16], ids=lambda d: d.name)
+# every (dtype, operation) with two of the four (inclusive, reverse) combinations - opposite ones - one per width of the offsets
+OFFSET_SEGMENTED = [(d, o, *SCAN_MODES[(j + m + 2 * w) % 4], (DataType.uint32, DataType.uint64)[(w + j) % 2])
+                    for j, d in enumerate([DataType.uint32, DataType.fp32, DataType.bf16])
+                    for m, o in enumerate([ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.arg_min, ScanOp.arg_max]) for w in range(2)]
+
+
+@pytest.mark.parametrize("dtype,op,inclusive,reverse,offsets_dtype", OFFSET_SEGMENTED,
+                         ids=[f"{d.name}-{o.name}-{'incl' if i else 'excl'}{'-rev' if r else ''}-off_{w.name}" for d, o, i, r, w in OFFSET_SEGMENTED])
 def test_offset_segmented_scans(stream, dtype, op, inclusive, reverse, offsets_dtype):
     rng = np.random.default_rng(43)
     n = 60000
@@ -162,10 +171,13 @@ def test_validation(stream):
         ph.scan(x, gpu_tensor([64], DataType.fp32), stream, segment_offsets=copy_numpy_to_gpu(np.zeros(3, np.float32), stream, DataType.fp32))
 
 
-@pytest.mark.parametrize("reverse", [False, True], ids=["forward", "reverse"])
-@pytest.mark.parametrize("dtype,op", [(DataType.uint32, ScanOp.sum), (DataType.fp32, ScanOp.min), (DataType.bf16, ScanOp.arg_max),
-                                      (DataType.fp32, ScanOp.sum)], ids=["u32-sum", "fp32-min", "bf16-argmax", "fp32-sum"])
-@pytest.mark.parametrize("n,segments", [(16_800_001, 0), (16_800_001, 3), (1_000_000, 2000)], ids=["flat-4102-chunks", "3-segments", "2000-segments"])
+PUBLISHED = [  # (n, segments, dtype, op, reverse): every level of totals, every class of operation, both directions
+    (16_800_001, 0, DataType.uint32, ScanOp.sum, False), (16_800_001, 0, DataType.fp32, ScanOp.sum, True), (16_800_001, 3, DataType.fp32, ScanOp.min, False),
+    (16_800_001, 3, DataType.bf16, ScanOp.arg_max, True), (1_000_000, 2000, DataType.uint32, ScanOp.sum, True),
+    (1_000_000, 2000, DataType.fp32, ScanOp.sum, False), (1_000_000, 2000, DataType.bf16, ScanOp.arg_max, False), (1_000_000, 0, DataType.fp32, ScanOp.min, True)]
+
+
+@pytest.mark.parametrize("n,segments,dtype,op,reverse", PUBLISHED, ids=[f"{n}-{s}seg-{d.name}-{o.name}{'-rev' if r else ''}" for n, s, d, o, r in PUBLISHED])
 def test_published_totals_agree_with_separate_passes(stream, monkeypatch, n, segments, dtype, op, reverse):
     """Chunks that read what precedes them from the totals other blocks publish (one launch over the data) against the same
     scan with totals and carries computed by launches of their own: the same bits for exact operations; float sums agree with
@@ -216,15 +228,39 @@ def test_rows_longer_than_a_chunk_at_a_size_that_takes_the_large_blocks(stream, 
     check(got, carrier, dtype, op, inclusive, reverse, segment_size=length)
 
 
-def test_a_wait_that_gives_up_is_reported(stream, monkeypatch):
-    """Waits between blocks are bounded so that every wavefront has an exit.  With the bound forced to zero polls a chunk that
-    needs a total gives up at once (every kernel still runs to its end), and thor_scan reports that instead of handing back
-    incomplete results; the same scan with the ordinary bound is exact."""
-    x = np.ones(1 << 22, np.uint32)
+def test_a_wait_that_gives_up_works_its_totals_out_again(stream, monkeypatch):
+    """Waits between blocks are bounded so that every wavefront has an exit.  With the bound forced to zero polls every chunk
+    that needs the total of an earlier one gives up at once and works that total out from the input, in the order its owner
+    would have: flat, ragged and float-sum scans return the bits of the ordinary run, through thor_scan and through the Scan
+    stage of a stamped Expression, and thor_scan counts the waits that took the way out."""
+    rng = np.random.default_rng(59)
+    ones = np.ones(1 << 22, np.uint32)
+    noisy = rng.standard_normal(1_300_003).astype(np.float32)      # odd length: single elements, 318 chunks, five groups
+    cuts = np.sort(rng.integers(0, noisy.size, 99))
+    offsets = np.concatenate([[0], cuts, [noisy.size]])
+    rows = rng.integers(0, 1 << 32, (3, 70_001), dtype=np.uint64).astype(np.uint32)
+    ordinary = {
+        "flat": run_scan(ones, DataType.uint32, stream, ScanOp.sum, True, False),
+        "float": run_scan(noisy, DataType.fp32, stream, ScanOp.sum, False, True),
+        "ragged": run_scan(noisy, DataType.fp32, stream, ScanOp.arg_max, True, False, offsets=offsets),
+    }
+    for got, variant in ordinary.values():
+        assert "published_totals" in variant, variant
+    np.testing.assert_array_equal(ordinary["flat"][0], np.arange(1, ones.size + 1, dtype=np.uint32))
+    before = ph.scan_waits_recovered()
     monkeypatch.setenv("THOR_SCAN_WAIT_LIMIT", "0")
-    with pytest.raises(RuntimeError, match="gave up"):
-        run_scan(x, DataType.uint32, stream, ScanOp.sum, True, False)
-    monkeypatch.delenv("THOR_SCAN_WAIT_LIMIT")
-    got, variant = run_scan(x, DataType.uint32, stream, ScanOp.sum, True, False)
-    assert "published_totals" in variant, variant
-    np.testing.assert_array_equal(got, np.arange(1, x.size + 1, dtype=np.uint32))
+    recovered = {
+        "flat": run_scan(ones, DataType.uint32, stream, ScanOp.sum, True, False),
+        "float": run_scan(noisy, DataType.fp32, stream, ScanOp.sum, False, True),
+        "ragged": run_scan(noisy, DataType.fp32, stream, ScanOp.arg_max, True, False, offsets=offsets),
+    }
+    assert ph.scan_waits_recovered() >= before + 3 * 100  # nearly every chunk waits for an earlier one of its group
+    for name, (got, variant) in recovered.items():
+        assert "published_totals" in variant, variant
+        np.testing.assert_array_equal(got.view(np.uint32), ordinary[name][0].view(np.uint32), err_msg=name)
+    # the Scan stage of a stamped Expression: rows longer than a chunk, so chunks inside a row read earlier totals
+    x = copy_numpy_to_gpu(rows, stream, DataType.uint32)
+    plan = ph.Expression.compile(ph.Expression.input("x").scan(ScanOp.sum), 0).stamp({"x": x}, stream)
+    assert plan.stage_kind_names() == ["Scan"]
+    plan.run()
+    np.testing.assert_array_equal(copy_gpu_to_numpy(plan.output(), stream), np.cumsum(rows, axis=1, dtype=np.uint32))

@@ -47,8 +47,12 @@ def partitions(rng, rows, segments):
 CASES = [((5000,), 37), ((4096, 8), 19), ((777, 3, 5), 12), ((300, 1024), 7), ((100000, 2), 5000), ((70000, 3), 1), ((200000,), 90000), ((33, 4099), 9)]
 
 
-@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16, DataType.fp16, DataType.fp8_e4m3, DataType.fp8_e5m2], ids=lambda d: d.name)
-@pytest.mark.parametrize("shape,segments", CASES, ids=[f"{s}-{b}" for s, b in CASES])
+# every shape in fp32 and in one narrower dtype (the four take turns down the list: each meets two shapes)
+NARROW = (DataType.bf16, DataType.fp16, DataType.fp8_e4m3, DataType.fp8_e5m2)
+BROADCAST_CASES = [(s, b, d) for i, (s, b) in enumerate(CASES) for d in (DataType.fp32, NARROW[i % 4])]
+
+
+@pytest.mark.parametrize("shape,segments,dtype", BROADCAST_CASES, ids=[f"{s}-{b}-{d.name}" for s, b, d in BROADCAST_CASES])
 def test_broadcast_matches_a_loop_over_segments(stream, shape, segments, dtype):
     rng = np.random.default_rng(len(shape) * 1000 + segments)
     per_segment_shape = (segments,) + shape[1:]
@@ -60,6 +64,8 @@ def test_broadcast_matches_a_loop_over_segments(stream, shape, segments, dtype):
             carrier = offsets.astype(np.uint64 if offsets_dtype == DataType.uint64 else np.uint32)
             toff = copy_numpy_to_gpu(carrier, stream, offsets_dtype)
             for normalize in (False, True):
+                if offsets_dtype == DataType.uint64 and not normalize:
+                    continue  # the offsets' width only changes how the partition is read
                 filler = to_storage(np.full(shape, 77.0, np.float32), dtype)
                 out = copy_numpy_to_gpu(filler, stream, dtype)
                 ph.segmented_broadcast(tv, toff, out, normalize, stream)

@@ -93,8 +93,11 @@ def ragged_offsets(rng, rows, segments):
 SHAPES = [((5000,), 37), ((4096, 8), 19), ((777, 3, 5), 12), ((300, 1024), 7), ((100000, 2), 5), ((64, 4099), 9), ((200000,), 1)]
 
 
-@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.bf16, DataType.fp16, DataType.fp8_e4m3], ids=lambda d: d.name)
-@pytest.mark.parametrize("shape,segments", SHAPES, ids=[f"{s}-{b}" for s, b in SHAPES])
+# every shape in fp32 and in one narrower dtype (bf16, fp16 and fp8 take turns down the list)
+RAGGED_CASES = [(s, b, d) for i, (s, b) in enumerate(SHAPES) for d in (DataType.fp32, (DataType.bf16, DataType.fp16, DataType.fp8_e4m3)[i % 3])]
+
+
+@pytest.mark.parametrize("shape,segments,dtype", RAGGED_CASES, ids=[f"{s}-{b}-{d.name}" for s, b, d in RAGGED_CASES])
 def test_random_ragged_partitions_against_numpy(stream, shape, segments, dtype):
     rng = np.random.default_rng(hash((shape, segments)) % 2**32)
     x = to_storage(rng.standard_normal(shape).astype(np.float32), dtype)
@@ -138,13 +141,15 @@ def awkward_offsets(rows):
     return np.array(cuts + [min(rows, 2900)] * 3, dtype=np.int64)
 
 
-SEGMENT_KERNELS = [("teams", {}), ("rows", {}), ("rows", {"THOR_SEGMENT_THREADS": "64"}),
-                   ("rows", {"THOR_SEGMENT_GROUP": "16", "THOR_SEGMENT_BATCH": "8"}), ("rows", {"THOR_SEGMENT_GROUP": "2", "THOR_SEGMENT_THREADS": "128"})]
+AWKWARD_SHAPES = [((3000, 64), DataType.fp32), ((3000, 200), DataType.fp16), ((2100, 3), DataType.fp32), ((3000, 512), DataType.bf16)]
+# both kernels over every shape; the other block sizes and walking groups of the by-rows kernel over one shape each
+SEGMENT_KERNELS = [(k, {}, s, d) for k in ("teams", "rows") for s, d in AWKWARD_SHAPES] + [
+    ("rows", {"THOR_SEGMENT_THREADS": "64"}, *AWKWARD_SHAPES[0]), ("rows", {"THOR_SEGMENT_GROUP": "16", "THOR_SEGMENT_BATCH": "8"}, *AWKWARD_SHAPES[1]),
+    ("rows", {"THOR_SEGMENT_GROUP": "2", "THOR_SEGMENT_THREADS": "128"}, *AWKWARD_SHAPES[3])]
 
 
-@pytest.mark.parametrize("kernel,switches", SEGMENT_KERNELS, ids=[k + "".join(f"-{n[13:].lower()}{v}" for n, v in e.items()) for k, e in SEGMENT_KERNELS])
-@pytest.mark.parametrize("shape,dtype", [((3000, 64), DataType.fp32), ((3000, 200), DataType.fp16), ((2100, 3), DataType.fp32), ((3000, 512), DataType.bf16)],
-                         ids=["3000x64-fp32", "3000x200-fp16", "2100x3-fp32", "3000x512-bf16"])
+@pytest.mark.parametrize("kernel,switches,shape,dtype", SEGMENT_KERNELS,
+                         ids=[f"{k}" + "".join(f"-{n[13:].lower()}{v}" for n, v in e.items()) + f"-{s[0]}x{s[1]}-{d.name}" for k, e, s, d in SEGMENT_KERNELS])
 def test_both_segment_kernels_on_awkward_partitions(stream, monkeypatch, kernel, switches, shape, dtype):
     """The planner picks between two kernels (segments dealt out to teams of lanes, rows dealt out to lanes) by the shape; the
     tuning switches force each of them, and other block sizes and walking groups, on the same partitions."""
@@ -160,7 +165,10 @@ def test_both_segment_kernels_on_awkward_partitions(stream, monkeypatch, kernel,
     for offsets_dtype in (DataType.uint32, DataType.uint64):
         toff = upload_offsets(offsets, stream, offsets_dtype)
         lengths = np.diff(offsets).reshape(-1, 1)
+        wide = offsets_dtype == DataType.uint64  # 64-bit offsets change how the partition is read, not what is folded: two operations
         for name, op in VALUE_OPS.items():
+            if wide and name != "Mean":
+                continue
             stamped = ph.CubSegmentedReduction(op, DataType.fp32).stamp(tx, toff, stream)
             assert ("by_rows" if kernel == "rows" else "by_teams") in stamped.get_kernel_variant()
             stamped.run()
@@ -173,6 +181,8 @@ def test_both_segment_kernels_on_awkward_partitions(stream, monkeypatch, kernel,
                 assert np.array_equal(np.isnan(got), np.isnan(want)), f"{name} {stamped.get_kernel_variant()}"
                 assert np.all(np.isnan(want) | (np.abs(got - want) <= 1e-5 * absolute + 1e-30)), f"{name} {stamped.get_kernel_variant()}"
         for name, op in ARG_OPS.items():
+            if wide and name != "ArgMax":
+                continue
             stamped = ph.CubSegmentedArgReduction(op).stamp(tx, toff, stream)
             stamped.run()
             got = copy_gpu_to_numpy(stamped.get_index_output_tensor(), stream).reshape(len(offsets) - 1, shape[1])
@@ -185,7 +195,7 @@ def test_both_segment_kernels_on_awkward_partitions(stream, monkeypatch, kernel,
                     np.testing.assert_array_equal(got[b], (offsets[b] + winner) * shape[1] + np.arange(shape[1]), err_msg=f"{name} segment {b} {stamped.get_kernel_variant()}")
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", range(6))
 def test_random_partitions_give_the_same_answer_through_both_kernels(stream, monkeypatch, seed):
     """Random partitions with many empty and one-row segments, rows of 1 to 260 elements: maxima and winners must agree bit for
     bit between the two segment kernels and with numpy, sums within the accumulation-order tolerance."""
@@ -321,6 +331,8 @@ def test_segments_that_begin_and_end_on_block_boundaries(stream, shape):
         offsets = np.array(partition, dtype=np.int64)
         toff = upload_offsets(offsets, stream, DataType.uint64)
         for name, op in VALUE_OPS.items():
+            if name == "Min":
+                continue
             stamped = ph.CubSegmentedReduction(op, DataType.fp32).stamp(tx, toff, stream)
             stamped.run()
             got = gpu_to_f32(stamped.get_output_tensor(), stream).astype(np.float64)
@@ -334,6 +346,8 @@ def test_segments_that_begin_and_end_on_block_boundaries(stream, shape):
                 assert np.all(np.abs(got - want) <= 1e-5 * scale + 1e-30), f"{name} {partition}"
         flat = x.reshape(n, trailing)
         for name, op in ARG_OPS.items():
+            if name == "ArgMax":
+                continue
             stamped = ph.CubSegmentedArgReduction(op, DataType.uint32).stamp(tx, toff, stream)
             stamped.run()
             got = copy_gpu_to_numpy(stamped.get_index_output_tensor(), stream).reshape(len(offsets) - 1, trailing)

@@ -78,8 +78,14 @@ def test_select_reference_vectors(stream, case):
     np.testing.assert_array_equal(bits_of(got[:count]), bits_of(carriers(case["expected"], dtype)))
 
 
-@pytest.mark.parametrize("dtype", KEY_DTYPES, ids=lambda d: d.name)
-@pytest.mark.parametrize("n", [1, 63, 4095, 4096, 4097, 1_000_003])
+# elements are copied as raw words: one dtype of each width meets every length, the other dtypes two lengths each
+SELECT_LENGTHS = [1, 63, 4095, 4096, 4097, 1_000_003]
+SELECT_CASES = [(d, n) for d in (DataType.uint8, DataType.bf16, DataType.fp32) for n in SELECT_LENGTHS]
+SELECT_CASES += [(d, SELECT_LENGTHS[(2 * i + j) % 6]) for i, d in enumerate(d for d in KEY_DTYPES if d not in (DataType.uint8, DataType.bf16, DataType.fp32))
+                 for j in (0, 3)]
+
+
+@pytest.mark.parametrize("dtype,n", SELECT_CASES, ids=[f"{d.name}-{n}" for d, n in SELECT_CASES])
 def test_select_keeps_the_flagged_elements_in_order(stream, dtype, n):
     rng = np.random.default_rng(n * 31 + int(dtype))
     values = random_keys(rng, n, dtype)
@@ -195,9 +201,12 @@ def test_top_k_reference_vectors(stream, case):
         assert pairs == sorted(zip(bits_of(expected.reshape(-1)).tolist(), case["expected_values"]))
 
 
-@pytest.mark.parametrize("dtype", KEY_DTYPES, ids=lambda d: d.name)
-@pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
-@pytest.mark.parametrize("n,k", [(1, 1), (257, 256), (2049, 2049), (100_003, 1), (100_003, 1000), (1_000_000, 65_537)])
+# every key dtype meets every (n, k); the order alternates so that every dtype and every (n, k) sees both
+TOPK_SIZES = [(1, 1), (257, 256), (2049, 2049), (100_003, 1), (100_003, 1000), (1_000_000, 65_537)]
+TOPK_KEY_CASES = [(d, (i + j) % 2 == 0, n, k) for i, d in enumerate(KEY_DTYPES) for j, (n, k) in enumerate(TOPK_SIZES)]
+
+
+@pytest.mark.parametrize("dtype,largest,n,k", TOPK_KEY_CASES, ids=[f"{d.name}-{'largest' if l else 'smallest'}-{n}-{k}" for d, l, n, k in TOPK_KEY_CASES])
 def test_top_k_keys(stream, dtype, largest, n, k):
     rng = np.random.default_rng(n * 7 + k + int(dtype))
     keys = random_keys(rng, n, dtype)
@@ -216,9 +225,13 @@ def test_top_k_pairs_with_many_equal_keys(stream, dtype, largest):
         check_top_k(keys, dtype, k, largest, got, got_values)
 
 
-@pytest.mark.parametrize("dtype", [d for d in KEY_DTYPES if d not in (DataType.uint8, DataType.int8)], ids=lambda d: d.name)
-@pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
-@pytest.mark.parametrize("region", [None, "1"], ids=["roomy", "overflowing"])
+# the key kinds of two and four bytes (unsigned, signed, float), each with roomy and with overflowing regions, orders alternating
+CANDIDATE_CASES = [(d, (i + j) % 2 == 0, r) for i, d in enumerate([DataType.uint16, DataType.int32, DataType.bf16, DataType.fp32, DataType.fp16])
+                   for j, r in enumerate([None, "1"])]
+
+
+@pytest.mark.parametrize("dtype,largest,region", CANDIDATE_CASES,
+                         ids=[f"{d.name}-{'largest' if l else 'smallest'}-{'overflowing' if r else 'roomy'}" for d, l, r in CANDIDATE_CASES])
 def test_top_k_over_candidates(stream, monkeypatch, dtype, largest, region):
     """Long inputs copy the keys at or above a floor taken from a sample (the keys that can still be part of the answer) during
     the one pass over the input and finish on those candidates; the switch asks for that on short inputs and large k too.  With one entry per wavefront the candidate regions overflow and the passes over
@@ -227,13 +240,14 @@ def test_top_k_over_candidates(stream, monkeypatch, dtype, largest, region):
     if region:
         monkeypatch.setenv("THOR_TOPK_REGION", region)
     rng = np.random.default_rng(int(dtype) * 3 + largest)
-    for n, k, levels in ((100_003, 1, None), (100_003, 1000, None), (300_001, 4_000, 20), (300_001, 250_000, 20), (65_536, 65_536, None)):
+    for index, (n, k, levels) in enumerate(((100_003, 1, None), (100_003, 1000, None), (300_001, 4_000, 20), (300_001, 250_000, 20), (65_536, 65_536, None))):
         keys = random_keys(rng, n, dtype, distinct_levels=levels)
         got, got_values, variant = run_top_k(keys, dtype, k, largest, stream, pairs=True)
         assert "candidates(" in variant
         check_top_k(keys, dtype, k, largest, got, got_values)
-        got, _, _ = run_top_k(keys, dtype, k, largest, stream)
-        check_top_k(keys, dtype, k, largest, got, None)
+        if index in (1, 3):  # the key-only kernels are the pair kernels without the positions: two of the five sizes
+            got, _, _ = run_top_k(keys, dtype, k, largest, stream)
+            check_top_k(keys, dtype, k, largest, got, None)
 
 
 def test_top_k_long_inputs_use_candidates_by_default(stream):
@@ -277,22 +291,68 @@ def test_top_k_zero_k_leaves_the_output_alone(stream):
     np.testing.assert_array_equal(copy_gpu_to_numpy(out, stream), 99)
 
 
-@pytest.mark.parametrize("dtype", KEY_DTYPES, ids=lambda d: d.name)
-@pytest.mark.parametrize("largest", [True, False], ids=["largest", "smallest"])
-@pytest.mark.parametrize("segments,segment_size,k", [(1, 2, 1), (33, 257, 256), (100, 1000, 10), (16, 8192, 8191), (3000, 64, 8)])
+# Rows a wavefront can hold (at most 64 keys per lane) take the kernel with one wavefront per row: a bit-by-bit search over the
+# keys in registers, or - when at most 64 keys are wanted and every lane holds two groups of vectors - over the few keys at or
+# above a floor taken from the groups' maxima ("floor-candidates"); longer rows take one block per row.  Every key dtype meets every shape, the
+# order alternating: rows of two keys, rows no vector divides, almost all keys wanted, rows of one vector per lane, full rows of
+# 4096, the longest rows, many short rows.
+ROW_SHAPES = [(1, 2, 1), (33, 257, 256), (100, 1000, 10), (37, 4096, 64), (6, 8192, 8191), (3000, 64, 8), (50, 3000, 3)]
+ROW_CASES = [(d, (i + j) % 2 == 0, *shape) for i, d in enumerate(KEY_DTYPES) for j, shape in enumerate(ROW_SHAPES)]
+
+
+def row_kernel_form(dtype, segment_size, k):
+    """What the variant text of a row top-k says about the kernel the planner must have chosen."""
+    vec = 16 // np.dtype(numpy_carrier(dtype)).itemsize
+    vectors_per_lane = -(-segment_size // (64 * vec))
+    if vectors_per_lane * vec > 64:
+        return "block-per-row"
+    floor = k <= 64 and vectors_per_lane % 2 == 0 and segment_size >= 32 * vec * vectors_per_lane and vectors_per_lane * vec > 16
+    return "wavefront-per-row" + (" floor-candidates" if floor else "")
+
+
+@pytest.mark.parametrize("dtype,largest,segments,segment_size,k", ROW_CASES,
+                         ids=[f"{d.name}-{'largest' if l else 'smallest'}-{s}x{n}-k{k}" for d, l, s, n, k in ROW_CASES])
 def test_top_k_of_rows(stream, dtype, largest, segments, segment_size, k):
     rng = np.random.default_rng(segments * 13 + segment_size + k + int(dtype))
     keys = random_keys(rng, segments * segment_size, dtype)
     got, got_values, variant = run_top_k(keys, dtype, k, largest, stream, pairs=True, segment_size=segment_size)
-    assert "row top-k" in variant
+    form = row_kernel_form(dtype, segment_size, k)
+    assert "row top-k" in variant and form.split()[0] in variant and ("floor-candidates" in variant) == ("floor-candidates" in form), variant
     check_top_k(keys, dtype, k, largest, got, got_values, segment_size=segment_size)
 
 
-def test_top_k_of_rows_keys_only_with_ties(stream):
+@pytest.mark.parametrize("dtype,segment_size,k,levels", [(DataType.bf16, 300, 100, 6), (DataType.bf16, 4096, 64, 6), (DataType.fp32, 2048, 33, 3),
+                                                         (DataType.uint8, 4096, 5, None), (DataType.int16, 1536, 64, 40)],
+                         ids=["bf16-300-k100", "bf16-4096-k64", "fp32-2048-k33", "uint8-4096-k5", "int16-1536-k64"])
+def test_top_k_of_rows_keys_only_with_ties(stream, dtype, segment_size, k, levels):
+    """Few distinct keys: the threshold key is shared by many, and with a floor most of a row lies at or above it - more
+    candidates than a wavefront's part of LDS holds, so those rows finish with the search over all keys.  One row is a single
+    repeated key, one holds the extremes of the order."""
     rng = np.random.default_rng(77)
-    keys = random_keys(rng, 512 * 300, DataType.bf16, distinct_levels=6)
-    got, _, _ = run_top_k(keys, DataType.bf16, 100, True, stream, segment_size=300)
-    check_top_k(keys, DataType.bf16, 100, True, got, None, segment_size=300)
+    rows = 96
+    keys = random_keys(rng, rows * segment_size, dtype, distinct_levels=levels).reshape(rows, segment_size)
+    keys[3] = keys[3, 0]
+    if dtype in FLOATS:
+        keys[5, :7] = to_storage(np.array([np.inf, -np.inf, np.nan, 0.0, -0.0, np.inf, np.nan], np.float32), dtype)
+    for largest in (True, False):
+        got, _, variant = run_top_k(keys, dtype, k, largest, stream, segment_size=segment_size)
+        assert "wavefront-per-row" in variant, variant
+        check_top_k(keys, dtype, k, largest, got, None, segment_size=segment_size)
+
+
+def test_both_row_kernels_agree(stream, monkeypatch):
+    """The switch forces one block per row on rows a wavefront could hold: the same keys, sorted, from both kernels."""
+    rng = np.random.default_rng(78)
+    keys = random_keys(rng, 64 * 4096, DataType.fp16).reshape(64, 4096)
+    by_wavefront, values_w, variant = run_top_k(keys, DataType.fp16, 64, True, stream, pairs=True, segment_size=4096)
+    assert "wavefront-per-row" in variant and "floor-candidates" in variant, variant
+    monkeypatch.setenv("THOR_TOPK_ROW_KERNEL", "block")
+    by_block, values_b, variant = run_top_k(keys, DataType.fp16, 64, True, stream, pairs=True, segment_size=4096)
+    assert "block-per-row" in variant, variant
+    for row in range(64):
+        np.testing.assert_array_equal(sorted_by_order(by_wavefront[row], DataType.fp16, True), sorted_by_order(by_block[row], DataType.fp16, True))
+    check_top_k(keys, DataType.fp16, 64, True, by_wavefront, values_w, segment_size=4096)
+    check_top_k(keys, DataType.fp16, 64, True, by_block, values_b, segment_size=4096)
 
 
 def test_top_k_full_size_against_a_host_partition(stream):

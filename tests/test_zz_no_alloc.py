@@ -91,3 +91,16 @@ def test_refuses_requests_larger_than_the_block(stream):
     off = copy_numpy_to_gpu(np.array([0, n // 2, n], np.uint32), stream, DataType.uint32)
     with pytest.raises(Exception, match="fixed scratch block"):
         ph.scan(x, out, stream, ScanOp.sum, segment_offsets=off, no_alloc=True)
+
+
+def test_a_wait_that_gives_up_still_returns_complete_results(stream, monkeypatch):
+    """This entry point has no temporary storage of the caller's to look into afterwards, so nothing could report a wait
+    between blocks that gave up: such a wait works the totals it lacks out of the input instead.  Forced here with a bound of
+    zero polls (a kernel of its own, loaded by the allocating call first)."""
+    monkeypatch.setenv("THOR_SCAN_WAIT_LIMIT", "0")
+    rng = np.random.default_rng(10)
+    x = rng.integers(0, 1 << 20, 900_001, dtype=np.uint32)
+    want, got, variant = both(stream, x, DataType.uint32, ScanOp.sum)
+    assert "published_totals" in variant, variant
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(got, np.cumsum(x, dtype=np.uint32))

@@ -15,7 +15,9 @@
 // of its group of 64, of the earlier groups of its super-group of 64 groups, and of the earlier super-groups (the last chunk
 // of a group publishes the group's total, the last of a super-group that one's).  A block only ever waits for chunks with
 // smaller tickets, which are running or done, and the shape of the fold does not depend on who arrived when: results are
-// the same from run to run.  Every element is read once and written once.  Beyond 64^3 chunks three launches, none of which
+// the same from run to run.  Waits are bounded (kWaitLimit polls).  A block whose wait gives up finishes its chunk with what it
+// has, then - its registers free again - works the totals it lacks out of the input, in the order their owners would have, and
+// does its chunk once more: the result is the same bits whether or not a wait gave up.  Every element is read once and written once.  Beyond 64^3 chunks three launches, none of which
 // waits on another block, do the same: the kernel without stores writes each chunk's total, one block turns the totals into
 // carries, the full kernel applies them.
 //
@@ -164,9 +166,21 @@ struct ScanRunSum {
     static constexpr int kOp = 0;
 };
 
+// bit k set: logical position p + k starts a segment (p is a multiple of kVec)
+template <typename Cfg>
+__device__ __forceinline__ u32 scanHeadBits(const u32* heads, u64 p) {
+    constexpr int V = Cfg::kVec;
+    if (Cfg::kRow == 0) return (heads[p / 32] >> (p % 32)) & ((1u << V) - 1u);
+    if (Cfg::kRow % V == 0) return p % Cfg::kRow == 0 ? 1u : 0u;
+    u32 bits = 0;
+#pragma unroll
+    for (int k = 0; k < V; ++k) bits |= ((p + k) % Cfg::kRow == 0 ? 1u : 0u) << k;
+    return bits;
+}
+
 // ---- published totals (Cfg::kLookback) ----------------------------------------------------------------------------------------
 // The block of memory a scan with published totals works in: 32 control words of 8 bytes (word 0: the ticket counter, word 1:
-// the number of waits that gave up), then one entry of two 8-byte words per chunk, per group and per super-group.  A word
+// the number of waits that gave up and worked their totals out again), then one entry of two 8-byte words per chunk, per group and per super-group.  A word
 // holds 32 bits of state above a tag (bit 0: written, bit 1: a head lies in the summarised range); the first word carries
 // the value, the second (min / max only) the index.  Every word is written once per run, whole, after the block was
 // cleared, so a reader that sees the tag sees the state: no fences.
@@ -197,36 +211,139 @@ __device__ __forceinline__ ScanGlimpse scanGlimpse(u64* entries, u64 first, u32 
     return g;
 }
 
-// The combination, in order, of entries [first, first + count), count <= 64: called by one whole wavefront, lane l waits for
-// entry first + l (`seen`: an earlier look at the same entries, or zeros); every lane returns the result.
+// ---- totals worked out again from the input (the way out of a wait that gave up) -----------------------------------------------
+// Every published total is a function of the input alone, folded in a fixed order.  A block whose wait for an entry gave up
+// therefore computes that entry itself, with the operations and the order of the block that owes it, so the scan's result does
+// not depend on whether the wait succeeded (same bits, float sums included).  Slow (one wavefront walks whole chunks) and, while
+// blocks take chunks by ticket, never needed: it is what makes a bounded wait safe to give up.  The code runs between the two
+// passes a block then makes over its chunk, when none of the chunk is held in registers.
 template <typename Cfg>
-__device__ __forceinline__ ScanState<Cfg> scanAwait(u64* entries, u64 first, u32 count, u64* control, ScanGlimpse seen) {
+struct ScanSource {
+    const typename Cfg::T* in;
+    const u32* heads;
+};
+
+template <typename Cfg>
+__device__ __forceinline__ ScanState<Cfg> scanLastLane(const ScanState<Cfg>& s) {
+    ScanState<Cfg> all;
+    all.v = __shfl(s.v, kWave - 1, kWave);
+    all.i = (Cfg::kOp == 1 || Cfg::kOp == 2) ? __shfl(s.i, kWave - 1, kWave) : kNoIndex;
+    all.head = __shfl(s.head, kWave - 1, kWave);
+    return all;
+}
+
+// the total of chunk `chunk` as its block computes it (scanChunkCore: vectors serially, lanes, then the wavefronts' totals),
+// by one whole wavefront that plays the block's wavefronts in turn; every lane returns it
+template <typename Cfg>
+__device__ __noinline__ ScanState<Cfg> scanChunkTotalAgain(ScanSource<Cfg> src, u64 chunk) {
+    typedef typename Cfg::T T;
+    typedef ScanState<Cfg> S;
+    constexpr int V = Cfg::kVec, ITEMS = Cfg::kItems, THREADS = Cfg::kThreads, WAVES = THREADS / kWave;
+    constexpr bool kPlain = Cfg::kRow != 0 && (Cfg::kRow % ((u64)THREADS * V) == 0 || Cfg::kRow == Cfg::kTotal);
+    const int lane = threadIdx.x % kWave;
+    const u64 chunkBase = chunk * Cfg::kChunkElems;
+    S mine = scanEmpty<Cfg>();
+#pragma unroll 1
+    for (int slot = 0; slot < ITEMS * WAVES; ++slot) {
+        const int it = slot / WAVES, wave = slot % WAVES;
+        const u64 local = ((u64)it * THREADS + (u64)wave * kWave + lane) * V;
+        const u64 p = chunkBase + local;
+        const bool live = local < Cfg::kChunkElems && p < Cfg::kTotal;
+        const u64 physical = Cfg::kReverse ? Cfg::kTotal - (live ? p : 0) - V : (live ? p : 0);
+        Pack<T, V> x;
+        u32 headBits = 0;
+        if (live) {
+            x.load(src.in + physical);
+            headBits = scanHeadBits<Cfg>(src.heads, p);
+        }
+        S run = scanEmpty<Cfg>();
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            S e;
+            e.v = live ? scanLoad(x.v[Cfg::kReverse ? V - 1 - k : k]) : scanIdentity<Cfg>();
+            e.i = live ? (u32)(physical + (Cfg::kReverse ? V - 1 - k : k)) : kNoIndex;
+            e.head = (headBits >> k) & 1u;
+            run = scanCombine<Cfg>(run, e);
+        }
+        S inclusive;
+        if (kPlain) {
+            const u32 roundHead = (chunkBase + (u64)it * THREADS * V) % Cfg::kRow == 0 ? 1u : 0u;
+            inclusive = scanWave<Cfg, false>(run);
+            inclusive.head = wave == 0 ? roundHead : 0u;
+        } else {
+            inclusive = scanWave<Cfg, true>(run);
+        }
+        const S total = scanLastLane<Cfg>(inclusive);
+        if (lane == slot) mine = total;
+    }
+    return scanLastLane<Cfg>(scanWave<Cfg>(mine));
+}
+
+// LEVEL 0: the total of chunk `entry`; 1: of group `entry` (64 chunks); 2: of super-group `entry` (64 groups) - each folded
+// like scanLookBack folds what it publishes: the first 63 parts across a wavefront, then the last part
+template <typename Cfg, int LEVEL>
+__device__ __forceinline__ ScanState<Cfg> scanTotalAgain(ScanSource<Cfg> src, u64 entry) {
+    typedef ScanState<Cfg> S;
+    if constexpr (LEVEL == 0) {
+        return scanChunkTotalAgain<Cfg>(src, entry);
+    } else {
+        const u32 lane = threadIdx.x % kWave;
+        S mine = scanEmpty<Cfg>();
+#pragma unroll 1
+        for (u32 part = 0; part < 63; ++part) {
+            const S t = scanTotalAgain<Cfg, LEVEL - 1>(src, entry * 64 + part);
+            if (lane == part) mine = t;
+        }
+        const S before = scanLastLane<Cfg>(scanWave<Cfg>(mine));
+        return scanCombine<Cfg>(before, scanTotalAgain<Cfg, LEVEL - 1>(src, entry * 64 + 63));
+    }
+}
+
+// The combination, in order, of entries [first, first + count), count <= 64, of level LEVEL: called by one whole wavefront,
+// lane l waits for entry first + l (`seen`: an earlier look at the same entries, or zeros); every lane returns the result.
+// RECOVER false: polls until every entry is there; after kWaitLimit polls the wait gives up: `gaveUp` is set (in every lane) and
+// the result means nothing.  RECOVER true: one look, and the entries that are not there are computed from the input.
+template <typename Cfg, int LEVEL, bool RECOVER>
+__device__ __forceinline__ ScanState<Cfg> scanAwait(u64* entries, u64 first, u32 count, u64* control, ScanGlimpse seen, ScanSource<Cfg> src,
+                                                    bool& gaveUp) {
     typedef ScanState<Cfg> S;
     constexpr bool kIndexed = Cfg::kOp == 1 || Cfg::kOp == 2;
     const u32 lane = threadIdx.x % kWave;
     const bool mine = lane < count;
-    for (u32 polls = 0;; ++polls) {
+    if constexpr (RECOVER) {
+        seen = scanGlimpse<Cfg>(entries, first, count);
         const bool ready = !mine || ((seen.w0 & 1u) != 0 && (!kIndexed || (seen.w1 & 1u) != 0));
-        if (__ballot(!ready) == 0) break;
-        if (polls >= Cfg::kWaitLimit) {  // polls before a wait gives up: seconds' worth, never reached while earlier tickets run
-            if (lane == 0) atomicAdd(reinterpret_cast<u32*>(control + 1), 1u);
-            break;
+        u64 missing = __ballot(!ready);
+        while (missing) {
+            const u32 l = (u32)__builtin_ctzll(missing);
+            missing &= missing - 1;
+            const S again = scanTotalAgain<Cfg, LEVEL>(src, first + l);
+            if (lane == l) {
+                const u64 tag = 1u | (again.head ? 2u : 0u);
+                seen.w0 = ((u64)__builtin_bit_cast(u32, again.v) << 32) | tag;
+                seen.w1 = ((u64)again.i << 32) | tag;
+            }
         }
-        if (polls) __builtin_amdgcn_s_sleep(1);
-        if (!ready) seen = scanGlimpse<Cfg>(entries, first, count);
+    } else {
+        for (u32 polls = 0;; ++polls) {
+            const bool ready = !mine || ((seen.w0 & 1u) != 0 && (!kIndexed || (seen.w1 & 1u) != 0));
+            if (__ballot(!ready) == 0) break;
+            if (polls >= Cfg::kWaitLimit) {  // polls before a wait gives up: seconds' worth, never reached while earlier tickets run
+                if (lane == 0) atomicAdd(reinterpret_cast<u32*>(control + 1), 1u);
+                gaveUp = true;
+                return scanEmpty<Cfg>();
+            }
+            if (polls) __builtin_amdgcn_s_sleep(1);
+            if (!ready) seen = scanGlimpse<Cfg>(entries, first, count);
+        }
     }
     S s = scanEmpty<Cfg>();
-    if (mine && (seen.w0 & 1u) != 0 && (!kIndexed || (seen.w1 & 1u) != 0)) {
+    if (mine) {
         s.v = __builtin_bit_cast(typename Cfg::Acc, (u32)(seen.w0 >> 32));
         s.i = kIndexed ? (u32)(seen.w1 >> 32) : kNoIndex;
         s.head = (u32)(seen.w0 >> 1) & 1u;
     }
-    s = scanWave<Cfg>(s);
-    S all;
-    all.v = __shfl(s.v, kWave - 1, kWave);
-    all.i = kIndexed ? __shfl(s.i, kWave - 1, kWave) : kNoIndex;
-    all.head = __shfl(s.head, kWave - 1, kWave);
-    return all;
+    return scanLastLane<Cfg>(scanWave<Cfg>(s));
 }
 
 // Where chunk `chunk` sits in the tree of totals, and the arrays of the tree inside the block of memory.
@@ -264,39 +381,34 @@ __device__ __forceinline__ ScanEarlyLook<Cfg> scanLookEarly(void* block, u64 chu
 }
 
 // What precedes chunk `chunk`, given its own total (the same in every lane of the calling wavefront); publishes the totals
-// this chunk owes to later ones.
-template <typename Cfg>
-__device__ __forceinline__ ScanState<Cfg> scanLookBack(void* block, u64 chunk, const ScanState<Cfg>& total, const ScanEarlyLook<Cfg>& early) {
+// this chunk owes to later ones.  RECOVER false: the first call; when a wait gives up `gaveUp` is set, the totals not yet
+// published stay owed and the result means nothing.  RECOVER true: the call that follows such a first one: nothing is waited
+// for, what is missing is computed from the input, what is still owed is published.
+template <typename Cfg, bool RECOVER>
+__device__ __forceinline__ ScanState<Cfg> scanLookBack(void* block, u64 chunk, const ScanState<Cfg>& total, const ScanEarlyLook<Cfg>& early,
+                                                       ScanSource<Cfg> src, bool& gaveUp) {
     typedef ScanState<Cfg> S;
     const ScanPlace<Cfg> at(block, chunk);
     const u32 lane = threadIdx.x % kWave;
     const bool closesGroup = at.inGroup == 63, closesSuper = closesGroup && at.inSuper == 63;
-    if (lane == 0 && !closesGroup) scanPublish<Cfg>(at.chunkTotals, chunk, total);  // the closing chunk's own total has no reader
+    // the closing chunk's own total has no reader; a second call finds the chunk's total published by the first
+    if (!RECOVER && lane == 0 && !closesGroup) scanPublish<Cfg>(at.chunkTotals, chunk, total);
     S chunksBefore = scanEmpty<Cfg>(), groupsBefore = scanEmpty<Cfg>(), supersBefore = scanEmpty<Cfg>();
     const ScanGlimpse nothing = {0, 0};
-    if (at.inGroup > 0) chunksBefore = scanAwait<Cfg>(at.chunkTotals, chunk - at.inGroup, at.inGroup, at.control, nothing);
+    if (at.inGroup > 0) chunksBefore = scanAwait<Cfg, 0, RECOVER>(at.chunkTotals, chunk - at.inGroup, at.inGroup, at.control, nothing, src, gaveUp);
+    if (gaveUp) return chunksBefore;
     const S groupTotal = scanCombine<Cfg>(chunksBefore, total);
+    // (publishing an entry twice writes the same words twice: a first call may have come this far before a later wait gave up)
     if (closesGroup && lane == 0) scanPublish<Cfg>(at.groupTotals, at.group, groupTotal);
     // a head in what was folded so far cuts off everything earlier: no need to wait for it
     if (at.inSuper > 0 && (!chunksBefore.head || closesSuper)) {
-        groupsBefore = scanAwait<Cfg>(at.groupTotals, at.group - at.inSuper, at.inSuper, at.control, early.groups);
+        groupsBefore = scanAwait<Cfg, 1, RECOVER>(at.groupTotals, at.group - at.inSuper, at.inSuper, at.control, early.groups, src, gaveUp);
+        if (gaveUp) return groupsBefore;
     }
     if (closesSuper && lane == 0) scanPublish<Cfg>(at.superTotals, at.super, scanCombine<Cfg>(groupsBefore, groupTotal));
     const S lower = scanCombine<Cfg>(groupsBefore, chunksBefore);
-    if (at.super > 0 && !lower.head) supersBefore = scanAwait<Cfg>(at.superTotals, 0, (u32)at.super, at.control, early.supers);
+    if (at.super > 0 && !lower.head) supersBefore = scanAwait<Cfg, 2, RECOVER>(at.superTotals, 0, (u32)at.super, at.control, early.supers, src, gaveUp);
     return scanCombine<Cfg>(supersBefore, lower);
-}
-
-// bit k set: logical position p + k starts a segment (p is a multiple of kVec)
-template <typename Cfg>
-__device__ __forceinline__ u32 scanHeadBits(const u32* heads, u64 p) {
-    constexpr int V = Cfg::kVec;
-    if (Cfg::kRow == 0) return (heads[p / 32] >> (p % 32)) & ((1u << V) - 1u);
-    if (Cfg::kRow % V == 0) return p % Cfg::kRow == 0 ? 1u : 0u;
-    u32 bits = 0;
-#pragma unroll
-    for (int k = 0; k < V; ++k) bits |= ((p + k) % Cfg::kRow == 0 ? 1u : 0u) << k;
-    return bits;
 }
 
 // AGGREGATE_ONLY: write the chunk's total to `aggregates` and nothing else.  Otherwise: take the chunk's carry from
@@ -307,9 +419,17 @@ __device__ __forceinline__ u32 scanHeadBits(const u32* heads, u64 p) {
 // the element itself (after it, for an exclusive scan) and end before the next element that beats it.  So a second scan over
 // the same chunk sums `gradient` over those runs, the last position of each run puts the run's sum where the winner lies in a
 // zeroed copy of the chunk in LDS, and the copy is written out with full vectors: every element of `routed` is written once.
-template <typename Cfg, bool AGGREGATE_ONLY, bool ROUTE>
+//
+// SECOND (published totals only): the pass that follows a first pass one of whose waits gave up.  The chunk is `again[0]`, its
+// total `again[1..3]` (LDS of the block, written by the first pass); what precedes the chunk is taken from the totals that are
+// there and, for the rest, worked out of the input before the chunk is loaded; nothing is waited for.
+template <typename Cfg>
+__device__ __forceinline__ void scanChunkSecondPass(const typename Cfg::T* in, const u32* heads, const void* carries, typename Cfg::T* outValue,
+                                                 u32* outIndex, u32* again);
+
+template <typename Cfg, bool AGGREGATE_ONLY, bool ROUTE, bool SECOND = false>
 __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u32* heads, const void* carries, void* aggregates,
-                                              typename Cfg::T* outValue, u32* outIndex, const float* gradient, float* routed) {
+                                              typename Cfg::T* outValue, u32* outIndex, const float* gradient, float* routed, u32* again = nullptr) {
     typedef typename Cfg::T T;
     typedef typename Cfg::Acc Acc;
     typedef ScanState<Cfg> S;
@@ -320,17 +440,18 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     constexpr bool kLook = Cfg::kLookback && Cfg::kCarry && !AGGREGATE_ONLY && !ROUTE;
     u64 chunk = blockIdx.x;
-    if constexpr (kLook) {
+    // first pass: [0] the chunk, [1..3] its total, [4] a wait gave up; second pass: [1..3] become what precedes the chunk
+    __shared__ u32 recovery[kLook && !SECOND ? 5 : 1];
+    if constexpr (kLook && !SECOND) {
         // chunks in the order blocks start: whoever a block waits for has started before it
-        __shared__ u32 ticket;
-        if (threadIdx.x == 0) ticket = atomicAdd(static_cast<u32*>(const_cast<void*>(carries)), 1u);
+        if (threadIdx.x == 0) {
+            recovery[0] = atomicAdd(static_cast<u32*>(const_cast<void*>(carries)), 1u);
+            recovery[4] = 0;
+        }
         __syncthreads();
-        chunk = ticket;
+        chunk = recovery[0];
     }
-    ScanEarlyLook<Cfg> early = {};
-    if constexpr (kLook) {
-        if (wave == 0) early = scanLookEarly<Cfg>(const_cast<void*>(carries), chunk);
-    }
+    if constexpr (SECOND) chunk = again[0];
     const u64 chunkBase = chunk * Cfg::kChunkElems;
 
     __shared__ u32 totalValue[ITEMS * WAVES], totalIndex[ITEMS * WAVES], totalHead[ITEMS * WAVES];
@@ -344,6 +465,11 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
     __shared__ float routeTile[ROUTE ? ITEMS * THREADS * V : 1];  // indexed by the position inside the chunk
     Pack<float, V> upstream[ROUTE ? ITEMS : 1];
     u32 rowHeads[ROUTE ? ITEMS : 1];
+    u32 winners[ROUTE ? ITEMS : 1][V];  // in scan order
+    ScanEarlyLook<Cfg> early = {};
+    if constexpr (kLook && !SECOND) {
+        if (wave == 0) early = scanLookEarly<Cfg>(const_cast<void*>(carries), chunk);
+    }
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         const u64 local = ((u64)it * THREADS + threadIdx.x) * V;
@@ -413,12 +539,24 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
         } else {
             S before = scanShuffleUp<Cfg>(inclusive, 1);
             if (lane == 0) before = scanEmpty<Cfg>();
-            if constexpr (kLook) {
-                S total;
-                total.v = __shfl(inclusive.v, kWave - 1, kWave);
-                total.i = (Cfg::kOp == 1 || Cfg::kOp == 2) ? __shfl(inclusive.i, kWave - 1, kWave) : kNoIndex;
-                total.head = __shfl(inclusive.head, kWave - 1, kWave);
-                before = scanCombine<Cfg>(scanLookBack<Cfg>(const_cast<void*>(carries), chunk, total, early), before);
+            if constexpr (kLook && !SECOND) {
+                const S total = scanLastLane<Cfg>(inclusive);
+                const ScanSource<Cfg> src = {in, heads};
+                bool gaveUp = false;
+                // a wait that gave up leaves this pass with a result that means nothing: a second pass follows
+                before = scanCombine<Cfg>(scanLookBack<Cfg, false>(const_cast<void*>(carries), chunk, total, early, src, gaveUp), before);
+                if (gaveUp && lane == 0) {
+                    recovery[1] = __builtin_bit_cast(u32, total.v);
+                    recovery[2] = total.i;
+                    recovery[3] = total.head;
+                    recovery[4] = 1;
+                }
+            } else if constexpr (SECOND) {
+                S preceding;
+                preceding.v = __builtin_bit_cast(Acc, again[1]);
+                preceding.i = again[2];
+                preceding.head = again[3];
+                before = scanCombine<Cfg>(preceding, before);
             } else if (Cfg::kCarry) {
                 before = scanCombine<Cfg>(scanLoadState<Cfg>(carries, chunk), before);
             }
@@ -431,7 +569,6 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
     }
     if (AGGREGATE_ONLY) return;
     __syncthreads();
-    u32 winners[ROUTE ? ITEMS : 1][V];  // in scan order
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         if (!live[it]) continue;
@@ -458,6 +595,11 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
             if (Cfg::kWriteValue) values.storeStream(outValue + physical[it]);
             if (Cfg::kWriteIndex) indices.storeStream(outIndex + physical[it]);
         }
+    }
+    if constexpr (kLook && !SECOND) {
+        // the flag was written before the barrier above: every thread of the block reads the same value.  Nothing of the first
+        // pass is needed any more, so the call costs the ordinary pass no registers.
+        if (recovery[4] != 0) scanChunkSecondPass<Cfg>(in, heads, carries, outValue, outIndex, recovery);
     }
     if constexpr (ROUTE) {
         typedef ScanRunSum R;
@@ -548,6 +690,32 @@ __device__ __forceinline__ void scanChunkCore(const typename Cfg::T* in, const u
             out.storeStream(routed + physical[it]);
         }
     }
+}
+
+// again[1..3]: the total of chunk again[0] -> what precedes that chunk (called by the block's first wavefront)
+template <typename Cfg>
+__device__ __forceinline__ void scanPrecedingAgain(const typename Cfg::T* in, const u32* heads, const void* carries, u32* again) {
+    typedef ScanState<Cfg> S;
+    S total;
+    total.v = __builtin_bit_cast(typename Cfg::Acc, again[1]);
+    total.i = again[2];
+    total.head = again[3];
+    const ScanSource<Cfg> src = {in, heads};
+    const ScanEarlyLook<Cfg> unused = {};
+    bool never = false;
+    const S preceding = scanLookBack<Cfg, true>(const_cast<void*>(carries), again[0], total, unused, src, never);
+    if (threadIdx.x % kWave == 0) {
+        again[1] = __builtin_bit_cast(u32, preceding.v);
+        again[2] = preceding.i;
+        again[3] = preceding.head;
+    }
+}
+
+template <typename Cfg>
+__device__ __forceinline__ void scanChunkSecondPass(const typename Cfg::T* in, const u32* heads, const void* carries, typename Cfg::T* outValue,
+                                                 u32* outIndex, u32* again) {
+    if (threadIdx.x < kWave) scanPrecedingAgain<Cfg>(in, heads, carries, again);
+    scanChunkCore<Cfg, false, false, true>(in, heads, carries, nullptr, outValue, outIndex, nullptr, nullptr, again);
 }
 
 template <typename Cfg, bool AGGREGATE_ONLY>

@@ -724,4 +724,207 @@ __device__ __forceinline__ void topkRows(const typename Cfg::Raw* keys, const u3
     }
 }
 
+// ---- top-k of every row: one wavefront per row ---------------------------------------------------------------------------------------
+// Rows of at most 64 * kVec * kItems keys (kVec = 16 bytes' worth of keys, at most 64 keys per lane; the kernel above takes
+// longer rows).  A wavefront keeps its row in registers as images - lane l holds vector (it * 64 + l) of the row for every
+// it < kItems, read with 16-byte loads at whatever alignment the row has; 16-bit keys stay two to a register - and finds the
+// image of the kK-th largest key bit by bit: the largest T with count(image >= T) >= kK.  Nothing is shared between
+// wavefronts, so the kernel has no barrier; a block of kThreads / 64 wavefronts takes that many consecutive rows.  The
+// kernel is bound by instruction issue (a row of 4096 16-bit keys is 8 KiB: at the memory's rate a wavefront may spend about
+// a dozen instructions per key), so the work per key is what is designed:
+//   * Direct form: every lane counts its own keys against T (a compare and an add-with-carry per key and bit), the counts
+//     meet in a wavefront sum: kBits steps over all kVec * kItems keys of a lane.
+//   * Few keys wanted (kK <= 64, rows of at least two vectors per lane): every lane takes the maxima of the first and of the
+//     second half of its keys, and the kK-th largest of those 128 maxima is a floor: kK different keys, at least, lie at or
+//     above it.  For keys in random order that leaves about 1.4 kK candidates (for kK = 64 of 4096), which every lane pushes
+//     on a small stack of its own in LDS (entry e of lane l at word e * 64 + l: no two lanes share a bank); the bit-by-bit
+//     search and the output then run over the stacks alone.  A row that overflows a stack (many equal keys at the top, a
+//     lane that holds most of the large keys) takes the direct form.
+// Cfg additionally: kRows.  Positions inside a row: p = (it * 64 + lane) * kVec + e.
+constexpr int kTopkRowStack = 8;  // candidates per lane
+
+template <typename Cfg>
+__device__ __forceinline__ u32 topkWaveSum(u32 x) {
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) x += __shfl_xor(x, d, kWave);
+    return x;
+}
+
+typedef unsigned short topk_u16x2 __attribute__((ext_vector_type(2)));
+typedef short topk_i16x2 __attribute__((ext_vector_type(2)));
+
+// The images of the two 16-bit keys of one word, in place (see topkImage).
+template <typename Cfg>
+__device__ __forceinline__ u32 topkImagePair(u32 w) {
+    if (Cfg::kKind == 1) w ^= 0x80008000u;
+    if (Cfg::kKind == 2) {
+        const topk_i16x2 negative = __builtin_bit_cast(topk_i16x2, w) >> (short)15;  // all ones in the halves whose sign is set
+        w ^= __builtin_bit_cast(u32, negative) | 0x80008000u;
+    }
+    return Cfg::kLargest ? w : ~w;
+}
+__device__ __forceinline__ u32 topkMaxPair(u32 a, u32 b) {
+    return __builtin_bit_cast(u32, __builtin_elementwise_max(__builtin_bit_cast(topk_u16x2, a), __builtin_bit_cast(topk_u16x2, b)));
+}
+
+// Output of one row from `SLOTS` keys per lane: image(j) counts only where live(j), position(j) is the key's place in the row.
+// prefix: the image of the kK-th largest key; `remaining`: how many keys equal to it belong to the answer.
+template <typename Cfg, int SLOTS, typename Image, typename Position, typename Live>
+__device__ __forceinline__ void topkRowEmit(const Image& image, const Position& position, const Live& live, u32 prefix, u32 remaining,
+                                            const typename Cfg::Raw* rowIn, const u32* rowValuesIn, typename Cfg::Raw* rowKeys, u32* rowValues) {
+    const int lane = threadIdx.x % kWave;
+    const u64 lowerLanes = ((u64)1 << lane) - 1;
+    const u32 firstTieSlot = (u32)Cfg::kK - remaining;
+    u32 aboveAt = 0, tieAt = 0;
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) {
+        const bool isAbove = live(j) && image(j) > prefix, isTie = live(j) && image(j) == prefix;
+        const u64 aboveVotes = __builtin_amdgcn_ballot_w64(isAbove), tieVotes = __builtin_amdgcn_ballot_w64(isTie);
+        if ((aboveVotes | tieVotes) == 0) continue;
+        u32 slot = 0xffffffffu;
+        if (isAbove) slot = aboveAt + (u32)__builtin_popcountll(aboveVotes & lowerLanes);
+        if (isTie) {
+            const u32 rank = tieAt + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+            if (rank < remaining) slot = firstTieSlot + rank;
+        }
+        aboveAt += (u32)__builtin_popcountll(aboveVotes);
+        tieAt += (u32)__builtin_popcountll(tieVotes);
+        if (slot != 0xffffffffu) {
+            rowKeys[slot] = rowIn[position(j)];
+            if (Cfg::kPairs) rowValues[slot] = rowValuesIn[position(j)];
+        }
+    }
+}
+
+template <typename Cfg>
+__device__ __forceinline__ void topkRowsWave(const typename Cfg::Raw* keys, const u32* values, typename Cfg::Raw* outKeys, u32* outValues) {
+    typedef typename Cfg::Raw Raw;
+    constexpr int V = Cfg::kVec, ITEMS = Cfg::kItems, R = V * ITEMS, kWaves = Cfg::kThreads / kWave;
+    constexpr int P = Cfg::kBits == 16 ? 2 : 1;  // images per register
+    constexpr int W = R / P;
+    constexpr int E = kTopkRowStack;
+    constexpr bool kFullRows = Cfg::kSegment == (u32)(kWave * R);  // no slot lies past the row
+    // the floor wants two groups of whole vectors in every lane, all of the first group inside the row, and at most one wanted
+    // key for every two groups
+    constexpr bool kFloor = Cfg::kK <= (u64)kWave && ITEMS % 2 == 0 && Cfg::kSegment >= (u32)(kWave * R / 2) && R > 2 * E;
+    constexpr bool kWideEntries = Cfg::kBits == 32;  // an entry of a stack is (image << 16 | slot), or two words for 32-bit images
+    __shared__ u32 stackEntries[kFloor ? kWaves * (E + 1) * kWave : 1];
+    __shared__ u32 stackImages[kFloor && kWideEntries ? kWaves * (E + 1) * kWave : 1];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const u64 row = (u64)blockIdx.x * kWaves + wave;
+    if (row >= Cfg::kRows) return;  // the whole wavefront leaves; nothing in this kernel waits for it
+    const Raw* rowIn = keys + row * Cfg::kSegment;
+    const u32* rowValuesIn = Cfg::kPairs ? values + row * Cfg::kSegment : nullptr;
+    Raw* rowKeys = outKeys + row * Cfg::kK;
+    u32* rowValues = Cfg::kPairs ? outValues + row * Cfg::kK : nullptr;
+
+    const auto position = [&](int j) { return (u32)((j / V) * kWave + lane) * V + (u32)(j % V); };
+    const auto live = [&](int j) { return kFullRows || position(j) < Cfg::kSegment; };
+    u32 words[W];  // a test image is never 0: slots past the row hold 0 and count for nothing
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const u32 first = (u32)(it * kWave + lane) * V;
+        Pack<Raw, V> x;
+        const bool whole = kFullRows || first + V <= Cfg::kSegment;
+        if (whole) {
+            x.loadStreamUnaligned(rowIn + first);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e) x.v[e] = first + e < Cfg::kSegment ? rowIn[first + e] : (Raw)0;
+        }
+        if constexpr (P == 2) {
+#pragma unroll
+            for (int e = 0; e < V; e += 2) {
+                const u32 pair = (u32)x.v[e] | ((u32)x.v[e + 1] << 16);
+                u32 images = topkImagePair<Cfg>(pair);
+                if (!whole) images = (live(it * V + e) ? images & 0xffffu : 0u) | (live(it * V + e + 1) ? images & 0xffff0000u : 0u);
+                words[(it * V + e) / 2] = images;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; ++e) words[it * V + e] = live(it * V + e) ? topkImage<Cfg>(x.v[e]) : 0u;
+        }
+    }
+    const auto image = [&](int j) { return P == 2 ? (j % 2 ? words[j / 2] >> 16 : words[j / 2] & 0xffffu) : words[j]; };
+
+    if constexpr (kFloor) {
+        // the maxima of the two halves of the lane's keys
+        u32 group[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            u32 best = words[t * (W / 2)];
+#pragma unroll
+            for (int w = 1; w < W / 2; ++w) {
+                const u32 other = words[t * (W / 2) + w];
+                best = P == 2 ? topkMaxPair(best, other) : (other > best ? other : best);
+            }
+            if (P == 2) best = (best >> 16) > (best & 0xffffu) ? best >> 16 : best & 0xffffu;
+            group[t] = best;
+        }
+        // the kK-th largest of the 128 maxima (0 when fewer than kK groups hold a key: then every key is a candidate)
+        u32 floorImage = 0;
+#pragma unroll 1
+        for (int bit = Cfg::kBits - 1; bit >= 0; --bit) {
+            const u32 test = floorImage | (1u << bit);
+            const u32 count = (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(group[0] >= test)) +
+                              (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(group[1] >= test));
+            if (count >= (u32)Cfg::kK) floorImage = test;
+        }
+        // every lane pushes its candidates on its own stack; pushes beyond the stack's height land in one more, unused, row
+        u32* entries = stackEntries + wave * (E + 1) * kWave + lane;
+        u32* wideImages = stackImages + (kWideEntries ? wave * (E + 1) * kWave + lane : 0);
+        u32 height = 0;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            if (live(j) && image(j) >= floorImage) {
+                const u32 at = (height < (u32)E ? height : (u32)E) * kWave;
+                entries[at] = kWideEntries ? (u32)j : (image(j) << 16) | (u32)j;
+                if (kWideEntries) wideImages[at] = image(j);
+                ++height;
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(height > (u32)E) == 0) {
+            u32 cImage[E], cSlot[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const u32 entry = (u32)e < height ? entries[e * kWave] : 0u;
+                cImage[e] = kWideEntries ? ((u32)e < height ? wideImages[e * kWave] : 0u) : entry >> 16;
+                cSlot[e] = entry & 0xffffu;
+            }
+            u32 prefix = 0;
+#pragma unroll 1
+            for (int bit = Cfg::kBits - 1; bit >= 0; --bit) {
+                const u32 test = prefix | (1u << bit);
+                u32 count = 0;
+#pragma unroll
+                for (int e = 0; e < E; ++e) count += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(cImage[e] >= test));
+                if (count >= (u32)Cfg::kK) prefix = test;
+            }
+            const auto cLive = [&](int e) { return (u32)e < height; };
+            u32 above = 0;
+#pragma unroll
+            for (int e = 0; e < E; ++e) above += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(cLive(e) && cImage[e] > prefix));
+            topkRowEmit<Cfg, E>([&](int e) { return cImage[e]; },
+                                [&](int e) { return ((cSlot[e] / (u32)V) * kWave + (u32)lane) * (u32)V + cSlot[e] % (u32)V; }, cLive, prefix,
+                                (u32)Cfg::kK - above, rowIn, rowValuesIn, rowKeys, rowValues);
+            return;
+        }
+    }
+
+    u32 prefix = 0;
+#pragma unroll 1
+    for (int bit = Cfg::kBits - 1; bit >= 0; --bit) {
+        const u32 test = prefix | (1u << bit);
+        u32 mine = 0;
+#pragma unroll
+        for (int j = 0; j < R; ++j) mine += image(j) >= test ? 1u : 0u;
+        if (topkWaveSum<Cfg>(mine) >= (u32)Cfg::kK) prefix = test;
+    }
+    u32 mineAbove = 0;
+#pragma unroll
+    for (int j = 0; j < R; ++j) mineAbove += live(j) && image(j) > prefix ? 1u : 0u;
+    const u32 above = topkWaveSum<Cfg>(mineAbove);
+    topkRowEmit<Cfg, R>(image, position, live, prefix, (u32)Cfg::kK - above, rowIn, rowValuesIn, rowKeys, rowValues);
+}
+
 }  // namespace thor

@@ -10,6 +10,7 @@
 #include "thorhip_numeric_embed.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <numeric>
 #include <sstream>
@@ -96,7 +97,7 @@ ScanChunking chooseScanChunking(const ScanRequest& r) {
 void writeScanTraits(std::ostringstream& s, const ScanRequest& r, bool isUnsigned, uint64_t threads, uint64_t vec, uint64_t items, uint64_t chunkElems,
                      const CubScanKernels& k) {
     // Waits between blocks are bounded so that every wavefront has an exit: 2^22 polls are seconds.  The test switch makes the
-    // bound so small that waits give up, to exercise how that is reported (the kernels still run to their end).
+    // bound so small that waits give up, to exercise the way out: the wavefront works the missing totals out from the input.
     unsigned long waitLimit = 1ul << 22;
     if (const char* env = std::getenv("THOR_SCAN_WAIT_LIMIT")) waitLimit = std::min<unsigned long>(std::strtoul(env, nullptr, 10), 1ul << 30);
     s << "namespace gen {\nstruct Cfg {\n    typedef " << scanStorageName(r.dtype) << " T;\n    typedef " << (isUnsigned ? "thor::u32" : "float")
@@ -260,7 +261,12 @@ void launchScan(const CubScanKernels& k, const void* input, const void* offsets,
     k.mainKernel->launch(static_cast<uint32_t>(k.chunks), 1, 1, k.threads, raw, mainArgs);
 }
 
-uint32_t scanWaitsGivenUp(const CubScanKernels& k, const void* temp, Stream& stream) {
+namespace {
+std::atomic<uint64_t> gWaitsRecovered{0};
+}
+uint64_t scanWaitsRecoveredTotal() { return gWaitsRecovered.load(); }
+
+uint32_t scanWaitsRecovered(const CubScanKernels& k, const void* temp, Stream& stream) {
     if (!k.lookback || temp == nullptr) return 0;
     ScopedGpu scoped(k.request.deviceNum);
     uint32_t count = 0;
@@ -269,6 +275,7 @@ uint32_t scanWaitsGivenUp(const CubScanKernels& k, const void* temp, Stream& str
     if (thorhip_memcpy_async(&count, word, sizeof count, THORHIP_D2H, stream.getStream()) != 0 || thorhip_stream_synchronize(stream.getStream()) != 0) {
         throw std::runtime_error(std::string("CUB scan: reading the wait counter failed: ") + thorhip_last_error());
     }
+    gWaitsRecovered += count;
     return count;
 }
 
@@ -299,6 +306,10 @@ void StampedScan::runOn(Stream& stream) const {
 std::string StampedScan::getKernelVariant() const { return kernels->variant; }
 
 std::string cubScanKernelVariant(const std::shared_ptr<const CubScanKernels>& kernels) { return kernels ? kernels->variant : std::string(); }
+uint32_t cubScanWaitsRecovered(const std::shared_ptr<const CubScanKernels>& kernels, const Tensor& temp, Stream& stream) {
+    if (!kernels || !temp.isInitialized()) return 0;
+    return scanWaitsRecovered(*kernels, const_cast<Tensor&>(temp).getMemPtr(), stream);
+}
 
 // ---- the reference's plan / run entry points ----------------------------------------------------------------------------------
 namespace {

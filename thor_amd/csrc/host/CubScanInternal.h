@@ -53,10 +53,13 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& reques
 void launchScan(const CubScanKernels& kernels, const void* input, const void* offsets, void* temp, size_t tempBytes, void* outValue, void* outIndex,
                 Stream& stream);
 
-// How many waits of the last launch on `temp` gave up (scans that publish totals between blocks bound every wait so that
-// each wavefront has an exit; a wait that gives up leaves wrong results behind).  Waits for the stream, then reads one word
-// of `temp`: for callers that synchronise anyway.  Always 0 for kernels that do not wait on each other.
-uint32_t scanWaitsGivenUp(const CubScanKernels& kernels, const void* temp, Stream& stream);
+// How many waits of the last launch on `temp` gave up.  Scans that publish totals between blocks bound every wait so that each
+// wavefront has an exit; a wait that gives up works the totals it lacks out again from the input, so the results are complete
+// and the same bits either way: this is a diagnostic, not an error.  Waits for the stream, then reads one word of `temp`: for
+// callers that synchronise anyway.  Always 0 for kernels that do not wait on each other.
+uint32_t scanWaitsRecovered(const CubScanKernels& kernels, const void* temp, Stream& stream);
+// The sum of what scanWaitsRecovered returned in this process (every thor_scan call adds its count).
+uint64_t scanWaitsRecoveredTotal();
 
 // One scan (flat: offsets null and segmentSize 0; rows of segmentSize; or the numSegments segments of *offsets) that compiles, loads
 // and allocates nothing: its kernels must be in the process-wide cache already (std::runtime_error otherwise) and its temporary

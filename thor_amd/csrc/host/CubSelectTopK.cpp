@@ -362,18 +362,29 @@ std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, u
     sel.threads = 256;
     sel.digits = static_cast<int>(digitPlanFor(dataTypeSizeInBytes(dtype) * 8).size());
     sel.chunks = numSegments;
-    const uint64_t items = (segmentSize + 255) / 256;
+    // Rows that a wavefront can hold (at most 64 keys per lane: 4096 keys) take the kernel with one wavefront per row and four
+    // rows per block; longer rows the one with a block per row.  THOR_TOPK_ROW_KERNEL=block forces the latter (a test switch).
+    const uint64_t vec = 16 / dataTypeSizeInBytes(dtype);
+    const uint64_t vectorsPerLane = (segmentSize + 64 * vec - 1) / (64 * vec);
+    const char* forced = std::getenv("THOR_TOPK_ROW_KERNEL");
+    const bool wavePerRow = vectorsPerLane * vec <= 64 && !(forced && std::string(forced) == "block");
+    const uint64_t items = wavePerRow ? vectorsPerLane : (segmentSize + 255) / 256;
+    sel.chunks = wavePerRow ? (numSegments + 3) / 4 : numSegments;
     std::ostringstream s;
     s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
     s << "namespace gen {\nstruct Cfg {\n";
     writeKeyTraits(s, dtype, largest, pairs);
     s << "    static constexpr thor::u32 kSegment = " << segmentSize << "u;\n    static constexpr thor::u64 kK = " << k
-      << "ull;\n    static constexpr int kThreads = 256;\n    static constexpr int kItems = " << items << ";\n};\n}  // namespace gen\n";
+      << "ull;\n    static constexpr thor::u64 kRows = " << numSegments << "ull;\n    static constexpr int kVec = " << vec
+      << ";\n    static constexpr int kThreads = 256;\n    static constexpr int kItems = " << items << ";\n};\n}  // namespace gen\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_rows(const gen::Cfg::Raw* keys, const thor::u32* values, gen::Cfg::Raw* outKeys, "
-         "thor::u32* outValues) {\n    thor::topkRows<gen::Cfg>(keys, values, outKeys, outValues);\n}\n";
+         "thor::u32* outValues) {\n    thor::" << (wavePerRow ? "topkRowsWave" : "topkRows") << "<gen::Cfg>(keys, values, outKeys, outValues);\n}\n";
     sel.first = compileKernel(s.str(), "thor_topk_rows", deviceNum, false);
     std::ostringstream v;
-    v << "row top-k radix-select bits" << dataTypeSizeInBytes(dtype) * 8 << " digits" << sel.digits << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of "
+    v << "row top-k " << (wavePerRow ? "bit-select wavefront-per-row" : "radix-select block-per-row") << " bits" << dataTypeSizeInBytes(dtype) * 8
+      << (wavePerRow ? " vec" + std::to_string(vec) + "x" + std::to_string(items) + (k <= 64 && vectorsPerLane % 2 == 0 && segmentSize >= 32 * vec * vectorsPerLane && vectorsPerLane * vec > 16 ? " floor-candidates" : "")
+                     : " digits" + std::to_string(sel.digits))
+      << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys") << " k" << k << " of "
       << segmentSize << " rows" << numSegments << " launches1 [" << sel.first->kernelName << "]";
     sel.variant = v.str();
     return kernels;

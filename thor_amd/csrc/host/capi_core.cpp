@@ -469,13 +469,13 @@ int thor_scan(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, 
             cubDeviceScan(plan, temp, in, out, stream->stream);
             kernels = plan.kernels;
         }
-        // this entry point frees its temporary storage on return, which waits for the device anyway: a wait between blocks that
-        // gave up is reported here
-        if (const uint32_t gaveUp = scanWaitsGivenUp(*kernels, temp.getMemPtr(), stream->stream)) {
-            throw std::runtime_error("CUB scan: " + std::to_string(gaveUp) + " wait(s) for the totals of earlier chunks gave up; the results are incomplete.");
-        }
+        // this entry point frees its temporary storage on return, which waits for the device anyway: waits between blocks that
+        // gave up (and worked their totals out again, so the results are complete) are counted here
+        scanWaitsRecovered(*kernels, temp.getMemPtr(), stream->stream);
         if (variant) copyOut(cubScanKernelVariant(kernels), variant, variant_capacity, nullptr);)
 }
+
+uint64_t thor_scan_waits_recovered(void) { return scanWaitsRecoveredTotal(); }
 
 int thor_scan_no_alloc(thor_tensor_t input, thor_tensor_t output, thor_tensor_t offsets, uint64_t num_items, uint64_t num_segments,
                        uint64_t segment_size, int op, int arg, int inclusive, int reverse, thor_stream_t stream, char* variant, size_t variant_capacity) {

@@ -62,6 +62,7 @@ PROTOTYPES = {
     "thor_stamped_segmented_reduction_variant": (_i, [_vp, _cp, _sz]),
     "thor_segmented_broadcast": (_i, [_vp, _vp, _vp, _i, _vp]),
     "thor_scan": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
+    "thor_scan_waits_recovered": (ctypes.c_uint64, []),
     "thor_scan_no_alloc": (_i, [_vp, _vp, _vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _i, _i, _i, _i, _vp, _cp, _sz]),
     "thor_select_flagged": (_i, [_vp, _vp, _vp, _vp, ctypes.c_uint64, _vp, _cp, _sz]),
     "thor_select_flagged_prepare": (_vp, [_vp, _vp, _vp, _vp, ctypes.c_uint64]),
@@ -578,6 +579,12 @@ def scan(input: PhysicalTensor, output: PhysicalTensor, stream: Stream, op: Scan
     _check(entry(input._h, output._h, segment_offsets._h if segment_offsets is not None else None, n, segments, segment_size, code, int(arg),
                  int(inclusive), int(reverse), stream._h, text, 512), "scan")
     return text.value.decode()
+
+
+def scan_waits_recovered() -> int:
+    """How many bounded waits between the blocks of one-launch scans gave up, and recomputed what they waited for, over all
+    ``scan`` calls of this process (a diagnostic; results are complete either way)."""
+    return int(lib().thor_scan_waits_recovered())
 
 
 class SelectionPlan:
