@@ -27,8 +27,12 @@ namespace ThorImplementation {
 
 inline constexpr const char* DEFAULT_BACKWARD_UPSTREAM_INPUT_NAME = "__grad_output";
 
-// Shapes are needed to undo broadcasting and to expand reduced gradients, so `forward_input_dims` (by input name) must be
-// given; std::runtime_error otherwise.
+// With `forward_input_dims` (by input name) every gradient has exactly the shape of its input: contributions to an operand that
+// the forward op broadcast are summed back, gradients of reductions are expanded.  Without them (the reference's shape-free form)
+// nothing is expanded or summed back - the implicit seed is the scalar 1, contributions keep the shape broadcasting gives them -
+// which is the gradient itself for graphs whose operands all have one shape; reshapes, squeezing reductions, means, min / max
+// reductions, softmax, strided views and segmented ops need shapes and throw std::runtime_error ("... requires forward shape
+// information.").  FusedEquation::compileBackward always builds with the shapes of the tensors it is stamped with.
 PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forward_outputs, const std::vector<std::string>& wrt_names = {},
                                      const std::optional<std::string>& upstream_input_name = std::nullopt,
                                      const std::optional<std::unordered_map<std::string, std::vector<uint64_t>>>& forward_input_dims = std::nullopt,
@@ -37,6 +41,22 @@ PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forward_outputs, con
 // Explicit upstream gradient input per forward output (may name a subset: outputs without an entry contribute nothing).
 PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forward_outputs, const std::vector<std::string>& wrt_names,
                                      const std::unordered_map<std::string, std::string>& upstream_input_names_by_output,
+                                     const std::optional<std::unordered_map<std::string, std::vector<uint64_t>>>& forward_input_dims = std::nullopt,
+                                     bool accumulate_grad_outputs = false);
+
+// As above, with the runtime dtype of each upstream gradient input (by forward-output name; an input named without its dtype
+// throws): the seed's INPUT node carries it, so dtype resolution of the backward graph starts from the tensor that will be bound.
+PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forward_outputs, const std::vector<std::string>& wrt_names,
+                                     const std::unordered_map<std::string, std::string>& upstream_input_names_by_output,
+                                     const std::unordered_map<std::string, DataType>& upstream_input_dtypes_by_output,
+                                     const std::optional<std::unordered_map<std::string, std::vector<uint64_t>>>& forward_input_dims = std::nullopt,
+                                     bool accumulate_grad_outputs = false);
+
+// As above, with upstream gradients that are values of the forward graph itself (node indices by forward-output name; they take
+// precedence over an input named for the same output).
+PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forward_outputs, const std::vector<std::string>& wrt_names,
+                                     const std::unordered_map<std::string, std::string>& upstream_input_names_by_output,
+                                     const std::unordered_map<std::string, uint32_t>& upstream_node_indices_by_output,
                                      const std::optional<std::unordered_map<std::string, std::vector<uint64_t>>>& forward_input_dims = std::nullopt,
                                      bool accumulate_grad_outputs = false);
 

@@ -72,6 +72,15 @@ inline bool isValueReductionOp(ExprOp op) {
 // other coordinate (NCHW semantics; the last axis of an [N, C] matrix), Instance = over every axis but the first.
 enum class SoftmaxAlgorithm : uint8_t { Fast = 0, Accurate = 1, Log = 2 };
 enum class SoftmaxMode : uint8_t { Instance = 0, Channel = 1 };
+}  // namespace ThorImplementation
+
+// The two enumerations the reference's softmax signatures are spelled with (Expression.h:736-738 there; they come from cudnn.h),
+// under cuDNN's type names, enumerator names and values, so that a caller written against the reference compiles unchanged:
+// `x.softmax(CUDNN_SOFTMAX_ACCURATE, CUDNN_SOFTMAX_MODE_CHANNEL)`.  They are names only: nothing of cuDNN is used or needed.
+enum cudnnSoftmaxAlgorithm_t { CUDNN_SOFTMAX_FAST = 0, CUDNN_SOFTMAX_ACCURATE = 1, CUDNN_SOFTMAX_LOG = 2 };
+enum cudnnSoftmaxMode_t { CUDNN_SOFTMAX_MODE_INSTANCE = 0, CUDNN_SOFTMAX_MODE_CHANNEL = 1 };
+
+namespace ThorImplementation {
 
 // Prefix scans along the last axis (Expression.h:181-193 there).  ArgMin / ArgMax return the UINT32 flattened index of the
 // element that holds the running minimum / maximum (the first one among equals), 0xFFFFFFFF where the prefix is empty.
@@ -424,6 +433,11 @@ class Expression {
     // register-resident row kernel.
     Expression softmax(SoftmaxAlgorithm algorithm = SoftmaxAlgorithm::Accurate, SoftmaxMode mode = SoftmaxMode::Channel) const;
     Expression logSoftmax(SoftmaxMode mode = SoftmaxMode::Channel) const;
+    // the reference's spelling of the same two (the enumerators map one to one)
+    Expression softmax(cudnnSoftmaxAlgorithm_t algorithm, cudnnSoftmaxMode_t mode = CUDNN_SOFTMAX_MODE_CHANNEL) const {
+        return softmax(static_cast<SoftmaxAlgorithm>(algorithm), static_cast<SoftmaxMode>(mode));
+    }
+    Expression logSoftmax(cudnnSoftmaxMode_t mode) const { return logSoftmax(static_cast<SoftmaxMode>(mode)); }
 
     // ---- shape -------------------------------------------------------------------------------------------------------
     Expression reshape(const std::vector<uint64_t>& new_dims) const;

@@ -263,7 +263,48 @@ static void autodiffGraphStructure() {
     CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"x"}, std::string("w"), dims); }));        // collides with an input
     CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"nope"}, std::nullopt, dims); }));         // unknown input
     CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"x", "x"}, std::nullopt, dims); }));       // duplicate
-    CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"x"}, std::nullopt, std::nullopt); }));    // shapes are required
+    {
+        // the shape-free forms (AutoDiff.h:15-27 there: forward_input_dims defaults to nullopt in every overload): the implicit seed
+        // is the scalar 1, nothing is summed back or expanded, rules that need a shape say so
+        const PhysicalOutputs shapeless = buildBackwardOutputs(forward, {"x", "w"});
+        CHECK(shapeless.outputs.size() == 2 && shapeless.outputs[0].name == "x_grad" && shapeless.outputs[1].name == "w_grad");
+        int sums = 0, fills = 0, ones = 0;
+        for (const ExprNode& node : shapeless.expr->nodes) {
+            sums += node.op == ExprOp::REDUCE_SUM;
+            fills += node.op == ExprOp::FILL;
+            ones += node.op == ExprOp::SCALAR_FP && node.scalar_fp == 1.0;
+        }
+        CHECK(sums == 0 && fills == 0 && ones >= 1);
+        CHECK((shapeless.expr->getInputNames() == std::set<std::string>{"x", "w"}));
+        const PhysicalOutputs named = buildBackwardOutputs(forward, {"x"}, std::unordered_map<std::string, std::string>{{"y", "__gy"}});
+        CHECK((named.expr->getInputNames() == std::set<std::string>{"x", "w", "__gy"}));
+        const PhysicalOutputs summed = buildBackwardOutputs(Expression::outputs({{"s", (x * x).reduce_sum({1}, {})}}).physicalOutputs(), {"x"});
+        CHECK(summed.outputs.size() == 1);  // a reduction that keeps its axes broadcasts back by itself
+        CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(Expression::outputs({{"r", x.reshape({12})}}).physicalOutputs(), {"x"}); }));
+        CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(Expression::outputs({{"m", x.reduce_mean({1}, {})}}).physicalOutputs(), {"x"}); }));
+        CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(Expression::outputs({{"m", x.reduce_sum({1}, {1})}}).physicalOutputs(), {"x"}); }));
+        // the overloads that carry the seeds' runtime dtypes, or take the seeds from the forward graph (AutoDiff.h:29-48 there)
+        const std::unordered_map<std::string, std::string> seedNames{{"y", "__gy"}};
+        const PhysicalOutputs typedSeed = buildBackwardOutputs(forward, {"x"}, seedNames, std::unordered_map<std::string, DataType>{{"y", DataType::FP16}}, dims);
+        bool carries = false;
+        for (const ExprNode& node : typedSeed.expr->nodes) {
+            carries = carries || (node.op == ExprOp::INPUT && typedSeed.expr->inputs.at(node.input_slot).name == "__gy" && node.output_dtype == DataType::FP16);
+        }
+        CHECK(carries);
+        CHECK(throwsAs<std::runtime_error>([&] { (void)buildBackwardOutputs(forward, {"x"}, seedNames, std::unordered_map<std::string, DataType>{}, dims); }));
+        const PhysicalOutputs nodeSeed =
+            buildBackwardOutputs(forward, {"x"}, seedNames, std::unordered_map<std::string, uint32_t>{{"y", forward.outputs[0].node_idx}}, dims);
+        CHECK((nodeSeed.expr->getInputNames() == std::set<std::string>{"x", "w"}));  // the seed is tanh(x * w) itself: no gradient input
+    }
+    {
+        // the reference's softmax spelling (Expression.h:736-738 there takes cuDNN's enumerations): the same nodes as this build's own
+        const Expression a = x.softmax(CUDNN_SOFTMAX_ACCURATE, CUDNN_SOFTMAX_MODE_CHANNEL), b = x.softmax(SoftmaxAlgorithm::Accurate, SoftmaxMode::Channel);
+        CHECK(a.expression().nodes.back().softmax_algorithm == b.expression().nodes.back().softmax_algorithm);
+        CHECK(a.expression().nodes.back().softmax_mode == SoftmaxMode::Channel);
+        CHECK(x.softmax(CUDNN_SOFTMAX_FAST, CUDNN_SOFTMAX_MODE_INSTANCE).expression().nodes.back().softmax_mode == SoftmaxMode::Instance);
+        CHECK(x.logSoftmax(CUDNN_SOFTMAX_MODE_INSTANCE).expression().nodes.back().softmax_algorithm == SoftmaxAlgorithm::Log);
+        CHECK(throwsAs<std::invalid_argument>([&] { (void)x.softmax(CUDNN_SOFTMAX_LOG); }));
+    }
     CHECK(throwsAs<std::runtime_error>([&] {
         (void)buildBackwardOutputs(Expression::outputs({{"y", x.floor() * w}}).physicalOutputs(), {"x"}, std::nullopt, dims);  // no rule for floor
     }));

@@ -20,6 +20,7 @@
 #include <dlfcn.h>
 #include <poll.h>
 #include <spawn.h>
+#include <fcntl.h>
 #include <sys/socket.h>
 #include <sys/wait.h>
 #include <unistd.h>
@@ -320,15 +321,39 @@ static bool sendString(int fd, const std::string& s) {
 static int compileInWorker(const std::string& source, const std::string& name, const std::string& arch, const std::vector<std::string>& flags,
                            void** code, size_t* code_size, char* log, size_t log_capacity) {
     const std::string path = workerPath();
-    int toWorker[2], fromWorker[2], errWorker[2];
-    if (socketpair(AF_UNIX, SOCK_STREAM, 0, toWorker) != 0) return fail(-7, "thorhip_compile: socketpair failed: %s", std::strerror(errno));
-    if (pipe(fromWorker) != 0 || pipe(errWorker) != 0) return fail(-7, "thorhip_compile: pipe failed: %s", std::strerror(errno));
+    // Every descriptor is close-on-exec from its creation, so a worker started by another thread at the same moment inherits none
+    // of them (it would hold this call's pipes open and keep its reader waiting for an end that never comes); the three the
+    // worker needs are duplicated onto its standard descriptors, which clears the flag on the copies.
+    int toWorker[2] = {-1, -1}, fromWorker[2] = {-1, -1}, errWorker[2] = {-1, -1};
+    auto closeAll = [&] {
+        for (int* pair : {toWorker, fromWorker, errWorker})
+            for (int k = 0; k < 2; ++k)
+                if (pair[k] >= 0) ::close(pair[k]);
+    };
+    if (socketpair(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0, toWorker) != 0) return fail(-7, "thorhip_compile: socketpair failed: %s", std::strerror(errno));
+    if (pipe2(fromWorker, O_CLOEXEC) != 0 || pipe2(errWorker, O_CLOEXEC) != 0) {
+        const int reason = errno;
+        closeAll();
+        return fail(-7, "thorhip_compile: pipe failed: %s", std::strerror(reason));
+    }
+    // a process that runs with closed standard descriptors may have been handed 0, 1 or 2 here: duplicating a descriptor onto itself
+    // would leave its close-on-exec flag set, so the worker's ends are moved out of that range first
+    for (int* end : {&toWorker[0], &fromWorker[1], &errWorker[1]}) {
+        if (*end > STDERR_FILENO) continue;
+        const int moved = fcntl(*end, F_DUPFD_CLOEXEC, STDERR_FILENO + 1);
+        if (moved < 0) {
+            const int reason = errno;
+            closeAll();
+            return fail(-7, "thorhip_compile: cannot move a descriptor: %s", std::strerror(reason));
+        }
+        ::close(*end);
+        *end = moved;
+    }
     posix_spawn_file_actions_t actions;
     posix_spawn_file_actions_init(&actions);
     posix_spawn_file_actions_adddup2(&actions, toWorker[0], STDIN_FILENO);
     posix_spawn_file_actions_adddup2(&actions, fromWorker[1], STDOUT_FILENO);
     posix_spawn_file_actions_adddup2(&actions, errWorker[1], STDERR_FILENO);
-    for (int fd : {toWorker[0], toWorker[1], fromWorker[0], fromWorker[1], errWorker[0], errWorker[1]}) posix_spawn_file_actions_addclose(&actions, fd);
     char* const argv[] = {const_cast<char*>(path.c_str()), nullptr};
     pid_t pid = -1;
     const int spawned = posix_spawn(&pid, path.c_str(), &actions, nullptr, argv, environ);

@@ -43,8 +43,11 @@ Dims broadcastOf(const Dims& a, const Dims& b) {
 // The backward graph under construction: nodes are appended in dependency order and every node's shape is tracked.
 class BackwardGraph {
    public:
-    BackwardGraph(const PhysicalExpression& forward, const std::vector<Dims>& forwardDims) : forward(forward), forwardDims(forwardDims) {}
+    // shapeless: the caller gave no dimensions; no shape is tracked and nothing is expanded or summed back
+    BackwardGraph(const PhysicalExpression& forward, const std::vector<Dims>& forwardDims, bool shapeless = false)
+        : shapeless(shapeless), forward(forward), forwardDims(forwardDims) {}
 
+    const bool shapeless;
     PhysicalExpression graph;
     std::vector<Dims> dims;
 
@@ -108,7 +111,7 @@ class BackwardGraph {
         n.op = op;
         n.lhs = a;
         n.rhs = b;
-        return push(std::move(n), broadcastOf(dims[a], dims[b]));
+        return push(std::move(n), shapeless ? Dims{} : broadcastOf(dims[a], dims[b]));
     }
     uint32_t add(uint32_t a, uint32_t b) { return binary(ExprOp::ADD, a, b); }
     uint32_t sub(uint32_t a, uint32_t b) { return binary(ExprOp::SUB, a, b); }
@@ -143,7 +146,7 @@ class BackwardGraph {
     }
     uint32_t transpose(uint32_t a) {
         Dims d = dims[a];
-        std::swap(d[d.size() - 1], d[d.size() - 2]);
+        if (d.size() >= 2) std::swap(d[d.size() - 1], d[d.size() - 2]);
         ExprNode n;
         n.op = ExprOp::TRANSPOSE;
         n.lhs = a;
@@ -293,7 +296,7 @@ class BackwardGraph {
     // `a`, which broadcasts against `target`, brought to exactly `target`: expanded where it is smaller, summed over the
     // axes along which the forward op broadcast the operand
     uint32_t sumToShape(uint32_t a, const Dims& target) {
-        if (dims[a] == target) return a;
+        if (shapeless || dims[a] == target) return a;
         const Dims full = broadcastOf(dims[a], target);
         if (dims[a] != full) a = add(a, fill(0.0, full));
         if (full == target) return a;
@@ -349,7 +352,9 @@ std::unordered_set<std::string> rowPartitionInputs(const PhysicalExpression& for
 // are undone to and that gradients are delivered in come from it.
 PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const PhysicalExpression* typed, const std::vector<std::string>& wrtNames,
                               const std::optional<std::unordered_map<std::string, std::string>>& upstreamByOutput,
-                              const std::optional<std::unordered_map<std::string, Dims>>& inputDimsByName, bool accumulate) {
+                              const std::optional<std::unordered_map<std::string, Dims>>& inputDimsByName, bool accumulate,
+                              const std::unordered_map<std::string, DataType>* seedDTypes = nullptr,
+                              const std::unordered_map<std::string, uint32_t>* seedNodes = nullptr) {
     if (!forwardOutputs.expr) throw std::runtime_error("buildBackwardOutputs requires non-null forward_outputs.expr.");
     const PhysicalExpression& forward = *forwardOutputs.expr;
     if (typed && typed->nodes.size() != forward.nodes.size()) throw std::logic_error("Autodiff: the dtype-resolved graph does not match the forward graph.");
@@ -367,19 +372,26 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
             "buildBackwardOutputs for multi-output forward equations requires an explicit upstream seed map. The map may be partial when "
             "some outputs have no incoming gradient.");
     }
-    if (upstreamByOutput.has_value() && upstreamByOutput->empty()) {
+    if (upstreamByOutput.has_value() && upstreamByOutput->empty() && !(seedNodes && !seedNodes->empty())) {
         throw std::runtime_error("buildBackwardOutputs explicit upstream seed map must contain at least one forward output.");
     }
-    if (!inputDimsByName.has_value()) {
-        throw std::runtime_error("buildBackwardOutputs requires the dimensions of the forward inputs (forward_input_dims).");
-    }
-
-    const std::vector<Dims> fdims = inferExpressionShapes(forward, [&](uint32_t slot) {
-        const std::string& name = forward.inputs.at(slot).name;
-        auto it = inputDimsByName->find(name);
-        if (it == inputDimsByName->end()) throw std::runtime_error("buildBackwardOutputs is missing the dimensions of forward input: " + name);
-        return it->second;
-    });
+    // Without the dimensions of the forward inputs (the reference's shape-free form, AutoDiff.cpp:3756,3829-3870 there) no
+    // gradient is expanded over reduced axes or summed back over broadcast ones: every contribution keeps the shape that
+    // broadcasting gives it, the implicit seed is the scalar 1, and a gradient nothing reaches is the scalar 0.  That is the
+    // gradient itself for graphs whose operands all have one shape; rules that cannot be written without shapes throw.
+    const bool shapeless = !inputDimsByName.has_value();
+    const std::vector<Dims> fdims = shapeless ? std::vector<Dims>(forward.nodes.size())
+                                              : inferExpressionShapes(forward, [&](uint32_t slot) {
+                                                    const std::string& name = forward.inputs.at(slot).name;
+                                                    auto it = inputDimsByName->find(name);
+                                                    if (it == inputDimsByName->end()) {
+                                                        throw std::runtime_error("buildBackwardOutputs is missing the dimensions of forward input: " + name);
+                                                    }
+                                                    return it->second;
+                                                });
+    auto needsShapes = [&](const char* what) {
+        if (shapeless) throw std::runtime_error(std::string("AutoDiff ") + what + " backward requires forward shape information.");
+    };
 
     // nodes through which a requested input is reached
     std::unordered_set<std::string> wanted(wrt.begin(), wrt.end());
@@ -397,7 +409,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
             if (c != kNone && reaches[c]) reaches[i] = 1;
     }
 
-    BackwardGraph b(forward, fdims);
+    BackwardGraph b(forward, fdims, shapeless);
     std::vector<uint32_t> adjoint(forward.nodes.size(), kNone);
     auto contribute = [&](uint32_t child, uint32_t contribution) {
         if (child == kNone || !reaches[child]) return;
@@ -409,10 +421,27 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
         if (!reaches[o.node_idx]) continue;
         uint32_t seed;
         if (upstreamByOutput.has_value()) {
+            const auto node = seedNodes ? seedNodes->find(o.name) : decltype(seedNodes->find(o.name)){};
             auto it = upstreamByOutput->find(o.name);
-            if (it == upstreamByOutput->end()) continue;
-            seed = b.input(it->second);
-            b.setDims(seed, fdims[o.node_idx]);
+            if (seedNodes && node != seedNodes->end()) {
+                // the upstream gradient is a value of the forward graph itself
+                if (node->second >= forward.nodes.size()) throw std::runtime_error("buildBackwardOutputs upstream node index is out of range for output: " + o.name);
+                seed = b.value(node->second);
+            } else if (it != upstreamByOutput->end()) {
+                seed = b.input(it->second);
+                b.setDims(seed, fdims[o.node_idx]);
+                if (seedDTypes) {
+                    auto dtype = seedDTypes->find(o.name);
+                    if (dtype == seedDTypes->end()) {
+                        throw std::runtime_error("buildBackwardOutputs received an upstream gradient input without its runtime dtype for output: " + o.name);
+                    }
+                    b.graph.nodes[seed].output_dtype = dtype->second;
+                }
+            } else {
+                continue;  // a partial map: this output received no gradient
+            }
+        } else if (shapeless) {
+            seed = b.scalar(1.0);
         } else {
             seed = b.fill(1.0, fdims[o.node_idx].empty() ? Dims{1} : fdims[o.node_idx]);
         }
@@ -435,6 +464,11 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
         };
         // the gradient of a reduction's output, shaped like the reduced operand with size-1 reduced axes, then expanded
         auto expandedOverReducedAxes = [&](uint32_t node) {
+            if (shapeless) {
+                // a reduction that kept its axes broadcasts back by itself; squeezed axes cannot be put back without the rank
+                if (!n.squeeze_axes.empty()) needsShapes("squeezing reduction");
+                return node;
+            }
             Dims keptAsOnes = fdims[n.lhs];
             for (uint64_t axis : resolveReductionAxes(n.reduction_axes, keptAsOnes.size())) keptAsOnes[axis] = 1;
             return b.sumToShape(b.reshape(node, keptAsOnes), fdims[n.lhs]);
@@ -524,6 +558,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
             case ExprOp::RESHAPE:
             case ExprOp::UNSQUEEZE:
             case ExprOp::SQUEEZE:
+                needsShapes("reshape");
                 contribute(n.lhs, b.reshape(g, fdims[n.lhs]));
                 break;
             case ExprOp::TRANSPOSE:
@@ -533,6 +568,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
                 // the gradient lands on the elements the view addresses, 0 elsewhere (Utilities/Expression/AutoDiff.cpp:2100-2125 there);
                 // a view of a view addresses storage that is not the operand's own index space
                 if (isStorageViewOp(forward.nodes[n.lhs].op)) throw std::runtime_error(noRule(n.op) + " The operand is itself a view.");
+                needsShapes("strided view");
                 contribute(n.lhs, b.viewGradient(b.cast(g, DataType::FP32), n, fdims[n.lhs]));
                 break;
 
@@ -540,6 +576,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
                 contribute(n.lhs, expandedOverReducedAxes(g));
                 break;
             case ExprOp::REDUCE_AVG: {
+                needsShapes("reduce_mean");
                 const uint64_t count = elementCount(fdims[n.lhs]) / elementCount(fdims[i]);
                 contribute(n.lhs, b.div(expandedOverReducedAxes(g), b.scalar(static_cast<double>(count))));
                 break;
@@ -556,10 +593,12 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
                 break;
             case ExprOp::REDUCE_MIN:
             case ExprOp::REDUCE_MAX:
+                needsShapes("reduce_min / reduce_max");
                 contribute(n.lhs, b.routeToWinner(n.op == ExprOp::REDUCE_MIN ? ExprOp::REDUCE_MIN_BACKWARD : ExprOp::REDUCE_MAX_BACKWARD, x(), g, n));
                 break;
 
             case ExprOp::SOFTMAX: {
+                needsShapes("softmax");
                 const Dims& d = fdims[n.lhs];
                 if (d.size() < 2) throw std::runtime_error("Autodiff for softmax expects tensors of rank 2 or more.");
                 Dims axes;
@@ -582,6 +621,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
             case ExprOp::SEGMENTED_REDUCE_SUM:
             case ExprOp::SEGMENTED_REDUCE_MEAN:
                 // every row of a segment receives the segment's gradient (divided by the segment's length for a mean)
+                needsShapes("segmented reduction");
                 contribute(n.lhs, b.segmentedBroadcast(g, b.value(n.rhs), fdims[n.lhs].at(0), n.op == ExprOp::SEGMENTED_REDUCE_MEAN));
                 break;
             case ExprOp::SEGMENTED_REDUCE_MIN:
@@ -590,6 +630,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
                 contribute(n.lhs, b.segmentWinnerGradient(x(), b.cast(g, DataType::FP32), b.value(n.rhs), n));
                 break;
             case ExprOp::SEGMENTED_BROADCAST:
+                needsShapes("segmented broadcast");
                 contribute(n.lhs, b.segmentedReduce(n.segmented_broadcast_normalize_by_length ? ExprOp::SEGMENTED_REDUCE_MEAN : ExprOp::SEGMENTED_REDUCE_SUM,
                                                     g, b.value(n.rhs), n));
                 break;
@@ -641,7 +682,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
         const Dims shape = fdims[firstNode].empty() ? Dims{1} : fdims[firstNode];
         const std::optional<DataType>& dtype = dtypeOf(firstNode);
         const std::string outputName = name + "_grad";
-        if (total == kNone) total = b.fill(0.0, shape, dtype);
+        if (total == kNone) total = shapeless ? b.scalar(0.0) : b.fill(0.0, shape, dtype);
         if (accumulate) {
             const uint32_t running = b.input(outputName);
             b.setDims(running, shape);
@@ -651,7 +692,7 @@ PhysicalOutputs differentiate(const PhysicalOutputs& forwardOutputs, const Physi
         const uint32_t repeats = timesNamed[total]++;
         uint32_t terminal = total;
         for (uint32_t r = 0; r < repeats; ++r) terminal = b.add(terminal, b.scalar(0.0));
-        terminal = dtype.has_value() ? b.cast(terminal, dtype.value()) : b.add(terminal, b.fill(0.0, shape));
+        terminal = dtype.has_value() ? b.cast(terminal, dtype.value()) : b.add(terminal, shapeless ? b.scalar(0.0) : b.fill(0.0, shape));
         named.push_back(NamedOutput{outputName, terminal});
     }
     result.expr = std::make_shared<PhysicalExpression>(std::move(b.graph));
@@ -728,6 +769,27 @@ PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forwardOutputs, cons
                                      const std::unordered_map<std::string, std::string>& upstreamByOutput,
                                      const std::optional<std::unordered_map<std::string, std::vector<uint64_t>>>& inputDims, bool accumulate) {
     return differentiate(forwardOutputs, nullptr, wrtNames, normalizeBackwardUpstreamNames(forwardOutputs, upstreamByOutput), inputDims, accumulate);
+}
+
+PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forwardOutputs, const std::vector<std::string>& wrtNames,
+                                     const std::unordered_map<std::string, std::string>& upstreamByOutput,
+                                     const std::unordered_map<std::string, DataType>& upstreamDTypesByOutput,
+                                     const std::optional<std::unordered_map<std::string, std::vector<uint64_t>>>& inputDims, bool accumulate) {
+    return differentiate(forwardOutputs, nullptr, wrtNames, normalizeBackwardUpstreamNames(forwardOutputs, upstreamByOutput), inputDims, accumulate,
+                         &upstreamDTypesByOutput);
+}
+
+PhysicalOutputs buildBackwardOutputs(const PhysicalOutputs& forwardOutputs, const std::vector<std::string>& wrtNames,
+                                     const std::unordered_map<std::string, std::string>& upstreamByOutput,
+                                     const std::unordered_map<std::string, uint32_t>& upstreamNodeIndicesByOutput,
+                                     const std::optional<std::unordered_map<std::string, std::vector<uint64_t>>>& inputDims, bool accumulate) {
+    if (upstreamByOutput.empty() && !upstreamNodeIndicesByOutput.empty()) {
+        // seeds given as forward nodes only: the name map may be empty then
+        return differentiate(forwardOutputs, nullptr, wrtNames, std::unordered_map<std::string, std::string>{}, inputDims, accumulate, nullptr,
+                             &upstreamNodeIndicesByOutput);
+    }
+    return differentiate(forwardOutputs, nullptr, wrtNames, normalizeBackwardUpstreamNames(forwardOutputs, upstreamByOutput), inputDims, accumulate, nullptr,
+                         &upstreamNodeIndicesByOutput);
 }
 
 PhysicalOutputs buildBackwardOutputsTyped(const PhysicalOutputs& forwardOutputs, const PhysicalExpression& typedForward,

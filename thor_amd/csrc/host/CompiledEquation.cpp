@@ -114,11 +114,38 @@ std::string moduleKeyOf(const std::string& source, int deviceNum, bool fastContr
                   source.size());
     return text;
 }
+
+// A digest is not the text: a kernel taken from a cache is held against the source it was asked for.  `tagged` is what was compiled:
+// `plain` with "_<tag>" inserted behind every kernel name.
+bool sameSource(const std::string& tagged, const std::string& plain, const std::string& tag) {
+    const std::string inserted = "_" + tag;
+    size_t i = 0, j = 0;
+    while (i < tagged.size()) {
+        if (j < plain.size() && tagged[i] == plain[j]) {
+            ++i;
+            ++j;
+        } else if (tagged.compare(i, inserted.size(), inserted) == 0) {
+            i += inserted.size();
+        } else {
+            return false;
+        }
+    }
+    return j == plain.size();
+}
+
+void requireSameSource(const std::shared_ptr<CompiledKernel>& kernel, const std::string& source, const std::string& kernelName) {
+    if (!kernel || !kernel->module || !kernel->module->source) return;
+    if (!sameSource(*kernel->module->source, source, sourceTag(source))) {
+        throw std::logic_error("Kernel cache: two different sources of kernel '" + kernelName + "' share one 128-bit digest.");
+    }
+}
 }  // namespace
 
 std::shared_ptr<CompiledKernel> findLoadedKernel(const std::string& source, const std::string& kernelName, int deviceNum, bool fastContract) {
     auto hit = kernelCache().get(kernelName + "|" + moduleKeyOf(source, deviceNum, fastContract));
-    return hit ? *hit : nullptr;
+    if (!hit) return nullptr;
+    requireSameSource(*hit, source, kernelName);
+    return *hit;
 }
 
 std::shared_ptr<CompiledKernel> compileKernel(const std::string& plainSource, const std::string& kernelName, int deviceNum, bool fastContract) {
@@ -126,7 +153,7 @@ std::shared_ptr<CompiledKernel> compileKernel(const std::string& plainSource, co
     const std::string source = std::getenv("THOR_PLAIN_STREAM_STORES") ? "#define THOR_PLAIN_STREAM_STORES 1\n" + plainSource : plainSource;
     const std::string moduleKey = moduleKeyOf(source, deviceNum, fastContract);
     const std::string kernelKey = kernelName + "|" + moduleKey;
-    return kernelCache().getOrCreate(kernelKey, [&] {
+    std::shared_ptr<CompiledKernel> result = kernelCache().getOrCreate(kernelKey, [&] {
         ScopedGpu scoped(deviceNum);
         const std::string tag = sourceTag(source);
         const std::string taggedName = kernelName + "_" + tag;
@@ -167,6 +194,8 @@ std::shared_ptr<CompiledKernel> compileKernel(const std::string& plainSource, co
         (void)thorhip_function_get_attributes(kernel->function, &kernel->numRegisters, &kernel->staticLdsBytes, nullptr);
         return kernel;
     });
+    requireSameSource(result, source, kernelName);  // a hit of either cache is held against the text it was asked for
+    return result;
 }
 
 }  // namespace ThorImplementation

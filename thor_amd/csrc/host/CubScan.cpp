@@ -8,9 +8,11 @@
 #include "ReductionPlanner.h"
 #include "Utilities/Common/ScopedGpu.h"
 #include "thorhip_numeric_embed.h"
+#include "Utilities/Cache/LruCache.h"
 
 #include <algorithm>
 #include <atomic>
+#include <cstdio>
 #include <cstdlib>
 #include <numeric>
 #include <sstream>
@@ -127,7 +129,44 @@ Tensor allocateCubTemporaryStorage(const TensorPlacement& placement, size_t byte
     return Tensor(placement, TensorDescriptor(DataType::UINT8, {std::max<uint64_t>(bytes, 1)}));
 }
 
+namespace {
+// The kernels of the requests seen so far, by request and by the switches that enter the generated source: a caller that repeats
+// a request (a serving loop through the entry point that allocates nothing) gets them without the source being generated and
+// hashed again.
+const char* switchText(const char* name) {
+    const char* value = std::getenv(name);
+    return value ? value : "";
+}
+std::string requestKey(const ScanRequest& r) {
+    char text[320];
+    std::snprintf(text, sizeof text, "%d|%llu|%llu|%llu|%d|%d|%d%d%d%d%d|%llu|%d|%s|%s|%s", static_cast<int>(r.dtype), (unsigned long long)r.total,
+                  (unsigned long long)r.row, (unsigned long long)r.segments, r.offsets64 ? 1 : 0, r.op, r.writeValue ? 1 : 0, r.writeIndex ? 1 : 0,
+                  r.inclusive ? 1 : 0, r.reverse ? 1 : 0, r.route ? 1 : 0, (unsigned long long)r.alignmentBytes, r.deviceNum,
+                  switchText("THOR_SCAN_WAIT_LIMIT"), switchText("THOR_SCAN_THREADS"), switchText("THOR_SCAN_PASSES"));
+    return text;
+}
+LruCacheThreadSafe<std::string, std::shared_ptr<const CubScanKernels>>& builtScans() {
+    static LruCacheThreadSafe<std::string, std::shared_ptr<const CubScanKernels>> cache(1024);
+    return cache;
+}
+std::shared_ptr<const CubScanKernels> buildScanKernelsUncached(const ScanRequest& r, bool loadedOnly, size_t tempLimitBytes);
+}  // namespace
+
 std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, bool loadedOnly, size_t tempLimitBytes) {
+    const std::string key = requestKey(r);
+    if (auto known = builtScans().get(key)) {
+        if ((*known)->tempBytes > tempLimitBytes) {
+            throw std::invalid_argument("CUB scan: this request needs " + std::to_string((*known)->tempBytes) + " bytes of temporary storage, more than the " +
+                                        std::to_string(tempLimitBytes) + " bytes of the fixed scratch block; use the allocating scan.");
+        }
+        return *known;
+    }
+    std::shared_ptr<const CubScanKernels> built = buildScanKernelsUncached(r, loadedOnly, tempLimitBytes);
+    return builtScans().getOrCreate(key, [&] { return built; });
+}
+
+namespace {
+std::shared_ptr<const CubScanKernels> buildScanKernelsUncached(const ScanRequest& r, bool loadedOnly, size_t tempLimitBytes) {
     if (!isCubScanDTypeSupported(r.dtype)) throw std::invalid_argument(std::string("Unsupported CUB scan dtype ") + dataTypeName(r.dtype) + ".");
     if (r.total == 0) throw std::invalid_argument("CUB scan requires at least one element.");
     if ((r.writeIndex || r.op == 1 || r.op == 2) && r.total > 0xfffffffeull) {
@@ -211,7 +250,8 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
         std::shared_ptr<CompiledKernel> loaded = findLoadedKernel(source, name, r.deviceNum, false);
         if (!loaded) {
             throw std::runtime_error(std::string("CUB scan: kernel ") + name +
-                                     " of this request is not loaded yet; an ordinary scan of the same dtype, operation, sizes and alignment loads it.");
+                                     " of this request is not loaded yet; an ordinary scan of the same dtype, operation, sizes and alignment - made "
+                                     "with the same THOR_SCAN_WAIT_LIMIT / THOR_SCAN_THREADS / THOR_SCAN_PASSES in the environment - loads it.");
         }
         return loaded;
     };
@@ -229,6 +269,7 @@ std::shared_ptr<const CubScanKernels> buildScanKernels(const ScanRequest& r, boo
     k.variant = variant.str();
     return kernels;
 }
+}  // namespace
 
 void launchScan(const CubScanKernels& k, const void* input, const void* offsets, void* temp, size_t tempBytes, void* outValue, void* outIndex,
                 Stream& stream) {
