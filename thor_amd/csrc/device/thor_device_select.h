@@ -201,6 +201,17 @@ __device__ __forceinline__ u32 topkImage(typename Cfg::Raw raw) {
     return Cfg::kLargest ? u : (~u & kMask);
 }
 
+// The key whose image is `image` (topkImage is a bijection of the key's bits).
+template <typename Cfg>
+__device__ __forceinline__ typename Cfg::Raw topkKeyOfImage(u32 image) {
+    constexpr u32 kMask = Cfg::kBits == 32 ? 0xffffffffu : ((1u << Cfg::kBits) - 1u);
+    constexpr u32 kSign = 1u << (Cfg::kBits - 1);
+    u32 u = Cfg::kLargest ? image : (~image & kMask);
+    if (Cfg::kKind == 1) u ^= kSign;
+    if (Cfg::kKind == 2) u = (u & kSign) ? (u & ~kSign) : (~u & kMask);
+    return (typename Cfg::Raw)u;
+}
+
 // Digits are taken from the most significant end: 11, 11 and 10 bits of a 32-bit image, 8 and 8 of a 16-bit one, 8 of an 8-bit one.
 constexpr int kTopkMaxBins = 2048;
 constexpr int kTopkBinsPerThread = kTopkMaxBins / 256;
@@ -771,7 +782,7 @@ __device__ __forceinline__ u32 topkMaxPair(u32 a, u32 b) {
 // prefix: the image of the kK-th largest key; `remaining`: how many keys equal to it belong to the answer.
 template <typename Cfg, int SLOTS, typename Image, typename Position, typename Live>
 __device__ __forceinline__ void topkRowEmit(const Image& image, const Position& position, const Live& live, u32 prefix, u32 remaining,
-                                            const typename Cfg::Raw* rowIn, const u32* rowValuesIn, typename Cfg::Raw* rowKeys, u32* rowValues) {
+                                            const u32* rowValuesIn, typename Cfg::Raw* rowKeys, u32* rowValues) {
     const int lane = threadIdx.x % kWave;
     const u64 lowerLanes = ((u64)1 << lane) - 1;
     const u32 firstTieSlot = (u32)Cfg::kK - remaining;
@@ -790,7 +801,7 @@ __device__ __forceinline__ void topkRowEmit(const Image& image, const Position& 
         aboveAt += (u32)__builtin_popcountll(aboveVotes);
         tieAt += (u32)__builtin_popcountll(tieVotes);
         if (slot != 0xffffffffu) {
-            rowKeys[slot] = rowIn[position(j)];
+            rowKeys[slot] = topkKeyOfImage<Cfg>(image(j));  // the key's bits, from its image: no second read of the row
             if (Cfg::kPairs) rowValues[slot] = rowValuesIn[position(j)];
         }
     }
@@ -891,9 +902,17 @@ __device__ __forceinline__ void topkRowsWave(const typename Cfg::Raw* keys, cons
                 cImage[e] = kWideEntries ? ((u32)e < height ? wideImages[e * kWave] : 0u) : entry >> 16;
                 cSlot[e] = entry & 0xffffu;
             }
-            u32 prefix = 0;
+            // the wanted image lies between the floor and the row's largest image: the bits those two share are its own
+            u32 largest = group[0] > group[1] ? group[0] : group[1];
+#pragma unroll
+            for (int d = kWave / 2; d > 0; d >>= 1) {
+                const u32 other = __shfl_xor(largest, d, kWave);
+                largest = other > largest ? other : largest;
+            }
+            const int open = 32 - __builtin_clz((floorImage ^ largest) | 1u);  // bits below this one may differ
+            u32 prefix = open >= 32 ? 0u : (floorImage >> open) << open;
 #pragma unroll 1
-            for (int bit = Cfg::kBits - 1; bit >= 0; --bit) {
+            for (int bit = open - 1; bit >= 0; --bit) {
                 const u32 test = prefix | (1u << bit);
                 u32 count = 0;
 #pragma unroll
@@ -906,7 +925,7 @@ __device__ __forceinline__ void topkRowsWave(const typename Cfg::Raw* keys, cons
             for (int e = 0; e < E; ++e) above += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(cLive(e) && cImage[e] > prefix));
             topkRowEmit<Cfg, E>([&](int e) { return cImage[e]; },
                                 [&](int e) { return ((cSlot[e] / (u32)V) * kWave + (u32)lane) * (u32)V + cSlot[e] % (u32)V; }, cLive, prefix,
-                                (u32)Cfg::kK - above, rowIn, rowValuesIn, rowKeys, rowValues);
+                                (u32)Cfg::kK - above, rowValuesIn, rowKeys, rowValues);
             return;
         }
     }
@@ -924,7 +943,7 @@ __device__ __forceinline__ void topkRowsWave(const typename Cfg::Raw* keys, cons
 #pragma unroll
     for (int j = 0; j < R; ++j) mineAbove += live(j) && image(j) > prefix ? 1u : 0u;
     const u32 above = topkWaveSum<Cfg>(mineAbove);
-    topkRowEmit<Cfg, R>(image, position, live, prefix, (u32)Cfg::kK - above, rowIn, rowValuesIn, rowKeys, rowValues);
+    topkRowEmit<Cfg, R>(image, position, live, prefix, (u32)Cfg::kK - above, rowValuesIn, rowKeys, rowValues);
 }
 
 }  // namespace thor

@@ -377,7 +377,15 @@ std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, u
     s << "    static constexpr thor::u32 kSegment = " << segmentSize << "u;\n    static constexpr thor::u64 kK = " << k
       << "ull;\n    static constexpr thor::u64 kRows = " << numSegments << "ull;\n    static constexpr int kVec = " << vec
       << ";\n    static constexpr int kThreads = 256;\n    static constexpr int kItems = " << items << ";\n};\n}  // namespace gen\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_rows(const gen::Cfg::Raw* keys, const thor::u32* values, gen::Cfg::Raw* outKeys, "
+    // A wavefront of the one-per-row kernel spends most of its life waiting (the row's loads, then chains of votes and counts), so
+    // what counts is how many of them a SIMD holds: the compiler is asked to leave room for as many as the row's registers
+    // (two 16-bit images to a register) plus about 40 others allow.  Measured on [16384, 4096] bf16, k = 64 (wavefronts per SIMD
+    // asked for -> time): none 38.1 us, 5 34.0, 6 31.6, 7 30.8, 8 37.1 (spills).  THOR_TOPK_ROW_WAVES overrides it (a tuning switch).
+    const uint64_t rowRegisters = vectorsPerLane * vec / (dataTypeSizeInBytes(dtype) == 2 ? 2 : 1);
+    const char* forcedWaves = std::getenv("THOR_TOPK_ROW_WAVES");
+    const int wavesPerSimd = forcedWaves ? std::max(1, std::atoi(forcedWaves)) : static_cast<int>(std::min<uint64_t>(8, std::max<uint64_t>(1, 512 / (rowRegisters + 41))));
+    s << "extern \"C\" __global__ __launch_bounds__(256" << (wavePerRow ? ", " + std::to_string(wavesPerSimd) : std::string())
+      << ") void thor_topk_rows(const gen::Cfg::Raw* keys, const thor::u32* values, gen::Cfg::Raw* outKeys, "
          "thor::u32* outValues) {\n    thor::" << (wavePerRow ? "topkRowsWave" : "topkRows") << "<gen::Cfg>(keys, values, outKeys, outValues);\n}\n";
     sel.first = compileKernel(s.str(), "thor_topk_rows", deviceNum, false);
     std::ostringstream v;
