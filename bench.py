@@ -233,6 +233,23 @@ def bench_other_configs(only=None):
     timed("c5_relu_and_channel_statistics_one_pass_fp16", [p_.run for p_ in plans], 4 * n, n,
           ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
     del xc, xc8, plans, csum
+    # the same kernels on four times the batch ([256, 256, 56, 56], 392 MiB per tensor): a launch on the BASELINE tensor lasts 18 us, so its
+    # ramp and tail weigh on its rate; these lines show what the kernels stream at once they run long enough
+    shape4 = (256, 256, 56, 56)
+    n4 = int(np.prod(shape4))
+    big = [ph.PhysicalTensor(ph.Placement(ph.DeviceType.gpu, 0), ph.PhysicalTensor.Descriptor(DataType.fp16, list(shape4))) for _ in range(3)]
+    quarter = gpu_from(rng.standard_normal(shape, dtype=np.float32), DataType.fp16)
+    for t in big:
+        for part in range(4):
+            _lib.check(_lib.load().thorhip_memcpy_async(t.mem_ptr() + part * n * 2, quarter.mem_ptr(), n * 2, 3, stream.handle), "d2d")
+    stream.synchronize()
+    csum = [ph.CubReduction(ph.CubReductionOp.Sum, [0, 2, 3], DataType.fp32).stamp(t, stream) for t in big]
+    timed("c5_channel_sum_fp16_batch256", [c.run for c in csum], 2 * n4, n4, csum[0].get_kernel_variant())
+    plans = [stats.stamp({"x": t}, stream) for t in big]
+    timed("c5_channel_sum_and_sumsq_fp16_batch256", [p_.run for p_ in plans], 2 * n4, n4, ">".join(plans[0].stage_kind_names()) + " " + plans[0].stage_descriptions()[0])
+    plans = [relu.stamp({"x": t, "scale": scale, "bias": bias}, stream) for t in big[:2]]
+    timed("c5_relu_scale_bias_fp16_batch256", [p_.run for p_ in plans], 4 * n4, n4, "+".join(plans[0].stage_descriptions()))
+    del big, quarter, plans, csum
 
     # ---- ragged batches (the rows next to the dense path): [2^22, 64] fp32 values (1 GiB) in 65 536 segments of log-normal
     # length; bytes counted are the values read once (reductions), written once (broadcast), read + written once (softmax)

@@ -264,6 +264,33 @@ bool tryFoldConstant(const PhysicalExpression& expr, uint32_t nodeIndex, double&
     }
 }
 
+namespace {
+// exp(-max(-x, 0)) evaluated in fp32 - the numerator of the reference's overflow-safe sigmoid, exp(-max(-x, 0)) / (1 + exp(-|x|))
+// (Expression.cpp:3261-3296 there).  For x < 0 its argument -(-x) is x = -|x| bit for bit; otherwise (x >= 0, -0, NaN: the
+// maximum ignores a NaN) the argument is -0 and the value exactly 1.  Written as `x < 0 ? exp(-|x|) : 1` it gives the same
+// bits and shares its exponential with the denominator's: one exponential per sigmoid instead of two.
+bool isExpOfMinusPositivePart(const PhysicalExpression& expr, uint32_t nodeIndex, uint32_t& x) {
+    auto fp32 = [&](uint32_t i) { return i != UINT32_MAX && emittedValueDType(expr.nodes[i]) == DataType::FP32; };
+    const ExprNode& e = expr.nodes[nodeIndex];
+    if (e.op != ExprOp::EXP || !fp32(nodeIndex) || !fp32(e.lhs)) return false;
+    if (std::getenv("THOR_SIGMOID_TWO_EXPONENTIALS")) return false;  // diagnostic switch: the literal form, for A/B runs
+    const ExprNode& outer = expr.nodes[e.lhs];
+    if (outer.op != ExprOp::NEG || !fp32(outer.lhs)) return false;
+    const ExprNode& larger = expr.nodes[outer.lhs];
+    if (larger.op != ExprOp::MAX) return false;
+    for (int side = 0; side < 2; ++side) {
+        const uint32_t negated = side == 0 ? larger.lhs : larger.rhs, zero = side == 0 ? larger.rhs : larger.lhs;
+        double constant;
+        if (!tryFoldConstant(expr, zero, constant) || constant != 0.0 || !fp32(negated)) continue;
+        const ExprNode& inner = expr.nodes[negated];
+        if (inner.op != ExprOp::NEG || inner.lhs == UINT32_MAX) continue;
+        x = inner.lhs;
+        return true;
+    }
+    return false;
+}
+}  // namespace
+
 BodyEmitter::BodyEmitter(const PhysicalExpression& expr)
     : expr(expr), valueDType(expr.nodes.size()), names(expr.nodes.size()), rowDivisors(expr.nodes.size()) {}
 
@@ -331,6 +358,10 @@ uint64_t BodyEmitter::emit(std::string& out, uint32_t nodeIndex, const std::stri
         flops = 1;
     } else if (Expression::isBinaryOp(n.op)) {
         out += decl + binary(n, dtype) + ";\n";
+        flops = opFlops(n.op);
+    } else if (uint32_t x; isExpOfMinusPositivePart(expr, nodeIndex, x) && defined(x)) {
+        const std::string value = ref(x, DataType::FP32);
+        out += decl + "((" + value + " < 0.0f) ? expf((-fabsf(" + value + "))) : 1.0f);\n";
         flops = opFlops(n.op);
     } else {
         out += decl + unary(n, dtype) + ";\n";

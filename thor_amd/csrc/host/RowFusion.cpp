@@ -393,6 +393,10 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         while (T < 256 && T * vectorsPerLane < vectors) T <<= 1;
         while (T < 1024 && T < vectors && (vectors + T - 1) / T * vec * registersPerElement > softTarget) T <<= 1;
         while (T < 1024 && ((vectors + T - 1) / T * vec > 64 || (vectors + T - 1) / T * vec * registersPerElement > budget(T))) T <<= 1;
+        if (const char* forced = std::getenv("THOR_ROW_THREADS")) {  // tuning switch: lanes per row (a power of two up to 1024)
+            const uint64_t wanted = static_cast<uint64_t>(std::max(1, std::atoi(forced)));
+            if ((wanted & (wanted - 1)) == 0 && wanted <= 1024 && (vectors + wanted - 1) / wanted * vec <= 64) T = wanted;
+        }
         items = (vectors + T - 1) / T;
         return !(items * vec > 64 || items * vec * registersPerElement > budget(T));
     };
@@ -408,8 +412,20 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     const bool subWave = T <= 64;
     const uint64_t threads = subWave ? 256 : T;
     const uint64_t rowsPerBlock = subWave ? 256 / T : 1;
+    // A block that owns a row spends part of its life in folds and barriers with no load in flight.  THOR_ROW_TURNS (a tuning
+    // switch) makes it take that many consecutive rows in turn, the loads of the next row issued before it works on the current
+    // one (the row's sources are the only registers that double).  Measured, it loses: eight resident blocks per compute unit
+    // already overlap one block's folds with the others' loads, and fewer, longer blocks overlap less - softmax bf16
+    // [16384, 4096] 68 / 71 / 78 / 87 us with 1 / 2 / 4 / 8 rows in turn, normalisation fp32 [32768, 1024] 44.5 / 46.7 / 50.7 /
+    // 51.6 us.  So the default is one row per block.
+    uint64_t turns = 1;
+    if (const char* forced = std::getenv("THOR_ROW_TURNS")) turns = subWave ? 1 : static_cast<uint64_t>(std::max(1, std::atoi(forced)));
+    turns = std::min<uint64_t>(turns, std::max<uint64_t>(rg.rows / 2048, 1));  // not at the price of an idle compute unit
+    for (uint32_t sNode : em.sourceNodes)
+        if (rg.cls[sNode] == Cls::ColVec) turns = 1;  // operands shared by all rows are loaded once, ahead of everything
+    const bool inTurns = turns > 1;
     em.threads = static_cast<uint32_t>(threads);
-    em.gridX = static_cast<uint32_t>((rg.rows + rowsPerBlock - 1) / rowsPerBlock);
+    em.gridX = static_cast<uint32_t>((rg.rows + rowsPerBlock * turns - 1) / (rowsPerBlock * turns));
 
     em.fastContract = true;
     for (uint32_t m : members) {
@@ -433,18 +449,25 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         s << "    const unsigned long long row = (unsigned long long)thor::xcdBlock<" << xcdRunLength(1) << ">(blockIdx.x, gridDim.x) * " << rowsPerBlock
           << "ull + threadIdx.x / T;\n";
         s << "    const int lane = threadIdx.x % T;\n";
+    } else if (inTurns) {
+        s << "    constexpr int TURNS = " << turns << ";\n";
+        s << "    const unsigned long long firstRow = (unsigned long long)thor::xcdBlock<" << xcdRunLength(1) << ">(blockIdx.x, gridDim.x) * TURNS;\n"
+             "    const int lane = threadIdx.x;\n";
     } else {
         s << "    const unsigned long long row = thor::xcdBlock<" << xcdRunLength(1) << ">(blockIdx.x, gridDim.x);\n    const int lane = threadIdx.x;\n";
     }
-    s << "    const bool rowLive = row < ROWS;\n";
-    s << "    const unsigned long long rowIndex = rowLive ? row : 0ull;\n";
-    s << "    const unsigned long long rowBase = rowIndex * R;\n";
     // when every lane of every block has a whole vector of a real row, the bounds checks vanish at compile time
-    const bool allLive = vectors % T == 0 && rg.rows % rowsPerBlock == 0 && tail == 0;
+    const bool allLive = vectors % T == 0 && rg.rows % (rowsPerBlock * turns) == 0 && tail == 0;
     const std::string liveIf = allLive ? "" : "if (live[it]) ";
-    s << "    bool live[ITEMS];\n    unsigned long long column[ITEMS];\n";
+    // what depends on the row: emitted once, or at the top of every turn
+    const std::string rowLines =
+        std::string("    const bool rowLive = row < ROWS;\n    const unsigned long long rowIndex = rowLive ? row : 0ull;\n"
+                    "    const unsigned long long rowBase = rowIndex * R;\n    bool live[ITEMS];\n"
+                    "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) live[it] = rowLive && (unsigned long long)it * T + lane < VECTORS;\n");
+    s << "    unsigned long long column[ITEMS];\n";
     s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        const unsigned long long v = (unsigned long long)it * T + lane;\n"
-         "        live[it] = rowLive && v < VECTORS;\n        column[it] = (v < VECTORS ? v : 0ull) * V;\n    }\n";
+         "        column[it] = (v < VECTORS ? v : 0ull) * V;\n    }\n";
+    if (!inTurns) s << rowLines;
     if (tail != 0) {
         // The row's last vector is read (and written) V - tail elements early, so that it ends with the row: it overlaps the
         // vector before it, folds skip the elements it shares with that one, and the stores write those twice with the same bits.
@@ -464,12 +487,25 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     std::map<uint32_t, size_t> sourceIndex;
     for (size_t o = 0; o < em.sourceNodes.size(); ++o) sourceIndex[em.sourceNodes[o]] = o;
     BodyEmitter uniform(expr);  // values that exist once per row (function scope)
+    std::string turnPrefetch, turnHandOver, turnUniform;  // in turns: the next row's loads, p = next, the row's own scalars
     for (size_t o = 0; o < em.sourceNodes.size(); ++o) {
         const uint32_t node = em.sourceNodes[o];
         const DataType storage = ctx.tensorOf[node].getDataType();
         const DataType valueDType = expr.nodes[node].output_dtype.value();
         const char* type = deviceTypeName(storage);
-        if (isElem(rg.cls[node])) {
+        if (isElem(rg.cls[node]) && inTurns && rg.cls[node] == Cls::RowVec) {
+            // the first row's loads here; every turn then issues the next row's before it works on its own
+            const std::string pack = "p" + std::to_string(o), in = "in" + std::to_string(o);
+            const std::string guard = allLive ? "" : "if (firstRow < ROWS && (unsigned long long)it * T + lane < VECTORS) ";
+            s << "    thor::Pack<" << type << ", V> " << pack << "[ITEMS];\n";
+            s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        " << pack << "[it] = {};\n        " << guard << pack << "[it]"
+              << (unaligned ? ".loadStreamUnaligned(" : ".loadStream(") << in << " + firstRow * R + column[it]);\n    }\n";
+            const std::string nextGuard = allLive ? "if (turn + 1 < TURNS) " : "if (turn + 1 < TURNS && row + 1 < ROWS && (unsigned long long)it * T + lane < VECTORS) ";
+            turnPrefetch += "    thor::Pack<" + std::string(type) + ", V> n" + pack + "[ITEMS];\n#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        n" + pack +
+                            "[it] = {};\n        " + nextGuard + "n" + pack + "[it]" + (unaligned ? ".loadStreamUnaligned(" : ".loadStream(") + in +
+                            " + (row + 1) * R + column[it]);\n    }\n";
+            turnHandOver += "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) " + pack + "[it] = n" + pack + "[it];\n";
+        } else if (isElem(rg.cls[node])) {
             s << "    thor::Pack<" << type << ", V> p" << o << "[ITEMS];\n";
             s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n        p" << o << "[it] = {};\n";
             if (rg.cls[node] == Cls::RowVec) {
@@ -481,9 +517,18 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         } else {
             const std::string index = rg.cls[node] == Cls::Scalar ? "0" : "rowIndex";
             std::string value = castValueExpr(storageToValueExpr("in" + std::to_string(o) + "[" + index + "]", storage), storage, valueDType);
-            s << "    const " << valueCType(valueDType) << " t" << node << " = " << value << ";\n";
+            const std::string line = "    const " + std::string(valueCType(valueDType)) + " t" + std::to_string(node) + " = " + value + ";\n";
+            if (inTurns) {
+                turnUniform += line;
+            } else {
+                s << line;
+            }
             uniform.defineSource(node, valueDType);
         }
+    }
+    if (inTurns) {
+        s << "#pragma unroll 1\n    for (int turn = 0; turn < TURNS; ++turn) {\n    const unsigned long long row = firstRow + turn;\n" << rowLines << turnPrefetch
+          << turnUniform;
     }
 
     auto isStoredOutput = [&](uint32_t node) { return rg.stored[node] != 0; };
@@ -554,6 +599,16 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
             const std::string name = "d" + std::to_string(n.rhs);
             s << "    const thor::RowDivisor " << name << "(" << uniform.ref(n.rhs, DataType::FP32) << ");\n";
             rowDivisorOf[n.rhs] = name;
+        }
+        // The next row's registers are taken over before the last loop when that loop reads no source: the wait for those loads
+        // then comes before this turn's stores are issued and does not have to sit through them.
+        bool lastLoopReadsSources = recompute;
+        for (uint32_t m : elemNodes)
+            for (uint32_t c : {expr.nodes[m].lhs, expr.nodes[m].rhs, expr.nodes[m].aux})
+                if (c != UINT32_MAX && rg.isSource[c] && rg.cls[c] == Cls::RowVec) lastLoopReadsSources = true;
+        if (inTurns && loop == numLoops - 1 && !lastLoopReadsSources) {
+            s << turnHandOver;
+            turnHandOver.clear();
         }
         s << "#pragma unroll\n    for (int it = 0; it < ITEMS; ++it) {\n";
         std::vector<uint32_t> storedHere;
@@ -681,6 +736,7 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
         }
         emitUniformUpTo(loop + 1);
     }
+    if (inTurns) s << turnHandOver << "    }\n";
     s << "}\n";
     // every member must have been produced
     for (uint32_t m : members) {
@@ -692,7 +748,8 @@ bool emitRegion(const RowFusionContext& ctx, const Region& rg, Emission& em) {
     em.source = s.str();
     em.flops *= rg.rows;
     em.description = "row_fused(rows=" + std::to_string(rg.rows) + ",R=" + std::to_string(rg.R) + ",lanes_per_row=" + std::to_string(T) +
-                     ",items=" + std::to_string(items) + ",vec=" + std::to_string(vec) + (unaligned ? ",unaligned_vectors" : "") + (recompute ? ",values_recomputed" : "") + ",loops=" + std::to_string(numLoops) + ")";
+                     ",items=" + std::to_string(items) + ",vec=" + std::to_string(vec) + (inTurns ? ",rows_in_turn=" + std::to_string(turns) : "") +
+                     (unaligned ? ",unaligned_vectors" : "") + (recompute ? ",values_recomputed" : "") + ",loops=" + std::to_string(numLoops) + ")";
     return true;
 }
 
