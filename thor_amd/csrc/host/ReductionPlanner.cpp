@@ -197,8 +197,9 @@ ReductionShape planReductionShape(const ReductionKernelRequest& request) {
     // output group are whole blocks.  THOR_REDUCE_TICKETS=0 keeps the finishing launch (tuning switch).
     // Measured on MI355X, finishing launch against last share: per-channel sums of an NCHW tensor (strided, 256 x 16 blocks) 21.0 /
     // 21.2 us, 16 rows of 2^22 (rows, 16 x 8 blocks) 49.5 / 48.9 us: as fast with one launch fewer, so these two kinds take
-    // tickets.  Whole-tensor sums (1024 arrivals on one word: 42 / 47 us) and column sums (256 device-wide partial stores per
-    // block: 53 / 84 us) keep the finishing launch unless THOR_REDUCE_TICKETS=2 forces tickets everywhere.
+    // tickets.  Whole-tensor sums (1024 arrivals on one word: 42 / 47 us) and column sums (47.5 / 53.9 us with the shares of one
+    // output apart and adjacent lanes on adjacent words, 84 us before that; with 48 shares instead of 64 the two are equal) keep
+    // the finishing launch unless THOR_REDUCE_TICKETS=2 forces tickets everywhere.
     const char* env = std::getenv("THOR_REDUCE_TICKETS");
     const bool wanted = env == nullptr || std::atoi(env) != 0;
     const bool forced = env != nullptr && std::atoi(env) == 2;
