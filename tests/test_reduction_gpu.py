@@ -351,3 +351,28 @@ def test_config3_full_size_properties(stream):
     # invariants: the sum of the row sums equals the full sum; the value at the argmax is the row max
     assert abs(got_rows.astype(np.float64).sum() - got_full) <= 1e-5 * abs_rows.sum() * 1e-3 + 1e-5 * abs(got_full)
     np.testing.assert_array_equal(x[np.arange(8192), got_arg], got_max)
+
+
+def test_split_reductions_whose_last_share_folds_agree_with_the_finishing_launch(stream, monkeypatch):
+    """THOR_REDUCE_TICKETS=2 makes every split reduction fold inside its main launch (the share that arrives last does it); the
+    default keeps a finishing launch for whole-tensor and column reductions.  Small integers: every order gives the same bits."""
+    rng = np.random.default_rng(21)
+    for dims, axes in (([8192, 1024], [0]), ([4096, 1001], [0]), ([3, 6000, 260], [1]), ([1 << 21], [0])):
+        x = rng.integers(-4, 5, size=dims).astype(np.float32)
+        t = copy_numpy_to_gpu(x, stream, DataType.fp32)
+        results = {}
+        for mode in ("0", "2"):
+            monkeypatch.setenv("THOR_REDUCE_TICKETS", mode)
+            stamped = ph.CubReduction(ph.CubReductionOp.Sum, axes, DataType.fp32).stamp(t, stream)
+            assert ("last_share_folds" in stamped.get_kernel_variant()) == (mode == "2"), stamped.get_kernel_variant()
+            for _ in range(2):  # the ticket words are left at zero for the next run
+                stamped.run()
+            arg = ph.CubArgReduction(ph.CubArgReductionOp.ArgMax, axes, value_output_dtype=DataType.fp32).stamp(t, stream)
+            arg.run()
+            results[mode] = (gpu_to_f32(stamped.get_output_tensor(), stream), copy_gpu_to_numpy(arg.get_index_output_tensor(), stream))
+        want = oracle.reduce_f64(oracle.SUM, x, oracle.FP32, axes).astype(np.float32)
+        np.testing.assert_array_equal(results["0"][0].reshape(want.shape), want)
+        np.testing.assert_array_equal(results["2"][0].reshape(want.shape), want)
+        want_idx, _ = oracle.arg_reduce(oracle.ARGMAX, x, oracle.FP32, axes)
+        np.testing.assert_array_equal(results["0"][1].astype(np.uint64).reshape(want_idx.shape), want_idx)
+        np.testing.assert_array_equal(results["2"][1].astype(np.uint64).reshape(want_idx.shape), want_idx)
