@@ -225,29 +225,52 @@ def test_top_k_pairs_with_many_equal_keys(stream, dtype, largest):
         check_top_k(keys, dtype, k, largest, got, got_values)
 
 
-# the key kinds of two and four bytes (unsigned, signed, float), each with roomy and with overflowing regions, orders alternating
-CANDIDATE_CASES = [(d, (i + j) % 2 == 0, r) for i, d in enumerate([DataType.uint16, DataType.int32, DataType.bf16, DataType.fp32, DataType.fp16])
-                   for j, r in enumerate([None, "1"])]
+# the key kinds of two and four bytes (unsigned, signed, float), each with roomy lists and with lists that overflow, orders alternating
+CANDIDATE_MODES = [("roomy", {}), ("short-list", {"THOR_TOPK_REGION": "1"}), ("short-second-list", {"THOR_TOPK_AMBIGUOUS": "2"}),
+                   ("both-short", {"THOR_TOPK_REGION": "1", "THOR_TOPK_AMBIGUOUS": "2"})]
+CANDIDATE_CASES = [(d, (i + j) % 2 == 0, CANDIDATE_MODES[j][0], CANDIDATE_MODES[j][1])
+                   for i, d in enumerate([DataType.uint16, DataType.int32, DataType.bf16, DataType.fp32, DataType.fp16]) for j in ((0, 1, 2, 3) if d in (DataType.fp32, DataType.uint16) else ((i % 2) * 3, 1 + i % 2))]
 
 
-@pytest.mark.parametrize("dtype,largest,region", CANDIDATE_CASES,
-                         ids=[f"{d.name}-{'largest' if l else 'smallest'}-{'overflowing' if r else 'roomy'}" for d, l, r in CANDIDATE_CASES])
-def test_top_k_over_candidates(stream, monkeypatch, dtype, largest, region):
-    """Long inputs copy the keys at or above a floor taken from a sample (the keys that can still be part of the answer) during
-    the one pass over the input and finish on those candidates; the switch asks for that on short inputs and large k too.  With one entry per wavefront the candidate regions overflow and the passes over
-    the whole input take over: both ways must give the same answer."""
+@pytest.mark.parametrize("dtype,largest,mode,switches", CANDIDATE_CASES,
+                         ids=[f"{d.name}-{'largest' if l else 'smallest'}-{m}" for d, l, m, _ in CANDIDATE_CASES])
+def test_top_k_over_candidates(stream, monkeypatch, dtype, largest, mode, switches):
+    """Long inputs list the keys above a floor taken from a sample (the keys that can still be part of the answer) during the one
+    pass over the input and finish on that list; the switch asks for that on short inputs and large k too (down to no sample: a
+    floor of zero).  A list that is too short makes the last launch walk the whole input, a second list (the keys of the
+    bucket that holds the k-th) that is too short makes its last block walk the candidates again: every way must give the same answer."""
     monkeypatch.setenv("THOR_TOPK_CANDIDATES", "1")
-    if region:
-        monkeypatch.setenv("THOR_TOPK_REGION", region)
+    for name, value in switches.items():
+        monkeypatch.setenv(name, value)
     rng = np.random.default_rng(int(dtype) * 3 + largest)
-    for index, (n, k, levels) in enumerate(((100_003, 1, None), (100_003, 1000, None), (300_001, 4_000, 20), (300_001, 250_000, 20), (65_536, 65_536, None))):
+    for index, (n, k, levels) in enumerate(((100_003, 1, None), (100_003, 1000, None), (300_001, 4_000, 20), (300_001, 250_000, 20), (65_536, 65_536, None),
+                                            (1 << 20, 300, None))):
         keys = random_keys(rng, n, dtype, distinct_levels=levels)
         got, got_values, variant = run_top_k(keys, dtype, k, largest, stream, pairs=True)
-        assert "candidates(" in variant
+        assert "candidates(" in variant and "launches3" in variant
         check_top_k(keys, dtype, k, largest, got, got_values)
-        if index in (1, 3):  # the key-only kernels are the pair kernels without the positions: two of the five sizes
+        if index in (1, 3, 5):  # the key-only kernels are the pair kernels without the positions: three of the six sizes
             got, _, _ = run_top_k(keys, dtype, k, largest, stream)
             check_top_k(keys, dtype, k, largest, got, None)
+
+
+def test_top_k_with_fewer_than_k_keys_above_the_floor(stream):
+    """Many keys equal to the k-th largest: the floor is that key, the list holds the few keys above it and the rest of the
+    answer are keys equal to the floor, from positions noted during the pass (pairs) or written as copies of the key."""
+    rng = np.random.default_rng(5)
+    keys = np.maximum(rng.standard_normal(1 << 21).astype(np.float32), 0)  # half of them zero
+    keys[rng.integers(0, keys.size, 1 << 19)] = np.float32(2.5)               # and about a quarter the same positive value
+    for k, largest in ((700_000, True), (8_000, True), (100, False), (5_000, False)):
+        for pairs in (True, False):
+            if k * 256 > keys.size:
+                continue
+            got, got_values, variant = run_top_k(keys, DataType.fp32, k, largest, stream, pairs=pairs)
+            assert "candidates(" in variant
+            check_top_k(keys, DataType.fp32, k, largest, got, got_values if pairs else None)
+    ints = rng.integers(0, 3, 1 << 20).astype(np.int32)  # three values: every k-th largest has a third of the input equal to it
+    for k in (1, 4_000):
+        got, got_values, _ = run_top_k(ints, DataType.int32, k, True, stream, pairs=True)
+        check_top_k(ints, DataType.int32, k, True, got, got_values)
 
 
 def test_top_k_long_inputs_use_candidates_by_default(stream):

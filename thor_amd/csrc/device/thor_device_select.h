@@ -217,10 +217,10 @@ constexpr int kTopkMaxBins = 2048;
 constexpr int kTopkBinsPerThread = kTopkMaxBins / 256;
 
 // The bucket of a histogram of `numBins` bins (a power of two, at most 2048) that holds the `wanted`-th largest digit (1-based,
-// wanted <= the histogram's total), found by the 256 threads of a block: thread t looks at the 8 bins of descending ranks
+// wanted <= the histogram's total, which `totalOut` receives: the result means nothing otherwise), found by the 256 threads of a block: thread t looks at the 8 bins of descending ranks
 // [8 t, 8 t + 8).  Returns the bucket in every thread; `above` receives the number of entries in larger buckets.  `lds`: 6 words.
 template <typename Bins>
-__device__ __forceinline__ u32 topkPickBucket(const Bins& bins, u32 numBins, u32 wanted, u32* lds, u32& above) {
+__device__ __forceinline__ u32 topkPickBucket(const Bins& bins, u32 numBins, u32 wanted, u32* lds, u32& above, u32* totalOut = nullptr) {
     u32 counts[kTopkBinsPerThread];
     u32 mine = 0;
 #pragma unroll
@@ -231,6 +231,7 @@ __device__ __forceinline__ u32 topkPickBucket(const Bins& bins, u32 numBins, u32
     }
     u32 total;
     u32 before = blockExclusiveSum<256>(mine, lds, total);  // entries in the bins of the threads before this one: all larger
+    if (totalOut) *totalOut = total;
     if (before < wanted && wanted <= before + mine) {
 #pragma unroll
         for (int i = 0; i < kTopkBinsPerThread; ++i) {
@@ -251,62 +252,50 @@ __device__ __forceinline__ u32 topkPickBucket(const Bins& bins, u32 numBins, u32
 // ---- device-wide top-k -----------------------------------------------------------------------------------------------------------
 // Cfg: Raw (u8 / u16 / u32 word of the key), kKind, kBits, kLargest, kTotal, kK (already capped at kTotal, > 0), kPairs, kVec (keys
 // per vector load: 16 bytes' worth when the key tensor is aligned and kTotal divides, else 1), kItems (vectors per thread of the
-// gathering pass).  Temporary storage: 2048 histogram words, then the eight state words below (then the candidates, see there).
+// gathering pass).  Temporary storage: 2048 histogram words, then the sixteen state words below (then the candidates, see there).
 struct TopkState {
     u32 prefix;     // the digits fixed so far, in place
     u32 remaining;  // the rank (1-based) of the wanted key among the keys that match the prefix
     u32 taken;      // output slots handed out to keys above the threshold
     u32 ties;       // keys equal to the threshold seen so far by the gathering pass
-    u32 overflow;   // candidate regions (below) were too small for this input: the passes over the whole input take over
-    u32 arrived;    // blocks of the running counting pass that have added their histogram (zero between passes)
-    u32 floor;      // candidates (below): keys whose image is at least this can still be part of the answer
-    u32 floorRemaining;  // while the floor is being fixed digit by digit over the sample: what `remaining` is for the prefix
+    u32 arrived;    // blocks of the running launch that have finished their part (zero between launches)
+    // candidates (below)
+    u32 reserved[2];
+    u32 overflow;    // a region of the candidate list was too short for this input: the third launch walks the whole input
+    u32 floorTies;   // keys equal to F whose positions were asked to be noted
+    u32 ambiguous;   // entries asked for in the second list
+    u32 unused[6];
 };
-constexpr int kTopkStateWords = 8;
+constexpr int kTopkStateWords = 16;
 
 template <typename Cfg>
 __device__ __forceinline__ void topkInit(u32* temp) {
     for (int b = threadIdx.x; b < kTopkMaxBins; b += 256) temp[b] = 0;
-    if (threadIdx.x == 0) {
-        TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-        state->prefix = 0;
-        state->remaining = (u32)Cfg::kK;
-        state->taken = 0;
-        state->ties = 0;
-        state->overflow = 0;
-        state->arrived = 0;
-        state->floor = 0;
-        state->floorRemaining = (u32)Cfg::kK;
-    }
+    if (threadIdx.x < kTopkStateWords) temp[kTopkMaxBins + threadIdx.x] = 0;
+    __syncthreads();
+    if (threadIdx.x == 0) reinterpret_cast<TopkState*>(temp + kTopkMaxBins)->remaining = (u32)Cfg::kK;
 }
 
 // One block of 256 threads: fixes the digit at `shift` and clears the histogram for the next pass.  The histogram words were
 // added to by blocks all over the device: they are read at device scope.
-// FLOOR: the histogram is that of a sample of the input, and the digits of the sample's kK-th largest key are fixed in
-// `floor` / `floorRemaining` instead (at least kK keys of the input lie at or above that key's digits: those of the sample).
-template <typename Cfg, bool FLOOR = false>
+template <typename Cfg>
 __device__ __forceinline__ void topkPick(u32* temp, u32 shift, u32 bits) {
     __shared__ u32 lds[8];
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-    const u32 wanted = FLOOR ? state->floorRemaining : state->remaining, prefix = FLOOR ? state->floor : state->prefix;
+    const u32 wanted = state->remaining, prefix = state->prefix;
     u32 above;
     const u32 bucket = topkPickBucket([&](u32 b) { return loadDeviceWide(&temp[b]); }, 1u << bits, wanted, lds, above);
     for (int b = threadIdx.x; b < kTopkMaxBins; b += 256) temp[b] = 0;
     if (threadIdx.x == 0) {
-        if (FLOOR) {
-            state->floor = prefix | (bucket << shift);
-            state->floorRemaining = wanted - above;
-        } else {
-            state->prefix = prefix | (bucket << shift);
-            state->remaining = wanted - above;
-        }
+        state->prefix = prefix | (bucket << shift);
+        state->remaining = wanted - above;
     }
 }
 
 // The end of a counting pass, called by every block (256 threads) once it has added its histogram to the shared one: the
 // block waits until those additions are acknowledged and counts itself in; the block that counts in last fixes the digit,
 // so the pass needs no launch of its own for that.
-template <typename Cfg, bool FLOOR = false>
+template <typename Cfg>
 __device__ __forceinline__ void topkPickWhenLast(u32* temp, u32 shift, u32 bits) {
     __shared__ u32 last;
     partialsWritten();
@@ -318,7 +307,7 @@ __device__ __forceinline__ void topkPickWhenLast(u32* temp, u32 shift, u32 bits)
         if (last) storeDeviceWide(&state->arrived, 0u);
     }
     __syncthreads();
-    if (last) topkPick<Cfg, FLOOR>(temp, shift, bits);
+    if (last) topkPick<Cfg>(temp, shift, bits);
 }
 
 // Histogram of the `bits`-wide digit at `shift` over the keys whose higher digits equal the prefix.  Blocks stride over the keys
@@ -446,232 +435,575 @@ __device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const 
 }
 
 // ---- candidates ------------------------------------------------------------------------------------------------------------------
-// Long inputs are read in full once instead of once per digit and once more for the output.  A first small launch counts the
-// first digit over a sample of the input (runs of 256 vectors spread evenly, max(2^16, 128 kK) keys), a second one the second
-// digit, and the two leading digits of the sample's kK-th largest key become the floor: at least kK keys of the input lie at or
-// above it, so the answer does too, whatever the sample missed.  The pass over the whole input then counts the first digit of the keys at or above the floor only (the
-// others cannot change which bucket holds the kK-th largest key, nor how many keys lie above it) and copies those keys, the
-// candidates, into the temporary storage; the later digits and the output are taken from the candidates.  With a floor most
-// keys fail one comparison and touch no histogram: the pass streams.  Every wavefront of the copying pass owns a region of
-// kRegion entries (keys as 32-bit words; for pairs the key's position as well) and counts what it wrote: no wavefront asks
-// another for room.  A region that would overflow (a bucket that holds a large part of the input: many equal keys, k close to
-// kTotal) raises `overflow`; the launches over the candidates then walk the whole input instead, with the blocks they have.
-// Cfg additionally: kCompact, kRegion, kRegions (wavefronts of the copying pass), kSampleVectors (a multiple of 256; 0: no
-// sample, the floor stays 0), kSampleRunStride (vectors from one run of the sample to the next).  Temporary storage after the
-// state: kRegions counts, kRegions * kRegion keys, the same number of positions (pairs).
+// Long inputs are read in full once, in three launches:
+//   1. the floor (topkFloor): wavefronts read a sample of the input (runs of 256 vectors spread evenly), every lane keeps the
+//      largest images of eight groups of its vectors, and each wavefront finds, by a bit search over votes, a value that at least
+//      kFloorRank of those maxima reach.  The smallest of the wavefronts' values is the floor F: wavefronts * kFloorRank >= kK
+//      sampled keys lie at or above it, so the kK-th largest key of the input does too, whatever the sample missed.  Block 0
+//      also clears the shared histogram and the state words (no launch of its own for that).
+//   2. the pass over the input (topkCollect): keys above F, the candidates, go into the candidate list (image and position;
+//      every wavefront owns a region of kRegion entries and counts what it wrote), and their distance from F is counted in a
+//      histogram whose buckets grow with the distance (below), so one histogram resolves keys just above F and keys far
+//      above it alike.  Keys equal to F are not listed: they can be any part of the input (many equal keys); the positions
+//      of the first kK of them are noted (pairs).
+//   3. the output (topkFinish): every block picks the bucket that holds the kK-th largest key out of the histogram, or finds
+//      that fewer than kK keys lie above F: then the answer is all candidates plus keys equal to F.  Blocks walk the list;
+//      candidates in buckets above the picked one are written out, those in
+//      the picked bucket go to a second, short list; the block that finishes last selects from that list (digits of the
+//      distance inside the bucket, histogram in LDS) and writes the rest of the output, or the keys equal to F.
+// A region that would overflow (the sample was not representative: inputs that repeat with the sample's period) raises
+// `overflow`: the histogram still counted every candidate, and the third launch walks the whole input instead of the list.
+// A picked bucket that holds more than kAmbiguous keys which are not all equal (clustered keys around the threshold that the
+// sample did not see) makes the last block of the third launch walk the list (the input) by itself: slow, and correct.
+// Cfg additionally: kCompact, kFloorBlocks (blocks of 256 threads of the first launch), kFloorItems (vectors per lane there),
+// kFloorRank, kSampleRunStride (vectors from one run of the sample to the next), kRegion, kRegions (wavefronts of the second
+// launch), kAmbiguous (entries of the second list).
+// Temporary storage after the state: kFloorBlocks * 4 floors, kK positions of keys equal to F, the second list (images,
+// positions), kRegions counts, the candidate list (kRegions * kRegion images, as many positions for pairs).
 template <typename Cfg>
 struct TopkCandidates {
-    __device__ __forceinline__ static u32* counts(u32* temp) { return temp + kTopkMaxBins + kTopkStateWords; }
-    __device__ __forceinline__ static u32* keys(u32* temp) { return counts(temp) + Cfg::kRegions; }
-    __device__ __forceinline__ static u32* positions(u32* temp) { return keys(temp) + (u64)Cfg::kRegions * Cfg::kRegion; }
+    static constexpr u32 kFloors = Cfg::kFloorBlocks * 4;
+    __device__ __forceinline__ static u32* floors(u32* temp) { return temp + kTopkMaxBins + kTopkStateWords; }
+    __device__ __forceinline__ static u32* tiePositions(u32* temp) { return floors(temp) + kFloors; }
+    __device__ __forceinline__ static u32* ambiguousImages(u32* temp) { return tiePositions(temp) + (u32)Cfg::kK; }
+    __device__ __forceinline__ static u32* ambiguousPositions(u32* temp) { return ambiguousImages(temp) + Cfg::kAmbiguous; }
+    __device__ __forceinline__ static u32* counts(u32* temp) { return ambiguousPositions(temp) + Cfg::kAmbiguous; }
+    __device__ __forceinline__ static u32* images(u32* temp) { return counts(temp) + Cfg::kRegions; }
+    __device__ __forceinline__ static u32* positions(u32* temp) { return images(temp) + (u64)Cfg::kRegions * Cfg::kRegion; }
 };
 
-// The digit at `shift` over the keys of the sample whose higher digits equal the floor's; the block that finishes last fixes
-// that digit of the floor.  Launched for the first digit and then for the second: a floor of one digit would make candidates of
-// the whole bucket of that digit, which for keys that crowd a few leading digits is a large part of the input.
+// The bucket of a distance d >= 0 (image - F - 1): d itself below 64, else the position q of d's leading bit and the six bits
+// after it: ((q - 5) << 6) | six bits, at most 1727.  Buckets order like distances.
+__device__ __forceinline__ u32 topkDistanceBucket(u32 d) {
+    if (d < 64u) return d;
+    const u32 q = 31u - (u32)__builtin_clz(d);
+    return ((q - 5u) << 6) | ((d >> (q - 6u)) & 63u);
+}
+// The distances of a bucket: [first, first + 2^bits).
+__device__ __forceinline__ void topkBucketRange(u32 bucket, u32& first, u32& bits) {
+    if (bucket < 64u) {
+        first = bucket;
+        bits = 0;
+        return;
+    }
+    const u32 q = (bucket >> 6) + 5u;
+    bits = q - 6u;
+    first = (64u | (bucket & 63u)) << bits;
+}
+constexpr int kTopkDistanceBuckets = 1728;
+
+// First launch: kFloorBlocks blocks of 256 threads.  A lane reads kFloorItems vectors (a multiple of kTopkFloorGroups) and keeps
+// kTopkFloorGroups maxima.
+constexpr int kTopkFloorGroups = 8;
 template <typename Cfg>
-__device__ __forceinline__ void topkSample(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
+__device__ __forceinline__ void topkFloor(const typename Cfg::Raw* keys, u32* temp) {
     typedef typename Cfg::Raw Raw;
-    constexpr int V = Cfg::kVec;
-    __shared__ u32 bins[kTopkMaxBins];
-    const u32 numBins = 1u << bits;
-    for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
-    __syncthreads();
-    const u32 floorSoFar = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins)->floor;
-    const u32 fixedBits = shift + bits >= 32 ? 0u : (0xffffffffu << (shift + bits));
-    const u32 digitMask = numBins - 1u;
-    constexpr int kUnroll = 4;
-    const u64 stride = (u64)gridDim.x * 256;
-    for (u64 j0 = (u64)blockIdx.x * 256 + threadIdx.x; j0 < Cfg::kSampleVectors; j0 += stride * kUnroll) {
-        Pack<Raw, V> x[kUnroll];
+    constexpr int V = Cfg::kVec, I = Cfg::kFloorItems;
+    if (blockIdx.x == 0) topkInit<Cfg>(temp);  // nothing else touches the histogram or the state during this launch
+    if (Cfg::kFloorRank == 0) {  // no sample: every key lies at or above zero
+        if (threadIdx.x % kWave == 0) TopkCandidates<Cfg>::floors(temp)[blockIdx.x * 4 + threadIdx.x / kWave] = 0;
+        return;
+    }
+    Pack<Raw, V> x[I];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const u64 j = j0 + u * stride;
-            if (j < Cfg::kSampleVectors) x[u].load(keys + ((j / 256) * Cfg::kSampleRunStride + j % 256) * V);
-        }
+    for (int it = 0; it < I; ++it) {
+        // run `run` of the sample lies somewhere in the run-th stretch of kSampleRunStride vectors: evenly spaced runs would
+        // show a sample of few distinct keys when the input repeats itself with a period that the spacing divides
+        const u64 run = (u64)it * Cfg::kFloorBlocks + blockIdx.x;
+        const u64 shift = (u64)(((u32)run * 2654435761u) >> 8) % (Cfg::kSampleRunStride - 255);
+        x[it].load(keys + (run * Cfg::kSampleRunStride + shift + threadIdx.x) * V);
+    }
+    constexpr int G = kTopkFloorGroups;  // maxima per lane: of the vectors it, it + G, ...
+    u32 largest[G];
+    u32 all = 0;
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            if (j0 + u * stride < Cfg::kSampleVectors) {
+    for (int g = 0; g < G; ++g) largest[g] = 0;
 #pragma unroll
-                for (int k = 0; k < V; ++k) {
-                    const u32 image = topkImage<Cfg>(x[u].v[k]);
-                    if ((image & fixedBits) == (floorSoFar & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
-                }
-            }
+    for (int it = 0; it < I; ++it) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const u32 image = topkImage<Cfg>(x[it].v[k]);
+            largest[it % G] = image > largest[it % G] ? image : largest[it % G];
         }
     }
-    __syncthreads();
-    for (u32 b = threadIdx.x; b < numBins; b += 256) {
-        const u32 mine = bins[b];
-        if (mine != 0) atomicAdd(&temp[b], mine);
+#pragma unroll
+    for (int g = 0; g < G; ++g) all = largest[g] > all ? largest[g] : all;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const u32 other = (u32)__shfl_xor((int)all, d, kWave);
+        all = other > all ? other : all;
     }
-    topkPickWhenLast<Cfg, true>(temp, shift, bits);
+    // The largest value, with the bits below the 20 under the wavefront's leading bit left zero, that kFloorRank of the
+    // wavefront's 64 * G maxima reach (zero is reached by all of them).
+    u32 value = 0;
+    if (all != 0) {
+        const int top = 31 - __builtin_clz(all);
+        const int low = top > 19 ? top - 19 : 0;
+        for (int bit = top; bit >= low; --bit) {
+            const u32 trial = value | (1u << bit);
+            u32 reached = 0;
+#pragma unroll
+            for (int g = 0; g < G; ++g) reached += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(largest[g] >= trial));
+            if (reached >= Cfg::kFloorRank) value = trial;
+        }
+    }
+    if (threadIdx.x % kWave == 0) TopkCandidates<Cfg>::floors(temp)[blockIdx.x * 4 + threadIdx.x / kWave] = value;
 }
 
-// Launched with kRegions / 4 blocks of 256 threads: histogram of the first digit (at `shift`) over the keys at or above the
-// floor, and those keys, the candidates of every wavefront, into its region; the block that finishes last fixes the digit.
+// The smallest of the first launch's values, in every thread of a block of 256.  `lds`: 4 words.
 template <typename Cfg>
-__device__ __forceinline__ void topkCompact(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
+__device__ __forceinline__ u32 topkFloorOfAll(const u32* temp, u32* lds) {
+    const u32* floors = TopkCandidates<Cfg>::floors(const_cast<u32*>(temp));
+    u32 smallest = 0xffffffffu;
+    for (u32 i = threadIdx.x; i < TopkCandidates<Cfg>::kFloors; i += 256) {
+        const u32 f = floors[i];
+        smallest = f < smallest ? f : smallest;
+    }
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const u32 other = (u32)__shfl_xor((int)smallest, d, kWave);
+        smallest = other < smallest ? other : smallest;
+    }
+    if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = smallest;
+    __syncthreads();
+    u32 result = lds[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) result = lds[w] < result ? lds[w] : result;
+    __syncthreads();
+    return result;
+}
+
+// Second launch: kRegions / 4 blocks of 256 threads stride over the input in vectors, the next turn's vectors on their way
+// while this turn's are looked at.  Every wavefront owns a region of the list and counts what it wrote: no wavefront asks
+// another for room, and no block waits for anything at its end (the bucket is picked by the third launch).  A wavefront
+// gathers its candidates in LDS and copies them to its region when kTopkStage have come together, as a rule once, at the
+// end: a store in the loop would make the wait for the next turn's vectors a wait for that store as well (the compiler
+// cannot count the memory operations in flight across the branches around the stores, and waits for all of them).
+constexpr u32 kTopkStage = 512;
+template <typename Cfg>
+__device__ __forceinline__ void topkCollect(const typename Cfg::Raw* keys, u32* temp) {
     typedef typename Cfg::Raw Raw;
     constexpr int V = Cfg::kVec, kUnroll = Cfg::kCompactUnroll;
     __shared__ u32 bins[kTopkMaxBins];
-    const u32 numBins = 1u << bits;
-    for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
-    __syncthreads();
+    __shared__ u32 lds[8];
+    __shared__ u32 stageImages[256 / kWave][kTopkStage];
+    __shared__ u32 stagePositions[Cfg::kPairs ? 256 / kWave : 1][Cfg::kPairs ? kTopkStage : 1];
+    constexpr u64 kVectors = Cfg::kTotal / V;
+    const u64 stride = (u64)gridDim.x * 256;
+    u64 v0 = (u64)blockIdx.x * 256 + threadIdx.x;
+    Pack<Raw, V> x[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+        if (v0 + u * stride < kVectors) x[u].loadStream(keys + (v0 + u * stride) * V);
+    for (u32 b = threadIdx.x; b < kTopkMaxBins; b += 256) bins[b] = 0;
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-    const u32 floorImage = state->floor;  // images at or above it are candidates
-    const u32 digitMask = numBins - 1u;
+    const u32 floorImage = topkFloorOfAll<Cfg>(temp, lds);  // (its barriers also order the cleared bins)
     const int lane = threadIdx.x % kWave;
     const u64 lowerLanes = ((u64)1 << lane) - 1;
     const u32 region = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
-    u32* regionKeys = TopkCandidates<Cfg>::keys(temp) + (u64)region * Cfg::kRegion;
+    u32* regionImages = TopkCandidates<Cfg>::images(temp) + (u64)region * Cfg::kRegion;
     u32* regionPositions = TopkCandidates<Cfg>::positions(temp) + (u64)region * Cfg::kRegion;
-    u32 cursor = 0;  // candidates of this wavefront so far: the same in every lane that is still in the loop (lane 0 leaves last)
-    constexpr u64 kVectors = Cfg::kTotal / V;
-    const u64 stride = (u64)gridDim.x * 256;
-    for (u64 v0 = (u64)blockIdx.x * 256 + threadIdx.x; v0 < kVectors; v0 += stride * kUnroll) {
-        Pack<Raw, V> x[kUnroll];
+    u32* tiePositions = TopkCandidates<Cfg>::tiePositions(temp);
+    const int wave = threadIdx.x / kWave;
+    u32 cursor = 0;          // candidates of this wavefront so far: the same in every lane
+    u32 copied = 0;          // of them, in the region already (the rest is in LDS)
+    bool tiesNoted = false;  // kK keys equal to F have been noted (by anyone): no more requests
+    auto copyStage = [&]() {  // (the wavefront's LDS writes and reads are in program order)
+        for (u32 i = lane; i < cursor - copied; i += kWave) {
+            if (copied + i < Cfg::kRegion) {
+                regionImages[copied + i] = stageImages[wave][i];
+                if (Cfg::kPairs) regionPositions[copied + i] = stagePositions[Cfg::kPairs ? wave : 0][Cfg::kPairs ? i : 0];
+            }
+        }
+        copied = cursor;
+    };
+    while ((v0 - lane) < kVectors) {  // (every lane of a wavefront makes the same number of turns)
+        const u64 next = v0 + stride * kUnroll;
+        Pack<Raw, V> y[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
-            if (v0 + u * stride < kVectors) x[u].loadStream(keys + (v0 + u * stride) * V);
+            if (next + u * stride < kVectors) y[u].loadStream(keys + (next + u * stride) * V);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const bool live = v0 + u * stride < kVectors;
             u32 image[V];
-            bool any = false;
+            u32 mask = 0;  // bit k: key k of the vector is a candidate
+            bool tie = false;
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 image[k] = live ? topkImage<Cfg>(x[u].v[k]) : 0u;
-                any |= live && image[k] >= floorImage;
+                mask |= (live && image[k] > floorImage ? 1u : 0u) << k;
+                tie |= Cfg::kPairs && live && image[k] == floorImage;
             }
-            if (__builtin_amdgcn_ballot_w64(any) == 0) continue;  // the usual case when k is small next to the input
+            if (__builtin_amdgcn_ballot_w64(mask != 0 || (tie && !tiesNoted)) == 0) continue;  // the usual case when k is small next to the input
+            // The lanes' candidate counts (0 .. V) turn into places in the region through votes on the counts' bits.
+            const u32 mine = (u32)__builtin_popcount(mask);
+            u32 before = 0, all = 0;
 #pragma unroll
-            for (int k = 0; k < V; ++k) {
-                const bool candidate = live && image[k] >= floorImage;
-                const u64 votes = __builtin_amdgcn_ballot_w64(candidate);
-                if (candidate) {
-                    const u32 slot = cursor + (u32)__builtin_popcountll(votes & lowerLanes);
-                    if (slot < Cfg::kRegion) {
-                        regionKeys[slot] = (u32)x[u].v[k];
-                        if (Cfg::kPairs) regionPositions[slot] = (u32)((v0 + u * stride) * V + k);
+            for (int b = 0; (1 << b) <= V; ++b) {
+                const u64 votes = __builtin_amdgcn_ballot_w64(((mine >> b) & 1u) != 0);
+                before += (u32)__builtin_popcountll(votes & lowerLanes) << b;
+                all += (u32)__builtin_popcountll(votes) << b;
+            }
+            if (cursor - copied + all > kTopkStage) copyStage();
+            u32 slot = cursor - copied + before;
+            cursor += all;
+            while (mask != 0) {  // (as many turns as the lane with most candidates has: one, as a rule)
+                const int k = __builtin_ctz(mask);
+                mask &= mask - 1u;
+                u32 chosen = image[0];
+#pragma unroll
+                for (int j = 1; j < V; ++j) chosen = k == j ? image[j] : chosen;
+                stageImages[wave][slot] = chosen;
+                if (Cfg::kPairs) stagePositions[Cfg::kPairs ? wave : 0][Cfg::kPairs ? slot : 0] = (u32)((v0 + u * stride) * V + k);
+                atomicAdd(&bins[topkDistanceBucket(chosen - floorImage - 1u)], 1u);
+                ++slot;
+            }
+            if (Cfg::kPairs && !tiesNoted) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) {
+                    const bool tieHere = live && image[k] == floorImage;
+                    const u64 tieVotes = __builtin_amdgcn_ballot_w64(tieHere);
+                    if (tieVotes != 0 && !tiesNoted) {
+                        const int first = __builtin_ctzll(tieVotes);
+                        u32 noted = 0;
+                        if (lane == first) noted = atomicAdd(&state->floorTies, (u32)__builtin_popcountll(tieVotes));
+                        noted = (u32)__shfl((int)noted, first, kWave);
+                        if (tieHere) {
+                            const u32 rank = noted + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+                            if (rank < (u32)Cfg::kK) tiePositions[rank] = (u32)((v0 + u * stride) * V + k);
+                        }
+                        tiesNoted = noted >= (u32)Cfg::kK;
                     }
-                    atomicAdd(&bins[(image[k] >> shift) & digitMask], 1u);
                 }
-                cursor += (u32)__builtin_popcountll(votes);
             }
         }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) x[u] = y[u];
+        v0 = next;
     }
+    copyStage();
     if (lane == 0) {
         TopkCandidates<Cfg>::counts(temp)[region] = cursor < Cfg::kRegion ? cursor : Cfg::kRegion;
         if (cursor > Cfg::kRegion) atomicOr(&state->overflow, 1u);
     }
     __syncthreads();
-    for (u32 b = threadIdx.x; b < numBins; b += 256) {
+    for (u32 b = threadIdx.x; b < kTopkDistanceBuckets; b += 256) {
         const u32 mine = bins[b];
         if (mine != 0) atomicAdd(&temp[b], mine);
     }
-    topkPickWhenLast<Cfg>(temp, shift, bits);
 }
 
-// A wavefront's walk over its candidate regions (region = first, first + step, ...): the counts of kTopkRegionBatch regions
-// are loaded together, then the first 64 entries of each (most regions hold fewer), so a region costs no round trip of its
-// own; `visit(word, region, index)` sees every entry once.
+// A walk over the candidates: `visit(image, position)` sees every key above F of the wavefront's share once and in the same
+// order for every run; `position()` is the key's place in the input.  Wavefront `first` of `step`: regions first,
+// first + step, ..., the counts of kTopkRegionBatch regions loaded together, then up to kWalkPerLane * 64 entries of each at a
+// time, so a region costs no round trip of its own.  issue() asks for the first regions' counts, settle() (any time later)
+// takes them; the first entries of the first regions stay in registers from one run to the next.  When a region overflowed,
+// the whole input is walked instead (the same share of it for every run).
 constexpr int kTopkRegionBatch = 4;
-template <typename Cfg, typename Visit>
-__device__ __forceinline__ void topkWalkRegions(const u32* counts, const u32* entries, u32 first, u32 step, const Visit& visit) {
-    const u32 lane = threadIdx.x % kWave;
-    for (u32 r0 = first; r0 < Cfg::kRegions; r0 += step * kTopkRegionBatch) {
-        u32 count[kTopkRegionBatch], word[kTopkRegionBatch];
-#pragma unroll
-        for (int j = 0; j < kTopkRegionBatch; ++j) count[j] = r0 + j * step < Cfg::kRegions ? counts[r0 + j * step] : 0u;
-#pragma unroll
-        for (int j = 0; j < kTopkRegionBatch; ++j)
-            if (lane < count[j]) word[j] = entries[(u64)(r0 + j * step) * Cfg::kRegion + lane];
+template <typename Cfg>
+struct TopkWalk {
+    static constexpr int kPerLane = Cfg::kRegion < Cfg::kWalkPerLane * kWave ? (int)((Cfg::kRegion + kWave - 1) / kWave) : Cfg::kWalkPerLane;
+    const typename Cfg::Raw* keys;
+    u32* temp;
+    u32 first, step, floorImage;
+    u32 overflow;
+    u32 firstCounts[kTopkRegionBatch];
+    u32 firstWords[kTopkRegionBatch][kPerLane];
+    bool haveWords;
+
+    __device__ __forceinline__ void loadCounts(u32 r0, u32 (&count)[kTopkRegionBatch]) const {
+        const u32* counts = TopkCandidates<Cfg>::counts(temp);
 #pragma unroll
         for (int j = 0; j < kTopkRegionBatch; ++j) {
-            if (lane < count[j]) visit(word[j], r0 + j * step, lane);
-            for (u32 i = lane + kWave; i < count[j]; i += kWave) visit(entries[(u64)(r0 + j * step) * Cfg::kRegion + i], r0 + j * step, i);
+            const u32 r = r0 + j * step;
+            count[j] = counts[r < Cfg::kRegions ? r : Cfg::kRegions - 1];
         }
     }
-}
-
-// kCandidateBlocks blocks of 256 threads: histogram of the digit at `shift` over the candidates that match the digits fixed so far.
-template <typename Cfg>
-__device__ __forceinline__ void topkCandidateHistogram(const typename Cfg::Raw* keys, u32* temp, u32 shift, u32 bits) {
-    typedef typename Cfg::Raw Raw;
-    __shared__ u32 bins[kTopkMaxBins];
-    const TopkState* state = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins);
-    if (state->overflow != 0) {  // the regions were too small: count over the whole input, with the blocks of this launch
-        topkHistogram<Cfg>(keys, temp, shift, bits);
-        return;
+    __device__ __forceinline__ void issue(const typename Cfg::Raw* keys_, u32* temp_, u32 first_, u32 step_) {
+        keys = keys_;
+        temp = temp_;
+        first = first_;
+        step = step_;
+        haveWords = false;
+        overflow = reinterpret_cast<const TopkState*>(temp + kTopkMaxBins)->overflow;
+        loadCounts(first, firstCounts);
     }
-    const u32 numBins = 1u << bits;
-    for (u32 b = threadIdx.x; b < numBins; b += 256) bins[b] = 0;
-    __syncthreads();
-    const u32 prefix = state->prefix;
-    const u32 fixedBits = shift + bits >= 32 ? 0u : (0xffffffffu << (shift + bits));
-    const u32 digitMask = numBins - 1u;
-    const u32* counts = TopkCandidates<Cfg>::counts(temp);
-    const u32* candidateKeys = TopkCandidates<Cfg>::keys(temp);
-    topkWalkRegions<Cfg>(counts, candidateKeys, blockIdx.x * (256 / kWave) + threadIdx.x / kWave, gridDim.x * (256 / kWave), [&](u32 word, u32, u32) {
-        const u32 image = topkImage<Cfg>((Raw)word);
-        if ((image & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(image >> shift) & digitMask], 1u);
-    });
-    __syncthreads();
-    for (u32 b = threadIdx.x; b < numBins; b += 256) {
-        const u32 mine = bins[b];
-        if (mine != 0) atomicAdd(&temp[b], mine);
+    __device__ __forceinline__ void settle(u32 floorImage_) {
+        floorImage = floorImage_;
+#pragma unroll
+        for (int j = 0; j < kTopkRegionBatch; ++j) {
+            firstCounts[j] = first + j * step < Cfg::kRegions ? (u32)__builtin_amdgcn_readfirstlane((int)firstCounts[j]) : 0u;
+        }
     }
-    topkPickWhenLast<Cfg>(temp, shift, bits);
-}
+    template <typename Visit>
+    __device__ __forceinline__ void run(const Visit& visit) {
+        const u32 lane = threadIdx.x % kWave;
+        if (overflow != 0) {
+            for (u64 i = (u64)first * kWave + lane; i < Cfg::kTotal; i += (u64)step * kWave) {
+                const u32 image = topkImage<Cfg>(keys[i]);
+                if (image > floorImage) visit(image, [&]() { return (u32)i; });
+            }
+            return;
+        }
+        const u32* images = TopkCandidates<Cfg>::images(temp);
+        const u32* positions = TopkCandidates<Cfg>::positions(temp);
+        for (u32 r0 = first; r0 < Cfg::kRegions; r0 += step * kTopkRegionBatch) {
+            u32 count[kTopkRegionBatch];
+            u32 most = 0;
+            if (r0 == first) {
+#pragma unroll
+                for (int j = 0; j < kTopkRegionBatch; ++j) count[j] = firstCounts[j];
+            } else {
+                loadCounts(r0, count);
+#pragma unroll
+                for (int j = 0; j < kTopkRegionBatch; ++j) count[j] = r0 + j * step < Cfg::kRegions ? (u32)__builtin_amdgcn_readfirstlane((int)count[j]) : 0u;
+            }
+#pragma unroll
+            for (int j = 0; j < kTopkRegionBatch; ++j) most = count[j] > most ? count[j] : most;
+            for (u32 at = 0; at < most; at += kPerLane * kWave) {
+                const bool kept = r0 == first && at == 0;  // these entries stay in registers for the next run
+                u32 word[kTopkRegionBatch][kPerLane];
+                if (!(kept && haveWords)) {
+#pragma unroll
+                    for (int j = 0; j < kTopkRegionBatch; ++j) {
+#pragma unroll
+                        for (int e = 0; e < kPerLane; ++e) {
+                            const u32 i = at + e * kWave + lane;
+                            word[j][e] = i < count[j] ? images[(u64)(r0 + j * step) * Cfg::kRegion + i] : 0u;
+                        }
+                    }
+                }
+                if (kept) {
+#pragma unroll
+                    for (int j = 0; j < kTopkRegionBatch; ++j) {
+#pragma unroll
+                        for (int e = 0; e < kPerLane; ++e) {
+                            if (haveWords) word[j][e] = firstWords[j][e];
+                            else firstWords[j][e] = word[j][e];
+                        }
+                    }
+                    haveWords = true;
+                }
+#pragma unroll
+                for (int j = 0; j < kTopkRegionBatch; ++j) {
+#pragma unroll
+                    for (int e = 0; e < kPerLane; ++e) {
+                        const u32 i = at + e * kWave + lane;
+                        if (i < count[j]) visit(word[j][e], [&]() { return positions[(u64)(r0 + j * step) * Cfg::kRegion + i]; });
+                    }
+                }
+            }
+        }
+    }
+};
 
-// kCandidateBlocks blocks of 256 threads: the output out of the candidates.  Every thread counts the candidates it will write
-// (above the threshold; equal to it), a block scan turns the counts into ranks inside the block, one thread asks for the
-// block's output slots, and a second walk over the same candidates writes them.
+// Third launch: kFinishBlocks blocks of 256 threads.  Every block finds F and picks the bucket out of the second launch's
+// histogram by itself.  Every thread counts the candidates of its share above the picked bucket and those in it, a block scan
+// turns the counts into ranks inside the block, one thread asks for the block's output slots and its room in the second
+// list (requests from all over the grid meet at one address each, and the memory system serves those one after the other:
+// about 10 ns a request), and a second walk over the same candidates puts them into LDS in rank order, from where the block
+// writes them out (a store between the walk's loads would make every later load wait for it).
+constexpr int kTopkAmbiguousPerThread = 8;  // a second list of up to 256 * this entries stays in the last block's registers
+constexpr u32 kTopkStageOut = 1792, kTopkStageAmbiguous = 256;  // entries of a block that go through LDS (the rest: stored from the walk)
 template <typename Cfg>
-__device__ __forceinline__ void topkCandidateGather(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
+__device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const u32* values, u32* temp, typename Cfg::Raw* outKeys, u32* outValues) {
     typedef typename Cfg::Raw Raw;
+    __shared__ u32 stage[Cfg::kPairs ? 2 : 1][kTopkMaxBins];  // [0]: images (later the digit histogram), [1]: positions
     __shared__ u32 lds[8];
     __shared__ u32 bases[2];
+    __shared__ u32 last;
+    static_assert(kTopkStageOut + kTopkStageAmbiguous == kTopkMaxBins, "the stage is the histogram's memory");
+    u32* bins = stage[0];
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
-    if (state->overflow != 0) {  // the regions were too small: gather from the whole input, with the blocks of this launch
-        topkGather<Cfg>(keys, values, temp, outKeys, outValues);
-        return;
+    const u32 firstWave = blockIdx.x * (256 / kWave) + threadIdx.x / kWave, waveStep = gridDim.x * (256 / kWave);
+    TopkWalk<Cfg> share;  // this wavefront's share of the candidates
+    share.issue(keys, temp, firstWave, waveStep);
+    const u32 floorImage = topkFloorOfAll<Cfg>(temp, lds);
+    u32 aboveBucket, listed;
+    const u32 picked = topkPickBucket([&](u32 b) { return temp[b]; }, kTopkMaxBins, (u32)Cfg::kK, lds, aboveBucket, &listed);
+    // fewer than kK keys above F: every candidate belongs to the answer (bucket -1), and `wanted` keys equal to F
+    const int bucket = listed >= (u32)Cfg::kK ? (int)picked : -1;
+    const u32 wanted = listed >= (u32)Cfg::kK ? (u32)Cfg::kK - aboveBucket : (u32)Cfg::kK - listed;
+    u32* ambiguousImages = TopkCandidates<Cfg>::ambiguousImages(temp);
+    u32* ambiguousPositions = TopkCandidates<Cfg>::ambiguousPositions(temp);
+    share.settle(floorImage);
+    {
+        u32 out = 0, ambiguous = 0;
+        share.run([&](u32 image, auto) {
+            const int mine = (int)topkDistanceBucket(image - floorImage - 1u);
+            out += mine > bucket;
+            ambiguous += mine == bucket;
+        });
+        u32 blockOut, blockAmbiguous;
+        u32 outAt = blockExclusiveSum<256>(out, lds, blockOut);                    // ranks inside the block
+        u32 ambiguousAt = blockExclusiveSum<256>(ambiguous, lds, blockAmbiguous);
+        if (blockOut + blockAmbiguous != 0) {  // (the same in every thread)
+            if (threadIdx.x == 0) {
+                bases[0] = blockOut ? atomicAdd(&state->taken, blockOut) : 0u;
+                bases[1] = blockAmbiguous ? atomicAdd(&state->ambiguous, blockAmbiguous) : 0u;
+            }
+            __syncthreads();
+            const u32 outBase = bases[0], ambiguousBase = bases[1];
+            if (out + ambiguous != 0) {
+                share.run([&](u32 image, auto position) {
+                    const int mine = (int)topkDistanceBucket(image - floorImage - 1u);
+                    if (mine > bucket) {
+                        const u32 rank = outAt++;
+                        if (rank < kTopkStageOut) {
+                            stage[0][rank] = image;
+                            if (Cfg::kPairs) stage[Cfg::kPairs ? 1 : 0][rank] = position();
+                        } else {
+                            outKeys[outBase + rank] = topkKeyOfImage<Cfg>(image);
+                            if (Cfg::kPairs) outValues[outBase + rank] = values[position()];
+                        }
+                    } else if (mine == bucket) {
+                        const u32 rank = ambiguousAt++;
+                        if (rank < kTopkStageAmbiguous) {
+                            stage[0][kTopkStageOut + rank] = image;
+                            if (Cfg::kPairs) stage[Cfg::kPairs ? 1 : 0][kTopkStageOut + rank] = position();
+                        } else if (ambiguousBase + rank < Cfg::kAmbiguous) {
+                            storeDeviceWide(&ambiguousImages[ambiguousBase + rank], image);  // read by the last block of this launch
+                            if (Cfg::kPairs) storeDeviceWide(&ambiguousPositions[ambiguousBase + rank], position());
+                        }
+                    }
+                });
+            }
+            __syncthreads();
+            const u32 stagedOut = blockOut < kTopkStageOut ? blockOut : kTopkStageOut;
+            for (u32 i = threadIdx.x; i < stagedOut; i += 256) {
+                outKeys[outBase + i] = topkKeyOfImage<Cfg>(stage[0][i]);
+                if (Cfg::kPairs) outValues[outBase + i] = values[stage[Cfg::kPairs ? 1 : 0][i]];
+            }
+            const u32 stagedAmbiguous = blockAmbiguous < kTopkStageAmbiguous ? blockAmbiguous : kTopkStageAmbiguous;
+            for (u32 i = threadIdx.x; i < stagedAmbiguous; i += 256) {
+                if (ambiguousBase + i < Cfg::kAmbiguous) {
+                    storeDeviceWide(&ambiguousImages[ambiguousBase + i], stage[0][kTopkStageOut + i]);
+                    if (Cfg::kPairs) storeDeviceWide(&ambiguousPositions[ambiguousBase + i], stage[Cfg::kPairs ? 1 : 0][kTopkStageOut + i]);
+                }
+            }
+        }
     }
-    const u32 threshold = state->prefix, wantedTies = state->remaining, firstTieSlot = (u32)Cfg::kK - wantedTies;
-    const u32* counts = TopkCandidates<Cfg>::counts(temp);
-    const u32* candidateKeys = TopkCandidates<Cfg>::keys(temp);
-    const u32* candidatePositions = TopkCandidates<Cfg>::positions(temp);
-    const u32 firstRegion = blockIdx.x * (256 / kWave) + threadIdx.x / kWave, regionStep = gridDim.x * (256 / kWave);
-    u32 above = 0, ties = 0;
-    topkWalkRegions<Cfg>(counts, candidateKeys, firstRegion, regionStep, [&](u32 word, u32, u32) {
-        const u32 image = topkImage<Cfg>((Raw)word);
-        above += image > threshold;
-        ties += image == threshold;
-    });
-    u32 blockAbove, blockTies;
-    u32 aboveAt = blockExclusiveSum<256>(above, lds, blockAbove);
-    u32 tieAt = blockExclusiveSum<256>(ties, lds, blockTies);
-    if (blockAbove + blockTies == 0) return;
+    partialsWritten();
+    __syncthreads();
     if (threadIdx.x == 0) {
-        bases[0] = blockAbove ? atomicAdd(&state->taken, blockAbove) : 0u;
-        bases[1] = blockTies ? atomicAdd(&state->ties, blockTies) : 0u;
+        const u32 before = __hip_atomic_fetch_add(&state->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last = before + 1u == gridDim.x ? 1u : 0u;
+        if (last) storeDeviceWide(&state->arrived, 0u);
     }
     __syncthreads();
-    aboveAt += bases[0];
-    tieAt += bases[1];
-    // the same entries per thread as in the count above: every thread hands out the ranks it counted
-    topkWalkRegions<Cfg>(counts, candidateKeys, firstRegion, regionStep, [&](u32 word, u32 region, u32 index) {
-        const u32 image = topkImage<Cfg>((Raw)word);
-        u32 slot = 0xffffffffu;
-        if (image > threshold) slot = aboveAt++;
-        if (image == threshold) {
-            const u32 rank = tieAt++;
-            if (rank < wantedTies) slot = firstTieSlot + rank;
+    if (!last) return;
+    if (bucket < 0) {
+        // the rest of the answer are keys equal to F, from the positions noted by the second launch
+        const u32* tiePositions = TopkCandidates<Cfg>::tiePositions(temp);
+        for (u32 j = threadIdx.x; j < wanted; j += 256) {
+            outKeys[listed + j] = topkKeyOfImage<Cfg>(floorImage);
+            if (Cfg::kPairs) outValues[listed + j] = values[tiePositions[j]];
         }
+        return;
+    }
+    // The picked bucket holds `held` keys and `wanted` of them belong to the answer: the largest ones, into the output's last
+    // `wanted` slots.  The keys are in the second list, which the block holds in registers when it is short (thread t: entries
+    // t, t + 256, ...), or, when that list was too short, found by walking the candidates again for every step.
+    const u32 held = loadDeviceWide(&state->ambiguous);
+    const bool listedAll = held <= Cfg::kAmbiguous;
+    u32 firstDistance, bits;
+    topkBucketRange((u32)bucket, firstDistance, bits);
+    const u32 firstImage = floorImage + 1u + firstDistance;  // images of the bucket: firstImage + [0, 2^bits)
+    constexpr int E = kTopkAmbiguousPerThread;
+    u32 offsets[E], places[E];
+    const bool inRegisters = listedAll && held <= 256u * E;
+    if (inRegisters) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            offsets[e] = 0;
+            places[e] = 0;
+            const u32 i = (u32)e * 256 + threadIdx.x;
+            if (i < held) {
+                offsets[e] = loadDeviceWide(&ambiguousImages[i]) - firstImage;
+                if (Cfg::kPairs) places[e] = loadDeviceWide(&ambiguousPositions[i]);
+            }
+        }
+    }
+    TopkWalk<Cfg> all;  // every candidate, for this block alone
+    if (!listedAll) {
+        all.issue(keys, temp, threadIdx.x / kWave, 256 / kWave);
+        all.settle(floorImage);
+    }
+    auto walk = [&](const auto& visit) {  // visit(offset inside the bucket, position): the same order for every call
+        if (inRegisters) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                if ((u32)e * 256 + threadIdx.x < held) visit(offsets[e], [&]() { return places[e]; });
+            }
+        } else if (listedAll) {
+            for (u32 i = threadIdx.x; i < held; i += 256) {
+                visit(loadDeviceWide(&ambiguousImages[i]) - firstImage, [&]() { return Cfg::kPairs ? loadDeviceWide(&ambiguousPositions[i]) : 0u; });
+            }
+        } else {
+            all.run([&](u32 image, auto position) {
+                if ((int)topkDistanceBucket(image - floorImage - 1u) == bucket) visit(image - firstImage, position);
+            });
+        }
+    };
+    // digits of the offset, from the top: 11 bits at a time
+    u32 prefix = 0, remaining = wanted;
+    for (int shift = (int)bits; shift > 0;) {
+        const u32 digitBits = shift >= 11 ? 11u : (u32)shift;
+        shift -= (int)digitBits;
+        const u32 fixedBits = shift + digitBits >= 32 ? 0u : (0xffffffffu << (shift + digitBits));
+        __syncthreads();
+        for (u32 b = threadIdx.x; b < (1u << digitBits); b += 256) bins[b] = 0;
+        __syncthreads();
+        walk([&](u32 offset, auto) {
+            if ((offset & fixedBits) == (prefix & fixedBits)) atomicAdd(&bins[(offset >> shift) & ((1u << digitBits) - 1u)], 1u);
+        });
+        __syncthreads();
+        u32 above;
+        const u32 digit = topkPickBucket([&](u32 b) { return bins[b]; }, 1u << digitBits, remaining, lds, above);
+        prefix |= digit << shift;
+        remaining -= above;
+    }
+    // `prefix` is the offset of the kK-th largest key; `remaining` keys equal to it belong to the answer
+    u32 above = 0, ties = 0;
+    walk([&](u32 offset, auto) {
+        above += offset > prefix;
+        ties += offset == prefix;
+    });
+    u32 total;
+    u32 aboveAt = blockExclusiveSum<256>(above, lds, total) + ((u32)Cfg::kK - wanted);
+    u32 tieAt = blockExclusiveSum<256>(ties, lds, total);
+    auto slotOf = [&](u32 offset) {
+        u32 slot = 0xffffffffu;
+        if (offset > prefix) slot = aboveAt++;
+        if (offset == prefix) {
+            const u32 rank = tieAt++;
+            if (rank < remaining) slot = (u32)Cfg::kK - remaining + rank;
+        }
+        return slot;
+    };
+    if (inRegisters) {  // the values of all entries are asked for before the first one is stored
+        u32 slots[E], taken[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            slots[e] = (u32)e * 256 + threadIdx.x < held ? slotOf(offsets[e]) : 0xffffffffu;
+            taken[e] = 0;
+            if (Cfg::kPairs && slots[e] != 0xffffffffu) taken[e] = values[places[e]];
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            if (slots[e] != 0xffffffffu) {
+                outKeys[slots[e]] = topkKeyOfImage<Cfg>(firstImage + offsets[e]);
+                if (Cfg::kPairs) outValues[slots[e]] = taken[e];
+            }
+        }
+        return;
+    }
+    walk([&](u32 offset, auto position) {
+        const u32 slot = slotOf(offset);
         if (slot != 0xffffffffu) {
-            outKeys[slot] = (Raw)word;
-            if (Cfg::kPairs) outValues[slot] = values[candidatePositions[(u64)region * Cfg::kRegion + index]];
+            outKeys[slot] = topkKeyOfImage<Cfg>(firstImage + offset);
+            if (Cfg::kPairs) outValues[slot] = values[position()];
         }
     });
 }

@@ -26,9 +26,8 @@ struct CubSelectionKernels {
     std::shared_ptr<CompiledKernel> first, second, third, fourth;
     // device-wide top-k over candidates: the sample that sets their floor, the copying pass, the histogram and the gathering
     // pass over the candidates
-    std::shared_ptr<CompiledKernel> sample, compact, candidateHistogram, candidateGather;
-    uint32_t candidateBlocks = 0, sampleBlocks = 0;
-    uint64_t sampleVectors = 0;
+    std::shared_ptr<CompiledKernel> floor, collect, finish;  // candidates: the three launches of a long input
+    uint32_t floorBlocks = 0, finishBlocks = 0;
     uint64_t chunks = 0;          // blocks of the counting / scattering / gathering launches; rows for kind 2
     uint32_t histogramBlocks = 0;
     uint32_t threads = 256;
@@ -44,7 +43,7 @@ namespace {
 constexpr uint64_t kRowTopKMaxSegment = 8192, kRowTopKMaxK = 8192;
 constexpr uint32_t kSelectThreads = 256, kSelectRounds = 4;
 constexpr uint32_t kGatherThreads = 256, kGatherItems = 8;  // vectors per thread
-constexpr uint32_t kTopKBins = 2048, kTopKStateWords = 8;
+constexpr uint32_t kTopKBins = 2048, kTopKStateWords = 16;
 constexpr uint64_t kTopKCompactMinItems = 1ull << 20;
 
 size_t roundUp(size_t v, size_t to) { return (v + to - 1) / to * to; }
@@ -265,43 +264,63 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     sel.chunks = (vectors + chunkVectors - 1) / chunkVectors;
     // enough striding blocks to keep every compute unit busy, few enough that the global histogram sees little contention
     sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, 2048));
-    // Long inputs with more than one digit: the pass over the input that counts the first digit also copies the keys that can
-    // still be part of the answer, and the later digits and the output are taken from those candidates (one read of the input
-    // instead of one per digit plus one).  Every wavefront of that pass owns room for its share of a 32nd of the input, at
-    // least 64 entries.
-    // The floor of the candidates comes from a sample of max(2^16, 128 k) keys, in runs of 256 vectors: about k / sample of the
-    // input, and what shares the floor's bucket with it, becomes candidates.  When k is more than a 256th of the input the
-    // candidates would not fit their regions: every digit then reads the whole input.  (Half the sample, twice the candidates,
-    // still fits on average, but not when the input repeats itself: a 2^22-key block tiled to 2^26 keys shows every wavefront
-    // the same few hundred keys sixteen times, and some regions overflowed.)
+    // Long inputs with more than one digit are read once, in three launches (the kernels' file describes them): a floor from a
+    // sample, the pass over the input that lists the keys above the floor, and the output out of that list.
+    // The sample: max(2^17, 128 k) keys in runs of 256 vectors spread evenly, 8 vectors per lane (32 when that takes more than
+    // 256 blocks: fewer and larger wavefront samples, whose values scatter less), 512 maxima per wavefront; every wavefront's
+    // value is reached by floorRank = ceil(k / wavefronts) of its maxima.  Somewhat more than k * items / sample keys become
+    // candidates (the smallest of the wavefronts' values lies below what the whole sample would give); the list has room for
+    // a 32nd of the input.  When k is more than a 256th of the input the candidates would not fit: every digit then reads
+    // the whole input.
     bool compact = sel.digits >= 2 && numItems >= kTopKCompactMinItems && numItems < (1ull << 32) && k * 256 <= numItems;
+    bool forced = false;
     if (const char* env = std::getenv("THOR_TOPK_CANDIDATES")) {  // tuning / test switch: "0" reads the whole input in every pass
         if (std::string(env) == "0") compact = false;
-        if (std::string(env) == "1") compact = sel.digits >= 2 && numItems < (1ull << 32);
+        // "1": also short inputs and large k, down to no sample at all (a floor of zero: every key is a candidate)
+        if (std::string(env) == "1") compact = forced = sel.digits >= 2 && numItems < (1ull << 32);
     }
+    uint64_t floorBlocks = 0, floorRank = 0, sampleRunStride = 0, kFloorItems = 8;
     if (compact) {
-        // Every block of a counting pass ends with additions to the same few words of the shared histogram and a ticket, and those
-        // are served one after the other: 2^26 fp32 keys, k = 64 / 65 536, with 512 / 1024 / 2048 blocks in the pass over the input
-        // 95 / 87 / 97 us and 158 / 133 / 147 us (4096 blocks: regions too small, overflow).
+        const uint64_t sampleKeys = std::max<uint64_t>(uint64_t(1) << 17, 128 * k);
+        if ((sampleKeys + 256 * 8 * vec - 1) / (256 * 8 * vec) > 256) kFloorItems = 32;
+        if (const char* env = std::getenv("THOR_TOPK_SAMPLE_ITEMS")) kFloorItems = std::max(std::atoi(env) / 8, 1) * 8;  // tuning switch
+        const uint64_t blockKeys = 256 * kFloorItems * vec;
+        floorBlocks = std::min<uint64_t>({(sampleKeys + blockKeys - 1) / blockKeys, 512, vectors / (256 * kFloorItems)});
+        if (const char* env = std::getenv("THOR_TOPK_SAMPLE_BLOCKS")) {  // tuning switch
+            floorBlocks = std::min<uint64_t>(std::max<long>(std::atol(env), 1), vectors / (256 * kFloorItems));
+        }
+        if (floorBlocks != 0) {
+            floorRank = (k + floorBlocks * 4 - 1) / (floorBlocks * 4);
+            sampleRunStride = vectors / (floorBlocks * kFloorItems);  // >= 256: the runs do not overlap
+        }
+        if (floorBlocks == 0 || floorRank > 64 * 8 / 2) {  // a value that most of a wavefront's maxima must reach says little
+            compact = forced;
+            floorBlocks = 1;
+            floorRank = 0;  // no sample: the floor is zero
+            sampleRunStride = 0;
+        }
+    }
+    uint64_t regions = 0, regionEntries = 0, ambiguous = 0;
+    if (compact) {
+        // Every block of the pass over the input ends with additions to the same few words of the shared histogram, a request
+        // for room in the list and a ticket, and those are served one after the other: more blocks, longer tail.
         uint64_t limit = 1024;
         if (const char* env = std::getenv("THOR_TOPK_BLOCKS")) limit = std::max<long>(std::atol(env), 1);  // tuning switch
         sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, limit));
+        // every wavefront of that pass owns room for its share of a 32nd of the input, at least 64 entries
+        regions = uint64_t(sel.histogramBlocks) * (256 / 64);
+        regionEntries = std::max<uint64_t>((numItems / 32 + regions - 1) / regions, 64);
+        if (const char* env = std::getenv("THOR_TOPK_REGION")) regionEntries = std::max<long>(std::atol(env), 1);  // test switch: entries per wavefront
+        ambiguous = 16384;
+        if (const char* env = std::getenv("THOR_TOPK_AMBIGUOUS")) ambiguous = std::min<long>(std::max<long>(std::atol(env), 1), 16384);  // test switch: entries of the second list (at most what the last block holds in registers)
+        // the third launch: a wavefront per batch of regions; the same blocks walk the whole input when a region overflowed
+        long finishLimit = 256;
+        if (const char* env = std::getenv("THOR_TOPK_FINISH_BLOCKS")) finishLimit = std::max<long>(std::atol(env), 1);  // tuning switch
+        sel.finishBlocks = static_cast<uint32_t>(std::min<uint64_t>((regions + 15) / 16, static_cast<uint64_t>(finishLimit)));
+        sel.floorBlocks = static_cast<uint32_t>(floorBlocks);
     }
-    const uint64_t sampleRuns = std::min<uint64_t>(std::max<uint64_t>(uint64_t(1) << 16, 128 * k) / vec, vectors) / 256;
-    sel.sampleVectors = sampleRuns * 256 * vec >= k ? sampleRuns * 256 : 0;  // a sample that holds fewer than k keys gives no floor
-    const uint64_t sampleRunStride = sel.sampleVectors ? vectors / sampleRuns : 0;
-    uint64_t sampleBlockLimit = 256;  // 8.4 M sampled keys: 147 us for the whole top-k with 1024 blocks, 133 us with 256
-    if (const char* env = std::getenv("THOR_TOPK_SAMPLE_BLOCKS")) sampleBlockLimit = std::max<long>(std::atol(env), 1);  // tuning switch
-    sel.sampleBlocks = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(sel.sampleVectors / 1024, 1), sampleBlockLimit));
-    const uint64_t regions = uint64_t(sel.histogramBlocks) * (256 / 64);
-    uint64_t regionEntries = std::max<uint64_t>((numItems / 32 + regions - 1) / regions, 64);
-    if (const char* env = std::getenv("THOR_TOPK_REGION")) regionEntries = std::max<long>(std::atol(env), 1);  // test switch: entries per wavefront
-    // few blocks walk the candidates; the same launches walk the whole input when the regions overflowed, so not too few
-    long candidateBlockLimit = 256;
-    if (const char* env = std::getenv("THOR_TOPK_CANDIDATE_BLOCKS")) candidateBlockLimit = std::max<long>(std::atol(env), 1);  // tuning switch
-    sel.candidateBlocks = static_cast<uint32_t>(std::min<uint64_t>((regions + 3) / 4, static_cast<uint64_t>(candidateBlockLimit)));
     sel.tempBytes = (kTopKBins + kTopKStateWords) * 4;
-    if (compact) sel.tempBytes += (regions + regions * regionEntries * (pairs ? 2 : 1)) * 4;
+    if (compact) sel.tempBytes += (floorBlocks * 4 + k + 2 * ambiguous + regions + regions * regionEntries * (pairs ? 2 : 1)) * 4;
     std::ostringstream s;
     s << thor_embed::kDevicePrelude << thor_embed::kSelectKernels;
     s << "namespace gen {\nstruct Cfg {\n";
@@ -309,45 +328,47 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     s << "    static constexpr thor::u64 kTotal = " << numItems << "ull;\n    static constexpr thor::u64 kK = " << k
       << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = " << kGatherThreads
       << ";\n    static constexpr int kItems = " << kGatherItems << ";\n    static constexpr bool kCompact = " << (compact ? "true" : "false")
+      << ";\n    static constexpr int kWalkPerLane = " << (std::getenv("THOR_TOPK_WALK") ? std::max(std::atoi(std::getenv("THOR_TOPK_WALK")), 1) : 2)
       << ";\n    static constexpr int kCompactUnroll = " << (std::getenv("THOR_TOPK_COMPACT_UNROLL") ? std::max(std::atoi(std::getenv("THOR_TOPK_COMPACT_UNROLL")), 1) : 4)
-      << ";\n    static constexpr thor::u32 kRegion = " << regionEntries << "u;\n    static constexpr thor::u32 kRegions = " << regions
-      << "u;\n    static constexpr thor::u64 kSampleVectors = " << sel.sampleVectors << "ull;\n    static constexpr thor::u64 kSampleRunStride = "
-      << sampleRunStride << "ull;\n};\n}  // namespace gen\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_init(thor::u32* temp) { thor::topkInit<gen::Cfg>(temp); }\n";
-    // every counting pass ends with the pick of its digit, by the block that finishes last
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
-         "    thor::topkHistogram<gen::Cfg>(keys, temp, shift, bits);\n}\n";
-    s << "extern \"C\" __global__ __launch_bounds__(" << kGatherThreads
-      << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n"
-         "    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
-    if (compact) {
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_sample(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
-             "    thor::topkSample<gen::Cfg>(keys, temp, shift, bits);\n}\n";
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_compact(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
-             "    thor::topkCompact<gen::Cfg>(keys, temp, shift, bits);\n}\n";
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, "
-             "thor::u32 bits) {\n    thor::topkCandidateHistogram<gen::Cfg>(keys, temp, shift, bits);\n}\n";
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_candidate_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, "
-             "gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n    thor::topkCandidateGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
+      << ";\n    static constexpr thor::u32 kFloorBlocks = " << std::max<uint64_t>(floorBlocks, 1) << "u;\n    static constexpr int kFloorItems = " << kFloorItems
+      << ";\n    static constexpr thor::u32 kFloorRank = " << floorRank << "u;\n    static constexpr thor::u64 kSampleRunStride = " << sampleRunStride
+      << "ull;\n    static constexpr thor::u32 kRegion = " << regionEntries << "u;\n    static constexpr thor::u32 kRegions = " << regions
+      << "u;\n    static constexpr thor::u32 kAmbiguous = " << ambiguous << "u;\n};\n}  // namespace gen\n";
+    if (!compact) {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_init(thor::u32* temp) { thor::topkInit<gen::Cfg>(temp); }\n";
+        // every counting pass ends with the pick of its digit, by the block that finishes last
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_histogram(const gen::Cfg::Raw* keys, thor::u32* temp, thor::u32 shift, thor::u32 bits) {\n"
+             "    thor::topkHistogram<gen::Cfg>(keys, temp, shift, bits);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(" << kGatherThreads
+          << ") void thor_topk_gather(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n"
+             "    thor::topkGather<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
+    } else {
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_floor(const gen::Cfg::Raw* keys, thor::u32* temp) {\n"
+             "    thor::topkFloor<gen::Cfg>(keys, temp);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_collect(const gen::Cfg::Raw* keys, thor::u32* temp) {\n"
+             "    thor::topkCollect<gen::Cfg>(keys, temp);\n}\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_topk_finish(const gen::Cfg::Raw* keys, const thor::u32* values, thor::u32* temp, "
+             "gen::Cfg::Raw* outKeys, thor::u32* outValues) {\n    thor::topkFinish<gen::Cfg>(keys, values, temp, outKeys, outValues);\n}\n";
     }
     const std::string source = s.str();
-    sel.first = compileKernel(source, "thor_topk_init", deviceNum, false);
-    sel.second = compileKernel(source, "thor_topk_histogram", deviceNum, false);
-    sel.fourth = compileKernel(source, "thor_topk_gather", deviceNum, false);
     int launches = 2 + sel.digits;  // init, one counting pass per digit, the gathering pass
-    if (compact) {
-        if (sel.sampleVectors) {
-            sel.sample = compileKernel(source, "thor_topk_sample", deviceNum, false);
-            launches += 2;
-        }
-        sel.compact = compileKernel(source, "thor_topk_compact", deviceNum, false);
-        sel.candidateHistogram = compileKernel(source, "thor_topk_candidate_histogram", deviceNum, false);
-        sel.candidateGather = compileKernel(source, "thor_topk_candidate_gather", deviceNum, false);
+    if (!compact) {
+        sel.first = compileKernel(source, "thor_topk_init", deviceNum, false);
+        sel.second = compileKernel(source, "thor_topk_histogram", deviceNum, false);
+        sel.fourth = compileKernel(source, "thor_topk_gather", deviceNum, false);
+    } else {
+        sel.floor = compileKernel(source, "thor_topk_floor", deviceNum, false);
+        sel.collect = compileKernel(source, "thor_topk_collect", deviceNum, false);
+        sel.finish = compileKernel(source, "thor_topk_finish", deviceNum, false);
+        launches = 3;
     }
     std::ostringstream v;
     v << "top-k radix-select bits" << keyBytes * 8 << " digits" << sel.digits << " vec" << vec << (largest ? " largest" : " smallest") << (pairs ? " pairs" : " keys")
-      << " k" << k << " of " << numItems << (compact ? " candidates(regions=" + std::to_string(regions) + "x" + std::to_string(regionEntries) + ")" : std::string())
-      << " launches" << launches << " [" << sel.second->kernelName << "]";
+      << " k" << k << " of " << numItems
+      << (compact ? " candidates(sample=" + std::to_string(floorBlocks * 4) + "x" + std::to_string(64 * kFloorItems * vec) + ",rank=" + std::to_string(floorRank) +
+                        ",regions=" + std::to_string(regions) + "x" + std::to_string(regionEntries) + ")"
+                  : std::string())
+      << " launches" << launches << " [" << (compact ? sel.collect : sel.second)->kernelName << "]";
     sel.variant = v.str();
     return kernels;
 }
@@ -406,32 +427,22 @@ void launchTopK(const CubSelectionKernels& sel, const void* keysIn, const void* 
         sel.first->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, args);
         return;
     }
+    std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut};
+    if (sel.collect) {
+        std::vector<void*> readArgs = {&keysIn, &temp};
+        sel.floor->launch(sel.floorBlocks, 1, 1, 256, raw, readArgs);
+        sel.collect->launch(sel.histogramBlocks, 1, 1, 256, raw, readArgs);
+        sel.finish->launch(sel.finishBlocks, 1, 1, 256, raw, gatherArgs);
+        return;
+    }
     std::vector<void*> initArgs = {&temp};
     sel.first->launch(1, 1, 1, 256, raw, initArgs);
     for (size_t d = 0; d < sel.digitPlan.size(); ++d) {
         uint32_t shift = sel.digitPlan[d].first, bits = sel.digitPlan[d].second;
         std::vector<void*> countArgs = {&keysIn, &temp, &shift, &bits};
-        if (sel.compact && d == 0) {
-            if (sel.sample) {
-                // the floor of the candidates: the two leading digits of the sample's k-th largest key
-                sel.sample->launch(sel.sampleBlocks, 1, 1, 256, raw, countArgs);
-                uint32_t secondShift = sel.digitPlan[1].first, secondBits = sel.digitPlan[1].second;
-                std::vector<void*> secondArgs = {&keysIn, &temp, &secondShift, &secondBits};
-                sel.sample->launch(sel.sampleBlocks, 1, 1, 256, raw, secondArgs);
-            }
-            sel.compact->launch(sel.histogramBlocks, 1, 1, 256, raw, countArgs);
-        } else if (sel.compact) {
-            sel.candidateHistogram->launch(sel.candidateBlocks, 1, 1, 256, raw, countArgs);
-        } else {
-            sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, countArgs);
-        }
+        sel.second->launch(sel.histogramBlocks, 1, 1, 256, raw, countArgs);
     }
-    std::vector<void*> gatherArgs = {&keysIn, &valuesIn, &temp, &keysOut, &valuesOut};
-    if (sel.compact) {
-        sel.candidateGather->launch(sel.candidateBlocks, 1, 1, 256, raw, gatherArgs);
-    } else {
-        sel.fourth->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, gatherArgs);
-    }
+    sel.fourth->launch(static_cast<uint32_t>(sel.chunks), 1, 1, sel.threads, raw, gatherArgs);
 }
 
 void* tempPointer(const Tensor& temp) { return const_cast<Tensor&>(temp).getMemPtr(); }
