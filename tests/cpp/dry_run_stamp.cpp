@@ -297,6 +297,17 @@ static int runAll() {
         }
         Tensor rows(gpuPlacement, TensorDescriptor(dtype, {256, 4096})), rowBest(gpuPlacement, TensorDescriptor(dtype, {256, 64}));
         primitive(std::string("top-k of rows ") + dtypeName, [&] { (void)prepareCubDeviceSegmentedTopKKeys(rows, rowBest, 256, 4096, 64, CubTopKOrder::Largest); });
+        {  // rows a wavefront cannot hold (one block per row), rows searched bit by bit (more than 64 keys wanted), with values
+            Tensor longRows(gpuPlacement, TensorDescriptor(dtype, {16, 8192})), longBest(gpuPlacement, TensorDescriptor(dtype, {16, 100}));
+            Tensor rowValues(gpuPlacement, TensorDescriptor(DataType::UINT32, {16, 8192})), bestRowValues(gpuPlacement, TensorDescriptor(DataType::UINT32, {16, 100}));
+            primitive(std::string("top-k pairs of long rows ") + dtypeName,
+                      [&] { (void)prepareCubDeviceSegmentedTopKPairs(longRows, longBest, rowValues, bestRowValues, 16, 8192, 100, CubTopKOrder::Smallest); });
+            primitive(std::string("top-k pairs of rows, k = 100 ") + dtypeName,
+                      [&] { (void)prepareCubDeviceSegmentedTopKPairs(longRows, longBest, rowValues, bestRowValues, 16, 4096, 100, CubTopKOrder::Largest); });
+            Tensor manyKeys(gpuPlacement, TensorDescriptor(dtype, {uint64_t(1) << 24})), manyBest(gpuPlacement, TensorDescriptor(dtype, {uint64_t(1) << 16}));
+            primitive(std::string("top-k keys ") + dtypeName + ", 65536 of 2^24",
+                      [&] { (void)prepareCubDeviceTopKKeys(manyKeys, manyBest, uint64_t(1) << 24, uint64_t(1) << 16, CubTopKOrder::Largest); });
+        }
         Tensor x(gpuPlacement, TensorDescriptor(dtype, {uint64_t(1) << 20})), y(gpuPlacement, TensorDescriptor(dtype, {uint64_t(1) << 20}));
         Tensor flags(gpuPlacement, TensorDescriptor(DataType::UINT8, {uint64_t(1) << 20})), count(gpuPlacement, TensorDescriptor(DataType::UINT32, {1}));
         primitive(std::string("select-flagged ") + dtypeName, [&] { (void)prepareCubDeviceSelectFlagged(x, flags, y, count, uint64_t(1) << 20); });

@@ -472,25 +472,30 @@ struct TopkCandidates {
     __device__ __forceinline__ static u32* positions(u32* temp) { return images(temp) + (u64)Cfg::kRegions * Cfg::kRegion; }
 };
 
-// The bucket of a distance d >= 0 (image - F - 1): d itself below 64, else the position q of d's leading bit and the six bits
-// after it: ((q - 5) << 6) | six bits, at most 1727.  Buckets order like distances.
+// The bucket of a distance d >= 0 (image - F - 1), B = Cfg::kBucketBits (3 .. 6): d itself below 2^B, else the position q of
+// d's leading bit and the B bits after it: ((q - B + 1) << B) | those bits, at most (33 - B) * 2^B - 1 < 2048.  Buckets order
+// like distances.  More bits: fewer keys share the bucket of the kK-th largest; fewer bits: fewer histogram words that every
+// block of the second launch adds to at its end.
+template <typename Cfg>
 __device__ __forceinline__ u32 topkDistanceBucket(u32 d) {
-    if (d < 64u) return d;
+    constexpr u32 B = Cfg::kBucketBits;
+    if (d < (1u << B)) return d;
     const u32 q = 31u - (u32)__builtin_clz(d);
-    return ((q - 5u) << 6) | ((d >> (q - 6u)) & 63u);
+    return ((q - B + 1u) << B) | ((d >> (q - B)) & ((1u << B) - 1u));
 }
 // The distances of a bucket: [first, first + 2^bits).
+template <typename Cfg>
 __device__ __forceinline__ void topkBucketRange(u32 bucket, u32& first, u32& bits) {
-    if (bucket < 64u) {
+    constexpr u32 B = Cfg::kBucketBits;
+    if (bucket < (1u << B)) {
         first = bucket;
         bits = 0;
         return;
     }
-    const u32 q = (bucket >> 6) + 5u;
-    bits = q - 6u;
-    first = (64u | (bucket & 63u)) << bits;
+    const u32 q = (bucket >> B) + B - 1u;
+    bits = q - B;
+    first = ((1u << B) | (bucket & ((1u << B) - 1u))) << bits;
 }
-constexpr int kTopkDistanceBuckets = 1728;
 
 // First launch: kFloorBlocks blocks of 256 threads.  A lane reads kFloorItems vectors (a multiple of kTopkFloorGroups) and keeps
 // kTopkFloorGroups maxima.
@@ -656,7 +661,7 @@ __device__ __forceinline__ void topkCollect(const typename Cfg::Raw* keys, u32* 
                 for (int j = 1; j < V; ++j) chosen = k == j ? image[j] : chosen;
                 stageImages[wave][slot] = chosen;
                 if (Cfg::kPairs) stagePositions[Cfg::kPairs ? wave : 0][Cfg::kPairs ? slot : 0] = (u32)((v0 + u * stride) * V + k);
-                atomicAdd(&bins[topkDistanceBucket(chosen - floorImage - 1u)], 1u);
+                atomicAdd(&bins[topkDistanceBucket<Cfg>(chosen - floorImage - 1u)], 1u);
                 ++slot;
             }
             if (Cfg::kPairs && !tiesNoted) {
@@ -688,7 +693,7 @@ __device__ __forceinline__ void topkCollect(const typename Cfg::Raw* keys, u32* 
         if (cursor > Cfg::kRegion) atomicOr(&state->overflow, 1u);
     }
     __syncthreads();
-    for (u32 b = threadIdx.x; b < kTopkDistanceBuckets; b += 256) {
+    for (u32 b = threadIdx.x; b < (33u - Cfg::kBucketBits) << Cfg::kBucketBits; b += 256) {
         const u32 mine = bins[b];
         if (mine != 0) atomicAdd(&temp[b], mine);
     }
@@ -831,7 +836,7 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
     {
         u32 out = 0, ambiguous = 0;
         share.run([&](u32 image, auto) {
-            const int mine = (int)topkDistanceBucket(image - floorImage - 1u);
+            const int mine = (int)topkDistanceBucket<Cfg>(image - floorImage - 1u);
             out += mine > bucket;
             ambiguous += mine == bucket;
         });
@@ -847,13 +852,13 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
             const u32 outBase = bases[0], ambiguousBase = bases[1];
             if (out + ambiguous != 0) {
                 share.run([&](u32 image, auto position) {
-                    const int mine = (int)topkDistanceBucket(image - floorImage - 1u);
+                    const int mine = (int)topkDistanceBucket<Cfg>(image - floorImage - 1u);
                     if (mine > bucket) {
                         const u32 rank = outAt++;
                         if (rank < kTopkStageOut) {
                             stage[0][rank] = image;
                             if (Cfg::kPairs) stage[Cfg::kPairs ? 1 : 0][rank] = position();
-                        } else {
+                        } else if (outBase + rank < (u32)Cfg::kK) {
                             outKeys[outBase + rank] = topkKeyOfImage<Cfg>(image);
                             if (Cfg::kPairs) outValues[outBase + rank] = values[position()];
                         }
@@ -872,8 +877,10 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
             __syncthreads();
             const u32 stagedOut = blockOut < kTopkStageOut ? blockOut : kTopkStageOut;
             for (u32 i = threadIdx.x; i < stagedOut; i += 256) {
-                outKeys[outBase + i] = topkKeyOfImage<Cfg>(stage[0][i]);
-                if (Cfg::kPairs) outValues[outBase + i] = values[stage[Cfg::kPairs ? 1 : 0][i]];
+                if (outBase + i < (u32)Cfg::kK) {  // (always, when the histogram and the list agree)
+                    outKeys[outBase + i] = topkKeyOfImage<Cfg>(stage[0][i]);
+                    if (Cfg::kPairs) outValues[outBase + i] = values[stage[Cfg::kPairs ? 1 : 0][i]];
+                }
             }
             const u32 stagedAmbiguous = blockAmbiguous < kTopkStageAmbiguous ? blockAmbiguous : kTopkStageAmbiguous;
             for (u32 i = threadIdx.x; i < stagedAmbiguous; i += 256) {
@@ -898,7 +905,10 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
         const u32* tiePositions = TopkCandidates<Cfg>::tiePositions(temp);
         for (u32 j = threadIdx.x; j < wanted; j += 256) {
             outKeys[listed + j] = topkKeyOfImage<Cfg>(floorImage);
-            if (Cfg::kPairs) outValues[listed + j] = values[tiePositions[j]];
+            if (Cfg::kPairs) {
+                const u32 position = tiePositions[j];
+                outValues[listed + j] = values[position < Cfg::kTotal ? position : 0];
+            }
         }
         return;
     }
@@ -908,7 +918,7 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
     const u32 held = loadDeviceWide(&state->ambiguous);
     const bool listedAll = held <= Cfg::kAmbiguous;
     u32 firstDistance, bits;
-    topkBucketRange((u32)bucket, firstDistance, bits);
+    topkBucketRange<Cfg>((u32)bucket, firstDistance, bits);
     const u32 firstImage = floorImage + 1u + firstDistance;  // images of the bucket: firstImage + [0, 2^bits)
     constexpr int E = kTopkAmbiguousPerThread;
     u32 offsets[E], places[E];
@@ -942,7 +952,7 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
             }
         } else {
             all.run([&](u32 image, auto position) {
-                if ((int)topkDistanceBucket(image - floorImage - 1u) == bucket) visit(image - firstImage, position);
+                if ((int)topkDistanceBucket<Cfg>(image - floorImage - 1u) == bucket) visit(image - firstImage, position);
             });
         }
     };
@@ -988,11 +998,11 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
         for (int e = 0; e < E; ++e) {
             slots[e] = (u32)e * 256 + threadIdx.x < held ? slotOf(offsets[e]) : 0xffffffffu;
             taken[e] = 0;
-            if (Cfg::kPairs && slots[e] != 0xffffffffu) taken[e] = values[places[e]];
+            if (Cfg::kPairs && slots[e] < (u32)Cfg::kK) taken[e] = values[places[e]];
         }
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            if (slots[e] != 0xffffffffu) {
+            if (slots[e] < (u32)Cfg::kK) {
                 outKeys[slots[e]] = topkKeyOfImage<Cfg>(firstImage + offsets[e]);
                 if (Cfg::kPairs) outValues[slots[e]] = taken[e];
             }
@@ -1001,7 +1011,7 @@ __device__ __forceinline__ void topkFinish(const typename Cfg::Raw* keys, const 
     }
     walk([&](u32 offset, auto position) {
         const u32 slot = slotOf(offset);
-        if (slot != 0xffffffffu) {
+        if (slot < (u32)Cfg::kK) {
             outKeys[slot] = topkKeyOfImage<Cfg>(firstImage + offset);
             if (Cfg::kPairs) outValues[slot] = values[position()];
         }

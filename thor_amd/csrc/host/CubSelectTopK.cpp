@@ -19,7 +19,7 @@
 namespace ThorImplementation {
 
 // What one plan launches.  kind 0: select-flagged (count, offsets, scatter); 1: device-wide top-k (init, then one counting pass
-// per digit whose last block picks the digit, gather; `third` is not used); 2: top-k of rows (one launch).  A plan with nothing to do (no items, k == 0) holds no kernels.
+// per digit whose last block picks the digit, gather; `third` is not used; or, for long inputs, floor, collect, finish); 2: top-k of rows (one launch).  A plan with nothing to do (no items, k == 0) holds no kernels.
 struct CubSelectionKernels {
     int kind = 0;
     int deviceNum = 0;
@@ -266,13 +266,15 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     sel.histogramBlocks = static_cast<uint32_t>(std::min<uint64_t>((vectors + 255) / 256, 2048));
     // Long inputs with more than one digit are read once, in three launches (the kernels' file describes them): a floor from a
     // sample, the pass over the input that lists the keys above the floor, and the output out of that list.
-    // The sample: max(2^17, 128 k) keys in runs of 256 vectors spread evenly, 8 vectors per lane (32 when that takes more than
-    // 256 blocks: fewer and larger wavefront samples, whose values scatter less), 512 maxima per wavefront; every wavefront's
+    // The sample: max(2^19, 128 k) keys in runs of 256 vectors spread evenly, 32 vectors per lane (8 when the input is too short
+    // for that many runs of 256 vectors: larger wavefront samples give values that scatter less), 512 maxima per wavefront; every wavefront's
     // value is reached by floorRank = ceil(k / wavefronts) of its maxima.  Somewhat more than k * items / sample keys become
     // candidates (the smallest of the wavefronts' values lies below what the whole sample would give); the list has room for
     // a 32nd of the input.  When k is more than a 256th of the input the candidates would not fit: every digit then reads
     // the whole input.
-    bool compact = sel.digits >= 2 && numItems >= kTopKCompactMinItems && numItems < (1ull << 32) && k * 256 <= numItems;
+    // (k beyond 2^18: the keys that share the k-th largest key's bucket, about a 40th of k, would be more than the last block of
+    // the third launch holds in registers.)
+    bool compact = sel.digits >= 2 && numItems >= kTopKCompactMinItems && numItems < (1ull << 32) && k * 256 <= numItems && k <= (1ull << 18);
     bool forced = false;
     if (const char* env = std::getenv("THOR_TOPK_CANDIDATES")) {  // tuning / test switch: "0" reads the whole input in every pass
         if (std::string(env) == "0") compact = false;
@@ -281,8 +283,8 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     }
     uint64_t floorBlocks = 0, floorRank = 0, sampleRunStride = 0, kFloorItems = 8;
     if (compact) {
-        const uint64_t sampleKeys = std::max<uint64_t>(uint64_t(1) << 17, 128 * k);
-        if ((sampleKeys + 256 * 8 * vec - 1) / (256 * 8 * vec) > 256) kFloorItems = 32;
+        const uint64_t sampleKeys = std::max<uint64_t>(uint64_t(1) << 19, 128 * k);
+        if (vectors / (256 * 32) >= (sampleKeys + 256 * 32 * vec - 1) / (256 * 32 * vec)) kFloorItems = 32;
         if (const char* env = std::getenv("THOR_TOPK_SAMPLE_ITEMS")) kFloorItems = std::max(std::atoi(env) / 8, 1) * 8;  // tuning switch
         const uint64_t blockKeys = 256 * kFloorItems * vec;
         floorBlocks = std::min<uint64_t>({(sampleKeys + blockKeys - 1) / blockKeys, 512, vectors / (256 * kFloorItems)});
@@ -328,8 +330,9 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
     s << "    static constexpr thor::u64 kTotal = " << numItems << "ull;\n    static constexpr thor::u64 kK = " << k
       << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = " << kGatherThreads
       << ";\n    static constexpr int kItems = " << kGatherItems << ";\n    static constexpr bool kCompact = " << (compact ? "true" : "false")
+      << ";\n    static constexpr thor::u32 kBucketBits = " << (std::getenv("THOR_TOPK_BUCKET_BITS") ? std::min(std::max(std::atoi(std::getenv("THOR_TOPK_BUCKET_BITS")), 3), 6) : 6)
       << ";\n    static constexpr int kWalkPerLane = " << (std::getenv("THOR_TOPK_WALK") ? std::max(std::atoi(std::getenv("THOR_TOPK_WALK")), 1) : 2)
-      << ";\n    static constexpr int kCompactUnroll = " << (std::getenv("THOR_TOPK_COMPACT_UNROLL") ? std::max(std::atoi(std::getenv("THOR_TOPK_COMPACT_UNROLL")), 1) : 4)
+      << ";\n    static constexpr int kCompactUnroll = " << (std::getenv("THOR_TOPK_COMPACT_UNROLL") ? std::max(std::atoi(std::getenv("THOR_TOPK_COMPACT_UNROLL")), 1) : 2)
       << ";\n    static constexpr thor::u32 kFloorBlocks = " << std::max<uint64_t>(floorBlocks, 1) << "u;\n    static constexpr int kFloorItems = " << kFloorItems
       << ";\n    static constexpr thor::u32 kFloorRank = " << floorRank << "u;\n    static constexpr thor::u64 kSampleRunStride = " << sampleRunStride
       << "ull;\n    static constexpr thor::u32 kRegion = " << regionEntries << "u;\n    static constexpr thor::u32 kRegions = " << regions
