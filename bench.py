@@ -546,6 +546,128 @@ def summarize_counters(dbs, bench_json=None):
             print(f"{grid:11d} {row['us']:9.1f} " + " ".join(cells) + f"  {_short(kernel, 44)} <- {_line_of(kernel, tags)}")
 
 
+
+def run_experiment(name):
+    """A/B experiments whose tables are kept under profiles/ (each prints plain text; medians of 7 samples of 4 launches, HIP events on
+    the launch stream).  c1_address_stagger: config 1 at 2^28 with the four operands and the output shifted inside their allocations,
+    so that a wavefront's four loads do not start on the same offset of their 4 KiB pages ("c1_address_stagger:BYTES": that step only).  c1_operand_streams: the same size with 1,
+    2, 3 and 4 operands read per element written, a plain sum against config 1's arithmetic.  c1_sigmoid_exponentials: config 1 with
+    the stable sigmoid's two exponentials as written against the shared one.  stage_overlap: plans with independent branches on
+    helper streams (THOR_STAGE_OVERLAP=1) against one lane."""
+    from thor_amd import physical as ph
+    from thor_amd.dtypes import DataType
+    from thor_amd.physical import Expression as ex
+    from thor_amd.runtime import Event
+
+    name, _, only = name.partition(":")  # "c1_address_stagger:4352" runs the one line with steps of that many bytes (for counter runs)
+    stream = ph.Stream(0)
+
+    class RawStream:
+        handle = stream.handle
+
+    gpu = ph.Placement(ph.DeviceType.gpu, 0)
+
+    def time_runs(runs, launches=4, samples=7):
+        for run in runs:
+            run()
+        stream.synchronize()
+        taken = []
+        for _ in range(samples):
+            first, last = Event(), Event()
+            first.record(RawStream)
+            for k in range(launches):
+                runs[k % len(runs)]()
+            last.record(RawStream)
+            last.synchronize()
+            taken.append(first.elapsed_ms(last) / launches)
+        return float(np.median(taken))
+
+    def device_tensor(values, dtype=DataType.fp32):
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        host = ph.PhysicalTensor(ph.Placement(ph.DeviceType.cpu), ph.PhysicalTensor.Descriptor(DataType.fp32, list(values.shape)))
+        host.numpy()[...] = values
+        device = ph.PhysicalTensor(gpu, ph.PhysicalTensor.Descriptor(dtype, list(values.shape)))
+        device.copy_from_async(host, stream)
+        stream.synchronize()
+        return device
+
+    n = 1 << 28
+    if name in ("c1_address_stagger", "c1_operand_streams", "c1_sigmoid_exponentials"):
+        room = 1 << 22  # 16 MiB of slack per tensor
+        base = {k: ph.PhysicalTensor(gpu, ph.PhysicalTensor.Descriptor(DataType.fp32, [n + room])) for k in "abcdo"}
+        for t in base.values():
+            t.memset_async(0, stream)
+        stream.synchronize()
+        a, b, c, d = (ex.input(k) for k in "abcd")
+        c1 = (a * b + c) * d.sigmoid()
+
+        def line(label, expression, offsets, reads):
+            equation = ex.compile(ex.outputs({"o": expression}), 0)
+            names = "abcd"[:reads]
+            views = {k: base[k].alias_view([n], [1], element_offset=offsets[i]) for i, k in enumerate(names)}
+            out = base["o"].alias_view([n], [1], element_offset=offsets[4])
+            plan = equation.stamp(views, stream, preallocated_outputs={"o": out})
+            ms = time_runs([plan.run])
+            moved = 4 * (reads + 1) * n
+            print(f"{label:44s} {ms * 1000:8.1f} us  {moved / ms / 1e6:7.0f} GB/s  {moved / ms / 1e6 / 8000:.3f}  {plan.stage_descriptions()[0][:50]}", flush=True)
+
+        if name == "c1_address_stagger":
+            print("operand base addresses:", {k: hex(t.mem_ptr()) for k, t in base.items()}, flush=True)
+            page = 1024  # elements per 4 KiB
+            for label, step in (("no stagger", 0), ("256 B steps", 64), ("1 KiB steps", 256), ("4 KiB steps", page), ("16 KiB steps", 4 * page),
+                                ("64 KiB steps", 16 * page), ("256 KiB steps", 64 * page), ("1 MiB steps", 256 * page), ("4 KiB + 256 B steps", page + 64),
+                                ("no stagger (again)", 0)):
+                if not only or int(only) == step * 4:
+                    line(label, c1, [i * step for i in range(5)], 4)
+        elif name == "c1_operand_streams":
+            for round_ in range(2):
+                line(f"round {round_}: a*2 (1 read : 1 write)", a * 2.0, [0] * 5, 1)
+                line(f"round {round_}: a+b (2 : 1)", a + b, [0] * 5, 2)
+                line(f"round {round_}: a+b+c (3 : 1)", a + b + c, [0] * 5, 3)
+                line(f"round {round_}: a+b+c+d (4 : 1)", a + b + c + d, [0] * 5, 4)
+                line(f"round {round_}: (a*b+c)*sigmoid(d) (4 : 1)", c1, [0] * 5, 4)
+        else:
+            for round_ in range(3):
+                os.environ["THOR_SIGMOID_TWO_EXPONENTIALS"] = "1"
+                line(f"round {round_}: two exponentials", c1, [0] * 5, 4)
+                os.environ.pop("THOR_SIGMOID_TWO_EXPONENTIALS")
+                line(f"round {round_}: shared exponential", c1, [0] * 5, 4)
+        return
+    if name == "stage_overlap":
+        def clone(t):
+            c = ph.PhysicalTensor(gpu, ph.PhysicalTensor.Descriptor(t.get_data_type(), t.get_dimensions()))
+            c.copy_from_async(t, stream)
+            stream.synchronize()
+            return c
+
+        def compare(label, plans):
+            taken = {"forked": [], "one lane": []}
+            for _ in range(7):
+                os.environ["THOR_STAGE_OVERLAP"] = "1"
+                taken["forked"].append(time_runs([p.run for p in plans], launches=24, samples=1))
+                os.environ["THOR_STAGE_OVERLAP"] = "0"
+                taken["one lane"].append(time_runs([p.run for p in plans], launches=24, samples=1))
+            print(f"{label:44s} forked {np.median(taken['forked']) * 1e3:8.1f} us   one lane {np.median(taken['one lane']) * 1e3:8.1f} us   "
+                  f"stages {plans[0].stage_kind_names()}", flush=True)
+
+        rng = np.random.default_rng(0)
+        x = device_tensor(rng.standard_normal((8192, 8192), dtype=np.float32))
+        backward = ex.compile(ex.input("x").reduce_max(axis=1, squeeze=[1]), 0).compile_backward(["x"])
+        compare("backward of row max, 8192^2", [backward.stamp({"x": t}, stream) for t in (x, clone(x), clone(x))])
+        y = device_tensor(rng.standard_normal((4096, 8192), dtype=np.float32))
+        two = ex.compile(ex.input("x").reduce_sum(axis=1).reduce_sum(axis=[0, 1]) + ex.input("y").reduce_max(axis=1).reduce_sum(axis=[0, 1]), 0)
+        compare("two large independent reductions", [two.stamp({"x": x, "y": y}, stream)])
+        small = [device_tensor(rng.standard_normal((64, 256 + 8 * k), dtype=np.float32)) for k in range(4)]
+        total = None
+        for k in range(4):
+            term = ex.input(f"s{k}").reduce_sum(axis=1).reduce_sum(axis=[0, 1])
+            total = term if total is None else total + term
+        chains = ex.compile(total, 0)
+        compare("four small independent reduction chains", [chains.stamp({f"s{k}": t for k, t in enumerate(small)}, stream)])
+        return
+    raise SystemExit(f"unknown experiment {name!r}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--summarize-kernel-trace", nargs="+", metavar=("DB", "BENCH_JSON"),
@@ -565,7 +687,13 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="before the timed region, launch a plain copy kernel of known size (uint32->int32 over the same element count: "
                          "4 B read + 4 B written per element) so that hardware counters of a profiled run can be scaled against it")
+    ap.add_argument("--experiment", default="", metavar="NAME",
+                    help="run one A/B experiment instead of the bench and print its table: c1_address_stagger, c1_operand_streams, "
+                         "c1_sigmoid_exponentials or stage_overlap")
     args = ap.parse_args()
+    if args.experiment:
+        run_experiment(args.experiment)
+        return
     if args.summarize_kernel_trace:
         summarize_kernel_trace(*args.summarize_kernel_trace[:2])
         return
