@@ -378,6 +378,33 @@ def test_both_row_kernels_agree(stream, monkeypatch):
     check_top_k(keys, DataType.fp16, 64, True, by_block, values_b, segment_size=4096)
 
 
+@pytest.mark.parametrize("dtype", [DataType.bf16, DataType.fp32, DataType.int16], ids=lambda d: d.name)
+def test_rows_whose_candidates_crowd_one_lane(stream, dtype):
+    """The wavefront-per-row kernel keeps the keys at or above its floor on lane-private stacks: 8 entries of every lane in
+    registers as a rule, up to 16 with a wider search, beyond that the search over all of the row's registers.  Rows of 4 096
+    keys in which one lane (lane l holds keys (64 j + l) * V .. + V of every j) owns 0, 10, 16, 17, 40 ... of the best keys."""
+    rng = np.random.default_rng(int(dtype) + 500)
+    vec = 16 // np.dtype(numpy_carrier(dtype)).itemsize
+    crowds = [0, 10, 16, 17, 40, 12, 9, 64]
+    if dtype in FLOATS:
+        values = rng.standard_normal((len(crowds), 4096)).astype(np.float32) * 100
+    else:
+        values = rng.integers(-30000, 30000, (len(crowds), 4096)).astype(np.int32)
+    for largest in (True, False):
+        rows = values.copy()
+        for row, crowd in enumerate(crowds):
+            lane = 5 + row
+            own = np.array([(64 * j + lane) * vec + e for j in range(4096 // (64 * vec)) for e in range(vec)])  # the lane's 64 positions
+            order = np.argsort(rows[row])
+            best = (order[::-1] if largest else order)[:crowd]  # swap the row's `crowd` best keys into that lane
+            for target, source in zip(own[:crowd], best):
+                rows[row, [target, source]] = rows[row, [source, target]]
+        keys = to_storage(rows, dtype) if dtype in FLOATS else rows.astype(numpy_carrier(dtype))
+        got, got_values, variant = run_top_k(keys, dtype, 64, largest, stream, pairs=True, segment_size=4096)
+        assert "wavefront-per-row" in variant and "floor-candidates" in variant, variant
+        check_top_k(keys, dtype, 64, largest, got, got_values, segment_size=4096)
+
+
 def test_top_k_full_size_against_a_host_partition(stream):
     """2^26 fp32 keys, k = 2^16: the answer's smallest key is the k-th largest of the input and every key above it is present
     (checked with NumPy's partition, which shares nothing with the radix selection)."""

@@ -1095,6 +1095,10 @@ __device__ __forceinline__ void topkRows(const typename Cfg::Raw* keys, const u3
 //     lane that holds most of the large keys) takes the direct form.
 // Cfg additionally: kRows.  Positions inside a row: p = (it * 64 + lane) * kVec + e.
 constexpr int kTopkRowStack = 8;  // candidates per lane
+template <int N>
+struct TopkSlots {
+    static constexpr int value = N;
+};
 
 template <typename Cfg>
 __device__ __forceinline__ u32 topkWaveSum(u32 x) {
@@ -1161,8 +1165,9 @@ __device__ __forceinline__ void topkRowsWave(const typename Cfg::Raw* keys, cons
     // key for every two groups
     constexpr bool kFloor = Cfg::kK <= (u64)kWave && ITEMS % 2 == 0 && Cfg::kSegment >= (u32)(kWave * R / 2) && R > 2 * E;
     constexpr bool kWideEntries = Cfg::kBits == 32;  // an entry of a stack is (image << 16 | slot), or two words for 32-bit images
-    __shared__ u32 stackEntries[kFloor ? kWaves * (E + 1) * kWave : 1];
-    __shared__ u32 stackImages[kFloor && kWideEntries ? kWaves * (E + 1) * kWave : 1];
+    constexpr int kRows = 2 * E;  // a stack's height in LDS: E entries are the rule, up to twice as many take the wider search below
+    __shared__ u32 stackEntries[kFloor ? kWaves * (kRows + 1) * kWave : 1];
+    __shared__ u32 stackImages[kFloor && kWideEntries ? kWaves * (kRows + 1) * kWave : 1];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const u64 row = (u64)blockIdx.x * kWaves + wave;
     if (row >= Cfg::kRows) return;  // the whole wavefront leaves; nothing in this kernel waits for it
@@ -1224,22 +1229,26 @@ __device__ __forceinline__ void topkRowsWave(const typename Cfg::Raw* keys, cons
             if (count >= (u32)Cfg::kK) floorImage = test;
         }
         // every lane pushes its candidates on its own stack; pushes beyond the stack's height land in one more, unused, row
-        u32* entries = stackEntries + wave * (E + 1) * kWave + lane;
-        u32* wideImages = stackImages + (kWideEntries ? wave * (E + 1) * kWave + lane : 0);
+        u32* entries = stackEntries + wave * (kRows + 1) * kWave + lane;
+        u32* wideImages = stackImages + (kWideEntries ? wave * (kRows + 1) * kWave + lane : 0);
         u32 height = 0;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
             if (live(j) && image(j) >= floorImage) {
-                const u32 at = (height < (u32)E ? height : (u32)E) * kWave;
+                const u32 at = (height < (u32)kRows ? height : (u32)kRows) * kWave;
                 entries[at] = kWideEntries ? (u32)j : (image(j) << 16) | (u32)j;
                 if (kWideEntries) wideImages[at] = image(j);
                 ++height;
             }
         }
-        if (__builtin_amdgcn_ballot_w64(height > (u32)E) == 0) {
-            u32 cImage[E], cSlot[E];
+        // The search over the stacks, S entries of every lane in registers.  Almost every row fits E; a row in which some lane
+        // holds more (2 in 1 000 rows of 4 096 normal keys, k = 64) would otherwise take the search over all registers below,
+        // several times the time of a row that fits, and a few such rows near the end of the grid lengthen the whole launch.
+        const auto overStacks = [&](auto slots) {
+            constexpr int S = decltype(slots)::value;
+            u32 cImage[S], cSlot[S];
 #pragma unroll
-            for (int e = 0; e < E; ++e) {
+            for (int e = 0; e < S; ++e) {
                 const u32 entry = (u32)e < height ? entries[e * kWave] : 0u;
                 cImage[e] = kWideEntries ? ((u32)e < height ? wideImages[e * kWave] : 0u) : entry >> 16;
                 cSlot[e] = entry & 0xffffu;
@@ -1258,16 +1267,23 @@ __device__ __forceinline__ void topkRowsWave(const typename Cfg::Raw* keys, cons
                 const u32 test = prefix | (1u << bit);
                 u32 count = 0;
 #pragma unroll
-                for (int e = 0; e < E; ++e) count += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(cImage[e] >= test));
+                for (int e = 0; e < S; ++e) count += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(cImage[e] >= test));
                 if (count >= (u32)Cfg::kK) prefix = test;
             }
             const auto cLive = [&](int e) { return (u32)e < height; };
             u32 above = 0;
 #pragma unroll
-            for (int e = 0; e < E; ++e) above += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(cLive(e) && cImage[e] > prefix));
-            topkRowEmit<Cfg, E>([&](int e) { return cImage[e]; },
+            for (int e = 0; e < S; ++e) above += (u32)__builtin_popcountll(__builtin_amdgcn_ballot_w64(cLive(e) && cImage[e] > prefix));
+            topkRowEmit<Cfg, S>([&](int e) { return cImage[e]; },
                                 [&](int e) { return ((cSlot[e] / (u32)V) * kWave + (u32)lane) * (u32)V + cSlot[e] % (u32)V; }, cLive, prefix,
                                 (u32)Cfg::kK - above, rowValuesIn, rowKeys, rowValues);
+        };
+        if (__builtin_amdgcn_ballot_w64(height > (u32)E) == 0) {
+            overStacks(TopkSlots<E>());
+            return;
+        }
+        if (__builtin_amdgcn_ballot_w64(height > (u32)kRows) == 0) {
+            overStacks(TopkSlots<kRows>());
             return;
         }
     }
