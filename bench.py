@@ -280,9 +280,13 @@ def bench_other_configs(only=None):
         for t in values]
     timed("ragged_segment_argmax_fp32", [a_.run for a_ in args], 4 * n, n, args[0].get_kernel_variant())
     per_segment = sums[0].get_output_tensor()
-    timed("ragged_segmented_broadcast_fp32", [(lambda t=t: ph.segmented_broadcast(per_segment, offsets_u32, t, False, stream)) for t in values], 4 * n, n,
-          "thor_segmented_broadcast (output-chunked, LDS window of offsets)")
     rv, ro = ex.input("x.values"), ex.input("x.offsets")
+    # stamped once like every other line (the one-call form, ph.segmented_broadcast, builds its kernel's text on every call: about
+    # 280 us of host time per call, more than the launch takes)
+    spread_plan = ex.compile(ex.outputs({"rows": ex.input("per_segment").segmented_broadcast(ro, segments, rows, width)}), 0)
+    plans = [spread_plan.stamp({"per_segment": per_segment, "x.offsets": offsets_u32}, stream, preallocated_outputs={"rows": t}) for t in values]
+    timed("ragged_segmented_broadcast_fp32", [p_.run for p_ in plans], 4 * n, n, " | ".join(plans[0].stage_descriptions()))
+    del plans, spread_plan
     spread = lambda v: v.segmented_broadcast(ro, segments, rows, width)
     shifted = rv - spread(rv.segment_max(ro, segments, rows, width))
     soft = (shifted.exp() / spread(shifted.exp().segment_sum(ro, segments, rows, width))).with_ragged_runtime_extent(ro, segments, rows, width)
