@@ -138,6 +138,13 @@ static int runAll() {
         stampOne(std::string("rows ") + dtypeName + " standardise",
                  (x - x.reduce_mean({1})) / ((x - x.reduce_mean({1})) * (x - x.reduce_mean({1}))).reduce_mean({1}).sqrt(), inputs, stream);
         stampOne(std::string("columns ") + dtypeName + " sum of a * ln(b)", (x * y.abs().ln()).reduce_sum({0}), inputs, stream);
+        {  // operands that are broadcast along some of the kept axes: their offsets are worked out of the output's number
+            Tensor image(gpuPlacement, TensorDescriptor(dtype, {6, 10, 9, 12})), bias(gpuPlacement, TensorDescriptor(dtype, {10, 1, 1}));
+            Tensor gain(gpuPlacement, TensorDescriptor(dtype, {6, 1, 1, 1}));
+            const Expression v = (Expression::input("image") + Expression::input("bias")) * Expression::input("gain");
+            stampOne(std::string("per-image sums ") + dtypeName + " of (x + bias[C,1,1]) * gain[N,1,1,1]", v.reduce_sum({2, 3}),
+                     {{"image", image}, {"bias", bias}, {"gain", gain}}, stream, "FusedReduction");
+        }
         // backward equations: gradients of fused chains, row kernels that recompute the forward value, winner routing
         Tensor rowGradient(gpuPlacement, TensorDescriptor(dtype, {4096})), fullGradient(gpuPlacement, TensorDescriptor(dtype, {4096, 24}));
         stampBackward(std::string("backward ") + dtypeName + " tanh(a) * b + exp(a)", x.tanh() * y + x.exp(), inputs, fullGradient, stream, "FusedKernel");

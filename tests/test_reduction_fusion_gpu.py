@@ -164,6 +164,45 @@ def test_per_row_and_scalar_operands_in_row_and_column_geometries(gpu):
     np.testing.assert_allclose(outs["colsq"], (y.astype(np.float64) ** 2).sum(axis=0), rtol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [DataType.fp32, DataType.fp16], ids=lambda d: d.name)
+def test_operands_broadcast_along_some_of_the_kept_axes(gpu, dtype):
+    """A [C, 1, 1] bias and a [N, 1, 1, 1] gain under [N, C, H, W] -> [N, C] (reduced over H, W): both depend on the output alone but
+    have fewer elements than outputs, so their offsets are worked out of the output's number; likewise a [1, K] operand under
+    [B, R, K] reduced over R (columns) and a [B, 1, 1] one there."""
+    rng = np.random.default_rng(77)
+    n, c, h, w = 6, 10, 9, 12
+    x = to_storage(rng.standard_normal((n, c, h, w)).astype(np.float32), dtype)
+    bias = to_storage(rng.standard_normal((c, 1, 1)).astype(np.float32), dtype)
+    gain = to_storage(rng.uniform(0.5, 2.0, (n, 1, 1, 1)).astype(np.float32), dtype)
+    ix, ib, ig = ex.input("x"), ex.input("bias"), ex.input("gain")
+    v = (ix + ib) * ig
+    outputs = ex.outputs({"sum": v.reduce_sum(axis=[2, 3], squeeze=True), "peak": v.reduce_max(axis=[2, 3], squeeze=True)})
+    plan, outs = run_staged(outputs, {"x": x, "bias": bias, "gain": gain}, dtype)
+    assert plan.stage_kind_names() == ["FusedReduction"], plan.stage_descriptions()
+    _, outs_s = staged(outputs, {"x": x, "bias": bias, "gain": gain}, dtype)
+    xf, bf, gf = (from_storage(t, dtype).astype(np.float64) for t in (x, bias, gain))
+    if dtype == DataType.fp32:
+        want = (xf + bf) * gf
+    else:  # 16-bit arithmetic rounds every operation
+        step = from_storage(to_storage((xf + bf).astype(np.float32), dtype), dtype).astype(np.float64)
+        want = from_storage(to_storage((step * gf).astype(np.float32), dtype), dtype).astype(np.float64)
+    tolerance = 1e-5 if dtype == DataType.fp32 else 2e-3
+    np.testing.assert_allclose(outs["sum"].reshape(n, c), want.sum(axis=(2, 3)), rtol=tolerance, atol=tolerance * 50)
+    np.testing.assert_allclose(outs["peak"].reshape(n, c), want.max(axis=(2, 3)), rtol=tolerance)
+    np.testing.assert_array_equal(outs["peak"], outs_s["peak"])  # order-independent: the staged plan's bits
+    # columns: [B, R, K] over R with a [1, K] and a [B, 1, 1] operand
+    b, r, k = 5, 700, 24
+    y = rng.standard_normal((b, r, k)).astype(np.float32)
+    per_k = rng.uniform(0.5, 2.0, (1, k)).astype(np.float32)
+    per_b = rng.standard_normal((b, 1, 1)).astype(np.float32)
+    iy, ik, ip = ex.input("y"), ex.input("per_k"), ex.input("per_b")
+    outputs = ex.outputs({"a": (iy * ik + ip).reduce_sum(axis=1, squeeze=True), "b": (iy * iy).reduce_sum(axis=1, squeeze=True)})
+    plan, outs = run_staged(outputs, {"y": y, "per_k": per_k, "per_b": per_b}, DataType.fp32)
+    assert plan.stage_kind_names() == ["FusedReduction"], plan.stage_descriptions()
+    np.testing.assert_allclose(outs["a"].reshape(b, k), (y.astype(np.float64) * per_k + per_b).sum(axis=1), rtol=1e-5, atol=1e-3)
+    np.testing.assert_allclose(outs["b"].reshape(b, k), (y.astype(np.float64) ** 2).sum(axis=1), rtol=1e-5)
+
+
 def test_config5_per_channel_statistics_at_full_size(gpu):
     """fp16 NCHW [64, 256, 56, 56]: per-channel sum and sum of squares (fp32) in one 2-byte-per-element pass."""
     rng = np.random.default_rng(1238)

@@ -62,14 +62,39 @@ Leaf leafKind(const RowFusionContext& ctx, uint32_t node, const Geometry& g) {
     const std::vector<uint64_t>& d = ctx.dims[node];
     if (product(d) == 1) return Leaf::Scalar;
     if (d == g.shape) return Leaf::Vector;
-    // one element per output: extent 1 along every reduced axis and the full extent along every kept axis
+    // a function of the output alone: extent 1 along every reduced axis; along a kept axis the full extent or 1 (broadcast there
+    // too: a [C, 1, 1] bias under [N, C, H, W] -> [N, C])
     if (d.size() > g.shape.size()) return Leaf::No;
     const size_t shift = g.shape.size() - d.size();
     for (size_t a = 0; a < g.shape.size(); ++a) {
         const uint64_t extent = a < shift ? 1 : d[a - shift];
-        if (g.reduced(a) ? extent != 1 : extent != g.shape[a]) return Leaf::No;
+        if (g.reduced(a) ? extent != 1 : (extent != g.shape[a] && extent != 1)) return Leaf::No;
     }
     return Leaf::Kept;
+}
+
+// The offset of a Kept leaf's element as a C expression of `slot`, the output's number (row-major over the kept axes); empty
+// when the leaf has one element per output in that order.
+std::string keptOffsetOf(const std::vector<uint64_t>& d, const Geometry& g) {
+    const size_t shift = g.shape.size() - d.size();
+    bool identity = true;
+    for (size_t a = 0; a < g.shape.size(); ++a)
+        if (!g.reduced(a) && (a < shift ? 1 : d[a - shift]) != g.shape[a]) identity = false;
+    if (identity) return std::string();
+    std::string text;
+    uint64_t after = 1;   // outputs per step of the kept axis at hand: the product of the kept extents after it
+    uint64_t stride = 1;  // the leaf's own stride there: the product of its extents after it
+    for (size_t a = g.shape.size(); a-- > 0;) {
+        const uint64_t extent = a < shift ? 1 : d[a - shift];
+        if (!g.reduced(a)) {
+            if (extent != 1) {
+                text += (text.empty() ? "" : " + ") + ("((slot / " + std::to_string(after) + "ull) % " + std::to_string(g.shape[a]) + "ull) * " + std::to_string(stride) + "ull");
+            }
+            after *= g.shape[a];
+        }
+        stride *= extent;
+    }
+    return text.empty() ? std::string("0") : text;
 }
 
 struct Analysis {
@@ -257,6 +282,7 @@ void tryReductionFusion(RowFusionContext& ctx) {
             ReductionKernelRequest::Source source;
             source.storage = t.getDataType();
             source.kind = kind == Leaf::Vector ? SourceKind::Vector : (kind == Leaf::Scalar ? SourceKind::Scalar : SourceKind::Kept);
+            if (kind == Leaf::Kept) source.keptOffset = keptOffsetOf(ctx.dims[node], g);
             request.sources.push_back(source);
             if (kind == Leaf::Vector) {
                 request.inputAlignmentBytes = std::min(request.inputAlignmentBytes, pointerAlignment(t.getMemPtr()));

@@ -613,7 +613,9 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     s << "    static __device__ __forceinline__ void loadKept(const Sources& s, u64 slot, Kept& kk) {\n";
     for (size_t i = 0; i < sources.size(); ++i) {
         if (sources[i].kind == SourceKind::Scalar) s << "        kk.z" << i << " = s.in" << i << "[0];\n";
-        if (sources[i].kind == SourceKind::Kept) s << "        kk.z" << i << " = s.in" << i << "[slot];\n";
+        if (sources[i].kind == SourceKind::Kept) {
+            s << "        kk.z" << i << " = s.in" << i << "[" << (sources[i].keptOffset.empty() ? std::string("slot") : sources[i].keptOffset) << "];\n";
+        }
     }
     s << "        (void)s; (void)slot; (void)kk;\n    }\n";
 

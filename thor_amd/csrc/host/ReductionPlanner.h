@@ -41,6 +41,9 @@ struct ReductionKernelRequest {
         };
         DataType storage = DataType::FP32;
         Kind kind = Kind::Vector;
+        // Kept sources that are broadcast along some of the kept axes as well (a [C, 1, 1] bias under [N, C, H, W] -> [N, C]): the
+        // element's offset as a C expression of `slot`, the output's number; empty: the output's number itself.
+        std::string keptOffset;
     };
     struct Value {
         CubReductionOp op = CubReductionOp::Sum;

@@ -2,6 +2,7 @@
 #include "Utilities/Expression/SegmentedBroadcastKernel.h"
 
 #include "ReductionPlanner.h"
+#include "Utilities/Cache/LruCache.h"
 #include "Utilities/Common/ScopedGpu.h"
 #include "Utilities/Expression/CompiledEquation.h"
 #include "thorhip_numeric_embed.h"
@@ -103,19 +104,30 @@ std::shared_ptr<StampedSegmentedBroadcast> stampImpl(const Tensor& per_segment_v
     const uint64_t averageRows = std::max<uint64_t>(rows / segments, 1);
     const uint64_t window = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(2 * chunkRows / averageRows + 2), 16), 1024);
 
+    // What decides the kernel's text: calls that stamp on every run (the one-call C entry point) look the built kernel up by
+    // these few numbers instead of writing out and hashing a hundred kilobytes of source.
+    std::ostringstream key;
+    key << stream.getGpuNum() << ' ' << static_cast<int>(dtype) << ' ' << static_cast<int>(offsetType) << ' ' << elementsPerValue << ' ' << rows << ' ' << segments
+        << ' ' << chunkRows << ' ' << vec << ' ' << window << ' ' << normalize_by_segment_length << ' ' << ids;
+    static LruCacheThreadSafe<std::string, std::shared_ptr<CompiledKernel>> builtKernels(1024);
+    std::shared_ptr<CompiledKernel> kernel;
+    if (auto known = builtKernels.get(key.str())) kernel = *known;
     std::ostringstream s;
-    s << thor_embed::kDevicePrelude << thor_embed::kReduceKernels;
-    const std::string typeName = normalize_by_segment_length ? deviceTypeName(dtype) : rawWordName(elementBytes);
-    s << "namespace gen {\nstruct Cfg {\n    typedef " << typeName << " T;\n    typedef " << (offsetType == DataType::UINT64 ? "thor::u64" : "thor::u32")
-      << " OffsetT;\n    static constexpr thor::u64 kE = " << elementsPerValue << "ull;\n    static constexpr thor::u64 kRows = " << rows
-      << "ull;\n    static constexpr thor::u64 kSegments = " << segments << "ull;\n    static constexpr thor::u64 kChunkRows = " << chunkRows
-      << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = 256;\n    static constexpr int kWindow = " << window
-      << ";\n    static constexpr bool kNormalize = " << (normalize_by_segment_length ? "true" : "false")
-      << ";\n    static constexpr bool kViaHalf = " << (dtype == DataType::FP8_E5M2 ? "true" : "false") << ";\n    static constexpr bool kIds = "
-      << (ids ? "true" : "false") << ";\n};\n}  // namespace gen\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void thor_segmented_broadcast(const gen::Cfg::T* values, const void* offsets, gen::Cfg::T* out) "
-         "{\n    thor::broadcastSegments<gen::Cfg>(values, static_cast<const gen::Cfg::OffsetT*>(offsets), out);\n}\n";
-    const std::shared_ptr<CompiledKernel> kernel = compileKernel(s.str(), "thor_segmented_broadcast", stream.getGpuNum(), /*fastContract=*/false);
+    if (!kernel) {
+        s << thor_embed::kDevicePrelude << thor_embed::kReduceKernels;
+        const std::string typeName = normalize_by_segment_length ? deviceTypeName(dtype) : rawWordName(elementBytes);
+        s << "namespace gen {\nstruct Cfg {\n    typedef " << typeName << " T;\n    typedef " << (offsetType == DataType::UINT64 ? "thor::u64" : "thor::u32")
+          << " OffsetT;\n    static constexpr thor::u64 kE = " << elementsPerValue << "ull;\n    static constexpr thor::u64 kRows = " << rows
+          << "ull;\n    static constexpr thor::u64 kSegments = " << segments << "ull;\n    static constexpr thor::u64 kChunkRows = " << chunkRows
+          << "ull;\n    static constexpr int kVec = " << vec << ";\n    static constexpr int kThreads = 256;\n    static constexpr int kWindow = " << window
+          << ";\n    static constexpr bool kNormalize = " << (normalize_by_segment_length ? "true" : "false")
+          << ";\n    static constexpr bool kViaHalf = " << (dtype == DataType::FP8_E5M2 ? "true" : "false") << ";\n    static constexpr bool kIds = "
+          << (ids ? "true" : "false") << ";\n};\n}  // namespace gen\n";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_segmented_broadcast(const gen::Cfg::T* values, const void* offsets, gen::Cfg::T* out) "
+             "{\n    thor::broadcastSegments<gen::Cfg>(values, static_cast<const gen::Cfg::OffsetT*>(offsets), out);\n}\n";
+        kernel = compileKernel(s.str(), "thor_segmented_broadcast", stream.getGpuNum(), /*fastContract=*/false);
+        kernel = builtKernels.getOrCreate(key.str(), [&] { return kernel; });
+    }
 
     std::ostringstream variant;
     variant << (ids ? "segment_ids(chunk_rows=" : "segmented_broadcast(chunk_rows=") << chunkRows << ",window=" << window << ",vec=" << vec << ",grid=" << chunks << ") [" << kernel->kernelName
