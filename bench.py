@@ -556,7 +556,8 @@ def run_experiment(name):
     the launch stream).  c1_address_stagger: config 1 at 2^28 with the four operands and the output shifted inside their allocations,
     so that a wavefront's four loads do not start on the same offset of their 4 KiB pages ("c1_address_stagger:BYTES": that step only).  c1_operand_streams: the same size with 1,
     2, 3 and 4 operands read per element written, a plain sum against config 1's arithmetic.  c1_sigmoid_exponentials: config 1 with
-    the stable sigmoid's two exponentials as written against the shared one.  stage_overlap: plans with independent branches on
+    the stable sigmoid's two exponentials as written against the shared one.  c4_row_kernel_shapes: the two row kernels of config 4 with
+    other lane counts per row than the planner's and with several rows per block taken in turn.  stage_overlap: plans with independent branches on
     helper streams (THOR_STAGE_OVERLAP=1) against one lane."""
     from thor_amd import physical as ph
     from thor_amd.dtypes import DataType
@@ -637,6 +638,40 @@ def run_experiment(name):
                 os.environ.pop("THOR_SIGMOID_TWO_EXPONENTIALS")
                 line(f"round {round_}: shared exponential", c1, [0] * 5, 4)
         return
+    if name == "c4_row_kernel_shapes":
+        rng = np.random.default_rng(0)
+        ix = ex.input("x")
+        e = (ix - ix.reduce_max(axis=1)).exp()
+        centred = ix - ix.reduce_mean(axis=1)
+        lines = (("softmax bf16 -> fp32 [16384, 4096]", ex.compile(e / e.reduce_sum(axis=1), 0), (16384, 4096), DataType.bf16, 6, (64, 128, 256, 512)),
+                 ("normalise fp32 [32768, 1024]", ex.compile(centred / ((centred * centred).reduce_mean(axis=1) + 1e-5).sqrt(), 0), (32768, 1024), DataType.fp32, 8,
+                  (32, 64, 128, 256)))
+        for label, equation, shape, dtype, bytes_per_element, lane_counts in lines:
+            first = device_tensor(rng.standard_normal(shape, dtype=np.float32) * 3, dtype)
+            copies = [first]
+            for _ in range(3):
+                copy = ph.PhysicalTensor(gpu, ph.PhysicalTensor.Descriptor(dtype, list(shape)))
+                copy.copy_from_async(first, stream)
+                copies.append(copy)
+            stream.synchronize()
+            moved = bytes_per_element * shape[0] * shape[1]
+
+            def measure(what, switches):
+                for key, value in switches.items():
+                    os.environ[key] = str(value)
+                plans = [equation.stamp({"x": t}, stream) for t in copies]
+                for key in switches:
+                    os.environ.pop(key)
+                ms = time_runs([p.run for p in plans], launches=8)
+                print(f"{label:36s} {what:28s} {ms * 1000:7.1f} us  {moved / ms / 1e6 / 8000:.3f}  {plans[0].stage_descriptions()[0][:90]}", flush=True)
+
+            measure("the planner's choice", {})
+            for lanes in lane_counts:
+                measure(f"{lanes} lanes per row", {"THOR_ROW_THREADS": lanes})
+            for turns in (2, 4, 8):
+                measure(f"{turns} rows per block in turn", {"THOR_ROW_TURNS": turns})
+            del copies, first
+        return
     if name == "stage_overlap":
         def clone(t):
             c = ph.PhysicalTensor(gpu, ph.PhysicalTensor.Descriptor(t.get_data_type(), t.get_dimensions()))
@@ -693,7 +728,7 @@ def main():
                          "4 B read + 4 B written per element) so that hardware counters of a profiled run can be scaled against it")
     ap.add_argument("--experiment", default="", metavar="NAME",
                     help="run one A/B experiment instead of the bench and print its table: c1_address_stagger, c1_operand_streams, "
-                         "c1_sigmoid_exponentials or stage_overlap")
+                         "c1_sigmoid_exponentials, c4_row_kernel_shapes or stage_overlap")
     args = ap.parse_args()
     if args.experiment:
         run_experiment(args.experiment)
