@@ -74,10 +74,12 @@ SHAPES = [("rows", (300, 64)), ("rows", (5, 4099)), ("rows", (3, 70000)), ("rows
 SCAN_OPS = [ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.product, ScanOp.arg_min, ScanOp.arg_max]
 SCAN_DTYPES = [DataType.uint32, DataType.fp32, DataType.fp16, DataType.bf16]
 SCAN_MODES = [(True, False), (False, False), (True, True), (False, True)]  # (inclusive, reverse)
-# Shape (which chunking the planner picks), dtype and operation (the arithmetic) in full; mode and direction are switches of the
-# same code, so each (shape, dtype, operation) takes one of their four combinations, turning so that every (shape, dtype),
-# (shape, operation) and (dtype, operation) pair meets all four (or, for the six operations, at least three of them).
-ROWS_AND_FLAT = [(k, s, d, o, *SCAN_MODES[(i + j + m) % 4]) for i, (k, s) in enumerate(SHAPES) for j, d in enumerate(SCAN_DTYPES) for m, o in enumerate(SCAN_OPS)]
+# Shape (which chunking the planner picks), dtype and operation (the arithmetic): every pair of the three meets - a shape takes
+# every other (dtype, operation) pair, the halves alternating from shape to shape, so each (dtype, operation) pair runs on two or
+# three shapes (every generated kernel is compiled on the spot, about half a second each: the full product took twice the time).
+# Mode and direction are switches of the same code: each case takes one of their four combinations, turning.
+ROWS_AND_FLAT = [(k, s, d, o, *SCAN_MODES[(i + j + m) % 4]) for i, (k, s) in enumerate(SHAPES) for j, d in enumerate(SCAN_DTYPES) for m, o in enumerate(SCAN_OPS)
+                 if (i + j + m) % 2 == 0]
 
 
 @pytest.mark.parametrize("kind,shape,dtype,op,inclusive,reverse", ROWS_AND_FLAT,
@@ -103,10 +105,10 @@ def test_rows_and_flat_scans(stream, kind, shape, dtype, op, inclusive, reverse)
         assert "passes=scan)" in variant or "passes=scan," in variant  # rows that fit a block need no carries
 
 
-# every (dtype, operation) with two of the four (inclusive, reverse) combinations - opposite ones - one per width of the offsets
-OFFSET_SEGMENTED = [(d, o, *SCAN_MODES[(j + m + 2 * w) % 4], (DataType.uint32, DataType.uint64)[(w + j) % 2])
+# every (dtype, operation) with one of the four (inclusive, reverse) combinations and one of the two offset widths, both turning
+OFFSET_SEGMENTED = [(d, o, *SCAN_MODES[(j + m) % 4], (DataType.uint32, DataType.uint64)[(m + j) % 2])
                     for j, d in enumerate([DataType.uint32, DataType.fp32, DataType.bf16])
-                    for m, o in enumerate([ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.arg_min, ScanOp.arg_max]) for w in range(2)]
+                    for m, o in enumerate([ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.arg_min, ScanOp.arg_max])]
 
 
 @pytest.mark.parametrize("dtype,op,inclusive,reverse,offsets_dtype", OFFSET_SEGMENTED,

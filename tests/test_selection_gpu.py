@@ -229,7 +229,8 @@ def test_top_k_pairs_with_many_equal_keys(stream, dtype, largest):
 CANDIDATE_MODES = [("roomy", {}), ("short-list", {"THOR_TOPK_REGION": "1"}), ("short-second-list", {"THOR_TOPK_AMBIGUOUS": "2"}),
                    ("both-short", {"THOR_TOPK_REGION": "1", "THOR_TOPK_AMBIGUOUS": "2"})]
 CANDIDATE_CASES = [(d, (i + j) % 2 == 0, CANDIDATE_MODES[j][0], CANDIDATE_MODES[j][1])
-                   for i, d in enumerate([DataType.uint16, DataType.int32, DataType.bf16, DataType.fp32, DataType.fp16]) for j in ((0, 1, 2, 3) if d in (DataType.fp32, DataType.uint16) else ((i % 2) * 3, 1 + i % 2))]
+                   for i, d in enumerate([DataType.uint16, DataType.int32, DataType.bf16, DataType.fp32, DataType.fp16])
+                   for j in ((0, 1, 2, 3) if d in (DataType.fp32, DataType.uint16) else ({DataType.int32: 3, DataType.bf16: 2, DataType.fp16: 0}[d],))]
 
 
 @pytest.mark.parametrize("dtype,largest,mode,switches", CANDIDATE_CASES,
@@ -243,13 +244,16 @@ def test_top_k_over_candidates(stream, monkeypatch, dtype, largest, mode, switch
     for name, value in switches.items():
         monkeypatch.setenv(name, value)
     rng = np.random.default_rng(int(dtype) * 3 + largest)
-    for index, (n, k, levels) in enumerate(((100_003, 1, None), (100_003, 1000, None), (300_001, 4_000, 20), (300_001, 250_000, 20), (65_536, 65_536, None),
-                                            (1 << 20, 300, None))):
+    sizes = ((100_003, 1000, None), (300_001, 4_000, 20), (300_001, 250_000, 20), (65_536, 65_536, None), (1 << 20, 300, None))
+    turn = CANDIDATE_CASES.index((dtype, largest, mode, switches))  # three of the five sizes per case, turning (each size compiles six kernels)
+    for index, (n, k, levels) in enumerate(sizes):
+        if (index + turn) % 5 in (1, 3):
+            continue
         keys = random_keys(rng, n, dtype, distinct_levels=levels)
         got, got_values, variant = run_top_k(keys, dtype, k, largest, stream, pairs=True)
         assert "candidates(" in variant and "launches3" in variant
         check_top_k(keys, dtype, k, largest, got, got_values)
-        if index in (1, 3, 5):  # the key-only kernels are the pair kernels without the positions: three of the six sizes
+        if index in (0, 4):  # the key-only kernels are the pair kernels without the positions: two of the five sizes
             got, _, _ = run_top_k(keys, dtype, k, largest, stream)
             check_top_k(keys, dtype, k, largest, got, None)
 
@@ -316,11 +320,11 @@ def test_top_k_zero_k_leaves_the_output_alone(stream):
 
 # Rows a wavefront can hold (at most 64 keys per lane) take the kernel with one wavefront per row: a bit-by-bit search over the
 # keys in registers, or - when at most 64 keys are wanted and every lane holds two groups of vectors - over the few keys at or
-# above a floor taken from the groups' maxima ("floor-candidates"); longer rows take one block per row.  Every key dtype meets every shape, the
+# above a floor taken from the groups' maxima ("floor-candidates"); longer rows take one block per row.  Every key dtype meets five of the seven shapes (every shape at least six of the nine dtypes), the
 # order alternating: rows of two keys, rows no vector divides, almost all keys wanted, rows of one vector per lane, full rows of
 # 4096, the longest rows, many short rows.
 ROW_SHAPES = [(1, 2, 1), (33, 257, 256), (100, 1000, 10), (37, 4096, 64), (6, 8192, 8191), (3000, 64, 8), (50, 3000, 3)]
-ROW_CASES = [(d, (i + j) % 2 == 0, *shape) for i, d in enumerate(KEY_DTYPES) for j, shape in enumerate(ROW_SHAPES)]
+ROW_CASES = [(d, (i + j) % 2 == 0, *shape) for i, d in enumerate(KEY_DTYPES) for j, shape in enumerate(ROW_SHAPES) if (i + j) % 7 not in (2, 5)]
 
 
 def row_kernel_form(dtype, segment_size, k):
