@@ -328,6 +328,9 @@ def test_segments_that_begin_and_end_on_block_boundaries(stream, shape):
     ]
     trailing = int(np.prod(shape[1:])) if len(shape) > 1 else 1
     for partition in partitions:
+        # empty segments after the last one bring every partition to ten offsets: the kernels bake the segment count in, so the
+        # partitions share their compiled kernels
+        partition = partition + [partition[-1]] * (10 - len(partition))
         offsets = np.array(partition, dtype=np.int64)
         toff = upload_offsets(offsets, stream, DataType.uint64)
         for name, op in VALUE_OPS.items():
