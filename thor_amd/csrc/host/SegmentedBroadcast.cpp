@@ -8,6 +8,7 @@
 #include "thorhip_numeric_embed.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
 #include <sstream>
 #include <stdexcept>
@@ -97,9 +98,12 @@ std::shared_ptr<StampedSegmentedBroadcast> stampImpl(const Tensor& per_segment_v
     const uint64_t alignment = std::min(pointerAlignment(per_segment_values.getMemPtr()), pointerAlignment(output.getMemPtr()));
     int vec = static_cast<int>(16 / elementBytes);
     while (vec > 1 && alignment % (static_cast<uint64_t>(vec) * elementBytes) != 0) vec /= 2;
-    // about 128 KiB of output per block, fewer rows while that leaves under eight blocks per CU; always a multiple of 16 rows
-    uint64_t chunkRows = std::max<uint64_t>(pow2Floor(std::max<uint64_t>(131072 / (elementsPerValue * elementBytes), 1)), 16);
+    // about 32 KiB of output per block, fewer rows while that leaves under eight blocks per CU; always a multiple of 16 rows.
+    // (Measured on [65 536, 64] fp32 -> [2^22, 64], 1 GiB written: 16 / 32 / 64 / 128 / 256 / 512 KiB per block take 214 / 179 / 184 / 199 /
+    // 206 / 249 us: a block's search for its first segment and its window of offsets are round trips during which it stores nothing.)
+    uint64_t chunkRows = std::max<uint64_t>(pow2Floor(std::max<uint64_t>(32768 / (elementsPerValue * elementBytes), 1)), 16);
     while (chunkRows > 16 && (rows + chunkRows - 1) / chunkRows < 2048) chunkRows /= 2;
+    if (const char* env = std::getenv("THOR_BROADCAST_CHUNK_ROWS")) chunkRows = std::max<uint64_t>(pow2Floor(std::max<long>(std::atol(env), 16)), 16);  // tuning switch
     const uint64_t chunks = (rows + chunkRows - 1) / chunkRows;
     const uint64_t averageRows = std::max<uint64_t>(rows / segments, 1);
     const uint64_t window = std::min<uint64_t>(std::max<uint64_t>(pow2Ceil(2 * chunkRows / averageRows + 2), 16), 1024);
