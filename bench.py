@@ -554,7 +554,8 @@ def summarize_counters(dbs, bench_json=None):
 def run_experiment(name):
     """A/B experiments whose tables are kept under profiles/ (each prints plain text; medians of 7 samples of 4 launches, HIP events on
     the launch stream).  c1_address_stagger: config 1 at 2^28 with the four operands and the output shifted inside their allocations,
-    so that a wavefront's four loads do not start on the same offset of their 4 KiB pages ("c1_address_stagger:BYTES": that step only).  c1_operand_streams: the same size with 1,
+    so that a wavefront's four loads do not start on the same offset of their 4 KiB pages ("c1_address_stagger:BYTES": that step only).  c1_tensor_spacing: the five tensors
+    inside one allocation, 1 GiB plus a given distance apart ("c1_tensor_spacing:0,4,8": those MiB counts).  c1_operand_streams: the same size with 1,
     2, 3 and 4 operands read per element written, a plain sum against config 1's arithmetic.  c1_sigmoid_exponentials: config 1 with
     the stable sigmoid's two exponentials as written against the shared one.  c4_row_kernel_shapes: the two row kernels of config 4 with
     other lane counts per row than the planner's and with several rows per block taken in turn.  stage_overlap: plans with independent branches on
@@ -600,9 +601,14 @@ def run_experiment(name):
     if name in ("c1_address_stagger", "c1_operand_streams", "c1_sigmoid_exponentials"):
         room = 1 << 22  # 16 MiB of slack per tensor
         base = {k: ph.PhysicalTensor(gpu, ph.PhysicalTensor.Descriptor(DataType.fp32, [n + room])) for k in "abcdo"}
-        for t in base.values():
-            t.memset_async(0, stream)
-        stream.synchronize()
+        # the bench line's data (uniform in [-1, 1), a 2^22 block repeated): tensors of zeros stream 5-6 % faster
+        from thor_amd import _lib
+        block = np.random.default_rng(1234).uniform(-1, 1, 1 << 22).astype(np.float32)
+        for k, t in base.items():
+            source = device_tensor(np.roll(block, ord(k)))
+            for off in range(0, n + room, block.size):
+                _lib.check(_lib.load().thorhip_memcpy_async(t.mem_ptr() + off * 4, source.mem_ptr(), block.nbytes, 3, stream.handle), "d2d")
+            stream.synchronize()
         a, b, c, d = (ex.input(k) for k in "abcd")
         c1 = (a * b + c) * d.sigmoid()
 
@@ -637,6 +643,29 @@ def run_experiment(name):
                 line(f"round {round_}: two exponentials", c1, [0] * 5, 4)
                 os.environ.pop("THOR_SIGMOID_TWO_EXPONENTIALS")
                 line(f"round {round_}: shared exponential", c1, [0] * 5, 4)
+        return
+    if name == "c1_tensor_spacing":
+        # the five tensors of config 1 inside one allocation, a fixed distance apart: what the distance between the streams does
+        a, b, c, d = (ex.input(k) for k in "abcd")
+        equation = ex.compile(ex.outputs({"o": (a * b + c) * d.sigmoid()}), 0)
+        room = 1 << 24
+        pool = ph.PhysicalTensor(gpu, ph.PhysicalTensor.Descriptor(DataType.fp32, [5 * (n + room)]))
+        from thor_amd import _lib
+        block = device_tensor(np.random.default_rng(1234).uniform(-1, 1, 1 << 22).astype(np.float32))
+        for off in range(0, 5 * (n + room), 1 << 22):
+            _lib.check(_lib.load().thorhip_memcpy_async(pool.mem_ptr() + off * 4, block.mem_ptr(), 4 << 22, 3, stream.handle), "d2d")
+        stream.synchronize()
+        print("pool at", hex(pool.mem_ptr()), flush=True)
+        spacings = (0, 128, 256, 1024, 4096, 65536, 1 << 20, 2 << 20, 4 << 20, 20 << 20, (20 << 20) + 4096, 33 << 20, 48 << 20, 0)
+        if only:
+            spacings = tuple(int(v) << 20 for v in only.split(","))  # "c1_tensor_spacing:0,1,2,3": those MiB counts
+        for extra_bytes in spacings:
+            stride = n + extra_bytes // 4
+            views = {k: pool.alias_view([n], [1], element_offset=i * stride) for i, k in enumerate("abcd")}
+            out = pool.alias_view([n], [1], element_offset=4 * stride)
+            plan = equation.stamp(views, stream, preallocated_outputs={"o": out})
+            ms = time_runs([plan.run])
+            print(f"tensors 1 GiB + {extra_bytes:>9d} B apart   {ms * 1000:8.1f} us  {20 * n / ms / 1e6 / 8000:.3f}", flush=True)
         return
     if name == "c4_row_kernel_shapes":
         rng = np.random.default_rng(0)
@@ -728,7 +757,7 @@ def main():
                          "4 B read + 4 B written per element) so that hardware counters of a profiled run can be scaled against it")
     ap.add_argument("--experiment", default="", metavar="NAME",
                     help="run one A/B experiment instead of the bench and print its table: c1_address_stagger, c1_operand_streams, "
-                         "c1_sigmoid_exponentials, c4_row_kernel_shapes or stage_overlap")
+                         "c1_tensor_spacing, c1_sigmoid_exponentials, c4_row_kernel_shapes or stage_overlap")
     args = ap.parse_args()
     if args.experiment:
         run_experiment(args.experiment)
