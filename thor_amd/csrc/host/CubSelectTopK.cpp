@@ -8,6 +8,8 @@
 #include "Utilities/Expression/CompiledEquation.h"
 #include "thorhip_numeric_embed.h"
 
+#include "Utilities/Cache/LruCache.h"
+
 #include <algorithm>
 #include <cstdlib>
 #include <limits>
@@ -119,7 +121,7 @@ void validateSelect(const Tensor& input, const Tensor& flags, const Tensor& outp
     }
 }
 
-std::shared_ptr<const CubSelectionKernels> buildSelectKernels(DataType dtype, uint64_t numItems, int deviceNum, uint32_t vec) {
+std::shared_ptr<const CubSelectionKernels> buildSelectKernelsUncached(DataType dtype, uint64_t numItems, int deviceNum, uint32_t vec) {
     auto kernels = std::make_shared<CubSelectionKernels>();
     CubSelectionKernels& k = *kernels;
     k.kind = 0;
@@ -247,7 +249,7 @@ std::vector<std::pair<uint32_t, uint32_t>> digitPlanFor(uint32_t keyBits) {
 }
 
 // numItems > 0 and 0 < k (already capped at numItems)
-std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint64_t numItems, uint64_t k, bool largest, bool pairs, int deviceNum,
+std::shared_ptr<const CubSelectionKernels> buildTopKKernelsUncached(DataType dtype, uint64_t numItems, uint64_t k, bool largest, bool pairs, int deviceNum,
                                                             uint64_t keyAlignmentBytes) {
     auto kernels = std::make_shared<CubSelectionKernels>();
     CubSelectionKernels& sel = *kernels;
@@ -377,7 +379,7 @@ std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint
 }
 
 // numSegments > 0, 0 < k < segmentSize <= 8192
-std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, uint64_t numSegments, uint64_t segmentSize, uint64_t k, bool largest,
+std::shared_ptr<const CubSelectionKernels> buildRowTopKKernelsUncached(DataType dtype, uint64_t numSegments, uint64_t segmentSize, uint64_t k, bool largest,
                                                                bool pairs, int deviceNum) {
     auto kernels = std::make_shared<CubSelectionKernels>();
     CubSelectionKernels& sel = *kernels;
@@ -420,6 +422,45 @@ std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, u
       << segmentSize << " rows" << numSegments << " launches1 [" << sel.first->kernelName << "]";
     sel.variant = v.str();
     return kernels;
+}
+
+// Callers that prepare on every call (the one-call C entry points) find their kernels by the few numbers that decide the text,
+// and by the tuning switches' values, instead of writing out and hashing a hundred kilobytes of source each time.
+std::string requestKey(const char* family, std::initializer_list<uint64_t> numbers) {
+    std::string key = family;
+    for (uint64_t v : numbers) key += ' ' + std::to_string(v);
+    for (const char* name : {"THOR_TOPK_CANDIDATES", "THOR_TOPK_REGION", "THOR_TOPK_AMBIGUOUS", "THOR_TOPK_BLOCKS", "THOR_TOPK_SAMPLE_BLOCKS", "THOR_TOPK_SAMPLE_ITEMS",
+                             "THOR_TOPK_FINISH_BLOCKS", "THOR_TOPK_WALK", "THOR_TOPK_BUCKET_BITS", "THOR_TOPK_COMPACT_UNROLL", "THOR_TOPK_ROW_KERNEL", "THOR_TOPK_ROW_WAVES"}) {
+        const char* value = std::getenv(name);
+        key += '|';
+        if (value) key += value;
+    }
+    return key;
+}
+LruCacheThreadSafe<std::string, std::shared_ptr<const CubSelectionKernels>>& builtSelections() {
+    static LruCacheThreadSafe<std::string, std::shared_ptr<const CubSelectionKernels>> cache(1024);
+    return cache;
+}
+template <typename Build>
+std::shared_ptr<const CubSelectionKernels> builtOnce(const std::string& key, const Build& build) {
+    if (auto known = builtSelections().get(key)) return *known;
+    std::shared_ptr<const CubSelectionKernels> built = build();
+    return builtSelections().getOrCreate(key, [&] { return built; });
+}
+std::shared_ptr<const CubSelectionKernels> buildSelectKernels(DataType dtype, uint64_t numItems, int deviceNum, uint32_t vec) {
+    return builtOnce(requestKey("select", {static_cast<uint64_t>(dtype), numItems, static_cast<uint64_t>(deviceNum), vec}),
+                     [&] { return buildSelectKernelsUncached(dtype, numItems, deviceNum, vec); });
+}
+std::shared_ptr<const CubSelectionKernels> buildTopKKernels(DataType dtype, uint64_t numItems, uint64_t k, bool largest, bool pairs, int deviceNum,
+                                                            uint64_t keyAlignmentBytes) {
+    // (the alignment only matters up to the 16 bytes of a vector)
+    return builtOnce(requestKey("topk", {static_cast<uint64_t>(dtype), numItems, k, largest, pairs, static_cast<uint64_t>(deviceNum), std::min<uint64_t>(keyAlignmentBytes, 16)}),
+                     [&] { return buildTopKKernelsUncached(dtype, numItems, k, largest, pairs, deviceNum, keyAlignmentBytes); });
+}
+std::shared_ptr<const CubSelectionKernels> buildRowTopKKernels(DataType dtype, uint64_t numSegments, uint64_t segmentSize, uint64_t k, bool largest,
+                                                               bool pairs, int deviceNum) {
+    return builtOnce(requestKey("rows", {static_cast<uint64_t>(dtype), numSegments, segmentSize, k, largest, pairs, static_cast<uint64_t>(deviceNum)}),
+                     [&] { return buildRowTopKKernelsUncached(dtype, numSegments, segmentSize, k, largest, pairs, deviceNum); });
 }
 
 void launchTopK(const CubSelectionKernels& sel, const void* keysIn, const void* valuesIn, void* temp, void* keysOut, void* valuesOut, Stream& stream) {
