@@ -610,7 +610,7 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
 
     // one team per piece: as many teams as pieces (a power of two), teams never smaller than kMinTeam threads
     int teamCountBits = 0;
-    while (teamCountBits < kMaxTeamBits && ((u64)1 << teamCountBits) < pieces) ++teamCountBits;
+    while (teamCountBits < kMaxTeamBits && (u64)(1u << teamCountBits) < pieces) ++teamCountBits;
     const int teamBits = kThreadBits - teamCountBits;
     const u64 team = threadIdx.x >> teamBits;
     const int inTeam = threadIdx.x & ((1 << teamBits) - 1);
@@ -619,10 +619,11 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
     const u64 column = tile * Cfg::kLanesX + lx;
     const bool columnLive = column < kColumnsPerRow;
     const u64 columnOffset = (columnLive ? column : 0) * Cfg::kVec;  // dead lanes read column 0 and store nothing
-    const u64 passes = (pieces + ((u64)1 << teamCountBits) - 1) >> teamCountBits;
+    const u64 teams = (u64)(1u << teamCountBits);
+    const u64 passes = shiftRightBelow32(pieces + teams - 1, (u32)teamCountBits);
 
     for (u64 pass = 0; pass < passes; ++pass) {
-        const u64 segment = sLo + (pass << teamCountBits) + team;
+        const u64 segment = sLo + pass * teams + team;
         const bool pieceLive = segment < sEnd;
         u64 first = 0, last = 0;
         if (pieceLive) {
@@ -680,7 +681,7 @@ __device__ __forceinline__ void reduceSegments(const typename Cfg::Sources& src,
                 } else if (last > cEnd) {
                     acc[k].storePartial(workspace, (chunk * 2 + 1) * Cfg::kD + d, Workspace::kPartialSlots);
                 } else {
-                    Cfg::store(acc[k], segment * Cfg::kD + d, out, scale, (float)(last - first));
+                    Cfg::store(acc[k], segment * Cfg::kD + d, out, scale, toFloat((u64)(last - first)));
                 }
             }
         }
@@ -850,7 +851,7 @@ __device__ __forceinline__ void reduceSegmentsByRows(const typename Cfg::Sources
                         } else if (columnLive) {
 #pragma unroll
                             for (int k = 0; k < Cfg::kVec; ++k)
-                                Cfg::store(acc[k], s * Cfg::kD + column * Cfg::kVec + k, out, scale, (float)(last > first ? last - first : 0));
+                                Cfg::store(acc[k], s * Cfg::kD + column * Cfg::kVec + k, out, scale, toFloat((u64)(last > first ? last - first : 0)));
                         }
                         ++s;
                         if (s < Cfg::kSegments) enter();
@@ -898,7 +899,7 @@ __device__ __forceinline__ void reduceSegmentsByRows(const typename Cfg::Sources
                             if (first < cBegin) {
                                 total.storePartial(workspace, (chunk * 2 + 0) * Cfg::kD + d, Workspace::kPartialSlots);
                             } else {
-                                Cfg::store(total, ended * Cfg::kD + d, out, scale, (float)(last > first ? last - first : 0));
+                                Cfg::store(total, ended * Cfg::kD + d, out, scale, toFloat((u64)(last > first ? last - first : 0)));
                             }
                         }
                         running[k].reset();
@@ -967,7 +968,7 @@ __device__ __forceinline__ void finishSegments(const void* workspace, const type
         }
     }
     teamReduce<kThreads, Cfg::kFinishLanes, 1>(acc, floorLog2(kThreads), parked);
-    if (rowLane == 0 && columnLive) Cfg::store(acc[0], segment * Cfg::kD + d, out, scale, (float)(last - first));
+    if (rowLane == 0 && columnLive) Cfg::store(acc[0], segment * Cfg::kD + d, out, scale, toFloat((u64)(last - first)));
 }
 
 // ---- segmented broadcast: per-segment values [B, E] -> rows [N, E] ---------------------------------------------------------------
@@ -1008,7 +1009,7 @@ __device__ __forceinline__ typename Cfg::T broadcastValue(typename Cfg::T value,
     if constexpr (!Cfg::kNormalize) {
         return value;
     } else {
-        float x = toFloat(value) / (float)length;
+        float x = toFloat(value) / toFloat(length);
         if (Cfg::kViaHalf) x = roundF16(x);
         return fromFloat<typename Cfg::T>(x);
     }

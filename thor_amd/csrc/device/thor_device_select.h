@@ -46,6 +46,11 @@ __device__ __forceinline__ u32 blockExclusiveSum(u32 x, u32* lds, u32& total) {
     return before + inclusive - x;
 }
 
+// How many of the lanes below this one are set in `votes` (the result of a ballot).
+__device__ __forceinline__ u32 votesBelow(u64 votes) {
+    return __builtin_amdgcn_mbcnt_hi((u32)(votes >> 32), __builtin_amdgcn_mbcnt_lo((u32)votes, 0u));
+}
+
 // ---- select-flagged ----------------------------------------------------------------------------------------------------------
 // Cfg: Word (u8 / u16 / u32: elements are copied as raw words), kTotal, kThreads (256), kVec (4 when the tensors are aligned to
 // four elements, else 1), kRounds (4), kChunks.  A block owns kThreads * kVec * kRounds consecutive positions, read in rounds of
@@ -365,7 +370,6 @@ __device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const 
     constexpr u64 kChunkVectors = (u64)Cfg::kThreads * Cfg::kItems;
     constexpr u64 kChunks = (kVectors + kChunkVectors - 1) / kChunkVectors;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const u64 lowerLanes = ((u64)1 << lane) - 1;
     for (u64 chunk = blockIdx.x; chunk < kChunks; chunk += gridDim.x) {
         if (chunk != blockIdx.x) __syncthreads();  // the previous chunk's counts and bases have been read
         const u64 blockFirst = chunk * kChunkVectors;
@@ -418,9 +422,9 @@ __device__ __forceinline__ void topkGather(const typename Cfg::Raw* keys, const 
                 const bool isAbove = live && image > threshold, isTie = live && image == threshold;
                 const u64 aboveVotes = __builtin_amdgcn_ballot_w64(isAbove), tieVotes = __builtin_amdgcn_ballot_w64(isTie);
                 u32 slot = 0xffffffffu;
-                if (isAbove) slot = aboveAt + (u32)__builtin_popcountll(aboveVotes & lowerLanes);
+                if (isAbove) slot = aboveAt + votesBelow(aboveVotes);
                 if (isTie) {
-                    const u32 rank = tieAt + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+                    const u32 rank = tieAt + votesBelow(tieVotes);
                     if (rank < wantedTies) slot = firstTieSlot + rank;
                 }
                 aboveAt += (u32)__builtin_popcountll(aboveVotes);
@@ -604,7 +608,6 @@ __device__ __forceinline__ void topkCollect(const typename Cfg::Raw* keys, u32* 
     TopkState* state = reinterpret_cast<TopkState*>(temp + kTopkMaxBins);
     const u32 floorImage = topkFloorOfAll<Cfg>(temp, lds);  // (its barriers also order the cleared bins)
     const int lane = threadIdx.x % kWave;
-    const u64 lowerLanes = ((u64)1 << lane) - 1;
     const u32 region = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
     u32* regionImages = TopkCandidates<Cfg>::images(temp) + (u64)region * Cfg::kRegion;
     u32* regionPositions = TopkCandidates<Cfg>::positions(temp) + (u64)region * Cfg::kRegion;
@@ -647,7 +650,7 @@ __device__ __forceinline__ void topkCollect(const typename Cfg::Raw* keys, u32* 
 #pragma unroll
             for (int b = 0; (1 << b) <= V; ++b) {
                 const u64 votes = __builtin_amdgcn_ballot_w64(((mine >> b) & 1u) != 0);
-                before += (u32)__builtin_popcountll(votes & lowerLanes) << b;
+                before += votesBelow(votes) << b;
                 all += (u32)__builtin_popcountll(votes) << b;
             }
             if (cursor - copied + all > kTopkStage) copyStage();
@@ -675,7 +678,7 @@ __device__ __forceinline__ void topkCollect(const typename Cfg::Raw* keys, u32* 
                         if (lane == first) noted = atomicAdd(&state->floorTies, (u32)__builtin_popcountll(tieVotes));
                         noted = (u32)__shfl((int)noted, first, kWave);
                         if (tieHere) {
-                            const u32 rank = noted + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+                            const u32 rank = noted + votesBelow(tieVotes);
                             if (rank < (u32)Cfg::kK) tiePositions[rank] = (u32)((v0 + u * stride) * V + k);
                         }
                         tiesNoted = noted >= (u32)Cfg::kK;
@@ -1130,7 +1133,6 @@ template <typename Cfg, int SLOTS, typename Image, typename Position, typename L
 __device__ __forceinline__ void topkRowEmit(const Image& image, const Position& position, const Live& live, u32 prefix, u32 remaining,
                                             const u32* rowValuesIn, typename Cfg::Raw* rowKeys, u32* rowValues) {
     const int lane = threadIdx.x % kWave;
-    const u64 lowerLanes = ((u64)1 << lane) - 1;
     const u32 firstTieSlot = (u32)Cfg::kK - remaining;
     u32 aboveAt = 0, tieAt = 0;
 #pragma unroll
@@ -1139,9 +1141,9 @@ __device__ __forceinline__ void topkRowEmit(const Image& image, const Position& 
         const u64 aboveVotes = __builtin_amdgcn_ballot_w64(isAbove), tieVotes = __builtin_amdgcn_ballot_w64(isTie);
         if ((aboveVotes | tieVotes) == 0) continue;
         u32 slot = 0xffffffffu;
-        if (isAbove) slot = aboveAt + (u32)__builtin_popcountll(aboveVotes & lowerLanes);
+        if (isAbove) slot = aboveAt + votesBelow(aboveVotes);
         if (isTie) {
-            const u32 rank = tieAt + (u32)__builtin_popcountll(tieVotes & lowerLanes);
+            const u32 rank = tieAt + votesBelow(tieVotes);
             if (rank < remaining) slot = firstTieSlot + rank;
         }
         aboveAt += (u32)__builtin_popcountll(aboveVotes);

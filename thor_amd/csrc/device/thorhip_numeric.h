@@ -163,15 +163,46 @@ __device__ __forceinline__ float f64ToF32RoundOdd(double d) {
     return bitsF32(b | 1u);
 }
 
+// The value, unknown to the optimiser: keeps it from widening the conversion of a 32-bit half back into the conversion of the
+// 64-bit integer the half was taken from (whose expansion shifts 64 bits by a register amount, see below).
+__device__ __forceinline__ u32 opaque(u32 x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 __device__ __forceinline__ float u64ToF32RoundOdd(u64 v) {
-    if (v < (1ull << 24)) return (float)(u32)v;
+    if (v < (1ull << 24)) return (float)opaque((u32)v);
     const int lz = __builtin_clzll(v);
-    const int shift = 40 - lz;  // bits dropped below a 24-bit significand
-    u32 sig = (u32)(v >> shift);
-    if (v & ((1ull << shift) - 1ull)) sig |= 1u;
+    const int shift = 40 - lz;  // bits dropped below a 24-bit significand: 1..40
+    // Shifts of 32-bit halves only.  A 64-bit vector shift by an amount held in a register has been measured to go wrong on
+    // MI355X when that register is the last one the wavefront owns (one result in ten), and the compiler does not avoid it.
+    const u32 lo = (u32)v, hi = (u32)(v >> 32);
+    u32 sig, dropped;
+    if (shift >= 32) {
+        const u32 s = (u32)shift - 32u;
+        sig = hi >> s;
+        dropped = (hi & ((1u << s) - 1u)) | lo;
+    } else {
+        sig = (lo >> shift) | (hi << (32 - shift));
+        dropped = lo & ((1u << shift) - 1u);
+    }
+    if (dropped) sig |= 1u;
     const u32 exp = (u32)(127 + 23 + shift);
     return bitsF32((exp << 23) | (sig & 0x7fffffu));
 }
+
+// Round-to-nearest-even fp32 of 64-bit integers, as the cast gives it, without the 64-bit shift by a register amount that the
+// compiler's own expansion of the cast uses: the halves are normalised with 32-bit shifts, the bits that do not fit 32 become
+// a sticky bit, the 32-bit conversion rounds once, and the scaling is exact.
+__device__ __forceinline__ float u64ToF32(u64 v) {
+    const u32 hi = (u32)(v >> 32), lo = (u32)v;
+    if (hi == 0) return (float)opaque(lo);
+    const u32 lz = (u32)__builtin_clz(hi);
+    const u32 top = lz ? (hi << lz) | (lo >> (32u - lz)) : hi;
+    const u32 rest = lo << lz;
+    return __builtin_ldexpf((float)(top | (rest ? 1u : 0u)), 32 - (int)lz);
+}
+__device__ __forceinline__ float i64ToF32(i64 v) { return v < 0 ? -u64ToF32((u64)0 - (u64)v) : u64ToF32((u64)v); }
 
 __device__ __forceinline__ float i64ToF32RoundOdd(i64 v) {
     if (v >= 0) return u64ToF32RoundOdd((u64)v);
@@ -313,7 +344,15 @@ struct Store<boolean> {
             return (T)v;                                       \
         }                                                      \
     };
-THOR_PLAIN_STORE(float)
+template <>
+struct Store<float> {
+    template <typename C>
+    __device__ __forceinline__ static float from(C v) {
+        return (float)v;
+    }
+    __device__ __forceinline__ static float from(u64 v) { return u64ToF32(v); }
+    __device__ __forceinline__ static float from(i64 v) { return i64ToF32(v); }
+};
 THOR_PLAIN_STORE(double)
 THOR_PLAIN_STORE(i8)
 THOR_PLAIN_STORE(i16)

@@ -564,7 +564,7 @@ std::string generateReductionSource(const ReductionKernelRequest& request, const
     std::vector<ReductionKernelRequest::Value> values = request.values;
     std::string prologue = request.prologue;
     if (values.empty()) {
-        sources = {{request.inputDType, ReductionKernelRequest::Source::Kind::Vector}};
+        sources = {{request.inputDType, ReductionKernelRequest::Source::Kind::Vector, std::string()}};
         values = {{request.valueOp, request.valueOutputDType, "x0"}};
         prologue = "        const float x0 = toFloat(l.p0.v[k]);\n";
     } else if (request.isArg) {

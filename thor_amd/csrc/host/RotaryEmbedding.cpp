@@ -366,11 +366,11 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         if (positionIds.has_value()) {
             s << "            float angleBase = thor::toFloat(ids[position]);\n";
         } else {
-            s << "            float angleBase = (float)position + " << floatLiteral(static_cast<double>(n.rope_position_offset)) << ";\n";
+            s << "            float angleBase = thor::toFloat(position) + " << floatLiteral(static_cast<double>(n.rope_position_offset)) << ";\n";
         }
         if (n.rope_scaling_kind == RotaryScalingKind::Linear) s << "            angleBase = angleBase / " << floatLiteral(n.rope_scaling_factor) << ";\n";
         s << "            float freq = 0.0f;\n";
-        s << "            {\n" << frequencyStatements(n, rotary, "(float)pair", "                ") << "            }\n";
+        s << "            {\n" << frequencyStatements(n, rotary, "thor::toFloat(pair)", "                ") << "            }\n";
         s << "            const float theta = angleBase * freq;\n";
         s << "            sincosf(theta, &sn, &cs);\n";  // one argument reduction for both (a third fewer instructions than sinf + cosf)
         if (n.rope_attention_factor != 1.0) s << "            sn *= " << attention << ";\n            cs *= " << attention << ";\n";
@@ -421,7 +421,7 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "    __shared__ float frequencies[" << half << "];\n";
         s << "    for (thor::u32 pair = threadIdx.x; pair < " << half << "u; pair += " << threads << "u) {\n";
         s << "        float freq = 0.0f;\n";
-        s << "        {\n" << frequencyStatements(n, rotary, "(float)pair", "            ") << "        }\n";
+        s << "        {\n" << frequencyStatements(n, rotary, "thor::toFloat(pair)", "            ") << "        }\n";
         s << "        frequencies[pair] = freq;\n    }\n";
         s << "    __syncthreads();\n";
     }
@@ -456,7 +456,7 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
     if (positionIds.has_value()) {
         s << "    float angleBase = thor::toFloat(ids[position]);\n";
     } else {
-        s << "    float angleBase = (float)position + " << floatLiteral(static_cast<double>(n.rope_position_offset)) << ";\n";
+        s << "    float angleBase = thor::toFloat(position) + " << floatLiteral(static_cast<double>(n.rope_position_offset)) << ";\n";
     }
     if (n.rope_scaling_kind == RotaryScalingKind::Linear) s << "    angleBase = angleBase / " << floatLiteral(n.rope_scaling_factor) << ";\n";
     s << "    float sn[P], cs[P];\n";
@@ -466,7 +466,7 @@ std::shared_ptr<StampedEquation> stampRotaryEmbedding(const Tensor& values, cons
         s << "        const float freq = frequencies[pair];\n";
     } else {
         s << "        float freq = 0.0f;\n";
-        s << "        {\n" << frequencyStatements(n, rotary, "(float)pair", "            ") << "        }\n";
+        s << "        {\n" << frequencyStatements(n, rotary, "thor::toFloat(pair)", "            ") << "        }\n";
     }
     s << "        const float theta = angleBase * freq;\n";
     s << "        sincosf(theta, &sn[k], &cs[k]);\n";
