@@ -114,6 +114,47 @@ def test_every_pair_out_of_place(gpu, src, dst):
     assert_same_bits(got, want, dst)
 
 
+def wide_integers(src, rng):
+    """Integers of every magnitude the type holds: random bits cut to a random width, values one step either side of the ties of a
+    24-, 11- and 8-bit significand at every exponent, and the ends of the range."""
+    carrier = numpy_carrier(src)
+    bits = np.iinfo(carrier).bits
+    signed = np.iinfo(carrier).min < 0
+    width = rng.integers(1, bits + 1, 20000).astype(np.uint64)
+    magnitude = rng.integers(0, 1 << 63, 20000, dtype=np.uint64) * np.uint64(2) + rng.integers(0, 2, 20000).astype(np.uint64)
+    magnitude = magnitude >> (np.uint64(64) - width)
+    around = []
+    for significand in (24, 11, 8):
+        for exponent in range(significand, bits):
+            tie = (1 << exponent) + (1 << (exponent - significand))  # halfway between two neighbours of that significand
+            odd_tie = tie + (1 << (exponent - significand + 1))
+            around += [tie - 1, tie, tie + 1, odd_tie - 1, odd_tie, odd_tie + 1, (1 << exponent) - 1, 1 << exponent]
+    limit = (1 << (bits - 1)) - 1 if signed else (1 << bits) - 1
+    values = np.concatenate([magnitude, np.array([v for v in around if v <= limit], np.uint64), np.array([0, 1, limit], np.uint64)])
+    values = np.minimum(values, np.uint64(limit))
+    if not signed:
+        return values.astype(carrier)
+    out = values.astype(np.int64)
+    out[::2] = -out[::2]
+    out = np.concatenate([out, np.array([np.iinfo(carrier).min], np.int64)])
+    return out.astype(carrier)
+
+
+@pytest.mark.parametrize("src", [DataType.int64, DataType.uint64, DataType.int32, DataType.uint32], ids=lambda d: d.name)
+def test_wide_integers_round_once_to_every_float_type(gpu, src):
+    """A 64-bit integer becomes fp32 through 32-bit halves with a sticky bit, and a narrower float through a round-to-odd fp32
+    image (device code has no 64-bit shift by a register amount, which is what the compiler's expansion of the cast would use): the
+    results must be the bits of one round-to-nearest-even step from the integer, at every magnitude and either side of every tie."""
+    rng = np.random.default_rng(int(src) + 900)
+    x = wide_integers(src, rng)
+    for dst in (DataType.fp32, DataType.fp64, DataType.fp16, DataType.bf16, DataType.fp8_e4m3, DataType.fp8_e5m2):
+        got = gpu.convert_array(x, src, dst)
+        want = oracle.convert(x, int(src), int(dst))
+        assert_same_bits(got, want, dst)
+        if dst == DataType.fp32:  # and the oracle's rounding against NumPy's own
+            np.testing.assert_array_equal(want.view(np.uint32), x.astype(np.float32).view(np.uint32))
+
+
 @pytest.mark.parametrize("src,dst", [(DataType.fp32, DataType.fp16), (DataType.fp32, DataType.bf16), (DataType.fp16, DataType.fp32),
                                       (DataType.bf16, DataType.fp32), (DataType.fp64, DataType.uint8), (DataType.int8, DataType.fp64),
                                       (DataType.fp32, DataType.int32), (DataType.fp16, DataType.bf16)])

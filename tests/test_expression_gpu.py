@@ -180,6 +180,14 @@ def test_compare_where_logic_and_casts(gpu):
     assert got.tolist() == [0.5, -1.0, 150.0, 3.5]
     got = run_expr(ex.input("i", output_dtype=DataType.fp32) * 0.5, {"i": ints}, DataType.int32, out_dtype=DataType.fp32)
     assert got.tolist() == [0.5, -1.0, 150.0, 3.5]
+    # 64-bit integers of every magnitude, either side of the ties of a 24-bit significand: the cast rounds once, to nearest even
+    # (generated code converts through 32-bit halves: the compiler's expansion of the cast would shift 64 bits by a register amount)
+    ties = [(1 << e) + (1 << (e - 24)) + d for e in range(24, 63) for d in (-1, 0, 1)] + [(1 << e) + 3 * (1 << (e - 24)) for e in range(24, 62)]
+    for carrier, dtype, values in ((np.int64, DataType.int64, [0, 1, -1, -(1 << 63), (1 << 63) - 1] + ties + [-t for t in ties]),
+                                   (np.uint64, DataType.uint64, [0, 1, (1 << 64) - 1, (1 << 63) + (1 << 39)] + ties)):
+        wide = np.array(values, dtype=carrier)
+        got = run_expr(ex.input("i").cast(DataType.fp32) * 1.0, {"i": wide}, dtype, out_dtype=DataType.fp32)
+        np.testing.assert_array_equal(got.view(np.uint32), wide.astype(np.float32).view(np.uint32))
 
 
 def test_constants_fold_and_identities_vanish(gpu):
