@@ -166,7 +166,7 @@ __device__ __forceinline__ float f64ToF32RoundOdd(double d) {
 // The value, unknown to the optimiser: keeps it from widening the conversion of a 32-bit half back into the conversion of the
 // 64-bit integer the half was taken from (whose expansion shifts 64 bits by a register amount, see below).
 __device__ __forceinline__ u32 opaque(u32 x) {
-    asm volatile("" : "+v"(x));
+    asm("" : "+v"(x));  // not volatile: a conversion whose result is unused still disappears
     return x;
 }
 
