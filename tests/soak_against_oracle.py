@@ -1,0 +1,225 @@
+"""Random differential runs of the GPU kernels against the oracle, outside the collected suite (every case compiles its own kernels,
+0.3-1 s each on a cold box):
+
+    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: topk | topk_rows | scans | reductions | rows
+
+Shapes, dtypes, operations, orders and data kinds (normal, few levels, sorted either way, a narrow band, outliers over zeros, NaN /
+inf / signed zeros, a repeated block) are drawn at random; every case is printed before it runs and checked with the same helper
+the collected test of its family uses (bit-exact for selections, scans of exact operations, min / max and arg reductions; the
+tests' tolerances for float sums).  The first failure ends the run with the case on the last line.  This is the run that showed
+the 64-bit shift defect of the device (row top-k, sorted fp16 rows: tests/test_selection_gpu.py keeps that case)."""
+from __future__ import annotations
+
+import os
+import sys
+import time
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+sys.path.insert(0, HERE)
+
+from helpers import to_storage  # noqa: E402
+from thor_amd import physical as ph  # noqa: E402
+from thor_amd.dtypes import DataType, numpy_carrier  # noqa: E402
+from thor_amd.physical import ScanOp  # noqa: E402
+
+FLOATS = (DataType.fp16, DataType.bf16, DataType.fp32)
+KINDS = ["normal", "levels", "sorted", "reversed", "narrow", "outliers", "specials", "blocks"]
+
+
+def keys_of(rng, dtype, rows, size, kind, k):
+    """[rows, size] keys of one data kind (sorted kinds are sorted inside every row)."""
+    n = rows * size
+    if dtype in FLOATS:
+        if kind == "normal":
+            v = rng.standard_normal(n).astype(np.float32) * 100
+        elif kind == "levels":
+            v = np.round(rng.standard_normal(n) * rng.integers(1, 40)).astype(np.float32)
+        elif kind in ("sorted", "reversed"):
+            v = np.sort(rng.standard_normal((rows, size)).astype(np.float32), axis=1)
+            v = (v[:, ::-1] if kind == "reversed" else v).reshape(-1).copy()
+        elif kind == "narrow":
+            v = (1.0 + rng.random(n) * 2.0 ** -rng.integers(4, 20)).astype(np.float32) * (1 if rng.random() < 0.5 else -1)
+        elif kind == "outliers":
+            v = np.zeros(n, np.float32)
+            at = rng.integers(0, n, max(k // 2, 1))
+            v[at] = rng.standard_normal(at.size).astype(np.float32) * 50
+        elif kind == "specials":
+            v = rng.standard_normal(n).astype(np.float32)
+            at = rng.integers(0, n, max(n // 50, 1))
+            v[at] = rng.choice(np.array([np.inf, -np.inf, np.nan, 0.0, -0.0], np.float32), at.size)
+        else:
+            block = rng.standard_normal(min(1 << 16, n)).astype(np.float32)
+            v = np.tile(block, n // block.size + 1)[:n].copy()
+        return to_storage(v, dtype)
+    carrier = numpy_carrier(dtype)
+    info = np.iinfo(carrier)
+    if kind in ("levels", "narrow"):
+        return rng.integers(0, int(rng.integers(2, 50)), n).astype(carrier)
+    if kind in ("sorted", "reversed"):
+        v = np.sort(rng.integers(info.min, int(info.max) + 1, (rows, size)).astype(carrier), axis=1)
+        return (v[:, ::-1] if kind == "reversed" else v).reshape(-1).copy()
+    if kind == "outliers":
+        v = np.zeros(n, carrier)
+        at = rng.integers(0, n, max(k // 2, 1))
+        v[at] = rng.integers(info.min, int(info.max) + 1, at.size)
+        return v
+    return rng.integers(info.min, int(info.max) + 1, n).astype(carrier)
+
+
+def topk_case(rng, stream):
+    import test_selection_gpu as T
+    dtype = [DataType.fp32, DataType.fp32, DataType.bf16, DataType.fp16, DataType.int32, DataType.uint32, DataType.uint16, DataType.int16][rng.integers(0, 8)]
+    n = int(rng.integers(1 << 20, 1 << 23)) if rng.random() < 0.8 else int(rng.integers(1 << 23, 1 << 25))
+    if rng.random() < 0.5:
+        n = n // 4 * 4
+    k = int(max(1, 2 ** rng.uniform(0, np.log2(max(n // 256, 1)))))
+    largest, pairs, kind = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), KINDS[rng.integers(0, len(KINDS))]
+    print(f"{dtype.name} n={n} k={k} largest={largest} pairs={pairs} kind={kind}", flush=True)
+    keys = keys_of(rng, dtype, 1, n, kind, k)
+    got, got_values, variant = T.run_top_k(keys, dtype, k, largest, stream, pairs=pairs)
+    T.check_top_k(keys, dtype, k, largest, got, got_values)
+    return variant
+
+
+def topk_rows_case(rng, stream):
+    import test_selection_gpu as T
+    dtype = [DataType.fp32, DataType.bf16, DataType.fp16, DataType.int32, DataType.uint16, DataType.int8, DataType.uint8][rng.integers(0, 7)]
+    size = min(int(2 ** rng.uniform(1, 13.2)), 8192)
+    if rng.random() < 0.4:
+        size = max(size // 8 * 8, 8)
+    rows = int(max(1, min(2 ** rng.uniform(0, 14), (1 << 22) // size)))
+    k = int(max(1, min(size - 1, 2 ** rng.uniform(0, np.log2(size)))))
+    largest, pairs, kind = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), KINDS[rng.integers(0, 5)]
+    print(f"{dtype.name} rows={rows} size={size} k={k} largest={largest} pairs={pairs} kind={kind}", flush=True)
+    keys = keys_of(rng, dtype, rows, size, kind, k)
+    got, got_values, variant = T.run_top_k(keys, dtype, k, largest, stream, pairs=pairs, segment_size=size)
+    T.check_top_k(keys, dtype, k, largest, got, got_values, segment_size=size)
+    return variant
+
+
+def scans_case(rng, stream):
+    import oracle
+    import test_scan_gpu as S
+    import test_selection_gpu as T
+    what = ["rows", "flat", "segments", "select"][rng.integers(0, 4)]
+    if what == "select":
+        dtype = [DataType.fp32, DataType.fp16, DataType.uint8, DataType.int32, DataType.uint16][rng.integers(0, 5)]
+        n = int(2 ** rng.uniform(0, 23))
+        density = [0.0, 1.0, 0.5, 0.01, 0.99, rng.random()][rng.integers(0, 6)]
+        flag_dtype = [DataType.uint8, DataType.boolean][rng.integers(0, 2)]
+        print(f"select {dtype.name} n={n} density={density:.3f} flags={flag_dtype.name}", flush=True)
+        values = T.random_keys(rng, n, dtype)
+        flags = (rng.random(n) < density).astype(np.uint8) * (rng.integers(1, 255, n).astype(np.uint8) if flag_dtype == DataType.uint8 else 1)
+        out, count, variant = T.run_select(values, flags, dtype, flag_dtype, stream)
+        want = values[flags != 0]
+        assert count == want.size, (count, want.size)
+        np.testing.assert_array_equal(T.bits_of(out[:count]), T.bits_of(want))
+        return variant
+    dtype = [DataType.uint32, DataType.fp32, DataType.fp16, DataType.bf16][rng.integers(0, 4)]
+    op = [ScanOp.sum, ScanOp.min, ScanOp.max, ScanOp.product, ScanOp.arg_min, ScanOp.arg_max][rng.integers(0, 6)]
+    if what == "segments" and op == ScanOp.product:
+        op = ScanOp.sum
+    inclusive, reverse = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    if what == "rows":
+        cols = int(2 ** rng.uniform(0, 17))
+        shape = (int(max(1, min(2 ** rng.uniform(0, 12), (1 << 22) // cols))), cols)
+    else:
+        shape = (1, int(2 ** rng.uniform(0, 23.5))) if what == "flat" else (int(2 ** rng.uniform(4, 22)),)
+    n = int(np.prod(shape))
+    if dtype == DataType.uint32:
+        carrier = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32) if op != ScanOp.product else rng.integers(1, 4, n).astype(np.uint32)
+    elif op == ScanOp.product:  # signed powers of two whose running exponent stays small: exact in any order
+        steps = np.diff(np.concatenate([[0], np.clip(np.cumsum(rng.integers(-1, 2, n)), -6, 6)]))
+        carrier = to_storage((np.exp2(steps) * rng.choice([1.0, -1.0], n)).astype(np.float32), dtype)
+    else:
+        carrier = to_storage((np.round(rng.standard_normal(n) * 8) / 8).astype(np.float32), dtype)
+    carrier = carrier.reshape(shape)
+    if what == "segments":
+        segments = int(max(1, min(2 ** rng.uniform(0, 16), n)))
+        cuts = np.sort(rng.integers(0, n + 1, segments))
+        offsets = np.concatenate([[0], cuts, [max(n - int(rng.integers(0, 50)), int(cuts[-1]))]])
+        width = [DataType.uint32, DataType.uint64][rng.integers(0, 2)]
+        print(f"segments {dtype.name} n={n} segments={segments} {op.name} inclusive={inclusive} reverse={reverse} offsets={width.name}", flush=True)
+        got, variant = S.run_scan(carrier, dtype, stream, op, inclusive, reverse, offsets=offsets, offsets_dtype=width)
+        active = int(offsets[-1])
+        if dtype == DataType.uint32 or op != ScanOp.sum:
+            expected = oracle.scan(carrier, S.ORACLE_OP[op], inclusive, reverse, offsets=offsets, dtype=int(dtype))
+            np.testing.assert_array_equal(got[:active], expected[:active])
+        else:
+            S.check(got[:active], carrier[:active], dtype, op, inclusive, reverse, offsets=offsets)
+        return variant
+    segment_size = shape[1] if what == "rows" else 0
+    print(f"{what} {dtype.name} shape={shape} {op.name} inclusive={inclusive} reverse={reverse}", flush=True)
+    got, variant = S.run_scan(carrier, dtype, stream, op, inclusive, reverse, segment_size=segment_size)
+    S.check(got, carrier, dtype, op, inclusive, reverse, segment_size=segment_size)
+    return variant
+
+
+def reductions_case(rng, stream):
+    import test_reduction_gpu as R
+    import test_segmented_reduction_gpu as SR
+    what = ["value", "arg", "segments"][rng.integers(0, 3)]
+    if what == "segments":
+        rank = int(rng.integers(1, 4))
+        rest = [int(2 ** rng.uniform(0, 6)) for _ in range(rank - 1)]
+        rows = int(2 ** rng.uniform(3, 17))
+        while rows * int(np.prod(rest or [1])) > (1 << 21):
+            rows //= 2
+        shape = tuple([max(rows, 8)] + rest)
+        segments = int(max(6, min(2 ** rng.uniform(2, 12), shape[0])))
+        dtype = [DataType.fp32, DataType.bf16, DataType.fp16, DataType.fp8_e4m3][rng.integers(0, 4)]
+        print(f"segments shape={shape} segments={segments} {dtype.name}", flush=True)
+        SR.test_random_ragged_partitions_against_numpy(stream, shape, segments, dtype)
+        return ""
+    rank = int(rng.integers(1, 5))
+    left = 2 ** rng.uniform(0, 22)
+    dims = []
+    for d in range(rank):
+        extent = int(max(1, round(left if d == rank - 1 else 2 ** rng.uniform(0, np.log2(max(left, 1.0001))))))
+        if rng.random() < 0.3:
+            extent |= 1
+        dims.append(extent)
+        left = max(left / extent, 1)
+    axes = sorted(rng.choice(rank, int(rng.integers(1, rank + 1)), replace=False).tolist())
+    dtype = [DataType.fp32, DataType.fp16, DataType.bf16][rng.integers(0, 3)]
+    print(f"{what} dims={dims} axes={axes} {dtype.name}", flush=True)
+    if what == "value":
+        R.test_value_ops_against_oracle(stream, dims, axes, dtype)
+    else:
+        R.test_arg_ops_against_oracle_with_ties_and_nans(stream, dims, axes)
+    return ""
+
+
+def rows_case(rng, stream):
+    import test_row_fusion_gpu as RF
+    cols = int(2 ** rng.uniform(1, 15))
+    rows = int(max(2, min(2 ** rng.uniform(1, 13), (1 << 22) // cols)))
+    dtype = [DataType.fp32, DataType.fp16, DataType.bf16][rng.integers(0, 3)]
+    if rng.random() < 0.5:
+        print(f"softmax {(rows, cols)} {dtype.name}", flush=True)
+        RF.test_softmax_single_pass_matches_staged_and_closed_form(None, dtype, (rows, cols))
+    else:
+        cols = min(cols, 8192)
+        shape = (rows, cols) if rng.random() < 0.6 else (max(rows // 3, 1), 3, cols)
+        print(f"normalise {shape} {dtype.name}", flush=True)
+        RF.test_mean_variance_normalisation_single_pass(None, dtype, shape)
+    return ""
+
+
+FAMILIES = {"topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
+
+if __name__ == "__main__":
+    if len(sys.argv) != 4 or sys.argv[1] not in FAMILIES:
+        sys.exit(__doc__)
+    family, seed, cases = FAMILIES[sys.argv[1]], int(sys.argv[2]), int(sys.argv[3])
+    rng = np.random.default_rng(seed)
+    stream = ph.Stream(0)
+    start = time.time()
+    for case in range(cases):
+        print(f"case {case}: ", end="", flush=True)
+        variant = family(rng, stream)
+        print(f"   ok {variant[:100]}  t={time.time() - start:.0f}s", flush=True)
+    print(f"ALL OK: {cases} cases of {sys.argv[1]}, seed {seed}")
