@@ -1,7 +1,7 @@
 """Random differential runs of the GPU kernels against the oracle, outside the collected suite (every case compiles its own kernels,
 0.3-1 s each on a cold box):
 
-    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: topk | topk_rows | scans | reductions | rows
+    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: conversions | topk | topk_rows | scans | reductions | rows
 
 Shapes, dtypes, operations, orders and data kinds (normal, few levels, sorted either way, a narrow band, outliers over zeros, NaN /
 inf / signed zeros, a repeated block) are drawn at random; every case is printed before it runs and checked with the same helper
@@ -209,7 +209,43 @@ def rows_case(rng, stream):
     return ""
 
 
-FAMILIES = {"topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
+def conversions_case(rng, stream):
+    """Out of place and in place, random lengths and element offsets at both ends, guard bytes around the destination."""
+    import oracle
+    import test_convert_gpu as C
+    from thor_amd.dtypes import size_of
+    from thor_amd.runtime import DeviceBuffer, TypeConverter
+    src, dst = [C.ALL[i] for i in rng.choice(len(C.ALL), 2, replace=False)]
+    n = int(2 ** rng.uniform(0, 21))
+    in_place = rng.random() < 0.3
+    src_off, dst_off = (0, 0) if in_place else (int(rng.integers(0, 9)), int(rng.integers(0, 9)))
+    wide = src in (DataType.int64, DataType.uint64, DataType.int32, DataType.uint32) and dst in C.FLOATS and rng.random() < 0.5
+    print(f"{src.name} -> {dst.name} n={n} in_place={in_place} offsets={src_off},{dst_off} wide={wide}", flush=True)
+    x = np.resize(C.wide_integers(src, rng), n) if wide else C._sample_for(src, dst, n, rng)
+    want = oracle.convert(x, int(src), int(dst))
+    ssz, dsz = size_of(src), size_of(dst)
+    if in_place:
+        buf = DeviceBuffer(n * max(ssz, dsz) + 256)
+        guard = np.full(256, 0xA5, np.uint8)
+        buf.upload(guard, offset_bytes=n * max(ssz, dsz))
+        buf.upload(x)
+        TypeConverter.convert_type(buf.ptr, buf.ptr, src, dst, n)
+        got = buf.download(numpy_carrier(dst), n)
+        assert np.array_equal(buf.download(np.uint8, 256, offset_bytes=n * max(ssz, dsz)), guard), "wrote past the end"
+    else:
+        a, b = DeviceBuffer((n + src_off) * ssz + 256), DeviceBuffer((n + dst_off) * dsz + 512)
+        fill = np.full((n + dst_off) * dsz + 512, 0x5A, np.uint8)
+        b.upload(fill)
+        a.upload(x, offset_bytes=src_off * ssz)
+        TypeConverter.convert_type(a.ptr + src_off * ssz, b.ptr + 256 + dst_off * dsz, src, dst, n)
+        got = b.download(numpy_carrier(dst), n, offset_bytes=256 + dst_off * dsz)
+        assert np.all(b.download(np.uint8, 256 + dst_off * dsz) == 0x5A), "wrote before the destination"
+        assert np.all(b.download(np.uint8, 256 - dst_off * dsz, offset_bytes=256 + (dst_off + n) * dsz) == 0x5A), "wrote past the destination"
+    C.assert_same_bits(got, want, dst)
+    return ""
+
+
+FAMILIES = {"conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
 
 if __name__ == "__main__":
     if len(sys.argv) != 4 or sys.argv[1] not in FAMILIES:
