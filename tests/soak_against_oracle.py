@@ -1,7 +1,7 @@
 """Random differential runs of the GPU kernels against the oracle, outside the collected suite (every case compiles its own kernels,
 0.3-1 s each on a cold box):
 
-    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: conversions | topk | topk_rows | scans | reductions | rows
+    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: expressions | conversions | topk | topk_rows | scans | reductions | rows
 
 Shapes, dtypes, operations, orders and data kinds (normal, few levels, sorted either way, a narrow band, outliers over zeros, NaN /
 inf / signed zeros, a repeated block) are drawn at random; every case is printed before it runs and checked with the same helper
@@ -245,7 +245,81 @@ def conversions_case(rng, stream):
     return ""
 
 
-FAMILIES = {"conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
+def expressions_case(rng, stream):
+    """Fused elementwise expressions over broadcast operands, with or without a reduction over some axes at the end.  Operands hold
+    small integers and the tree keeps every intermediate below 200 in magnitude, so fp32, fp16 and bf16 arithmetic is exact in any
+    order and the result must equal NumPy's integer arithmetic bit for bit."""
+    from helpers import from_storage, run_staged
+    ex = ph.Expression
+    rank = int(rng.integers(1, 5))
+    left = 2 ** rng.uniform(0, 20)
+    dims = []
+    for d in range(rank):
+        extent = int(max(1, round(left if d == rank - 1 else 2 ** rng.uniform(0, np.log2(max(left, 1.0001))))))
+        dims.append(extent)
+        left = max(left / extent, 1)
+    dtype = [DataType.fp32, DataType.fp16, DataType.bf16][rng.integers(0, 3)]
+    names = "abcd"[:int(rng.integers(2, 5))]
+    arrays, nodes = {}, []
+    for i, name in enumerate(names):
+        shape = [e if i == 0 or rng.random() < 0.7 else 1 for e in dims]
+        values = rng.integers(-3, 4, shape)
+        arrays[name] = to_storage(values.astype(np.float32), dtype)
+        nodes.append((ex.input(name), values.astype(np.int64), 3))
+    text = list(names)
+    used = [{name} for name in names]
+    for _ in range(int(rng.integers(1, 6))):
+        i, j = int(rng.integers(0, len(nodes))), int(rng.integers(0, len(nodes)))
+        (x, xv, xb), (y, yv, yb) = nodes[i], nodes[j]
+        op = ["add", "sub", "mul", "min", "max", "where", "neg", "abs"][rng.integers(0, 8)]
+        if op == "mul" and xb * yb > 200 or op in ("add", "sub") and xb + yb > 200:
+            op = "max"
+        if op == "add":
+            node = (x + y, xv + yv, xb + yb)
+        elif op == "sub":
+            node = (x - y, xv - yv, xb + yb)
+        elif op == "mul":
+            node = (x * y, xv * yv, xb * yb)
+        elif op == "min":
+            node = (x.min(y), np.minimum(xv, yv), max(xb, yb))
+        elif op == "max":
+            node = (x.max(y), np.maximum(xv, yv), max(xb, yb))
+        elif op == "where":
+            node = (ex.where(x > y, x, y - 1.0), np.where(xv > yv, xv, yv - 1), max(xb, yb) + 1)
+        elif op == "neg":
+            node = (-x, -xv, xb)
+        else:
+            node = (x.abs(), np.abs(xv), xb)
+        nodes.append(node)
+        text.append(f"{op}({text[i]},{text[j]})" if op not in ("neg", "abs") else f"{op}({text[i]})")
+        used.append(used[i] | used[j] if op not in ("neg", "abs") else set(used[i]))
+    expr, want, bound = nodes[-1]
+    for name in names:  # every input takes part, so that the plan binds all of them
+        if name not in used[-1]:
+            k = names.index(name)
+            expr, want, bound = expr.max(nodes[k][0]), np.maximum(want, nodes[k][1]), max(bound, 3)
+            text[-1] = f"max({text[-1]},{name})"
+    want = np.broadcast_to(want, np.broadcast_shapes(*[arrays[n].shape for n in names])).copy()
+    reduce = None
+    if rng.random() < 0.5:
+        axes = sorted(rng.choice(rank, int(rng.integers(1, rank + 1)), replace=False).tolist())
+        count = int(np.prod([want.shape[a] for a in axes]))
+        reduce = ["sum", "max", "min"][rng.integers(0, 3)]
+        if reduce == "sum" and count * bound >= (1 << 24):
+            reduce = "max"
+        expr = {"sum": expr.reduce_sum, "max": expr.reduce_max, "min": expr.reduce_min}[reduce](axes)
+        want = {"sum": np.sum, "max": np.max, "min": np.min}[reduce](want, axis=tuple(axes), keepdims=True)
+        text[-1] = f"{reduce}{axes}({text[-1]})"
+    print(f"{dtype.name} dims={dims} shapes={[list(arrays[n].shape) for n in names]} {text[-1]}", flush=True)
+    plan, outs = run_staged(expr, arrays, dtype)
+    got = outs["output"]
+    got = got.astype(np.float64) if reduce else from_storage(got, dtype).astype(np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    np.testing.assert_array_equal(got, want.astype(np.float64), err_msg=str(plan.stage_descriptions()))
+    return " | ".join(plan.stage_kind_names())
+
+
+FAMILIES = {"expressions": expressions_case, "conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
 
 if __name__ == "__main__":
     if len(sys.argv) != 4 or sys.argv[1] not in FAMILIES:
