@@ -1,7 +1,7 @@
 """Random differential runs of the GPU kernels against the oracle, outside the collected suite (every case compiles its own kernels,
 0.3-1 s each on a cold box):
 
-    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: expressions | conversions | topk | topk_rows | scans | reductions | rows
+    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: views | expressions | conversions | topk | topk_rows | scans | reductions | rows
 
 Shapes, dtypes, operations, orders and data kinds (normal, few levels, sorted either way, a narrow band, outliers over zeros, NaN /
 inf / signed zeros, a repeated block) are drawn at random; every case is printed before it runs and checked with the same helper
@@ -319,7 +319,50 @@ def expressions_case(rng, stream):
     return " | ".join(plan.stage_kind_names())
 
 
-FAMILIES = {"expressions": expressions_case, "conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
+def views_case(rng, stream):
+    """An operand seen through a permuted (and possibly cropped) strided view, in elementwise work with a dense operand and under a
+    reduction over random axes; small integers, so that the result equals NumPy's bit for bit."""
+    from helpers import from_storage, run_staged
+    ex = ph.Expression
+    rank = int(rng.integers(2, 5))
+    left = 2 ** rng.uniform(2, 19)
+    dims = []
+    for d in range(rank):
+        extent = int(max(1, round(left if d == rank - 1 else 2 ** rng.uniform(0, np.log2(max(left, 1.0001))))))
+        dims.append(extent)
+        left = max(left / extent, 1)
+    dtype = [DataType.fp32, DataType.fp16, DataType.bf16][rng.integers(0, 3)]
+    x = rng.integers(-3, 4, dims)
+    strides = [int(np.prod(dims[d + 1:])) for d in range(rank)]
+    perm = rng.permutation(rank).tolist()
+    crop = [int(rng.integers(0, dims[a])) if rng.random() < 0.3 and dims[a] > 1 else 0 for a in range(rank)]  # first index kept, per storage axis
+    view_dims = [dims[a] - crop[a] for a in perm]
+    view_strides = [strides[a] for a in perm]
+    offset = sum(crop[a] * strides[a] for a in range(rank))
+    seen = x[tuple(slice(crop[a], None) for a in range(rank))].transpose(perm)
+    y = rng.integers(-3, 4, view_dims)
+    view = ex.input("x").strided_view(view_dims, view_strides, offset)
+    expr, want = view * ex.input("y") + view, seen * y + seen
+    text = f"x{dims} perm={perm} crop={crop}"
+    reduced = rng.random() < 0.6
+    if reduced:
+        axes = sorted(rng.choice(rank, int(rng.integers(1, rank + 1)), replace=False).tolist())
+        op = ["sum", "max", "min"][rng.integers(0, 3)]
+        if op == "sum" and int(np.prod([view_dims[a] for a in axes])) * 12 >= (1 << 24):
+            op = "max"
+        expr = {"sum": expr.reduce_sum, "max": expr.reduce_max, "min": expr.reduce_min}[op](axes)
+        want = {"sum": np.sum, "max": np.max, "min": np.min}[op](want, axis=tuple(axes), keepdims=True)
+        text += f" {op}{axes}"
+    print(f"{dtype.name} {text}", flush=True)
+    plan, outs = run_staged(expr, {"x": to_storage(x.astype(np.float32), dtype), "y": to_storage(y.astype(np.float32), dtype)}, dtype)
+    got = outs["output"]
+    got = got.astype(np.float64) if reduced else from_storage(got, dtype).astype(np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    np.testing.assert_array_equal(got, want.astype(np.float64), err_msg=str(plan.stage_descriptions()))
+    return " | ".join(plan.stage_kind_names())
+
+
+FAMILIES = {"views": views_case, "expressions": expressions_case, "conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
 
 if __name__ == "__main__":
     if len(sys.argv) != 4 or sys.argv[1] not in FAMILIES:
