@@ -1,7 +1,7 @@
 """Random differential runs of the GPU kernels against the oracle, outside the collected suite (every case compiles its own kernels,
 0.3-1 s each on a cold box):
 
-    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: views | expressions | conversions | topk | topk_rows | scans | reductions | rows
+    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: ragged | rope | views | expressions | conversions | topk | topk_rows | scans | reductions | rows
 
 Shapes, dtypes, operations, orders and data kinds (normal, few levels, sorted either way, a narrow band, outliers over zeros, NaN /
 inf / signed zeros, a repeated block) are drawn at random; every case is printed before it runs and checked with the same helper
@@ -362,7 +362,52 @@ def views_case(rng, stream):
     return " | ".join(plan.stage_kind_names())
 
 
-FAMILIES = {"views": views_case, "expressions": expressions_case, "conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
+def ragged_case(rng, stream):
+    """Ragged softmax / centering through the expression planner and the segmented broadcast, on random partitions."""
+    import test_ragged_expression_gpu as RE
+    import test_segmented_broadcast_gpu as SB
+    rank = int(rng.integers(1, 4))
+    rest = tuple(int(2 ** rng.uniform(0, 5)) for _ in range(rank - 1))
+    rows = int(2 ** rng.uniform(5, 17))
+    while rows * int(np.prod(rest or (1,))) > (1 << 20):
+        rows //= 2
+    shape = (max(rows, 32),) + rest
+    segments = int(max(2, min(2 ** rng.uniform(1, 13), shape[0] // 2)))
+    if rng.random() < 0.5:
+        dtype = [DataType.fp32, DataType.bf16][rng.integers(0, 2)]
+        print(f"softmax and centering shape={shape} segments={segments} {dtype.name}", flush=True)
+        RE.test_random_ragged_softmax_and_centering_against_numpy(stream, shape, segments, dtype)
+    else:
+        dtype = [DataType.fp32, DataType.bf16, DataType.fp16, DataType.fp8_e4m3, DataType.fp8_e5m2][rng.integers(0, 5)]
+        print(f"broadcast shape={shape} segments={segments} {dtype.name}", flush=True)
+        SB.test_broadcast_matches_a_loop_over_segments(stream, shape, segments, dtype)
+    return ""
+
+
+def rope_case(rng, stream):
+    import test_expression_rope_gpu as RP
+    head = int(rng.integers(1, 65)) * 2
+    options = {}
+    if rng.random() < 0.5:
+        shape = (int(rng.integers(1, 4)), int(rng.integers(1, 6)), int(2 ** rng.uniform(0, 9)), head)
+    else:
+        shape = (int(rng.integers(1, 4)), int(2 ** rng.uniform(0, 9)), int(rng.integers(1, 6)), head)
+        options.update(sequence_axis=1, head_dim_axis=3)
+    if rng.random() < 0.4:
+        options["rotary_dim"] = int(rng.integers(1, head // 2 + 1)) * 2
+    if rng.random() < 0.4:
+        options["interleaved"] = True
+    if rng.random() < 0.3:
+        options["inverse"] = True
+    if rng.random() < 0.4:
+        options["position_offset"] = int(rng.integers(0, 100))
+    dtype = [DataType.fp32, DataType.fp16, DataType.bf16][rng.integers(0, 3)]
+    print(f"{dtype.name} shape={shape} {options}", flush=True)
+    RP.test_layouts_against_the_oracle(stream, shape, options, dtype)
+    return ""
+
+
+FAMILIES = {"ragged": ragged_case, "rope": rope_case, "views": views_case, "expressions": expressions_case, "conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
 
 if __name__ == "__main__":
     if len(sys.argv) != 4 or sys.argv[1] not in FAMILIES:
