@@ -1,7 +1,7 @@
 """Random differential runs of the GPU kernels against the oracle, outside the collected suite (every case compiles its own kernels,
 0.3-1 s each on a cold box):
 
-    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: ragged | rope | views | expressions | conversions | topk | topk_rows | scans | reductions | rows
+    python tests/soak_against_oracle.py FAMILY SEED CASES      FAMILY: backward | ragged | rope | views | expressions | conversions | topk | topk_rows | scans | reductions | rows
 
 Shapes, dtypes, operations, orders and data kinds (normal, few levels, sorted either way, a narrow band, outliers over zeros, NaN /
 inf / signed zeros, a repeated block) are drawn at random; every case is printed before it runs and checked with the same helper
@@ -407,7 +407,96 @@ def rope_case(rng, stream):
     return ""
 
 
-FAMILIES = {"ragged": ragged_case, "rope": rope_case, "views": views_case, "expressions": expressions_case, "conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
+def backward_case(rng, stream):
+    """Gradients of random polynomial graphs over broadcast operands (exact in fp32 on small integers), and of min / max reductions
+    over rows of distinct values, against a reverse-mode walk in NumPy."""
+    import test_expression_backward_gpu as B
+    ex = ph.Expression
+    rank = int(rng.integers(1, 4))
+    left = 2 ** rng.uniform(0, 16)
+    dims = []
+    for d in range(rank):
+        extent = int(max(1, round(left if d == rank - 1 else 2 ** rng.uniform(0, np.log2(max(left, 1.0001))))))
+        dims.append(extent)
+        left = max(left / extent, 1)
+    total = int(np.prod(dims))
+
+    def unbroadcast(g, shape):
+        axes = tuple(a for a in range(len(shape)) if shape[a] == 1 and g.shape[a] != 1)
+        return g.sum(axis=axes, keepdims=True) if axes else g
+
+    if rng.random() < 0.3:
+        # the gradient of a max / min over some axes goes to the one winner of every reduced group (distinct values: no ties)
+        x = rng.permutation(total).reshape(dims).astype(np.int64) - total // 2
+        if total >= (1 << 23):
+            return ""
+        axes = sorted(rng.choice(rank, int(rng.integers(1, rank + 1)), replace=False).tolist())
+        scale = int(rng.choice([1, -1, 2]))
+        kind = ["max", "min"][rng.integers(0, 2)]
+        value = ex.input("x") * float(scale) + 1.0
+        forward = value.reduce_max(axes) if kind == "max" else value.reduce_min(axes)
+        seen = x * scale + 1
+        best = (np.max if kind == "max" else np.min)(seen, axis=tuple(axes), keepdims=True)
+        upstream = rng.integers(-3, 4, best.shape)
+        want = {"x_grad": (seen == best) * upstream * scale}
+        print(f"{kind}{axes} of x{dims} * {scale} + 1", flush=True)
+        plan, got, _, _ = B.backward(forward, {"x": x.astype(np.float32), "e": upstream.astype(np.float32)}, stream, ["x"], upstream="e")
+    else:
+        names = "abc"[:int(rng.integers(2, 4))]
+        values = {}
+        nodes = []  # (expression, value, parents as (node index, function of the node's gradient -> the parent's share))
+        for i, name in enumerate(names):
+            shape = [e if i == 0 or rng.random() < 0.7 else 1 for e in dims]
+            values[name] = rng.integers(-3, 4, shape).astype(np.int64)
+            nodes.append((ex.input(name), values[name], [], 3))
+        text = list(names)
+        for _ in range(int(rng.integers(1, 5))):
+            i, j = int(rng.integers(0, len(nodes))), int(rng.integers(0, len(nodes)))
+            (x, xv, _, xb), (y, yv, _, yb) = nodes[i], nodes[j]
+            op = ["add", "sub", "mul", "neg"][rng.integers(0, 4)]
+            if op == "mul" and xb * yb > 60 or op in ("add", "sub") and xb + yb > 60:
+                op = "neg"
+            if op == "add":
+                node = (x + y, xv + yv, [(i, lambda g: g), (j, lambda g: g)], xb + yb)
+            elif op == "sub":
+                node = (x - y, xv - yv, [(i, lambda g: g), (j, lambda g: -g)], xb + yb)
+            elif op == "mul":
+                node = (x * y, xv * yv, [(i, lambda g, yv=yv: g * yv), (j, lambda g, xv=xv: g * xv)], xb * yb)
+            else:
+                node = (-x, -xv, [(i, lambda g: -g)], xb)
+            nodes.append(node)
+            text.append(f"{op}({text[i]},{text[j]})" if op != "neg" else f"neg({text[i]})")
+        for k, name in enumerate(names):  # every input takes part
+            last = len(nodes) - 1
+            x, xv, _, xb = nodes[last]
+            y, yv, _, yb = nodes[k]
+            nodes.append((x + y, xv + yv, [(last, lambda g: g), (k, lambda g: g)], xb + yb))
+            text.append(f"add({text[last]},{name})")
+        forward, out_value = nodes[-1][0], nodes[-1][1]
+        out_shape = np.broadcast_shapes(*[values[n].shape for n in names])
+        upstream = rng.integers(-2, 3, out_shape).astype(np.int64)
+        grads = [None] * len(nodes)
+        grads[-1] = upstream
+        for index in range(len(nodes) - 1, -1, -1):
+            if grads[index] is None:
+                continue
+            for parent, share in nodes[index][2]:
+                g = unbroadcast(share(grads[index]), nodes[parent][1].shape)
+                grads[parent] = g if grads[parent] is None else grads[parent] + g
+        want = {name + "_grad": grads[k] for k, name in enumerate(names)}
+        if max(int(np.abs(g).max()) for g in want.values()) >= (1 << 24):
+            return ""
+        print(f"dims={dims} shapes={[list(values[n].shape) for n in names]} {text[-1]}", flush=True)
+        arrays = {n: values[n].astype(np.float32) for n in names}
+        arrays["e"] = upstream.astype(np.float32)
+        plan, got, _, _ = B.backward(forward, arrays, stream, list(names), upstream="e")
+    for name, expected in want.items():
+        assert got[name].shape == expected.shape, (name, got[name].shape, expected.shape)
+        np.testing.assert_array_equal(got[name], expected.astype(np.float64), err_msg=f"{name} {plan.stage_descriptions()}")
+    return " | ".join(plan.stage_kind_names())
+
+
+FAMILIES = {"backward": backward_case, "ragged": ragged_case, "rope": rope_case, "views": views_case, "expressions": expressions_case, "conversions": conversions_case, "topk": topk_case, "topk_rows": topk_rows_case, "scans": scans_case, "reductions": reductions_case, "rows": rows_case}
 
 if __name__ == "__main__":
     if len(sys.argv) != 4 or sys.argv[1] not in FAMILIES:
