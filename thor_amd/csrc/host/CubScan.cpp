@@ -143,7 +143,7 @@ std::string requestKey(const ScanRequest& r) {
                   (unsigned long long)r.row, (unsigned long long)r.segments, r.offsets64 ? 1 : 0, r.op, r.writeValue ? 1 : 0, r.writeIndex ? 1 : 0,
                   r.inclusive ? 1 : 0, r.reverse ? 1 : 0, r.route ? 1 : 0, (unsigned long long)r.alignmentBytes, r.deviceNum,
                   switchText("THOR_SCAN_WAIT_LIMIT"), switchText("THOR_SCAN_THREADS"), switchText("THOR_SCAN_PASSES"));
-    return text;
+    return std::string(text) + "|" + switchText("THOR_SCAN_MIN_WAVES");
 }
 LruCacheThreadSafe<std::string, std::shared_ptr<const CubScanKernels>>& builtScans() {
     static LruCacheThreadSafe<std::string, std::shared_ptr<const CubScanKernels>> cache(1024);
@@ -231,7 +231,15 @@ std::shared_ptr<const CubScanKernels> buildScanKernelsUncached(const ScanRequest
     s << thor_embed::kDevicePrelude << thor_embed::kScanKernels;
     writeScanTraits(s, r, isUnsigned, threads, vec, items, chunkElems, k);
 
-    s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void thor_scan_main(const gen::Cfg::T* in, const thor::u32* heads, const void* carries, "
+    // Blocks of 1 024 threads whose chunks wait for each other: two of them fit a compute unit only within 64 vector registers.  The
+    // head-aware value scans take about 93 and then run one block per compute unit, with nothing to cover a block's wait; asked
+    // for eight wavefronts per SIMD the compiler spills a few registers instead (ragged running sum of 2^26 fp32: 137 -> 126 us;
+    // kernels that fit anyway are unchanged).  Arg scans hold twice the state and are left alone, and with smaller blocks the
+    // bound costs more than it gives (512 threads: 137 -> 209 us).  THOR_SCAN_MIN_WAVES=<n> asks for n, 0 for no bound.
+    int minWaves = k.lookback && threads == 1024 && !r.writeIndex ? 8 : 0;
+    if (const char* env = std::getenv("THOR_SCAN_MIN_WAVES")) minWaves = std::atoi(env);
+    s << "extern \"C\" __global__ __launch_bounds__(" << threads << (minWaves > 0 ? ", " + std::to_string(minWaves) : std::string())
+      << ") void thor_scan_main(const gen::Cfg::T* in, const thor::u32* heads, const void* carries, "
          "gen::Cfg::T* outValue, thor::u32* outIndex) {\n    thor::scanChunk<gen::Cfg, false>(in, heads, carries, nullptr, outValue, outIndex);\n}\n";
     if (k.carry && !k.lookback) {
         s << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void thor_scan_totals(const gen::Cfg::T* in, const thor::u32* heads, void* totals) {\n"
