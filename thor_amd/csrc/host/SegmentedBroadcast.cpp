@@ -127,7 +127,9 @@ std::shared_ptr<StampedSegmentedBroadcast> stampImpl(const Tensor& per_segment_v
           << ";\n    static constexpr bool kNormalize = " << (normalize_by_segment_length ? "true" : "false")
           << ";\n    static constexpr bool kViaHalf = " << (dtype == DataType::FP8_E5M2 ? "true" : "false") << ";\n    static constexpr bool kIds = "
           << (ids ? "true" : "false") << ";\n};\n}  // namespace gen\n";
-        s << "extern \"C\" __global__ __launch_bounds__(256) void thor_segmented_broadcast(const gen::Cfg::T* values, const void* offsets, gen::Cfg::T* out) "
+        // eight wavefronts per SIMD: the fp32 form takes 65 vector registers unasked, one more than eight resident wavefronts allow
+        // (2^26 rows in 65 536 segments, four alternating runs on one device: 181-186 -> 170-172 us)
+        s << "extern \"C\" __global__ __launch_bounds__(256, 8) void thor_segmented_broadcast(const gen::Cfg::T* values, const void* offsets, gen::Cfg::T* out) "
              "{\n    thor::broadcastSegments<gen::Cfg>(values, static_cast<const gen::Cfg::OffsetT*>(offsets), out);\n}\n";
         kernel = compileKernel(s.str(), "thor_segmented_broadcast", stream.getGpuNum(), /*fastContract=*/false);
         kernel = builtKernels.getOrCreate(key.str(), [&] { return kernel; });
