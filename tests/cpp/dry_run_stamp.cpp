@@ -5,6 +5,7 @@
 // in-process compiler aborts the process, so each case prints its name first.
 #include "thorhip.h"
 
+#include "Utilities/Expression/CompiledEquation.h"
 #include "Utilities/Expression/FusedEquation.h"
 #include "Utilities/Expression/RaggedExpression.h"
 #include "Utilities/TensorOperations/Cub/CubDevicePrimitives.h"
@@ -14,6 +15,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -328,6 +330,29 @@ static int runAll() {
         Tensor odd(gpuPlacement, TensorDescriptor(dtype, {300, 1001}));
         primitive(std::string("column sum over an inner extent of 1001 ") + dtypeName, [&] { (void)CubReduction(CubReductionOp::Sum, {0}, DataType::FP32).stamp(odd, stream); });
         primitive(std::string("column arg-max over an inner extent of 1001 ") + dtypeName, [&] { (void)CubArgReduction(CubArgReductionOp::ArgMax, {0}).stamp(odd, stream); });
+    }
+    // A kernel whose machine code shifts 64 bits by an amount held in a vector register numbered 8n+7 must be refused when it is
+    // loaded (the device computes that shift wrong when the register is the last one a wavefront owns); the same kernel with the
+    // amount one register lower must load.
+    {
+        const auto shifting = [](int amountRegister) {
+            const std::string reg = "v" + std::to_string(amountRegister);
+            return "extern \"C\" __global__ void shift_probe(unsigned long long* out) {\n    unsigned long long r;\n    const unsigned lane = threadIdx.x & 63u;\n"
+                   "    asm volatile(\"v_mov_b32 " + reg + ", %1\\n s_nop 4\\n v_lshlrev_b64 %0, " + reg + ", -1\" : \"=&v\"(r) : \"v\"(lane) : \"" + reg +
+                   "\");\n    out[threadIdx.x] = r;\n}\n";
+        };
+        std::printf("[ RUN  ] a 64-bit shift by v14 loads, by v15 is refused\n");
+        (void)compileKernel(shifting(14), "shift_probe", 0, false);
+        bool refused = false;
+        try {
+            (void)compileKernel(shifting(15), "shift_probe", 0, false);
+        } catch (const std::runtime_error& e) {
+            refused = std::string(e.what()).find("64-bit vector shift") != std::string::npos;
+        }
+        if (!refused) {
+            std::printf("  a kernel with v_lshlrev_b64 by v15 was loaded\n");
+            return 1;
+        }
     }
     std::printf("%d expressions stamped, 0 failures\n", stamped);
     return 0;
