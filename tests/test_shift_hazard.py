@@ -37,3 +37,27 @@ def test_no_ahead_of_time_kernel_shifts_64_bits_by_a_vector_register():
     assert amounts.size > 100, "the library's gfx950 code is expected to be stored uncompressed (shifts by constants were always found)"
     in_registers = amounts[amounts >= 256] - 256
     assert in_registers.size == 0, f"64-bit vector shifts by register amounts: v{sorted(set(in_registers.tolist()))}"
+
+
+def u64_to_f32_through_halves(values):
+    """The steps of the device's u64ToF32 (thorhip_numeric.h), one NumPy operation per device operation: the high half normalised
+    with 32-bit shifts, the bits that do not fit 32 folded into a sticky bit, one rounding 32-bit conversion, exact scaling."""
+    values = np.asarray(values, np.uint64)
+    hi, lo = (values >> np.uint64(32)).astype(np.uint32), (values & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+    lz = np.where(hi == 0, 0, 31 - np.floor(np.log2(np.maximum(hi, 1).astype(np.float64))).astype(np.int64)).astype(np.uint32)
+    shifted_in = np.where(lz == 0, np.uint32(0), lo >> (np.uint32(32) - np.maximum(lz, 1)).astype(np.uint32))
+    top = ((hi << lz) | shifted_in).astype(np.uint32)
+    rest = (lo << lz).astype(np.uint32)
+    rounded = (top | (rest != 0).astype(np.uint32)).astype(np.float32)  # uint32 -> float32 rounds to nearest even
+    wide = np.ldexp(rounded, (32 - lz.astype(np.int64)).astype(np.int32)).astype(np.float32)
+    return np.where(hi == 0, lo.astype(np.float32), wide)
+
+
+def test_the_conversion_through_32_bit_halves_rounds_like_the_cast():
+    rng = np.random.default_rng(5)
+    width = rng.integers(1, 65, 200000).astype(np.uint64)
+    random = (rng.integers(0, 1 << 63, 200000, dtype=np.uint64) * np.uint64(2) + rng.integers(0, 2, 200000).astype(np.uint64)) >> (np.uint64(64) - width)
+    ties = [(1 << e) + (k << (e - 24)) + d for e in range(24, 64) for k in (1, 3, 5, 7) for d in (-1, 0, 1) if (1 << e) + (k << (e - 24)) + d < (1 << 64)]
+    edges = [0, 1, (1 << 24) - 1, 1 << 24, (1 << 32) - 1, 1 << 32, (1 << 32) + 1, (1 << 63), (1 << 64) - 1, (1 << 64) - (1 << 39), (1 << 64) - (1 << 39) - 1]
+    values = np.concatenate([random, np.array(ties + edges, np.uint64)])
+    np.testing.assert_array_equal(u64_to_f32_through_halves(values).view(np.uint32), values.astype(np.float32).view(np.uint32))
